@@ -1,0 +1,39 @@
+/*
+ * aclnnGridSampler2D -- two-phase C API, MI355X (gfx950) implementation.
+ *
+ * Drop-in for the reference interface image/grid_sample/op_api/aclnn_grid_sampler2d.h:53-82
+ * (implementation image/grid_sample/op_api/aclnn_grid_sampler2d.cpp:263-351).
+ *
+ * out[n,c,h,w] = sample(input[n,c,:,:], grid[n,h,w,:]) with grid in normalized [-1,1] coordinates
+ * (x first, then y).
+ *   interpolationMode : 0 bilinear, 1 nearest (2 = bicubic is validated but not implemented: 161002)
+ *   paddingMode       : 0 zeros, 1 border, 2 reflection
+ *   dtypes            : FLOAT, FLOAT16, BF16 (all three tensors equal); DOUBLE is rejected with 161002
+ *   shapes            : input (N,C,Hin,Win), grid (N,Hout,Wout,2), out (N,C,Hout,Wout); formats are ignored
+ *   views             : arbitrary strides/offsets are honoured (packed through the workspace)
+ * Validation order and status codes follow aclnn_grid_sampler2d.cpp:159-175.
+ */
+#ifndef OPSCV_ACLNN_GRID_SAMPLER2D_H_
+#define OPSCV_ACLNN_GRID_SAMPLER2D_H_
+
+#include "opscv_acl_base.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Phase 1 (host only, touches no device): validate, plan, report workspace bytes, hand out the executor. */
+ACLNN_API aclnnStatus aclnnGridSampler2DGetWorkspaceSize(const aclTensor* input, const aclTensor* grid,
+                                                         int64_t interpolationMode, int64_t paddingMode,
+                                                         bool alignCorners, aclTensor* out, uint64_t* workspaceSize,
+                                                         aclOpExecutor** executor);
+
+/* Phase 2: enqueue the kernels on `stream` (a hipStream_t) and free the executor.  Asynchronous. */
+ACLNN_API aclnnStatus aclnnGridSampler2D(void* workspace, uint64_t workspaceSize, aclOpExecutor* executor,
+                                         aclrtStream stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* OPSCV_ACLNN_GRID_SAMPLER2D_H_ */

@@ -1,0 +1,138 @@
+// Internal definitions behind the opaque ACL handles, the executor and the error-message channel.
+#pragma once
+
+#include <cstdarg>
+#include <cstdint>
+#include <vector>
+
+#include "opscv_acl_base.h"
+
+constexpr int kMaxDims = 8;
+
+struct aclTensor {
+    int64_t ndim = 0;
+    int64_t dims[kMaxDims] = {0};
+    int64_t strides[kMaxDims] = {0};  // in elements
+    int64_t offset = 0;               // in elements
+    aclDataType dtype = ACL_DT_UNDEFINED;
+    aclFormat format = ACL_FORMAT_ND;
+    int64_t storage_ndim = 0;
+    int64_t storage_dims[kMaxDims] = {0};
+    void* data = nullptr;
+
+    int64_t numel() const
+    {
+        int64_t n = 1;
+        for (int64_t i = 0; i < ndim; i++) {
+            n *= dims[i];
+        }
+        return n;
+    }
+    bool empty() const { return numel() == 0; }
+    bool contiguous() const
+    {
+        int64_t expect = 1;
+        for (int64_t i = ndim - 1; i >= 0; i--) {
+            if (dims[i] != 1 && strides[i] != expect) {
+                return false;
+            }
+            expect *= dims[i];
+        }
+        return true;
+    }
+};
+
+struct aclIntArray {
+    std::vector<int64_t> v;
+};
+
+struct aclFloatArray {
+    std::vector<float> v;
+};
+
+namespace opscv {
+
+enum class Elem : int { F32 = 0, F16 = 1, BF16 = 2 };
+
+inline int elem_size(Elem e) { return e == Elem::F32 ? 4 : 2; }
+
+// dtype -> element kind for the three types the kernels handle; false otherwise
+inline bool elem_of(aclDataType dt, Elem* e)
+{
+    switch (dt) {
+        case ACL_FLOAT: *e = Elem::F32; return true;
+        case ACL_FLOAT16: *e = Elem::F16; return true;
+        case ACL_BF16: *e = Elem::BF16; return true;
+        default: return false;
+    }
+}
+
+// A 4-D strided view that has to be packed into (or scattered from) a contiguous workspace slice.
+struct StridedView {
+    void* base = nullptr;      // tensor data pointer + offset, in bytes
+    int64_t dims[4] = {0};
+    int64_t strides[4] = {0};  // elements
+};
+
+enum class OpKind : int { Nop = 0, GridSampler2D = 1, Resize = 2 };
+
+// Where a kernel operand lives: the tensor's own memory (contiguous view) or a slice of the caller's
+// workspace, known only as an offset until the second phase receives the workspace address.
+struct PlannedPtr {
+    bool in_workspace = false;
+    uint64_t ws_offset = 0;
+    void* direct = nullptr;
+};
+
+struct GridSamplerArgs {
+    Elem elem = Elem::F32;
+    int interp = 0;
+    int pad = 0;
+    int align = 0;
+    int64_t N = 0, C = 0, Hin = 0, Win = 0, Hout = 0, Wout = 0;
+    const void* x = nullptr;
+    const void* grid = nullptr;
+    void* y = nullptr;
+};
+
+enum class ResizeMode : int { Bilinear = 0, Copy = 1, Broadcast = 2, FirstPixel = 3 };
+
+struct ResizeArgs {
+    Elem elem = Elem::F32;
+    ResizeMode mode = ResizeMode::Bilinear;
+    int half_pixel = 1;
+    int channels_last = 0;
+    float scale_h = 1.0f, scale_w = 1.0f;
+    int64_t N = 0, C = 0, Hs = 0, Ws = 0, Hd = 0, Wd = 0;
+    const void* x = nullptr;
+    void* y = nullptr;
+};
+
+}  // namespace opscv
+
+constexpr uint32_t kExecutorMagic = 0x0C5CA11Du;
+
+struct aclOpExecutor {
+    uint32_t magic = kExecutorMagic;
+    opscv::OpKind kind = opscv::OpKind::Nop;
+    uint64_t workspace_bytes = 0;
+    opscv::GridSamplerArgs gs;  // pointer members are filled in by the second phase
+    opscv::ResizeArgs rs;
+    opscv::PlannedPtr in0, in1, out0;  // input/self, grid, out
+    // packing work: views gathered into the workspace before the kernel, scattered after it
+    struct Pack {
+        opscv::StridedView view;
+        uint64_t ws_offset = 0;
+        int elem_bytes = 0;
+    };
+    std::vector<Pack> pack_in;
+    std::vector<Pack> unpack_out;
+};
+
+namespace opscv {
+
+// printf-style; stores the text for aclGetRecentErrMsg and, when OPSCV_LOG=1, prints it to stderr
+void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
+void clear_error();
+
+}  // namespace opscv

@@ -1,0 +1,170 @@
+// aclnnGridSampler2D: parameter validation, planning and the second-phase entry.
+//
+// Mirrors the checks, their order and their status codes of the reference implementation
+// image/grid_sample/op_api/aclnn_grid_sampler2d.cpp:55-175,263-351.
+#include <memory>
+#include <new>
+
+#include "aclnn_grid_sampler2d.h"
+#include "executor.hpp"
+
+using namespace opscv;
+
+namespace {
+
+constexpr int64_t kSpatialDims = 4;
+
+// aclnn_grid_sampler2d.cpp:78-92 : grid and out must match input's dtype; input's dtype must be in the list
+bool check_dtypes(const aclTensor* input, const aclTensor* grid, const aclTensor* out)
+{
+    if (grid->dtype != input->dtype) {
+        set_error("aclnnGridSampler2D: grid dtype %d differs from input dtype %d", (int)grid->dtype,
+                  (int)input->dtype);
+        return false;
+    }
+    if (out->dtype != input->dtype) {
+        set_error("aclnnGridSampler2D: out dtype %d differs from input dtype %d", (int)out->dtype,
+                  (int)input->dtype);
+        return false;
+    }
+    switch (input->dtype) {
+        case ACL_FLOAT:
+        case ACL_FLOAT16:
+        case ACL_BF16:
+        case ACL_DOUBLE: return true;
+        default: break;
+    }
+    set_error("aclnnGridSampler2D: dtype %d is not in {FLOAT, FLOAT16, BF16, DOUBLE}", (int)input->dtype);
+    return false;
+}
+
+// aclnn_grid_sampler2d.cpp:94-110
+bool check_attrs(int64_t interp, int64_t pad)
+{
+    if (interp < 0 || interp > 2) {
+        set_error("interpolationMode %lld should be in support list {0(bilinear), 1(nearest), 2(bicubic)}.",
+                  (long long)interp);
+        return false;
+    }
+    if (pad < 0 || pad > 2) {
+        set_error("paddingMode %lld should be in support list {0(zeros), 1(border), 2(reflection)}.",
+                  (long long)pad);
+        return false;
+    }
+    return true;
+}
+
+// aclnn_grid_sampler2d.cpp:112-157
+bool check_shapes(const aclTensor* input, const aclTensor* grid, const aclTensor* out)
+{
+    if (input->ndim != kSpatialDims || grid->ndim != kSpatialDims || out->ndim != kSpatialDims) {
+        set_error("aclnnGridSampler2D: input, grid and out must be 4-D, got %lld, %lld, %lld dims",
+                  (long long)input->ndim, (long long)grid->ndim, (long long)out->ndim);
+        return false;
+    }
+    if (input->dims[0] != grid->dims[0] || input->dims[0] != out->dims[0]) {
+        set_error("expect input, grid and out to have same batch size");
+        return false;
+    }
+    if (input->dims[1] != out->dims[1]) {
+        set_error("expect input and out to have same channel size");
+        return false;
+    }
+    if (grid->dims[1] != out->dims[2] || grid->dims[2] != out->dims[3]) {
+        set_error("expect grid and out to have same H and W size");
+        return false;
+    }
+    if (input->dims[2] == 0 || input->dims[3] == 0) {
+        set_error("expect input to have non-empty spatial dimensions");
+        return false;
+    }
+    if (grid->dims[3] != 2) {
+        set_error("expect grid to have size 2 in last dimension");
+        return false;
+    }
+    return true;
+}
+
+}  // namespace
+
+extern "C" {
+
+aclnnStatus aclnnGridSampler2DGetWorkspaceSize(const aclTensor* input, const aclTensor* grid,
+                                               int64_t interpolationMode, int64_t paddingMode, bool alignCorners,
+                                               aclTensor* out, uint64_t* workspaceSize, aclOpExecutor** executor)
+{
+    std::unique_ptr<aclOpExecutor> ex(new (std::nothrow) aclOpExecutor());
+    if (!ex) {
+        set_error("aclnnGridSampler2D: cannot allocate the executor");
+        return ACLNN_ERR_INNER_CREATE_EXECUTOR;
+    }
+    // 1. null pointers (aclnn_grid_sampler2d.cpp:55-61)
+    if (input == nullptr || grid == nullptr || out == nullptr) {
+        set_error("aclnnGridSampler2D: input, grid and out must not be NULL");
+        return ACLNN_ERR_PARAM_NULLPTR;
+    }
+    if (workspaceSize == nullptr || executor == nullptr) {
+        set_error("aclnnGridSampler2D: workspaceSize and executor must not be NULL");
+        return ACLNN_ERR_PARAM_NULLPTR;
+    }
+    // 2. dtypes, 3. attributes, 4. shapes
+    if (!check_dtypes(input, grid, out) || !check_attrs(interpolationMode, paddingMode) ||
+        !check_shapes(input, grid, out)) {
+        return ACLNN_ERR_PARAM_INVALID;
+    }
+    // empty tensors are a successful no-op that still hands out an executor (aclnn_grid_sampler2d.cpp:280-285)
+    if (input->empty() || grid->empty()) {
+        *workspaceSize = 0;
+        *executor = ex.release();
+        return ACLNN_SUCCESS;
+    }
+    // The reference routes DOUBLE to a host-CPU kernel that is not part of its tree and bicubic to a
+    // kernel outside this path; neither exists here.
+    Elem elem;
+    if (!elem_of(input->dtype, &elem)) {
+        set_error("aclnnGridSampler2D: DOUBLE tensors are not supported by the MI355X implementation");
+        return ACLNN_ERR_PARAM_INVALID;
+    }
+    if (interpolationMode == 2) {
+        set_error("aclnnGridSampler2D: bicubic interpolation is not supported by the MI355X implementation");
+        return ACLNN_ERR_PARAM_INVALID;
+    }
+    for (int i = 0; i < 4; i++) {
+        if (input->dims[i] > INT32_MAX || grid->dims[i] > INT32_MAX) {
+            set_error("aclnnGridSampler2D: every extent must fit in int32");
+            return ACLNN_ERR_PARAM_INVALID;
+        }
+    }
+    if (input->dims[2] * input->dims[3] > INT32_MAX) {
+        set_error("aclnnGridSampler2D: Hin*Win must fit in int32");
+        return ACLNN_ERR_PARAM_INVALID;
+    }
+
+    ex->kind = OpKind::GridSampler2D;
+    GridSamplerArgs& a = ex->gs;
+    a.elem = elem;
+    a.interp = (int)interpolationMode;
+    a.pad = (int)paddingMode;
+    a.align = alignCorners ? 1 : 0;
+    a.N = input->dims[0];
+    a.C = input->dims[1];
+    a.Hin = input->dims[2];
+    a.Win = input->dims[3];
+    a.Hout = grid->dims[1];
+    a.Wout = grid->dims[2];
+    const int esz = elem_size(elem);
+    ex->in0 = plan_view(ex.get(), input, esz, false);
+    ex->in1 = plan_view(ex.get(), grid, esz, false);
+    ex->out0 = plan_view(ex.get(), out, esz, true);
+
+    *workspaceSize = ex->workspace_bytes;
+    *executor = ex.release();
+    return ACLNN_SUCCESS;
+}
+
+aclnnStatus aclnnGridSampler2D(void* workspace, uint64_t workspaceSize, aclOpExecutor* executor, aclrtStream stream)
+{
+    return run_executor(workspace, workspaceSize, executor, stream, OpKind::GridSampler2D, "aclnnGridSampler2D");
+}
+
+}  // extern "C"

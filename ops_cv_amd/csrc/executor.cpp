@@ -1,0 +1,124 @@
+// Second-phase runner and view-packing plan shared by the aclnn entry points.
+#include "executor.hpp"
+
+#include <hip/hip_runtime_api.h>
+
+#include "kernels.hpp"
+
+namespace opscv {
+
+namespace {
+uint64_t align_up(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
+}  // namespace
+
+PlannedPtr plan_view(aclOpExecutor* ex, const aclTensor* t, int elem_bytes, bool is_output)
+{
+    PlannedPtr p;
+    char* base = (t->data == nullptr) ? nullptr : (char*)t->data + t->offset * (int64_t)elem_bytes;
+    if (t->contiguous()) {
+        p.direct = base;
+        return p;
+    }
+    aclOpExecutor::Pack pk;
+    pk.view.base = base;
+    for (int i = 0; i < 4; i++) {
+        pk.view.dims[i] = t->dims[i];
+        pk.view.strides[i] = t->strides[i];
+    }
+    pk.elem_bytes = elem_bytes;
+    pk.ws_offset = align_up(ex->workspace_bytes, 256);
+    ex->workspace_bytes = pk.ws_offset + (uint64_t)t->numel() * (uint64_t)elem_bytes;
+    p.in_workspace = true;
+    p.ws_offset = pk.ws_offset;
+    if (is_output) {
+        ex->unpack_out.push_back(pk);
+    } else {
+        ex->pack_in.push_back(pk);
+    }
+    return p;
+}
+
+aclnnStatus run_executor(void* workspace, uint64_t workspace_size, aclOpExecutor* ex, aclrtStream stream,
+                         OpKind expected, const char* api)
+{
+    if (ex == nullptr) {
+        set_error("%s: executor is NULL", api);
+        return ACLNN_ERR_PARAM_NULLPTR;
+    }
+    if (ex->magic != kExecutorMagic) {
+        set_error("%s: executor is not live (already consumed?)", api);
+        return ACLNN_ERR_PARAM_INVALID;
+    }
+    std::unique_ptr<aclOpExecutor> owner(ex);  // consumed whatever happens below
+    ex->magic = 0;
+    if (ex->kind != OpKind::Nop && ex->kind != expected) {
+        set_error("%s: executor was created by a different operator", api);
+        return ACLNN_ERR_PARAM_INVALID;
+    }
+    if (ex->workspace_bytes > 0) {
+        if (workspace == nullptr) {
+            set_error("%s: workspace is NULL but %llu bytes are required", api,
+                      (unsigned long long)ex->workspace_bytes);
+            return ACLNN_ERR_PARAM_NULLPTR;
+        }
+        if (workspace_size < ex->workspace_bytes) {
+            set_error("%s: workspace of %llu bytes is smaller than the %llu required", api,
+                      (unsigned long long)workspace_size, (unsigned long long)ex->workspace_bytes);
+            return ACLNN_ERR_PARAM_INVALID;
+        }
+    }
+    if (ex->kind == OpKind::Nop) {
+        return ACLNN_SUCCESS;
+    }
+    hipStream_t s = (hipStream_t)stream;
+    for (const auto& pk : ex->pack_in) {
+        if (pk.view.base == nullptr) {
+            set_error("%s: tensor data pointer is NULL", api);
+            return ACLNN_ERR_PARAM_NULLPTR;
+        }
+        hipError_t e = launch_strided_copy(pk.view, (char*)workspace + pk.ws_offset, pk.elem_bytes, true, s);
+        if (e != hipSuccess) {
+            set_error("%s: packing a strided input failed: %s", api, hipGetErrorString(e));
+            return ACLNN_ERR_RUNTIME_ERROR;
+        }
+    }
+    hipError_t e = hipSuccess;
+    if (ex->kind == OpKind::GridSampler2D) {
+        GridSamplerArgs a = ex->gs;
+        a.x = resolve(ex->in0, workspace);
+        a.grid = resolve(ex->in1, workspace);
+        a.y = resolve(ex->out0, workspace);
+        if (a.x == nullptr || a.grid == nullptr || a.y == nullptr) {
+            set_error("%s: tensor data pointer is NULL", api);
+            return ACLNN_ERR_PARAM_NULLPTR;
+        }
+        e = launch_grid_sampler2d(a, s);
+    } else {
+        ResizeArgs a = ex->rs;
+        a.x = resolve(ex->in0, workspace);
+        a.y = resolve(ex->out0, workspace);
+        if (a.x == nullptr || a.y == nullptr) {
+            set_error("%s: tensor data pointer is NULL", api);
+            return ACLNN_ERR_PARAM_NULLPTR;
+        }
+        e = launch_resize(a, s);
+    }
+    if (e != hipSuccess) {
+        set_error("%s: kernel launch failed: %s", api, hipGetErrorString(e));
+        return ACLNN_ERR_RUNTIME_ERROR;
+    }
+    for (const auto& pk : ex->unpack_out) {
+        if (pk.view.base == nullptr) {
+            set_error("%s: tensor data pointer is NULL", api);
+            return ACLNN_ERR_PARAM_NULLPTR;
+        }
+        e = launch_strided_copy(pk.view, (char*)workspace + pk.ws_offset, pk.elem_bytes, false, s);
+        if (e != hipSuccess) {
+            set_error("%s: scattering the strided output failed: %s", api, hipGetErrorString(e));
+            return ACLNN_ERR_RUNTIME_ERROR;
+        }
+    }
+    return ACLNN_SUCCESS;
+}
+
+}  // namespace opscv

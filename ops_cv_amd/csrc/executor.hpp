@@ -1,0 +1,25 @@
+// Shared pieces of the two-phase API: planning of view packing and the second-phase runner.
+#pragma once
+
+#include <memory>
+
+#include "acl_types.hpp"
+
+namespace opscv {
+
+// Chooses where the kernel operand for the 4-D tensor `t` lives: the tensor's own memory when the view is
+// contiguous, else a 256-byte aligned slice of the workspace; in that case a gather (input) or scatter
+// (output) step is queued on the executor and its workspace requirement grows.
+PlannedPtr plan_view(aclOpExecutor* ex, const aclTensor* t, int elem_bytes, bool is_output);
+
+inline void* resolve(const PlannedPtr& p, void* workspace)
+{
+    return p.in_workspace ? (void*)((char*)workspace + p.ws_offset) : p.direct;
+}
+
+// Second phase common to every operator: checks the executor and the workspace, gathers packed inputs,
+// launches the operator, scatters the packed output, frees the executor (always, also on failure).
+aclnnStatus run_executor(void* workspace, uint64_t workspace_size, aclOpExecutor* ex, aclrtStream stream,
+                         OpKind expected, const char* api);
+
+}  // namespace opscv

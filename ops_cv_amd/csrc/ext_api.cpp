@@ -1,0 +1,66 @@
+// Introspection entry points (no counterpart in the reference).
+#include "opscv_ext.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include "acl_types.hpp"
+#include "kernels.hpp"
+
+using namespace opscv;
+
+static_assert(sizeof(opscvTapRecord) == sizeof(TapRecord), "tap record layouts must match");
+
+extern "C" {
+
+aclnnStatus opscvGridSampler2DTaps(const void* grid, aclDataType dataType, int64_t N, int64_t Hin, int64_t Win,
+                                   int64_t Hout, int64_t Wout, int64_t interpolationMode, int64_t paddingMode,
+                                   bool alignCorners, opscvTapRecord* taps, aclrtStream stream)
+{
+    if (grid == nullptr || taps == nullptr) {
+        set_error("opscvGridSampler2DTaps: grid and taps must not be NULL");
+        return ACLNN_ERR_PARAM_NULLPTR;
+    }
+    GridSamplerArgs a;
+    if (!elem_of(dataType, &a.elem) || interpolationMode < 0 || interpolationMode > 1 || paddingMode < 0 ||
+        paddingMode > 2) {
+        set_error("opscvGridSampler2DTaps: unsupported dtype or mode");
+        return ACLNN_ERR_PARAM_INVALID;
+    }
+    a.interp = (int)interpolationMode;
+    a.pad = (int)paddingMode;
+    a.align = alignCorners ? 1 : 0;
+    a.N = N;
+    a.C = 1;
+    a.Hin = Hin;
+    a.Win = Win;
+    a.Hout = Hout;
+    a.Wout = Wout;
+    a.grid = grid;
+    hipError_t e = launch_grid_sampler2d_taps(a, (TapRecord*)taps, (hipStream_t)stream);
+    if (e == hipErrorInvalidValue) {
+        set_error("opscvGridSampler2DTaps: shapes out of range");
+        return ACLNN_ERR_PARAM_INVALID;
+    }
+    if (e != hipSuccess) {
+        set_error("opscvGridSampler2DTaps: launch failed: %s", hipGetErrorString(e));
+        return ACLNN_ERR_RUNTIME_ERROR;
+    }
+    return ACLNN_SUCCESS;
+}
+
+const char* opscvExecutorVariant(const aclOpExecutor* executor)
+{
+    if (executor == nullptr || executor->magic != kExecutorMagic) {
+        return "";
+    }
+    switch (executor->kind) {
+        case OpKind::GridSampler2D: return grid_sampler2d_variant(executor->gs);
+        case OpKind::Resize: return resize_variant(executor->rs);
+        default: break;
+    }
+    return "";
+}
+
+const char* opscvVersion(void) { return "opscv-amd 0.1 (gfx950)"; }
+
+}  // extern "C"

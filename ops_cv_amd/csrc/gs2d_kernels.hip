@@ -1,0 +1,261 @@
+// Grid sampler 2-D forward kernels for gfx950 (bilinear and nearest; zeros, border, reflection; align on/off).
+//
+// Replaces the reference device kernel image/grid_sampler2_d/op_kernel/arch35/grid_sampler2_d_simt.h:461-557 and
+// its host tiling image/grid_sampler2_d/op_host/arch35/grid_sampler2_d_tiling.cpp:208-271.
+//
+// Common shape of every variant: one lane owns one output pixel (n, h, w); the wavefront therefore reads a
+// contiguous run of grid values and writes a contiguous run of every output channel plane.  The source
+// coordinate, the four tap offsets, the four weights and the bounds masks are computed once and stay in
+// registers across the channel loop.
+#include <hip/hip_runtime.h>
+
+#include "kernels.hpp"
+#include "sampler_math.hpp"
+
+namespace opscv {
+
+namespace {
+
+constexpr int kDirectThreads = 256;
+
+// ---------------------------------------------------------------------------------------------------------
+// Direct variant: taps are read straight from global memory (through L1/L2).  Works for every shape.
+// ---------------------------------------------------------------------------------------------------------
+template <typename T, int INTERP, int PAD, bool ALIGN>
+__global__ __launch_bounds__(kDirectThreads) void gs2d_direct_kernel(const T* __restrict__ x,
+                                                                      const T* __restrict__ grid,
+                                                                      T* __restrict__ y, int64_t total_pixels,
+                                                                      int32_t C, int32_t H, int32_t W,
+                                                                      int64_t out_plane)
+{
+    const int64_t in_plane = (int64_t)H * W;
+    const int64_t stride = (int64_t)gridDim.x * kDirectThreads;
+    for (int64_t p = (int64_t)blockIdx.x * kDirectThreads + threadIdx.x; p < total_pixels; p += stride) {
+        const int64_t n = p / out_plane;
+        const int64_t rem = p - n * out_plane;
+        const float gx = ElemIO<T>::load(grid + 2 * p);
+        const float gy = ElemIO<T>::load(grid + 2 * p + 1);
+        const PixelTap t = decide_pixel<INTERP, PAD, ALIGN>(gx, gy, H, W);
+        const T* xp = x + n * C * in_plane;
+        T* yp = y + n * C * out_plane + rem;
+        if (INTERP == 0) {
+            if (t.flag) {
+                const float nan_val = __builtin_nanf("");
+                for (int32_t c = 0; c < C; c++) {
+                    ElemIO<T>::store(yp, nan_val);
+                    yp += out_plane;
+                }
+                continue;
+            }
+            const int32_t x0 = t.x0, y0 = t.y0;
+            const int32_t x1 = (x0 == INT32_MAX) ? x0 : x0 + 1;
+            const int32_t y1 = (y0 == INT32_MAX) ? y0 : y0 + 1;
+            const bool in_nw = within(y0, x0, H, W), in_ne = within(y0, x1, H, W);
+            const bool in_sw = within(y1, x0, H, W), in_se = within(y1, x1, H, W);
+            // offsets are only dereferenced under their mask; clamp them to 0 so that they are always valid
+            const int64_t o_nw = in_nw ? (int64_t)y0 * W + x0 : 0;
+            const int64_t o_ne = in_ne ? (int64_t)y0 * W + x1 : 0;
+            const int64_t o_sw = in_sw ? (int64_t)y1 * W + x0 : 0;
+            const int64_t o_se = in_se ? (int64_t)y1 * W + x1 : 0;
+#pragma unroll 4
+            for (int32_t c = 0; c < C; c++) {
+                // grid_sampler2_d_simt.h:321-338 : nw, ne, sw, se added in this order, skipped when outside
+                float out = 0.0f;
+                if (in_nw) {
+                    out += ElemIO<T>::load(xp + o_nw) * t.w[0];
+                }
+                if (in_ne) {
+                    out += ElemIO<T>::load(xp + o_ne) * t.w[1];
+                }
+                if (in_sw) {
+                    out += ElemIO<T>::load(xp + o_sw) * t.w[2];
+                }
+                if (in_se) {
+                    out += ElemIO<T>::load(xp + o_se) * t.w[3];
+                }
+                ElemIO<T>::store(yp, out);
+                xp += in_plane;
+                yp += out_plane;
+            }
+        } else {
+            const bool in = within(t.y0, t.x0, H, W);
+            const int64_t o = in ? (int64_t)t.y0 * W + t.x0 : 0;
+#pragma unroll 4
+            for (int32_t c = 0; c < C; c++) {
+                // grid_sampler2_d_simt.h:341-360 : the value passes through fp32, exact for 16-bit types
+                float out = 0.0f;
+                if (in) {
+                    out = ElemIO<T>::load(xp + o);
+                }
+                ElemIO<T>::store(yp, out);
+                xp += in_plane;
+                yp += out_plane;
+            }
+        }
+    }
+}
+
+template <typename T, int INTERP, int PAD, bool ALIGN>
+__global__ __launch_bounds__(kDirectThreads) void gs2d_taps_kernel(const T* __restrict__ grid,
+                                                                    TapRecord* __restrict__ taps,
+                                                                    int64_t total_pixels, int32_t H, int32_t W)
+{
+    const int64_t stride = (int64_t)gridDim.x * kDirectThreads;
+    for (int64_t p = (int64_t)blockIdx.x * kDirectThreads + threadIdx.x; p < total_pixels; p += stride) {
+        const float gx = ElemIO<T>::load(grid + 2 * p);
+        const float gy = ElemIO<T>::load(grid + 2 * p + 1);
+        const PixelTap t = decide_pixel<INTERP, PAD, ALIGN>(gx, gy, H, W);
+        TapRecord r;
+        r.x0 = t.x0;
+        r.y0 = t.y0;
+        r.w[0] = t.w[0];
+        r.w[1] = t.w[1];
+        r.w[2] = t.w[2];
+        r.w[3] = t.w[3];
+        r.flag = t.flag;
+        taps[p] = r;
+    }
+}
+
+inline int blocks_for(int64_t items, int threads)
+{
+    int64_t b = (items + threads - 1) / threads;
+    const int64_t cap = 256 * 64;  // 256 CUs; enough resident waves, the loops are grid-stride
+    if (b > cap) {
+        b = cap;
+    }
+    if (b < 1) {
+        b = 1;
+    }
+    return (int)b;
+}
+
+template <typename T, int INTERP, int PAD, bool ALIGN>
+hipError_t run_direct(const GridSamplerArgs& a, hipStream_t stream)
+{
+    const int64_t total = a.N * a.Hout * a.Wout;
+    hipLaunchKernelGGL((gs2d_direct_kernel<T, INTERP, PAD, ALIGN>), dim3(blocks_for(total, kDirectThreads)),
+                       dim3(kDirectThreads), 0, stream, (const T*)a.x, (const T*)a.grid, (T*)a.y, total,
+                       (int32_t)a.C, (int32_t)a.Hin, (int32_t)a.Win, a.Hout * a.Wout);
+    return hipGetLastError();
+}
+
+template <typename T, int INTERP, int PAD, bool ALIGN>
+hipError_t run_taps(const GridSamplerArgs& a, TapRecord* taps, hipStream_t stream)
+{
+    const int64_t total = a.N * a.Hout * a.Wout;
+    hipLaunchKernelGGL((gs2d_taps_kernel<T, INTERP, PAD, ALIGN>), dim3(blocks_for(total, kDirectThreads)),
+                       dim3(kDirectThreads), 0, stream, (const T*)a.grid, taps, total, (int32_t)a.Hin,
+                       (int32_t)a.Win);
+    return hipGetLastError();
+}
+
+// Expands the run-time (interp, pad, align) triple into the template instantiation.
+template <typename T, typename F>
+hipError_t dispatch_modes(const GridSamplerArgs& a, F&& f)
+{
+#define OPSCV_CASE(I, P, A)                                   \
+    if (a.interp == I && a.pad == P && (a.align != 0) == A) { \
+        return f.template operator()<T, I, P, A>();           \
+    }
+    OPSCV_CASE(0, 0, false)
+    OPSCV_CASE(0, 0, true)
+    OPSCV_CASE(0, 1, false)
+    OPSCV_CASE(0, 1, true)
+    OPSCV_CASE(0, 2, false)
+    OPSCV_CASE(0, 2, true)
+    OPSCV_CASE(1, 0, false)
+    OPSCV_CASE(1, 0, true)
+    OPSCV_CASE(1, 1, false)
+    OPSCV_CASE(1, 1, true)
+    OPSCV_CASE(1, 2, false)
+    OPSCV_CASE(1, 2, true)
+#undef OPSCV_CASE
+    return hipErrorInvalidValue;
+}
+
+template <typename F>
+hipError_t dispatch_elem(const GridSamplerArgs& a, F&& f)
+{
+    switch (a.elem) {
+        case Elem::F32: return dispatch_modes<float>(a, f);
+        case Elem::F16: return dispatch_modes<_Float16>(a, f);
+        case Elem::BF16: return dispatch_modes<__bf16>(a, f);
+    }
+    return hipErrorInvalidValue;
+}
+
+// Shape limits shared by every variant (the reference tiling enforces the same ones,
+// grid_sampler2_d_tiling.cpp:92-156): every extent and the input plane fit in int32.
+bool shapes_ok(const GridSamplerArgs& a)
+{
+    if (a.N < 0 || a.C < 0 || a.Hout < 0 || a.Wout < 0 || a.Hin <= 0 || a.Win <= 0) {
+        return false;
+    }
+    const int64_t lim = INT32_MAX;
+    if (a.N > lim || a.C > lim || a.Hin > lim || a.Win > lim || a.Hout > lim || a.Wout > lim) {
+        return false;
+    }
+    if (a.Hin * a.Win > lim) {
+        return false;
+    }
+    if (a.Hout != 0 && a.Wout != 0 && a.Hout > INT64_MAX / a.Wout / (a.N > 0 ? a.N : 1) / 2) {
+        return false;
+    }
+    return true;
+}
+
+struct DirectLauncher {
+    const GridSamplerArgs& a;
+    hipStream_t stream;
+    template <typename T, int I, int P, bool A>
+    hipError_t operator()() const
+    {
+        return run_direct<T, I, P, A>(a, stream);
+    }
+};
+
+struct TapsLauncher {
+    const GridSamplerArgs& a;
+    TapRecord* taps;
+    hipStream_t stream;
+    template <typename T, int I, int P, bool A>
+    hipError_t operator()() const
+    {
+        return run_taps<T, I, P, A>(a, taps, stream);
+    }
+};
+
+}  // namespace
+
+const char* grid_sampler2d_variant(const GridSamplerArgs&) { return "direct"; }
+
+hipError_t launch_grid_sampler2d(const GridSamplerArgs& a, hipStream_t stream)
+{
+    if (!shapes_ok(a) || a.interp < 0 || a.interp > 1 || a.pad < 0 || a.pad > 2) {
+        return hipErrorInvalidValue;
+    }
+    if (a.N == 0 || a.C == 0 || a.Hout == 0 || a.Wout == 0) {
+        return hipSuccess;
+    }
+    if (a.x == nullptr || a.grid == nullptr || a.y == nullptr) {
+        return hipErrorInvalidValue;
+    }
+    return dispatch_elem(a, DirectLauncher{a, stream});
+}
+
+hipError_t launch_grid_sampler2d_taps(const GridSamplerArgs& a, TapRecord* taps, hipStream_t stream)
+{
+    if (!shapes_ok(a) || a.interp < 0 || a.interp > 1 || a.pad < 0 || a.pad > 2) {
+        return hipErrorInvalidValue;
+    }
+    if (a.N == 0 || a.Hout == 0 || a.Wout == 0) {
+        return hipSuccess;
+    }
+    if (a.grid == nullptr || taps == nullptr) {
+        return hipErrorInvalidValue;
+    }
+    return dispatch_elem(a, TapsLauncher{a, taps, stream});
+}
+
+}  // namespace opscv

@@ -1,0 +1,32 @@
+// Launch interface between the aclnn host layer and the HIP kernels.
+#pragma once
+
+#include <hip/hip_runtime_api.h>
+
+#include "acl_types.hpp"
+
+namespace opscv {
+
+// Record written per output pixel by the tap-dump kernel (28 bytes, no padding).
+struct TapRecord {
+    int32_t x0;
+    int32_t y0;
+    float w[4];
+    int32_t flag;
+};
+
+// All tensors contiguous.  Each launcher validates the shapes against what its kernels assume and
+// returns hipErrorInvalidValue instead of launching when they do not fit.
+hipError_t launch_grid_sampler2d(const GridSamplerArgs& a, hipStream_t stream);
+hipError_t launch_grid_sampler2d_taps(const GridSamplerArgs& a, TapRecord* taps, hipStream_t stream);
+hipError_t launch_resize(const ResizeArgs& a, hipStream_t stream);
+
+// gather == true : strided view -> contiguous buffer;  false : contiguous buffer -> strided view
+hipError_t launch_strided_copy(const StridedView& v, void* contiguous, int elem_bytes, bool gather,
+                               hipStream_t stream);
+
+// Name of the kernel variant the launcher would pick for these arguments (for benchmarks and tests).
+const char* grid_sampler2d_variant(const GridSamplerArgs& a);
+const char* resize_variant(const ResizeArgs& a);
+
+}  // namespace opscv

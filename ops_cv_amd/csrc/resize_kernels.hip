@@ -1,0 +1,220 @@
+// Bilinear resize / upsample forward kernels for gfx950.
+//
+// Replaces the reference device kernels image/resize_bilinear_v2/op_kernel/arch35/resize_bilinear_v2_simt_nchw.h:77-146
+// (and the copy / broadcast templates selected in image/resize_bilinear_v2/op_kernel/resize_bilinear_v2_apt.cpp:42-115)
+// and the host tiling image/resize_bilinear_v2/op_host/arch35/resize_bilinear_v2_tiling_arch35.cpp:175-243,592-623.
+//
+// Per axis: src = (dst + 0.5) * scale - 0.5 (half-pixel) or dst * scale (align corners), clamped at 0;
+// taps floor/ceil clamped to size-1; lambda = src - floor(src);
+// out = (1-dy) * ((1-dx)*TL + dx*TR) + dy * ((1-dx)*BL + dx*BR), every product and sum rounded separately
+// (the file is compiled with -ffp-contract=off).
+#include <hip/hip_runtime.h>
+
+#include "kernels.hpp"
+#include "sampler_math.hpp"
+
+namespace opscv {
+
+namespace {
+
+constexpr int kThreads = 256;
+
+struct AxisTap {
+    int32_t i0, i1;
+    float lambda;
+};
+
+// resize_bilinear_v2_simt_nchw.h:108-134 for one axis
+template <bool HALF_PIXEL>
+__device__ __forceinline__ AxisTap axis_tap(int32_t d, float scale, int32_t len_src)
+{
+    float orig;
+    if (HALF_PIXEL) {
+        orig = ((float)d + 0.5f) * scale - 0.5f;
+    } else {
+        orig = (float)d * scale;
+    }
+    if (orig < 0.0f) {
+        orig = 0.0f;
+    }
+    const float fl = __builtin_floorf(orig);
+    const float lo = (orig > 0.0f) ? fl : 0.0f;
+    const float hi = (orig > 0.0f) ? __builtin_ceilf(orig) : 0.0f;
+    const float last = (float)(len_src - 1);
+    AxisTap t;
+    t.i0 = (lo < last) ? (int32_t)lo : len_src - 1;
+    t.i1 = (hi < last) ? (int32_t)hi : len_src - 1;
+    t.lambda = orig - fl;
+    return t;
+}
+
+// Generic NCHW variant: one lane per output pixel of a row, rows and planes on the other grid axes.
+template <typename T, bool HALF_PIXEL>
+__global__ __launch_bounds__(kThreads) void resize_nchw_generic_kernel(const T* __restrict__ x, T* __restrict__ y,
+                                                                        int64_t planes, int32_t Hs, int32_t Ws,
+                                                                        int32_t Hd, int32_t Wd, float scale_h,
+                                                                        float scale_w)
+{
+    const int64_t rows = planes * Hd;
+    const int32_t w = blockIdx.x * kThreads + threadIdx.x;
+    if (w >= Wd) {
+        return;
+    }
+    const AxisTap tx = axis_tap<HALF_PIXEL>(w, scale_w, Ws);
+    const float dx = tx.lambda;
+    for (int64_t r = blockIdx.y; r < rows; r += gridDim.y) {
+        const int64_t pl = r / Hd;
+        const int32_t h = (int32_t)(r - pl * Hd);
+        const AxisTap ty = axis_tap<HALF_PIXEL>(h, scale_h, Hs);
+        const float dy = ty.lambda;
+        const T* top = x + (pl * Hs + ty.i0) * (int64_t)Ws;
+        const T* bot = x + (pl * Hs + ty.i1) * (int64_t)Ws;
+        const float tl = ElemIO<T>::load(top + tx.i0);
+        const float tr = ElemIO<T>::load(top + tx.i1);
+        const float bl = ElemIO<T>::load(bot + tx.i0);
+        const float br = ElemIO<T>::load(bot + tx.i1);
+        const float out = (1.0f - dy) * ((1.0f - dx) * tl + dx * tr) + dy * ((1.0f - dx) * bl + dx * br);
+        ElemIO<T>::store(y + r * Wd + w, out);
+    }
+}
+
+// Generic NHWC variant: one lane per (w, c) element of an output row.
+template <typename T, bool HALF_PIXEL>
+__global__ __launch_bounds__(kThreads) void resize_nhwc_generic_kernel(const T* __restrict__ x, T* __restrict__ y,
+                                                                        int64_t N, int32_t C, int32_t Hs, int32_t Ws,
+                                                                        int32_t Hd, int32_t Wd, float scale_h,
+                                                                        float scale_w)
+{
+    const int64_t row_elems = (int64_t)Wd * C;
+    const int64_t e = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (e >= row_elems) {
+        return;
+    }
+    const int32_t w = (int32_t)(e / C);
+    const int32_t c = (int32_t)(e - (int64_t)w * C);
+    const AxisTap tx = axis_tap<HALF_PIXEL>(w, scale_w, Ws);
+    const float dx = tx.lambda;
+    const int64_t rows = N * Hd;
+    for (int64_t r = blockIdx.y; r < rows; r += gridDim.y) {
+        const int64_t n = r / Hd;
+        const int32_t h = (int32_t)(r - n * Hd);
+        const AxisTap ty = axis_tap<HALF_PIXEL>(h, scale_h, Hs);
+        const float dy = ty.lambda;
+        const T* top = x + ((n * Hs + ty.i0) * (int64_t)Ws) * C + c;
+        const T* bot = x + ((n * Hs + ty.i1) * (int64_t)Ws) * C + c;
+        const float tl = ElemIO<T>::load(top + (int64_t)tx.i0 * C);
+        const float tr = ElemIO<T>::load(top + (int64_t)tx.i1 * C);
+        const float bl = ElemIO<T>::load(bot + (int64_t)tx.i0 * C);
+        const float br = ElemIO<T>::load(bot + (int64_t)tx.i1 * C);
+        const float out = (1.0f - dy) * ((1.0f - dx) * tl + dx * tr) + dy * ((1.0f - dx) * bl + dx * br);
+        ElemIO<T>::store(y + r * row_elems + e, out);
+    }
+}
+
+// Broadcast of one source element per plane (mode Broadcast: 1x1 source; FirstPixel: 1x1 destination).
+// For NHWC the "plane" index is (n, c) with element stride C inside a batch.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void resize_fill_kernel(const T* __restrict__ x, T* __restrict__ y,
+                                                                int64_t N, int64_t C, int64_t src_hw, int64_t dst_hw,
+                                                                int channels_last)
+{
+    const int64_t total = N * C * dst_hw;
+    const int64_t stride = (int64_t)gridDim.x * kThreads;
+    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += stride) {
+        int64_t src;
+        if (channels_last) {
+            const int64_t n = i / (dst_hw * C);
+            const int64_t c = i % C;
+            src = n * src_hw * C + c;
+        } else {
+            src = (i / dst_hw) * src_hw;
+        }
+        y[i] = x[src];
+    }
+}
+
+template <typename T>
+hipError_t run_resize(const ResizeArgs& a, hipStream_t stream)
+{
+    const T* x = (const T*)a.x;
+    T* y = (T*)a.y;
+    const int64_t out_elems = a.N * a.C * a.Hd * a.Wd;
+    if (a.mode == ResizeMode::Copy) {
+        return hipMemcpyAsync(y, x, (size_t)out_elems * sizeof(T), hipMemcpyDeviceToDevice, stream);
+    }
+    if (a.mode == ResizeMode::Broadcast || a.mode == ResizeMode::FirstPixel) {
+        int64_t blocks = (out_elems + kThreads - 1) / kThreads;
+        if (blocks > 256 * 64) {
+            blocks = 256 * 64;
+        }
+        hipLaunchKernelGGL((resize_fill_kernel<T>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, x, y, a.N, a.C,
+                           a.Hs * a.Ws, a.Hd * a.Wd, a.channels_last);
+        return hipGetLastError();
+    }
+    if (a.channels_last) {
+        const int64_t row_elems = a.Wd * a.C;
+        const int64_t rows = a.N * a.Hd;
+        dim3 grid((unsigned)((row_elems + kThreads - 1) / kThreads), (unsigned)(rows < 65535 ? rows : 65535));
+        if (a.half_pixel) {
+            hipLaunchKernelGGL((resize_nhwc_generic_kernel<T, true>), grid, dim3(kThreads), 0, stream, x, y, a.N,
+                               (int32_t)a.C, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h,
+                               a.scale_w);
+        } else {
+            hipLaunchKernelGGL((resize_nhwc_generic_kernel<T, false>), grid, dim3(kThreads), 0, stream, x, y, a.N,
+                               (int32_t)a.C, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h,
+                               a.scale_w);
+        }
+        return hipGetLastError();
+    }
+    const int64_t planes = a.N * a.C;
+    const int64_t rows = planes * a.Hd;
+    dim3 grid((unsigned)((a.Wd + kThreads - 1) / kThreads), (unsigned)(rows < 65535 ? rows : 65535));
+    if (a.half_pixel) {
+        hipLaunchKernelGGL((resize_nchw_generic_kernel<T, true>), grid, dim3(kThreads), 0, stream, x, y, planes,
+                           (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h, a.scale_w);
+    } else {
+        hipLaunchKernelGGL((resize_nchw_generic_kernel<T, false>), grid, dim3(kThreads), 0, stream, x, y, planes,
+                           (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h, a.scale_w);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace
+
+const char* resize_variant(const ResizeArgs& a)
+{
+    switch (a.mode) {
+        case ResizeMode::Copy: return "copy";
+        case ResizeMode::Broadcast: return "broadcast";
+        case ResizeMode::FirstPixel: return "first_pixel";
+        default: break;
+    }
+    return a.channels_last ? "nhwc_generic" : "nchw_generic";
+}
+
+hipError_t launch_resize(const ResizeArgs& a, hipStream_t stream)
+{
+    const int64_t lim = INT32_MAX;
+    if (a.N < 0 || a.C < 0 || a.Hs <= 0 || a.Ws <= 0 || a.Hd < 0 || a.Wd < 0 || a.Hs > lim || a.Ws > lim ||
+        a.Hd > lim || a.Wd > lim || a.C > lim || a.N > lim) {
+        return hipErrorInvalidValue;
+    }
+    // one output row (NHWC: Wd*C elements) must be addressable by the x grid axis
+    if (a.Wd * (a.channels_last ? a.C : 1) > lim) {
+        return hipErrorInvalidValue;
+    }
+    if (a.N == 0 || a.C == 0 || a.Hd == 0 || a.Wd == 0) {
+        return hipSuccess;
+    }
+    if (a.x == nullptr || a.y == nullptr) {
+        return hipErrorInvalidValue;
+    }
+    switch (a.elem) {
+        case Elem::F32: return run_resize<float>(a, stream);
+        case Elem::F16: return run_resize<_Float16>(a, stream);
+        case Elem::BF16: return run_resize<__bf16>(a, stream);
+    }
+    return hipErrorInvalidValue;
+}
+
+}  // namespace opscv

@@ -1,0 +1,17 @@
+// Host-side planning of the bilinear resize: scale factors and kernel-template selection.
+#pragma once
+
+#include "acl_types.hpp"
+
+namespace opscv {
+
+// Scale handed to the kernel for one axis; user_scale <= 0 means "derive from the sizes".
+// image/resize_bilinear_v2/op_host/arch35/resize_bilinear_v2_tiling_arch35.cpp:175-184,228-243
+float resize_axis_scale(int64_t len_src, int64_t len_dst, bool align_corners, float user_scale);
+
+// Fills mode / half_pixel / scales of `a` from its shape fields (elem, channels_last, N, C, Hs, Ws, Hd, Wd).
+// Template choice follows resize_bilinear_v2_tiling_arch35.cpp:245-335,592-623 and
+// image/resize_bilinear_v2/op_kernel/resize_bilinear_v2_apt.cpp:91-140.
+void plan_resize(ResizeArgs* a, bool align_corners, float user_scale_h, float user_scale_w);
+
+}  // namespace opscv

@@ -1,0 +1,179 @@
+// Device-side coordinate arithmetic shared by the grid-sampler kernels.
+//
+// Every function mirrors, operation for operation, the scalar code of the reference SIMT kernel
+// image/grid_sampler2_d/op_kernel/arch35/grid_sampler2_d_simt.h.  The translation unit is compiled with
+// -ffp-contract=off, so a*b+c is two roundings everywhere except the single explicit fused multiply-add
+// in unnormalize(), exactly as in the reference (grid_sampler2_d_simt.h:74,131).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+namespace opscv {
+
+// ---- element <-> float conversion (round to nearest even on the way out) ----
+template <typename T>
+struct ElemIO;
+
+template <>
+struct ElemIO<float> {
+    static __device__ __forceinline__ float load(const float* p) { return *p; }
+    static __device__ __forceinline__ void store(float* p, float v) { *p = v; }
+};
+
+template <>
+struct ElemIO<_Float16> {
+    static __device__ __forceinline__ float load(const _Float16* p) { return (float)*p; }
+    static __device__ __forceinline__ void store(_Float16* p, float v) { *p = (_Float16)v; }
+};
+
+template <>
+struct ElemIO<__bf16> {
+    static __device__ __forceinline__ float load(const __bf16* p)
+    {
+        return __builtin_bit_cast(float, (uint32_t)(*(const uint16_t*)p) << 16);
+    }
+    static __device__ __forceinline__ void store(__bf16* p, float v) { *p = (__bf16)v; }
+};
+
+// grid_sampler2_d_simt.h:125-132
+template <bool ALIGN>
+__device__ __forceinline__ float unnormalize(float coord, int32_t size)
+{
+    if (ALIGN) {
+        return ((coord + 1.0f) / 2.0f) * (float)(size - 1);
+    }
+    float scaling = (float)size / 2.0f;
+    return __builtin_fmaf(scaling, coord + 1.0f, -0.5f);
+}
+
+// grid_sampler2_d_simt.h:136-143
+__device__ __forceinline__ float clip_coordinates(float coord, int32_t size)
+{
+    float max_val = (float)(size - 1);
+    if (__builtin_isnan(coord)) {
+        return 0.0f;
+    }
+    return __builtin_fminf(__builtin_fmaxf(coord, 0.0f), max_val);
+}
+
+// grid_sampler2_d_simt.h:171-185 (product and difference are rounded separately)
+__device__ __forceinline__ float reflect_coordinates(float coord, float low, float twice_span)
+{
+    if (twice_span == 0.0f) {
+        return 0.0f;
+    }
+    float abs_in = __builtin_fabsf(coord - low);
+    float flips = __builtin_truncf(abs_in / twice_span);
+    float product = flips * twice_span;
+    float extra = abs_in - product;
+    float complement = twice_span - extra;
+    return __builtin_fminf(extra, complement) + low;
+}
+
+// grid_sampler2_d_simt.h:187-207
+template <int PAD, bool ALIGN>
+__device__ __forceinline__ float compute_source_index(float coord, int32_t size)
+{
+    coord = unnormalize<ALIGN>(coord, size);
+    if (PAD == 1) {
+        coord = clip_coordinates(coord, size);
+    } else if (PAD == 2) {
+        if (ALIGN) {
+            coord = reflect_coordinates(coord, 0.0f, 2.0f * (float)(size - 1));
+        } else {
+            coord = reflect_coordinates(coord, -0.5f, 2.0f * (float)size);
+        }
+        coord = clip_coordinates(coord, size);
+    }
+    return coord;
+}
+
+__device__ __forceinline__ bool nan_or_inf(float x) { return __builtin_isnan(x) || __builtin_isinf(x); }
+
+// grid_sampler2_d_simt.h:209-215
+__device__ __forceinline__ float safe_downgrade(float x)
+{
+    if (x > 2147483646.0f || x < -2147483648.0f || nan_or_inf(x)) {
+        return -100.0f;
+    }
+    return x;
+}
+
+// float -> int32 with saturation (the hardware conversion saturates; 2^31 is out of bounds either way)
+__device__ __forceinline__ int32_t float_to_i32(float v)
+{
+    if (v >= 2147483648.0f) {
+        return INT32_MAX;
+    }
+    if (v < -2147483648.0f) {
+        return INT32_MIN;
+    }
+    return (int32_t)v;
+}
+
+// grid_sampler2_d_simt.h:219-234
+__device__ __forceinline__ int32_t banker_round(float x)
+{
+    float fl = __builtin_floorf(x);
+    float frac = x - fl;
+    int32_t fi = float_to_i32(fl);
+    int32_t up = (fi == INT32_MAX) ? fi : fi + 1;
+    if (frac < 0.5f) {
+        return fi;
+    }
+    if (frac > 0.5f) {
+        return up;
+    }
+    return ((fi & 1) == 0) ? fi : up;
+}
+
+// What the sampler decides per output pixel, before the channel loop.
+struct PixelTap {
+    int32_t x0, y0;  // bilinear: north-west corner; nearest: the selected texel
+    float w[4];      // nw, ne, sw, se (bilinear only)
+    int32_t flag;    // 1: write NaN to every channel (non-finite source coordinate, bilinear only)
+};
+
+// grid_sampler2_d_simt.h:479-498 and :307-316
+template <int INTERP, int PAD, bool ALIGN>
+__device__ __forceinline__ PixelTap decide_pixel(float gx, float gy, int32_t H, int32_t W)
+{
+    PixelTap t;
+    float ix = compute_source_index<PAD, ALIGN>(gx, W);
+    float iy = compute_source_index<PAD, ALIGN>(gy, H);
+    t.flag = 0;
+    t.w[0] = t.w[1] = t.w[2] = t.w[3] = 0.0f;
+    if (INTERP == 0) {
+        if (nan_or_inf(ix) || nan_or_inf(iy)) {
+            t.flag = 1;
+            t.x0 = 0;
+            t.y0 = 0;
+            return t;
+        }
+        ix = safe_downgrade(ix);
+        iy = safe_downgrade(iy);
+        float ixf = __builtin_floorf(ix);
+        float iyf = __builtin_floorf(iy);
+        t.x0 = float_to_i32(ixf);
+        t.y0 = float_to_i32(iyf);
+        t.w[0] = (ixf + 1.0f - ix) * (iyf + 1.0f - iy);
+        t.w[1] = (ix - ixf) * (iyf + 1.0f - iy);
+        t.w[2] = (ixf + 1.0f - ix) * (iy - iyf);
+        t.w[3] = (ix - ixf) * (iy - iyf);
+    } else {
+        ix = safe_downgrade(ix);
+        iy = safe_downgrade(iy);
+        t.x0 = banker_round(ix);
+        t.y0 = banker_round(iy);
+    }
+    return t;
+}
+
+__device__ __forceinline__ bool within(int32_t h, int32_t w, int32_t H, int32_t W)
+{
+    return h >= 0 && h < H && w >= 0 && w < W;
+}
+
+}  // namespace opscv

@@ -1,0 +1,514 @@
+/*
+ * CPU oracle for the bilinear gather/interpolate path -- TEST INFRASTRUCTURE ONLY.
+ *
+ * A plain-C restatement of the reference arithmetic.  It is the checker for the HIP kernels
+ * and the timed "cpu_baseline" of the benchmark; the shipped library never calls it.
+ * Build: gcc -O2 -ffp-contract=off -fopenmp (see oracle/Makefile).  -ffp-contract=off is part
+ * of the contract: the reference disables contraction file-wide and uses one explicit fmaf.
+ *
+ * Pinning status (how each function is checked by tests/, independent of this file's text):
+ *   half/bf16 conversions        : exhaustive round trip over all 65536 patterns + numpy/torch casts
+ *   oracle_unnormalize           : closed forms (g=-1,+1 -> -0.5,size-0.5 / 0,size-1), crafted fma-vs-mul point
+ *   oracle_clip/reflect          : range/evenness/periodicity invariants + torch grid_sample at large |g|
+ *   oracle_banker_round          : numpy rint on ties and near-ties
+ *   oracle_grid_sampler2d        : known answers recorded for the reference's own example inputs
+ *                                  (image/grid_sample/examples/test_aclnn_grid_sample2_d.cpp:96-98), identity
+ *                                  grid of image/grid_sampler2_d/examples/arch35/test_geir_grid_sampler2_d.cpp:84-90,
+ *                                  committed torch.nn.functional.grid_sample fixtures, live torch CPU comparison
+ *   oracle_upsample_bilinear2d   : known answers for image/upsample_bilinear2d/examples/
+ *                                  test_aclnn_upsample_bilinear2d.cpp:83-94, kernel-UT shapes (1,1,1,4)->(2,16),
+ *                                  (3,16), committed torch interpolate fixtures, live torch CPU comparison
+ *   oracle_resize_scale          : float bit patterns held by the reference's tiling UT
+ *                                  (image/resize_bilinear_v2/tests/ut/op_host/arch35/test_resize_bilinear_v2_tiling.cpp)
+ */
+#include "cv_oracle.h"
+
+#include <math.h>
+#include <stddef.h>
+#include <string.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+/* ------------------------------------------------------------------------------------------
+ * 16-bit float conversions (software, round-to-nearest-even; the reference converts through
+ * __half2float/__float2half and static_cast: grid_sampler2_d_simt.h:84-102)
+ * ---------------------------------------------------------------------------------------- */
+static inline uint32_t f2u(float f)
+{
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    return u;
+}
+static inline float u2f(uint32_t u)
+{
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+float oracle_half_to_float(uint16_t h)
+{
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1Fu;
+    uint32_t man = h & 0x3FFu;
+    if (exp == 0) {
+        if (man == 0) {
+            return u2f(sign);
+        }
+        /* subnormal: value = man * 2^-24, exact in fp32 */
+        float v = (float)man * 5.9604644775390625e-8f;
+        return (sign != 0) ? -v : v;
+    }
+    if (exp == 31) {
+        return u2f(sign | 0x7F800000u | (man << 13));
+    }
+    return u2f(sign | ((exp + 112u) << 23) | (man << 13));
+}
+
+uint16_t oracle_float_to_half(float f)
+{
+    uint32_t u = f2u(f);
+    uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+    uint32_t abs = u & 0x7FFFFFFFu;
+    if (abs >= 0x7F800000u) {
+        if (abs > 0x7F800000u) {
+            /* NaN: keep it a quiet NaN */
+            return (uint16_t)(sign | 0x7E00u | ((abs >> 13) & 0x3FFu));
+        }
+        return (uint16_t)(sign | 0x7C00u);
+    }
+    if (abs >= 0x477FF000u) {
+        /* >= 65520 rounds to infinity */
+        return (uint16_t)(sign | 0x7C00u);
+    }
+    if (abs < 0x38800000u) {
+        /* result is subnormal (or zero): quantum is 2^-24 */
+        if (abs < 0x33000000u) {
+            /* < 2^-25 : rounds to zero (2^-25 itself ties to even = 0) */
+            return sign;
+        }
+        uint32_t exp = abs >> 23;
+        uint32_t man = (abs & 0x7FFFFFu) | 0x800000u;
+        uint32_t shift = 126u - exp; /* 14..24 */
+        uint32_t q = man >> shift;
+        uint32_t rem = man & ((1u << shift) - 1u);
+        uint32_t half = 1u << (shift - 1u);
+        if (rem > half || (rem == half && (q & 1u))) {
+            q++;
+        }
+        return (uint16_t)(sign | q);
+    }
+    uint32_t man = abs & 0x7FFFFFu;
+    uint32_t exp = (abs >> 23) - 112u;
+    uint32_t q = (exp << 10) | (man >> 13);
+    uint32_t rem = man & 0x1FFFu;
+    if (rem > 0x1000u || (rem == 0x1000u && (q & 1u))) {
+        q++; /* carries into the exponent correctly */
+    }
+    return (uint16_t)(sign | q);
+}
+
+float oracle_bf16_to_float(uint16_t h) { return u2f((uint32_t)h << 16); }
+
+uint16_t oracle_float_to_bf16(float f)
+{
+    uint32_t u = f2u(f);
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) {
+        return (uint16_t)((u >> 16) | 0x0040u);
+    }
+    uint32_t lsb = (u >> 16) & 1u;
+    u += 0x7FFFu + lsb;
+    return (uint16_t)(u >> 16);
+}
+
+static inline float load_as_float(const void* p, int dtype, int64_t i)
+{
+    if (dtype == ORACLE_F32) {
+        return ((const float*)p)[i];
+    }
+    if (dtype == ORACLE_F16) {
+        return oracle_half_to_float(((const uint16_t*)p)[i]);
+    }
+    return oracle_bf16_to_float(((const uint16_t*)p)[i]);
+}
+
+static inline void store_from_float(void* p, int dtype, int64_t i, float v)
+{
+    if (dtype == ORACLE_F32) {
+        ((float*)p)[i] = v;
+    } else if (dtype == ORACLE_F16) {
+        ((uint16_t*)p)[i] = oracle_float_to_half(v);
+    } else {
+        ((uint16_t*)p)[i] = oracle_float_to_bf16(v);
+    }
+}
+
+/* ------------------------------------------------------------------------------------------
+ * Grid sampler coordinate pipeline
+ * ---------------------------------------------------------------------------------------- */
+
+/* grid_sampler2_d_simt.h:125-132 : align -> ((g+1)/2)*(size-1); else ONE fused multiply-add */
+float oracle_unnormalize(float coord, int32_t size, int32_t align_corners)
+{
+    if (align_corners != 0) {
+        return ((coord + 1.0f) / 2.0f) * (float)(size - 1);
+    }
+    float scaling = (float)size / 2.0f;
+    return fmaf(scaling, coord + 1.0f, -0.5f);
+}
+
+/* grid_sampler2_d_simt.h:136-143 */
+float oracle_clip_coordinates(float coord, int32_t size)
+{
+    float max_val = (float)(size - 1);
+    if (isnan(coord)) {
+        return 0.0f;
+    }
+    return fminf(fmaxf(coord, 0.0f), max_val);
+}
+
+/* grid_sampler2_d_simt.h:171-185 : a - trunc(a/b)*b with product and difference rounded separately */
+float oracle_reflect_coordinates(float coord, float low, float twice_span)
+{
+    if (twice_span == 0.0f) {
+        return 0.0f;
+    }
+    float abs_in = fabsf(coord - low);
+    float flips = truncf(abs_in / twice_span);
+    float product = flips * twice_span;
+    float extra = abs_in - product;
+    float complement = twice_span - extra;
+    return fminf(extra, complement) + low;
+}
+
+/* grid_sampler2_d_simt.h:187-207 */
+float oracle_compute_source_index(float coord, int32_t size, int32_t padding_mode, int32_t align_corners)
+{
+    coord = oracle_unnormalize(coord, size, align_corners);
+    if (padding_mode == 1) {
+        coord = oracle_clip_coordinates(coord, size);
+    } else if (padding_mode == 2) {
+        if (align_corners != 0) {
+            coord = oracle_reflect_coordinates(coord, 0.0f, 2.0f * (float)(size - 1));
+        } else {
+            coord = oracle_reflect_coordinates(coord, -0.5f, 2.0f * (float)size);
+        }
+        coord = oracle_clip_coordinates(coord, size);
+    }
+    return coord;
+}
+
+/* grid_sampler2_d_simt.h:209-215 ; 2147483646.0f is 2^31 once rounded to fp32 */
+float oracle_safe_downgrade(float x)
+{
+    if (x > 2147483646.0f || x < -2147483648.0f || isnan(x) || isinf(x)) {
+        return -100.0f;
+    }
+    return x;
+}
+
+/* float -> int32 for values the guard above lets through; 2^31 itself saturates (it is out of
+ * bounds for every legal tensor either way) */
+static inline int32_t float_to_i32(float v)
+{
+    if (v >= 2147483648.0f) {
+        return INT32_MAX;
+    }
+    if (v < -2147483648.0f) {
+        return INT32_MIN;
+    }
+    return (int32_t)v;
+}
+
+/* grid_sampler2_d_simt.h:219-234 : round half to even built from floor, frac and parity */
+int32_t oracle_banker_round(float x)
+{
+    float fl = floorf(x);
+    float frac = x - fl;
+    int32_t fi = float_to_i32(fl);
+    if (frac < 0.5f) {
+        return fi;
+    }
+    if (frac > 0.5f) {
+        return (fi == INT32_MAX) ? fi : fi + 1;
+    }
+    if ((fi & 1) == 0) {
+        return fi;
+    }
+    return (fi == INT32_MAX) ? fi : fi + 1;
+}
+
+static inline int within(int32_t h, int32_t w, int32_t H, int32_t W) { return h >= 0 && h < H && w >= 0 && w < W; }
+
+/* the per-pixel decision of grid_sampler2_d_simt.h:479-498 (bilinear, nearest) */
+static inline void gs_decide(float gx, float gy, int32_t Hin, int32_t Win, int interp, int pad, int align,
+                             oracle_gs_tap* t)
+{
+    float ix = oracle_compute_source_index(gx, Win, pad, align);
+    float iy = oracle_compute_source_index(gy, Hin, pad, align);
+    t->flag = 0;
+    t->w[0] = t->w[1] = t->w[2] = t->w[3] = 0.0f;
+    if (interp == 0) {
+        if (isnan(ix) || isinf(ix) || isnan(iy) || isinf(iy)) {
+            t->flag = 1;
+            t->ix0 = 0;
+            t->iy0 = 0;
+            return;
+        }
+        ix = oracle_safe_downgrade(ix);
+        iy = oracle_safe_downgrade(iy);
+        /* grid_sampler2_d_simt.h:307-316 */
+        float ixf = floorf(ix);
+        float iyf = floorf(iy);
+        t->ix0 = float_to_i32(ixf);
+        t->iy0 = float_to_i32(iyf);
+        t->w[0] = (ixf + 1.0f - ix) * (iyf + 1.0f - iy);
+        t->w[1] = (ix - ixf) * (iyf + 1.0f - iy);
+        t->w[2] = (ixf + 1.0f - ix) * (iy - iyf);
+        t->w[3] = (ix - ixf) * (iy - iyf);
+    } else {
+        ix = oracle_safe_downgrade(ix);
+        iy = oracle_safe_downgrade(iy);
+        t->ix0 = oracle_banker_round(ix);
+        t->iy0 = oracle_banker_round(iy);
+    }
+}
+
+int oracle_grid_sampler2d_taps(const void* grid, oracle_gs_tap* taps, int dtype, int64_t N, int64_t Hin,
+                               int64_t Win, int64_t Hout, int64_t Wout, int interp_mode, int padding_mode,
+                               int align_corners)
+{
+    if (interp_mode < 0 || interp_mode > 1 || padding_mode < 0 || padding_mode > 2 || dtype < 0 || dtype > 2) {
+        return -1;
+    }
+    int64_t total = N * Hout * Wout;
+    for (int64_t p = 0; p < total; p++) {
+        float gx = load_as_float(grid, dtype, 2 * p);
+        float gy = load_as_float(grid, dtype, 2 * p + 1);
+        gs_decide(gx, gy, (int32_t)Hin, (int32_t)Win, interp_mode, padding_mode, align_corners, &taps[p]);
+    }
+    return 0;
+}
+
+int oracle_grid_sampler2d(const void* x, const void* grid, void* y, int dtype, int64_t N, int64_t C, int64_t Hin,
+                          int64_t Win, int64_t Hout, int64_t Wout, int interp_mode, int padding_mode,
+                          int align_corners, int num_threads)
+{
+    if (interp_mode < 0 || interp_mode > 1 || padding_mode < 0 || padding_mode > 2 || dtype < 0 || dtype > 2) {
+        return -1;
+    }
+    if (Hin <= 0 || Win <= 0 || Hin > INT32_MAX || Win > INT32_MAX) {
+        return -2;
+    }
+    const int64_t total = N * Hout * Wout;
+    const int64_t x_step = Hin * Win;
+    const int64_t y_step = Hout * Wout;
+    const int32_t H = (int32_t)Hin;
+    const int32_t W = (int32_t)Win;
+    (void)num_threads;
+#ifdef _OPENMP
+    if (num_threads <= 0) {
+        num_threads = omp_get_max_threads();
+    }
+#pragma omp parallel for schedule(static) num_threads(num_threads)
+#endif
+    for (int64_t p = 0; p < total; p++) {
+        /* pixel decode of grid_sampler2_d_simt.h:473-479 */
+        int64_t hw = p / Wout;
+        int64_t w_out = p - hw * Wout;
+        int64_t n = hw / Hout;
+        int64_t h_out = hw - n * Hout;
+        float gx = load_as_float(grid, dtype, 2 * p);
+        float gy = load_as_float(grid, dtype, 2 * p + 1);
+        oracle_gs_tap t;
+        gs_decide(gx, gy, H, W, interp_mode, padding_mode, align_corners, &t);
+        int64_t x_base = n * C * x_step;
+        int64_t y_base = n * C * y_step + h_out * Wout + w_out;
+        if (t.flag) {
+            /* grid_sampler2_d_simt.h:236-247 */
+            float nan_val = NAN;
+            for (int64_t c = 0; c < C; c++) {
+                store_from_float(y, dtype, y_base, nan_val);
+                y_base += y_step;
+            }
+            continue;
+        }
+        if (interp_mode == 0) {
+            /* grid_sampler2_d_simt.h:321-338 : taps added in nw, ne, sw, se order, each skipped when outside */
+            int32_t x0 = t.ix0, y0 = t.iy0;
+            int32_t x1 = (x0 == INT32_MAX) ? x0 : x0 + 1;
+            int32_t y1 = (y0 == INT32_MAX) ? y0 : y0 + 1;
+            int in_nw = within(y0, x0, H, W), in_ne = within(y0, x1, H, W);
+            int in_sw = within(y1, x0, H, W), in_se = within(y1, x1, H, W);
+            for (int64_t c = 0; c < C; c++) {
+                float out = 0.0f;
+                if (in_nw) {
+                    out += load_as_float(x, dtype, x_base + (int64_t)y0 * W + x0) * t.w[0];
+                }
+                if (in_ne) {
+                    out += load_as_float(x, dtype, x_base + (int64_t)y0 * W + x1) * t.w[1];
+                }
+                if (in_sw) {
+                    out += load_as_float(x, dtype, x_base + (int64_t)y1 * W + x0) * t.w[2];
+                }
+                if (in_se) {
+                    out += load_as_float(x, dtype, x_base + (int64_t)y1 * W + x1) * t.w[3];
+                }
+                store_from_float(y, dtype, y_base, out);
+                x_base += x_step;
+                y_base += y_step;
+            }
+        } else {
+            /* grid_sampler2_d_simt.h:341-360 */
+            int in = within(t.iy0, t.ix0, H, W);
+            for (int64_t c = 0; c < C; c++) {
+                float out = 0.0f;
+                if (in) {
+                    out = load_as_float(x, dtype, x_base + (int64_t)t.iy0 * W + t.ix0);
+                }
+                store_from_float(y, dtype, y_base, out);
+                x_base += x_step;
+                y_base += y_step;
+            }
+        }
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------------------------------
+ * Upsample (resize_bilinear_v2, NCHW SIMT template)
+ * ---------------------------------------------------------------------------------------- */
+
+/* resize_bilinear_v2_tiling_arch35.cpp:175-184 (user scale -> reciprocal, else size ratio) and :228-243 */
+float oracle_resize_scale(int64_t len_src, int64_t len_dst, int align_corners, float user_scale)
+{
+    if (align_corners == 0) {
+        if (user_scale > 0.0f) {
+            return 1.0f / user_scale;
+        }
+        return (float)len_src / (float)len_dst;
+    }
+    if (len_dst > 1) {
+        return (float)(len_src - 1) / (float)(len_dst - 1);
+    }
+    return (float)len_src / (float)len_dst;
+}
+
+/* resize_bilinear_v2_simt_nchw.h:108-134 for one axis */
+static inline void axis_tap(int64_t d, float scale, int half_pixel, int64_t len_src, int32_t* i0, int32_t* i1,
+                            float* lambda)
+{
+    float orig;
+    if (half_pixel) {
+        orig = ((float)d + 0.5f) * scale - 0.5f;
+    } else {
+        orig = (float)d * scale;
+    }
+    if (orig < 0.0f) {
+        orig = 0.0f;
+    }
+    float fl = floorf(orig);
+    float lo = (orig > 0.0f) ? fl : 0.0f;
+    float hi = (orig > 0.0f) ? ceilf(orig) : 0.0f;
+    float last = (float)(len_src - 1);
+    /* the reference assigns the float to an unsigned index and then clamps; clamping first is the
+     * same for every in-range value and keeps the conversion defined for huge coordinates */
+    int64_t a = (lo < last) ? (int64_t)lo : len_src - 1;
+    int64_t b = (hi < last) ? (int64_t)hi : len_src - 1;
+    *i0 = (int32_t)a;
+    *i1 = (int32_t)b;
+    *lambda = orig - fl;
+}
+
+int oracle_upsample_axis_taps(int64_t len_src, int64_t len_dst, int align_corners, float user_scale, int32_t* i0,
+                              int32_t* i1, float* lambda)
+{
+    float scale = oracle_resize_scale(len_src, len_dst, align_corners, user_scale);
+    for (int64_t d = 0; d < len_dst; d++) {
+        axis_tap(d, scale, !align_corners, len_src, &i0[d], &i1[d], &lambda[d]);
+    }
+    return 0;
+}
+
+int oracle_upsample_bilinear2d(const void* x, void* y, int dtype, int64_t N, int64_t C, int64_t Hs, int64_t Ws,
+                               int64_t Hd, int64_t Wd, int align_corners, double scales_h, double scales_w,
+                               int num_threads)
+{
+    if (dtype < 0 || dtype > 2 || Hs <= 0 || Ws <= 0) {
+        return -1;
+    }
+    const int64_t planes = N * C;
+    const int64_t esz = (dtype == ORACLE_F32) ? 4 : 2;
+    (void)num_threads;
+#ifdef _OPENMP
+    if (num_threads <= 0) {
+        num_threads = omp_get_max_threads();
+    }
+#endif
+    /* template selection of resize_bilinear_v2_tiling_arch35.cpp:592-623 + resize_bilinear_v2_apt.cpp:91-115:
+     * same size -> copy; 1x1 source -> broadcast (always for align_corners, from 128 output bytes per plane
+     * otherwise); 1x1 destination with align_corners -> element (0,0) */
+    int mode = 0;
+    if (Hs == Hd && Ws == Wd) {
+        mode = 1;
+    } else if (Hs == 1 && Ws == 1 && (align_corners || Hd * Wd * esz >= 128)) {
+        mode = 2;
+    } else if (Hd == 1 && Wd == 1 && align_corners) {
+        mode = 3;
+    }
+    if (mode != 0) {
+#ifdef _OPENMP
+#pragma omp parallel for schedule(static) num_threads(num_threads)
+#endif
+        for (int64_t pl = 0; pl < planes; pl++) {
+            for (int64_t i = 0; i < Hd * Wd; i++) {
+                int64_t src = (mode == 1) ? pl * Hs * Ws + i : pl * Hs * Ws;
+                if (esz == 4) {
+                    ((uint32_t*)y)[pl * Hd * Wd + i] = ((const uint32_t*)x)[src];
+                } else {
+                    ((uint16_t*)y)[pl * Hd * Wd + i] = ((const uint16_t*)x)[src];
+                }
+            }
+        }
+        return 0;
+    }
+    /* aclnn_upsample_bilinear_2d.cpp:411-412 narrows the user scales to float before they reach the tiling */
+    const float scale_h = oracle_resize_scale(Hs, Hd, align_corners, (float)scales_h);
+    const float scale_w = oracle_resize_scale(Ws, Wd, align_corners, (float)scales_w);
+    const int half_pixel = !align_corners;
+    const int64_t rows = planes * Hd;
+#ifdef _OPENMP
+#pragma omp parallel for schedule(static) num_threads(num_threads)
+#endif
+    for (int64_t r = 0; r < rows; r++) {
+        int64_t pl = r / Hd;
+        int64_t h = r - pl * Hd;
+        int32_t top, bottom;
+        float dy;
+        axis_tap(h, scale_h, half_pixel, Hs, &top, &bottom, &dy);
+        const int64_t base = pl * Hs * Ws;
+        for (int64_t w = 0; w < Wd; w++) {
+            int32_t left, right;
+            float dx;
+            axis_tap(w, scale_w, half_pixel, Ws, &left, &right, &dx);
+            float tl = load_as_float(x, dtype, base + (int64_t)top * Ws + left);
+            float tr = load_as_float(x, dtype, base + (int64_t)top * Ws + right);
+            float bl = load_as_float(x, dtype, base + (int64_t)bottom * Ws + left);
+            float br = load_as_float(x, dtype, base + (int64_t)bottom * Ws + right);
+            /* resize_bilinear_v2_simt_nchw.h:143-144 */
+            float out = (1.0f - dy) * ((1.0f - dx) * tl + dx * tr) + dy * ((1.0f - dx) * bl + dx * br);
+            store_from_float(y, dtype, r * Wd + w, out);
+        }
+    }
+    return 0;
+}
+
+int oracle_max_threads(void)
+{
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}

@@ -1,0 +1,84 @@
+/*
+ * CPU oracle for the bilinear gather/interpolate path (TEST INFRASTRUCTURE ONLY).
+ *
+ * This library restates, in plain C, the arithmetic of the reference kernels so that the
+ * HIP kernels can be checked against it.  It is the checker, never the product: nothing
+ * under the shipped package may include, link or load it.  Only the test-suite, the smoke
+ * entry and the benchmark's "cpu_baseline" leg call it.
+ *
+ * Reference sources followed (paths relative to the reference tree):
+ *   grid sample : image/grid_sampler2_d/op_kernel/arch35/grid_sampler2_d_simt.h
+ *   upsample    : image/resize_bilinear_v2/op_kernel/arch35/resize_bilinear_v2_simt_nchw.h
+ *   scale rules : image/resize_bilinear_v2/op_host/arch35/resize_bilinear_v2_tiling_arch35.cpp:175-243
+ *
+ * Pinning status of each exported function is listed in cv_oracle.c's header comment.
+ */
+#ifndef CV_ORACLE_H_
+#define CV_ORACLE_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element type codes shared by every oracle entry point */
+enum { ORACLE_F32 = 0, ORACLE_F16 = 1, ORACLE_BF16 = 2 };
+
+/* ---- scalar building blocks (exported so that tests can pin each one separately) ---- */
+float oracle_half_to_float(uint16_t h);
+uint16_t oracle_float_to_half(float f);
+float oracle_bf16_to_float(uint16_t h);
+uint16_t oracle_float_to_bf16(float f);
+
+float oracle_unnormalize(float coord, int32_t size, int32_t align_corners);
+float oracle_clip_coordinates(float coord, int32_t size);
+float oracle_reflect_coordinates(float coord, float low, float twice_span);
+float oracle_compute_source_index(float coord, int32_t size, int32_t padding_mode, int32_t align_corners);
+float oracle_safe_downgrade(float x);
+int32_t oracle_banker_round(float x);
+
+/*
+ * Per-pixel tap record of the grid sampler: what the kernel decides before the channel loop.
+ * bilinear: ix0/iy0 = north-west corner, w[4] = nw,ne,sw,se weights, flag = 1 when the pixel
+ * is written as NaN (non-finite source coordinate).  nearest: ix0/iy0 = the selected texel,
+ * w unused (0), flag = 0.
+ */
+typedef struct {
+    int32_t ix0;
+    int32_t iy0;
+    float w[4];
+    int32_t flag;
+} oracle_gs_tap;
+
+/* ---- whole-tensor entry points; all tensors contiguous, NCHW, grid is (N,Ho,Wo,2) ---- */
+
+/* returns 0 on success, <0 on invalid arguments */
+int oracle_grid_sampler2d(const void* x, const void* grid, void* y, int dtype, int64_t N, int64_t C, int64_t Hin,
+                          int64_t Win, int64_t Hout, int64_t Wout, int interp_mode, int padding_mode,
+                          int align_corners, int num_threads);
+
+/* fills taps[N*Hout*Wout]; same decision code as oracle_grid_sampler2d */
+int oracle_grid_sampler2d_taps(const void* grid, oracle_gs_tap* taps, int dtype, int64_t N, int64_t Hin,
+                               int64_t Win, int64_t Hout, int64_t Wout, int interp_mode, int padding_mode,
+                               int align_corners);
+
+/* scale handed to the kernel for one axis (align_corners / user scale / size ratio) */
+float oracle_resize_scale(int64_t len_src, int64_t len_dst, int align_corners, float user_scale);
+
+/* scales_h / scales_w are the user-facing multipliers (0 = derive from sizes) */
+int oracle_upsample_bilinear2d(const void* x, void* y, int dtype, int64_t N, int64_t C, int64_t Hs, int64_t Ws,
+                               int64_t Hd, int64_t Wd, int align_corners, double scales_h, double scales_w,
+                               int num_threads);
+
+/* per-axis tap table of the upsample: i0[len_dst], i1[len_dst], lambda[len_dst] */
+int oracle_upsample_axis_taps(int64_t len_src, int64_t len_dst, int align_corners, float user_scale, int32_t* i0,
+                              int32_t* i1, float* lambda);
+
+int oracle_max_threads(void);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* CV_ORACLE_H_ */

@@ -1,0 +1,158 @@
+"""ctypes view of the CPU oracle (oracle/libcv_oracle.so).
+
+Test infrastructure: imported by tests/, the smoke entry and the benchmark's cpu_baseline leg only.
+The shipped package never imports this module.
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+_ORACLE_DIR = os.path.join(_ROOT, "oracle")
+_LIB_PATH = os.path.join(_ORACLE_DIR, "libcv_oracle.so")
+
+F32, F16, BF16 = 0, 1, 2
+
+
+class GsTap(ctypes.Structure):
+    _fields_ = [("ix0", ctypes.c_int32), ("iy0", ctypes.c_int32), ("w", ctypes.c_float * 4),
+                ("flag", ctypes.c_int32)]
+
+
+TAP_DTYPE = np.dtype([("ix0", "<i4"), ("iy0", "<i4"), ("w", "<f4", (4,)), ("flag", "<i4")])
+
+
+def build(force=False):
+    """Compile the oracle with gcc when the shared object is missing (or when forced)."""
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.check_call(["make", "-C", _ORACLE_DIR, "-B" if force else "-s", "libcv_oracle.so"])
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is not None:
+        return _lib
+    build()
+    L = ctypes.CDLL(_LIB_PATH)
+    i64, i32, f32, vp = ctypes.c_int64, ctypes.c_int32, ctypes.c_float, ctypes.c_void_p
+    L.oracle_half_to_float.restype = f32
+    L.oracle_half_to_float.argtypes = [ctypes.c_uint16]
+    L.oracle_float_to_half.restype = ctypes.c_uint16
+    L.oracle_float_to_half.argtypes = [f32]
+    L.oracle_bf16_to_float.restype = f32
+    L.oracle_bf16_to_float.argtypes = [ctypes.c_uint16]
+    L.oracle_float_to_bf16.restype = ctypes.c_uint16
+    L.oracle_float_to_bf16.argtypes = [f32]
+    L.oracle_unnormalize.restype = f32
+    L.oracle_unnormalize.argtypes = [f32, i32, i32]
+    L.oracle_clip_coordinates.restype = f32
+    L.oracle_clip_coordinates.argtypes = [f32, i32]
+    L.oracle_reflect_coordinates.restype = f32
+    L.oracle_reflect_coordinates.argtypes = [f32, f32, f32]
+    L.oracle_compute_source_index.restype = f32
+    L.oracle_compute_source_index.argtypes = [f32, i32, i32, i32]
+    L.oracle_safe_downgrade.restype = f32
+    L.oracle_safe_downgrade.argtypes = [f32]
+    L.oracle_banker_round.restype = i32
+    L.oracle_banker_round.argtypes = [f32]
+    L.oracle_grid_sampler2d.restype = ctypes.c_int
+    L.oracle_grid_sampler2d.argtypes = [vp, vp, vp, ctypes.c_int, i64, i64, i64, i64, i64, i64, ctypes.c_int,
+                                        ctypes.c_int, ctypes.c_int, ctypes.c_int]
+    L.oracle_grid_sampler2d_taps.restype = ctypes.c_int
+    L.oracle_grid_sampler2d_taps.argtypes = [vp, vp, ctypes.c_int, i64, i64, i64, i64, i64, ctypes.c_int,
+                                             ctypes.c_int, ctypes.c_int]
+    L.oracle_resize_scale.restype = f32
+    L.oracle_resize_scale.argtypes = [i64, i64, ctypes.c_int, f32]
+    L.oracle_upsample_bilinear2d.restype = ctypes.c_int
+    L.oracle_upsample_bilinear2d.argtypes = [vp, vp, ctypes.c_int, i64, i64, i64, i64, i64, i64, ctypes.c_int,
+                                             ctypes.c_double, ctypes.c_double, ctypes.c_int]
+    L.oracle_upsample_axis_taps.restype = ctypes.c_int
+    L.oracle_upsample_axis_taps.argtypes = [i64, i64, ctypes.c_int, f32, vp, vp, vp]
+    L.oracle_max_threads.restype = ctypes.c_int
+    L.oracle_max_threads.argtypes = []
+    _lib = L
+    return L
+
+
+def _code_of(arr):
+    """Element code for a numpy array: float32 -> F32, float16 -> F16; uint16 needs an explicit code."""
+    if arr.dtype == np.float32:
+        return F32
+    if arr.dtype == np.float16:
+        return F16
+    raise TypeError("pass dtype= explicitly for %s arrays (bf16 travels as uint16)" % arr.dtype)
+
+
+def _ptr(a):
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+def grid_sampler2d(x, grid, interp=0, pad=0, align=False, dtype=None, threads=0):
+    """x (N,C,H,W), grid (N,Ho,Wo,2) -> y (N,C,Ho,Wo); arrays are float32, float16, or uint16 holding bf16 bits."""
+    x = np.ascontiguousarray(x)
+    grid = np.ascontiguousarray(grid)
+    code = _code_of(x) if dtype is None else dtype
+    N, C, H, W = x.shape
+    _, Ho, Wo, two = grid.shape
+    assert two == 2 and grid.shape[0] == N and grid.dtype == x.dtype
+    y = np.empty((N, C, Ho, Wo), dtype=x.dtype)
+    rc = lib().oracle_grid_sampler2d(_ptr(x), _ptr(grid), _ptr(y), code, N, C, H, W, Ho, Wo, interp, pad,
+                                     int(bool(align)), threads)
+    if rc != 0:
+        raise ValueError("oracle_grid_sampler2d rc=%d" % rc)
+    return y
+
+
+def grid_sampler2d_taps(grid, H, W, interp=0, pad=0, align=False, dtype=None):
+    grid = np.ascontiguousarray(grid)
+    code = _code_of(grid) if dtype is None else dtype
+    N, Ho, Wo, _ = grid.shape
+    taps = np.zeros((N, Ho, Wo), dtype=TAP_DTYPE)
+    rc = lib().oracle_grid_sampler2d_taps(_ptr(grid), _ptr(taps), code, N, H, W, Ho, Wo, interp, pad,
+                                          int(bool(align)))
+    if rc != 0:
+        raise ValueError("oracle_grid_sampler2d_taps rc=%d" % rc)
+    return taps
+
+
+def upsample_bilinear2d(x, out_hw, align=False, scales_h=0.0, scales_w=0.0, dtype=None, threads=0):
+    x = np.ascontiguousarray(x)
+    code = _code_of(x) if dtype is None else dtype
+    N, C, Hs, Ws = x.shape
+    Hd, Wd = out_hw
+    y = np.empty((N, C, Hd, Wd), dtype=x.dtype)
+    rc = lib().oracle_upsample_bilinear2d(_ptr(x), _ptr(y), code, N, C, Hs, Ws, Hd, Wd, int(bool(align)),
+                                          float(scales_h), float(scales_w), threads)
+    if rc != 0:
+        raise ValueError("oracle_upsample_bilinear2d rc=%d" % rc)
+    return y
+
+
+def upsample_axis_taps(len_src, len_dst, align=False, user_scale=0.0):
+    i0 = np.zeros(len_dst, dtype=np.int32)
+    i1 = np.zeros(len_dst, dtype=np.int32)
+    lam = np.zeros(len_dst, dtype=np.float32)
+    lib().oracle_upsample_axis_taps(len_src, len_dst, int(bool(align)), float(user_scale), _ptr(i0), _ptr(i1),
+                                    _ptr(lam))
+    return i0, i1, lam
+
+
+def f32_to_bf16_bits(a):
+    """Round-to-nearest-even float32 -> bf16 bit patterns (uint16), NaN kept quiet."""
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    u = a.view(np.uint32)
+    nan = (u & 0x7FFFFFFF) > 0x7F800000
+    r = ((u + (0x7FFF + ((u >> 16) & 1))) >> 16).astype(np.uint16)
+    r[nan] = ((u[nan] >> 16) | 0x40).astype(np.uint16)
+    return r
+
+
+def bf16_bits_to_f32(b):
+    b = np.ascontiguousarray(b, dtype=np.uint16)
+    return (b.astype(np.uint32) << 16).view(np.float32)

@@ -1,0 +1,138 @@
+"""GPU parity: the HIP path, called through the C-ABI, against the CPU oracle on the same seeded inputs.
+
+Bars: nearest mode and every integer tap index bit-exact; bilinear max-abs <= 1e-5 (fp32) and <= 1e-3 relative
+(fp16/bf16) as stated for this path.  The kernels keep the oracle's operation order with contraction disabled,
+so the tests additionally report (and for fp32 require) bit equality where it holds.
+"""
+import numpy as np
+import pytest
+
+import inputs as I
+
+pytestmark = pytest.mark.gpu
+
+INTERP = {0: "bilinear", 1: "nearest"}
+PAD = {0: "zeros", 1: "border", 2: "reflection"}
+
+
+def _check(y_gpu, y_ref, dtype, interp, what):
+    a = I.as_f32(y_gpu, dtype)
+    b = I.as_f32(y_ref, dtype)
+    nan_a, nan_b = np.isnan(a), np.isnan(b)
+    assert np.array_equal(nan_a, nan_b), "%s: NaN positions differ" % what
+    a = np.where(nan_a, 0, a)
+    b = np.where(nan_b, 0, b)
+    if interp == 1:
+        assert np.array_equal(a, b), "%s: nearest must be bit-exact, %d mismatches" % (what, (a != b).sum())
+        return
+    inf = np.isinf(b)
+    assert np.array_equal(np.isinf(a), inf) and np.array_equal(a[inf], b[inf]), "%s: inf positions differ" % what
+    a = np.where(inf, 0, a)
+    b = np.where(inf, 0, b)
+    if dtype == "fp32":
+        err = np.abs(a - b).max() if a.size else 0.0
+        assert err <= 1e-5, "%s: max-abs %g > 1e-5" % (what, err)
+    else:
+        # 1e-3 relative; values that round to (sub)normal-small outputs are compared against a small absolute floor
+        tol = 1e-3 * np.maximum(np.abs(b), 1e-2)
+        bad = np.abs(a - b) > tol
+        assert not bad.any(), "%s: %d samples beyond 1e-3 relative, worst %g" % (
+            what, bad.sum(), (np.abs(a - b) / np.maximum(np.abs(b), 1e-2)).max())
+
+
+def _run_gs(oracle, device, x32, g32, dtype, interp, pad, align):
+    from ops_cv_amd import aclnn
+    x = I.cast_np(x32, dtype)
+    g = I.cast_np(g32, dtype)
+    y_ref = oracle.grid_sampler2d(x, g, interp, pad, align, dtype=I.oracle_code(dtype))
+    y = aclnn.grid_sampler2d(I.to_torch(x, dtype, device), I.to_torch(g, dtype, device), interp, pad, align)
+    import torch
+    torch.cuda.synchronize()
+    return I.from_torch(y, dtype), y_ref
+
+
+@pytest.mark.parametrize("dtype", I.DTYPES)
+@pytest.mark.parametrize("interp", [0, 1])
+@pytest.mark.parametrize("pad", [0, 1, 2])
+@pytest.mark.parametrize("align", [False, True])
+def test_grid_sampler_random(oracle, device, dtype, interp, pad, align):
+    rng = np.random.default_rng(1000 + interp * 100 + pad * 10 + int(align))
+    for (N, C, H, W, Ho, Wo) in [(2, 5, 13, 17, 19, 23), (1, 3, 64, 64, 32, 32), (3, 8, 1, 1, 7, 5),
+                                 (2, 16, 7, 64, 33, 65)]:
+        x32 = rng.standard_normal((N, C, H, W)).astype(np.float32)
+        g32 = rng.uniform(-1.3, 1.3, (N, Ho, Wo, 2)).astype(np.float32)
+        y, y_ref = _run_gs(oracle, device, x32, g32, dtype, interp, pad, align)
+        _check(y, y_ref, dtype, interp, "gs %s %s %s align=%s %s" % (dtype, INTERP[interp], PAD[pad], align,
+                                                                      (N, C, H, W, Ho, Wo)))
+
+
+@pytest.mark.parametrize("dtype", I.DTYPES)
+@pytest.mark.parametrize("interp", [0, 1])
+@pytest.mark.parametrize("pad", [0, 1, 2])
+@pytest.mark.parametrize("align", [False, True])
+def test_grid_sampler_special_coordinates(oracle, device, dtype, interp, pad, align):
+    """ties, borders, 1e10, inf and NaN grid values (what the reference handles at grid_sampler2_d_simt.h:136-247)"""
+    rng = np.random.default_rng(7)
+    g32 = I.special_grid()
+    for (H, W) in [(5, 8), (10, 10), (1, 7), (64, 64)]:
+        x32 = rng.standard_normal((1, 3, H, W)).astype(np.float32)
+        y, y_ref = _run_gs(oracle, device, x32, g32, dtype, interp, pad, align)
+        _check(y, y_ref, dtype, interp, "gs-special %s %s %s align=%s %s" % (dtype, INTERP[interp], PAD[pad], align,
+                                                                              (H, W)))
+
+
+@pytest.mark.parametrize("dtype", I.DTYPES)
+@pytest.mark.parametrize("interp", [0, 1])
+@pytest.mark.parametrize("pad", [0, 1, 2])
+@pytest.mark.parametrize("align", [False, True])
+def test_grid_sampler_taps_bit_exact(oracle, device, dtype, interp, pad, align):
+    """every integer corner index, weight and NaN flag equals the oracle's, bit for bit"""
+    from ops_cv_amd import aclnn
+    rng = np.random.default_rng(11)
+    grids = [I.special_grid(), rng.uniform(-1.5, 1.5, (2, 37, 41, 2)).astype(np.float32),
+             I.affine_grid(rng, 3, 64, 64)]
+    for g32 in grids:
+        for (H, W) in [(5, 8), (10, 10), (64, 64), (1080, 1920), (3, 1)]:
+            g = I.cast_np(g32, dtype)
+            ref = oracle.grid_sampler2d_taps(g, H, W, interp, pad, align, dtype=I.oracle_code(dtype))
+            got = aclnn.grid_sampler2d_taps(I.to_torch(g, dtype, device), H, W, interp, pad, align)
+            assert np.array_equal(got["flag"], ref["flag"])
+            live = ref["flag"] == 0
+            assert np.array_equal(got["ix0"][live], ref["ix0"][live])
+            assert np.array_equal(got["iy0"][live], ref["iy0"][live])
+            assert np.array_equal(got["w"][live].view(np.uint32), ref["w"][live].view(np.uint32))
+
+
+def _run_up(oracle, device, x32, out_hw, dtype, align, sh=0.0, sw=0.0):
+    from ops_cv_amd import aclnn
+    import torch
+    x = I.cast_np(x32, dtype)
+    y_ref = oracle.upsample_bilinear2d(x, out_hw, align, sh, sw, dtype=I.oracle_code(dtype))
+    y = aclnn.upsample_bilinear2d(I.to_torch(x, dtype, device), out_hw, align, sh, sw)
+    torch.cuda.synchronize()
+    return I.from_torch(y, dtype), y_ref
+
+
+@pytest.mark.parametrize("dtype", I.DTYPES)
+@pytest.mark.parametrize("align", [False, True])
+def test_upsample_random(oracle, device, dtype, align):
+    rng = np.random.default_rng(50 + int(align))
+    cases = [((2, 3, 7, 9), (14, 18)), ((1, 2, 5, 5), (13, 7)), ((2, 2, 16, 16), (5, 3)), ((1, 1, 1, 4), (2, 16)),
+             ((1, 1, 1, 4), (3, 16)), ((2, 3, 1, 1), (4, 4)), ((2, 3, 1, 1), (16, 16)), ((2, 3, 6, 6), (1, 1)),
+             ((1, 4, 9, 11), (9, 11)), ((1, 2, 56, 56), (112, 112)), ((1, 1, 33, 65), (67, 200)),
+             ((1, 2, 4, 2), (8, 4))]
+    for shape, out_hw in cases:
+        x32 = rng.standard_normal(shape).astype(np.float32)
+        y, y_ref = _run_up(oracle, device, x32, out_hw, dtype, align)
+        _check(y, y_ref, dtype, 0, "up %s align=%s %s->%s" % (dtype, align, shape, out_hw))
+        if dtype == "fp32":
+            assert np.array_equal(y.view(np.uint32), y_ref.view(np.uint32)), "fp32 upsample should be bit-exact"
+
+
+@pytest.mark.parametrize("dtype", I.DTYPES)
+def test_upsample_user_scales(oracle, device, dtype):
+    rng = np.random.default_rng(60)
+    x32 = rng.standard_normal((2, 3, 10, 12)).astype(np.float32)
+    for out_hw, sh, sw in [((20, 24), 2.0, 2.0), ((25, 18), 2.5, 1.5), ((15, 30), 1.7, 2.4)]:
+        y, y_ref = _run_up(oracle, device, x32, out_hw, dtype, False, sh, sw)
+        _check(y, y_ref, dtype, 0, "up-scales %s %s" % (dtype, out_hw))
