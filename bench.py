@@ -1,0 +1,354 @@
+#!/usr/bin/env python3
+"""Benchmark of the bilinear gather/interpolate path on one MI355X.
+
+A "step" is one full two-phase call (GetWorkspaceSize + launch) of the hot path over one synthetic batch whose
+tensors already live in HBM.  The headline workload is the grid_sampler2d fp16 N=16 C=256 configuration; the
+other configurations are reported beside it in "other_workloads".  Steps rotate over several independent
+tensor sets so that a step does not find its operands in the last-level cache left by the previous one.
+
+Prints ONE JSON line (see the keys below).  `roofline.achieved` = algorithmic bytes (every tensor touched
+once) / average launch duration measured with HIP events on the launch stream.  `cpu_baseline` = the CPU
+oracle (a port of the reference arithmetic) timed on this machine's host cores on the same workload.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "tests")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+HBM_PEAK_GBS = 8000.0
+
+# name -> description of the workloads (shapes as in the baseline configuration list)
+GS_WORKLOADS = {
+    "C1": dict(dtype="fp32", x=(1, 3, 64, 64), grid=(1, 32, 32), kind="uniform", interp=0, pad=0, align=False,
+               sets=4),
+    "C3": dict(dtype="fp16", x=(16, 256, 64, 64), grid=(16, 64, 64), kind="affine", interp=0, pad=0, align=False,
+               sets=8),
+    "C5": dict(dtype="bf16", x=(8, 128, 128, 128), grid=(8, 256, 256), kind="random", interp=0, pad=1, align=True,
+               sets=3),
+}
+UP_WORKLOADS = {
+    "C2": dict(dtype="fp32", x=(8, 64, 56, 56), out=(112, 112), align=False, scales=(2.0, 2.0), dist="normal",
+               sets=8),
+    "C4": dict(dtype="fp16", x=(4, 16, 1080, 1920), out=(2160, 3840), align=True, scales=(2.0, 2.0),
+               dist="uniform", sets=2),
+}
+INTERP_NAMES = {0: "bilinear", 1: "nearest"}
+PAD_NAMES = {0: "zeros", 1: "border", 2: "reflection"}
+
+
+def esize(dtype):
+    return 4 if dtype == "fp32" else 2
+
+
+def make_gs_inputs(name, seed_base):
+    import numpy as np
+    import inputs as I
+    w = GS_WORKLOADS[name]
+    N, C, H, W = w["x"]
+    _, Ho, Wo = w["grid"]
+    rng = np.random.default_rng(seed_base)
+    if name == "C1":
+        x32 = rng.uniform(0, 1, w["x"]).astype(np.float32)
+    else:
+        x32 = rng.standard_normal(w["x"], dtype=np.float32)
+    if w["kind"] == "uniform":
+        g32 = rng.uniform(-1, 1, (N, Ho, Wo, 2)).astype(np.float32)
+    elif w["kind"] == "affine":
+        g32 = I.affine_grid(rng, N, Ho, Wo)
+    else:
+        g32 = rng.uniform(-1.1, 1.1, (N, Ho, Wo, 2)).astype(np.float32)
+    return I.cast_np(x32, w["dtype"]), I.cast_np(g32, w["dtype"])
+
+
+def make_up_input(name, seed_base):
+    import numpy as np
+    import inputs as I
+    w = UP_WORKLOADS[name]
+    rng = np.random.default_rng(seed_base)
+    if w["dist"] == "normal":
+        x32 = rng.standard_normal(w["x"], dtype=np.float32)
+    else:
+        x32 = rng.random(w["x"], dtype=np.float32)
+    return I.cast_np(x32, w["dtype"])
+
+
+def load_bench_lib():
+    path = os.path.join(ROOT, "ops_cv_amd", "libopscv_bench.so")
+    if not os.path.exists(path):
+        raise RuntimeError("libopscv_bench.so is not built: run `python -m ops_cv_amd.build`")
+    L = ctypes.CDLL(path)
+    vp, i64, u64 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_uint64
+    pd = ctypes.POINTER(ctypes.c_double)
+    L.opscv_bench_grid_sampler2d.restype = ctypes.c_int
+    L.opscv_bench_grid_sampler2d.argtypes = [ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.c_int,
+                                            i64, i64, ctypes.c_bool, vp, u64, ctypes.c_int, vp, pd, pd]
+    L.opscv_bench_upsample_bilinear2d.restype = ctypes.c_int
+    L.opscv_bench_upsample_bilinear2d.argtypes = [ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.c_int, vp,
+                                                 ctypes.c_bool, ctypes.c_double, ctypes.c_double, vp, u64,
+                                                 ctypes.c_int, vp, pd, pd]
+    return L
+
+
+class Timed:
+    def __init__(self, event_ms, wall_ms, steps):
+        self.kernel_us = event_ms * 1e3 / steps
+        self.step_ms = wall_ms / steps
+
+
+def bench_gs(name, steps, warmup, interp=None, pad=None, align=None, sets=None, check=True):
+    import numpy as np
+    import torch
+    import inputs as I
+    import oracle_lib
+    from ops_cv_amd import aclnn
+    w = dict(GS_WORKLOADS[name])
+    if interp is not None:
+        w["interp"] = interp
+    if pad is not None:
+        w["pad"] = pad
+    if align is not None:
+        w["align"] = align
+    nsets = w["sets"] if sets is None else sets
+    dev = torch.device("cuda:0")
+    L = load_bench_lib()
+    N, C, H, W = w["x"]
+    _, Ho, Wo = w["grid"]
+    xs, gs, ys, hx, hg, hy = [], [], [], [], [], []
+    x0 = g0 = None
+    for s in range(nsets):
+        x, g = make_gs_inputs(name, 1000 + s)
+        if s == 0:
+            x0, g0 = x, g
+        xs.append(I.to_torch(x, w["dtype"], dev))
+        gs.append(I.to_torch(g, w["dtype"], dev))
+        ys.append(torch.empty((N, C, Ho, Wo), dtype=xs[-1].dtype, device=dev))
+        hx.append(aclnn.tensor_handle(xs[-1]))
+        hg.append(aclnn.tensor_handle(gs[-1]))
+        hy.append(aclnn.tensor_handle(ys[-1]))
+    arr = lambda hs: (ctypes.c_void_p * len(hs))(*hs)
+    ax, ag, ay = arr(hx), arr(hg), arr(hy)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ev, wall = ctypes.c_double(0), ctypes.c_double(0)
+
+    def run(k):
+        rc = L.opscv_bench_grid_sampler2d(ax, ag, ay, nsets, w["interp"], w["pad"], w["align"], None, 0, k, stream,
+                                          ctypes.byref(ev), ctypes.byref(wall))
+        if rc != 0:
+            raise RuntimeError("bench loop failed rc=%d: %s" % (rc, aclnn.load_library().aclGetRecentErrMsg()))
+        return Timed(ev.value, wall.value, k)
+
+    st, _, ex = aclnn.get_workspace_size_grid_sampler2d(hx[0], hg[0], w["interp"], w["pad"], w["align"], hy[0])
+    variant = aclnn.executor_variant(ex)
+    aclnn.destroy_executor(ex)
+    if warmup > 0:
+        run(warmup)
+    torch.cuda.synchronize()
+    t = run(steps)
+    torch.cuda.synchronize()
+    parity = None
+    if check:
+        ref = oracle_lib.grid_sampler2d(x0, g0, w["interp"], w["pad"], w["align"], dtype=I.oracle_code(w["dtype"]))
+        got = I.from_torch(ys[0], w["dtype"])
+        a, b = I.as_f32(got, w["dtype"]), I.as_f32(ref, w["dtype"])
+        nan = np.isnan(b)
+        assert np.array_equal(np.isnan(a), nan)
+        d = np.abs(np.where(nan, 0, a) - np.where(nan, 0, b))
+        parity = {"max_abs_err": float(d.max()), "bit_exact": bool(np.array_equal(got.view(np.uint8),
+                                                                                    ref.view(np.uint8)))}
+    for h in hx + hg + hy:
+        aclnn.destroy_tensor(h)
+    samples = N * C * Ho * Wo
+    e = esize(w["dtype"])
+    alg_bytes = (N * C * H * W + N * Ho * Wo * 2 + samples) * e
+    desc = "%s grid_sampler2d %s x%s grid%s %s %s align_corners=%s" % (
+        name, w["dtype"], tuple(w["x"]), (N, Ho, Wo, 2), INTERP_NAMES[w["interp"]], PAD_NAMES[w["pad"]], w["align"])
+    return dict(workload=desc, samples=samples, alg_bytes=alg_bytes, timed=t, variant=variant, parity=parity,
+                sets=nsets, cpu=(x0, g0, w))
+
+
+def bench_up(name, steps, warmup, sets=None, check=True):
+    import numpy as np
+    import torch
+    import inputs as I
+    import oracle_lib
+    from ops_cv_amd import aclnn
+    w = UP_WORKLOADS[name]
+    nsets = w["sets"] if sets is None else sets
+    dev = torch.device("cuda:0")
+    L = load_bench_lib()
+    N, C, Hs, Ws = w["x"]
+    Hd, Wd = w["out"]
+    xs, ys, hx, hy = [], [], [], []
+    x0 = None
+    for s in range(nsets):
+        x = make_up_input(name, 2000 + s)
+        if s == 0:
+            x0 = x
+        xs.append(I.to_torch(x, w["dtype"], dev))
+        ys.append(torch.empty((N, C, Hd, Wd), dtype=xs[-1].dtype, device=dev))
+        hx.append(aclnn.tensor_handle(xs[-1], aclnn.ACL_FORMAT_NCHW))
+        hy.append(aclnn.tensor_handle(ys[-1], aclnn.ACL_FORMAT_NCHW))
+    arr = lambda hs: (ctypes.c_void_p * len(hs))(*hs)
+    ax, ay = arr(hx), arr(hy)
+    size = aclnn.create_int_array([Hd, Wd])
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ev, wall = ctypes.c_double(0), ctypes.c_double(0)
+
+    def run(k):
+        rc = L.opscv_bench_upsample_bilinear2d(ax, ay, nsets, size, w["align"], w["scales"][0], w["scales"][1], None,
+                                               0, k, stream, ctypes.byref(ev), ctypes.byref(wall))
+        if rc != 0:
+            raise RuntimeError("bench loop failed rc=%d: %s" % (rc, aclnn.load_library().aclGetRecentErrMsg()))
+        return Timed(ev.value, wall.value, k)
+
+    st, _, ex = aclnn.get_workspace_size_upsample_bilinear2d(hx[0], size, w["align"], w["scales"][0], w["scales"][1],
+                                                             hy[0])
+    variant = aclnn.executor_variant(ex)
+    aclnn.destroy_executor(ex)
+    if warmup > 0:
+        run(warmup)
+    torch.cuda.synchronize()
+    t = run(steps)
+    torch.cuda.synchronize()
+    parity = None
+    if check:
+        # the oracle on the first plane block only (the full 4K case would take minutes on one core)
+        planes = min(N * C, 4)
+        xsub = x0.reshape(N * C, 1, Hs, Ws)[:planes]
+        ref = oracle_lib.upsample_bilinear2d(xsub, (Hd, Wd), w["align"], w["scales"][0], w["scales"][1],
+                                             dtype=I.oracle_code(w["dtype"]))
+        got = I.from_torch(ys[0], w["dtype"]).reshape(N * C, 1, Hd, Wd)[:planes]
+        d = np.abs(I.as_f32(got, w["dtype"]) - I.as_f32(ref, w["dtype"]))
+        parity = {"max_abs_err": float(d.max()), "bit_exact": bool(np.array_equal(got.view(np.uint8),
+                                                                                    ref.view(np.uint8))),
+                  "planes_checked": planes}
+    for h in hx + hy:
+        aclnn.destroy_tensor(h)
+    aclnn.destroy_int_array(size)
+    samples = N * C * Hd * Wd
+    e = esize(w["dtype"])
+    alg_bytes = (N * C * Hs * Ws + samples) * e
+    desc = "%s upsample_bilinear2d %s %s->%s align_corners=%s" % (name, w["dtype"], tuple(w["x"]),
+                                                                  (N, C, Hd, Wd), w["align"])
+    return dict(workload=desc, samples=samples, alg_bytes=alg_bytes, timed=t, variant=variant, parity=parity,
+                sets=nsets, cpu=(x0, w))
+
+
+def roofline_of(r):
+    gbs = r["alg_bytes"] / (r["timed"].kernel_us * 1e-6) / 1e9
+    return {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+            "kernel_us": round(r["timed"].kernel_us, 3), "algorithmic_bytes": r["alg_bytes"],
+            "kernel": r["variant"]}
+
+
+def summary_of(r):
+    t = r["timed"]
+    return {"workload": r["workload"], "samples_per_s": r["samples"] / (t.step_ms * 1e-3),
+            "ms_per_step": round(t.step_ms, 6), "roofline": roofline_of(r), "parity_vs_oracle": r["parity"],
+            "tensor_sets": r["sets"]}
+
+
+def cpu_baseline_gs(x0, g0, w, budget_s=12.0):
+    """The CPU oracle on the full headline workload, all host threads, repeated for about `budget_s` seconds."""
+    import inputs as I
+    import oracle_lib
+    threads = oracle_lib.lib().oracle_max_threads()
+    N, C = w["x"][0], w["x"][1]
+    Ho, Wo = w["grid"][1], w["grid"][2]
+    samples = N * C * Ho * Wo
+    reps, t0 = 0, time.perf_counter()
+    while True:
+        oracle_lib.grid_sampler2d(x0, g0, w["interp"], w["pad"], w["align"], dtype=I.oracle_code(w["dtype"]),
+                                  threads=threads)
+        reps += 1
+        el = time.perf_counter() - t0
+        if el > budget_s or reps >= 200:
+            break
+    t1 = time.perf_counter()
+    oracle_lib.grid_sampler2d(x0, g0, w["interp"], w["pad"], w["align"], dtype=I.oracle_code(w["dtype"]), threads=1)
+    one = time.perf_counter() - t1
+    return {"value": samples * reps / el, "unit": "samples/s", "cores": threads, "kind": "port",
+            "sample": "full workload (%d output samples) x %d repetitions, OpenMP static over output pixels" % (
+                samples, reps),
+            "single_thread_samples_per_s": samples / one}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="C3", help="headline workload (C1..C5)")
+    ap.add_argument("--only", action="store_true", help="skip the other workloads and the CPU baseline")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the path shards over the batch axis with no "
+              "communication); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
+        sys.exit(3)
+    torch.cuda.set_device(0)
+
+    head = args.workload
+    if head in GS_WORKLOADS:
+        r = bench_gs(head, args.steps, args.warmup)
+    else:
+        r = bench_up(head, args.steps, args.warmup)
+    t = r["timed"]
+    line = {
+        "metric": "output samples/s, grid_sampler2d fp16 N16 C256 (achieved HBM GB/s in roofline)" if head == "C3"
+        else "output samples/s",
+        "value": r["samples"] / (t.step_ms * 1e-3),
+        "unit": "samples/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": t.step_ms,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": r["workload"], "tensor_sets_rotated": r["sets"], "kernel": r["variant"],
+                   "parity_vs_oracle": r["parity"]},
+        "roofline": roofline_of(r),
+    }
+    if not args.only and not args.no_cpu and head in GS_WORKLOADS:
+        line["cpu_baseline"] = cpu_baseline_gs(*r["cpu"])
+    else:
+        line["cpu_baseline"] = None
+    if not args.only:
+        others = {}
+        if head == "C3":
+            for interp in (0, 1):
+                for pad in (0, 1, 2):
+                    if interp == 0 and pad == 0:
+                        continue
+                    rr = bench_gs("C3", args.steps, args.warmup, interp=interp, pad=pad)
+                    others["C3_%s_%s" % (INTERP_NAMES[interp], PAD_NAMES[pad])] = summary_of(rr)
+            rr = bench_gs("C3", args.steps, args.warmup, sets=1)
+            others["C3_bilinear_zeros_same_buffers_every_step"] = summary_of(rr)
+        for name in ("C1", "C5"):
+            if name != head:
+                others[name] = summary_of(bench_gs(name, args.steps, args.warmup))
+        for name in ("C2", "C4"):
+            if name != head:
+                k = args.steps if name == "C2" else max(5, args.steps // 10)
+                others[name] = summary_of(bench_up(name, k, max(2, args.warmup // 10)))
+        line["other_workloads"] = others
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
