@@ -1,0 +1,71 @@
+// Dispatch helpers shared by the grid-sampler translation units.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "kernels.hpp"
+
+namespace opscv {
+
+// Expands the run-time (interp, pad, align) triple into the template instantiation.
+template <typename T, typename F>
+inline hipError_t dispatch_modes(const GridSamplerArgs& a, F&& f)
+{
+#define OPSCV_CASE(I, P, A)                                   \
+    if (a.interp == I && a.pad == P && (a.align != 0) == A) { \
+        return f.template operator()<T, I, P, A>();           \
+    }
+    OPSCV_CASE(0, 0, false)
+    OPSCV_CASE(0, 0, true)
+    OPSCV_CASE(0, 1, false)
+    OPSCV_CASE(0, 1, true)
+    OPSCV_CASE(0, 2, false)
+    OPSCV_CASE(0, 2, true)
+    OPSCV_CASE(1, 0, false)
+    OPSCV_CASE(1, 0, true)
+    OPSCV_CASE(1, 1, false)
+    OPSCV_CASE(1, 1, true)
+    OPSCV_CASE(1, 2, false)
+    OPSCV_CASE(1, 2, true)
+#undef OPSCV_CASE
+    return hipErrorInvalidValue;
+}
+
+template <typename F>
+inline hipError_t dispatch_elem(const GridSamplerArgs& a, F&& f)
+{
+    switch (a.elem) {
+        case Elem::F32: return dispatch_modes<float>(a, f);
+        case Elem::F16: return dispatch_modes<_Float16>(a, f);
+        case Elem::BF16: return dispatch_modes<__bf16>(a, f);
+    }
+    return hipErrorInvalidValue;
+}
+
+// Shape limits shared by every variant (the reference tiling enforces the same ones,
+// grid_sampler2_d_tiling.cpp:92-156): every extent and the input plane fit in int32.
+inline bool gs_shapes_ok(const GridSamplerArgs& a)
+{
+    if (a.N < 0 || a.C < 0 || a.Hout < 0 || a.Wout < 0 || a.Hin <= 0 || a.Win <= 0) {
+        return false;
+    }
+    const int64_t lim = INT32_MAX;
+    if (a.N > lim || a.C > lim || a.Hin > lim || a.Win > lim || a.Hout > lim || a.Wout > lim) {
+        return false;
+    }
+    if (a.Hin * a.Win > lim) {
+        return false;
+    }
+    if (a.Hout != 0 && a.Wout != 0 && a.Hout > INT64_MAX / a.Wout / (a.N > 0 ? a.N : 1) / 2) {
+        return false;
+    }
+    return true;
+}
+
+
+// LDS-staged variant (gs2d_lds.hip).  Sets *handled to false, launching nothing, when the shape does not fit
+// its assumptions (input plane too large for LDS); the caller then falls back to the direct variant.
+hipError_t run_gs2d_lds(const GridSamplerArgs& a, hipStream_t stream, bool* handled);
+const char* gs2d_lds_variant_name(const GridSamplerArgs& a);
+
+}  // namespace opscv

@@ -9,6 +9,9 @@
 // registers across the channel loop.
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
+#include "gs2d_common.hpp"
 #include "kernels.hpp"
 #include "sampler_math.hpp"
 
@@ -150,61 +153,6 @@ hipError_t run_taps(const GridSamplerArgs& a, TapRecord* taps, hipStream_t strea
     return hipGetLastError();
 }
 
-// Expands the run-time (interp, pad, align) triple into the template instantiation.
-template <typename T, typename F>
-hipError_t dispatch_modes(const GridSamplerArgs& a, F&& f)
-{
-#define OPSCV_CASE(I, P, A)                                   \
-    if (a.interp == I && a.pad == P && (a.align != 0) == A) { \
-        return f.template operator()<T, I, P, A>();           \
-    }
-    OPSCV_CASE(0, 0, false)
-    OPSCV_CASE(0, 0, true)
-    OPSCV_CASE(0, 1, false)
-    OPSCV_CASE(0, 1, true)
-    OPSCV_CASE(0, 2, false)
-    OPSCV_CASE(0, 2, true)
-    OPSCV_CASE(1, 0, false)
-    OPSCV_CASE(1, 0, true)
-    OPSCV_CASE(1, 1, false)
-    OPSCV_CASE(1, 1, true)
-    OPSCV_CASE(1, 2, false)
-    OPSCV_CASE(1, 2, true)
-#undef OPSCV_CASE
-    return hipErrorInvalidValue;
-}
-
-template <typename F>
-hipError_t dispatch_elem(const GridSamplerArgs& a, F&& f)
-{
-    switch (a.elem) {
-        case Elem::F32: return dispatch_modes<float>(a, f);
-        case Elem::F16: return dispatch_modes<_Float16>(a, f);
-        case Elem::BF16: return dispatch_modes<__bf16>(a, f);
-    }
-    return hipErrorInvalidValue;
-}
-
-// Shape limits shared by every variant (the reference tiling enforces the same ones,
-// grid_sampler2_d_tiling.cpp:92-156): every extent and the input plane fit in int32.
-bool shapes_ok(const GridSamplerArgs& a)
-{
-    if (a.N < 0 || a.C < 0 || a.Hout < 0 || a.Wout < 0 || a.Hin <= 0 || a.Win <= 0) {
-        return false;
-    }
-    const int64_t lim = INT32_MAX;
-    if (a.N > lim || a.C > lim || a.Hin > lim || a.Win > lim || a.Hout > lim || a.Wout > lim) {
-        return false;
-    }
-    if (a.Hin * a.Win > lim) {
-        return false;
-    }
-    if (a.Hout != 0 && a.Wout != 0 && a.Hout > INT64_MAX / a.Wout / (a.N > 0 ? a.N : 1) / 2) {
-        return false;
-    }
-    return true;
-}
-
 struct DirectLauncher {
     const GridSamplerArgs& a;
     hipStream_t stream;
@@ -228,11 +176,29 @@ struct TapsLauncher {
 
 }  // namespace
 
-const char* grid_sampler2d_variant(const GridSamplerArgs&) { return "direct"; }
+namespace {
+// OPSCV_GS_VARIANT=direct forces the direct kernel (benchmark knob)
+bool force_direct()
+{
+    const char* v = getenv("OPSCV_GS_VARIANT");
+    return v != nullptr && v[0] == 'd';
+}
+}  // namespace
+
+const char* grid_sampler2d_variant(const GridSamplerArgs& a)
+{
+    if (!force_direct()) {
+        const char* n = gs2d_lds_variant_name(a);
+        if (n != nullptr) {
+            return n;
+        }
+    }
+    return "direct";
+}
 
 hipError_t launch_grid_sampler2d(const GridSamplerArgs& a, hipStream_t stream)
 {
-    if (!shapes_ok(a) || a.interp < 0 || a.interp > 1 || a.pad < 0 || a.pad > 2) {
+    if (!gs_shapes_ok(a) || a.interp < 0 || a.interp > 1 || a.pad < 0 || a.pad > 2) {
         return hipErrorInvalidValue;
     }
     if (a.N == 0 || a.C == 0 || a.Hout == 0 || a.Wout == 0) {
@@ -241,12 +207,19 @@ hipError_t launch_grid_sampler2d(const GridSamplerArgs& a, hipStream_t stream)
     if (a.x == nullptr || a.grid == nullptr || a.y == nullptr) {
         return hipErrorInvalidValue;
     }
+    if (!force_direct()) {
+        bool handled = false;
+        hipError_t e = run_gs2d_lds(a, stream, &handled);
+        if (handled || e != hipSuccess) {
+            return e;
+        }
+    }
     return dispatch_elem(a, DirectLauncher{a, stream});
 }
 
 hipError_t launch_grid_sampler2d_taps(const GridSamplerArgs& a, TapRecord* taps, hipStream_t stream)
 {
-    if (!shapes_ok(a) || a.interp < 0 || a.interp > 1 || a.pad < 0 || a.pad > 2) {
+    if (!gs_shapes_ok(a) || a.interp < 0 || a.interp > 1 || a.pad < 0 || a.pad > 2) {
         return hipErrorInvalidValue;
     }
     if (a.N == 0 || a.Hout == 0 || a.Wout == 0) {
