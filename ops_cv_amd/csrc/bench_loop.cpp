@@ -29,7 +29,7 @@ __attribute__((visibility("default"))) int opscv_bench_grid_sampler2d(
         return -1;
     }
     auto t0 = std::chrono::steady_clock::now();
-    hipEventRecord(e0, s);
+    (void)hipEventRecord(e0, s);
     for (int k = 0; k < steps; k++) {
         const int i = k % sets;
         uint64_t ws = 0;
@@ -43,17 +43,17 @@ __attribute__((visibility("default"))) int opscv_bench_grid_sampler2d(
             return st;
         }
     }
-    hipEventRecord(e1, s);
+    (void)hipEventRecord(e1, s);
     if (hipEventSynchronize(e1) != hipSuccess) {
         return -1;
     }
     auto t1 = std::chrono::steady_clock::now();
     float ms = 0.0f;
-    hipEventElapsedTime(&ms, e0, e1);
+    (void)hipEventElapsedTime(&ms, e0, e1);
     *event_ms = ms;
     *wall_ms = std::chrono::duration<double, std::milli>(t1 - t0).count();
-    hipEventDestroy(e0);
-    hipEventDestroy(e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
     return 0;
 }
 
@@ -71,7 +71,7 @@ __attribute__((visibility("default"))) int opscv_bench_upsample_bilinear2d(
         return -1;
     }
     auto t0 = std::chrono::steady_clock::now();
-    hipEventRecord(e0, s);
+    (void)hipEventRecord(e0, s);
     for (int k = 0; k < steps; k++) {
         const int i = k % sets;
         uint64_t ws = 0;
@@ -86,17 +86,17 @@ __attribute__((visibility("default"))) int opscv_bench_upsample_bilinear2d(
             return st;
         }
     }
-    hipEventRecord(e1, s);
+    (void)hipEventRecord(e1, s);
     if (hipEventSynchronize(e1) != hipSuccess) {
         return -1;
     }
     auto t1 = std::chrono::steady_clock::now();
     float ms = 0.0f;
-    hipEventElapsedTime(&ms, e0, e1);
+    (void)hipEventElapsedTime(&ms, e0, e1);
     *event_ms = ms;
     *wall_ms = std::chrono::duration<double, std::milli>(t1 - t0).count();
-    hipEventDestroy(e0);
-    hipEventDestroy(e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
     return 0;
 }
 

@@ -1,0 +1,88 @@
+// Grid sampler 2-D forward, LDS-staged variant: launch plan and the typed launch template.
+// The three element types are instantiated in separate translation units so that they compile in parallel.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "gs2d_common.hpp"
+#include "gs2d_lds_kernel.hpp"
+
+namespace opscv {
+
+struct LdsPlan {
+    bool ok = false;
+    int cls = 0;  // index into kPitch / kCgs
+    int ppt = 4;
+    int copy_gran = 16;
+    uint32_t lds_bytes = 0;
+    uint32_t tiles_per_n = 0, cblocks = 0;
+    int32_t chans_per_block = 0;
+};
+
+constexpr int kThreads = 512;
+// plane pitch in LDS and planes per stage for the four size classes; two stage buffers are resident
+constexpr int kPitch[4] = {2064, 8208, 32784, 81904};
+constexpr int kCgs[4] = {8, 4, 2, 1};
+
+LdsPlan make_lds_plan(const GridSamplerArgs& a);
+
+template <typename T, int I, int P, bool A, int PPT, int CGS, int PITCH>
+hipError_t launch_one(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t stream)
+{
+    auto kernel = gs2d_lds_kernel<T, I, P, A, kThreads, PPT, CGS, PITCH>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit);
+        if (e != hipSuccess) {
+            return e;
+        }
+        attr_set = true;
+    }
+    const int64_t esz = sizeof(T);
+    const int pair_aligned = (reinterpret_cast<uintptr_t>(a.grid) % (2 * esz) == 0);
+    const uint32_t blocks = (uint32_t)(a.N * p.tiles_per_n * p.cblocks);
+    hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kThreads), p.lds_bytes, stream, (const T*)a.x, (const T*)a.grid,
+                       (T*)a.y, (int32_t)a.C, (int32_t)a.Hin, (int32_t)a.Win, (int32_t)(a.Hout * a.Wout),
+                       p.tiles_per_n, p.cblocks, p.chans_per_block, p.copy_gran, pair_aligned);
+    return hipGetLastError();
+}
+
+template <typename T, int I, int P, bool A, int PPT>
+hipError_t launch_class(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t stream)
+{
+    switch (p.cls) {
+        case 0: return launch_one<T, I, P, A, PPT, kCgs[0], kPitch[0]>(a, p, stream);
+        case 1: return launch_one<T, I, P, A, PPT, kCgs[1], kPitch[1]>(a, p, stream);
+        case 2: return launch_one<T, I, P, A, PPT, kCgs[2], kPitch[2]>(a, p, stream);
+        default: return launch_one<T, I, P, A, PPT, kCgs[3], kPitch[3]>(a, p, stream);
+    }
+}
+
+// Expands (interp, pad, align, pixels per lane, size class) for one element type and launches.
+template <typename T>
+struct LdsTypedLauncher {
+    const GridSamplerArgs& a;
+    const LdsPlan& p;
+    hipStream_t stream;
+    template <typename U, int I, int P, bool A>
+    hipError_t operator()() const
+    {
+        if (p.ppt == 4) {
+            return launch_class<T, I, P, A, 4>(a, p, stream);
+        }
+        return launch_class<T, I, P, A, 1>(a, p, stream);
+    }
+};
+
+template <typename T>
+hipError_t lds_launch_typed(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t stream)
+{
+    return dispatch_modes<T>(a, LdsTypedLauncher<T>{a, p, stream});
+}
+
+extern template hipError_t lds_launch_typed<float>(const GridSamplerArgs&, const LdsPlan&, hipStream_t);
+extern template hipError_t lds_launch_typed<_Float16>(const GridSamplerArgs&, const LdsPlan&, hipStream_t);
+extern template hipError_t lds_launch_typed<__bf16>(const GridSamplerArgs&, const LdsPlan&, hipStream_t);
+
+}  // namespace opscv
