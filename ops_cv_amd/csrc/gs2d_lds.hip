@@ -21,7 +21,7 @@ LdsPlan make_lds_plan(const GridSamplerArgs& a)
         p.cls++;
     }
     const int cgs = kCgs[p.cls];
-    p.lds_bytes = (uint32_t)(2 * kPitch[p.cls] * cgs);
+    p.lds_bytes = (uint32_t)(kNbuf[p.cls] * kPitch[p.cls] * cgs);
     p.ppt = (out_plane >= 2 * kThreads) ? 4 : 1;
     const int64_t tile = (int64_t)kThreads * p.ppt;
     p.tiles_per_n = (uint32_t)((out_plane + tile - 1) / tile);
@@ -52,8 +52,10 @@ LdsPlan make_lds_plan(const GridSamplerArgs& a)
     } else if (plane_bytes % 4 == 0 && xa % 4 == 0) {
         p.copy_gran = 4;
     } else {
-        p.copy_gran = (int)esz;
+        return p;  // odd byte counts: the asynchronous copy moves whole dwords, leave it to the direct variant
     }
+    // all tiles of one (n, channel block) group on one XCD: needs the group count to be a multiple of 8
+    p.xcd_swizzle = ((a.N * cblocks) % 8 == 0) ? 1 : 0;
     p.ok = true;
     return p;
 }
@@ -64,8 +66,8 @@ const char* gs2d_lds_variant_name(const GridSamplerArgs& a)
     if (!p.ok) {
         return nullptr;
     }
-    static const char* names[4] = {"lds_planes_p2064x8", "lds_planes_p8208x4", "lds_planes_p32784x2",
-                                   "lds_planes_p81904x1"};
+    static const char* names[4] = {"lds_ring_p2064_4x4", "lds_ring_p8208_2x4", "lds_ring_p32784_1x4",
+                                   "lds_ring_p81904_1x2"};
     return names[p.cls];
 }
 

@@ -18,6 +18,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "sampler_math.hpp"
 
 namespace opscv {
@@ -94,10 +96,59 @@ __device__ __forceinline__ void buffer_store_elem(float v, __amdgpu_buffer_rsrc_
     }
 }
 
+// s_waitcnt that waits only for the vector-memory counter to drop to `n` (gfx9 encoding: vmcnt is split over
+// bits 3:0 and 15:14; the other counters are left at their "do not wait" maximum).
+template <int N>
+__device__ __forceinline__ void wait_vmcnt_imm()
+{
+    static_assert(N >= 0 && N <= 63, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4) | (0xF << 8));
+}
+
+// Waits until at most  per_copy_stage * mine + per_sampled_stage * sampled  vector-memory operations of this
+// wavefront are outstanding; `mine` (copy instructions per plane of this wavefront, 0..4) and `sampled`
+// (0..MAX_SAMPLED) are wave-uniform run-time values, the products are turned into immediates here.
+// Anything outside the table waits for everything.
+template <int PER_COPY, int PER_SAMPLED, int MAX_SAMPLED>
+__device__ __forceinline__ void wait_vmcnt_table(uint32_t mine, uint32_t sampled)
+{
+    static_assert(MAX_SAMPLED <= 3, "table covers up to three sampled stages");
+    constexpr int kMaxMine = 4;
+    if (mine > (uint32_t)kMaxMine || sampled > (uint32_t)MAX_SAMPLED ||
+        PER_COPY * kMaxMine + PER_SAMPLED * MAX_SAMPLED > 63) {
+        wait_vmcnt_imm<0>();
+        return;
+    }
+    const uint32_t key = __builtin_amdgcn_readfirstlane(mine * 4u + sampled);
+    switch (key) {
+#define OPSCV_W(M, S)                                                             \
+    case (M) * 4 + (S):                                                           \
+        wait_vmcnt_imm<(PER_COPY * (M) + PER_SAMPLED * (S)) <= 63 ? (PER_COPY * (M) + PER_SAMPLED * (S)) : 0>(); \
+        break;
+#define OPSCV_WM(M) OPSCV_W(M, 0) OPSCV_W(M, 1) OPSCV_W(M, 2) OPSCV_W(M, 3)
+        OPSCV_WM(0) OPSCV_WM(1) OPSCV_WM(2) OPSCV_WM(3) OPSCV_WM(4)
+#undef OPSCV_WM
+#undef OPSCV_W
+        default: wait_vmcnt_imm<0>(); break;
+    }
+}
+
+// Workgroup barrier without the memory fences of __syncthreads(): a fence would make the compiler drain the
+// vector-memory counter (the global->LDS copies count there), which is exactly what the ring must not do.
+// The caller has already waited for the operations it depends on; the empty asm statements keep the compiler
+// from moving LDS accesses across the barrier.
+__device__ __forceinline__ void lds_barrier()
+{
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
 // Starts the asynchronous copy of `nch` consecutive input planes (plane_bytes each, contiguous in global memory
 // from `src`) to LDS at `dst` with PITCH bytes between planes.  G = bytes per lane (16 or 4): the largest
 // granule that divides the plane size and the source alignment.  Each wavefront instruction moves 64*G
-// contiguous bytes; lanes past the end of a plane are masked off.
+// contiguous bytes; lanes past the end of a plane are masked off.  Wavefront w takes chunks w, w+NWAVES, ...
+// of every plane, so it issues the same number of instructions for every full stage.
 template <int G, int THREADS, int CGS, int PITCH>
 __device__ __forceinline__ void issue_stage_copy(const char* src, char* dst, uint32_t plane_bytes, int nch)
 {
@@ -126,59 +177,80 @@ __device__ __forceinline__ void issue_stage_copy(const char* src, char* dst, uin
     }
 }
 
-// PITCH: compile-time byte distance between staged planes in LDS (>= padded plane size + 16).  The LDS holds two
-// buffers of CGS planes each.  Compile-time so that a tap address is "register + immediate".
-template <typename T, int INTERP, int PAD, bool ALIGN, int THREADS, int PPT, int CGS, int PITCH>
-__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 4))) void gs2d_lds_kernel(const T* __restrict__ x, const T* __restrict__ grid,
-                                                           T* __restrict__ y, int32_t C, int32_t H, int32_t W,
-                                                           int32_t out_plane, uint32_t tiles_per_n,
-                                                           uint32_t cblocks, int32_t chans_per_block,
-                                                           int32_t copy_gran, int32_t pair_aligned)
+// LDS layout: a ring of NBUF stage slots, each CGS planes at PITCH bytes (PITCH >= padded plane size + 16,
+// compile-time so that a tap address is "register + immediate").  Stage s lives in slot s % NBUF and up to
+// NBUF-1 later stages are in flight while it is sampled.
+//
+// Completion of a stage copy is tracked with the wavefront's own vector-memory counter, which retires in issue
+// order: when stage s is needed, the operations this wavefront issued after the copy of stage s are the copies
+// of the NBUF-2 following stages and the output stores of the stages sampled since, so waiting until at most
+// that many operations are outstanding guarantees the copy has landed without draining the newer ones.  The
+// count is exact only while every stage involved is a full one; otherwise the wait is for everything.
+template <typename T, int INTERP, int PAD, bool ALIGN, int THREADS, int PPT, int CGS, int NBUF, int PITCH>
+__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 4))) void gs2d_lds_kernel(
+    const T* __restrict__ x, const T* __restrict__ grid, T* __restrict__ y, int32_t C, int32_t H, int32_t W,
+    int32_t out_plane, uint32_t tiles_per_n, uint32_t cblocks, int32_t chans_per_block, int32_t copy_gran,
+    int32_t pair_aligned, int32_t xcd_swizzle)
 {
     extern __shared__ uint4 smem_raw[];
     char* lds = reinterpret_cast<char*>(smem_raw);
     constexpr int NT = (INTERP == 0) ? 4 : 1;
-    constexpr int BUF_BYTES = CGS * PITCH;
+    constexpr int SLOT_BYTES = CGS * PITCH;
+    constexpr int DEPTH = NBUF - 1;          // stages in flight ahead of the one being sampled
+    constexpr int NWAVES = THREADS / 64;
+    constexpr uint32_t STORES_PER_STAGE = PPT * CGS;
     const int tid = threadIdx.x;
 
-    uint32_t b = blockIdx.x;
-    const uint32_t tile = b % tiles_per_n;
-    b /= tiles_per_n;
-    const uint32_t cb = b % cblocks;
-    const uint32_t n = b / cblocks;
+    // Block -> (group = (n, channel block), tile).  Workgroups are handed to the 8 XCDs round-robin by index;
+    // with the swizzle all tiles of one group (they read the same input planes) land on the same XCD next to
+    // each other in time, so the planes are fetched into one L2 once.
+    uint32_t group, tile;
+    if (xcd_swizzle) {
+        const uint32_t xcd = blockIdx.x & 7u;
+        const uint32_t i = blockIdx.x >> 3;
+        group = (i / tiles_per_n) * 8u + xcd;
+        tile = i % tiles_per_n;
+    } else {
+        group = blockIdx.x / tiles_per_n;
+        tile = blockIdx.x % tiles_per_n;
+    }
+    const uint32_t cb = group % cblocks;
+    const uint32_t n = group / cblocks;
 
     const int32_t plane_elems = H * W;
     const uint32_t plane_bytes = (uint32_t)plane_elems * (uint32_t)sizeof(T);
     const uint32_t zero_off = round_up16(plane_bytes);
     const int32_t c_begin = (int32_t)cb * chans_per_block;
     const int32_t c_end = (c_begin + chans_per_block < C) ? c_begin + chans_per_block : C;
-    const int32_t nstages = (c_end - c_begin + CGS - 1) / CGS;
+    const int32_t nchan = c_end - c_begin;
+    const int32_t nstages = (nchan + CGS - 1) / CGS;
+    const int32_t nfull = nchan / CGS;  // stages 0 .. nfull-1 hold CGS planes
     const char* xb = reinterpret_cast<const char*>(x + ((int64_t)n * C + c_begin) * plane_elems);
     const size_t stage_bytes = (size_t)CGS * plane_bytes;
 
-    auto start_stage = [&](int32_t s, int buf) {
-        const int32_t left = c_end - c_begin - s * CGS;
+    // copy instructions this wavefront issues per plane (copy_gran is 16 or 4 bytes per lane)
+    uint32_t copies_per_plane;
+    {
+        const uint32_t chunk = 64u * (uint32_t)copy_gran;
+        const uint32_t chunks = (plane_bytes + chunk - 1) / chunk;
+        const uint32_t wave = __builtin_amdgcn_readfirstlane((uint32_t)tid >> 6);
+        copies_per_plane = (chunks > wave) ? (chunks - wave + NWAVES - 1) / NWAVES : 0;
+    }
+
+    auto start_stage = [&](int32_t s, int slot) {
+        const int32_t left = nchan - s * CGS;
         const int nch = left < CGS ? left : CGS;
         const char* src = xb + (size_t)s * stage_bytes;
-        char* dst = lds + buf * BUF_BYTES;
+        char* dst = lds + slot * SLOT_BYTES;
         if (copy_gran == 16) {
             issue_stage_copy<16, THREADS, CGS, PITCH>(src, dst, plane_bytes, nch);
-        } else if (copy_gran == 4) {
-            issue_stage_copy<4, THREADS, CGS, PITCH>(src, dst, plane_bytes, nch);
         } else {
-            // planes whose size or address is not a multiple of 4 bytes: element-wise copy through registers
-            const T* se = reinterpret_cast<const T*>(src);
-            for (int k = 0; k < nch; k++) {
-                T* de = reinterpret_cast<T*>(dst + k * PITCH);
-                for (int32_t i = tid; i < plane_elems; i += THREADS) {
-                    de[i] = se[(int64_t)k * plane_elems + i];
-                }
-            }
+            issue_stage_copy<4, THREADS, CGS, PITCH>(src, dst, plane_bytes, nch);
         }
     };
 
-    // the zero slots behind each staged plane (both buffers); stage copies never touch them
-    if (tid < 2 * CGS * 4) {
+    // the zero slots behind each staged plane (all ring slots); stage copies never touch them
+    if (tid < NBUF * CGS * 4) {
         reinterpret_cast<uint32_t*>(lds + (tid >> 2) * PITCH + zero_off)[tid & 3] = 0u;
     }
     start_stage(0, 0);
@@ -223,11 +295,20 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 4)))
         }
     }
 
+    // the rest of the prologue: stages 1 .. DEPTH-1 (stage 0 went out before the grid loads so that the wait
+    // for the grid values does not also wait for these)
+#pragma unroll
+    for (int s = 1; s < DEPTH; s++) {
+        if (s < nstages) {
+            start_stage(s, s);
+        }
+    }
+
     T* yb = y + ((int64_t)n * C + c_begin) * out_plane;
     const uint32_t out_plane_bytes = (uint32_t)out_plane * (uint32_t)sizeof(T);
 
     auto sample_stage = [&](int32_t s, const char* buf) {
-        const int32_t left = c_end - c_begin - s * CGS;
+        const int32_t left = nchan - s * CGS;
         T* ys = yb + (int64_t)s * CGS * out_plane;
         if (left >= CGS) {
             // software pipeline over the channels of the stage: the taps of channel k+1 are read from LDS
@@ -269,22 +350,42 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 4)))
         }
     };
 
-    // Stage s lives in buffer s & 1.  Per stage: wait for its copy (issued one stage earlier), barrier (which
-    // also tells that everybody left the other buffer), start the next copy into the other buffer, sample.
-    for (int32_t s = 0; s < nstages; s += 2) {
-        __builtin_amdgcn_s_waitcnt(0);
-        __syncthreads();
-        if (s + 1 < nstages) {
-            start_stage(s + 1, 1);
+    // One step of the ring: wait for the copy of stage s, barrier (it also tells that every wavefront has left
+    // the slot that is refilled next), start the copy of stage s + DEPTH, sample stage s.
+    auto step = [&](int32_t s, auto slot_tag) {
+        constexpr int SLOT = decltype(slot_tag)::value;
+        // Operations issued after the copy of stage s: copies of stages s+1 .. s+DEPTH-1 and the stores of the
+        // min(s, DEPTH) stages sampled since.  Exact only when those later stages exist and are full.
+        if (s + DEPTH - 1 < nfull) {
+            const uint32_t sampled = (s < DEPTH) ? (uint32_t)s : (uint32_t)DEPTH;
+            wait_vmcnt_table<(DEPTH - 1) * CGS, STORES_PER_STAGE, (DEPTH < 3 ? DEPTH : 3)>(copies_per_plane, sampled);
+        } else {
+            wait_vmcnt_imm<0>();
         }
-        sample_stage(s, lds);
-        if (s + 1 < nstages) {
-            __builtin_amdgcn_s_waitcnt(0);
-            __syncthreads();
-            if (s + 2 < nstages) {
-                start_stage(s + 2, 0);
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the zero-slot writes before the first barrier
+        lds_barrier();
+        if (s + DEPTH < nstages) {
+            start_stage(s + DEPTH, (SLOT + DEPTH) % NBUF);
+        }
+        sample_stage(s, lds + SLOT * SLOT_BYTES);
+    };
+
+    for (int32_t s = 0; s < nstages; s += NBUF) {
+        step(s, std::integral_constant<int, 0>{});
+        if constexpr (NBUF > 1) {
+            if (s + 1 < nstages) {
+                step(s + 1, std::integral_constant<int, 1 % NBUF>{});
             }
-            sample_stage(s + 1, lds + BUF_BYTES);
+        }
+        if constexpr (NBUF > 2) {
+            if (s + 2 < nstages) {
+                step(s + 2, std::integral_constant<int, 2 % NBUF>{});
+            }
+        }
+        if constexpr (NBUF > 3) {
+            if (s + 3 < nstages) {
+                step(s + 3, std::integral_constant<int, 3 % NBUF>{});
+            }
         }
     }
 }

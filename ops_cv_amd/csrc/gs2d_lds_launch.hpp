@@ -14,6 +14,7 @@ struct LdsPlan {
     int cls = 0;  // index into kPitch / kCgs
     int ppt = 4;
     int copy_gran = 16;
+    int xcd_swizzle = 0;
     uint32_t lds_bytes = 0;
     uint32_t tiles_per_n = 0, cblocks = 0;
     int32_t chans_per_block = 0;
@@ -22,14 +23,15 @@ struct LdsPlan {
 constexpr int kThreads = 512;
 // plane pitch in LDS and planes per stage for the four size classes; two stage buffers are resident
 constexpr int kPitch[4] = {2064, 8208, 32784, 81904};
-constexpr int kCgs[4] = {8, 4, 2, 1};
+constexpr int kCgs[4] = {4, 2, 1, 1};   // planes per stage
+constexpr int kNbuf[4] = {4, 4, 4, 2};  // ring slots (stages resident in LDS)
 
 LdsPlan make_lds_plan(const GridSamplerArgs& a);
 
-template <typename T, int I, int P, bool A, int PPT, int CGS, int PITCH>
+template <typename T, int I, int P, bool A, int PPT, int CGS, int NBUF, int PITCH>
 hipError_t launch_one(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t stream)
 {
-    auto kernel = gs2d_lds_kernel<T, I, P, A, kThreads, PPT, CGS, PITCH>;
+    auto kernel = gs2d_lds_kernel<T, I, P, A, kThreads, PPT, CGS, NBUF, PITCH>;
     static bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -44,7 +46,7 @@ hipError_t launch_one(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t st
     const uint32_t blocks = (uint32_t)(a.N * p.tiles_per_n * p.cblocks);
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kThreads), p.lds_bytes, stream, (const T*)a.x, (const T*)a.grid,
                        (T*)a.y, (int32_t)a.C, (int32_t)a.Hin, (int32_t)a.Win, (int32_t)(a.Hout * a.Wout),
-                       p.tiles_per_n, p.cblocks, p.chans_per_block, p.copy_gran, pair_aligned);
+                       p.tiles_per_n, p.cblocks, p.chans_per_block, p.copy_gran, pair_aligned, p.xcd_swizzle);
     return hipGetLastError();
 }
 
@@ -52,10 +54,10 @@ template <typename T, int I, int P, bool A, int PPT>
 hipError_t launch_class(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t stream)
 {
     switch (p.cls) {
-        case 0: return launch_one<T, I, P, A, PPT, kCgs[0], kPitch[0]>(a, p, stream);
-        case 1: return launch_one<T, I, P, A, PPT, kCgs[1], kPitch[1]>(a, p, stream);
-        case 2: return launch_one<T, I, P, A, PPT, kCgs[2], kPitch[2]>(a, p, stream);
-        default: return launch_one<T, I, P, A, PPT, kCgs[3], kPitch[3]>(a, p, stream);
+        case 0: return launch_one<T, I, P, A, PPT, kCgs[0], kNbuf[0], kPitch[0]>(a, p, stream);
+        case 1: return launch_one<T, I, P, A, PPT, kCgs[1], kNbuf[1], kPitch[1]>(a, p, stream);
+        case 2: return launch_one<T, I, P, A, PPT, kCgs[2], kNbuf[2], kPitch[2]>(a, p, stream);
+        default: return launch_one<T, I, P, A, PPT, kCgs[3], kNbuf[3], kPitch[3]>(a, p, stream);
     }
 }
 
