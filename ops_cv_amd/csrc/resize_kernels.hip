@@ -10,6 +10,8 @@
 // (the file is compiled with -ffp-contract=off).
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
 #include "kernels.hpp"
 #include "sampler_math.hpp"
 
@@ -78,6 +80,88 @@ __global__ __launch_bounds__(kThreads) void resize_nchw_generic_kernel(const T* 
     }
 }
 
+// Row-band variant for NCHW when the output row is a whole number of 16-byte vectors.
+//
+// A lane owns V = 16/sizeof(T) consecutive output columns and walks down a band of output rows.  The column
+// taps (two source offsets and the lambda per column) are computed once per lane.  The reference formula
+//     out = (1-dy) * ((1-dx)*TL + dx*TR) + dy * ((1-dx)*BL + dx*BR)
+// is separable as written: the two inner terms depend on the source row only, so the horizontally blended
+// source row  Hrow(y)[col] = (1-dx)*x[y,x0] + dx*x[y,x1]  is kept in registers and reused by every output row
+// that touches source row y (two of them for a x2 upscale) -- same operations, same order, same bits.
+// Each lane writes one 16-byte vector per output row; a wavefront writes 1 KiB contiguous.
+template <typename T, bool HALF_PIXEL, int BAND>
+__global__ __launch_bounds__(kThreads) void resize_nchw_band_kernel(const T* __restrict__ x, T* __restrict__ y,
+                                                                     int64_t planes, int32_t Hs, int32_t Ws,
+                                                                     int32_t Hd, int32_t Wd, float scale_h,
+                                                                     float scale_w)
+{
+    constexpr int V = 16 / (int)sizeof(T);
+    const int32_t chunk = blockIdx.x * kThreads + threadIdx.x;
+    const int32_t col0 = chunk * V;
+    if (col0 >= Wd) {
+        return;
+    }
+    int32_t xo0[V], xo1[V];
+    float dx[V];
+#pragma unroll
+    for (int i = 0; i < V; i++) {
+        const AxisTap t = axis_tap<HALF_PIXEL>(col0 + i, scale_w, Ws);
+        xo0[i] = t.i0;
+        xo1[i] = t.i1;
+        dx[i] = t.lambda;
+    }
+    const int32_t h_begin = blockIdx.y * BAND;
+    const int32_t h_end = (h_begin + BAND < Hd) ? h_begin + BAND : Hd;
+
+    for (int64_t pl = blockIdx.z; pl < planes; pl += gridDim.z) {
+        const T* xp = x + pl * Hs * (int64_t)Ws;
+        T* yp = y + (pl * Hd + h_begin) * (int64_t)Wd + col0;
+        float ha[V], hb[V];  // blended source rows ya and yb
+        int32_t ya = -1, yb = -1;
+        auto blend_row = [&](float* hrow, int32_t ys) {
+            const T* row = xp + (int64_t)ys * Ws;
+#pragma unroll
+            for (int i = 0; i < V; i++) {
+                const float l = ElemIO<T>::load(row + xo0[i]);
+                const float r = ElemIO<T>::load(row + xo1[i]);
+                hrow[i] = (1.0f - dx[i]) * l + dx[i] * r;
+            }
+        };
+        for (int32_t h = h_begin; h < h_end; h++) {
+            const AxisTap ty = axis_tap<HALF_PIXEL>(h, scale_h, Hs);
+            const int32_t y0 = __builtin_amdgcn_readfirstlane(ty.i0);
+            const int32_t y1 = __builtin_amdgcn_readfirstlane(ty.i1);
+            const float dy = ty.lambda;
+            // top row -> ha
+            if (y0 != ya) {
+                if (y0 == yb) {
+#pragma unroll
+                    for (int i = 0; i < V; i++) {
+                        ha[i] = hb[i];
+                    }
+                } else {
+                    blend_row(ha, y0);
+                }
+                ya = y0;
+            }
+            // bottom row -> hb (or ha again when both taps are the same source row)
+            if (y1 != ya && y1 != yb) {
+                blend_row(hb, y1);
+                yb = y1;
+            }
+            T outv[V];
+#pragma unroll
+            for (int i = 0; i < V; i++) {
+                const float bot = (y1 == ya) ? ha[i] : hb[i];
+                const float o = (1.0f - dy) * ha[i] + dy * bot;
+                ElemIO<T>::store(&outv[i], o);
+            }
+            *reinterpret_cast<uint4*>(yp) = *reinterpret_cast<const uint4*>(outv);
+            yp += Wd;
+        }
+    }
+}
+
 // Generic NHWC variant: one lane per (w, c) element of an output row.
 template <typename T, bool HALF_PIXEL>
 __global__ __launch_bounds__(kThreads) void resize_nhwc_generic_kernel(const T* __restrict__ x, T* __restrict__ y,
@@ -133,6 +217,27 @@ __global__ __launch_bounds__(kThreads) void resize_fill_kernel(const T* __restri
     }
 }
 
+constexpr int kBand = 32;  // output rows a workgroup walks down (vertical reuse of blended source rows)
+
+// The band variant stores whole 16-byte vectors: needs Wd to be a multiple of the vector length, a 16-byte
+// aligned output and a band count that fits the grid.
+template <typename T>
+bool band_variant_ok(const ResizeArgs& a)
+{
+    constexpr int V = 16 / (int)sizeof(T);
+    if (a.channels_last || a.mode != ResizeMode::Bilinear) {
+        return false;
+    }
+    if (a.Wd % V != 0 || reinterpret_cast<uintptr_t>(a.y) % 16 != 0) {
+        return false;
+    }
+    if ((a.Hd + kBand - 1) / kBand > 65535) {
+        return false;
+    }
+    const char* v = getenv("OPSCV_RESIZE_VARIANT");
+    return !(v != nullptr && v[0] == 'g');  // OPSCV_RESIZE_VARIANT=generic forces the generic kernel
+}
+
 template <typename T>
 hipError_t run_resize(const ResizeArgs& a, hipStream_t stream)
 {
@@ -167,6 +272,23 @@ hipError_t run_resize(const ResizeArgs& a, hipStream_t stream)
         return hipGetLastError();
     }
     const int64_t planes = a.N * a.C;
+    if (band_variant_ok<T>(a)) {
+        constexpr int V = 16 / (int)sizeof(T);
+        const int64_t chunks = a.Wd / V;
+        const int64_t bands = (a.Hd + kBand - 1) / kBand;
+        dim3 grid((unsigned)((chunks + kThreads - 1) / kThreads), (unsigned)bands,
+                  (unsigned)(planes < 65535 ? planes : 65535));
+        if (a.half_pixel) {
+            hipLaunchKernelGGL((resize_nchw_band_kernel<T, true, kBand>), grid, dim3(kThreads), 0, stream, x, y,
+                               planes, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h,
+                               a.scale_w);
+        } else {
+            hipLaunchKernelGGL((resize_nchw_band_kernel<T, false, kBand>), grid, dim3(kThreads), 0, stream, x, y,
+                               planes, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h,
+                               a.scale_w);
+        }
+        return hipGetLastError();
+    }
     const int64_t rows = planes * a.Hd;
     dim3 grid((unsigned)((a.Wd + kThreads - 1) / kThreads), (unsigned)(rows < 65535 ? rows : 65535));
     if (a.half_pixel) {
@@ -189,7 +311,16 @@ const char* resize_variant(const ResizeArgs& a)
         case ResizeMode::FirstPixel: return "first_pixel";
         default: break;
     }
-    return a.channels_last ? "nhwc_generic" : "nchw_generic";
+    if (a.channels_last) {
+        return "nhwc_generic";
+    }
+    bool band = false;
+    switch (a.elem) {
+        case Elem::F32: band = band_variant_ok<float>(a); break;
+        case Elem::F16: band = band_variant_ok<_Float16>(a); break;
+        case Elem::BF16: band = band_variant_ok<__bf16>(a); break;
+    }
+    return band ? "nchw_band32" : "nchw_generic";
 }
 
 hipError_t launch_resize(const ResizeArgs& a, hipStream_t stream)
