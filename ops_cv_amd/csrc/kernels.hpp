@@ -25,6 +25,10 @@ hipError_t launch_resize(const ResizeArgs& a, hipStream_t stream);
 hipError_t launch_strided_copy(const StridedView& v, void* contiguous, int elem_bytes, bool gather,
                                hipStream_t stream);
 
+// LDS-staged row-band resize (resize_band_lds.hip); *handled is false when the shape does not qualify.
+hipError_t run_resize_band_lds(const ResizeArgs& a, hipStream_t stream, bool* handled);
+bool resize_band_lds_applicable(const ResizeArgs& a);
+
 // Name of the kernel variant the launcher would pick for these arguments (for benchmarks and tests).
 const char* grid_sampler2d_variant(const GridSamplerArgs& a);
 const char* resize_variant(const ResizeArgs& a);

@@ -1,0 +1,178 @@
+// Bilinear resize, NCHW, LDS-staged row-band variant for gfx950: device code.
+//
+// Arithmetic: image/resize_bilinear_v2/op_kernel/arch35/resize_bilinear_v2_simt_nchw.h:108-144 (see resize_math.hpp).
+//
+// A workgroup owns (plane, band of BAND output rows, block of THREADS*V output columns), V = 16/sizeof(T).
+//   * The source rows the band touches, cut to the columns the block touches, are copied from HBM into LDS
+//     once with the asynchronous global->LDS loads (16 or 4 bytes per lane), so every source element is read
+//     from memory once per workgroup and the unaligned two-byte tap reads never leave the CU.
+//   * A lane owns V consecutive output columns; its column taps (two LDS byte offsets and lambda per column)
+//     are computed once.  The reference formula  out = (1-dy)*((1-dx)*TL + dx*TR) + dy*((1-dx)*BL + dx*BR)  is
+//     separable as written: the horizontally blended source row  Hrow(y)[col] = (1-dx)*x[y,x0] + dx*x[y,x1]  is
+//     kept in registers and reused by every output row that touches source row y -- same operations in the
+//     same order, so the result is bit-identical to the per-pixel evaluation.
+//   * Row taps (y0, y1, dy) of the band are computed by the first BAND lanes once and broadcast per row.
+//   * Each lane writes one 16-byte vector per output row through a buffer descriptor (lanes past the row end
+//     are dropped by its range check); a wavefront writes 1 KiB contiguous.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "resize_math.hpp"
+#include "sampler_math.hpp"
+
+namespace opscv {
+
+typedef __attribute__((address_space(1))) const void* rs_global_cptr_t;
+typedef __attribute__((address_space(3))) void* rs_lds_ptr_t;
+
+constexpr uint32_t kRsBufferFlags = 0x00020000u;  // raw buffer, 32-bit data format
+
+struct BandLdsParams {
+    int64_t planes;
+    int32_t Hs, Ws, Hd, Wd;
+    float scale_h, scale_w;
+    int32_t lds_pitch;  // bytes between staged source rows (multiple of 16)
+    int32_t lds_rows;   // staged rows the LDS allocation holds
+    int32_t gran;       // bytes per lane of the asynchronous copy: 16 or 4
+};
+
+template <typename T, bool HALF_PIXEL, int THREADS, int BAND>
+__global__ __launch_bounds__(THREADS) void resize_band_lds_kernel(const T* __restrict__ x, T* __restrict__ y,
+                                                                   BandLdsParams p)
+{
+    static_assert(BAND <= 64, "row taps are held one per lane of a wavefront");
+    constexpr int V = 16 / (int)sizeof(T);
+    constexpr int NWAVES = THREADS / 64;
+    extern __shared__ uint4 smem_raw[];
+    char* lds = reinterpret_cast<char*>(smem_raw);
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+
+    // ---- block geometry (uniform) ----
+    const int32_t c_begin = blockIdx.x * (THREADS * V);
+    const int32_t c_last = ((c_begin + THREADS * V < p.Wd) ? c_begin + THREADS * V : p.Wd) - 1;
+    const int32_t h_begin = blockIdx.y * BAND;
+    const int32_t h_end = (h_begin + BAND < p.Hd) ? h_begin + BAND : p.Hd;
+    const int32_t ge = p.gran / (int)sizeof(T);  // elements per copy granule
+    const int32_t xs_lo = axis_tap<HALF_PIXEL>(c_begin, p.scale_w, p.Ws).i0;
+    const int32_t xs_hi = axis_tap<HALF_PIXEL>(c_last, p.scale_w, p.Ws).i1;
+    const int32_t seg_col0 = xs_lo / ge * ge;
+    const int32_t seg_elems = (xs_hi + 1 - seg_col0 + ge - 1) / ge * ge;  // stays inside the row: Ws % ge == 0
+    const uint32_t seg_bytes = (uint32_t)seg_elems * (uint32_t)sizeof(T);
+    const int32_t ys_lo = axis_tap<HALF_PIXEL>(h_begin, p.scale_h, p.Hs).i0;
+    const int32_t ys_hi = axis_tap<HALF_PIXEL>(h_end - 1, p.scale_h, p.Hs).i1;
+    int32_t rows = ys_hi - ys_lo + 1;
+    rows = (rows < p.lds_rows) ? rows : p.lds_rows;  // the host sized the allocation for the exact maximum
+
+    // ---- per-lane column taps ----
+    const int32_t col0 = c_begin + tid * V;
+    uint32_t to0[V], to1[V];
+    float dx[V], omdx[V];
+#pragma unroll
+    for (int i = 0; i < V; i++) {
+        int32_t c = col0 + i;
+        c = (c < p.Wd) ? c : p.Wd - 1;
+        const AxisTap t = axis_tap<HALF_PIXEL>(c, p.scale_w, p.Ws);
+        to0[i] = (uint32_t)(t.i0 - seg_col0) * (uint32_t)sizeof(T);
+        to1[i] = (uint32_t)(t.i1 - seg_col0) * (uint32_t)sizeof(T);
+        dx[i] = t.lambda;
+        omdx[i] = 1.0f - t.lambda;
+    }
+    // ---- row taps of the band: lane l holds output row h_begin + l ----
+    int32_t my_y0, my_y1;
+    float my_dy;
+    {
+        int32_t h = h_begin + lane;
+        h = (h < p.Hd) ? h : p.Hd - 1;
+        const AxisTap t = axis_tap<HALF_PIXEL>(h, p.scale_h, p.Hs);
+        my_y0 = t.i0 - ys_lo;
+        my_y1 = t.i1 - ys_lo;
+        my_dy = t.lambda;
+    }
+    const uint32_t out_row_bytes = (uint32_t)p.Wd * (uint32_t)sizeof(T);
+    const uint32_t out_off = (col0 < p.Wd) ? (uint32_t)col0 * (uint32_t)sizeof(T) : 0x80000000u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane((uint32_t)tid >> 6);
+
+    for (int64_t pl = blockIdx.z; pl < p.planes; pl += gridDim.z) {
+        // ---- stage the source rows of this band ----
+        const char* src0 = reinterpret_cast<const char*>(x + (pl * p.Hs + ys_lo) * (int64_t)p.Ws + seg_col0);
+        const uint32_t chunk = 64u * (uint32_t)p.gran;
+        const uint32_t chunks_per_row = (seg_bytes + chunk - 1) / chunk;
+        const uint32_t total_chunks = chunks_per_row * (uint32_t)rows;
+        for (uint32_t q = wave; q < total_chunks; q += NWAVES) {
+            const uint32_t r = q / chunks_per_row;
+            const uint32_t cb = (q - r * chunks_per_row) * chunk;
+            const uint32_t lane_off = cb + (uint32_t)lane * (uint32_t)p.gran;
+            if (lane_off < seg_bytes) {
+                const rs_global_cptr_t g = (rs_global_cptr_t)(src0 + (size_t)r * p.Ws * sizeof(T) + lane_off);
+                const rs_lds_ptr_t l = (rs_lds_ptr_t)(lds + r * p.lds_pitch + cb);
+                if (p.gran == 16) {
+                    __builtin_amdgcn_global_load_lds(g, l, 16, 0, 0);
+                } else {
+                    __builtin_amdgcn_global_load_lds(g, l, 4, 0, 0);
+                }
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+
+        T* yp = y + (pl * p.Hd + h_begin) * (int64_t)p.Wd;
+        float ha[V], hb[V];  // blended source rows ya and yb (row indices relative to ys_lo)
+        int32_t ya = -1, yb = -1;
+        auto blend_row = [&](float* hrow, int32_t ys) {
+            const char* row = lds + ys * p.lds_pitch;
+            T l[V], r[V];
+#pragma unroll
+            for (int i = 0; i < V; i++) {
+                l[i] = *reinterpret_cast<const T*>(row + to0[i]);
+                r[i] = *reinterpret_cast<const T*>(row + to1[i]);
+            }
+#pragma unroll
+            for (int i = 0; i < V; i++) {
+                hrow[i] = omdx[i] * ElemIO<T>::load(&l[i]) + dx[i] * ElemIO<T>::load(&r[i]);
+            }
+        };
+        for (int32_t h = h_begin; h < h_end; h++) {
+            const int32_t y0 = __builtin_amdgcn_readlane(my_y0, h - h_begin);
+            const int32_t y1 = __builtin_amdgcn_readlane(my_y1, h - h_begin);
+            const float dy = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int32_t, my_dy),
+                                                                                  h - h_begin));
+            if (y0 != ya) {
+                if (y0 == yb) {
+#pragma unroll
+                    for (int i = 0; i < V; i++) {
+                        ha[i] = hb[i];
+                    }
+                } else {
+                    blend_row(ha, y0);
+                }
+                ya = y0;
+            }
+            if (y1 != ya && y1 != yb) {
+                blend_row(hb, y1);
+                yb = y1;
+            }
+            const float omdy = 1.0f - dy;
+            T outv[V];
+            if (y1 == ya) {
+#pragma unroll
+                for (int i = 0; i < V; i++) {
+                    ElemIO<T>::store(&outv[i], omdy * ha[i] + dy * ha[i]);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < V; i++) {
+                    ElemIO<T>::store(&outv[i], omdy * ha[i] + dy * hb[i]);
+                }
+            }
+            const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(yp, 0, out_row_bytes, kRsBufferFlags);
+            typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+            __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4*>(outv), rsrc, (int)out_off, 0, 0);
+            yp += p.Wd;
+        }
+        __syncthreads();  // everybody is done with the staged rows before the next plane overwrites them
+    }
+}
+
+}  // namespace opscv

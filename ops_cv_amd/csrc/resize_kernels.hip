@@ -13,6 +13,7 @@
 #include <cstdlib>
 
 #include "kernels.hpp"
+#include "resize_math.hpp"
 #include "sampler_math.hpp"
 
 namespace opscv {
@@ -20,35 +21,6 @@ namespace opscv {
 namespace {
 
 constexpr int kThreads = 256;
-
-struct AxisTap {
-    int32_t i0, i1;
-    float lambda;
-};
-
-// resize_bilinear_v2_simt_nchw.h:108-134 for one axis
-template <bool HALF_PIXEL>
-__device__ __forceinline__ AxisTap axis_tap(int32_t d, float scale, int32_t len_src)
-{
-    float orig;
-    if (HALF_PIXEL) {
-        orig = ((float)d + 0.5f) * scale - 0.5f;
-    } else {
-        orig = (float)d * scale;
-    }
-    if (orig < 0.0f) {
-        orig = 0.0f;
-    }
-    const float fl = __builtin_floorf(orig);
-    const float lo = (orig > 0.0f) ? fl : 0.0f;
-    const float hi = (orig > 0.0f) ? __builtin_ceilf(orig) : 0.0f;
-    const float last = (float)(len_src - 1);
-    AxisTap t;
-    t.i0 = (lo < last) ? (int32_t)lo : len_src - 1;
-    t.i1 = (hi < last) ? (int32_t)hi : len_src - 1;
-    t.lambda = orig - fl;
-    return t;
-}
 
 // Generic NCHW variant: one lane per output pixel of a row, rows and planes on the other grid axes.
 template <typename T, bool HALF_PIXEL>
@@ -272,6 +244,13 @@ hipError_t run_resize(const ResizeArgs& a, hipStream_t stream)
         return hipGetLastError();
     }
     const int64_t planes = a.N * a.C;
+    {
+        bool handled = false;
+        const hipError_t e = run_resize_band_lds(a, stream, &handled);
+        if (handled || e != hipSuccess) {
+            return e;
+        }
+    }
     if (band_variant_ok<T>(a)) {
         constexpr int V = 16 / (int)sizeof(T);
         const int64_t chunks = a.Wd / V;
@@ -313,6 +292,9 @@ const char* resize_variant(const ResizeArgs& a)
     }
     if (a.channels_last) {
         return "nhwc_generic";
+    }
+    if (resize_band_lds_applicable(a)) {
+        return "nchw_band32_lds";
     }
     bool band = false;
     switch (a.elem) {
