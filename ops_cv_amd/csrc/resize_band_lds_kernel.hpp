@@ -35,6 +35,8 @@ struct BandLdsParams {
     int32_t lds_pitch;  // bytes between staged source rows (multiple of 16)
     int32_t lds_rows;   // staged rows the LDS allocation holds
     int32_t gran;       // bytes per lane of the asynchronous copy: 16 or 4
+    int32_t streaming;  // 1: mark the output stores non-temporal (outputs much larger than the caches)
+    float neg_zero;     // -0.0f, passed in so that fma(v, w, -0) is not folded back into a multiply
 };
 
 template <typename T, bool HALF_PIXEL, int THREADS, int BAND>
@@ -93,6 +95,7 @@ __global__ __launch_bounds__(THREADS) void resize_band_lds_kernel(const T* __res
     const uint32_t out_row_bytes = (uint32_t)p.Wd * (uint32_t)sizeof(T);
     const uint32_t out_off = (col0 < p.Wd) ? (uint32_t)col0 * (uint32_t)sizeof(T) : 0x80000000u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane((uint32_t)tid >> 6);
+    const float neg_zero = p.neg_zero;
 
     for (int64_t pl = blockIdx.z; pl < p.planes; pl += gridDim.z) {
         // ---- stage the source rows of this band ----
@@ -130,7 +133,11 @@ __global__ __launch_bounds__(THREADS) void resize_band_lds_kernel(const T* __res
             }
 #pragma unroll
             for (int i = 0; i < V; i++) {
-                hrow[i] = omdx[i] * ElemIO<T>::load(&l[i]) + dx[i] * ElemIO<T>::load(&r[i]);
+                // fma(v, w, -0) is v * w bit for bit (also for zero products of either sign); written as an
+                // fma with an addend the compiler cannot see through so that, for 16-bit floats, the conversion
+                // rides on the multiply (mixed-precision fma) instead of costing an instruction of its own
+                hrow[i] = __builtin_fmaf(ElemIO<T>::load(&l[i]), omdx[i], neg_zero) +
+                          __builtin_fmaf(ElemIO<T>::load(&r[i]), dx[i], neg_zero);
             }
         };
         for (int32_t h = h_begin; h < h_end; h++) {
@@ -168,7 +175,11 @@ __global__ __launch_bounds__(THREADS) void resize_band_lds_kernel(const T* __res
             }
             const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(yp, 0, out_row_bytes, kRsBufferFlags);
             typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-            __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4*>(outv), rsrc, (int)out_off, 0, 0);
+            if (p.streaming) {
+                __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4*>(outv), rsrc, (int)out_off, 0, 2);
+            } else {
+                __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4*>(outv), rsrc, (int)out_off, 0, 0);
+            }
             yp += p.Wd;
         }
         __syncthreads();  // everybody is done with the staged rows before the next plane overwrites them

@@ -294,7 +294,7 @@ const char* resize_variant(const ResizeArgs& a)
         return "nhwc_generic";
     }
     if (resize_band_lds_applicable(a)) {
-        return "nchw_band32_lds";
+        return "nchw_band_lds";
     }
     bool band = false;
     switch (a.elem) {
