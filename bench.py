@@ -96,6 +96,22 @@ def load_bench_lib():
     return L
 
 
+PREHEAT_MS = 300.0
+
+
+def preheat(run, warmup):
+    """`warmup` untimed steps, then more untimed steps until PREHEAT_MS of GPU work have run: the clocks of an
+    idle MI355X take tens of milliseconds of load to settle, far longer than a few 20-microsecond launches."""
+    done_ms = 0.0
+    if warmup > 0:
+        done_ms += run(warmup).step_ms * warmup
+    chunk = max(warmup, 10)
+    while done_ms < PREHEAT_MS:
+        t = run(chunk)
+        done_ms += t.step_ms * chunk
+        chunk = min(chunk * 2, 4096)
+
+
 class Timed:
     def __init__(self, event_ms, wall_ms, steps):
         self.kernel_us = event_ms * 1e3 / steps
@@ -147,8 +163,7 @@ def bench_gs(name, steps, warmup, interp=None, pad=None, align=None, sets=None, 
     st, _, ex = aclnn.get_workspace_size_grid_sampler2d(hx[0], hg[0], w["interp"], w["pad"], w["align"], hy[0])
     variant = aclnn.executor_variant(ex)
     aclnn.destroy_executor(ex)
-    if warmup > 0:
-        run(warmup)
+    preheat(run, warmup)
     torch.cuda.synchronize()
     t = run(steps)
     torch.cuda.synchronize()
@@ -212,8 +227,7 @@ def bench_up(name, steps, warmup, sets=None, check=True):
                                                              hy[0])
     variant = aclnn.executor_variant(ex)
     aclnn.destroy_executor(ex)
-    if warmup > 0:
-        run(warmup)
+    preheat(run, warmup)
     torch.cuda.synchronize()
     t = run(steps)
     torch.cuda.synchronize()
@@ -289,7 +303,11 @@ def main():
     ap.add_argument("--workload", default="C3", help="headline workload (C1..C5)")
     ap.add_argument("--only", action="store_true", help="skip the other workloads and the CPU baseline")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--preheat-ms", type=float, default=300.0,
+                    help="untimed GPU work before each timed region, on top of --warmup steps")
     args = ap.parse_args()
+    global PREHEAT_MS
+    PREHEAT_MS = args.preheat_ms
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the path shards over the batch axis with no "
               "communication); run with --gpus 1", file=sys.stderr)
@@ -314,6 +332,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "preheat_ms": args.preheat_ms,
         "ms_per_step": t.step_ms,
         "higher_is_better": True,
         "scaling": "weak",
@@ -344,8 +363,8 @@ def main():
                 others[name] = summary_of(bench_gs(name, args.steps, args.warmup))
         for name in ("C2", "C4"):
             if name != head:
-                k = args.steps if name == "C2" else max(5, args.steps // 10)
-                others[name] = summary_of(bench_up(name, k, max(2, args.warmup // 10)))
+                k = args.steps if name == "C2" else max(5, args.steps // 4)
+                others[name] = summary_of(bench_up(name, k, max(2, args.warmup // 4)))
         line["other_workloads"] = others
     print(json.dumps(line))
 

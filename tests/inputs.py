@@ -15,7 +15,8 @@ def cast_np(a32, dtype):
     if dtype == "fp32":
         return np.ascontiguousarray(a32, dtype=np.float32)
     if dtype == "fp16":
-        return np.ascontiguousarray(a32).astype(np.float16)
+        with np.errstate(over="ignore"):  # special-value grids hold 1e10 and 3e38 on purpose (they become inf)
+            return np.ascontiguousarray(a32).astype(np.float16)
     if dtype == "bf16":
         return f32_to_bf16_bits(a32)
     raise ValueError(dtype)

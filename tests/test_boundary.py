@@ -1,0 +1,234 @@
+"""The C-ABI boundary without a GPU: exported symbols, phase-1 validation order and status codes.
+
+The cases mirror the reference's op_api unit tests, which build descriptors with NULL data pointers and call only
+the GetWorkspaceSize phase: image/grid_sample/tests/ut/op_host/op_api/test_aclnn_grid_sampler2d.cpp and
+image/upsample_bilinear2d/tests/ut/op_host/op_api/test_aclnn_upsample_bilinear_2d.cpp.
+"""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol(aclnn):
+    L = aclnn.load_library()
+    declared = set()
+    for name in os.listdir(os.path.join(ROOT, "include")):
+        text = open(os.path.join(ROOT, "include", name)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        declared |= set(re.findall(r"ACLNN_API\s+[\w\s\*]+?\b(\w+)\s*\(", text))
+    assert {"aclnnGridSampler2DGetWorkspaceSize", "aclnnGridSampler2D", "aclnnUpsampleBilinear2dGetWorkspaceSize",
+            "aclnnUpsampleBilinear2d", "aclCreateTensor", "aclGetRecentErrMsg"} <= declared
+    for sym in sorted(declared):
+        assert hasattr(L, sym), "libopscv_amd.so does not export %s" % sym
+    assert b"gfx950" in L.opscvVersion()
+
+
+class Desc:
+    """Descriptor builder in the spirit of the reference's TensorDesc (NULL data pointer)."""
+
+    def __init__(self, aclnn):
+        self.a = aclnn
+        self.handles = []
+
+    def t(self, dims, dtype, fmt=None, strides=None, offset=0, storage=None):
+        if dims is None:
+            return None
+        fmt = self.a.ACL_FORMAT_ND if fmt is None else fmt
+        h = self.a.create_tensor(dims, dtype, fmt, strides, offset, storage)
+        assert h
+        self.handles.append(h)
+        return h
+
+    def close(self):
+        for h in self.handles:
+            self.a.destroy_tensor(h)
+
+
+@pytest.fixture
+def desc(aclnn):
+    d = Desc(aclnn)
+    yield d
+    d.close()
+
+
+def _gs(aclnn, desc, inp=(1, 1, 5, 8), grid=(1, 3, 3, 2), out=(1, 1, 3, 3), dt=None, gdt=None, odt=None, interp=0, pad=0,
+        align=False, fmts=(None, None, None), **kw):
+    dt = aclnn.ACL_FLOAT if dt is None else dt
+    i = desc.t(inp, dt, fmts[0], **kw)
+    g = desc.t(grid, dt if gdt is None else gdt, fmts[1])
+    o = desc.t(out, dt if odt is None else odt, fmts[2])
+    st, ws, ex = aclnn.get_workspace_size_grid_sampler2d(i, g, interp, pad, align, o)
+    if ex:
+        assert aclnn.destroy_executor(ex) == 0
+    return st, ws, bool(ex)
+
+
+def test_grid_sampler_success_cases(aclnn, desc):
+    for dt in (aclnn.ACL_FLOAT, aclnn.ACL_FLOAT16, aclnn.ACL_BF16):  # reference cases 1, 5, 6
+        st, ws, ex = _gs(aclnn, desc, dt=dt)
+        assert (st, ws, ex) == (0, 0, True)
+    # formats are ignored (cases "nchw nhwc", "hwcn nchw", "nhwc nhwc" with nearest/border)
+    assert _gs(aclnn, desc, fmts=(aclnn.ACL_FORMAT_NCHW, aclnn.ACL_FORMAT_NHWC, aclnn.ACL_FORMAT_ND))[0] == 0
+    assert _gs(aclnn, desc, fmts=(aclnn.ACL_FORMAT_HWCN, aclnn.ACL_FORMAT_NCHW, aclnn.ACL_FORMAT_ND))[0] == 0
+    assert _gs(aclnn, desc, interp=1, pad=1, fmts=(aclnn.ACL_FORMAT_NCHW, aclnn.ACL_FORMAT_NHWC, None))[0] == 0
+    for interp in (0, 1):
+        for pad in (0, 1, 2):
+            for align in (False, True):
+                assert _gs(aclnn, desc, interp=interp, pad=pad, align=align)[0] == 0
+
+
+def test_grid_sampler_null_pointers(aclnn, desc):
+    assert _gs(aclnn, desc, inp=None)[0] == aclnn.ACLNN_ERR_PARAM_NULLPTR
+    assert _gs(aclnn, desc, grid=None)[0] == aclnn.ACLNN_ERR_PARAM_NULLPTR
+    assert _gs(aclnn, desc, out=None)[0] == aclnn.ACLNN_ERR_PARAM_NULLPTR
+    L = aclnn.load_library()
+    i, g, o = desc.t((1, 1, 5, 8), 0), desc.t((1, 3, 3, 2), 0), desc.t((1, 1, 3, 3), 0)
+    ex = ctypes.c_void_p()
+    assert L.aclnnGridSampler2DGetWorkspaceSize(i, g, 0, 0, False, o, None, ctypes.byref(ex)) == 161001
+    assert b"NULL" in L.aclGetRecentErrMsg()
+
+
+def test_grid_sampler_dtype_checks(aclnn, desc):
+    bad = [aclnn.ACL_UINT8, aclnn.ACL_INT8, aclnn.ACL_INT16, aclnn.ACL_INT32, aclnn.ACL_INT64, aclnn.ACL_BOOL,
+           aclnn.ACL_COMPLEX64, aclnn.ACL_COMPLEX128]
+    for dt in bad:  # reference cases 8-15
+        assert _gs(aclnn, desc, dt=dt)[0] == aclnn.ACLNN_ERR_PARAM_INVALID
+    # mismatching dtypes (reference case "format not same": DOUBLE input with FLOAT grid/out)
+    assert _gs(aclnn, desc, dt=aclnn.ACL_DOUBLE, gdt=aclnn.ACL_FLOAT, odt=aclnn.ACL_FLOAT)[0] == 161002
+    assert _gs(aclnn, desc, odt=aclnn.ACL_FLOAT16)[0] == 161002
+    # DOUBLE passes the reference's checks but has no kernel here: documented gap, same status class
+    assert _gs(aclnn, desc, dt=aclnn.ACL_DOUBLE)[0] == 161002
+
+
+def test_grid_sampler_attr_and_shape_checks(aclnn, desc):
+    assert _gs(aclnn, desc, interp=3)[0] == 161002
+    assert _gs(aclnn, desc, interp=-1)[0] == 161002
+    assert _gs(aclnn, desc, pad=3)[0] == 161002
+    assert _gs(aclnn, desc, grid=(2, 3, 3, 2))[0] == 161002          # batch mismatch
+    assert _gs(aclnn, desc, grid=(1, 3, 3, 3))[0] == 161002          # last grid dim must be 2
+    assert _gs(aclnn, desc, inp=(1, 1, 0, 8))[0] == 161002           # empty spatial input
+    assert _gs(aclnn, desc, inp=(1, 1, 5))[0] == 161002              # not 4-D
+    assert _gs(aclnn, desc, out=(1, 2, 3, 3))[0] == 161002           # channel mismatch
+    assert _gs(aclnn, desc, out=(1, 1, 3, 2))[0] == 161002           # grid/out W mismatch
+    # validation order: dtype is reported before attributes and shapes, attributes before shapes
+    L = aclnn.load_library()
+    _gs(aclnn, desc, dt=aclnn.ACL_INT32, interp=7, grid=(2, 3, 3, 2))
+    assert b"dtype" in L.aclGetRecentErrMsg()
+    _gs(aclnn, desc, interp=7, grid=(2, 3, 3, 2))
+    assert b"interpolationMode" in L.aclGetRecentErrMsg()
+    # bicubic is in the validated range but outside this implementation
+    assert _gs(aclnn, desc, interp=2)[0] == 161002
+
+
+def test_grid_sampler_empty_and_views(aclnn, desc):
+    # empty batch / empty grid: success, no workspace, an executor is still handed out
+    assert _gs(aclnn, desc, inp=(0, 1, 5, 8), grid=(0, 3, 3, 2), out=(0, 1, 3, 3)) == (0, 0, True)
+    assert _gs(aclnn, desc, grid=(1, 0, 3, 2), out=(1, 1, 0, 3)) == (0, 0, True)
+    # non-contiguous input view (reference case "not contiguous"): accepted, packed through the workspace
+    st, ws, ex = _gs(aclnn, desc, strides=(40, 40, 1, 5), storage=(1, 1, 8, 5))
+    assert st == 0 and ex and ws >= 40 * 4
+    # contiguous with an offset needs no workspace
+    st, ws, ex = _gs(aclnn, desc, offset=16, storage=(100,))
+    assert (st, ws) == (0, 0)
+
+
+def test_executor_lifecycle(aclnn, desc):
+    L = aclnn.load_library()
+    i, g, o = desc.t((0, 1, 5, 8), 0), desc.t((0, 3, 3, 2), 0), desc.t((0, 1, 3, 3), 0)
+    st, ws, ex = aclnn.get_workspace_size_grid_sampler2d(i, g, 0, 0, False, o)
+    assert st == 0 and ex
+    # phase 2 on a no-op executor touches no device and consumes the executor
+    assert L.aclnnGridSampler2D(None, 0, ex, None) == 0
+    assert L.aclnnGridSampler2D(None, 0, None, None) == aclnn.ACLNN_ERR_PARAM_NULLPTR
+    assert L.aclDestroyAclOpExecutor(None) == aclnn.ACLNN_ERR_PARAM_NULLPTR
+    # an executor of one operator is refused by the other operator's phase 2 (and is consumed by the call)
+    i2, g2, o2 = desc.t((1, 1, 5, 8), 0), desc.t((1, 3, 3, 2), 0), desc.t((1, 1, 3, 3), 0)
+    st, ws, ex = aclnn.get_workspace_size_grid_sampler2d(i2, g2, 0, 0, False, o2)
+    assert st == 0
+    assert L.aclnnUpsampleBilinear2d(None, 0, ex, None) == aclnn.ACLNN_ERR_PARAM_INVALID
+    # NULL data pointers are only rejected when something has to run
+    st, ws, ex = aclnn.get_workspace_size_grid_sampler2d(i2, g2, 0, 0, False, o2)
+    assert L.aclnnGridSampler2D(None, 0, ex, None) == aclnn.ACLNN_ERR_PARAM_NULLPTR
+    # workspace smaller than requested
+    v = desc.t((1, 1, 5, 8), 0, None, (40, 40, 1, 5), 0, (1, 1, 8, 5))
+    st, ws, ex = aclnn.get_workspace_size_grid_sampler2d(v, g2, 0, 0, False, o2)
+    assert st == 0 and ws > 0
+    assert L.aclnnGridSampler2D(None, 0, ex, None) == aclnn.ACLNN_ERR_PARAM_NULLPTR
+    st, ws, ex = aclnn.get_workspace_size_grid_sampler2d(v, g2, 0, 0, False, o2)
+    buf = ctypes.create_string_buffer(8)
+    assert L.aclnnGridSampler2D(buf, 8, ex, None) == aclnn.ACLNN_ERR_PARAM_INVALID
+
+
+def _up(aclnn, desc, inp=(1, 1, 3, 3), out=(1, 1, 6, 6), size=(6, 6), dt=None, odt=None, fmt=None, ofmt=None, align=False,
+        sh=2.0, sw=2.0):
+    dt = aclnn.ACL_FLOAT if dt is None else dt
+    fmt = aclnn.ACL_FORMAT_NCHW if fmt is None else fmt
+    s = desc.t(inp, dt, fmt)
+    o = desc.t(out, dt if odt is None else odt, fmt if ofmt is None else ofmt)
+    arr = aclnn.create_int_array(list(size)) if size is not None else None
+    st, ws, ex = aclnn.get_workspace_size_upsample_bilinear2d(s, arr, align, sh, sw, o)
+    variant = aclnn.executor_variant(ex) if ex else None
+    if ex:
+        aclnn.destroy_executor(ex)
+    aclnn.destroy_int_array(arr)
+    return st, ws, variant
+
+
+def test_upsample_status_codes(aclnn, desc):
+    INV, INNER = aclnn.ACLNN_ERR_PARAM_INVALID, aclnn.ACLNN_ERR_INNER_NULLPTR
+    # test_001: empty tensors but outputSize {2,2} != out H,W -> the size check comes before the empty check
+    assert _up(aclnn, desc, inp=(1, 1, 0, 0), out=(1, 1, 0, 0), size=(2, 2))[0] == INV
+    # test_002: same size
+    st, ws, variant = _up(aclnn, desc, out=(1, 1, 3, 3), size=(3, 3), sh=1.0, sw=1.0)
+    assert (st, ws, variant) == (0, 0, "copy")
+    # nullptr self / out -> inner nullptr (this operator, unlike the grid sampler)
+    assert _up(aclnn, desc, inp=None)[0] == INNER
+    assert _up(aclnn, desc, out=None)[0] == INNER
+    # dtype mismatch, unsupported dtype
+    assert _up(aclnn, desc, odt=aclnn.ACL_FLOAT16)[0] == INV
+    assert _up(aclnn, desc, dt=aclnn.ACL_INT32)[0] == INV
+    # N/C checks (ncdim001..004)
+    assert _up(aclnn, desc, out=(1, 1, 2, 2), size=(2, 2), dt=aclnn.ACL_FLOAT16, sh=1.0, sw=1.0)[0] == 0
+    assert _up(aclnn, desc, inp=(1, 2, 3, 3), out=(1, 1, 2, 2), size=(2, 2), dt=aclnn.ACL_FLOAT16)[0] == INV
+    assert _up(aclnn, desc, inp=(1, 1, 3, 3), out=(1, 1, 3, 3), size=(2, 2), fmt=aclnn.ACL_FORMAT_NHWC)[0] == INV
+    assert _up(aclnn, desc, inp=(1, 1, 3, 4), out=(1, 1, 2, 3), size=(2, 2), fmt=aclnn.ACL_FORMAT_NHWC)[0] == INV
+    # negative scales
+    assert _up(aclnn, desc, sh=-2.0, sw=-2.0)[0] == INV
+    assert _up(aclnn, desc, sh=1.0, sw=-2.0)[0] == INV
+    # formats
+    assert _up(aclnn, desc, ofmt=aclnn.ACL_FORMAT_NHWC)[0] == INV
+    assert _up(aclnn, desc, fmt=aclnn.ACL_FORMAT_ND)[0] == INV
+    assert _up(aclnn, desc, inp=(1, 3, 3), out=(1, 6, 6))[0] == INV
+    assert _up(aclnn, desc, dt=aclnn.ACL_DOUBLE)[0] == INV  # DOUBLE only with NHWC in the reference
+    # outputSize checks (Ascend910B2 cases 1001-1004)
+    assert _up(aclnn, desc)[0] == 0
+    assert _up(aclnn, desc, size=(0, 0))[0] == INV
+    assert _up(aclnn, desc, size=None)[0] == INV
+    assert _up(aclnn, desc, size=(6, 6, 6))[0] == INV
+    # empty tensors with consistent sizes: success, nothing to run
+    st, ws, variant = _up(aclnn, desc, inp=(0, 1, 3, 3), out=(0, 1, 6, 6))
+    assert (st, ws, variant) == (0, 0, "")
+
+
+def test_upsample_template_selection(aclnn, desc):
+    """kernel-template choice for the shapes of the reference tiling UT (keys 40000 copy, 40002 broadcast, 3000x
+    bilinear): image/resize_bilinear_v2/tests/ut/op_host/arch35/test_resize_bilinear_v2_tiling.cpp"""
+    f16, f32 = aclnn.ACL_FLOAT16, aclnn.ACL_FLOAT
+    # case12/13: 1x1 -> 11x21 is the broadcast template for both align_corners and half-pixel
+    assert _up(aclnn, desc, inp=(1, 1, 1, 1), out=(1, 1, 11, 21), size=(11, 21), align=True, sh=0, sw=0)[2] == "broadcast"
+    assert _up(aclnn, desc, inp=(1, 1, 1, 1), out=(1, 1, 11, 21), size=(11, 21), dt=f16, sh=0, sw=0)[2] == "broadcast"
+    # below 128 output bytes per plane the half-pixel case stays on the bilinear template
+    v = _up(aclnn, desc, inp=(1, 1, 1, 1), out=(1, 1, 4, 4), size=(4, 4), dt=f16, sh=0, sw=0)[2]
+    assert v.startswith("nchw")
+    assert _up(aclnn, desc, inp=(1, 1, 1, 1), out=(1, 1, 4, 4), size=(4, 4), dt=f16, align=True, sh=0, sw=0)[2] == "broadcast"
+    # 1x1 destination with align_corners -> first pixel; case16: equal sizes -> copy
+    assert _up(aclnn, desc, inp=(1, 1, 5, 5), out=(1, 1, 1, 1), size=(1, 1), align=True, sh=0, sw=0)[2] == "first_pixel"
+    assert _up(aclnn, desc, inp=(3, 5, 11, 21), out=(3, 5, 11, 21), size=(11, 21), dt=aclnn.ACL_BF16, sh=0, sw=0)[2] == "copy"
+    # case01/02/06: ordinary NCHW bilinear; NHWC has its own kernel
+    assert _up(aclnn, desc, inp=(2, 256, 12, 12), out=(2, 256, 18, 18), size=(18, 18), dt=f32, sh=1.5, sw=1.5)[2].startswith("nchw")
+    assert _up(aclnn, desc, inp=(2, 128, 128, 256), out=(2, 192, 192, 256), size=(192, 192), dt=f32,
+               fmt=aclnn.ACL_FORMAT_NHWC, align=True)[2] == "nhwc_generic"

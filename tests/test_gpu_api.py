@@ -1,0 +1,156 @@
+"""GPU tests of the boundary behaviour: strided views, offsets, NHWC, fallback variants, full-size configurations."""
+import ctypes
+
+import numpy as np
+import pytest
+
+import inputs as I
+
+pytestmark = pytest.mark.gpu
+
+
+def _torch():
+    import torch
+    return torch
+
+
+def test_noncontiguous_views_are_honoured(oracle, device, aclnn):
+    torch = _torch()
+    rng = np.random.default_rng(21)
+    x32 = rng.standard_normal((2, 3, 9, 12)).astype(np.float32)
+    g32 = rng.uniform(-1.2, 1.2, (2, 7, 5, 2)).astype(np.float32)
+    ref = oracle.grid_sampler2d(x32, g32, 0, 0, False)
+    # input as a transposed view of an (N,C,W,H) buffer, grid as a slice of a larger buffer, out as a strided slice
+    xt = torch.from_numpy(np.ascontiguousarray(x32.transpose(0, 1, 3, 2))).to(device).transpose(2, 3)
+    assert not xt.is_contiguous()
+    gbig = torch.zeros((2, 7, 10, 2), device=device)
+    gbig[:, :, ::2, :] = torch.from_numpy(g32).to(device)
+    gv = gbig[:, :, ::2, :]
+    obig = torch.full((2, 3, 7, 9), -7.0, device=device)
+    ov = obig[:, :, :, 2:7]
+    out = aclnn.grid_sampler2d(xt, gv, 0, 0, False, out=ov)
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy(), ref)
+    rest = obig.cpu().numpy()
+    assert (rest[..., :2] == -7.0).all() and (rest[..., 7:] == -7.0).all()  # nothing outside the view is touched
+    # upsample on a view with a storage offset
+    u32 = rng.standard_normal((2, 2, 6, 8)).astype(np.float32)
+    ubig = torch.zeros((3, 2, 6, 8), device=device)
+    ubig[1:] = torch.from_numpy(u32).to(device)
+    y = aclnn.upsample_bilinear2d(ubig[1:], (12, 16), False, 2.0, 2.0)
+    torch.cuda.synchronize()
+    assert np.array_equal(y.cpu().numpy(), oracle.upsample_bilinear2d(u32, (12, 16), False, 2.0, 2.0))
+
+
+@pytest.mark.parametrize("dtype", I.DTYPES)
+@pytest.mark.parametrize("align", [False, True])
+def test_upsample_nhwc(oracle, device, aclnn, dtype, align):
+    torch = _torch()
+    rng = np.random.default_rng(22)
+    for (N, C, H, W), size in [((2, 5, 7, 9), (14, 18)), ((1, 64, 1, 1), (6, 6)), ((1, 3, 8, 8), (8, 8)),
+                               ((2, 3, 6, 6), (1, 1)), ((1, 130, 3, 3), (5, 7))]:
+        x32 = rng.standard_normal((N, C, H, W)).astype(np.float32)
+        x = I.cast_np(x32, dtype)
+        ref = oracle.upsample_bilinear2d(x, size, align, dtype=I.oracle_code(dtype))
+        xh = np.ascontiguousarray(x.transpose(0, 2, 3, 1))
+        y = aclnn.upsample_bilinear2d(I.to_torch(xh, dtype, device), size, align, channels_last=True)
+        torch.cuda.synchronize()
+        got = I.from_torch(y, dtype).transpose(0, 3, 1, 2)
+        a, b = I.as_f32(got, dtype), I.as_f32(ref, dtype)
+        assert np.array_equal(a, b), "nhwc %s %s align=%s" % (dtype, (N, C, H, W), align)
+
+
+@pytest.mark.parametrize("dtype", I.DTYPES)
+def test_grid_sampler_variants_agree(oracle, device, aclnn, dtype):
+    """every kernel variant (LDS ring classes, direct fallback for odd or oversized planes) matches the oracle"""
+    torch = _torch()
+    rng = np.random.default_rng(23)
+    L = aclnn.load_library()
+    seen = set()
+    shapes = [(2, 5, 13, 17, 19, 23),    # odd byte count for 16-bit types -> direct
+              (2, 9, 16, 16, 40, 40),    # small planes
+              (1, 6, 64, 64, 64, 64),    # 8 KiB planes (16-bit)
+              (1, 5, 128, 128, 50, 70),  # 32 KiB planes (16-bit)
+              (1, 3, 160, 200, 33, 65),  # 64-128 KiB planes
+              (1, 2, 300, 320, 31, 33)]  # beyond LDS -> direct
+    for (N, C, H, W, Ho, Wo) in shapes:
+        x = I.cast_np(rng.standard_normal((N, C, H, W)).astype(np.float32), dtype)
+        g = I.cast_np(rng.uniform(-1.2, 1.2, (N, Ho, Wo, 2)).astype(np.float32), dtype)
+        xt, gt = I.to_torch(x, dtype, device), I.to_torch(g, dtype, device)
+        out = torch.empty((N, C, Ho, Wo), dtype=xt.dtype, device=device)
+        hs = [aclnn.tensor_handle(t) for t in (xt, gt, out)]
+        for interp in (0, 1):
+            for pad in (0, 2):
+                st, ws, ex = aclnn.get_workspace_size_grid_sampler2d(hs[0], hs[1], interp, pad, False, hs[2])
+                assert st == 0
+                seen.add(aclnn.executor_variant(ex))
+                assert L.aclnnGridSampler2D(None, 0, ex, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)) == 0
+                torch.cuda.synchronize()
+                ref = oracle.grid_sampler2d(x, g, interp, pad, False, dtype=I.oracle_code(dtype))
+                assert np.array_equal(I.from_torch(out, dtype).view(np.uint8), ref.view(np.uint8)), (
+                    dtype, (N, C, H, W, Ho, Wo), interp, pad)
+        for h in hs:
+            aclnn.destroy_tensor(h)
+    assert "direct" in seen and len(seen) >= 4, seen
+
+
+def test_full_size_grid_sampler_fp16_n16_c256(oracle, device, aclnn):
+    """the headline configuration at full size, all six mode/padding variants, against the oracle"""
+    torch = _torch()
+    rng = np.random.default_rng(31)
+    x = I.cast_np(rng.standard_normal((16, 256, 64, 64), dtype=np.float32), "fp16")
+    g32 = I.affine_grid(rng, 16, 64, 64)
+    outside = (np.abs(g32) > 1).any(-1).mean()
+    assert 0.01 <= outside <= 0.15, outside
+    g = I.cast_np(g32, "fp16")
+    xt, gt = I.to_torch(x, "fp16", device), I.to_torch(g, "fp16", device)
+    for interp in (0, 1):
+        for pad in (0, 1, 2):
+            y = aclnn.grid_sampler2d(xt, gt, interp, pad, False)
+            torch.cuda.synchronize()
+            ref = oracle.grid_sampler2d(x, g, interp, pad, False)
+            assert np.array_equal(I.from_torch(y, "fp16").view(np.uint16), ref.view(np.uint16)), (interp, pad)
+
+
+def test_full_size_random_gather_bf16(oracle, device, aclnn):
+    torch = _torch()
+    rng = np.random.default_rng(32)
+    x = I.cast_np(rng.standard_normal((8, 128, 128, 128), dtype=np.float32), "bf16")
+    g = I.cast_np(rng.uniform(-1.1, 1.1, (8, 256, 256, 2)).astype(np.float32), "bf16")
+    y = aclnn.grid_sampler2d(I.to_torch(x, "bf16", device), I.to_torch(g, "bf16", device), 0, 1, True)
+    torch.cuda.synchronize()
+    ref = oracle.grid_sampler2d(x, g, 0, 1, True, dtype=oracle.BF16)
+    assert np.array_equal(I.from_torch(y, "bf16"), ref)
+
+
+def test_full_size_4k_upscale_properties(oracle, device, aclnn):
+    """(4,16,1080,1920) -> (2160,3840) fp16 align_corners: oracle on a few planes, invariants on everything"""
+    torch = _torch()
+    rng = np.random.default_rng(33)
+    x = torch.from_numpy(rng.random((4, 16, 1080, 1920), dtype=np.float32)).to(torch.float16)
+    x[1, 3] = 0.625  # a constant plane stays constant
+    xt = x.to(device)
+    y = aclnn.upsample_bilinear2d(xt, (2160, 3840), True)
+    torch.cuda.synchronize()
+    yc = y.cpu()
+    assert (yc[1, 3] == 0.625).all()
+    # align_corners keeps the four corner samples of every plane
+    for (a, b) in [((0, 0), (0, 0)), ((0, 3839), (0, 1919)), ((2159, 0), (1079, 0)), ((2159, 3839), (1079, 1919))]:
+        assert torch.equal(yc[:, :, a[0], a[1]], x[:, :, b[0], b[1]])
+    # convexity: every output lies within the range of its plane
+    assert (yc.amax((2, 3)) <= x.amax((2, 3))).all() and (yc.amin((2, 3)) >= x.amin((2, 3))).all()
+    planes = [(0, 0), (2, 7), (3, 15)]
+    xs = np.stack([x[n, c].numpy() for n, c in planes])[:, None]
+    ref = oracle.upsample_bilinear2d(xs, (2160, 3840), True)
+    got = np.stack([yc[n, c].numpy() for n, c in planes])[:, None]
+    assert np.array_equal(got.view(np.uint16), ref.view(np.uint16))
+
+
+def test_full_size_upsample_fp32_56_to_112(oracle, device, aclnn):
+    torch = _torch()
+    rng = np.random.default_rng(34)
+    x = rng.standard_normal((8, 64, 56, 56), dtype=np.float32)
+    y = aclnn.upsample_bilinear2d(torch.from_numpy(x).to(device), (112, 112), False, 2.0, 2.0)
+    torch.cuda.synchronize()
+    ref = oracle.upsample_bilinear2d(x, (112, 112), False, 2.0, 2.0)
+    assert np.array_equal(y.cpu().numpy().view(np.uint32), ref.view(np.uint32))

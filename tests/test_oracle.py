@@ -1,0 +1,330 @@
+"""Pins the CPU oracle (oracle/cv_oracle.c) independently of its own text.
+
+Sources of truth used here: known answers for the reference's own example inputs, closed forms and invariants of
+the coordinate pipeline, numpy/torch library conversions, the committed PyTorch fixtures under tests/golden/, a
+live PyTorch CPU comparison, and the scale bit patterns held by the reference's tiling unit test.
+"""
+import os
+
+import numpy as np
+import pytest
+
+import inputs as I
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+MODES = ["bilinear", "nearest"]
+PADS = ["zeros", "border", "reflection"]
+
+
+# ------------------------------------------------------------------------------------------ conversions
+def test_half_roundtrip_exhaustive(oracle):
+    L = oracle.lib()
+    bits = np.arange(65536, dtype=np.uint16)
+    ref = bits.view(np.float16).astype(np.float32)
+    for b in range(0, 65536, 7):  # every 7th pattern through ctypes; the vectorised check below covers all
+        f = L.oracle_half_to_float(int(b))
+        r = ref[b]
+        assert (np.isnan(f) and np.isnan(r)) or f == r
+        if not np.isnan(r):
+            assert L.oracle_float_to_half(float(r)) == b or (r == 0 and L.oracle_float_to_half(float(r)) in (0, 0x8000))
+
+
+def test_float_to_half_matches_numpy(oracle):
+    L = oracle.lib()
+    rng = np.random.default_rng(3)
+    vals = np.concatenate([
+        rng.standard_normal(4000).astype(np.float32) * np.float32(10.0) ** rng.integers(-8, 5, 4000),
+        np.array([0.0, -0.0, 65504.0, 65519.9, 65520.0, 1e-8, 5.9604645e-8, 2.9802322e-8, 2.98023224e-8 * 1.0000001,
+                  6.1035156e-5, 6.0975552e-5, 1.0009766, 1.00048828125, 1.00146484375, np.inf, -np.inf],
+                 dtype=np.float32)]).astype(np.float32)
+    with np.errstate(over="ignore"):
+        want = vals.astype(np.float16).view(np.uint16)
+    got = np.array([L.oracle_float_to_half(float(v)) for v in vals], dtype=np.uint16)
+    assert np.array_equal(got, want)
+
+
+def test_bf16_matches_torch(oracle):
+    import torch
+    L = oracle.lib()
+    rng = np.random.default_rng(4)
+    vals = (rng.standard_normal(4000).astype(np.float32) * np.float32(10.0) ** rng.integers(-20, 20, 4000))
+    vals = np.concatenate([vals, np.array([0.0, -0.0, 1.00390625, 1.01171875, 3.3895314e38, np.inf],
+                                          np.float32)]).astype(np.float32)
+    want = torch.from_numpy(vals).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    got = np.array([L.oracle_float_to_bf16(float(v)) for v in vals], dtype=np.uint16)
+    assert np.array_equal(got, want)
+    assert np.array_equal(oracle.f32_to_bf16_bits(vals), want)
+    back = np.array([L.oracle_bf16_to_float(int(b)) for b in want], dtype=np.float32)
+    assert np.array_equal(back, oracle.bf16_bits_to_f32(want))
+
+
+# ------------------------------------------------------------------------------------------ coordinate pipeline
+def test_unnormalize_closed_forms(oracle):
+    L = oracle.lib()
+    for size in (1, 2, 5, 8, 64, 1920):
+        assert L.oracle_unnormalize(-1.0, size, 0) == -0.5
+        assert L.oracle_unnormalize(1.0, size, 0) == size - 0.5
+        assert L.oracle_unnormalize(-1.0, size, 1) == 0.0
+        assert L.oracle_unnormalize(1.0, size, 1) == float(size - 1)
+        assert L.oracle_unnormalize(0.0, size, 0) == size / 2 - 0.5
+    # single rounding of scaling*(g+1) - 0.5: the fused result stays below 8, mul-then-sub would round up to 8.0
+    assert L.oracle_unnormalize(np.float32(0.6999999), 10, 0) == np.float32(7.9999995)
+
+
+def test_clip_and_reflect_invariants(oracle):
+    L = oracle.lib()
+    rng = np.random.default_rng(5)
+    assert L.oracle_clip_coordinates(float("nan"), 7) == 0.0
+    assert L.oracle_clip_coordinates(-3.0, 7) == 0.0 and L.oracle_clip_coordinates(99.0, 7) == 6.0
+    assert L.oracle_reflect_coordinates(3.0, 0.0, 0.0) == 0.0  # size 1 with align_corners: span is zero
+    for size in (2, 5, 8, 64):
+        for align in (0, 1):
+            low, span2 = (0.0, 2.0 * (size - 1)) if align else (-0.5, 2.0 * size)
+            for c in rng.uniform(-5 * size, 5 * size, 300).astype(np.float32):
+                r = L.oracle_reflect_coordinates(float(c), low, span2)
+                assert low - 1e-4 <= r <= low + span2 / 2 + 1e-4
+                mirrored = L.oracle_reflect_coordinates(float(np.float32(2 * low) - c), low, span2)
+                assert abs(mirrored - r) <= 1e-3 * size  # even about `low`
+                shifted = L.oracle_reflect_coordinates(float(c + np.float32(span2)), low, span2)
+                assert abs(shifted - r) <= 1e-3 * size  # period 2*span
+                s = L.oracle_compute_source_index(float(c) / size, size, 2, align)
+                assert 0.0 <= s <= size - 1
+            for c in rng.uniform(-3, 3, 100).astype(np.float32):
+                s = L.oracle_compute_source_index(float(c), size, 1, align)
+                assert 0.0 <= s <= size - 1
+    # catastrophic-cancellation case spelled out by the reference (grid_sampler2_d_simt.h:152-158): 3e10 mod 12
+    assert L.oracle_reflect_coordinates(3e10, 0.0, 12.0) == 0.0
+
+
+def test_safe_downgrade(oracle):
+    L = oracle.lib()
+    assert L.oracle_safe_downgrade(5.25) == 5.25
+    for v in (float("nan"), float("inf"), float("-inf"), 3e9, -3e9, 2147483904.0):
+        assert L.oracle_safe_downgrade(v) == -100.0
+    assert L.oracle_safe_downgrade(-2147483648.0) == -2147483648.0
+
+
+def test_banker_round_matches_rint(oracle):
+    L = oracle.lib()
+    rng = np.random.default_rng(6)
+    ties = np.arange(-20, 20, dtype=np.float32) + np.float32(0.5)
+    near = np.concatenate([np.nextafter(ties, np.float32(100)), np.nextafter(ties, np.float32(-100))])
+    vals = np.concatenate([ties, near, rng.uniform(-1000, 1000, 3000).astype(np.float32), [0.0, -0.0, -100.0, 7.0]])
+    got = np.array([L.oracle_banker_round(float(v)) for v in vals])
+    assert np.array_equal(got, np.rint(vals).astype(np.int64))
+
+
+# ------------------------------------------------------------------------------------------ known answers
+def _example_inputs():
+    # image/grid_sample/examples/test_aclnn_grid_sample2_d.cpp:96-98: x = 1..40 as (1,1,5,8), 3x3 lattice grid
+    x = np.arange(1, 41, dtype=np.float32).reshape(1, 1, 5, 8)
+    g = np.array([[-1, -1], [0, -1], [1, -1], [-1, 0], [0, 0], [1, 0], [-1, 1], [0, 1], [1, 1]],
+                 dtype=np.float32).reshape(1, 3, 3, 2)
+    return x, g
+
+
+def test_grid_sampler_known_answers(oracle):
+    x, g = _example_inputs()
+    inner = [1, 4.5, 8, 17, 20.5, 24, 33, 36.5, 40]
+    assert oracle.grid_sampler2d(x, g, 0, 0, False).ravel().tolist() == [0.25, 2.25, 2.0, 8.5, 20.5, 12.0, 8.25, 18.25,
+                                                                           10.0]
+    for pad, align in [(0, True), (1, False), (1, True), (2, False), (2, True)]:
+        assert oracle.grid_sampler2d(x, g, 0, pad, align).ravel().tolist() == inner
+    assert oracle.grid_sampler2d(x, g, 1, 0, False).ravel().tolist() == [1, 5, 0, 17, 21, 0, 33, 37, 0]
+    near = [1, 5, 8, 17, 21, 24, 33, 37, 40]
+    for pad, align in [(0, True), (1, False), (1, True), (2, False), (2, True)]:
+        assert oracle.grid_sampler2d(x, g, 1, pad, align).ravel().tolist() == near
+    # half-even tie: W=8, gx=+1, align_corners=False -> ix = 7.5 -> 8 -> outside -> 0 under zeros padding
+    t = oracle.grid_sampler2d_taps(np.array([[[[1.0, 0.0]]]], np.float32), 5, 8, 1, 0, False)
+    assert t["ix0"][0, 0, 0] == 8 and t["iy0"][0, 0, 0] == 2
+
+
+def test_grid_sampler_identity(oracle):
+    # image/grid_sampler2_d/examples/arch35/test_geir_grid_sampler2_d.cpp:84-90,158: sampling at the pixel
+    # centres returns the image (tolerance 1e-4 there); with align_corners the lattice is exact
+    rng = np.random.default_rng(8)
+    for (H, W) in [(2, 2), (5, 8), (16, 16)]:
+        x = rng.standard_normal((2, 3, H, W)).astype(np.float32)
+        xs = np.linspace(-1, 1, W, dtype=np.float32) if W > 1 else np.zeros(1, np.float32)
+        ys = np.linspace(-1, 1, H, dtype=np.float32) if H > 1 else np.zeros(1, np.float32)
+        gx, gy = np.meshgrid(xs, ys)
+        g = np.broadcast_to(np.stack([gx, gy], -1)[None], (2, H, W, 2)).astype(np.float32)
+        for interp in (0, 1):
+            for pad in (0, 1, 2):
+                y = oracle.grid_sampler2d(x, g, interp, pad, True)
+                assert np.abs(y - x).max() <= 1e-4
+        # align_corners=False pixel centres
+        xs = ((2 * np.arange(W) + 1) / W - 1).astype(np.float32)
+        ys = ((2 * np.arange(H) + 1) / H - 1).astype(np.float32)
+        gx, gy = np.meshgrid(xs, ys)
+        g = np.broadcast_to(np.stack([gx, gy], -1)[None], (2, H, W, 2)).astype(np.float32)
+        assert np.abs(oracle.grid_sampler2d(x, g, 0, 0, False) - x).max() <= 1e-4
+
+
+def test_grid_sampler_weights_sum_to_one_and_constant_image(oracle):
+    rng = np.random.default_rng(9)
+    g = rng.uniform(-0.95, 0.95, (1, 20, 20, 2)).astype(np.float32)
+    taps = oracle.grid_sampler2d_taps(g, 9, 11, 0, 1, True)
+    assert np.abs(taps["w"].sum(-1) - 1.0).max() <= 1e-6
+    x = np.full((1, 2, 9, 11), 3.25, np.float32)
+    assert np.abs(oracle.grid_sampler2d(x, g, 0, 1, True) - 3.25).max() <= 1e-6
+
+
+def test_grid_sampler_nonfinite_grid(oracle):
+    # grid_sampler2_d_simt.h:485-487: bilinear writes NaN to every channel; :497-498 nearest maps to an
+    # always-outside coordinate (zeros padding -> 0); border/reflection clip NaN to 0 first
+    x = np.arange(1, 41, dtype=np.float32).reshape(1, 2, 4, 5)
+    g = np.array([[[[np.nan, 0.0], [np.inf, 0.0], [0.0, -np.inf], [1e10, 0.0]]]], np.float32)
+    y = oracle.grid_sampler2d(x, g, 0, 0, False)
+    assert np.isnan(y[0, :, 0, :3]).all() and (y[0, :, 0, 3] == 0).all()
+    y = oracle.grid_sampler2d(x, g, 1, 0, False)
+    assert (y == 0).all()
+    y = oracle.grid_sampler2d(x, g, 0, 1, False)
+    assert np.isfinite(y).all()
+
+
+# ------------------------------------------------------------------------------------------ fixtures
+def test_grid_sampler_against_committed_fixtures(oracle):
+    z = np.load(os.path.join(GOLD, "grid_sampler2d.npz"))
+    for prefix, count in (("gs", 4), ("sp", 3)):
+        for si in range(count):
+            x, g = z["%s%d_x" % (prefix, si)], z["%s%d_grid" % (prefix, si)]
+            for m in range(2):
+                for p in range(3):
+                    for a in (0, 1):
+                        want = z["%s%d_y_m%d_p%d_a%d" % (prefix, si, m, p, a)]
+                        got = oracle.grid_sampler2d(x, g, m, p, bool(a))
+                        assert np.array_equal(np.isnan(got), np.isnan(want)), (prefix, si, m, p, a)
+                        w, q = np.nan_to_num(want), np.nan_to_num(got)
+                        if m == 1:
+                            assert np.array_equal(q, w), (prefix, si, m, p, a)
+                        else:
+                            assert np.abs(q - w).max() <= 2e-6 * max(1.0, np.abs(w).max()), (prefix, si, m, p, a)
+    # the tap below 8.0 that only the fused unnormalize selects
+    got = oracle.grid_sampler2d(z["fma_x"], z["fma_grid"], 0, 0, False)
+    assert got.ravel()[0] == z["fma_y"].ravel()[0] == np.float32(999999.5)
+    # 16-bit: fp32 compute, one rounding at the end
+    for name, code in (("f16", oracle.F16), ("bf16", oracle.BF16)):
+        x, g = z["h_%s_x" % name], z["h_%s_grid" % name]
+        if name == "f16":
+            x, g = x.view(np.float16), g.view(np.float16)
+        for m in range(2):
+            for p in range(3):
+                for a in (0, 1):
+                    want = z["h_%s_y_m%d_p%d_a%d" % (name, m, p, a)]
+                    got = oracle.grid_sampler2d(x, g, m, p, bool(a), dtype=code).view(np.uint16)
+                    if m == 1:
+                        assert np.array_equal(got, want)
+                    else:
+                        # same fp32 value up to summation order: at most one unit in the last 16-bit place
+                        assert np.abs(got.astype(np.int32) - want.astype(np.int32)).max() <= 1
+
+
+def test_upsample_against_committed_fixtures(oracle):
+    z = np.load(os.path.join(GOLD, "upsample_bilinear2d.npz"))
+    for ci in range(10):
+        x, size = z["up%d_x" % ci], tuple(int(v) for v in z["up%d_size" % ci])
+        for a in (0, 1):
+            want = z["up%d_y_a%d" % (ci, a)]
+            got = oracle.upsample_bilinear2d(x, size, bool(a))
+            assert np.abs(got - want).max() <= 1e-5 * max(1.0, np.abs(want).max()), (ci, a)
+    for si in range(3):
+        sh, sw = z["ups_scale_%d" % si]
+        want = z["ups_y_%d" % si]
+        got = oracle.upsample_bilinear2d(z["ups_x"], want.shape[2:], False, sh, sw)
+        assert np.abs(got - want).max() <= 1e-5
+
+
+def test_upsample_known_answers(oracle):
+    # image/upsample_bilinear2d/examples/test_aclnn_upsample_bilinear2d.cpp:83-94: x = 0..7 as (1,1,4,2) -> (8,4)
+    x = np.arange(8, dtype=np.float32).reshape(1, 1, 4, 2)
+    y = oracle.upsample_bilinear2d(x, (8, 4), True)
+    assert np.allclose(y[0, 0, 0], [0, 1 / 3, 2 / 3, 1], atol=1e-6)
+    assert np.allclose(y[0, 0, -1], [6, 6 + 1 / 3, 6 + 2 / 3, 7], atol=1e-6)
+    assert np.allclose(y[0, 0, :, 0], np.arange(8) * 6 / 7, atol=1e-6)
+    y = oracle.upsample_bilinear2d(x, (8, 4), False, 2.0, 2.0)
+    assert y[0, 0, 0].tolist() == [0, 0.25, 0.75, 1] and y[0, 0, 1].tolist() == [0.5, 0.75, 1.25, 1.5]
+
+
+def test_upsample_invariants(oracle):
+    rng = np.random.default_rng(10)
+    x = rng.standard_normal((2, 2, 6, 7)).astype(np.float32)
+    assert np.array_equal(oracle.upsample_bilinear2d(x, (6, 7), False), x)  # same size is a copy
+    c = np.full((1, 1, 5, 5), -2.5, np.float32)
+    for align in (False, True):
+        assert np.abs(oracle.upsample_bilinear2d(c, (13, 9), align) + 2.5).max() <= 1e-6
+    ramp = np.broadcast_to(np.arange(9, dtype=np.float32), (1, 1, 4, 9)).copy()
+    y = oracle.upsample_bilinear2d(ramp, (4, 25), True)
+    assert np.abs(y[0, 0, 0] - np.linspace(0, 8, 25)).max() <= 1e-5  # align_corners reproduces linear ramps
+    one = rng.standard_normal((2, 3, 1, 1)).astype(np.float32)
+    for align in (False, True):
+        y = oracle.upsample_bilinear2d(one, (16, 16), align)
+        assert np.array_equal(y, np.broadcast_to(one, y.shape))  # 1x1 source broadcasts exactly
+    i0, i1, lam = oracle.upsample_axis_taps(5, 13, False)
+    assert (i0 >= 0).all() and (i1 <= 4).all() and (i1 - i0 >= 0).all() and (i1 - i0 <= 1).all()
+    assert (lam >= 0).all() and (lam < 1).all()
+
+
+# scale bit patterns held by image/resize_bilinear_v2/tests/ut/op_host/arch35/test_resize_bilinear_v2_tiling.cpp
+# (the number before the last one in each expectTilingData string packs scaleW in the low and scaleH in the
+# high 32 bits): (Hs, Ws, Hd, Wd, align_corners, scale_h, scale_w, packed)
+TILING_SCALES = [
+    (12, 12, 18, 18, False, 1.5, 1.5, 4551638025887197867),
+    (128, 128, 192, 192, True, 1.5, 1.5, 4551512269244741707),
+    (128, 128, 64, 64, False, 0.5, 0.5, 4611686019501129728),
+    (14, 16, 5, 8, False, 3.0, 3.0, 4515609228859845291),
+    (10, 10, 64, 1024, False, 2.0, 2.0, 4539628425446424576),
+    (36, 15, 12, 5, False, 0.0, 0.0, 4629700418014806016),
+    (36, 15, 12, 5, False, 0.2, 0.2, 4656722015785320448),
+    (22, 79, 13, 43, False, 0.31269457412229545, 0.27077088627767687, 4633267427011747001),
+    (1, 1, 11, 21, True, 0.0, 0.0, 0),
+    (1, 1, 11, 21, False, 0.0, 0.0, 4447918761839889457),
+    (11, 21, 11, 21, False, 0.0, 0.0, 4575657222473777152),
+]
+
+
+@pytest.mark.parametrize("case", TILING_SCALES)
+def test_resize_scale_bit_patterns(oracle, case):
+    Hs, Ws, Hd, Wd, align, sh, sw, packed = case
+    L = oracle.lib()
+    h = np.float32(L.oracle_resize_scale(Hs, Hd, int(align), np.float32(sh)))
+    w = np.float32(L.oracle_resize_scale(Ws, Wd, int(align), np.float32(sw)))
+    got = (int(h.view(np.uint32)) << 32) | int(w.view(np.uint32))
+    assert got == packed
+
+
+# ------------------------------------------------------------------------------------------ live PyTorch CPU
+def test_live_torch_grid_sample(oracle):
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(12)
+    for trial in range(12):
+        N, C = 2, 3
+        H, W = rng.integers(1, 40, 2)
+        Ho, Wo = rng.integers(1, 50, 2)
+        x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+        g = rng.uniform(-1.6, 1.6, (N, Ho, Wo, 2)).astype(np.float32)
+        for m in range(2):
+            for p in range(3):
+                for a in (False, True):
+                    got = oracle.grid_sampler2d(x, g, m, p, a)
+                    want = F.grid_sample(torch.from_numpy(x), torch.from_numpy(g), mode=MODES[m], padding_mode=PADS[p],
+                                         align_corners=a).numpy()
+                    if m == 1:
+                        assert np.array_equal(got, want)
+                    else:
+                        assert np.abs(got - want).max() <= 2e-6 * max(1.0, np.abs(want).max())
+
+
+def test_live_torch_interpolate(oracle):
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(13)
+    for trial in range(20):
+        H, W = rng.integers(1, 40, 2)
+        Ho, Wo = rng.integers(1, 90, 2)
+        x = rng.standard_normal((2, 2, H, W)).astype(np.float32)
+        for a in (False, True):
+            got = oracle.upsample_bilinear2d(x, (int(Ho), int(Wo)), a)
+            want = F.interpolate(torch.from_numpy(x), size=(int(Ho), int(Wo)), mode="bilinear", align_corners=a).numpy()
+            assert np.abs(got - want).max() <= 2e-5
