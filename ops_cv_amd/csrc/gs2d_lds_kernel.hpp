@@ -70,15 +70,18 @@ __device__ __forceinline__ void load_taps(const char* plane, const uint32_t* tof
 
 // One output sample from its tap values: grid_sampler2_d_simt.h:321-338 (0 + nw + ne + sw + se, products and
 // sums rounded separately) for bilinear, :341-360 (the value passes through fp32) for nearest.
+// fma(v, w, +0) is "0 + v*w" with one rounding of the exact product, i.e. the reference's first step bit for
+// bit; fma(v, w, -0) is "v*w" bit for bit (also for zero products of either sign).  Writing the products as
+// fmas lets the 16-bit -> fp32 conversion ride on the multiply (mixed-precision fma) for fp16; `neg_zero` is
+// -0.0f handed in at run time so that the compiler cannot fold the fma back into a multiply.
 template <typename T, int INTERP>
-__device__ __forceinline__ float blend(const T* raw, const float* tw)
+__device__ __forceinline__ float blend(const T* raw, const float* tw, float neg_zero)
 {
     if (INTERP == 0) {
-        float out = 0.0f;
-        out += ElemIO<T>::load(&raw[0]) * tw[0];
-        out += ElemIO<T>::load(&raw[1]) * tw[1];
-        out += ElemIO<T>::load(&raw[2]) * tw[2];
-        out += ElemIO<T>::load(&raw[3]) * tw[3];
+        float out = __builtin_fmaf(ElemIO<T>::load(&raw[0]), tw[0], 0.0f);
+        out += __builtin_fmaf(ElemIO<T>::load(&raw[1]), tw[1], neg_zero);
+        out += __builtin_fmaf(ElemIO<T>::load(&raw[2]), tw[2], neg_zero);
+        out += __builtin_fmaf(ElemIO<T>::load(&raw[3]), tw[3], neg_zero);
         return out;
     }
     return ElemIO<T>::load(&raw[0]);
@@ -105,29 +108,16 @@ __device__ __forceinline__ void wait_vmcnt_imm()
     __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4) | (0xF << 8));
 }
 
-// Waits until at most  per_copy_stage * mine + per_sampled_stage * sampled  vector-memory operations of this
-// wavefront are outstanding; `mine` (copy instructions per plane of this wavefront, 0..4) and `sampled`
-// (0..MAX_SAMPLED) are wave-uniform run-time values, the products are turned into immediates here.
-// Anything outside the table waits for everything.
-template <int PER_COPY, int PER_SAMPLED, int MAX_SAMPLED>
-__device__ __forceinline__ void wait_vmcnt_table(uint32_t mine, uint32_t sampled)
+// Run-time `n` (wave-uniform, 0..63) -> the matching immediate form; larger values cannot be expressed and wait
+// for everything.
+__device__ __forceinline__ void wait_vmcnt(uint32_t n)
 {
-    static_assert(MAX_SAMPLED <= 3, "table covers up to three sampled stages");
-    constexpr int kMaxMine = 4;
-    if (mine > (uint32_t)kMaxMine || sampled > (uint32_t)MAX_SAMPLED ||
-        PER_COPY * kMaxMine + PER_SAMPLED * MAX_SAMPLED > 63) {
-        wait_vmcnt_imm<0>();
-        return;
-    }
-    const uint32_t key = __builtin_amdgcn_readfirstlane(mine * 4u + sampled);
-    switch (key) {
-#define OPSCV_W(M, S)                                                             \
-    case (M) * 4 + (S):                                                           \
-        wait_vmcnt_imm<(PER_COPY * (M) + PER_SAMPLED * (S)) <= 63 ? (PER_COPY * (M) + PER_SAMPLED * (S)) : 0>(); \
-        break;
-#define OPSCV_WM(M) OPSCV_W(M, 0) OPSCV_W(M, 1) OPSCV_W(M, 2) OPSCV_W(M, 3)
-        OPSCV_WM(0) OPSCV_WM(1) OPSCV_WM(2) OPSCV_WM(3) OPSCV_WM(4)
-#undef OPSCV_WM
+    switch (__builtin_amdgcn_readfirstlane(n)) {
+#define OPSCV_W(N) \
+    case N: wait_vmcnt_imm<N>(); break;
+#define OPSCV_W8(B) OPSCV_W(B) OPSCV_W(B + 1) OPSCV_W(B + 2) OPSCV_W(B + 3) OPSCV_W(B + 4) OPSCV_W(B + 5) OPSCV_W(B + 6) OPSCV_W(B + 7)
+        OPSCV_W8(0) OPSCV_W8(8) OPSCV_W8(16) OPSCV_W8(24) OPSCV_W8(32) OPSCV_W8(40) OPSCV_W8(48) OPSCV_W8(56)
+#undef OPSCV_W8
 #undef OPSCV_W
         default: wait_vmcnt_imm<0>(); break;
     }
@@ -147,21 +137,21 @@ __device__ __forceinline__ void lds_barrier()
 // Starts the asynchronous copy of `nch` consecutive input planes (plane_bytes each, contiguous in global memory
 // from `src`) to LDS at `dst` with PITCH bytes between planes.  G = bytes per lane (16 or 4): the largest
 // granule that divides the plane size and the source alignment.  Each wavefront instruction moves 64*G
-// contiguous bytes; lanes past the end of a plane are masked off.  Wavefront w takes chunks w, w+NWAVES, ...
-// of every plane, so it issues the same number of instructions for every full stage.
-template <int G, int THREADS, int CGS, int PITCH>
-__device__ __forceinline__ void issue_stage_copy(const char* src, char* dst, uint32_t plane_bytes, int nch)
+// contiguous bytes; lanes past the end of a plane are masked off.  The LWAVES loader wavefronts share the
+// chunks of every plane round-robin (`lwave` = index of the calling one).  Returns nothing; the number of
+// instructions issued per plane by this wavefront is copies_per_plane() below.
+template <int G, int LWAVES, int CGS, int PITCH>
+__device__ __forceinline__ void issue_stage_copy(const char* src, char* dst, uint32_t plane_bytes, int nch,
+                                                 uint32_t lwave, uint32_t lane)
 {
-    constexpr int NWAVES = THREADS / 64;
     constexpr uint32_t CHUNK = 64u * G;
-    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const uint32_t lane_off = (threadIdx.x & 63u) * G;
+    const uint32_t lane_off = lane * G;
 #pragma unroll
     for (int k = 0; k < CGS; k++) {
         if (k < nch) {
             const char* sp = src + (size_t)k * plane_bytes;
             char* dp = dst + k * PITCH;
-            for (uint32_t base = wave * CHUNK; base < plane_bytes; base += NWAVES * CHUNK) {
+            for (uint32_t base = lwave * CHUNK; base < plane_bytes; base += LWAVES * CHUNK) {
                 if (base + lane_off < plane_bytes) {
                     const global_cptr_t gsrc = (global_cptr_t)(sp + base + lane_off);
                     const lds_ptr_t ldst = (lds_ptr_t)(dp + base);
@@ -181,25 +171,27 @@ __device__ __forceinline__ void issue_stage_copy(const char* src, char* dst, uin
 // compile-time so that a tap address is "register + immediate").  Stage s lives in slot s % NBUF and up to
 // NBUF-1 later stages are in flight while it is sampled.
 //
-// Completion of a stage copy is tracked with the wavefront's own vector-memory counter, which retires in issue
-// order: when stage s is needed, the operations this wavefront issued after the copy of stage s are the copies
-// of the NBUF-2 following stages and the output stores of the stages sampled since, so waiting until at most
-// that many operations are outstanding guarantees the copy has landed without draining the newer ones.  The
-// count is exact only while every stage involved is a full one; otherwise the wait is for everything.
-template <typename T, int INTERP, int PAD, bool ALIGN, int THREADS, int PPT, int CGS, int NBUF, int PITCH>
-__global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 4))) void gs2d_lds_kernel(
+// The workgroup is split by role.  SWAVES sampler wavefronts own the output pixels (one lane = PPT pixels); they
+// only read LDS and store results, and they never wait for their stores.  LWAVES loader wavefronts only issue
+// the global->LDS copies.  On this architecture one counter per wavefront tracks loads and stores together and
+// retires in issue order, so a wavefront that both copied and stored would have every copy wait behind its
+// older stores; with the roles split the loader's counter sees copies only, and "stage s has landed" is "at most
+// the copies of the later stages are outstanding".  One workgroup barrier per stage hands the stage over and
+// tells the loaders that the slot sampled before is free again.
+template <typename T, int INTERP, int PAD, bool ALIGN, int SWAVES, int LWAVES, int PPT, int CGS, int NBUF, int PITCH>
+__global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves_per_eu(1, 5))) void gs2d_lds_kernel(
     const T* __restrict__ x, const T* __restrict__ grid, T* __restrict__ y, int32_t C, int32_t H, int32_t W,
     int32_t out_plane, uint32_t tiles_per_n, uint32_t cblocks, int32_t chans_per_block, int32_t copy_gran,
-    int32_t pair_aligned, int32_t xcd_swizzle)
+    int32_t pair_aligned, int32_t xcd_swizzle, float neg_zero)
 {
     extern __shared__ uint4 smem_raw[];
     char* lds = reinterpret_cast<char*>(smem_raw);
     constexpr int NT = (INTERP == 0) ? 4 : 1;
     constexpr int SLOT_BYTES = CGS * PITCH;
-    constexpr int DEPTH = NBUF - 1;          // stages in flight ahead of the one being sampled
-    constexpr int NWAVES = THREADS / 64;
-    constexpr uint32_t STORES_PER_STAGE = PPT * CGS;
+    constexpr int DEPTH = NBUF - 1;  // stages in flight ahead of the one being sampled
+    constexpr int STHREADS = SWAVES * 64;
     const int tid = threadIdx.x;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane((uint32_t)tid >> 6);
 
     // Block -> (group = (n, channel block), tile).  Workgroups are handed to the 8 XCDs round-robin by index;
     // with the swizzle all tiles of one group (they read the same input planes) land on the same XCD next to
@@ -224,44 +216,68 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 4)))
     const int32_t c_end = (c_begin + chans_per_block < C) ? c_begin + chans_per_block : C;
     const int32_t nchan = c_end - c_begin;
     const int32_t nstages = (nchan + CGS - 1) / CGS;
-    const int32_t nfull = nchan / CGS;  // stages 0 .. nfull-1 hold CGS planes
-    const char* xb = reinterpret_cast<const char*>(x + ((int64_t)n * C + c_begin) * plane_elems);
-    const size_t stage_bytes = (size_t)CGS * plane_bytes;
 
-    // copy instructions this wavefront issues per plane (copy_gran is 16 or 4 bytes per lane)
-    uint32_t copies_per_plane;
-    {
+    if (wave >= (uint32_t)SWAVES) {
+        // ------------------------------------------------ loader wavefronts ------------------------------------
+        const uint32_t lwave = wave - SWAVES;
+        const uint32_t lane = (uint32_t)tid & 63u;
+        const char* xb = reinterpret_cast<const char*>(x + ((int64_t)n * C + c_begin) * plane_elems);
+        const size_t stage_bytes = (size_t)CGS * plane_bytes;
+        // copy instructions this wavefront issues per plane
         const uint32_t chunk = 64u * (uint32_t)copy_gran;
         const uint32_t chunks = (plane_bytes + chunk - 1) / chunk;
-        const uint32_t wave = __builtin_amdgcn_readfirstlane((uint32_t)tid >> 6);
-        copies_per_plane = (chunks > wave) ? (chunks - wave + NWAVES - 1) / NWAVES : 0;
+        const uint32_t per_plane = (chunks > lwave) ? (chunks - lwave + LWAVES - 1) / LWAVES : 0;
+        auto planes_of = [&](int32_t s) {
+            const int32_t left = nchan - s * CGS;
+            return left < CGS ? left : CGS;
+        };
+        auto start_stage = [&](int32_t s, int slot) {
+            const char* src = xb + (size_t)s * stage_bytes;
+            char* dst = lds + slot * SLOT_BYTES;
+            if (copy_gran == 16) {
+                issue_stage_copy<16, LWAVES, CGS, PITCH>(src, dst, plane_bytes, planes_of(s), lwave, lane);
+            } else {
+                issue_stage_copy<4, LWAVES, CGS, PITCH>(src, dst, plane_bytes, planes_of(s), lwave, lane);
+            }
+        };
+#pragma unroll
+        for (int s = 0; s < DEPTH; s++) {
+            if (s < nstages) {
+                start_stage(s, s);
+            }
+        }
+        int slot = 0;
+        for (int32_t s = 0; s < nstages; s++) {
+            // outstanding after stage s has landed: the copies of stages s+1 .. min(s+DEPTH, nstages)-1
+            int32_t later_planes = 0;
+            for (int32_t q = s + 1; q < s + DEPTH && q < nstages; q++) {
+                later_planes += planes_of(q);
+            }
+            wait_vmcnt((uint32_t)later_planes * per_plane);
+            lds_barrier();
+            if (s + DEPTH < nstages) {
+                int refill = slot + DEPTH;
+                refill = (refill >= NBUF) ? refill - NBUF : refill;
+                start_stage(s + DEPTH, refill);
+            }
+            slot = (slot + 1 == NBUF) ? 0 : slot + 1;
+        }
+        return;
     }
 
-    auto start_stage = [&](int32_t s, int slot) {
-        const int32_t left = nchan - s * CGS;
-        const int nch = left < CGS ? left : CGS;
-        const char* src = xb + (size_t)s * stage_bytes;
-        char* dst = lds + slot * SLOT_BYTES;
-        if (copy_gran == 16) {
-            issue_stage_copy<16, THREADS, CGS, PITCH>(src, dst, plane_bytes, nch);
-        } else {
-            issue_stage_copy<4, THREADS, CGS, PITCH>(src, dst, plane_bytes, nch);
-        }
-    };
-
+    // ---------------------------------------------------- sampler wavefronts -----------------------------------
     // the zero slots behind each staged plane (all ring slots); stage copies never touch them
     if (tid < NBUF * CGS * 4) {
         reinterpret_cast<uint32_t*>(lds + (tid >> 2) * PITCH + zero_off)[tid & 3] = 0u;
     }
-    start_stage(0, 0);
 
-    // ---- per-pixel decisions, once for the whole channel range (overlaps the first stage copy) ----
+    // per-pixel decisions, once for the whole channel range
     uint32_t toff[PPT][NT];
     float tw[PPT][4];
     uint32_t pixoff[PPT];  // byte offset of the pixel inside an output plane; out of range for lanes past the end
 #pragma unroll
     for (int j = 0; j < PPT; j++) {
-        const int32_t pix = (int32_t)tile * (THREADS * PPT) + j * THREADS + tid;
+        const int32_t pix = (int32_t)tile * (STHREADS * PPT) + j * STHREADS + tid;
         const bool valid = pix < out_plane;
         const int32_t pc = valid ? pix : out_plane - 1;
         pixoff[j] = valid ? (uint32_t)pc * (uint32_t)sizeof(T) : 0x80000000u;
@@ -295,15 +311,6 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 4)))
         }
     }
 
-    // the rest of the prologue: stages 1 .. DEPTH-1 (stage 0 went out before the grid loads so that the wait
-    // for the grid values does not also wait for these)
-#pragma unroll
-    for (int s = 1; s < DEPTH; s++) {
-        if (s < nstages) {
-            start_stage(s, s);
-        }
-    }
-
     T* yb = y + ((int64_t)n * C + c_begin) * out_plane;
     const uint32_t out_plane_bytes = (uint32_t)out_plane * (uint32_t)sizeof(T);
 
@@ -330,7 +337,7 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 4)))
                     __builtin_amdgcn_make_buffer_rsrc(ys + (int64_t)k * out_plane, 0, out_plane_bytes, kBufferFlags);
 #pragma unroll
                 for (int j = 0; j < PPT; j++) {
-                    buffer_store_elem<T>(blend<T, INTERP>(raw[k & 1][j], tw[j]), rsrc, pixoff[j]);
+                    buffer_store_elem<T>(blend<T, INTERP>(raw[k & 1][j], tw[j], neg_zero), rsrc, pixoff[j]);
                 }
             }
         } else {
@@ -344,47 +351,21 @@ __global__ __launch_bounds__(THREADS) __attribute__((amdgpu_waves_per_eu(1, 4)))
                 }
 #pragma unroll
                 for (int j = 0; j < PPT; j++) {
-                    buffer_store_elem<T>(blend<T, INTERP>(raw[j], tw[j]), rsrc, pixoff[j]);
+                    buffer_store_elem<T>(blend<T, INTERP>(raw[j], tw[j], neg_zero), rsrc, pixoff[j]);
                 }
             }
         }
     };
 
-    // One step of the ring: wait for the copy of stage s, barrier (it also tells that every wavefront has left
-    // the slot that is refilled next), start the copy of stage s + DEPTH, sample stage s.
-    auto step = [&](int32_t s, auto slot_tag) {
-        constexpr int SLOT = decltype(slot_tag)::value;
-        // Operations issued after the copy of stage s: copies of stages s+1 .. s+DEPTH-1 and the stores of the
-        // min(s, DEPTH) stages sampled since.  Exact only when those later stages exist and are full.
-        if (s + DEPTH - 1 < nfull) {
-            const uint32_t sampled = (s < DEPTH) ? (uint32_t)s : (uint32_t)DEPTH;
-            wait_vmcnt_table<(DEPTH - 1) * CGS, STORES_PER_STAGE, (DEPTH < 3 ? DEPTH : 3)>(copies_per_plane, sampled);
-        } else {
-            wait_vmcnt_imm<0>();
-        }
-        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the zero-slot writes before the first barrier
-        lds_barrier();
-        if (s + DEPTH < nstages) {
-            start_stage(s + DEPTH, (SLOT + DEPTH) % NBUF);
-        }
-        sample_stage(s, lds + SLOT * SLOT_BYTES);
-    };
-
+    // the ring, unrolled by NBUF so that the slot offset is an immediate; one barrier per stage, matched by the
+    // loaders' loop above
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the zero-slot writes, before the first barrier publishes them
     for (int32_t s = 0; s < nstages; s += NBUF) {
-        step(s, std::integral_constant<int, 0>{});
-        if constexpr (NBUF > 1) {
-            if (s + 1 < nstages) {
-                step(s + 1, std::integral_constant<int, 1 % NBUF>{});
-            }
-        }
-        if constexpr (NBUF > 2) {
-            if (s + 2 < nstages) {
-                step(s + 2, std::integral_constant<int, 2 % NBUF>{});
-            }
-        }
-        if constexpr (NBUF > 3) {
-            if (s + 3 < nstages) {
-                step(s + 3, std::integral_constant<int, 3 % NBUF>{});
+#pragma unroll
+        for (int u = 0; u < NBUF; u++) {
+            if (s + u < nstages) {
+                lds_barrier();
+                sample_stage(s + u, lds + u * SLOT_BYTES);
             }
         }
     }

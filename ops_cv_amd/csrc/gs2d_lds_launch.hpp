@@ -20,7 +20,11 @@ struct LdsPlan {
     int32_t chans_per_block = 0;
 };
 
-constexpr int kThreads = 512;
+constexpr int kSamplerWaves = 8;  // 512 lanes own output pixels
+// loader wavefronts per size class: enough that (NBUF-2) stages of one loader's copy instructions fit the
+// 6-bit outstanding-operation counter (a 1 KiB chunk per instruction)
+constexpr int kLoaderWaves[4] = {1, 1, 2, 4};
+constexpr int kThreads = kSamplerWaves * 64;  // pixels per tile = kThreads * ppt
 // plane pitch in LDS and planes per stage for the four size classes; two stage buffers are resident
 constexpr int kPitch[4] = {2064, 8208, 32784, 81904};
 constexpr int kCgs[4] = {4, 2, 1, 1};   // planes per stage
@@ -28,10 +32,10 @@ constexpr int kNbuf[4] = {4, 4, 4, 2};  // ring slots (stages resident in LDS)
 
 LdsPlan make_lds_plan(const GridSamplerArgs& a);
 
-template <typename T, int I, int P, bool A, int PPT, int CGS, int NBUF, int PITCH>
+template <typename T, int I, int P, bool A, int PPT, int CGS, int NBUF, int PITCH, int LWAVES>
 hipError_t launch_one(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t stream)
 {
-    auto kernel = gs2d_lds_kernel<T, I, P, A, kThreads, PPT, CGS, NBUF, PITCH>;
+    auto kernel = gs2d_lds_kernel<T, I, P, A, kSamplerWaves, LWAVES, PPT, CGS, NBUF, PITCH>;
     static bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -44,9 +48,9 @@ hipError_t launch_one(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t st
     const int64_t esz = sizeof(T);
     const int pair_aligned = (reinterpret_cast<uintptr_t>(a.grid) % (2 * esz) == 0);
     const uint32_t blocks = (uint32_t)(a.N * p.tiles_per_n * p.cblocks);
-    hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kThreads), p.lds_bytes, stream, (const T*)a.x, (const T*)a.grid,
+    hipLaunchKernelGGL(kernel, dim3(blocks), dim3((kSamplerWaves + LWAVES) * 64), p.lds_bytes, stream, (const T*)a.x, (const T*)a.grid,
                        (T*)a.y, (int32_t)a.C, (int32_t)a.Hin, (int32_t)a.Win, (int32_t)(a.Hout * a.Wout),
-                       p.tiles_per_n, p.cblocks, p.chans_per_block, p.copy_gran, pair_aligned, p.xcd_swizzle);
+                       p.tiles_per_n, p.cblocks, p.chans_per_block, p.copy_gran, pair_aligned, p.xcd_swizzle, -0.0f);
     return hipGetLastError();
 }
 
@@ -54,10 +58,10 @@ template <typename T, int I, int P, bool A, int PPT>
 hipError_t launch_class(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t stream)
 {
     switch (p.cls) {
-        case 0: return launch_one<T, I, P, A, PPT, kCgs[0], kNbuf[0], kPitch[0]>(a, p, stream);
-        case 1: return launch_one<T, I, P, A, PPT, kCgs[1], kNbuf[1], kPitch[1]>(a, p, stream);
-        case 2: return launch_one<T, I, P, A, PPT, kCgs[2], kNbuf[2], kPitch[2]>(a, p, stream);
-        default: return launch_one<T, I, P, A, PPT, kCgs[3], kNbuf[3], kPitch[3]>(a, p, stream);
+        case 0: return launch_one<T, I, P, A, PPT, kCgs[0], kNbuf[0], kPitch[0], kLoaderWaves[0]>(a, p, stream);
+        case 1: return launch_one<T, I, P, A, PPT, kCgs[1], kNbuf[1], kPitch[1], kLoaderWaves[1]>(a, p, stream);
+        case 2: return launch_one<T, I, P, A, PPT, kCgs[2], kNbuf[2], kPitch[2], kLoaderWaves[2]>(a, p, stream);
+        default: return launch_one<T, I, P, A, PPT, kCgs[3], kNbuf[3], kPitch[3], kLoaderWaves[3]>(a, p, stream);
     }
 }
 
