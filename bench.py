@@ -24,6 +24,13 @@ for _p in (ROOT, os.path.join(ROOT, "tests")):
 
 HBM_PEAK_GBS = 8000.0
 
+# HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs summarised under profiles/ (scaled by a
+# plain copy of known size), keyed by (workload, kernel variant); anything else reports null
+MEASURED_TRAFFIC = {
+    ("C3", "lds_ring_p8208_2x4"): 69.41e6,   # profiles/gs2d_lds_ring_C3_fp16_n16_c256.md
+    ("C4", "nchw_band_lds"): 1415.4e6,       # profiles/resize_band_lds_C4_fp16_4k_upscale.md
+}
+
 # name -> description of the workloads (shapes as in the baseline configuration list)
 GS_WORKLOADS = {
     "C1": dict(dtype="fp32", x=(1, 3, 64, 64), grid=(1, 32, 32), kind="uniform", interp=0, pad=0, align=False,
@@ -185,7 +192,7 @@ def bench_gs(name, steps, warmup, interp=None, pad=None, align=None, sets=None, 
     desc = "%s grid_sampler2d %s x%s grid%s %s %s align_corners=%s" % (
         name, w["dtype"], tuple(w["x"]), (N, Ho, Wo, 2), INTERP_NAMES[w["interp"]], PAD_NAMES[w["pad"]], w["align"])
     return dict(workload=desc, samples=samples, alg_bytes=alg_bytes, timed=t, variant=variant, parity=parity,
-                sets=nsets, cpu=(x0, g0, w))
+                sets=nsets, cpu=(x0, g0, w), default_modes=(interp is None and pad is None and align is None))
 
 
 def bench_up(name, steps, warmup, sets=None, check=True):
@@ -257,8 +264,10 @@ def bench_up(name, steps, warmup, sets=None, check=True):
 
 def roofline_of(r):
     gbs = r["alg_bytes"] / (r["timed"].kernel_us * 1e-6) / 1e9
+    name = r["workload"].split(" ")[0]
+    traffic = MEASURED_TRAFFIC.get((name, r["variant"])) if r.get("default_modes", True) else None
     return {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+            "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
             "kernel_us": round(r["timed"].kernel_us, 3), "algorithmic_bytes": r["alg_bytes"],
             "kernel": r["variant"]}
 
@@ -303,6 +312,9 @@ def main():
     ap.add_argument("--workload", default="C3", help="headline workload (C1..C5)")
     ap.add_argument("--only", action="store_true", help="skip the other workloads and the CPU baseline")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 256 MiB device copy (torch copy_) so that a counter run of this command "
+                         "holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
     ap.add_argument("--preheat-ms", type=float, default=300.0,
                     help="untimed GPU work before each timed region, on top of --warmup steps")
     args = ap.parse_args()
@@ -317,6 +329,14 @@ def main():
         print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
         sys.exit(3)
     torch.cuda.set_device(0)
+
+    if args.copy_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda:0").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     head = args.workload
     if head in GS_WORKLOADS:
