@@ -22,7 +22,12 @@ LdsPlan make_lds_plan(const GridSamplerArgs& a)
     }
     const int cgs = kCgs[p.cls];
     p.lds_bytes = (uint32_t)(kNbuf[p.cls] * kPitch[p.cls] * cgs);
+    // pixels per lane: every tile of an output plane streams all staged input planes through LDS again, so large
+    // output planes over large input planes take eight (half the tiles, half the LDS fill traffic)
     p.ppt = (out_plane >= 2 * kThreads) ? 4 : 1;
+    if (p.cls >= 2 && out_plane >= 32 * kThreads) {
+        p.ppt = 8;
+    }
     const int64_t tile = (int64_t)kThreads * p.ppt;
     p.tiles_per_n = (uint32_t)((out_plane + tile - 1) / tile);
     // channels per workgroup: as many stages as possible (the pixel decisions are reused across them) while

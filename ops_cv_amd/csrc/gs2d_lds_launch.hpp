@@ -22,8 +22,9 @@ struct LdsPlan {
 
 constexpr int kSamplerWaves = 8;  // 512 lanes own output pixels
 // loader wavefronts per size class: enough that (NBUF-2) stages of one loader's copy instructions fit the
-// 6-bit outstanding-operation counter (a 1 KiB chunk per instruction)
-constexpr int kLoaderWaves[4] = {1, 1, 2, 4};
+// 6-bit outstanding-operation counter (a 1 KiB chunk per instruction), and for the 8 KiB class four of them
+// because one wavefront alone issues the copies of a stage too slowly to keep the ring full
+constexpr int kLoaderWaves[4] = {1, 4, 2, 4};
 constexpr int kThreads = kSamplerWaves * 64;  // pixels per tile = kThreads * ppt
 // plane pitch in LDS and planes per stage for the four size classes; two stage buffers are resident
 constexpr int kPitch[4] = {2064, 8208, 32784, 81904};
@@ -54,18 +55,14 @@ hipError_t launch_one(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t st
     return hipGetLastError();
 }
 
-template <typename T, int I, int P, bool A, int PPT>
-hipError_t launch_class(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t stream)
+template <typename T, int I, int P, bool A, int CLS, int PPT>
+hipError_t launch_cls(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t stream)
 {
-    switch (p.cls) {
-        case 0: return launch_one<T, I, P, A, PPT, kCgs[0], kNbuf[0], kPitch[0], kLoaderWaves[0]>(a, p, stream);
-        case 1: return launch_one<T, I, P, A, PPT, kCgs[1], kNbuf[1], kPitch[1], kLoaderWaves[1]>(a, p, stream);
-        case 2: return launch_one<T, I, P, A, PPT, kCgs[2], kNbuf[2], kPitch[2], kLoaderWaves[2]>(a, p, stream);
-        default: return launch_one<T, I, P, A, PPT, kCgs[3], kNbuf[3], kPitch[3], kLoaderWaves[3]>(a, p, stream);
-    }
+    return launch_one<T, I, P, A, PPT, kCgs[CLS], kNbuf[CLS], kPitch[CLS], kLoaderWaves[CLS]>(a, p, stream);
 }
 
-// Expands (interp, pad, align, pixels per lane, size class) for one element type and launches.
+// Expands (interp, pad, align, size class, pixels per lane) for one element type and launches.  Eight pixels per
+// lane exist for the two large-plane classes only.
 template <typename T>
 struct LdsTypedLauncher {
     const GridSamplerArgs& a;
@@ -74,10 +71,19 @@ struct LdsTypedLauncher {
     template <typename U, int I, int P, bool A>
     hipError_t operator()() const
     {
-        if (p.ppt == 4) {
-            return launch_class<T, I, P, A, 4>(a, p, stream);
+        switch (p.cls * 16 + p.ppt) {
+            case 0 * 16 + 1: return launch_cls<T, I, P, A, 0, 1>(a, p, stream);
+            case 0 * 16 + 4: return launch_cls<T, I, P, A, 0, 4>(a, p, stream);
+            case 1 * 16 + 1: return launch_cls<T, I, P, A, 1, 1>(a, p, stream);
+            case 1 * 16 + 4: return launch_cls<T, I, P, A, 1, 4>(a, p, stream);
+            case 2 * 16 + 1: return launch_cls<T, I, P, A, 2, 1>(a, p, stream);
+            case 2 * 16 + 4: return launch_cls<T, I, P, A, 2, 4>(a, p, stream);
+            case 2 * 16 + 8: return launch_cls<T, I, P, A, 2, 8>(a, p, stream);
+            case 3 * 16 + 1: return launch_cls<T, I, P, A, 3, 1>(a, p, stream);
+            case 3 * 16 + 4: return launch_cls<T, I, P, A, 3, 4>(a, p, stream);
+            case 3 * 16 + 8: return launch_cls<T, I, P, A, 3, 8>(a, p, stream);
+            default: return hipErrorInvalidValue;
         }
-        return launch_class<T, I, P, A, 1>(a, p, stream);
     }
 };
 

@@ -68,6 +68,22 @@ def test_grid_sampler_random(oracle, device, dtype, interp, pad, align):
 
 @pytest.mark.parametrize("dtype", I.DTYPES)
 @pytest.mark.parametrize("interp", [0, 1])
+def test_grid_sampler_large_planes(oracle, device, dtype, interp):
+    """input planes of 20-160 KB and output planes of several tiles with a ragged last one: the staged variants
+    that keep eight pixels per lane, and the largest plane class"""
+    rng = np.random.default_rng(1500 + interp)
+    for (N, C, H, W, Ho, Wo, pad, align) in [(1, 3, 100, 100, 130, 131, 1, True), (2, 2, 120, 96, 129, 129, 0, False),
+                                             (1, 2, 200, 100, 150, 150, 2, False)]:
+        x32 = rng.standard_normal((N, C, H, W)).astype(np.float32)
+        g32 = rng.uniform(-1.1, 1.1, (N, Ho, Wo, 2)).astype(np.float32)
+        y, y_ref = _run_gs(oracle, device, x32, g32, dtype, interp, pad, align)
+        _check(y, y_ref, dtype, interp, "gs-large %s %s %s" % (dtype, INTERP[interp], (N, C, H, W, Ho, Wo)))
+        if dtype == "fp32":
+            assert np.array_equal(y.view(np.uint32), y_ref.view(np.uint32))
+
+
+@pytest.mark.parametrize("dtype", I.DTYPES)
+@pytest.mark.parametrize("interp", [0, 1])
 @pytest.mark.parametrize("pad", [0, 1, 2])
 @pytest.mark.parametrize("align", [False, True])
 def test_grid_sampler_special_coordinates(oracle, device, dtype, interp, pad, align):
