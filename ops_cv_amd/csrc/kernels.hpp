@@ -27,7 +27,8 @@ hipError_t launch_strided_copy(const StridedView& v, void* contiguous, int elem_
 
 // LDS-staged row-band resize (resize_band_lds.hip); *handled is false when the shape does not qualify.
 hipError_t run_resize_band_lds(const ResizeArgs& a, hipStream_t stream, bool* handled);
-bool resize_band_lds_applicable(const ResizeArgs& a);
+// name of the LDS-staged variant that would run, or nullptr when neither applies
+const char* resize_lds_variant(const ResizeArgs& a);
 
 // Name of the kernel variant the launcher would pick for these arguments (for benchmarks and tests).
 const char* grid_sampler2d_variant(const GridSamplerArgs& a);

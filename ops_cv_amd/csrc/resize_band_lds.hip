@@ -6,6 +6,7 @@
 
 #include "kernels.hpp"
 #include "resize_band_lds_kernel.hpp"
+#include "resize_flat_lds_kernel.hpp"
 
 namespace opscv {
 
@@ -110,9 +111,125 @@ BandPlan make_plan(const ResizeArgs& a)
     return bp;
 }
 
+// ---- narrow images: 2-D lane arrangement (resize_flat_lds_kernel.hpp) ----
+constexpr int kFlatThreads = 256;
+constexpr int kFlatMaxColumnLanes = 128;   // wider rows keep at least half of the band variant's lanes busy
+constexpr int kFlatLdsBudget = 32 * 1024;  // per workgroup: several workgroups per CU hide the staging latency
+constexpr int64_t kFlatWantBlocks = 2048;
+
+struct FlatPlan {
+    bool ok = false;
+    FlatLdsParams p{};
+    uint32_t lds_bytes = 0;
+    dim3 grid;
+};
+
+template <typename T, bool HALF_PIXEL>
+int32_t flat_max_rows(const ResizeArgs& a, int32_t band_rows)
+{
+    const int32_t Hd = (int32_t)a.Hd, Hs = (int32_t)a.Hs;
+    int32_t mr = 0;
+    for (int32_t hb = 0; hb < Hd; hb += band_rows) {
+        const int32_t he = (hb + band_rows < Hd) ? hb + band_rows : Hd;
+        const int32_t lo = axis_tap<HALF_PIXEL>(hb, a.scale_h, Hs).i0;
+        const int32_t hi = axis_tap<HALF_PIXEL>(he - 1, a.scale_h, Hs).i1;
+        mr = (hi - lo + 1 > mr) ? hi - lo + 1 : mr;
+    }
+    return mr;
+}
+
+template <typename T>
+FlatPlan make_flat_plan(const ResizeArgs& a)
+{
+    FlatPlan fp;
+    constexpr int V = 16 / (int)sizeof(T);
+    if (a.channels_last || a.mode != ResizeMode::Bilinear) {
+        return fp;
+    }
+    // whole 16-byte output vectors, 16-byte aligned output planes, 32-bit byte offsets inside an output plane
+    if (a.Wd % V != 0 || reinterpret_cast<uintptr_t>(a.y) % 16 != 0 ||
+        a.Hd * a.Wd * (int64_t)sizeof(T) >= (1ll << 31)) {
+        return fp;
+    }
+    const int64_t cl = a.Wd / V;
+    if (cl > kFlatMaxColumnLanes) {
+        return fp;
+    }
+    const uintptr_t xa = reinterpret_cast<uintptr_t>(a.x);
+    int gran;
+    if ((a.Ws * sizeof(T)) % 16 == 0 && xa % 16 == 0) {
+        gran = 16;
+    } else if ((a.Ws * sizeof(T)) % 4 == 0 && xa % 4 == 0) {
+        gran = 4;
+    } else {
+        return fp;
+    }
+    const int32_t rg = kFlatThreads / (int32_t)cl;
+    const int64_t planes = a.N * a.C;
+    // bands: enough workgroups to fill the chip several times over, each a whole number of row-group passes
+    int64_t bands = (kFlatWantBlocks + planes - 1) / planes;
+    int64_t band_rows = (a.Hd + bands - 1) / bands;
+    band_rows = (band_rows + rg - 1) / rg * rg;
+    int32_t rows = 0;
+    for (;;) {
+        rows = a.half_pixel ? flat_max_rows<T, true>(a, (int32_t)band_rows) : flat_max_rows<T, false>(a, (int32_t)band_rows);
+        if ((int64_t)rows * a.Ws * (int64_t)sizeof(T) <= kFlatLdsBudget) {
+            break;
+        }
+        if (band_rows <= rg) {
+            return fp;  // even one pass of the row groups touches more source rows than the budget holds
+        }
+        band_rows = (band_rows / 2 + rg - 1) / rg * rg;
+    }
+    bands = (a.Hd + band_rows - 1) / band_rows;
+    if (bands > INT32_MAX) {
+        return fp;
+    }
+    fp.p.planes = planes;
+    fp.p.Hs = (int32_t)a.Hs;
+    fp.p.Ws = (int32_t)a.Ws;
+    fp.p.Hd = (int32_t)a.Hd;
+    fp.p.Wd = (int32_t)a.Wd;
+    fp.p.scale_h = a.scale_h;
+    fp.p.scale_w = a.scale_w;
+    fp.p.band_rows = (int32_t)band_rows;
+    fp.p.cl = (int32_t)cl;
+    fp.p.rg = rg;
+    fp.p.gran = gran;
+    fp.p.neg_zero = -0.0f;
+    fp.lds_bytes = (uint32_t)(((int64_t)rows * a.Ws * (int64_t)sizeof(T) + 15) / 16 * 16);
+    fp.grid = dim3((unsigned)bands, (unsigned)(planes < 65535 ? planes : 65535));
+    const char* v = getenv("OPSCV_RESIZE_VARIANT");
+    // generic / register-band / LDS band forced (benchmark knob)
+    fp.ok = !(v != nullptr && (v[0] == 'g' || v[0] == 'r' || v[0] == 'b'));
+    return fp;
+}
+
+template <typename T>
+hipError_t run_flat_typed(const ResizeArgs& a, hipStream_t stream, bool* handled)
+{
+    const FlatPlan fp = make_flat_plan<T>(a);
+    if (!fp.ok) {
+        return hipSuccess;
+    }
+    *handled = true;
+    if (a.half_pixel) {
+        hipLaunchKernelGGL((resize_flat_lds_kernel<T, true, kFlatThreads>), fp.grid, dim3(kFlatThreads), fp.lds_bytes,
+                           stream, (const T*)a.x, (T*)a.y, fp.p);
+    } else {
+        hipLaunchKernelGGL((resize_flat_lds_kernel<T, false, kFlatThreads>), fp.grid, dim3(kFlatThreads), fp.lds_bytes,
+                           stream, (const T*)a.x, (T*)a.y, fp.p);
+    }
+    return hipGetLastError();
+}
+
 template <typename T>
 hipError_t run_typed(const ResizeArgs& a, hipStream_t stream, bool* handled)
 {
+    const hipError_t e = run_flat_typed<T>(a, stream, handled);
+    if (*handled || e != hipSuccess) {
+        return e;
+    }
     const BandPlan bp = make_plan<T>(a);
     if (!bp.ok) {
         return hipSuccess;
@@ -140,14 +257,15 @@ hipError_t run_typed(const ResizeArgs& a, hipStream_t stream, bool* handled)
 
 }  // namespace
 
-bool resize_band_lds_applicable(const ResizeArgs& a)
+const char* resize_lds_variant(const ResizeArgs& a)
 {
+    bool flat = false, band = false;
     switch (a.elem) {
-        case Elem::F32: return make_plan<float>(a).ok;
-        case Elem::F16: return make_plan<_Float16>(a).ok;
-        case Elem::BF16: return make_plan<__bf16>(a).ok;
+        case Elem::F32: flat = make_flat_plan<float>(a).ok; band = make_plan<float>(a).ok; break;
+        case Elem::F16: flat = make_flat_plan<_Float16>(a).ok; band = make_plan<_Float16>(a).ok; break;
+        case Elem::BF16: flat = make_flat_plan<__bf16>(a).ok; band = make_plan<__bf16>(a).ok; break;
     }
-    return false;
+    return flat ? "nchw_flat_lds" : (band ? "nchw_band_lds" : nullptr);
 }
 
 hipError_t run_resize_band_lds(const ResizeArgs& a, hipStream_t stream, bool* handled)

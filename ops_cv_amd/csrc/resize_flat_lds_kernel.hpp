@@ -1,0 +1,128 @@
+// Bilinear resize, NCHW, LDS-staged variant for narrow images on gfx950: device code.
+//
+// Arithmetic: image/resize_bilinear_v2/op_kernel/arch35/resize_bilinear_v2_simt_nchw.h:108-144 (see resize_math.hpp).
+//
+// The row-band variant gives a lane one 16-byte output vector of a row, so an output row narrower than the
+// workgroup leaves most lanes idle.  Here the lanes of a workgroup form a 2-D arrangement instead:
+// `cl` column lanes (one 16-byte output vector each, together a whole output row) times `rg` row groups.
+//   * A workgroup owns (plane, band of output rows).  The source rows the band touches are whole rows and
+//     therefore one contiguous byte range; they are copied from HBM into LDS once with the asynchronous
+//     global->LDS loads.
+//   * A lane computes its column taps once; it then walks the band rows  hb + group, hb + group + rg, ...  and
+//     evaluates the reference formula per output element from eight (fp32: four-byte, else two-byte) LDS reads
+//     per column pair -- same operations in the same order as the per-pixel reference.
+//   * One 16-byte store per lane and row through a buffer descriptor over the output plane.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "resize_band_lds_kernel.hpp"
+
+namespace opscv {
+
+struct FlatLdsParams {
+    int64_t planes;
+    int32_t Hs, Ws, Hd, Wd;
+    float scale_h, scale_w;
+    int32_t band_rows;  // output rows per workgroup (a multiple of rg)
+    int32_t cl;         // column lanes = Wd / V
+    int32_t rg;         // row groups = THREADS / cl
+    int32_t gran;       // bytes per lane of the asynchronous copy: 16 or 4
+    float neg_zero;     // -0.0f, passed in so that fma(v, w, -0) is not folded back into a multiply
+};
+
+template <typename T, bool HALF_PIXEL, int THREADS>
+__global__ __launch_bounds__(THREADS) void resize_flat_lds_kernel(const T* __restrict__ x, T* __restrict__ y,
+                                                                   FlatLdsParams p)
+{
+    constexpr int V = 16 / (int)sizeof(T);
+    constexpr int NWAVES = THREADS / 64;
+    extern __shared__ uint4 smem_raw[];
+    char* lds = reinterpret_cast<char*>(smem_raw);
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane((uint32_t)tid >> 6);
+
+    const int32_t group = tid / p.cl;
+    const int32_t cvec = tid - group * p.cl;
+    const bool active = group < p.rg;
+
+    const int32_t h_begin = blockIdx.x * p.band_rows;
+    const int32_t h_end = (h_begin + p.band_rows < p.Hd) ? h_begin + p.band_rows : p.Hd;
+    const int32_t ys_lo = axis_tap<HALF_PIXEL>(h_begin, p.scale_h, p.Hs).i0;
+    const int32_t ys_hi = axis_tap<HALF_PIXEL>(h_end - 1, p.scale_h, p.Hs).i1;
+    const uint32_t src_row_bytes = (uint32_t)p.Ws * (uint32_t)sizeof(T);
+    const uint32_t stage_bytes = (uint32_t)(ys_hi - ys_lo + 1) * src_row_bytes;
+
+    // ---- per-lane column taps ----
+    const int32_t col0 = cvec * V;
+    uint32_t to0[V], to1[V];
+    float dx[V], omdx[V];
+#pragma unroll
+    for (int i = 0; i < V; i++) {
+        int32_t c = col0 + i;
+        c = (c < p.Wd) ? c : p.Wd - 1;
+        const AxisTap t = axis_tap<HALF_PIXEL>(c, p.scale_w, p.Ws);
+        to0[i] = (uint32_t)t.i0 * (uint32_t)sizeof(T);
+        to1[i] = (uint32_t)t.i1 * (uint32_t)sizeof(T);
+        dx[i] = t.lambda;
+        omdx[i] = 1.0f - t.lambda;
+    }
+    const uint32_t out_row_bytes = (uint32_t)p.Wd * (uint32_t)sizeof(T);
+    const uint32_t out_plane_bytes = (uint32_t)p.Hd * out_row_bytes;
+    const uint32_t col_off = (uint32_t)col0 * (uint32_t)sizeof(T);
+    const float neg_zero = p.neg_zero;
+    const uint32_t chunk = 64u * (uint32_t)p.gran;
+
+    for (int64_t pl = blockIdx.y; pl < p.planes; pl += gridDim.y) {
+        const char* src0 = reinterpret_cast<const char*>(x + (pl * p.Hs + ys_lo) * (int64_t)p.Ws);
+        for (uint32_t cb = wave * chunk; cb < stage_bytes; cb += NWAVES * chunk) {
+            const uint32_t lane_off = cb + (uint32_t)lane * (uint32_t)p.gran;
+            if (lane_off < stage_bytes) {
+                const rs_global_cptr_t g = (rs_global_cptr_t)(src0 + lane_off);
+                const rs_lds_ptr_t l = (rs_lds_ptr_t)(lds + cb);
+                if (p.gran == 16) {
+                    __builtin_amdgcn_global_load_lds(g, l, 16, 0, 0);
+                } else {
+                    __builtin_amdgcn_global_load_lds(g, l, 4, 0, 0);
+                }
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+
+        const __amdgpu_buffer_rsrc_t rsrc =
+            __builtin_amdgcn_make_buffer_rsrc(y + pl * (int64_t)p.Hd * p.Wd, 0, out_plane_bytes, kRsBufferFlags);
+        for (int32_t h = active ? h_begin + group : h_end; h < h_end; h += p.rg) {
+            const AxisTap t = axis_tap<HALF_PIXEL>(h, p.scale_h, p.Hs);
+            const char* r0 = lds + (uint32_t)(t.i0 - ys_lo) * src_row_bytes;
+            const char* r1 = lds + (uint32_t)(t.i1 - ys_lo) * src_row_bytes;
+            T tl[V], tr[V], bl[V], br[V];
+#pragma unroll
+            for (int i = 0; i < V; i++) {
+                tl[i] = *reinterpret_cast<const T*>(r0 + to0[i]);
+                tr[i] = *reinterpret_cast<const T*>(r0 + to1[i]);
+                bl[i] = *reinterpret_cast<const T*>(r1 + to0[i]);
+                br[i] = *reinterpret_cast<const T*>(r1 + to1[i]);
+            }
+            const float dy = t.lambda;
+            const float omdy = 1.0f - dy;
+            T outv[V];
+#pragma unroll
+            for (int i = 0; i < V; i++) {
+                // fma(v, w, -0) is v * w bit for bit; see resize_band_lds_kernel.hpp
+                const float top = __builtin_fmaf(ElemIO<T>::load(&tl[i]), omdx[i], neg_zero) +
+                                  __builtin_fmaf(ElemIO<T>::load(&tr[i]), dx[i], neg_zero);
+                const float bot = __builtin_fmaf(ElemIO<T>::load(&bl[i]), omdx[i], neg_zero) +
+                                  __builtin_fmaf(ElemIO<T>::load(&br[i]), dx[i], neg_zero);
+                ElemIO<T>::store(&outv[i], omdy * top + dy * bot);
+            }
+            typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+            __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4*>(outv), rsrc,
+                                                   (int)((uint32_t)h * out_row_bytes + col_off), 0, 0);
+        }
+        __syncthreads();  // everybody is done with the staged rows before the next plane overwrites them
+    }
+}
+
+}  // namespace opscv

@@ -293,8 +293,8 @@ const char* resize_variant(const ResizeArgs& a)
     if (a.channels_last) {
         return "nhwc_generic";
     }
-    if (resize_band_lds_applicable(a)) {
-        return "nchw_band_lds";
+    if (const char* lds_variant = resize_lds_variant(a)) {
+        return lds_variant;
     }
     bool band = false;
     switch (a.elem) {

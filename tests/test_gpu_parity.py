@@ -136,7 +136,8 @@ def test_upsample_random(oracle, device, dtype, align):
     cases = [((2, 3, 7, 9), (14, 18)), ((1, 2, 5, 5), (13, 7)), ((2, 2, 16, 16), (5, 3)), ((1, 1, 1, 4), (2, 16)),
              ((1, 1, 1, 4), (3, 16)), ((2, 3, 1, 1), (4, 4)), ((2, 3, 1, 1), (16, 16)), ((2, 3, 6, 6), (1, 1)),
              ((1, 4, 9, 11), (9, 11)), ((1, 2, 56, 56), (112, 112)), ((1, 1, 33, 65), (67, 200)),
-             ((1, 2, 4, 2), (8, 4))]
+             ((1, 2, 4, 2), (8, 4)), ((3, 5, 20, 24), (40, 48)), ((2, 2, 30, 16), (11, 8)),
+             ((1, 3, 64, 32), (200, 64)), ((600, 1, 8, 8), (16, 16)), ((1, 1, 700, 8), (1400, 16))]
     for shape, out_hw in cases:
         x32 = rng.standard_normal(shape).astype(np.float32)
         y, y_ref = _run_up(oracle, device, x32, out_hw, dtype, align)
