@@ -46,7 +46,7 @@ UP_WORKLOADS = {
     "C4": dict(dtype="fp16", x=(4, 16, 1080, 1920), out=(2160, 3840), align=True, scales=(2.0, 2.0),
                dist="uniform", sets=2),
 }
-INTERP_NAMES = {0: "bilinear", 1: "nearest"}
+INTERP_NAMES = {0: "bilinear", 1: "nearest", 2: "bicubic"}
 PAD_NAMES = {0: "zeros", 1: "border", 2: "reflection"}
 
 
@@ -413,6 +413,8 @@ def main():
                     others["C3_%s_%s" % (INTERP_NAMES[interp], PAD_NAMES[pad])] = summary_of(rr)
             rr = bench_gs("C3", args.steps, args.warmup, sets=1)
             others["C3_bilinear_zeros_same_buffers_every_step"] = summary_of(rr)
+            # the third interpolation mode on the same tensors (not part of the headline set)
+            others["C3_bicubic_zeros"] = summary_of(bench_gs("C3", max(10, args.steps // 2), args.warmup, interp=2))
         for name in ("C1", "C5"):
             if name != head:
                 others[name] = summary_of(bench_gs(name, args.steps, args.warmup))

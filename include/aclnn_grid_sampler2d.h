@@ -6,7 +6,7 @@
  *
  * out[n,c,h,w] = sample(input[n,c,:,:], grid[n,h,w,:]) with grid in normalized [-1,1] coordinates
  * (x first, then y).
- *   interpolationMode : 0 bilinear, 1 nearest (2 = bicubic is validated but not implemented: 161002)
+ *   interpolationMode : 0 bilinear, 1 nearest, 2 bicubic (A = -0.75)
  *   paddingMode       : 0 zeros, 1 border, 2 reflection
  *   dtypes            : FLOAT, FLOAT16, BF16 (all three tensors equal); DOUBLE is rejected with 161002
  *   shapes            : input (N,C,Hin,Win), grid (N,Hout,Wout,2), out (N,C,Hout,Wout); formats are ignored

@@ -30,6 +30,21 @@ ACLNN_API aclnnStatus opscvGridSampler2DTaps(const void* grid, aclDataType dataT
                                              int64_t paddingMode, bool alignCorners, opscvTapRecord* taps,
                                              aclrtStream stream);
 
+/* Per-pixel record of the bicubic mode written by opscvGridSampler2DBicubicTaps (68 bytes, packed). */
+typedef struct {
+    int32_t bx[4]; /* tap columns after padding, -1 = outside the image */
+    int32_t by[4]; /* tap rows after padding, -1 = outside the image */
+    float cx[4];   /* column coefficients */
+    float cy[4];   /* row coefficients */
+    int32_t flag;  /* 1 when the pixel is written as NaN (non-finite source coordinate) */
+} opscvBicubicTapRecord;
+
+/* Same as opscvGridSampler2DTaps for interpolationMode 2 (bicubic). */
+ACLNN_API aclnnStatus opscvGridSampler2DBicubicTaps(const void* grid, aclDataType dataType, int64_t N, int64_t Hin,
+                                                    int64_t Win, int64_t Hout, int64_t Wout, int64_t paddingMode,
+                                                    bool alignCorners, opscvBicubicTapRecord* taps,
+                                                    aclrtStream stream);
+
 /*
  * Name of the kernel variant phase 2 would launch for an executor returned by a GetWorkspaceSize call
  * ("" for a no-op executor).  The string is static.

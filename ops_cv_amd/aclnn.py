@@ -101,6 +101,8 @@ def load_library():
     L.aclnnUpsampleBilinear2d.argtypes = [vp, u64, vp, vp]
     L.opscvGridSampler2DTaps.restype = i32
     L.opscvGridSampler2DTaps.argtypes = [vp, ctypes.c_int, i64, i64, i64, i64, i64, i64, i64, ctypes.c_bool, vp, vp]
+    L.opscvGridSampler2DBicubicTaps.restype = i32
+    L.opscvGridSampler2DBicubicTaps.argtypes = [vp, ctypes.c_int, i64, i64, i64, i64, i64, i64, ctypes.c_bool, vp, vp]
     L.opscvExecutorVariant.restype = ctypes.c_char_p
     L.opscvExecutorVariant.argtypes = [vp]
     L.opscvVersion.restype = ctypes.c_char_p
@@ -282,4 +284,23 @@ def grid_sampler2d_taps(grid, h_in, w_in, interpolation_mode=0, padding_mode=0, 
         raise AclnnError("opscvGridSampler2DTaps", st)
     torch.cuda.synchronize()
     dt = np.dtype([("ix0", "<i4"), ("iy0", "<i4"), ("w", "<f4", (4,)), ("flag", "<i4")])
+    return raw.cpu().numpy().view(dt).reshape(n, ho, wo)
+
+
+def grid_sampler2d_bicubic_taps(grid, h_in, w_in, padding_mode=0, align_corners=False, stream=None):
+    """Per-pixel records of the bicubic mode: tap columns/rows after padding, coefficients, NaN flag."""
+    import numpy as np
+    torch = _torch()
+    L = load_library()
+    grid = grid.contiguous()
+    n, ho, wo, _ = grid.shape
+    dt = np.dtype([("bx", "<i4", (4,)), ("by", "<i4", (4,)), ("cx", "<f4", (4,)), ("cy", "<f4", (4,)),
+                   ("flag", "<i4")])
+    raw = torch.empty((n * ho * wo, dt.itemsize), dtype=torch.uint8, device=grid.device)
+    st = L.opscvGridSampler2DBicubicTaps(ctypes.c_void_p(grid.data_ptr()), acl_dtype_of(grid), n, h_in, w_in, ho, wo,
+                                         padding_mode, bool(align_corners), ctypes.c_void_p(raw.data_ptr()),
+                                         _stream_handle(stream))
+    if st != ACLNN_SUCCESS:
+        raise AclnnError("opscvGridSampler2DBicubicTaps", st)
+    torch.cuda.synchronize()
     return raw.cpu().numpy().view(dt).reshape(n, ho, wo)

@@ -118,15 +118,10 @@ aclnnStatus aclnnGridSampler2DGetWorkspaceSize(const aclTensor* input, const acl
         *executor = ex.release();
         return ACLNN_SUCCESS;
     }
-    // The reference routes DOUBLE to a host-CPU kernel that is not part of its tree and bicubic to a
-    // kernel outside this path; neither exists here.
+    // The reference routes DOUBLE to a host-CPU kernel that is not part of its tree; it does not exist here.
     Elem elem;
     if (!elem_of(input->dtype, &elem)) {
         set_error("aclnnGridSampler2D: DOUBLE tensors are not supported by the MI355X implementation");
-        return ACLNN_ERR_PARAM_INVALID;
-    }
-    if (interpolationMode == 2) {
-        set_error("aclnnGridSampler2D: bicubic interpolation is not supported by the MI355X implementation");
         return ACLNN_ERR_PARAM_INVALID;
     }
     for (int i = 0; i < 4; i++) {

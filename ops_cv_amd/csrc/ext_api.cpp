@@ -9,6 +9,7 @@
 using namespace opscv;
 
 static_assert(sizeof(opscvTapRecord) == sizeof(TapRecord), "tap record layouts must match");
+static_assert(sizeof(opscvBicubicTapRecord) == sizeof(BicubicTapRecord), "tap record layouts must match");
 
 extern "C" {
 
@@ -43,6 +44,41 @@ aclnnStatus opscvGridSampler2DTaps(const void* grid, aclDataType dataType, int64
     }
     if (e != hipSuccess) {
         set_error("opscvGridSampler2DTaps: launch failed: %s", hipGetErrorString(e));
+        return ACLNN_ERR_RUNTIME_ERROR;
+    }
+    return ACLNN_SUCCESS;
+}
+
+aclnnStatus opscvGridSampler2DBicubicTaps(const void* grid, aclDataType dataType, int64_t N, int64_t Hin, int64_t Win,
+                                          int64_t Hout, int64_t Wout, int64_t paddingMode, bool alignCorners,
+                                          opscvBicubicTapRecord* taps, aclrtStream stream)
+{
+    if (grid == nullptr || taps == nullptr) {
+        set_error("opscvGridSampler2DBicubicTaps: grid and taps must not be NULL");
+        return ACLNN_ERR_PARAM_NULLPTR;
+    }
+    GridSamplerArgs a;
+    if (!elem_of(dataType, &a.elem) || paddingMode < 0 || paddingMode > 2) {
+        set_error("opscvGridSampler2DBicubicTaps: unsupported dtype or mode");
+        return ACLNN_ERR_PARAM_INVALID;
+    }
+    a.interp = 2;
+    a.pad = (int)paddingMode;
+    a.align = alignCorners ? 1 : 0;
+    a.N = N;
+    a.C = 1;
+    a.Hin = Hin;
+    a.Win = Win;
+    a.Hout = Hout;
+    a.Wout = Wout;
+    a.grid = grid;
+    hipError_t e = launch_grid_sampler2d_bicubic_taps(a, (BicubicTapRecord*)taps, (hipStream_t)stream);
+    if (e == hipErrorInvalidValue) {
+        set_error("opscvGridSampler2DBicubicTaps: shapes out of range");
+        return ACLNN_ERR_PARAM_INVALID;
+    }
+    if (e != hipSuccess) {
+        set_error("opscvGridSampler2DBicubicTaps: launch failed: %s", hipGetErrorString(e));
         return ACLNN_ERR_RUNTIME_ERROR;
     }
     return ACLNN_SUCCESS;

@@ -27,6 +27,12 @@ inline hipError_t dispatch_modes(const GridSamplerArgs& a, F&& f)
     OPSCV_CASE(1, 1, true)
     OPSCV_CASE(1, 2, false)
     OPSCV_CASE(1, 2, true)
+    OPSCV_CASE(2, 0, false)
+    OPSCV_CASE(2, 0, true)
+    OPSCV_CASE(2, 1, false)
+    OPSCV_CASE(2, 1, true)
+    OPSCV_CASE(2, 2, false)
+    OPSCV_CASE(2, 2, true)
 #undef OPSCV_CASE
     return hipErrorInvalidValue;
 }

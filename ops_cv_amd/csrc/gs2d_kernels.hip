@@ -1,4 +1,5 @@
-// Grid sampler 2-D forward kernels for gfx950 (bilinear and nearest; zeros, border, reflection; align on/off).
+// Grid sampler 2-D forward kernels for gfx950 (bilinear, nearest and bicubic; zeros, border, reflection; align
+// on/off).
 //
 // Replaces the reference device kernel image/grid_sampler2_d/op_kernel/arch35/grid_sampler2_d_simt.h:461-557 and
 // its host tiling image/grid_sampler2_d/op_host/arch35/grid_sampler2_d_tiling.cpp:208-271.
@@ -38,9 +39,48 @@ __global__ __launch_bounds__(kDirectThreads) void gs2d_direct_kernel(const T* __
         const int64_t rem = p - n * out_plane;
         const float gx = ElemIO<T>::load(grid + 2 * p);
         const float gy = ElemIO<T>::load(grid + 2 * p + 1);
-        const PixelTap t = decide_pixel<INTERP, PAD, ALIGN>(gx, gy, H, W);
         const T* xp = x + n * C * in_plane;
         T* yp = y + n * C * out_plane + rem;
+        if constexpr (INTERP == 2) {
+            // grid_sampler2_d_simt.h:375-458
+            const BicubicTap b = decide_bicubic<PAD, ALIGN>(gx, gy, H, W);
+            if (b.flag) {
+                const float nan_val = __builtin_nanf("");
+                for (int32_t c = 0; c < C; c++) {
+                    ElemIO<T>::store(yp, nan_val);
+                    yp += out_plane;
+                }
+                continue;
+            }
+            bool col_in[4], row_in[4];
+            int64_t row_off[4];
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                col_in[k] = b.bx[k] >= 0 && b.bx[k] < W;
+                row_in[k] = b.by[k] >= 0 && b.by[k] < H;
+                row_off[k] = row_in[k] ? (int64_t)b.by[k] * W : 0;
+            }
+            for (int32_t c = 0; c < C; c++) {
+                float r[4];
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    r[j] = 0.0f;
+                    if (row_in[j]) {
+                        float v[4];
+#pragma unroll
+                        for (int k = 0; k < 4; k++) {
+                            v[k] = col_in[k] ? ElemIO<T>::load(xp + row_off[j] + b.bx[k]) : 0.0f;
+                        }
+                        r[j] = bicubic_weighted_sum(b.cx[0], b.cx[1], b.cx[2], b.cx[3], v[0], v[1], v[2], v[3]);
+                    }
+                }
+                ElemIO<T>::store(yp, bicubic_weighted_sum(b.cy[0], b.cy[1], b.cy[2], b.cy[3], r[0], r[1], r[2], r[3]));
+                xp += in_plane;
+                yp += out_plane;
+            }
+            continue;
+        }
+        const PixelTap t = decide_pixel<(INTERP == 2 ? 0 : INTERP), PAD, ALIGN>(gx, gy, H, W);
         if (INTERP == 0) {
             if (t.flag) {
                 const float nan_val = __builtin_nanf("");
@@ -120,6 +160,29 @@ __global__ __launch_bounds__(kDirectThreads) void gs2d_taps_kernel(const T* __re
     }
 }
 
+template <typename T, int PAD, bool ALIGN>
+__global__ __launch_bounds__(kDirectThreads) void gs2d_bicubic_taps_kernel(const T* __restrict__ grid,
+                                                                            BicubicTapRecord* __restrict__ taps,
+                                                                            int64_t total_pixels, int32_t H, int32_t W)
+{
+    const int64_t stride = (int64_t)gridDim.x * kDirectThreads;
+    for (int64_t p = (int64_t)blockIdx.x * kDirectThreads + threadIdx.x; p < total_pixels; p += stride) {
+        const float gx = ElemIO<T>::load(grid + 2 * p);
+        const float gy = ElemIO<T>::load(grid + 2 * p + 1);
+        const BicubicTap t = decide_bicubic<PAD, ALIGN>(gx, gy, H, W);
+        BicubicTapRecord r;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            r.bx[k] = t.bx[k];
+            r.by[k] = t.by[k];
+            r.cx[k] = t.cx[k];
+            r.cy[k] = t.cy[k];
+        }
+        r.flag = t.flag;
+        taps[p] = r;
+    }
+}
+
 inline int blocks_for(int64_t items, int threads)
 {
     int64_t b = (items + threads - 1) / threads;
@@ -147,7 +210,24 @@ template <typename T, int INTERP, int PAD, bool ALIGN>
 hipError_t run_taps(const GridSamplerArgs& a, TapRecord* taps, hipStream_t stream)
 {
     const int64_t total = a.N * a.Hout * a.Wout;
-    hipLaunchKernelGGL((gs2d_taps_kernel<T, INTERP, PAD, ALIGN>), dim3(blocks_for(total, kDirectThreads)),
+    if constexpr (INTERP == 2) {
+        (void)taps;
+        (void)stream;
+        (void)total;
+        return hipErrorInvalidValue;  // the bicubic record has its own entry point
+    } else {
+        hipLaunchKernelGGL((gs2d_taps_kernel<T, INTERP, PAD, ALIGN>), dim3(blocks_for(total, kDirectThreads)),
+                           dim3(kDirectThreads), 0, stream, (const T*)a.grid, taps, total, (int32_t)a.Hin,
+                           (int32_t)a.Win);
+        return hipGetLastError();
+    }
+}
+
+template <typename T, int INTERP, int PAD, bool ALIGN>
+hipError_t run_bicubic_taps(const GridSamplerArgs& a, BicubicTapRecord* taps, hipStream_t stream)
+{
+    const int64_t total = a.N * a.Hout * a.Wout;
+    hipLaunchKernelGGL((gs2d_bicubic_taps_kernel<T, PAD, ALIGN>), dim3(blocks_for(total, kDirectThreads)),
                        dim3(kDirectThreads), 0, stream, (const T*)a.grid, taps, total, (int32_t)a.Hin,
                        (int32_t)a.Win);
     return hipGetLastError();
@@ -171,6 +251,17 @@ struct TapsLauncher {
     hipError_t operator()() const
     {
         return run_taps<T, I, P, A>(a, taps, stream);
+    }
+};
+
+struct BicubicTapsLauncher {
+    const GridSamplerArgs& a;
+    BicubicTapRecord* taps;
+    hipStream_t stream;
+    template <typename T, int I, int P, bool A>
+    hipError_t operator()() const
+    {
+        return run_bicubic_taps<T, I, P, A>(a, taps, stream);
     }
 };
 
@@ -198,7 +289,7 @@ const char* grid_sampler2d_variant(const GridSamplerArgs& a)
 
 hipError_t launch_grid_sampler2d(const GridSamplerArgs& a, hipStream_t stream)
 {
-    if (!gs_shapes_ok(a) || a.interp < 0 || a.interp > 1 || a.pad < 0 || a.pad > 2) {
+    if (!gs_shapes_ok(a) || a.interp < 0 || a.interp > 2 || a.pad < 0 || a.pad > 2) {
         return hipErrorInvalidValue;
     }
     if (a.N == 0 || a.C == 0 || a.Hout == 0 || a.Wout == 0) {
@@ -229,6 +320,20 @@ hipError_t launch_grid_sampler2d_taps(const GridSamplerArgs& a, TapRecord* taps,
         return hipErrorInvalidValue;
     }
     return dispatch_elem(a, TapsLauncher{a, taps, stream});
+}
+
+hipError_t launch_grid_sampler2d_bicubic_taps(const GridSamplerArgs& a, BicubicTapRecord* taps, hipStream_t stream)
+{
+    if (!gs_shapes_ok(a) || a.interp != 2 || a.pad < 0 || a.pad > 2) {
+        return hipErrorInvalidValue;
+    }
+    if (a.N == 0 || a.Hout == 0 || a.Wout == 0) {
+        return hipSuccess;
+    }
+    if (a.grid == nullptr || taps == nullptr) {
+        return hipErrorInvalidValue;
+    }
+    return dispatch_elem(a, BicubicTapsLauncher{a, taps, stream});
 }
 
 }  // namespace opscv

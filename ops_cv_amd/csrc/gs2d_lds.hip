@@ -28,6 +28,9 @@ LdsPlan make_lds_plan(const GridSamplerArgs& a)
     if (p.cls >= 2 && out_plane >= 32 * kThreads) {
         p.ppt = 8;
     }
+    if (a.interp == 2) {
+        p.ppt = (out_plane >= 4 * kThreads) ? 2 : 1;  // sixteen tap offsets per pixel live in registers
+    }
     const int64_t tile = (int64_t)kThreads * p.ppt;
     p.tiles_per_n = (uint32_t)((out_plane + tile - 1) / tile);
     // channels per workgroup: as many stages as possible (the pixel decisions are reused across them) while

@@ -4,8 +4,8 @@
 // image/grid_sampler2_d/op_kernel/arch35/grid_sampler2_d_simt.h:461-514), different data movement:
 //
 //   * a workgroup owns (batch n, a tile of THREADS*PPT output pixels, a range of channels);
-//   * every lane decides its PPT pixels once -- four LDS byte offsets and four weights per pixel stay in
-//     registers for the whole channel range;
+//   * every lane decides its PPT pixels once -- four LDS byte offsets and four weights per pixel (bicubic:
+//     sixteen offsets, eight coefficients) stay in registers for the whole channel range;
 //   * the channel range is walked in stages of CGS whole input planes.  The planes go from HBM straight into
 //     LDS with the asynchronous global->LDS loads of gfx950 (no registers, 16 bytes per lane, 1 KiB per
 //     wavefront instruction), double-buffered: stage s+1 is in flight while stage s is sampled;
@@ -74,9 +74,31 @@ __device__ __forceinline__ void load_taps(const char* plane, const uint32_t* tof
 // bit; fma(v, w, -0) is "v*w" bit for bit (also for zero products of either sign).  Writing the products as
 // fmas lets the 16-bit -> fp32 conversion ride on the multiply (mixed-precision fma) for fp16; `neg_zero` is
 // -0.0f handed in at run time so that the compiler cannot fold the fma back into a multiply.
+//
+// Bicubic (grid_sampler2_d_simt.h:362-371 and :418-455): raw[4*j + k] is the tap of row j, column k; tw[0..3] are
+// the column coefficients, tw[4..7] the row coefficients.  Each row is  c0*v0  followed by three fused
+// multiply-adds, and so is the column of the four row results.  A tap outside the image reads the zero slot; a
+// row outside the image therefore evaluates to +0 like the reference's literal 0 (the products are zeros and at
+// least one of the two middle coefficients is positive, so the sum cannot be -0).
 template <typename T, int INTERP>
 __device__ __forceinline__ float blend(const T* raw, const float* tw, float neg_zero)
 {
+    if (INTERP == 2) {
+        float r[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            float acc = __builtin_fmaf(ElemIO<T>::load(&raw[4 * j]), tw[0], neg_zero);
+            acc = __builtin_fmaf(tw[1], ElemIO<T>::load(&raw[4 * j + 1]), acc);
+            acc = __builtin_fmaf(tw[2], ElemIO<T>::load(&raw[4 * j + 2]), acc);
+            acc = __builtin_fmaf(tw[3], ElemIO<T>::load(&raw[4 * j + 3]), acc);
+            r[j] = acc;
+        }
+        float out = tw[4] * r[0];
+        out = __builtin_fmaf(tw[5], r[1], out);
+        out = __builtin_fmaf(tw[6], r[2], out);
+        out = __builtin_fmaf(tw[7], r[3], out);
+        return as_fp32_value(out);
+    }
     if (INTERP == 0) {
         float out = __builtin_fmaf(ElemIO<T>::load(&raw[0]), tw[0], 0.0f);
         out += __builtin_fmaf(ElemIO<T>::load(&raw[1]), tw[1], neg_zero);
@@ -186,7 +208,8 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
 {
     extern __shared__ uint4 smem_raw[];
     char* lds = reinterpret_cast<char*>(smem_raw);
-    constexpr int NT = (INTERP == 0) ? 4 : 1;
+    constexpr int NT = (INTERP == 0) ? 4 : (INTERP == 1 ? 1 : 16);  // taps per pixel
+    constexpr int NW = (INTERP == 2) ? 8 : 4;                        // weights per pixel
     constexpr int SLOT_BYTES = CGS * PITCH;
     constexpr int DEPTH = NBUF - 1;  // stages in flight ahead of the one being sampled
     constexpr int STHREADS = SWAVES * 64;
@@ -273,7 +296,7 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
 
     // per-pixel decisions, once for the whole channel range
     uint32_t toff[PPT][NT];
-    float tw[PPT][4];
+    float tw[PPT][NW];
     uint32_t pixoff[PPT];  // byte offset of the pixel inside an output plane; out of range for lanes past the end
 #pragma unroll
     for (int j = 0; j < PPT; j++) {
@@ -283,7 +306,26 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
         pixoff[j] = valid ? (uint32_t)pc * (uint32_t)sizeof(T) : 0x80000000u;
         float gx, gy;
         load_grid_pair<T>(grid + ((int64_t)n * out_plane + pc) * 2, pair_aligned != 0, &gx, &gy);
-        const PixelTap t = decide_pixel<INTERP, PAD, ALIGN>(gx, gy, H, W);
+        if constexpr (INTERP == 2) {
+            const BicubicTap b = decide_bicubic<PAD, ALIGN>(gx, gy, H, W);
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const bool row_in = b.by[r] >= 0 && b.by[r] < H && !b.flag;
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    const bool in = row_in && b.bx[k] >= 0 && b.bx[k] < W;
+                    toff[j][4 * r + k] =
+                        in ? ((uint32_t)b.by[r] * (uint32_t)W + (uint32_t)b.bx[k]) * (uint32_t)sizeof(T) : zero_off;
+                }
+                tw[j][r] = b.cx[r];
+                tw[j][4 + r] = b.cy[r];
+            }
+            if (b.flag) {
+                tw[j][0] = __builtin_nanf("");  // 0 * NaN: every channel becomes NaN, as the reference writes
+            }
+            continue;
+        }
+        const PixelTap t = decide_pixel<(INTERP == 2 ? 0 : INTERP), PAD, ALIGN>(gx, gy, H, W);
         if (INTERP == 0) {
             const int32_t x0 = t.x0, y0 = t.y0;
             const int32_t x1 = (x0 == INT32_MAX) ? x0 : x0 + 1;

@@ -71,6 +71,20 @@ struct LdsTypedLauncher {
     template <typename U, int I, int P, bool A>
     hipError_t operator()() const
     {
+        if constexpr (I == 2) {
+            // bicubic keeps sixteen tap offsets per pixel: one or two pixels per lane
+            switch (p.cls * 16 + p.ppt) {
+                case 0 * 16 + 1: return launch_cls<T, I, P, A, 0, 1>(a, p, stream);
+                case 0 * 16 + 2: return launch_cls<T, I, P, A, 0, 2>(a, p, stream);
+                case 1 * 16 + 1: return launch_cls<T, I, P, A, 1, 1>(a, p, stream);
+                case 1 * 16 + 2: return launch_cls<T, I, P, A, 1, 2>(a, p, stream);
+                case 2 * 16 + 1: return launch_cls<T, I, P, A, 2, 1>(a, p, stream);
+                case 2 * 16 + 2: return launch_cls<T, I, P, A, 2, 2>(a, p, stream);
+                case 3 * 16 + 1: return launch_cls<T, I, P, A, 3, 1>(a, p, stream);
+                case 3 * 16 + 2: return launch_cls<T, I, P, A, 3, 2>(a, p, stream);
+                default: return hipErrorInvalidValue;
+            }
+        }
         switch (p.cls * 16 + p.ppt) {
             case 0 * 16 + 1: return launch_cls<T, I, P, A, 0, 1>(a, p, stream);
             case 0 * 16 + 4: return launch_cls<T, I, P, A, 0, 4>(a, p, stream);

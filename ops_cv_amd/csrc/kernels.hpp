@@ -15,10 +15,20 @@ struct TapRecord {
     int32_t flag;
 };
 
+// Record of the bicubic mode (68 bytes, no padding).
+struct BicubicTapRecord {
+    int32_t bx[4];
+    int32_t by[4];
+    float cx[4];
+    float cy[4];
+    int32_t flag;
+};
+
 // All tensors contiguous.  Each launcher validates the shapes against what its kernels assume and
 // returns hipErrorInvalidValue instead of launching when they do not fit.
 hipError_t launch_grid_sampler2d(const GridSamplerArgs& a, hipStream_t stream);
 hipError_t launch_grid_sampler2d_taps(const GridSamplerArgs& a, TapRecord* taps, hipStream_t stream);
+hipError_t launch_grid_sampler2d_bicubic_taps(const GridSamplerArgs& a, BicubicTapRecord* taps, hipStream_t stream);
 hipError_t launch_resize(const ResizeArgs& a, hipStream_t stream);
 
 // gather == true : strided view -> contiguous buffer;  false : contiguous buffer -> strided view

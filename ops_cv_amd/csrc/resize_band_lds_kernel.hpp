@@ -175,10 +175,12 @@ __global__ __launch_bounds__(THREADS) void resize_band_lds_kernel(const T* __res
             }
             const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(yp, 0, out_row_bytes, kRsBufferFlags);
             typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+            u32x4 packed;
+            __builtin_memcpy(&packed, outv, sizeof(packed));
             if (p.streaming) {
-                __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4*>(outv), rsrc, (int)out_off, 0, 2);
+                __builtin_amdgcn_raw_buffer_store_b128(packed, rsrc, (int)out_off, 0, 2);
             } else {
-                __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4*>(outv), rsrc, (int)out_off, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b128(packed, rsrc, (int)out_off, 0, 0);
             }
             yp += p.Wd;
         }

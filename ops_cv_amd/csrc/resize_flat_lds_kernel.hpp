@@ -118,7 +118,9 @@ __global__ __launch_bounds__(THREADS) void resize_flat_lds_kernel(const T* __res
                 ElemIO<T>::store(&outv[i], omdy * top + dy * bot);
             }
             typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-            __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const u32x4*>(outv), rsrc,
+            u32x4 packed;
+            __builtin_memcpy(&packed, outv, sizeof(packed));
+            __builtin_amdgcn_raw_buffer_store_b128(packed, rsrc,
                                                    (int)((uint32_t)h * out_row_bytes + col_off), 0, 0);
         }
         __syncthreads();  // everybody is done with the staged rows before the next plane overwrites them

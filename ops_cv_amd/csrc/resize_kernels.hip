@@ -128,7 +128,9 @@ __global__ __launch_bounds__(kThreads) void resize_nchw_band_kernel(const T* __r
                 const float o = (1.0f - dy) * ha[i] + dy * bot;
                 ElemIO<T>::store(&outv[i], o);
             }
-            *reinterpret_cast<uint4*>(yp) = *reinterpret_cast<const uint4*>(outv);
+            uint4 packed;
+            __builtin_memcpy(&packed, outv, sizeof(packed));
+            *reinterpret_cast<uint4*>(yp) = packed;
             yp += Wd;
         }
     }

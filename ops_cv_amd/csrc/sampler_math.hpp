@@ -32,7 +32,9 @@ template <>
 struct ElemIO<__bf16> {
     static __device__ __forceinline__ float load(const __bf16* p)
     {
-        return __builtin_bit_cast(float, (uint32_t)(*(const uint16_t*)p) << 16);
+        // the object is read as what it is and its bits reinterpreted afterwards (reading it through a
+        // uint16_t lvalue would let the compiler reorder the read against writes of the __bf16 object)
+        return __builtin_bit_cast(float, (uint32_t)__builtin_bit_cast(uint16_t, *p) << 16);
     }
     static __device__ __forceinline__ void store(__bf16* p, float v) { *p = (__bf16)v; }
 };
@@ -72,11 +74,10 @@ __device__ __forceinline__ float reflect_coordinates(float coord, float low, flo
     return __builtin_fminf(extra, complement) + low;
 }
 
-// grid_sampler2_d_simt.h:187-207
+// grid_sampler2_d_simt.h:187-200
 template <int PAD, bool ALIGN>
-__device__ __forceinline__ float compute_source_index(float coord, int32_t size)
+__device__ __forceinline__ float compute_coordinates(float coord, int32_t size)
 {
-    coord = unnormalize<ALIGN>(coord, size);
     if (PAD == 1) {
         coord = clip_coordinates(coord, size);
     } else if (PAD == 2) {
@@ -88,6 +89,13 @@ __device__ __forceinline__ float compute_source_index(float coord, int32_t size)
         coord = clip_coordinates(coord, size);
     }
     return coord;
+}
+
+// grid_sampler2_d_simt.h:202-207
+template <int PAD, bool ALIGN>
+__device__ __forceinline__ float compute_source_index(float coord, int32_t size)
+{
+    return compute_coordinates<PAD, ALIGN>(unnormalize<ALIGN>(coord, size), size);
 }
 
 __device__ __forceinline__ bool nan_or_inf(float x) { return __builtin_isnan(x) || __builtin_isinf(x); }
@@ -168,6 +176,100 @@ __device__ __forceinline__ PixelTap decide_pixel(float gx, float gy, int32_t H, 
         t.x0 = banker_round(ix);
         t.y0 = banker_round(iy);
     }
+    return t;
+}
+
+// ---- bicubic mode (A = -0.75), grid_sampler2_d_simt.h:271-298 and :375-412 ----
+
+// every product, sum and difference rounds separately (the translation unit has contraction off)
+__device__ __forceinline__ float cubic_convolution1(float x, float a)
+{
+    float t0 = (a + 2.0f) * x;
+    float t1 = t0 - (a + 3.0f);
+    float t2 = t1 * x;
+    float t3 = t2 * x;
+    return t3 + 1.0f;
+}
+
+__device__ __forceinline__ float cubic_convolution2(float x, float a)
+{
+    float t0 = a * x;
+    float t1 = t0 - 5.0f * a;
+    float t2 = t1 * x;
+    float t3 = t2 + 8.0f * a;
+    float t4 = t3 * x;
+    return t4 - 4.0f * a;
+}
+
+__device__ __forceinline__ int32_t safe_float_to_i32(float f)
+{
+    if (f >= 0.0f && f < 2147483648.0f) {
+        return (int32_t)f;
+    }
+    return -1;
+}
+
+// Pins a value as an fp32 register.  The reference rounds the last fused multiply-add of the bicubic sum to fp32
+// and then converts to the 16-bit output type (two roundings); without this the compiler merges that
+// multiply-add and the conversion into one instruction that rounds once, which differs on exact ties.
+__device__ __forceinline__ float as_fp32_value(float v)
+{
+    asm volatile("" : "+v"(v));
+    return v;
+}
+
+// grid_sampler2_d_simt.h:362-371: a plain product, then three explicit fused multiply-adds
+__device__ __forceinline__ float bicubic_weighted_sum(float c0, float c1, float c2, float c3, float v0, float v1,
+                                                      float v2, float v3)
+{
+    float r = c0 * v0;
+    r = __builtin_fmaf(c1, v1, r);
+    r = __builtin_fmaf(c2, v2, r);
+    r = __builtin_fmaf(c3, v3, r);
+    return as_fp32_value(r);
+}
+
+struct BicubicTap {
+    int32_t bx[4], by[4];  // tap columns / rows after padding; -1 = outside
+    float cx[4], cy[4];    // column / row coefficients
+    int32_t flag;          // 1: write NaN to every channel (non-finite source coordinate)
+};
+
+// grid_sampler2_d_simt.h:499-503 (the coordinate is only unnormalized; padding applies to every tap) and :379-412
+template <int PAD, bool ALIGN>
+__device__ __forceinline__ BicubicTap decide_bicubic(float gx, float gy, int32_t H, int32_t W)
+{
+    constexpr float A = -0.75f;
+    BicubicTap t;
+    const float ix = unnormalize<ALIGN>(gx, W);
+    const float iy = unnormalize<ALIGN>(gy, H);
+    t.flag = 0;
+    if (nan_or_inf(ix) || nan_or_inf(iy)) {
+        t.flag = 1;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            t.bx[k] = t.by[k] = 0;
+            t.cx[k] = t.cy[k] = 0.0f;
+        }
+        return t;
+    }
+    const float ixf = __builtin_floorf(ix);
+    const float iyf = __builtin_floorf(iy);
+    const float tx = ix - ixf;
+    const float ty = iy - iyf;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        t.bx[k] = safe_float_to_i32(compute_coordinates<PAD, ALIGN>(ixf + (float)(k - 1), W));
+        t.by[k] = safe_float_to_i32(compute_coordinates<PAD, ALIGN>(iyf + (float)(k - 1), H));
+    }
+    t.cx[0] = cubic_convolution2(tx + 1.0f, A);
+    t.cx[1] = cubic_convolution1(tx, A);
+    t.cx[2] = cubic_convolution1(1.0f - tx, A);
+    t.cx[3] = cubic_convolution2(2.0f - tx, A);
+    t.cy[0] = cubic_convolution2(ty + 1.0f, A);
+    t.cy[1] = cubic_convolution1(ty, A);
+    t.cy[2] = cubic_convolution1(1.0f - ty, A);
+    t.cy[3] = cubic_convolution2(2.0f - ty, A);
     return t;
 }
 

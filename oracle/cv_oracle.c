@@ -15,6 +15,9 @@
  *                                  (image/grid_sample/examples/test_aclnn_grid_sample2_d.cpp:96-98), identity
  *                                  grid of image/grid_sampler2_d/examples/arch35/test_geir_grid_sampler2_d.cpp:84-90,
  *                                  committed torch.nn.functional.grid_sample fixtures, live torch CPU comparison
+ *   bicubic mode (interp 2)      : coefficient closed forms (t=0 -> 0,1,0,0; partition of unity; symmetry),
+ *                                  identity grid, committed and live torch grid_sample(mode="bicubic") comparison,
+ *                                  integer-coordinate samples reproduce the source pixel
  *   oracle_upsample_bilinear2d   : known answers for image/upsample_bilinear2d/examples/
  *                                  test_aclnn_upsample_bilinear2d.cpp:83-94, kernel-UT shapes (1,1,1,4)->(2,16),
  *                                  (3,16), committed torch interpolate fixtures, live torch CPU comparison
@@ -182,10 +185,9 @@ float oracle_reflect_coordinates(float coord, float low, float twice_span)
     return fminf(extra, complement) + low;
 }
 
-/* grid_sampler2_d_simt.h:187-207 */
-float oracle_compute_source_index(float coord, int32_t size, int32_t padding_mode, int32_t align_corners)
+/* grid_sampler2_d_simt.h:187-200 */
+float oracle_compute_coordinates(float coord, int32_t size, int32_t padding_mode, int32_t align_corners)
 {
-    coord = oracle_unnormalize(coord, size, align_corners);
     if (padding_mode == 1) {
         coord = oracle_clip_coordinates(coord, size);
     } else if (padding_mode == 2) {
@@ -197,6 +199,13 @@ float oracle_compute_source_index(float coord, int32_t size, int32_t padding_mod
         coord = oracle_clip_coordinates(coord, size);
     }
     return coord;
+}
+
+/* grid_sampler2_d_simt.h:202-207 */
+float oracle_compute_source_index(float coord, int32_t size, int32_t padding_mode, int32_t align_corners)
+{
+    coord = oracle_unnormalize(coord, size, align_corners);
+    return oracle_compute_coordinates(coord, size, padding_mode, align_corners);
 }
 
 /* grid_sampler2_d_simt.h:209-215 ; 2147483646.0f is 2^31 once rounded to fp32 */
@@ -275,6 +284,95 @@ static inline void gs_decide(float gx, float gy, int32_t Hin, int32_t Win, int i
     }
 }
 
+/* ---- bicubic (A = -0.75) ---- */
+
+/* grid_sampler2_d_simt.h:273-280 : every product, sum and difference rounded separately */
+float oracle_cubic_convolution1(float x, float a)
+{
+    float t0 = (a + 2.0f) * x;
+    float t1 = t0 - (a + 3.0f);
+    float t2 = t1 * x;
+    float t3 = t2 * x;
+    return t3 + 1.0f;
+}
+
+/* grid_sampler2_d_simt.h:282-290 */
+float oracle_cubic_convolution2(float x, float a)
+{
+    float t0 = a * x;
+    float t1 = t0 - 5.0f * a;
+    float t2 = t1 * x;
+    float t3 = t2 + 8.0f * a;
+    float t4 = t3 * x;
+    return t4 - 4.0f * a;
+}
+
+/* grid_sampler2_d_simt.h:292-298 */
+static inline int32_t safe_float_to_i32(float f)
+{
+    if (f >= 0.0f && f < 2147483648.0f) {
+        return (int32_t)f;
+    }
+    return -1;
+}
+
+/* grid_sampler2_d_simt.h:362-371 : plain product, then three explicit fused multiply-adds */
+static inline float bicubic_weighted_sum(float c0, float c1, float c2, float c3, float v0, float v1, float v2,
+                                         float v3)
+{
+    float r = c0 * v0;
+    r = fmaf(c1, v1, r);
+    r = fmaf(c2, v2, r);
+    r = fmaf(c3, v3, r);
+    return r;
+}
+
+/* grid_sampler2_d_simt.h:499-503 (coordinates) and :379-412 (taps and coefficients) */
+static inline void gs_decide_bicubic(float gx, float gy, int32_t Hin, int32_t Win, int pad, int align,
+                                     oracle_gs_bicubic_tap* t)
+{
+    const float A = -0.75f;
+    float ix = oracle_unnormalize(gx, Win, align);
+    float iy = oracle_unnormalize(gy, Hin, align);
+    memset(t, 0, sizeof(*t));
+    if (isnan(ix) || isinf(ix) || isnan(iy) || isinf(iy)) {
+        t->flag = 1;
+        return;
+    }
+    float ixf = floorf(ix);
+    float iyf = floorf(iy);
+    float tx = ix - ixf;
+    float ty = iy - iyf;
+    for (int k = 0; k < 4; k++) {
+        t->bx[k] = safe_float_to_i32(oracle_compute_coordinates(ixf + (float)(k - 1), Win, pad, align));
+        t->by[k] = safe_float_to_i32(oracle_compute_coordinates(iyf + (float)(k - 1), Hin, pad, align));
+    }
+    t->cx[0] = oracle_cubic_convolution2(tx + 1.0f, A);
+    t->cx[1] = oracle_cubic_convolution1(tx, A);
+    t->cx[2] = oracle_cubic_convolution1(1.0f - tx, A);
+    t->cx[3] = oracle_cubic_convolution2(2.0f - tx, A);
+    t->cy[0] = oracle_cubic_convolution2(ty + 1.0f, A);
+    t->cy[1] = oracle_cubic_convolution1(ty, A);
+    t->cy[2] = oracle_cubic_convolution1(1.0f - ty, A);
+    t->cy[3] = oracle_cubic_convolution2(2.0f - ty, A);
+}
+
+int oracle_grid_sampler2d_bicubic_taps(const void* grid, oracle_gs_bicubic_tap* taps, int dtype, int64_t N,
+                                       int64_t Hin, int64_t Win, int64_t Hout, int64_t Wout, int padding_mode,
+                                       int align_corners)
+{
+    if (padding_mode < 0 || padding_mode > 2 || dtype < 0 || dtype > 2) {
+        return -1;
+    }
+    int64_t total = N * Hout * Wout;
+    for (int64_t p = 0; p < total; p++) {
+        float gx = load_as_float(grid, dtype, 2 * p);
+        float gy = load_as_float(grid, dtype, 2 * p + 1);
+        gs_decide_bicubic(gx, gy, (int32_t)Hin, (int32_t)Win, padding_mode, align_corners, &taps[p]);
+    }
+    return 0;
+}
+
 int oracle_grid_sampler2d_taps(const void* grid, oracle_gs_tap* taps, int dtype, int64_t N, int64_t Hin,
                                int64_t Win, int64_t Hout, int64_t Wout, int interp_mode, int padding_mode,
                                int align_corners)
@@ -295,7 +393,7 @@ int oracle_grid_sampler2d(const void* x, const void* grid, void* y, int dtype, i
                           int64_t Win, int64_t Hout, int64_t Wout, int interp_mode, int padding_mode,
                           int align_corners, int num_threads)
 {
-    if (interp_mode < 0 || interp_mode > 1 || padding_mode < 0 || padding_mode > 2 || dtype < 0 || dtype > 2) {
+    if (interp_mode < 0 || interp_mode > 2 || padding_mode < 0 || padding_mode > 2 || dtype < 0 || dtype > 2) {
         return -1;
     }
     if (Hin <= 0 || Win <= 0 || Hin > INT32_MAX || Win > INT32_MAX) {
@@ -321,10 +419,41 @@ int oracle_grid_sampler2d(const void* x, const void* grid, void* y, int dtype, i
         int64_t h_out = hw - n * Hout;
         float gx = load_as_float(grid, dtype, 2 * p);
         float gy = load_as_float(grid, dtype, 2 * p + 1);
-        oracle_gs_tap t;
-        gs_decide(gx, gy, H, W, interp_mode, padding_mode, align_corners, &t);
         int64_t x_base = n * C * x_step;
         int64_t y_base = n * C * y_step + h_out * Wout + w_out;
+        if (interp_mode == 2) {
+            oracle_gs_bicubic_tap b;
+            gs_decide_bicubic(gx, gy, H, W, padding_mode, align_corners, &b);
+            if (b.flag) {
+                for (int64_t c = 0; c < C; c++) {
+                    store_from_float(y, dtype, y_base, NAN);
+                    y_base += y_step;
+                }
+                continue;
+            }
+            /* grid_sampler2_d_simt.h:418-455 : a row outside the image contributes 0, a column outside reads 0 */
+            for (int64_t c = 0; c < C; c++) {
+                float r[4];
+                for (int j = 0; j < 4; j++) {
+                    r[j] = 0.0f;
+                    if (b.by[j] >= 0 && b.by[j] < H) {
+                        int64_t off = x_base + (int64_t)b.by[j] * W;
+                        float v[4];
+                        for (int k = 0; k < 4; k++) {
+                            v[k] = (b.bx[k] >= 0 && b.bx[k] < W) ? load_as_float(x, dtype, off + b.bx[k]) : 0.0f;
+                        }
+                        r[j] = bicubic_weighted_sum(b.cx[0], b.cx[1], b.cx[2], b.cx[3], v[0], v[1], v[2], v[3]);
+                    }
+                }
+                float out = bicubic_weighted_sum(b.cy[0], b.cy[1], b.cy[2], b.cy[3], r[0], r[1], r[2], r[3]);
+                store_from_float(y, dtype, y_base, out);
+                x_base += x_step;
+                y_base += y_step;
+            }
+            continue;
+        }
+        oracle_gs_tap t;
+        gs_decide(gx, gy, H, W, interp_mode, padding_mode, align_corners, &t);
         if (t.flag) {
             /* grid_sampler2_d_simt.h:236-247 */
             float nan_val = NAN;

@@ -7,7 +7,7 @@
  * entry and the benchmark's "cpu_baseline" leg call it.
  *
  * Reference sources followed (paths relative to the reference tree):
- *   grid sample : image/grid_sampler2_d/op_kernel/arch35/grid_sampler2_d_simt.h
+ *   grid sample : image/grid_sampler2_d/op_kernel/arch35/grid_sampler2_d_simt.h (bilinear, nearest, bicubic)
  *   upsample    : image/resize_bilinear_v2/op_kernel/arch35/resize_bilinear_v2_simt_nchw.h
  *   scale rules : image/resize_bilinear_v2/op_host/arch35/resize_bilinear_v2_tiling_arch35.cpp:175-243
  *
@@ -50,6 +50,25 @@ typedef struct {
     float w[4];
     int32_t flag;
 } oracle_gs_tap;
+
+/*
+ * Per-pixel record of the bicubic mode (grid_sampler2_d_simt.h:375-403): the four tap columns and rows after
+ * padding (-1 = outside), the four column and row coefficients, flag = 1 when the pixel is written as NaN.
+ */
+typedef struct {
+    int32_t bx[4];
+    int32_t by[4];
+    float cx[4];
+    float cy[4];
+    int32_t flag;
+} oracle_gs_bicubic_tap;
+
+float oracle_compute_coordinates(float coord, int32_t size, int32_t padding_mode, int32_t align_corners);
+float oracle_cubic_convolution1(float x, float a);
+float oracle_cubic_convolution2(float x, float a);
+int oracle_grid_sampler2d_bicubic_taps(const void* grid, oracle_gs_bicubic_tap* taps, int dtype, int64_t N,
+                                       int64_t Hin, int64_t Win, int64_t Hout, int64_t Wout, int padding_mode,
+                                       int align_corners);
 
 /* ---- whole-tensor entry points; all tensors contiguous, NCHW, grid is (N,Ho,Wo,2) ---- */
 

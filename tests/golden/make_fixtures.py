@@ -79,6 +79,28 @@ def main():
                     out["h_%s_y_m%d_p%d_a%d" % (name, m, p, a)] = y.view(torch.int16).numpy().view(np.uint16)
     np.savez_compressed(os.path.join(HERE, "grid_sampler2d.npz"), **out)
 
+    # ---- bicubic mode on the same inputs (outputs only; inputs are read from grid_sampler2d.npz) ----
+    bic = {}
+    for key in sorted(out):
+        if not key.endswith("_x") or key == "fma_x":
+            continue
+        stem = key[:-2]
+        x, g = out[key], out[stem + "_grid"]
+        if stem.startswith("h_"):
+            dt = torch.float16 if stem == "h_f16" else torch.bfloat16
+            xt = torch.from_numpy(x.view(np.int16)).view(dt)
+            gt = torch.from_numpy(g.view(np.int16)).view(dt)
+        for p in range(3):
+            for a in (0, 1):
+                if stem.startswith("h_"):
+                    y = F.grid_sample(xt.float(), gt.float(), mode="bicubic", padding_mode=PADS[p],
+                                      align_corners=bool(a)).to(dt).view(torch.int16).numpy().view(np.uint16)
+                else:
+                    y = F.grid_sample(torch.from_numpy(x), torch.from_numpy(g), mode="bicubic", padding_mode=PADS[p],
+                                      align_corners=bool(a)).numpy()
+                bic["%s_y_m2_p%d_a%d" % (stem, p, a)] = y
+    np.savez_compressed(os.path.join(HERE, "grid_sampler2d_bicubic.npz"), **bic)
+
     # ---- upsample ----
     up = {}
     cases = [((1, 1, 4, 2), (8, 4)), ((2, 3, 7, 9), (14, 18)), ((1, 2, 5, 5), (13, 7)), ((2, 2, 16, 16), (5, 3)),

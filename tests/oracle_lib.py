@@ -22,6 +22,8 @@ class GsTap(ctypes.Structure):
 
 
 TAP_DTYPE = np.dtype([("ix0", "<i4"), ("iy0", "<i4"), ("w", "<f4", (4,)), ("flag", "<i4")])
+BICUBIC_TAP_DTYPE = np.dtype([("bx", "<i4", (4,)), ("by", "<i4", (4,)), ("cx", "<f4", (4,)), ("cy", "<f4", (4,)),
+                              ("flag", "<i4")])
 
 
 def build(force=False):
@@ -67,6 +69,15 @@ def lib():
     L.oracle_grid_sampler2d_taps.restype = ctypes.c_int
     L.oracle_grid_sampler2d_taps.argtypes = [vp, vp, ctypes.c_int, i64, i64, i64, i64, i64, ctypes.c_int,
                                              ctypes.c_int, ctypes.c_int]
+    L.oracle_compute_coordinates.restype = f32
+    L.oracle_compute_coordinates.argtypes = [f32, i32, i32, i32]
+    L.oracle_cubic_convolution1.restype = f32
+    L.oracle_cubic_convolution1.argtypes = [f32, f32]
+    L.oracle_cubic_convolution2.restype = f32
+    L.oracle_cubic_convolution2.argtypes = [f32, f32]
+    L.oracle_grid_sampler2d_bicubic_taps.restype = ctypes.c_int
+    L.oracle_grid_sampler2d_bicubic_taps.argtypes = [vp, vp, ctypes.c_int, i64, i64, i64, i64, i64, ctypes.c_int,
+                                                     ctypes.c_int]
     L.oracle_resize_scale.restype = f32
     L.oracle_resize_scale.argtypes = [i64, i64, ctypes.c_int, f32]
     L.oracle_upsample_bilinear2d.restype = ctypes.c_int
@@ -118,6 +129,18 @@ def grid_sampler2d_taps(grid, H, W, interp=0, pad=0, align=False, dtype=None):
                                           int(bool(align)))
     if rc != 0:
         raise ValueError("oracle_grid_sampler2d_taps rc=%d" % rc)
+    return taps
+
+
+def grid_sampler2d_bicubic_taps(grid, H, W, pad=0, align=False, dtype=None):
+    grid = np.ascontiguousarray(grid)
+    code = _code_of(grid) if dtype is None else dtype
+    N, Ho, Wo, _ = grid.shape
+    taps = np.zeros((N, Ho, Wo), dtype=BICUBIC_TAP_DTYPE)
+    rc = lib().oracle_grid_sampler2d_bicubic_taps(_ptr(grid), _ptr(taps), code, N, H, W, Ho, Wo, pad,
+                                                  int(bool(align)))
+    if rc != 0:
+        raise ValueError("oracle_grid_sampler2d_bicubic_taps rc=%d" % rc)
     return taps
 
 

@@ -75,7 +75,7 @@ def test_grid_sampler_success_cases(aclnn, desc):
     assert _gs(aclnn, desc, fmts=(aclnn.ACL_FORMAT_NCHW, aclnn.ACL_FORMAT_NHWC, aclnn.ACL_FORMAT_ND))[0] == 0
     assert _gs(aclnn, desc, fmts=(aclnn.ACL_FORMAT_HWCN, aclnn.ACL_FORMAT_NCHW, aclnn.ACL_FORMAT_ND))[0] == 0
     assert _gs(aclnn, desc, interp=1, pad=1, fmts=(aclnn.ACL_FORMAT_NCHW, aclnn.ACL_FORMAT_NHWC, None))[0] == 0
-    for interp in (0, 1):
+    for interp in (0, 1, 2):
         for pad in (0, 1, 2):
             for align in (False, True):
                 assert _gs(aclnn, desc, interp=interp, pad=pad, align=align)[0] == 0
@@ -120,8 +120,8 @@ def test_grid_sampler_attr_and_shape_checks(aclnn, desc):
     assert b"dtype" in L.aclGetRecentErrMsg()
     _gs(aclnn, desc, interp=7, grid=(2, 3, 3, 2))
     assert b"interpolationMode" in L.aclGetRecentErrMsg()
-    # bicubic is in the validated range but outside this implementation
-    assert _gs(aclnn, desc, interp=2)[0] == 161002
+    # bicubic is the third supported mode
+    assert _gs(aclnn, desc, interp=2)[0] == 0
 
 
 def test_grid_sampler_empty_and_views(aclnn, desc):

@@ -11,7 +11,7 @@ import inputs as I
 
 pytestmark = pytest.mark.gpu
 
-INTERP = {0: "bilinear", 1: "nearest"}
+INTERP = {0: "bilinear", 1: "nearest", 2: "bicubic"}
 PAD = {0: "zeros", 1: "border", 2: "reflection"}
 
 
@@ -40,6 +40,17 @@ def _check(y_gpu, y_ref, dtype, interp, what):
             what, bad.sum(), (np.abs(a - b) / np.maximum(np.abs(b), 1e-2)).max())
 
 
+def _assert_same_bits(y_gpu, y_ref, what):
+    """The kernels keep the oracle's operation order and rounding, so outside NaN (whose sign and payload are not
+    part of the contract) every output has to carry the same bits."""
+    nan = np.isnan(I.as_f32(y_ref, "fp16" if y_ref.dtype == np.float16 else ("fp32" if y_ref.dtype == np.float32
+                                                                             else "bf16")))
+    view = np.uint32 if y_ref.dtype == np.float32 else np.uint16
+    a = np.where(nan, 0, y_gpu.view(view))
+    b = np.where(nan, 0, y_ref.view(view))
+    assert np.array_equal(a, b), "%s: %d outputs differ in their bits" % (what, (a != b).sum())
+
+
 def _run_gs(oracle, device, x32, g32, dtype, interp, pad, align):
     from ops_cv_amd import aclnn
     x = I.cast_np(x32, dtype)
@@ -52,7 +63,7 @@ def _run_gs(oracle, device, x32, g32, dtype, interp, pad, align):
 
 
 @pytest.mark.parametrize("dtype", I.DTYPES)
-@pytest.mark.parametrize("interp", [0, 1])
+@pytest.mark.parametrize("interp", [0, 1, 2])
 @pytest.mark.parametrize("pad", [0, 1, 2])
 @pytest.mark.parametrize("align", [False, True])
 def test_grid_sampler_random(oracle, device, dtype, interp, pad, align):
@@ -64,10 +75,11 @@ def test_grid_sampler_random(oracle, device, dtype, interp, pad, align):
         y, y_ref = _run_gs(oracle, device, x32, g32, dtype, interp, pad, align)
         _check(y, y_ref, dtype, interp, "gs %s %s %s align=%s %s" % (dtype, INTERP[interp], PAD[pad], align,
                                                                       (N, C, H, W, Ho, Wo)))
+        _assert_same_bits(y, y_ref, "gs %s %s %s align=%s" % (dtype, INTERP[interp], PAD[pad], align))
 
 
 @pytest.mark.parametrize("dtype", I.DTYPES)
-@pytest.mark.parametrize("interp", [0, 1])
+@pytest.mark.parametrize("interp", [0, 1, 2])
 def test_grid_sampler_large_planes(oracle, device, dtype, interp):
     """input planes of 20-160 KB and output planes of several tiles with a ragged last one: the staged variants
     that keep eight pixels per lane, and the largest plane class"""
@@ -78,12 +90,11 @@ def test_grid_sampler_large_planes(oracle, device, dtype, interp):
         g32 = rng.uniform(-1.1, 1.1, (N, Ho, Wo, 2)).astype(np.float32)
         y, y_ref = _run_gs(oracle, device, x32, g32, dtype, interp, pad, align)
         _check(y, y_ref, dtype, interp, "gs-large %s %s %s" % (dtype, INTERP[interp], (N, C, H, W, Ho, Wo)))
-        if dtype == "fp32":
-            assert np.array_equal(y.view(np.uint32), y_ref.view(np.uint32))
+        _assert_same_bits(y, y_ref, "gs-large %s %s" % (dtype, INTERP[interp]))
 
 
 @pytest.mark.parametrize("dtype", I.DTYPES)
-@pytest.mark.parametrize("interp", [0, 1])
+@pytest.mark.parametrize("interp", [0, 1, 2])
 @pytest.mark.parametrize("pad", [0, 1, 2])
 @pytest.mark.parametrize("align", [False, True])
 def test_grid_sampler_special_coordinates(oracle, device, dtype, interp, pad, align):
@@ -117,6 +128,29 @@ def test_grid_sampler_taps_bit_exact(oracle, device, dtype, interp, pad, align):
             assert np.array_equal(got["ix0"][live], ref["ix0"][live])
             assert np.array_equal(got["iy0"][live], ref["iy0"][live])
             assert np.array_equal(got["w"][live].view(np.uint32), ref["w"][live].view(np.uint32))
+
+
+@pytest.mark.parametrize("dtype", I.DTYPES)
+@pytest.mark.parametrize("pad", [0, 1, 2])
+@pytest.mark.parametrize("align", [False, True])
+def test_grid_sampler_bicubic_taps_bit_exact(oracle, device, dtype, pad, align):
+    """bicubic: the four tap columns and rows after padding, the eight coefficients and the NaN flag equal the
+    oracle's, bit for bit"""
+    from ops_cv_amd import aclnn
+    rng = np.random.default_rng(12)
+    grids = [I.special_grid(), rng.uniform(-1.5, 1.5, (2, 37, 41, 2)).astype(np.float32),
+             I.affine_grid(rng, 3, 64, 64)]
+    for g32 in grids:
+        for (H, W) in [(5, 8), (10, 10), (64, 64), (1080, 1920), (3, 1)]:
+            g = I.cast_np(g32, dtype)
+            ref = oracle.grid_sampler2d_bicubic_taps(g, H, W, pad, align, dtype=I.oracle_code(dtype))
+            got = aclnn.grid_sampler2d_bicubic_taps(I.to_torch(g, dtype, device), H, W, pad, align)
+            assert np.array_equal(got["flag"], ref["flag"])
+            live = ref["flag"] == 0
+            for f in ("bx", "by"):
+                assert np.array_equal(got[f][live], ref[f][live]), f
+            for f in ("cx", "cy"):
+                assert np.array_equal(got[f][live].view(np.uint32), ref[f][live].view(np.uint32)), f
 
 
 def _run_up(oracle, device, x32, out_hw, dtype, align, sh=0.0, sw=0.0):

@@ -294,6 +294,110 @@ def test_resize_scale_bit_patterns(oracle, case):
 
 
 # ------------------------------------------------------------------------------------------ live PyTorch CPU
+def test_bicubic_coefficients_closed_forms(oracle):
+    """grid_sampler2_d_simt.h:271-290: at t = 0 the coefficients are exactly (0, 1, 0, 0), they form a partition
+    of unity, and they are those of the Keys kernel with A = -0.75 evaluated in double precision"""
+    L = oracle.lib()
+    A = np.float32(-0.75)
+    assert L.oracle_cubic_convolution1(0.0, A) == 1.0
+    assert L.oracle_cubic_convolution1(1.0, A) == 0.0
+    assert L.oracle_cubic_convolution2(1.0, A) == 0.0
+    assert L.oracle_cubic_convolution2(2.0, A) == 0.0
+
+    def keys(d, a=-0.75):
+        d = abs(d)
+        if d <= 1:
+            return (a + 2) * d ** 3 - (a + 3) * d ** 2 + 1
+        if d < 2:
+            return a * d ** 3 - 5 * a * d ** 2 + 8 * a * d - 4 * a
+        return 0.0
+
+    for t in np.linspace(0, 1, 257, dtype=np.float32)[:-1]:
+        t = np.float32(t)
+        c = [L.oracle_cubic_convolution2(np.float32(t + np.float32(1)), A), L.oracle_cubic_convolution1(t, A),
+             L.oracle_cubic_convolution1(np.float32(np.float32(1) - t), A),
+             L.oracle_cubic_convolution2(np.float32(np.float32(2) - t), A)]
+        want = [keys(float(t) + 1), keys(float(t)), keys(1 - float(t)), keys(2 - float(t))]
+        assert np.allclose(c, want, atol=1e-6)
+        assert abs(sum(c) - 1.0) < 1e-6
+
+
+def test_bicubic_taps_and_identity(oracle):
+    """tap columns are floor-1 .. floor+2 passed through the padding rule; integer coordinates reproduce the
+    source pixel exactly (coefficients 0,1,0,0)"""
+    rng = np.random.default_rng(31)
+    H, W = 6, 9
+    x = rng.standard_normal((1, 2, H, W)).astype(np.float32)
+    # identity grid with align_corners=True lands on integer source coordinates
+    ys, xs = np.meshgrid(np.arange(H, dtype=np.float32), np.arange(W, dtype=np.float32), indexing="ij")
+    g = np.stack([xs * 2 / (W - 1) - 1, ys * 2 / (H - 1) - 1], axis=-1)[None].astype(np.float32)
+    for pad in range(3):
+        taps = oracle.grid_sampler2d_bicubic_taps(g, H, W, pad, True)
+        y = oracle.grid_sampler2d(x, g, 2, pad, True)
+        exact = (taps["cx"][..., 1] == 1.0) & (taps["cy"][..., 1] == 1.0)
+        assert exact.mean() > 0.3   # where the unnormalized coordinate is exactly an integer
+        assert np.array_equal(y[0, :, exact[0]], x[0, :, exact[0]])
+        assert np.abs(y - x).max() < 1e-5
+    # zeros padding: columns/rows outside are -1; border: clamped; reflection(align=True): mirrored about 0 and W-1
+    g1 = np.array([[[[-1.0, -1.0]]]], dtype=np.float32)   # source coordinate (0, 0) with align_corners=True
+    t = oracle.grid_sampler2d_bicubic_taps(g1, H, W, 0, True)[0, 0, 0]
+    assert list(t["bx"]) == [-1, 0, 1, 2] and list(t["by"]) == [-1, 0, 1, 2]
+    t = oracle.grid_sampler2d_bicubic_taps(g1, H, W, 1, True)[0, 0, 0]
+    assert list(t["bx"]) == [0, 0, 1, 2] and list(t["by"]) == [0, 0, 1, 2]
+    t = oracle.grid_sampler2d_bicubic_taps(g1, H, W, 2, True)[0, 0, 0]
+    assert list(t["bx"]) == [1, 0, 1, 2] and list(t["by"]) == [1, 0, 1, 2]
+    g2 = np.array([[[[1.0, 1.0]]]], dtype=np.float32)     # source coordinate (W-1, H-1)
+    t = oracle.grid_sampler2d_bicubic_taps(g2, H, W, 0, True)[0, 0, 0]
+    assert list(t["bx"]) == [W - 2, W - 1, W, W + 1]      # only negative columns become -1; >= W fails the bounds test
+    t = oracle.grid_sampler2d_bicubic_taps(g2, H, W, 2, True)[0, 0, 0]
+    assert list(t["bx"]) == [W - 2, W - 1, W - 2, W - 3]
+    # non-finite coordinate: NaN in every channel
+    g3 = np.array([[[[np.nan, 0.0], [0.0, np.inf]]]], dtype=np.float32)
+    assert np.isnan(oracle.grid_sampler2d(x, g3, 2, 0, False)).all()
+
+
+def test_bicubic_against_committed_fixtures(oracle):
+    z = np.load(os.path.join(GOLD, "grid_sampler2d.npz"))
+    b = np.load(os.path.join(GOLD, "grid_sampler2d_bicubic.npz"))
+    for prefix, count in (("gs", 4), ("sp", 3)):
+        for si in range(count):
+            x, g = z["%s%d_x" % (prefix, si)], z["%s%d_grid" % (prefix, si)]
+            for p in range(3):
+                for a in (0, 1):
+                    want = b["%s%d_y_m2_p%d_a%d" % (prefix, si, p, a)]
+                    got = oracle.grid_sampler2d(x, g, 2, p, bool(a))
+                    assert np.array_equal(np.isnan(got), np.isnan(want)), (prefix, si, p, a)
+                    w, q = np.nan_to_num(want), np.nan_to_num(got)
+                    assert np.abs(q - w).max() <= 4e-6 * max(1.0, np.abs(w).max()), (prefix, si, p, a)
+    for name, code in (("f16", oracle.F16), ("bf16", oracle.BF16)):
+        x, g = z["h_%s_x" % name], z["h_%s_grid" % name]
+        if name == "f16":
+            x, g = x.view(np.float16), g.view(np.float16)
+        for p in range(3):
+            for a in (0, 1):
+                want = b["h_%s_y_m2_p%d_a%d" % (name, p, a)]
+                got = oracle.grid_sampler2d(x, g, 2, p, bool(a), dtype=code).view(np.uint16)
+                assert np.abs(got.astype(np.int32) - want.astype(np.int32)).max() <= 1
+
+
+def test_live_torch_bicubic(oracle):
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(13)
+    for trial in range(8):
+        N, C = 2, 3
+        H, W = rng.integers(1, 40, 2)
+        Ho, Wo = rng.integers(1, 50, 2)
+        x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+        g = rng.uniform(-1.6, 1.6, (N, Ho, Wo, 2)).astype(np.float32)
+        for p in range(3):
+            for a in (False, True):
+                got = oracle.grid_sampler2d(x, g, 2, p, a)
+                want = F.grid_sample(torch.from_numpy(x), torch.from_numpy(g), mode="bicubic", padding_mode=PADS[p],
+                                     align_corners=a).numpy()
+                assert np.abs(got - want).max() <= 4e-6 * max(1.0, np.abs(want).max())
+
+
 def test_live_torch_grid_sample(oracle):
     import torch
     import torch.nn.functional as F
