@@ -99,6 +99,10 @@ def load_library():
                                                          vp, p_u64, p_vp]
     L.aclnnUpsampleBilinear2d.restype = i32
     L.aclnnUpsampleBilinear2d.argtypes = [vp, u64, vp, vp]
+    L.aclnnResizeGetWorkspaceSize.restype = i32
+    L.aclnnResizeGetWorkspaceSize.argtypes = [vp, vp, ctypes.c_char_p, vp, ctypes.POINTER(u64), ctypes.POINTER(vp)]
+    L.aclnnResize.restype = i32
+    L.aclnnResize.argtypes = [vp, u64, vp, vp]
     L.opscvGridSampler2DTaps.restype = i32
     L.opscvGridSampler2DTaps.argtypes = [vp, ctypes.c_int, i64, i64, i64, i64, i64, i64, i64, ctypes.c_bool, vp, vp]
     L.opscvGridSampler2DBicubicTaps.restype = i32
@@ -164,6 +168,25 @@ def get_workspace_size_upsample_bilinear2d(self_t, output_size, align_corners, s
     ex = ctypes.c_void_p(None)
     st = L.aclnnUpsampleBilinear2dGetWorkspaceSize(self_t, output_size, bool(align_corners), float(scales_h),
                                                    float(scales_w), out, ctypes.byref(ws), ctypes.byref(ex))
+    return st, ws.value, ex.value
+
+
+def create_float_array(values):
+    arr = (ctypes.c_float * len(values))(*[float(v) for v in values])
+    return load_library().aclCreateFloatArray(arr, len(values))
+
+
+def destroy_float_array(handle):
+    if handle:
+        load_library().aclDestroyFloatArray(handle)
+
+
+def get_workspace_size_resize(self_t, scales, mode, out):
+    """Phase 1 of aclnnResize on raw handles; `mode` is bytes or None."""
+    L = load_library()
+    ws = ctypes.c_uint64(0)
+    ex = ctypes.c_void_p(None)
+    st = L.aclnnResizeGetWorkspaceSize(self_t, scales, mode, out, ctypes.byref(ws), ctypes.byref(ex))
     return st, ws.value, ex.value
 
 
@@ -266,6 +289,37 @@ def upsample_bilinear2d(self_t, output_size, align_corners=False, scales_h=0.0, 
         for h in hs:
             destroy_tensor(h)
         destroy_int_array(size)
+    return out
+
+
+def resize(self_t, scales, mode="bilinear", out=None, stream=None, channels_last=False, workspace=None):
+    """Both phases of aclnnResize.  `scales` holds four floats in the order of the tensor's dimensions; the output
+    extents are trunc(in * scale).  Tensors are NCHW views, or NHWC views when channels_last."""
+    torch = _torch()
+    L = load_library()
+    fmt = ACL_FORMAT_NHWC if channels_last else ACL_FORMAT_NCHW
+    if out is None:
+        shape = list(self_t.shape)
+        for d in ((1, 2) if channels_last else (2, 3)):
+            shape[d] = int(float(self_t.shape[d]) * float(scales[d]))
+        out = torch.empty(shape, dtype=self_t.dtype, device=self_t.device)
+    hs = [tensor_handle(self_t, fmt), tensor_handle(out, fmt)]
+    sc = create_float_array(list(scales))
+    try:
+        st, ws, ex = get_workspace_size_resize(hs[0], sc, mode.encode(), hs[1])
+        if st != ACLNN_SUCCESS:
+            raise AclnnError("aclnnResizeGetWorkspaceSize", st)
+        if ws > 0 and (workspace is None or workspace.numel() * workspace.element_size() < ws):
+            workspace = torch.empty(ws, dtype=torch.uint8, device=self_t.device)
+        wptr = ctypes.c_void_p(workspace.data_ptr()) if ws > 0 else None
+        wsize = workspace.numel() * workspace.element_size() if ws > 0 else 0
+        st = L.aclnnResize(wptr, wsize, ex, _stream_handle(stream))
+        if st != ACLNN_SUCCESS:
+            raise AclnnError("aclnnResize", st)
+    finally:
+        for h in hs:
+            destroy_tensor(h)
+        destroy_float_array(sc)
     return out
 
 

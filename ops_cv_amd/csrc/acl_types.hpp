@@ -95,7 +95,7 @@ struct GridSamplerArgs {
     void* y = nullptr;
 };
 
-enum class ResizeMode : int { Bilinear = 0, Copy = 1, Broadcast = 2, FirstPixel = 3 };
+enum class ResizeMode : int { Bilinear = 0, Copy = 1, Broadcast = 2, FirstPixel = 3, Nearest = 4 };
 
 struct ResizeArgs {
     Elem elem = Elem::F32;

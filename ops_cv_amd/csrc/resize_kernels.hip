@@ -169,6 +169,68 @@ __global__ __launch_bounds__(kThreads) void resize_nhwc_generic_kernel(const T* 
     }
 }
 
+// Nearest-neighbour resize (align_corners = false, half_pixel_centers = false):
+//   src = min(floor(float(dst) * scale), len_src - 1)
+// image/resize_nearest_neighbor_v2/op_kernel/arch35/resize_nearest_neighbor_v2_simt.h:103-124.
+__device__ __forceinline__ int32_t nearest_src(int32_t d, float scale, int32_t len_src)
+{
+    const float f = __builtin_floorf((float)d * scale);
+    // the reference converts to an unsigned index and clamps from above only; dst and scale are non-negative
+    const int32_t i = (f >= 2147483648.0f) ? INT32_MAX : (int32_t)f;
+    return (i < len_src - 1) ? i : len_src - 1;
+}
+
+// A pure gather-copy: V = 16/sizeof(T) (VEC) or 1 output elements per lane along the contiguous axis.
+// NCHW: the contiguous axis is w, each element has its own source column.  NHWC: the contiguous axis is (w, c);
+// a vector never straddles a pixel because VEC requires C % V == 0.
+template <typename T, bool NHWC, bool VEC>
+__global__ __launch_bounds__(kThreads) void resize_nearest_kernel(const T* __restrict__ x, T* __restrict__ y,
+                                                                   int64_t outer, int32_t C, int32_t Hs, int32_t Ws,
+                                                                   int32_t Hd, int32_t Wd, float scale_h, float scale_w)
+{
+    constexpr int V = VEC ? 16 / (int)sizeof(T) : 1;
+    const int64_t row_elems = NHWC ? (int64_t)Wd * C : (int64_t)Wd;
+    const int64_t src_row_elems = NHWC ? (int64_t)Ws * C : (int64_t)Ws;
+    const int64_t e0 = ((int64_t)blockIdx.x * kThreads + threadIdx.x) * V;
+    if (e0 >= row_elems) {
+        return;
+    }
+    int64_t src_off[NHWC ? 1 : V];
+    if (NHWC) {
+        const int32_t w = (int32_t)(e0 / C);
+        const int32_t c = (int32_t)(e0 - (int64_t)w * C);
+        src_off[0] = (int64_t)nearest_src(w, scale_w, Ws) * C + c;
+    } else {
+#pragma unroll
+        for (int i = 0; i < V; i++) {
+            src_off[i] = nearest_src((int32_t)e0 + i, scale_w, Ws);
+        }
+    }
+    const int64_t rows = outer * Hd;  // outer = N*C planes (NCHW) or N images (NHWC)
+    for (int64_t r = blockIdx.y; r < rows; r += gridDim.y) {
+        const int64_t o = r / Hd;
+        const int32_t h = (int32_t)(r - o * Hd);
+        const T* src = x + (o * Hs + nearest_src(h, scale_h, Hs)) * src_row_elems;
+        T* dst = y + r * row_elems + e0;
+        if (VEC) {
+            uint4 packed;
+            if (NHWC) {
+                packed = *reinterpret_cast<const uint4*>(src + src_off[0]);
+            } else {
+                T v[V];
+#pragma unroll
+                for (int i = 0; i < V; i++) {
+                    v[i] = src[src_off[i]];
+                }
+                __builtin_memcpy(&packed, v, sizeof(packed));
+            }
+            *reinterpret_cast<uint4*>(dst) = packed;
+        } else {
+            dst[0] = src[src_off[0]];
+        }
+    }
+}
+
 // Broadcast of one source element per plane (mode Broadcast: 1x1 source; FirstPixel: 1x1 destination).
 // For NHWC the "plane" index is (n, c) with element stride C inside a batch.
 template <typename T>
@@ -228,6 +290,36 @@ hipError_t run_resize(const ResizeArgs& a, hipStream_t stream)
         }
         hipLaunchKernelGGL((resize_fill_kernel<T>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, x, y, a.N, a.C,
                            a.Hs * a.Ws, a.Hd * a.Wd, a.channels_last);
+        return hipGetLastError();
+    }
+    if (a.mode == ResizeMode::Nearest) {
+        constexpr int V = 16 / (int)sizeof(T);
+        const bool nhwc = a.channels_last != 0;
+        const int64_t row_elems = nhwc ? a.Wd * a.C : a.Wd;
+        const int64_t outer = nhwc ? a.N : a.N * a.C;
+        const int64_t rows = outer * a.Hd;
+        const bool aligned = reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0;
+        // whole 16-byte vectors: rows start aligned (row_elems % V == 0); for NHWC a vector stays inside one pixel
+        const bool vec = aligned && row_elems % V == 0 && (!nhwc || (a.C % V == 0 && (a.Ws * a.C) % V == 0));
+        const int64_t lanes = vec ? row_elems / V : row_elems;
+        dim3 grid((unsigned)((lanes + kThreads - 1) / kThreads), (unsigned)(rows < 65535 ? rows : 65535));
+#define OPSCV_NEAREST(NHWC_, VEC_)                                                                                  \
+    hipLaunchKernelGGL((resize_nearest_kernel<T, NHWC_, VEC_>), grid, dim3(kThreads), 0, stream, x, y, outer,      \
+                       (int32_t)a.C, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h, a.scale_w)
+        if (nhwc) {
+            if (vec) {
+                OPSCV_NEAREST(true, true);
+            } else {
+                OPSCV_NEAREST(true, false);
+            }
+        } else {
+            if (vec) {
+                OPSCV_NEAREST(false, true);
+            } else {
+                OPSCV_NEAREST(false, false);
+            }
+        }
+#undef OPSCV_NEAREST
         return hipGetLastError();
     }
     if (a.channels_last) {
@@ -290,6 +382,7 @@ const char* resize_variant(const ResizeArgs& a)
         case ResizeMode::Copy: return "copy";
         case ResizeMode::Broadcast: return "broadcast";
         case ResizeMode::FirstPixel: return "first_pixel";
+        case ResizeMode::Nearest: return a.channels_last ? "nearest_nhwc" : "nearest_nchw";
         default: break;
     }
     if (a.channels_last) {

@@ -37,4 +37,17 @@ void plan_resize(ResizeArgs* a, bool align_corners, float user_scale_h, float us
     }
 }
 
+void plan_resize_nearest(ResizeArgs* a)
+{
+    a->half_pixel = 0;
+    a->scale_h = (float)a->Hs / (float)a->Hd;
+    a->scale_w = (float)a->Ws / (float)a->Wd;
+    a->mode = ResizeMode::Nearest;
+    if (a->Hs == a->Hd && a->Ws == a->Wd) {
+        a->mode = ResizeMode::Copy;  // every index maps to itself: floor(i * 1.0f) = i
+    } else if (a->Hs == 1 && a->Ws == 1) {
+        a->mode = ResizeMode::Broadcast;
+    }
+}
+
 }  // namespace opscv

@@ -14,4 +14,9 @@ float resize_axis_scale(int64_t len_src, int64_t len_dst, bool align_corners, fl
 // image/resize_bilinear_v2/op_kernel/resize_bilinear_v2_apt.cpp:91-140.
 void plan_resize(ResizeArgs* a, bool align_corners, float user_scale_h, float user_scale_w);
 
+// Nearest-neighbour resize with align_corners = false and half_pixel_centers = false, the only combination
+// aclnnResize requests (image/resize_bilinear_v2/op_api/aclnn_resize.cpp:286-288): scale = in / out
+// (image/resize_nearest_neighbor_v2/op_host/arch35/resize_nearest_neighbor_v2_tiling_base.cpp:253-263).
+void plan_resize_nearest(ResizeArgs* a);
+
 }  // namespace opscv

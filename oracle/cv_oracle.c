@@ -21,6 +21,8 @@
  *   oracle_upsample_bilinear2d   : known answers for image/upsample_bilinear2d/examples/
  *                                  test_aclnn_upsample_bilinear2d.cpp:83-94, kernel-UT shapes (1,1,1,4)->(2,16),
  *                                  (3,16), committed torch interpolate fixtures, live torch CPU comparison
+ *   oracle_resize_nearest        : integer-factor upscales equal element repetition, committed and live
+ *                                  torch interpolate(mode="nearest") comparison (bit-exact: a pure copy)
  *   oracle_resize_scale          : float bit patterns held by the reference's tiling UT
  *                                  (image/resize_bilinear_v2/tests/ut/op_host/arch35/test_resize_bilinear_v2_tiling.cpp)
  */
@@ -628,6 +630,48 @@ int oracle_upsample_bilinear2d(const void* x, void* y, int dtype, int64_t N, int
             /* resize_bilinear_v2_simt_nchw.h:143-144 */
             float out = (1.0f - dy) * ((1.0f - dx) * tl + dx * tr) + dy * ((1.0f - dx) * bl + dx * br);
             store_from_float(y, dtype, r * Wd + w, out);
+        }
+    }
+    return 0;
+}
+
+/* resize_nearest_neighbor_v2_simt.h:103-124 (the !align_corner && !half_pixel branch) */
+static inline int64_t nearest_src(int64_t d, float scale, int64_t len_src)
+{
+    float f = floorf((float)d * scale);
+    int64_t i = (int64_t)f;
+    return (i < len_src - 1) ? i : len_src - 1;
+}
+
+int oracle_resize_nearest(const void* x, void* y, int dtype, int64_t N, int64_t C, int64_t Hs, int64_t Ws,
+                          int64_t Hd, int64_t Wd, int channels_last)
+{
+    if (dtype < 0 || dtype > 2 || Hs <= 0 || Ws <= 0 || Hd <= 0 || Wd <= 0) {
+        return -1;
+    }
+    const int64_t esz = (dtype == ORACLE_F32) ? 4 : 2;
+    /* resize_nearest_neighbor_v2_tiling_base.cpp:257,262 */
+    const float scale_h = (float)Hs / (float)Hd;
+    const float scale_w = (float)Ws / (float)Wd;
+    const char* src = (const char*)x;
+    char* dst = (char*)y;
+    for (int64_t n = 0; n < N; n++) {
+        for (int64_t c = 0; c < C; c++) {
+            for (int64_t h = 0; h < Hd; h++) {
+                const int64_t sy = nearest_src(h, scale_h, Hs);
+                for (int64_t w = 0; w < Wd; w++) {
+                    const int64_t sx = nearest_src(w, scale_w, Ws);
+                    int64_t so, dof;
+                    if (channels_last) {
+                        so = ((n * Hs + sy) * Ws + sx) * C + c;
+                        dof = ((n * Hd + h) * Wd + w) * C + c;
+                    } else {
+                        so = ((n * C + c) * Hs + sy) * Ws + sx;
+                        dof = ((n * C + c) * Hd + h) * Wd + w;
+                    }
+                    memcpy(dst + dof * esz, src + so * esz, (size_t)esz);
+                }
+            }
         }
     }
     return 0;

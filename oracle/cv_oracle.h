@@ -90,6 +90,16 @@ int oracle_upsample_bilinear2d(const void* x, void* y, int dtype, int64_t N, int
                                int64_t Hd, int64_t Wd, int align_corners, double scales_h, double scales_w,
                                int num_threads);
 
+/*
+ * nearest-neighbour resize with align_corners = false and half_pixel_centers = false, scale = in / out:
+ * src = min(floor(float(dst) * scale), in - 1)
+ * (image/resize_nearest_neighbor_v2/op_kernel/arch35/resize_nearest_neighbor_v2_simt.h:103-124, scale rule
+ * image/resize_nearest_neighbor_v2/op_host/arch35/resize_nearest_neighbor_v2_tiling_base.cpp:253-263).
+ * channels_last = 0: x is (N,C,Hs,Ws); 1: x is (N,Hs,Ws,C).
+ */
+int oracle_resize_nearest(const void* x, void* y, int dtype, int64_t N, int64_t C, int64_t Hs, int64_t Ws,
+                          int64_t Hd, int64_t Wd, int channels_last);
+
 /* per-axis tap table of the upsample: i0[len_dst], i1[len_dst], lambda[len_dst] */
 int oracle_upsample_axis_taps(int64_t len_src, int64_t len_dst, int align_corners, float user_scale, int32_t* i0,
                               int32_t* i1, float* lambda);

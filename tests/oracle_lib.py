@@ -78,6 +78,8 @@ def lib():
     L.oracle_grid_sampler2d_bicubic_taps.restype = ctypes.c_int
     L.oracle_grid_sampler2d_bicubic_taps.argtypes = [vp, vp, ctypes.c_int, i64, i64, i64, i64, i64, ctypes.c_int,
                                                      ctypes.c_int]
+    L.oracle_resize_nearest.restype = ctypes.c_int
+    L.oracle_resize_nearest.argtypes = [vp, vp, ctypes.c_int, i64, i64, i64, i64, i64, i64, ctypes.c_int]
     L.oracle_resize_scale.restype = f32
     L.oracle_resize_scale.argtypes = [i64, i64, ctypes.c_int, f32]
     L.oracle_upsample_bilinear2d.restype = ctypes.c_int
@@ -142,6 +144,22 @@ def grid_sampler2d_bicubic_taps(grid, H, W, pad=0, align=False, dtype=None):
     if rc != 0:
         raise ValueError("oracle_grid_sampler2d_bicubic_taps rc=%d" % rc)
     return taps
+
+
+def resize_nearest(x, out_hw, channels_last=False, dtype=None):
+    """x (N,C,H,W) or, with channels_last, (N,H,W,C) -> the same layout at out_hw"""
+    x = np.ascontiguousarray(x)
+    code = _code_of(x) if dtype is None else dtype
+    if channels_last:
+        N, Hs, Ws, C = x.shape
+        y = np.empty((N, out_hw[0], out_hw[1], C), dtype=x.dtype)
+    else:
+        N, C, Hs, Ws = x.shape
+        y = np.empty((N, C, out_hw[0], out_hw[1]), dtype=x.dtype)
+    rc = lib().oracle_resize_nearest(_ptr(x), _ptr(y), code, N, C, Hs, Ws, out_hw[0], out_hw[1], int(channels_last))
+    if rc != 0:
+        raise ValueError("oracle_resize_nearest rc=%d" % rc)
+    return y
 
 
 def upsample_bilinear2d(x, out_hw, align=False, scales_h=0.0, scales_w=0.0, dtype=None, threads=0):

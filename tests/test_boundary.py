@@ -2,7 +2,8 @@
 
 The cases mirror the reference's op_api unit tests, which build descriptors with NULL data pointers and call only
 the GetWorkspaceSize phase: image/grid_sample/tests/ut/op_host/op_api/test_aclnn_grid_sampler2d.cpp and
-image/upsample_bilinear2d/tests/ut/op_host/op_api/test_aclnn_upsample_bilinear_2d.cpp.
+image/upsample_bilinear2d/tests/ut/op_host/op_api/test_aclnn_upsample_bilinear_2d.cpp,
+image/resize_bilinear_v2/tests/ut/op_host/op_api/test_aclnn_resize.cpp.
 """
 import ctypes
 import os
@@ -232,3 +233,58 @@ def test_upsample_template_selection(aclnn, desc):
     assert _up(aclnn, desc, inp=(2, 256, 12, 12), out=(2, 256, 18, 18), size=(18, 18), dt=f32, sh=1.5, sw=1.5)[2].startswith("nchw")
     assert _up(aclnn, desc, inp=(2, 128, 128, 256), out=(2, 192, 192, 256), size=(192, 192), dt=f32,
                fmt=aclnn.ACL_FORMAT_NHWC, align=True)[2] == "nhwc_generic"
+
+
+def _rs(aclnn, desc, inp=(1, 1, 2, 2), out=(1, 1, 4, 4), scales=(1, 1, 2, 2), mode=b"nearest", dt=None, odt=None,
+        fmt=None, ofmt=None):
+    dt = aclnn.ACL_FLOAT if dt is None else dt
+    fmt = aclnn.ACL_FORMAT_NCHW if fmt is None else fmt
+    s = desc.t(inp, dt, fmt)
+    o = desc.t(out, dt if odt is None else odt, fmt if ofmt is None else ofmt)
+    arr = aclnn.create_float_array(list(scales)) if scales is not None else None
+    st, ws, ex = aclnn.get_workspace_size_resize(s, arr, mode, o)
+    variant = aclnn.executor_variant(ex) if ex else None
+    if ex:
+        aclnn.destroy_executor(ex)
+    aclnn.destroy_float_array(arr)
+    return st, ws, variant
+
+
+def test_resize_status_codes(aclnn, desc):
+    """test_aclnn_resize.cpp case_1 .. case_11 and the element checks of aclnn_resize.cpp:82-121"""
+    INV, NULL = aclnn.ACLNN_ERR_PARAM_INVALID, aclnn.ACLNN_ERR_PARAM_NULLPTR
+    for dt in (aclnn.ACL_FLOAT, aclnn.ACL_FLOAT16, aclnn.ACL_BF16):
+        assert _rs(aclnn, desc, dt=dt, mode=b"nearest") == (0, 0, "nearest_nchw")          # case_1, case_2
+        st, ws, variant = _rs(aclnn, desc, dt=dt, mode=b"bilinear")                        # case_3, case_4
+        assert st == 0 and ws == 0 and variant.startswith("nchw")
+    assert _rs(aclnn, desc, scales=(1, 1, 2))[0] == INV                                    # case_5
+    assert _rs(aclnn, desc, inp=None)[0] == NULL                                           # case_6
+    assert _rs(aclnn, desc, scales=None)[0] == NULL                                        # case_7
+    assert _rs(aclnn, desc, out=None)[0] == NULL                                           # case_8
+    assert _rs(aclnn, desc, mode=None)[0] == NULL
+    assert _rs(aclnn, desc, mode=b"trilinear")[0] == INV                                   # case_9
+    assert _rs(aclnn, desc, odt=aclnn.ACL_FLOAT16)[0] == INV                               # case_10
+    assert _rs(aclnn, desc, out=(1, 2, 4, 4))[0] == INV                                    # case_11
+    # the mode is matched by prefix
+    assert _rs(aclnn, desc, mode=b"nearest-exact")[0] == 0
+    assert _rs(aclnn, desc, mode=b"bilinear_v2")[0] == 0
+    # unsupported dtype, unequal / unsupported formats
+    assert _rs(aclnn, desc, dt=aclnn.ACL_DOUBLE)[0] == INV
+    assert _rs(aclnn, desc, ofmt=aclnn.ACL_FORMAT_NHWC)[0] == INV
+    assert _rs(aclnn, desc, fmt=aclnn.ACL_FORMAT_ND)[0] == INV
+    # output extents must equal trunc(in * scale) within scale +- 1e-5
+    assert _rs(aclnn, desc, out=(1, 1, 5, 4))[0] == INV
+    assert _rs(aclnn, desc, out=(1, 1, 4, 2))[0] == INV
+    # ... where the lower bound truncates 2 * (2 - 1e-5) = 3.99998 to 3, so 3 passes as it does in the reference
+    assert _rs(aclnn, desc, out=(1, 1, 4, 3))[0] == 0
+    assert _rs(aclnn, desc, inp=(1, 1, 3, 3), out=(1, 1, 4, 7), scales=(1, 1, 1.5, 2.5))[0] == 0
+    # NHWC: dimensions and scales are read in N,H,W,C order
+    st, ws, variant = _rs(aclnn, desc, inp=(1, 2, 2, 8), out=(1, 4, 4, 8), scales=(1, 2, 2, 1), fmt=aclnn.ACL_FORMAT_NHWC)
+    assert (st, variant) == (0, "nearest_nhwc")
+    assert _rs(aclnn, desc, inp=(1, 2, 2, 8), out=(1, 4, 4, 8), scales=(1, 1, 2, 2), fmt=aclnn.ACL_FORMAT_NHWC)[0] == INV
+    # rank
+    assert _rs(aclnn, desc, inp=(1, 2, 2), out=(1, 4, 4), scales=(1, 2, 2, 1))[0] == INV
+    # same size -> copy; 1x1 source -> broadcast; empty -> no-op
+    assert _rs(aclnn, desc, out=(1, 1, 2, 2), scales=(1, 1, 1, 1))[2] == "copy"
+    assert _rs(aclnn, desc, inp=(1, 1, 1, 1), out=(1, 1, 4, 4), scales=(1, 1, 4, 4))[2] == "broadcast"
+    assert _rs(aclnn, desc, inp=(0, 1, 2, 2), out=(0, 1, 4, 4))[:2] == (0, 0)

@@ -154,3 +154,49 @@ def test_full_size_upsample_fp32_56_to_112(oracle, device, aclnn):
     torch.cuda.synchronize()
     ref = oracle.upsample_bilinear2d(x, (112, 112), False, 2.0, 2.0)
     assert np.array_equal(y.cpu().numpy().view(np.uint32), ref.view(np.uint32))
+
+
+@pytest.mark.parametrize("dtype", I.DTYPES)
+@pytest.mark.parametrize("channels_last", [False, True])
+def test_resize_entry_point(oracle, device, aclnn, dtype, channels_last):
+    """aclnnResize: bilinear is the upsample kernel with align_corners=False and scale = in/out; nearest is
+    floor(dst * in/out).  Both bit-exact against the oracle, NCHW and NHWC, vector and scalar shapes."""
+    import torch
+    rng = np.random.default_rng(300 + int(channels_last))
+    cases = [((1, 1, 2, 2), (2.0, 2.0)), ((2, 8, 9, 12), (2.0, 2.0)), ((1, 16, 7, 5), (1.5, 2.5)),
+             ((2, 3, 16, 16), (0.5, 0.75)), ((1, 4, 1, 1), (4.0, 8.0)), ((1, 2, 6, 6), (1.0, 1.0)),
+             ((1, 8, 33, 64), (3.0, 2.0))]
+    for shape, (sh, sw) in cases:
+        N, C, H, W = shape
+        Ho, Wo = int(float(H) * sh), int(float(W) * sw)
+        x = I.cast_np(rng.standard_normal(shape).astype(np.float32), dtype)
+        xin = np.ascontiguousarray(x.transpose(0, 2, 3, 1)) if channels_last else x
+        scales = (1.0, sh, sw, 1.0) if channels_last else (1.0, 1.0, sh, sw)
+        xt = I.to_torch(xin, dtype, device)
+        for mode in ("nearest", "bilinear"):
+            y = I.from_torch(aclnn.resize(xt, scales, mode, channels_last=channels_last), dtype)
+            torch.cuda.synchronize()
+            if mode == "nearest":
+                ref = oracle.resize_nearest(xin, (Ho, Wo), channels_last=channels_last, dtype=I.oracle_code(dtype))
+            else:
+                ref = oracle.upsample_bilinear2d(x, (Ho, Wo), False, 0.0, 0.0, dtype=I.oracle_code(dtype))
+                if channels_last:
+                    ref = np.ascontiguousarray(ref.transpose(0, 2, 3, 1))
+            view = np.uint32 if dtype == "fp32" else np.uint16
+            assert y.shape == ref.shape
+            assert np.array_equal(y.view(view), ref.view(view)), (mode, shape, sh, sw, dtype, channels_last)
+
+
+def test_resize_strided_views(oracle, device, aclnn):
+    """aclnnResize honours non-contiguous self and out views (packed through the workspace)"""
+    import torch
+    rng = np.random.default_rng(301)
+    big = torch.from_numpy(rng.standard_normal((2, 4, 10, 24)).astype(np.float32)).to(device)
+    xv = big[:, 1:3, 2:9, 3:19:2]
+    outbig = torch.zeros((2, 2, 14, 40), device=device)
+    ov = outbig[:, :, :, ::2][..., :16]
+    aclnn.resize(xv, (1.0, 1.0, 2.0, 2.0), "nearest", out=ov)
+    torch.cuda.synchronize()
+    ref = oracle.resize_nearest(xv.contiguous().cpu().numpy(), (14, 16))
+    assert np.array_equal(ov.cpu().numpy(), ref)
+    assert float(outbig[:, :, :, 1::2].abs().max()) == 0.0

@@ -432,3 +432,27 @@ def test_live_torch_interpolate(oracle):
             got = oracle.upsample_bilinear2d(x, (int(Ho), int(Wo)), a)
             want = F.interpolate(torch.from_numpy(x), size=(int(Ho), int(Wo)), mode="bilinear", align_corners=a).numpy()
             assert np.abs(got - want).max() <= 2e-5
+
+
+def test_resize_nearest_oracle(oracle):
+    """resize_nearest_neighbor_v2_simt.h:103-124: integer factors repeat elements; the rule is PyTorch's legacy
+    "nearest" (floor(dst * in/out)), so torch reproduces it exactly -- a copy has no rounding"""
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(77)
+    x = rng.standard_normal((2, 3, 5, 7)).astype(np.float32)
+    y = oracle.resize_nearest(x, (10, 21))
+    assert np.array_equal(y, np.repeat(np.repeat(x, 2, axis=2), 3, axis=3))
+    # the reference example: 1,2,3,4 as 2x2 -> 4x4
+    e = oracle.resize_nearest(np.array([1, 2, 3, 4], dtype=np.float32).reshape(1, 1, 2, 2), (4, 4))
+    assert e[0, 0].tolist() == [[1, 1, 2, 2], [1, 1, 2, 2], [3, 3, 4, 4], [3, 3, 4, 4]]
+    for (H, W, Ho, Wo) in [(5, 7, 13, 4), (9, 9, 3, 20), (1, 6, 4, 4), (17, 31, 40, 77), (64, 64, 100, 37)]:
+        x = rng.standard_normal((2, 3, H, W)).astype(np.float32)
+        want = F.interpolate(torch.from_numpy(x), size=(Ho, Wo), mode="nearest").numpy()
+        assert np.array_equal(oracle.resize_nearest(x, (Ho, Wo)), want), (H, W, Ho, Wo)
+        xl = np.ascontiguousarray(x.transpose(0, 2, 3, 1))
+        assert np.array_equal(oracle.resize_nearest(xl, (Ho, Wo), channels_last=True), want.transpose(0, 2, 3, 1))
+    xh = rng.standard_normal((1, 2, 6, 5)).astype(np.float16)
+    assert np.array_equal(oracle.resize_nearest(xh, (9, 11)),
+                          F.interpolate(torch.from_numpy(xh.astype(np.float32)), size=(9, 11),
+                                        mode="nearest").numpy().astype(np.float16))
