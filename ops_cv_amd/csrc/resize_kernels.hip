@@ -22,6 +22,16 @@ namespace {
 
 constexpr int kThreads = 256;
 
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+// 16-byte store that bypasses the caches (for outputs much larger than them)
+__device__ __forceinline__ void store_streaming(uint4* dst, uint4 v)
+{
+    u32x4_t t;
+    __builtin_memcpy(&t, &v, 16);
+    __builtin_nontemporal_store(t, reinterpret_cast<u32x4_t*>(dst));
+}
+
 // Generic NCHW variant: one lane per output pixel of a row, rows and planes on the other grid axes.
 template <typename T, bool HALF_PIXEL>
 __global__ __launch_bounds__(kThreads) void resize_nchw_generic_kernel(const T* __restrict__ x, T* __restrict__ y,
@@ -169,6 +179,65 @@ __global__ __launch_bounds__(kThreads) void resize_nhwc_generic_kernel(const T* 
     }
 }
 
+// Vector NHWC variant: one lane per 16-byte run of channels of an output pixel (V = 16/sizeof(T) channels, needs
+// C % V == 0 and 16-byte aligned tensors).  The four taps are 16-byte loads that neighbouring lanes extend to
+// whole pixels, the result is one 16-byte store; per channel the arithmetic is the reference formula.
+template <typename T, bool HALF_PIXEL>
+__global__ __launch_bounds__(kThreads) void resize_nhwc_vec_kernel(const T* __restrict__ x, T* __restrict__ y,
+                                                                    int64_t N, int32_t C, int32_t Hs, int32_t Ws,
+                                                                    int32_t Hd, int32_t Wd, float scale_h,
+                                                                    float scale_w, int streaming)
+{
+    constexpr int V = 16 / (int)sizeof(T);
+    const int32_t cvecs = C / V;
+    const int64_t row_vecs = (int64_t)Wd * cvecs;
+    const int64_t e = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (e >= row_vecs) {
+        return;
+    }
+    const int32_t w = (int32_t)(e / cvecs);
+    const int32_t c = (int32_t)(e - (int64_t)w * cvecs) * V;
+    const AxisTap tx = axis_tap<HALF_PIXEL>(w, scale_w, Ws);
+    const float dx = tx.lambda;
+    const float omdx = 1.0f - dx;
+    const int64_t o0 = (int64_t)tx.i0 * C + c;
+    const int64_t o1 = (int64_t)tx.i1 * C + c;
+    const int64_t rows = N * Hd;
+    const int64_t src_row = (int64_t)Ws * C;
+    for (int64_t r = blockIdx.y; r < rows; r += gridDim.y) {
+        const int64_t n = r / Hd;
+        const int32_t h = (int32_t)(r - n * Hd);
+        const AxisTap ty = axis_tap<HALF_PIXEL>(h, scale_h, Hs);
+        const float dy = ty.lambda;
+        const float omdy = 1.0f - dy;
+        const T* top = x + (n * Hs + ty.i0) * src_row;
+        const T* bot = x + (n * Hs + ty.i1) * src_row;
+        T tl[V], tr[V], bl[V], br[V], outv[V];
+        uint4 raw;
+        raw = *reinterpret_cast<const uint4*>(top + o0);
+        __builtin_memcpy(tl, &raw, 16);
+        raw = *reinterpret_cast<const uint4*>(top + o1);
+        __builtin_memcpy(tr, &raw, 16);
+        raw = *reinterpret_cast<const uint4*>(bot + o0);
+        __builtin_memcpy(bl, &raw, 16);
+        raw = *reinterpret_cast<const uint4*>(bot + o1);
+        __builtin_memcpy(br, &raw, 16);
+#pragma unroll
+        for (int i = 0; i < V; i++) {
+            const float t = omdx * ElemIO<T>::load(&tl[i]) + dx * ElemIO<T>::load(&tr[i]);
+            const float b = omdx * ElemIO<T>::load(&bl[i]) + dx * ElemIO<T>::load(&br[i]);
+            ElemIO<T>::store(&outv[i], omdy * t + dy * b);
+        }
+        __builtin_memcpy(&raw, outv, 16);
+        uint4* dst = reinterpret_cast<uint4*>(y + (r * row_vecs + e) * V);
+        if (streaming) {
+            store_streaming(dst, raw);
+        } else {
+            *dst = raw;
+        }
+    }
+}
+
 // Nearest-neighbour resize (align_corners = false, half_pixel_centers = false):
 //   src = min(floor(float(dst) * scale), len_src - 1)
 // image/resize_nearest_neighbor_v2/op_kernel/arch35/resize_nearest_neighbor_v2_simt.h:103-124.
@@ -186,7 +255,8 @@ __device__ __forceinline__ int32_t nearest_src(int32_t d, float scale, int32_t l
 template <typename T, bool NHWC, bool VEC>
 __global__ __launch_bounds__(kThreads) void resize_nearest_kernel(const T* __restrict__ x, T* __restrict__ y,
                                                                    int64_t outer, int32_t C, int32_t Hs, int32_t Ws,
-                                                                   int32_t Hd, int32_t Wd, float scale_h, float scale_w)
+                                                                   int32_t Hd, int32_t Wd, float scale_h, float scale_w,
+                                                                   int streaming)
 {
     constexpr int V = VEC ? 16 / (int)sizeof(T) : 1;
     const int64_t row_elems = NHWC ? (int64_t)Wd * C : (int64_t)Wd;
@@ -224,7 +294,11 @@ __global__ __launch_bounds__(kThreads) void resize_nearest_kernel(const T* __res
                 }
                 __builtin_memcpy(&packed, v, sizeof(packed));
             }
-            *reinterpret_cast<uint4*>(dst) = packed;
+            if (streaming) {
+                store_streaming(reinterpret_cast<uint4*>(dst), packed);
+            } else {
+                *reinterpret_cast<uint4*>(dst) = packed;
+            }
         } else {
             dst[0] = src[src_off[0]];
         }
@@ -274,6 +348,15 @@ bool band_variant_ok(const ResizeArgs& a)
     return !(v != nullptr && v[0] == 'g');  // OPSCV_RESIZE_VARIANT=generic forces the generic kernel
 }
 
+// The vector NHWC variant moves whole 16-byte runs of channels.
+template <typename T>
+bool nhwc_vec_ok(const ResizeArgs& a)
+{
+    constexpr int V = 16 / (int)sizeof(T);
+    return a.channels_last && a.mode == ResizeMode::Bilinear && a.C % V == 0 &&
+           reinterpret_cast<uintptr_t>(a.x) % 16 == 0 && reinterpret_cast<uintptr_t>(a.y) % 16 == 0;
+}
+
 template <typename T>
 hipError_t run_resize(const ResizeArgs& a, hipStream_t stream)
 {
@@ -305,7 +388,9 @@ hipError_t run_resize(const ResizeArgs& a, hipStream_t stream)
         dim3 grid((unsigned)((lanes + kThreads - 1) / kThreads), (unsigned)(rows < 65535 ? rows : 65535));
 #define OPSCV_NEAREST(NHWC_, VEC_)                                                                                  \
     hipLaunchKernelGGL((resize_nearest_kernel<T, NHWC_, VEC_>), grid, dim3(kThreads), 0, stream, x, y, outer,      \
-                       (int32_t)a.C, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h, a.scale_w)
+                       (int32_t)a.C, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h, a.scale_w, \
+                       streaming)
+        const int streaming = (out_elems * (int64_t)sizeof(T) >= (128ll << 20)) ? 1 : 0;
         if (nhwc) {
             if (vec) {
                 OPSCV_NEAREST(true, true);
@@ -320,6 +405,23 @@ hipError_t run_resize(const ResizeArgs& a, hipStream_t stream)
             }
         }
 #undef OPSCV_NEAREST
+        return hipGetLastError();
+    }
+    if (nhwc_vec_ok<T>(a)) {
+        constexpr int V = 16 / (int)sizeof(T);
+        const int64_t row_vecs = a.Wd * (a.C / V);
+        const int64_t rows = a.N * a.Hd;
+        const int streaming = (out_elems * (int64_t)sizeof(T) >= (128ll << 20)) ? 1 : 0;
+        dim3 grid((unsigned)((row_vecs + kThreads - 1) / kThreads), (unsigned)(rows < 65535 ? rows : 65535));
+        if (a.half_pixel) {
+            hipLaunchKernelGGL((resize_nhwc_vec_kernel<T, true>), grid, dim3(kThreads), 0, stream, x, y, a.N,
+                               (int32_t)a.C, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h,
+                               a.scale_w, streaming);
+        } else {
+            hipLaunchKernelGGL((resize_nhwc_vec_kernel<T, false>), grid, dim3(kThreads), 0, stream, x, y, a.N,
+                               (int32_t)a.C, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h,
+                               a.scale_w, streaming);
+        }
         return hipGetLastError();
     }
     if (a.channels_last) {
@@ -386,7 +488,13 @@ const char* resize_variant(const ResizeArgs& a)
         default: break;
     }
     if (a.channels_last) {
-        return "nhwc_generic";
+        bool vec = false;
+        switch (a.elem) {
+            case Elem::F32: vec = nhwc_vec_ok<float>(a); break;
+            case Elem::F16: vec = nhwc_vec_ok<_Float16>(a); break;
+            case Elem::BF16: vec = nhwc_vec_ok<__bf16>(a); break;
+        }
+        return vec ? "nhwc_vec" : "nhwc_generic";
     }
     if (const char* lds_variant = resize_lds_variant(a)) {
         return lds_variant;

@@ -232,6 +232,8 @@ def test_upsample_template_selection(aclnn, desc):
     # case01/02/06: ordinary NCHW bilinear; NHWC has its own kernel
     assert _up(aclnn, desc, inp=(2, 256, 12, 12), out=(2, 256, 18, 18), size=(18, 18), dt=f32, sh=1.5, sw=1.5)[2].startswith("nchw")
     assert _up(aclnn, desc, inp=(2, 128, 128, 256), out=(2, 192, 192, 256), size=(192, 192), dt=f32,
+               fmt=aclnn.ACL_FORMAT_NHWC, align=True)[2] == "nhwc_vec"
+    assert _up(aclnn, desc, inp=(2, 12, 12, 5), out=(2, 18, 18, 5), size=(18, 18), dt=f32,
                fmt=aclnn.ACL_FORMAT_NHWC, align=True)[2] == "nhwc_generic"
 
 

@@ -48,7 +48,8 @@ def test_upsample_nhwc(oracle, device, aclnn, dtype, align):
     torch = _torch()
     rng = np.random.default_rng(22)
     for (N, C, H, W), size in [((2, 5, 7, 9), (14, 18)), ((1, 64, 1, 1), (6, 6)), ((1, 3, 8, 8), (8, 8)),
-                               ((2, 3, 6, 6), (1, 1)), ((1, 130, 3, 3), (5, 7))]:
+                               ((2, 3, 6, 6), (1, 1)), ((1, 130, 3, 3), (5, 7)), ((2, 16, 9, 11), (20, 17)),
+                               ((1, 64, 12, 10), (5, 23)), ((1, 8, 1, 6), (4, 4))]:
         x32 = rng.standard_normal((N, C, H, W)).astype(np.float32)
         x = I.cast_np(x32, dtype)
         ref = oracle.upsample_bilinear2d(x, size, align, dtype=I.oracle_code(dtype))
