@@ -89,6 +89,7 @@ struct GridSamplerArgs {
     int interp = 0;
     int pad = 0;
     int align = 0;
+    int channels_last = 0;  // 1: x is (N,Hin,Win,C) and y is (N,Hout,Wout,C) in memory
     int64_t N = 0, C = 0, Hin = 0, Win = 0, Hout = 0, Wout = 0;
     const void* x = nullptr;
     const void* grid = nullptr;

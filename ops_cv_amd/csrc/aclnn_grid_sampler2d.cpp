@@ -39,6 +39,19 @@ bool check_dtypes(const aclTensor* input, const aclTensor* grid, const aclTensor
 }
 
 // aclnn_grid_sampler2d.cpp:94-110
+// (N,C,H,W) view whose elements lie in memory as a dense (N,H,W,C) array
+bool channels_last_dense(const aclTensor* t)
+{
+    const int64_t C = t->dims[1], H = t->dims[2], W = t->dims[3];
+    const int64_t want[4] = {H * W * C, 1, W * C, C};
+    for (int i = 0; i < 4; i++) {
+        if (t->dims[i] != 1 && t->strides[i] != want[i]) {
+            return false;
+        }
+    }
+    return true;
+}
+
 bool check_attrs(int64_t interp, int64_t pad)
 {
     if (interp < 0 || interp > 2) {
@@ -148,9 +161,17 @@ aclnnStatus aclnnGridSampler2DGetWorkspaceSize(const aclTensor* input, const acl
     a.Hout = grid->dims[1];
     a.Wout = grid->dims[2];
     const int esz = elem_size(elem);
-    ex->in0 = plan_view(ex.get(), input, esz, false);
+    // Views that are dense in channels-last order (what a framework hands over for its channels_last memory
+    // format) are sampled in place by the channels-last kernel instead of being repacked to NCHW and back.
+    if (!input->contiguous() && !out->contiguous() && channels_last_dense(input) && channels_last_dense(out)) {
+        a.channels_last = 1;
+        ex->in0.direct = (input->data == nullptr) ? nullptr : (char*)input->data + input->offset * (int64_t)esz;
+        ex->out0.direct = (out->data == nullptr) ? nullptr : (char*)out->data + out->offset * (int64_t)esz;
+    } else {
+        ex->in0 = plan_view(ex.get(), input, esz, false);
+        ex->out0 = plan_view(ex.get(), out, esz, true);
+    }
     ex->in1 = plan_view(ex.get(), grid, esz, false);
-    ex->out0 = plan_view(ex.get(), out, esz, true);
 
     *workspaceSize = ex->workspace_bytes;
     *executor = ex.release();

@@ -278,6 +278,9 @@ bool force_direct()
 
 const char* grid_sampler2d_variant(const GridSamplerArgs& a)
 {
+    if (a.channels_last) {
+        return "nhwc";
+    }
     if (!force_direct()) {
         const char* n = gs2d_lds_variant_name(a);
         if (n != nullptr) {
@@ -297,6 +300,9 @@ hipError_t launch_grid_sampler2d(const GridSamplerArgs& a, hipStream_t stream)
     }
     if (a.x == nullptr || a.grid == nullptr || a.y == nullptr) {
         return hipErrorInvalidValue;
+    }
+    if (a.channels_last) {
+        return run_gs2d_nhwc(a, stream);
     }
     if (!force_direct()) {
         bool handled = false;

@@ -1,0 +1,174 @@
+// Grid sampler 2-D forward for channels-last tensors (input (N,Hin,Win,C) and output (N,Hout,Wout,C) in memory)
+// on gfx950.
+//
+// Same arithmetic as the NCHW variants (see sampler_math.hpp; reference kernel
+// image/grid_sampler2_d/op_kernel/arch35/grid_sampler2_d_simt.h:303-360,375-458).  With the channels innermost
+// every tap of a pixel is one contiguous run of C elements, so the gather needs no staging:
+//   * `lpp` neighbouring lanes (a power of two, at most 16) share one output pixel; each takes every lpp-th
+//     16-byte run of channels, so a pixel's tap is read -- and its output written -- as contiguous 16*lpp bytes;
+//   * every lane decides its pixel once (tap offsets, weights, bounds masks) and keeps that across its channel runs;
+//   * a tap outside the image is replaced by zeros after the (clamped, always valid) load, which is the
+//     reference's "skip the tap": 0 * w adds nothing.
+// When C is not a multiple of the vector length, or a tensor is not 16-byte aligned, the same kernel runs with
+// one element per lane and step.
+#include <hip/hip_runtime.h>
+
+#include "gs2d_common.hpp"
+#include "gs2d_lds_kernel.hpp"
+#include "kernels.hpp"
+#include "sampler_math.hpp"
+
+namespace opscv {
+
+namespace {
+
+constexpr int kNhwcThreads = 256;
+
+template <typename T, int INTERP, int PAD, bool ALIGN, bool VEC>
+__global__ __launch_bounds__(kNhwcThreads) void gs2d_nhwc_kernel(const T* __restrict__ x, const T* __restrict__ grid,
+                                                                  T* __restrict__ y, int64_t total_pixels, int32_t C,
+                                                                  int32_t H, int32_t W, int64_t out_plane,
+                                                                  int32_t lpp_shift, float neg_zero)
+{
+    constexpr int V = VEC ? 16 / (int)sizeof(T) : 1;
+    constexpr int NT = (INTERP == 0) ? 4 : (INTERP == 1 ? 1 : 16);
+    constexpr int NW = (INTERP == 2) ? 8 : 4;
+    const int32_t lpp = 1 << lpp_shift;
+    const int32_t sub = threadIdx.x & (lpp - 1);
+    const int64_t p = (int64_t)blockIdx.x * (kNhwcThreads >> lpp_shift) + (threadIdx.x >> lpp_shift);
+    if (p >= total_pixels) {
+        return;
+    }
+    const int64_t n = p / out_plane;
+    const float gx = ElemIO<T>::load(grid + 2 * p);
+    const float gy = ElemIO<T>::load(grid + 2 * p + 1);
+
+    int64_t toff[NT];  // element offset of the tap's pixel inside image n; 0 (always valid) when outside
+    bool tin[NT];
+    float tw[NW];
+    if constexpr (INTERP == 2) {
+        const BicubicTap b = decide_bicubic<PAD, ALIGN>(gx, gy, H, W);
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const bool row_in = b.by[r] >= 0 && b.by[r] < H && !b.flag;
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const bool in = row_in && b.bx[k] >= 0 && b.bx[k] < W;
+                tin[4 * r + k] = in;
+                toff[4 * r + k] = in ? ((int64_t)b.by[r] * W + b.bx[k]) * C : 0;
+            }
+            tw[r] = b.cx[r];
+            tw[4 + r] = b.cy[r];
+        }
+        if (b.flag) {
+            tw[0] = __builtin_nanf("");  // 0 * NaN: every channel becomes NaN, as the reference writes
+        }
+    } else {
+        const PixelTap t = decide_pixel<(INTERP == 2 ? 0 : INTERP), PAD, ALIGN>(gx, gy, H, W);
+        if (INTERP == 0) {
+            const int32_t x0 = t.x0, y0 = t.y0;
+            const int32_t x1 = (x0 == INT32_MAX) ? x0 : x0 + 1;
+            const int32_t y1 = (y0 == INT32_MAX) ? y0 : y0 + 1;
+            const int32_t xs[4] = {x0, x1, x0, x1};
+            const int32_t ys[4] = {y0, y0, y1, y1};
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const bool in = within(ys[k], xs[k], H, W) && !t.flag;
+                tin[k % NT] = in;
+                toff[k % NT] = in ? ((int64_t)ys[k] * W + xs[k]) * C : 0;
+                tw[k] = t.w[k];
+            }
+            if (t.flag) {
+                tw[0] = __builtin_nanf("");
+            }
+        } else {
+            const bool in = within(t.y0, t.x0, H, W);
+            tin[0] = in;
+            toff[0] = in ? ((int64_t)t.y0 * W + t.x0) * C : 0;
+            tw[0] = tw[1] = tw[2] = tw[3] = 0.0f;
+        }
+    }
+
+    const T* xn = x + n * (int64_t)H * W * C;
+    T* yp = y + p * C;
+    const int32_t runs = C / V;  // VEC: C % V == 0
+    for (int32_t cv = sub; cv < runs; cv += lpp) {
+        const int32_t c = cv * V;
+        T tap[NT][V];
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            if constexpr (VEC) {
+                uint4 raw = *reinterpret_cast<const uint4*>(xn + toff[t] + c);
+                if (!tin[t]) {
+                    raw = make_uint4(0u, 0u, 0u, 0u);
+                }
+                __builtin_memcpy(tap[t], &raw, 16);
+            } else {
+                T v = xn[toff[t] + c];
+                if (!tin[t]) {
+                    ElemIO<T>::store(&v, 0.0f);
+                }
+                tap[t][0] = v;
+            }
+        }
+        T outv[V];
+#pragma unroll
+        for (int i = 0; i < V; i++) {
+            T raw[NT];
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                raw[t] = tap[t][i];
+            }
+            ElemIO<T>::store(&outv[i], blend<T, INTERP>(raw, tw, neg_zero));
+        }
+        if constexpr (VEC) {
+            uint4 packed;
+            __builtin_memcpy(&packed, outv, 16);
+            *reinterpret_cast<uint4*>(yp + c) = packed;
+        } else {
+            yp[c] = outv[0];
+        }
+    }
+}
+
+struct NhwcLauncher {
+    const GridSamplerArgs& a;
+    hipStream_t stream;
+    template <typename T, int I, int P, bool A>
+    hipError_t operator()() const
+    {
+        constexpr int V = 16 / (int)sizeof(T);
+        const bool vec = a.C % V == 0 && reinterpret_cast<uintptr_t>(a.x) % 16 == 0 &&
+                         reinterpret_cast<uintptr_t>(a.y) % 16 == 0;
+        const int64_t runs = vec ? a.C / V : a.C;
+        int shift = 0;
+        while (shift < 4 && (2ll << shift) <= runs) {
+            shift++;
+        }
+        const int64_t total = a.N * a.Hout * a.Wout;
+        const int64_t per_block = kNhwcThreads >> shift;
+        const int64_t blocks = (total + per_block - 1) / per_block;
+        if (blocks > INT32_MAX) {
+            return hipErrorInvalidValue;
+        }
+        if (vec) {
+            hipLaunchKernelGGL((gs2d_nhwc_kernel<T, I, P, A, true>), dim3((unsigned)blocks), dim3(kNhwcThreads), 0, stream,
+                               (const T*)a.x, (const T*)a.grid, (T*)a.y, total, (int32_t)a.C, (int32_t)a.Hin,
+                               (int32_t)a.Win, a.Hout * a.Wout, shift, -0.0f);
+        } else {
+            hipLaunchKernelGGL((gs2d_nhwc_kernel<T, I, P, A, false>), dim3((unsigned)blocks), dim3(kNhwcThreads), 0, stream,
+                               (const T*)a.x, (const T*)a.grid, (T*)a.y, total, (int32_t)a.C, (int32_t)a.Hin,
+                               (int32_t)a.Win, a.Hout * a.Wout, shift, -0.0f);
+        }
+        return hipGetLastError();
+    }
+};
+
+}  // namespace
+
+hipError_t run_gs2d_nhwc(const GridSamplerArgs& a, hipStream_t stream)
+{
+    return dispatch_elem(a, NhwcLauncher{a, stream});
+}
+
+}  // namespace opscv

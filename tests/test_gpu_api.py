@@ -201,3 +201,44 @@ def test_resize_strided_views(oracle, device, aclnn):
     ref = oracle.resize_nearest(xv.contiguous().cpu().numpy(), (14, 16))
     assert np.array_equal(ov.cpu().numpy(), ref)
     assert float(outbig[:, :, :, 1::2].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("dtype", I.DTYPES)
+@pytest.mark.parametrize("interp", [0, 1, 2])
+def test_grid_sampler_channels_last_views(oracle, device, aclnn, dtype, interp):
+    """input and out handed over as channels_last views (N,C,H,W dims, NHWC memory): sampled in place by the
+    channels-last kernel, bit-exact against the oracle; vector (C % 8 or 4 == 0) and scalar channel counts"""
+    import torch
+    rng = np.random.default_rng(400 + interp)
+    for (N, C, H, W, Ho, Wo, pad, align) in [(2, 16, 9, 11, 13, 7, 0, False), (1, 64, 32, 32, 40, 24, 1, True),
+                                             (2, 5, 7, 6, 9, 9, 2, False), (1, 24, 5, 8, 4, 33, 0, True),
+                                             (1, 3, 1, 1, 5, 5, 1, False)]:
+        x = I.cast_np(rng.standard_normal((N, C, H, W)).astype(np.float32), dtype)
+        g = I.cast_np(rng.uniform(-1.3, 1.3, (N, Ho, Wo, 2)).astype(np.float32), dtype)
+        if C >= 16:
+            g[0, 0, 0] = np.array([np.nan, 0.0]).astype(np.float32).view(np.float32) if dtype == "fp32" else g[0, 0, 0]
+        ref = oracle.grid_sampler2d(x, g, interp, pad, align, dtype=I.oracle_code(dtype))
+        xt = I.to_torch(x, dtype, device).contiguous(memory_format=torch.channels_last)
+        gt = I.to_torch(g, dtype, device)
+        out = torch.empty((N, C, Ho, Wo), dtype=xt.dtype, device=device).contiguous(memory_format=torch.channels_last)
+        hs = [aclnn.tensor_handle(xt), aclnn.tensor_handle(gt), aclnn.tensor_handle(out)]
+        st, ws, ex = aclnn.get_workspace_size_grid_sampler2d(hs[0], hs[1], interp, pad, align, hs[2])
+        assert st == 0
+        expect_inplace = C > 1 and (H * W > 1) and (Ho * Wo > 1)
+        if expect_inplace:
+            assert ws == 0 and aclnn.executor_variant(ex) == "nhwc"
+        aclnn.destroy_executor(ex)
+        for h in hs:
+            aclnn.destroy_tensor(h)
+        y = aclnn.grid_sampler2d(xt, gt, interp, pad, align, out=out)
+        torch.cuda.synchronize()
+        got = I.from_torch(y.contiguous(), dtype)
+        nan = np.isnan(I.as_f32(ref, dtype))
+        assert np.array_equal(np.isnan(I.as_f32(got, dtype)), nan)
+        view = np.uint32 if dtype == "fp32" else np.uint16
+        assert np.array_equal(np.where(nan, 0, got.view(view)), np.where(nan, 0, ref.view(view))), (N, C, H, W, pad, align)
+        # mixed layouts fall back to packing and give the same result
+        out2 = aclnn.grid_sampler2d(xt, gt, interp, pad, align)
+        torch.cuda.synchronize()
+        got2 = I.from_torch(out2, dtype)
+        assert np.array_equal(np.where(nan, 0, got2.view(view)), np.where(nan, 0, ref.view(view)))
