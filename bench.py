@@ -150,7 +150,7 @@ class Timed:
         self.stream_us = None
 
 
-def bench_gs(name, steps, warmup, interp=None, pad=None, align=None, sets=None, check=True):
+def bench_gs(name, steps, warmup, interp=None, pad=None, align=None, sets=None, check=True, channels_last=False):
     import numpy as np
     import torch
     import inputs as I
@@ -177,6 +177,10 @@ def bench_gs(name, steps, warmup, interp=None, pad=None, align=None, sets=None, 
         xs.append(I.to_torch(x, w["dtype"], dev))
         gs.append(I.to_torch(g, w["dtype"], dev))
         ys.append(torch.empty((N, C, Ho, Wo), dtype=xs[-1].dtype, device=dev))
+        if channels_last:
+            # (N,C,H,W) views over NHWC memory, as a framework's channels_last tensors are handed over
+            xs[-1] = xs[-1].contiguous(memory_format=torch.channels_last)
+            ys[-1] = ys[-1].contiguous(memory_format=torch.channels_last)
         hx.append(aclnn.tensor_handle(xs[-1]))
         hg.append(aclnn.tensor_handle(gs[-1]))
         hy.append(aclnn.tensor_handle(ys[-1]))
@@ -216,10 +220,11 @@ def bench_gs(name, steps, warmup, interp=None, pad=None, align=None, sets=None, 
     samples = N * C * Ho * Wo
     e = esize(w["dtype"])
     alg_bytes = (N * C * H * W + N * Ho * Wo * 2 + samples) * e
-    desc = "%s grid_sampler2d %s x%s grid%s %s %s align_corners=%s" % (
-        name, w["dtype"], tuple(w["x"]), (N, Ho, Wo, 2), INTERP_NAMES[w["interp"]], PAD_NAMES[w["pad"]], w["align"])
+    desc = "%s grid_sampler2d %s x%s grid%s %s %s align_corners=%s%s" % (
+        name, w["dtype"], tuple(w["x"]), (N, Ho, Wo, 2), INTERP_NAMES[w["interp"]], PAD_NAMES[w["pad"]], w["align"],
+        " channels_last views" if channels_last else "")
     return dict(workload=desc, samples=samples, alg_bytes=alg_bytes, timed=t, variant=variant, parity=parity,
-                sets=nsets, cpu=(x0, g0, w), default_modes=(interp is None and pad is None and align is None))
+                sets=nsets, cpu=(x0, g0, w), default_modes=(interp is None and pad is None and align is None and not channels_last))
 
 
 def bench_up(name, steps, warmup, sets=None, check=True):
@@ -413,6 +418,8 @@ def main():
                     others["C3_%s_%s" % (INTERP_NAMES[interp], PAD_NAMES[pad])] = summary_of(rr)
             rr = bench_gs("C3", args.steps, args.warmup, sets=1)
             others["C3_bilinear_zeros_same_buffers_every_step"] = summary_of(rr)
+            others["C3_bilinear_zeros_channels_last"] = summary_of(bench_gs("C3", args.steps, args.warmup,
+                                                                             channels_last=True))
             # the third interpolation mode on the same tensors (not part of the headline set)
             others["C3_bicubic_zeros"] = summary_of(bench_gs("C3", max(10, args.steps // 2), args.warmup, interp=2))
         for name in ("C1", "C5"):
