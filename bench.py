@@ -29,6 +29,8 @@ HBM_PEAK_GBS = 8000.0
 MEASURED_TRAFFIC = {
     ("C3", "lds_ring_p8208_2x4"): 69.41e6,   # profiles/gs2d_lds_ring_C3_fp16_n16_c256.md
     ("C4", "nchw_band_lds"): 1415.4e6,       # profiles/resize_band_lds_C4_fp16_4k_upscale.md
+    ("C2", "nchw_flat_lds"): 33.08e6,        # profiles/resize_flat_lds_C2_fp32_56_to_112.md
+    ("C5", "lds_ring_p32784_1x4"): 176.4e6,  # profiles/gs2d_lds_ring_C5_bf16_random_gather.md
 }
 
 # name -> description of the workloads (shapes as in the baseline configuration list)
