@@ -156,6 +156,19 @@ __device__ __forceinline__ void lds_barrier()
     asm volatile("" ::: "memory");
 }
 
+// Bank-spreading layout of a staged plane whose rows are exactly 128 bytes (row_shift = 7; 0 = plain layout).
+// LDS has 32 four-byte banks, i.e. 128 bytes per "line"; with that row pitch column x of every row falls into the
+// same bank, and coordinates clamped to the first or last column (border padding) make a wavefront read one bank
+// 64 times.  The 16-byte chunks of each line are therefore permuted by the low three bits of the row number:
+// byte offset o of the plane lives at o ^ ((row & 7) << 4).  The permutation stays inside the line, so it maps the
+// plane onto itself.  The copy applies it to the source address (the LDS side of the asynchronous copy is fixed per
+// lane); a copy instruction covers eight whole rows starting at a multiple of 1 KiB, so the permuted source offset
+// of a lane inside that block is a per-lane constant.  The samplers apply it once per tap when they compute offsets.
+__device__ __forceinline__ uint32_t lds_swizzle(uint32_t byte_off, uint32_t row_shift)
+{
+    return row_shift ? (byte_off ^ (((byte_off >> row_shift) & 7u) << 4)) : byte_off;
+}
+
 // Starts the asynchronous copy of `nch` consecutive input planes (plane_bytes each, contiguous in global memory
 // from `src`) to LDS at `dst` with PITCH bytes between planes.  G = bytes per lane (16 or 4): the largest
 // granule that divides the plane size and the source alignment.  Each wavefront instruction moves 64*G
@@ -164,7 +177,7 @@ __device__ __forceinline__ void lds_barrier()
 // instructions issued per plane by this wavefront is copies_per_plane() below.
 template <int G, int LWAVES, int CGS, int PITCH>
 __device__ __forceinline__ void issue_stage_copy(const char* src, char* dst, uint32_t plane_bytes, int nch,
-                                                 uint32_t lwave, uint32_t lane)
+                                                 uint32_t lwave, uint32_t lane, uint32_t lane_src_off)
 {
     constexpr uint32_t CHUNK = 64u * G;
     const uint32_t lane_off = lane * G;
@@ -175,7 +188,8 @@ __device__ __forceinline__ void issue_stage_copy(const char* src, char* dst, uin
             char* dp = dst + k * PITCH;
             for (uint32_t base = lwave * CHUNK; base < plane_bytes; base += LWAVES * CHUNK) {
                 if (base + lane_off < plane_bytes) {
-                    const global_cptr_t gsrc = (global_cptr_t)(sp + base + lane_off);
+                    // lane_src_off: the chunk of this 1 KiB block that belongs at the lane's LDS position
+                    const global_cptr_t gsrc = (global_cptr_t)(sp + base + lane_src_off);
                     const lds_ptr_t ldst = (lds_ptr_t)(dp + base);
                     // the size operand must be a literal
                     if constexpr (G == 16) {
@@ -204,7 +218,7 @@ template <typename T, int INTERP, int PAD, bool ALIGN, int SWAVES, int LWAVES, i
 __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves_per_eu(1, 5))) void gs2d_lds_kernel(
     const T* __restrict__ x, const T* __restrict__ grid, T* __restrict__ y, int32_t C, int32_t H, int32_t W,
     int32_t out_plane, uint32_t tiles_per_n, uint32_t cblocks, int32_t chans_per_block, int32_t copy_gran,
-    int32_t pair_aligned, int32_t xcd_swizzle, float neg_zero)
+    int32_t pair_aligned, int32_t xcd_swizzle, int32_t row_shift, float neg_zero)
 {
     extern __shared__ uint4 smem_raw[];
     char* lds = reinterpret_cast<char*>(smem_raw);
@@ -254,13 +268,14 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
             const int32_t left = nchan - s * CGS;
             return left < CGS ? left : CGS;
         };
+        const uint32_t lane_src16 = lds_swizzle(lane * 16u, (uint32_t)row_shift);
         auto start_stage = [&](int32_t s, int slot) {
             const char* src = xb + (size_t)s * stage_bytes;
             char* dst = lds + slot * SLOT_BYTES;
             if (copy_gran == 16) {
-                issue_stage_copy<16, LWAVES, CGS, PITCH>(src, dst, plane_bytes, planes_of(s), lwave, lane);
+                issue_stage_copy<16, LWAVES, CGS, PITCH>(src, dst, plane_bytes, planes_of(s), lwave, lane, lane_src16);
             } else {
-                issue_stage_copy<4, LWAVES, CGS, PITCH>(src, dst, plane_bytes, planes_of(s), lwave, lane);
+                issue_stage_copy<4, LWAVES, CGS, PITCH>(src, dst, plane_bytes, planes_of(s), lwave, lane, lane * 4u);
             }
         };
 #pragma unroll
@@ -315,7 +330,9 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
                 for (int k = 0; k < 4; k++) {
                     const bool in = row_in && b.bx[k] >= 0 && b.bx[k] < W;
                     toff[j][4 * r + k] =
-                        in ? ((uint32_t)b.by[r] * (uint32_t)W + (uint32_t)b.bx[k]) * (uint32_t)sizeof(T) : zero_off;
+                        in ? lds_swizzle(((uint32_t)b.by[r] * (uint32_t)W + (uint32_t)b.bx[k]) * (uint32_t)sizeof(T),
+                                         (uint32_t)row_shift)
+                           : zero_off;
                 }
                 tw[j][r] = b.cx[r];
                 tw[j][4 + r] = b.cy[r];
@@ -333,10 +350,11 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
             const bool in_nw = within(y0, x0, H, W), in_ne = within(y0, x1, H, W);
             const bool in_sw = within(y1, x0, H, W), in_se = within(y1, x1, H, W);
             const uint32_t uw = (uint32_t)W, es = (uint32_t)sizeof(T);
-            toff[j][0] = in_nw ? ((uint32_t)y0 * uw + (uint32_t)x0) * es : zero_off;
-            toff[j][1] = in_ne ? ((uint32_t)y0 * uw + (uint32_t)x1) * es : zero_off;
-            toff[j][2] = in_sw ? ((uint32_t)y1 * uw + (uint32_t)x0) * es : zero_off;
-            toff[j][3] = in_se ? ((uint32_t)y1 * uw + (uint32_t)x1) * es : zero_off;
+            const uint32_t rs = (uint32_t)row_shift;
+            toff[j][0] = in_nw ? lds_swizzle(((uint32_t)y0 * uw + (uint32_t)x0) * es, rs) : zero_off;
+            toff[j][1] = in_ne ? lds_swizzle(((uint32_t)y0 * uw + (uint32_t)x1) * es, rs) : zero_off;
+            toff[j][2] = in_sw ? lds_swizzle(((uint32_t)y1 * uw + (uint32_t)x0) * es, rs) : zero_off;
+            toff[j][3] = in_se ? lds_swizzle(((uint32_t)y1 * uw + (uint32_t)x1) * es, rs) : zero_off;
             tw[j][0] = t.w[0];
             tw[j][1] = t.w[1];
             tw[j][2] = t.w[2];
@@ -348,7 +366,9 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
             }
         } else {
             const bool in = within(t.y0, t.x0, H, W);
-            toff[j][0] = in ? ((uint32_t)t.y0 * (uint32_t)W + (uint32_t)t.x0) * (uint32_t)sizeof(T) : zero_off;
+            toff[j][0] = in ? lds_swizzle(((uint32_t)t.y0 * (uint32_t)W + (uint32_t)t.x0) * (uint32_t)sizeof(T),
+                                          (uint32_t)row_shift)
+                            : zero_off;
             tw[j][0] = tw[j][1] = tw[j][2] = tw[j][3] = 0.0f;
         }
     }

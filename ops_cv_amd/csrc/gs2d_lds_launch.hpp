@@ -15,6 +15,7 @@ struct LdsPlan {
     int ppt = 4;
     int copy_gran = 16;
     int xcd_swizzle = 0;
+    int row_shift = 0;  // 7 when the staged planes (128-byte rows) use the bank-spreading layout, else 0
     uint32_t lds_bytes = 0;
     uint32_t tiles_per_n = 0, cblocks = 0;
     int32_t chans_per_block = 0;
@@ -51,7 +52,8 @@ hipError_t launch_one(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t st
     const uint32_t blocks = (uint32_t)(a.N * p.tiles_per_n * p.cblocks);
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3((kSamplerWaves + LWAVES) * 64), p.lds_bytes, stream, (const T*)a.x, (const T*)a.grid,
                        (T*)a.y, (int32_t)a.C, (int32_t)a.Hin, (int32_t)a.Win, (int32_t)(a.Hout * a.Wout),
-                       p.tiles_per_n, p.cblocks, p.chans_per_block, p.copy_gran, pair_aligned, p.xcd_swizzle, -0.0f);
+                       p.tiles_per_n, p.cblocks, p.chans_per_block, p.copy_gran, pair_aligned, p.xcd_swizzle, p.row_shift,
+                       -0.0f);
     return hipGetLastError();
 }
 
