@@ -268,7 +268,7 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
             const int32_t left = nchan - s * CGS;
             return left < CGS ? left : CGS;
         };
-        const uint32_t lane_src16 = lds_swizzle(lane * 16u, (uint32_t)row_shift);
+        const uint32_t lane_src16 = lds_swizzle(lane * 16u, (PAD == 1) ? (uint32_t)row_shift : 0u);
         auto start_stage = [&](int32_t s, int slot) {
             const char* src = xb + (size_t)s * stage_bytes;
             char* dst = lds + slot * SLOT_BYTES;
@@ -313,14 +313,22 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
     uint32_t toff[PPT][NT];
     float tw[PPT][NW];
     uint32_t pixoff[PPT];  // byte offset of the pixel inside an output plane; out of range for lanes past the end
+    // all grid points of the lane are requested before the first is used: one memory latency, not PPT of them
+    float gxs[PPT], gys[PPT];
+    const T* gridn = grid + (int64_t)n * out_plane * 2;
 #pragma unroll
     for (int j = 0; j < PPT; j++) {
         const int32_t pix = (int32_t)tile * (STHREADS * PPT) + j * STHREADS + tid;
         const bool valid = pix < out_plane;
         const int32_t pc = valid ? pix : out_plane - 1;
         pixoff[j] = valid ? (uint32_t)pc * (uint32_t)sizeof(T) : 0x80000000u;
-        float gx, gy;
-        load_grid_pair<T>(grid + ((int64_t)n * out_plane + pc) * 2, pair_aligned != 0, &gx, &gy);
+        load_grid_pair<T>(gridn + (int64_t)pc * 2, pair_aligned != 0, &gxs[j], &gys[j]);
+    }
+    // the bank-spreading layout exists for border padding only (see make_lds_plan)
+    const uint32_t rs = (PAD == 1) ? (uint32_t)row_shift : 0u;
+#pragma unroll
+    for (int j = 0; j < PPT; j++) {
+        const float gx = gxs[j], gy = gys[j];
         if constexpr (INTERP == 2) {
             const BicubicTap b = decide_bicubic<PAD, ALIGN>(gx, gy, H, W);
 #pragma unroll
@@ -330,8 +338,7 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
                 for (int k = 0; k < 4; k++) {
                     const bool in = row_in && b.bx[k] >= 0 && b.bx[k] < W;
                     toff[j][4 * r + k] =
-                        in ? lds_swizzle(((uint32_t)b.by[r] * (uint32_t)W + (uint32_t)b.bx[k]) * (uint32_t)sizeof(T),
-                                         (uint32_t)row_shift)
+                        in ? lds_swizzle(((uint32_t)b.by[r] * (uint32_t)W + (uint32_t)b.bx[k]) * (uint32_t)sizeof(T), rs)
                            : zero_off;
                 }
                 tw[j][r] = b.cx[r];
@@ -342,33 +349,51 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
             }
             continue;
         }
-        const PixelTap t = decide_pixel<(INTERP == 2 ? 0 : INTERP), PAD, ALIGN>(gx, gy, H, W);
+        // Bilinear and nearest: the decisions of decide_pixel() (sampler_math.hpp; grid_sampler2_d_simt.h:479-498,
+        // 307-316, 341-349) written without branches -- this prologue runs once per workgroup for every one of its
+        // pixels and is on the critical path to the first sampled stage, so its instruction count matters.
+        // Bounds tests are single unsigned compares (a negative index is a huge unsigned one), tap offsets follow
+        // from the north-west one by modular arithmetic, and the "+1" of an index saturated at INT32_MAX wraps to
+        // 0x80000000, which is out of bounds like the saturated value itself.
+        float ix = compute_source_index<PAD, ALIGN>(gx, W);
+        float iy = compute_source_index<PAD, ALIGN>(gy, H);
+        const bool finite = __builtin_fabsf(ix) < __builtin_inff() && __builtin_fabsf(iy) < __builtin_inff();
+        const bool x_far = ix > 2147483646.0f || ix < -2147483648.0f;  // safe_downgrade: -> -100, always outside
+        const bool y_far = iy > 2147483646.0f || iy < -2147483648.0f;
+        const uint32_t uw = (uint32_t)W, uh = (uint32_t)H, es = (uint32_t)sizeof(T);
         if (INTERP == 0) {
-            const int32_t x0 = t.x0, y0 = t.y0;
-            const int32_t x1 = (x0 == INT32_MAX) ? x0 : x0 + 1;
-            const int32_t y1 = (y0 == INT32_MAX) ? y0 : y0 + 1;
-            const bool in_nw = within(y0, x0, H, W), in_ne = within(y0, x1, H, W);
-            const bool in_sw = within(y1, x0, H, W), in_se = within(y1, x1, H, W);
-            const uint32_t uw = (uint32_t)W, es = (uint32_t)sizeof(T);
-            const uint32_t rs = (uint32_t)row_shift;
-            toff[j][0] = in_nw ? lds_swizzle(((uint32_t)y0 * uw + (uint32_t)x0) * es, rs) : zero_off;
-            toff[j][1] = in_ne ? lds_swizzle(((uint32_t)y0 * uw + (uint32_t)x1) * es, rs) : zero_off;
-            toff[j][2] = in_sw ? lds_swizzle(((uint32_t)y1 * uw + (uint32_t)x0) * es, rs) : zero_off;
-            toff[j][3] = in_se ? lds_swizzle(((uint32_t)y1 * uw + (uint32_t)x1) * es, rs) : zero_off;
-            tw[j][0] = t.w[0];
-            tw[j][1] = t.w[1];
-            tw[j][2] = t.w[2];
-            tw[j][3] = t.w[3];
-            if (t.flag) {
-                // non-finite source coordinate: every channel becomes NaN (0 * NaN), as the reference writes
-                toff[j][0] = toff[j][1] = toff[j][2] = toff[j][3] = zero_off;
-                tw[j][0] = __builtin_nanf("");
-            }
+            ix = x_far ? -100.0f : ix;
+            iy = y_far ? -100.0f : iy;
+            const float ixf = __builtin_floorf(ix), iyf = __builtin_floorf(iy);
+            const uint32_t x0 = (uint32_t)float_to_i32(ixf), y0 = (uint32_t)float_to_i32(iyf);
+            const uint32_t x1 = x0 + 1u, y1 = y0 + 1u;
+            const bool in_x0 = x0 < uw && finite, in_x1 = x1 < uw && finite;
+            const bool in_y0 = y0 < uh, in_y1 = y1 < uh;
+            const uint32_t o_nw = (y0 * uw + x0) * es;
+            const uint32_t o_sw = o_nw + uw * es;
+            toff[j][0] = (in_y0 && in_x0) ? lds_swizzle(o_nw, rs) : zero_off;
+            toff[j][1] = (in_y0 && in_x1) ? lds_swizzle(o_nw + es, rs) : zero_off;
+            toff[j][2] = (in_y1 && in_x0) ? lds_swizzle(o_sw, rs) : zero_off;
+            toff[j][3] = (in_y1 && in_x1) ? lds_swizzle(o_sw + es, rs) : zero_off;
+            const float wx1 = ix - ixf, wx0 = ixf + 1.0f - ix;
+            const float wy1 = iy - iyf, wy0 = iyf + 1.0f - iy;
+            // non-finite source coordinate: every tap reads the zero slot and 0 * NaN makes every channel NaN,
+            // as the reference writes (grid_sampler2_d_simt.h:485-487)
+            tw[j][0] = finite ? wx0 * wy0 : __builtin_nanf("");
+            tw[j][1] = wx1 * wy0;
+            tw[j][2] = wx0 * wy1;
+            tw[j][3] = wx1 * wy1;
         } else {
-            const bool in = within(t.y0, t.x0, H, W);
-            toff[j][0] = in ? lds_swizzle(((uint32_t)t.y0 * (uint32_t)W + (uint32_t)t.x0) * (uint32_t)sizeof(T),
-                                          (uint32_t)row_shift)
-                            : zero_off;
+            ix = (x_far || !finite) ? -100.0f : ix;
+            iy = (y_far || !finite) ? -100.0f : iy;
+            // round half to even from floor, fraction and parity (grid_sampler2_d_simt.h:219-234)
+            const float xf = __builtin_floorf(ix), yf = __builtin_floorf(iy);
+            const float fx = ix - xf, fy = iy - yf;
+            const uint32_t xi = (uint32_t)float_to_i32(xf), yi = (uint32_t)float_to_i32(yf);
+            const uint32_t xr = xi + ((fx > 0.5f || (fx == 0.5f && (xi & 1u))) ? 1u : 0u);
+            const uint32_t yr = yi + ((fy > 0.5f || (fy == 0.5f && (yi & 1u))) ? 1u : 0u);
+            const bool in = xr < uw && yr < uh;
+            toff[j][0] = in ? lds_swizzle((yr * uw + xr) * es, rs) : zero_off;
             tw[j][0] = tw[j][1] = tw[j][2] = tw[j][3] = 0.0f;
         }
     }
