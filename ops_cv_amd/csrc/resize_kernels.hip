@@ -179,10 +179,14 @@ __global__ __launch_bounds__(kThreads) void resize_nhwc_generic_kernel(const T* 
     }
 }
 
-// Vector NHWC variant: one lane per 16-byte run of channels of an output pixel (V = 16/sizeof(T) channels, needs
-// C % V == 0 and 16-byte aligned tensors).  The four taps are 16-byte loads that neighbouring lanes extend to
-// whole pixels, the result is one 16-byte store; per channel the arithmetic is the reference formula.
-template <typename T, bool HALF_PIXEL>
+// Vector NHWC variant: one lane per 16-byte run of channels of an output column (V = 16/sizeof(T) channels, needs
+// C % V == 0 and 16-byte aligned tensors), walking down a band of BAND output rows.  The reference formula is
+// separable as written, so the horizontally blended source row  (1-dx)*x[y,x0,c] + dx*x[y,x1,c]  stays in
+// registers and is reused by every output row of the band that touches source row y (two of them for a x2
+// upscale): two 16-byte loads per source row instead of four per output row, same operations in the same order.
+constexpr int kNhwcBand = 8;
+
+template <typename T, bool HALF_PIXEL, int BAND>
 __global__ __launch_bounds__(kThreads) void resize_nhwc_vec_kernel(const T* __restrict__ x, T* __restrict__ y,
                                                                     int64_t N, int32_t C, int32_t Hs, int32_t Ws,
                                                                     int32_t Hd, int32_t Wd, float scale_h,
@@ -202,38 +206,60 @@ __global__ __launch_bounds__(kThreads) void resize_nhwc_vec_kernel(const T* __re
     const float omdx = 1.0f - dx;
     const int64_t o0 = (int64_t)tx.i0 * C + c;
     const int64_t o1 = (int64_t)tx.i1 * C + c;
-    const int64_t rows = N * Hd;
     const int64_t src_row = (int64_t)Ws * C;
-    for (int64_t r = blockIdx.y; r < rows; r += gridDim.y) {
-        const int64_t n = r / Hd;
-        const int32_t h = (int32_t)(r - n * Hd);
-        const AxisTap ty = axis_tap<HALF_PIXEL>(h, scale_h, Hs);
-        const float dy = ty.lambda;
-        const float omdy = 1.0f - dy;
-        const T* top = x + (n * Hs + ty.i0) * src_row;
-        const T* bot = x + (n * Hs + ty.i1) * src_row;
-        T tl[V], tr[V], bl[V], br[V], outv[V];
-        uint4 raw;
-        raw = *reinterpret_cast<const uint4*>(top + o0);
-        __builtin_memcpy(tl, &raw, 16);
-        raw = *reinterpret_cast<const uint4*>(top + o1);
-        __builtin_memcpy(tr, &raw, 16);
-        raw = *reinterpret_cast<const uint4*>(bot + o0);
-        __builtin_memcpy(bl, &raw, 16);
-        raw = *reinterpret_cast<const uint4*>(bot + o1);
-        __builtin_memcpy(br, &raw, 16);
+    const int32_t h_begin = blockIdx.y * BAND;
+    const int32_t h_end = (h_begin + BAND < Hd) ? h_begin + BAND : Hd;
+    for (int64_t n = blockIdx.z; n < N; n += gridDim.z) {
+        const T* xn = x + n * Hs * src_row;
+        float ha[V], hb[V];  // blended source rows ya and yb
+        int32_t ya = -1, yb = -1;
+        auto blend_row = [&](float* hrow, int32_t ys) {
+            const T* row = xn + (int64_t)ys * src_row;
+            T l[V], r[V];
+            uint4 raw = *reinterpret_cast<const uint4*>(row + o0);
+            __builtin_memcpy(l, &raw, 16);
+            raw = *reinterpret_cast<const uint4*>(row + o1);
+            __builtin_memcpy(r, &raw, 16);
 #pragma unroll
-        for (int i = 0; i < V; i++) {
-            const float t = omdx * ElemIO<T>::load(&tl[i]) + dx * ElemIO<T>::load(&tr[i]);
-            const float b = omdx * ElemIO<T>::load(&bl[i]) + dx * ElemIO<T>::load(&br[i]);
-            ElemIO<T>::store(&outv[i], omdy * t + dy * b);
-        }
-        __builtin_memcpy(&raw, outv, 16);
-        uint4* dst = reinterpret_cast<uint4*>(y + (r * row_vecs + e) * V);
-        if (streaming) {
-            store_streaming(dst, raw);
-        } else {
-            *dst = raw;
+            for (int i = 0; i < V; i++) {
+                hrow[i] = omdx * ElemIO<T>::load(&l[i]) + dx * ElemIO<T>::load(&r[i]);
+            }
+        };
+        for (int32_t h = h_begin; h < h_end; h++) {
+            const AxisTap ty = axis_tap<HALF_PIXEL>(h, scale_h, Hs);
+            const int32_t y0 = __builtin_amdgcn_readfirstlane(ty.i0);
+            const int32_t y1 = __builtin_amdgcn_readfirstlane(ty.i1);
+            const float dy = ty.lambda;
+            const float omdy = 1.0f - dy;
+            if (y0 != ya) {
+                if (y0 == yb) {
+#pragma unroll
+                    for (int i = 0; i < V; i++) {
+                        ha[i] = hb[i];
+                    }
+                } else {
+                    blend_row(ha, y0);
+                }
+                ya = y0;
+            }
+            if (y1 != ya && y1 != yb) {
+                blend_row(hb, y1);
+                yb = y1;
+            }
+            T outv[V];
+#pragma unroll
+            for (int i = 0; i < V; i++) {
+                const float bot = (y1 == ya) ? ha[i] : hb[i];
+                ElemIO<T>::store(&outv[i], omdy * ha[i] + dy * bot);
+            }
+            uint4 raw;
+            __builtin_memcpy(&raw, outv, 16);
+            uint4* dst = reinterpret_cast<uint4*>(y + ((n * Hd + h) * row_vecs + e) * V);
+            if (streaming) {
+                store_streaming(dst, raw);
+            } else {
+                *dst = raw;
+            }
         }
     }
 }
@@ -248,6 +274,8 @@ __device__ __forceinline__ int32_t nearest_src(int32_t d, float scale, int32_t l
     const int32_t i = (f >= 2147483648.0f) ? INT32_MAX : (int32_t)f;
     return (i < len_src - 1) ? i : len_src - 1;
 }
+
+constexpr int kNearestBand = 8;
 
 // A pure gather-copy: V = 16/sizeof(T) (VEC) or 1 output elements per lane along the contiguous axis.
 // NCHW: the contiguous axis is w, each element has its own source column.  NHWC: the contiguous axis is (w, c);
@@ -277,7 +305,11 @@ __global__ __launch_bounds__(kThreads) void resize_nearest_kernel(const T* __res
         }
     }
     const int64_t rows = outer * Hd;  // outer = N*C planes (NCHW) or N images (NHWC)
-    for (int64_t r = blockIdx.y; r < rows; r += gridDim.y) {
+    // a workgroup copies kNearestBand consecutive output rows per step: the column offsets above are reused and
+    // neighbouring output rows of an upscale read the same source row out of L1
+    for (int64_t r0 = (int64_t)blockIdx.y * kNearestBand; r0 < rows; r0 += (int64_t)gridDim.y * kNearestBand) {
+      const int64_t r_end = (r0 + kNearestBand < rows) ? r0 + kNearestBand : rows;
+      for (int64_t r = r0; r < r_end; r++) {
         const int64_t o = r / Hd;
         const int32_t h = (int32_t)(r - o * Hd);
         const T* src = x + (o * Hs + nearest_src(h, scale_h, Hs)) * src_row_elems;
@@ -302,6 +334,7 @@ __global__ __launch_bounds__(kThreads) void resize_nearest_kernel(const T* __res
         } else {
             dst[0] = src[src_off[0]];
         }
+      }
     }
 }
 
@@ -354,7 +387,8 @@ bool nhwc_vec_ok(const ResizeArgs& a)
 {
     constexpr int V = 16 / (int)sizeof(T);
     return a.channels_last && a.mode == ResizeMode::Bilinear && a.C % V == 0 &&
-           reinterpret_cast<uintptr_t>(a.x) % 16 == 0 && reinterpret_cast<uintptr_t>(a.y) % 16 == 0;
+           (a.Hd + kNhwcBand - 1) / kNhwcBand <= 65535 && reinterpret_cast<uintptr_t>(a.x) % 16 == 0 &&
+           reinterpret_cast<uintptr_t>(a.y) % 16 == 0;
 }
 
 template <typename T>
@@ -385,7 +419,8 @@ hipError_t run_resize(const ResizeArgs& a, hipStream_t stream)
         // whole 16-byte vectors: rows start aligned (row_elems % V == 0); for NHWC a vector stays inside one pixel
         const bool vec = aligned && row_elems % V == 0 && (!nhwc || (a.C % V == 0 && (a.Ws * a.C) % V == 0));
         const int64_t lanes = vec ? row_elems / V : row_elems;
-        dim3 grid((unsigned)((lanes + kThreads - 1) / kThreads), (unsigned)(rows < 65535 ? rows : 65535));
+        const int64_t bands = (rows + kNearestBand - 1) / kNearestBand;
+        dim3 grid((unsigned)((lanes + kThreads - 1) / kThreads), (unsigned)(bands < 65535 ? bands : 65535));
 #define OPSCV_NEAREST(NHWC_, VEC_)                                                                                  \
     hipLaunchKernelGGL((resize_nearest_kernel<T, NHWC_, VEC_>), grid, dim3(kThreads), 0, stream, x, y, outer,      \
                        (int32_t)a.C, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h, a.scale_w, \
@@ -410,15 +445,16 @@ hipError_t run_resize(const ResizeArgs& a, hipStream_t stream)
     if (nhwc_vec_ok<T>(a)) {
         constexpr int V = 16 / (int)sizeof(T);
         const int64_t row_vecs = a.Wd * (a.C / V);
-        const int64_t rows = a.N * a.Hd;
+        const int64_t bands = (a.Hd + kNhwcBand - 1) / kNhwcBand;
         const int streaming = (out_elems * (int64_t)sizeof(T) >= (128ll << 20)) ? 1 : 0;
-        dim3 grid((unsigned)((row_vecs + kThreads - 1) / kThreads), (unsigned)(rows < 65535 ? rows : 65535));
+        dim3 grid((unsigned)((row_vecs + kThreads - 1) / kThreads), (unsigned)bands,
+                  (unsigned)(a.N < 65535 ? a.N : 65535));
         if (a.half_pixel) {
-            hipLaunchKernelGGL((resize_nhwc_vec_kernel<T, true>), grid, dim3(kThreads), 0, stream, x, y, a.N,
+            hipLaunchKernelGGL((resize_nhwc_vec_kernel<T, true, kNhwcBand>), grid, dim3(kThreads), 0, stream, x, y, a.N,
                                (int32_t)a.C, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h,
                                a.scale_w, streaming);
         } else {
-            hipLaunchKernelGGL((resize_nhwc_vec_kernel<T, false>), grid, dim3(kThreads), 0, stream, x, y, a.N,
+            hipLaunchKernelGGL((resize_nhwc_vec_kernel<T, false, kNhwcBand>), grid, dim3(kThreads), 0, stream, x, y, a.N,
                                (int32_t)a.C, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h,
                                a.scale_w, streaming);
         }
