@@ -103,6 +103,12 @@ def load_library():
     L.aclnnResizeGetWorkspaceSize.argtypes = [vp, vp, ctypes.c_char_p, vp, ctypes.POINTER(u64), ctypes.POINTER(vp)]
     L.aclnnResize.restype = i32
     L.aclnnResize.argtypes = [vp, u64, vp, vp]
+    L.aclnnUpsampleBilinear2dBackwardGetWorkspaceSize.restype = i32
+    L.aclnnUpsampleBilinear2dBackwardGetWorkspaceSize.argtypes = [vp, vp, vp, ctypes.c_bool, ctypes.c_double,
+                                                                  ctypes.c_double, vp, ctypes.POINTER(u64),
+                                                                  ctypes.POINTER(vp)]
+    L.aclnnUpsampleBilinear2dBackward.restype = i32
+    L.aclnnUpsampleBilinear2dBackward.argtypes = [vp, u64, vp, vp]
     L.opscvGridSampler2DTaps.restype = i32
     L.opscvGridSampler2DTaps.argtypes = [vp, ctypes.c_int, i64, i64, i64, i64, i64, i64, i64, ctypes.c_bool, vp, vp]
     L.opscvGridSampler2DBicubicTaps.restype = i32
@@ -187,6 +193,17 @@ def get_workspace_size_resize(self_t, scales, mode, out):
     ws = ctypes.c_uint64(0)
     ex = ctypes.c_void_p(None)
     st = L.aclnnResizeGetWorkspaceSize(self_t, scales, mode, out, ctypes.byref(ws), ctypes.byref(ex))
+    return st, ws.value, ex.value
+
+
+def get_workspace_size_upsample_bilinear2d_backward(grad_out, output_size, input_size, align_corners, scales_h,
+                                                    scales_w, out):
+    L = load_library()
+    ws = ctypes.c_uint64(0)
+    ex = ctypes.c_void_p(None)
+    st = L.aclnnUpsampleBilinear2dBackwardGetWorkspaceSize(grad_out, output_size, input_size, bool(align_corners),
+                                                           float(scales_h), float(scales_w), out, ctypes.byref(ws),
+                                                           ctypes.byref(ex))
     return st, ws.value, ex.value
 
 
@@ -320,6 +337,40 @@ def resize(self_t, scales, mode="bilinear", out=None, stream=None, channels_last
         for h in hs:
             destroy_tensor(h)
         destroy_float_array(sc)
+    return out
+
+
+def upsample_bilinear2d_backward(grad_out, input_size, align_corners=False, scales_h=0.0, scales_w=0.0, out=None,
+                                 stream=None, channels_last=False, out_dtype=None, workspace=None):
+    """Both phases of aclnnUpsampleBilinear2dBackward.  `input_size` holds the four extents of the tensor that was
+    upsampled, in the order of the tensors' layout (NCHW, or NHWC when channels_last)."""
+    torch = _torch()
+    L = load_library()
+    fmt = ACL_FORMAT_NHWC if channels_last else ACL_FORMAT_NCHW
+    if out is None:
+        out = torch.empty(tuple(input_size), dtype=grad_out.dtype if out_dtype is None else out_dtype,
+                          device=grad_out.device)
+    hw = (1, 2) if channels_last else (2, 3)
+    hs = [tensor_handle(grad_out, fmt), tensor_handle(out, fmt)]
+    osz = create_int_array([grad_out.shape[hw[0]], grad_out.shape[hw[1]]])
+    isz = create_int_array(list(input_size))
+    try:
+        st, ws, ex = get_workspace_size_upsample_bilinear2d_backward(hs[0], osz, isz, align_corners, scales_h,
+                                                                     scales_w, hs[1])
+        if st != ACLNN_SUCCESS:
+            raise AclnnError("aclnnUpsampleBilinear2dBackwardGetWorkspaceSize", st)
+        if ws > 0 and (workspace is None or workspace.numel() * workspace.element_size() < ws):
+            workspace = torch.empty(ws, dtype=torch.uint8, device=grad_out.device)
+        wptr = ctypes.c_void_p(workspace.data_ptr()) if ws > 0 else None
+        wsize = workspace.numel() * workspace.element_size() if ws > 0 else 0
+        st = L.aclnnUpsampleBilinear2dBackward(wptr, wsize, ex, _stream_handle(stream))
+        if st != ACLNN_SUCCESS:
+            raise AclnnError("aclnnUpsampleBilinear2dBackward", st)
+    finally:
+        for h in hs:
+            destroy_tensor(h)
+        destroy_int_array(osz)
+        destroy_int_array(isz)
     return out
 
 

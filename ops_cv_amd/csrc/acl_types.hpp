@@ -74,7 +74,7 @@ struct StridedView {
     int64_t strides[4] = {0};  // elements
 };
 
-enum class OpKind : int { Nop = 0, GridSampler2D = 1, Resize = 2 };
+enum class OpKind : int { Nop = 0, GridSampler2D = 1, Resize = 2, ResizeGrad = 3 };
 
 // Where a kernel operand lives: the tensor's own memory (contiguous view) or a slice of the caller's
 // workspace, known only as an offset until the second phase receives the workspace address.
@@ -109,6 +109,21 @@ struct ResizeArgs {
     void* y = nullptr;
 };
 
+// Backward of the bilinear resize.  "src" is the tensor that was upsampled (the extents of the result `y`), "dst"
+// the upsampled one (the extents of the incoming gradient `x`).
+struct ResizeGradArgs {
+    Elem elem_in = Elem::F32;   // gradient coming in
+    Elem elem_out = Elem::F32;  // gradient going out
+    int copy = 0;               // equal sizes: y = x
+    int user_scales = 0;        // scales that are not the ratio of the sizes: the user-scale template
+    int half_pixel = 1;
+    int channels_last = 0;
+    float scale_h = 1.0f, scale_w = 1.0f, inv_scale_h = 1.0f, inv_scale_w = 1.0f;
+    int64_t N = 0, C = 0, Hs = 0, Ws = 0, Hd = 0, Wd = 0;
+    const void* x = nullptr;
+    void* y = nullptr;
+};
+
 }  // namespace opscv
 
 constexpr uint32_t kExecutorMagic = 0x0C5CA11Du;
@@ -119,6 +134,7 @@ struct aclOpExecutor {
     uint64_t workspace_bytes = 0;
     opscv::GridSamplerArgs gs;  // pointer members are filled in by the second phase
     opscv::ResizeArgs rs;
+    opscv::ResizeGradArgs rg;
     opscv::PlannedPtr in0, in1, out0;  // input/self, grid, out
     // packing work: views gathered into the workspace before the kernel, scattered after it
     struct Pack {

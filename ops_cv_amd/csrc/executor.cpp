@@ -93,6 +93,15 @@ aclnnStatus run_executor(void* workspace, uint64_t workspace_size, aclOpExecutor
             return ACLNN_ERR_PARAM_NULLPTR;
         }
         e = launch_grid_sampler2d(a, s);
+    } else if (ex->kind == OpKind::ResizeGrad) {
+        ResizeGradArgs a = ex->rg;
+        a.x = resolve(ex->in0, workspace);
+        a.y = resolve(ex->out0, workspace);
+        if (a.x == nullptr || a.y == nullptr) {
+            set_error("%s: tensor data pointer is NULL", api);
+            return ACLNN_ERR_PARAM_NULLPTR;
+        }
+        e = launch_resize_grad(a, s);
     } else {
         ResizeArgs a = ex->rs;
         a.x = resolve(ex->in0, workspace);

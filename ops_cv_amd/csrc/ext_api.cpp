@@ -92,6 +92,7 @@ const char* opscvExecutorVariant(const aclOpExecutor* executor)
     switch (executor->kind) {
         case OpKind::GridSampler2D: return grid_sampler2d_variant(executor->gs);
         case OpKind::Resize: return resize_variant(executor->rs);
+        case OpKind::ResizeGrad: return executor->rg.copy ? "copy" : (executor->rg.user_scales ? "resize_grad_gather_scales" : "resize_grad_gather");
         default: break;
     }
     return "";

@@ -23,6 +23,8 @@
  *                                  (3,16), committed torch interpolate fixtures, live torch CPU comparison
  *   oracle_resize_nearest        : integer-factor upscales equal element repetition, committed and live
  *                                  torch interpolate(mode="nearest") comparison (bit-exact: a pure copy)
+ *   oracle_upsample_bilinear2d_backward : adjointness with the forward oracle (<forward(x), g> = <x, backward(g)>),
+ *                                  gradient mass conservation, x2 closed form, live torch autograd comparison
  *   oracle_resize_scale          : float bit patterns held by the reference's tiling UT
  *                                  (image/resize_bilinear_v2/tests/ut/op_host/arch35/test_resize_bilinear_v2_tiling.cpp)
  */
@@ -670,6 +672,115 @@ int oracle_resize_nearest(const void* x, void* y, int dtype, int64_t N, int64_t 
                         dof = ((n * C + c) * Hd + h) * Wd + w;
                     }
                     memcpy(dst + dof * esz, src + so * esz, (size_t)esz);
+                }
+            }
+        }
+    }
+    return 0;
+}
+
+/* resize_bilinear_v2_grad_tiling_arch35.cpp:352-394 (deterministic templates) */
+static float grad_scale(int64_t len_src, int64_t len_dst, int align_corners, float user_scale)
+{
+    if (align_corners) {
+        if (len_src > 1 && len_dst > 1) {
+            return (float)(len_src - 1) / (float)(len_dst - 1);
+        }
+        return (float)len_src / (float)len_dst;
+    }
+    if (user_scale > 0.0f) {
+        return 1.0f / user_scale;
+    }
+    return (float)len_src / (float)len_dst;
+}
+
+/* resize_bilinear_v2_grad_simt_determine_scales.h:55-63 */
+static float grad_source_index(float scale, int64_t i, int half_pixel)
+{
+    return half_pixel ? scale * ((float)i + 0.5f) - 0.5f : scale * (float)i;
+}
+
+int oracle_upsample_bilinear2d_backward(const void* grads, void* y, int dtype_in, int dtype_out, int64_t N, int64_t C,
+                                        int64_t Hs, int64_t Ws, int64_t Hd, int64_t Wd, int align_corners,
+                                        int channels_last, double scales_h, double scales_w)
+{
+    if (dtype_in < 0 || dtype_in > 2 || dtype_out < 0 || dtype_out > 2 || Hs <= 0 || Ws <= 0 || Hd <= 0 || Wd <= 0) {
+        return -1;
+    }
+    const float scale_h = grad_scale(Hs, Hd, align_corners, (float)scales_h);
+    const float scale_w = grad_scale(Ws, Wd, align_corners, (float)scales_w);
+    const float inv_h = 1.0f / scale_h, inv_w = 1.0f / scale_w;
+    const int half_pixel = !align_corners;
+    const float offset = half_pixel ? 0.5f : 0.0f;
+    /* template choice: resize_bilinear_v2_grad_tiling_arch35.cpp:422-436 */
+    const int user_scales = !align_corners && (fabsf((float)Hs / (float)Hd - scale_h) >= 1.1920929e-7f ||
+                                               fabsf((float)Ws / (float)Wd - scale_w) >= 1.1920929e-7f);
+    for (int64_t n = 0; n < N; n++) {
+        for (int64_t c = 0; c < C; c++) {
+            for (int64_t H = 0; H < Hs; H++) {
+                for (int64_t W = 0; W < Ws; W++) {
+                    /* start of the walk: resize_bilinear_v2_grad_simt_determine.h:83-91 (both templates) */
+                    float fy0 = ceilf(((float)H - 1.0f + offset) * inv_h - offset);
+                    float fx0 = ceilf(((float)W - 1.0f + offset) * inv_w - offset);
+                    int64_t in_y_start = (fy0 > 0.0f) ? (int64_t)fy0 : 0;
+                    int64_t in_x_start = (fx0 > 0.0f) ? (int64_t)fx0 : 0;
+                    float out_y_start = ((float)in_y_start + offset) * scale_h - offset;
+                    float out_x_start = ((float)in_x_start + offset) * scale_w - offset;
+                    /* first/last row or column: only in the user-scale template (…determine_scales.h:264-282) */
+                    int hb = user_scales && (H == 0 || H == Hs - 1);
+                    int wb = user_scales && (W == 0 || W == Ws - 1);
+                    float acc = 0.0f;
+                    float out_y = out_y_start;
+                    int64_t in_y = in_y_start;
+                    while ((hb || out_y < (float)H + 1.0f) && in_y < Hd) {
+                        float out_x = out_x_start;
+                        int64_t in_x = in_x_start;
+                        while ((wb || out_x < (float)W + 1.0f) && in_x < Wd) {
+                            int64_t gi = channels_last ? ((n * Hd + in_y) * Wd + in_x) * C + c
+                                                       : ((n * C + c) * Hd + in_y) * Wd + in_x;
+                            float g = load_as_float(grads, dtype_in, gi);
+                            float yc = fmaxf(0.0f, fminf(out_y, (float)Hs - 1.0f));
+                            float xc = fmaxf(0.0f, fminf(out_x, (float)Ws - 1.0f));
+                            float y_lerp = 1.0f - fabsf(yc - (float)H);
+                            float x_lerp = 1.0f - fabsf(xc - (float)W);
+                            if (!hb && !wb) {
+                                acc += g * y_lerp * x_lerp;
+                            } else {
+                                float yt = fminf(floorf(yc), (float)(Hs - 1));
+                                float xt = fminf(floorf(xc), (float)(Ws - 1));
+                                float lepy[2] = {y_lerp, yc - yt};
+                                float lepx[2] = {x_lerp, xc - xt};
+                                if (!hb) {
+                                    for (int j = 0; j < 2; j++) {
+                                        if (xt + (float)j == (float)W) {
+                                            acc += g * lepx[j] * y_lerp;
+                                        }
+                                    }
+                                } else if (!wb) {
+                                    for (int i = 0; i < 2; i++) {
+                                        if (yt + (float)i == (float)H) {
+                                            acc += g * lepy[i] * x_lerp;
+                                        }
+                                    }
+                                } else {
+                                    for (int i = 0; i < 2; i++) {
+                                        for (int j = 0; j < 2; j++) {
+                                            if (yt + (float)i == (float)H && xt + (float)j == (float)W) {
+                                                acc += g * lepx[j] * lepy[i];
+                                            }
+                                        }
+                                    }
+                                }
+                            }
+                            in_x++;
+                            /* the plain template accumulates the coordinate, the user-scale one recomputes it */
+                            out_x = user_scales ? grad_source_index(scale_w, in_x, half_pixel) : out_x + scale_w;
+                        }
+                        in_y++;
+                        out_y = user_scales ? grad_source_index(scale_h, in_y, half_pixel) : out_y + scale_h;
+                    }
+                    int64_t yi = channels_last ? ((n * Hs + H) * Ws + W) * C + c : ((n * C + c) * Hs + H) * Ws + W;
+                    store_from_float(y, dtype_out, yi, acc);
                 }
             }
         }

@@ -100,6 +100,18 @@ int oracle_upsample_bilinear2d(const void* x, void* y, int dtype, int64_t N, int
 int oracle_resize_nearest(const void* x, void* y, int dtype, int64_t N, int64_t C, int64_t Hs, int64_t Ws,
                           int64_t Hd, int64_t Wd, int channels_last);
 
+/*
+ * Backward of the bilinear resize, deterministic gather formulation
+ * (image/resize_bilinear_v2_grad/op_kernel/arch35/resize_bilinear_v2_grad_simt_determine.h:56-117; scales
+ * image/resize_bilinear_v2_grad/op_host/arch35/resize_bilinear_v2_grad_tiling_arch35.cpp:352-394).
+ * scales_h/scales_w > 0 (align_corners false) that differ from Hd/Hs, Wd/Ws follow the user-scale template
+ * resize_bilinear_v2_grad_simt_determine_scales.h:77-305.
+ * grads: (N,C,Hd,Wd) or channels_last (N,Hd,Wd,C), dtype_in; y: (N,C,Hs,Ws) / (N,Hs,Ws,C), dtype_out.
+ */
+int oracle_upsample_bilinear2d_backward(const void* grads, void* y, int dtype_in, int dtype_out, int64_t N, int64_t C,
+                                        int64_t Hs, int64_t Ws, int64_t Hd, int64_t Wd, int align_corners,
+                                        int channels_last, double scales_h, double scales_w);
+
 /* per-axis tap table of the upsample: i0[len_dst], i1[len_dst], lambda[len_dst] */
 int oracle_upsample_axis_taps(int64_t len_src, int64_t len_dst, int align_corners, float user_scale, int32_t* i0,
                               int32_t* i1, float* lambda);

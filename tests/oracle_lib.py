@@ -80,6 +80,9 @@ def lib():
                                                      ctypes.c_int]
     L.oracle_resize_nearest.restype = ctypes.c_int
     L.oracle_resize_nearest.argtypes = [vp, vp, ctypes.c_int, i64, i64, i64, i64, i64, i64, ctypes.c_int]
+    L.oracle_upsample_bilinear2d_backward.restype = ctypes.c_int
+    L.oracle_upsample_bilinear2d_backward.argtypes = [vp, vp, ctypes.c_int, ctypes.c_int, i64, i64, i64, i64, i64,
+                                                      i64, ctypes.c_int, ctypes.c_int, ctypes.c_double, ctypes.c_double]
     L.oracle_resize_scale.restype = f32
     L.oracle_resize_scale.argtypes = [i64, i64, ctypes.c_int, f32]
     L.oracle_upsample_bilinear2d.restype = ctypes.c_int
@@ -159,6 +162,27 @@ def resize_nearest(x, out_hw, channels_last=False, dtype=None):
     rc = lib().oracle_resize_nearest(_ptr(x), _ptr(y), code, N, C, Hs, Ws, out_hw[0], out_hw[1], int(channels_last))
     if rc != 0:
         raise ValueError("oracle_resize_nearest rc=%d" % rc)
+    return y
+
+
+def upsample_bilinear2d_backward(grads, in_hw, align=False, channels_last=False, dtype=None, out_dtype=None,
+                                 out_numpy_dtype=None, scales_h=0.0, scales_w=0.0):
+    """grads (N,C,Hd,Wd) or channels_last (N,Hd,Wd,C) -> gradient of the (.., in_hw) tensor that was upsampled"""
+    grads = np.ascontiguousarray(grads)
+    code = _code_of(grads) if dtype is None else dtype
+    ocode = code if out_dtype is None else out_dtype
+    if channels_last:
+        N, Hd, Wd, C = grads.shape
+        shape = (N, in_hw[0], in_hw[1], C)
+    else:
+        N, C, Hd, Wd = grads.shape
+        shape = (N, C, in_hw[0], in_hw[1])
+    y = np.empty(shape, dtype=grads.dtype if out_numpy_dtype is None else out_numpy_dtype)
+    rc = lib().oracle_upsample_bilinear2d_backward(_ptr(grads), _ptr(y), code, ocode, N, C, in_hw[0], in_hw[1], Hd, Wd,
+                                                   int(bool(align)), int(channels_last), float(scales_h),
+                                                   float(scales_w))
+    if rc != 0:
+        raise ValueError("oracle_upsample_bilinear2d_backward rc=%d" % rc)
     return y
 
 

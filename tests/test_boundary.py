@@ -3,7 +3,8 @@
 The cases mirror the reference's op_api unit tests, which build descriptors with NULL data pointers and call only
 the GetWorkspaceSize phase: image/grid_sample/tests/ut/op_host/op_api/test_aclnn_grid_sampler2d.cpp and
 image/upsample_bilinear2d/tests/ut/op_host/op_api/test_aclnn_upsample_bilinear_2d.cpp,
-image/resize_bilinear_v2/tests/ut/op_host/op_api/test_aclnn_resize.cpp.
+image/resize_bilinear_v2/tests/ut/op_host/op_api/test_aclnn_resize.cpp,
+image/resize_bilinear_v2_grad/tests/ut/op_host/op_api/test_aclnn_upsample_bilineard_2d_backward.cpp.
 """
 import ctypes
 import os
@@ -290,3 +291,61 @@ def test_resize_status_codes(aclnn, desc):
     assert _rs(aclnn, desc, out=(1, 1, 2, 2), scales=(1, 1, 1, 1))[2] == "copy"
     assert _rs(aclnn, desc, inp=(1, 1, 1, 1), out=(1, 1, 4, 4), scales=(1, 1, 4, 4))[2] == "broadcast"
     assert _rs(aclnn, desc, inp=(0, 1, 2, 2), out=(0, 1, 4, 4))[:2] == (0, 0)
+
+
+def _ub(aclnn, desc, grad=(1, 1, 2, 2), out=(1, 1, 3, 3), osize=(2, 2), isize=(1, 1, 3, 3), dt=None, odt=None, fmt=None,
+        ofmt=None, align=False, sh=2.0, sw=2.0):
+    dt = aclnn.ACL_FLOAT if dt is None else dt
+    fmt = aclnn.ACL_FORMAT_NCHW if fmt is None else fmt
+    g = desc.t(grad, dt, fmt)
+    o = desc.t(out, dt if odt is None else odt, fmt if ofmt is None else ofmt)
+    a1 = aclnn.create_int_array(list(osize)) if osize is not None else None
+    a2 = aclnn.create_int_array(list(isize)) if isize is not None else None
+    st, ws, ex = aclnn.get_workspace_size_upsample_bilinear2d_backward(g, a1, a2, align, sh, sw, o)
+    variant = aclnn.executor_variant(ex) if ex else None
+    if ex:
+        aclnn.destroy_executor(ex)
+    aclnn.destroy_int_array(a1)
+    aclnn.destroy_int_array(a2)
+    return st, ws, variant
+
+
+def test_upsample_backward_status_codes(aclnn, desc):
+    """test_aclnn_upsample_bilineard_2d_backward.cpp cases 001-017 and the checks of
+    aclnn_upsample_bilinear_2d_backward.cpp:48-230"""
+    INV, NULL = aclnn.ACLNN_ERR_PARAM_INVALID, aclnn.ACLNN_ERR_PARAM_NULLPTR
+    # 001/002 (+ bf16, supported on the newest parts): scales 2.0 with sizes 2x2 <- 3x3 do not match the size ratio:
+    # accepted, the user-scale template runs
+    for dt in (aclnn.ACL_FLOAT, aclnn.ACL_FLOAT16, aclnn.ACL_BF16):
+        assert _ub(aclnn, desc, dt=dt) == (0, 0, "resize_grad_gather_scales")
+    assert _ub(aclnn, desc, sh=0.0, sw=0.0)[2] == "resize_grad_gather"
+    assert _ub(aclnn, desc, align=True)[2] == "resize_grad_gather"
+    # 003-012: unsupported dtypes
+    for dt in (aclnn.ACL_DOUBLE, aclnn.ACL_INT32):
+        assert _ub(aclnn, desc, dt=dt)[0] == INV
+    # 013: empty tensor
+    assert _ub(aclnn, desc, grad=(0, 1, 2, 2), out=(0, 1, 3, 3), isize=(0, 1, 3, 3))[:2] == (0, 0)
+    # 014/015: rank
+    assert _ub(aclnn, desc, grad=(2, 2))[0] == INV
+    assert _ub(aclnn, desc, grad=(1, 1, 1, 2, 2))[0] == INV
+    # 016: null arguments
+    assert _ub(aclnn, desc, grad=None)[0] == NULL
+    assert _ub(aclnn, desc, out=None)[0] == NULL
+    assert _ub(aclnn, desc, osize=None)[0] == NULL
+    assert _ub(aclnn, desc, isize=None)[0] == NULL
+    # 017: out dtype; a FLOAT gradient may be reduced into a 16-bit out, a 16-bit one may not change type
+    assert _ub(aclnn, desc, odt=aclnn.ACL_FLOAT16)[0] == 0
+    assert _ub(aclnn, desc, dt=aclnn.ACL_FLOAT16, odt=aclnn.ACL_FLOAT)[0] == INV
+    # sizes: array lengths, positive extents, gradOut == (N,C,outputSize), out == inputSize
+    assert _ub(aclnn, desc, osize=(2, 2, 2))[0] == INV
+    assert _ub(aclnn, desc, isize=(1, 3, 3))[0] == INV
+    assert _ub(aclnn, desc, osize=(0, 2), grad=(1, 1, 0, 2))[0] == INV
+    assert _ub(aclnn, desc, osize=(3, 2))[0] == INV
+    assert _ub(aclnn, desc, out=(1, 1, 3, 4))[0] == INV
+    assert _ub(aclnn, desc, out=(1, 2, 3, 3))[0] == INV
+    # formats: equal, NCHW or NHWC; NHWC reads the four extents as N,H,W,C
+    assert _ub(aclnn, desc, ofmt=aclnn.ACL_FORMAT_NHWC)[0] == INV
+    assert _ub(aclnn, desc, grad=(1, 2, 2, 5), out=(1, 3, 3, 5), isize=(1, 3, 3, 5), fmt=aclnn.ACL_FORMAT_NHWC,
+               sh=0, sw=0) == (0, 0, "resize_grad_gather")
+    # equal sizes: a copy
+    assert _ub(aclnn, desc, grad=(1, 1, 3, 3), osize=(3, 3), sh=1.0, sw=1.0)[2] == "copy"

@@ -242,3 +242,48 @@ def test_grid_sampler_channels_last_views(oracle, device, aclnn, dtype, interp):
         torch.cuda.synchronize()
         got2 = I.from_torch(out2, dtype)
         assert np.array_equal(np.where(nan, 0, got2.view(view)), np.where(nan, 0, ref.view(view)))
+
+
+@pytest.mark.parametrize("dtype", I.DTYPES)
+@pytest.mark.parametrize("channels_last", [False, True])
+def test_upsample_backward(oracle, device, aclnn, dtype, channels_last):
+    """aclnnUpsampleBilinear2dBackward: bit-exact against the oracle's restatement of the reference's deterministic
+    templates (size-ratio and user scales), NCHW and NHWC, and reproducible from run to run"""
+    import torch
+    rng = np.random.default_rng(500 + int(channels_last))
+    cases = [((2, 3, 5, 7), (10, 14), False, 0.0, 0.0), ((1, 4, 8, 8), (3, 5), True, 0.0, 0.0),
+             ((2, 2, 16, 16), (33, 47), False, 0.0, 0.0), ((1, 5, 1, 5), (4, 10), True, 0.0, 0.0),
+             ((1, 2, 4, 6), (10, 10), False, 2.5, 1.7), ((2, 1, 8, 8), (4, 3), False, 0.6, 0.45),
+             ((1, 3, 6, 6), (6, 6), False, 0.0, 0.0), ((1, 8, 56, 56), (112, 112), False, 2.0, 2.0)]
+    for in_shape, (Ho, Wo), align, sh, sw in cases:
+        N, C, H, W = in_shape
+        g = I.cast_np(rng.standard_normal((N, C, Ho, Wo)).astype(np.float32), dtype)
+        gin = np.ascontiguousarray(g.transpose(0, 2, 3, 1)) if channels_last else g
+        isz = (N, H, W, C) if channels_last else (N, C, H, W)
+        ref = oracle.upsample_bilinear2d_backward(gin, (H, W), align, channels_last=channels_last,
+                                                  dtype=I.oracle_code(dtype), scales_h=sh, scales_w=sw)
+        gt = I.to_torch(gin, dtype, device)
+        y1 = I.from_torch(aclnn.upsample_bilinear2d_backward(gt, isz, align, sh, sw, channels_last=channels_last), dtype)
+        y2 = I.from_torch(aclnn.upsample_bilinear2d_backward(gt, isz, align, sh, sw, channels_last=channels_last), dtype)
+        torch.cuda.synchronize()
+        view = np.uint32 if dtype == "fp32" else np.uint16
+        assert np.array_equal(y1.view(view), ref.view(view)), (in_shape, Ho, Wo, align, sh, sw, dtype, channels_last)
+        assert np.array_equal(y1.view(view), y2.view(view))
+
+
+def test_upsample_backward_fp32_into_fp16(oracle, device, aclnn):
+    """a FLOAT gradient reduced into a FLOAT16 result, and a strided gradient view"""
+    import torch
+    rng = np.random.default_rng(510)
+    g = rng.standard_normal((2, 3, 12, 10)).astype(np.float32)
+    ref = oracle.upsample_bilinear2d_backward(g, (6, 5), False, dtype=oracle.F32, out_dtype=oracle.F16,
+                                              out_numpy_dtype=np.float16)
+    y = aclnn.upsample_bilinear2d_backward(torch.from_numpy(g).to(device), (2, 3, 6, 5), False, out_dtype=torch.float16)
+    torch.cuda.synchronize()
+    assert np.array_equal(y.cpu().numpy().view(np.uint16), ref.view(np.uint16))
+    big = torch.from_numpy(rng.standard_normal((2, 3, 12, 20)).astype(np.float32)).to(device)
+    gv = big[:, :, :, ::2]
+    y = aclnn.upsample_bilinear2d_backward(gv, (2, 3, 6, 5), False)
+    torch.cuda.synchronize()
+    ref = oracle.upsample_bilinear2d_backward(gv.contiguous().cpu().numpy(), (6, 5), False)
+    assert np.array_equal(y.cpu().numpy(), ref)

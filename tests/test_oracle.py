@@ -456,3 +456,41 @@ def test_resize_nearest_oracle(oracle):
     assert np.array_equal(oracle.resize_nearest(xh, (9, 11)),
                           F.interpolate(torch.from_numpy(xh.astype(np.float32)), size=(9, 11),
                                         mode="nearest").numpy().astype(np.float16))
+
+
+def test_upsample_backward_oracle(oracle):
+    """resize_bilinear_v2_grad_simt_determine.h / _determine_scales.h: the gather form is the adjoint of the
+    forward resize (<forward(x), g> = <x, backward(g)>), keeps the gradient mass when no source pixel is skipped,
+    and agrees with torch autograd on both templates (size-ratio scales and user scales)"""
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(88)
+    for (H, W, Ho, Wo) in [(5, 7, 10, 14), (4, 4, 9, 6), (8, 8, 3, 5), (1, 5, 4, 10), (6, 6, 13, 13), (3, 2, 3, 9)]:
+        for align in (False, True):
+            x = rng.standard_normal((2, 3, H, W)).astype(np.float32)
+            g = rng.standard_normal((2, 3, Ho, Wo)).astype(np.float32)
+            fwd = oracle.upsample_bilinear2d(x, (Ho, Wo), align)
+            bwd = oracle.upsample_bilinear2d_backward(g, (H, W), align)
+            lhs = float((fwd.astype(np.float64) * g).sum())
+            rhs = float((x.astype(np.float64) * bwd).sum())
+            assert abs(lhs - rhs) <= 1e-4 * max(1.0, abs(lhs)), (H, W, Ho, Wo, align)
+            assert abs(float(bwd.sum(dtype=np.float64)) - float(g.sum(dtype=np.float64))) <= 1e-3
+            xt = torch.from_numpy(x).requires_grad_(True)
+            F.interpolate(xt, size=(Ho, Wo), mode="bilinear", align_corners=align).backward(torch.from_numpy(g))
+            assert np.abs(bwd - xt.grad.numpy()).max() <= 1e-5, (H, W, Ho, Wo, align)
+            # channels-last layout gives the same numbers
+            gl = np.ascontiguousarray(g.transpose(0, 2, 3, 1))
+            bl = oracle.upsample_bilinear2d_backward(gl, (H, W), align, channels_last=True)
+            assert np.array_equal(bl.transpose(0, 3, 1, 2), bwd)
+    # user scales that are not the ratio of the sizes (the second template)
+    for (H, W, sh, sw) in [(4, 6, 2.5, 1.7), (8, 8, 0.6, 0.45), (3, 9, 3.3, 1.2), (5, 5, 1.9, 2.0)]:
+        xt = torch.randn(2, 2, H, W, requires_grad=True)
+        yt = F.interpolate(xt, scale_factor=(sh, sw), mode="bilinear", align_corners=False,
+                           recompute_scale_factor=False)
+        g = rng.standard_normal(tuple(yt.shape)).astype(np.float32)
+        yt.backward(torch.from_numpy(g))
+        bwd = oracle.upsample_bilinear2d_backward(g, (H, W), False, scales_h=sh, scales_w=sw)
+        assert np.abs(bwd - xt.grad.numpy()).max() <= 1e-5, (H, W, sh, sw)
+    # x2 of a single source pixel: all the gradient lands on it
+    g = np.arange(4, dtype=np.float32).reshape(1, 1, 2, 2)
+    assert oracle.upsample_bilinear2d_backward(g, (1, 1), False)[0, 0, 0, 0] == 6.0
