@@ -36,6 +36,8 @@ ACL_FORMAT_NCHW = 0
 ACL_FORMAT_NHWC = 1
 ACL_FORMAT_ND = 2
 ACL_FORMAT_HWCN = 16
+ACL_FORMAT_NDHWC = 27
+ACL_FORMAT_NCDHW = 30
 
 ACLNN_SUCCESS = 0
 ACLNN_ERR_PARAM_NULLPTR = 161001
@@ -94,6 +96,10 @@ def load_library():
     L.aclnnGridSampler2DGetWorkspaceSize.argtypes = [vp, vp, i64, i64, ctypes.c_bool, vp, p_u64, p_vp]
     L.aclnnGridSampler2D.restype = i32
     L.aclnnGridSampler2D.argtypes = [vp, u64, vp, vp]
+    L.aclnnGridSampler3DGetWorkspaceSize.restype = i32
+    L.aclnnGridSampler3DGetWorkspaceSize.argtypes = [vp, vp, i64, i64, ctypes.c_bool, vp, p_u64, p_vp]
+    L.aclnnGridSampler3D.restype = i32
+    L.aclnnGridSampler3D.argtypes = [vp, u64, vp, vp]
     L.aclnnUpsampleBilinear2dGetWorkspaceSize.restype = i32
     L.aclnnUpsampleBilinear2dGetWorkspaceSize.argtypes = [vp, vp, ctypes.c_bool, ctypes.c_double, ctypes.c_double,
                                                          vp, p_u64, p_vp]
@@ -164,6 +170,16 @@ def get_workspace_size_grid_sampler2d(inp, grid, interpolation_mode, padding_mod
     ws = ctypes.c_uint64(0)
     ex = ctypes.c_void_p(None)
     st = L.aclnnGridSampler2DGetWorkspaceSize(inp, grid, interpolation_mode, padding_mode, bool(align_corners), out,
+                                              ctypes.byref(ws), ctypes.byref(ex))
+    return st, ws.value, ex.value
+
+
+def get_workspace_size_grid_sampler3d(inp, grid, interpolation_mode, padding_mode, align_corners, out):
+    """Phase 1 of aclnnGridSampler3D on raw handles; returns (status, workspace_bytes, executor_handle)."""
+    L = load_library()
+    ws = ctypes.c_uint64(0)
+    ex = ctypes.c_void_p(None)
+    st = L.aclnnGridSampler3DGetWorkspaceSize(inp, grid, interpolation_mode, padding_mode, bool(align_corners), out,
                                               ctypes.byref(ws), ctypes.byref(ex))
     return st, ws.value, ex.value
 
@@ -271,6 +287,41 @@ def grid_sampler2d(inp, grid, interpolation_mode=0, padding_mode=0, align_corner
         st = L.aclnnGridSampler2D(wptr, wsize, ex, _stream_handle(stream))
         if st != ACLNN_SUCCESS:
             raise AclnnError("aclnnGridSampler2D", st)
+    finally:
+        for h in hs:
+            destroy_tensor(h)
+    return out
+
+
+def grid_sampler3d(inp, grid, interpolation_mode=0, padding_mode=0, align_corners=False, out=None, stream=None,
+                   channels_last=False, workspace=None):
+    """Both phases of aclnnGridSampler3D on torch CUDA tensors.
+
+    inp is (N,C,D,H,W) and the result (N,C,Do,Ho,Wo); with channels_last inp is (N,D,H,W,C) and the result
+    (N,Do,Ho,Wo,C) (format NDHWC).  grid is (N,Do,Ho,Wo,3).
+    """
+    torch = _torch()
+    L = load_library()
+    fmt = ACL_FORMAT_NDHWC if channels_last else ACL_FORMAT_NCDHW
+    if out is None:
+        if channels_last:
+            shape = (inp.shape[0], grid.shape[1], grid.shape[2], grid.shape[3], inp.shape[4])
+        else:
+            shape = (inp.shape[0], inp.shape[1], grid.shape[1], grid.shape[2], grid.shape[3])
+        out = torch.empty(shape, dtype=inp.dtype, device=inp.device)
+    hs = [tensor_handle(inp, fmt), tensor_handle(grid), tensor_handle(out, fmt)]
+    try:
+        st, ws, ex = get_workspace_size_grid_sampler3d(hs[0], hs[1], interpolation_mode, padding_mode,
+                                                       align_corners, hs[2])
+        if st != ACLNN_SUCCESS:
+            raise AclnnError("aclnnGridSampler3DGetWorkspaceSize", st)
+        if ws > 0 and (workspace is None or workspace.numel() * workspace.element_size() < ws):
+            workspace = torch.empty(ws, dtype=torch.uint8, device=inp.device)
+        wptr = ctypes.c_void_p(workspace.data_ptr()) if ws > 0 else None
+        wsize = workspace.numel() * workspace.element_size() if ws > 0 else 0
+        st = L.aclnnGridSampler3D(wptr, wsize, ex, _stream_handle(stream))
+        if st != ACLNN_SUCCESS:
+            raise AclnnError("aclnnGridSampler3D", st)
     finally:
         for h in hs:
             destroy_tensor(h)

@@ -67,14 +67,16 @@ inline bool elem_of(aclDataType dt, Elem* e)
     }
 }
 
-// A 4-D strided view that has to be packed into (or scattered from) a contiguous workspace slice.
+// A strided view of up to five dimensions (shorter ones are padded in front with extent 1) that has to be packed
+// into (or scattered from) a contiguous workspace slice.
+constexpr int kViewDims = 5;
 struct StridedView {
-    void* base = nullptr;      // tensor data pointer + offset, in bytes
-    int64_t dims[4] = {0};
-    int64_t strides[4] = {0};  // elements
+    void* base = nullptr;              // tensor data pointer + offset, in bytes
+    int64_t dims[kViewDims] = {0};
+    int64_t strides[kViewDims] = {0};  // elements
 };
 
-enum class OpKind : int { Nop = 0, GridSampler2D = 1, Resize = 2, ResizeGrad = 3 };
+enum class OpKind : int { Nop = 0, GridSampler2D = 1, Resize = 2, ResizeGrad = 3, GridSampler3D = 4 };
 
 // Where a kernel operand lives: the tensor's own memory (contiguous view) or a slice of the caller's
 // workspace, known only as an offset until the second phase receives the workspace address.
@@ -91,6 +93,18 @@ struct GridSamplerArgs {
     int align = 0;
     int channels_last = 0;  // 1: x is (N,Hin,Win,C) and y is (N,Hout,Wout,C) in memory
     int64_t N = 0, C = 0, Hin = 0, Win = 0, Hout = 0, Wout = 0;
+    const void* x = nullptr;
+    const void* grid = nullptr;
+    void* y = nullptr;
+};
+
+// Volumetric sampler: x is (N,C,Din,Hin,Win), grid (N,Dout,Hout,Wout,3) ordered x,y,z, y (N,C,Dout,Hout,Wout).
+struct GridSampler3DArgs {
+    Elem elem = Elem::F32;
+    int interp = 0;  // 0 bilinear (trilinear blend of eight corners), 1 nearest
+    int pad = 0;
+    int align = 0;
+    int64_t N = 0, C = 0, Din = 0, Hin = 0, Win = 0, Dout = 0, Hout = 0, Wout = 0;
     const void* x = nullptr;
     const void* grid = nullptr;
     void* y = nullptr;
@@ -135,6 +149,7 @@ struct aclOpExecutor {
     opscv::GridSamplerArgs gs;  // pointer members are filled in by the second phase
     opscv::ResizeArgs rs;
     opscv::ResizeGradArgs rg;
+    opscv::GridSampler3DArgs gs3;
     opscv::PlannedPtr in0, in1, out0;  // input/self, grid, out
     // packing work: views gathered into the workspace before the kernel, scattered after it
     struct Pack {

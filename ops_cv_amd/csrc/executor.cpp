@@ -11,19 +11,34 @@ namespace {
 uint64_t align_up(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
 }  // namespace
 
-PlannedPtr plan_view(aclOpExecutor* ex, const aclTensor* t, int elem_bytes, bool is_output)
+PlannedPtr plan_view(aclOpExecutor* ex, const aclTensor* t, int elem_bytes, bool is_output, const int* perm)
 {
     PlannedPtr p;
     char* base = (t->data == nullptr) ? nullptr : (char*)t->data + t->offset * (int64_t)elem_bytes;
-    if (t->contiguous()) {
-        p.direct = base;
-        return p;
-    }
     aclOpExecutor::Pack pk;
     pk.view.base = base;
-    for (int i = 0; i < 4; i++) {
-        pk.view.dims[i] = t->dims[i];
-        pk.view.strides[i] = t->strides[i];
+    const int n = (int)t->ndim;
+    const int lead = kViewDims - n;
+    for (int i = 0; i < lead; i++) {
+        pk.view.dims[i] = 1;
+        pk.view.strides[i] = 0;
+    }
+    for (int i = 0; i < n; i++) {
+        const int src = (perm != nullptr) ? perm[i] : i;
+        pk.view.dims[lead + i] = t->dims[src];
+        pk.view.strides[lead + i] = t->strides[src];
+    }
+    bool dense = true;
+    int64_t expect = 1;
+    for (int i = kViewDims - 1; i >= 0; i--) {
+        if (pk.view.dims[i] != 1 && pk.view.strides[i] != expect) {
+            dense = false;
+        }
+        expect *= pk.view.dims[i];
+    }
+    if (dense) {
+        p.direct = base;
+        return p;
     }
     pk.elem_bytes = elem_bytes;
     pk.ws_offset = align_up(ex->workspace_bytes, 256);
@@ -93,6 +108,16 @@ aclnnStatus run_executor(void* workspace, uint64_t workspace_size, aclOpExecutor
             return ACLNN_ERR_PARAM_NULLPTR;
         }
         e = launch_grid_sampler2d(a, s);
+    } else if (ex->kind == OpKind::GridSampler3D) {
+        GridSampler3DArgs a = ex->gs3;
+        a.x = resolve(ex->in0, workspace);
+        a.grid = resolve(ex->in1, workspace);
+        a.y = resolve(ex->out0, workspace);
+        if (a.x == nullptr || a.grid == nullptr || a.y == nullptr) {
+            set_error("%s: tensor data pointer is NULL", api);
+            return ACLNN_ERR_PARAM_NULLPTR;
+        }
+        e = launch_grid_sampler3d(a, s);
     } else if (ex->kind == OpKind::ResizeGrad) {
         ResizeGradArgs a = ex->rg;
         a.x = resolve(ex->in0, workspace);

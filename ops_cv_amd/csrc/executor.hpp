@@ -7,10 +7,13 @@
 
 namespace opscv {
 
-// Chooses where the kernel operand for the 4-D tensor `t` lives: the tensor's own memory when the view is
-// contiguous, else a 256-byte aligned slice of the workspace; in that case a gather (input) or scatter
-// (output) step is queued on the executor and its workspace requirement grows.
-PlannedPtr plan_view(aclOpExecutor* ex, const aclTensor* t, int elem_bytes, bool is_output);
+// Chooses where the kernel operand for the tensor `t` (at most five dimensions) lives: the tensor's own memory
+// when the view is contiguous, else a 256-byte aligned slice of the workspace; in that case a gather (input) or
+// scatter (output) step is queued on the executor and its workspace requirement grows.  With `perm`, the
+// operand's dimension i is the view's dimension perm[i] (a transposed operand: contiguity is judged and the
+// packing done in the permuted order).
+PlannedPtr plan_view(aclOpExecutor* ex, const aclTensor* t, int elem_bytes, bool is_output,
+                     const int* perm = nullptr);
 
 inline void* resolve(const PlannedPtr& p, void* workspace)
 {

@@ -1,0 +1,262 @@
+// Volumetric grid sampler (5-D), forward, NCDHW: device code and launcher.
+//
+// Arithmetic of the bilinear mode follows, operation for operation, the reference SIMT kernel
+//   image/grid_sample/op_kernel/arch35/grid_sampler_3d_bilinear_smit.h:66-135  (eight-corner blend)
+//   image/grid_sample/op_kernel/arch35/grid_sampler_3d_bilinear_smit.h:168-183 (unnormalize, clip order d, w, h)
+//   image/grid_sample/op_kernel/arch35/grid_sampler_bilinear_smit_common.h:37-94 (ClipCoordinates,
+//   reflectCoordinates, safeDowngradeToIntRange, Clip)
+// with every product and sum rounded separately (the translation unit is compiled with -ffp-contract=off).
+// The nearest mode uses the same coordinate pipeline and rounds each coordinate half to even, as the reference's
+// vector kernel does (image/grid_sample/op_kernel/grid_sampler_3d_nearest.h:569-571, CAST_RINT).
+//
+// Work split: the reference gives one thread to every (n, c, d, h, w) output element and repeats the coordinate
+// arithmetic per channel.  Here a lane owns one output point (n, d, h, w): it computes the eight corner offsets and
+// weights once and then walks a chunk of channels, so the grid is read once per channel chunk and the stores of a
+// wavefront are 64 consecutive elements of one output row.  The weights do not depend on the channel, so hoisting
+// them changes no bit of the result.
+#include <hip/hip_runtime.h>
+
+#include "kernels.hpp"
+#include "sampler_math.hpp"
+
+namespace opscv {
+
+namespace {
+
+constexpr int kThreads = 256;
+
+// grid_sampler_bilinear_smit_common.h:37-46 (size is an unsigned index type there: size - 1 is converted to
+// float for the comparison, the replacement value is float(size) - 1)
+__device__ __forceinline__ float clip3_coordinates(float coord, int32_t size)
+{
+    coord = (coord < 0.0f) ? 0.0f : coord;
+    coord = (coord > (float)(size - 1)) ? (float)size - 1.0f : coord;
+    if (__builtin_isnan(coord) || __builtin_isinf(coord)) {
+        return 0.0f;
+    }
+    return coord;
+}
+
+// grid_sampler_bilinear_smit_common.h:48-66.  `low2` is twiceLow (0 or -1), `span2` is twiceHigh - twiceLow.
+// The parity of floor(coord / span) is taken from the float itself: every float of 2^24 or more is an even
+// integer, below that the conversion to an integer is exact.
+__device__ __forceinline__ float reflect3_coordinates(float coord, int32_t low2, int64_t span2)
+{
+    if (span2 == 0) {
+        return 0.0f;
+    }
+    const float mn = (float)low2 / 2.0f;
+    const float span = (float)span2 / 2.0f;
+    coord = __builtin_fabsf(coord - mn);
+    const float extra = __builtin_fmodf(coord, span);
+    const float fl = __builtin_floorf(coord / span);
+    const bool odd = (fl < 16777216.0f) && (((int32_t)fl & 1) != 0);
+    if (!odd) {
+        return extra + mn;
+    }
+    return span - extra + mn;
+}
+
+// grid_sampler_bilinear_smit_common.h:76-92
+template <int PAD, bool ALIGN>
+__device__ __forceinline__ float clip3(float coord, int32_t size)
+{
+    if (PAD == 1) {
+        coord = clip3_coordinates(coord, size);
+    } else if (PAD == 2) {
+        if (ALIGN) {
+            coord = reflect3_coordinates(coord, 0, 2 * ((int64_t)size - 1));
+        } else {
+            coord = reflect3_coordinates(coord, -1, 2 * (int64_t)size);
+        }
+        coord = clip3_coordinates(coord, size);
+    }
+    if (nan_or_inf(coord)) {
+        return -100.0f;
+    }
+    return coord;
+}
+
+// grid_sampler_3d_bilinear_smit.h:171-179
+template <bool ALIGN>
+__device__ __forceinline__ float unnormalize3(float g, int32_t size)
+{
+    if (ALIGN) {
+        return (g + 1.0f) / 2.0f * (float)(size - 1);
+    }
+    return ((g + 1.0f) * (float)size - 1.0f) / 2.0f;
+}
+
+struct Gs3dParams {
+    int32_t C, Din, Hin, Win;
+    int64_t out_vol;     // Dout * Hout * Wout
+    int64_t points;      // N * out_vol
+    int32_t chan_chunk;  // channels per blockIdx.y
+};
+
+template <typename T, int INTERP, int PAD, bool ALIGN>
+__global__ __launch_bounds__(kThreads) void gs3d_kernel(const T* __restrict__ x, const T* __restrict__ grid,
+                                                         T* __restrict__ y, Gs3dParams p)
+{
+    const int64_t pt = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (pt >= p.points) {
+        return;
+    }
+    const int64_t n = pt / p.out_vol;
+    const int64_t sp = pt - n * p.out_vol;
+    const T* g = grid + pt * 3;
+    const float gw = ElemIO<T>::load(g);
+    const float gh = ElemIO<T>::load(g + 1);
+    const float gd = ElemIO<T>::load(g + 2);
+    const float pd = clip3<PAD, ALIGN>(unnormalize3<ALIGN>(gd, p.Din), p.Din);
+    const float pw = clip3<PAD, ALIGN>(unnormalize3<ALIGN>(gw, p.Win), p.Win);
+    const float ph = clip3<PAD, ALIGN>(unnormalize3<ALIGN>(gh, p.Hin), p.Hin);
+
+    const int32_t in_plane = p.Hin * p.Win;
+    const int64_t in_vol = (int64_t)p.Din * in_plane;
+    const int32_t c_begin = blockIdx.y * p.chan_chunk;
+    const int32_t c_end = (c_begin + p.chan_chunk < p.C) ? c_begin + p.chan_chunk : p.C;
+    const T* xc = x + (n * p.C + c_begin) * in_vol;
+    T* yc = y + (n * p.C + c_begin) * p.out_vol + sp;
+
+    if (INTERP == 1) {
+        const int32_t id = float_to_i32(__builtin_rintf(pd));
+        const int32_t ih = float_to_i32(__builtin_rintf(ph));
+        const int32_t iw = float_to_i32(__builtin_rintf(pw));
+        const bool in = id >= 0 && id < p.Din && ih >= 0 && ih < p.Hin && iw >= 0 && iw < p.Win;
+        const int64_t off = in ? (int64_t)id * in_plane + ih * p.Win + iw : 0;
+        T zero;
+        ElemIO<T>::store(&zero, 0.0f);
+        for (int32_t c = c_begin; c < c_end; c++) {
+            *yc = in ? xc[off] : zero;
+            xc += in_vol;
+            yc += p.out_vol;
+        }
+        return;
+    }
+
+    const float fd = __builtin_floorf(pd), fh = __builtin_floorf(ph), fw = __builtin_floorf(pw);
+    const float dd = pd - fd, dh = ph - fh, dw = pw - fw;
+    const int32_t d0 = float_to_i32(fd), d1 = float_to_i32(fd + 1.0f);
+    const int32_t h0 = float_to_i32(fh), h1 = float_to_i32(fh + 1.0f);
+    const int32_t w0 = float_to_i32(fw), w1 = float_to_i32(fw + 1.0f);
+    const bool vd0 = d0 >= 0 && d0 < p.Din, vd1 = d1 >= 0 && d1 < p.Din;
+    const bool vh0 = h0 >= 0 && h0 < p.Hin, vh1 = h1 >= 0 && h1 < p.Hin;
+    const bool vw0 = w0 >= 0 && w0 < p.Win, vw1 = w1 >= 0 && w1 < p.Win;
+    // corner order of the reference: (d0,h0,w0) (d0,h0,w1) (d0,h1,w0) (d0,h1,w1) (d1,h0,w0) (d1,h0,w1) (d1,h1,w0) (d1,h1,w1)
+    float wt[8];
+    wt[0] = (1.0f - dw) * (1.0f - dh) * (1.0f - dd);
+    wt[1] = dw * (1.0f - dh) * (1.0f - dd);
+    wt[2] = (1.0f - dw) * dh * (1.0f - dd);
+    wt[3] = dw * dh * (1.0f - dd);
+    wt[4] = (1.0f - dw) * (1.0f - dh) * dd;
+    wt[5] = dw * (1.0f - dh) * dd;
+    wt[6] = (1.0f - dw) * dh * dd;
+    wt[7] = dw * dh * dd;
+    bool ok[8];
+    int64_t off[8];
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        const bool vd = (k & 4) ? vd1 : vd0;
+        const bool vh = (k & 2) ? vh1 : vh0;
+        const bool vw = (k & 1) ? vw1 : vw0;
+        ok[k] = vd && vh && vw;
+        const int32_t d = (k & 4) ? d1 : d0, h = (k & 2) ? h1 : h0, w = (k & 1) ? w1 : w0;
+        off[k] = ok[k] ? (int64_t)d * in_plane + h * p.Win + w : 0;
+    }
+    for (int32_t c = c_begin; c < c_end; c++) {
+        float v[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            v[k] = ok[k] ? ElemIO<T>::load(xc + off[k]) : 0.0f;
+        }
+        float acc = v[0] * wt[0];
+#pragma unroll
+        for (int k = 1; k < 8; k++) {
+            acc += v[k] * wt[k];
+        }
+        ElemIO<T>::store(yc, acc);
+        xc += in_vol;
+        yc += p.out_vol;
+    }
+}
+
+template <typename T, int INTERP, int PAD, bool ALIGN>
+hipError_t launch_one(const GridSampler3DArgs& a, hipStream_t stream)
+{
+    Gs3dParams p;
+    p.C = (int32_t)a.C;
+    p.Din = (int32_t)a.Din;
+    p.Hin = (int32_t)a.Hin;
+    p.Win = (int32_t)a.Win;
+    p.out_vol = a.Dout * a.Hout * a.Wout;
+    p.points = a.N * p.out_vol;
+    const int64_t pblocks = (p.points + kThreads - 1) / kThreads;
+    // enough workgroups to fill 256 compute units several times over, else whole channel ranges per lane
+    int64_t chunks = 1;
+    while (pblocks * chunks < 4096 && chunks * 2 <= a.C) {
+        chunks *= 2;
+    }
+    p.chan_chunk = (int32_t)((a.C + chunks - 1) / chunks);
+    const int64_t ychunks = (a.C + p.chan_chunk - 1) / p.chan_chunk;
+    if (pblocks > INT32_MAX || ychunks > 65535) {
+        return hipErrorInvalidValue;
+    }
+    hipLaunchKernelGGL((gs3d_kernel<T, INTERP, PAD, ALIGN>), dim3((unsigned)pblocks, (unsigned)ychunks),
+                       dim3(kThreads), 0, stream, (const T*)a.x, (const T*)a.grid, (T*)a.y, p);
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t launch_typed(const GridSampler3DArgs& a, hipStream_t stream)
+{
+    const int key = a.interp * 6 + a.pad * 2 + a.align;
+    switch (key) {
+#define OPSCV_GS3D_CASE(I, P, A) \
+    case (I) * 6 + (P) * 2 + (A): return launch_one<T, I, P, (A) != 0>(a, stream);
+        OPSCV_GS3D_CASE(0, 0, 0)
+        OPSCV_GS3D_CASE(0, 0, 1)
+        OPSCV_GS3D_CASE(0, 1, 0)
+        OPSCV_GS3D_CASE(0, 1, 1)
+        OPSCV_GS3D_CASE(0, 2, 0)
+        OPSCV_GS3D_CASE(0, 2, 1)
+        OPSCV_GS3D_CASE(1, 0, 0)
+        OPSCV_GS3D_CASE(1, 0, 1)
+        OPSCV_GS3D_CASE(1, 1, 0)
+        OPSCV_GS3D_CASE(1, 1, 1)
+        OPSCV_GS3D_CASE(1, 2, 0)
+        OPSCV_GS3D_CASE(1, 2, 1)
+#undef OPSCV_GS3D_CASE
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace
+
+hipError_t launch_grid_sampler3d(const GridSampler3DArgs& a, hipStream_t stream)
+{
+    if (a.x == nullptr || a.grid == nullptr || a.y == nullptr) {
+        return hipErrorInvalidValue;
+    }
+    if (a.interp < 0 || a.interp > 1 || a.pad < 0 || a.pad > 2) {
+        return hipErrorInvalidValue;
+    }
+    if (a.N <= 0 || a.C <= 0 || a.Din <= 0 || a.Hin <= 0 || a.Win <= 0 || a.Dout < 0 || a.Hout < 0 || a.Wout < 0) {
+        return hipErrorInvalidValue;
+    }
+    if (a.C > INT32_MAX || a.Din > INT32_MAX || a.Hin > INT32_MAX || a.Win > INT32_MAX ||
+        a.Hin * a.Win > INT32_MAX) {
+        return hipErrorInvalidValue;
+    }
+    if (a.N * a.Dout * a.Hout * a.Wout == 0) {
+        return hipSuccess;
+    }
+    switch (a.elem) {
+        case Elem::F32: return launch_typed<float>(a, stream);
+        case Elem::F16: return launch_typed<_Float16>(a, stream);
+        case Elem::BF16: return launch_typed<__bf16>(a, stream);
+    }
+    return hipErrorInvalidValue;
+}
+
+}  // namespace opscv

@@ -1,4 +1,4 @@
-// Packing of non-contiguous 4-D views into contiguous workspace slices and back.
+// Packing of non-contiguous views of up to five dimensions into contiguous workspace slices and back.
 //
 // Takes the place of the reference's l0op::Contiguous (inputs) and l0op::ViewCopy (output) steps,
 // image/grid_sample/op_api/aclnn_grid_sampler2d.cpp:288-293,337-338.
@@ -12,25 +12,27 @@ namespace {
 
 constexpr int kThreads = 256;
 
-struct View4 {
-    int64_t d1, d2, d3;          // extents of dims 1..3 (dim 0 follows from the total)
-    int64_t s0, s1, s2, s3;      // element strides
+struct View5 {
+    int64_t d1, d2, d3, d4;      // extents of dims 1..4 (dim 0 follows from the total)
+    int64_t s0, s1, s2, s3, s4;  // element strides
 };
 
 template <typename U, bool GATHER>
 __global__ __launch_bounds__(kThreads) void strided_copy_kernel(U* __restrict__ strided, U* __restrict__ packed,
-                                                                 int64_t total, View4 v)
+                                                                 int64_t total, View5 v)
 {
     const int64_t stride = (int64_t)gridDim.x * kThreads;
     for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += stride) {
         int64_t r = i;
+        const int64_t i4 = r % v.d4;
+        r /= v.d4;
         const int64_t i3 = r % v.d3;
         r /= v.d3;
         const int64_t i2 = r % v.d2;
         r /= v.d2;
         const int64_t i1 = r % v.d1;
         const int64_t i0 = r / v.d1;
-        const int64_t off = i0 * v.s0 + i1 * v.s1 + i2 * v.s2 + i3 * v.s3;
+        const int64_t off = i0 * v.s0 + i1 * v.s1 + i2 * v.s2 + i3 * v.s3 + i4 * v.s4;
         if (GATHER) {
             packed[i] = strided[off];
         } else {
@@ -42,11 +44,12 @@ __global__ __launch_bounds__(kThreads) void strided_copy_kernel(U* __restrict__ 
 template <typename U>
 hipError_t run(const StridedView& sv, void* contiguous, bool gather, hipStream_t stream)
 {
-    const int64_t total = sv.dims[0] * sv.dims[1] * sv.dims[2] * sv.dims[3];
+    const int64_t total = sv.dims[0] * sv.dims[1] * sv.dims[2] * sv.dims[3] * sv.dims[4];
     if (total == 0) {
         return hipSuccess;
     }
-    View4 v{sv.dims[1], sv.dims[2], sv.dims[3], sv.strides[0], sv.strides[1], sv.strides[2], sv.strides[3]};
+    View5 v{sv.dims[1],    sv.dims[2],    sv.dims[3],    sv.dims[4],   sv.strides[0],
+            sv.strides[1], sv.strides[2], sv.strides[3], sv.strides[4]};
     int64_t blocks = (total + kThreads - 1) / kThreads;
     if (blocks > 256 * 64) {
         blocks = 256 * 64;
@@ -69,7 +72,7 @@ hipError_t launch_strided_copy(const StridedView& v, void* contiguous, int elem_
     if (v.base == nullptr || contiguous == nullptr) {
         return hipErrorInvalidValue;
     }
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < kViewDims; i++) {
         if (v.dims[i] < 0) {
             return hipErrorInvalidValue;
         }

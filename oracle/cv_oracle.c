@@ -25,6 +25,12 @@
  *                                  torch interpolate(mode="nearest") comparison (bit-exact: a pure copy)
  *   oracle_upsample_bilinear2d_backward : adjointness with the forward oracle (<forward(x), g> = <x, backward(g)>),
  *                                  gradient mass conservation, x2 closed form, live torch autograd comparison
+ *   oracle_grid_sampler3d        : identity grid reproduces the volume, a grid constant in z reduces to the 2-D
+ *                                  sampler's geometry on one slice, reflection invariants, live torch
+ *                                  grid_sample on 5-D inputs (both modes, all paddings); the reference's source
+ *                                  does not fix whether its compiler contracts a*b+c in this file: restated with
+ *                                  separate roundings, so bit-exactness to the reference is "parity unpinned",
+ *                                  agreement with torch to 1e-5 is what is pinned
  *   oracle_resize_scale          : float bit patterns held by the reference's tiling UT
  *                                  (image/resize_bilinear_v2/tests/ut/op_host/arch35/test_resize_bilinear_v2_tiling.cpp)
  */
@@ -783,6 +789,153 @@ int oracle_upsample_bilinear2d_backward(const void* grads, void* y, int dtype_in
                     store_from_float(y, dtype_out, yi, acc);
                 }
             }
+        }
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------------------------------
+ * Volumetric grid sampler (5-D)
+ *   image/grid_sample/op_kernel/arch35/grid_sampler_3d_bilinear_smit.h:53-135,146-191
+ *   image/grid_sample/op_kernel/arch35/grid_sampler_bilinear_smit_common.h:37-94
+ * The reference's index types are unsigned (uint32_t/uint64_t) for sizes and signed for the corner
+ * indices; sizes here are positive int32 so (size - 1) converts to the same float.  Conversions the
+ * reference leaves undefined (a float beyond the index type) are treated as out of bounds.
+ * ---------------------------------------------------------------------------------------- */
+static float gs3_clip_coordinates(float coord, int32_t size)
+{
+    coord = coord < 0 ? 0 : coord;
+    coord = coord > (float)(size - 1) ? (float)size - 1 : coord;
+    if (isnan(coord) || isinf(coord)) {
+        return 0.0f;
+    }
+    return coord;
+}
+
+static float gs3_reflect_coordinates(float coord, int64_t twice_low, int64_t twice_high)
+{
+    if (twice_low == twice_high) {
+        return 0;
+    }
+    float min = (float)twice_low / 2;
+    float span = (float)(twice_high - twice_low) / 2;
+    coord = fabsf(coord - min);
+    float extra = fmodf(coord, span);
+    float fl = floorf(coord / span);
+    /* parity of the quotient: floats of 2^24 and more are even integers */
+    int odd = (fl < 16777216.0f) && (((int64_t)fl) % 2 != 0);
+    if (!odd) {
+        return extra + min;
+    }
+    return span - extra + min;
+}
+
+float oracle_gs3d_clip(float coord, int32_t size, int32_t padding_mode, int32_t align_corners)
+{
+    if (padding_mode == 1) {
+        coord = gs3_clip_coordinates(coord, size);
+    } else if (padding_mode == 2) {
+        if (align_corners) {
+            coord = gs3_reflect_coordinates(coord, 0, 2 * ((int64_t)size - 1));
+        } else {
+            coord = gs3_reflect_coordinates(coord, -1, 2 * (int64_t)size - 1);
+        }
+        coord = gs3_clip_coordinates(coord, size);
+    }
+    if (!isfinite(coord)) {
+        return -100.0f;
+    }
+    return coord;
+}
+
+float oracle_gs3d_unnormalize(float g, int32_t size, int32_t align_corners)
+{
+    if (align_corners == 1) {
+        return (g + 1) / 2 * (float)(size - 1);
+    }
+    return ((g + 1) * (float)size - 1) / 2;
+}
+
+static int64_t gs3_index(float f)
+{
+    if (!(f >= -2147483648.0f && f < 2147483648.0f)) {
+        return -1; /* outside every volume */
+    }
+    return (int64_t)f;
+}
+
+static float gs3_point_value(const void* x, int dtype, int64_t base, int64_t d, int64_t h, int64_t w, int64_t D,
+                             int64_t H, int64_t W)
+{
+    if (d >= 0 && h >= 0 && w >= 0 && d < D && h < H && w < W) {
+        return load_as_float(x, dtype, base + d * H * W + h * W + w);
+    }
+    return 0.0f;
+}
+
+int oracle_grid_sampler3d(const void* x, const void* grid, void* y, int dtype, int64_t N, int64_t C, int64_t Din,
+                          int64_t Hin, int64_t Win, int64_t Dout, int64_t Hout, int64_t Wout, int interp, int pad,
+                          int align, int threads)
+{
+    if (x == NULL || grid == NULL || y == NULL || dtype < 0 || dtype > 2 || interp < 0 || interp > 1 || pad < 0 ||
+        pad > 2 || Din <= 0 || Hin <= 0 || Win <= 0) {
+        return -1;
+    }
+    const int64_t out_vol = Dout * Hout * Wout;
+    const int64_t in_vol = Din * Hin * Win;
+    const int64_t points = N * out_vol;
+    (void)threads;
+#ifdef _OPENMP
+    int nt = threads > 0 ? threads : omp_get_max_threads();
+#pragma omp parallel for num_threads(nt) schedule(static)
+#endif
+    for (int64_t p = 0; p < points; p++) {
+        const int64_t n = p / out_vol;
+        const int64_t sp = p - n * out_vol;
+        float gd = load_as_float(grid, dtype, 3 * p + 2);
+        float gh = load_as_float(grid, dtype, 3 * p + 1);
+        float gw = load_as_float(grid, dtype, 3 * p);
+        gd = oracle_gs3d_clip(oracle_gs3d_unnormalize(gd, (int32_t)Din, align), (int32_t)Din, pad, align);
+        gw = oracle_gs3d_clip(oracle_gs3d_unnormalize(gw, (int32_t)Win, align), (int32_t)Win, pad, align);
+        gh = oracle_gs3d_clip(oracle_gs3d_unnormalize(gh, (int32_t)Hin, align), (int32_t)Hin, pad, align);
+        for (int64_t c = 0; c < C; c++) {
+            const int64_t base = (n * C + c) * in_vol;
+            const int64_t yo = (n * C + c) * out_vol + sp;
+            if (interp == 1) {
+                float v = gs3_point_value(x, dtype, base, gs3_index(rintf(gd)), gs3_index(rintf(gh)),
+                                          gs3_index(rintf(gw)), Din, Hin, Win);
+                store_from_float(y, dtype, yo, v);
+                continue;
+            }
+            float df = floorf(gd), hf = floorf(gh), wf = floorf(gw);
+            float dd = gd - df, dh = gh - hf, dw = gw - wf;
+            float v, wgt, acc;
+            v = gs3_point_value(x, dtype, base, gs3_index(df), gs3_index(hf), gs3_index(wf), Din, Hin, Win);
+            wgt = (1.0f - dw) * (1.0f - dh) * (1.0f - dd);
+            acc = v * wgt;
+            v = gs3_point_value(x, dtype, base, gs3_index(df), gs3_index(hf), gs3_index(wf + 1), Din, Hin, Win);
+            wgt = dw * (1.0f - dh) * (1.0f - dd);
+            acc += v * wgt;
+            v = gs3_point_value(x, dtype, base, gs3_index(df), gs3_index(hf + 1), gs3_index(wf), Din, Hin, Win);
+            wgt = (1.0f - dw) * dh * (1.0f - dd);
+            acc += v * wgt;
+            v = gs3_point_value(x, dtype, base, gs3_index(df), gs3_index(hf + 1), gs3_index(wf + 1), Din, Hin, Win);
+            wgt = dw * dh * (1.0f - dd);
+            acc += v * wgt;
+            v = gs3_point_value(x, dtype, base, gs3_index(df + 1), gs3_index(hf), gs3_index(wf), Din, Hin, Win);
+            wgt = (1.0f - dw) * (1.0f - dh) * dd;
+            acc += v * wgt;
+            v = gs3_point_value(x, dtype, base, gs3_index(df + 1), gs3_index(hf), gs3_index(wf + 1), Din, Hin, Win);
+            wgt = dw * (1.0f - dh) * dd;
+            acc += v * wgt;
+            v = gs3_point_value(x, dtype, base, gs3_index(df + 1), gs3_index(hf + 1), gs3_index(wf), Din, Hin, Win);
+            wgt = (1.0f - dw) * dh * dd;
+            acc += v * wgt;
+            v = gs3_point_value(x, dtype, base, gs3_index(df + 1), gs3_index(hf + 1), gs3_index(wf + 1), Din, Hin,
+                                Win);
+            wgt = dw * dh * dd;
+            acc += v * wgt;
+            store_from_float(y, dtype, yo, acc);
         }
     }
     return 0;

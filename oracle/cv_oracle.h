@@ -116,6 +116,17 @@ int oracle_upsample_bilinear2d_backward(const void* grads, void* y, int dtype_in
 int oracle_upsample_axis_taps(int64_t len_src, int64_t len_dst, int align_corners, float user_scale, int32_t* i0,
                               int32_t* i1, float* lambda);
 
+/*
+ * Volumetric grid sampler, forward (image/grid_sample/op_kernel/arch35/grid_sampler_3d_bilinear_smit.h:146-191).
+ * x (N,C,Din,Hin,Win), grid (N,Dout,Hout,Wout,3) ordered x,y,z, y (N,C,Dout,Hout,Wout); interp 0 bilinear,
+ * 1 nearest (round half to even, image/grid_sample/op_kernel/grid_sampler_3d_nearest.h:569-571).
+ */
+float oracle_gs3d_unnormalize(float g, int32_t size, int32_t align_corners);
+float oracle_gs3d_clip(float coord, int32_t size, int32_t padding_mode, int32_t align_corners);
+int oracle_grid_sampler3d(const void* x, const void* grid, void* y, int dtype, int64_t N, int64_t C, int64_t Din,
+                          int64_t Hin, int64_t Win, int64_t Dout, int64_t Hout, int64_t Wout, int interp, int pad,
+                          int align, int threads);
+
 int oracle_max_threads(void);
 
 #ifdef __cplusplus

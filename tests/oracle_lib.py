@@ -90,6 +90,12 @@ def lib():
                                              ctypes.c_double, ctypes.c_double, ctypes.c_int]
     L.oracle_upsample_axis_taps.restype = ctypes.c_int
     L.oracle_upsample_axis_taps.argtypes = [i64, i64, ctypes.c_int, f32, vp, vp, vp]
+    L.oracle_grid_sampler3d.restype = ctypes.c_int
+    L.oracle_grid_sampler3d.argtypes = [vp, vp, vp, ctypes.c_int] + [i64] * 8 + [ctypes.c_int] * 4
+    L.oracle_gs3d_unnormalize.restype = f32
+    L.oracle_gs3d_unnormalize.argtypes = [f32, ctypes.c_int32, ctypes.c_int32]
+    L.oracle_gs3d_clip.restype = f32
+    L.oracle_gs3d_clip.argtypes = [f32, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32]
     L.oracle_max_threads.restype = ctypes.c_int
     L.oracle_max_threads.argtypes = []
     _lib = L
@@ -183,6 +189,22 @@ def upsample_bilinear2d_backward(grads, in_hw, align=False, channels_last=False,
                                                    float(scales_w))
     if rc != 0:
         raise ValueError("oracle_upsample_bilinear2d_backward rc=%d" % rc)
+    return y
+
+
+def grid_sampler3d(x, grid, interp=0, pad=0, align=False, dtype=None, threads=0):
+    """x (N,C,D,H,W), grid (N,Do,Ho,Wo,3) -> y (N,C,Do,Ho,Wo); float32, float16, or uint16 holding bf16 bits."""
+    x = np.ascontiguousarray(x)
+    grid = np.ascontiguousarray(grid)
+    code = _code_of(x) if dtype is None else dtype
+    N, C, D, H, W = x.shape
+    _, Do, Ho, Wo, three = grid.shape
+    assert three == 3 and grid.shape[0] == N and grid.dtype == x.dtype
+    y = np.empty((N, C, Do, Ho, Wo), dtype=x.dtype)
+    rc = lib().oracle_grid_sampler3d(_ptr(x), _ptr(grid), _ptr(y), code, N, C, D, H, W, Do, Ho, Wo, interp, pad,
+                                     int(bool(align)), threads)
+    if rc != 0:
+        raise ValueError("oracle_grid_sampler3d rc=%d" % rc)
     return y
 
 

@@ -4,7 +4,8 @@ The cases mirror the reference's op_api unit tests, which build descriptors with
 the GetWorkspaceSize phase: image/grid_sample/tests/ut/op_host/op_api/test_aclnn_grid_sampler2d.cpp and
 image/upsample_bilinear2d/tests/ut/op_host/op_api/test_aclnn_upsample_bilinear_2d.cpp,
 image/resize_bilinear_v2/tests/ut/op_host/op_api/test_aclnn_resize.cpp,
-image/resize_bilinear_v2_grad/tests/ut/op_host/op_api/test_aclnn_upsample_bilineard_2d_backward.cpp.
+image/resize_bilinear_v2_grad/tests/ut/op_host/op_api/test_aclnn_upsample_bilineard_2d_backward.cpp,
+image/grid_sample/tests/ut/op_host/op_api/test_aclnn_grid_sampler3d.cpp.
 """
 import ctypes
 import os
@@ -349,3 +350,69 @@ def test_upsample_backward_status_codes(aclnn, desc):
                sh=0, sw=0) == (0, 0, "resize_grad_gather")
     # equal sizes: a copy
     assert _ub(aclnn, desc, grad=(1, 1, 3, 3), osize=(3, 3), sh=1.0, sw=1.0)[2] == "copy"
+
+
+def _gs3(aclnn, desc, inp=(2, 1, 1, 3, 3), grid=(2, 1, 2, 2, 3), out=(2, 1, 1, 2, 2), dt=None, gdt=None, odt=None,
+         interp=0, pad=0, align=False, fmt=None, ofmt=None, **kw):
+    dt = aclnn.ACL_FLOAT if dt is None else dt
+    fmt = aclnn.ACL_FORMAT_NCDHW if fmt is None else fmt
+    i = desc.t(inp, dt, fmt, **kw)
+    g = desc.t(grid, dt if gdt is None else gdt, aclnn.ACL_FORMAT_NCDHW)
+    o = desc.t(out, dt if odt is None else odt, fmt if ofmt is None else ofmt)
+    st, ws, ex = aclnn.get_workspace_size_grid_sampler3d(i, g, interp, pad, align, o)
+    variant = aclnn.executor_variant(ex) if ex else None
+    if ex:
+        assert aclnn.destroy_executor(ex) == 0
+    return st, ws, variant
+
+
+def test_grid_sampler3d_status_codes(aclnn, desc):
+    """test_aclnn_grid_sampler3d.cpp:33-289 and the check order of aclnn_grid_sampler3d.cpp:194-208"""
+    INV, NULL = aclnn.ACLNN_ERR_PARAM_INVALID, aclnn.ACLNN_ERR_PARAM_NULLPTR
+    # input_nullptr, grid_nullptr, out_nullptr
+    assert _gs3(aclnn, desc, inp=None)[0] == NULL
+    assert _gs3(aclnn, desc, grid=None)[0] == NULL
+    assert _gs3(aclnn, desc, out=None)[0] == NULL
+    # input_empty: success, no workspace, an executor that does nothing
+    assert _gs3(aclnn, desc, inp=(2, 0, 1, 3, 3), out=(2, 0, 1, 2, 2)) == (0, 0, "")
+    # dtype_float16 / float32 / bf16 accepted, int8 rejected; DOUBLE passes the reference's list but has no kernel here
+    for dt in (aclnn.ACL_FLOAT16, aclnn.ACL_FLOAT, aclnn.ACL_BF16):
+        assert _gs3(aclnn, desc, dt=dt) == (0, 0, "gs3d_bilinear")
+    assert _gs3(aclnn, desc, dt=aclnn.ACL_INT8)[0] == INV
+    assert _gs3(aclnn, desc, dt=aclnn.ACL_DOUBLE)[0] == INV
+    assert _gs3(aclnn, desc, gdt=aclnn.ACL_FLOAT16)[0] == INV
+    assert _gs3(aclnn, desc, odt=aclnn.ACL_FLOAT16)[0] == INV
+    # shape_n_input1_grid2, shape_c_input1_out2, shape_h_grid2_out3, shape_w_grid2_out4, shape_grid_not_3
+    assert _gs3(aclnn, desc, inp=(1, 1, 1, 3, 3), out=(1, 1, 1, 2, 2))[0] == INV
+    assert _gs3(aclnn, desc, out=(2, 3, 1, 2, 2))[0] == INV
+    assert _gs3(aclnn, desc, out=(2, 1, 1, 3, 2))[0] == INV
+    assert _gs3(aclnn, desc, out=(2, 1, 1, 2, 4))[0] == INV
+    assert _gs3(aclnn, desc, grid=(2, 1, 2, 2, 4))[0] == INV
+    # rank and empty spatial extents
+    assert _gs3(aclnn, desc, inp=(2, 1, 3, 3))[0] == INV
+    assert _gs3(aclnn, desc, inp=(2, 1, 1, 0, 3))[0] == INV
+    # mode_3, padding_mode_3 (interpolation is 0 or 1 only; there is no volumetric bicubic)
+    assert _gs3(aclnn, desc, interp=3)[0] == INV
+    assert _gs3(aclnn, desc, interp=2)[0] == INV
+    assert _gs3(aclnn, desc, pad=3)[0] == INV
+    assert _gs3(aclnn, desc, interp=1, pad=2, align=True) == (0, 0, "gs3d_nearest")
+    # input_format_invalid, out_format_invalid
+    assert _gs3(aclnn, desc, fmt=aclnn.ACL_FORMAT_NCHW, ofmt=aclnn.ACL_FORMAT_NCDHW)[0] == INV
+    assert _gs3(aclnn, desc, ofmt=aclnn.ACL_FORMAT_NCHW)[0] == INV
+    assert _gs3(aclnn, desc, fmt=aclnn.ACL_FORMAT_ND)[0] == 0
+    # format errors come before attribute errors, dtype errors before both
+    msg = aclnn.load_library().aclGetRecentErrMsg
+    _gs3(aclnn, desc, fmt=aclnn.ACL_FORMAT_NCHW, interp=7)
+    assert b"format" in msg()
+    _gs3(aclnn, desc, dt=aclnn.ACL_INT8, fmt=aclnn.ACL_FORMAT_NCHW)
+    assert b"dtype" in msg()
+    # isNCDHW_special_case: an ordinary shape here
+    assert _gs3(aclnn, desc, inp=(22, 4, 16, 64, 64), grid=(22, 16, 64, 64, 3), out=(22, 4, 16, 64, 64))[0] == 0
+    # ascend910B2_NDHWC_case_01: channels-last extents (N,D,H,W,C); the operand is a permuted view, so a channel
+    # count above one needs workspace for the input and for the output
+    assert _gs3(aclnn, desc, inp=(2, 1, 3, 3, 1), out=(2, 1, 2, 2, 1), fmt=aclnn.ACL_FORMAT_NDHWC)[:2] == (0, 0)
+    st, ws, _ = _gs3(aclnn, desc, inp=(2, 1, 3, 3, 4), out=(2, 1, 2, 2, 4), fmt=aclnn.ACL_FORMAT_NDHWC)
+    assert st == 0 and ws >= (2 * 9 * 4 + 2 * 4 * 4) * 4
+    # a strided NCDHW view is packed too
+    st, ws, _ = _gs3(aclnn, desc, strides=(18, 18, 18, 6, 2), storage=(36,))
+    assert st == 0 and ws >= 2 * 9 * 4

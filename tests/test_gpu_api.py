@@ -287,3 +287,73 @@ def test_upsample_backward_fp32_into_fp16(oracle, device, aclnn):
     torch.cuda.synchronize()
     ref = oracle.upsample_bilinear2d_backward(gv.contiguous().cpu().numpy(), (6, 5), False)
     assert np.array_equal(y.cpu().numpy(), ref)
+
+
+def _bits(a, dtype):
+    return a.view(np.uint32 if dtype == "fp32" else np.uint16)
+
+
+@pytest.mark.parametrize("dtype", I.DTYPES)
+@pytest.mark.parametrize("interp", [0, 1])
+def test_grid_sampler3d(oracle, device, aclnn, dtype, interp):
+    """aclnnGridSampler3D against the oracle, bit for bit: every padding and alignment, grids reaching well outside
+    the volume, special values (NaN, infinities, huge and tie coordinates), single-voxel axes"""
+    torch = _torch()
+    rng = np.random.default_rng(500 + interp)
+    shapes = [(2, 3, 5, 6, 7, 4, 5, 9), (1, 8, 1, 1, 1, 2, 2, 2), (1, 2, 9, 3, 1, 3, 7, 5), (2, 1, 2, 17, 33, 6, 3, 70),
+              (1, 20, 4, 4, 4, 1, 1, 3)]
+    for (N, C, D, H, W, Do, Ho, Wo) in shapes:
+        x = I.cast_np(rng.standard_normal((N, C, D, H, W)).astype(np.float32), dtype)
+        g32 = rng.uniform(-2.5, 2.5, (N, Do, Ho, Wo, 3)).astype(np.float32)
+        flat = g32.reshape(-1, 3)
+        special = np.array([np.nan, np.inf, -np.inf, 1e30, -1e30, 1.0, -1.0, 0.0, 3e9, 0.5], np.float32)
+        k = min(len(special), flat.shape[0])
+        for j in range(k):
+            flat[j, j % 3] = special[j]
+        g = I.cast_np(g32, dtype)
+        for pad in range(3):
+            for align in (False, True):
+                ref = oracle.grid_sampler3d(x, g, interp, pad, align, dtype=I.oracle_code(dtype))
+                y = aclnn.grid_sampler3d(I.to_torch(x, dtype, device), I.to_torch(g, dtype, device), interp, pad, align)
+                torch.cuda.synchronize()
+                got = I.from_torch(y, dtype)
+                rn = np.isnan(I.as_f32(ref, dtype))
+                assert np.array_equal(np.isnan(I.as_f32(got, dtype)), rn), (N, C, D, H, W, pad, align)
+                assert np.array_equal(np.where(rn, 0, _bits(got, dtype)), np.where(rn, 0, _bits(ref, dtype))), \
+                    (N, C, D, H, W, Do, Ho, Wo, pad, align)
+
+
+def test_grid_sampler3d_layouts_and_views(oracle, device, aclnn):
+    """NDHWC tensors (permuted operands), strided NCDHW views, the reference's own example shape"""
+    torch = _torch()
+    rng = np.random.default_rng(510)
+    N, C, D, H, W, Do, Ho, Wo = 2, 5, 4, 6, 7, 3, 5, 8
+    x = rng.standard_normal((N, C, D, H, W)).astype(np.float32)
+    g = rng.uniform(-1.3, 1.3, (N, Do, Ho, Wo, 3)).astype(np.float32)
+    for interp, pad, align in [(0, 0, False), (0, 2, True), (1, 1, False)]:
+        ref = oracle.grid_sampler3d(x, g, interp, pad, align)
+        # channels-last extents (N,D,H,W,C) in and out
+        xl = torch.from_numpy(np.ascontiguousarray(x.transpose(0, 2, 3, 4, 1))).to(device)
+        y = aclnn.grid_sampler3d(xl, torch.from_numpy(g).to(device), interp, pad, align, channels_last=True)
+        torch.cuda.synchronize()
+        assert y.shape == (N, Do, Ho, Wo, C)
+        assert np.array_equal(y.cpu().numpy().transpose(0, 4, 1, 2, 3), ref)
+        # NCDHW views: input a transposed view, grid a slice with a storage offset, out a strided slice
+        xv = torch.from_numpy(np.ascontiguousarray(x.transpose(0, 1, 2, 4, 3))).to(device).transpose(3, 4)
+        assert not xv.is_contiguous()
+        gbig = torch.zeros((N + 1, Do, Ho, Wo, 3), device=device)
+        gbig[1:] = torch.from_numpy(g).to(device)
+        obig = torch.full((N, C, Do, Ho, Wo + 4), -3.0, device=device)
+        out = aclnn.grid_sampler3d(xv, gbig[1:], interp, pad, align, out=obig[..., 2:2 + Wo])
+        torch.cuda.synchronize()
+        assert np.array_equal(out.cpu().numpy(), ref)
+        rest = obig.cpu().numpy()
+        assert (rest[..., :2] == -3.0).all() and (rest[..., 2 + Wo:] == -3.0).all()
+    # the shape of the reference's special case (aclnn_grid_sampler3d.cpp:277-312): 22 x 4 x 16 x 64 x 64, fp16,
+    # against live torch on the host through the oracle at a tolerance-free comparison with the oracle only
+    x = I.cast_np(rng.standard_normal((22, 4, 16, 64, 64)).astype(np.float32), "fp16")
+    g = I.cast_np(rng.uniform(-1.1, 1.1, (22, 16, 64, 64, 3)).astype(np.float32), "fp16")
+    ref = oracle.grid_sampler3d(x, g, 0, 0, False)
+    y = aclnn.grid_sampler3d(I.to_torch(x, "fp16", device), I.to_torch(g, "fp16", device), 0, 0, False)
+    torch.cuda.synchronize()
+    assert np.array_equal(I.from_torch(y, "fp16").view(np.uint16), ref.view(np.uint16))

@@ -494,3 +494,98 @@ def test_upsample_backward_oracle(oracle):
     # x2 of a single source pixel: all the gradient lands on it
     g = np.arange(4, dtype=np.float32).reshape(1, 1, 2, 2)
     assert oracle.upsample_bilinear2d_backward(g, (1, 1), False)[0, 0, 0, 0] == 6.0
+
+
+# ---- volumetric (5-D) sampler ----
+
+def _identity_grid3(D, H, W, align):
+    def axis(n):
+        i = np.arange(n, dtype=np.float64)
+        return (2 * i / (n - 1) - 1) if align else ((2 * i + 1) / n - 1)
+    gz, gy, gx = np.meshgrid(axis(D), axis(H), axis(W), indexing="ij")
+    return np.stack([gx, gy, gz], -1)[None].astype(np.float32)
+
+
+def test_grid_sampler3d_identity_and_slice_reduction(oracle):
+    rng = np.random.default_rng(31)
+    D, H, W = 4, 8, 16  # powers of two: the identity grid's coordinates are exact in fp32
+    x = rng.standard_normal((1, 3, D, H, W)).astype(np.float32)
+    for a in (False, True):
+        g = _identity_grid3(D, H, W, a) if not a else _identity_grid3(5, 9, 17, a)
+        xs = x if not a else rng.standard_normal((1, 3, 5, 9, 17)).astype(np.float32)
+        for m in range(2):
+            for p in range(3):
+                got = oracle.grid_sampler3d(xs, g, m, p, a)
+                assert np.allclose(got, xs, atol=1e-6), (a, m, p)
+    # a grid whose z coordinate sits exactly on slice k samples that slice with the 2-D geometry:
+    # compare with torch's 2-D sampler on the slice (different arithmetic order, so a tolerance)
+    import torch
+    import torch.nn.functional as F
+    g2 = rng.uniform(-1.3, 1.3, (1, 6, 7, 2)).astype(np.float32)
+    k = 2
+    z = np.float32(2.0 * k / (D - 1) - 1.0)  # align_corners=True: slice k exactly (D - 1 = 3 is not a power of two,
+    zc = oracle.lib().oracle_gs3d_unnormalize(z, D, 1)  # so check the slice is hit exactly before relying on it)
+    assert zc == float(k)
+    g3 = np.concatenate([g2, np.full((1, 6, 7, 1), z, np.float32)], -1)[:, None]
+    for p in range(3):
+        got = oracle.grid_sampler3d(x, g3, 0, p, True)[:, :, 0]
+        want = F.grid_sample(torch.from_numpy(x[:, :, k]), torch.from_numpy(g2), mode="bilinear",
+                             padding_mode=PADS[p], align_corners=True).numpy()
+        assert np.abs(got - want).max() <= 2e-6 * max(1.0, np.abs(want).max())
+
+
+def test_grid_sampler3d_clip_invariants(oracle):
+    L = oracle.lib()
+    rng = np.random.default_rng(32)
+    for size in (1, 2, 3, 7, 32):
+        for a in (0, 1):
+            for c in rng.uniform(-300, 300, 400).astype(np.float32):
+                b = L.oracle_gs3d_clip(c, size, 1, a)
+                assert 0.0 <= b <= size - 1
+                r = L.oracle_gs3d_clip(c, size, 2, a)
+                assert 0.0 <= r <= size - 1
+                # reflection is periodic with period 2*(size-1) (align) or 2*size (no align)
+                period = 2 * (size - 1) if a else 2 * size
+                if period:
+                    r2 = L.oracle_gs3d_clip(np.float32(c + period), size, 2, a)
+                    assert abs(r - r2) <= 1e-3
+            # zeros padding leaves finite coordinates alone; non-finite ones land at -100 or, clipped, at 0
+            assert L.oracle_gs3d_clip(np.float32(12.5), size, 0, a) == 12.5
+            for bad in (np.nan, np.inf, -np.inf):
+                assert L.oracle_gs3d_clip(np.float32(bad), size, 0, a) == -100.0
+                assert L.oracle_gs3d_clip(np.float32(bad), size, 2, a) == 0.0
+            assert L.oracle_gs3d_clip(np.float32(np.nan), size, 1, a) == 0.0
+            assert L.oracle_gs3d_clip(np.float32(np.inf), size, 1, a) == size - 1
+    # closed forms of the unnormalization
+    assert L.oracle_gs3d_unnormalize(-1.0, 8, 1) == 0.0 and L.oracle_gs3d_unnormalize(1.0, 8, 1) == 7.0
+    assert L.oracle_gs3d_unnormalize(-1.0, 8, 0) == -0.5 and L.oracle_gs3d_unnormalize(1.0, 8, 0) == 7.5
+
+
+def test_live_torch_grid_sample3d(oracle):
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(33)
+    for trial in range(8):
+        N, C = 2, 3
+        D, H, W = rng.integers(1, 12, 3)
+        Do, Ho, Wo = rng.integers(1, 10, 3)
+        x = rng.standard_normal((N, C, D, H, W)).astype(np.float32)
+        g = rng.uniform(-1.7, 1.7, (N, Do, Ho, Wo, 3)).astype(np.float32)
+        for m in range(2):
+            for p in range(3):
+                for a in (False, True):
+                    got = oracle.grid_sampler3d(x, g, m, p, a)
+                    want = F.grid_sample(torch.from_numpy(x), torch.from_numpy(g), mode=MODES[m],
+                                         padding_mode=PADS[p], align_corners=a).numpy()
+                    if m == 1:
+                        # a pure selection: bit-exact unless a coordinate sits within rounding of a tie
+                        assert (got != want).mean() <= 0.01, (trial, p, a)
+                    else:
+                        assert np.abs(got - want).max() <= 1e-5 * max(1.0, np.abs(want).max()), (trial, m, p, a)
+    # 16-bit types round once at the end
+    x = rng.standard_normal((1, 2, 5, 6, 7)).astype(np.float16)
+    g = rng.uniform(-1.2, 1.2, (1, 3, 4, 5, 3)).astype(np.float16)
+    got = oracle.grid_sampler3d(x, g, 0, 0, False).astype(np.float32)
+    want = F.grid_sample(torch.from_numpy(x.astype(np.float32)), torch.from_numpy(g.astype(np.float32)),
+                         mode="bilinear", padding_mode="zeros", align_corners=False).numpy()
+    assert np.abs(got - want).max() <= 2e-3 * max(1.0, np.abs(want).max())
