@@ -102,6 +102,15 @@ def load_bench_lib():
     L.opscv_bench_upsample_bilinear2d.argtypes = [ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.c_int, vp,
                                                  ctypes.c_bool, ctypes.c_double, ctypes.c_double, vp, u64,
                                                  ctypes.c_int, vp, pd, pd]
+    L.opscv_bench_grid_sampler3d.restype = ctypes.c_int
+    L.opscv_bench_grid_sampler3d.argtypes = L.opscv_bench_grid_sampler2d.argtypes
+    L.opscv_bench_upsample_bilinear2d_backward.restype = ctypes.c_int
+    L.opscv_bench_upsample_bilinear2d_backward.argtypes = [ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.c_int, vp,
+                                                          vp, ctypes.c_bool, ctypes.c_double, ctypes.c_double, vp,
+                                                          u64, ctypes.c_int, vp, pd, pd]
+    L.opscv_bench_resize.restype = ctypes.c_int
+    L.opscv_bench_resize.argtypes = [ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.c_int, vp, ctypes.c_char_p, vp,
+                                     u64, ctypes.c_int, vp, pd, pd]
     L.opscv_bench_stream.restype = ctypes.c_int
     L.opscv_bench_stream.argtypes = [ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.c_int, u64, u64, ctypes.c_int, vp,
                                      pd]
@@ -298,6 +307,154 @@ def bench_up(name, steps, warmup, sets=None, check=True):
                 sets=nsets, cpu=(x0, w))
 
 
+def _finish(L, run, xs, ys, steps, warmup, stream):
+    import torch
+    preheat(run, warmup)
+    torch.cuda.synchronize()
+    t = run(steps)
+    torch.cuda.synchronize()
+    t.stream_us = stream_reference_us(L, xs, ys, steps, stream)
+    torch.cuda.synchronize()
+    return t
+
+
+def _parity(got, ref, dtype, **extra):
+    import numpy as np
+    import inputs as I
+    d = np.abs(I.as_f32(got, dtype) - I.as_f32(ref, dtype))
+    out = {"max_abs_err": float(d.max()), "bit_exact": bool(np.array_equal(got.view(np.uint8), ref.view(np.uint8)))}
+    out.update(extra)
+    return out
+
+
+def bench_gs3d(steps, warmup, sets=4):
+    """Volumetric sampler on the shape the reference singles out (22 x 4 x 16 x 64 x 64, fp16, an affine warp)."""
+    import numpy as np
+    import torch
+    import inputs as I
+    import oracle_lib
+    from ops_cv_amd import aclnn
+    dev = torch.device("cuda:0")
+    L = load_bench_lib()
+    N, C, D, H, W = 22, 4, 16, 64, 64
+    dtype = "fp16"
+    xs, gs, ys, hs = [], [], [], [[], [], []]
+    x0 = g0 = None
+    for s in range(sets):
+        rng = np.random.default_rng(3000 + s)
+        x = I.cast_np(rng.standard_normal((N, C, D, H, W)).astype(np.float32), dtype)
+        # identity lattice, mildly scaled and shifted per batch item, with jitter: a registration-style warp
+        ax = [np.linspace(-1, 1, n, dtype=np.float32) for n in (D, H, W)]
+        gz, gy, gx = np.meshgrid(*ax, indexing="ij")
+        base = np.stack([gx, gy, gz], -1)[None]
+        g = base * rng.uniform(0.9, 1.1, (N, 1, 1, 1, 3)) + rng.uniform(-0.1, 0.1, (N, 1, 1, 1, 3))
+        g = I.cast_np((g + rng.normal(0, 0.01, g.shape)).astype(np.float32), dtype)
+        if s == 0:
+            x0, g0 = x, g
+        xs.append(I.to_torch(x, dtype, dev))
+        gs.append(I.to_torch(g, dtype, dev))
+        ys.append(torch.empty((N, C, D, H, W), dtype=xs[-1].dtype, device=dev))
+        for lst, t in zip(hs, (xs[-1], gs[-1], ys[-1])):
+            lst.append(aclnn.tensor_handle(t, aclnn.ACL_FORMAT_NCDHW))
+    arr = lambda h: (ctypes.c_void_p * len(h))(*h)
+    ax_, ag, ay = arr(hs[0]), arr(hs[1]), arr(hs[2])
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ev, wall = ctypes.c_double(0), ctypes.c_double(0)
+
+    def run(k):
+        rc = L.opscv_bench_grid_sampler3d(ax_, ag, ay, sets, 0, 0, False, None, 0, k, stream, ctypes.byref(ev),
+                                          ctypes.byref(wall))
+        if rc != 0:
+            raise RuntimeError("bench loop failed rc=%d: %s" % (rc, aclnn.load_library().aclGetRecentErrMsg()))
+        return Timed(ev.value, wall.value, k)
+
+    st, _, ex = aclnn.get_workspace_size_grid_sampler3d(hs[0][0], hs[1][0], 0, 0, False, hs[2][0])
+    variant = aclnn.executor_variant(ex)
+    aclnn.destroy_executor(ex)
+    t = _finish(L, run, xs, ys, steps, warmup, stream)
+    ref = oracle_lib.grid_sampler3d(x0, g0, 0, 0, False, dtype=I.oracle_code(dtype))
+    parity = _parity(I.from_torch(ys[0], dtype), ref, dtype)
+    for lst in hs:
+        for h in lst:
+            aclnn.destroy_tensor(h)
+    samples = N * C * D * H * W
+    alg = (N * C * D * H * W * 2 + N * D * H * W * 3) * esize(dtype)
+    return dict(workload="V1 grid_sampler3d fp16 x(22,4,16,64,64) grid(22,16,64,64,3) bilinear zeros "
+                         "align_corners=False", samples=samples, alg_bytes=alg, timed=t, variant=variant,
+                parity=parity, sets=sets, default_modes=True)
+
+
+def bench_resize_like(kind, steps, warmup, sets=2):
+    """The 4K workload through the neighbouring entry points: kind "backward" (aclnnUpsampleBilinear2dBackward, the
+    gradient of the 2x upscale) or "nearest" (aclnnResize, mode nearest)."""
+    import numpy as np
+    import torch
+    import inputs as I
+    import oracle_lib
+    from ops_cv_amd import aclnn
+    dev = torch.device("cuda:0")
+    L = load_bench_lib()
+    dtype = "fp16"
+    N, C, Hs, Ws, Hd, Wd = 4, 16, 1080, 1920, 2160, 3840
+    in_shape = (N, C, Hd, Wd) if kind == "backward" else (N, C, Hs, Ws)
+    out_shape = (N, C, Hs, Ws) if kind == "backward" else (N, C, Hd, Wd)
+    xs, ys, hx, hy = [], [], [], []
+    x0 = None
+    for s in range(sets):
+        rng = np.random.default_rng(4000 + s)
+        x = I.cast_np(rng.uniform(-1, 1, in_shape).astype(np.float32), dtype)
+        if s == 0:
+            x0 = x
+        xs.append(I.to_torch(x, dtype, dev))
+        ys.append(torch.empty(out_shape, dtype=xs[-1].dtype, device=dev))
+        hx.append(aclnn.tensor_handle(xs[-1], aclnn.ACL_FORMAT_NCHW))
+        hy.append(aclnn.tensor_handle(ys[-1], aclnn.ACL_FORMAT_NCHW))
+    arr = lambda h: (ctypes.c_void_p * len(h))(*h)
+    ax, ay = arr(hx), arr(hy)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ev, wall = ctypes.c_double(0), ctypes.c_double(0)
+    planes = 2
+    if kind == "backward":
+        osz, isz = aclnn.create_int_array([Hd, Wd]), aclnn.create_int_array([N, C, Hs, Ws])
+
+        def run(k):
+            rc = L.opscv_bench_upsample_bilinear2d_backward(ax, ay, sets, osz, isz, True, 2.0, 2.0, None, 0, k, stream,
+                                                            ctypes.byref(ev), ctypes.byref(wall))
+            if rc != 0:
+                raise RuntimeError("bench loop failed rc=%d: %s" % (rc, aclnn.load_library().aclGetRecentErrMsg()))
+            return Timed(ev.value, wall.value, k)
+
+        st, _, ex = aclnn.get_workspace_size_upsample_bilinear2d_backward(hx[0], osz, isz, True, 2.0, 2.0, hy[0])
+        ref = oracle_lib.upsample_bilinear2d_backward(x0.reshape(N * C, 1, Hd, Wd)[:planes], (Hs, Ws), True,
+                                                      dtype=I.oracle_code(dtype))
+        desc = "B4 upsample_bilinear2d_backward fp16 grad(4,16,2160,3840)->(4,16,1080,1920) align_corners=True"
+    else:
+        sc = aclnn.create_float_array([1.0, 1.0, 2.0, 2.0])
+
+        def run(k):
+            rc = L.opscv_bench_resize(ax, ay, sets, sc, b"nearest", None, 0, k, stream, ctypes.byref(ev),
+                                      ctypes.byref(wall))
+            if rc != 0:
+                raise RuntimeError("bench loop failed rc=%d: %s" % (rc, aclnn.load_library().aclGetRecentErrMsg()))
+            return Timed(ev.value, wall.value, k)
+
+        st, _, ex = aclnn.get_workspace_size_resize(hx[0], sc, b"nearest", hy[0])
+        ref = oracle_lib.resize_nearest(x0.reshape(N * C, 1, Hs, Ws)[:planes], (Hd, Wd), dtype=I.oracle_code(dtype))
+        desc = "R4 resize nearest fp16 (4,16,1080,1920)->(4,16,2160,3840)"
+    assert st == 0, aclnn.load_library().aclGetRecentErrMsg()
+    variant = aclnn.executor_variant(ex)
+    aclnn.destroy_executor(ex)
+    t = _finish(L, run, xs, ys, steps, warmup, stream)
+    got = I.from_torch(ys[0], dtype).reshape((N * C, 1) + out_shape[2:])[:planes]
+    parity = _parity(got, ref, dtype, planes_checked=planes)
+    for h in hx + hy:
+        aclnn.destroy_tensor(h)
+    samples = int(np.prod(out_shape))
+    alg = (int(np.prod(in_shape)) + samples) * esize(dtype)
+    return dict(workload=desc, samples=samples, alg_bytes=alg, timed=t, variant=variant, parity=parity, sets=sets,
+                default_modes=True)
+
+
 def roofline_of(r):
     gbs = r["alg_bytes"] / (r["timed"].kernel_us * 1e-6) / 1e9
     name = r["workload"].split(" ")[0]
@@ -431,6 +588,11 @@ def main():
             if name != head:
                 k = args.steps if name == "C2" else max(5, args.steps // 4)
                 others[name] = summary_of(bench_up(name, k, max(2, args.warmup // 4)))
+        # the entry points either side of the path, on shapes of the same scale
+        others["V1_grid_sampler3d"] = summary_of(bench_gs3d(max(10, args.steps // 2), args.warmup))
+        k4 = max(5, args.steps // 4)
+        others["B4_upsample_backward"] = summary_of(bench_resize_like("backward", k4, max(2, args.warmup // 4)))
+        others["R4_resize_nearest"] = summary_of(bench_resize_like("nearest", k4, max(2, args.warmup // 4)))
         line["other_workloads"] = others
     print(json.dumps(line))
 

@@ -81,6 +81,7 @@ typedef enum {
 typedef struct aclTensor aclTensor;
 typedef struct aclIntArray aclIntArray;
 typedef struct aclFloatArray aclFloatArray;
+typedef struct aclBoolArray aclBoolArray;
 typedef struct aclOpExecutor aclOpExecutor;
 typedef void* aclrtStream;
 
@@ -102,6 +103,10 @@ ACLNN_API aclnnStatus aclGetIntArraySize(const aclIntArray* array, uint64_t* siz
 ACLNN_API aclFloatArray* aclCreateFloatArray(const float* value, uint64_t size);
 ACLNN_API aclnnStatus aclDestroyFloatArray(const aclFloatArray* array);
 ACLNN_API aclnnStatus aclGetFloatArraySize(const aclFloatArray* array, uint64_t* size);
+
+ACLNN_API aclBoolArray* aclCreateBoolArray(const bool* value, uint64_t size);
+ACLNN_API aclnnStatus aclDestroyBoolArray(const aclBoolArray* array);
+ACLNN_API aclnnStatus aclGetBoolArraySize(const aclBoolArray* array, uint64_t* size);
 
 /*
  * Releases an executor whose second-phase call will never be made (the second-phase call itself frees

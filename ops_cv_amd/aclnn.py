@@ -96,6 +96,15 @@ def load_library():
     L.aclnnGridSampler2DGetWorkspaceSize.argtypes = [vp, vp, i64, i64, ctypes.c_bool, vp, p_u64, p_vp]
     L.aclnnGridSampler2D.restype = i32
     L.aclnnGridSampler2D.argtypes = [vp, u64, vp, vp]
+    L.aclCreateBoolArray.restype = vp
+    L.aclCreateBoolArray.argtypes = [ctypes.POINTER(ctypes.c_bool), u64]
+    L.aclDestroyBoolArray.restype = i32
+    L.aclDestroyBoolArray.argtypes = [vp]
+    L.aclnnGridSampler2DBackwardGetWorkspaceSize.restype = i32
+    L.aclnnGridSampler2DBackwardGetWorkspaceSize.argtypes = [vp, vp, vp, i64, i64, ctypes.c_bool, vp, vp, vp, p_u64,
+                                                             p_vp]
+    L.aclnnGridSampler2DBackward.restype = i32
+    L.aclnnGridSampler2DBackward.argtypes = [vp, u64, vp, vp]
     L.aclnnGridSampler3DGetWorkspaceSize.restype = i32
     L.aclnnGridSampler3DGetWorkspaceSize.argtypes = [vp, vp, i64, i64, ctypes.c_bool, vp, p_u64, p_vp]
     L.aclnnGridSampler3D.restype = i32
@@ -171,6 +180,29 @@ def get_workspace_size_grid_sampler2d(inp, grid, interpolation_mode, padding_mod
     ex = ctypes.c_void_p(None)
     st = L.aclnnGridSampler2DGetWorkspaceSize(inp, grid, interpolation_mode, padding_mode, bool(align_corners), out,
                                               ctypes.byref(ws), ctypes.byref(ex))
+    return st, ws.value, ex.value
+
+
+def create_bool_array(values):
+    L = load_library()
+    arr = (ctypes.c_bool * len(values))(*[bool(v) for v in values])
+    return L.aclCreateBoolArray(arr, len(values))
+
+
+def destroy_bool_array(handle):
+    if handle:
+        load_library().aclDestroyBoolArray(handle)
+
+
+def get_workspace_size_grid_sampler2d_backward(grad_out, inp, grid, interpolation_mode, padding_mode, align_corners,
+                                               output_mask, input_grad, grid_grad):
+    """Phase 1 of aclnnGridSampler2DBackward on raw handles; returns (status, workspace_bytes, executor_handle)."""
+    L = load_library()
+    ws = ctypes.c_uint64(0)
+    ex = ctypes.c_void_p(None)
+    st = L.aclnnGridSampler2DBackwardGetWorkspaceSize(grad_out, inp, grid, interpolation_mode, padding_mode,
+                                                      bool(align_corners), output_mask, input_grad, grid_grad,
+                                                      ctypes.byref(ws), ctypes.byref(ex))
     return st, ws.value, ex.value
 
 
@@ -291,6 +323,37 @@ def grid_sampler2d(inp, grid, interpolation_mode=0, padding_mode=0, align_corner
         for h in hs:
             destroy_tensor(h)
     return out
+
+
+def grid_sampler2d_backward(grad_out, inp, grid, interpolation_mode=0, padding_mode=0, align_corners=False,
+                            output_mask=(True, True), input_grad=None, grid_grad=None, stream=None, workspace=None):
+    """Both phases of aclnnGridSampler2DBackward on torch CUDA tensors; returns (input_grad, grid_grad).  A gradient
+    whose mask flag is false is left untouched."""
+    torch = _torch()
+    L = load_library()
+    if input_grad is None:
+        input_grad = torch.empty_like(inp)
+    if grid_grad is None:
+        grid_grad = torch.empty_like(grid)
+    hs = [tensor_handle(t) for t in (grad_out, inp, grid, input_grad, grid_grad)]
+    mask = create_bool_array(list(output_mask))
+    try:
+        st, ws, ex = get_workspace_size_grid_sampler2d_backward(hs[0], hs[1], hs[2], interpolation_mode, padding_mode,
+                                                                align_corners, mask, hs[3], hs[4])
+        if st != ACLNN_SUCCESS:
+            raise AclnnError("aclnnGridSampler2DBackwardGetWorkspaceSize", st)
+        if ws > 0 and (workspace is None or workspace.numel() * workspace.element_size() < ws):
+            workspace = torch.empty(ws, dtype=torch.uint8, device=inp.device)
+        wptr = ctypes.c_void_p(workspace.data_ptr()) if ws > 0 else None
+        wsize = workspace.numel() * workspace.element_size() if ws > 0 else 0
+        st = L.aclnnGridSampler2DBackward(wptr, wsize, ex, _stream_handle(stream))
+        if st != ACLNN_SUCCESS:
+            raise AclnnError("aclnnGridSampler2DBackward", st)
+    finally:
+        for h in hs:
+            destroy_tensor(h)
+        destroy_bool_array(mask)
+    return input_grad, grid_grad
 
 
 def grid_sampler3d(inp, grid, interpolation_mode=0, padding_mode=0, align_corners=False, out=None, stream=None,

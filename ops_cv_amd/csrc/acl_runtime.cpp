@@ -131,6 +131,33 @@ aclnnStatus aclGetFloatArraySize(const aclFloatArray* array, uint64_t* size)
     return ACLNN_SUCCESS;
 }
 
+aclBoolArray* aclCreateBoolArray(const bool* value, uint64_t size)
+{
+    if (size > 0 && value == nullptr) {
+        return nullptr;
+    }
+    aclBoolArray* a = new (std::nothrow) aclBoolArray();
+    if (a != nullptr) {
+        a->v.assign(value, value + size);
+    }
+    return a;
+}
+
+aclnnStatus aclDestroyBoolArray(const aclBoolArray* array)
+{
+    delete array;
+    return ACLNN_SUCCESS;
+}
+
+aclnnStatus aclGetBoolArraySize(const aclBoolArray* array, uint64_t* size)
+{
+    if (array == nullptr || size == nullptr) {
+        return ACLNN_ERR_PARAM_NULLPTR;
+    }
+    *size = array->v.size();
+    return ACLNN_SUCCESS;
+}
+
 aclnnStatus aclDestroyAclOpExecutor(aclOpExecutor* executor)
 {
     if (executor == nullptr) {

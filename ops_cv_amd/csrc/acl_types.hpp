@@ -50,6 +50,10 @@ struct aclFloatArray {
     std::vector<float> v;
 };
 
+struct aclBoolArray {
+    std::vector<char> v;  // one byte per flag
+};
+
 namespace opscv {
 
 enum class Elem : int { F32 = 0, F16 = 1, BF16 = 2 };
@@ -76,7 +80,7 @@ struct StridedView {
     int64_t strides[kViewDims] = {0};  // elements
 };
 
-enum class OpKind : int { Nop = 0, GridSampler2D = 1, Resize = 2, ResizeGrad = 3, GridSampler3D = 4 };
+enum class OpKind : int { Nop = 0, GridSampler2D = 1, Resize = 2, ResizeGrad = 3, GridSampler3D = 4, GridSampler2DGrad = 5 };
 
 // Where a kernel operand lives: the tensor's own memory (contiguous view) or a slice of the caller's
 // workspace, known only as an offset until the second phase receives the workspace address.
@@ -108,6 +112,20 @@ struct GridSampler3DArgs {
     const void* x = nullptr;
     const void* grid = nullptr;
     void* y = nullptr;
+};
+
+// Backward of the 2-D sampler.  dx / dgrid may be null (output mask): that gradient is then not computed.
+struct GridSamplerGradArgs {
+    Elem elem = Elem::F32;
+    int interp = 0;
+    int pad = 0;
+    int align = 0;
+    int64_t N = 0, C = 0, Hin = 0, Win = 0, Hout = 0, Wout = 0;
+    const void* gout = nullptr;  // (N,C,Hout,Wout)
+    const void* x = nullptr;     // (N,C,Hin,Win)
+    const void* grid = nullptr;  // (N,Hout,Wout,2)
+    void* dx = nullptr;          // (N,C,Hin,Win)
+    void* dgrid = nullptr;       // (N,Hout,Wout,2)
 };
 
 enum class ResizeMode : int { Bilinear = 0, Copy = 1, Broadcast = 2, FirstPixel = 3, Nearest = 4 };
@@ -150,7 +168,10 @@ struct aclOpExecutor {
     opscv::ResizeArgs rs;
     opscv::ResizeGradArgs rg;
     opscv::GridSampler3DArgs gs3;
+    opscv::GridSamplerGradArgs gsg;
+    int want_out0 = 1, want_out1 = 0;  // which outputs the operator produces (backward output mask)
     opscv::PlannedPtr in0, in1, out0;  // input/self, grid, out
+    opscv::PlannedPtr in2, out1;       // third input and second output of the operators that have them
     // packing work: views gathered into the workspace before the kernel, scattered after it
     struct Pack {
         opscv::StridedView view;

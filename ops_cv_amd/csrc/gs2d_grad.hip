@@ -1,0 +1,268 @@
+// Backward of grid_sampler2d for gfx950: gradient of the input (scatter) and of the grid, both deterministic.
+//
+// Replaces the reference device kernels
+//   image/grid_sampler2_d_grad/op_kernel/arch35/grid_sampler2_d_grad_simt_det.h (deterministic mode) and
+//   image/grid_sampler2_d_grad/op_kernel/arch35/grid_sampler2_d_grad_simt.h      (atomic mode).
+//
+// Gradient of the input.  The reference's deterministic mode walks the grid points of one batch item in chunks of
+// 256; within a chunk it adds, tap after tap (nw, ne, sw, se; or the 16 bicubic taps in index order), the 256
+// contributions one by one in point order, each add rounding to the tensor's element type
+// (grid_sampler2_d_grad_simt_det.h:75-101).  The sum that reaches one element of the gradient is therefore a fixed
+// sequence: its contributions ordered by (chunk, tap, point).  Adds to different elements commute, so only that
+// per-element order has to be kept.  Here a workgroup owns one (batch item, channel, band of the plane): the band
+// lives in LDS, the workgroup walks the chunks in order, and inside a chunk the pending contributions to one
+// element are applied in rounds -- each round an LDS max-reduction elects, per element, the pending contribution
+// that comes first in (tap, point) order, and only the elected ones are added.  The result does not depend on
+// scheduling and equals the sequential order above bit for bit.
+//
+// Gradient of the grid.  One lane per grid point walks the channels in order, as the reference does
+// (grid_sampler2_d_grad_simt_det.h:103-196,279-343); no atomics are involved.
+#include <hip/hip_runtime.h>
+
+#include "gs2d_grad_math.hpp"
+#include "kernels.hpp"
+
+namespace opscv {
+
+namespace {
+
+constexpr int kThreads = 256;         // also the chunk length of the accumulation order
+constexpr uint32_t kKeyBits = 12;     // 16 taps x 256 points
+constexpr uint32_t kEpochMax = (1u << (32 - kKeyBits)) - 1;
+
+struct GradParams {
+    int32_t C, H, W, Ho, Wo;
+    int32_t pad, align;
+    int32_t band_px;  // plane elements per workgroup (dx kernel)
+};
+
+template <typename T, int INTERP>
+__global__ __launch_bounds__(kThreads) void gs2d_grad_input_kernel(const T* __restrict__ gout,
+                                                                    const T* __restrict__ grid, T* __restrict__ dx,
+                                                                    GradParams p)
+{
+    using Taps = GradTaps<T, INTERP>;
+    constexpr int NT = Taps::NT;
+    extern __shared__ uint32_t smem_u32[];
+    float* plane = reinterpret_cast<float*>(smem_u32);
+    uint32_t* owner = smem_u32 + p.band_px;
+
+    const int t = threadIdx.x;
+    const int32_t plane_px = p.H * p.W;
+    const int32_t b0 = blockIdx.x * p.band_px;
+    const int32_t b1 = (b0 + p.band_px < plane_px) ? b0 + p.band_px : plane_px;
+    const int32_t c = blockIdx.y;
+    const int64_t n = blockIdx.z;
+    for (int32_t i = t; i < b1 - b0; i += kThreads) {
+        plane[i] = 0.0f;
+        owner[i] = 0u;
+    }
+    const int32_t points = p.Ho * p.Wo;
+    const T* g_n = grid + n * (int64_t)points * 2;
+    const T* go_nc = gout + (n * p.C + c) * (int64_t)points;
+    uint32_t epoch = 1;
+    for (int32_t base = 0; base < points; base += kThreads) {
+        const int32_t pt = base + t;
+        int32_t off[NT];
+        float val[NT];
+        uint32_t pend = 0;
+        if (pt < points) {
+            Taps tp;
+            decide_grad_taps<T, INTERP>(tp, ElemIO<T>::load(g_n + 2 * (int64_t)pt),
+                                        ElemIO<T>::load(g_n + 2 * (int64_t)pt + 1), p.H, p.W, p.pad, p.align);
+            const float go = ElemIO<T>::load(go_nc + pt);
+#pragma unroll
+            for (int k = 0; k < NT; k++) {
+                off[k] = tp.off[k] - b0;
+                // the contribution is rounded to the element type before it is added
+                val[k] = rt<T>(INTERP == 1 ? go : (INTERP == 0 ? tp.w[k] * go : go * tp.w[k]));
+                if (tp.off[k] >= b0 && tp.off[k] < b1) {
+                    pend |= 1u << k;
+                }
+            }
+        }
+        while (__syncthreads_or((int)pend) != 0) {
+#pragma unroll
+            for (int k = 0; k < NT; k++) {
+                if (pend & (1u << k)) {
+                    atomicMax(&owner[off[k]], (epoch << kKeyBits) | (4095u - (uint32_t)(k * kThreads + t)));
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int k = 0; k < NT; k++) {
+                if ((pend & (1u << k)) &&
+                    owner[off[k]] == ((epoch << kKeyBits) | (4095u - (uint32_t)(k * kThreads + t)))) {
+                    plane[off[k]] = rt<T>(plane[off[k]] + val[k]);
+                    pend &= ~(1u << k);
+                }
+            }
+            epoch++;
+            if (epoch == kEpochMax) {  // uniform: start the election tags over
+                __syncthreads();
+                for (int32_t i = t; i < b1 - b0; i += kThreads) {
+                    owner[i] = 0u;
+                }
+                epoch = 1;
+            }
+        }
+    }
+    // the loop's last barrier has made every add visible
+    T* dx_nc = dx + (n * p.C + c) * (int64_t)plane_px + b0;
+    for (int32_t i = t; i < b1 - b0; i += kThreads) {
+        ElemIO<T>::store(dx_nc + i, plane[i]);
+    }
+}
+
+template <typename T, int INTERP>
+__global__ __launch_bounds__(kThreads) void gs2d_grad_grid_kernel(const T* __restrict__ gout, const T* __restrict__ x,
+                                                                   const T* __restrict__ grid, T* __restrict__ dgrid,
+                                                                   int64_t total, GradParams p)
+{
+    using Taps = GradTaps<T, INTERP>;
+    const int64_t idx = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (idx >= total) {
+        return;
+    }
+    const int32_t points = p.Ho * p.Wo;
+    const int64_t n = idx / points;
+    const int32_t pt = (int32_t)(idx - n * points);
+    if (INTERP == 1) {
+        ElemIO<T>::store(dgrid + 2 * idx, 0.0f);
+        ElemIO<T>::store(dgrid + 2 * idx + 1, 0.0f);
+        return;
+    }
+    Taps tp;
+    decide_grad_taps<T, INTERP>(tp, ElemIO<T>::load(grid + 2 * idx), ElemIO<T>::load(grid + 2 * idx + 1), p.H, p.W,
+                                p.pad, p.align);
+    const int32_t plane_px = p.H * p.W;
+    const T* x_n = x + n * p.C * (int64_t)plane_px;
+    const T* go_n = gout + n * p.C * (int64_t)points + pt;
+    float gix = 0.0f, giy = 0.0f;
+    if (INTERP == 0) {
+        const float dxe = (float)(tp.x0 == INT32_MAX ? tp.x0 : tp.x0 + 1) - tp.fx, dxw = tp.fx - (float)tp.x0;
+        const float dys = (float)(tp.y0 == INT32_MAX ? tp.y0 : tp.y0 + 1) - tp.fy, dyn = tp.fy - (float)tp.y0;
+        for (int32_t c = 0; c < p.C; c++) {
+            const float go = ElemIO<T>::load(go_n + (int64_t)c * points);
+            const T* xc = x_n + (int64_t)c * plane_px;
+            if (tp.off[0] >= 0) {
+                const float v = ElemIO<T>::load(xc + tp.off[0]);
+                gix -= v * dys * go;
+                giy -= v * dxe * go;
+            }
+            if (tp.off[1] >= 0) {
+                const float v = ElemIO<T>::load(xc + tp.off[1]);
+                gix += v * dys * go;
+                giy -= v * dxw * go;
+            }
+            if (tp.off[2] >= 0) {
+                const float v = ElemIO<T>::load(xc + tp.off[2]);
+                gix -= v * dyn * go;
+                giy += v * dxe * go;
+            }
+            if (tp.off[3] >= 0) {
+                const float v = ElemIO<T>::load(xc + tp.off[3]);
+                gix += v * dyn * go;
+                giy += v * dxw * go;
+            }
+        }
+    } else {
+        const float xf = __builtin_floorf(tp.fx), yf = __builtin_floorf(tp.fy);
+        float cx[4], cy[4], cxg[4], cyg[4];
+        cubic_coefficients(cy, tp.fy - yf);
+        cubic_coefficients(cx, tp.fx - xf);
+        cubic_coefficients_grad(cyg, tp.fy - yf);
+        cubic_coefficients_grad(cxg, tp.fx - xf);
+        for (int32_t c = 0; c < p.C; c++) {
+            const float go = ElemIO<T>::load(go_n + (int64_t)c * points);
+            const T* xc = x_n + (int64_t)c * plane_px;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const int32_t o = tp.off[i * 4 + j];
+                    const float v = (o >= 0) ? ElemIO<T>::load(xc + o) : 0.0f;
+                    giy += v * cyg[j] * cx[i] * go;
+                    gix += v * cxg[i] * cy[j] * go;
+                }
+            }
+        }
+    }
+    ElemIO<T>::store(dgrid + 2 * idx, tp.mx * gix);
+    ElemIO<T>::store(dgrid + 2 * idx + 1, tp.my * giy);
+}
+
+template <typename T, int INTERP>
+hipError_t launch_interp(const GridSamplerGradArgs& a, hipStream_t stream)
+{
+    GradParams p;
+    p.C = (int32_t)a.C;
+    p.H = (int32_t)a.Hin;
+    p.W = (int32_t)a.Win;
+    p.Ho = (int32_t)a.Hout;
+    p.Wo = (int32_t)a.Wout;
+    p.pad = a.pad;
+    p.align = a.align;
+    const int64_t plane_px = a.Hin * a.Win;
+    // 8 bytes of LDS per plane element (value + election tag); bands of at most 4096 elements keep a workgroup
+    // at 32 KB so that several share a compute unit
+    p.band_px = (int32_t)(plane_px < 4096 ? plane_px : 4096);
+    if (a.dx != nullptr) {
+        const int64_t bands = (plane_px + p.band_px - 1) / p.band_px;
+        if (bands > INT32_MAX || a.C > 65535 || a.N > 65535) {
+            return hipErrorInvalidValue;
+        }
+        hipLaunchKernelGGL((gs2d_grad_input_kernel<T, INTERP>), dim3((unsigned)bands, (unsigned)a.C, (unsigned)a.N),
+                           dim3(kThreads), (size_t)p.band_px * 8, stream, (const T*)a.gout, (const T*)a.grid,
+                           (T*)a.dx, p);
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) {
+            return e;
+        }
+    }
+    if (a.dgrid != nullptr) {
+        const int64_t total = a.N * a.Hout * a.Wout;
+        const int64_t blocks = (total + kThreads - 1) / kThreads;
+        if (blocks > INT32_MAX) {
+            return hipErrorInvalidValue;
+        }
+        hipLaunchKernelGGL((gs2d_grad_grid_kernel<T, INTERP>), dim3((unsigned)blocks), dim3(kThreads), 0, stream,
+                           (const T*)a.gout, (const T*)a.x, (const T*)a.grid, (T*)a.dgrid, total, p);
+        return hipGetLastError();
+    }
+    return hipSuccess;
+}
+
+template <typename T>
+hipError_t launch_typed(const GridSamplerGradArgs& a, hipStream_t stream)
+{
+    switch (a.interp) {
+        case 0: return launch_interp<T, 0>(a, stream);
+        case 1: return launch_interp<T, 1>(a, stream);
+        case 2: return launch_interp<T, 2>(a, stream);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace
+
+hipError_t launch_grid_sampler2d_grad(const GridSamplerGradArgs& a, hipStream_t stream)
+{
+    if (a.gout == nullptr || a.x == nullptr || a.grid == nullptr || (a.dx == nullptr && a.dgrid == nullptr)) {
+        return hipErrorInvalidValue;
+    }
+    if (a.pad < 0 || a.pad > 2 || a.N <= 0 || a.C <= 0 || a.Hin <= 0 || a.Win <= 0 || a.Hout <= 0 || a.Wout <= 0) {
+        return hipErrorInvalidValue;
+    }
+    if (a.Hin * a.Win > INT32_MAX || a.Hout * a.Wout > INT32_MAX) {
+        return hipErrorInvalidValue;
+    }
+    switch (a.elem) {
+        case Elem::F32: return launch_typed<float>(a, stream);
+        case Elem::F16: return launch_typed<_Float16>(a, stream);
+        case Elem::BF16: return launch_typed<__bf16>(a, stream);
+    }
+    return hipErrorInvalidValue;
+}
+
+}  // namespace opscv

@@ -31,12 +31,21 @@
  *                                  does not fix whether its compiler contracts a*b+c in this file: restated with
  *                                  separate roundings, so bit-exactness to the reference is "parity unpinned",
  *                                  agreement with torch to 1e-5 is what is pinned
+ *   oracle_grid_sampler2d_backward : live torch autograd of grid_sample (all modes, paddings, alignments; fp32 to
+ *                                  1e-5), adjointness with the forward oracle (<forward(x), g> = <x, dx>), finite
+ *                                  differences of the forward oracle for the grid gradient, the reference's example
+ *                                  (examples/test_aclnn_grid_sampler2_d_backward.cpp) against torch.  The reference's
+ *                                  source does not fix whether its compiler contracts a*b+c in these files and its
+ *                                  default mode adds with atomics in arbitrary order: bit-level parity with the
+ *                                  reference is "parity unpinned"; the accumulation order restated is that of its
+ *                                  deterministic mode
  *   oracle_resize_scale          : float bit patterns held by the reference's tiling UT
  *                                  (image/resize_bilinear_v2/tests/ut/op_host/arch35/test_resize_bilinear_v2_tiling.cpp)
  */
 #include "cv_oracle.h"
 
 #include <math.h>
+#include <stdint.h>
 #include <stddef.h>
 #include <string.h>
 #ifdef _OPENMP
@@ -936,6 +945,303 @@ int oracle_grid_sampler3d(const void* x, const void* grid, void* y, int dtype, i
             wgt = dw * dh * dd;
             acc += v * wgt;
             store_from_float(y, dtype, yo, acc);
+        }
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------------------------------
+ * Backward of grid_sampler2d, deterministic mode
+ *   image/grid_sampler2_d_grad/op_kernel/arch35/grid_sampler2_d_grad_simt_det.h:75-413
+ *   image/grid_sampler3_d_grad/op_kernel/arch35/grid_sampler3_d_grad_simt_base.h:50-311
+ * Several intermediates of the reference live in the tensor's element type T; rt() rounds to it.
+ * The reference assigns whole batch items to a core (one per core while N does not exceed the core
+ * count) and walks the item's grid points in chunks of 256 threads; per chunk, channel and tap a
+ * single thread adds the 256 staged contributions in thread order, each add in T.  That loop nest is
+ * restated literally below.  Adds of a staged zero to element 0 for taps outside the image
+ * (grid_sampler2_d_grad_simt_det.h:86-88,93-97) are left out: they can only turn a -0 into +0.
+ * ---------------------------------------------------------------------------------------- */
+static float rt(int dtype, float v)
+{
+    if (dtype == ORACLE_F16) {
+        return oracle_half_to_float(oracle_float_to_half(v));
+    }
+    if (dtype == ORACLE_BF16) {
+        return oracle_bf16_to_float(oracle_float_to_bf16(v));
+    }
+    return v;
+}
+
+static float gsg_unnormalize(int dtype, float coord, int32_t size, int align, float* mult)
+{
+    float c;
+    if (align == 1) {
+        c = (coord + 1) / 2 * (float)(size - 1);
+        *mult = rt(dtype, (float)(size - 1) / 2);
+    } else {
+        c = ((coord + 1) * (float)size - 1) / 2;
+        *mult = rt(dtype, (float)size / 2);
+    }
+    return rt(dtype, c);
+}
+
+static float gsg_clip(int dtype, float coord, int32_t limit, float* g)
+{
+    if (coord <= 0.0f) {
+        *g = 0.0f;
+        return 0.0f;
+    }
+    float max = rt(dtype, (float)(limit - 1));
+    if (coord >= max) {
+        *g = 0.0f;
+        return max;
+    }
+    *g = 1.0f;
+    return coord;
+}
+
+static float gsg_reflect(int dtype, float coord, int64_t twice_low, int64_t twice_high, float* g)
+{
+    if (twice_low == twice_high) {
+        *g = 0.0f;
+        return 0.0f;
+    }
+    float mult;
+    float min = (float)twice_low / 2;
+    float span = (float)(twice_high - twice_low) / 2;
+    coord = rt(dtype, coord - min);
+    if (coord < 0.0f) {
+        mult = -1.0f;
+        coord = -coord;
+    } else {
+        mult = 1.0f;
+    }
+    float extra = fmodf(coord, span);
+    float fl = floorf(coord / span);
+    int odd = (fl < 16777216.0f) && (((int64_t)fl) % 2 != 0);
+    if (!odd) {
+        *g = mult;
+        return rt(dtype, extra + min);
+    }
+    *g = -mult;
+    return rt(dtype, span - extra + min);
+}
+
+static float gsg_source_index(int dtype, float coord, int32_t size, int pad, int align, float* mult)
+{
+    float gc = 0, gr = 0;
+    coord = gsg_unnormalize(dtype, coord, size, align, mult);
+    if (pad == 1) {
+        coord = gsg_clip(dtype, coord, size, &gc);
+        *mult = rt(dtype, *mult * gc);
+    } else if (pad == 2) {
+        if (align) {
+            coord = gsg_reflect(dtype, coord, 0, 2 * ((int64_t)size - 1), &gr);
+        } else {
+            coord = gsg_reflect(dtype, coord, -1, 2 * (int64_t)size - 1, &gr);
+        }
+        coord = gsg_clip(dtype, coord, size, &gc);
+        *mult = rt(dtype, *mult * gr * gc);
+    }
+    if (!isfinite(coord)) {
+        return -100.0f;
+    }
+    return coord;
+}
+
+static int32_t gsg_to_i32(float f)
+{
+    if (f >= 2147483648.0f) {
+        return INT32_MAX;
+    }
+    if (f < -2147483648.0f) {
+        return INT32_MIN;
+    }
+    return (int32_t)f;
+}
+
+/* plane offset of a bicubic tap after padding, -1 outside (simt_base.h:249-311, simt_det.h:239-277) */
+static int64_t gsg_bounded(float x, float y, int32_t W, int32_t H, int pad, int align)
+{
+    if (pad == 0) {
+        if (x < 0 || x >= (float)W || y < 0 || y >= (float)H) {
+            return -1;
+        }
+    } else if (pad == 1) {
+        x = x < 0 ? 0 : (x >= (float)W ? (float)W - 1 : x);
+        y = y < 0 ? 0 : (y >= (float)H ? (float)H - 1 : y);
+    } else {
+        float g;
+        if (align) {
+            x = gsg_reflect(ORACLE_F32, x, 0, 2 * ((int64_t)W - 1), &g);
+            y = gsg_reflect(ORACLE_F32, y, 0, 2 * ((int64_t)H - 1), &g);
+        } else {
+            x = gsg_reflect(ORACLE_F32, x, -1, 2 * (int64_t)W - 1, &g);
+            y = gsg_reflect(ORACLE_F32, y, -1, 2 * (int64_t)H - 1, &g);
+        }
+        x = gsg_clip(ORACLE_F32, x, W, &g);
+        y = gsg_clip(ORACLE_F32, y, H, &g);
+    }
+    int32_t ix = gsg_to_i32(isfinite(x) ? x : -100.0f);
+    int32_t iy = gsg_to_i32(isfinite(y) ? y : -100.0f);
+    if (ix >= 0 && ix < W && iy >= 0 && iy < H) {
+        return (int64_t)iy * W + ix;
+    }
+    return -1;
+}
+
+static void gsg_cubic_coeffs(float c[4], float t)
+{
+    c[0] = oracle_cubic_convolution2(t + 1.0f, -0.75f);
+    c[1] = oracle_cubic_convolution1(t, -0.75f);
+    c[2] = oracle_cubic_convolution1(1.0f - t, -0.75f);
+    c[3] = oracle_cubic_convolution2(2.0f - t, -0.75f);
+}
+
+static void gsg_cubic_coeffs_grad(float c[4], float t)
+{
+    float A = -0.75f;
+    float x = t + 1.0f;
+    c[0] = (3.0f * A * x - 10.0f * A) * x + 8.0f * A;
+    x = t;
+    c[1] = (3.0f * (A + 2.0f) * x - 2.0f * (A + 3.0f)) * x;
+    x = 1.0f - t;
+    c[2] = -((3.0f * (A + 2.0f) * x - 2.0f * (A + 3.0f)) * x);
+    x = 2.0f - t;
+    c[3] = -((3.0f * A * x - 10.0f * A) * x + 8.0f * A);
+}
+
+#define GSG_CHUNK 256
+
+int oracle_grid_sampler2d_backward(const void* gout, const void* x, const void* grid, void* dx, void* dgrid,
+                                   int dtype, int64_t N, int64_t C, int64_t H, int64_t W, int64_t Ho, int64_t Wo,
+                                   int interp, int pad, int align)
+{
+    if (gout == NULL || x == NULL || grid == NULL || dtype < 0 || dtype > 2 || interp < 0 || interp > 2 || pad < 0 ||
+        pad > 2 || H <= 0 || W <= 0) {
+        return -1;
+    }
+    const int64_t points = Ho * Wo, plane = H * W;
+    if (dx != NULL) {
+        for (int64_t i = 0; i < N * C * plane; i++) {
+            store_from_float(dx, dtype, i, 0.0f);
+        }
+    }
+    /* staged contributions of one chunk: [tap][thread] */
+    static _Thread_local int64_t st_idx[16][GSG_CHUNK];
+    static _Thread_local float st_val[16][GSG_CHUNK];
+#ifdef _OPENMP
+#pragma omp parallel for schedule(dynamic)
+#endif
+    for (int64_t n = 0; n < N; n++) {
+        for (int64_t base = 0; base < points; base += GSG_CHUNK) {
+            const int64_t cnt = (points - base < GSG_CHUNK) ? points - base : GSG_CHUNK;
+            float gix[GSG_CHUNK], giy[GSG_CHUNK], mx[GSG_CHUNK], my[GSG_CHUNK];
+            for (int64_t t = 0; t < cnt; t++) {
+                gix[t] = giy[t] = 0.0f;
+            }
+            for (int64_t c = 0; c < C; c++) {
+                const int64_t xin = (n * C + c) * plane;
+                int ntaps = 0;
+                for (int64_t t = 0; t < cnt; t++) {
+                    const int64_t p = base + t;
+                    float fx = load_as_float(grid, dtype, (n * points + p) * 2);
+                    float fy = load_as_float(grid, dtype, (n * points + p) * 2 + 1);
+                    const float go = load_as_float(gout, dtype, (n * C + c) * points + p);
+                    if (interp == 2) {
+                        fy = gsg_unnormalize(dtype, fy, (int32_t)H, align, &my[t]);
+                        fx = gsg_unnormalize(dtype, fx, (int32_t)W, align, &mx[t]);
+                        float xf = floorf(fx), yf = floorf(fy);
+                        float cx[4], cy[4], cxg[4], cyg[4];
+                        gsg_cubic_coeffs(cy, fy - yf);
+                        gsg_cubic_coeffs(cx, fx - xf);
+                        gsg_cubic_coeffs_grad(cyg, fy - yf);
+                        gsg_cubic_coeffs_grad(cxg, fx - xf);
+                        ntaps = 16;
+                        for (int i = 0; i < 4; i++) {
+                            for (int j = 0; j < 4; j++) {
+                                float nx = xf - 1 + i;
+                                float ny = yf - 1 + j;
+                                float weight = cx[i] * cy[j];
+                                float delta = go * weight;
+                                int64_t o = gsg_bounded(nx, ny, (int32_t)W, (int32_t)H, pad, align);
+                                st_idx[i * 4 + j][t] = o;
+                                st_val[i * 4 + j][t] = rt(dtype, delta);
+                                float val = (o >= 0) ? load_as_float(x, dtype, xin + o) : 0.0f;
+                                giy[t] += val * cyg[j] * cx[i] * go;
+                                gix[t] += val * cxg[i] * cy[j] * go;
+                            }
+                        }
+                        continue;
+                    }
+                    fy = gsg_source_index(dtype, fy, (int32_t)H, pad, align, &my[t]);
+                    fx = gsg_source_index(dtype, fx, (int32_t)W, pad, align, &mx[t]);
+                    if (interp == 1) {
+                        int32_t xi = gsg_to_i32(rintf(fx)), yi = gsg_to_i32(rintf(fy));
+                        ntaps = 1;
+                        st_idx[0][t] = (yi >= 0 && xi >= 0 && yi < H && xi < W) ? (int64_t)yi * W + xi : -1;
+                        st_val[0][t] = rt(dtype, go);
+                        continue;
+                    }
+                    int32_t x0 = gsg_to_i32(floorf(fx)), y0 = gsg_to_i32(floorf(fy));
+                    int32_t x1 = (x0 == INT32_MAX) ? x0 : x0 + 1, y1 = (y0 == INT32_MAX) ? y0 : y0 + 1;
+                    float tnw = rt(dtype, ((float)x1 - fx) * ((float)y1 - fy));
+                    float tne = rt(dtype, (fx - (float)x0) * ((float)y1 - fy));
+                    float tsw = rt(dtype, ((float)x1 - fx) * (fy - (float)y0));
+                    float tse = rt(dtype, (fx - (float)x0) * (fy - (float)y0));
+                    const int32_t cxs[4] = {x0, x1, x0, x1}, cys[4] = {y0, y0, y1, y1};
+                    const float ws[4] = {tnw, tne, tsw, tse};
+                    ntaps = 4;
+                    for (int k = 0; k < 4; k++) {
+                        const int in = cys[k] >= 0 && cxs[k] >= 0 && cys[k] < H && cxs[k] < W;
+                        st_idx[k][t] = in ? (int64_t)cys[k] * W + cxs[k] : -1;
+                        st_val[k][t] = rt(dtype, ws[k] * go);
+                    }
+                    if (st_idx[0][t] >= 0) {
+                        float v = load_as_float(x, dtype, xin + st_idx[0][t]);
+                        gix[t] -= v * ((float)y1 - fy) * go;
+                        giy[t] -= v * ((float)x1 - fx) * go;
+                    }
+                    if (st_idx[1][t] >= 0) {
+                        float v = load_as_float(x, dtype, xin + st_idx[1][t]);
+                        gix[t] += v * ((float)y1 - fy) * go;
+                        giy[t] -= v * (fx - (float)x0) * go;
+                    }
+                    if (st_idx[2][t] >= 0) {
+                        float v = load_as_float(x, dtype, xin + st_idx[2][t]);
+                        gix[t] -= v * (fy - (float)y0) * go;
+                        giy[t] += v * ((float)x1 - fx) * go;
+                    }
+                    if (st_idx[3][t] >= 0) {
+                        float v = load_as_float(x, dtype, xin + st_idx[3][t]);
+                        gix[t] += v * (fy - (float)y0) * go;
+                        giy[t] += v * (fx - (float)x0) * go;
+                    }
+                }
+                /* thread 0 of the reference: tap after tap, 256 sequential adds in the element type */
+                if (dx != NULL) {
+                    for (int k = 0; k < ntaps; k++) {
+                        for (int64_t t = 0; t < cnt; t++) {
+                            if (st_idx[k][t] >= 0) {
+                                const int64_t e = xin + st_idx[k][t];
+                                store_from_float(dx, dtype, e, load_as_float(dx, dtype, e) + st_val[k][t]);
+                            }
+                        }
+                    }
+                }
+            }
+            if (dgrid != NULL) {
+                for (int64_t t = 0; t < cnt; t++) {
+                    const int64_t o = (n * points + base + t) * 2;
+                    if (interp == 1) {
+                        store_from_float(dgrid, dtype, o, 0.0f);
+                        store_from_float(dgrid, dtype, o + 1, 0.0f);
+                    } else {
+                        store_from_float(dgrid, dtype, o, mx[t] * gix[t]);
+                        store_from_float(dgrid, dtype, o + 1, my[t] * giy[t]);
+                    }
+                }
+            }
         }
     }
     return 0;

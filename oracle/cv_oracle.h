@@ -127,6 +127,15 @@ int oracle_grid_sampler3d(const void* x, const void* grid, void* y, int dtype, i
                           int64_t Hin, int64_t Win, int64_t Dout, int64_t Hout, int64_t Wout, int interp, int pad,
                           int align, int threads);
 
+/*
+ * Backward of grid_sampler2d in the accumulation order of the reference's deterministic mode
+ * (image/grid_sampler2_d_grad/op_kernel/arch35/grid_sampler2_d_grad_simt_det.h).  gout (N,C,Ho,Wo), x (N,C,H,W),
+ * grid (N,Ho,Wo,2); dx (N,C,H,W) and dgrid (N,Ho,Wo,2) may each be NULL.
+ */
+int oracle_grid_sampler2d_backward(const void* gout, const void* x, const void* grid, void* dx, void* dgrid,
+                                   int dtype, int64_t N, int64_t C, int64_t H, int64_t W, int64_t Ho, int64_t Wo,
+                                   int interp, int pad, int align);
+
 int oracle_max_threads(void);
 
 #ifdef __cplusplus

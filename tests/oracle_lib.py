@@ -96,6 +96,8 @@ def lib():
     L.oracle_gs3d_unnormalize.argtypes = [f32, ctypes.c_int32, ctypes.c_int32]
     L.oracle_gs3d_clip.restype = f32
     L.oracle_gs3d_clip.argtypes = [f32, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32]
+    L.oracle_grid_sampler2d_backward.restype = ctypes.c_int
+    L.oracle_grid_sampler2d_backward.argtypes = [vp] * 5 + [ctypes.c_int] + [i64] * 6 + [ctypes.c_int] * 3
     L.oracle_max_threads.restype = ctypes.c_int
     L.oracle_max_threads.argtypes = []
     _lib = L
@@ -190,6 +192,23 @@ def upsample_bilinear2d_backward(grads, in_hw, align=False, channels_last=False,
     if rc != 0:
         raise ValueError("oracle_upsample_bilinear2d_backward rc=%d" % rc)
     return y
+
+
+def grid_sampler2d_backward(gout, x, grid, interp=0, pad=0, align=False, dtype=None, want=(True, True)):
+    """gout (N,C,Ho,Wo), x (N,C,H,W), grid (N,Ho,Wo,2) -> (dx or None, dgrid or None)"""
+    gout, x, grid = (np.ascontiguousarray(a) for a in (gout, x, grid))
+    code = _code_of(x) if dtype is None else dtype
+    N, C, H, W = x.shape
+    _, Ho, Wo, _ = grid.shape
+    assert gout.shape == (N, C, Ho, Wo)
+    dx = np.empty_like(x) if want[0] else None
+    dg = np.empty_like(grid) if want[1] else None
+    rc = lib().oracle_grid_sampler2d_backward(_ptr(gout), _ptr(x), _ptr(grid), _ptr(dx) if want[0] else None,
+                                              _ptr(dg) if want[1] else None, code, N, C, H, W, Ho, Wo, interp, pad,
+                                              int(bool(align)))
+    if rc != 0:
+        raise ValueError("oracle_grid_sampler2d_backward rc=%d" % rc)
+    return dx, dg
 
 
 def grid_sampler3d(x, grid, interp=0, pad=0, align=False, dtype=None, threads=0):

@@ -5,7 +5,8 @@ the GetWorkspaceSize phase: image/grid_sample/tests/ut/op_host/op_api/test_aclnn
 image/upsample_bilinear2d/tests/ut/op_host/op_api/test_aclnn_upsample_bilinear_2d.cpp,
 image/resize_bilinear_v2/tests/ut/op_host/op_api/test_aclnn_resize.cpp,
 image/resize_bilinear_v2_grad/tests/ut/op_host/op_api/test_aclnn_upsample_bilineard_2d_backward.cpp,
-image/grid_sample/tests/ut/op_host/op_api/test_aclnn_grid_sampler3d.cpp.
+image/grid_sample/tests/ut/op_host/op_api/test_aclnn_grid_sampler3d.cpp,
+image/grid_sampler2_d_grad/tests/ut/op_host/op_api/test_aclnn_grid_sampler2d_backward.cpp.
 """
 import ctypes
 import os
@@ -416,3 +417,67 @@ def test_grid_sampler3d_status_codes(aclnn, desc):
     # a strided NCDHW view is packed too
     st, ws, _ = _gs3(aclnn, desc, strides=(18, 18, 18, 6, 2), storage=(36,))
     assert st == 0 and ws >= 2 * 9 * 4
+
+
+_KEEP = object()
+
+
+def _gsb(aclnn, desc, gout=(1, 1, 3, 3), inp=(1, 1, 5, 8), grid=(1, 3, 3, 2), dx=_KEEP, dgrid=_KEEP, dt=None,
+         dts=None, interp=0, pad=0, align=False, mask=(True, True), **kw):
+    dt = aclnn.ACL_FLOAT if dt is None else dt
+    dts = dts or {}
+    dx = inp if dx is _KEEP else dx
+    dgrid = grid if dgrid is _KEEP else dgrid
+    hs = [desc.t(shape, dts.get(name, dt), **(kw if name == "inp" else {}))
+          for name, shape in (("gout", gout), ("inp", inp), ("grid", grid), ("dx", dx), ("dgrid", dgrid))]
+    m = aclnn.create_bool_array(list(mask)) if mask is not None else None
+    st, ws, ex = aclnn.get_workspace_size_grid_sampler2d_backward(hs[0], hs[1], hs[2], interp, pad, align, m, hs[3],
+                                                                  hs[4])
+    variant = aclnn.executor_variant(ex) if ex else None
+    if ex:
+        assert aclnn.destroy_executor(ex) == 0
+    aclnn.destroy_bool_array(m)
+    return st, ws, variant
+
+
+def test_grid_sampler2d_backward_status_codes(aclnn, desc):
+    """test_aclnn_grid_sampler2d_backward.cpp and the check order of aclnn_grid_sampler2d_backward.cpp:195-243"""
+    INV, NULL = aclnn.ACLNN_ERR_PARAM_INVALID, aclnn.ACLNN_ERR_PARAM_NULLPTR
+    # case_1: the example shapes, float; 16-bit types as on the newest parts
+    for dt in (aclnn.ACL_FLOAT, aclnn.ACL_FLOAT16, aclnn.ACL_BF16):
+        assert _gsb(aclnn, desc, dt=dt) == (0, 0, "gs2d_grad_ordered")
+    # case_2..case_6: each tensor missing in turn
+    for missing in ("gout", "inp", "grid", "dx", "dgrid"):
+        assert _gsb(aclnn, desc, **{missing: None})[0] == NULL, missing
+    # a missing mask succeeds as a no-op before anything else is looked at, even with tensors missing
+    assert _gsb(aclnn, desc, mask=None, inp=None) == (0, 0, "")
+    # both flags false: a no-op; one flag: that gradient only
+    assert _gsb(aclnn, desc, mask=(False, False)) == (0, 0, "")
+    assert _gsb(aclnn, desc, mask=(True, False))[0] == 0 and _gsb(aclnn, desc, mask=(False, True))[0] == 0
+    assert _gsb(aclnn, desc, mask=(True,))[0] == INV
+    assert _gsb(aclnn, desc, mask=(True, True, True))[0] == INV
+    # dtypes: all five equal, from the list; DOUBLE passes the list but has no kernel here
+    for name in ("gout", "grid", "dx", "dgrid"):
+        assert _gsb(aclnn, desc, dts={name: aclnn.ACL_FLOAT16})[0] == INV, name
+    assert _gsb(aclnn, desc, dt=aclnn.ACL_INT32)[0] == INV
+    assert _gsb(aclnn, desc, dt=aclnn.ACL_DOUBLE)[0] == INV
+    # attributes
+    assert _gsb(aclnn, desc, interp=3)[0] == INV and _gsb(aclnn, desc, interp=-1)[0] == INV
+    assert _gsb(aclnn, desc, pad=3)[0] == INV
+    assert _gsb(aclnn, desc, interp=2, pad=2, align=True)[0] == 0
+    # shapes
+    assert _gsb(aclnn, desc, inp=(1, 5, 8), dx=(1, 5, 8))[0] == INV
+    assert _gsb(aclnn, desc, gout=(2, 1, 3, 3))[0] == INV          # batch
+    assert _gsb(aclnn, desc, gout=(1, 2, 3, 3))[0] == INV          # channels
+    assert _gsb(aclnn, desc, inp=(1, 1, 0, 8), dx=(1, 1, 0, 8))[0] == INV
+    assert _gsb(aclnn, desc, gout=(1, 1, 3, 4))[0] == INV          # grid vs gradOutput
+    assert _gsb(aclnn, desc, grid=(1, 3, 3, 3), dgrid=(1, 3, 3, 3))[0] == INV
+    assert _gsb(aclnn, desc, dx=(1, 1, 5, 7))[0] == INV
+    assert _gsb(aclnn, desc, dgrid=(1, 3, 2, 2))[0] == INV
+    # empty tensors: success without work
+    assert _gsb(aclnn, desc, gout=(0, 1, 3, 3), inp=(0, 1, 5, 8), grid=(0, 3, 3, 2)) == (0, 0, "")
+    # case_9_BIGC: 4096 channels are fine
+    assert _gsb(aclnn, desc, gout=(1, 4096, 3, 3), inp=(1, 4096, 5, 8))[0] == 0
+    # a strided input view needs workspace
+    st, ws, _ = _gsb(aclnn, desc, strides=(80, 80, 16, 2), storage=(80,))
+    assert st == 0 and ws >= 40 * 4

@@ -357,3 +357,74 @@ def test_grid_sampler3d_layouts_and_views(oracle, device, aclnn):
     y = aclnn.grid_sampler3d(I.to_torch(x, "fp16", device), I.to_torch(g, "fp16", device), 0, 0, False)
     torch.cuda.synchronize()
     assert np.array_equal(I.from_torch(y, "fp16").view(np.uint16), ref.view(np.uint16))
+
+
+@pytest.mark.parametrize("dtype", I.DTYPES)
+@pytest.mark.parametrize("interp", [0, 1, 2])
+def test_grid_sampler2d_backward(oracle, device, aclnn, dtype, interp):
+    """aclnnGridSampler2DBackward against the oracle, bit for bit, both gradients: every padding and alignment,
+    several chunks of 256 points, planes larger than one LDS band, points piling up on few texels, special grid
+    values"""
+    torch = _torch()
+    rng = np.random.default_rng(600 + interp)
+    shapes = [(2, 3, 5, 8, 3, 3), (1, 2, 9, 11, 23, 29), (2, 1, 70, 80, 20, 30), (1, 4, 1, 1, 17, 31),
+              (1, 2, 3, 2, 40, 40)]
+    for (N, C, H, W, Ho, Wo) in shapes:
+        x = I.cast_np(rng.standard_normal((N, C, H, W)).astype(np.float32), dtype)
+        g32 = rng.uniform(-1.5, 1.5, (N, Ho, Wo, 2)).astype(np.float32)
+        flat = g32.reshape(-1, 2)
+        special = np.array([np.nan, np.inf, -np.inf, 1e30, -1e30, 1.0, -1.0, 0.0], np.float32)
+        for j in range(min(len(special), flat.shape[0])):
+            flat[j, j % 2] = special[j]
+        g = I.cast_np(g32, dtype)
+        go = I.cast_np(rng.standard_normal((N, C, Ho, Wo)).astype(np.float32), dtype)
+        for pad in range(3):
+            for align in (False, True):
+                rdx, rdg = oracle.grid_sampler2d_backward(go, x, g, interp, pad, align, dtype=I.oracle_code(dtype))
+                dx, dg = aclnn.grid_sampler2d_backward(I.to_torch(go, dtype, device), I.to_torch(x, dtype, device),
+                                                       I.to_torch(g, dtype, device), interp, pad, align)
+                torch.cuda.synchronize()
+                for got, ref, what in ((I.from_torch(dx, dtype), rdx, "dx"), (I.from_torch(dg, dtype), rdg, "dgrid")):
+                    rn = np.isnan(I.as_f32(ref, dtype))
+                    assert np.array_equal(np.isnan(I.as_f32(got, dtype)), rn), (what, N, C, H, W, pad, align)
+                    assert np.array_equal(np.where(rn, 0, _bits(got, dtype)), np.where(rn, 0, _bits(ref, dtype))), \
+                        (what, N, C, H, W, Ho, Wo, pad, align)
+
+
+def test_grid_sampler2d_backward_mask_views_and_torch(oracle, device, aclnn):
+    torch = _torch()
+    import torch.nn.functional as F
+    rng = np.random.default_rng(610)
+    N, C, H, W, Ho, Wo = 2, 3, 12, 10, 9, 14
+    x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+    g = rng.uniform(-1.2, 1.2, (N, Ho, Wo, 2)).astype(np.float32)
+    go = rng.standard_normal((N, C, Ho, Wo)).astype(np.float32)
+    xt, gt, got = (torch.from_numpy(a).to(device) for a in (x, g, go))
+    # masked outputs stay untouched
+    dx = torch.full((N, C, H, W), 7.0, device=device)
+    dg = torch.full((N, Ho, Wo, 2), 7.0, device=device)
+    aclnn.grid_sampler2d_backward(got, xt, gt, 0, 0, False, (True, False), dx, dg)
+    torch.cuda.synchronize()
+    rdx, rdg = oracle.grid_sampler2d_backward(go, x, g, 0, 0, False)
+    assert np.array_equal(dx.cpu().numpy(), rdx) and (dg == 7.0).all()
+    dx.fill_(7.0)
+    aclnn.grid_sampler2d_backward(got, xt, gt, 0, 0, False, (False, True), dx, dg)
+    torch.cuda.synchronize()
+    assert np.array_equal(dg.cpu().numpy(), rdg) and (dx == 7.0).all()
+    # strided views on both sides
+    xv = torch.from_numpy(np.ascontiguousarray(x.transpose(0, 1, 3, 2))).to(device).transpose(2, 3)
+    dxbig = torch.full((N, C, H, W + 3), -1.0, device=device)
+    dgbig = torch.full((N, Ho, Wo, 4), -1.0, device=device)
+    aclnn.grid_sampler2d_backward(got, xv, gt, 0, 1, True, (True, True), dxbig[..., 1:1 + W], dgbig[..., 1:3])
+    torch.cuda.synchronize()
+    rdx, rdg = oracle.grid_sampler2d_backward(go, x, g, 0, 1, True)
+    assert np.array_equal(dxbig[..., 1:1 + W].cpu().numpy(), rdx) and np.array_equal(dgbig[..., 1:3].cpu().numpy(), rdg)
+    assert (dxbig[..., 0] == -1.0).all() and (dgbig[..., 3] == -1.0).all()
+    # live torch autograd on the device (tolerance: another summation order)
+    for mode, m in (("bilinear", 0), ("bicubic", 2)):
+        xa, ga = xt.clone().requires_grad_(True), gt.clone().requires_grad_(True)
+        F.grid_sample(xa, ga, mode=mode, padding_mode="border", align_corners=False).backward(got)
+        dx, dg = aclnn.grid_sampler2d_backward(got, xt, gt, m, 1, False)
+        torch.cuda.synchronize()
+        assert (dx - xa.grad).abs().max().item() <= 1e-4
+        assert ((dg - ga.grad).abs() > 1e-3).float().mean().item() <= 0.02

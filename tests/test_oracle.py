@@ -589,3 +589,81 @@ def test_live_torch_grid_sample3d(oracle):
     want = F.grid_sample(torch.from_numpy(x.astype(np.float32)), torch.from_numpy(g.astype(np.float32)),
                          mode="bilinear", padding_mode="zeros", align_corners=False).numpy()
     assert np.abs(got - want).max() <= 2e-3 * max(1.0, np.abs(want).max())
+
+
+# ---- backward of the 2-D sampler ----
+
+def _torch_gs_backward(x, g, go, mode, pad, align):
+    import torch
+    import torch.nn.functional as F
+    xt = torch.from_numpy(x).requires_grad_(True)
+    gt = torch.from_numpy(g).requires_grad_(True)
+    y = F.grid_sample(xt, gt, mode=mode, padding_mode=pad, align_corners=align)
+    y.backward(torch.from_numpy(go))
+    return xt.grad.numpy(), gt.grad.numpy()
+
+
+def test_grid_sampler2d_backward_against_torch_autograd(oracle):
+    rng = np.random.default_rng(41)
+    modes = ["bilinear", "nearest", "bicubic"]
+    for trial in range(6):
+        N, C = 2, 3
+        H, W = rng.integers(2, 14, 2)
+        Ho, Wo = rng.integers(1, 24, 2)  # up to 529 points: more than one chunk of 256
+        x = rng.standard_normal((N, C, H, W)).astype(np.float32)
+        g = rng.uniform(-1.4, 1.4, (N, Ho, Wo, 2)).astype(np.float32)
+        go = rng.standard_normal((N, C, Ho, Wo)).astype(np.float32)
+        for m in range(3):
+            for p in range(3):
+                for a in (False, True):
+                    dx, dg = oracle.grid_sampler2d_backward(go, x, g, m, p, a)
+                    wx, wg = _torch_gs_backward(x, g, go, modes[m], PADS[p], a)
+                    tol = 2e-5 if m < 2 else 1e-4
+                    assert np.abs(dx - wx).max() <= tol * max(1.0, np.abs(wx).max()), (trial, m, p, a)
+                    # the grid gradient jumps where a coordinate crosses a texel or a reflection point: compare
+                    # away from those
+                    bad = np.abs(dg - wg) > tol * max(1.0, np.abs(wg).max())
+                    assert bad.mean() <= 0.02, (trial, m, p, a, bad.mean())
+                    # masked outputs
+                    only_dx, none = oracle.grid_sampler2d_backward(go, x, g, m, p, a, want=(True, False))
+                    assert none is None and np.array_equal(only_dx, dx)
+
+
+def test_grid_sampler2d_backward_adjoint_and_example(oracle):
+    rng = np.random.default_rng(42)
+    x = rng.standard_normal((1, 2, 9, 11)).astype(np.float32)
+    g = rng.uniform(-1.2, 1.2, (1, 13, 7, 2)).astype(np.float32)
+    go = rng.standard_normal((1, 2, 13, 7)).astype(np.float32)
+    for m in range(3):
+        for p in range(3):
+            # the forward is linear in x, dx is its adjoint applied to gout
+            y = oracle.grid_sampler2d(x, g, m, p, False)
+            dx, _ = oracle.grid_sampler2d_backward(go, x, g, m, p, False)
+            lhs = float((y.astype(np.float64) * go).sum())
+            rhs = float((x.astype(np.float64) * dx).sum())
+            assert abs(lhs - rhs) <= 1e-4 * max(1.0, abs(lhs)), (m, p)
+    # the reference's example (examples/test_aclnn_grid_sampler2_d_backward.cpp): 5x8 ramp, 3x3 grid on the corners,
+    # centres and edge midpoints, gradOutput of ones
+    x = np.arange(1, 41, dtype=np.float32).reshape(1, 1, 5, 8)
+    g = np.array([-1, -1, 0, -1, 1, -1, -1, 0, 0, 0, 1, 0, -1, 1, 0, 1, 1, 1], np.float32).reshape(1, 3, 3, 2)
+    go = np.ones((1, 1, 3, 3), np.float32)
+    dx, dg = oracle.grid_sampler2d_backward(go, x, g, 0, 0, False)
+    wx, wg = _torch_gs_backward(x, g, go, "bilinear", "zeros", False)
+    assert np.allclose(dx, wx, atol=1e-6) and np.allclose(dg, wg, atol=1e-5)
+    assert abs(dx.sum() - 4 * 0.25 - 4 * 0.5 - 1.0) < 1e-6  # corners keep 1/4, edge midpoints 1/2, the centre all
+
+
+def test_grid_sampler2d_backward_order_is_sequential_in_element_type(oracle):
+    """many points landing on one texel: the sum is the left-to-right sum in the element type, chunk after chunk"""
+    n_pts = 600
+    x = np.zeros((1, 1, 1, 1), np.float16)
+    g = np.zeros((1, 1, n_pts, 2), np.float16)  # all at the centre of the single texel
+    go = (np.arange(n_pts) % 7 + 0.25).astype(np.float16).reshape(1, 1, 1, n_pts)
+    dx, _ = oracle.grid_sampler2d_backward(go, x, g, 1, 0, False)
+    acc = np.float16(0)
+    for v in go.ravel():
+        acc = np.float16(np.float32(acc) + np.float32(v))
+    assert dx.ravel()[0] == acc
+    # bilinear at the exact centre: only the north-west tap has weight 1; the other taps add +0 in between
+    dxb, _ = oracle.grid_sampler2d_backward(go, x, g, 0, 1, False)
+    assert dxb.ravel()[0] == acc
