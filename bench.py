@@ -102,6 +102,9 @@ def load_bench_lib():
     L.opscv_bench_upsample_bilinear2d.argtypes = [ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.c_int, vp,
                                                  ctypes.c_bool, ctypes.c_double, ctypes.c_double, vp, u64,
                                                  ctypes.c_int, vp, pd, pd]
+    L.opscv_bench_grid_sampler2d_backward.restype = ctypes.c_int
+    L.opscv_bench_grid_sampler2d_backward.argtypes = [ctypes.POINTER(vp)] * 5 + [ctypes.c_int, i64, i64, ctypes.c_bool,
+                                                                                 vp, vp, u64, ctypes.c_int, vp, pd, pd]
     L.opscv_bench_grid_sampler3d.restype = ctypes.c_int
     L.opscv_bench_grid_sampler3d.argtypes = L.opscv_bench_grid_sampler2d.argtypes
     L.opscv_bench_upsample_bilinear2d_backward.restype = ctypes.c_int
@@ -384,6 +387,66 @@ def bench_gs3d(steps, warmup, sets=4):
                 parity=parity, sets=sets, default_modes=True)
 
 
+def bench_gs_backward(steps, warmup, sets=4, mask=(True, True)):
+    """Backward of the headline sampler workload (fp16 N16 C256 64x64, affine grid): both gradients."""
+    import numpy as np
+    import torch
+    import inputs as I
+    import oracle_lib
+    from ops_cv_amd import aclnn
+    dev = torch.device("cuda:0")
+    L = load_bench_lib()
+    w = GS_WORKLOADS["C3"]
+    dtype = w["dtype"]
+    N, C, H, W = w["x"]
+    _, Ho, Wo = w["grid"]
+    ts, hs = [[] for _ in range(5)], [[] for _ in range(5)]
+    first = None
+    for s in range(sets):
+        x, g = make_gs_inputs("C3", 5000 + s)
+        go = I.cast_np(np.random.default_rng(5100 + s).standard_normal((N, C, Ho, Wo)).astype(np.float32), dtype)
+        if s == 0:
+            first = (go, x, g)
+        tens = [I.to_torch(go, dtype, dev), I.to_torch(x, dtype, dev), I.to_torch(g, dtype, dev)]
+        tens += [torch.empty_like(tens[1]), torch.empty_like(tens[2])]
+        for lst, hl, t in zip(ts, hs, tens):
+            lst.append(t)
+            hl.append(aclnn.tensor_handle(t))
+    arr = lambda h: (ctypes.c_void_p * len(h))(*h)
+    arrs = [arr(h) for h in hs]
+    m = aclnn.create_bool_array(list(mask))
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ev, wall = ctypes.c_double(0), ctypes.c_double(0)
+
+    def run(k):
+        rc = L.opscv_bench_grid_sampler2d_backward(*arrs, sets, 0, 0, False, m, None, 0, k, stream, ctypes.byref(ev),
+                                                   ctypes.byref(wall))
+        if rc != 0:
+            raise RuntimeError("bench loop failed rc=%d: %s" % (rc, aclnn.load_library().aclGetRecentErrMsg()))
+        return Timed(ev.value, wall.value, k)
+
+    st, _, ex = aclnn.get_workspace_size_grid_sampler2d_backward(hs[0][0], hs[1][0], hs[2][0], 0, 0, False, m,
+                                                                 hs[3][0], hs[4][0])
+    assert st == 0
+    variant = aclnn.executor_variant(ex)
+    aclnn.destroy_executor(ex)
+    t = _finish(L, run, ts[0], ts[3], steps, warmup, stream)
+    rdx, rdg = oracle_lib.grid_sampler2d_backward(*first, 0, 0, False, dtype=I.oracle_code(dtype))
+    parity = _parity(I.from_torch(ts[3][0], dtype), rdx, dtype)
+    parity["grid_grad_bit_exact"] = bool(np.array_equal(I.from_torch(ts[4][0], dtype).view(np.uint8),
+                                                        rdg.view(np.uint8)))
+    for hl in hs:
+        for h in hl:
+            aclnn.destroy_tensor(h)
+    aclnn.destroy_bool_array(m)
+    e = esize(dtype)
+    # gradOutput read for both gradients' kernels, input read once, grid read, both gradients written
+    alg = (N * C * Ho * Wo + 2 * N * C * H * W + 2 * N * Ho * Wo * 2) * e
+    return dict(workload="G3 grid_sampler2d_backward fp16 x(16,256,64,64) grid(16,64,64,2) bilinear zeros "
+                         "align_corners=False both gradients", samples=N * C * Ho * Wo, alg_bytes=alg, timed=t,
+                variant=variant, parity=parity, sets=sets, default_modes=True)
+
+
 def bench_resize_like(kind, steps, warmup, sets=2):
     """The 4K workload through the neighbouring entry points: kind "backward" (aclnnUpsampleBilinear2dBackward, the
     gradient of the 2x upscale) or "nearest" (aclnnResize, mode nearest)."""
@@ -591,6 +654,7 @@ def main():
         # the entry points either side of the path, on shapes of the same scale
         others["V1_grid_sampler3d"] = summary_of(bench_gs3d(max(10, args.steps // 2), args.warmup))
         k4 = max(5, args.steps // 4)
+        others["G3_grid_sampler2d_backward"] = summary_of(bench_gs_backward(k4, max(2, args.warmup // 4)))
         others["B4_upsample_backward"] = summary_of(bench_resize_like("backward", k4, max(2, args.warmup // 4)))
         others["R4_resize_nearest"] = summary_of(bench_resize_like("nearest", k4, max(2, args.warmup // 4)))
         line["other_workloads"] = others

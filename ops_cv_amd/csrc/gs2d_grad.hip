@@ -61,16 +61,27 @@ __global__ __launch_bounds__(kThreads) void gs2d_grad_input_kernel(const T* __re
     const T* g_n = grid + n * (int64_t)points * 2;
     const T* go_nc = gout + (n * p.C + c) * (int64_t)points;
     uint32_t epoch = 1;
+    // the grid point and incoming gradient of the next chunk are requested before the rounds of this one
+    float gx_next = 0.0f, gy_next = 0.0f, go_next = 0.0f;
+    if (t < points) {
+        gx_next = ElemIO<T>::load(g_n + 2 * (int64_t)t);
+        gy_next = ElemIO<T>::load(g_n + 2 * (int64_t)t + 1);
+        go_next = ElemIO<T>::load(go_nc + t);
+    }
     for (int32_t base = 0; base < points; base += kThreads) {
         const int32_t pt = base + t;
+        const float gx = gx_next, gy = gy_next, go = go_next;
+        if (pt + kThreads < points) {
+            gx_next = ElemIO<T>::load(g_n + 2 * (int64_t)(pt + kThreads));
+            gy_next = ElemIO<T>::load(g_n + 2 * (int64_t)(pt + kThreads) + 1);
+            go_next = ElemIO<T>::load(go_nc + pt + kThreads);
+        }
         int32_t off[NT];
         float val[NT];
         uint32_t pend = 0;
         if (pt < points) {
             Taps tp;
-            decide_grad_taps<T, INTERP>(tp, ElemIO<T>::load(g_n + 2 * (int64_t)pt),
-                                        ElemIO<T>::load(g_n + 2 * (int64_t)pt + 1), p.H, p.W, p.pad, p.align);
-            const float go = ElemIO<T>::load(go_nc + pt);
+            decide_grad_taps<T, INTERP>(tp, gx, gy, p.H, p.W, p.pad, p.align);
 #pragma unroll
             for (int k = 0; k < NT; k++) {
                 off[k] = tp.off[k] - b0;
@@ -142,29 +153,51 @@ __global__ __launch_bounds__(kThreads) void gs2d_grad_grid_kernel(const T* __res
     if (INTERP == 0) {
         const float dxe = (float)(tp.x0 == INT32_MAX ? tp.x0 : tp.x0 + 1) - tp.fx, dxw = tp.fx - (float)tp.x0;
         const float dys = (float)(tp.y0 == INT32_MAX ? tp.y0 : tp.y0 + 1) - tp.fy, dyn = tp.fy - (float)tp.y0;
-        for (int32_t c = 0; c < p.C; c++) {
-            const float go = ElemIO<T>::load(go_n + (int64_t)c * points);
+        // The sums run over the channels in order; the loads do not depend on them, so they are issued a group of
+        // channels ahead (a lane has one grid point and would otherwise wait out every load in turn).
+        constexpr int U = 8;
+        const bool ok0 = tp.off[0] >= 0, ok1 = tp.off[1] >= 0, ok2 = tp.off[2] >= 0, ok3 = tp.off[3] >= 0;
+        const int32_t o0 = ok0 ? tp.off[0] : 0, o1 = ok1 ? tp.off[1] : 0, o2 = ok2 ? tp.off[2] : 0,
+                      o3 = ok3 ? tp.off[3] : 0;
+        auto accumulate = [&](float go, float v0, float v1, float v2, float v3) {
+            if (ok0) {
+                gix -= v0 * dys * go;
+                giy -= v0 * dxe * go;
+            }
+            if (ok1) {
+                gix += v1 * dys * go;
+                giy -= v1 * dxw * go;
+            }
+            if (ok2) {
+                gix -= v2 * dyn * go;
+                giy += v2 * dxe * go;
+            }
+            if (ok3) {
+                gix += v3 * dyn * go;
+                giy += v3 * dxw * go;
+            }
+        };
+        int32_t c = 0;
+        for (; c + U <= p.C; c += U) {
+            float go[U], v[U][4];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const T* xc = x_n + (int64_t)(c + u) * plane_px;
+                go[u] = ElemIO<T>::load(go_n + (int64_t)(c + u) * points);
+                v[u][0] = ElemIO<T>::load(xc + o0);
+                v[u][1] = ElemIO<T>::load(xc + o1);
+                v[u][2] = ElemIO<T>::load(xc + o2);
+                v[u][3] = ElemIO<T>::load(xc + o3);
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                accumulate(go[u], v[u][0], v[u][1], v[u][2], v[u][3]);
+            }
+        }
+        for (; c < p.C; c++) {
             const T* xc = x_n + (int64_t)c * plane_px;
-            if (tp.off[0] >= 0) {
-                const float v = ElemIO<T>::load(xc + tp.off[0]);
-                gix -= v * dys * go;
-                giy -= v * dxe * go;
-            }
-            if (tp.off[1] >= 0) {
-                const float v = ElemIO<T>::load(xc + tp.off[1]);
-                gix += v * dys * go;
-                giy -= v * dxw * go;
-            }
-            if (tp.off[2] >= 0) {
-                const float v = ElemIO<T>::load(xc + tp.off[2]);
-                gix -= v * dyn * go;
-                giy += v * dxe * go;
-            }
-            if (tp.off[3] >= 0) {
-                const float v = ElemIO<T>::load(xc + tp.off[3]);
-                gix += v * dyn * go;
-                giy += v * dxw * go;
-            }
+            accumulate(ElemIO<T>::load(go_n + (int64_t)c * points), ElemIO<T>::load(xc + o0),
+                       ElemIO<T>::load(xc + o1), ElemIO<T>::load(xc + o2), ElemIO<T>::load(xc + o3));
         }
     } else {
         const float xf = __builtin_floorf(tp.fx), yf = __builtin_floorf(tp.fy);
