@@ -92,7 +92,7 @@ const char* opscvExecutorVariant(const aclOpExecutor* executor)
     switch (executor->kind) {
         case OpKind::GridSampler2D: return grid_sampler2d_variant(executor->gs);
         case OpKind::Resize: return resize_variant(executor->rs);
-        case OpKind::ResizeGrad: return executor->rg.copy ? "copy" : (executor->rg.user_scales ? "resize_grad_gather_scales" : "resize_grad_gather");
+        case OpKind::ResizeGrad: return executor->rg.copy ? "copy" : resize_grad_variant(executor->rg);
         case OpKind::GridSampler2DGrad: return "gs2d_grad_ordered";
         case OpKind::GridSampler3D: return executor->gs3.interp == 0 ? "gs3d_bilinear" : "gs3d_nearest";
         default: break;

@@ -31,6 +31,7 @@ hipError_t launch_grid_sampler2d_taps(const GridSamplerArgs& a, TapRecord* taps,
 hipError_t launch_grid_sampler2d_bicubic_taps(const GridSamplerArgs& a, BicubicTapRecord* taps, hipStream_t stream);
 hipError_t launch_resize(const ResizeArgs& a, hipStream_t stream);
 hipError_t launch_resize_grad(const ResizeGradArgs& a, hipStream_t stream);
+const char* resize_grad_variant(const ResizeGradArgs& a);  // which kernel launch_resize_grad picks (x may be null)
 hipError_t launch_grid_sampler2d_grad(const GridSamplerGradArgs& a, hipStream_t stream);
 hipError_t launch_grid_sampler3d(const GridSampler3DArgs& a, hipStream_t stream);
 

@@ -173,9 +173,173 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_kernel(const TI* __r
     }
 }
 
+
+// LDS-tiled variant of resize_grad_kernel for NCHW.  A workgroup owns (plane, tile of kTileRows x 128 elements of
+// the outgoing gradient).  The incoming-gradient rows and columns the tile's lanes will visit form one rectangle
+// (start of the first lane, largest end over all lanes, found with the very loops the lanes run later); it is
+// copied into LDS with independent 4-byte loads -- all in flight together, where the gather variant waits for one
+// two-byte load per visit -- and the lanes then run the unchanged visiting loops on LDS.  A rectangle that does not
+// fit the LDS capacity is read from global memory instead (same loops, same result).
+// The visiting loops of resize_grad_kernel over a row-major array whose element (y0, x0) is base[0].
+template <typename TI>
+__device__ __forceinline__ float visit_sum(const TI* base, int32_t pitch, int32_t y0, int32_t x0, int32_t in_y_start,
+                                           int32_t in_x_start, float out_y_start, float out_x_start, float fh,
+                                           float fw, float scale_h, float scale_w, float last_y, float last_x,
+                                           int32_t Hd, int32_t Wd)
+{
+    float acc = 0.0f;
+    float out_y = out_y_start;
+    for (int32_t in_y = in_y_start; out_y < fh + 1.0f && in_y < Hd; in_y++) {
+        const float yc = __builtin_fmaxf(0.0f, __builtin_fminf(out_y, last_y));
+        const float y_lerp = 1.0f - __builtin_fabsf(yc - fh);
+        const TI* row = base + (int64_t)(in_y - y0) * pitch;
+        float out_x = out_x_start;
+        for (int32_t in_x = in_x_start; out_x < fw + 1.0f && in_x < Wd; in_x++) {
+            const float xc = __builtin_fmaxf(0.0f, __builtin_fminf(out_x, last_x));
+            const float x_lerp = 1.0f - __builtin_fabsf(xc - fw);
+            acc += ElemIO<TI>::load(row + (in_x - x0)) * y_lerp * x_lerp;
+            out_x += scale_w;
+        }
+        out_y += scale_h;
+    }
+    return acc;
+}
+
+constexpr int kTileCols = 128;
+constexpr int kTileGroups = kGradThreads / kTileCols;  // row groups of a workgroup
+
+template <typename TI, typename TO, bool HALF_PIXEL>
+__global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI* __restrict__ g, TO* __restrict__ y,
+                                                                        int64_t planes, int32_t Hs, int32_t Ws,
+                                                                        int32_t Hd, int32_t Wd, float scale_h,
+                                                                        float scale_w, float inv_scale_h,
+                                                                        float inv_scale_w, int32_t tile_rows,
+                                                                        int32_t cap_words)
+{
+    constexpr int EPW = 4 / (int)sizeof(TI);  // elements per 4-byte word
+    extern __shared__ uint32_t tile_words[];
+    __shared__ int32_t s_x1, s_y1;
+    const int tx = threadIdx.x % kTileCols, ty = threadIdx.x / kTileCols;
+    const int32_t W0 = blockIdx.x * kTileCols, H0 = blockIdx.y * tile_rows;
+    const float offset = HALF_PIXEL ? 0.5f : 0.0f;
+    const float last_y = (float)Hs - 1.0f, last_x = (float)Ws - 1.0f;
+    auto first_visit = [&](int32_t i, float inv_scale, int32_t len_dst) {
+        const float f = __builtin_ceilf(((float)i - 1.0f + offset) * inv_scale - offset);
+        // a start at or beyond the end visits nothing, whatever its exact value
+        return (f > 0.0f) ? ((f < (float)len_dst) ? (int32_t)f : len_dst) : 0;
+    };
+    auto end_visit = [&](int32_t i, int32_t start, float scale, int32_t len_dst) {
+        float out = ((float)start + offset) * scale - offset;
+        int32_t in = start;
+        for (; out < (float)i + 1.0f && in < len_dst; in++) {
+            out += scale;
+        }
+        return in;
+    };
+    const int32_t W = W0 + tx;
+    const bool col_ok = W < Ws;
+    const int32_t in_x_start = first_visit(col_ok ? W : W0, inv_scale_w, Wd);
+    const int32_t tile_x0 = first_visit(W0, inv_scale_w, Wd) / EPW * EPW;
+    const int32_t tile_y0 = first_visit(H0, inv_scale_h, Hd);
+    if (threadIdx.x == 0) {
+        s_x1 = 0;
+        s_y1 = 0;
+    }
+    __syncthreads();
+    if (col_ok) {
+        atomicMax(&s_x1, end_visit(W, in_x_start, scale_w, Wd));
+    }
+    if (tx == 0) {
+        for (int32_t H = H0 + ty; H < H0 + tile_rows && H < Hs; H += kTileGroups) {
+            atomicMax(&s_y1, end_visit(H, first_visit(H, inv_scale_h, Hd), scale_h, Hd));
+        }
+    }
+    __syncthreads();
+    const int32_t tile_x1 = (s_x1 + EPW - 1) / EPW * EPW;  // Wd is a multiple of EPW (host check): stays inside the row
+    const int32_t tile_y1 = s_y1;
+    const int32_t pitch_w = (tile_x1 > tile_x0) ? (tile_x1 - tile_x0) / EPW : 0;
+    const int32_t rows = (tile_y1 > tile_y0) ? tile_y1 - tile_y0 : 0;
+    const bool use_lds = (int64_t)rows * pitch_w <= cap_words;
+    const int32_t pitch = pitch_w * EPW;
+    const TI* tile = reinterpret_cast<const TI*>(tile_words);
+    const float out_x_start = ((float)in_x_start + offset) * scale_w - offset;
+    const float fw = (float)W;
+
+    for (int64_t pl = blockIdx.z; pl < planes; pl += gridDim.z) {
+        const TI* gp = g + pl * (int64_t)Hd * Wd;
+        if (use_lds) {
+            const int32_t total = rows * pitch_w;
+#pragma unroll 4
+            for (int32_t i = threadIdx.x; i < total; i += kGradThreads) {
+                const int32_t r = i / pitch_w;
+                const int32_t cw = i - r * pitch_w;
+                tile_words[i] = *reinterpret_cast<const uint32_t*>(gp + (int64_t)(tile_y0 + r) * Wd + tile_x0 + cw * EPW);
+            }
+            __syncthreads();
+        }
+        if (col_ok) {
+            for (int32_t H = H0 + ty; H < H0 + tile_rows && H < Hs; H += kTileGroups) {
+                const int32_t in_y_start = first_visit(H, inv_scale_h, Hd);
+                const float out_y_start = ((float)in_y_start + offset) * scale_h - offset;
+                // two call sites so that each is compiled for its own address space (LDS reads, global loads)
+                const float acc =
+                    use_lds ? visit_sum<TI>(tile, pitch, tile_y0, tile_x0, in_y_start, in_x_start, out_y_start,
+                                            out_x_start, (float)H, fw, scale_h, scale_w, last_y, last_x, Hd, Wd)
+                            : visit_sum<TI>(gp, Wd, 0, 0, in_y_start, in_x_start, out_y_start, out_x_start, (float)H,
+                                            fw, scale_h, scale_w, last_y, last_x, Hd, Wd);
+                ElemIO<TO>::store(y + (pl * Hs + H) * (int64_t)Ws + W, acc);
+            }
+        }
+        if (use_lds) {
+            __syncthreads();  // the tile is overwritten by the next plane
+        }
+    }
+}
+
+// Output rows per workgroup for the LDS variant (0: use the gather kernel).  The estimate only sizes the launch;
+// the kernel measures the rectangle itself.
+template <typename TI>
+int32_t lds_tile_rows(const ResizeGradArgs& a, int32_t cap_words)
+{
+    constexpr int EPW = 4 / (int)sizeof(TI);
+    if (a.channels_last || a.user_scales || a.Wd % EPW != 0 || reinterpret_cast<uintptr_t>(a.x) % 4 != 0) {
+        return 0;
+    }
+    const double per_col = (double)a.Wd / (double)a.Ws, per_row = (double)a.Hd / (double)a.Hs;
+    const double cols = kTileCols * per_col + 2.0 * per_col + 2.0 + EPW;
+    for (int32_t rows = 8; rows >= kTileGroups; rows /= 2) {
+        const double need = (rows * per_row + 2.0 * per_row + 2.0) * cols / EPW;
+        if (need <= (double)cap_words) {
+            return rows;
+        }
+    }
+    return 0;
+}
+
 template <typename TI, typename TO>
 hipError_t run(const ResizeGradArgs& a, hipStream_t stream)
 {
+    constexpr int32_t kCapWords = 8192;  // 32 KB of LDS per workgroup
+    const int32_t tile_rows = lds_tile_rows<TI>(a, kCapWords);
+    if (tile_rows > 0) {
+        const int64_t planes = a.N * a.C;
+        dim3 grid((unsigned)((a.Ws + kTileCols - 1) / kTileCols), (unsigned)((a.Hs + tile_rows - 1) / tile_rows),
+                  (unsigned)(planes < 65535 ? planes : 65535));
+        if (grid.y <= 65535) {
+            if (a.half_pixel) {
+                hipLaunchKernelGGL((resize_grad_lds_kernel<TI, TO, true>), grid, dim3(kGradThreads), kCapWords * 4,
+                                   stream, (const TI*)a.x, (TO*)a.y, planes, (int32_t)a.Hs, (int32_t)a.Ws,
+                                   (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h, a.scale_w, a.inv_scale_h, a.inv_scale_w,
+                                   tile_rows, kCapWords);
+            } else {
+                hipLaunchKernelGGL((resize_grad_lds_kernel<TI, TO, false>), grid, dim3(kGradThreads), kCapWords * 4,
+                                   stream, (const TI*)a.x, (TO*)a.y, planes, (int32_t)a.Hs, (int32_t)a.Ws,
+                                   (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h, a.scale_w, a.inv_scale_h, a.inv_scale_w,
+                                   tile_rows, kCapWords);
+            }
+            return hipGetLastError();
+        }
+    }
     const int64_t total = a.N * a.C * a.Hs * a.Ws;
     int64_t blocks = (total + kGradThreads - 1) / kGradThreads;
     if (blocks > 256 * 256) {
@@ -209,6 +373,17 @@ hipError_t run(const ResizeGradArgs& a, hipStream_t stream)
 }
 
 }  // namespace
+
+const char* resize_grad_variant(const ResizeGradArgs& a)
+{
+    if (a.user_scales) {
+        return "resize_grad_gather_scales";
+    }
+    constexpr int32_t kCapWords = 8192;
+    const int32_t rows = (a.elem_in == Elem::F32) ? lds_tile_rows<float>(a, kCapWords)
+                                                  : lds_tile_rows<uint16_t>(a, kCapWords);
+    return (rows > 0 && (a.Hs + rows - 1) / rows <= 65535) ? "resize_grad_lds" : "resize_grad_gather";
+}
 
 hipError_t launch_resize_grad(const ResizeGradArgs& a, hipStream_t stream)
 {

@@ -13,6 +13,7 @@
 #include <cstdlib>
 
 #include "kernels.hpp"
+#include "resize_band_lds_kernel.hpp"
 #include "resize_math.hpp"
 #include "sampler_math.hpp"
 
@@ -338,6 +339,117 @@ __global__ __launch_bounds__(kThreads) void resize_nearest_kernel(const T* __res
     }
 }
 
+// Nearest, NCHW, whole 16-byte output vectors, source rows staged in LDS.  Per element the gather-copy above issues a
+// two-byte global load, which binds it to the address rate of the memory pipeline rather than to memory.  Here a
+// workgroup owns (chunk of 256 output vectors, band of kNearestBand output rows): the source-row segments the chunk
+// reads -- one per distinct source row of the band, each a single 16-byte aligned byte range -- are copied into LDS
+// with the asynchronous global->LDS loads, and a lane assembles its vector from V two-byte LDS reads, once per
+// distinct source row.  Needs source rows that are whole 16-byte vectors (Ws % V == 0, aligned base).
+template <typename T>
+__global__ __launch_bounds__(kThreads) void resize_nearest_lds_kernel(const T* __restrict__ x, T* __restrict__ y,
+                                                                       int64_t outer, int32_t Hs, int32_t Ws,
+                                                                       int32_t Hd, int32_t Wd, float scale_h,
+                                                                       float scale_w, uint32_t slot_bytes,
+                                                                       int streaming)
+{
+    constexpr int V = 16 / (int)sizeof(T);
+    extern __shared__ uint4 nearest_smem[];
+    char* lds = reinterpret_cast<char*>(nearest_smem);
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane((uint32_t)tid >> 6);
+    const int32_t col_first = blockIdx.x * kThreads * V;
+    const int32_t col_last = ((col_first + kThreads * V < Wd) ? col_first + kThreads * V : Wd) - 1;
+    const int32_t s_lo = nearest_src(col_first, scale_w, Ws) / V * V;
+    const int32_t s_hi = nearest_src(col_last, scale_w, Ws);
+    const uint32_t seg_bytes = (uint32_t)((s_hi - s_lo) / V + 1) * 16u;
+    const bool use_lds = seg_bytes <= slot_bytes;  // uniform; the launch sizes the slots so that this holds
+    const int32_t e0 = col_first + tid * V;
+    const bool active = e0 < Wd;
+    int32_t src_col[V];
+#pragma unroll
+    for (int i = 0; i < V; i++) {
+        const int32_t c = (e0 + i < Wd) ? e0 + i : Wd - 1;
+        src_col[i] = nearest_src(c, scale_w, Ws);
+    }
+    const int64_t rows = outer * Hd;
+    for (int64_t r0 = (int64_t)blockIdx.y * kNearestBand; r0 < rows; r0 += (int64_t)gridDim.y * kNearestBand) {
+        int64_t src_row[kNearestBand];
+        int slot_of[kNearestBand];
+        int nslots = 0;
+        int64_t prev = -1;
+#pragma unroll
+        for (int j = 0; j < kNearestBand; j++) {
+            const int64_t r = r0 + j;
+            if (r < rows) {
+                const int64_t o = r / Hd;
+                const int32_t h = (int32_t)(r - o * Hd);
+                src_row[j] = o * Hs + nearest_src(h, scale_h, Hs);
+                if (src_row[j] != prev) {
+                    if (use_lds) {
+                        const char* src = reinterpret_cast<const char*>(x + src_row[j] * (int64_t)Ws + s_lo);
+                        for (uint32_t cb = wave * 1024u; cb < seg_bytes; cb += (kThreads / 64) * 1024u) {
+                            const uint32_t lane_off = cb + (uint32_t)lane * 16u;
+                            if (lane_off < seg_bytes) {
+                                __builtin_amdgcn_global_load_lds((rs_global_cptr_t)(src + lane_off),
+                                                                 (rs_lds_ptr_t)(lds + nslots * slot_bytes + cb), 16, 0,
+                                                                 0);
+                            }
+                        }
+                    }
+                    nslots++;
+                    prev = src_row[j];
+                }
+                slot_of[j] = nslots - 1;
+            } else {
+                src_row[j] = -1;
+                slot_of[j] = -1;
+            }
+        }
+        if (use_lds) {
+            __builtin_amdgcn_s_waitcnt(0);
+            __syncthreads();
+        }
+        if (active) {
+            int last = -1;
+            uint4 packed = make_uint4(0, 0, 0, 0);
+#pragma unroll
+            for (int j = 0; j < kNearestBand; j++) {
+                if (slot_of[j] < 0) {
+                    continue;
+                }
+                if (slot_of[j] != last) {
+                    T v[V];
+                    if (use_lds) {
+                        const T* seg = reinterpret_cast<const T*>(lds + slot_of[j] * slot_bytes);
+#pragma unroll
+                        for (int i = 0; i < V; i++) {
+                            v[i] = seg[src_col[i] - s_lo];
+                        }
+                    } else {
+                        const T* src = x + src_row[j] * (int64_t)Ws;
+#pragma unroll
+                        for (int i = 0; i < V; i++) {
+                            v[i] = src[src_col[i]];
+                        }
+                    }
+                    __builtin_memcpy(&packed, v, sizeof(packed));
+                    last = slot_of[j];
+                }
+                uint4* dst = reinterpret_cast<uint4*>(y + (r0 + j) * (int64_t)Wd + e0);
+                if (streaming) {
+                    store_streaming(dst, packed);
+                } else {
+                    *dst = packed;
+                }
+            }
+        }
+        if (use_lds) {
+            __syncthreads();  // the slots are refilled by the next band
+        }
+    }
+}
+
 // Broadcast of one source element per plane (mode Broadcast: 1x1 source; FirstPixel: 1x1 destination).
 // For NHWC the "plane" index is (n, c) with element stride C inside a batch.
 template <typename T>
@@ -426,6 +538,18 @@ hipError_t run_resize(const ResizeArgs& a, hipStream_t stream)
                        (int32_t)a.C, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h, a.scale_w, \
                        streaming)
         const int streaming = (out_elems * (int64_t)sizeof(T) >= (128ll << 20)) ? 1 : 0;
+        if (!nhwc && vec && a.Ws % V == 0 && !(getenv("OPSCV_NEAREST_VARIANT") && getenv("OPSCV_NEAREST_VARIANT")[0] == 'g')) {
+            // slot = the longest source segment a chunk of kThreads vectors can touch, with slack for the rounding of
+            // the per-column products; the kernel checks the real length and gathers from global memory otherwise
+            const double span = (double)(kThreads * V) * (double)a.scale_w * 1.001 + 2.0 + 2.0 * V;
+            const uint64_t slot = ((uint64_t)(span * sizeof(T)) + 15u) / 16u * 16u;
+            if (slot * kNearestBand <= 64u * 1024u) {
+                hipLaunchKernelGGL((resize_nearest_lds_kernel<T>), grid, dim3(kThreads), slot * kNearestBand, stream, x,
+                                   y, outer, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h,
+                                   a.scale_w, (uint32_t)slot, streaming);
+                return hipGetLastError();
+            }
+        }
         if (nhwc) {
             if (vec) {
                 OPSCV_NEAREST(true, true);
@@ -520,7 +644,17 @@ const char* resize_variant(const ResizeArgs& a)
         case ResizeMode::Copy: return "copy";
         case ResizeMode::Broadcast: return "broadcast";
         case ResizeMode::FirstPixel: return "first_pixel";
-        case ResizeMode::Nearest: return a.channels_last ? "nearest_nhwc" : "nearest_nchw";
+        case ResizeMode::Nearest: {
+            if (a.channels_last) {
+                return "nearest_nhwc";
+            }
+            // rows of whole 16-byte vectors on both sides and slots that fit: the LDS-staged kernel (see run_resize)
+            const int64_t V = 16 / elem_size(a.elem);
+            const double span = 256.0 * (double)V * (double)a.scale_w * 1.001 + 2.0 + 2.0 * (double)V;
+            const uint64_t slot = ((uint64_t)(span * elem_size(a.elem)) + 15u) / 16u * 16u;
+            const bool lds = a.Wd % V == 0 && a.Ws % V == 0 && slot * kNearestBand <= 64u * 1024u;
+            return lds ? "nearest_nchw_lds" : "nearest_nchw";
+        }
         default: break;
     }
     if (a.channels_last) {

@@ -320,8 +320,8 @@ def test_upsample_backward_status_codes(aclnn, desc):
     # accepted, the user-scale template runs
     for dt in (aclnn.ACL_FLOAT, aclnn.ACL_FLOAT16, aclnn.ACL_BF16):
         assert _ub(aclnn, desc, dt=dt) == (0, 0, "resize_grad_gather_scales")
-    assert _ub(aclnn, desc, sh=0.0, sw=0.0)[2] == "resize_grad_gather"
-    assert _ub(aclnn, desc, align=True)[2] == "resize_grad_gather"
+    assert _ub(aclnn, desc, sh=0.0, sw=0.0)[2] == "resize_grad_lds"
+    assert _ub(aclnn, desc, align=True)[2] == "resize_grad_lds"
     # 003-012: unsupported dtypes
     for dt in (aclnn.ACL_DOUBLE, aclnn.ACL_INT32):
         assert _ub(aclnn, desc, dt=dt)[0] == INV

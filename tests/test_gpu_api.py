@@ -254,7 +254,11 @@ def test_upsample_backward(oracle, device, aclnn, dtype, channels_last):
     cases = [((2, 3, 5, 7), (10, 14), False, 0.0, 0.0), ((1, 4, 8, 8), (3, 5), True, 0.0, 0.0),
              ((2, 2, 16, 16), (33, 47), False, 0.0, 0.0), ((1, 5, 1, 5), (4, 10), True, 0.0, 0.0),
              ((1, 2, 4, 6), (10, 10), False, 2.5, 1.7), ((2, 1, 8, 8), (4, 3), False, 0.6, 0.45),
-             ((1, 3, 6, 6), (6, 6), False, 0.0, 0.0), ((1, 8, 56, 56), (112, 112), False, 2.0, 2.0)]
+             ((1, 3, 6, 6), (6, 6), False, 0.0, 0.0), ((1, 8, 56, 56), (112, 112), False, 2.0, 2.0),
+             # several column tiles and ragged row tiles of the LDS variant; an odd incoming width (16-bit types
+             # then take the gather kernel); a x20 upscale whose tile exceeds the LDS capacity; a strong downscale
+             ((1, 2, 37, 300), (75, 610), True, 0.0, 0.0), ((2, 1, 19, 131), (40, 263), False, 0.0, 0.0),
+             ((1, 1, 9, 130), (180, 2600), False, 0.0, 0.0), ((1, 2, 90, 260), (11, 40), True, 0.0, 0.0)]
     for in_shape, (Ho, Wo), align, sh, sw in cases:
         N, C, H, W = in_shape
         g = I.cast_np(rng.standard_normal((N, C, Ho, Wo)).astype(np.float32), dtype)
@@ -428,3 +432,24 @@ def test_grid_sampler2d_backward_mask_views_and_torch(oracle, device, aclnn):
         torch.cuda.synchronize()
         assert (dx - xa.grad).abs().max().item() <= 1e-4
         assert ((dg - ga.grad).abs() > 1e-3).float().mean().item() <= 0.02
+
+
+@pytest.mark.parametrize("dtype", I.DTYPES)
+def test_resize_nearest_wide_rows(oracle, device, aclnn, dtype):
+    """nearest NCHW with whole-vector rows (the LDS-staged kernel): several column chunks, bands that straddle
+    planes, non-integer factors, down-scaling, and a factor whose source segment exceeds the LDS slots"""
+    import torch
+    rng = np.random.default_rng(320)
+    cases = [((2, 3, 5, 1040), (13, 4160)), ((1, 2, 9, 2560), (7, 1600)), ((3, 1, 4, 64), (11, 8)),
+             ((1, 1, 3, 8192), (5, 256)), ((1, 4, 7, 528), (7, 2072)), ((1, 2, 6, 24), (12, 48))]
+    for shape, (Ho, Wo) in cases:
+        N, C, H, W = shape
+        x = I.cast_np(rng.standard_normal(shape).astype(np.float32), dtype)
+        ref = oracle.resize_nearest(x, (Ho, Wo), dtype=I.oracle_code(dtype))
+        out = torch.empty((N, C, Ho, Wo), dtype=I.to_torch(x[:1, :1, :1, :1], dtype, device).dtype, device=device)
+        # scales such that trunc(in * scale) == out and the kernel's scale is in/out
+        y = aclnn.resize(I.to_torch(x, dtype, device), (1.0, 1.0, Ho / H, Wo / W), "nearest", out=out)
+        torch.cuda.synchronize()
+        got = I.from_torch(y, dtype)
+        view = np.uint32 if dtype == "fp32" else np.uint16
+        assert np.array_equal(got.view(view), ref.view(view)), (shape, Ho, Wo, dtype)
