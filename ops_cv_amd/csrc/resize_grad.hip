@@ -205,6 +205,30 @@ __device__ __forceinline__ float visit_sum(const TI* base, int32_t pitch, int32_
     return acc;
 }
 
+// The same sum with the column part of the loop taken out: a lane keeps the weights of the (at most KX) columns it
+// visits -- computed once, by the same repeated additions -- and a row costs one LDS read, two products and an add
+// per column.  Column k of a lane with fewer than k + 1 visits re-reads its last column and leaves the sum alone.
+template <typename TI, int KX>
+__device__ __forceinline__ float visit_sum_fixed(const TI* tile_xy, int32_t pitch, int32_t y0, int32_t in_y_start,
+                                                 int32_t nx, const float (&xl)[KX], const int32_t (&xo)[KX],
+                                                 float out_y_start, float fh, float scale_h, float last_y, int32_t Hd)
+{
+    float acc = 0.0f;
+    float out_y = out_y_start;
+    for (int32_t in_y = in_y_start; out_y < fh + 1.0f && in_y < Hd; in_y++) {
+        const float yc = __builtin_fmaxf(0.0f, __builtin_fminf(out_y, last_y));
+        const float y_lerp = 1.0f - __builtin_fabsf(yc - fh);
+        const TI* row = tile_xy + (in_y - y0) * pitch;
+#pragma unroll
+        for (int k = 0; k < KX; k++) {
+            const float t = ElemIO<TI>::load(row + xo[k]) * y_lerp * xl[k];
+            acc = (k < nx) ? acc + t : acc;
+        }
+        out_y += scale_h;
+    }
+    return acc;
+}
+
 constexpr int kTileCols = 128;
 constexpr int kTileGroups = kGradThreads / kTileCols;  // row groups of a workgroup
 
@@ -218,7 +242,7 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
 {
     constexpr int EPW = 4 / (int)sizeof(TI);  // elements per 4-byte word
     extern __shared__ uint32_t tile_words[];
-    __shared__ int32_t s_x1, s_y1;
+    __shared__ int32_t s_x1, s_y1, s_nx;
     const int tx = threadIdx.x % kTileCols, ty = threadIdx.x / kTileCols;
     const int32_t W0 = blockIdx.x * kTileCols, H0 = blockIdx.y * tile_rows;
     const float offset = HALF_PIXEL ? 0.5f : 0.0f;
@@ -244,10 +268,15 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
     if (threadIdx.x == 0) {
         s_x1 = 0;
         s_y1 = 0;
+        s_nx = 0;
     }
     __syncthreads();
+    int32_t nx = 0;
     if (col_ok) {
-        atomicMax(&s_x1, end_visit(W, in_x_start, scale_w, Wd));
+        const int32_t x_end = end_visit(W, in_x_start, scale_w, Wd);
+        nx = x_end - in_x_start;
+        atomicMax(&s_x1, x_end);
+        atomicMax(&s_nx, nx);
     }
     if (tx == 0) {
         for (int32_t H = H0 + ty; H < H0 + tile_rows && H < Hs; H += kTileGroups) {
@@ -265,6 +294,23 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
     const float out_x_start = ((float)in_x_start + offset) * scale_w - offset;
     const float fw = (float)W;
 
+    // column weights of this lane, for the variants with a fixed column count
+    constexpr int KMAX = 8;
+    float xl[KMAX];
+    int32_t xo[KMAX];
+    {
+        float out_x = out_x_start;
+#pragma unroll
+        for (int k = 0; k < KMAX; k++) {
+            const float xc = __builtin_fmaxf(0.0f, __builtin_fminf(out_x, last_x));
+            xl[k] = 1.0f - __builtin_fabsf(xc - fw);
+            xo[k] = (k < nx) ? k : ((nx > 0) ? nx - 1 : 0);
+            out_x += scale_w;
+        }
+    }
+    const int32_t nx_max = s_nx;
+    const int32_t x_base = (nx > 0) ? in_x_start - tile_x0 : 0;
+
     for (int64_t pl = blockIdx.z; pl < planes; pl += gridDim.z) {
         const TI* gp = g + pl * (int64_t)Hd * Wd;
         if (use_lds) {
@@ -281,12 +327,28 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
             for (int32_t H = H0 + ty; H < H0 + tile_rows && H < Hs; H += kTileGroups) {
                 const int32_t in_y_start = first_visit(H, inv_scale_h, Hd);
                 const float out_y_start = ((float)in_y_start + offset) * scale_h - offset;
-                // two call sites so that each is compiled for its own address space (LDS reads, global loads)
-                const float acc =
-                    use_lds ? visit_sum<TI>(tile, pitch, tile_y0, tile_x0, in_y_start, in_x_start, out_y_start,
-                                            out_x_start, (float)H, fw, scale_h, scale_w, last_y, last_x, Hd, Wd)
-                            : visit_sum<TI>(gp, Wd, 0, 0, in_y_start, in_x_start, out_y_start, out_x_start, (float)H,
-                                            fw, scale_h, scale_w, last_y, last_x, Hd, Wd);
+                float acc;
+                // separate call sites so that each is compiled for its own address space (LDS reads, global loads)
+                if (use_lds && nx_max <= 4) {
+                    const float(&xl4)[4] = reinterpret_cast<const float(&)[4]>(xl);
+                    const int32_t(&xo4)[4] = reinterpret_cast<const int32_t(&)[4]>(xo);
+                    acc = visit_sum_fixed<TI, 4>(tile + x_base, pitch, tile_y0, in_y_start, nx, xl4, xo4, out_y_start,
+                                                 (float)H, scale_h, last_y, Hd);
+                } else if (use_lds && nx_max <= 6) {
+                    const float(&xl6)[6] = reinterpret_cast<const float(&)[6]>(xl);
+                    const int32_t(&xo6)[6] = reinterpret_cast<const int32_t(&)[6]>(xo);
+                    acc = visit_sum_fixed<TI, 6>(tile + x_base, pitch, tile_y0, in_y_start, nx, xl6, xo6, out_y_start,
+                                                 (float)H, scale_h, last_y, Hd);
+                } else if (use_lds && nx_max <= 8) {
+                    acc = visit_sum_fixed<TI, 8>(tile + x_base, pitch, tile_y0, in_y_start, nx, xl, xo, out_y_start,
+                                                 (float)H, scale_h, last_y, Hd);
+                } else if (use_lds) {
+                    acc = visit_sum<TI>(tile, pitch, tile_y0, tile_x0, in_y_start, in_x_start, out_y_start,
+                                        out_x_start, (float)H, fw, scale_h, scale_w, last_y, last_x, Hd, Wd);
+                } else {
+                    acc = visit_sum<TI>(gp, Wd, 0, 0, in_y_start, in_x_start, out_y_start, out_x_start, (float)H, fw,
+                                        scale_h, scale_w, last_y, last_x, Hd, Wd);
+                }
                 ElemIO<TO>::store(y + (pl * Hs + H) * (int64_t)Ws + W, acc);
             }
         }
