@@ -31,6 +31,10 @@ MEASURED_TRAFFIC = {
     ("C4", "nchw_band_lds"): 1415.4e6,       # profiles/resize_band_lds_C4_fp16_4k_upscale.md
     ("C2", "nchw_flat_lds"): 33.08e6,        # profiles/resize_flat_lds_C2_fp32_56_to_112.md
     ("C5", "lds_ring_p32784_1x4"): 176.4e6,  # profiles/gs2d_lds_ring_C5_bf16_random_gather.md
+    ("V1", "gs3d_bilinear"): 38.65e6,        # profiles/gs3d_V1_fp16_22x4x16x64x64.md
+    ("G3", "gs2d_grad_ordered"): 250.7e6,    # profiles/gs2d_grad_G3_fp16_n16_c256.md (both kernels of a step)
+    ("B4", "resize_grad_lds"): 1954.4e6,     # profiles/resize_grad_lds_B4_fp16_4k.md
+    ("R4", "nearest_nchw_lds"): 1327.3e6,    # profiles/resize_nearest_lds_R4_fp16_4k.md
 }
 
 # name -> description of the workloads (shapes as in the baseline configuration list)
@@ -571,7 +575,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="C3", help="headline workload (C1..C5)")
+    ap.add_argument("--workload", default="C3", help="headline workload: C1..C5, or one of the neighbouring entry points V1 (3-D sampler), G3 "
+                         "(sampler backward), B4 (resize backward), R4 (nearest resize)")
     ap.add_argument("--only", action="store_true", help="skip the other workloads and the CPU baseline")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -603,8 +608,19 @@ def main():
     head = args.workload
     if head in GS_WORKLOADS:
         r = bench_gs(head, args.steps, args.warmup)
-    else:
+    elif head in UP_WORKLOADS:
         r = bench_up(head, args.steps, args.warmup)
+    elif head == "V1":
+        r = bench_gs3d(args.steps, args.warmup)
+    elif head == "G3":
+        r = bench_gs_backward(args.steps, args.warmup)
+    elif head == "B4":
+        r = bench_resize_like("backward", args.steps, args.warmup)
+    elif head == "R4":
+        r = bench_resize_like("nearest", args.steps, args.warmup)
+    else:
+        print("bench.py: unknown workload %s" % head, file=sys.stderr)
+        sys.exit(2)
     t = r["timed"]
     line = {
         "metric": "output samples/s, grid_sampler2d fp16 N16 C256 (achieved HBM GB/s in roofline)" if head == "C3"
