@@ -9,11 +9,13 @@
 // contributions one by one in point order, each add rounding to the tensor's element type
 // (grid_sampler2_d_grad_simt_det.h:75-101).  The sum that reaches one element of the gradient is therefore a fixed
 // sequence: its contributions ordered by (chunk, tap, point).  Adds to different elements commute, so only that
-// per-element order has to be kept.  Here a workgroup owns one (batch item, channel, band of the plane): the band
-// lives in LDS, the workgroup walks the chunks in order, and inside a chunk the pending contributions to one
-// element are applied in rounds -- each round an LDS max-reduction elects, per element, the pending contribution
-// that comes first in (tap, point) order, and only the elected ones are added.  The result does not depend on
-// scheduling and equals the sequential order above bit for bit.
+// per-element order has to be kept.  Here a workgroup owns one (batch item, group of channels, band of the plane):
+// the band of every channel of the group lives in LDS, the workgroup walks the chunks in order and, inside a chunk,
+// the taps in order.  The contributions of one tap that land on the same element are applied in rounds: an LDS
+// max-reduction elects, per element, the waiting contribution of the lowest point; the elected ones are added (to
+// every channel's plane) and retire.  Distinct points of a chunk rarely share a corner texel, so a tap mostly needs
+// a single round with all lanes at work.  The result does not depend on scheduling and equals the sequential order
+// above bit for bit.
 //
 // Gradient of the grid.  One lane per grid point walks the channels in order, as the reference does
 // (grid_sampler2_d_grad_simt_det.h:103-196,279-343); no atomics are involved.
@@ -27,7 +29,7 @@ namespace opscv {
 namespace {
 
 constexpr int kThreads = 256;         // also the chunk length of the accumulation order
-constexpr uint32_t kKeyBits = 12;     // 16 taps x 256 points
+constexpr uint32_t kKeyBits = 8;      // 256 points of a chunk
 constexpr uint32_t kEpochMax = (1u << (32 - kKeyBits)) - 1;
 
 struct GradParams {
@@ -36,7 +38,9 @@ struct GradParams {
     int32_t band_px;  // plane elements per workgroup (dx kernel)
 };
 
-template <typename T, int INTERP>
+// CB channels of one batch item per workgroup: the grid points, their taps and the election of a round are the
+// same for every channel, only the values added differ, so that work is shared by the CB planes held in LDS.
+template <typename T, int INTERP, int CB>
 __global__ __launch_bounds__(kThreads) void gs2d_grad_input_kernel(const T* __restrict__ gout,
                                                                     const T* __restrict__ grid, T* __restrict__ dx,
                                                                     GradParams p)
@@ -44,40 +48,65 @@ __global__ __launch_bounds__(kThreads) void gs2d_grad_input_kernel(const T* __re
     using Taps = GradTaps<T, INTERP>;
     constexpr int NT = Taps::NT;
     extern __shared__ uint32_t smem_u32[];
-    float* plane = reinterpret_cast<float*>(smem_u32);
-    uint32_t* owner = smem_u32 + p.band_px;
+    __shared__ uint32_t s_flag[2];
+    uint32_t* owner = smem_u32;
+    T* planes = reinterpret_cast<T*>(smem_u32 + p.band_px);  // [CB][band_px], values already in the element type
 
     const int t = threadIdx.x;
     const int32_t plane_px = p.H * p.W;
     const int32_t b0 = blockIdx.x * p.band_px;
     const int32_t b1 = (b0 + p.band_px < plane_px) ? b0 + p.band_px : plane_px;
-    const int32_t c = blockIdx.y;
+    const int32_t c0 = blockIdx.y * CB;
+    const int32_t nc = (c0 + CB <= p.C) ? CB : p.C - c0;
     const int64_t n = blockIdx.z;
     for (int32_t i = t; i < b1 - b0; i += kThreads) {
-        plane[i] = 0.0f;
         owner[i] = 0u;
+#pragma unroll
+        for (int cb = 0; cb < CB; cb++) {
+            ElemIO<T>::store(planes + cb * p.band_px + i, 0.0f);
+        }
     }
+    if (t == 0) {
+        s_flag[0] = s_flag[1] = 0u;
+    }
+    __syncthreads();
     const int32_t points = p.Ho * p.Wo;
     const T* g_n = grid + n * (int64_t)points * 2;
-    const T* go_nc = gout + (n * p.C + c) * (int64_t)points;
+    const T* go_n = gout + (n * p.C + c0) * (int64_t)points;
     uint32_t epoch = 1;
-    // the grid point and incoming gradient of the next chunk are requested before the rounds of this one
-    float gx_next = 0.0f, gy_next = 0.0f, go_next = 0.0f;
+    int fl = 0;
+    // the grid point and incoming gradients of the next chunk are requested before the rounds of this one
+    float gx_next = 0.0f, gy_next = 0.0f, go_next[CB];
+#pragma unroll
+    for (int cb = 0; cb < CB; cb++) {
+        go_next[cb] = 0.0f;
+    }
+    auto request = [&](int32_t pt) {
+        gx_next = ElemIO<T>::load(g_n + 2 * (int64_t)pt);
+        gy_next = ElemIO<T>::load(g_n + 2 * (int64_t)pt + 1);
+#pragma unroll
+        for (int cb = 0; cb < CB; cb++) {
+            if (cb < nc) {
+                go_next[cb] = ElemIO<T>::load(go_n + (int64_t)cb * points + pt);
+            }
+        }
+    };
     if (t < points) {
-        gx_next = ElemIO<T>::load(g_n + 2 * (int64_t)t);
-        gy_next = ElemIO<T>::load(g_n + 2 * (int64_t)t + 1);
-        go_next = ElemIO<T>::load(go_nc + t);
+        request(t);
     }
     for (int32_t base = 0; base < points; base += kThreads) {
         const int32_t pt = base + t;
-        const float gx = gx_next, gy = gy_next, go = go_next;
+        const float gx = gx_next, gy = gy_next;
+        float go[CB];
+#pragma unroll
+        for (int cb = 0; cb < CB; cb++) {
+            go[cb] = go_next[cb];
+        }
         if (pt + kThreads < points) {
-            gx_next = ElemIO<T>::load(g_n + 2 * (int64_t)(pt + kThreads));
-            gy_next = ElemIO<T>::load(g_n + 2 * (int64_t)(pt + kThreads) + 1);
-            go_next = ElemIO<T>::load(go_nc + pt + kThreads);
+            request(pt + kThreads);
         }
         int32_t off[NT];
-        float val[NT];
+        float wt[NT];
         uint32_t pend = 0;
         if (pt < points) {
             Taps tp;
@@ -85,43 +114,86 @@ __global__ __launch_bounds__(kThreads) void gs2d_grad_input_kernel(const T* __re
 #pragma unroll
             for (int k = 0; k < NT; k++) {
                 off[k] = tp.off[k] - b0;
-                // the contribution is rounded to the element type before it is added
-                val[k] = rt<T>(INTERP == 1 ? go : (INTERP == 0 ? tp.w[k] * go : go * tp.w[k]));
+                wt[k] = tp.w[k];
                 if (tp.off[k] >= b0 && tp.off[k] < b1) {
                     pend |= 1u << k;
                 }
             }
         }
-        while (__syncthreads_or((int)pend) != 0) {
+        // Tap after tap, as the order demands.  Contributions of one tap rarely collide (two grid points of a chunk
+        // with the same corner texel), so a tap usually takes one round in which every lane is busy.  A flag word
+        // holds the number of the last round for which a contribution of tap k is still waiting; round numbers only
+        // grow, so a stale value never matches.
+        if (epoch > kEpochMax - 2u * NT * kThreads) {  // uniform: start the election tags over
+            __syncthreads();
+            for (int32_t i = t; i < b1 - b0; i += kThreads) {
+                owner[i] = 0u;
+            }
+            if (t == 0) {
+                s_flag[0] = s_flag[1] = 0u;
+            }
+            epoch = 1;
+            __syncthreads();
+        }
 #pragma unroll
-            for (int k = 0; k < NT; k++) {
-                if (pend & (1u << k)) {
-                    atomicMax(&owner[off[k]], (epoch << kKeyBits) | (4095u - (uint32_t)(k * kThreads + t)));
-                }
+        for (int k = 0; k < NT; k++) {
+            bool waiting = (pend & (1u << k)) != 0;
+            fl ^= 1;  // the other flag than the tap before: its last readers are behind this tap's first barrier
+            if (waiting) {
+                s_flag[fl] = epoch;
             }
             __syncthreads();
-#pragma unroll
-            for (int k = 0; k < NT; k++) {
-                if ((pend & (1u << k)) &&
-                    owner[off[k]] == ((epoch << kKeyBits) | (4095u - (uint32_t)(k * kThreads + t)))) {
-                    plane[off[k]] = rt<T>(plane[off[k]] + val[k]);
-                    pend &= ~(1u << k);
+            while (s_flag[fl] == epoch) {
+                const uint32_t key = (epoch << kKeyBits) | (uint32_t)(kThreads - 1 - t);
+                if (waiting) {
+                    atomicMax(&owner[off[k]], key);
                 }
+                __syncthreads();
+                if (waiting) {
+                    if (owner[off[k]] == key) {
+                        // the contribution is rounded to the element type before it is added, and so is the sum
+                        T* e = planes + off[k];
+                        if (nc == CB) {
+                            // all planes read before any is written: the channels' updates overlap
+                            float cur[CB];
+#pragma unroll
+                            for (int cb = 0; cb < CB; cb++) {
+                                cur[cb] = ElemIO<T>::load(e + cb * p.band_px);
+                            }
+#pragma unroll
+                            for (int cb = 0; cb < CB; cb++) {
+                                const float val =
+                                    rt<T>(INTERP == 1 ? go[cb] : (INTERP == 0 ? wt[k] * go[cb] : go[cb] * wt[k]));
+                                ElemIO<T>::store(e + cb * p.band_px, cur[cb] + val);
+                            }
+                        } else {
+#pragma unroll
+                            for (int cb = 0; cb < CB; cb++) {
+                                if (cb < nc) {
+                                    const float val =
+                                        rt<T>(INTERP == 1 ? go[cb] : (INTERP == 0 ? wt[k] * go[cb] : go[cb] * wt[k]));
+                                    ElemIO<T>::store(e + cb * p.band_px, ElemIO<T>::load(e + cb * p.band_px) + val);
+                                }
+                            }
+                        }
+                        waiting = false;
+                    } else {
+                        s_flag[fl] = epoch + 1;  // somebody is left for the next round
+                    }
+                }
+                __syncthreads();
+                epoch++;
             }
             epoch++;
-            if (epoch == kEpochMax) {  // uniform: start the election tags over
-                __syncthreads();
-                for (int32_t i = t; i < b1 - b0; i += kThreads) {
-                    owner[i] = 0u;
-                }
-                epoch = 1;
-            }
         }
     }
-    // the loop's last barrier has made every add visible
-    T* dx_nc = dx + (n * p.C + c) * (int64_t)plane_px + b0;
-    for (int32_t i = t; i < b1 - b0; i += kThreads) {
-        ElemIO<T>::store(dx_nc + i, plane[i]);
+    __syncthreads();
+    for (int cb = 0; cb < nc; cb++) {
+        T* dx_nc = dx + (n * p.C + c0 + cb) * (int64_t)plane_px + b0;
+        const T* pl = planes + cb * p.band_px;
+        for (int32_t i = t; i < b1 - b0; i += kThreads) {
+            dx_nc[i] = pl[i];
+        }
     }
 }
 
@@ -237,17 +309,38 @@ hipError_t launch_interp(const GridSamplerGradArgs& a, hipStream_t stream)
     p.pad = a.pad;
     p.align = a.align;
     const int64_t plane_px = a.Hin * a.Win;
-    // 8 bytes of LDS per plane element (value + election tag); bands of at most 4096 elements keep a workgroup
-    // at 32 KB so that several share a compute unit
+    // bands of at most 4096 plane elements: election tags (4 bytes each) plus the planes of a channel group
     p.band_px = (int32_t)(plane_px < 4096 ? plane_px : 4096);
     if (a.dx != nullptr) {
         const int64_t bands = (plane_px + p.band_px - 1) / p.band_px;
-        if (bands > INT32_MAX || a.C > 65535 || a.N > 65535) {
+        // 8 bytes of planes per band element: 4 channels of a 16-bit type, 2 of fp32 (48 KB of LDS with the tags, three
+        // workgroups per compute unit); fewer channels than that run one per workgroup
+        constexpr int CBMAX = 8 / (int)sizeof(T);
+        const bool grouped = a.C >= CBMAX;
+        const int64_t cgroups = grouped ? (a.C + CBMAX - 1) / CBMAX : a.C;
+        if (bands > INT32_MAX || cgroups > 65535 || a.N > 65535) {
             return hipErrorInvalidValue;
         }
-        hipLaunchKernelGGL((gs2d_grad_input_kernel<T, INTERP>), dim3((unsigned)bands, (unsigned)a.C, (unsigned)a.N),
-                           dim3(kThreads), (size_t)p.band_px * 8, stream, (const T*)a.gout, (const T*)a.grid,
-                           (T*)a.dx, p);
+        const dim3 grid((unsigned)bands, (unsigned)cgroups, (unsigned)a.N);
+        if (grouped) {
+            static bool attr_set = false;  // more than the default 64 KB of dynamic LDS
+            if (!attr_set) {
+                const hipError_t ea = hipFuncSetAttribute(
+                    reinterpret_cast<const void*>(gs2d_grad_input_kernel<T, INTERP, CBMAX>),
+                    hipFuncAttributeMaxDynamicSharedMemorySize, 4096 * (4 + CBMAX * (int)sizeof(T)));
+                if (ea != hipSuccess) {
+                    return ea;
+                }
+                attr_set = true;
+            }
+            hipLaunchKernelGGL((gs2d_grad_input_kernel<T, INTERP, CBMAX>), grid, dim3(kThreads),
+                               (size_t)p.band_px * (4 + CBMAX * sizeof(T)), stream, (const T*)a.gout,
+                               (const T*)a.grid, (T*)a.dx, p);
+        } else {
+            hipLaunchKernelGGL((gs2d_grad_input_kernel<T, INTERP, 1>), grid, dim3(kThreads),
+                               (size_t)p.band_px * (4 + sizeof(T)), stream, (const T*)a.gout, (const T*)a.grid,
+                               (T*)a.dx, p);
+        }
         const hipError_t e = hipGetLastError();
         if (e != hipSuccess) {
             return e;
