@@ -128,7 +128,7 @@ struct GridSamplerGradArgs {
     void* dgrid = nullptr;       // (N,Hout,Wout,2)
 };
 
-enum class ResizeMode : int { Bilinear = 0, Copy = 1, Broadcast = 2, FirstPixel = 3, Nearest = 4 };
+enum class ResizeMode : int { Bilinear = 0, Copy = 1, Broadcast = 2, FirstPixel = 3, Nearest = 4, PointCopy = 5 };
 
 struct ResizeArgs {
     Elem elem = Elem::F32;
@@ -136,6 +136,7 @@ struct ResizeArgs {
     int half_pixel = 1;
     int channels_last = 0;
     float scale_h = 1.0f, scale_w = 1.0f;
+    int64_t point_step_h = 1, point_step_w = 1;  // PointCopy: integer source stride per destination pixel
     int64_t N = 0, C = 0, Hs = 0, Ws = 0, Hd = 0, Wd = 0;
     const void* x = nullptr;
     void* y = nullptr;

@@ -450,6 +450,33 @@ __global__ __launch_bounds__(kThreads) void resize_nearest_lds_kernel(const T* _
     }
 }
 
+// Point copy (channels-last, whole shrink factors whose sampling points are source pixels): every destination pixel
+// is the copy of one source pixel.  Source index as in
+// image/resize_bilinear_v2/op_kernel/arch35/resize_bilinear_v2_point_copy.h:117-124, clamped to the last pixel.
+// U is the unit copied per lane: a 16-byte vector when a pixel's channels are whole vectors, else one element.
+template <typename U>
+__global__ __launch_bounds__(kThreads) void resize_point_copy_kernel(const U* __restrict__ x, U* __restrict__ y,
+                                                                      int64_t total, int32_t units, int32_t Hs,
+                                                                      int32_t Ws, int32_t Hd, int32_t Wd,
+                                                                      int64_t step_h, int64_t step_w, int half_pixel)
+{
+    const int64_t stride = (int64_t)gridDim.x * kThreads;
+    for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += stride) {
+        int64_t r = i;
+        const int32_t u = (int32_t)(r % units);
+        r /= units;
+        const int64_t w = r % Wd;
+        r /= Wd;
+        const int64_t h = r % Hd;
+        const int64_t n = r / Hd;
+        int64_t hs = half_pixel ? ((2 * h + 1) * step_h - 1) / 2 : h * step_h;
+        int64_t ws = half_pixel ? ((2 * w + 1) * step_w - 1) / 2 : w * step_w;
+        hs = (hs < Hs - 1) ? hs : Hs - 1;
+        ws = (ws < Ws - 1) ? ws : Ws - 1;
+        y[i] = x[((n * Hs + hs) * Ws + ws) * units + u];
+    }
+}
+
 // Broadcast of one source element per plane (mode Broadcast: 1x1 source; FirstPixel: 1x1 destination).
 // For NHWC the "plane" index is (n, c) with element stride C inside a batch.
 template <typename T>
@@ -511,6 +538,27 @@ hipError_t run_resize(const ResizeArgs& a, hipStream_t stream)
     const int64_t out_elems = a.N * a.C * a.Hd * a.Wd;
     if (a.mode == ResizeMode::Copy) {
         return hipMemcpyAsync(y, x, (size_t)out_elems * sizeof(T), hipMemcpyDeviceToDevice, stream);
+    }
+    if (a.mode == ResizeMode::PointCopy) {
+        constexpr int V = 16 / (int)sizeof(T);
+        const bool vec = a.C % V == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0;
+        const int64_t units = vec ? a.C / V : a.C;
+        const int64_t total = a.N * a.Hd * a.Wd * units;
+        int64_t blocks = (total + kThreads - 1) / kThreads;
+        if (blocks > 256 * 256) {
+            blocks = 256 * 256;
+        }
+        if (vec) {
+            hipLaunchKernelGGL((resize_point_copy_kernel<uint4>), dim3((unsigned)blocks), dim3(kThreads), 0, stream,
+                               reinterpret_cast<const uint4*>(x), reinterpret_cast<uint4*>(y), total, (int32_t)units,
+                               (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.point_step_h,
+                               a.point_step_w, a.half_pixel);
+        } else {
+            hipLaunchKernelGGL((resize_point_copy_kernel<T>), dim3((unsigned)blocks), dim3(kThreads), 0, stream, x, y,
+                               total, (int32_t)units, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd,
+                               a.point_step_h, a.point_step_w, a.half_pixel);
+        }
+        return hipGetLastError();
     }
     if (a.mode == ResizeMode::Broadcast || a.mode == ResizeMode::FirstPixel) {
         int64_t blocks = (out_elems + kThreads - 1) / kThreads;
@@ -644,6 +692,7 @@ const char* resize_variant(const ResizeArgs& a)
         case ResizeMode::Copy: return "copy";
         case ResizeMode::Broadcast: return "broadcast";
         case ResizeMode::FirstPixel: return "first_pixel";
+        case ResizeMode::PointCopy: return "point_copy";
         case ResizeMode::Nearest: {
             if (a.channels_last) {
                 return "nearest_nhwc";

@@ -1,5 +1,8 @@
 #include "resize_plan.hpp"
 
+#include <cfloat>
+#include <cmath>
+
 namespace opscv {
 
 float resize_axis_scale(int64_t len_src, int64_t len_dst, bool align_corners, float user_scale)
@@ -16,6 +19,33 @@ float resize_axis_scale(int64_t len_src, int64_t len_dst, bool align_corners, fl
     return (float)len_src / (float)len_dst;
 }
 
+// resize_bilinear_v2_tiling_arch35.cpp:254-303 (MatchPointCopyCondition, IsMatchPointCopy): channels-last data
+// with runs of at least 128 bytes, shrunk by whole factors whose sampling points fall exactly on source pixels
+// (always with align_corners; with half-pixel centres only for odd factors).  Every destination pixel is then a
+// copy of one source pixel, and the reference copies instead of interpolating.
+static bool point_copy_steps(const ResizeArgs& a, bool align_corners, int64_t* step_h, int64_t* step_w)
+{
+    if (!a.channels_last || a.C * elem_size(a.elem) < 128) {
+        return false;
+    }
+    if (a.scale_h < 1.0f || a.scale_w < 1.0f) {
+        return false;
+    }
+    const int64_t fh = (int64_t)(a.scale_h + FLT_EPSILON), fw = (int64_t)(a.scale_w + FLT_EPSILON);
+    if (std::fabs(a.scale_h - (float)fh) >= FLT_EPSILON || std::fabs(a.scale_w - (float)fw) >= FLT_EPSILON) {
+        return false;
+    }
+    *step_h = fh;
+    *step_w = fw;
+    if (align_corners) {
+        return true;
+    }
+    if (!a.half_pixel) {
+        return true;
+    }
+    return fh % 2 == 1 && fw % 2 == 1;
+}
+
 void plan_resize(ResizeArgs* a, bool align_corners, float user_scale_h, float user_scale_w)
 {
     a->half_pixel = align_corners ? 0 : 1;
@@ -30,6 +60,8 @@ void plan_resize(ResizeArgs* a, bool align_corners, float user_scale_h, float us
     a->mode = ResizeMode::Bilinear;
     if (a->Hs == a->Hd && a->Ws == a->Wd) {
         a->mode = ResizeMode::Copy;
+    } else if (point_copy_steps(*a, align_corners, &a->point_step_h, &a->point_step_w)) {
+        a->mode = ResizeMode::PointCopy;
     } else if (one_src && (run_bytes >= kMinRunBytes || align_corners)) {
         a->mode = ResizeMode::Broadcast;
     } else if (one_dst && align_corners) {

@@ -21,6 +21,10 @@
  *   oracle_upsample_bilinear2d   : known answers for image/upsample_bilinear2d/examples/
  *                                  test_aclnn_upsample_bilinear2d.cpp:83-94, kernel-UT shapes (1,1,1,4)->(2,16),
  *                                  (3,16), committed torch interpolate fixtures, live torch CPU comparison
+ *   oracle_resize_point_copy     : equals a strided numpy slice x[:, off::f, off::f, :] (off = 0 or (f-1)/2), equals the
+ *                                  interpolating oracle on finite data (all weights there are exactly 0 or 1), and
+ *                                  differs from it exactly where a sampled value is infinite (the formula multiplies
+ *                                  it by its zero weight too)
  *   oracle_resize_nearest        : integer-factor upscales equal element repetition, committed and live
  *                                  torch interpolate(mode="nearest") comparison (bit-exact: a pure copy)
  *   oracle_upsample_bilinear2d_backward : adjointness with the forward oracle (<forward(x), g> = <x, backward(g)>),
@@ -801,6 +805,51 @@ int oracle_upsample_bilinear2d_backward(const void* grads, void* y, int dtype_in
         }
     }
     return 0;
+}
+
+/* ------------------------------------------------------------------------------------------
+ * Point-copy template of the bilinear resize (channels-last only)
+ *   selection: image/resize_bilinear_v2/op_host/arch35/resize_bilinear_v2_tiling_arch35.cpp:254-303
+ *   indices  : image/resize_bilinear_v2/op_kernel/arch35/resize_bilinear_v2_point_copy.h:117-124
+ * Returns 1 and fills y (N,Hd,Wd,C) when the template applies, 0 when the interpolating templates apply.
+ * ---------------------------------------------------------------------------------------- */
+int oracle_resize_point_copy(const void* x, void* y, int dtype, int64_t N, int64_t C, int64_t Hs, int64_t Ws,
+                             int64_t Hd, int64_t Wd, int align_corners, double scales_h, double scales_w)
+{
+    const int64_t esz = (dtype == ORACLE_F32) ? 4 : 2;
+    if (Hs == Hd && Ws == Wd) {
+        return 0; /* the all-copy template comes first */
+    }
+    if (C * esz < 128) {
+        return 0;
+    }
+    const float scale_h = oracle_resize_scale(Hs, Hd, align_corners, (float)scales_h);
+    const float scale_w = oracle_resize_scale(Ws, Wd, align_corners, (float)scales_w);
+    if (scale_h < 1.0 || scale_w < 1.0) {
+        return 0;
+    }
+    const int64_t fh = (int64_t)(scale_h + 1.1920928955078125e-7f);
+    const int64_t fw = (int64_t)(scale_w + 1.1920928955078125e-7f);
+    if (fabsf(scale_h - (float)fh) >= 1.1920928955078125e-7f || fabsf(scale_w - (float)fw) >= 1.1920928955078125e-7f) {
+        return 0;
+    }
+    const int half_pixel = !align_corners;
+    if (half_pixel && !(fh % 2 == 1 && fw % 2 == 1)) {
+        return 0;
+    }
+    for (int64_t n = 0; n < N; n++) {
+        for (int64_t h = 0; h < Hd; h++) {
+            int64_t hs = half_pixel ? ((2 * h + 1) * fh - 1) / 2 : h * fh;
+            hs = hs < Hs - 1 ? hs : Hs - 1;
+            for (int64_t w = 0; w < Wd; w++) {
+                int64_t ws = half_pixel ? ((2 * w + 1) * fw - 1) / 2 : w * fw;
+                ws = ws < Ws - 1 ? ws : Ws - 1;
+                memcpy((char*)y + ((n * Hd + h) * Wd + w) * C * esz, (const char*)x + ((n * Hs + hs) * Ws + ws) * C * esz,
+                       (size_t)(C * esz));
+            }
+        }
+    }
+    return 1;
 }
 
 /* ------------------------------------------------------------------------------------------

@@ -117,6 +117,14 @@ int oracle_upsample_axis_taps(int64_t len_src, int64_t len_dst, int align_corner
                               int32_t* i1, float* lambda);
 
 /*
+ * Point-copy template of the bilinear resize, channels-last (N,H,W,C) tensors
+ * (image/resize_bilinear_v2/op_host/arch35/resize_bilinear_v2_tiling_arch35.cpp:254-303).  Returns 1 and fills y when
+ * the template applies, else 0.
+ */
+int oracle_resize_point_copy(const void* x, void* y, int dtype, int64_t N, int64_t C, int64_t Hs, int64_t Ws,
+                             int64_t Hd, int64_t Wd, int align_corners, double scales_h, double scales_w);
+
+/*
  * Volumetric grid sampler, forward (image/grid_sample/op_kernel/arch35/grid_sampler_3d_bilinear_smit.h:146-191).
  * x (N,C,Din,Hin,Win), grid (N,Dout,Hout,Wout,3) ordered x,y,z, y (N,C,Dout,Hout,Wout); interp 0 bilinear,
  * 1 nearest (round half to even, image/grid_sample/op_kernel/grid_sampler_3d_nearest.h:569-571).

@@ -98,6 +98,9 @@ def lib():
     L.oracle_gs3d_clip.argtypes = [f32, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32]
     L.oracle_grid_sampler2d_backward.restype = ctypes.c_int
     L.oracle_grid_sampler2d_backward.argtypes = [vp] * 5 + [ctypes.c_int] + [i64] * 6 + [ctypes.c_int] * 3
+    L.oracle_resize_point_copy.restype = ctypes.c_int
+    L.oracle_resize_point_copy.argtypes = [vp, vp, ctypes.c_int] + [i64] * 6 + [ctypes.c_int, ctypes.c_double,
+                                                                            ctypes.c_double]
     L.oracle_max_threads.restype = ctypes.c_int
     L.oracle_max_threads.argtypes = []
     _lib = L
@@ -192,6 +195,17 @@ def upsample_bilinear2d_backward(grads, in_hw, align=False, channels_last=False,
     if rc != 0:
         raise ValueError("oracle_upsample_bilinear2d_backward rc=%d" % rc)
     return y
+
+
+def resize_point_copy(x_nhwc, out_hw, align=False, scales_h=0.0, scales_w=0.0, dtype=None):
+    """x (N,H,W,C) -> y (N,Ho,Wo,C) when the reference's point-copy template applies, else None"""
+    x = np.ascontiguousarray(x_nhwc)
+    code = _code_of(x) if dtype is None else dtype
+    N, Hs, Ws, C = x.shape
+    y = np.empty((N, out_hw[0], out_hw[1], C), dtype=x.dtype)
+    rc = lib().oracle_resize_point_copy(_ptr(x), _ptr(y), code, N, C, Hs, Ws, out_hw[0], out_hw[1], int(bool(align)),
+                                        float(scales_h), float(scales_w))
+    return y if rc == 1 else None
 
 
 def grid_sampler2d_backward(gout, x, grid, interp=0, pad=0, align=False, dtype=None, want=(True, True)):

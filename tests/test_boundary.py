@@ -481,3 +481,17 @@ def test_grid_sampler2d_backward_status_codes(aclnn, desc):
     # a strided input view needs workspace
     st, ws, _ = _gsb(aclnn, desc, strides=(80, 80, 16, 2), storage=(80,))
     assert st == 0 and ws >= 40 * 4
+
+
+def test_resize_template_selection_point_copy(aclnn, desc):
+    """resize_bilinear_v2_tiling_arch35.cpp:254-303: channels-last runs of 128 bytes and more, shrunk by whole factors
+    (odd ones with half-pixel centres), are copied instead of interpolated"""
+    nhwc = aclnn.ACL_FORMAT_NHWC
+    kw = dict(mode=b"bilinear", fmt=nhwc)
+    assert _rs(aclnn, desc, inp=(1, 9, 15, 32), out=(1, 3, 5, 32), scales=(1, 1 / 3, 1 / 3, 1), **kw)[2] == "point_copy"
+    # factor 2 with half-pixel centres samples between pixels; 31 channels of fp32 are under 128 bytes
+    assert _rs(aclnn, desc, inp=(1, 8, 8, 32), out=(1, 4, 4, 32), scales=(1, 0.5, 0.5, 1), **kw)[2] != "point_copy"
+    assert _rs(aclnn, desc, inp=(1, 9, 15, 31), out=(1, 3, 5, 31), scales=(1, 1 / 3, 1 / 3, 1), **kw)[2] != "point_copy"
+    # NCHW never takes the template
+    assert _rs(aclnn, desc, inp=(1, 32, 9, 15), out=(1, 32, 3, 5), scales=(1, 1, 1 / 3, 1 / 3), mode=b"bilinear")[2] != \
+        "point_copy"

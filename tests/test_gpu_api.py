@@ -453,3 +453,30 @@ def test_resize_nearest_wide_rows(oracle, device, aclnn, dtype):
         got = I.from_torch(y, dtype)
         view = np.uint32 if dtype == "fp32" else np.uint16
         assert np.array_equal(got.view(view), ref.view(view)), (shape, Ho, Wo, dtype)
+
+
+@pytest.mark.parametrize("dtype", I.DTYPES)
+def test_resize_point_copy(oracle, device, aclnn, dtype):
+    """channels-last shrinks by whole factors take the reference's point-copy template: bit-exact copies, also of
+    infinities and NaNs, through aclnnUpsampleBilinear2d and aclnnResize; vector and scalar channel counts"""
+    torch = _torch()
+    rng = np.random.default_rng(330)
+    C_vec, C_odd = 128, 130
+    for (N, Hs, Ws, C, Ho, Wo, align) in [(2, 12, 15, C_vec, 4, 5, False), (1, 11, 13, C_vec, 6, 5, True),
+                                          (1, 9, 9, C_odd, 3, 3, False), (1, 5, 7, C_vec, 1, 7, False)]:
+        x32 = rng.standard_normal((N, Hs, Ws, C)).astype(np.float32)
+        x32[0, 1, 1, :4] = [np.inf, -np.inf, np.nan, -0.0]
+        x = I.cast_np(x32, dtype)
+        ref = oracle.resize_point_copy(x, (Ho, Wo), align=align, dtype=I.oracle_code(dtype))
+        assert ref is not None
+        xt = I.to_torch(x, dtype, device)
+        hs = [aclnn.tensor_handle(xt, aclnn.ACL_FORMAT_NHWC)]
+        y = aclnn.upsample_bilinear2d(xt, (Ho, Wo), align, channels_last=True)
+        torch.cuda.synchronize()
+        aclnn.destroy_tensor(hs[0])
+        got = I.from_torch(y, dtype)
+        assert np.array_equal(_bits(got, dtype), _bits(ref, dtype)), (N, Hs, Ws, C, Ho, Wo, align, dtype)
+        if not align:
+            y2 = aclnn.resize(xt, (1.0, Ho / Hs, Wo / Ws, 1.0), "bilinear", channels_last=True)
+            torch.cuda.synchronize()
+            assert np.array_equal(_bits(I.from_torch(y2, dtype), dtype), _bits(ref, dtype))

@@ -667,3 +667,34 @@ def test_grid_sampler2d_backward_order_is_sequential_in_element_type(oracle):
     # bilinear at the exact centre: only the north-west tap has weight 1; the other taps add +0 in between
     dxb, _ = oracle.grid_sampler2d_backward(go, x, g, 0, 1, False)
     assert dxb.ravel()[0] == acc
+
+
+def test_resize_point_copy_oracle(oracle):
+    """the point-copy template: a strided slice of the source, equal to the interpolating oracle on finite data
+    and different from it exactly where a sampled value is infinite"""
+    rng = np.random.default_rng(51)
+    C = 64  # 256 bytes of fp32 per pixel: above the 128-byte threshold
+    x = rng.standard_normal((2, 12, 15, C)).astype(np.float32)
+    # half-pixel centres (align_corners=False): odd factors only, sampling point (f - 1) / 2
+    y = oracle.resize_point_copy(x, (4, 5), align=False)
+    assert y is not None and np.array_equal(y, x[:, 1::3, 1::3, :])
+    assert oracle.resize_point_copy(x, (6, 5), align=False) is None        # factor 2 along H
+    assert oracle.resize_point_copy(x, (4, 4), align=False) is None        # 15 / 4 is not whole
+    # align_corners: (in - 1) / (out - 1) whole, sampling point 0
+    y = oracle.resize_point_copy(x[:, :11, :13], (6, 5), align=True)       # factors 2 and 3
+    assert y is not None and np.array_equal(y, x[:, 0:11:2, 0:13:3, :])
+    # runs under 128 bytes, equal sizes and upscales do not take the template
+    assert oracle.resize_point_copy(x[..., :16], (4, 5), align=False) is None
+    assert oracle.resize_point_copy(x, (12, 15), align=False) is None
+    assert oracle.resize_point_copy(x, (36, 45), align=False) is None
+    # finite data: the interpolating formula gives the same numbers
+    y = oracle.resize_point_copy(x, (4, 5), align=False)
+    gen = oracle.upsample_bilinear2d(np.ascontiguousarray(x.transpose(0, 3, 1, 2)), (4, 5), False).transpose(0, 2, 3, 1)
+    assert np.array_equal(y, gen)
+    # an infinite sample: the copy hands it over, the interpolation multiplies it by its zero weights as well
+    # (both taps of an axis coincide when the coordinate is whole: 1 * inf + 0 * inf)
+    xi = x.copy()
+    xi[0, 1, 1, 0] = np.inf
+    y = oracle.resize_point_copy(xi, (4, 5), align=False)
+    gen = oracle.upsample_bilinear2d(np.ascontiguousarray(xi.transpose(0, 3, 1, 2)), (4, 5), False).transpose(0, 2, 3, 1)
+    assert y[0, 0, 0, 0] == np.inf and np.isnan(gen[0, 0, 0, 0])
