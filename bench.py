@@ -334,8 +334,9 @@ def _parity(got, ref, dtype, **extra):
     return out
 
 
-def bench_gs3d(steps, warmup, sets=4):
-    """Volumetric sampler on the shape the reference singles out (22 x 4 x 16 x 64 x 64, fp16, an affine warp)."""
+def bench_gs3d(steps, warmup, sets=4, channels_last=False):
+    """Volumetric sampler on the shape the reference singles out (22 x 4 x 16 x 64 x 64, fp16, an affine warp);
+    with channels_last the same data as dense NDHWC tensors."""
     import numpy as np
     import torch
     import inputs as I
@@ -358,11 +359,16 @@ def bench_gs3d(steps, warmup, sets=4):
         g = I.cast_np((g + rng.normal(0, 0.01, g.shape)).astype(np.float32), dtype)
         if s == 0:
             x0, g0 = x, g
-        xs.append(I.to_torch(x, dtype, dev))
+        if channels_last:
+            xs.append(I.to_torch(np.ascontiguousarray(x.transpose(0, 2, 3, 4, 1)), dtype, dev))
+            ys.append(torch.empty((N, D, H, W, C), dtype=xs[-1].dtype, device=dev))
+        else:
+            xs.append(I.to_torch(x, dtype, dev))
+            ys.append(torch.empty((N, C, D, H, W), dtype=xs[-1].dtype, device=dev))
         gs.append(I.to_torch(g, dtype, dev))
-        ys.append(torch.empty((N, C, D, H, W), dtype=xs[-1].dtype, device=dev))
-        for lst, t in zip(hs, (xs[-1], gs[-1], ys[-1])):
-            lst.append(aclnn.tensor_handle(t, aclnn.ACL_FORMAT_NCDHW))
+        fmt = aclnn.ACL_FORMAT_NDHWC if channels_last else aclnn.ACL_FORMAT_NCDHW
+        for lst, t, f in zip(hs, (xs[-1], gs[-1], ys[-1]), (fmt, aclnn.ACL_FORMAT_NCDHW, fmt)):
+            lst.append(aclnn.tensor_handle(t, f))
     arr = lambda h: (ctypes.c_void_p * len(h))(*h)
     ax_, ag, ay = arr(hs[0]), arr(hs[1]), arr(hs[2])
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
@@ -380,14 +386,17 @@ def bench_gs3d(steps, warmup, sets=4):
     aclnn.destroy_executor(ex)
     t = _finish(L, run, xs, ys, steps, warmup, stream)
     ref = oracle_lib.grid_sampler3d(x0, g0, 0, 0, False, dtype=I.oracle_code(dtype))
-    parity = _parity(I.from_torch(ys[0], dtype), ref, dtype)
+    got = I.from_torch(ys[0], dtype)
+    if channels_last:
+        got = np.ascontiguousarray(got.transpose(0, 4, 1, 2, 3))
+    parity = _parity(got, ref, dtype)
     for lst in hs:
         for h in lst:
             aclnn.destroy_tensor(h)
     samples = N * C * D * H * W
     alg = (N * C * D * H * W * 2 + N * D * H * W * 3) * esize(dtype)
     return dict(workload="V1 grid_sampler3d fp16 x(22,4,16,64,64) grid(22,16,64,64,3) bilinear zeros "
-                         "align_corners=False", samples=samples, alg_bytes=alg, timed=t, variant=variant,
+                         "align_corners=False" + (" NDHWC tensors" if channels_last else ""), samples=samples, alg_bytes=alg, timed=t, variant=variant,
                 parity=parity, sets=sets, default_modes=True)
 
 
@@ -612,6 +621,8 @@ def main():
         r = bench_up(head, args.steps, args.warmup)
     elif head == "V1":
         r = bench_gs3d(args.steps, args.warmup)
+    elif head == "V1cl":
+        r = bench_gs3d(args.steps, args.warmup, channels_last=True)
     elif head == "G3":
         r = bench_gs_backward(args.steps, args.warmup)
     elif head == "B4":
@@ -669,6 +680,8 @@ def main():
                 others[name] = summary_of(bench_up(name, k, max(2, args.warmup // 4)))
         # the entry points either side of the path, on shapes of the same scale
         others["V1_grid_sampler3d"] = summary_of(bench_gs3d(max(10, args.steps // 2), args.warmup))
+        others["V1_grid_sampler3d_ndhwc"] = summary_of(bench_gs3d(max(10, args.steps // 2), args.warmup,
+                                                                  channels_last=True))
         k4 = max(5, args.steps // 4)
         others["G3_grid_sampler2d_backward"] = summary_of(bench_gs_backward(k4, max(2, args.warmup // 4)))
         others["B4_upsample_backward"] = summary_of(bench_resize_like("backward", k4, max(2, args.warmup // 4)))

@@ -108,6 +108,7 @@ struct GridSampler3DArgs {
     int interp = 0;  // 0 bilinear (trilinear blend of eight corners), 1 nearest
     int pad = 0;
     int align = 0;
+    int channels_last = 0;  // 1: x is (N,Din,Hin,Win,C) and y is (N,Dout,Hout,Wout,C) in memory
     int64_t N = 0, C = 0, Din = 0, Hin = 0, Win = 0, Dout = 0, Hout = 0, Wout = 0;
     const void* x = nullptr;
     const void* grid = nullptr;

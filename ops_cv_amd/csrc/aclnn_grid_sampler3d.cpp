@@ -177,10 +177,17 @@ aclnnStatus aclnnGridSampler3DGetWorkspaceSize(const aclTensor* input, const acl
     // The kernel works on (N,C,D,H,W) operands.  A channels-last tensor is that operand seen through a permuted
     // view, which is packed (and the result scattered) like any other non-contiguous view; this takes the place of
     // the reference's transposes around its kernel (aclnn_grid_sampler3d.cpp:247-274).
+    // Dense NDHWC tensors on both sides are sampled in place by the channels-last kernel.
     static const int kToNcdhw[5] = {0, 4, 1, 2, 3};
-    ex->in0 = plan_view(ex.get(), input, esz, false, ndhwc ? kToNcdhw : nullptr);
+    if (ndhwc && input->contiguous() && out->contiguous()) {
+        a.channels_last = 1;
+        ex->in0 = plan_view(ex.get(), input, esz, false);
+        ex->out0 = plan_view(ex.get(), out, esz, true);
+    } else {
+        ex->in0 = plan_view(ex.get(), input, esz, false, ndhwc ? kToNcdhw : nullptr);
+        ex->out0 = plan_view(ex.get(), out, esz, true, ndhwc ? kToNcdhw : nullptr);
+    }
     ex->in1 = plan_view(ex.get(), grid, esz, false);
-    ex->out0 = plan_view(ex.get(), out, esz, true, ndhwc ? kToNcdhw : nullptr);
 
     *workspaceSize = ex->workspace_bytes;
     *executor = ex.release();

@@ -181,9 +181,141 @@ __global__ __launch_bounds__(kThreads) void gs3d_kernel(const T* __restrict__ x,
     }
 }
 
+// Channels-last (NDHWC) variant: the C values of a voxel are contiguous, so a corner is one load of up to 16 bytes
+// instead of C scattered two- or four-byte loads.  A lane owns one unit of UE consecutive channels of one output
+// point (consecutive lanes own consecutive units, so loads and stores of neighbouring lanes are contiguous); the
+// lanes of a point compute its coordinates redundantly.  Arithmetic per element as in gs3d_kernel.
+template <typename T, int INTERP, int PAD, bool ALIGN, int UE>
+__global__ __launch_bounds__(kThreads) void gs3d_ndhwc_kernel(const T* __restrict__ x, const T* __restrict__ grid,
+                                                               T* __restrict__ y, Gs3dParams p, int32_t units)
+{
+    typedef T Unit __attribute__((ext_vector_type(UE)));
+    const int64_t idx = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (idx >= p.points * units) {
+        return;
+    }
+    const int64_t pt = idx / units;
+    const int32_t u = (int32_t)(idx - pt * units);
+    const int64_t n = pt / p.out_vol;
+    const T* g = grid + pt * 3;
+    const float gw = ElemIO<T>::load(g);
+    const float gh = ElemIO<T>::load(g + 1);
+    const float gd = ElemIO<T>::load(g + 2);
+    const float pd = clip3<PAD, ALIGN>(unnormalize3<ALIGN>(gd, p.Din), p.Din);
+    const float pw = clip3<PAD, ALIGN>(unnormalize3<ALIGN>(gw, p.Win), p.Win);
+    const float ph = clip3<PAD, ALIGN>(unnormalize3<ALIGN>(gh, p.Hin), p.Hin);
+    const int64_t in_vol = (int64_t)p.Din * p.Hin * p.Win;
+    const Unit* xu = reinterpret_cast<const Unit*>(x + n * in_vol * p.C) + u;  // voxel v, unit u: xu[v * units]
+    Unit* yu = reinterpret_cast<Unit*>(y) + idx;
+    Unit zero;
+#pragma unroll
+    for (int e = 0; e < UE; e++) {
+        T z;
+        ElemIO<T>::store(&z, 0.0f);
+        zero[e] = z;
+    }
+    if (INTERP == 1) {
+        const int32_t id = float_to_i32(__builtin_rintf(pd));
+        const int32_t ih = float_to_i32(__builtin_rintf(ph));
+        const int32_t iw = float_to_i32(__builtin_rintf(pw));
+        const bool in = id >= 0 && id < p.Din && ih >= 0 && ih < p.Hin && iw >= 0 && iw < p.Win;
+        *yu = in ? xu[(((int64_t)id * p.Hin + ih) * p.Win + iw) * units] : zero;
+        return;
+    }
+    const float fd = __builtin_floorf(pd), fh = __builtin_floorf(ph), fw = __builtin_floorf(pw);
+    const float dd = pd - fd, dh = ph - fh, dw = pw - fw;
+    const int32_t d0 = float_to_i32(fd), d1 = float_to_i32(fd + 1.0f);
+    const int32_t h0 = float_to_i32(fh), h1 = float_to_i32(fh + 1.0f);
+    const int32_t w0 = float_to_i32(fw), w1 = float_to_i32(fw + 1.0f);
+    const bool vd0 = d0 >= 0 && d0 < p.Din, vd1 = d1 >= 0 && d1 < p.Din;
+    const bool vh0 = h0 >= 0 && h0 < p.Hin, vh1 = h1 >= 0 && h1 < p.Hin;
+    const bool vw0 = w0 >= 0 && w0 < p.Win, vw1 = w1 >= 0 && w1 < p.Win;
+    float wt[8];
+    wt[0] = (1.0f - dw) * (1.0f - dh) * (1.0f - dd);
+    wt[1] = dw * (1.0f - dh) * (1.0f - dd);
+    wt[2] = (1.0f - dw) * dh * (1.0f - dd);
+    wt[3] = dw * dh * (1.0f - dd);
+    wt[4] = (1.0f - dw) * (1.0f - dh) * dd;
+    wt[5] = dw * (1.0f - dh) * dd;
+    wt[6] = (1.0f - dw) * dh * dd;
+    wt[7] = dw * dh * dd;
+    Unit v[8];
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        const bool ok = ((k & 4) ? vd1 : vd0) && ((k & 2) ? vh1 : vh0) && ((k & 1) ? vw1 : vw0);
+        const int32_t d = (k & 4) ? d1 : d0, h = (k & 2) ? h1 : h0, w = (k & 1) ? w1 : w0;
+        // an always valid address for the corners outside the volume, their values replaced by zeros
+        const int64_t vox = ok ? ((int64_t)d * p.Hin + h) * p.Win + w : 0;
+        const Unit raw = xu[vox * units];
+        v[k] = ok ? raw : zero;
+    }
+    Unit out;
+#pragma unroll
+    for (int e = 0; e < UE; e++) {
+        T t0 = v[0][e];
+        float acc = ElemIO<T>::load(&t0) * wt[0];
+#pragma unroll
+        for (int k = 1; k < 8; k++) {
+            T tk = v[k][e];
+            acc += ElemIO<T>::load(&tk) * wt[k];
+        }
+        T o;
+        ElemIO<T>::store(&o, acc);
+        out[e] = o;
+    }
+    *yu = out;
+}
+
+template <typename T, int INTERP, int PAD, bool ALIGN>
+hipError_t launch_ndhwc(const GridSampler3DArgs& a, hipStream_t stream)
+{
+    Gs3dParams p;
+    p.C = (int32_t)a.C;
+    p.Din = (int32_t)a.Din;
+    p.Hin = (int32_t)a.Hin;
+    p.Win = (int32_t)a.Win;
+    p.out_vol = a.Dout * a.Hout * a.Wout;
+    p.points = a.N * p.out_vol;
+    p.chan_chunk = 0;
+    // the widest unit (16, 8, 4 bytes or one element) that divides a voxel's channels and keeps every access aligned
+    const int64_t vox_bytes = a.C * (int64_t)sizeof(T);
+    const uintptr_t both = reinterpret_cast<uintptr_t>(a.x) | reinterpret_cast<uintptr_t>(a.y);
+    int ub = (int)sizeof(T);
+    for (int cand = 16; cand > (int)sizeof(T); cand /= 2) {
+        if (vox_bytes % cand == 0 && both % cand == 0) {
+            ub = cand;
+            break;
+        }
+    }
+    const int64_t units = vox_bytes / ub;
+    const int64_t blocks = (p.points * units + kThreads - 1) / kThreads;
+    if (blocks > INT32_MAX || units > INT32_MAX) {
+        return hipErrorInvalidValue;
+    }
+#define OPSCV_GS3D_CL(UE_)                                                                                          \
+    hipLaunchKernelGGL((gs3d_ndhwc_kernel<T, INTERP, PAD, ALIGN, UE_>), dim3((unsigned)blocks), dim3(kThreads), 0,  \
+                       stream, (const T*)a.x, (const T*)a.grid, (T*)a.y, p, (int32_t)units)
+    switch (ub / (int)sizeof(T)) {
+        case 1: OPSCV_GS3D_CL(1); break;
+        case 2: OPSCV_GS3D_CL(2); break;
+        case 4: OPSCV_GS3D_CL(4); break;
+        case 8:
+            if constexpr (sizeof(T) == 2) {
+                OPSCV_GS3D_CL(8);
+            }
+            break;
+        default: return hipErrorInvalidValue;
+    }
+#undef OPSCV_GS3D_CL
+    return hipGetLastError();
+}
+
 template <typename T, int INTERP, int PAD, bool ALIGN>
 hipError_t launch_one(const GridSampler3DArgs& a, hipStream_t stream)
 {
+    if (a.channels_last) {
+        return launch_ndhwc<T, INTERP, PAD, ALIGN>(a, stream);
+    }
     Gs3dParams p;
     p.C = (int32_t)a.C;
     p.Din = (int32_t)a.Din;

@@ -412,8 +412,12 @@ def test_grid_sampler3d_status_codes(aclnn, desc):
     # ascend910B2_NDHWC_case_01: channels-last extents (N,D,H,W,C); the operand is a permuted view, so a channel
     # count above one needs workspace for the input and for the output
     assert _gs3(aclnn, desc, inp=(2, 1, 3, 3, 1), out=(2, 1, 2, 2, 1), fmt=aclnn.ACL_FORMAT_NDHWC)[:2] == (0, 0)
-    st, ws, _ = _gs3(aclnn, desc, inp=(2, 1, 3, 3, 4), out=(2, 1, 2, 2, 4), fmt=aclnn.ACL_FORMAT_NDHWC)
-    assert st == 0 and ws >= (2 * 9 * 4 + 2 * 4 * 4) * 4
+    # dense channels-last tensors are sampled in place; a strided one is packed as a permuted view
+    assert _gs3(aclnn, desc, inp=(2, 1, 3, 3, 4), out=(2, 1, 2, 2, 4), fmt=aclnn.ACL_FORMAT_NDHWC) == \
+        (0, 0, "gs3d_ndhwc_bilinear")
+    st, ws, variant = _gs3(aclnn, desc, inp=(2, 1, 3, 3, 4), out=(2, 1, 2, 2, 4), fmt=aclnn.ACL_FORMAT_NDHWC,
+                           strides=(72, 72, 24, 8, 1), storage=(144,))
+    assert st == 0 and variant == "gs3d_bilinear" and ws >= 2 * 9 * 4 * 4
     # a strided NCDHW view is packed too
     st, ws, _ = _gs3(aclnn, desc, strides=(18, 18, 18, 6, 2), storage=(36,))
     assert st == 0 and ws >= 2 * 9 * 4

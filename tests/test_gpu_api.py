@@ -480,3 +480,33 @@ def test_resize_point_copy(oracle, device, aclnn, dtype):
             y2 = aclnn.resize(xt, (1.0, Ho / Hs, Wo / Ws, 1.0), "bilinear", channels_last=True)
             torch.cuda.synchronize()
             assert np.array_equal(_bits(I.from_torch(y2, dtype), dtype), _bits(ref, dtype))
+
+
+@pytest.mark.parametrize("dtype", I.DTYPES)
+@pytest.mark.parametrize("interp", [0, 1])
+def test_grid_sampler3d_channels_last(oracle, device, aclnn, dtype, interp):
+    """dense NDHWC tensors are sampled in place: every vector width of the channel run (16, 8, 4 bytes, one element),
+    all paddings, special grid values; bit-exact against the oracle on the transposed data"""
+    torch = _torch()
+    rng = np.random.default_rng(520 + interp)
+    for (N, C, D, H, W, Do, Ho, Wo) in [(2, 4, 5, 6, 7, 4, 5, 9), (1, 8, 3, 4, 5, 2, 3, 33), (1, 1, 4, 4, 4, 3, 3, 3),
+                                        (2, 3, 2, 9, 5, 3, 7, 5), (1, 20, 3, 3, 3, 2, 2, 17), (1, 64, 2, 2, 2, 1, 3, 5)]:
+        x = I.cast_np(rng.standard_normal((N, C, D, H, W)).astype(np.float32), dtype)
+        g32 = rng.uniform(-1.8, 1.8, (N, Do, Ho, Wo, 3)).astype(np.float32)
+        flat = g32.reshape(-1, 3)
+        special = np.array([np.nan, np.inf, -np.inf, 1e30, 1.0, -1.0, 0.0], np.float32)
+        for j in range(min(len(special), flat.shape[0])):
+            flat[j, j % 3] = special[j]
+        g = I.cast_np(g32, dtype)
+        xl = I.to_torch(np.ascontiguousarray(x.transpose(0, 2, 3, 4, 1)), dtype, device)
+        gt = I.to_torch(g, dtype, device)
+        for pad in range(3):
+            for align in (False, True):
+                ref = oracle.grid_sampler3d(x, g, interp, pad, align, dtype=I.oracle_code(dtype))
+                y = aclnn.grid_sampler3d(xl, gt, interp, pad, align, channels_last=True)
+                torch.cuda.synchronize()
+                got = I.from_torch(y, dtype).transpose(0, 4, 1, 2, 3)
+                rn = np.isnan(I.as_f32(ref, dtype))
+                assert np.array_equal(np.isnan(I.as_f32(got, dtype)), rn), (N, C, D, H, W, pad, align)
+                assert np.array_equal(np.where(rn, 0, _bits(np.ascontiguousarray(got), dtype)),
+                                      np.where(rn, 0, _bits(ref, dtype))), (N, C, D, H, W, Do, Ho, Wo, pad, align)
