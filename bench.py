@@ -573,7 +573,16 @@ def cpu_baseline_gs(x0, g0, w, budget_s=12.0):
     t1 = time.perf_counter()
     oracle_lib.grid_sampler2d(x0, g0, w["interp"], w["pad"], w["align"], dtype=I.oracle_code(w["dtype"]), threads=1)
     one = time.perf_counter() - t1
-    return {"value": samples * reps / el, "unit": "samples/s", "cores": threads, "kind": "port",
+    model = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for ln in f:
+                if ln.startswith("model name"):
+                    model = ln.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return {"value": samples * reps / el, "unit": "samples/s", "cores": threads, "kind": "port", "cpu_model": model,
             "sample": "full workload (%d output samples) x %d repetitions, OpenMP static over output pixels" % (
                 samples, reps),
             "single_thread_samples_per_s": samples / one}
@@ -652,6 +661,14 @@ def main():
                    "parity_vs_oracle": r["parity"]},
         "roofline": roofline_of(r),
     }
+    try:
+        props = torch.cuda.get_device_properties(0)
+        line["device"] = {"name": props.name, "compute_units": props.multi_processor_count,
+                          "memory_GiB": round(props.total_memory / 2**30, 1),
+                          "memory_clock_kHz": getattr(props, "memory_clock_rate", None),
+                          "memory_bus_bits": getattr(props, "memory_bus_width", None)}
+    except Exception:  # informational only
+        line["device"] = None
     if not args.only and not args.no_cpu and head in GS_WORKLOADS:
         line["cpu_baseline"] = cpu_baseline_gs(*r["cpu"])
     else:
@@ -667,6 +684,7 @@ def main():
                     others["C3_%s_%s" % (INTERP_NAMES[interp], PAD_NAMES[pad])] = summary_of(rr)
             rr = bench_gs("C3", args.steps, args.warmup, sets=1)
             others["C3_bilinear_zeros_same_buffers_every_step"] = summary_of(rr)
+            others["C3_bilinear_zeros_align_corners"] = summary_of(bench_gs("C3", args.steps, args.warmup, align=True))
             others["C3_bilinear_zeros_channels_last"] = summary_of(bench_gs("C3", args.steps, args.warmup,
                                                                              channels_last=True))
             # the third interpolation mode on the same tensors (not part of the headline set)
