@@ -207,11 +207,11 @@ __device__ __forceinline__ float visit_sum(const TI* base, int32_t pitch, int32_
 
 // The same sum with the column part of the loop taken out: a lane keeps the weights of the (at most KX) columns it
 // visits -- computed once, by the same repeated additions -- and a row costs one LDS read, two products and an add
-// per column.  Column k of a lane with fewer than k + 1 visits re-reads its last column and leaves the sum alone.
+// per column.  Column k of a lane with fewer than k + 1 visits leaves the sum alone.
 template <typename TI, int KX>
 __device__ __forceinline__ float visit_sum_fixed(const TI* tile_xy, int32_t pitch, int32_t y0, int32_t in_y_start,
-                                                 int32_t nx, const float (&xl)[KX], const int32_t (&xo)[KX],
-                                                 float out_y_start, float fh, float scale_h, float last_y, int32_t Hd)
+                                                 int32_t nx, const float (&xl)[KX], float out_y_start, float fh,
+                                                 float scale_h, float last_y, int32_t Hd, float neg_zero)
 {
     float acc = 0.0f;
     float out_y = out_y_start;
@@ -221,7 +221,9 @@ __device__ __forceinline__ float visit_sum_fixed(const TI* tile_xy, int32_t pitc
         const TI* row = tile_xy + (in_y - y0) * pitch;
 #pragma unroll
         for (int k = 0; k < KX; k++) {
-            const float t = ElemIO<TI>::load(row + xo[k]) * y_lerp * xl[k];
+            // fma(g, w, -0) is g * w bit for bit and lets a 16-bit element be converted by the multiply itself; the
+            // read of a column past the lane's last one may fetch anything (it stays inside LDS) and is dropped
+            const float t = __builtin_fmaf(ElemIO<TI>::load(row + k), y_lerp, neg_zero) * xl[k];
             acc = (k < nx) ? acc + t : acc;
         }
         out_y += scale_h;
@@ -238,7 +240,7 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
                                                                         int32_t Hd, int32_t Wd, float scale_h,
                                                                         float scale_w, float inv_scale_h,
                                                                         float inv_scale_w, int32_t tile_rows,
-                                                                        int32_t cap_words)
+                                                                        int32_t cap_words, float neg_zero)
 {
     constexpr int EPW = 4 / (int)sizeof(TI);  // elements per 4-byte word
     extern __shared__ uint32_t tile_words[];
@@ -297,29 +299,39 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
     // column weights of this lane, for the variants with a fixed column count
     constexpr int KMAX = 8;
     float xl[KMAX];
-    int32_t xo[KMAX];
     {
         float out_x = out_x_start;
 #pragma unroll
         for (int k = 0; k < KMAX; k++) {
             const float xc = __builtin_fmaxf(0.0f, __builtin_fminf(out_x, last_x));
             xl[k] = 1.0f - __builtin_fabsf(xc - fw);
-            xo[k] = (k < nx) ? k : ((nx > 0) ? nx - 1 : 0);
             out_x += scale_w;
         }
     }
     const int32_t nx_max = s_nx;
+    // starting position and step of this lane in the tile's (row, word) grid for the copy loop
+    const int32_t pw1 = (pitch_w > 0) ? pitch_w : 1;
+    const int32_t ld_r0 = (int32_t)threadIdx.x / pw1, ld_c0 = (int32_t)threadIdx.x % pw1;
+    const int32_t ld_dr = kGradThreads / pw1, ld_dc = kGradThreads % pw1;
     const int32_t x_base = (nx > 0) ? in_x_start - tile_x0 : 0;
 
     for (int64_t pl = blockIdx.z; pl < planes; pl += gridDim.z) {
         const TI* gp = g + pl * (int64_t)Hd * Wd;
         if (use_lds) {
+            // word i of the tile is (row i / pitch_w, word i % pitch_w); the pair is advanced instead of divided
             const int32_t total = rows * pitch_w;
+            int32_t r = ld_r0, cw = ld_c0;
+            const uint32_t* src = reinterpret_cast<const uint32_t*>(gp + (int64_t)tile_y0 * Wd + tile_x0);
+            const int32_t row_words = Wd / EPW;
 #pragma unroll 4
             for (int32_t i = threadIdx.x; i < total; i += kGradThreads) {
-                const int32_t r = i / pitch_w;
-                const int32_t cw = i - r * pitch_w;
-                tile_words[i] = *reinterpret_cast<const uint32_t*>(gp + (int64_t)(tile_y0 + r) * Wd + tile_x0 + cw * EPW);
+                tile_words[i] = src[(int64_t)r * row_words + cw];
+                r += ld_dr;
+                cw += ld_dc;
+                if (cw >= pitch_w) {
+                    cw -= pitch_w;
+                    r++;
+                }
             }
             __syncthreads();
         }
@@ -331,17 +343,15 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
                 // separate call sites so that each is compiled for its own address space (LDS reads, global loads)
                 if (use_lds && nx_max <= 4) {
                     const float(&xl4)[4] = reinterpret_cast<const float(&)[4]>(xl);
-                    const int32_t(&xo4)[4] = reinterpret_cast<const int32_t(&)[4]>(xo);
-                    acc = visit_sum_fixed<TI, 4>(tile + x_base, pitch, tile_y0, in_y_start, nx, xl4, xo4, out_y_start,
-                                                 (float)H, scale_h, last_y, Hd);
+                    acc = visit_sum_fixed<TI, 4>(tile + x_base, pitch, tile_y0, in_y_start, nx, xl4, out_y_start,
+                                                 (float)H, scale_h, last_y, Hd, neg_zero);
                 } else if (use_lds && nx_max <= 6) {
                     const float(&xl6)[6] = reinterpret_cast<const float(&)[6]>(xl);
-                    const int32_t(&xo6)[6] = reinterpret_cast<const int32_t(&)[6]>(xo);
-                    acc = visit_sum_fixed<TI, 6>(tile + x_base, pitch, tile_y0, in_y_start, nx, xl6, xo6, out_y_start,
-                                                 (float)H, scale_h, last_y, Hd);
+                    acc = visit_sum_fixed<TI, 6>(tile + x_base, pitch, tile_y0, in_y_start, nx, xl6, out_y_start,
+                                                 (float)H, scale_h, last_y, Hd, neg_zero);
                 } else if (use_lds && nx_max <= 8) {
-                    acc = visit_sum_fixed<TI, 8>(tile + x_base, pitch, tile_y0, in_y_start, nx, xl, xo, out_y_start,
-                                                 (float)H, scale_h, last_y, Hd);
+                    acc = visit_sum_fixed<TI, 8>(tile + x_base, pitch, tile_y0, in_y_start, nx, xl, out_y_start,
+                                                 (float)H, scale_h, last_y, Hd, neg_zero);
                 } else if (use_lds) {
                     acc = visit_sum<TI>(tile, pitch, tile_y0, tile_x0, in_y_start, in_x_start, out_y_start,
                                         out_x_start, (float)H, fw, scale_h, scale_w, last_y, last_x, Hd, Wd);
@@ -392,12 +402,12 @@ hipError_t run(const ResizeGradArgs& a, hipStream_t stream)
                 hipLaunchKernelGGL((resize_grad_lds_kernel<TI, TO, true>), grid, dim3(kGradThreads), kCapWords * 4,
                                    stream, (const TI*)a.x, (TO*)a.y, planes, (int32_t)a.Hs, (int32_t)a.Ws,
                                    (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h, a.scale_w, a.inv_scale_h, a.inv_scale_w,
-                                   tile_rows, kCapWords);
+                                   tile_rows, kCapWords, -0.0f);
             } else {
                 hipLaunchKernelGGL((resize_grad_lds_kernel<TI, TO, false>), grid, dim3(kGradThreads), kCapWords * 4,
                                    stream, (const TI*)a.x, (TO*)a.y, planes, (int32_t)a.Hs, (int32_t)a.Ws,
                                    (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h, a.scale_w, a.inv_scale_h, a.inv_scale_w,
-                                   tile_rows, kCapWords);
+                                   tile_rows, kCapWords, -0.0f);
             }
             return hipGetLastError();
         }
