@@ -59,12 +59,16 @@ __device__ __forceinline__ void load_grid_pair(const T* gp, bool pair_aligned, f
 
 // Raw tap values of one pixel from a staged plane (LDS reads only, no arithmetic, so that the reads of
 // many pixels can be in flight together).
+// `taddr` holds absolute LDS addresses of the taps in the first plane of the ring (base of the LDS allocation
+// already added, once, in the prologue); `plane_off` is the compile-time distance of the plane being sampled, which
+// ends up in the instruction's immediate offset.
 template <typename T, int NT>
-__device__ __forceinline__ void load_taps(const char* plane, const uint32_t* toff, T* raw)
+__device__ __forceinline__ void load_taps(uint32_t plane_off, const uint32_t* taddr, T* raw)
 {
+    typedef const T __attribute__((address_space(3))) * lds_elem_ptr_t;
 #pragma unroll
     for (int t = 0; t < NT; t++) {
-        raw[t] = *reinterpret_cast<const T*>(plane + toff[t]);
+        raw[t] = *reinterpret_cast<lds_elem_ptr_t>((uintptr_t)(taddr[t] + plane_off));
     }
 }
 
@@ -398,10 +402,28 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
         }
     }
 
+    // tap offsets become absolute LDS addresses (left as offsets, the compiler re-adds the allocation's base to
+    // every tap in every stage)
+    {
+        uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
+        // opaque to the compiler from here on: seen as the allocation's symbol, the base would be split off the sum
+        // again and re-added at every use
+        asm volatile("" : "+s"(lds_base));
+#pragma unroll
+        for (int j = 0; j < PPT; j++) {
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                toff[j][t] += lds_base;
+                asm volatile("" : "+v"(toff[j][t]));  // the sum itself is what stays in the register
+            }
+        }
+    }
+
     T* yb = y + ((int64_t)n * C + c_begin) * out_plane;
     const uint32_t out_plane_bytes = (uint32_t)out_plane * (uint32_t)sizeof(T);
 
-    auto sample_stage = [&](int32_t s, const char* buf) {
+    // `buf` is the byte offset of the stage's slot inside the ring
+    auto sample_stage = [&](int32_t s, uint32_t buf) {
         const int32_t left = nchan - s * CGS;
         T* ys = yb + (int64_t)s * CGS * out_plane;
         if (left >= CGS) {
@@ -452,7 +474,7 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
         for (int u = 0; u < NBUF; u++) {
             if (s + u < nstages) {
                 lds_barrier();
-                sample_stage(s + u, lds + u * SLOT_BYTES);
+                sample_stage(s + u, (uint32_t)(u * SLOT_BYTES));
             }
         }
     }
