@@ -34,8 +34,10 @@ LdsPlan make_lds_plan(const GridSamplerArgs& a)
     const int64_t tile = (int64_t)kThreads * p.ppt;
     p.tiles_per_n = (uint32_t)((out_plane + tile - 1) / tile);
     // channels per workgroup: as many stages as possible (the pixel decisions are reused across them) while
-    // still giving the 256 CUs at least two workgroups each
-    const int64_t want_blocks = 512;
+    // still giving the 256 CUs at least two workgroups each -- one each where the ring takes more than half of a
+    // CU's LDS and a second workgroup could not be resident anyway (bf16 N8 C128 128x128 -> 256x256 random grid:
+    // 95 us with 32 channels per workgroup, 87 us with 64)
+    const int64_t want_blocks = (p.lds_bytes > kLdsLimit / 2) ? 256 : 512;
     const int64_t base = a.N * p.tiles_per_n;
     int64_t cblocks = (want_blocks + base - 1) / base;
     const int64_t max_cblocks = (a.C + cgs - 1) / cgs;
