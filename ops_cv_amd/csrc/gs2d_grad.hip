@@ -32,6 +32,18 @@ constexpr int kThreads = 256;         // also the chunk length of the accumulati
 constexpr uint32_t kKeyBits = 8;      // 256 points of a chunk
 constexpr uint32_t kEpochMax = (1u << (32 - kKeyBits)) - 1;
 
+// What a tap adds: the incoming gradient times the tap weight, rounded to fp32 and then to the element type (two
+// roundings, as the reference's float product followed by a cast).  The fp32 value is pinned in a register: left
+// alone, the compiler merges product and conversion into one instruction that rounds once, which differs on ties.
+template <typename T, int INTERP>
+__device__ __forceinline__ float contribution(float go, float w)
+{
+    if (INTERP == 1) {
+        return rt<T>(go);
+    }
+    return rt<T>(as_fp32_value(INTERP == 0 ? w * go : go * w));
+}
+
 struct GradParams {
     int32_t C, H, W, Ho, Wo;
     int32_t pad, align;
@@ -163,7 +175,7 @@ __global__ __launch_bounds__(kThreads) void gs2d_grad_input_kernel(const T* __re
 #pragma unroll
                             for (int cb = 0; cb < CB; cb++) {
                                 const float val =
-                                    rt<T>(INTERP == 1 ? go[cb] : (INTERP == 0 ? wt[k] * go[cb] : go[cb] * wt[k]));
+                                    contribution<T, INTERP>(go[cb], wt[k]);
                                 ElemIO<T>::store(e + cb * p.band_px, cur[cb] + val);
                             }
                         } else {
@@ -171,7 +183,7 @@ __global__ __launch_bounds__(kThreads) void gs2d_grad_input_kernel(const T* __re
                             for (int cb = 0; cb < CB; cb++) {
                                 if (cb < nc) {
                                     const float val =
-                                        rt<T>(INTERP == 1 ? go[cb] : (INTERP == 0 ? wt[k] * go[cb] : go[cb] * wt[k]));
+                                        contribution<T, INTERP>(go[cb], wt[k]);
                                     ElemIO<T>::store(e + cb * p.band_px, ElemIO<T>::load(e + cb * p.band_px) + val);
                                 }
                             }
@@ -293,8 +305,9 @@ __global__ __launch_bounds__(kThreads) void gs2d_grad_grid_kernel(const T* __res
             }
         }
     }
-    ElemIO<T>::store(dgrid + 2 * idx, tp.mx * gix);
-    ElemIO<T>::store(dgrid + 2 * idx + 1, tp.my * giy);
+    // products in fp32 first, then the conversion (see contribution())
+    ElemIO<T>::store(dgrid + 2 * idx, as_fp32_value(tp.mx * gix));
+    ElemIO<T>::store(dgrid + 2 * idx + 1, as_fp32_value(tp.my * giy));
 }
 
 template <typename T, int INTERP>

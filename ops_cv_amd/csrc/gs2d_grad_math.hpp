@@ -40,7 +40,9 @@ __device__ __forceinline__ float unnormalize_set_grad(float coord, int32_t size,
         c = ((coord + 1.0f) * (float)size - 1.0f) / 2.0f;
         *mult = rt<T>((float)size / 2.0f);
     }
-    return rt<T>(c);
+    // the fp32 result is pinned before it is rounded to T: product and conversion merged into one instruction would
+    // round once where the reference rounds twice
+    return rt<T>(as_fp32_value(c));
 }
 
 // grid_sampler3_d_grad_simt_base.h:68-86

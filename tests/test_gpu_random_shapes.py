@@ -1,0 +1,151 @@
+"""Seeded random shapes and modes for every entry point, bit-exact against the oracle.
+
+The enumerated tests pick shapes by hand around the kernels' size classes; this sweep draws them, so that tile
+edges, odd extents and class boundaries nobody thought of are met as well.  Every case prints its parameters first.
+"""
+import sys
+
+import numpy as np
+import pytest
+
+import inputs as I
+
+pytestmark = pytest.mark.gpu
+
+
+def _bits(a, dtype):
+    return np.ascontiguousarray(a).view(np.uint32 if dtype == "fp32" else np.uint16)
+
+
+def _same(got, ref, dtype, what):
+    rn = np.isnan(I.as_f32(ref, dtype))
+    assert np.array_equal(np.isnan(I.as_f32(got, dtype)), rn), what
+    assert np.array_equal(np.where(rn, 0, _bits(got, dtype)), np.where(rn, 0, _bits(ref, dtype))), what
+
+
+def _say(*what):
+    print("case:", *what)
+    sys.stdout.flush()
+
+
+def _dims(rng, lo, hi, n):
+    # log-uniform extents: small ones are as likely as large ones
+    return [int(round(np.exp(rng.uniform(np.log(lo), np.log(hi))))) for _ in range(n)]
+
+
+def test_random_grid_sampler2d(oracle, device, aclnn):
+    import torch
+    rng = np.random.default_rng(9001)
+    for case in range(240):
+        dtype = I.DTYPES[case % 3]
+        N, C = _dims(rng, 1, 5, 1)[0], _dims(rng, 1, 40, 1)[0]
+        H, W = _dims(rng, 1, 150, 2)
+        Ho, Wo = _dims(rng, 1, 120, 2)
+        interp, pad, align = int(rng.integers(0, 3)), int(rng.integers(0, 3)), bool(rng.integers(0, 2))
+        _say("gs2d", dtype, N, C, H, W, Ho, Wo, interp, pad, align)
+        x = I.cast_np(rng.standard_normal((N, C, H, W)).astype(np.float32), dtype)
+        g = I.cast_np(rng.uniform(-1.4, 1.4, (N, Ho, Wo, 2)).astype(np.float32), dtype)
+        ref = oracle.grid_sampler2d(x, g, interp, pad, align, dtype=I.oracle_code(dtype))
+        y = aclnn.grid_sampler2d(I.to_torch(x, dtype, device), I.to_torch(g, dtype, device), interp, pad, align)
+        torch.cuda.synchronize()
+        _same(I.from_torch(y, dtype), ref, dtype, (case, dtype, N, C, H, W, Ho, Wo, interp, pad, align))
+
+
+def test_random_grid_sampler2d_large_planes(oracle, device, aclnn):
+    """input planes from a few KB to beyond the largest LDS class (the direct kernel), few channels"""
+    import torch
+    rng = np.random.default_rng(9004)
+    for case in range(45):
+        dtype = I.DTYPES[case % 3]
+        N, C = int(rng.integers(1, 3)), int(rng.integers(1, 7))
+        H, W = _dims(rng, 40, 420, 2)
+        Ho, Wo = _dims(rng, 8, 300, 2)
+        interp, pad, align = int(rng.integers(0, 3)), int(rng.integers(0, 3)), bool(rng.integers(0, 2))
+        _say("gs2d large", dtype, N, C, H, W, Ho, Wo, interp, pad, align)
+        x = I.cast_np(rng.standard_normal((N, C, H, W)).astype(np.float32), dtype)
+        g = I.cast_np(rng.uniform(-1.2, 1.2, (N, Ho, Wo, 2)).astype(np.float32), dtype)
+        ref = oracle.grid_sampler2d(x, g, interp, pad, align, dtype=I.oracle_code(dtype))
+        y = aclnn.grid_sampler2d(I.to_torch(x, dtype, device), I.to_torch(g, dtype, device), interp, pad, align)
+        torch.cuda.synchronize()
+        _same(I.from_torch(y, dtype), ref, dtype, (case, dtype, N, C, H, W, Ho, Wo, interp, pad, align))
+
+
+def test_random_resize_family(oracle, device, aclnn):
+    import torch
+    rng = np.random.default_rng(9002)
+    for case in range(240):
+        dtype = I.DTYPES[case % 3]
+        N, C = _dims(rng, 1, 4, 1)[0], _dims(rng, 1, 70, 1)[0]
+        H, W = _dims(rng, 1, 90, 2)
+        Ho, Wo = _dims(rng, 1, 200, 2)
+        align, cl = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        _say("upsample", dtype, N, C, H, W, Ho, Wo, align, cl)
+        x = I.cast_np(rng.standard_normal((N, C, H, W)).astype(np.float32), dtype)
+        xin = np.ascontiguousarray(x.transpose(0, 2, 3, 1)) if cl else x
+        ref = oracle.resize_point_copy(xin, (Ho, Wo), align=align, dtype=I.oracle_code(dtype)) if cl else None
+        if ref is None:
+            ref = oracle.upsample_bilinear2d(x, (Ho, Wo), align, dtype=I.oracle_code(dtype))
+            ref = np.ascontiguousarray(ref.transpose(0, 2, 3, 1)) if cl else ref
+        y = aclnn.upsample_bilinear2d(I.to_torch(xin, dtype, device), (Ho, Wo), align, channels_last=cl)
+        torch.cuda.synchronize()
+        _same(I.from_torch(y, dtype), ref, dtype, (case, "up", dtype, N, C, H, W, Ho, Wo, align, cl))
+        # nearest through aclnnResize on the same tensors
+        _say("nearest", dtype, N, C, H, W, Ho, Wo, cl)
+        scales = (1.0, Ho / H, Wo / W, 1.0) if cl else (1.0, 1.0, Ho / H, Wo / W)
+        shape = (N, Ho, Wo, C) if cl else (N, C, Ho, Wo)
+        out = torch.empty(shape, dtype=I.to_torch(xin[:1, :1, :1, :1], dtype, device).dtype, device=device)
+        try:
+            y = aclnn.resize(I.to_torch(xin, dtype, device), scales, "nearest", out=out, channels_last=cl)
+        except aclnn.AclnnError:
+            continue  # float scales that do not reproduce the extents exactly are rejected, as in the reference
+        torch.cuda.synchronize()
+        ref = oracle.resize_nearest(xin, (Ho, Wo), channels_last=cl, dtype=I.oracle_code(dtype))
+        _same(I.from_torch(y, dtype), ref, dtype, (case, "nearest", dtype, N, C, H, W, Ho, Wo, cl))
+        # gradient of the upsample
+        _say("upsample backward", dtype, N, C, H, W, Ho, Wo, align, cl)
+        gshape = (N, Ho, Wo, C) if cl else (N, C, Ho, Wo)
+        go = I.cast_np(rng.standard_normal(gshape).astype(np.float32), dtype)
+        ref = oracle.upsample_bilinear2d_backward(go, (H, W), align, channels_last=cl, dtype=I.oracle_code(dtype))
+        isz = (N, H, W, C) if cl else (N, C, H, W)
+        y = aclnn.upsample_bilinear2d_backward(I.to_torch(go, dtype, device), isz, align, channels_last=cl)
+        torch.cuda.synchronize()
+        _same(I.from_torch(y, dtype), ref, dtype, (case, "upbwd", dtype, N, C, H, W, Ho, Wo, align, cl))
+
+
+def test_random_sampler_backward_and_3d(oracle, device, aclnn):
+    import torch
+    rng = np.random.default_rng(9003)
+    for case in range(150):
+        dtype = I.DTYPES[case % 3]
+        N, C = _dims(rng, 1, 3, 1)[0], _dims(rng, 1, 12, 1)[0]
+        H, W = _dims(rng, 1, 90, 2)
+        Ho, Wo = _dims(rng, 1, 60, 2)
+        interp, pad, align = int(rng.integers(0, 3)), int(rng.integers(0, 3)), bool(rng.integers(0, 2))
+        _say("gs2d backward", dtype, N, C, H, W, Ho, Wo, interp, pad, align)
+        x = I.cast_np(rng.standard_normal((N, C, H, W)).astype(np.float32), dtype)
+        g = I.cast_np(rng.uniform(-1.3, 1.3, (N, Ho, Wo, 2)).astype(np.float32), dtype)
+        go = I.cast_np(rng.standard_normal((N, C, Ho, Wo)).astype(np.float32), dtype)
+        rdx, rdg = oracle.grid_sampler2d_backward(go, x, g, interp, pad, align, dtype=I.oracle_code(dtype))
+        dx, dg = aclnn.grid_sampler2d_backward(I.to_torch(go, dtype, device), I.to_torch(x, dtype, device),
+                                               I.to_torch(g, dtype, device), interp, pad, align)
+        torch.cuda.synchronize()
+        _same(I.from_torch(dx, dtype), rdx, dtype, (case, "dx", dtype, N, C, H, W, Ho, Wo, interp, pad, align))
+        _same(I.from_torch(dg, dtype), rdg, dtype, (case, "dgrid", dtype, N, C, H, W, Ho, Wo, interp, pad, align))
+    for case in range(150):
+        dtype = I.DTYPES[case % 3]
+        N, C = _dims(rng, 1, 3, 1)[0], _dims(rng, 1, 20, 1)[0]
+        D, H, W = _dims(rng, 1, 20, 3)
+        Do, Ho, Wo = _dims(rng, 1, 16, 3)
+        interp, pad, align, cl = int(rng.integers(0, 2)), int(rng.integers(0, 3)), bool(rng.integers(0, 2)), bool(
+            rng.integers(0, 2))
+        _say("gs3d", dtype, N, C, D, H, W, Do, Ho, Wo, interp, pad, align, cl)
+        x = I.cast_np(rng.standard_normal((N, C, D, H, W)).astype(np.float32), dtype)
+        g = I.cast_np(rng.uniform(-1.4, 1.4, (N, Do, Ho, Wo, 3)).astype(np.float32), dtype)
+        ref = oracle.grid_sampler3d(x, g, interp, pad, align, dtype=I.oracle_code(dtype))
+        xin = np.ascontiguousarray(x.transpose(0, 2, 3, 4, 1)) if cl else x
+        y = aclnn.grid_sampler3d(I.to_torch(xin, dtype, device), I.to_torch(g, dtype, device), interp, pad, align,
+                                 channels_last=cl)
+        torch.cuda.synchronize()
+        got = I.from_torch(y, dtype)
+        got = got.transpose(0, 4, 1, 2, 3) if cl else got
+        _same(got, ref, dtype, (case, "gs3d", dtype, N, C, D, H, W, Do, Ho, Wo, interp, pad, align, cl))
