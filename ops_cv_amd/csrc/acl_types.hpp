@@ -129,7 +129,15 @@ struct GridSamplerGradArgs {
     void* dgrid = nullptr;       // (N,Hout,Wout,2)
 };
 
-enum class ResizeMode : int { Bilinear = 0, Copy = 1, Broadcast = 2, FirstPixel = 3, Nearest = 4, PointCopy = 5 };
+enum class ResizeMode : int {
+    Bilinear = 0,
+    Copy = 1,
+    Broadcast = 2,
+    FirstPixel = 3,
+    Nearest = 4,
+    PointCopy = 5,
+    FourWeights = 6  // channels-last: sum of four weighted taps instead of two nested blends
+};
 
 struct ResizeArgs {
     Elem elem = Elem::F32;

@@ -265,6 +265,80 @@ __global__ __launch_bounds__(kThreads) void resize_nhwc_vec_kernel(const T* __re
     }
 }
 
+// Four-weights NHWC variant (image/resize_bilinear_v2/op_kernel/arch35/resize_bilinear_v2_c_parallel.h:122-147,190-232):
+// the reference's template for channel runs of 128 bytes and more shrunk to half or less forms the four corner weights
+//   (1-dy)(1-dx), (1-dy)dx, dy(1-dx), dy*dx
+// first and adds  (NW*w + NE*w) + (SW*w + SE*w),  which rounds differently from the nested blends of the per-element
+// template.  Its taps are "floor, then +1 when the fraction is positive"; for the non-negative source positions that a
+// scale of two or more produces these are the floor/ceil taps of axis_tap().  One lane per run of UE channels of an
+// output pixel; a shrink of two or more touches every source pixel at most once, so there is nothing to reuse.
+template <typename T, bool HALF_PIXEL, int UE>
+__global__ __launch_bounds__(kThreads) void resize_nhwc_four_weights_kernel(const T* __restrict__ x, T* __restrict__ y,
+                                                                             int64_t N, int32_t C, int32_t Hs,
+                                                                             int32_t Ws, int32_t Hd, int32_t Wd,
+                                                                             float scale_h, float scale_w,
+                                                                             int streaming)
+{
+    typedef uint32_t words_t __attribute__((ext_vector_type((UE * sizeof(T) >= 4) ? UE * sizeof(T) / 4 : 1)));
+    const int32_t units = C / UE;
+    const int64_t row_units = (int64_t)Wd * units;
+    const int64_t e = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (e >= row_units) {
+        return;
+    }
+    const int32_t w = (int32_t)(e / units);
+    const int32_t c = (int32_t)(e - (int64_t)w * units) * UE;
+    const AxisTap tx = axis_tap<HALF_PIXEL>(w, scale_w, Ws);
+    const float dx = tx.lambda;
+    const int64_t o0 = (int64_t)tx.i0 * C + c;
+    const int64_t o1 = (int64_t)tx.i1 * C + c;
+    const int64_t src_row = (int64_t)Ws * C;
+    const int64_t rows = N * Hd;
+    auto fetch = [&](T* dst, const T* src) {
+        if (UE * sizeof(T) >= 4) {
+            const words_t raw = *reinterpret_cast<const words_t*>(src);
+            __builtin_memcpy(dst, &raw, UE * sizeof(T));
+        } else {
+            dst[0] = src[0];
+        }
+    };
+    for (int64_t r = blockIdx.y; r < rows; r += gridDim.y) {
+        const int64_t n = r / Hd;
+        const int32_t h = (int32_t)(r - n * Hd);
+        const AxisTap ty = axis_tap<HALF_PIXEL>(h, scale_h, Hs);
+        const float dy = ty.lambda;
+        const float w_nw = (1.0f - dy) * (1.0f - dx);
+        const float w_ne = (1.0f - dy) * dx;
+        const float w_sw = dy * (1.0f - dx);
+        const float w_se = dy * dx;
+        const T* top = x + (n * Hs + ty.i0) * src_row;
+        const T* bot = x + (n * Hs + ty.i1) * src_row;
+        T nw[UE], ne[UE], sw[UE], se[UE], outv[UE];
+        fetch(nw, top + o0);
+        fetch(ne, top + o1);
+        fetch(sw, bot + o0);
+        fetch(se, bot + o1);
+#pragma unroll
+        for (int i = 0; i < UE; i++) {
+            const float sum_top = ElemIO<T>::load(&nw[i]) * w_nw + ElemIO<T>::load(&ne[i]) * w_ne;
+            const float sum_bot = ElemIO<T>::load(&sw[i]) * w_sw + ElemIO<T>::load(&se[i]) * w_se;
+            ElemIO<T>::store(&outv[i], sum_top + sum_bot);
+        }
+        T* dst = y + (r * row_units + e) * UE;
+        if (UE * sizeof(T) >= 4) {
+            words_t raw;
+            __builtin_memcpy(&raw, outv, UE * sizeof(T));
+            if (streaming) {
+                __builtin_nontemporal_store(raw, reinterpret_cast<words_t*>(dst));
+            } else {
+                *reinterpret_cast<words_t*>(dst) = raw;
+            }
+        } else {
+            dst[0] = outv[0];
+        }
+    }
+}
+
 // Nearest-neighbour resize (align_corners = false, half_pixel_centers = false):
 //   src = min(floor(float(dst) * scale), len_src - 1)
 // image/resize_nearest_neighbor_v2/op_kernel/arch35/resize_nearest_neighbor_v2_simt.h:103-124.
@@ -530,6 +604,22 @@ bool nhwc_vec_ok(const ResizeArgs& a)
            reinterpret_cast<uintptr_t>(a.y) % 16 == 0;
 }
 
+// Channels per lane of the four-weights kernel: the widest of 16 bytes, 8 bytes or one element that divides C and
+// that both tensors are aligned to.
+template <typename T>
+int four_weights_unit(const ResizeArgs& a)
+{
+    constexpr int V = 16 / (int)sizeof(T);
+    const uintptr_t both = reinterpret_cast<uintptr_t>(a.x) | reinterpret_cast<uintptr_t>(a.y);
+    if (a.C % V == 0 && both % 16 == 0) {
+        return V;
+    }
+    if (a.C % (V / 2) == 0 && both % 8 == 0) {
+        return V / 2;
+    }
+    return 1;
+}
+
 template <typename T>
 hipError_t run_resize(const ResizeArgs& a, hipStream_t stream)
 {
@@ -614,6 +704,37 @@ hipError_t run_resize(const ResizeArgs& a, hipStream_t stream)
 #undef OPSCV_NEAREST
         return hipGetLastError();
     }
+    if (a.mode == ResizeMode::FourWeights) {
+        constexpr int V = 16 / (int)sizeof(T);
+        const int ue = four_weights_unit<T>(a);
+        const int64_t row_units = a.Wd * (a.C / ue);
+        const int64_t rows = a.N * a.Hd;
+        const int streaming = (out_elems * (int64_t)sizeof(T) >= (128ll << 20)) ? 1 : 0;
+        dim3 grid((unsigned)((row_units + kThreads - 1) / kThreads), (unsigned)(rows < 65535 ? rows : 65535));
+#define OPSCV_FOUR(HP, UE)                                                                                           \
+    hipLaunchKernelGGL((resize_nhwc_four_weights_kernel<T, HP, UE>), grid, dim3(kThreads), 0, stream, x, y, a.N,      \
+                       (int32_t)a.C, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h,           \
+                       a.scale_w, streaming)
+        if (a.half_pixel) {
+            if (ue == V) {
+                OPSCV_FOUR(true, V);
+            } else if (ue == V / 2) {
+                OPSCV_FOUR(true, V / 2);
+            } else {
+                OPSCV_FOUR(true, 1);
+            }
+        } else {
+            if (ue == V) {
+                OPSCV_FOUR(false, V);
+            } else if (ue == V / 2) {
+                OPSCV_FOUR(false, V / 2);
+            } else {
+                OPSCV_FOUR(false, 1);
+            }
+        }
+#undef OPSCV_FOUR
+        return hipGetLastError();
+    }
     if (nhwc_vec_ok<T>(a)) {
         constexpr int V = 16 / (int)sizeof(T);
         const int64_t row_vecs = a.Wd * (a.C / V);
@@ -693,6 +814,7 @@ const char* resize_variant(const ResizeArgs& a)
         case ResizeMode::Broadcast: return "broadcast";
         case ResizeMode::FirstPixel: return "first_pixel";
         case ResizeMode::PointCopy: return "point_copy";
+        case ResizeMode::FourWeights: return "nhwc_four_weights";
         case ResizeMode::Nearest: {
             if (a.channels_last) {
                 return "nearest_nhwc";

@@ -62,7 +62,14 @@ void plan_resize(ResizeArgs* a, bool align_corners, float user_scale_h, float us
         a->mode = ResizeMode::Copy;
     } else if (point_copy_steps(*a, align_corners, &a->point_step_h, &a->point_step_w)) {
         a->mode = ResizeMode::PointCopy;
-    } else if (one_src && (run_bytes >= kMinRunBytes || align_corners)) {
+    } else if (one_src && run_bytes >= kMinRunBytes) {
+        a->mode = ResizeMode::Broadcast;
+    } else if (a->channels_last && a->C * esz >= kMinRunBytes && a->scale_w >= 2.0f && a->scale_h >= 2.0f) {
+        // resize_bilinear_v2_tiling_arch35.cpp:337-352,604 (IsMatchCParallel): long channel runs shrunk to half or less
+        // go to the template that sums four weighted taps (resize_bilinear_v2_c_parallel.h:122-232); it comes before
+        // the per-element template and its special cases
+        a->mode = ResizeMode::FourWeights;
+    } else if (one_src && align_corners) {
         a->mode = ResizeMode::Broadcast;
     } else if (one_dst && align_corners) {
         a->mode = ResizeMode::FirstPixel;

@@ -853,6 +853,94 @@ int oracle_resize_point_copy(const void* x, void* y, int dtype, int64_t N, int64
 }
 
 /* ------------------------------------------------------------------------------------------
+ * Channels-last bilinear resize: x (N,Hs,Ws,C) -> y (N,Hd,Wd,C)
+ *   template order : image/resize_bilinear_v2/op_host/arch35/resize_bilinear_v2_tiling_arch35.cpp:592-623
+ *                    (all copy, point copy, broadcast from C * esz >= 128, channel-parallel from C * esz >= 128
+ *                    and both scales >= 2, else the per-element template)
+ *   channel-parallel arithmetic : image/resize_bilinear_v2/op_kernel/arch35/resize_bilinear_v2_c_parallel.h:122-147
+ *                    (taps and weights) and :190-232 (four products, top sum, bottom sum, total)
+ *   per-element template : image/resize_bilinear_v2/op_kernel/arch35/resize_bilinear_v2_simt_nhwc.h:60-150 with the
+ *                    special cases picked in image/resize_bilinear_v2/op_kernel/resize_bilinear_v2_apt.cpp:117-142
+ * Returns the template that produced y: 0 per-element, 1 all copy, 2 broadcast, 3 first pixel, 4 point copy,
+ * 5 channel-parallel; -1 on bad arguments.
+ * ---------------------------------------------------------------------------------------- */
+int oracle_upsample_bilinear2d_nhwc(const void* x, void* y, int dtype, int64_t N, int64_t C, int64_t Hs, int64_t Ws,
+                                    int64_t Hd, int64_t Wd, int align_corners, double scales_h, double scales_w)
+{
+    if (dtype < 0 || dtype > 2 || Hs <= 0 || Ws <= 0) {
+        return -1;
+    }
+    const int64_t esz = (dtype == ORACLE_F32) ? 4 : 2;
+    const int half_pixel = !align_corners;
+    const float scale_h = oracle_resize_scale(Hs, Hd, align_corners, (float)scales_h);
+    const float scale_w = oracle_resize_scale(Ws, Wd, align_corners, (float)scales_w);
+    const int wide = C * esz >= 128;
+    int mode = 0;
+    if (Hs == Hd && Ws == Wd) {
+        mode = 1;
+    } else if (oracle_resize_point_copy(x, y, dtype, N, C, Hs, Ws, Hd, Wd, align_corners, scales_h, scales_w) == 1) {
+        return 4;
+    } else if (wide && Hs == 1 && Ws == 1) {
+        mode = 2;
+    } else if (wide && scale_w >= 2.0f && scale_h >= 2.0f) {
+        mode = 5;
+    } else if (!half_pixel && Hs == 1 && Ws == 1) {
+        mode = 2;
+    } else if (!half_pixel && Hd == 1 && Wd == 1) {
+        mode = 3;
+    }
+    for (int64_t n = 0; n < N; n++) {
+        for (int64_t h = 0; h < Hd; h++) {
+            int32_t top, bottom;
+            float dy;
+            axis_tap(h, scale_h, half_pixel, Hs, &top, &bottom, &dy);
+            for (int64_t w = 0; w < Wd; w++) {
+                int32_t left, right;
+                float dx;
+                axis_tap(w, scale_w, half_pixel, Ws, &left, &right, &dx);
+                const int64_t dst = ((n * Hd + h) * Wd + w) * C;
+                if (mode >= 1 && mode <= 3) {
+                    const int64_t src = (mode == 1) ? dst : n * Hs * Ws * C;
+                    memcpy((char*)y + dst * esz, (const char*)x + src * esz, (size_t)(C * esz));
+                    continue;
+                }
+                const int64_t tl_i = ((n * Hs + top) * Ws + left) * C, tr_i = ((n * Hs + top) * Ws + right) * C;
+                const int64_t bl_i = ((n * Hs + bottom) * Ws + left) * C, br_i = ((n * Hs + bottom) * Ws + right) * C;
+                if (mode == 5) {
+                    /* c_parallel.h:122-142.  Its source position is not clamped at zero, which cannot matter: with a
+                     * scale of two or more the position is at least 0.5 (half pixel) or 0 (otherwise); from there on
+                     * "floor, then +1 when the fraction is positive" and floor/ceil name the same taps */
+                    const float w_nw = (1.0f - dy) * (1.0f - dx);
+                    const float w_ne = (1.0f - dy) * dx;
+                    const float w_sw = dy * (1.0f - dx);
+                    const float w_se = dy * dx;
+                    for (int64_t c = 0; c < C; c++) {
+                        float nw = load_as_float(x, dtype, tl_i + c) * w_nw;
+                        float ne = load_as_float(x, dtype, tr_i + c) * w_ne;
+                        float sw = load_as_float(x, dtype, bl_i + c) * w_sw;
+                        float se = load_as_float(x, dtype, br_i + c) * w_se;
+                        float sum_top = nw + ne;
+                        float sum_bot = sw + se;
+                        store_from_float(y, dtype, dst + c, sum_top + sum_bot);
+                    }
+                    continue;
+                }
+                for (int64_t c = 0; c < C; c++) {
+                    float tl = load_as_float(x, dtype, tl_i + c);
+                    float tr = load_as_float(x, dtype, tr_i + c);
+                    float bl = load_as_float(x, dtype, bl_i + c);
+                    float br = load_as_float(x, dtype, br_i + c);
+                    /* resize_bilinear_v2_simt_nhwc.h:147-148 */
+                    float out = (1.0f - dy) * ((1.0f - dx) * tl + dx * tr) + dy * ((1.0f - dx) * bl + dx * br);
+                    store_from_float(y, dtype, dst + c, out);
+                }
+            }
+        }
+    }
+    return mode;
+}
+
+/* ------------------------------------------------------------------------------------------
  * Volumetric grid sampler (5-D)
  *   image/grid_sample/op_kernel/arch35/grid_sampler_3d_bilinear_smit.h:53-135,146-191
  *   image/grid_sample/op_kernel/arch35/grid_sampler_bilinear_smit_common.h:37-94

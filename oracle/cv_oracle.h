@@ -125,6 +125,16 @@ int oracle_resize_point_copy(const void* x, void* y, int dtype, int64_t N, int64
                              int64_t Hd, int64_t Wd, int align_corners, double scales_h, double scales_w);
 
 /*
+ * Bilinear resize of channels-last tensors, x (N,Hs,Ws,C) -> y (N,Hd,Wd,C), with the reference's template choice for
+ * that layout (image/resize_bilinear_v2/op_host/arch35/resize_bilinear_v2_tiling_arch35.cpp:592-623): the
+ * channel-parallel template (image/resize_bilinear_v2/op_kernel/arch35/resize_bilinear_v2_c_parallel.h:122-232) sums
+ * four weighted taps where the per-element template (resize_bilinear_v2_simt_nhwc.h:60-150) nests two blends.
+ * Returns the template used: 0 per-element, 1 all copy, 2 broadcast, 3 first pixel, 4 point copy, 5 channel-parallel.
+ */
+int oracle_upsample_bilinear2d_nhwc(const void* x, void* y, int dtype, int64_t N, int64_t C, int64_t Hs, int64_t Ws,
+                                    int64_t Hd, int64_t Wd, int align_corners, double scales_h, double scales_w);
+
+/*
  * Volumetric grid sampler, forward (image/grid_sample/op_kernel/arch35/grid_sampler_3d_bilinear_smit.h:146-191).
  * x (N,C,Din,Hin,Win), grid (N,Dout,Hout,Wout,3) ordered x,y,z, y (N,C,Dout,Hout,Wout); interp 0 bilinear,
  * 1 nearest (round half to even, image/grid_sample/op_kernel/grid_sampler_3d_nearest.h:569-571).

@@ -98,6 +98,9 @@ def lib():
     L.oracle_gs3d_clip.argtypes = [f32, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32]
     L.oracle_grid_sampler2d_backward.restype = ctypes.c_int
     L.oracle_grid_sampler2d_backward.argtypes = [vp] * 5 + [ctypes.c_int] + [i64] * 6 + [ctypes.c_int] * 3
+    L.oracle_upsample_bilinear2d_nhwc.restype = ctypes.c_int
+    L.oracle_upsample_bilinear2d_nhwc.argtypes = [vp, vp, ctypes.c_int] + [i64] * 6 + [ctypes.c_int, ctypes.c_double,
+                                                                                         ctypes.c_double]
     L.oracle_resize_point_copy.restype = ctypes.c_int
     L.oracle_resize_point_copy.argtypes = [vp, vp, ctypes.c_int] + [i64] * 6 + [ctypes.c_int, ctypes.c_double,
                                                                             ctypes.c_double]
@@ -252,6 +255,22 @@ def upsample_bilinear2d(x, out_hw, align=False, scales_h=0.0, scales_w=0.0, dtyp
     if rc != 0:
         raise ValueError("oracle_upsample_bilinear2d rc=%d" % rc)
     return y
+
+
+NHWC_TEMPLATES = ("per_element", "copy", "broadcast", "first_pixel", "point_copy", "channel_parallel")
+
+
+def upsample_bilinear2d_nhwc(x_nhwc, out_hw, align=False, scales_h=0.0, scales_w=0.0, dtype=None, with_template=False):
+    """x (N,H,W,C) -> y (N,Ho,Wo,C) with the reference's template choice for channels-last tensors"""
+    x = np.ascontiguousarray(x_nhwc)
+    code = _code_of(x) if dtype is None else dtype
+    N, Hs, Ws, C = x.shape
+    y = np.empty((N, out_hw[0], out_hw[1], C), dtype=x.dtype)
+    rc = lib().oracle_upsample_bilinear2d_nhwc(_ptr(x), _ptr(y), code, N, C, Hs, Ws, out_hw[0], out_hw[1],
+                                               int(bool(align)), float(scales_h), float(scales_w))
+    if rc < 0:
+        raise ValueError("oracle_upsample_bilinear2d_nhwc rc=%d" % rc)
+    return (y, NHWC_TEMPLATES[rc]) if with_template else y
 
 
 def upsample_axis_taps(len_src, len_dst, align=False, user_scale=0.0):

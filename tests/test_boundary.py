@@ -240,6 +240,40 @@ def test_upsample_template_selection(aclnn, desc):
                fmt=aclnn.ACL_FORMAT_NHWC, align=True)[2] == "nhwc_generic"
 
 
+def test_upsample_template_selection_channels_last(aclnn, desc):
+    """the channels-last cases of the reference tiling UT whose attributes this entry point can express
+    (image/resize_bilinear_v2/tests/ut/op_host/arch35/test_resize_bilinear_v2_tiling.cpp case04, 05, 07, 09, 10, 11,
+    15, 16): keys 30000/30002 per-element, 40001 point copy, 10000 channel-parallel (four weights), 40003 broadcast,
+    40000 copy"""
+    f16, f32, nhwc = aclnn.ACL_FLOAT16, aclnn.ACL_FLOAT, aclnn.ACL_FORMAT_NHWC
+
+    def variant(inp, out, dt, align, sh=0.0, sw=0.0):
+        st, ws, v = _up(aclnn, desc, inp=inp, out=out, size=out[1:3], dt=dt, fmt=nhwc, align=align, sh=sh, sw=sw)
+        assert st == 0 and ws == 0
+        return v
+
+    assert variant((2, 128, 128, 256), (2, 192, 192, 256), f32, True, 1.5, 1.5) == "nhwc_vec"                 # case04
+    assert variant((128, 14, 16, 256), (128, 5, 8, 256), f32, False, 3.0, 3.0) == "nhwc_vec"                  # case05
+    assert variant((128, 14, 16, 256), (128, 5, 8, 256), f32, False) == "nhwc_four_weights"   # size ratios 2.8 and 2
+    assert variant((1, 36, 15, 128), (1, 12, 5, 128), f32, False) == "point_copy"                             # case07
+    assert variant((1, 36, 15, 128), (1, 12, 5, 128), f32, False, 0.2, 0.2) == "point_copy"                   # case09
+    assert variant((190, 22, 79, 128), (190, 13, 43, 128), f16, False, 0.31269457412229545,
+                   0.27077088627767687) == "nhwc_four_weights"                                                # case10
+    assert variant((190, 22, 79, 128), (190, 13, 43, 128), f16, False) == "nhwc_vec"          # 22 / 13 is under two
+    assert variant((1, 1, 1, 64), (1, 59, 32, 64), f32, True) == "broadcast"                                  # case11
+    assert variant((12768, 128, 128, 256), (12768, 192, 192, 256), f32, True, 1.5, 1.5) == "nhwc_vec"         # case15
+    assert variant((3, 11, 21, 5), (3, 11, 21, 5), aclnn.ACL_BF16, False) == "copy"                           # case16
+    # runs under 128 bytes never take the four-weights template; a 1x1 source of such runs is interpolated with
+    # half-pixel centres and broadcast with align_corners
+    assert variant((1, 8, 8, 32), (1, 3, 3, 32), f32, False) == "nhwc_four_weights"
+    assert variant((1, 8, 8, 32), (1, 3, 3, 32), f16, False) == "nhwc_vec"
+    assert variant((1, 1, 1, 14), (1, 13, 7, 14), f32, False) == "nhwc_generic"
+    assert variant((1, 1, 1, 14), (1, 13, 7, 14), f32, True) == "broadcast"
+    assert variant((1, 8, 8, 8), (1, 1, 1, 8), f32, True) == "first_pixel"
+    assert variant((1, 8, 8, 32), (1, 1, 1, 32), f32, True) == "point_copy"
+    assert variant((1, 8, 8, 32), (1, 1, 3, 32), f32, True) == "nhwc_four_weights"
+
+
 def _rs(aclnn, desc, inp=(1, 1, 2, 2), out=(1, 1, 4, 4), scales=(1, 1, 2, 2), mode=b"nearest", dt=None, odt=None,
         fmt=None, ofmt=None):
     dt = aclnn.ACL_FLOAT if dt is None else dt

@@ -47,18 +47,25 @@ def test_noncontiguous_views_are_honoured(oracle, device, aclnn):
 def test_upsample_nhwc(oracle, device, aclnn, dtype, align):
     torch = _torch()
     rng = np.random.default_rng(22)
+    seen = set()
     for (N, C, H, W), size in [((2, 5, 7, 9), (14, 18)), ((1, 64, 1, 1), (6, 6)), ((1, 3, 8, 8), (8, 8)),
                                ((2, 3, 6, 6), (1, 1)), ((1, 130, 3, 3), (5, 7)), ((2, 16, 9, 11), (20, 17)),
-                               ((1, 64, 12, 10), (5, 23)), ((1, 8, 1, 6), (4, 4))]:
+                               ((1, 64, 12, 10), (5, 23)), ((1, 8, 1, 6), (4, 4)), ((1, 14, 1, 1), (13, 7)),
+                               # long channel runs shrunk to half or less: the four-weights template, with channel
+                               # counts for every vector width of its kernel (16 bytes, 8 bytes, one element)
+                               ((2, 64, 12, 10), (5, 4)), ((1, 68, 23, 17), (7, 8)), ((1, 67, 9, 31), (4, 3)),
+                               ((2, 128, 16, 16), (1, 1)), ((1, 72, 40, 6), (3, 3))]:
         x32 = rng.standard_normal((N, C, H, W)).astype(np.float32)
         x = I.cast_np(x32, dtype)
-        ref = oracle.upsample_bilinear2d(x, size, align, dtype=I.oracle_code(dtype))
         xh = np.ascontiguousarray(x.transpose(0, 2, 3, 1))
+        ref, template = oracle.upsample_bilinear2d_nhwc(xh, size, align, dtype=I.oracle_code(dtype), with_template=True)
+        seen.add(template)
         y = aclnn.upsample_bilinear2d(I.to_torch(xh, dtype, device), size, align, channels_last=True)
         torch.cuda.synchronize()
-        got = I.from_torch(y, dtype).transpose(0, 3, 1, 2)
-        a, b = I.as_f32(got, dtype), I.as_f32(ref, dtype)
-        assert np.array_equal(a, b), "nhwc %s %s align=%s" % (dtype, (N, C, H, W), align)
+        got = I.from_torch(y, dtype)
+        assert np.array_equal(_bits(got, dtype), _bits(ref, dtype)), \
+            "nhwc %s %s align=%s template %s" % (dtype, (N, C, H, W), align, template)
+    assert {"per_element", "copy", "broadcast", "channel_parallel"} <= seen
 
 
 @pytest.mark.parametrize("dtype", I.DTYPES)
@@ -166,7 +173,7 @@ def test_resize_entry_point(oracle, device, aclnn, dtype, channels_last):
     rng = np.random.default_rng(300 + int(channels_last))
     cases = [((1, 1, 2, 2), (2.0, 2.0)), ((2, 8, 9, 12), (2.0, 2.0)), ((1, 16, 7, 5), (1.5, 2.5)),
              ((2, 3, 16, 16), (0.5, 0.75)), ((1, 4, 1, 1), (4.0, 8.0)), ((1, 2, 6, 6), (1.0, 1.0)),
-             ((1, 8, 33, 64), (3.0, 2.0))]
+             ((1, 8, 33, 64), (3.0, 2.0)), ((1, 64, 20, 18), (0.25, 0.5)), ((2, 66, 9, 14), (0.4, 0.3))]
     for shape, (sh, sw) in cases:
         N, C, H, W = shape
         Ho, Wo = int(float(H) * sh), int(float(W) * sw)
@@ -179,10 +186,10 @@ def test_resize_entry_point(oracle, device, aclnn, dtype, channels_last):
             torch.cuda.synchronize()
             if mode == "nearest":
                 ref = oracle.resize_nearest(xin, (Ho, Wo), channels_last=channels_last, dtype=I.oracle_code(dtype))
+            elif channels_last:
+                ref = oracle.upsample_bilinear2d_nhwc(xin, (Ho, Wo), False, 0.0, 0.0, dtype=I.oracle_code(dtype))
             else:
                 ref = oracle.upsample_bilinear2d(x, (Ho, Wo), False, 0.0, 0.0, dtype=I.oracle_code(dtype))
-                if channels_last:
-                    ref = np.ascontiguousarray(ref.transpose(0, 2, 3, 1))
             view = np.uint32 if dtype == "fp32" else np.uint16
             assert y.shape == ref.shape
             assert np.array_equal(y.view(view), ref.view(view)), (mode, shape, sh, sw, dtype, channels_last)

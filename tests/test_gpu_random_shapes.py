@@ -3,6 +3,7 @@
 The enumerated tests pick shapes by hand around the kernels' size classes; this sweep draws them, so that tile
 edges, odd extents and class boundaries nobody thought of are met as well.  Every case prints its parameters first.
 """
+import os
 import sys
 
 import numpy as np
@@ -11,6 +12,9 @@ import pytest
 import inputs as I
 
 pytestmark = pytest.mark.gpu
+
+# the committed runs use the fixed seeds below; OPSCV_TEST_SEED shifts them all for an extra hunt
+SEED_SHIFT = int(os.environ.get("OPSCV_TEST_SEED", "0"))
 
 
 def _bits(a, dtype):
@@ -35,7 +39,7 @@ def _dims(rng, lo, hi, n):
 
 def test_random_grid_sampler2d(oracle, device, aclnn):
     import torch
-    rng = np.random.default_rng(9001)
+    rng = np.random.default_rng(9001 + SEED_SHIFT)
     for case in range(240):
         dtype = I.DTYPES[case % 3]
         N, C = _dims(rng, 1, 5, 1)[0], _dims(rng, 1, 40, 1)[0]
@@ -54,7 +58,7 @@ def test_random_grid_sampler2d(oracle, device, aclnn):
 def test_random_grid_sampler2d_large_planes(oracle, device, aclnn):
     """input planes from a few KB to beyond the largest LDS class (the direct kernel), few channels"""
     import torch
-    rng = np.random.default_rng(9004)
+    rng = np.random.default_rng(9004 + SEED_SHIFT)
     for case in range(45):
         dtype = I.DTYPES[case % 3]
         N, C = int(rng.integers(1, 3)), int(rng.integers(1, 7))
@@ -72,7 +76,7 @@ def test_random_grid_sampler2d_large_planes(oracle, device, aclnn):
 
 def test_random_resize_family(oracle, device, aclnn):
     import torch
-    rng = np.random.default_rng(9002)
+    rng = np.random.default_rng(9002 + SEED_SHIFT)
     for case in range(240):
         dtype = I.DTYPES[case % 3]
         N, C = _dims(rng, 1, 4, 1)[0], _dims(rng, 1, 70, 1)[0]
@@ -82,10 +86,10 @@ def test_random_resize_family(oracle, device, aclnn):
         _say("upsample", dtype, N, C, H, W, Ho, Wo, align, cl)
         x = I.cast_np(rng.standard_normal((N, C, H, W)).astype(np.float32), dtype)
         xin = np.ascontiguousarray(x.transpose(0, 2, 3, 1)) if cl else x
-        ref = oracle.resize_point_copy(xin, (Ho, Wo), align=align, dtype=I.oracle_code(dtype)) if cl else None
-        if ref is None:
+        if cl:
+            ref = oracle.upsample_bilinear2d_nhwc(xin, (Ho, Wo), align, dtype=I.oracle_code(dtype))
+        else:
             ref = oracle.upsample_bilinear2d(x, (Ho, Wo), align, dtype=I.oracle_code(dtype))
-            ref = np.ascontiguousarray(ref.transpose(0, 2, 3, 1)) if cl else ref
         y = aclnn.upsample_bilinear2d(I.to_torch(xin, dtype, device), (Ho, Wo), align, channels_last=cl)
         torch.cuda.synchronize()
         _same(I.from_torch(y, dtype), ref, dtype, (case, "up", dtype, N, C, H, W, Ho, Wo, align, cl))
@@ -114,7 +118,7 @@ def test_random_resize_family(oracle, device, aclnn):
 
 def test_random_sampler_backward_and_3d(oracle, device, aclnn):
     import torch
-    rng = np.random.default_rng(9003)
+    rng = np.random.default_rng(9003 + SEED_SHIFT)
     for case in range(150):
         dtype = I.DTYPES[case % 3]
         N, C = _dims(rng, 1, 3, 1)[0], _dims(rng, 1, 12, 1)[0]

@@ -698,3 +698,106 @@ def test_resize_point_copy_oracle(oracle):
     y = oracle.resize_point_copy(xi, (4, 5), align=False)
     gen = oracle.upsample_bilinear2d(np.ascontiguousarray(xi.transpose(0, 3, 1, 2)), (4, 5), False).transpose(0, 2, 3, 1)
     assert y[0, 0, 0, 0] == np.inf and np.isnan(gen[0, 0, 0, 0])
+
+
+# (input NHWC shape, output H W, dtype, align_corners, user scales h w, tiling key the reference's unit test expects)
+# image/resize_bilinear_v2/tests/ut/op_host/arch35/test_resize_bilinear_v2_tiling.cpp, the channels-last cases whose
+# attributes the upsample entry point can express (half_pixel_centers = !align_corners)
+NHWC_TILING_UT = [
+    ((2, 128, 128, 256), (192, 192), "fp32", True, (1.5, 1.5), 30000),                              # case04
+    ((128, 14, 16, 256), (5, 8), "fp32", False, (3.0, 3.0), 30000),                                 # case05
+    ((1, 36, 15, 128), (12, 5), "fp32", False, (0.0, 0.0), 40001),                                  # case07
+    ((1, 36, 15, 128), (12, 5), "fp32", False, (0.2, 0.2), 40001),                                  # case09
+    ((190, 22, 79, 128), (13, 43), "fp16", False, (0.31269457412229545, 0.27077088627767687), 10000),  # case10
+    ((1, 1, 1, 64), (59, 32), "fp32", True, (0.0, 0.0), 40003),                                     # case11
+    ((3, 11, 21, 5), (11, 21), "bf16", False, (0.0, 0.0), 40000),                                   # case16
+]
+NHWC_KEY_TEMPLATE = {30000: "per_element", 40001: "point_copy", 10000: "channel_parallel", 40003: "broadcast",
+                     40000: "copy"}
+
+
+def test_upsample_nhwc_oracle_templates(oracle):
+    """template choice for channels-last tensors against the tiling keys held by the reference's unit test"""
+    rng = np.random.default_rng(61)
+    for shape, out_hw, dtype, align, (sh, sw), key in NHWC_TILING_UT:
+        x = I.cast_np(rng.standard_normal(shape, dtype=np.float32), dtype)
+        _, template = oracle.upsample_bilinear2d_nhwc(x, out_hw, align, sh, sw, dtype=I.oracle_code(dtype),
+                                                      with_template=True)
+        assert template == NHWC_KEY_TEMPLATE[key], (shape, out_hw, dtype, align, sh, sw, key)
+    # without the user scales case10 shrinks by 22/13 along H: under two, so the per-element template
+    x = I.cast_np(rng.standard_normal((1, 22, 79, 128), dtype=np.float32), "fp16")
+    assert oracle.upsample_bilinear2d_nhwc(x, (13, 43), False, dtype=I.oracle_code("fp16"), with_template=True)[1] == \
+        "per_element"
+    # the 128-byte rule counts bytes: 32 fp32 channels take the template, 32 fp16 channels do not
+    x32 = rng.standard_normal((1, 8, 8, 32), dtype=np.float32)
+    assert oracle.upsample_bilinear2d_nhwc(x32, (3, 3), False, with_template=True)[1] == "channel_parallel"
+    assert oracle.upsample_bilinear2d_nhwc(x32.astype(np.float16), (3, 3), False, with_template=True)[1] == "per_element"
+    # a 1x1 source of short channel runs is interpolated with half-pixel centres and broadcast with align_corners
+    x1 = rng.standard_normal((1, 1, 1, 14), dtype=np.float32)
+    assert oracle.upsample_bilinear2d_nhwc(x1, (13, 7), False, with_template=True)[1] == "per_element"
+    assert oracle.upsample_bilinear2d_nhwc(x1, (13, 7), True, with_template=True)[1] == "broadcast"
+    # align_corners, 1x1 destination: first pixel for short runs; for long runs the scale is the whole source extent,
+    # which the point-copy template takes
+    assert oracle.upsample_bilinear2d_nhwc(x32[..., :8], (1, 1), True, with_template=True)[1] == "first_pixel"
+    assert oracle.upsample_bilinear2d_nhwc(x32, (1, 1), True, with_template=True)[1] == "point_copy"
+    assert oracle.upsample_bilinear2d_nhwc(x32, (1, 3), True, with_template=True)[1] == "channel_parallel"  # 8, 3.5
+
+
+def test_upsample_nhwc_oracle_arithmetic(oracle):
+    """the two interpolating templates of the channels-last resize: same taps, different order of operations"""
+    torch = pytest.importorskip("torch")
+    rng = np.random.default_rng(62)
+    # both against torch (different formula, so a tolerance) -- catches a wrong tap, stride or transposition
+    for shape, out_hw, align in [((2, 9, 14, 40), (4, 5), False), ((1, 23, 17, 33), (7, 8), True),
+                                 ((2, 9, 14, 8), (4, 5), False), ((1, 5, 6, 40), (11, 9), False)]:
+        x = rng.standard_normal(shape, dtype=np.float32)
+        y = oracle.upsample_bilinear2d_nhwc(x, out_hw, align)
+        ref = torch.nn.functional.interpolate(torch.from_numpy(x).permute(0, 3, 1, 2), size=out_hw, mode="bilinear",
+                                              align_corners=align).permute(0, 2, 3, 1).numpy()
+        assert np.max(np.abs(y - ref)) <= 1e-5, (shape, out_hw, align)
+    # the per-element template is the NCHW formula on transposed data
+    x = rng.standard_normal((2, 9, 14, 8), dtype=np.float32)
+    y, template = oracle.upsample_bilinear2d_nhwc(x, (4, 5), False, with_template=True)
+    assert template == "per_element"
+    nchw = oracle.upsample_bilinear2d(np.ascontiguousarray(x.transpose(0, 3, 1, 2)), (4, 5), False)
+    assert np.array_equal(y, nchw.transpose(0, 2, 3, 1))
+    # channel-parallel, one tap at a time: with a single non-zero source pixel the output pixel that touches it is
+    # value * (product of its two axis weights, rounded to fp32 first) -- the nested blends of the per-element
+    # template round value * (x weight) first, which gives other bits for weights that are not dyadic
+    Hs, Ws, Hd, Wd, C = 22, 31, 7, 9, 32
+    i0y, i1y, ly = oracle.upsample_axis_taps(Hs, Hd, False)
+    i0x, i1x, lx = oracle.upsample_axis_taps(Ws, Wd, False)
+    differs = 0
+    inner = [(h, w) for h in range(Hd) for w in range(Wd)
+             if i1y[h] == i0y[h] + 1 and i1x[w] == i0x[w] + 1 and 0 < ly[h] < 1 and 0 < lx[w] < 1]
+    assert len(inner) > 20
+    for h, w in inner[3::11]:
+        corners = {"nw": (i0y[h], i0x[w], (np.float32(1) - ly[h]) * (np.float32(1) - lx[w])),
+                   "ne": (i0y[h], i1x[w], (np.float32(1) - ly[h]) * lx[w]),
+                   "sw": (i1y[h], i0x[w], ly[h] * (np.float32(1) - lx[w])),
+                   "se": (i1y[h], i1x[w], ly[h] * lx[w])}
+        for name, (ys, xs, weight) in corners.items():
+            x = np.zeros((1, Hs, Ws, C), np.float32)
+            v = rng.standard_normal(C, dtype=np.float32)
+            x[0, ys, xs] = v
+            y, template = oracle.upsample_bilinear2d_nhwc(x, (Hd, Wd), False, with_template=True)
+            assert template == "channel_parallel"
+            assert weight.dtype == np.float32
+            assert np.array_equal(y[0, h, w], v * weight), (h, w, name)
+            nested = oracle.upsample_bilinear2d(np.ascontiguousarray(x.transpose(0, 3, 1, 2)), (Hd, Wd), False)
+            differs += int(not np.array_equal(nested[0, :, h, w], y[0, h, w]))
+            # 16-bit elements: the sum is formed in fp32 and rounded once
+            y16 = oracle.upsample_bilinear2d_nhwc(x.astype(np.float16)[..., :64].repeat(2, axis=3), (Hd, Wd), False)
+            v16 = x.astype(np.float16)[0, ys, xs].repeat(2).astype(np.float32)
+            assert np.array_equal(y16[0, h, w], (v16 * weight).astype(np.float16)), (h, w, name)
+    assert differs > 0
+    # dyadic weights and small integers: every product and sum is exact, so both templates give the exact value
+    x = rng.integers(-8, 9, (1, 10, 10, 32)).astype(np.float32)
+    y, template = oracle.upsample_bilinear2d_nhwc(x, (4, 4), False, with_template=True)   # scale 2.5: fractions .25 / .75
+    assert template == "channel_parallel"
+    pos = (np.arange(4) + 0.5) * 2.5 - 0.5
+    lo, fr = np.floor(pos).astype(int), pos - np.floor(pos)
+    x64 = x.astype(np.float64)
+    exact = ((1 - fr)[:, None, None] * ((1 - fr)[None, :, None] * x64[0, lo][:, lo] + fr[None, :, None] * x64[0, lo][:, lo + 1]) +
+             fr[:, None, None] * ((1 - fr)[None, :, None] * x64[0, lo + 1][:, lo] + fr[None, :, None] * x64[0, lo + 1][:, lo + 1]))
+    assert np.array_equal(y[0].astype(np.float64), exact)
