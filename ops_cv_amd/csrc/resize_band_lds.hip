@@ -103,6 +103,7 @@ BandPlan make_plan(const ResizeArgs& a)
     bp.p.lds_rows = rows;
     bp.p.gran = gran;
     bp.p.neg_zero = -0.0f;
+    bp.p.raw_lambda = a.raw_lambda;
     bp.p.streaming = (a.N * a.C * a.Hd * a.Wd * (int64_t)sizeof(T) >= kStreamingBytes) ? 1 : 0;
     bp.lds_bytes = (uint32_t)bytes;
     bp.grid = dim3((unsigned)cblocks, (unsigned)bands, (unsigned)(planes < 65535 ? planes : 65535));
@@ -197,6 +198,7 @@ FlatPlan make_flat_plan(const ResizeArgs& a)
     fp.p.rg = rg;
     fp.p.gran = gran;
     fp.p.neg_zero = -0.0f;
+    fp.p.raw_lambda = a.raw_lambda;
     fp.lds_bytes = (uint32_t)(((int64_t)rows * a.Ws * (int64_t)sizeof(T) + 15) / 16 * 16);
     fp.grid = dim3((unsigned)bands, (unsigned)(planes < 65535 ? planes : 65535));
     const char* v = getenv("OPSCV_RESIZE_VARIANT");

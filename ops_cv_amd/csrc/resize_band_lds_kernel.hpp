@@ -36,6 +36,7 @@ struct BandLdsParams {
     int32_t lds_rows;   // staged rows the LDS allocation holds
     int32_t gran;       // bytes per lane of the asynchronous copy: 16 or 4
     int32_t streaming;  // 1: mark the output stores non-temporal (outputs much larger than the caches)
+    int32_t raw_lambda;  // fraction from the unclamped source coordinate (see axis_tap)
     float neg_zero;     // -0.0f, passed in so that fma(v, w, -0) is not folded back into a multiply
 };
 
@@ -75,7 +76,7 @@ __global__ __launch_bounds__(THREADS) void resize_band_lds_kernel(const T* __res
     for (int i = 0; i < V; i++) {
         int32_t c = col0 + i;
         c = (c < p.Wd) ? c : p.Wd - 1;
-        const AxisTap t = axis_tap<HALF_PIXEL>(c, p.scale_w, p.Ws);
+        const AxisTap t = axis_tap<HALF_PIXEL>(c, p.scale_w, p.Ws, p.raw_lambda);
         to0[i] = (uint32_t)(t.i0 - seg_col0) * (uint32_t)sizeof(T);
         to1[i] = (uint32_t)(t.i1 - seg_col0) * (uint32_t)sizeof(T);
         dx[i] = t.lambda;
@@ -87,7 +88,7 @@ __global__ __launch_bounds__(THREADS) void resize_band_lds_kernel(const T* __res
     {
         int32_t h = h_begin + lane;
         h = (h < p.Hd) ? h : p.Hd - 1;
-        const AxisTap t = axis_tap<HALF_PIXEL>(h, p.scale_h, p.Hs);
+        const AxisTap t = axis_tap<HALF_PIXEL>(h, p.scale_h, p.Hs, p.raw_lambda);
         my_y0 = t.i0 - ys_lo;
         my_y1 = t.i1 - ys_lo;
         my_dy = t.lambda;

@@ -28,6 +28,7 @@ struct FlatLdsParams {
     int32_t cl;         // column lanes = Wd / V
     int32_t rg;         // row groups = THREADS / cl
     int32_t gran;       // bytes per lane of the asynchronous copy: 16 or 4
+    int32_t raw_lambda;  // fraction from the unclamped source coordinate (see axis_tap)
     float neg_zero;     // -0.0f, passed in so that fma(v, w, -0) is not folded back into a multiply
 };
 
@@ -62,7 +63,7 @@ __global__ __launch_bounds__(THREADS) void resize_flat_lds_kernel(const T* __res
     for (int i = 0; i < V; i++) {
         int32_t c = col0 + i;
         c = (c < p.Wd) ? c : p.Wd - 1;
-        const AxisTap t = axis_tap<HALF_PIXEL>(c, p.scale_w, p.Ws);
+        const AxisTap t = axis_tap<HALF_PIXEL>(c, p.scale_w, p.Ws, p.raw_lambda);
         to0[i] = (uint32_t)t.i0 * (uint32_t)sizeof(T);
         to1[i] = (uint32_t)t.i1 * (uint32_t)sizeof(T);
         dx[i] = t.lambda;
@@ -94,7 +95,7 @@ __global__ __launch_bounds__(THREADS) void resize_flat_lds_kernel(const T* __res
         const __amdgpu_buffer_rsrc_t rsrc =
             __builtin_amdgcn_make_buffer_rsrc(y + pl * (int64_t)p.Hd * p.Wd, 0, out_plane_bytes, kRsBufferFlags);
         for (int32_t h = active ? h_begin + group : h_end; h < h_end; h += p.rg) {
-            const AxisTap t = axis_tap<HALF_PIXEL>(h, p.scale_h, p.Hs);
+            const AxisTap t = axis_tap<HALF_PIXEL>(h, p.scale_h, p.Hs, p.raw_lambda);
             const char* r0 = lds + (uint32_t)(t.i0 - ys_lo) * src_row_bytes;
             const char* r1 = lds + (uint32_t)(t.i1 - ys_lo) * src_row_bytes;
             T tl[V], tr[V], bl[V], br[V];

@@ -38,19 +38,19 @@ template <typename T, bool HALF_PIXEL>
 __global__ __launch_bounds__(kThreads) void resize_nchw_generic_kernel(const T* __restrict__ x, T* __restrict__ y,
                                                                         int64_t planes, int32_t Hs, int32_t Ws,
                                                                         int32_t Hd, int32_t Wd, float scale_h,
-                                                                        float scale_w)
+                                                                        float scale_w, int raw_lambda)
 {
     const int64_t rows = planes * Hd;
     const int32_t w = blockIdx.x * kThreads + threadIdx.x;
     if (w >= Wd) {
         return;
     }
-    const AxisTap tx = axis_tap<HALF_PIXEL>(w, scale_w, Ws);
+    const AxisTap tx = axis_tap<HALF_PIXEL>(w, scale_w, Ws, raw_lambda);
     const float dx = tx.lambda;
     for (int64_t r = blockIdx.y; r < rows; r += gridDim.y) {
         const int64_t pl = r / Hd;
         const int32_t h = (int32_t)(r - pl * Hd);
-        const AxisTap ty = axis_tap<HALF_PIXEL>(h, scale_h, Hs);
+        const AxisTap ty = axis_tap<HALF_PIXEL>(h, scale_h, Hs, raw_lambda);
         const float dy = ty.lambda;
         const T* top = x + (pl * Hs + ty.i0) * (int64_t)Ws;
         const T* bot = x + (pl * Hs + ty.i1) * (int64_t)Ws;
@@ -76,7 +76,7 @@ template <typename T, bool HALF_PIXEL, int BAND>
 __global__ __launch_bounds__(kThreads) void resize_nchw_band_kernel(const T* __restrict__ x, T* __restrict__ y,
                                                                      int64_t planes, int32_t Hs, int32_t Ws,
                                                                      int32_t Hd, int32_t Wd, float scale_h,
-                                                                     float scale_w)
+                                                                     float scale_w, int raw_lambda)
 {
     constexpr int V = 16 / (int)sizeof(T);
     const int32_t chunk = blockIdx.x * kThreads + threadIdx.x;
@@ -88,7 +88,7 @@ __global__ __launch_bounds__(kThreads) void resize_nchw_band_kernel(const T* __r
     float dx[V];
 #pragma unroll
     for (int i = 0; i < V; i++) {
-        const AxisTap t = axis_tap<HALF_PIXEL>(col0 + i, scale_w, Ws);
+        const AxisTap t = axis_tap<HALF_PIXEL>(col0 + i, scale_w, Ws, raw_lambda);
         xo0[i] = t.i0;
         xo1[i] = t.i1;
         dx[i] = t.lambda;
@@ -111,7 +111,7 @@ __global__ __launch_bounds__(kThreads) void resize_nchw_band_kernel(const T* __r
             }
         };
         for (int32_t h = h_begin; h < h_end; h++) {
-            const AxisTap ty = axis_tap<HALF_PIXEL>(h, scale_h, Hs);
+            const AxisTap ty = axis_tap<HALF_PIXEL>(h, scale_h, Hs, raw_lambda);
             const int32_t y0 = __builtin_amdgcn_readfirstlane(ty.i0);
             const int32_t y1 = __builtin_amdgcn_readfirstlane(ty.i1);
             const float dy = ty.lambda;
@@ -785,11 +785,11 @@ hipError_t run_resize(const ResizeArgs& a, hipStream_t stream)
         if (a.half_pixel) {
             hipLaunchKernelGGL((resize_nchw_band_kernel<T, true, kBand>), grid, dim3(kThreads), 0, stream, x, y,
                                planes, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h,
-                               a.scale_w);
+                               a.scale_w, a.raw_lambda);
         } else {
             hipLaunchKernelGGL((resize_nchw_band_kernel<T, false, kBand>), grid, dim3(kThreads), 0, stream, x, y,
                                planes, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h,
-                               a.scale_w);
+                               a.scale_w, a.raw_lambda);
         }
         return hipGetLastError();
     }
@@ -797,10 +797,12 @@ hipError_t run_resize(const ResizeArgs& a, hipStream_t stream)
     dim3 grid((unsigned)((a.Wd + kThreads - 1) / kThreads), (unsigned)(rows < 65535 ? rows : 65535));
     if (a.half_pixel) {
         hipLaunchKernelGGL((resize_nchw_generic_kernel<T, true>), grid, dim3(kThreads), 0, stream, x, y, planes,
-                           (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h, a.scale_w);
+                           (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h, a.scale_w,
+                           a.raw_lambda);
     } else {
         hipLaunchKernelGGL((resize_nchw_generic_kernel<T, false>), grid, dim3(kThreads), 0, stream, x, y, planes,
-                           (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h, a.scale_w);
+                           (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h, a.scale_w,
+                           a.raw_lambda);
     }
     return hipGetLastError();
 }

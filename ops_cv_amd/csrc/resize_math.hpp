@@ -13,9 +13,17 @@ struct AxisTap {
     float lambda;
 };
 
-// image/resize_bilinear_v2/op_kernel/arch35/resize_bilinear_v2_simt_nchw.h:108-134 for one axis
+// image/resize_bilinear_v2/op_kernel/arch35/resize_bilinear_v2_simt_nchw.h:108-134 for one axis.
+//
+// raw_lambda selects the arithmetic of the reference's template for large outputs
+// (image/resize_bilinear_v2/op_kernel/arch35/resize_bilinear_v2_simt_hw.h:79-86): it does not clamp the source
+// coordinate at zero before taking the fraction, so the first rows and columns of a half-pixel upscale (coordinate
+// in [-0.5, 0)) blend the border pixel with itself, (1-l)*v + l*v with l = coordinate + 1, instead of passing it
+// through with l = 0.  Its taps are the same: floor and ceil converted to an unsigned index and capped at size-1,
+// a negative floor taken as index 0 (the conversion is undefined in C++; zero is what the clamp the reference
+// writes around it intends).
 template <bool HALF_PIXEL>
-__host__ __device__ __forceinline__ AxisTap axis_tap(int32_t d, float scale, int32_t len_src)
+__host__ __device__ __forceinline__ AxisTap axis_tap(int32_t d, float scale, int32_t len_src, int raw_lambda = 0)
 {
     float orig;
     if (HALF_PIXEL) {
@@ -23,6 +31,7 @@ __host__ __device__ __forceinline__ AxisTap axis_tap(int32_t d, float scale, int
     } else {
         orig = (float)d * scale;
     }
+    const float raw = orig;
     if (orig < 0.0f) {
         orig = 0.0f;
     }
@@ -34,6 +43,9 @@ __host__ __device__ __forceinline__ AxisTap axis_tap(int32_t d, float scale, int
     t.i0 = (lo < last) ? (int32_t)lo : len_src - 1;
     t.i1 = (hi < last) ? (int32_t)hi : len_src - 1;
     t.lambda = orig - fl;
+    if (HALF_PIXEL && raw_lambda != 0) {
+        t.lambda = raw - __builtin_floorf(raw);
+    }
     return t;
 }
 

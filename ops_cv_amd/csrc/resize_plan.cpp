@@ -2,6 +2,8 @@
 
 #include <cfloat>
 #include <cmath>
+#include <cstdint>
+#include <cstdlib>
 
 namespace opscv {
 
@@ -74,6 +76,29 @@ void plan_resize(ResizeArgs* a, bool align_corners, float user_scale_h, float us
     } else if (one_dst && align_corners) {
         a->mode = ResizeMode::FirstPixel;
     }
+    // resize_bilinear_v2_tiling_arch35.cpp:592-595,606-615: NCHW outputs of at least cores * 1024 pixels (cores * 512
+    // when a tensor needs 64-bit indices) go to the template that splits H*W over the cores; it takes the fraction from
+    // the unclamped source coordinate (see axis_tap), which only differs with half-pixel centres
+    a->raw_lambda = 0;
+    if (a->mode == ResizeMode::Bilinear && !a->channels_last && a->half_pixel) {
+        const int64_t x_elems = a->N * a->C * a->Hs * a->Ws, y_elems = a->N * a->C * a->Hd * a->Wd;
+        const bool idx32 = y_elems < (int64_t)UINT32_MAX && x_elems < (int64_t)UINT32_MAX;
+        const int64_t threshold = reference_vector_cores() * (idx32 ? 1024 : 512);
+        if (x_elems != 1 && a->Hd * a->Wd >= threshold) {
+            a->raw_lambda = 1;
+        }
+    }
+}
+
+int64_t reference_vector_cores()
+{
+    if (const char* v = getenv("OPSCV_REFERENCE_CORES")) {
+        const long n = strtol(v, nullptr, 10);
+        if (n > 0) {
+            return n;
+        }
+    }
+    return 64;  // the core count of the reference's tiling unit test (test_resize_bilinear_v2_tiling.cpp: {64, 245760})
 }
 
 void plan_resize_nearest(ResizeArgs* a)

@@ -14,6 +14,11 @@ float resize_axis_scale(int64_t len_src, int64_t len_dst, bool align_corners, fl
 // image/resize_bilinear_v2/op_kernel/resize_bilinear_v2_apt.cpp:91-140.
 void plan_resize(ResizeArgs* a, bool align_corners, float user_scale_h, float user_scale_w);
 
+// Vector cores of the device the reference would run on.  Its choice between the per-plane and the H*W-split NCHW
+// template depends on that number (resize_bilinear_v2_tiling_arch35.cpp:606-609,877), and the two templates differ in
+// the border pixels of fp32 half-pixel upscales.  OPSCV_REFERENCE_CORES overrides the default of 64.
+int64_t reference_vector_cores();
+
 // Nearest-neighbour resize with align_corners = false and half_pixel_centers = false, the only combination
 // aclnnResize requests (image/resize_bilinear_v2/op_api/aclnn_resize.cpp:286-288): scale = in / out
 // (image/resize_nearest_neighbor_v2/op_host/arch35/resize_nearest_neighbor_v2_tiling_base.cpp:253-263).

@@ -573,6 +573,42 @@ static inline void axis_tap(int64_t d, float scale, int half_pixel, int64_t len_
     *lambda = orig - fl;
 }
 
+/* The template for large NCHW outputs, one axis: resize_bilinear_v2_simt_hw.h:76-86.  The coordinate is not clamped at
+ * zero before the fraction is taken.  floor and ceil are converted to the unsigned index type and capped at
+ * len_src - 1; for the coordinates in [-0.5, 0) that half-pixel centres produce the floor is -1, whose conversion to
+ * unsigned the language leaves undefined: taken as index 0, which is what the max(..., 0) written around it intends
+ * (ceil is -0 -> 0 there). */
+static inline void axis_tap_hw(int64_t d, float scale, int half_pixel, int64_t len_src, int32_t* i0, int32_t* i1,
+                               float* lambda)
+{
+    const float offset = half_pixel ? 0.5f : 0.0f;
+    const float orig = ((float)d + offset) * scale - offset;
+    const float fl = floorf(orig), ce = ceilf(orig);
+    const float last = (float)(len_src - 1);
+    *i0 = (int32_t)((fl < 0.0f) ? 0 : ((fl < last) ? (int64_t)fl : len_src - 1));
+    *i1 = (int32_t)((ce < 0.0f) ? 0 : ((ce < last) ? (int64_t)ce : len_src - 1));
+    *lambda = orig - fl;
+}
+
+static int64_t g_reference_cores = 64;
+
+/* Vector cores of the device the reference would run on (64 in the compile info of its tiling unit test); the NCHW
+ * template choice depends on it: resize_bilinear_v2_tiling_arch35.cpp:606-615,877 */
+void oracle_set_reference_cores(int64_t cores)
+{
+    g_reference_cores = cores > 0 ? cores : 64;
+}
+
+/* resize_bilinear_v2_tiling_arch35.cpp:592-595,606-615: 1 when the H*W-split template is chosen for an NCHW resize
+ * that reached the interpolating templates */
+int oracle_resize_uses_hw_split(int64_t N, int64_t C, int64_t Hs, int64_t Ws, int64_t Hd, int64_t Wd)
+{
+    const int64_t x_elems = N * C * Hs * Ws, y_elems = N * C * Hd * Wd;
+    const int idx32 = y_elems < (int64_t)UINT32_MAX && x_elems < (int64_t)UINT32_MAX;
+    const int64_t threshold = g_reference_cores * (idx32 ? 1024 : 512);
+    return x_elems != 1 && (Ws != Wd || Hs != Hd) && Hd * Wd >= threshold;
+}
+
 int oracle_upsample_axis_taps(int64_t len_src, int64_t len_dst, int align_corners, float user_scale, int32_t* i0,
                               int32_t* i1, float* lambda)
 {
@@ -630,6 +666,7 @@ int oracle_upsample_bilinear2d(const void* x, void* y, int dtype, int64_t N, int
     const float scale_w = oracle_resize_scale(Ws, Wd, align_corners, (float)scales_w);
     const int half_pixel = !align_corners;
     const int64_t rows = planes * Hd;
+    const int hw_split = oracle_resize_uses_hw_split(N, C, Hs, Ws, Hd, Wd);
 #ifdef _OPENMP
 #pragma omp parallel for schedule(static) num_threads(num_threads)
 #endif
@@ -638,17 +675,25 @@ int oracle_upsample_bilinear2d(const void* x, void* y, int dtype, int64_t N, int
         int64_t h = r - pl * Hd;
         int32_t top, bottom;
         float dy;
-        axis_tap(h, scale_h, half_pixel, Hs, &top, &bottom, &dy);
+        if (hw_split) {
+            axis_tap_hw(h, scale_h, half_pixel, Hs, &top, &bottom, &dy);
+        } else {
+            axis_tap(h, scale_h, half_pixel, Hs, &top, &bottom, &dy);
+        }
         const int64_t base = pl * Hs * Ws;
         for (int64_t w = 0; w < Wd; w++) {
             int32_t left, right;
             float dx;
-            axis_tap(w, scale_w, half_pixel, Ws, &left, &right, &dx);
+            if (hw_split) {
+                axis_tap_hw(w, scale_w, half_pixel, Ws, &left, &right, &dx);
+            } else {
+                axis_tap(w, scale_w, half_pixel, Ws, &left, &right, &dx);
+            }
             float tl = load_as_float(x, dtype, base + (int64_t)top * Ws + left);
             float tr = load_as_float(x, dtype, base + (int64_t)top * Ws + right);
             float bl = load_as_float(x, dtype, base + (int64_t)bottom * Ws + left);
             float br = load_as_float(x, dtype, base + (int64_t)bottom * Ws + right);
-            /* resize_bilinear_v2_simt_nchw.h:143-144 */
+            /* resize_bilinear_v2_simt_nchw.h:143-144 and resize_bilinear_v2_simt_hw.h:96-97 */
             float out = (1.0f - dy) * ((1.0f - dx) * tl + dx * tr) + dy * ((1.0f - dx) * bl + dx * br);
             store_from_float(y, dtype, r * Wd + w, out);
         }

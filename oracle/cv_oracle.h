@@ -85,6 +85,17 @@ int oracle_grid_sampler2d_taps(const void* grid, oracle_gs_tap* taps, int dtype,
 /* scale handed to the kernel for one axis (align_corners / user scale / size ratio) */
 float oracle_resize_scale(int64_t len_src, int64_t len_dst, int align_corners, float user_scale);
 
+/*
+ * The reference picks between two NCHW interpolating templates by the output size and the number of vector cores of
+ * its device (image/resize_bilinear_v2/op_host/arch35/resize_bilinear_v2_tiling_arch35.cpp:606-615): from
+ * cores * 1024 output pixels per plane on, the H*W-split template
+ * (image/resize_bilinear_v2/op_kernel/arch35/resize_bilinear_v2_simt_hw.h:76-97), which takes the fraction from the
+ * unclamped source coordinate.  oracle_set_reference_cores sets the core count (default 64, that of the reference's
+ * tiling unit test); oracle_resize_uses_hw_split tells which template oracle_upsample_bilinear2d restates for a shape.
+ */
+void oracle_set_reference_cores(int64_t cores);
+int oracle_resize_uses_hw_split(int64_t N, int64_t C, int64_t Hs, int64_t Ws, int64_t Hd, int64_t Wd);
+
 /* scales_h / scales_w are the user-facing multipliers (0 = derive from sizes) */
 int oracle_upsample_bilinear2d(const void* x, void* y, int dtype, int64_t N, int64_t C, int64_t Hs, int64_t Ws,
                                int64_t Hd, int64_t Wd, int align_corners, double scales_h, double scales_w,

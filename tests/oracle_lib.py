@@ -98,6 +98,10 @@ def lib():
     L.oracle_gs3d_clip.argtypes = [f32, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32]
     L.oracle_grid_sampler2d_backward.restype = ctypes.c_int
     L.oracle_grid_sampler2d_backward.argtypes = [vp] * 5 + [ctypes.c_int] + [i64] * 6 + [ctypes.c_int] * 3
+    L.oracle_set_reference_cores.restype = None
+    L.oracle_set_reference_cores.argtypes = [i64]
+    L.oracle_resize_uses_hw_split.restype = ctypes.c_int
+    L.oracle_resize_uses_hw_split.argtypes = [i64] * 6
     L.oracle_upsample_bilinear2d_nhwc.restype = ctypes.c_int
     L.oracle_upsample_bilinear2d_nhwc.argtypes = [vp, vp, ctypes.c_int] + [i64] * 6 + [ctypes.c_int, ctypes.c_double,
                                                                                          ctypes.c_double]
@@ -255,6 +259,15 @@ def upsample_bilinear2d(x, out_hw, align=False, scales_h=0.0, scales_w=0.0, dtyp
     if rc != 0:
         raise ValueError("oracle_upsample_bilinear2d rc=%d" % rc)
     return y
+
+
+def set_reference_cores(cores):
+    """vector cores of the device the reference would run on (its NCHW template choice depends on it); 0 -> default"""
+    lib().oracle_set_reference_cores(int(cores))
+
+
+def resize_uses_hw_split(N, C, Hs, Ws, Hd, Wd):
+    return bool(lib().oracle_resize_uses_hw_split(N, C, Hs, Ws, Hd, Wd))
 
 
 NHWC_TEMPLATES = ("per_element", "copy", "broadcast", "first_pixel", "point_copy", "channel_parallel")

@@ -187,3 +187,38 @@ def test_upsample_user_scales(oracle, device, dtype):
     for out_hw, sh, sw in [((20, 24), 2.0, 2.0), ((25, 18), 2.5, 1.5), ((15, 30), 1.7, 2.4)]:
         y, y_ref = _run_up(oracle, device, x32, out_hw, dtype, False, sh, sw)
         _check(y, y_ref, dtype, 0, "up-scales %s %s" % (dtype, out_hw))
+
+
+@pytest.mark.parametrize("dtype", I.DTYPES)
+def test_upsample_hw_split_template(oracle, device, dtype, monkeypatch):
+    """the reference's NCHW template for large outputs (fraction from the unclamped coordinate), reached at small
+    sizes by telling library and oracle that the reference device has one vector core; every NCHW kernel variant"""
+    from ops_cv_amd import aclnn
+    rng = np.random.default_rng(70)
+    cases = [((1, 2, 56, 56), (112, 112), 0, 0), ((1, 1, 33, 65), (67, 200), 0, 0), ((1, 3, 64, 32), (200, 64), 0, 0),
+             ((1, 1, 700, 8), (1400, 16), 0, 0), ((2, 2, 20, 300), (47, 1031), 0, 0), ((1, 2, 16, 600), (40, 1536), 0, 0),
+             ((2, 3, 30, 36), (75, 54), 2.5, 1.5), ((1, 2, 40, 40), (24, 48), 0, 0)]
+    monkeypatch.setenv("OPSCV_REFERENCE_CORES", "1")
+    differs = 0
+    try:
+        for forced in ("", "b", "r", "g"):
+            monkeypatch.setenv("OPSCV_RESIZE_VARIANT", forced)
+            for shape, out_hw, sh, sw in cases:
+                x32 = rng.standard_normal(shape).astype(np.float32)
+                oracle.set_reference_cores(1)
+                assert oracle.resize_uses_hw_split(*shape, *out_hw)
+                y, y_ref = _run_up(oracle, device, x32, out_hw, dtype, False, sh, sw)
+                bits = np.uint32 if dtype == "fp32" else np.uint16
+                assert np.array_equal(y.view(bits), y_ref.view(bits)), (dtype, forced, shape, out_hw)
+                oracle.set_reference_cores(64)
+                plain = oracle.upsample_bilinear2d(I.cast_np(x32, dtype), out_hw, False, sh, sw, dtype=I.oracle_code(dtype))
+                differs += int(not np.array_equal(plain.view(bits), y_ref.view(bits)))
+        # align_corners never has a negative coordinate: both templates agree
+        oracle.set_reference_cores(1)
+        x32 = rng.standard_normal((1, 2, 56, 56)).astype(np.float32)
+        y, y_ref = _run_up(oracle, device, x32, (112, 112), dtype, True)
+        assert np.array_equal(y, y_ref)
+    finally:
+        oracle.set_reference_cores(0)
+    # the test would be vacuous if the two templates agreed on these inputs (16-bit results mostly round back)
+    assert differs > 0 or dtype != "fp32"

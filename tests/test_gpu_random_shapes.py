@@ -74,9 +74,19 @@ def test_random_grid_sampler2d_large_planes(oracle, device, aclnn):
         _same(I.from_torch(y, dtype), ref, dtype, (case, dtype, N, C, H, W, Ho, Wo, interp, pad, align))
 
 
-def test_random_resize_family(oracle, device, aclnn):
+def test_random_resize_family(oracle, device, aclnn, monkeypatch):
     import torch
     rng = np.random.default_rng(9002 + SEED_SHIFT)
+    # the reference picks its NCHW template by output pixels against cores * 1024: four cores put both templates in reach
+    monkeypatch.setenv("OPSCV_REFERENCE_CORES", "4")
+    oracle.set_reference_cores(4)
+    try:
+        _random_resize_family(oracle, device, aclnn, torch, rng)
+    finally:
+        oracle.set_reference_cores(0)
+
+
+def _random_resize_family(oracle, device, aclnn, torch, rng):
     for case in range(240):
         dtype = I.DTYPES[case % 3]
         N, C = _dims(rng, 1, 4, 1)[0], _dims(rng, 1, 70, 1)[0]

@@ -801,3 +801,60 @@ def test_upsample_nhwc_oracle_arithmetic(oracle):
     exact = ((1 - fr)[:, None, None] * ((1 - fr)[None, :, None] * x64[0, lo][:, lo] + fr[None, :, None] * x64[0, lo][:, lo + 1]) +
              fr[:, None, None] * ((1 - fr)[None, :, None] * x64[0, lo + 1][:, lo] + fr[None, :, None] * x64[0, lo + 1][:, lo + 1]))
     assert np.array_equal(y[0].astype(np.float64), exact)
+
+
+def test_upsample_hw_split_template(oracle):
+    """the reference's template for large NCHW outputs (resize_bilinear_v2_simt_hw.h): chosen by output size and core
+    count as its tiling unit test expects, equal to the per-plane template wherever the source coordinate is not
+    negative, and a self-blend of the border pixel where it is"""
+    # test_resize_bilinear_v2_tiling.cpp, 64 cores: case01 -> 30001, case02 -> 30001, case06 -> 30004, case14 -> 30005
+    assert not oracle.resize_uses_hw_split(2, 256, 12, 12, 18, 18)
+    assert not oracle.resize_uses_hw_split(2, 256, 128, 128, 192, 192)
+    assert oracle.resize_uses_hw_split(10, 10, 10, 10, 64, 1024)
+    assert oracle.resize_uses_hw_split(12768, 10, 128, 256, 128, 1024)
+    assert not oracle.resize_uses_hw_split(10, 10, 10, 10, 64, 1023)          # one column short of 64 * 1024
+    assert oracle.resize_uses_hw_split(12768, 10, 128, 256, 48, 1024)          # 64-bit indices: from 64 * 512 on
+    assert not oracle.resize_uses_hw_split(12768, 10, 128, 256, 32, 1024)      # fits 32-bit indices: from 64 * 1024 on
+    rng = np.random.default_rng(71)
+    x = rng.standard_normal((2, 3, 16, 20), dtype=np.float32)
+    moved = 0
+    try:
+        for out_hw, align in [((32, 40), False), ((40, 52), False), ((32, 40), True), ((9, 120), False)]:
+            oracle.set_reference_cores(64)
+            assert not oracle.resize_uses_hw_split(2, 3, 16, 20, *out_hw)
+            plain = oracle.upsample_bilinear2d(x, out_hw, align)
+            oracle.set_reference_cores(1)
+            assert oracle.resize_uses_hw_split(2, 3, 16, 20, *out_hw)
+            split = oracle.upsample_bilinear2d(x, out_hw, align)
+            i0y, _, _ = oracle.upsample_axis_taps(16, out_hw[0], align)
+            if align:
+                assert np.array_equal(plain, split)        # coordinates are never negative
+                continue
+            # rows / columns whose source coordinate is negative: (d + 0.5) * scale < 0.5
+            neg_r = np.array([(d + 0.5) * (16 / out_hw[0]) < 0.5 for d in range(out_hw[0])])
+            neg_c = np.array([(d + 0.5) * (20 / out_hw[1]) < 0.5 for d in range(out_hw[1])])
+            inner = ~neg_r[:, None] & ~neg_c[None, :]
+            assert neg_r.any() or neg_c.any()
+            assert np.array_equal(plain[:, :, inner], split[:, :, inner])
+            # on the border both taps of that axis are the same pixel; blending it with itself moves an fp32 value by
+            # a rounding error or two of the values involved
+            border = ~inner
+            d = np.abs(plain[:, :, border].astype(np.float64) - split[:, :, border])
+            assert d.max() <= 2.0 ** -22 * np.abs(x).max(), d.max()
+            moved += int(d.max() > 0)
+            # 16-bit elements: where both coordinates are negative the corner pixel is blended with itself in fp32
+            # and rounds back to itself
+            x16 = x.astype(np.float16)
+            s16 = oracle.upsample_bilinear2d(x16, out_hw, align)
+            corner = neg_r[:, None] & neg_c[None, :]
+            if corner.any():   # the case that shrinks along H has no such rows
+                assert np.array_equal(s16[:, :, corner], np.repeat(x16[:, :, :1, 0], corner.sum(), axis=2))
+        assert moved >= 1   # fractions that are not dyadic (0.7 at a scale of 0.4) do move values
+        # the corner pixel of a x2 upscale: coordinate -0.25 on both axes, fraction 0.75; values with short mantissas
+        # come through exactly (0.25 v and 0.75 v are exact), 1 + 2^-23 + ... need not
+        oracle.set_reference_cores(1)
+        xs = np.zeros((1, 1, 16, 32), np.float32)
+        xs[0, 0, 0, 0] = 1.3125
+        assert oracle.upsample_bilinear2d(xs, (32, 64), False)[0, 0, 0, 0] == np.float32(1.3125)
+    finally:
+        oracle.set_reference_cores(0)
