@@ -12,6 +12,8 @@
 // the result does not depend on scheduling.  The translation unit is compiled with -ffp-contract=off.
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
 #include "kernels.hpp"
 #include "sampler_math.hpp"
 
@@ -208,23 +210,25 @@ __device__ __forceinline__ float visit_sum(const TI* base, int32_t pitch, int32_
 // The same sum with the column part of the loop taken out: a lane keeps the weights of the (at most KX) columns it
 // visits -- computed once, by the same repeated additions -- and a row costs one LDS read, two products and an add
 // per column.  Column k of a lane with fewer than k + 1 visits leaves the sum alone.
-template <typename TI, int KX>
+template <typename TI, int KX, int KMIN>
 __device__ __forceinline__ float visit_sum_fixed(const TI* tile_xy, int32_t pitch, int32_t y0, int32_t in_y_start,
-                                                 int32_t nx, const float (&xl)[KX], float out_y_start, float fh,
+                                                 int32_t nx, const float* xl, float out_y_start, float fh,
                                                  float scale_h, float last_y, int32_t Hd, float neg_zero)
 {
     float acc = 0.0f;
     float out_y = out_y_start;
     for (int32_t in_y = in_y_start; out_y < fh + 1.0f && in_y < Hd; in_y++) {
-        const float yc = __builtin_fmaxf(0.0f, __builtin_fminf(out_y, last_y));
+        // max(0, min(out_y, last_y)) as one median: out_y is never a NaN
+        const float yc = __builtin_amdgcn_fmed3f(out_y, 0.0f, last_y);
         const float y_lerp = 1.0f - __builtin_fabsf(yc - fh);
         const TI* row = tile_xy + (in_y - y0) * pitch;
 #pragma unroll
         for (int k = 0; k < KX; k++) {
             // fma(g, w, -0) is g * w bit for bit and lets a 16-bit element be converted by the multiply itself; the
-            // read of a column past the lane's last one may fetch anything (it stays inside LDS) and is dropped
+            // read of a column past the lane's last one may fetch anything (it stays inside LDS) and is dropped.
+            // Every lane of the workgroup visits at least KMIN columns: those need no test.
             const float t = __builtin_fmaf(ElemIO<TI>::load(row + k), y_lerp, neg_zero) * xl[k];
-            acc = (k < nx) ? acc + t : acc;
+            acc = (k < KMIN || k < nx) ? acc + t : acc;
         }
         out_y += scale_h;
     }
@@ -232,6 +236,7 @@ __device__ __forceinline__ float visit_sum_fixed(const TI* tile_xy, int32_t pitc
 }
 
 constexpr int kTileCols = 128;
+constexpr int32_t kGradCapWords = 12288;  // at most 48 KB of LDS per workgroup (fp32 words, one per tile element)
 constexpr int kTileGroups = kGradThreads / kTileCols;  // row groups of a workgroup
 
 template <typename TI, typename TO, bool HALF_PIXEL>
@@ -243,8 +248,8 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
                                                                         int32_t cap_words, float neg_zero)
 {
     constexpr int EPW = 4 / (int)sizeof(TI);  // elements per 4-byte word
-    extern __shared__ uint32_t tile_words[];
-    __shared__ int32_t s_x1, s_y1, s_nx;
+    extern __shared__ __attribute__((aligned(16))) uint32_t tile_words[];
+    __shared__ int32_t s_x1, s_y1, s_nx, s_nx_min;
     const int tx = threadIdx.x % kTileCols, ty = threadIdx.x / kTileCols;
     const int32_t W0 = blockIdx.x * kTileCols, H0 = blockIdx.y * tile_rows;
     const float offset = HALF_PIXEL ? 0.5f : 0.0f;
@@ -271,14 +276,31 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
         s_x1 = 0;
         s_y1 = 0;
         s_nx = 0;
+        s_nx_min = INT32_MAX;
     }
     __syncthreads();
     int32_t nx = 0;
-    if (col_ok) {
-        const int32_t x_end = end_visit(W, in_x_start, scale_w, Wd);
-        nx = x_end - in_x_start;
-        atomicMax(&s_x1, x_end);
-        atomicMax(&s_nx, nx);
+    {
+        // largest end and largest visit count over the wavefront by a butterfly of lane exchanges, then one LDS atomic
+        // per wavefront (an atomic per lane is serialised lane by lane on the scalar unit)
+        int32_t x_end = 0;
+        if (col_ok) {
+            x_end = end_visit(W, in_x_start, scale_w, Wd);
+            nx = x_end - in_x_start;
+        }
+        int32_t m_end = x_end, m_nx = nx, m_min = col_ok ? nx : INT32_MAX;  // lanes past the last column do not count
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) {
+            const int32_t o_end = __shfl_xor(m_end, d), o_nx = __shfl_xor(m_nx, d), o_min = __shfl_xor(m_min, d);
+            m_end = (o_end > m_end) ? o_end : m_end;
+            m_nx = (o_nx > m_nx) ? o_nx : m_nx;
+            m_min = (o_min < m_min) ? o_min : m_min;
+        }
+        if ((threadIdx.x & 63) == 0) {
+            atomicMax(&s_x1, m_end);
+            atomicMax(&s_nx, m_nx);
+            atomicMin(&s_nx_min, m_min);
+        }
     }
     if (tx == 0) {
         for (int32_t H = H0 + ty; H < H0 + tile_rows && H < Hs; H += kTileGroups) {
@@ -290,9 +312,11 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
     const int32_t tile_y1 = s_y1;
     const int32_t pitch_w = (tile_x1 > tile_x0) ? (tile_x1 - tile_x0) / EPW : 0;
     const int32_t rows = (tile_y1 > tile_y0) ? tile_y1 - tile_y0 : 0;
-    const bool use_lds = (int64_t)rows * pitch_w <= cap_words;
+    // the tile holds fp32 values (16-bit gradients are widened by the copy, which is exact): a lane's run of columns
+    // then starts on a 4-byte boundary whatever its parity, and LDS reads that straddle words are several times slower
     const int32_t pitch = pitch_w * EPW;
-    const TI* tile = reinterpret_cast<const TI*>(tile_words);
+    const bool use_lds = (int64_t)rows * pitch <= cap_words;
+    const float* tile = reinterpret_cast<const float*>(tile_words);
     const float out_x_start = ((float)in_x_start + offset) * scale_w - offset;
     const float fw = (float)W;
 
@@ -308,7 +332,7 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
             out_x += scale_w;
         }
     }
-    const int32_t nx_max = s_nx;
+    const int32_t nx_max = s_nx, nx_min = s_nx_min;
     // starting position and step of this lane in the tile's (row, word) grid for the copy loop
     const int32_t pw1 = (pitch_w > 0) ? pitch_w : 1;
     const int32_t ld_r0 = (int32_t)threadIdx.x / pw1, ld_c0 = (int32_t)threadIdx.x % pw1;
@@ -323,9 +347,19 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
             int32_t r = ld_r0, cw = ld_c0;
             const uint32_t* src = reinterpret_cast<const uint32_t*>(gp + (int64_t)tile_y0 * Wd + tile_x0);
             const int32_t row_words = Wd / EPW;
-#pragma unroll 4
+#pragma unroll 8
             for (int32_t i = threadIdx.x; i < total; i += kGradThreads) {
-                tile_words[i] = src[(int64_t)r * row_words + cw];
+                const uint32_t word = src[(int64_t)r * row_words + cw];
+                if (EPW == 1) {
+                    tile_words[i] = word;
+                } else {
+                    TI pair[2];
+                    __builtin_memcpy(pair, &word, 4);
+                    float2 wide;
+                    wide.x = ElemIO<TI>::load(&pair[0]);
+                    wide.y = ElemIO<TI>::load(&pair[1]);
+                    reinterpret_cast<float2*>(tile_words)[i] = wide;
+                }
                 r += ld_dr;
                 cw += ld_dc;
                 if (cw >= pitch_w) {
@@ -341,24 +375,25 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
                 const float out_y_start = ((float)in_y_start + offset) * scale_h - offset;
                 float acc;
                 // separate call sites so that each is compiled for its own address space (LDS reads, global loads)
+#define OPSCV_VISIT(KX, KMIN)                                                                                       \
+    visit_sum_fixed<float, KX, KMIN>(tile + x_base, pitch, tile_y0, in_y_start, nx, xl, out_y_start, (float)H, scale_h,  \
+                                  last_y, Hd, neg_zero)
                 if (use_lds && nx_max <= 4) {
-                    const float(&xl4)[4] = reinterpret_cast<const float(&)[4]>(xl);
-                    acc = visit_sum_fixed<TI, 4>(tile + x_base, pitch, tile_y0, in_y_start, nx, xl4, out_y_start,
-                                                 (float)H, scale_h, last_y, Hd, neg_zero);
+                    acc = (nx_min >= 4) ? OPSCV_VISIT(4, 4) : OPSCV_VISIT(4, 0);
+                } else if (use_lds && nx_max <= 5) {
+                    acc = (nx_min >= 4) ? OPSCV_VISIT(5, 4) : OPSCV_VISIT(5, 0);
                 } else if (use_lds && nx_max <= 6) {
-                    const float(&xl6)[6] = reinterpret_cast<const float(&)[6]>(xl);
-                    acc = visit_sum_fixed<TI, 6>(tile + x_base, pitch, tile_y0, in_y_start, nx, xl6, out_y_start,
-                                                 (float)H, scale_h, last_y, Hd, neg_zero);
+                    acc = (nx_min >= 4) ? OPSCV_VISIT(6, 4) : OPSCV_VISIT(6, 0);
                 } else if (use_lds && nx_max <= 8) {
-                    acc = visit_sum_fixed<TI, 8>(tile + x_base, pitch, tile_y0, in_y_start, nx, xl, out_y_start,
-                                                 (float)H, scale_h, last_y, Hd, neg_zero);
+                    acc = OPSCV_VISIT(8, 0);
                 } else if (use_lds) {
-                    acc = visit_sum<TI>(tile, pitch, tile_y0, tile_x0, in_y_start, in_x_start, out_y_start,
+                    acc = visit_sum<float>(tile, pitch, tile_y0, tile_x0, in_y_start, in_x_start, out_y_start,
                                         out_x_start, (float)H, fw, scale_h, scale_w, last_y, last_x, Hd, Wd);
                 } else {
                     acc = visit_sum<TI>(gp, Wd, 0, 0, in_y_start, in_x_start, out_y_start, out_x_start, (float)H, fw,
                                         scale_h, scale_w, last_y, last_x, Hd, Wd);
                 }
+#undef OPSCV_VISIT
                 ElemIO<TO>::store(y + (pl * Hs + H) * (int64_t)Ws + W, acc);
             }
         }
@@ -371,7 +406,7 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
 // Output rows per workgroup for the LDS variant (0: use the gather kernel).  The estimate only sizes the launch;
 // the kernel measures the rectangle itself.
 template <typename TI>
-int32_t lds_tile_rows(const ResizeGradArgs& a, int32_t cap_words)
+int32_t lds_tile_rows(const ResizeGradArgs& a, int32_t cap_words, int32_t* need_words = nullptr)
 {
     constexpr int EPW = 4 / (int)sizeof(TI);
     if (a.channels_last || a.user_scales || a.Wd % EPW != 0 || reinterpret_cast<uintptr_t>(a.x) % 4 != 0) {
@@ -380,8 +415,11 @@ int32_t lds_tile_rows(const ResizeGradArgs& a, int32_t cap_words)
     const double per_col = (double)a.Wd / (double)a.Ws, per_row = (double)a.Hd / (double)a.Hs;
     const double cols = kTileCols * per_col + 2.0 * per_col + 2.0 + EPW;
     for (int32_t rows = 8; rows >= kTileGroups; rows /= 2) {
-        const double need = (rows * per_row + 2.0 * per_row + 2.0) * cols / EPW;
+        const double need = (rows * per_row + 2.0 * per_row + 2.0) * cols;  // fp32 words: one per element
         if (need <= (double)cap_words) {
+            if (need_words != nullptr) {
+                *need_words = (int32_t)need + 1;
+            }
             return rows;
         }
     }
@@ -391,23 +429,38 @@ int32_t lds_tile_rows(const ResizeGradArgs& a, int32_t cap_words)
 template <typename TI, typename TO>
 hipError_t run(const ResizeGradArgs& a, hipStream_t stream)
 {
-    constexpr int32_t kCapWords = 8192;  // 32 KB of LDS per workgroup
-    const int32_t tile_rows = lds_tile_rows<TI>(a, kCapWords);
+    constexpr int32_t kCapWords = kGradCapWords;
+    int32_t lds_words = kCapWords;
+    const int32_t tile_rows = lds_tile_rows<TI>(a, kCapWords, &lds_words);
+    // the allocation follows the estimate so that more workgroups share a CU (their load and compute phases overlap);
+    // a rectangle that turns out larger than the estimate is read from global memory by the kernel
+    lds_words = (lds_words + 63) / 64 * 64;
+    lds_words = lds_words < kCapWords ? lds_words : kCapWords;
     if (tile_rows > 0) {
         const int64_t planes = a.N * a.C;
+        // A workgroup walks over several planes with the tile geometry and column weights it computed once; enough
+        // workgroups are launched to keep every CU supplied (want_blocks), the rest of the planes are looped over.
+        const int64_t tiles = ((a.Ws + kTileCols - 1) / kTileCols) * ((a.Hs + tile_rows - 1) / tile_rows);
+        int64_t want_blocks = 16384;
+        if (const char* v = getenv("OPSCV_RGRAD_BLOCKS")) {
+            want_blocks = atoll(v) > 0 ? atoll(v) : want_blocks;
+        }
+        int64_t zdim = (want_blocks + tiles - 1) / tiles;
+        zdim = zdim < planes ? zdim : planes;
+        zdim = zdim < 65535 ? zdim : 65535;
         dim3 grid((unsigned)((a.Ws + kTileCols - 1) / kTileCols), (unsigned)((a.Hs + tile_rows - 1) / tile_rows),
-                  (unsigned)(planes < 65535 ? planes : 65535));
+                  (unsigned)zdim);
         if (grid.y <= 65535) {
             if (a.half_pixel) {
-                hipLaunchKernelGGL((resize_grad_lds_kernel<TI, TO, true>), grid, dim3(kGradThreads), kCapWords * 4,
+                hipLaunchKernelGGL((resize_grad_lds_kernel<TI, TO, true>), grid, dim3(kGradThreads), lds_words * 4,
                                    stream, (const TI*)a.x, (TO*)a.y, planes, (int32_t)a.Hs, (int32_t)a.Ws,
                                    (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h, a.scale_w, a.inv_scale_h, a.inv_scale_w,
-                                   tile_rows, kCapWords, -0.0f);
+                                   tile_rows, lds_words, -0.0f);
             } else {
-                hipLaunchKernelGGL((resize_grad_lds_kernel<TI, TO, false>), grid, dim3(kGradThreads), kCapWords * 4,
+                hipLaunchKernelGGL((resize_grad_lds_kernel<TI, TO, false>), grid, dim3(kGradThreads), lds_words * 4,
                                    stream, (const TI*)a.x, (TO*)a.y, planes, (int32_t)a.Hs, (int32_t)a.Ws,
                                    (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h, a.scale_w, a.inv_scale_h, a.inv_scale_w,
-                                   tile_rows, kCapWords, -0.0f);
+                                   tile_rows, lds_words, -0.0f);
             }
             return hipGetLastError();
         }
@@ -451,7 +504,7 @@ const char* resize_grad_variant(const ResizeGradArgs& a)
     if (a.user_scales) {
         return "resize_grad_gather_scales";
     }
-    constexpr int32_t kCapWords = 8192;
+    constexpr int32_t kCapWords = kGradCapWords;
     const int32_t rows = (a.elem_in == Elem::F32) ? lds_tile_rows<float>(a, kCapWords)
                                                   : lds_tile_rows<uint16_t>(a, kCapWords);
     return (rows > 0 && (a.Hs + rows - 1) / rows <= 65535) ? "resize_grad_lds" : "resize_grad_gather";
