@@ -13,6 +13,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdlib>
+#include <type_traits>
 
 #include "kernels.hpp"
 #include "sampler_math.hpp"
@@ -235,6 +236,36 @@ __device__ __forceinline__ float visit_sum_fixed(const TI* tile_xy, int32_t pitc
     return acc;
 }
 
+// The same sum once more with the row part taken out as well.  The rows an outgoing row H visits, and their weights,
+// do not depend on the plane or the column: a workgroup that walks over planes computes them once per H (by the very
+// loop above) and keeps count and weights in registers.  H is the same for all lanes of a wavefront, so the count is
+// a scalar and the row loop needs no lane masks.  A visited row then costs the LDS reads, one address add and, per
+// column, two products and an add.
+constexpr int kRowWeights = 6;  // visited rows per outgoing row kept in registers (more: the loops above)
+
+template <int KX, int KMIN, int Q>
+__device__ __forceinline__ float tile_sum_fixed(const float* lane_rows, int32_t pitch, int32_t n_rows, float lerp_pack,
+                                                int32_t nx, const float* xl, float neg_zero)
+{
+    float acc = 0.0f;
+#pragma unroll
+    for (int j = 0; j < kRowWeights; j++) {
+        if (j < n_rows) {  // n_rows is uniform over the wavefront
+            // weight of visited row j of this wavefront's outgoing row Q: lane Q * kRowWeights + j of lerp_pack
+            const float y_lerp = __builtin_bit_cast(
+                float, __builtin_amdgcn_readlane(__builtin_bit_cast(int32_t, lerp_pack), Q * kRowWeights + j));
+#pragma unroll
+            for (int k = 0; k < KX; k++) {
+                // fma(g, w, -0) is g * w bit for bit; the compiler may not fold it into the following product
+                const float t = __builtin_fmaf(lane_rows[k], y_lerp, neg_zero) * xl[k];
+                acc = (k < KMIN || k < nx) ? acc + t : acc;
+            }
+            lane_rows += pitch;
+        }
+    }
+    return acc;
+}
+
 constexpr int kTileCols = 128;
 constexpr int32_t kGradCapWords = 12288;  // at most 48 KB of LDS per workgroup (fp32 words, one per tile element)
 constexpr int kTileGroups = kGradThreads / kTileCols;  // row groups of a workgroup
@@ -245,13 +276,26 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
                                                                         int32_t Hd, int32_t Wd, float scale_h,
                                                                         float scale_w, float inv_scale_h,
                                                                         float inv_scale_w, int32_t tile_rows,
-                                                                        int32_t cap_words, float neg_zero)
+                                                                        int32_t cap_words, float neg_zero,
+                                                                        uint32_t tiles_x, uint32_t tiles_y,
+                                                                        uint32_t plane_slots)
 {
+    // Workgroups are handed to the eight XCDs in turn, each with its own L2.  The launch is one-dimensional and padded
+    // to a multiple of eight; workgroup L becomes tile (L % 8) * (count / 8) + L / 8, so that an XCD works through a
+    // contiguous run of tiles and the rows and 128-byte lines that neighbouring tiles share are fetched from memory
+    // once per XCD rather than once per tile.
+    const uint32_t per_xcd = gridDim.x / 8u;
+    const uint32_t tile_id = (blockIdx.x % 8u) * per_xcd + blockIdx.x / 8u;
+    if (tile_id >= tiles_x * tiles_y * plane_slots) {
+        return;
+    }
+    const uint32_t block_x = tile_id % tiles_x, block_y = (tile_id / tiles_x) % tiles_y;
+    const uint32_t block_z = tile_id / (tiles_x * tiles_y);
     constexpr int EPW = 4 / (int)sizeof(TI);  // elements per 4-byte word
     extern __shared__ __attribute__((aligned(16))) uint32_t tile_words[];
     __shared__ int32_t s_x1, s_y1, s_nx, s_nx_min;
     const int tx = threadIdx.x % kTileCols, ty = threadIdx.x / kTileCols;
-    const int32_t W0 = blockIdx.x * kTileCols, H0 = blockIdx.y * tile_rows;
+    const int32_t W0 = (int32_t)block_x * kTileCols, H0 = (int32_t)block_y * tile_rows;
     const float offset = HALF_PIXEL ? 0.5f : 0.0f;
     const float last_y = (float)Hs - 1.0f, last_x = (float)Ws - 1.0f;
     auto first_visit = [&](int32_t i, float inv_scale, int32_t len_dst) {
@@ -339,14 +383,45 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
     const int32_t ld_dr = kGradThreads / pw1, ld_dc = kGradThreads % pw1;
     const int32_t x_base = (nx > 0) ? in_x_start - tile_x0 : 0;
 
-    for (int64_t pl = blockIdx.z; pl < planes; pl += gridDim.z) {
+    // rows visited by each of this wavefront's outgoing rows, and their weights (see tile_sum_fixed)
+    constexpr int HQ = 8 / kTileGroups;  // outgoing rows per lane at the largest tile height
+    static_assert(HQ * kRowWeights <= 64, "the row weights of a wavefront are packed one per lane");
+    int32_t hy_start[HQ], hy_n[HQ];
+    float lerp_pack = 0.0f;  // lane q * kRowWeights + j: weight of visited row j of outgoing row q (a uniform table)
+    bool rows_fixed = true;
+    const int32_t lane_id = (int32_t)threadIdx.x & 63;
+#pragma unroll
+    for (int q = 0; q < HQ; q++) {
+        const int32_t H = __builtin_amdgcn_readfirstlane(H0 + ty + q * kTileGroups);
+        hy_start[q] = 0;
+        hy_n[q] = -1;  // no such row in this tile
+        if (H < H0 + tile_rows && H < Hs) {
+            const int32_t start = first_visit(H, inv_scale_h, Hd);
+            float out_y = ((float)start + offset) * scale_h - offset;
+            const float fh = (float)H;
+            int32_t n = 0;
+            for (int32_t in_y = start; out_y < fh + 1.0f && in_y < Hd; in_y++) {
+                const float w = 1.0f - __builtin_fabsf(__builtin_amdgcn_fmed3f(out_y, 0.0f, last_y) - fh);
+                lerp_pack = (n < kRowWeights && lane_id == q * kRowWeights + n) ? w : lerp_pack;
+                n++;
+                out_y += scale_h;
+            }
+            hy_start[q] = __builtin_amdgcn_readfirstlane(start);
+            hy_n[q] = __builtin_amdgcn_readfirstlane(n);
+            rows_fixed = rows_fixed && (hy_n[q] <= kRowWeights);
+        }
+    }
+
+    // Copy of the rectangle into LDS: word i of the tile is (row i / pitch_w, word i % pitch_w) of the rectangle.
+    const int32_t total = rows * pitch_w;
+    const int32_t row_words = Wd / EPW;
+
+    for (int64_t pl = block_z; pl < planes; pl += plane_slots) {
         const TI* gp = g + pl * (int64_t)Hd * Wd;
         if (use_lds) {
-            // word i of the tile is (row i / pitch_w, word i % pitch_w); the pair is advanced instead of divided
-            const int32_t total = rows * pitch_w;
+            // the pair (row, word) is advanced instead of divided
             int32_t r = ld_r0, cw = ld_c0;
             const uint32_t* src = reinterpret_cast<const uint32_t*>(gp + (int64_t)tile_y0 * Wd + tile_x0);
-            const int32_t row_words = Wd / EPW;
 #pragma unroll 8
             for (int32_t i = threadIdx.x; i < total; i += kGradThreads) {
                 const uint32_t word = src[(int64_t)r * row_words + cw];
@@ -369,7 +444,32 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
             }
             __syncthreads();
         }
-        if (col_ok) {
+        if (col_ok && use_lds && rows_fixed && nx_max <= 6) {
+            TO* yp = y + (pl * Hs + H0 + ty) * (int64_t)Ws + W;
+            auto one_row = [&](auto qc) {
+                constexpr int q = decltype(qc)::value;
+                if (hy_n[q] >= 0) {
+                    const float* lane_rows = tile + (hy_start[q] - tile_y0) * pitch + x_base;
+                    float acc;
+#define OPSCV_TILE_SUM(KX, KMIN) \
+    tile_sum_fixed<KX, KMIN, q>(lane_rows, pitch, hy_n[q], lerp_pack, nx, xl, neg_zero)
+                    if (nx_max <= 4) {
+                        acc = (nx_min >= 4) ? OPSCV_TILE_SUM(4, 4) : OPSCV_TILE_SUM(4, 0);
+                    } else if (nx_max <= 5) {
+                        acc = (nx_min >= 4) ? OPSCV_TILE_SUM(5, 4) : OPSCV_TILE_SUM(5, 0);
+                    } else {
+                        acc = (nx_min >= 4) ? OPSCV_TILE_SUM(6, 4) : OPSCV_TILE_SUM(6, 0);
+                    }
+#undef OPSCV_TILE_SUM
+                    ElemIO<TO>::store(yp + (int64_t)q * kTileGroups * Ws, acc);
+                }
+            };
+            static_assert(HQ == 4, "one call per outgoing row of a lane");
+            one_row(std::integral_constant<int, 0>{});
+            one_row(std::integral_constant<int, 1>{});
+            one_row(std::integral_constant<int, 2>{});
+            one_row(std::integral_constant<int, 3>{});
+        } else if (col_ok) {
             for (int32_t H = H0 + ty; H < H0 + tile_rows && H < Hs; H += kTileGroups) {
                 const int32_t in_y_start = first_visit(H, inv_scale_h, Hd);
                 const float out_y_start = ((float)in_y_start + offset) * scale_h - offset;
@@ -441,27 +541,25 @@ hipError_t run(const ResizeGradArgs& a, hipStream_t stream)
         // A workgroup walks over several planes with the tile geometry and column weights it computed once; enough
         // workgroups are launched to keep every CU supplied (want_blocks), the rest of the planes are looped over.
         const int64_t tiles = ((a.Ws + kTileCols - 1) / kTileCols) * ((a.Hs + tile_rows - 1) / tile_rows);
-        int64_t want_blocks = 16384;
-        if (const char* v = getenv("OPSCV_RGRAD_BLOCKS")) {
-            want_blocks = atoll(v) > 0 ? atoll(v) : want_blocks;
-        }
+        const int64_t want_blocks = 8192;
         int64_t zdim = (want_blocks + tiles - 1) / tiles;
         zdim = zdim < planes ? zdim : planes;
         zdim = zdim < 65535 ? zdim : 65535;
-        dim3 grid((unsigned)((a.Ws + kTileCols - 1) / kTileCols), (unsigned)((a.Hs + tile_rows - 1) / tile_rows),
-                  (unsigned)zdim);
-        if (grid.y <= 65535) {
+        const int64_t tiles_x = (a.Ws + kTileCols - 1) / kTileCols, tiles_y = (a.Hs + tile_rows - 1) / tile_rows;
+        const int64_t blocks = (tiles * zdim + 7) / 8 * 8;  // padded for the XCD mapping of the kernel
+        if (tiles_y <= 65535 && blocks <= (int64_t)INT32_MAX) {
+            const dim3 grid((unsigned)blocks);
+#define OPSCV_RGL(HP)                                                                                                \
+    hipLaunchKernelGGL((resize_grad_lds_kernel<TI, TO, HP>), grid, dim3(kGradThreads), lds_words * 4, stream,         \
+                       (const TI*)a.x, (TO*)a.y, planes, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, \
+                       a.scale_h, a.scale_w, a.inv_scale_h, a.inv_scale_w, tile_rows, lds_words, -0.0f,              \
+                       (uint32_t)tiles_x, (uint32_t)tiles_y, (uint32_t)zdim)
             if (a.half_pixel) {
-                hipLaunchKernelGGL((resize_grad_lds_kernel<TI, TO, true>), grid, dim3(kGradThreads), lds_words * 4,
-                                   stream, (const TI*)a.x, (TO*)a.y, planes, (int32_t)a.Hs, (int32_t)a.Ws,
-                                   (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h, a.scale_w, a.inv_scale_h, a.inv_scale_w,
-                                   tile_rows, lds_words, -0.0f);
+                OPSCV_RGL(true);
             } else {
-                hipLaunchKernelGGL((resize_grad_lds_kernel<TI, TO, false>), grid, dim3(kGradThreads), lds_words * 4,
-                                   stream, (const TI*)a.x, (TO*)a.y, planes, (int32_t)a.Hs, (int32_t)a.Ws,
-                                   (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h, a.scale_w, a.inv_scale_h, a.inv_scale_w,
-                                   tile_rows, lds_words, -0.0f);
+                OPSCV_RGL(false);
             }
+#undef OPSCV_RGL
             return hipGetLastError();
         }
     }
