@@ -771,6 +771,13 @@ int oracle_upsample_bilinear2d_backward(const void* grads, void* y, int dtype_in
     if (dtype_in < 0 || dtype_in > 2 || dtype_out < 0 || dtype_out > 2 || Hs <= 0 || Ws <= 0 || Hd <= 0 || Wd <= 0) {
         return -1;
     }
+    /* equal sizes: the entry point hands the incoming gradient on without running the operator, whatever the scales
+     * (image/resize_bilinear_v2_grad/op_api/aclnn_upsample_bilinear_2d_backward.cpp:251-252; the operator's own
+     * all-copy template says the same, resize_bilinear_v2_grad_tiling_arch35.cpp:310-313) */
+    if (Hs == Hd && Ws == Wd && dtype_in == dtype_out) {
+        memcpy(y, grads, (size_t)(N * C * Hs * Ws) * (size_t)((dtype_in == ORACLE_F32) ? 4 : 2));
+        return 0;
+    }
     const float scale_h = grad_scale(Hs, Hd, align_corners, (float)scales_h);
     const float scale_w = grad_scale(Ws, Wd, align_corners, (float)scales_w);
     const float inv_h = 1.0f / scale_h, inv_w = 1.0f / scale_w;

@@ -93,16 +93,18 @@ def _random_resize_family(oracle, device, aclnn, torch, rng):
         H, W = _dims(rng, 1, 90, 2)
         Ho, Wo = _dims(rng, 1, 200, 2)
         align, cl = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
-        _say("upsample", dtype, N, C, H, W, Ho, Wo, align, cl)
+        # a third of the cases hand over scales of their own (they replace the size ratio when align_corners is off)
+        sh, sw = (float(rng.uniform(0.3, 3.0)), float(rng.uniform(0.3, 3.0))) if case % 3 == 1 else (0.0, 0.0)
+        _say("upsample", dtype, N, C, H, W, Ho, Wo, align, cl, sh, sw)
         x = I.cast_np(rng.standard_normal((N, C, H, W)).astype(np.float32), dtype)
         xin = np.ascontiguousarray(x.transpose(0, 2, 3, 1)) if cl else x
         if cl:
-            ref = oracle.upsample_bilinear2d_nhwc(xin, (Ho, Wo), align, dtype=I.oracle_code(dtype))
+            ref = oracle.upsample_bilinear2d_nhwc(xin, (Ho, Wo), align, sh, sw, dtype=I.oracle_code(dtype))
         else:
-            ref = oracle.upsample_bilinear2d(x, (Ho, Wo), align, dtype=I.oracle_code(dtype))
-        y = aclnn.upsample_bilinear2d(I.to_torch(xin, dtype, device), (Ho, Wo), align, channels_last=cl)
+            ref = oracle.upsample_bilinear2d(x, (Ho, Wo), align, sh, sw, dtype=I.oracle_code(dtype))
+        y = aclnn.upsample_bilinear2d(I.to_torch(xin, dtype, device), (Ho, Wo), align, sh, sw, channels_last=cl)
         torch.cuda.synchronize()
-        _same(I.from_torch(y, dtype), ref, dtype, (case, "up", dtype, N, C, H, W, Ho, Wo, align, cl))
+        _same(I.from_torch(y, dtype), ref, dtype, (case, "up", dtype, N, C, H, W, Ho, Wo, align, cl, sh, sw))
         # nearest through aclnnResize on the same tensors
         _say("nearest", dtype, N, C, H, W, Ho, Wo, cl)
         scales = (1.0, Ho / H, Wo / W, 1.0) if cl else (1.0, 1.0, Ho / H, Wo / W)
@@ -115,15 +117,25 @@ def _random_resize_family(oracle, device, aclnn, torch, rng):
         torch.cuda.synchronize()
         ref = oracle.resize_nearest(xin, (Ho, Wo), channels_last=cl, dtype=I.oracle_code(dtype))
         _same(I.from_torch(y, dtype), ref, dtype, (case, "nearest", dtype, N, C, H, W, Ho, Wo, cl))
+        # bilinear through aclnnResize: align_corners off, the size ratio as scale
+        _say("resize bilinear", dtype, N, C, H, W, Ho, Wo, cl)
+        y = aclnn.resize(I.to_torch(xin, dtype, device), scales, "bilinear", out=out, channels_last=cl)
+        torch.cuda.synchronize()
+        if cl:
+            ref = oracle.upsample_bilinear2d_nhwc(xin, (Ho, Wo), False, dtype=I.oracle_code(dtype))
+        else:
+            ref = oracle.upsample_bilinear2d(x, (Ho, Wo), False, dtype=I.oracle_code(dtype))
+        _same(I.from_torch(y, dtype), ref, dtype, (case, "resize bilinear", dtype, N, C, H, W, Ho, Wo, cl))
         # gradient of the upsample
         _say("upsample backward", dtype, N, C, H, W, Ho, Wo, align, cl)
         gshape = (N, Ho, Wo, C) if cl else (N, C, Ho, Wo)
         go = I.cast_np(rng.standard_normal(gshape).astype(np.float32), dtype)
-        ref = oracle.upsample_bilinear2d_backward(go, (H, W), align, channels_last=cl, dtype=I.oracle_code(dtype))
+        ref = oracle.upsample_bilinear2d_backward(go, (H, W), align, channels_last=cl, dtype=I.oracle_code(dtype),
+                                                  scales_h=sh, scales_w=sw)
         isz = (N, H, W, C) if cl else (N, C, H, W)
-        y = aclnn.upsample_bilinear2d_backward(I.to_torch(go, dtype, device), isz, align, channels_last=cl)
+        y = aclnn.upsample_bilinear2d_backward(I.to_torch(go, dtype, device), isz, align, sh, sw, channels_last=cl)
         torch.cuda.synchronize()
-        _same(I.from_torch(y, dtype), ref, dtype, (case, "upbwd", dtype, N, C, H, W, Ho, Wo, align, cl))
+        _same(I.from_torch(y, dtype), ref, dtype, (case, "upbwd", dtype, N, C, H, W, Ho, Wo, align, cl, sh, sw))
 
 
 def test_random_sampler_backward_and_3d(oracle, device, aclnn):

@@ -858,3 +858,18 @@ def test_upsample_hw_split_template(oracle):
         assert oracle.upsample_bilinear2d(xs, (32, 64), False)[0, 0, 0, 0] == np.float32(1.3125)
     finally:
         oracle.set_reference_cores(0)
+
+
+def test_upsample_backward_equal_sizes_is_a_copy(oracle):
+    """equal sizes: the incoming gradient is handed on, also when scales are given (the reference's entry point skips
+    the operator there, aclnn_upsample_bilinear_2d_backward.cpp:251-252), bits and non-finite values included"""
+    rng = np.random.default_rng(81)
+    g = rng.standard_normal((2, 3, 5, 7), dtype=np.float32)
+    g[0, 0, 0, :3] = [np.inf, np.nan, -0.0]
+    for align in (False, True):
+        for sh, sw in ((0.0, 0.0), (1.7, 0.4)):
+            y = oracle.upsample_bilinear2d_backward(g, (5, 7), align, scales_h=sh, scales_w=sw)
+            assert np.array_equal(y.view(np.uint32), g.view(np.uint32))
+    yh = oracle.upsample_bilinear2d_backward(np.ascontiguousarray(g.transpose(0, 2, 3, 1)), (5, 7), False,
+                                             channels_last=True, scales_h=2.0, scales_w=2.0)
+    assert np.array_equal(yh.view(np.uint32), g.transpose(0, 2, 3, 1).view(np.uint32))
