@@ -37,6 +37,28 @@ def _dims(rng, lo, hi, n):
     return [int(round(np.exp(rng.uniform(np.log(lo), np.log(hi))))) for _ in range(n)]
 
 
+SPECIAL_COORDS = np.array([np.nan, np.inf, -np.inf, 1e30, -1e30, 3e9, -3e9, 1.0, -1.0, 0.0, -0.0, 0.5, -0.5, 2.0, -2.0],
+                          np.float32)
+
+
+def _sprinkle(rng, g32, H, W, align):
+    """a few per cent of the coordinates replaced: non-finite and huge values, the borders, and coordinates that
+    land exactly on pixel centres and on the ties between them"""
+    flat = g32.reshape(-1)
+    k = max(1, flat.size // 25)
+    idx = rng.integers(0, flat.size, k)
+    flat[idx] = SPECIAL_COORDS[rng.integers(0, len(SPECIAL_COORDS), k)]
+    idx = rng.integers(0, flat.size, k)
+    size = np.where(idx % 2 == 0, W, H).astype(np.float32)   # x coordinates at even positions
+    half = rng.integers(0, 2 * int(max(H, W)) + 2, k).astype(np.float32) / 2.0   # pixel centres and half-way points
+    half = np.minimum(half, size)
+    if align:
+        flat[idx] = np.where(size > 1, 2.0 * half / np.maximum(size - 1, 1) - 1.0, 0.0).astype(np.float32)
+    else:
+        flat[idx] = ((2.0 * half + 1.0) / size - 1.0).astype(np.float32)
+    return g32
+
+
 def test_random_grid_sampler2d(oracle, device, aclnn):
     import torch
     rng = np.random.default_rng(9001 + SEED_SHIFT)
@@ -46,13 +68,23 @@ def test_random_grid_sampler2d(oracle, device, aclnn):
         H, W = _dims(rng, 1, 150, 2)
         Ho, Wo = _dims(rng, 1, 120, 2)
         interp, pad, align = int(rng.integers(0, 3)), int(rng.integers(0, 3)), bool(rng.integers(0, 2))
-        _say("gs2d", dtype, N, C, H, W, Ho, Wo, interp, pad, align)
+        cl = case % 4 == 3   # a quarter of the cases: input and out as channels-last views
+        _say("gs2d", dtype, N, C, H, W, Ho, Wo, interp, pad, align, cl)
         x = I.cast_np(rng.standard_normal((N, C, H, W)).astype(np.float32), dtype)
-        g = I.cast_np(rng.uniform(-1.4, 1.4, (N, Ho, Wo, 2)).astype(np.float32), dtype)
+        g32 = rng.uniform(-1.4, 1.4, (N, Ho, Wo, 2)).astype(np.float32)
+        if case % 2 == 1:
+            g32 = _sprinkle(rng, g32, H, W, align)
+        g = I.cast_np(g32, dtype)
         ref = oracle.grid_sampler2d(x, g, interp, pad, align, dtype=I.oracle_code(dtype))
-        y = aclnn.grid_sampler2d(I.to_torch(x, dtype, device), I.to_torch(g, dtype, device), interp, pad, align)
+        xt, gt = I.to_torch(x, dtype, device), I.to_torch(g, dtype, device)
+        if cl:
+            xt = xt.contiguous(memory_format=torch.channels_last)
+            out = torch.empty((N, C, Ho, Wo), dtype=xt.dtype, device=device).contiguous(memory_format=torch.channels_last)
+            y = aclnn.grid_sampler2d(xt, gt, interp, pad, align, out=out).contiguous()
+        else:
+            y = aclnn.grid_sampler2d(xt, gt, interp, pad, align)
         torch.cuda.synchronize()
-        _same(I.from_torch(y, dtype), ref, dtype, (case, dtype, N, C, H, W, Ho, Wo, interp, pad, align))
+        _same(I.from_torch(y, dtype), ref, dtype, (case, dtype, N, C, H, W, Ho, Wo, interp, pad, align, cl))
 
 
 def test_random_grid_sampler2d_large_planes(oracle, device, aclnn):
@@ -67,7 +99,10 @@ def test_random_grid_sampler2d_large_planes(oracle, device, aclnn):
         interp, pad, align = int(rng.integers(0, 3)), int(rng.integers(0, 3)), bool(rng.integers(0, 2))
         _say("gs2d large", dtype, N, C, H, W, Ho, Wo, interp, pad, align)
         x = I.cast_np(rng.standard_normal((N, C, H, W)).astype(np.float32), dtype)
-        g = I.cast_np(rng.uniform(-1.2, 1.2, (N, Ho, Wo, 2)).astype(np.float32), dtype)
+        g32 = rng.uniform(-1.2, 1.2, (N, Ho, Wo, 2)).astype(np.float32)
+        if case % 2 == 1:
+            g32 = _sprinkle(rng, g32, H, W, align)
+        g = I.cast_np(g32, dtype)
         ref = oracle.grid_sampler2d(x, g, interp, pad, align, dtype=I.oracle_code(dtype))
         y = aclnn.grid_sampler2d(I.to_torch(x, dtype, device), I.to_torch(g, dtype, device), interp, pad, align)
         torch.cuda.synchronize()
@@ -149,7 +184,10 @@ def test_random_sampler_backward_and_3d(oracle, device, aclnn):
         interp, pad, align = int(rng.integers(0, 3)), int(rng.integers(0, 3)), bool(rng.integers(0, 2))
         _say("gs2d backward", dtype, N, C, H, W, Ho, Wo, interp, pad, align)
         x = I.cast_np(rng.standard_normal((N, C, H, W)).astype(np.float32), dtype)
-        g = I.cast_np(rng.uniform(-1.3, 1.3, (N, Ho, Wo, 2)).astype(np.float32), dtype)
+        g32 = rng.uniform(-1.3, 1.3, (N, Ho, Wo, 2)).astype(np.float32)
+        if case % 2 == 1:
+            g32 = _sprinkle(rng, g32, H, W, align)
+        g = I.cast_np(g32, dtype)
         go = I.cast_np(rng.standard_normal((N, C, Ho, Wo)).astype(np.float32), dtype)
         rdx, rdg = oracle.grid_sampler2d_backward(go, x, g, interp, pad, align, dtype=I.oracle_code(dtype))
         dx, dg = aclnn.grid_sampler2d_backward(I.to_torch(go, dtype, device), I.to_torch(x, dtype, device),
@@ -166,7 +204,12 @@ def test_random_sampler_backward_and_3d(oracle, device, aclnn):
             rng.integers(0, 2))
         _say("gs3d", dtype, N, C, D, H, W, Do, Ho, Wo, interp, pad, align, cl)
         x = I.cast_np(rng.standard_normal((N, C, D, H, W)).astype(np.float32), dtype)
-        g = I.cast_np(rng.uniform(-1.4, 1.4, (N, Do, Ho, Wo, 3)).astype(np.float32), dtype)
+        g32 = rng.uniform(-1.4, 1.4, (N, Do, Ho, Wo, 3)).astype(np.float32)
+        if case % 2 == 1:
+            flat = g32.reshape(-1)
+            k = max(1, flat.size // 25)
+            flat[rng.integers(0, flat.size, k)] = SPECIAL_COORDS[rng.integers(0, len(SPECIAL_COORDS), k)]
+        g = I.cast_np(g32, dtype)
         ref = oracle.grid_sampler3d(x, g, interp, pad, align, dtype=I.oracle_code(dtype))
         xin = np.ascontiguousarray(x.transpose(0, 2, 3, 4, 1)) if cl else x
         y = aclnn.grid_sampler3d(I.to_torch(xin, dtype, device), I.to_torch(g, dtype, device), interp, pad, align,
