@@ -218,3 +218,117 @@ def test_random_sampler_backward_and_3d(oracle, device, aclnn):
         got = I.from_torch(y, dtype)
         got = got.transpose(0, 4, 1, 2, 3) if cl else got
         _same(got, ref, dtype, (case, "gs3d", dtype, N, C, D, H, W, Do, Ho, Wo, interp, pad, align, cl))
+
+
+def _as_view(torch, rng, t, kind):
+    """a tensor with the values and shape of `t` and another memory layout: 1 = a strided window of a larger
+    buffer (offset, steps, padding), 2 = dimensions stored in another order; returns (view, backing buffer)"""
+    if kind == 1:
+        steps = [int(rng.integers(1, 3)) for _ in t.shape]
+        offs = [int(rng.integers(0, 3)) for _ in t.shape]
+        big = torch.full([o + s * n + int(rng.integers(0, 2)) for o, s, n in zip(offs, steps, t.shape)], 77.0,
+                         dtype=t.dtype, device=t.device)
+        view = big[tuple(slice(o, o + s * n, s) for o, s, n in zip(offs, steps, t.shape))]
+        view.copy_(t)
+        return view, big
+    if kind == 2:
+        perm = [int(i) for i in rng.permutation(t.dim())]
+        inv = [perm.index(i) for i in range(t.dim())]
+        back = t.permute(perm).contiguous()
+        return back.permute(inv), back
+    return t, t
+
+
+def test_random_views(oracle, device, aclnn):
+    """every operand of every entry point as a non-contiguous view: strided windows with offsets, permuted storage;
+    results land in the view and nowhere else"""
+    import torch
+    rng = np.random.default_rng(9005 + SEED_SHIFT)
+
+    def views(*arrays_and_dtype):
+        *arrays, dtype = arrays_and_dtype
+        return [_as_view(torch, rng, I.to_torch(a, dtype, device), int(rng.integers(0, 3)))[0] for a in arrays]
+
+    def out_view(shape, like):
+        kind = int(rng.integers(0, 3))
+        view, big = _as_view(torch, rng, torch.full(shape, 55.0, dtype=like.dtype, device=device), kind)
+        return view, big, kind
+
+    def check_untouched(big, view, kind, what):
+        if kind == 1:   # everything outside the window still holds the fill value
+            probe = big.clone()
+            view_in_probe = probe.as_strided(view.shape, view.stride(), view.storage_offset())
+            view_in_probe.fill_(77.0)
+            assert bool((probe == 77.0).all()), what
+
+    for case in range(90):
+        dtype = I.DTYPES[case % 3]
+        op = case % 6
+        N, C = int(rng.integers(1, 3)), int(rng.integers(1, 10))
+        H, W = _dims(rng, 1, 40, 2)
+        Ho, Wo = _dims(rng, 1, 40, 2)
+        interp, pad, align = int(rng.integers(0, 3)), int(rng.integers(0, 3)), bool(rng.integers(0, 2))
+        _say("views", op, dtype, N, C, H, W, Ho, Wo, interp, pad, align)
+        x = I.cast_np(rng.standard_normal((N, C, H, W)).astype(np.float32), dtype)
+        g = I.cast_np(rng.uniform(-1.3, 1.3, (N, Ho, Wo, 2)).astype(np.float32), dtype)
+        what = (case, op, dtype, N, C, H, W, Ho, Wo, interp, pad, align)
+        if op == 0:
+            ref = oracle.grid_sampler2d(x, g, interp, pad, align, dtype=I.oracle_code(dtype))
+            xt, gt = views(x, g, dtype)
+            out, big, kind = out_view((N, C, Ho, Wo), xt)
+            aclnn.grid_sampler2d(xt, gt, interp, pad, align, out=out)
+            torch.cuda.synchronize()
+            _same(I.from_torch(out.contiguous(), dtype), ref, dtype, what)
+            check_untouched(big, out, kind, what)
+        elif op == 1:
+            ref = oracle.upsample_bilinear2d(x, (Ho, Wo), align, dtype=I.oracle_code(dtype))
+            (xt,) = views(x, dtype)
+            out, big, kind = out_view((N, C, Ho, Wo), xt)
+            aclnn.upsample_bilinear2d(xt, (Ho, Wo), align, out=out)
+            torch.cuda.synchronize()
+            _same(I.from_torch(out.contiguous(), dtype), ref, dtype, what)
+            check_untouched(big, out, kind, what)
+        elif op == 2:
+            ref = oracle.resize_nearest(x, (Ho, Wo), dtype=I.oracle_code(dtype))
+            (xt,) = views(x, dtype)
+            out, big, kind = out_view((N, C, Ho, Wo), xt)
+            try:
+                aclnn.resize(xt, (1.0, 1.0, Ho / H, Wo / W), "nearest", out=out)
+            except aclnn.AclnnError:
+                continue
+            torch.cuda.synchronize()
+            _same(I.from_torch(out.contiguous(), dtype), ref, dtype, what)
+            check_untouched(big, out, kind, what)
+        elif op == 3:
+            go = I.cast_np(rng.standard_normal((N, C, Ho, Wo)).astype(np.float32), dtype)
+            rdx, rdg = oracle.grid_sampler2d_backward(go, x, g, interp, pad, align, dtype=I.oracle_code(dtype))
+            got, xt, gt = views(go, x, g, dtype)
+            dx, bigx, kx = out_view((N, C, H, W), xt)
+            dg, bigg, kg = out_view((N, Ho, Wo, 2), xt)
+            aclnn.grid_sampler2d_backward(got, xt, gt, interp, pad, align, input_grad=dx, grid_grad=dg)
+            torch.cuda.synchronize()
+            _same(I.from_torch(dx.contiguous(), dtype), rdx, dtype, what + ("dx",))
+            _same(I.from_torch(dg.contiguous(), dtype), rdg, dtype, what + ("dgrid",))
+            check_untouched(bigx, dx, kx, what)
+            check_untouched(bigg, dg, kg, what)
+        elif op == 4:
+            go = I.cast_np(rng.standard_normal((N, C, Ho, Wo)).astype(np.float32), dtype)
+            ref = oracle.upsample_bilinear2d_backward(go, (H, W), align, dtype=I.oracle_code(dtype))
+            (got,) = views(go, dtype)
+            out, big, kind = out_view((N, C, H, W), got)
+            aclnn.upsample_bilinear2d_backward(got, (N, C, H, W), align, out=out)
+            torch.cuda.synchronize()
+            _same(I.from_torch(out.contiguous(), dtype), ref, dtype, what)
+            check_untouched(big, out, kind, what)
+        else:
+            D, Do = int(rng.integers(1, 7)), int(rng.integers(1, 7))
+            i3 = interp % 2
+            x5 = I.cast_np(rng.standard_normal((N, C, D, H, W)).astype(np.float32), dtype)
+            g5 = I.cast_np(rng.uniform(-1.3, 1.3, (N, Do, Ho, Wo, 3)).astype(np.float32), dtype)
+            ref = oracle.grid_sampler3d(x5, g5, i3, pad, align, dtype=I.oracle_code(dtype))
+            xt, gt = views(x5, g5, dtype)
+            out, big, kind = out_view((N, C, Do, Ho, Wo), xt)
+            aclnn.grid_sampler3d(xt, gt, i3, pad, align, out=out)
+            torch.cuda.synchronize()
+            _same(I.from_torch(out.contiguous(), dtype), ref, dtype, what + (D, Do))
+            check_untouched(big, out, kind, what)
