@@ -386,15 +386,13 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
     // rows visited by each of this wavefront's outgoing rows, and their weights (see tile_sum_fixed)
     constexpr int HQ = 8 / kTileGroups;  // outgoing rows per lane at the largest tile height
     static_assert(HQ * kRowWeights <= 64, "the row weights of a wavefront are packed one per lane");
-    int32_t hy_start[HQ], hy_n[HQ];
     float lerp_pack = 0.0f;  // lane q * kRowWeights + j: weight of visited row j of outgoing row q (a uniform table)
+    int32_t meta_pack = -1;  // lane q: rows outgoing row q visits (-1: no such row in this tile); lane 8 + q: the first
     bool rows_fixed = true;
     const int32_t lane_id = (int32_t)threadIdx.x & 63;
 #pragma unroll
     for (int q = 0; q < HQ; q++) {
         const int32_t H = __builtin_amdgcn_readfirstlane(H0 + ty + q * kTileGroups);
-        hy_start[q] = 0;
-        hy_n[q] = -1;  // no such row in this tile
         if (H < H0 + tile_rows && H < Hs) {
             const int32_t start = first_visit(H, inv_scale_h, Hd);
             float out_y = ((float)start + offset) * scale_h - offset;
@@ -406,9 +404,8 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
                 n++;
                 out_y += scale_h;
             }
-            hy_start[q] = __builtin_amdgcn_readfirstlane(start);
-            hy_n[q] = __builtin_amdgcn_readfirstlane(n);
-            rows_fixed = rows_fixed && (hy_n[q] <= kRowWeights);
+            meta_pack = (lane_id == q) ? n : ((lane_id == 8 + q) ? start : meta_pack);
+            rows_fixed = rows_fixed && (__builtin_amdgcn_readfirstlane(n) <= kRowWeights);
         }
     }
 
@@ -446,13 +443,19 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
         }
         if (col_ok && use_lds && rows_fixed && nx_max <= 6) {
             TO* yp = y + (pl * Hs + H0 + ty) * (int64_t)Ws + W;
+            // -0 in a vector register: with the row weight in a scalar one, a second scalar operand would be copied
+            // into a vector register before every product
+            const float neg_zero_v = as_fp32_value(neg_zero);
             auto one_row = [&](auto qc) {
                 constexpr int q = decltype(qc)::value;
-                if (hy_n[q] >= 0) {
-                    const float* lane_rows = tile + (hy_start[q] - tile_y0) * pitch + x_base;
+                // read where they are used: kept in scalar registers from the set-up on, they would be spilled
+                const int32_t n_rows = __builtin_amdgcn_readlane(meta_pack, q);
+                if (n_rows >= 0) {
+                    const int32_t first_row = __builtin_amdgcn_readlane(meta_pack, 8 + q);
+                    const float* lane_rows = tile + (first_row - tile_y0) * pitch + x_base;
                     float acc;
 #define OPSCV_TILE_SUM(KX, KMIN) \
-    tile_sum_fixed<KX, KMIN, q>(lane_rows, pitch, hy_n[q], lerp_pack, nx, xl, neg_zero)
+    tile_sum_fixed<KX, KMIN, q>(lane_rows, pitch, n_rows, lerp_pack, nx, xl, neg_zero_v)
                     if (nx_max <= 4) {
                         acc = (nx_min >= 4) ? OPSCV_TILE_SUM(4, 4) : OPSCV_TILE_SUM(4, 0);
                     } else if (nx_max <= 5) {
