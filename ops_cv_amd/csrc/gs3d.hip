@@ -16,6 +16,8 @@
 // them changes no bit of the result.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "kernels.hpp"
 #include "sampler_math.hpp"
 
@@ -163,6 +165,54 @@ __global__ __launch_bounds__(kThreads) void gs3d_kernel(const T* __restrict__ x,
         ok[k] = vd && vh && vw;
         const int32_t d = (k & 4) ? d1 : d0, h = (k & 2) ? h1 : h0, w = (k & 1) ? w1 : w0;
         off[k] = ok[k] ? (int64_t)d * in_plane + h * p.Win + w : 0;
+    }
+    if (p.Win >= 2) {
+        // The two corners of a row, w0 and w0 + 1, are neighbours in memory: one load of two elements (aligned to one
+        // element only, which global memory accesses allow) instead of two loads halves the number of addresses the
+        // gather puts through the memory pipeline, which is what bounds it.  The pair is taken at column
+        // pb = clamp(w0, 0, Win - 2) so that it never leaves the row; which half is which corner follows from pb.
+        const int32_t pb = (w0 < 0) ? 0 : ((w0 > p.Win - 2) ? p.Win - 2 : w0);
+        const bool lo_is_w0 = (w0 == pb), lo_is_w1 = (w1 == pb);  // else the high half (or the corner is outside)
+        int64_t poff[4];
+        bool pok[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const bool vd = (r & 2) ? vd1 : vd0;
+            const bool vh = (r & 1) ? vh1 : vh0;
+            const int32_t d = (r & 2) ? d1 : d0, h = (r & 1) ? h1 : h0;
+            pok[r] = vd && vh && (vw0 || vw1);
+            poff[r] = pok[r] ? (int64_t)d * in_plane + h * p.Win + pb : 0;
+        }
+        // the pair as one integer of twice the element size, so that it is fetched by a single load instruction
+        using PairBits = typename std::conditional<sizeof(T) == 2, uint32_t, uint64_t>::type;
+        for (int32_t c = c_begin; c < c_end; c++) {
+            PairBits pr[4];
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                pr[r] = 0;
+                if (pok[r]) {
+                    __builtin_memcpy(&pr[r], xc + poff[r], sizeof(PairBits));
+                }
+            }
+            float v[8];
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                T halves[2];
+                __builtin_memcpy(halves, &pr[r], sizeof(PairBits));
+                const float lo = ElemIO<T>::load(&halves[0]), hi = ElemIO<T>::load(&halves[1]);
+                v[2 * r] = ok[2 * r] ? (lo_is_w0 ? lo : hi) : 0.0f;
+                v[2 * r + 1] = ok[2 * r + 1] ? (lo_is_w1 ? lo : hi) : 0.0f;
+            }
+            float acc = v[0] * wt[0];
+#pragma unroll
+            for (int k = 1; k < 8; k++) {
+                acc += v[k] * wt[k];
+            }
+            ElemIO<T>::store(yc, acc);
+            xc += in_vol;
+            yc += p.out_vol;
+        }
+        return;
     }
     for (int32_t c = c_begin; c < c_end; c++) {
         float v[8];
