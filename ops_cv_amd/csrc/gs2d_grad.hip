@@ -21,6 +21,8 @@
 // (grid_sampler2_d_grad_simt_det.h:103-196,279-343); no atomics are involved.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "gs2d_grad_math.hpp"
 #include "kernels.hpp"
 
@@ -262,6 +264,39 @@ __global__ __launch_bounds__(kThreads) void gs2d_grad_grid_kernel(const T* __res
             }
         };
         int32_t c = 0;
+        if (p.W >= 2) {
+            // The west and east corner of a row are neighbours in memory: one load of two elements (aligned to one
+            // element only) per row instead of two loads halves the addresses the gather puts through the memory
+            // pipeline.  The pair sits at column pb = clamp(x0, 0, W - 2), so it never leaves the row; which half is
+            // which corner follows from pb.  Corners outside the image are skipped by accumulate() as before.
+            using PairBits = typename std::conditional<sizeof(T) == 2, uint32_t, uint64_t>::type;
+            const int32_t x0 = tp.x0, x1 = (tp.x0 == INT32_MAX) ? tp.x0 : tp.x0 + 1;
+            const int32_t y1 = (tp.y0 == INT32_MAX) ? tp.y0 : tp.y0 + 1;
+            const int32_t pb = (x0 < 0) ? 0 : ((x0 > p.W - 2) ? p.W - 2 : x0);
+            const bool lo_w = (x0 == pb), lo_e = (x1 == pb);
+            const int32_t r0 = (tp.y0 >= 0 && tp.y0 < p.H) ? tp.y0 * p.W + pb : 0;
+            const int32_t r1 = (y1 >= 0 && y1 < p.H) ? y1 * p.W + pb : 0;
+            for (; c + U <= p.C; c += U) {
+                float go[U];
+                PairBits north[U], south[U];
+#pragma unroll
+                for (int u = 0; u < U; u++) {
+                    const T* xc = x_n + (int64_t)(c + u) * plane_px;
+                    go[u] = ElemIO<T>::load(go_n + (int64_t)(c + u) * points);
+                    __builtin_memcpy(&north[u], xc + r0, sizeof(PairBits));
+                    __builtin_memcpy(&south[u], xc + r1, sizeof(PairBits));
+                }
+#pragma unroll
+                for (int u = 0; u < U; u++) {
+                    T n2[2], s2[2];
+                    __builtin_memcpy(n2, &north[u], sizeof(PairBits));
+                    __builtin_memcpy(s2, &south[u], sizeof(PairBits));
+                    const float nlo = ElemIO<T>::load(&n2[0]), nhi = ElemIO<T>::load(&n2[1]);
+                    const float slo = ElemIO<T>::load(&s2[0]), shi = ElemIO<T>::load(&s2[1]);
+                    accumulate(go[u], lo_w ? nlo : nhi, lo_e ? nlo : nhi, lo_w ? slo : shi, lo_e ? slo : shi);
+                }
+            }
+        }
         for (; c + U <= p.C; c += U) {
             float go[U], v[U][4];
 #pragma unroll
