@@ -10,6 +10,8 @@
 // registers across the channel loop.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include <cstdlib>
 
 #include "gs2d_common.hpp"
@@ -29,9 +31,12 @@ template <typename T, int INTERP, int PAD, bool ALIGN>
 __global__ __launch_bounds__(kDirectThreads) void gs2d_direct_kernel(const T* __restrict__ x,
                                                                       const T* __restrict__ grid,
                                                                       T* __restrict__ y, int64_t total_pixels,
-                                                                      int32_t C, int32_t H, int32_t W,
-                                                                      int64_t out_plane)
+                                                                      int32_t C_all, int32_t H, int32_t W,
+                                                                      int64_t out_plane, int32_t chan_chunk)
 {
+    // blockIdx.y selects a run of channels: with few output pixels the channels are what fills the GPU
+    const int32_t c_first = (int32_t)blockIdx.y * chan_chunk;
+    const int32_t C = (c_first + chan_chunk < C_all) ? chan_chunk : C_all - c_first;
     const int64_t in_plane = (int64_t)H * W;
     const int64_t stride = (int64_t)gridDim.x * kDirectThreads;
     for (int64_t p = (int64_t)blockIdx.x * kDirectThreads + threadIdx.x; p < total_pixels; p += stride) {
@@ -39,8 +44,8 @@ __global__ __launch_bounds__(kDirectThreads) void gs2d_direct_kernel(const T* __
         const int64_t rem = p - n * out_plane;
         const float gx = ElemIO<T>::load(grid + 2 * p);
         const float gy = ElemIO<T>::load(grid + 2 * p + 1);
-        const T* xp = x + n * C * in_plane;
-        T* yp = y + n * C * out_plane + rem;
+        const T* xp = x + (n * C_all + c_first) * in_plane;
+        T* yp = y + (n * C_all + c_first) * out_plane + rem;
         if constexpr (INTERP == 2) {
             // grid_sampler2_d_simt.h:375-458
             const BicubicTap b = decide_bicubic<PAD, ALIGN>(gx, gy, H, W);
@@ -100,6 +105,51 @@ __global__ __launch_bounds__(kDirectThreads) void gs2d_direct_kernel(const T* __
             const int64_t o_ne = in_ne ? (int64_t)y0 * W + x1 : 0;
             const int64_t o_sw = in_sw ? (int64_t)y1 * W + x0 : 0;
             const int64_t o_se = in_se ? (int64_t)y1 * W + x1 : 0;
+            if (W >= 2) {
+                // The west and east corner of a row are neighbours in memory: one load of two elements (aligned to
+                // one element only, which global memory accesses allow) per row instead of two loads halves the
+                // addresses the gather puts through the memory pipeline, which is what bounds it.  The pair sits at
+                // column pb = clamp(x0, 0, W - 2), so it never leaves the row; which half is which corner follows
+                // from pb.  Same sums in the same order.
+                using PairBits = typename std::conditional<sizeof(T) == 2, uint32_t, uint64_t>::type;
+                const int32_t pb = (x0 < 0) ? 0 : ((x0 > W - 2) ? W - 2 : x0);
+                const bool lo_w = (x0 == pb), lo_e = (x1 == pb);
+                const bool row_n = in_nw || in_ne, row_s = in_sw || in_se;
+                const int64_t o_n = row_n ? (int64_t)y0 * W + pb : 0;
+                const int64_t o_s = row_s ? (int64_t)y1 * W + pb : 0;
+#pragma unroll 4
+                for (int32_t c = 0; c < C; c++) {
+                    PairBits north = 0, south = 0;
+                    if (row_n) {
+                        __builtin_memcpy(&north, xp + o_n, sizeof(PairBits));
+                    }
+                    if (row_s) {
+                        __builtin_memcpy(&south, xp + o_s, sizeof(PairBits));
+                    }
+                    T n2[2], s2[2];
+                    __builtin_memcpy(n2, &north, sizeof(PairBits));
+                    __builtin_memcpy(s2, &south, sizeof(PairBits));
+                    const float nlo = ElemIO<T>::load(&n2[0]), nhi = ElemIO<T>::load(&n2[1]);
+                    const float slo = ElemIO<T>::load(&s2[0]), shi = ElemIO<T>::load(&s2[1]);
+                    float out = 0.0f;
+                    if (in_nw) {
+                        out += (lo_w ? nlo : nhi) * t.w[0];
+                    }
+                    if (in_ne) {
+                        out += (lo_e ? nlo : nhi) * t.w[1];
+                    }
+                    if (in_sw) {
+                        out += (lo_w ? slo : shi) * t.w[2];
+                    }
+                    if (in_se) {
+                        out += (lo_e ? slo : shi) * t.w[3];
+                    }
+                    ElemIO<T>::store(yp, out);
+                    xp += in_plane;
+                    yp += out_plane;
+                }
+                continue;
+            }
 #pragma unroll 4
             for (int32_t c = 0; c < C; c++) {
                 // grid_sampler2_d_simt.h:321-338 : nw, ne, sw, se added in this order, skipped when outside
@@ -200,9 +250,20 @@ template <typename T, int INTERP, int PAD, bool ALIGN>
 hipError_t run_direct(const GridSamplerArgs& a, hipStream_t stream)
 {
     const int64_t total = a.N * a.Hout * a.Wout;
-    hipLaunchKernelGGL((gs2d_direct_kernel<T, INTERP, PAD, ALIGN>), dim3(blocks_for(total, kDirectThreads)),
+    const int blocks = blocks_for(total, kDirectThreads);
+    // a lane walks its channels one after the other, each step waiting for its loads: aim at 8192 workgroups (eight
+    // wavefronts per SIMD) by giving runs of channels to different workgroups when the pixels alone are too few
+    int64_t chunks = (8192 + blocks - 1) / blocks;
+    chunks = chunks < a.C ? chunks : a.C;
+    chunks = chunks < 1 ? 1 : chunks;
+    const int64_t chan_chunk = (a.C + chunks - 1) / chunks;
+    const int64_t grid_y = (a.C + chan_chunk - 1) / chan_chunk;
+    if (grid_y > 65535) {
+        return hipErrorInvalidValue;
+    }
+    hipLaunchKernelGGL((gs2d_direct_kernel<T, INTERP, PAD, ALIGN>), dim3((unsigned)blocks, (unsigned)grid_y),
                        dim3(kDirectThreads), 0, stream, (const T*)a.x, (const T*)a.grid, (T*)a.y, total,
-                       (int32_t)a.C, (int32_t)a.Hin, (int32_t)a.Win, a.Hout * a.Wout);
+                       (int32_t)a.C, (int32_t)a.Hin, (int32_t)a.Win, a.Hout * a.Wout, (int32_t)chan_chunk);
     return hipGetLastError();
 }
 
