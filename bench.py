@@ -45,6 +45,9 @@ GS_WORKLOADS = {
                sets=8),
     "C5": dict(dtype="bf16", x=(8, 128, 128, 128), grid=(8, 256, 256), kind="random", interp=0, pad=1, align=True,
                sets=3),
+    # not a BASELINE configuration: input planes of 4 MB, far beyond LDS, which only the direct kernel serves
+    "L1": dict(dtype="fp16", x=(2, 32, 1080, 1920), grid=(2, 1080, 1920), kind="affine", interp=0, pad=0, align=False,
+               sets=2),
 }
 UP_WORKLOADS = {
     "C2": dict(dtype="fp32", x=(8, 64, 56, 56), out=(112, 112), align=False, scales=(2.0, 2.0), dist="normal",
@@ -593,7 +596,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="C3", help="headline workload: C1..C5, or one of the neighbouring entry points V1 (3-D sampler), G3 "
+    ap.add_argument("--workload", default="C3", help="headline workload: C1..C5, L1 (sampler on 1080p planes), or one of the neighbouring entry points V1 (3-D sampler), G3 "
                          "(sampler backward), B4 (resize backward), R4 (nearest resize)")
     ap.add_argument("--only", action="store_true", help="skip the other workloads and the CPU baseline")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")

@@ -65,6 +65,34 @@ __global__ __launch_bounds__(kDirectThreads) void gs2d_direct_kernel(const T* __
                 row_in[k] = b.by[k] >= 0 && b.by[k] < H;
                 row_off[k] = row_in[k] ? (int64_t)b.by[k] * W : 0;
             }
+            // Away from the left and right edge the four columns of a row are neighbours in memory and inside the
+            // image: one load of four elements (aligned to one element only) instead of four.  Taken when that holds
+            // for every lane of the wavefront, so that the choice costs no divergence.
+            const bool in_a_row = b.bx[0] >= 0 && b.bx[3] < W && b.bx[1] == b.bx[0] + 1 && b.bx[2] == b.bx[0] + 2 &&
+                                  b.bx[3] == b.bx[0] + 3;
+            if (__builtin_amdgcn_ballot_w64(!in_a_row) == 0) {
+                for (int32_t c = 0; c < C; c++) {
+                    float r[4];
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        r[j] = 0.0f;
+                        if (row_in[j]) {
+                            uint64_t bits[sizeof(T) / 2];  // 8 bytes for 16-bit elements, 16 for fp32
+                            __builtin_memcpy(bits, xp + row_off[j] + b.bx[0], 4 * sizeof(T));
+                            T q[4];
+                            __builtin_memcpy(q, bits, 4 * sizeof(T));
+                            r[j] = bicubic_weighted_sum(b.cx[0], b.cx[1], b.cx[2], b.cx[3], ElemIO<T>::load(&q[0]),
+                                                        ElemIO<T>::load(&q[1]), ElemIO<T>::load(&q[2]),
+                                                        ElemIO<T>::load(&q[3]));
+                        }
+                    }
+                    ElemIO<T>::store(yp,
+                                     bicubic_weighted_sum(b.cy[0], b.cy[1], b.cy[2], b.cy[3], r[0], r[1], r[2], r[3]));
+                    xp += in_plane;
+                    yp += out_plane;
+                }
+                continue;
+            }
             for (int32_t c = 0; c < C; c++) {
                 float r[4];
 #pragma unroll
