@@ -11,6 +11,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdlib>
+#include <type_traits>
 
 #include "kernels.hpp"
 #include "resize_band_lds_kernel.hpp"
@@ -63,7 +64,7 @@ __global__ __launch_bounds__(kThreads) void resize_nchw_generic_kernel(const T* 
     }
 }
 
-// Row-band variant for NCHW when the output row is a whole number of 16-byte vectors.
+// Row-band variant for NCHW, any width.
 //
 // A lane owns V = 16/sizeof(T) consecutive output columns and walks down a band of output rows.  The column
 // taps (two source offsets and the lambda per column) are computed once per lane.  The reference formula
@@ -71,7 +72,10 @@ __global__ __launch_bounds__(kThreads) void resize_nchw_generic_kernel(const T* 
 // is separable as written: the two inner terms depend on the source row only, so the horizontally blended
 // source row  Hrow(y)[col] = (1-dx)*x[y,x0] + dx*x[y,x1]  is kept in registers and reused by every output row
 // that touches source row y (two of them for a x2 upscale) -- same operations, same order, same bits.
-// Each lane writes one 16-byte vector per output row; a wavefront writes 1 KiB contiguous.
+// The two taps of a column are the same element or neighbours: they are fetched as one load of two elements
+// (aligned to one element only, which global memory accesses allow) at column min(x0, Ws - 2).  Each lane writes
+// one 16-byte vector per output row, at whatever alignment the row has (again element-aligned: rows of a width that
+// is not a multiple of V start anywhere); the lane that holds the ragged end of a row stores its elements singly.
 template <typename T, bool HALF_PIXEL, int BAND>
 __global__ __launch_bounds__(kThreads) void resize_nchw_band_kernel(const T* __restrict__ x, T* __restrict__ y,
                                                                      int64_t planes, int32_t Hs, int32_t Ws,
@@ -79,19 +83,30 @@ __global__ __launch_bounds__(kThreads) void resize_nchw_band_kernel(const T* __r
                                                                      float scale_w, int raw_lambda)
 {
     constexpr int V = 16 / (int)sizeof(T);
+    using PairBits = typename std::conditional<sizeof(T) == 2, uint32_t, uint64_t>::type;
     const int32_t chunk = blockIdx.x * kThreads + threadIdx.x;
     const int32_t col0 = chunk * V;
     if (col0 >= Wd) {
         return;
     }
-    int32_t xo0[V], xo1[V];
+    const int32_t nvalid = (Wd - col0 < V) ? Wd - col0 : V;
+    const bool pairs = Ws >= 2;
+    int32_t xo0[V], xo1[V];  // pairs: xo0 = column of the pair; else the two tap columns
+    uint32_t left_is_lo = 0, right_is_lo = 0;
     float dx[V];
 #pragma unroll
     for (int i = 0; i < V; i++) {
-        const AxisTap t = axis_tap<HALF_PIXEL>(col0 + i, scale_w, Ws, raw_lambda);
+        const int32_t c = (col0 + i < Wd) ? col0 + i : Wd - 1;
+        const AxisTap t = axis_tap<HALF_PIXEL>(c, scale_w, Ws, raw_lambda);
         xo0[i] = t.i0;
         xo1[i] = t.i1;
         dx[i] = t.lambda;
+        if (pairs) {
+            const int32_t pb = (t.i0 < Ws - 2) ? t.i0 : Ws - 2;
+            left_is_lo |= (uint32_t)(t.i0 == pb) << i;
+            right_is_lo |= (uint32_t)(t.i1 == pb) << i;
+            xo0[i] = pb;
+        }
     }
     const int32_t h_begin = blockIdx.y * BAND;
     const int32_t h_end = (h_begin + BAND < Hd) ? h_begin + BAND : Hd;
@@ -103,11 +118,28 @@ __global__ __launch_bounds__(kThreads) void resize_nchw_band_kernel(const T* __r
         int32_t ya = -1, yb = -1;
         auto blend_row = [&](float* hrow, int32_t ys) {
             const T* row = xp + (int64_t)ys * Ws;
+            if (pairs) {
+                PairBits pr[V];
 #pragma unroll
-            for (int i = 0; i < V; i++) {
-                const float l = ElemIO<T>::load(row + xo0[i]);
-                const float r = ElemIO<T>::load(row + xo1[i]);
-                hrow[i] = (1.0f - dx[i]) * l + dx[i] * r;
+                for (int i = 0; i < V; i++) {
+                    __builtin_memcpy(&pr[i], row + xo0[i], sizeof(PairBits));
+                }
+#pragma unroll
+                for (int i = 0; i < V; i++) {
+                    T two[2];
+                    __builtin_memcpy(two, &pr[i], sizeof(PairBits));
+                    const float lo = ElemIO<T>::load(&two[0]), hi = ElemIO<T>::load(&two[1]);
+                    const float l = ((left_is_lo >> i) & 1u) ? lo : hi;
+                    const float r = ((right_is_lo >> i) & 1u) ? lo : hi;
+                    hrow[i] = (1.0f - dx[i]) * l + dx[i] * r;
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < V; i++) {
+                    const float l = ElemIO<T>::load(row + xo0[i]);
+                    const float r = ElemIO<T>::load(row + xo1[i]);
+                    hrow[i] = (1.0f - dx[i]) * l + dx[i] * r;
+                }
             }
         };
         for (int32_t h = h_begin; h < h_end; h++) {
@@ -139,9 +171,19 @@ __global__ __launch_bounds__(kThreads) void resize_nchw_band_kernel(const T* __r
                 const float o = (1.0f - dy) * ha[i] + dy * bot;
                 ElemIO<T>::store(&outv[i], o);
             }
-            uint4 packed;
-            __builtin_memcpy(&packed, outv, sizeof(packed));
-            *reinterpret_cast<uint4*>(yp) = packed;
+            if (nvalid == V) {
+                typedef uint32_t u32x4_any __attribute__((ext_vector_type(4), aligned(2)));
+                u32x4_any packed;
+                __builtin_memcpy(&packed, outv, sizeof(packed));
+                *reinterpret_cast<u32x4_any*>(yp) = packed;
+            } else {
+#pragma unroll
+                for (int i = 0; i < V; i++) {
+                    if (i < nvalid) {
+                        yp[i] = outv[i];
+                    }
+                }
+            }
             yp += Wd;
         }
     }
@@ -575,16 +617,14 @@ __global__ __launch_bounds__(kThreads) void resize_fill_kernel(const T* __restri
 
 constexpr int kBand = 32;  // output rows a workgroup walks down (vertical reuse of blended source rows)
 
-// The band variant stores whole 16-byte vectors: needs Wd to be a multiple of the vector length, a 16-byte
-// aligned output and a band count that fits the grid.
+// The band variant serves every NCHW shape whose band count fits the grid (its vector stores are element-aligned).
 template <typename T>
 bool band_variant_ok(const ResizeArgs& a)
 {
-    constexpr int V = 16 / (int)sizeof(T);
     if (a.channels_last || a.mode != ResizeMode::Bilinear) {
         return false;
     }
-    if (a.Wd % V != 0 || reinterpret_cast<uintptr_t>(a.y) % 16 != 0) {
+    if (reinterpret_cast<uintptr_t>(a.x) % sizeof(T) != 0 || reinterpret_cast<uintptr_t>(a.y) % sizeof(T) != 0) {
         return false;
     }
     if ((a.Hd + kBand - 1) / kBand > 65535) {
@@ -778,7 +818,7 @@ hipError_t run_resize(const ResizeArgs& a, hipStream_t stream)
     }
     if (band_variant_ok<T>(a)) {
         constexpr int V = 16 / (int)sizeof(T);
-        const int64_t chunks = a.Wd / V;
+        const int64_t chunks = (a.Wd + V - 1) / V;
         const int64_t bands = (a.Hd + kBand - 1) / kBand;
         dim3 grid((unsigned)((chunks + kThreads - 1) / kThreads), (unsigned)bands,
                   (unsigned)(planes < 65535 ? planes : 65535));
