@@ -59,8 +59,13 @@ BandPlan make_plan(const ResizeArgs& a)
     if (a.channels_last || a.mode != ResizeMode::Bilinear) {
         return bp;
     }
-    // whole 16-byte output vectors, 16-byte aligned output, 32-bit row byte offsets
-    if (a.Wd % V != 0 || reinterpret_cast<uintptr_t>(a.y) % 16 != 0 || a.Wd * (int64_t)sizeof(T) >= (1ll << 31)) {
+    // element-aligned output (the vector stores are), 32-bit row byte offsets
+    if (reinterpret_cast<uintptr_t>(a.y) % sizeof(T) != 0 || a.Wd * (int64_t)sizeof(T) >= (1ll << 31)) {
+        return bp;
+    }
+    // short rows leave most of this kernel's lanes idle; the flat variant that serves them takes whole vectors only,
+    // so short ragged rows are left to the register-band kernel
+    if (a.Wd % V != 0 && a.Wd / V <= 128) {
         return bp;
     }
     const uintptr_t xa = reinterpret_cast<uintptr_t>(a.x);
@@ -73,7 +78,7 @@ BandPlan make_plan(const ResizeArgs& a)
         return bp;
     }
     // one workgroup spans the whole output row when it fits in 512 lanes (fewer, longer row segments)
-    const int kThreads = (a.Wd / V > 256) ? 512 : 256;
+    const int kThreads = ((a.Wd + V - 1) / V > 256) ? 512 : 256;
     bp.threads = kThreads;
     int32_t rows = 0, seg = 0;
     if (a.half_pixel) {

@@ -13,7 +13,8 @@
 //     same order, so the result is bit-identical to the per-pixel evaluation.
 //   * Row taps (y0, y1, dy) of the band are computed by the first BAND lanes once and broadcast per row.
 //   * Each lane writes one 16-byte vector per output row through a buffer descriptor (lanes past the row end
-//     are dropped by its range check); a wavefront writes 1 KiB contiguous.
+//     are dropped by its range check; the lane holding the ragged end of a row whose width is not a multiple of V
+//     stores its elements singly); a wavefront writes 1 KiB contiguous.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -95,6 +96,7 @@ __global__ __launch_bounds__(THREADS) void resize_band_lds_kernel(const T* __res
     }
     const uint32_t out_row_bytes = (uint32_t)p.Wd * (uint32_t)sizeof(T);
     const uint32_t out_off = (col0 < p.Wd) ? (uint32_t)col0 * (uint32_t)sizeof(T) : 0x80000000u;
+    const int32_t nvalid = (p.Wd - col0 < V) ? p.Wd - col0 : V;  // output columns of this lane inside the row
     const uint32_t wave = __builtin_amdgcn_readfirstlane((uint32_t)tid >> 6);
     const float neg_zero = p.neg_zero;
 
@@ -178,10 +180,28 @@ __global__ __launch_bounds__(THREADS) void resize_band_lds_kernel(const T* __res
             typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
             u32x4 packed;
             __builtin_memcpy(&packed, outv, sizeof(packed));
-            if (p.streaming) {
-                __builtin_amdgcn_raw_buffer_store_b128(packed, rsrc, (int)out_off, 0, 2);
+            if (nvalid == V) {
+                // rows of a width that is not a multiple of V start anywhere: the store is element-aligned
+                if (p.streaming) {
+                    __builtin_amdgcn_raw_buffer_store_b128(packed, rsrc, (int)out_off, 0, 2);
+                } else {
+                    __builtin_amdgcn_raw_buffer_store_b128(packed, rsrc, (int)out_off, 0, 0);
+                }
             } else {
-                __builtin_amdgcn_raw_buffer_store_b128(packed, rsrc, (int)out_off, 0, 0);
+                // the lane that holds the ragged end of the row stores its elements singly (lanes past the end
+                // have nvalid <= 0 and an offset outside the descriptor's range)
+#pragma unroll
+                for (int i = 0; i < V; i++) {
+                    if (i < nvalid) {
+                        if constexpr (sizeof(T) == 4) {
+                            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, outv[i]), rsrc,
+                                                                  (int)(out_off + i * 4), 0, 0);
+                        } else {
+                            __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(uint16_t, outv[i]), rsrc,
+                                                                  (int)(out_off + i * 2), 0, 0);
+                        }
+                    }
+                }
             }
             yp += p.Wd;
         }
