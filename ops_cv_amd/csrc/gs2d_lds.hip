@@ -10,7 +10,14 @@ LdsPlan make_lds_plan(const GridSamplerArgs& a)
     LdsPlan p;
     const int64_t esz = elem_size(a.elem);
     const int64_t plane_bytes = a.Hin * a.Win * esz;
-    const int64_t need = ((plane_bytes + 15) & ~(int64_t)15) + 16;
+    // planes that start on 16-byte boundaries and are whole 16-byte units are copied as they are; every other
+    // element-aligned plane in the shifted layout (gs2d_lds_kernel.hpp, issue_stage_copy), up to 14 bytes into its slot
+    const uintptr_t xa = reinterpret_cast<uintptr_t>(a.x);
+    const bool plain = plane_bytes % 16 == 0 && xa % 16 == 0;
+    if (!plain && xa % esz != 0) {
+        return p;  // a misaligned tensor: leave it to the direct variant
+    }
+    const int64_t need = ((plane_bytes + (plain ? 0 : 14) + 15) & ~(int64_t)15) + 16;
     const int64_t out_plane = a.Hout * a.Wout;
     // output-plane byte offsets are kept in 32 bits (and below the out-of-range marker 0x80000000)
     if (out_plane * esz >= ((int64_t)1 << 31) || need > kPitch[3]) {
@@ -55,15 +62,7 @@ LdsPlan make_lds_plan(const GridSamplerArgs& a)
     if (a.N * p.tiles_per_n * cblocks > INT32_MAX) {
         return p;
     }
-    // bytes per lane of the global->LDS copy: must divide the plane size and the alignment of the input
-    const uintptr_t xa = reinterpret_cast<uintptr_t>(a.x);
-    if (plane_bytes % 16 == 0 && xa % 16 == 0) {
-        p.copy_gran = 16;
-    } else if (plane_bytes % 4 == 0 && xa % 4 == 0) {
-        p.copy_gran = 4;
-    } else {
-        return p;  // odd byte counts: the asynchronous copy moves whole dwords, leave it to the direct variant
-    }
+    p.copy_gran = plain ? 16 : 2;  // 2: 16-byte units in the shifted layout
     // Bank-spreading layout (gs2d_lds_kernel.hpp): rows of exactly 128 bytes, 16-byte copy granule.  Only for
     // border padding, where clamped coordinates pile up on the first and last column (one bank in the plain
     // layout: 21.2 -> 18.7 us on the fp16 N16 C256 64x64 case).  Elsewhere the plain layout is the better one: the
@@ -97,10 +96,16 @@ hipError_t run_gs2d_lds(const GridSamplerArgs& a, hipStream_t stream, bool* hand
         return hipSuccess;
     }
     *handled = true;
+    const bool shifted = p.copy_gran == 2;
     switch (a.elem) {
-        case Elem::F32: return lds_launch_typed<float>(a, p, stream);
-        case Elem::F16: return lds_launch_typed<_Float16>(a, p, stream);
-        case Elem::BF16: return lds_launch_typed<__bf16>(a, p, stream);
+        case Elem::F32:
+            return shifted ? lds_launch_typed<float, true>(a, p, stream) : lds_launch_typed<float, false>(a, p, stream);
+        case Elem::F16:
+            return shifted ? lds_launch_typed<_Float16, true>(a, p, stream)
+                           : lds_launch_typed<_Float16, false>(a, p, stream);
+        case Elem::BF16:
+            return shifted ? lds_launch_typed<__bf16, true>(a, p, stream)
+                           : lds_launch_typed<__bf16, false>(a, p, stream);
     }
     return hipErrorInvalidValue;
 }

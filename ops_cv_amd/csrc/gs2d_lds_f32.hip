@@ -1,8 +1,8 @@
-// LDS-staged grid sampler kernels for float tensors.
+// LDS-staged grid sampler kernels for float tensors, planes on the 16-byte grid.
 #include "gs2d_lds_launch.hpp"
 
 namespace opscv {
 
-template hipError_t lds_launch_typed<float>(const GridSamplerArgs&, const LdsPlan&, hipStream_t);
+template hipError_t lds_launch_typed<float, false>(const GridSamplerArgs&, const LdsPlan&, hipStream_t);
 
 }  // namespace opscv

@@ -178,8 +178,15 @@ __device__ __forceinline__ uint32_t lds_swizzle(uint32_t byte_off, uint32_t row_
 // granule that divides the plane size and the source alignment.  Each wavefront instruction moves 64*G
 // contiguous bytes; lanes past the end of a plane are masked off.  The LWAVES loader wavefronts share the
 // chunks of every plane round-robin (`lwave` = index of the calling one).  Returns nothing; the number of
-// instructions issued per plane by this wavefront is copies_per_plane() below.
-template <int G, int LWAVES, int CGS, int PITCH>
+// instructions issued per plane by this wavefront is copies_of() in the kernel.
+//
+// SHIFTED (G = 16): planes that do not start on a 16-byte boundary or are not whole 16-byte units -- an odd number of
+// elements per plane, a tensor view that starts anywhere.  The copy of such a plane starts up to 14 bytes early, on
+// the boundary, and ends on the boundary after the plane's last byte, so the plane's first element lands `shift`
+// bytes into its LDS slot; the samplers add the same shift (plane_shift() in the kernel).  The bytes read outside the
+// plane share an aligned 16-byte unit with bytes inside it, so they are readable wherever the plane is; they land
+// in the slot's padding.  The number of copy instructions then depends on the plane: stage_copy_count() below.
+template <int G, int LWAVES, int CGS, int PITCH, bool SHIFTED = false>
 __device__ __forceinline__ void issue_stage_copy(const char* src, char* dst, uint32_t plane_bytes, int nch,
                                                  uint32_t lwave, uint32_t lane, uint32_t lane_src_off)
 {
@@ -190,8 +197,14 @@ __device__ __forceinline__ void issue_stage_copy(const char* src, char* dst, uin
         if (k < nch) {
             const char* sp = src + (size_t)k * plane_bytes;
             char* dp = dst + k * PITCH;
-            for (uint32_t base = lwave * CHUNK; base < plane_bytes; base += LWAVES * CHUNK) {
-                if (base + lane_off < plane_bytes) {
+            uint32_t copy_bytes = plane_bytes;
+            if constexpr (SHIFTED) {
+                const uint32_t shift = (uint32_t)(reinterpret_cast<uintptr_t>(sp) & 15u);
+                sp -= shift;
+                copy_bytes = (shift + plane_bytes + 15u) & ~15u;
+            }
+            for (uint32_t base = lwave * CHUNK; base < copy_bytes; base += LWAVES * CHUNK) {
+                if (base + lane_off < copy_bytes) {
                     // lane_src_off: the chunk of this 1 KiB block that belongs at the lane's LDS position
                     const global_cptr_t gsrc = (global_cptr_t)(sp + base + lane_src_off);
                     const lds_ptr_t ldst = (lds_ptr_t)(dp + base);
@@ -218,7 +231,11 @@ __device__ __forceinline__ void issue_stage_copy(const char* src, char* dst, uin
 // older stores; with the roles split the loader's counter sees copies only, and "stage s has landed" is "at most
 // the copies of the later stages are outstanding".  One workgroup barrier per stage hands the stage over and
 // tells the loaders that the slot sampled before is free again.
-template <typename T, int INTERP, int PAD, bool ALIGN, int SWAVES, int LWAVES, int PPT, int CGS, int NBUF, int PITCH>
+//
+// SHIFTED_PLANES selects the layout for planes off the 16-byte grid (issue_stage_copy); it is a template parameter so
+// that the kernels for whole, aligned planes carry no trace of it.
+template <typename T, int INTERP, int PAD, bool ALIGN, int SWAVES, int LWAVES, int PPT, int CGS, int NBUF, int PITCH,
+          bool SHIFTED_PLANES = false>
 __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves_per_eu(1, 5))) void gs2d_lds_kernel(
     const T* __restrict__ x, const T* __restrict__ grid, T* __restrict__ y, int32_t C, int32_t H, int32_t W,
     int32_t out_plane, uint32_t tiles_per_n, uint32_t cblocks, int32_t chans_per_block, int32_t copy_gran,
@@ -252,7 +269,8 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
 
     const int32_t plane_elems = H * W;
     const uint32_t plane_bytes = (uint32_t)plane_elems * (uint32_t)sizeof(T);
-    const uint32_t zero_off = round_up16(plane_bytes);
+    // behind the plane, which in the shifted layout (copy_gran == 2) may sit up to 14 bytes into its slot
+    const uint32_t zero_off = round_up16(plane_bytes + (SHIFTED_PLANES ? 14u : 0u));
     const int32_t c_begin = (int32_t)cb * chans_per_block;
     const int32_t c_end = (c_begin + chans_per_block < C) ? c_begin + chans_per_block : C;
     const int32_t nchan = c_end - c_begin;
@@ -265,18 +283,35 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
         const char* xb = reinterpret_cast<const char*>(x + ((int64_t)n * C + c_begin) * plane_elems);
         const size_t stage_bytes = (size_t)CGS * plane_bytes;
         // copy instructions this wavefront issues per plane
-        const uint32_t chunk = 64u * (uint32_t)copy_gran;
-        const uint32_t chunks = (plane_bytes + chunk - 1) / chunk;
-        const uint32_t per_plane = (chunks > lwave) ? (chunks - lwave + LWAVES - 1) / LWAVES : 0;
+        constexpr bool shifted = SHIFTED_PLANES;  // 16-byte granule, planes off the 16-byte grid (see issue_stage_copy)
+        const uint32_t chunk = 64u * (uint32_t)(shifted ? 16 : copy_gran);
         auto planes_of = [&](int32_t s) {
             const int32_t left = nchan - s * CGS;
             return left < CGS ? left : CGS;
+        };
+        // copy instructions this wavefront issues per plane (whole planes: the same for every plane)
+        const uint32_t chunks = (plane_bytes + chunk - 1) / chunk;
+        const uint32_t per_plane = (chunks > lwave) ? (chunks - lwave + LWAVES - 1) / LWAVES : 0;
+        // ... and for the planes of stage s in the shifted layout, where a plane's copy starts `shift` bytes early and
+        // is rounded out to 16-byte units, so that the count depends on the plane
+        const uint32_t xb_low = (uint32_t)(reinterpret_cast<uintptr_t>(xb) & 15u);
+        auto shifted_copy_count = [&](int32_t s) -> uint32_t {
+            uint32_t total = 0;
+            for (int32_t k = 0; k < planes_of(s); k++) {
+                const uint32_t shift = (xb_low + (uint32_t)(s * CGS + k) * (plane_bytes & 15u)) & 15u;
+                const uint32_t units = (((shift + plane_bytes + 15u) & ~15u) + chunk - 1) / chunk;
+                total += (units > lwave) ? (units - lwave + LWAVES - 1) / LWAVES : 0;
+            }
+            return total;
         };
         const uint32_t lane_src16 = lds_swizzle(lane * 16u, (PAD == 1) ? (uint32_t)row_shift : 0u);
         auto start_stage = [&](int32_t s, int slot) {
             const char* src = xb + (size_t)s * stage_bytes;
             char* dst = lds + slot * SLOT_BYTES;
-            if (copy_gran == 16) {
+            if constexpr (shifted) {
+                issue_stage_copy<16, LWAVES, CGS, PITCH, true>(src, dst, plane_bytes, planes_of(s), lwave, lane,
+                                                               lane * 16u);
+            } else if (copy_gran == 16) {
                 issue_stage_copy<16, LWAVES, CGS, PITCH>(src, dst, plane_bytes, planes_of(s), lwave, lane, lane_src16);
             } else {
                 issue_stage_copy<4, LWAVES, CGS, PITCH>(src, dst, plane_bytes, planes_of(s), lwave, lane, lane * 4u);
@@ -291,11 +326,19 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
         int slot = 0;
         for (int32_t s = 0; s < nstages; s++) {
             // outstanding after stage s has landed: the copies of stages s+1 .. min(s+DEPTH, nstages)-1
-            int32_t later_planes = 0;
-            for (int32_t q = s + 1; q < s + DEPTH && q < nstages; q++) {
-                later_planes += planes_of(q);
+            if constexpr (shifted) {
+                uint32_t later_copies = 0;
+                for (int32_t q = s + 1; q < s + DEPTH && q < nstages; q++) {
+                    later_copies += shifted_copy_count(q);
+                }
+                wait_vmcnt(later_copies);
+            } else {
+                int32_t later_planes = 0;
+                for (int32_t q = s + 1; q < s + DEPTH && q < nstages; q++) {
+                    later_planes += planes_of(q);
+                }
+                wait_vmcnt((uint32_t)later_planes * per_plane);
             }
-            wait_vmcnt((uint32_t)later_planes * per_plane);
             lds_barrier();
             if (s + DEPTH < nstages) {
                 int refill = slot + DEPTH;
@@ -423,7 +466,23 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
     const uint32_t out_plane_bytes = (uint32_t)out_plane * (uint32_t)sizeof(T);
 
     // `buf` is the byte offset of the stage's slot inside the ring
+    // the bytes by which a plane's copy started early (SHIFTED_PLANES, see issue_stage_copy): the low four bits of the
+    // plane's first byte address, from those of the tensor's address and of the plane size
+    const uint32_t addr_low = (uint32_t)(reinterpret_cast<uintptr_t>(x) & 15u);
+    const uint32_t size_low = plane_bytes & 15u;
+    const uint32_t first_plane = (uint32_t)n * (uint32_t)C + (uint32_t)c_begin;
+    // The shift makes the plane distance a run-time value where it is a literal otherwise (one more add per tap).
     auto sample_stage = [&](int32_t s, uint32_t buf) {
+        constexpr bool SHIFTED = SHIFTED_PLANES;
+        auto plane_shift = [&](int32_t stage, int k) -> uint32_t {
+            if constexpr (SHIFTED) {
+                return (addr_low + (first_plane + (uint32_t)(stage * CGS + k)) * size_low) & 15u;
+            } else {
+                (void)stage;
+                (void)k;
+                return 0u;
+            }
+        };
         const int32_t left = nchan - s * CGS;
         T* ys = yb + (int64_t)s * CGS * out_plane;
         if (left >= CGS) {
@@ -432,14 +491,14 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
             T raw[2][PPT][NT];
 #pragma unroll
             for (int j = 0; j < PPT; j++) {
-                load_taps<T, NT>(buf, toff[j], raw[0][j]);
+                load_taps<T, NT>(buf + plane_shift(s, 0), toff[j], raw[0][j]);
             }
 #pragma unroll
             for (int k = 0; k < CGS; k++) {
                 if (k + 1 < CGS) {
 #pragma unroll
                     for (int j = 0; j < PPT; j++) {
-                        load_taps<T, NT>(buf + (k + 1) * PITCH, toff[j], raw[(k + 1) & 1][j]);
+                        load_taps<T, NT>(buf + (k + 1) * PITCH + plane_shift(s, k + 1), toff[j], raw[(k + 1) & 1][j]);
                     }
                 }
                 const __amdgpu_buffer_rsrc_t rsrc =
@@ -456,7 +515,7 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
                 T raw[PPT][NT];
 #pragma unroll
                 for (int j = 0; j < PPT; j++) {
-                    load_taps<T, NT>(buf + k * PITCH, toff[j], raw[j]);
+                    load_taps<T, NT>(buf + k * PITCH + plane_shift(s, k), toff[j], raw[j]);
                 }
 #pragma unroll
                 for (int j = 0; j < PPT; j++) {

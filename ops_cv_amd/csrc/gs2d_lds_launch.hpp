@@ -1,5 +1,6 @@
 // Grid sampler 2-D forward, LDS-staged variant: launch plan and the typed launch template.
-// The three element types are instantiated in separate translation units so that they compile in parallel.
+// The element types, and for each the two plane layouts, are instantiated in separate translation units so that they
+// compile in parallel.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -34,10 +35,10 @@ constexpr int kNbuf[4] = {4, 4, 4, 2};  // ring slots (stages resident in LDS)
 
 LdsPlan make_lds_plan(const GridSamplerArgs& a);
 
-template <typename T, int I, int P, bool A, int PPT, int CGS, int NBUF, int PITCH, int LWAVES>
+template <typename T, int I, int P, bool A, int PPT, int CGS, int NBUF, int PITCH, int LWAVES, bool SHIFTED>
 hipError_t launch_one(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t stream)
 {
-    auto kernel = gs2d_lds_kernel<T, I, P, A, kSamplerWaves, LWAVES, PPT, CGS, NBUF, PITCH>;
+    auto kernel = gs2d_lds_kernel<T, I, P, A, kSamplerWaves, LWAVES, PPT, CGS, NBUF, PITCH, SHIFTED>;
     static bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -57,15 +58,15 @@ hipError_t launch_one(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t st
     return hipGetLastError();
 }
 
-template <typename T, int I, int P, bool A, int CLS, int PPT>
+template <typename T, int I, int P, bool A, int CLS, int PPT, bool SHIFTED>
 hipError_t launch_cls(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t stream)
 {
-    return launch_one<T, I, P, A, PPT, kCgs[CLS], kNbuf[CLS], kPitch[CLS], kLoaderWaves[CLS]>(a, p, stream);
+    return launch_one<T, I, P, A, PPT, kCgs[CLS], kNbuf[CLS], kPitch[CLS], kLoaderWaves[CLS], SHIFTED>(a, p, stream);
 }
 
 // Expands (interp, pad, align, size class, pixels per lane) for one element type and launches.  Eight pixels per
 // lane exist for the two large-plane classes only.
-template <typename T>
+template <typename T, bool SHIFTED>
 struct LdsTypedLauncher {
     const GridSamplerArgs& a;
     const LdsPlan& p;
@@ -76,41 +77,45 @@ struct LdsTypedLauncher {
         if constexpr (I == 2) {
             // bicubic keeps sixteen tap offsets per pixel: one or two pixels per lane
             switch (p.cls * 16 + p.ppt) {
-                case 0 * 16 + 1: return launch_cls<T, I, P, A, 0, 1>(a, p, stream);
-                case 0 * 16 + 2: return launch_cls<T, I, P, A, 0, 2>(a, p, stream);
-                case 1 * 16 + 1: return launch_cls<T, I, P, A, 1, 1>(a, p, stream);
-                case 1 * 16 + 2: return launch_cls<T, I, P, A, 1, 2>(a, p, stream);
-                case 2 * 16 + 1: return launch_cls<T, I, P, A, 2, 1>(a, p, stream);
-                case 2 * 16 + 2: return launch_cls<T, I, P, A, 2, 2>(a, p, stream);
-                case 3 * 16 + 1: return launch_cls<T, I, P, A, 3, 1>(a, p, stream);
-                case 3 * 16 + 2: return launch_cls<T, I, P, A, 3, 2>(a, p, stream);
+                case 0 * 16 + 1: return launch_cls<T, I, P, A, 0, 1, SHIFTED>(a, p, stream);
+                case 0 * 16 + 2: return launch_cls<T, I, P, A, 0, 2, SHIFTED>(a, p, stream);
+                case 1 * 16 + 1: return launch_cls<T, I, P, A, 1, 1, SHIFTED>(a, p, stream);
+                case 1 * 16 + 2: return launch_cls<T, I, P, A, 1, 2, SHIFTED>(a, p, stream);
+                case 2 * 16 + 1: return launch_cls<T, I, P, A, 2, 1, SHIFTED>(a, p, stream);
+                case 2 * 16 + 2: return launch_cls<T, I, P, A, 2, 2, SHIFTED>(a, p, stream);
+                case 3 * 16 + 1: return launch_cls<T, I, P, A, 3, 1, SHIFTED>(a, p, stream);
+                case 3 * 16 + 2: return launch_cls<T, I, P, A, 3, 2, SHIFTED>(a, p, stream);
                 default: return hipErrorInvalidValue;
             }
         }
         switch (p.cls * 16 + p.ppt) {
-            case 0 * 16 + 1: return launch_cls<T, I, P, A, 0, 1>(a, p, stream);
-            case 0 * 16 + 4: return launch_cls<T, I, P, A, 0, 4>(a, p, stream);
-            case 1 * 16 + 1: return launch_cls<T, I, P, A, 1, 1>(a, p, stream);
-            case 1 * 16 + 4: return launch_cls<T, I, P, A, 1, 4>(a, p, stream);
-            case 2 * 16 + 1: return launch_cls<T, I, P, A, 2, 1>(a, p, stream);
-            case 2 * 16 + 4: return launch_cls<T, I, P, A, 2, 4>(a, p, stream);
-            case 2 * 16 + 8: return launch_cls<T, I, P, A, 2, 8>(a, p, stream);
-            case 3 * 16 + 1: return launch_cls<T, I, P, A, 3, 1>(a, p, stream);
-            case 3 * 16 + 4: return launch_cls<T, I, P, A, 3, 4>(a, p, stream);
-            case 3 * 16 + 8: return launch_cls<T, I, P, A, 3, 8>(a, p, stream);
+            case 0 * 16 + 1: return launch_cls<T, I, P, A, 0, 1, SHIFTED>(a, p, stream);
+            case 0 * 16 + 4: return launch_cls<T, I, P, A, 0, 4, SHIFTED>(a, p, stream);
+            case 1 * 16 + 1: return launch_cls<T, I, P, A, 1, 1, SHIFTED>(a, p, stream);
+            case 1 * 16 + 4: return launch_cls<T, I, P, A, 1, 4, SHIFTED>(a, p, stream);
+            case 2 * 16 + 1: return launch_cls<T, I, P, A, 2, 1, SHIFTED>(a, p, stream);
+            case 2 * 16 + 4: return launch_cls<T, I, P, A, 2, 4, SHIFTED>(a, p, stream);
+            case 2 * 16 + 8: return launch_cls<T, I, P, A, 2, 8, SHIFTED>(a, p, stream);
+            case 3 * 16 + 1: return launch_cls<T, I, P, A, 3, 1, SHIFTED>(a, p, stream);
+            case 3 * 16 + 4: return launch_cls<T, I, P, A, 3, 4, SHIFTED>(a, p, stream);
+            case 3 * 16 + 8: return launch_cls<T, I, P, A, 3, 8, SHIFTED>(a, p, stream);
             default: return hipErrorInvalidValue;
         }
     }
 };
 
-template <typename T>
+// SHIFTED: the kernels for planes off the 16-byte grid (plan.copy_gran == 2)
+template <typename T, bool SHIFTED>
 hipError_t lds_launch_typed(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t stream)
 {
-    return dispatch_modes<T>(a, LdsTypedLauncher<T>{a, p, stream});
+    return dispatch_modes<T>(a, LdsTypedLauncher<T, SHIFTED>{a, p, stream});
 }
 
-extern template hipError_t lds_launch_typed<float>(const GridSamplerArgs&, const LdsPlan&, hipStream_t);
-extern template hipError_t lds_launch_typed<_Float16>(const GridSamplerArgs&, const LdsPlan&, hipStream_t);
-extern template hipError_t lds_launch_typed<__bf16>(const GridSamplerArgs&, const LdsPlan&, hipStream_t);
+extern template hipError_t lds_launch_typed<float, false>(const GridSamplerArgs&, const LdsPlan&, hipStream_t);
+extern template hipError_t lds_launch_typed<_Float16, false>(const GridSamplerArgs&, const LdsPlan&, hipStream_t);
+extern template hipError_t lds_launch_typed<__bf16, false>(const GridSamplerArgs&, const LdsPlan&, hipStream_t);
+extern template hipError_t lds_launch_typed<float, true>(const GridSamplerArgs&, const LdsPlan&, hipStream_t);
+extern template hipError_t lds_launch_typed<_Float16, true>(const GridSamplerArgs&, const LdsPlan&, hipStream_t);
+extern template hipError_t lds_launch_typed<__bf16, true>(const GridSamplerArgs&, const LdsPlan&, hipStream_t);
 
 }  // namespace opscv
