@@ -20,7 +20,7 @@ LdsPlan make_lds_plan(const GridSamplerArgs& a)
     const int64_t need = ((plane_bytes + (plain ? 0 : 14) + 15) & ~(int64_t)15) + 16;
     const int64_t out_plane = a.Hout * a.Wout;
     // output-plane byte offsets are kept in 32 bits (and below the out-of-range marker 0x80000000)
-    if (out_plane * esz >= ((int64_t)1 << 31) || need > kPitch[3]) {
+    if (out_plane * esz >= ((int64_t)1 << 31) || need > kPitch[4]) {
         return p;
     }
     p.cls = 0;
@@ -83,8 +83,8 @@ const char* gs2d_lds_variant_name(const GridSamplerArgs& a)
     if (!p.ok) {
         return nullptr;
     }
-    static const char* names[4] = {"lds_ring_p2064_4x4", "lds_ring_p8208_2x4", "lds_ring_p32784_1x4",
-                                   "lds_ring_p81904_1x2"};
+    static const char* names[5] = {"lds_ring_p2064_4x4", "lds_ring_p8208_2x4", "lds_ring_p16400_1x4",
+                                   "lds_ring_p32784_1x4", "lds_ring_p81904_1x2"};
     return names[p.cls];
 }
 

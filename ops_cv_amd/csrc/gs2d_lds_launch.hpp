@@ -23,15 +23,16 @@ struct LdsPlan {
 };
 
 constexpr int kSamplerWaves = 8;  // 512 lanes own output pixels
-// loader wavefronts per size class: enough that (NBUF-2) stages of one loader's copy instructions fit the
+// loader wavefronts per size class (the 16 KiB class as the 8 KiB one): enough that (NBUF-2) stages of one loader's copy instructions fit the
 // 6-bit outstanding-operation counter (a 1 KiB chunk per instruction), and for the 8 KiB class four of them
 // because one wavefront alone issues the copies of a stage too slowly to keep the ring full
-constexpr int kLoaderWaves[4] = {1, 4, 2, 4};
+constexpr int kLoaderWaves[5] = {1, 4, 4, 2, 4};
 constexpr int kThreads = kSamplerWaves * 64;  // pixels per tile = kThreads * ppt
-// plane pitch in LDS and planes per stage for the four size classes; two stage buffers are resident
-constexpr int kPitch[4] = {2064, 8208, 32784, 81904};
-constexpr int kCgs[4] = {4, 2, 1, 1};   // planes per stage
-constexpr int kNbuf[4] = {4, 4, 4, 2};  // ring slots (stages resident in LDS)
+// plane pitch in LDS and planes per stage for the five size classes (the 16 KiB class keeps two workgroups per CU
+// for planes a little over 8 KiB, which the 32 KiB class would run one per CU at a third of the speed)
+constexpr int kPitch[5] = {2064, 8208, 16400, 32784, 81904};
+constexpr int kCgs[5] = {4, 2, 1, 1, 1};   // planes per stage
+constexpr int kNbuf[5] = {4, 4, 4, 4, 2};  // ring slots (stages resident in LDS)
 
 LdsPlan make_lds_plan(const GridSamplerArgs& a);
 
@@ -85,6 +86,8 @@ struct LdsTypedLauncher {
                 case 2 * 16 + 2: return launch_cls<T, I, P, A, 2, 2, SHIFTED>(a, p, stream);
                 case 3 * 16 + 1: return launch_cls<T, I, P, A, 3, 1, SHIFTED>(a, p, stream);
                 case 3 * 16 + 2: return launch_cls<T, I, P, A, 3, 2, SHIFTED>(a, p, stream);
+                case 4 * 16 + 1: return launch_cls<T, I, P, A, 4, 1, SHIFTED>(a, p, stream);
+                case 4 * 16 + 2: return launch_cls<T, I, P, A, 4, 2, SHIFTED>(a, p, stream);
                 default: return hipErrorInvalidValue;
             }
         }
@@ -99,6 +102,9 @@ struct LdsTypedLauncher {
             case 3 * 16 + 1: return launch_cls<T, I, P, A, 3, 1, SHIFTED>(a, p, stream);
             case 3 * 16 + 4: return launch_cls<T, I, P, A, 3, 4, SHIFTED>(a, p, stream);
             case 3 * 16 + 8: return launch_cls<T, I, P, A, 3, 8, SHIFTED>(a, p, stream);
+            case 4 * 16 + 1: return launch_cls<T, I, P, A, 4, 1, SHIFTED>(a, p, stream);
+            case 4 * 16 + 4: return launch_cls<T, I, P, A, 4, 4, SHIFTED>(a, p, stream);
+            case 4 * 16 + 8: return launch_cls<T, I, P, A, 4, 8, SHIFTED>(a, p, stream);
             default: return hipErrorInvalidValue;
         }
     }
