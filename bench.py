@@ -31,9 +31,9 @@ MEASURED_TRAFFIC = {
     ("C4", "nchw_band_lds"): 1415.4e6,       # profiles/resize_band_lds_C4_fp16_4k_upscale.md
     ("C2", "nchw_flat_lds"): 33.08e6,        # profiles/resize_flat_lds_C2_fp32_56_to_112.md
     ("C5", "lds_ring_p32784_1x4"): 176.4e6,  # profiles/gs2d_lds_ring_C5_bf16_random_gather.md
-    ("V1", "gs3d_bilinear"): 38.65e6,        # profiles/gs3d_V1_fp16_22x4x16x64x64.md
-    ("G3", "gs2d_grad_ordered"): 250.7e6,    # profiles/gs2d_grad_G3_fp16_n16_c256.md (both kernels of a step)
-    ("B4", "resize_grad_lds"): 1338.5e6,     # profiles/resize_grad_lds_B4_fp16_4k.md
+    ("V1", "gs3d_bilinear"): 38.67e6,        # profiles/gs3d_V1_fp16_22x4x16x64x64.md
+    ("G3", "gs2d_grad_ordered"): 255.3e6,    # profiles/gs2d_grad_G3_fp16_n16_c256.md (both kernels of a step)
+    ("B4", "resize_grad_lds"): 1340.0e6,     # profiles/resize_grad_lds_B4_fp16_4k.md
     ("R4", "nearest_nchw_lds"): 1327.3e6,    # profiles/resize_nearest_lds_R4_fp16_4k.md
 }
 
