@@ -418,9 +418,12 @@ __global__ __launch_bounds__(kThreads) void resize_nearest_kernel(const T* __res
     } else {
 #pragma unroll
         for (int i = 0; i < V; i++) {
-            src_off[i] = nearest_src((int32_t)e0 + i, scale_w, Ws);
+            const int32_t col = ((int32_t)e0 + i < Wd) ? (int32_t)e0 + i : Wd - 1;  // past a ragged row end: unused
+            src_off[i] = nearest_src(col, scale_w, Ws);
         }
     }
+    // NCHW rows of any width: the vector store is element-aligned, the lane at a ragged row end stores singly
+    const int nvalid = (row_elems - e0 < V) ? (int)(row_elems - e0) : V;
     const int64_t rows = outer * Hd;  // outer = N*C planes (NCHW) or N images (NHWC)
     // a workgroup copies kNearestBand consecutive output rows per step: the column offsets above are reused and
     // neighbouring output rows of an upscale read the same source row out of L1
@@ -443,10 +446,30 @@ __global__ __launch_bounds__(kThreads) void resize_nearest_kernel(const T* __res
                 }
                 __builtin_memcpy(&packed, v, sizeof(packed));
             }
-            if (streaming) {
-                store_streaming(reinterpret_cast<uint4*>(dst), packed);
+            if (NHWC) {
+                if (streaming) {
+                    store_streaming(reinterpret_cast<uint4*>(dst), packed);
+                } else {
+                    *reinterpret_cast<uint4*>(dst) = packed;
+                }
+            } else if (nvalid == V) {
+                typedef uint32_t u32x4_any __attribute__((ext_vector_type(4), aligned(2)));
+                u32x4_any t;
+                __builtin_memcpy(&t, &packed, 16);
+                if (streaming) {
+                    __builtin_nontemporal_store(t, reinterpret_cast<u32x4_any*>(dst));
+                } else {
+                    *reinterpret_cast<u32x4_any*>(dst) = t;
+                }
             } else {
-                *reinterpret_cast<uint4*>(dst) = packed;
+                T v[V];
+                __builtin_memcpy(v, &packed, 16);
+#pragma unroll
+                for (int i = 0; i < V; i++) {
+                    if (i < nvalid) {
+                        dst[i] = v[i];
+                    }
+                }
             }
         } else {
             dst[0] = src[src_off[0]];
@@ -460,7 +483,8 @@ __global__ __launch_bounds__(kThreads) void resize_nearest_kernel(const T* __res
 // workgroup owns (chunk of 256 output vectors, band of kNearestBand output rows): the source-row segments the chunk
 // reads -- one per distinct source row of the band, each a single 16-byte aligned byte range -- are copied into LDS
 // with the asynchronous global->LDS loads, and a lane assembles its vector from V two-byte LDS reads, once per
-// distinct source row.  Needs source rows that are whole 16-byte vectors (Ws % V == 0, aligned base).
+// distinct source row.  Needs source rows that are whole 16-byte vectors (Ws % V == 0, aligned base); the output may
+// have any width.
 template <typename T>
 __global__ __launch_bounds__(kThreads) void resize_nearest_lds_kernel(const T* __restrict__ x, T* __restrict__ y,
                                                                        int64_t outer, int32_t Hs, int32_t Ws,
@@ -482,6 +506,7 @@ __global__ __launch_bounds__(kThreads) void resize_nearest_lds_kernel(const T* _
     const bool use_lds = seg_bytes <= slot_bytes;  // uniform; the launch sizes the slots so that this holds
     const int32_t e0 = col_first + tid * V;
     const bool active = e0 < Wd;
+    const int nvalid = (Wd - e0 < V) ? Wd - e0 : V;
     int32_t src_col[V];
 #pragma unroll
     for (int i = 0; i < V; i++) {
@@ -552,11 +577,27 @@ __global__ __launch_bounds__(kThreads) void resize_nearest_lds_kernel(const T* _
                     __builtin_memcpy(&packed, v, sizeof(packed));
                     last = slot_of[j];
                 }
-                uint4* dst = reinterpret_cast<uint4*>(y + (r0 + j) * (int64_t)Wd + e0);
-                if (streaming) {
-                    store_streaming(dst, packed);
+                // rows of a width that is not a multiple of V start anywhere: the vector store is element-aligned,
+                // and the lane at the ragged end of a row stores its elements singly
+                T* dst = y + (r0 + j) * (int64_t)Wd + e0;
+                if (nvalid == V) {
+                    typedef uint32_t u32x4_any __attribute__((ext_vector_type(4), aligned(2)));
+                    u32x4_any t;
+                    __builtin_memcpy(&t, &packed, 16);
+                    if (streaming) {
+                        __builtin_nontemporal_store(t, reinterpret_cast<u32x4_any*>(dst));
+                    } else {
+                        *reinterpret_cast<u32x4_any*>(dst) = t;
+                    }
                 } else {
-                    *dst = packed;
+                    T v[V];
+                    __builtin_memcpy(v, &packed, 16);
+#pragma unroll
+                    for (int i = 0; i < V; i++) {
+                        if (i < nvalid) {
+                            dst[i] = v[i];
+                        }
+                    }
                 }
             }
         }
@@ -707,8 +748,10 @@ hipError_t run_resize(const ResizeArgs& a, hipStream_t stream)
         const int64_t rows = outer * a.Hd;
         const bool aligned = reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(y) % 16 == 0;
         // whole 16-byte vectors: rows start aligned (row_elems % V == 0); for NHWC a vector stays inside one pixel
-        const bool vec = aligned && row_elems % V == 0 && (!nhwc || (a.C % V == 0 && (a.Ws * a.C) % V == 0));
-        const int64_t lanes = vec ? row_elems / V : row_elems;
+        // (NCHW takes vectors at any width and alignment: its loads are per element, its stores element-aligned)
+        const bool whole = aligned && row_elems % V == 0;
+        const bool vec = nhwc ? (whole && a.C % V == 0 && (a.Ws * a.C) % V == 0) : true;
+        const int64_t lanes = vec ? (row_elems + V - 1) / V : row_elems;
         const int64_t bands = (rows + kNearestBand - 1) / kNearestBand;
         dim3 grid((unsigned)((lanes + kThreads - 1) / kThreads), (unsigned)(bands < 65535 ? bands : 65535));
 #define OPSCV_NEAREST(NHWC_, VEC_)                                                                                  \
@@ -716,7 +759,7 @@ hipError_t run_resize(const ResizeArgs& a, hipStream_t stream)
                        (int32_t)a.C, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h, a.scale_w, \
                        streaming)
         const int streaming = (out_elems * (int64_t)sizeof(T) >= (128ll << 20)) ? 1 : 0;
-        if (!nhwc && vec && a.Ws % V == 0 && !(getenv("OPSCV_NEAREST_VARIANT") && getenv("OPSCV_NEAREST_VARIANT")[0] == 'g')) {
+        if (!nhwc && reinterpret_cast<uintptr_t>(x) % 16 == 0 && a.Ws % V == 0 && !(getenv("OPSCV_NEAREST_VARIANT") && getenv("OPSCV_NEAREST_VARIANT")[0] == 'g')) {
             // slot = the longest source segment a chunk of kThreads vectors can touch, with slack for the rounding of
             // the per-column products; the kernel checks the real length and gathers from global memory otherwise
             const double span = (double)(kThreads * V) * (double)a.scale_w * 1.001 + 2.0 + 2.0 * V;
@@ -861,11 +904,11 @@ const char* resize_variant(const ResizeArgs& a)
             if (a.channels_last) {
                 return "nearest_nhwc";
             }
-            // rows of whole 16-byte vectors on both sides and slots that fit: the LDS-staged kernel (see run_resize)
+            // source rows of whole 16-byte vectors and slots that fit: the LDS-staged kernel (see run_resize)
             const int64_t V = 16 / elem_size(a.elem);
             const double span = 256.0 * (double)V * (double)a.scale_w * 1.001 + 2.0 + 2.0 * (double)V;
             const uint64_t slot = ((uint64_t)(span * elem_size(a.elem)) + 15u) / 16u * 16u;
-            const bool lds = a.Wd % V == 0 && a.Ws % V == 0 && slot * kNearestBand <= 64u * 1024u;
+            const bool lds = a.Ws % V == 0 && slot * kNearestBand <= 64u * 1024u;
             return lds ? "nearest_nchw_lds" : "nearest_nchw";
         }
         default: break;
