@@ -30,7 +30,7 @@ template <typename T, bool HALF_PIXEL>
 void staged_extent(const ResizeArgs& a, int gran, int kThreads, int32_t* max_rows, int32_t* max_seg_elems)
 {
     constexpr int V = 16 / (int)sizeof(T);
-    const int32_t ge = gran / (int)sizeof(T);
+    const int32_t ge = (gran == 1) ? 1 : gran / (int)sizeof(T);
     const int32_t Wd = (int32_t)a.Wd, Hd = (int32_t)a.Hd, Ws = (int32_t)a.Ws, Hs = (int32_t)a.Hs;
     int32_t mr = 0, ms = 0;
     for (int32_t hb = 0; hb < Hd; hb += kBand) {
@@ -72,8 +72,8 @@ BandPlan make_plan(const ResizeArgs& a)
     int gran;
     if ((a.Ws * sizeof(T)) % 16 == 0 && xa % 16 == 0) {
         gran = 16;
-    } else if ((a.Ws * sizeof(T)) % 4 == 0 && xa % 4 == 0) {
-        gran = 4;
+    } else if (xa % sizeof(T) == 0) {
+        gran = 1;  // rows off the 16-byte grid: 16-byte copies in the shifted layout (see the kernel)
     } else {
         return bp;
     }
@@ -86,7 +86,7 @@ BandPlan make_plan(const ResizeArgs& a)
     } else {
         staged_extent<T, false>(a, gran, kThreads, &rows, &seg);
     }
-    const int64_t pitch = ((int64_t)seg * sizeof(T) + 15) / 16 * 16;
+    const int64_t pitch = ((int64_t)seg * sizeof(T) + (gran == 1 ? 15 : 0) + 15) / 16 * 16;
     const int64_t bytes = pitch * rows;
     if (bytes > kLdsBudget || bytes <= 0) {
         return bp;  // strong down-scaling: the band touches too many source rows/columns

@@ -35,7 +35,7 @@ struct BandLdsParams {
     float scale_h, scale_w;
     int32_t lds_pitch;  // bytes between staged source rows (multiple of 16)
     int32_t lds_rows;   // staged rows the LDS allocation holds
-    int32_t gran;       // bytes per lane of the asynchronous copy: 16 or 4
+    int32_t gran;       // bytes per lane of the asynchronous copy: 16 or 4; 1: 16 in the shifted layout (kernel)
     int32_t streaming;  // 1: mark the output stores non-temporal (outputs much larger than the caches)
     int32_t raw_lambda;  // fraction from the unclamped source coordinate (see axis_tap)
     float neg_zero;     // -0.0f, passed in so that fma(v, w, -0) is not folded back into a multiply
@@ -58,7 +58,13 @@ __global__ __launch_bounds__(THREADS) void resize_band_lds_kernel(const T* __res
     const int32_t c_last = ((c_begin + THREADS * V < p.Wd) ? c_begin + THREADS * V : p.Wd) - 1;
     const int32_t h_begin = blockIdx.y * BAND;
     const int32_t h_end = (h_begin + BAND < p.Hd) ? h_begin + BAND : p.Hd;
-    const int32_t ge = p.gran / (int)sizeof(T);  // elements per copy granule
+    // gran 16 or 4: source rows on that grid, copied as they are.  gran 1: rows anywhere (an odd width of 16-bit
+    // elements, a view that starts anywhere) -- a row's segment is then copied in 16-byte units from the boundary
+    // before its first byte to the boundary after its last (the bytes outside share an aligned unit with bytes inside,
+    // so they are readable), and lands `shift` bytes into its LDS row; the shift goes into the row's base address.
+    const bool shifted = p.gran == 1;
+    const int32_t ge = shifted ? 1 : p.gran / (int)sizeof(T);  // elements per copy granule
+    const uint32_t copy_unit = shifted ? 16u : (uint32_t)p.gran;
     const int32_t xs_lo = axis_tap<HALF_PIXEL>(c_begin, p.scale_w, p.Ws).i0;
     const int32_t xs_hi = axis_tap<HALF_PIXEL>(c_last, p.scale_w, p.Ws).i1;
     const int32_t seg_col0 = xs_lo / ge * ge;
@@ -103,17 +109,24 @@ __global__ __launch_bounds__(THREADS) void resize_band_lds_kernel(const T* __res
     for (int64_t pl = blockIdx.z; pl < p.planes; pl += gridDim.z) {
         // ---- stage the source rows of this band ----
         const char* src0 = reinterpret_cast<const char*>(x + (pl * p.Hs + ys_lo) * (int64_t)p.Ws + seg_col0);
-        const uint32_t chunk = 64u * (uint32_t)p.gran;
-        const uint32_t chunks_per_row = (seg_bytes + chunk - 1) / chunk;
+        const uint32_t chunk = 64u * copy_unit;
+        const uint32_t chunks_per_row = (seg_bytes + (shifted ? 15u : 0u) + chunk - 1) / chunk;
         const uint32_t total_chunks = chunks_per_row * (uint32_t)rows;
+        const uint32_t src0_low = (uint32_t)(reinterpret_cast<uintptr_t>(src0) & 15u);
+        const uint32_t row_low = (uint32_t)(((uint32_t)p.Ws * (uint32_t)sizeof(T)) & 15u);
+        // bytes by which the copy of staged row r starts before the row's segment
+        auto row_shift = [&](uint32_t r) -> uint32_t { return shifted ? ((src0_low + r * row_low) & 15u) : 0u; };
         for (uint32_t q = wave; q < total_chunks; q += NWAVES) {
             const uint32_t r = q / chunks_per_row;
             const uint32_t cb = (q - r * chunks_per_row) * chunk;
-            const uint32_t lane_off = cb + (uint32_t)lane * (uint32_t)p.gran;
-            if (lane_off < seg_bytes) {
-                const rs_global_cptr_t g = (rs_global_cptr_t)(src0 + (size_t)r * p.Ws * sizeof(T) + lane_off);
+            const uint32_t lane_off = cb + (uint32_t)lane * copy_unit;
+            const uint32_t shift = row_shift(r);
+            const uint32_t limit = shifted ? ((seg_bytes + shift + 15u) & ~15u) : seg_bytes;
+            if (lane_off < limit) {
+                const rs_global_cptr_t g =
+                    (rs_global_cptr_t)(src0 + (size_t)r * p.Ws * sizeof(T) - shift + lane_off);
                 const rs_lds_ptr_t l = (rs_lds_ptr_t)(lds + r * p.lds_pitch + cb);
-                if (p.gran == 16) {
+                if (copy_unit == 16u) {
                     __builtin_amdgcn_global_load_lds(g, l, 16, 0, 0);
                 } else {
                     __builtin_amdgcn_global_load_lds(g, l, 4, 0, 0);
@@ -127,7 +140,7 @@ __global__ __launch_bounds__(THREADS) void resize_band_lds_kernel(const T* __res
         float ha[V], hb[V];  // blended source rows ya and yb (row indices relative to ys_lo)
         int32_t ya = -1, yb = -1;
         auto blend_row = [&](float* hrow, int32_t ys) {
-            const char* row = lds + ys * p.lds_pitch;
+            const char* row = lds + ys * p.lds_pitch + row_shift((uint32_t)ys);
             T l[V], r[V];
 #pragma unroll
             for (int i = 0; i < V; i++) {
