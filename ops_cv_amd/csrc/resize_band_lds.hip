@@ -63,11 +63,7 @@ BandPlan make_plan(const ResizeArgs& a)
     if (reinterpret_cast<uintptr_t>(a.y) % sizeof(T) != 0 || a.Wd * (int64_t)sizeof(T) >= (1ll << 31)) {
         return bp;
     }
-    // short rows leave most of this kernel's lanes idle; the flat variant that serves them takes whole vectors only,
-    // so short ragged rows are left to the register-band kernel
-    if (a.Wd % V != 0 && a.Wd / V <= 128) {
-        return bp;
-    }
+
     const uintptr_t xa = reinterpret_cast<uintptr_t>(a.x);
     int gran;
     if ((a.Ws * sizeof(T)) % 16 == 0 && xa % 16 == 0) {
@@ -152,12 +148,11 @@ FlatPlan make_flat_plan(const ResizeArgs& a)
     if (a.channels_last || a.mode != ResizeMode::Bilinear) {
         return fp;
     }
-    // whole 16-byte output vectors, 16-byte aligned output planes, 32-bit byte offsets inside an output plane
-    if (a.Wd % V != 0 || reinterpret_cast<uintptr_t>(a.y) % 16 != 0 ||
-        a.Hd * a.Wd * (int64_t)sizeof(T) >= (1ll << 31)) {
+    // element-aligned output (the vector stores are), 32-bit byte offsets inside an output plane
+    if (reinterpret_cast<uintptr_t>(a.y) % sizeof(T) != 0 || a.Hd * a.Wd * (int64_t)sizeof(T) >= (1ll << 31)) {
         return fp;
     }
-    const int64_t cl = a.Wd / V;
+    const int64_t cl = (a.Wd + V - 1) / V;
     if (cl > kFlatMaxColumnLanes) {
         return fp;
     }
@@ -165,8 +160,8 @@ FlatPlan make_flat_plan(const ResizeArgs& a)
     int gran;
     if ((a.Ws * sizeof(T)) % 16 == 0 && xa % 16 == 0) {
         gran = 16;
-    } else if ((a.Ws * sizeof(T)) % 4 == 0 && xa % 4 == 0) {
-        gran = 4;
+    } else if (xa % sizeof(T) == 0) {
+        gran = 1;  // rows off the 16-byte grid: 16-byte copies in the shifted layout (see the kernel)
     } else {
         return fp;
     }
@@ -204,7 +199,7 @@ FlatPlan make_flat_plan(const ResizeArgs& a)
     fp.p.gran = gran;
     fp.p.neg_zero = -0.0f;
     fp.p.raw_lambda = a.raw_lambda;
-    fp.lds_bytes = (uint32_t)(((int64_t)rows * a.Ws * (int64_t)sizeof(T) + 15) / 16 * 16);
+    fp.lds_bytes = (uint32_t)(((int64_t)rows * a.Ws * (int64_t)sizeof(T) + (gran == 1 ? 15 : 0) + 15) / 16 * 16);
     fp.grid = dim3((unsigned)bands, (unsigned)(planes < 65535 ? planes : 65535));
     const char* v = getenv("OPSCV_RESIZE_VARIANT");
     // generic / register-band / LDS band forced (benchmark knob)

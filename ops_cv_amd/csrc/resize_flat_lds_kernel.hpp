@@ -25,9 +25,9 @@ struct FlatLdsParams {
     int32_t Hs, Ws, Hd, Wd;
     float scale_h, scale_w;
     int32_t band_rows;  // output rows per workgroup (a multiple of rg)
-    int32_t cl;         // column lanes = Wd / V
+    int32_t cl;         // column lanes = ceil(Wd / V)
     int32_t rg;         // row groups = THREADS / cl
-    int32_t gran;       // bytes per lane of the asynchronous copy: 16 or 4
+    int32_t gran;       // bytes per lane of the asynchronous copy: 16 or 4; 1: 16 in the shifted layout (kernel)
     int32_t raw_lambda;  // fraction from the unclamped source coordinate (see axis_tap)
     float neg_zero;     // -0.0f, passed in so that fma(v, w, -0) is not folded back into a multiply
 };
@@ -57,6 +57,7 @@ __global__ __launch_bounds__(THREADS) void resize_flat_lds_kernel(const T* __res
 
     // ---- per-lane column taps ----
     const int32_t col0 = cvec * V;
+    const int32_t nvalid = (p.Wd - col0 < V) ? p.Wd - col0 : V;  // output columns of this lane inside the row
     uint32_t to0[V], to1[V];
     float dx[V], omdx[V];
 #pragma unroll
@@ -73,16 +74,24 @@ __global__ __launch_bounds__(THREADS) void resize_flat_lds_kernel(const T* __res
     const uint32_t out_plane_bytes = (uint32_t)p.Hd * out_row_bytes;
     const uint32_t col_off = (uint32_t)col0 * (uint32_t)sizeof(T);
     const float neg_zero = p.neg_zero;
-    const uint32_t chunk = 64u * (uint32_t)p.gran;
+    const uint32_t copy_unit = (p.gran == 1) ? 16u : (uint32_t)p.gran;
+    const uint32_t chunk = 64u * copy_unit;
 
     for (int64_t pl = blockIdx.y; pl < p.planes; pl += gridDim.y) {
+        // gran 1: source rows anywhere (an odd width of 16-bit elements, a view that starts anywhere).  The band's
+        // rows are one contiguous byte range; it is copied in 16-byte units from the boundary before its first byte to
+        // the boundary after its last (the bytes outside share an aligned unit with bytes inside, so they are
+        // readable) and lands `shift` bytes into LDS.
         const char* src0 = reinterpret_cast<const char*>(x + (pl * p.Hs + ys_lo) * (int64_t)p.Ws);
-        for (uint32_t cb = wave * chunk; cb < stage_bytes; cb += NWAVES * chunk) {
-            const uint32_t lane_off = cb + (uint32_t)lane * (uint32_t)p.gran;
-            if (lane_off < stage_bytes) {
+        const uint32_t shift = (p.gran == 1) ? (uint32_t)(reinterpret_cast<uintptr_t>(src0) & 15u) : 0u;
+        const uint32_t copy_bytes = (p.gran == 1) ? ((stage_bytes + shift + 15u) & ~15u) : stage_bytes;
+        src0 -= shift;
+        for (uint32_t cb = wave * chunk; cb < copy_bytes; cb += NWAVES * chunk) {
+            const uint32_t lane_off = cb + (uint32_t)lane * copy_unit;
+            if (lane_off < copy_bytes) {
                 const rs_global_cptr_t g = (rs_global_cptr_t)(src0 + lane_off);
                 const rs_lds_ptr_t l = (rs_lds_ptr_t)(lds + cb);
-                if (p.gran == 16) {
+                if (copy_unit == 16u) {
                     __builtin_amdgcn_global_load_lds(g, l, 16, 0, 0);
                 } else {
                     __builtin_amdgcn_global_load_lds(g, l, 4, 0, 0);
@@ -96,8 +105,8 @@ __global__ __launch_bounds__(THREADS) void resize_flat_lds_kernel(const T* __res
             __builtin_amdgcn_make_buffer_rsrc(y + pl * (int64_t)p.Hd * p.Wd, 0, out_plane_bytes, kRsBufferFlags);
         for (int32_t h = active ? h_begin + group : h_end; h < h_end; h += p.rg) {
             const AxisTap t = axis_tap<HALF_PIXEL>(h, p.scale_h, p.Hs, p.raw_lambda);
-            const char* r0 = lds + (uint32_t)(t.i0 - ys_lo) * src_row_bytes;
-            const char* r1 = lds + (uint32_t)(t.i1 - ys_lo) * src_row_bytes;
+            const char* r0 = lds + shift + (uint32_t)(t.i0 - ys_lo) * src_row_bytes;
+            const char* r1 = lds + shift + (uint32_t)(t.i1 - ys_lo) * src_row_bytes;
             T tl[V], tr[V], bl[V], br[V];
 #pragma unroll
             for (int i = 0; i < V; i++) {
@@ -121,8 +130,25 @@ __global__ __launch_bounds__(THREADS) void resize_flat_lds_kernel(const T* __res
             typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
             u32x4 packed;
             __builtin_memcpy(&packed, outv, sizeof(packed));
-            __builtin_amdgcn_raw_buffer_store_b128(packed, rsrc,
-                                                   (int)((uint32_t)h * out_row_bytes + col_off), 0, 0);
+            const uint32_t out_off = (uint32_t)h * out_row_bytes + col_off;
+            if (nvalid == V) {
+                // rows of a width that is not a multiple of V start anywhere: the store is element-aligned
+                __builtin_amdgcn_raw_buffer_store_b128(packed, rsrc, (int)out_off, 0, 0);
+            } else {
+                // the lane that holds the ragged end of the row stores its elements singly
+#pragma unroll
+                for (int i = 0; i < V; i++) {
+                    if (i < nvalid) {
+                        if constexpr (sizeof(T) == 4) {
+                            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, outv[i]), rsrc,
+                                                                  (int)(out_off + i * 4), 0, 0);
+                        } else {
+                            __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(uint16_t, outv[i]), rsrc,
+                                                                  (int)(out_off + i * 2), 0, 0);
+                        }
+                    }
+                }
+            }
         }
         __syncthreads();  // everybody is done with the staged rows before the next plane overwrites them
     }
