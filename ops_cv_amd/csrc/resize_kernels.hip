@@ -307,6 +307,107 @@ __global__ __launch_bounds__(kThreads) void resize_nhwc_vec_kernel(const T* __re
     }
 }
 
+// Element-aligned copies of VB bytes (a run of channels of one pixel), built from power-of-two pieces so that each
+// piece is one memory instruction: global memory accesses need only element alignment.
+template <int VB>
+__device__ __forceinline__ void copy_unit(void* dst, const void* src)
+{
+    char* d = static_cast<char*>(dst);
+    const char* s = static_cast<const char*>(src);
+    if constexpr (VB == 16) {
+        typedef uint32_t u32x4_any __attribute__((ext_vector_type(4), aligned(2)));
+        *reinterpret_cast<u32x4_any*>(d) = *reinterpret_cast<const u32x4_any*>(s);
+    } else {
+        if constexpr (VB >= 8) {
+            uint64_t t;
+            __builtin_memcpy(&t, s, 8);
+            __builtin_memcpy(d, &t, 8);
+        }
+        if constexpr ((VB & 4) != 0) {
+            uint32_t t;
+            __builtin_memcpy(&t, s + (VB & 8), 4);
+            __builtin_memcpy(d + (VB & 8), &t, 4);
+        }
+        if constexpr ((VB & 2) != 0) {
+            uint16_t t;
+            __builtin_memcpy(&t, s + (VB & 12), 2);
+            __builtin_memcpy(d + (VB & 12), &t, 2);
+        }
+    }
+}
+
+// NHWC variant for channel counts that are not whole aligned 16-byte vectors (three-channel images, C = 20 ...): the
+// band kernel above with a unit of VB bytes -- the widest of 16, 12, 8, 6, 4 that divides a pixel's channels --
+// moved by element-aligned loads and stores.  Same operations in the same order.
+template <typename T, bool HALF_PIXEL, int BAND, int VB>
+__global__ __launch_bounds__(kThreads) void resize_nhwc_unit_kernel(const T* __restrict__ x, T* __restrict__ y,
+                                                                     int64_t N, int32_t C, int32_t Hs, int32_t Ws,
+                                                                     int32_t Hd, int32_t Wd, float scale_h,
+                                                                     float scale_w)
+{
+    constexpr int V = VB / (int)sizeof(T);
+    const int32_t cvecs = C / V;
+    const int64_t row_vecs = (int64_t)Wd * cvecs;
+    const int64_t e = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (e >= row_vecs) {
+        return;
+    }
+    const int32_t w = (int32_t)(e / cvecs);
+    const int32_t c = (int32_t)(e - (int64_t)w * cvecs) * V;
+    const AxisTap tx = axis_tap<HALF_PIXEL>(w, scale_w, Ws);
+    const float dx = tx.lambda;
+    const float omdx = 1.0f - dx;
+    const int64_t o0 = (int64_t)tx.i0 * C + c;
+    const int64_t o1 = (int64_t)tx.i1 * C + c;
+    const int64_t src_row = (int64_t)Ws * C;
+    const int32_t h_begin = blockIdx.y * BAND;
+    const int32_t h_end = (h_begin + BAND < Hd) ? h_begin + BAND : Hd;
+    for (int64_t n = blockIdx.z; n < N; n += gridDim.z) {
+        const T* xn = x + n * Hs * src_row;
+        float ha[V], hb[V];  // blended source rows ya and yb
+        int32_t ya = -1, yb = -1;
+        auto blend_row = [&](float* hrow, int32_t ys) {
+            const T* row = xn + (int64_t)ys * src_row;
+            T l[V], r[V];
+            copy_unit<VB>(l, row + o0);
+            copy_unit<VB>(r, row + o1);
+#pragma unroll
+            for (int i = 0; i < V; i++) {
+                hrow[i] = omdx * ElemIO<T>::load(&l[i]) + dx * ElemIO<T>::load(&r[i]);
+            }
+        };
+        for (int32_t h = h_begin; h < h_end; h++) {
+            const AxisTap ty = axis_tap<HALF_PIXEL>(h, scale_h, Hs);
+            const int32_t y0 = __builtin_amdgcn_readfirstlane(ty.i0);
+            const int32_t y1 = __builtin_amdgcn_readfirstlane(ty.i1);
+            const float dy = ty.lambda;
+            const float omdy = 1.0f - dy;
+            if (y0 != ya) {
+                if (y0 == yb) {
+#pragma unroll
+                    for (int i = 0; i < V; i++) {
+                        ha[i] = hb[i];
+                    }
+                } else {
+                    blend_row(ha, y0);
+                }
+                ya = y0;
+            }
+            if (y1 != ya && y1 != yb) {
+                blend_row(hb, y1);
+                yb = y1;
+            }
+            T outv[V];
+#pragma unroll
+            for (int i = 0; i < V; i++) {
+                const float bot = (y1 == ya) ? ha[i] : hb[i];
+                ElemIO<T>::store(&outv[i], omdy * ha[i] + dy * bot);
+            }
+            copy_unit<VB>(y + ((n * Hd + h) * row_vecs + e) * V, outv);
+        }
+    }
+}
+
 // Four-weights NHWC variant (image/resize_bilinear_v2/op_kernel/arch35/resize_bilinear_v2_c_parallel.h:122-147,190-232):
 // the reference's template for channel runs of 128 bytes and more shrunk to half or less forms the four corner weights
 //   (1-dy)(1-dx), (1-dy)dx, dy(1-dx), dy*dx
@@ -685,6 +786,26 @@ bool nhwc_vec_ok(const ResizeArgs& a)
            reinterpret_cast<uintptr_t>(a.y) % 16 == 0;
 }
 
+// Bytes per lane of the element-aligned NHWC band variant: the widest of 16, 12, 8, 6, 4 that divides the bytes of a
+// pixel's channels and holds more than one element; sizeof(T) when there is none (the per-element kernel).
+template <typename T>
+int nhwc_unit_bytes(const ResizeArgs& a)
+{
+    const int esz = (int)sizeof(T);
+    if (!a.channels_last || a.mode != ResizeMode::Bilinear || (a.Hd + kNhwcBand - 1) / kNhwcBand > 65535 ||
+        reinterpret_cast<uintptr_t>(a.x) % esz != 0 || reinterpret_cast<uintptr_t>(a.y) % esz != 0) {
+        return esz;
+    }
+    const int64_t pixel_bytes = a.C * esz;
+    static const int kUnits[5] = {16, 12, 8, 6, 4};
+    for (int u : kUnits) {
+        if (u > esz && u % esz == 0 && pixel_bytes % u == 0) {
+            return u;
+        }
+    }
+    return esz;
+}
+
 // Channels per lane of the four-weights kernel: the widest of 16 bytes, 8 bytes or one element that divides C and
 // that both tensors are aligned to.
 template <typename T>
@@ -837,6 +958,32 @@ hipError_t run_resize(const ResizeArgs& a, hipStream_t stream)
         return hipGetLastError();
     }
     if (a.channels_last) {
+        const int vb = nhwc_unit_bytes<T>(a);
+        if (vb > (int)sizeof(T)) {
+            const int64_t row_vecs = a.Wd * (a.C * (int64_t)sizeof(T) / vb);
+            const int64_t bands = (a.Hd + kNhwcBand - 1) / kNhwcBand;
+            dim3 grid((unsigned)((row_vecs + kThreads - 1) / kThreads), (unsigned)bands,
+                      (unsigned)(a.N < 65535 ? a.N : 65535));
+#define OPSCV_NHWC_UNIT(HP, VB)                                                                                      \
+    hipLaunchKernelGGL((resize_nhwc_unit_kernel<T, HP, kNhwcBand, VB>), grid, dim3(kThreads), 0, stream, x, y, a.N,   \
+                       (int32_t)a.C, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h, a.scale_w)
+#define OPSCV_NHWC_UNITS(HP)                                                                                         \
+    switch (vb) {                                                                                                    \
+        case 16: OPSCV_NHWC_UNIT(HP, 16); break;                                                                     \
+        case 12: OPSCV_NHWC_UNIT(HP, 12); break;                                                                     \
+        case 8: OPSCV_NHWC_UNIT(HP, 8); break;                                                                       \
+        case 6: if constexpr (sizeof(T) == 2) { OPSCV_NHWC_UNIT(HP, 6); } break;                                     \
+        default: if constexpr (sizeof(T) == 2) { OPSCV_NHWC_UNIT(HP, 4); } break;                                    \
+    }
+            if (a.half_pixel) {
+                OPSCV_NHWC_UNITS(true)
+            } else {
+                OPSCV_NHWC_UNITS(false)
+            }
+#undef OPSCV_NHWC_UNITS
+#undef OPSCV_NHWC_UNIT
+            return hipGetLastError();
+        }
         const int64_t row_elems = a.Wd * a.C;
         const int64_t rows = a.N * a.Hd;
         dim3 grid((unsigned)((row_elems + kThreads - 1) / kThreads), (unsigned)(rows < 65535 ? rows : 65535));
@@ -920,7 +1067,16 @@ const char* resize_variant(const ResizeArgs& a)
             case Elem::F16: vec = nhwc_vec_ok<_Float16>(a); break;
             case Elem::BF16: vec = nhwc_vec_ok<__bf16>(a); break;
         }
-        return vec ? "nhwc_vec" : "nhwc_generic";
+        if (vec) {
+            return "nhwc_vec";
+        }
+        int vb = 0, esz = elem_size(a.elem);
+        switch (a.elem) {
+            case Elem::F32: vb = nhwc_unit_bytes<float>(a); break;
+            case Elem::F16: vb = nhwc_unit_bytes<_Float16>(a); break;
+            case Elem::BF16: vb = nhwc_unit_bytes<__bf16>(a); break;
+        }
+        return vb > esz ? "nhwc_unit" : "nhwc_generic";
     }
     if (const char* lds_variant = resize_lds_variant(a)) {
         return lds_variant;

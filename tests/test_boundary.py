@@ -267,7 +267,10 @@ def test_upsample_template_selection_channels_last(aclnn, desc):
     # half-pixel centres and broadcast with align_corners
     assert variant((1, 8, 8, 32), (1, 3, 3, 32), f32, False) == "nhwc_four_weights"
     assert variant((1, 8, 8, 32), (1, 3, 3, 32), f16, False) == "nhwc_vec"
-    assert variant((1, 1, 1, 14), (1, 13, 7, 14), f32, False) == "nhwc_generic"
+    assert variant((1, 1, 1, 14), (1, 13, 7, 14), f32, False) == "nhwc_unit"      # 56-byte pixels: 8-byte units
+    assert variant((1, 1, 1, 7), (1, 13, 7, 7), f32, False) == "nhwc_generic"     # no unit wider than an element
+    assert variant((1, 4, 4, 3), (1, 13, 7, 3), f32, False) == "nhwc_unit"        # three-channel images: 12 bytes
+    assert variant((1, 4, 4, 3), (1, 13, 7, 3), f16, False) == "nhwc_unit"        # ... and 6 bytes
     assert variant((1, 1, 1, 14), (1, 13, 7, 14), f32, True) == "broadcast"
     assert variant((1, 8, 8, 8), (1, 1, 1, 8), f32, True) == "first_pixel"
     assert variant((1, 8, 8, 32), (1, 1, 1, 32), f32, True) == "point_copy"

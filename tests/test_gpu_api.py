@@ -54,7 +54,11 @@ def test_upsample_nhwc(oracle, device, aclnn, dtype, align):
                                # long channel runs shrunk to half or less: the four-weights template, with channel
                                # counts for every vector width of its kernel (16 bytes, 8 bytes, one element)
                                ((2, 64, 12, 10), (5, 4)), ((1, 68, 23, 17), (7, 8)), ((1, 67, 9, 31), (4, 3)),
-                               ((2, 128, 16, 16), (1, 1)), ((1, 72, 40, 6), (3, 3))]:
+                               ((2, 128, 16, 16), (1, 1)), ((1, 72, 40, 6), (3, 3)),
+                               # pixels that are not whole 16-byte vectors: units of 12, 8, 6 and 4 bytes
+                               ((2, 3, 9, 11), (20, 17)), ((1, 6, 5, 7), (11, 13)), ((1, 10, 6, 4), (9, 9)),
+                               ((1, 9, 6, 4), (5, 10)), ((1, 2, 6, 4), (9, 7)), ((1, 20, 5, 5), (12, 12)),
+                               ((3, 3, 33, 47), (70, 129))]:
         x32 = rng.standard_normal((N, C, H, W)).astype(np.float32)
         x = I.cast_np(x32, dtype)
         xh = np.ascontiguousarray(x.transpose(0, 2, 3, 1))
@@ -65,6 +69,14 @@ def test_upsample_nhwc(oracle, device, aclnn, dtype, align):
         got = I.from_torch(y, dtype)
         assert np.array_equal(_bits(got, dtype), _bits(ref, dtype)), \
             "nhwc %s %s align=%s template %s" % (dtype, (N, C, H, W), align, template)
+        # the same tensors one element into their allocations: dense, but off the 16-byte grid
+        xo = torch.zeros(xh.size + 1, device=device, dtype=y.dtype)
+        xo[1:] = I.to_torch(xh, dtype, device).reshape(-1)
+        yo = torch.zeros(y.numel() + 2, device=device, dtype=y.dtype)
+        aclnn.upsample_bilinear2d(xo[1:].view(xh.shape), size, align, out=yo[1:-1].view(y.shape), channels_last=True)
+        torch.cuda.synchronize()
+        assert torch.equal(yo[1:-1].view(y.shape), y) and yo[0] == 0 and yo[-1] == 0, \
+            "nhwc offset %s %s align=%s" % (dtype, (N, C, H, W), align)
     assert {"per_element", "copy", "broadcast", "channel_parallel"} <= seen
 
 
