@@ -337,9 +337,10 @@ __device__ __forceinline__ void copy_unit(void* dst, const void* src)
 }
 
 // NHWC variant for channel counts that are not whole aligned 16-byte vectors (three-channel images, C = 20 ...): the
-// band kernel above with a unit of VB bytes -- the widest of 16, 12, 8, 6, 4 that divides a pixel's channels --
-// moved by element-aligned loads and stores.  Same operations in the same order.
-template <typename T, bool HALF_PIXEL, int BAND, int VB>
+// band kernel above with a unit of VB bytes -- the widest of 16, 12, 8, 6, 4, 2 that divides a pixel's channels --
+// moved by element-aligned loads and stores.  A lane owns UPL units next to each other in the output row and stores
+// them as one run of UPL * VB bytes.  Same operations in the same order.
+template <typename T, bool HALF_PIXEL, int BAND, int VB, int UPL>
 __global__ __launch_bounds__(kThreads) void resize_nhwc_unit_kernel(const T* __restrict__ x, T* __restrict__ y,
                                                                      int64_t N, int32_t C, int32_t Hs, int32_t Ws,
                                                                      int32_t Hd, int32_t Wd, float scale_h,
@@ -348,32 +349,42 @@ __global__ __launch_bounds__(kThreads) void resize_nhwc_unit_kernel(const T* __r
     constexpr int V = VB / (int)sizeof(T);
     const int32_t cvecs = C / V;
     const int64_t row_vecs = (int64_t)Wd * cvecs;
-    const int64_t e = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    const int64_t e = ((int64_t)blockIdx.x * kThreads + threadIdx.x) * UPL;
     if (e >= row_vecs) {
         return;
     }
-    const int32_t w = (int32_t)(e / cvecs);
-    const int32_t c = (int32_t)(e - (int64_t)w * cvecs) * V;
-    const AxisTap tx = axis_tap<HALF_PIXEL>(w, scale_w, Ws);
-    const float dx = tx.lambda;
-    const float omdx = 1.0f - dx;
-    const int64_t o0 = (int64_t)tx.i0 * C + c;
-    const int64_t o1 = (int64_t)tx.i1 * C + c;
+    const bool whole = e + UPL <= row_vecs;
+    float dx[UPL], omdx[UPL];
+    int64_t o0[UPL], o1[UPL];
+#pragma unroll
+    for (int u = 0; u < UPL; u++) {
+        const int64_t eu = (e + u < row_vecs) ? e + u : row_vecs - 1;  // past the row: a repeat that is never stored
+        const int32_t w = (int32_t)(eu / cvecs);
+        const int32_t c = (int32_t)(eu - (int64_t)w * cvecs) * V;
+        const AxisTap tx = axis_tap<HALF_PIXEL>(w, scale_w, Ws);
+        dx[u] = tx.lambda;
+        omdx[u] = 1.0f - tx.lambda;
+        o0[u] = (int64_t)tx.i0 * C + c;
+        o1[u] = (int64_t)tx.i1 * C + c;
+    }
     const int64_t src_row = (int64_t)Ws * C;
     const int32_t h_begin = blockIdx.y * BAND;
     const int32_t h_end = (h_begin + BAND < Hd) ? h_begin + BAND : Hd;
     for (int64_t n = blockIdx.z; n < N; n += gridDim.z) {
         const T* xn = x + n * Hs * src_row;
-        float ha[V], hb[V];  // blended source rows ya and yb
+        float ha[UPL * V], hb[UPL * V];  // blended source rows ya and yb
         int32_t ya = -1, yb = -1;
         auto blend_row = [&](float* hrow, int32_t ys) {
             const T* row = xn + (int64_t)ys * src_row;
-            T l[V], r[V];
-            copy_unit<VB>(l, row + o0);
-            copy_unit<VB>(r, row + o1);
+            T l[UPL * V], r[UPL * V];
 #pragma unroll
-            for (int i = 0; i < V; i++) {
-                hrow[i] = omdx * ElemIO<T>::load(&l[i]) + dx * ElemIO<T>::load(&r[i]);
+            for (int u = 0; u < UPL; u++) {
+                copy_unit<VB>(l + u * V, row + o0[u]);
+                copy_unit<VB>(r + u * V, row + o1[u]);
+            }
+#pragma unroll
+            for (int i = 0; i < UPL * V; i++) {
+                hrow[i] = omdx[i / V] * ElemIO<T>::load(&l[i]) + dx[i / V] * ElemIO<T>::load(&r[i]);
             }
         };
         for (int32_t h = h_begin; h < h_end; h++) {
@@ -385,7 +396,7 @@ __global__ __launch_bounds__(kThreads) void resize_nhwc_unit_kernel(const T* __r
             if (y0 != ya) {
                 if (y0 == yb) {
 #pragma unroll
-                    for (int i = 0; i < V; i++) {
+                    for (int i = 0; i < UPL * V; i++) {
                         ha[i] = hb[i];
                     }
                 } else {
@@ -397,13 +408,20 @@ __global__ __launch_bounds__(kThreads) void resize_nhwc_unit_kernel(const T* __r
                 blend_row(hb, y1);
                 yb = y1;
             }
-            T outv[V];
+            T outv[UPL * V];
 #pragma unroll
-            for (int i = 0; i < V; i++) {
+            for (int i = 0; i < UPL * V; i++) {
                 const float bot = (y1 == ya) ? ha[i] : hb[i];
                 ElemIO<T>::store(&outv[i], omdy * ha[i] + dy * bot);
             }
-            copy_unit<VB>(y + ((n * Hd + h) * row_vecs + e) * V, outv);
+            T* dst = y + ((n * Hd + h) * row_vecs + e) * V;
+            if (whole) {
+                copy_unit<UPL * VB>(dst, outv);
+            } else {
+                for (int u = 0; u < UPL && e + u < row_vecs; u++) {
+                    copy_unit<VB>(dst + u * V, outv + u * V);
+                }
+            }
         }
     }
 }
@@ -786,24 +804,28 @@ bool nhwc_vec_ok(const ResizeArgs& a)
            reinterpret_cast<uintptr_t>(a.y) % 16 == 0;
 }
 
-// Bytes per lane of the element-aligned NHWC band variant: the widest of 16, 12, 8, 6, 4 that divides the bytes of a
-// pixel's channels and holds more than one element; sizeof(T) when there is none (the per-element kernel).
+// Bytes per lane of the element-aligned NHWC band variant: the widest of 16, 12, 8, 6, 4, 2 that divides the bytes of
+// a pixel's channels; 0 when the variant does not apply (the per-element kernel runs).
 template <typename T>
 int nhwc_unit_bytes(const ResizeArgs& a)
 {
     const int esz = (int)sizeof(T);
     if (!a.channels_last || a.mode != ResizeMode::Bilinear || (a.Hd + kNhwcBand - 1) / kNhwcBand > 65535 ||
         reinterpret_cast<uintptr_t>(a.x) % esz != 0 || reinterpret_cast<uintptr_t>(a.y) % esz != 0) {
-        return esz;
+        return 0;
+    }
+    const char* v = getenv("OPSCV_RESIZE_VARIANT");
+    if (v != nullptr && v[0] == 'g') {
+        return 0;
     }
     const int64_t pixel_bytes = a.C * esz;
-    static const int kUnits[5] = {16, 12, 8, 6, 4};
+    static const int kUnits[6] = {16, 12, 8, 6, 4, 2};
     for (int u : kUnits) {
-        if (u > esz && u % esz == 0 && pixel_bytes % u == 0) {
+        if (u % esz == 0 && pixel_bytes % u == 0) {
             return u;
         }
     }
-    return esz;
+    return 0;
 }
 
 // Channels per lane of the four-weights kernel: the widest of 16 bytes, 8 bytes or one element that divides C and
@@ -959,21 +981,29 @@ hipError_t run_resize(const ResizeArgs& a, hipStream_t stream)
     }
     if (a.channels_last) {
         const int vb = nhwc_unit_bytes<T>(a);
-        if (vb > (int)sizeof(T)) {
-            const int64_t row_vecs = a.Wd * (a.C * (int64_t)sizeof(T) / vb);
+        if (vb != 0) {
+            // Units per lane.  Several units of 2 or 4 bytes per lane make the stores 16 bytes wide, which pays when
+            // rows grow (neighbouring units read neighbouring source pixels); when rows shrink, and for wider units,
+            // the lanes' loads coalesce better with one unit each.
+            const int upl = (vb > 4 || a.Wd < a.Ws) ? 1 : 16 / vb;
+            const int64_t row_lanes = (a.Wd * (a.C * (int64_t)sizeof(T) / vb) + upl - 1) / upl;
             const int64_t bands = (a.Hd + kNhwcBand - 1) / kNhwcBand;
-            dim3 grid((unsigned)((row_vecs + kThreads - 1) / kThreads), (unsigned)bands,
+            dim3 grid((unsigned)((row_lanes + kThreads - 1) / kThreads), (unsigned)bands,
                       (unsigned)(a.N < 65535 ? a.N : 65535));
-#define OPSCV_NHWC_UNIT(HP, VB)                                                                                      \
-    hipLaunchKernelGGL((resize_nhwc_unit_kernel<T, HP, kNhwcBand, VB>), grid, dim3(kThreads), 0, stream, x, y, a.N,   \
-                       (int32_t)a.C, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h, a.scale_w)
+#define OPSCV_NHWC_UNIT(HP, VB, UPL)                                                                                 \
+    hipLaunchKernelGGL((resize_nhwc_unit_kernel<T, HP, kNhwcBand, VB, UPL>), grid, dim3(kThreads), 0, stream, x, y,   \
+                       a.N, (int32_t)a.C, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h,      \
+                       a.scale_w)
 #define OPSCV_NHWC_UNITS(HP)                                                                                         \
-    switch (vb) {                                                                                                    \
-        case 16: OPSCV_NHWC_UNIT(HP, 16); break;                                                                     \
-        case 12: OPSCV_NHWC_UNIT(HP, 12); break;                                                                     \
-        case 8: OPSCV_NHWC_UNIT(HP, 8); break;                                                                       \
-        case 6: if constexpr (sizeof(T) == 2) { OPSCV_NHWC_UNIT(HP, 6); } break;                                     \
-        default: if constexpr (sizeof(T) == 2) { OPSCV_NHWC_UNIT(HP, 4); } break;                                    \
+    switch (vb * 16 + upl) {                                                                                         \
+        case 16 * 16 + 1: OPSCV_NHWC_UNIT(HP, 16, 1); break;                                                         \
+        case 12 * 16 + 1: OPSCV_NHWC_UNIT(HP, 12, 1); break;                                                         \
+        case 8 * 16 + 1: OPSCV_NHWC_UNIT(HP, 8, 1); break;                                                           \
+        case 6 * 16 + 1: if constexpr (sizeof(T) == 2) { OPSCV_NHWC_UNIT(HP, 6, 1); } break;                         \
+        case 4 * 16 + 1: OPSCV_NHWC_UNIT(HP, 4, 1); break;                                                           \
+        case 4 * 16 + 4: OPSCV_NHWC_UNIT(HP, 4, 4); break;                                                           \
+        case 2 * 16 + 1: if constexpr (sizeof(T) == 2) { OPSCV_NHWC_UNIT(HP, 2, 1); } break;                         \
+        default: if constexpr (sizeof(T) == 2) { OPSCV_NHWC_UNIT(HP, 2, 8); } break;                                 \
     }
             if (a.half_pixel) {
                 OPSCV_NHWC_UNITS(true)
@@ -1070,13 +1100,13 @@ const char* resize_variant(const ResizeArgs& a)
         if (vec) {
             return "nhwc_vec";
         }
-        int vb = 0, esz = elem_size(a.elem);
+        int vb = 0;
         switch (a.elem) {
             case Elem::F32: vb = nhwc_unit_bytes<float>(a); break;
             case Elem::F16: vb = nhwc_unit_bytes<_Float16>(a); break;
             case Elem::BF16: vb = nhwc_unit_bytes<__bf16>(a); break;
         }
-        return vb > esz ? "nhwc_unit" : "nhwc_generic";
+        return vb != 0 ? "nhwc_unit" : "nhwc_generic";
     }
     if (const char* lds_variant = resize_lds_variant(a)) {
         return lds_variant;

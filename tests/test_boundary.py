@@ -237,7 +237,7 @@ def test_upsample_template_selection(aclnn, desc):
     assert _up(aclnn, desc, inp=(2, 128, 128, 256), out=(2, 192, 192, 256), size=(192, 192), dt=f32,
                fmt=aclnn.ACL_FORMAT_NHWC, align=True)[2] == "nhwc_vec"
     assert _up(aclnn, desc, inp=(2, 12, 12, 5), out=(2, 18, 18, 5), size=(18, 18), dt=f32,
-               fmt=aclnn.ACL_FORMAT_NHWC, align=True)[2] == "nhwc_generic"
+               fmt=aclnn.ACL_FORMAT_NHWC, align=True)[2] == "nhwc_unit"
 
 
 def test_upsample_template_selection_channels_last(aclnn, desc):
@@ -268,7 +268,7 @@ def test_upsample_template_selection_channels_last(aclnn, desc):
     assert variant((1, 8, 8, 32), (1, 3, 3, 32), f32, False) == "nhwc_four_weights"
     assert variant((1, 8, 8, 32), (1, 3, 3, 32), f16, False) == "nhwc_vec"
     assert variant((1, 1, 1, 14), (1, 13, 7, 14), f32, False) == "nhwc_unit"      # 56-byte pixels: 8-byte units
-    assert variant((1, 1, 1, 7), (1, 13, 7, 7), f32, False) == "nhwc_generic"     # no unit wider than an element
+    assert variant((1, 1, 1, 7), (1, 13, 7, 7), f32, False) == "nhwc_unit"        # one element per unit
     assert variant((1, 4, 4, 3), (1, 13, 7, 3), f32, False) == "nhwc_unit"        # three-channel images: 12 bytes
     assert variant((1, 4, 4, 3), (1, 13, 7, 3), f16, False) == "nhwc_unit"        # ... and 6 bytes
     assert variant((1, 1, 1, 14), (1, 13, 7, 14), f32, True) == "broadcast"
