@@ -81,6 +81,22 @@ def test_upsample_nhwc(oracle, device, aclnn, dtype, align):
 
 
 @pytest.mark.parametrize("dtype", I.DTYPES)
+def test_upsample_nhwc_per_element_kernel(oracle, device, aclnn, dtype, monkeypatch):
+    """the per-element channels-last kernel (kept for band counts beyond the grid limit) is reachable through
+    OPSCV_RESIZE_VARIANT=generic and matches the oracle like the band kernels"""
+    torch = _torch()
+    monkeypatch.setenv("OPSCV_RESIZE_VARIANT", "generic")
+    rng = np.random.default_rng(29)
+    for (N, C, H, W), size, align in [((2, 5, 7, 9), (14, 18), False), ((1, 3, 9, 6), (4, 11), True),
+                                      ((1, 7, 12, 10), (5, 23), False)]:
+        x = I.cast_np(rng.standard_normal((N, H, W, C)).astype(np.float32), dtype)
+        ref = oracle.upsample_bilinear2d_nhwc(x, size, align, dtype=I.oracle_code(dtype))
+        y = aclnn.upsample_bilinear2d(I.to_torch(x, dtype, device), size, align, channels_last=True)
+        torch.cuda.synchronize()
+        assert np.array_equal(_bits(I.from_torch(y, dtype), dtype), _bits(ref, dtype)), (dtype, N, C, H, W, align)
+
+
+@pytest.mark.parametrize("dtype", I.DTYPES)
 def test_grid_sampler_variants_agree(oracle, device, aclnn, dtype):
     """every kernel variant (LDS ring classes, direct fallback for odd or oversized planes) matches the oracle"""
     torch = _torch()
