@@ -105,6 +105,10 @@ def load_library():
                                                              p_vp]
     L.aclnnGridSampler2DBackward.restype = i32
     L.aclnnGridSampler2DBackward.argtypes = [vp, u64, vp, vp]
+    L.aclnnGridSampler3DBackwardGetWorkspaceSize.restype = i32
+    L.aclnnGridSampler3DBackwardGetWorkspaceSize.argtypes = L.aclnnGridSampler2DBackwardGetWorkspaceSize.argtypes
+    L.aclnnGridSampler3DBackward.restype = i32
+    L.aclnnGridSampler3DBackward.argtypes = [vp, u64, vp, vp]
     L.aclnnGridSampler3DGetWorkspaceSize.restype = i32
     L.aclnnGridSampler3DGetWorkspaceSize.argtypes = [vp, vp, i64, i64, ctypes.c_bool, vp, p_u64, p_vp]
     L.aclnnGridSampler3D.restype = i32
@@ -201,6 +205,18 @@ def get_workspace_size_grid_sampler2d_backward(grad_out, inp, grid, interpolatio
     ws = ctypes.c_uint64(0)
     ex = ctypes.c_void_p(None)
     st = L.aclnnGridSampler2DBackwardGetWorkspaceSize(grad_out, inp, grid, interpolation_mode, padding_mode,
+                                                      bool(align_corners), output_mask, input_grad, grid_grad,
+                                                      ctypes.byref(ws), ctypes.byref(ex))
+    return st, ws.value, ex.value
+
+
+def get_workspace_size_grid_sampler3d_backward(grad_out, inp, grid, interpolation_mode, padding_mode, align_corners,
+                                               output_mask, input_grad, grid_grad):
+    """Phase 1 of aclnnGridSampler3DBackward on raw handles; returns (status, workspace_bytes, executor_handle)."""
+    L = load_library()
+    ws = ctypes.c_uint64(0)
+    ex = ctypes.c_void_p(None)
+    st = L.aclnnGridSampler3DBackwardGetWorkspaceSize(grad_out, inp, grid, interpolation_mode, padding_mode,
                                                       bool(align_corners), output_mask, input_grad, grid_grad,
                                                       ctypes.byref(ws), ctypes.byref(ex))
     return st, ws.value, ex.value
@@ -349,6 +365,40 @@ def grid_sampler2d_backward(grad_out, inp, grid, interpolation_mode=0, padding_m
         st = L.aclnnGridSampler2DBackward(wptr, wsize, ex, _stream_handle(stream))
         if st != ACLNN_SUCCESS:
             raise AclnnError("aclnnGridSampler2DBackward", st)
+    finally:
+        for h in hs:
+            destroy_tensor(h)
+        destroy_bool_array(mask)
+    return input_grad, grid_grad
+
+
+def grid_sampler3d_backward(grad_out, inp, grid, interpolation_mode=0, padding_mode=0, align_corners=False,
+                            output_mask=(True, True), input_grad=None, grid_grad=None, stream=None, workspace=None,
+                            channels_last=False):
+    """Both phases of aclnnGridSampler3DBackward on torch CUDA tensors; returns (input_grad, grid_grad).  A gradient
+    whose mask flag is false is left untouched.  With channels_last, grad_out, inp and input_grad are (N,D,H,W,C)."""
+    torch = _torch()
+    L = load_library()
+    if input_grad is None:
+        input_grad = torch.empty_like(inp)
+    if grid_grad is None:
+        grid_grad = torch.empty_like(grid)
+    fmt = ACL_FORMAT_NDHWC if channels_last else ACL_FORMAT_NCDHW
+    hs = [tensor_handle(grad_out, fmt), tensor_handle(inp, fmt), tensor_handle(grid), tensor_handle(input_grad, fmt),
+          tensor_handle(grid_grad)]
+    mask = create_bool_array(list(output_mask))
+    try:
+        st, ws, ex = get_workspace_size_grid_sampler3d_backward(hs[0], hs[1], hs[2], interpolation_mode, padding_mode,
+                                                                align_corners, mask, hs[3], hs[4])
+        if st != ACLNN_SUCCESS:
+            raise AclnnError("aclnnGridSampler3DBackwardGetWorkspaceSize", st)
+        if ws > 0 and (workspace is None or workspace.numel() * workspace.element_size() < ws):
+            workspace = torch.empty(ws, dtype=torch.uint8, device=inp.device)
+        wptr = ctypes.c_void_p(workspace.data_ptr()) if ws > 0 else None
+        wsize = workspace.numel() * workspace.element_size() if ws > 0 else 0
+        st = L.aclnnGridSampler3DBackward(wptr, wsize, ex, _stream_handle(stream))
+        if st != ACLNN_SUCCESS:
+            raise AclnnError("aclnnGridSampler3DBackward", st)
     finally:
         for h in hs:
             destroy_tensor(h)

@@ -80,7 +80,8 @@ struct StridedView {
     int64_t strides[kViewDims] = {0};  // elements
 };
 
-enum class OpKind : int { Nop = 0, GridSampler2D = 1, Resize = 2, ResizeGrad = 3, GridSampler3D = 4, GridSampler2DGrad = 5 };
+enum class OpKind : int { Nop = 0, GridSampler2D = 1, Resize = 2, ResizeGrad = 3, GridSampler3D = 4, GridSampler2DGrad = 5,
+                          GridSampler3DGrad = 6 };
 
 // Where a kernel operand lives: the tensor's own memory (contiguous view) or a slice of the caller's
 // workspace, known only as an offset until the second phase receives the workspace address.
@@ -127,6 +128,21 @@ struct GridSamplerGradArgs {
     const void* grid = nullptr;  // (N,Hout,Wout,2)
     void* dx = nullptr;          // (N,C,Hin,Win)
     void* dgrid = nullptr;       // (N,Hout,Wout,2)
+};
+
+// Backward of the 3-D sampler.  dx / dgrid may be null (output mask): that gradient is then not computed.
+struct GridSampler3DGradArgs {
+    Elem elem = Elem::F32;
+    int interp = 0;  // 0 bilinear, 1 nearest
+    int pad = 0;
+    int align = 0;
+    int64_t N = 0, C = 0, Din = 0, Hin = 0, Win = 0, Dout = 0, Hout = 0, Wout = 0;
+    int64_t items_per_core = 1;  // batch items the reference walks as one run of grid points (chunk boundaries)
+    const void* gout = nullptr;  // (N,C,Dout,Hout,Wout)
+    const void* x = nullptr;     // (N,C,Din,Hin,Win)
+    const void* grid = nullptr;  // (N,Dout,Hout,Wout,3)
+    void* dx = nullptr;          // (N,C,Din,Hin,Win)
+    void* dgrid = nullptr;       // (N,Dout,Hout,Wout,3)
 };
 
 enum class ResizeMode : int {
@@ -180,6 +196,7 @@ struct aclOpExecutor {
     opscv::ResizeGradArgs rg;
     opscv::GridSampler3DArgs gs3;
     opscv::GridSamplerGradArgs gsg;
+    opscv::GridSampler3DGradArgs gsg3;
     int want_out0 = 1, want_out1 = 0;  // which outputs the operator produces (backward output mask)
     opscv::PlannedPtr in0, in1, out0;  // input/self, grid, out
     opscv::PlannedPtr in2, out1;       // third input and second output of the operators that have them

@@ -121,6 +121,19 @@ aclnnStatus run_executor(void* workspace, uint64_t workspace_size, aclOpExecutor
             return ACLNN_ERR_PARAM_NULLPTR;
         }
         e = launch_grid_sampler2d_grad(a, s);
+    } else if (ex->kind == OpKind::GridSampler3DGrad) {
+        GridSampler3DGradArgs a = ex->gsg3;
+        a.gout = resolve(ex->in0, workspace);
+        a.x = resolve(ex->in1, workspace);
+        a.grid = resolve(ex->in2, workspace);
+        a.dx = ex->want_out0 ? resolve(ex->out0, workspace) : nullptr;
+        a.dgrid = ex->want_out1 ? resolve(ex->out1, workspace) : nullptr;
+        if (a.gout == nullptr || a.x == nullptr || a.grid == nullptr || (ex->want_out0 && a.dx == nullptr) ||
+            (ex->want_out1 && a.dgrid == nullptr)) {
+            set_error("%s: tensor data pointer is NULL", api);
+            return ACLNN_ERR_PARAM_NULLPTR;
+        }
+        e = launch_grid_sampler3d_grad(a, s);
     } else if (ex->kind == OpKind::GridSampler3D) {
         GridSampler3DArgs a = ex->gs3;
         a.x = resolve(ex->in0, workspace);

@@ -94,6 +94,7 @@ const char* opscvExecutorVariant(const aclOpExecutor* executor)
         case OpKind::Resize: return resize_variant(executor->rs);
         case OpKind::ResizeGrad: return executor->rg.copy ? "copy" : resize_grad_variant(executor->rg);
         case OpKind::GridSampler2DGrad: return "gs2d_grad_ordered";
+        case OpKind::GridSampler3DGrad: return "gs3d_grad_ordered";
         case OpKind::GridSampler3D:
             if (executor->gs3.channels_last) {
                 return executor->gs3.interp == 0 ? "gs3d_ndhwc_bilinear" : "gs3d_ndhwc_nearest";

@@ -1,0 +1,444 @@
+// Backward of the 3-D grid sampler for gfx950: gradient of the input volume (scatter) and of the grid, deterministic.
+//
+// Replaces the reference device kernel
+//   image/grid_sampler3_d_grad/op_kernel/arch35/grid_sampler3_d_grad_simt_det.h (deterministic mode)
+// and, up to the order of additions, its atomic mode (grid_sampler3_d_grad_simt.h).
+//
+// Gradient of the input.  The reference gives a core whole batch items and walks their grid points as one run of
+// indices in chunks of 256; within a chunk it adds, channel after channel and corner after corner (tnw, tne, tsw, tse,
+// bnw, bne, bsw, bse), the 256 contributions one by one in point order, each add rounding to the element type
+// (grid_sampler3_d_grad_simt_det.h:63-96).  The sum that reaches one voxel of the gradient is therefore a fixed
+// sequence: its contributions ordered by (chunk, corner, point).  Adds to different voxels commute.  A workgroup here
+// owns one (batch item, group of channels, band of the volume) held in LDS, walks the chunks in order and the corners
+// in order; contributions of one corner that land on the same voxel are applied in rounds, an LDS max-reduction
+// electing per voxel the waiting contribution of the lowest point.  When a core of the reference holds several batch
+// items, the chunk boundaries of its later items are shifted by (item * points) mod 256
+// (grid_sampler3_d_grad_tiling.cpp:183-191); `items_per_core` carries that.
+//
+// Gradient of the grid.  One lane per grid point walks the channels in order (grid_sampler3_d_grad_simt_det.h:
+// 98-330); no atomics are involved.
+#include <hip/hip_runtime.h>
+
+#include "gs2d_grad_math.hpp"
+#include "kernels.hpp"
+
+namespace opscv {
+
+namespace {
+
+constexpr int kThreads = 256;  // also the chunk length of the accumulation order
+constexpr uint32_t kKeyBits = 8;
+constexpr uint32_t kEpochMax = (1u << (32 - kKeyBits)) - 1;
+constexpr int kBandMax = 8192;  // voxels of the gradient a workgroup keeps in LDS
+
+struct Grad3Params {
+    int32_t C, D, H, W, points;
+    int32_t pad, align;
+    int32_t band_px;
+    int32_t items_per_core;
+};
+
+// Where the contributions of a grid point land in the (D, H, W) volume and with what weight.
+//   INTERP 0: eight corners, index = x-high + 2 * y-high + 4 * z-high; weight = rt<T>(wx * wy * wz)
+//   INTERP 1: one tap, weight 1
+// off[k] = -1 marks a corner outside the volume.
+template <typename T, int INTERP>
+struct GradTaps3 {
+    static constexpr int NT = (INTERP == 0) ? 8 : 1;
+    int32_t off[NT];
+    float w[NT];
+    float wx[2], wy[2], wz[2];  // per axis: weight of the low and of the high corner
+    float mx, my, mz;           // chain-rule multipliers of the grid gradient
+};
+
+__device__ __forceinline__ int32_t next_index(int32_t i)
+{
+    return (i == INT32_MAX) ? i : i + 1;
+}
+
+template <typename T, int INTERP>
+__device__ __forceinline__ void decide_grad_taps3(GradTaps3<T, INTERP>& t, float gx, float gy, float gz, int32_t D,
+                                                  int32_t H, int32_t W, int pad, int align)
+{
+    // grid_sampler3_d_grad_simt_det.h:381-383
+    const float fx = source_index_set_grad<T>(gx, W, pad, align, &t.mx);
+    const float fy = source_index_set_grad<T>(gy, H, pad, align, &t.my);
+    const float fz = source_index_set_grad<T>(gz, D, pad, align, &t.mz);
+    if (INTERP == 1) {
+        // grid_sampler3_d_grad_simt_det.h:340-342
+        const int32_t xi = float_to_i32(__builtin_rintf(fx));
+        const int32_t yi = float_to_i32(__builtin_rintf(fy));
+        const int32_t zi = float_to_i32(__builtin_rintf(fz));
+        const bool in = (uint32_t)xi < (uint32_t)W && (uint32_t)yi < (uint32_t)H && (uint32_t)zi < (uint32_t)D;
+        t.off[0] = in ? (zi * H + yi) * W + xi : -1;
+        t.w[0] = 1.0f;
+        return;
+    }
+    // grid_sampler3_d_grad_simt_det.h:281-297
+    const int32_t x0 = float_to_i32(__builtin_floorf(fx));
+    const int32_t y0 = float_to_i32(__builtin_floorf(fy));
+    const int32_t z0 = float_to_i32(__builtin_floorf(fz));
+    const int32_t x1 = next_index(x0), y1 = next_index(y0), z1 = next_index(z0);
+    t.wx[0] = (float)x1 - fx;
+    t.wx[1] = fx - (float)x0;
+    t.wy[0] = (float)y1 - fy;
+    t.wy[1] = fy - (float)y0;
+    t.wz[0] = (float)z1 - fz;
+    t.wz[1] = fz - (float)z0;
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        const int xs = k & 1, ys = (k >> 1) & 1, zs = k >> 2;
+        const int32_t cx = xs ? x1 : x0, cy = ys ? y1 : y0, cz = zs ? z1 : z0;
+        const bool in = (uint32_t)cx < (uint32_t)W && (uint32_t)cy < (uint32_t)H && (uint32_t)cz < (uint32_t)D;
+        t.off[k] = in ? (cz * H + cy) * W + cx : -1;
+        // the fp32 product is pinned before it is rounded to T (one rounding each, as in the reference)
+        t.w[k] = rt<T>(as_fp32_value(t.wx[xs] * t.wy[ys] * t.wz[zs]));
+    }
+}
+
+// What a corner adds: weight times incoming gradient in fp32, then rounded to the element type
+// (grid_sampler3_d_grad_simt_det.h:116-118,72-73).
+template <typename T, int INTERP>
+__device__ __forceinline__ float contribution3(float go, float w)
+{
+    if (INTERP == 1) {
+        return rt<T>(go);
+    }
+    return rt<T>(as_fp32_value(w * go));
+}
+
+// Thread of the chunk that holds the first grid point of batch item n.
+__device__ __forceinline__ int32_t chunk_phase(int64_t n, const Grad3Params& p)
+{
+    return (int32_t)(((n % p.items_per_core) * (int64_t)p.points) % kThreads);
+}
+
+template <typename T, int INTERP, int CB>
+__global__ __launch_bounds__(kThreads) void gs3d_grad_input_kernel(const T* __restrict__ gout,
+                                                                    const T* __restrict__ grid, T* __restrict__ dx,
+                                                                    Grad3Params p)
+{
+    using Taps = GradTaps3<T, INTERP>;
+    constexpr int NT = Taps::NT;
+    extern __shared__ uint32_t smem_u32[];
+    __shared__ uint32_t s_flag[2];
+    uint32_t* owner = smem_u32;
+    T* planes = reinterpret_cast<T*>(smem_u32 + p.band_px);  // [CB][band_px], values already in the element type
+
+    const int t = threadIdx.x;
+    const int32_t vol = p.D * p.H * p.W;
+    const int32_t b0 = blockIdx.x * p.band_px;
+    const int32_t b1 = (b0 + p.band_px < vol) ? b0 + p.band_px : vol;
+    const int32_t c0 = blockIdx.y * CB;
+    const int32_t nc = (c0 + CB <= p.C) ? CB : p.C - c0;
+    const int64_t n = blockIdx.z;
+    for (int32_t i = t; i < b1 - b0; i += kThreads) {
+        owner[i] = 0u;
+#pragma unroll
+        for (int cb = 0; cb < CB; cb++) {
+            ElemIO<T>::store(planes + cb * p.band_px + i, 0.0f);
+        }
+    }
+    if (t == 0) {
+        s_flag[0] = s_flag[1] = 0u;
+    }
+    __syncthreads();
+    const int32_t points = p.points;
+    const T* g_n = grid + n * (int64_t)points * 3;
+    const T* go_n = gout + (n * p.C + c0) * (int64_t)points;
+    uint32_t epoch = 1;
+    int fl = 0;
+    // the grid point and incoming gradients of the next chunk are requested before the rounds of this one
+    float gx_next = 0.0f, gy_next = 0.0f, gz_next = 0.0f, go_next[CB];
+#pragma unroll
+    for (int cb = 0; cb < CB; cb++) {
+        go_next[cb] = 0.0f;
+    }
+    auto request = [&](int32_t pt) {
+        gx_next = ElemIO<T>::load(g_n + 3 * (int64_t)pt);
+        gy_next = ElemIO<T>::load(g_n + 3 * (int64_t)pt + 1);
+        gz_next = ElemIO<T>::load(g_n + 3 * (int64_t)pt + 2);
+#pragma unroll
+        for (int cb = 0; cb < CB; cb++) {
+            if (cb < nc) {
+                go_next[cb] = ElemIO<T>::load(go_n + (int64_t)cb * points + pt);
+            }
+        }
+    };
+    const int32_t first = -chunk_phase(n, p);
+    if (first + t >= 0 && first + t < points) {
+        request(first + t);
+    }
+    for (int32_t base = first; base < points; base += kThreads) {
+        const int32_t pt = base + t;
+        const float gx = gx_next, gy = gy_next, gz = gz_next;
+        float go[CB];
+#pragma unroll
+        for (int cb = 0; cb < CB; cb++) {
+            go[cb] = go_next[cb];
+        }
+        if (pt + kThreads >= 0 && pt + kThreads < points) {
+            request(pt + kThreads);
+        }
+        int32_t off[NT];
+        float wt[NT];
+        uint32_t pend = 0;
+        if (pt >= 0 && pt < points) {
+            Taps tp;
+            decide_grad_taps3<T, INTERP>(tp, gx, gy, gz, p.D, p.H, p.W, p.pad, p.align);
+#pragma unroll
+            for (int k = 0; k < NT; k++) {
+                off[k] = tp.off[k] - b0;
+                wt[k] = tp.w[k];
+                if (tp.off[k] >= b0 && tp.off[k] < b1) {
+                    pend |= 1u << k;
+                }
+            }
+        }
+        // a chunk none of whose points touches this band costs one barrier
+        if (__syncthreads_or((int)pend) == 0) {
+            continue;
+        }
+        if (epoch > kEpochMax - 2u * NT * kThreads) {  // uniform: start the election tags over
+            __syncthreads();
+            for (int32_t i = t; i < b1 - b0; i += kThreads) {
+                owner[i] = 0u;
+            }
+            if (t == 0) {
+                s_flag[0] = s_flag[1] = 0u;
+            }
+            epoch = 1;
+            __syncthreads();
+        }
+        // Corner after corner, as the order demands.  A flag word holds the number of the last round for which a
+        // contribution of corner k is still waiting; round numbers only grow, so a stale value never matches.
+#pragma unroll
+        for (int k = 0; k < NT; k++) {
+            bool waiting = (pend & (1u << k)) != 0;
+            fl ^= 1;  // the other flag than the corner before: its last readers are behind this corner's first barrier
+            if (waiting) {
+                s_flag[fl] = epoch;
+            }
+            __syncthreads();
+            while (s_flag[fl] == epoch) {
+                const uint32_t key = (epoch << kKeyBits) | (uint32_t)(kThreads - 1 - t);
+                if (waiting) {
+                    atomicMax(&owner[off[k]], key);
+                }
+                __syncthreads();
+                if (waiting) {
+                    if (owner[off[k]] == key) {
+                        T* e = planes + off[k];
+#pragma unroll
+                        for (int cb = 0; cb < CB; cb++) {
+                            if (cb < nc) {
+                                const float val = contribution3<T, INTERP>(go[cb], wt[k]);
+                                ElemIO<T>::store(e + cb * p.band_px, ElemIO<T>::load(e + cb * p.band_px) + val);
+                            }
+                        }
+                        waiting = false;
+                    } else {
+                        s_flag[fl] = epoch + 1;  // somebody is left for the next round
+                    }
+                }
+                __syncthreads();
+                epoch++;
+            }
+            epoch++;
+        }
+    }
+    __syncthreads();
+    for (int cb = 0; cb < nc; cb++) {
+        T* dx_nc = dx + (n * p.C + c0 + cb) * (int64_t)vol + b0;
+        const T* pl = planes + cb * p.band_px;
+        for (int32_t i = t; i < b1 - b0; i += kThreads) {
+            dx_nc[i] = pl[i];
+        }
+    }
+}
+
+template <typename T, int INTERP>
+__global__ __launch_bounds__(kThreads) void gs3d_grad_grid_kernel(const T* __restrict__ gout, const T* __restrict__ x,
+                                                                   const T* __restrict__ grid, T* __restrict__ dgrid,
+                                                                   int64_t total, Grad3Params p)
+{
+    using Taps = GradTaps3<T, INTERP>;
+    const int64_t idx = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (idx >= total) {
+        return;
+    }
+    if (INTERP == 1) {
+        // grid_sampler3_d_grad_simt_det.h:354-356
+        ElemIO<T>::store(dgrid + 3 * idx, 0.0f);
+        ElemIO<T>::store(dgrid + 3 * idx + 1, 0.0f);
+        ElemIO<T>::store(dgrid + 3 * idx + 2, 0.0f);
+        return;
+    }
+    const int32_t points = p.points;
+    const int64_t n = idx / points;
+    const int32_t pt = (int32_t)(idx - n * points);
+    Taps tp;
+    decide_grad_taps3<T, INTERP>(tp, ElemIO<T>::load(grid + 3 * idx), ElemIO<T>::load(grid + 3 * idx + 1),
+                                 ElemIO<T>::load(grid + 3 * idx + 2), p.D, p.H, p.W, p.pad, p.align);
+    const int32_t vol = p.D * p.H * p.W;
+    const T* x_n = x + n * p.C * (int64_t)vol;
+    const T* go_n = gout + n * p.C * (int64_t)points + pt;
+    float gix = 0.0f, giy = 0.0f, giz = 0.0f;
+    bool ok[8];
+    int32_t o[8];
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        ok[k] = tp.off[k] >= 0;
+        o[k] = ok[k] ? tp.off[k] : 0;
+    }
+    // grid_sampler3_d_grad_simt_det.h:119-124 and the seven corners after it: value times two distances times the
+    // incoming gradient, left to right, subtracted for a low corner of the axis and added for a high one
+    auto accumulate = [&](float go, const float* v) {
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const int xs = k & 1, ys = (k >> 1) & 1, zs = k >> 2;
+            if (ok[k]) {
+                const float tx = v[k] * tp.wy[ys] * tp.wz[zs] * go;
+                const float ty = v[k] * tp.wx[xs] * tp.wz[zs] * go;
+                const float tz = v[k] * tp.wx[xs] * tp.wy[ys] * go;
+                gix = xs ? gix + tx : gix - tx;
+                giy = ys ? giy + ty : giy - ty;
+                giz = zs ? giz + tz : giz - tz;
+            }
+        }
+    };
+    // The sums run over the channels in order; the loads do not depend on them and are issued a group ahead.
+    constexpr int U = 4;
+    int32_t c = 0;
+    for (; c + U <= p.C; c += U) {
+        float go[U], v[U][8];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const T* xc = x_n + (int64_t)(c + u) * vol;
+            go[u] = ElemIO<T>::load(go_n + (int64_t)(c + u) * points);
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                v[u][k] = ElemIO<T>::load(xc + o[k]);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            accumulate(go[u], v[u]);
+        }
+    }
+    for (; c < p.C; c++) {
+        const T* xc = x_n + (int64_t)c * vol;
+        float v[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            v[k] = ElemIO<T>::load(xc + o[k]);
+        }
+        accumulate(ElemIO<T>::load(go_n + (int64_t)c * points), v);
+    }
+    // grid_sampler3_d_grad_simt_det.h:324-326: product in fp32, then the conversion
+    ElemIO<T>::store(dgrid + 3 * idx, as_fp32_value(tp.mx * gix));
+    ElemIO<T>::store(dgrid + 3 * idx + 1, as_fp32_value(tp.my * giy));
+    ElemIO<T>::store(dgrid + 3 * idx + 2, as_fp32_value(tp.mz * giz));
+}
+
+template <typename T, int INTERP>
+hipError_t launch_interp(const GridSampler3DGradArgs& a, hipStream_t stream)
+{
+    Grad3Params p;
+    p.C = (int32_t)a.C;
+    p.D = (int32_t)a.Din;
+    p.H = (int32_t)a.Hin;
+    p.W = (int32_t)a.Win;
+    p.points = (int32_t)(a.Dout * a.Hout * a.Wout);
+    p.pad = a.pad;
+    p.align = a.align;
+    p.items_per_core = (int32_t)(a.items_per_core > 0 ? a.items_per_core : 1);
+    const int64_t vol = a.Din * a.Hin * a.Win;
+    p.band_px = (int32_t)(vol < kBandMax ? vol : kBandMax);
+    if (a.dx != nullptr) {
+        const int64_t bands = (vol + p.band_px - 1) / p.band_px;
+        // 8 bytes of gradient per band voxel: 4 channels of a 16-bit type, 2 of fp32 (96 KB of LDS with the election
+        // tags); fewer channels than that run one per workgroup
+        constexpr int CBMAX = 8 / (int)sizeof(T);
+        const bool grouped = a.C >= CBMAX;
+        const int64_t cgroups = grouped ? (a.C + CBMAX - 1) / CBMAX : a.C;
+        if (bands > INT32_MAX || cgroups > 65535 || a.N > 65535) {
+            return hipErrorInvalidValue;
+        }
+        const dim3 grid((unsigned)bands, (unsigned)cgroups, (unsigned)a.N);
+        // more than the default 64 KB of dynamic LDS
+        static bool attr_set = false;
+        if (!attr_set) {
+            hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(gs3d_grad_input_kernel<T, INTERP, CBMAX>),
+                                                hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                kBandMax * (4 + CBMAX * (int)sizeof(T)));
+            if (ea == hipSuccess) {
+                ea = hipFuncSetAttribute(reinterpret_cast<const void*>(gs3d_grad_input_kernel<T, INTERP, 1>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         kBandMax * (4 + (int)sizeof(T)));
+            }
+            if (ea != hipSuccess) {
+                return ea;
+            }
+            attr_set = true;
+        }
+        if (grouped) {
+            hipLaunchKernelGGL((gs3d_grad_input_kernel<T, INTERP, CBMAX>), grid, dim3(kThreads),
+                               (size_t)p.band_px * (4 + CBMAX * sizeof(T)), stream, (const T*)a.gout,
+                               (const T*)a.grid, (T*)a.dx, p);
+        } else {
+            hipLaunchKernelGGL((gs3d_grad_input_kernel<T, INTERP, 1>), grid, dim3(kThreads),
+                               (size_t)p.band_px * (4 + sizeof(T)), stream, (const T*)a.gout, (const T*)a.grid,
+                               (T*)a.dx, p);
+        }
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) {
+            return e;
+        }
+    }
+    if (a.dgrid != nullptr) {
+        const int64_t total = a.N * (int64_t)p.points;
+        const int64_t blocks = (total + kThreads - 1) / kThreads;
+        if (blocks > INT32_MAX) {
+            return hipErrorInvalidValue;
+        }
+        hipLaunchKernelGGL((gs3d_grad_grid_kernel<T, INTERP>), dim3((unsigned)blocks), dim3(kThreads), 0, stream,
+                           (const T*)a.gout, (const T*)a.x, (const T*)a.grid, (T*)a.dgrid, total, p);
+        return hipGetLastError();
+    }
+    return hipSuccess;
+}
+
+template <typename T>
+hipError_t launch_typed(const GridSampler3DGradArgs& a, hipStream_t stream)
+{
+    switch (a.interp) {
+        case 0: return launch_interp<T, 0>(a, stream);
+        case 1: return launch_interp<T, 1>(a, stream);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace
+
+hipError_t launch_grid_sampler3d_grad(const GridSampler3DGradArgs& a, hipStream_t stream)
+{
+    if (a.gout == nullptr || a.x == nullptr || a.grid == nullptr || (a.dx == nullptr && a.dgrid == nullptr)) {
+        return hipErrorInvalidValue;
+    }
+    if (a.pad < 0 || a.pad > 2 || a.N <= 0 || a.C <= 0 || a.Din <= 0 || a.Hin <= 0 || a.Win <= 0 || a.Dout <= 0 ||
+        a.Hout <= 0 || a.Wout <= 0) {
+        return hipErrorInvalidValue;
+    }
+    if (a.Din * a.Hin * a.Win > INT32_MAX || a.Dout * a.Hout * a.Wout > INT32_MAX || a.C > INT32_MAX) {
+        return hipErrorInvalidValue;
+    }
+    switch (a.elem) {
+        case Elem::F32: return launch_typed<float>(a, stream);
+        case Elem::F16: return launch_typed<_Float16>(a, stream);
+        case Elem::BF16: return launch_typed<__bf16>(a, stream);
+    }
+    return hipErrorInvalidValue;
+}
+
+}  // namespace opscv

@@ -34,6 +34,7 @@ hipError_t launch_resize_grad(const ResizeGradArgs& a, hipStream_t stream);
 const char* resize_grad_variant(const ResizeGradArgs& a);  // which kernel launch_resize_grad picks (x may be null)
 hipError_t launch_grid_sampler2d_grad(const GridSamplerGradArgs& a, hipStream_t stream);
 hipError_t launch_grid_sampler3d(const GridSampler3DArgs& a, hipStream_t stream);
+hipError_t launch_grid_sampler3d_grad(const GridSampler3DGradArgs& a, hipStream_t stream);
 
 // gather == true : strided view -> contiguous buffer;  false : contiguous buffer -> strided view
 hipError_t launch_strided_copy(const StridedView& v, void* contiguous, int elem_bytes, bool gather,

@@ -1436,6 +1436,115 @@ int oracle_grid_sampler2d_backward(const void* gout, const void* x, const void* 
     return 0;
 }
 
+/* ------------------------------------------------------------------------------------------
+ * Backward of the 3-D grid sampler, deterministic mode
+ *   image/grid_sampler3_d_grad/op_kernel/arch35/grid_sampler3_d_grad_simt_det.h:63-398
+ *   image/grid_sampler3_d_grad/op_host/grid_sampler3_d_grad_tiling.cpp:175-192 (items per core)
+ * A core owns `per_core` whole batch items (1 while N does not exceed the core count, else
+ * ceil(N / cores)) and walks their grid points as one run of indices in chunks of 256 threads, so the
+ * chunk boundaries inside the second and later items of a core are shifted by (item * points) mod 256.
+ * Per chunk, channel and corner (tnw, tne, tsw, tse, bnw, bne, bsw, bse) one thread adds the staged
+ * contributions in thread order, each add in the element type.  Staged zeros added to element 0 for
+ * corners outside the volume are left out (they can only turn a -0 into +0).
+ * ---------------------------------------------------------------------------------------- */
+int oracle_grid_sampler3d_backward(const void* gout, const void* x, const void* grid, void* dx, void* dgrid,
+                                   int dtype, int64_t N, int64_t C, int64_t D, int64_t H, int64_t W, int64_t Do,
+                                   int64_t Ho, int64_t Wo, int interp, int pad, int align)
+{
+    if (gout == NULL || x == NULL || grid == NULL || dtype < 0 || dtype > 2 || interp < 0 || interp > 1 || pad < 0 ||
+        pad > 2 || D <= 0 || H <= 0 || W <= 0) {
+        return -1;
+    }
+    const int64_t points = Do * Ho * Wo, vol = D * H * W;
+    if (dx != NULL) {
+        for (int64_t i = 0; i < N * C * vol; i++) {
+            store_from_float(dx, dtype, i, 0.0f);
+        }
+    }
+    const int64_t per_core = (N > g_reference_cores) ? (N + g_reference_cores - 1) / g_reference_cores : 1;
+    static _Thread_local int64_t st_idx[8][GSG_CHUNK];
+    static _Thread_local float st_val[8][GSG_CHUNK];
+#ifdef _OPENMP
+#pragma omp parallel for schedule(dynamic)
+#endif
+    for (int64_t n = 0; n < N; n++) {
+        const int64_t phase = ((n % per_core) * points) % GSG_CHUNK; /* thread of the item's first point */
+        for (int64_t base = -phase; base < points; base += GSG_CHUNK) {
+            const int64_t t_lo = (base < 0) ? -base : 0;
+            const int64_t t_hi = (points - base < GSG_CHUNK) ? points - base : GSG_CHUNK;
+            float gi[3][GSG_CHUNK], mult[3][GSG_CHUNK];
+            for (int64_t t = t_lo; t < t_hi; t++) {
+                gi[0][t] = gi[1][t] = gi[2][t] = 0.0f;
+            }
+            for (int64_t c = 0; c < C; c++) {
+                const int64_t xin = (n * C + c) * vol;
+                const int ntaps = (interp == 1) ? 1 : 8;
+                for (int64_t t = t_lo; t < t_hi; t++) {
+                    const int64_t p = base + t;
+                    float fx = load_as_float(grid, dtype, (n * points + p) * 3);
+                    float fy = load_as_float(grid, dtype, (n * points + p) * 3 + 1);
+                    float fz = load_as_float(grid, dtype, (n * points + p) * 3 + 2);
+                    const float go = load_as_float(gout, dtype, (n * C + c) * points + p);
+                    fx = gsg_source_index(dtype, fx, (int32_t)W, pad, align, &mult[0][t]);
+                    fy = gsg_source_index(dtype, fy, (int32_t)H, pad, align, &mult[1][t]);
+                    fz = gsg_source_index(dtype, fz, (int32_t)D, pad, align, &mult[2][t]);
+                    if (interp == 1) {
+                        int32_t zi = gsg_to_i32(rintf(fz)), yi = gsg_to_i32(rintf(fy)), xi = gsg_to_i32(rintf(fx));
+                        const int in = zi >= 0 && yi >= 0 && xi >= 0 && zi < D && yi < H && xi < W;
+                        st_idx[0][t] = in ? ((int64_t)zi * H + yi) * W + xi : -1;
+                        st_val[0][t] = rt(dtype, go);
+                        continue;
+                    }
+                    const int32_t x0 = gsg_to_i32(floorf(fx)), y0 = gsg_to_i32(floorf(fy)),
+                                  z0 = gsg_to_i32(floorf(fz));
+                    const int32_t x1 = (x0 == INT32_MAX) ? x0 : x0 + 1, y1 = (y0 == INT32_MAX) ? y0 : y0 + 1,
+                                  z1 = (z0 == INT32_MAX) ? z0 : z0 + 1;
+                    /* distance to the far corner per axis: index 0 weighs the low corner, 1 the high one */
+                    const float wx[2] = {(float)x1 - fx, fx - (float)x0};
+                    const float wy[2] = {(float)y1 - fy, fy - (float)y0};
+                    const float wz[2] = {(float)z1 - fz, fz - (float)z0};
+                    for (int k = 0; k < 8; k++) {
+                        const int xs = k & 1, ys = (k >> 1) & 1, zs = k >> 2;
+                        const int32_t cx = xs ? x1 : x0, cy = ys ? y1 : y0, cz = zs ? z1 : z0;
+                        const int in = cz >= 0 && cy >= 0 && cx >= 0 && cz < D && cy < H && cx < W;
+                        const float w = rt(dtype, wx[xs] * wy[ys] * wz[zs]);
+                        st_idx[k][t] = in ? ((int64_t)cz * H + cy) * W + cx : -1;
+                        st_val[k][t] = rt(dtype, w * go);
+                        if (in) {
+                            const float v = load_as_float(x, dtype, xin + st_idx[k][t]);
+                            const float tx = v * wy[ys] * wz[zs] * go;
+                            const float ty = v * wx[xs] * wz[zs] * go;
+                            const float tz = v * wx[xs] * wy[ys] * go;
+                            gi[0][t] = xs ? gi[0][t] + tx : gi[0][t] - tx;
+                            gi[1][t] = ys ? gi[1][t] + ty : gi[1][t] - ty;
+                            gi[2][t] = zs ? gi[2][t] + tz : gi[2][t] - tz;
+                        }
+                    }
+                }
+                if (dx != NULL) {
+                    for (int k = 0; k < ntaps; k++) {
+                        for (int64_t t = t_lo; t < t_hi; t++) {
+                            if (st_idx[k][t] >= 0) {
+                                const int64_t e = xin + st_idx[k][t];
+                                store_from_float(dx, dtype, e, load_as_float(dx, dtype, e) + st_val[k][t]);
+                            }
+                        }
+                    }
+                }
+            }
+            if (dgrid != NULL) {
+                for (int64_t t = t_lo; t < t_hi; t++) {
+                    const int64_t o = (n * points + base + t) * 3;
+                    for (int a = 0; a < 3; a++) {
+                        store_from_float(dgrid, dtype, o + a, (interp == 1 || C == 0) ? 0.0f : mult[a][t] * gi[a][t]);
+                    }
+                }
+            }
+        }
+    }
+    return 0;
+}
+
 int oracle_max_threads(void)
 {
 #ifdef _OPENMP

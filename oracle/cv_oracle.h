@@ -165,6 +165,16 @@ int oracle_grid_sampler2d_backward(const void* gout, const void* x, const void* 
                                    int dtype, int64_t N, int64_t C, int64_t H, int64_t W, int64_t Ho, int64_t Wo,
                                    int interp, int pad, int align);
 
+/*
+ * Backward of the 3-D grid sampler in the accumulation order of the reference's deterministic mode
+ * (image/grid_sampler3_d_grad/op_kernel/arch35/grid_sampler3_d_grad_simt_det.h).  gout (N,C,Do,Ho,Wo),
+ * x (N,C,D,H,W), grid (N,Do,Ho,Wo,3) ordered x,y,z; dx (N,C,D,H,W) and dgrid (N,Do,Ho,Wo,3) may each be NULL.
+ * interp 0 bilinear, 1 nearest.  The chunking follows oracle_set_reference_cores().
+ */
+int oracle_grid_sampler3d_backward(const void* gout, const void* x, const void* grid, void* dx, void* dgrid,
+                                   int dtype, int64_t N, int64_t C, int64_t D, int64_t H, int64_t W, int64_t Do,
+                                   int64_t Ho, int64_t Wo, int interp, int pad, int align);
+
 int oracle_max_threads(void);
 
 #ifdef __cplusplus

@@ -98,6 +98,8 @@ def lib():
     L.oracle_gs3d_clip.argtypes = [f32, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32]
     L.oracle_grid_sampler2d_backward.restype = ctypes.c_int
     L.oracle_grid_sampler2d_backward.argtypes = [vp] * 5 + [ctypes.c_int] + [i64] * 6 + [ctypes.c_int] * 3
+    L.oracle_grid_sampler3d_backward.restype = ctypes.c_int
+    L.oracle_grid_sampler3d_backward.argtypes = [vp] * 5 + [ctypes.c_int] + [i64] * 8 + [ctypes.c_int] * 3
     L.oracle_set_reference_cores.restype = None
     L.oracle_set_reference_cores.argtypes = [i64]
     L.oracle_resize_uses_hw_split.restype = ctypes.c_int
@@ -229,6 +231,23 @@ def grid_sampler2d_backward(gout, x, grid, interp=0, pad=0, align=False, dtype=N
                                               int(bool(align)))
     if rc != 0:
         raise ValueError("oracle_grid_sampler2d_backward rc=%d" % rc)
+    return dx, dg
+
+
+def grid_sampler3d_backward(gout, x, grid, interp=0, pad=0, align=False, dtype=None, want=(True, True)):
+    """gout (N,C,Do,Ho,Wo), x (N,C,D,H,W), grid (N,Do,Ho,Wo,3) -> (dx or None, dgrid or None)"""
+    gout, x, grid = (np.ascontiguousarray(a) for a in (gout, x, grid))
+    code = _code_of(x) if dtype is None else dtype
+    N, C, D, H, W = x.shape
+    _, Do, Ho, Wo, _ = grid.shape
+    assert gout.shape == (N, C, Do, Ho, Wo)
+    dx = np.empty_like(x) if want[0] else None
+    dg = np.empty_like(grid) if want[1] else None
+    rc = lib().oracle_grid_sampler3d_backward(_ptr(gout), _ptr(x), _ptr(grid), _ptr(dx) if want[0] else None,
+                                              _ptr(dg) if want[1] else None, code, N, C, D, H, W, Do, Ho, Wo, interp,
+                                              pad, int(bool(align)))
+    if rc != 0:
+        raise ValueError("oracle_grid_sampler3d_backward rc=%d" % rc)
     return dx, dg
 
 

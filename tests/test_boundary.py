@@ -524,6 +524,71 @@ def test_grid_sampler2d_backward_status_codes(aclnn, desc):
     assert st == 0 and ws >= 40 * 4
 
 
+def _gsb3(aclnn, desc, gout=(1, 1, 1, 2, 2), inp=(1, 1, 1, 3, 3), grid=(1, 1, 2, 2, 3), dx=_KEEP, dgrid=_KEEP, dt=None,
+          dts=None, interp=0, pad=0, align=False, mask=(True, True), fmt=None, **kw):
+    dt = aclnn.ACL_FLOAT if dt is None else dt
+    fmt = aclnn.ACL_FORMAT_NCDHW if fmt is None else fmt
+    dts = dts or {}
+    dx = inp if dx is _KEEP else dx
+    dgrid = grid if dgrid is _KEEP else dgrid
+    hs = [desc.t(shape, dts.get(name, dt), fmt=fmt, **(kw if name == "inp" else {}))
+          for name, shape in (("gout", gout), ("inp", inp), ("grid", grid), ("dx", dx), ("dgrid", dgrid))]
+    m = aclnn.create_bool_array(list(mask)) if mask is not None else None
+    st, ws, ex = aclnn.get_workspace_size_grid_sampler3d_backward(hs[0], hs[1], hs[2], interp, pad, align, m, hs[3],
+                                                                  hs[4])
+    variant = aclnn.executor_variant(ex) if ex else None
+    if ex:
+        assert aclnn.destroy_executor(ex) == 0
+    aclnn.destroy_bool_array(m)
+    return st, ws, variant
+
+
+def test_grid_sampler3d_backward_status_codes(aclnn, desc):
+    """image/grid_sampler3_d_grad/tests/ut/op_host/op_api/test_aclnn_grid_sampler3d_backward.cpp and the check order
+    of aclnn_grid_sampler3d_backward.cpp:174-238"""
+    INV, NULL = aclnn.ACLNN_ERR_PARAM_INVALID, aclnn.ACLNN_ERR_PARAM_NULLPTR
+    # dtype_float16 / dtype_float32 / dtype_bf16: the unit test's shapes
+    for dt in (aclnn.ACL_FLOAT, aclnn.ACL_FLOAT16, aclnn.ACL_BF16):
+        assert _gsb3(aclnn, desc, dt=dt) == (0, 0, "gs3d_grad_ordered")
+    # gradOutput_nullptr .. gridGrad_nullptr
+    for missing in ("gout", "inp", "grid", "dx", "dgrid"):
+        assert _gsb3(aclnn, desc, **{missing: None})[0] == NULL, missing
+    # a missing mask succeeds as a no-op before anything else is looked at
+    assert _gsb3(aclnn, desc, mask=None, inp=None) == (0, 0, "")
+    # output_mask_false_false: success, no work; a mask of another length is checked after the shapes
+    assert _gsb3(aclnn, desc, mask=(False, False)) == (0, 0, "")
+    assert _gsb3(aclnn, desc, mask=(True, False))[0] == 0 and _gsb3(aclnn, desc, mask=(False, True))[0] == 0
+    assert _gsb3(aclnn, desc, mask=(True,))[0] == INV
+    assert _gsb3(aclnn, desc, mask=(True, True, True))[0] == INV
+    # dtypes
+    for name in ("gout", "grid", "dx", "dgrid"):
+        assert _gsb3(aclnn, desc, dts={name: aclnn.ACL_FLOAT16})[0] == INV, name
+    assert _gsb3(aclnn, desc, dt=aclnn.ACL_INT32)[0] == INV
+    assert _gsb3(aclnn, desc, dt=aclnn.ACL_DOUBLE)[0] == INV
+    # mode_3, padding_mode_3; bicubic does not exist in three dimensions
+    assert _gsb3(aclnn, desc, interp=3)[0] == INV and _gsb3(aclnn, desc, interp=2)[0] == INV
+    assert _gsb3(aclnn, desc, interp=-1)[0] == INV
+    assert _gsb3(aclnn, desc, pad=3)[0] == INV
+    assert _gsb3(aclnn, desc, interp=1, pad=2, align=True)[0] == 0
+    # shape_n_input1_grid2, shape_c_input1_output2, shape_h_grid2_output3, shape_w_grid2_output4
+    assert _gsb3(aclnn, desc, grid=(2, 1, 2, 2, 3), dgrid=(2, 1, 2, 2, 3))[0] == INV
+    assert _gsb3(aclnn, desc, gout=(1, 2, 1, 2, 2))[0] == INV
+    assert _gsb3(aclnn, desc, gout=(1, 1, 1, 3, 2))[0] == INV
+    assert _gsb3(aclnn, desc, gout=(1, 1, 1, 2, 4))[0] == INV
+    assert _gsb3(aclnn, desc, gout=(1, 1, 2, 2, 2))[0] == INV
+    assert _gsb3(aclnn, desc, inp=(1, 1, 3, 3), dx=(1, 1, 3, 3))[0] == INV
+    assert _gsb3(aclnn, desc, grid=(1, 1, 2, 2, 2), dgrid=(1, 1, 2, 2, 2))[0] == INV
+    assert _gsb3(aclnn, desc, dx=(1, 1, 1, 3, 4))[0] == INV
+    assert _gsb3(aclnn, desc, dgrid=(1, 1, 2, 1, 3))[0] == INV
+    # empty tensors: success without work
+    assert _gsb3(aclnn, desc, gout=(0, 1, 1, 2, 2), inp=(0, 1, 1, 3, 3), grid=(0, 1, 2, 2, 3)) == (0, 0, "")
+    # channels-last: the format of input says where the channels are; such tensors are packed through the workspace
+    nd = aclnn.ACL_FORMAT_NDHWC
+    st, ws, v = _gsb3(aclnn, desc, gout=(1, 1, 2, 2, 5), inp=(1, 1, 3, 3, 5), fmt=nd)
+    assert st == 0 and v == "gs3d_grad_ordered" and ws >= (20 + 45 + 45) * 4
+    assert _gsb3(aclnn, desc, gout=(1, 1, 2, 2, 4), inp=(1, 1, 3, 3, 5), fmt=nd)[0] == INV
+
+
 def test_resize_template_selection_point_copy(aclnn, desc):
     """resize_bilinear_v2_tiling_arch35.cpp:254-303: channels-last runs of 128 bytes and more, shrunk by whole factors
     (odd ones with half-pixel centres), are copied instead of interpolated"""

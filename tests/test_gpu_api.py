@@ -470,6 +470,100 @@ def test_grid_sampler2d_backward_mask_views_and_torch(oracle, device, aclnn):
 
 
 @pytest.mark.parametrize("dtype", I.DTYPES)
+@pytest.mark.parametrize("interp", [0, 1])
+def test_grid_sampler3d_backward(oracle, device, aclnn, dtype, interp):
+    """aclnnGridSampler3DBackward against the oracle, bit for bit, both gradients: every padding and alignment,
+    several chunks of 256 points, volumes larger than one LDS band, points piling up on few voxels, special grid
+    values, channel counts around the group size"""
+    torch = _torch()
+    rng = np.random.default_rng(700 + interp)
+    shapes = [(2, 3, 2, 5, 8, 2, 3, 3), (1, 2, 4, 9, 11, 5, 7, 9), (2, 1, 30, 20, 17, 6, 20, 10),
+              (1, 5, 1, 1, 1, 3, 17, 31), (1, 2, 2, 3, 2, 10, 12, 10), (1, 4, 3, 3, 3, 1, 1, 1)]
+    for (N, C, D, H, W, Do, Ho, Wo) in shapes:
+        x = I.cast_np(rng.standard_normal((N, C, D, H, W)).astype(np.float32), dtype)
+        g32 = rng.uniform(-1.5, 1.5, (N, Do, Ho, Wo, 3)).astype(np.float32)
+        flat = g32.reshape(-1, 3)
+        special = np.array([np.nan, np.inf, -np.inf, 1e30, -1e30, 1.0, -1.0, 0.0], np.float32)
+        for j in range(min(len(special), flat.shape[0])):
+            flat[j, j % 3] = special[j]
+        g = I.cast_np(g32, dtype)
+        go = I.cast_np(rng.standard_normal((N, C, Do, Ho, Wo)).astype(np.float32), dtype)
+        for pad in range(3):
+            for align in (False, True):
+                rdx, rdg = oracle.grid_sampler3d_backward(go, x, g, interp, pad, align, dtype=I.oracle_code(dtype))
+                dx, dg = aclnn.grid_sampler3d_backward(I.to_torch(go, dtype, device), I.to_torch(x, dtype, device),
+                                                       I.to_torch(g, dtype, device), interp, pad, align)
+                torch.cuda.synchronize()
+                for got, ref, what in ((I.from_torch(dx, dtype), rdx, "dx"), (I.from_torch(dg, dtype), rdg, "dgrid")):
+                    rn = np.isnan(I.as_f32(ref, dtype))
+                    assert np.array_equal(np.isnan(I.as_f32(got, dtype)), rn), (what, N, C, D, H, W, pad, align)
+                    assert np.array_equal(np.where(rn, 0, _bits(got, dtype)), np.where(rn, 0, _bits(ref, dtype))), \
+                        (what, N, C, D, H, W, Do, Ho, Wo, pad, align)
+
+
+def test_grid_sampler3d_backward_core_split_mask_layouts_and_torch(oracle, device, aclnn, monkeypatch):
+    torch = _torch()
+    import torch.nn.functional as F
+    rng = np.random.default_rng(710)
+    # more batch items than cores of the reference device: a core walks several items as one run of points, which
+    # moves the chunk boundaries of the later ones (300 points: item 1 of a core starts at thread 44)
+    N, C, D, H, W, Do, Ho, Wo = 5, 2, 2, 3, 3, 3, 10, 10
+    x = rng.standard_normal((N, C, D, H, W)).astype(np.float16)
+    g = rng.uniform(-1.1, 1.1, (N, Do, Ho, Wo, 3)).astype(np.float16)
+    go = rng.standard_normal((N, C, Do, Ho, Wo)).astype(np.float16)
+    results = []
+    try:
+        for cores in (2, 64):
+            monkeypatch.setenv("OPSCV_REFERENCE_CORES", str(cores))
+            oracle.set_reference_cores(cores)
+            rdx, rdg = oracle.grid_sampler3d_backward(go, x, g, 0, 1, False)
+            dx, dg = aclnn.grid_sampler3d_backward(*(torch.from_numpy(a).to(device) for a in (go, x, g)), 0, 1, False)
+            torch.cuda.synchronize()
+            assert np.array_equal(dx.cpu().numpy().view(np.uint16), rdx.view(np.uint16)), cores
+            assert np.array_equal(dg.cpu().numpy().view(np.uint16), rdg.view(np.uint16)), cores
+            results.append(rdx)
+    finally:
+        oracle.set_reference_cores(64)
+        monkeypatch.delenv("OPSCV_REFERENCE_CORES")
+    assert not np.array_equal(results[0].view(np.uint16), results[1].view(np.uint16))  # the order is visible in fp16
+    # masks, strided views, channels-last, torch autograd (fp32)
+    N, C, D, H, W, Do, Ho, Wo = 2, 3, 4, 6, 5, 3, 7, 6
+    x = rng.standard_normal((N, C, D, H, W)).astype(np.float32)
+    g = rng.uniform(-1.2, 1.2, (N, Do, Ho, Wo, 3)).astype(np.float32)
+    go = rng.standard_normal((N, C, Do, Ho, Wo)).astype(np.float32)
+    xt, gt, got = (torch.from_numpy(a).to(device) for a in (x, g, go))
+    rdx, rdg = oracle.grid_sampler3d_backward(go, x, g, 0, 0, False)
+    dx = torch.full((N, C, D, H, W), 7.0, device=device)
+    dg = torch.full((N, Do, Ho, Wo, 3), 7.0, device=device)
+    aclnn.grid_sampler3d_backward(got, xt, gt, 0, 0, False, (True, False), dx, dg)
+    torch.cuda.synchronize()
+    assert np.array_equal(dx.cpu().numpy(), rdx) and (dg == 7.0).all()
+    dx.fill_(7.0)
+    aclnn.grid_sampler3d_backward(got, xt, gt, 0, 0, False, (False, True), dx, dg)
+    torch.cuda.synchronize()
+    assert np.array_equal(dg.cpu().numpy(), rdg) and (dx == 7.0).all()
+    dxbig = torch.full((N, C, D, H, W + 3), -1.0, device=device)
+    dgbig = torch.full((N, Do, Ho, Wo, 5), -1.0, device=device)
+    xv = torch.from_numpy(np.ascontiguousarray(x.transpose(0, 1, 2, 4, 3))).to(device).transpose(3, 4)
+    aclnn.grid_sampler3d_backward(got, xv, gt, 0, 0, False, (True, True), dxbig[..., 1:1 + W], dgbig[..., 1:4])
+    torch.cuda.synchronize()
+    assert np.array_equal(dxbig[..., 1:1 + W].cpu().numpy(), rdx) and np.array_equal(dgbig[..., 1:4].cpu().numpy(), rdg)
+    assert (dxbig[..., 0] == -1.0).all() and (dgbig[..., 4] == -1.0).all()
+    # channels-last operands give the channels-last gradient
+    xl, gol = (t.permute(0, 2, 3, 4, 1).contiguous() for t in (xt, got))
+    dxl, dgl = aclnn.grid_sampler3d_backward(gol, xl, gt, 0, 0, False, channels_last=True)
+    torch.cuda.synchronize()
+    assert np.array_equal(dxl.permute(0, 4, 1, 2, 3).cpu().numpy(), rdx) and np.array_equal(dgl.cpu().numpy(), rdg)
+    for mode, m in (("bilinear", 0), ("nearest", 1)):
+        xa, ga = xt.clone().requires_grad_(True), gt.clone().requires_grad_(True)
+        F.grid_sample(xa, ga, mode=mode, padding_mode="reflection", align_corners=True).backward(got)
+        dx, dg = aclnn.grid_sampler3d_backward(got, xt, gt, m, 2, True)
+        torch.cuda.synchronize()
+        assert (dx - xa.grad).abs().max().item() <= 1e-4
+        assert ((dg - ga.grad).abs() > 1e-3).float().mean().item() <= 0.02
+
+
+@pytest.mark.parametrize("dtype", I.DTYPES)
 def test_resize_nearest_wide_rows(oracle, device, aclnn, dtype):
     """nearest NCHW with whole-vector rows (the LDS-staged kernel): several column chunks, bands that straddle
     planes, non-integer factors, down-scaling, and a factor whose source segment exceeds the LDS slots"""

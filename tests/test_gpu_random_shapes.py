@@ -218,6 +218,24 @@ def test_random_sampler_backward_and_3d(oracle, device, aclnn):
         got = I.from_torch(y, dtype)
         got = got.transpose(0, 4, 1, 2, 3) if cl else got
         _same(got, ref, dtype, (case, "gs3d", dtype, N, C, D, H, W, Do, Ho, Wo, interp, pad, align, cl))
+        if case % 3 == 0:
+            # the backward of the same call; volumes above 8192 voxels span several LDS bands
+            if case % 6 == 0:
+                D, H, W = D + 12, H + 14, W + 16
+                x = I.cast_np(rng.standard_normal((N, C, D, H, W)).astype(np.float32), dtype)
+            _say("gs3d backward", dtype, N, C, D, H, W, Do, Ho, Wo, interp, pad, align, cl)
+            go = I.cast_np(rng.standard_normal((N, C, Do, Ho, Wo)).astype(np.float32), dtype)
+            rdx, rdg = oracle.grid_sampler3d_backward(go, x, g, interp, pad, align, dtype=I.oracle_code(dtype))
+            xin = np.ascontiguousarray(x.transpose(0, 2, 3, 4, 1)) if cl else x
+            gin = np.ascontiguousarray(go.transpose(0, 2, 3, 4, 1)) if cl else go
+            dx, dg = aclnn.grid_sampler3d_backward(I.to_torch(gin, dtype, device), I.to_torch(xin, dtype, device),
+                                                   I.to_torch(g, dtype, device), interp, pad, align, channels_last=cl)
+            torch.cuda.synchronize()
+            gdx = I.from_torch(dx, dtype)
+            gdx = gdx.transpose(0, 4, 1, 2, 3) if cl else gdx
+            what = (case, dtype, N, C, D, H, W, Do, Ho, Wo, interp, pad, align, cl)
+            _same(gdx, rdx, dtype, ("gs3d dx",) + what)
+            _same(I.from_torch(dg, dtype), rdg, dtype, ("gs3d dgrid",) + what)
 
 
 def _as_view(torch, rng, t, kind):

@@ -669,6 +669,75 @@ def test_grid_sampler2d_backward_order_is_sequential_in_element_type(oracle):
     assert dxb.ravel()[0] == acc
 
 
+def test_grid_sampler3d_backward_against_torch_autograd(oracle):
+    """both gradients of the 3-D sampler against torch autograd on 5-D inputs (fp32), and the adjoint identity with
+    the forward oracle"""
+    rng = np.random.default_rng(43)
+    modes = ["bilinear", "nearest"]
+    for trial in range(4):
+        N, C = 2, 3
+        D, H, W = rng.integers(2, 9, 3)
+        Do, Ho, Wo = rng.integers(1, 9, 3)  # up to 512 points: more than one chunk of 256
+        x = rng.standard_normal((N, C, D, H, W)).astype(np.float32)
+        g = rng.uniform(-1.4, 1.4, (N, Do, Ho, Wo, 3)).astype(np.float32)
+        go = rng.standard_normal((N, C, Do, Ho, Wo)).astype(np.float32)
+        for m in range(2):
+            for p in range(3):
+                for a in (False, True):
+                    dx, dg = oracle.grid_sampler3d_backward(go, x, g, m, p, a)
+                    wx, wg = _torch_gs_backward(x, g, go, modes[m], PADS[p], a)
+                    assert np.abs(dx - wx).max() <= 2e-5 * max(1.0, np.abs(wx).max()), (trial, m, p, a)
+                    bad = np.abs(dg - wg) > 2e-5 * max(1.0, np.abs(wg).max())
+                    assert bad.mean() <= 0.02, (trial, m, p, a, bad.mean())
+                    only_dg = oracle.grid_sampler3d_backward(go, x, g, m, p, a, want=(False, True))
+                    assert only_dg[0] is None and np.array_equal(only_dg[1], dg)
+                    y = oracle.grid_sampler3d(x, g, m, p, a)
+                    lhs = float((y.astype(np.float64) * go).sum())
+                    rhs = float((x.astype(np.float64) * dx).sum())
+                    assert abs(lhs - rhs) <= 1e-4 * max(1.0, abs(lhs)), (trial, m, p, a)
+
+
+def test_grid_sampler3d_backward_order_and_core_split(oracle):
+    """many points landing on one voxel: the sum is the left-to-right sum in the element type.  When the batch exceeds
+    the reference's core count, a core walks several items as one run of points, which moves the chunk boundaries of
+    its later items: values agree to rounding, the orders are both sequential per voxel, so a single voxel sees the
+    same sum either way"""
+    n_pts = 300
+    N = 3
+    x = np.zeros((N, 1, 1, 1, 1), np.float16)
+    g = np.zeros((N, 1, 1, n_pts, 3), np.float16)
+    go = (np.arange(N * n_pts) % 7 + 0.25).astype(np.float16).reshape(N, 1, 1, 1, n_pts)
+    want = []
+    for n in range(N):
+        acc = np.float16(0)
+        for v in go[n].ravel():
+            acc = np.float16(np.float32(acc) + np.float32(v))
+        want.append(acc)
+    try:
+        for cores in (64, 1):
+            oracle.set_reference_cores(cores)
+            for m in (0, 1):
+                dx, _ = oracle.grid_sampler3d_backward(go, x, g, m, 1, False)
+                assert [dx[n].ravel()[0] for n in range(N)] == want, (cores, m)
+        # two voxels hit alternately by points 0, 1, 2, ...: chunk boundaries do not reorder one voxel's own adds
+        x2 = np.zeros((N, 1, 1, 1, 2), np.float16)
+        g2 = np.zeros((N, 1, 1, n_pts, 3), np.float16)
+        g2[..., 0] = np.where(np.arange(n_pts) % 2 == 0, -1.0, 1.0)
+        res = []
+        for cores in (64, 1):
+            oracle.set_reference_cores(cores)
+            res.append(oracle.grid_sampler3d_backward(go, x2, g2, 1, 1, True)[0])
+        assert np.array_equal(res[0], res[1])
+        for n in range(N):
+            for v in range(2):
+                acc = np.float16(0)
+                for q in go[n].ravel()[v::2]:
+                    acc = np.float16(np.float32(acc) + np.float32(q))
+                assert res[0][n].ravel()[v] == acc
+    finally:
+        oracle.set_reference_cores(64)
+
+
 def test_resize_point_copy_oracle(oracle):
     """the point-copy template: a strided slice of the source, equal to the interpolating oracle on finite data
     and different from it exactly where a sampled value is infinite"""
