@@ -143,6 +143,9 @@ struct GridSampler3DGradArgs {
     const void* grid = nullptr;  // (N,Dout,Hout,Wout,3)
     void* dx = nullptr;          // (N,C,Din,Hin,Win)
     void* dgrid = nullptr;       // (N,Dout,Hout,Wout,3)
+    // optional scratch of gs3d_grad_range_words() 32-bit words: the span of voxels every chunk of grid points
+    // touches, which lets a band of the input gradient pass over the chunks that miss it; null: every chunk is looked at
+    void* chunk_ranges = nullptr;
 };
 
 enum class ResizeMode : int {
@@ -200,6 +203,7 @@ struct aclOpExecutor {
     int want_out0 = 1, want_out1 = 0;  // which outputs the operator produces (backward output mask)
     opscv::PlannedPtr in0, in1, out0;  // input/self, grid, out
     opscv::PlannedPtr in2, out1;       // third input and second output of the operators that have them
+    opscv::PlannedPtr scratch;         // kernel scratch inside the workspace (operators that use one)
     // packing work: views gathered into the workspace before the kernel, scattered after it
     struct Pack {
         opscv::StridedView view;

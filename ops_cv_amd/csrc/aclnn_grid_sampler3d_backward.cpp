@@ -7,6 +7,7 @@
 
 #include "aclnn_grid_sampler3d_backward.h"
 #include "executor.hpp"
+#include "kernels.hpp"
 #include "resize_plan.hpp"
 
 using namespace opscv;
@@ -206,6 +207,15 @@ aclnnStatus aclnnGridSampler3DBackwardGetWorkspaceSize(const aclTensor* gradOutp
     }
     if (want_dgrid) {
         ex->out1 = plan_view(ex.get(), gridGrad, esz, true);
+    }
+    if (want_dx) {
+        // scratch of the input-gradient kernel: the voxel span of every chunk of grid points
+        const int64_t words = gs3d_grad_range_words(a);
+        if (words > 0) {
+            ex->scratch.in_workspace = true;
+            ex->scratch.ws_offset = (ex->workspace_bytes + 255) / 256 * 256;
+            ex->workspace_bytes = ex->scratch.ws_offset + (uint64_t)words * 4;
+        }
     }
     *workspaceSize = ex->workspace_bytes;
     *executor = ex.release();

@@ -128,6 +128,7 @@ aclnnStatus run_executor(void* workspace, uint64_t workspace_size, aclOpExecutor
         a.grid = resolve(ex->in2, workspace);
         a.dx = ex->want_out0 ? resolve(ex->out0, workspace) : nullptr;
         a.dgrid = ex->want_out1 ? resolve(ex->out1, workspace) : nullptr;
+        a.chunk_ranges = ex->scratch.in_workspace ? resolve(ex->scratch, workspace) : nullptr;
         if (a.gout == nullptr || a.x == nullptr || a.grid == nullptr || (ex->want_out0 && a.dx == nullptr) ||
             (ex->want_out1 && a.dgrid == nullptr)) {
             set_error("%s: tensor data pointer is NULL", api);

@@ -9,9 +9,9 @@
 // bnw, bne, bsw, bse), the 256 contributions one by one in point order, each add rounding to the element type
 // (grid_sampler3_d_grad_simt_det.h:63-96).  The sum that reaches one voxel of the gradient is therefore a fixed
 // sequence: its contributions ordered by (chunk, corner, point).  Adds to different voxels commute.  A workgroup here
-// owns one (batch item, group of channels, band of the volume) held in LDS, walks the chunks in order and the corners
-// in order; contributions of one corner that land on the same voxel are applied in rounds, an LDS max-reduction
-// electing per voxel the waiting contribution of the lowest point.  When a core of the reference holds several batch
+// owns one (batch item, group of channels, band of the volume) held in LDS and walks the chunks in order; the
+// contributions of a chunk that land on the same voxel are applied in rounds, an LDS max-reduction electing per voxel
+// the waiting contribution of the lowest (corner, point).  When a core of the reference holds several batch
 // items, the chunk boundaries of its later items are shifted by (item * points) mod 256
 // (grid_sampler3_d_grad_tiling.cpp:183-191); `items_per_core` carries that.
 //
@@ -27,7 +27,8 @@ namespace opscv {
 namespace {
 
 constexpr int kThreads = 256;  // also the chunk length of the accumulation order
-constexpr uint32_t kKeyBits = 8;
+constexpr uint32_t kLaneBits = 8;              // 256 points of a chunk
+constexpr uint32_t kKeyBits = kLaneBits + 3;   // ... times eight corners
 constexpr uint32_t kEpochMax = (1u << (32 - kKeyBits)) - 1;
 constexpr int kBandMax = 8192;  // voxels of the gradient a workgroup keeps in LDS
 
@@ -36,6 +37,7 @@ struct Grad3Params {
     int32_t pad, align;
     int32_t band_px;
     int32_t items_per_core;
+    int32_t chunks;  // chunks a batch item is walked in, a possibly empty leading one included
 };
 
 // Where the contributions of a grid point land in the (D, H, W) volume and with what weight.
@@ -113,10 +115,65 @@ __device__ __forceinline__ int32_t chunk_phase(int64_t n, const Grad3Params& p)
     return (int32_t)(((n % p.items_per_core) * (int64_t)p.points) % kThreads);
 }
 
+// Chunks a batch item is walked in: with several items per core the first chunk of an item may start before its
+// first point.
+__host__ __device__ inline int32_t chunk_count(int64_t points, int64_t items_per_core)
+{
+    return (int32_t)(((items_per_core > 1 ? kThreads - 1 : 0) + points + kThreads - 1) / kThreads);
+}
+
+// Per (batch item, chunk): lowest and highest voxel any corner of the chunk's points lands on (lowest > highest for a
+// chunk with none).  One workgroup per chunk.
+template <typename T, int INTERP>
+__global__ __launch_bounds__(kThreads) void gs3d_grad_range_kernel(const T* __restrict__ grid,
+                                                                    int32_t* __restrict__ ranges, Grad3Params p)
+{
+    using Taps = GradTaps3<T, INTERP>;
+    __shared__ int32_t s_lo[kThreads / 64], s_hi[kThreads / 64];
+    const int t = threadIdx.x;
+    const int64_t n = blockIdx.y;
+    const int32_t pt = -chunk_phase(n, p) + (int32_t)blockIdx.x * kThreads + t;
+    int32_t lo = INT32_MAX, hi = -1;
+    if (pt >= 0 && pt < p.points) {
+        const T* g = grid + (n * (int64_t)p.points + pt) * 3;
+        Taps tp;
+        decide_grad_taps3<T, INTERP>(tp, ElemIO<T>::load(g), ElemIO<T>::load(g + 1), ElemIO<T>::load(g + 2), p.D, p.H,
+                                     p.W, p.pad, p.align);
+#pragma unroll
+        for (int k = 0; k < Taps::NT; k++) {
+            if (tp.off[k] >= 0) {
+                lo = tp.off[k] < lo ? tp.off[k] : lo;
+                hi = tp.off[k] > hi ? tp.off[k] : hi;
+            }
+        }
+    }
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+        const int32_t olo = __shfl_xor(lo, d), ohi = __shfl_xor(hi, d);
+        lo = olo < lo ? olo : lo;
+        hi = ohi > hi ? ohi : hi;
+    }
+    if ((t & 63) == 0) {
+        s_lo[t >> 6] = lo;
+        s_hi[t >> 6] = hi;
+    }
+    __syncthreads();
+    if (t == 0) {
+#pragma unroll
+        for (int w = 1; w < kThreads / 64; w++) {
+            lo = s_lo[w] < lo ? s_lo[w] : lo;
+            hi = s_hi[w] > hi ? s_hi[w] : hi;
+        }
+        int32_t* r = ranges + (n * (int64_t)p.chunks + blockIdx.x) * 2;
+        r[0] = lo;
+        r[1] = hi;
+    }
+}
+
 template <typename T, int INTERP, int CB>
 __global__ __launch_bounds__(kThreads) void gs3d_grad_input_kernel(const T* __restrict__ gout,
                                                                     const T* __restrict__ grid, T* __restrict__ dx,
-                                                                    Grad3Params p)
+                                                                    const int32_t* __restrict__ ranges, Grad3Params p)
 {
     using Taps = GradTaps3<T, INTERP>;
     constexpr int NT = Taps::NT;
@@ -166,20 +223,35 @@ __global__ __launch_bounds__(kThreads) void gs3d_grad_input_kernel(const T* __re
         }
     };
     const int32_t first = -chunk_phase(n, p);
-    if (first + t >= 0 && first + t < points) {
-        request(first + t);
-    }
-    for (int32_t base = first; base < points; base += kThreads) {
-        const int32_t pt = base + t;
+    // Chunks whose voxel span misses this band are passed over (the spans come from gs3d_grad_range_kernel; without
+    // them every chunk is looked at).  The choice is the same for the whole workgroup.
+    const int32_t* rng_n = (ranges != nullptr) ? ranges + n * 2 * (int64_t)p.chunks : nullptr;
+    auto next_busy = [&](int32_t ci) {
+        if (rng_n != nullptr) {
+            while (ci < p.chunks && (rng_n[2 * ci + 1] < b0 || rng_n[2 * ci] >= b1)) {
+                ci++;
+            }
+        }
+        return ci;
+    };
+    auto request_chunk = [&](int32_t ci) {
+        const int32_t pt = first + ci * kThreads + t;
+        if (ci < p.chunks && pt >= 0 && pt < points) {
+            request(pt);
+        }
+    };
+    int32_t ci = next_busy(0);
+    request_chunk(ci);
+    while (ci < p.chunks) {
+        const int32_t pt = first + ci * kThreads + t;
         const float gx = gx_next, gy = gy_next, gz = gz_next;
         float go[CB];
 #pragma unroll
         for (int cb = 0; cb < CB; cb++) {
             go[cb] = go_next[cb];
         }
-        if (pt + kThreads >= 0 && pt + kThreads < points) {
-            request(pt + kThreads);
-        }
+        ci = next_busy(ci + 1);
+        request_chunk(ci);
         int32_t off[NT];
         float wt[NT];
         uint32_t pend = 0;
@@ -195,10 +267,6 @@ __global__ __launch_bounds__(kThreads) void gs3d_grad_input_kernel(const T* __re
                 }
             }
         }
-        // a chunk none of whose points touches this band costs one barrier
-        if (__syncthreads_or((int)pend) == 0) {
-            continue;
-        }
         if (epoch > kEpochMax - 2u * NT * kThreads) {  // uniform: start the election tags over
             __syncthreads();
             for (int32_t i = t; i < b1 - b0; i += kThreads) {
@@ -210,42 +278,48 @@ __global__ __launch_bounds__(kThreads) void gs3d_grad_input_kernel(const T* __re
             epoch = 1;
             __syncthreads();
         }
-        // Corner after corner, as the order demands.  A flag word holds the number of the last round for which a
-        // contribution of corner k is still waiting; round numbers only grow, so a stale value never matches.
+        // All corners of the chunk take part in one election: per voxel the waiting contribution with the lowest
+        // (corner, point) wins the round, is added and retires, so a voxel receives its contributions in the order
+        // corner after corner, point after point, and a chunk takes as many rounds as its busiest voxel has
+        // contributions (mostly one or two) instead of at least one per corner.  The corners of one point are
+        // different voxels, so a lane may win several of them in a round.  A flag word holds the number of the last
+        // round for which a contribution is still waiting; round numbers only grow, so a stale value never matches.
+        // A chunk none of whose points touches this band costs one barrier.
+        fl ^= 1;  // the other flag than the chunk before: its last readers are behind this chunk's first barrier
+        if (pend != 0) {
+            s_flag[fl] = epoch;
+        }
+        __syncthreads();
+        while (s_flag[fl] == epoch) {
+            const uint32_t key = (epoch << kKeyBits) | (uint32_t)(kThreads - 1 - t);
 #pragma unroll
-        for (int k = 0; k < NT; k++) {
-            bool waiting = (pend & (1u << k)) != 0;
-            fl ^= 1;  // the other flag than the corner before: its last readers are behind this corner's first barrier
-            if (waiting) {
-                s_flag[fl] = epoch;
+            for (int k = 0; k < NT; k++) {
+                if (pend & (1u << k)) {
+                    atomicMax(&owner[off[k]], key | ((uint32_t)(NT - 1 - k) << kLaneBits));
+                }
             }
             __syncthreads();
-            while (s_flag[fl] == epoch) {
-                const uint32_t key = (epoch << kKeyBits) | (uint32_t)(kThreads - 1 - t);
-                if (waiting) {
-                    atomicMax(&owner[off[k]], key);
-                }
-                __syncthreads();
-                if (waiting) {
-                    if (owner[off[k]] == key) {
-                        T* e = planes + off[k];
 #pragma unroll
-                        for (int cb = 0; cb < CB; cb++) {
-                            if (cb < nc) {
-                                const float val = contribution3<T, INTERP>(go[cb], wt[k]);
-                                ElemIO<T>::store(e + cb * p.band_px, ElemIO<T>::load(e + cb * p.band_px) + val);
-                            }
+            for (int k = 0; k < NT; k++) {
+                if ((pend & (1u << k)) && owner[off[k]] == (key | ((uint32_t)(NT - 1 - k) << kLaneBits))) {
+                    T* e = planes + off[k];
+#pragma unroll
+                    for (int cb = 0; cb < CB; cb++) {
+                        if (cb < nc) {
+                            const float val = contribution3<T, INTERP>(go[cb], wt[k]);
+                            ElemIO<T>::store(e + cb * p.band_px, ElemIO<T>::load(e + cb * p.band_px) + val);
                         }
-                        waiting = false;
-                    } else {
-                        s_flag[fl] = epoch + 1;  // somebody is left for the next round
                     }
+                    pend &= ~(1u << k);
                 }
-                __syncthreads();
-                epoch++;
             }
+            if (pend != 0) {
+                s_flag[fl] = epoch + 1;  // somebody is left for the next round
+            }
+            __syncthreads();
             epoch++;
         }
+        epoch++;
     }
     __syncthreads();
     for (int cb = 0; cb < nc; cb++) {
@@ -353,6 +427,7 @@ hipError_t launch_interp(const GridSampler3DGradArgs& a, hipStream_t stream)
     p.pad = a.pad;
     p.align = a.align;
     p.items_per_core = (int32_t)(a.items_per_core > 0 ? a.items_per_core : 1);
+    p.chunks = chunk_count(p.points, p.items_per_core);
     const int64_t vol = a.Din * a.Hin * a.Win;
     p.band_px = (int32_t)(vol < kBandMax ? vol : kBandMax);
     if (a.dx != nullptr) {
@@ -366,6 +441,15 @@ hipError_t launch_interp(const GridSampler3DGradArgs& a, hipStream_t stream)
             return hipErrorInvalidValue;
         }
         const dim3 grid((unsigned)bands, (unsigned)cgroups, (unsigned)a.N);
+        const int32_t* ranges = nullptr;
+        if (bands > 1 && a.chunk_ranges != nullptr) {
+            if (p.chunks > 0x7fffffff / 2) {
+                return hipErrorInvalidValue;
+            }
+            hipLaunchKernelGGL((gs3d_grad_range_kernel<T, INTERP>), dim3((unsigned)p.chunks, (unsigned)a.N),
+                               dim3(kThreads), 0, stream, (const T*)a.grid, (int32_t*)a.chunk_ranges, p);
+            ranges = (const int32_t*)a.chunk_ranges;
+        }
         // more than the default 64 KB of dynamic LDS
         static bool attr_set = false;
         if (!attr_set) {
@@ -385,11 +469,11 @@ hipError_t launch_interp(const GridSampler3DGradArgs& a, hipStream_t stream)
         if (grouped) {
             hipLaunchKernelGGL((gs3d_grad_input_kernel<T, INTERP, CBMAX>), grid, dim3(kThreads),
                                (size_t)p.band_px * (4 + CBMAX * sizeof(T)), stream, (const T*)a.gout,
-                               (const T*)a.grid, (T*)a.dx, p);
+                               (const T*)a.grid, (T*)a.dx, ranges, p);
         } else {
             hipLaunchKernelGGL((gs3d_grad_input_kernel<T, INTERP, 1>), grid, dim3(kThreads),
                                (size_t)p.band_px * (4 + sizeof(T)), stream, (const T*)a.gout, (const T*)a.grid,
-                               (T*)a.dx, p);
+                               (T*)a.dx, ranges, p);
         }
         const hipError_t e = hipGetLastError();
         if (e != hipSuccess) {
@@ -420,6 +504,15 @@ hipError_t launch_typed(const GridSampler3DGradArgs& a, hipStream_t stream)
 }
 
 }  // namespace
+
+int64_t gs3d_grad_range_words(const GridSampler3DGradArgs& a)
+{
+    if (a.Din * a.Hin * a.Win <= kBandMax) {
+        return 0;  // one band: every chunk concerns it
+    }
+    const int64_t per_core = a.items_per_core > 0 ? a.items_per_core : 1;
+    return a.N * 2 * (int64_t)chunk_count(a.Dout * a.Hout * a.Wout, per_core);
+}
 
 hipError_t launch_grid_sampler3d_grad(const GridSampler3DGradArgs& a, hipStream_t stream)
 {

@@ -35,6 +35,8 @@ const char* resize_grad_variant(const ResizeGradArgs& a);  // which kernel launc
 hipError_t launch_grid_sampler2d_grad(const GridSamplerGradArgs& a, hipStream_t stream);
 hipError_t launch_grid_sampler3d(const GridSampler3DArgs& a, hipStream_t stream);
 hipError_t launch_grid_sampler3d_grad(const GridSampler3DGradArgs& a, hipStream_t stream);
+// 32-bit words of GridSampler3DGradArgs::chunk_ranges that make the input gradient faster; 0 when it would not help
+int64_t gs3d_grad_range_words(const GridSampler3DGradArgs& a);
 
 // gather == true : strided view -> contiguous buffer;  false : contiguous buffer -> strided view
 hipError_t launch_strided_copy(const StridedView& v, void* contiguous, int elem_bytes, bool gather,

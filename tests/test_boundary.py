@@ -587,6 +587,11 @@ def test_grid_sampler3d_backward_status_codes(aclnn, desc):
     st, ws, v = _gsb3(aclnn, desc, gout=(1, 1, 2, 2, 5), inp=(1, 1, 3, 3, 5), fmt=nd)
     assert st == 0 and v == "gs3d_grad_ordered" and ws >= (20 + 45 + 45) * 4
     assert _gsb3(aclnn, desc, gout=(1, 1, 2, 2, 4), inp=(1, 1, 3, 3, 5), fmt=nd)[0] == INV
+    # volumes of more than one LDS band ask for scratch: two words per chunk of 256 grid points and batch item, only
+    # when the input gradient is wanted
+    big = dict(gout=(3, 1, 2, 30, 10), inp=(3, 1, 10, 30, 30), grid=(3, 2, 30, 10, 3))
+    assert _gsb3(aclnn, desc, **big)[:2] == (0, 3 * 3 * 2 * 4)
+    assert _gsb3(aclnn, desc, mask=(False, True), **big)[:2] == (0, 0)
 
 
 def test_resize_template_selection_point_copy(aclnn, desc):

@@ -507,25 +507,30 @@ def test_grid_sampler3d_backward_core_split_mask_layouts_and_torch(oracle, devic
     rng = np.random.default_rng(710)
     # more batch items than cores of the reference device: a core walks several items as one run of points, which
     # moves the chunk boundaries of the later ones (300 points: item 1 of a core starts at thread 44)
-    N, C, D, H, W, Do, Ho, Wo = 5, 2, 2, 3, 3, 3, 10, 10
-    x = rng.standard_normal((N, C, D, H, W)).astype(np.float16)
-    g = rng.uniform(-1.1, 1.1, (N, Do, Ho, Wo, 3)).astype(np.float16)
-    go = rng.standard_normal((N, C, Do, Ho, Wo)).astype(np.float16)
-    results = []
-    try:
-        for cores in (2, 64):
-            monkeypatch.setenv("OPSCV_REFERENCE_CORES", str(cores))
-            oracle.set_reference_cores(cores)
-            rdx, rdg = oracle.grid_sampler3d_backward(go, x, g, 0, 1, False)
-            dx, dg = aclnn.grid_sampler3d_backward(*(torch.from_numpy(a).to(device) for a in (go, x, g)), 0, 1, False)
-            torch.cuda.synchronize()
-            assert np.array_equal(dx.cpu().numpy().view(np.uint16), rdx.view(np.uint16)), cores
-            assert np.array_equal(dg.cpu().numpy().view(np.uint16), rdg.view(np.uint16)), cores
-            results.append(rdx)
-    finally:
-        oracle.set_reference_cores(64)
-        monkeypatch.delenv("OPSCV_REFERENCE_CORES")
-    assert not np.array_equal(results[0].view(np.uint16), results[1].view(np.uint16))  # the order is visible in fp16
+    # the second volume spans two LDS bands, which brings in the per-chunk voxel spans
+    for (N, C, D, H, W, Do, Ho, Wo) in [(5, 2, 2, 3, 3, 3, 10, 10), (5, 2, 3, 60, 50, 3, 10, 10)]:
+        x = rng.standard_normal((N, C, D, H, W)).astype(np.float16)
+        g = rng.uniform(-1.1, 1.1, (N, Do, Ho, Wo, 3)).astype(np.float16)
+        if D > 2:
+            g[..., :2] *= 0.05  # pile the points up on few voxels
+        go = rng.standard_normal((N, C, Do, Ho, Wo)).astype(np.float16)
+        results = []
+        try:
+            for cores in (2, 64):
+                monkeypatch.setenv("OPSCV_REFERENCE_CORES", str(cores))
+                oracle.set_reference_cores(cores)
+                rdx, rdg = oracle.grid_sampler3d_backward(go, x, g, 0, 1, False)
+                dx, dg = aclnn.grid_sampler3d_backward(*(torch.from_numpy(a).to(device) for a in (go, x, g)), 0, 1,
+                                                       False)
+                torch.cuda.synchronize()
+                assert np.array_equal(dx.cpu().numpy().view(np.uint16), rdx.view(np.uint16)), (cores, D)
+                assert np.array_equal(dg.cpu().numpy().view(np.uint16), rdg.view(np.uint16)), (cores, D)
+                results.append(rdx)
+        finally:
+            oracle.set_reference_cores(64)
+            monkeypatch.delenv("OPSCV_REFERENCE_CORES")
+        # the order is visible in fp16
+        assert not np.array_equal(results[0].view(np.uint16), results[1].view(np.uint16))
     # masks, strided views, channels-last, torch autograd (fp32)
     N, C, D, H, W, Do, Ho, Wo = 2, 3, 4, 6, 5, 3, 7, 6
     x = rng.standard_normal((N, C, D, H, W)).astype(np.float32)
