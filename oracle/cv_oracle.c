@@ -43,6 +43,12 @@
  *                                  default mode adds with atomics in arbitrary order: bit-level parity with the
  *                                  reference is "parity unpinned"; the accumulation order restated is that of its
  *                                  deterministic mode
+ *   oracle_grid_sampler3d_backward : live torch autograd of grid_sample on 5-D inputs (both modes, all paddings
+ *                                  and alignments; fp32 to 2e-5, both gradients), adjointness with the forward
+ *                                  oracle, left-to-right sums in the element type for points piled on one voxel,
+ *                                  with and without the chunk shift of several items per core.  Bit-level parity
+ *                                  with the reference is "parity unpinned" for the reasons given for the 2-D
+ *                                  backward; the accumulation order restated is that of its deterministic mode
  *   oracle_resize_scale          : float bit patterns held by the reference's tiling UT
  *                                  (image/resize_bilinear_v2/tests/ut/op_host/arch35/test_resize_bilinear_v2_tiling.cpp)
  */
