@@ -112,6 +112,8 @@ def load_bench_lib():
     L.opscv_bench_grid_sampler2d_backward.restype = ctypes.c_int
     L.opscv_bench_grid_sampler2d_backward.argtypes = [ctypes.POINTER(vp)] * 5 + [ctypes.c_int, i64, i64, ctypes.c_bool,
                                                                                  vp, vp, u64, ctypes.c_int, vp, pd, pd]
+    L.opscv_bench_grid_sampler3d_backward.restype = ctypes.c_int
+    L.opscv_bench_grid_sampler3d_backward.argtypes = L.opscv_bench_grid_sampler2d_backward.argtypes
     L.opscv_bench_grid_sampler3d.restype = ctypes.c_int
     L.opscv_bench_grid_sampler3d.argtypes = L.opscv_bench_grid_sampler2d.argtypes
     L.opscv_bench_upsample_bilinear2d_backward.restype = ctypes.c_int
@@ -401,6 +403,73 @@ def bench_gs3d(steps, warmup, sets=4, channels_last=False):
     return dict(workload="V1 grid_sampler3d fp16 x(22,4,16,64,64) grid(22,16,64,64,3) bilinear zeros "
                          "align_corners=False" + (" NDHWC tensors" if channels_last else ""), samples=samples, alg_bytes=alg, timed=t, variant=variant,
                 parity=parity, sets=sets, default_modes=True)
+
+
+def bench_gs3d_backward(steps, warmup, sets=2, mask=(True, True)):
+    """Backward of the volumetric workload (fp16 22 x 4 x 16 x 64 x 64, the same registration-style warp): both
+    gradients."""
+    import numpy as np
+    import torch
+    import inputs as I
+    import oracle_lib
+    from ops_cv_amd import aclnn
+    dev = torch.device("cuda:0")
+    L = load_bench_lib()
+    N, C, D, H, W = 22, 4, 16, 64, 64
+    dtype = "fp16"
+    ts, hs = [[] for _ in range(5)], [[] for _ in range(5)]
+    first = None
+    for s in range(sets):
+        rng = np.random.default_rng(3100 + s)
+        x = I.cast_np(rng.standard_normal((N, C, D, H, W)).astype(np.float32), dtype)
+        ax = [np.linspace(-1, 1, n, dtype=np.float32) for n in (D, H, W)]
+        gz, gy, gx = np.meshgrid(*ax, indexing="ij")
+        base = np.stack([gx, gy, gz], -1)[None]
+        g = base * rng.uniform(0.9, 1.1, (N, 1, 1, 1, 3)) + rng.uniform(-0.1, 0.1, (N, 1, 1, 1, 3))
+        g = I.cast_np((g + rng.normal(0, 0.01, g.shape)).astype(np.float32), dtype)
+        go = I.cast_np(rng.standard_normal((N, C, D, H, W)).astype(np.float32), dtype)
+        if s == 0:
+            first = (go, x, g)
+        tens = [I.to_torch(go, dtype, dev), I.to_torch(x, dtype, dev), I.to_torch(g, dtype, dev)]
+        tens += [torch.empty_like(tens[1]), torch.empty_like(tens[2])]
+        for lst, hl, t in zip(ts, hs, tens):
+            lst.append(t)
+            hl.append(aclnn.tensor_handle(t, aclnn.ACL_FORMAT_NCDHW))
+    arr = lambda h: (ctypes.c_void_p * len(h))(*h)
+    arrs = [arr(h) for h in hs]
+    m = aclnn.create_bool_array(list(mask))
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ev, wall = ctypes.c_double(0), ctypes.c_double(0)
+    st, ws_bytes, ex = aclnn.get_workspace_size_grid_sampler3d_backward(hs[0][0], hs[1][0], hs[2][0], 0, 0, False, m,
+                                                                        hs[3][0], hs[4][0])
+    assert st == 0
+    variant = aclnn.executor_variant(ex)
+    aclnn.destroy_executor(ex)
+    work = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)  # the spans of the chunks of grid points
+    wptr = ctypes.c_void_p(work.data_ptr())
+
+    def run(k):
+        rc = L.opscv_bench_grid_sampler3d_backward(*arrs, sets, 0, 0, False, m, wptr, ws_bytes, k, stream,
+                                                   ctypes.byref(ev), ctypes.byref(wall))
+        if rc != 0:
+            raise RuntimeError("bench loop failed rc=%d: %s" % (rc, aclnn.load_library().aclGetRecentErrMsg()))
+        return Timed(ev.value, wall.value, k)
+
+    t = _finish(L, run, ts[0], ts[3], steps, warmup, stream)
+    rdx, rdg = oracle_lib.grid_sampler3d_backward(*first, 0, 0, False, dtype=I.oracle_code(dtype))
+    parity = _parity(I.from_torch(ts[3][0], dtype), rdx, dtype)
+    parity["grid_grad_bit_exact"] = bool(np.array_equal(I.from_torch(ts[4][0], dtype).view(np.uint8),
+                                                        rdg.view(np.uint8)))
+    for hl in hs:
+        for h in hl:
+            aclnn.destroy_tensor(h)
+    aclnn.destroy_bool_array(m)
+    e = esize(dtype)
+    # gradOutput read by both gradients' kernels, input read once, grid read twice, both gradients written
+    alg = (2 * N * C * D * H * W + 2 * N * C * D * H * W + 3 * N * D * H * W * 3) * e
+    return dict(workload="W1 grid_sampler3d_backward fp16 x(22,4,16,64,64) grid(22,16,64,64,3) bilinear zeros "
+                         "align_corners=False both gradients", samples=N * C * D * H * W, alg_bytes=alg, timed=t,
+                variant=variant, parity=parity, sets=sets, default_modes=True)
 
 
 def bench_gs_backward(steps, warmup, sets=4, mask=(True, True)):
@@ -705,6 +774,7 @@ def main():
                                                                   channels_last=True))
         k4 = max(5, args.steps // 4)
         others["G3_grid_sampler2d_backward"] = summary_of(bench_gs_backward(k4, max(2, args.warmup // 4)))
+        others["W1_grid_sampler3d_backward"] = summary_of(bench_gs3d_backward(k4, max(2, args.warmup // 4)))
         others["B4_upsample_backward"] = summary_of(bench_resize_like("backward", k4, max(2, args.warmup // 4)))
         others["R4_resize_nearest"] = summary_of(bench_resize_like("nearest", k4, max(2, args.warmup // 4)))
         line["other_workloads"] = others

@@ -10,6 +10,7 @@
 
 #include "aclnn_grid_sampler2d.h"
 #include "aclnn_grid_sampler2d_backward.h"
+#include "aclnn_grid_sampler3d_backward.h"
 #include "aclnn_grid_sampler3d.h"
 #include "aclnn_resize.h"
 #include "aclnn_upsample_bilinear_2d.h"
@@ -83,6 +84,22 @@ OPSCV_BENCH_API int opscv_bench_grid_sampler2d_backward(const aclTensor* const* 
         aclnnStatus st = aclnnGridSampler2DBackwardGetWorkspaceSize(gouts[i], inputs[i], grids[i], interp, pad, align,
                                                                     mask, dxs[i], dgrids[i], &ws, &ex);
         return st != ACLNN_SUCCESS ? st : aclnnGridSampler2DBackward(workspace, workspace_size, ex, stream);
+    });
+}
+
+OPSCV_BENCH_API int opscv_bench_grid_sampler3d_backward(const aclTensor* const* gouts, const aclTensor* const* inputs,
+                                                        const aclTensor* const* grids, aclTensor* const* dxs,
+                                                        aclTensor* const* dgrids, int sets, int64_t interp,
+                                                        int64_t pad, bool align, const aclBoolArray* mask,
+                                                        void* workspace, uint64_t workspace_size, int steps,
+                                                        void* stream, double* event_ms, double* wall_ms)
+{
+    return timed_loop(sets, steps, stream, event_ms, wall_ms, [&](int i) {
+        uint64_t ws = 0;
+        aclOpExecutor* ex = nullptr;
+        aclnnStatus st = aclnnGridSampler3DBackwardGetWorkspaceSize(gouts[i], inputs[i], grids[i], interp, pad, align,
+                                                                    mask, dxs[i], dgrids[i], &ws, &ex);
+        return st != ACLNN_SUCCESS ? st : aclnnGridSampler3DBackward(workspace, workspace_size, ex, stream);
     });
 }
 

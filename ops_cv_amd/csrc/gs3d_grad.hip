@@ -30,7 +30,7 @@ constexpr int kThreads = 256;  // also the chunk length of the accumulation orde
 constexpr uint32_t kLaneBits = 8;              // 256 points of a chunk
 constexpr uint32_t kKeyBits = kLaneBits + 3;   // ... times eight corners
 constexpr uint32_t kEpochMax = (1u << (32 - kKeyBits)) - 1;
-constexpr int kBandMax = 8192;  // voxels of the gradient a workgroup keeps in LDS
+constexpr int kBandMax = 8192;  // most voxels of the gradient a workgroup keeps in LDS
 
 struct Grad3Params {
     int32_t C, D, H, W, points;
@@ -415,6 +415,21 @@ __global__ __launch_bounds__(kThreads) void gs3d_grad_grid_kernel(const T* __res
     ElemIO<T>::store(dgrid + 3 * idx + 2, as_fp32_value(tp.mz * giz));
 }
 
+// Voxels per band.  Every workgroup is a chain of dependent LDS round trips, so the chip is filled by workgroups
+// next to each other: bands are halved (down to a quarter) until there are about two workgroups per compute unit.
+// Measured on fp16 22x4x16x64x64 with an affine grid: 582 us with 8192 voxels, 383 with 4096, 280 with 2048.
+int64_t band_voxels(const GridSampler3DGradArgs& a)
+{
+    const int64_t vol = a.Din * a.Hin * a.Win;
+    const int cbmax = 8 / elem_size(a.elem);
+    const int64_t cgroups = (a.C >= cbmax) ? (a.C + cbmax - 1) / cbmax : a.C;
+    int64_t band = kBandMax;
+    while (band > kBandMax / 4 && ((vol + band - 1) / band) * cgroups * a.N < 512) {
+        band /= 2;
+    }
+    return vol < band ? vol : band;
+}
+
 template <typename T, int INTERP>
 hipError_t launch_interp(const GridSampler3DGradArgs& a, hipStream_t stream)
 {
@@ -429,7 +444,7 @@ hipError_t launch_interp(const GridSampler3DGradArgs& a, hipStream_t stream)
     p.items_per_core = (int32_t)(a.items_per_core > 0 ? a.items_per_core : 1);
     p.chunks = chunk_count(p.points, p.items_per_core);
     const int64_t vol = a.Din * a.Hin * a.Win;
-    p.band_px = (int32_t)(vol < kBandMax ? vol : kBandMax);
+    p.band_px = (int32_t)band_voxels(a);
     if (a.dx != nullptr) {
         const int64_t bands = (vol + p.band_px - 1) / p.band_px;
         // 8 bytes of gradient per band voxel: 4 channels of a 16-bit type, 2 of fp32 (96 KB of LDS with the election
@@ -507,7 +522,7 @@ hipError_t launch_typed(const GridSampler3DGradArgs& a, hipStream_t stream)
 
 int64_t gs3d_grad_range_words(const GridSampler3DGradArgs& a)
 {
-    if (a.Din * a.Hin * a.Win <= kBandMax) {
+    if (a.Din * a.Hin * a.Win <= band_voxels(a)) {
         return 0;  // one band: every chunk concerns it
     }
     const int64_t per_core = a.items_per_core > 0 ? a.items_per_core : 1;
