@@ -33,6 +33,7 @@ MEASURED_TRAFFIC = {
     ("C5", "lds_ring_p32784_1x4"): 176.4e6,  # profiles/gs2d_lds_ring_C5_bf16_random_gather.md
     ("V1", "gs3d_bilinear"): 38.67e6,        # profiles/gs3d_V1_fp16_22x4x16x64x64.md
     ("G3", "gs2d_grad_ordered"): 255.3e6,    # profiles/gs2d_grad_G3_fp16_n16_c256.md (both kernels of a step)
+    ("W1", "gs3d_grad_ordered"): 140.0e6,    # profiles/gs3d_grad_W1_fp16_22x4x16x64x64.md (three kernels of a step)
     ("B4", "resize_grad_lds"): 1340.0e6,     # profiles/resize_grad_lds_B4_fp16_4k.md
     ("R4", "nearest_nchw_lds"): 1327.3e6,    # profiles/resize_nearest_lds_R4_fp16_4k.md
 }
@@ -666,7 +667,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="C3", help="headline workload: C1..C5, L1 (sampler on 1080p planes), or one of the neighbouring entry points V1 (3-D sampler), G3 "
-                         "(sampler backward), B4 (resize backward), R4 (nearest resize)")
+                         "(sampler backward), W1 (3-D sampler backward), B4 (resize backward), R4 (nearest resize)")
     ap.add_argument("--only", action="store_true", help="skip the other workloads and the CPU baseline")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -706,6 +707,8 @@ def main():
         r = bench_gs3d(args.steps, args.warmup, channels_last=True)
     elif head == "G3":
         r = bench_gs_backward(args.steps, args.warmup)
+    elif head == "W1":
+        r = bench_gs3d_backward(args.steps, args.warmup)
     elif head == "B4":
         r = bench_resize_like("backward", args.steps, args.warmup)
     elif head == "R4":
