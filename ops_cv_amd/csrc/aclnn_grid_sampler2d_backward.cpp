@@ -163,7 +163,8 @@ aclnnStatus aclnnGridSampler2DBackwardGetWorkspaceSize(const aclTensor* gradOutp
             return ACLNN_ERR_PARAM_INVALID;
         }
     }
-    if (input->dims[2] * input->dims[3] > INT32_MAX || grid->dims[1] * grid->dims[2] > INT32_MAX ||
+    // the walk over chunks of 256 grid points runs up to a chunk past the last point
+    if (input->dims[2] * input->dims[3] > INT32_MAX || grid->dims[1] * grid->dims[2] > INT32_MAX - 1024 ||
         input->dims[0] > 65535 || input->dims[1] > 65535) {
         set_error("%s: Hin*Win and Hout*Wout must fit in int32, N and C in 16 bits", kApi);
         return ACLNN_ERR_PARAM_INVALID;

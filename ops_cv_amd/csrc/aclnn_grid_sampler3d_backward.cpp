@@ -168,7 +168,8 @@ aclnnStatus aclnnGridSampler3DBackwardGetWorkspaceSize(const aclTensor* gradOutp
     }
     if (input->dims[di] * input->dims[hi] > INT32_MAX ||
         input->dims[di] * input->dims[hi] * input->dims[wi] > INT32_MAX ||
-        grid->dims[1] * grid->dims[2] > INT32_MAX || grid->dims[1] * grid->dims[2] * grid->dims[3] > INT32_MAX ||
+        grid->dims[1] * grid->dims[2] > INT32_MAX ||
+        grid->dims[1] * grid->dims[2] * grid->dims[3] > INT32_MAX - 1024 ||  // chunk arithmetic runs a chunk past it
         input->dims[0] > 65535 || input->dims[ci] > 65535) {
         set_error("%s: Din*Hin*Win and Dout*Hout*Wout must fit in int32, N and C in 16 bits", kApi);
         return ACLNN_ERR_PARAM_INVALID;

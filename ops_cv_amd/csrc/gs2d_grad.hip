@@ -428,7 +428,7 @@ hipError_t launch_grid_sampler2d_grad(const GridSamplerGradArgs& a, hipStream_t 
     if (a.pad < 0 || a.pad > 2 || a.N <= 0 || a.C <= 0 || a.Hin <= 0 || a.Win <= 0 || a.Hout <= 0 || a.Wout <= 0) {
         return hipErrorInvalidValue;
     }
-    if (a.Hin * a.Win > INT32_MAX || a.Hout * a.Wout > INT32_MAX) {
+    if (a.Hin * a.Win > INT32_MAX || a.Hout * a.Wout > INT32_MAX - 1024) {
         return hipErrorInvalidValue;
     }
     switch (a.elem) {

@@ -19,6 +19,8 @@
 // 98-330); no atomics are involved.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "gs2d_grad_math.hpp"
 #include "kernels.hpp"
 
@@ -50,6 +52,7 @@ struct GradTaps3 {
     int32_t off[NT];
     float w[NT];
     float wx[2], wy[2], wz[2];  // per axis: weight of the low and of the high corner
+    int32_t x0, y0, z0;         // bilinear: the low corner
     float mx, my, mz;           // chain-rule multipliers of the grid gradient
 };
 
@@ -81,6 +84,9 @@ __device__ __forceinline__ void decide_grad_taps3(GradTaps3<T, INTERP>& t, float
     const int32_t y0 = float_to_i32(__builtin_floorf(fy));
     const int32_t z0 = float_to_i32(__builtin_floorf(fz));
     const int32_t x1 = next_index(x0), y1 = next_index(y0), z1 = next_index(z0);
+    t.x0 = x0;
+    t.y0 = y0;
+    t.z0 = z0;
     t.wx[0] = (float)x1 - fx;
     t.wx[1] = fx - (float)x0;
     t.wy[0] = (float)y1 - fy;
@@ -384,6 +390,48 @@ __global__ __launch_bounds__(kThreads) void gs3d_grad_grid_kernel(const T* __res
     // The sums run over the channels in order; the loads do not depend on them and are issued a group ahead.
     constexpr int U = 4;
     int32_t c = 0;
+    if (p.W >= 2) {
+        // The low and high corner along x are neighbours in memory: one load of two elements (aligned to one element
+        // only) per row of corners instead of two halves the addresses the gather puts through the memory pipeline.
+        // The pair sits at column pb = clamp(x0, 0, W - 2), so it never leaves the row; which half is which corner
+        // follows from pb.  Corners outside the volume are skipped by accumulate() as before.
+        using PairBits = typename std::conditional<sizeof(T) == 2, uint32_t, uint64_t>::type;
+        const int32_t pb = (tp.x0 < 0) ? 0 : ((tp.x0 > p.W - 2) ? p.W - 2 : tp.x0);
+        const bool lo_w = (tp.x0 == pb), lo_e = (next_index(tp.x0) == pb);
+        int32_t rowoff[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int32_t cy = (r & 1) ? next_index(tp.y0) : tp.y0, cz = (r >> 1) ? next_index(tp.z0) : tp.z0;
+            const bool in = (uint32_t)cy < (uint32_t)p.H && (uint32_t)cz < (uint32_t)p.D;
+            rowoff[r] = in ? (cz * p.H + cy) * p.W + pb : 0;
+        }
+        for (; c + U <= p.C; c += U) {
+            float go[U];
+            PairBits pr[U][4];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const T* xc = x_n + (int64_t)(c + u) * vol;
+                go[u] = ElemIO<T>::load(go_n + (int64_t)(c + u) * points);
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    __builtin_memcpy(&pr[u][r], xc + rowoff[r], sizeof(PairBits));
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                float v[8];
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    T two[2];
+                    __builtin_memcpy(two, &pr[u][r], sizeof(PairBits));
+                    const float lo = ElemIO<T>::load(&two[0]), hi = ElemIO<T>::load(&two[1]);
+                    v[2 * r] = lo_w ? lo : hi;
+                    v[2 * r + 1] = lo_e ? lo : hi;
+                }
+                accumulate(go[u], v);
+            }
+        }
+    }
     for (; c + U <= p.C; c += U) {
         float go[U], v[U][8];
 #pragma unroll
@@ -538,7 +586,7 @@ hipError_t launch_grid_sampler3d_grad(const GridSampler3DGradArgs& a, hipStream_
         a.Hout <= 0 || a.Wout <= 0) {
         return hipErrorInvalidValue;
     }
-    if (a.Din * a.Hin * a.Win > INT32_MAX || a.Dout * a.Hout * a.Wout > INT32_MAX || a.C > INT32_MAX) {
+    if (a.Din * a.Hin * a.Win > INT32_MAX || a.Dout * a.Hout * a.Wout > INT32_MAX - 1024 || a.C > INT32_MAX) {
         return hipErrorInvalidValue;
     }
     switch (a.elem) {
