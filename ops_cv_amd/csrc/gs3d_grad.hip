@@ -32,6 +32,7 @@ constexpr int kThreads = 256;  // also the chunk length of the accumulation orde
 constexpr uint32_t kLaneBits = 8;              // 256 points of a chunk
 constexpr uint32_t kKeyBits = kLaneBits + 3;   // ... times eight corners
 constexpr uint32_t kEpochMax = (1u << (32 - kKeyBits)) - 1;
+constexpr int kTagsMax = 4096;  // election tags of a band (bands of 8192 voxels share them in pairs: two workgroups per CU)
 constexpr int kBandMax = 8192;  // most voxels of the gradient a workgroup keeps in LDS
 
 struct Grad3Params {
@@ -40,7 +41,15 @@ struct Grad3Params {
     int32_t band_px;
     int32_t items_per_core;
     int32_t chunks;  // chunks a batch item is walked in, a possibly empty leading one included
+    int32_t tags;    // election tags, a power of two (tag_of)
 };
+
+// Tag of a band element.  Elements that share a tag are elected as if they were one; folding the high bits in keeps
+// neighbours along every axis (offsets 1, W, H * W, often powers of two) on different tags.
+__device__ __forceinline__ int32_t tag_of(int32_t off, int32_t tag_mask)
+{
+    return (off ^ (off >> 10)) & tag_mask;
+}
 
 // Where the contributions of a grid point land in the (D, H, W) volume and with what weight.
 //   INTERP 0: eight corners, index = x-high + 2 * y-high + 4 * z-high; weight = rt<T>(wx * wy * wz)
@@ -186,7 +195,8 @@ __global__ __launch_bounds__(kThreads) void gs3d_grad_input_kernel(const T* __re
     extern __shared__ uint32_t smem_u32[];
     __shared__ uint32_t s_flag[2];
     uint32_t* owner = smem_u32;
-    T* planes = reinterpret_cast<T*>(smem_u32 + p.band_px);  // [CB][band_px], values already in the element type
+    T* planes = reinterpret_cast<T*>(smem_u32 + p.tags);  // [CB][band_px], values already in the element type
+    const int32_t tag_mask = p.tags - 1;
 
     const int t = threadIdx.x;
     const int32_t vol = p.D * p.H * p.W;
@@ -195,8 +205,10 @@ __global__ __launch_bounds__(kThreads) void gs3d_grad_input_kernel(const T* __re
     const int32_t c0 = blockIdx.y * CB;
     const int32_t nc = (c0 + CB <= p.C) ? CB : p.C - c0;
     const int64_t n = blockIdx.z;
-    for (int32_t i = t; i < b1 - b0; i += kThreads) {
+    for (int32_t i = t; i < p.tags; i += kThreads) {
         owner[i] = 0u;
+    }
+    for (int32_t i = t; i < b1 - b0; i += kThreads) {
 #pragma unroll
         for (int cb = 0; cb < CB; cb++) {
             ElemIO<T>::store(planes + cb * p.band_px + i, 0.0f);
@@ -275,7 +287,7 @@ __global__ __launch_bounds__(kThreads) void gs3d_grad_input_kernel(const T* __re
         }
         if (epoch > kEpochMax - 2u * NT * kThreads) {  // uniform: start the election tags over
             __syncthreads();
-            for (int32_t i = t; i < b1 - b0; i += kThreads) {
+            for (int32_t i = t; i < p.tags; i += kThreads) {
                 owner[i] = 0u;
             }
             if (t == 0) {
@@ -301,13 +313,13 @@ __global__ __launch_bounds__(kThreads) void gs3d_grad_input_kernel(const T* __re
 #pragma unroll
             for (int k = 0; k < NT; k++) {
                 if (pend & (1u << k)) {
-                    atomicMax(&owner[off[k]], key | ((uint32_t)(NT - 1 - k) << kLaneBits));
+                    atomicMax(&owner[tag_of(off[k], tag_mask)], key | ((uint32_t)(NT - 1 - k) << kLaneBits));
                 }
             }
             __syncthreads();
 #pragma unroll
             for (int k = 0; k < NT; k++) {
-                if ((pend & (1u << k)) && owner[off[k]] == (key | ((uint32_t)(NT - 1 - k) << kLaneBits))) {
+                if ((pend & (1u << k)) && owner[tag_of(off[k], tag_mask)] == (key | ((uint32_t)(NT - 1 - k) << kLaneBits))) {
                     T* e = planes + off[k];
 #pragma unroll
                     for (int cb = 0; cb < CB; cb++) {
@@ -493,6 +505,11 @@ hipError_t launch_interp(const GridSampler3DGradArgs& a, hipStream_t stream)
     p.chunks = chunk_count(p.points, p.items_per_core);
     const int64_t vol = a.Din * a.Hin * a.Win;
     p.band_px = (int32_t)band_voxels(a);
+    // voxels that share a tag are elected as if they were one: never out of order, at worst a round more
+    p.tags = 64;
+    while (p.tags < p.band_px && p.tags < kTagsMax) {
+        p.tags *= 2;
+    }
     if (a.dx != nullptr) {
         const int64_t bands = (vol + p.band_px - 1) / p.band_px;
         // 8 bytes of gradient per band voxel: 4 channels of a 16-bit type, 2 of fp32 (96 KB of LDS with the election
@@ -518,11 +535,11 @@ hipError_t launch_interp(const GridSampler3DGradArgs& a, hipStream_t stream)
         if (!attr_set) {
             hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(gs3d_grad_input_kernel<T, INTERP, CBMAX>),
                                                 hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                kBandMax * (4 + CBMAX * (int)sizeof(T)));
+                                                kTagsMax * 4 + kBandMax * CBMAX * (int)sizeof(T));
             if (ea == hipSuccess) {
                 ea = hipFuncSetAttribute(reinterpret_cast<const void*>(gs3d_grad_input_kernel<T, INTERP, 1>),
                                          hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         kBandMax * (4 + (int)sizeof(T)));
+                                         kTagsMax * 4 + kBandMax * (int)sizeof(T));
             }
             if (ea != hipSuccess) {
                 return ea;
@@ -531,11 +548,11 @@ hipError_t launch_interp(const GridSampler3DGradArgs& a, hipStream_t stream)
         }
         if (grouped) {
             hipLaunchKernelGGL((gs3d_grad_input_kernel<T, INTERP, CBMAX>), grid, dim3(kThreads),
-                               (size_t)p.band_px * (4 + CBMAX * sizeof(T)), stream, (const T*)a.gout,
+                               (size_t)p.tags * 4 + (size_t)p.band_px * CBMAX * sizeof(T), stream, (const T*)a.gout,
                                (const T*)a.grid, (T*)a.dx, ranges, p);
         } else {
             hipLaunchKernelGGL((gs3d_grad_input_kernel<T, INTERP, 1>), grid, dim3(kThreads),
-                               (size_t)p.band_px * (4 + sizeof(T)), stream, (const T*)a.gout, (const T*)a.grid,
+                               (size_t)p.tags * 4 + (size_t)p.band_px * sizeof(T), stream, (const T*)a.gout, (const T*)a.grid,
                                (T*)a.dx, ranges, p);
         }
         const hipError_t e = hipGetLastError();
