@@ -32,6 +32,8 @@ void staged_extent(const ResizeArgs& a, int gran, int kThreads, int32_t* max_row
     constexpr int V = 16 / (int)sizeof(T);
     const int32_t ge = (gran == 1) ? 1 : gran / (int)sizeof(T);
     const int32_t Wd = (int32_t)a.Wd, Hd = (int32_t)a.Hd, Ws = (int32_t)a.Ws, Hs = (int32_t)a.Hs;
+    const int32_t ci = a.channels_last ? (int32_t)a.C : 1;  // row elements per pixel
+    const int32_t Wde = Wd * ci;
     int32_t mr = 0, ms = 0;
     for (int32_t hb = 0; hb < Hd; hb += kBand) {
         const int32_t he = (hb + kBand < Hd) ? hb + kBand : Hd;
@@ -39,10 +41,10 @@ void staged_extent(const ResizeArgs& a, int gran, int kThreads, int32_t* max_row
         const int32_t hi = axis_tap<HALF_PIXEL>(he - 1, a.scale_h, Hs).i1;
         mr = (hi - lo + 1 > mr) ? hi - lo + 1 : mr;
     }
-    for (int32_t cb = 0; cb < Wd; cb += kThreads * V) {
-        const int32_t cl = ((cb + kThreads * V < Wd) ? cb + kThreads * V : Wd) - 1;
-        const int32_t lo = axis_tap<HALF_PIXEL>(cb, a.scale_w, Ws).i0;
-        const int32_t hi = axis_tap<HALF_PIXEL>(cl, a.scale_w, Ws).i1;
+    for (int32_t cb = 0; cb < Wde; cb += kThreads * V) {
+        const int32_t cl = ((cb + kThreads * V < Wde) ? cb + kThreads * V : Wde) - 1;
+        const int32_t lo = axis_tap<HALF_PIXEL>(cb / ci, a.scale_w, Ws).i0 * ci;
+        const int32_t hi = axis_tap<HALF_PIXEL>(cl / ci, a.scale_w, Ws).i1 * ci + ci - 1;
         const int32_t c0 = lo / ge * ge;
         const int32_t se = (hi + 1 - c0 + ge - 1) / ge * ge;
         ms = (se > ms) ? se : ms;
@@ -56,17 +58,27 @@ BandPlan make_plan(const ResizeArgs& a)
 {
     BandPlan bp;
     constexpr int V = 16 / (int)sizeof(T);
-    if (a.channels_last || a.mode != ResizeMode::Bilinear) {
+    if (a.mode != ResizeMode::Bilinear) {
         return bp;
     }
+    // Channels-last images whose pixels are not whole 16-byte vectors are resized as planes with rows of Ws * C
+    // elements (taps C elements apart); whole vectors per pixel have their own kernel.
+    const int64_t ci = a.channels_last ? a.C : 1;
+    // Staging pays when source rows are reused: images that at least double in area (3-channel fp16 1080p to 4K: 211 ->
+    // 101 us; 224 -> 256 is faster without staging).
+    if (a.channels_last && ((a.C * sizeof(T)) % 16 == 0 || a.Ws * ci > INT32_MAX || a.Wd * ci > INT32_MAX ||
+                            a.Hd * a.Wd < 2 * a.Hs * a.Ws)) {
+        return bp;
+    }
+    const int64_t Wse = a.Ws * ci, Wde = a.Wd * ci;
     // element-aligned output (the vector stores are), 32-bit row byte offsets
-    if (reinterpret_cast<uintptr_t>(a.y) % sizeof(T) != 0 || a.Wd * (int64_t)sizeof(T) >= (1ll << 31)) {
+    if (reinterpret_cast<uintptr_t>(a.y) % sizeof(T) != 0 || Wde * (int64_t)sizeof(T) >= (1ll << 31)) {
         return bp;
     }
 
     const uintptr_t xa = reinterpret_cast<uintptr_t>(a.x);
     int gran;
-    if ((a.Ws * sizeof(T)) % 16 == 0 && xa % 16 == 0) {
+    if ((Wse * sizeof(T)) % 16 == 0 && xa % 16 == 0) {
         gran = 16;
     } else if (xa % sizeof(T) == 0) {
         gran = 1;  // rows off the 16-byte grid: 16-byte copies in the shifted layout (see the kernel)
@@ -74,7 +86,7 @@ BandPlan make_plan(const ResizeArgs& a)
         return bp;
     }
     // one workgroup spans the whole output row when it fits in 512 lanes (fewer, longer row segments)
-    const int kThreads = ((a.Wd + V - 1) / V > 256) ? 512 : 256;
+    const int kThreads = ((Wde + V - 1) / V > 256) ? 512 : 256;
     bp.threads = kThreads;
     int32_t rows = 0, seg = 0;
     if (a.half_pixel) {
@@ -88,8 +100,8 @@ BandPlan make_plan(const ResizeArgs& a)
         return bp;  // strong down-scaling: the band touches too many source rows/columns
     }
     const int64_t bands = (a.Hd + kBand - 1) / kBand;
-    const int64_t cblocks = (a.Wd + kThreads * V - 1) / (kThreads * V);
-    const int64_t planes = a.N * a.C;
+    const int64_t cblocks = (Wde + kThreads * V - 1) / (kThreads * V);
+    const int64_t planes = a.channels_last ? a.N : a.N * a.C;
     if (bands > 65535 || cblocks > INT32_MAX) {
         return bp;
     }
@@ -105,6 +117,7 @@ BandPlan make_plan(const ResizeArgs& a)
     bp.p.gran = gran;
     bp.p.neg_zero = -0.0f;
     bp.p.raw_lambda = a.raw_lambda;
+    bp.p.interleave = (int32_t)ci;
     bp.p.streaming = (a.N * a.C * a.Hd * a.Wd * (int64_t)sizeof(T) >= kStreamingBytes) ? 1 : 0;
     bp.lds_bytes = (uint32_t)bytes;
     bp.grid = dim3((unsigned)cblocks, (unsigned)bands, (unsigned)(planes < 65535 ? planes : 65535));
@@ -267,7 +280,7 @@ const char* resize_lds_variant(const ResizeArgs& a)
         case Elem::F16: flat = make_flat_plan<_Float16>(a).ok; band = make_plan<_Float16>(a).ok; break;
         case Elem::BF16: flat = make_flat_plan<__bf16>(a).ok; band = make_plan<__bf16>(a).ok; break;
     }
-    return flat ? "nchw_flat_lds" : (band ? "nchw_band_lds" : nullptr);
+    return flat ? "nchw_flat_lds" : (band ? (a.channels_last ? "nhwc_band_lds" : "nchw_band_lds") : nullptr);
 }
 
 hipError_t run_resize_band_lds(const ResizeArgs& a, hipStream_t stream, bool* handled)

@@ -1,4 +1,5 @@
-// Bilinear resize, NCHW, LDS-staged row-band variant for gfx950: device code.
+// Bilinear resize, NCHW (and channels-last images of few channels), LDS-staged row-band variant for gfx950: device
+// code.
 //
 // Arithmetic: image/resize_bilinear_v2/op_kernel/arch35/resize_bilinear_v2_simt_nchw.h:108-144 (see resize_math.hpp).
 //
@@ -38,6 +39,7 @@ struct BandLdsParams {
     int32_t gran;       // bytes per lane of the asynchronous copy: 16 or 4; 1: 16 in the shifted layout (kernel)
     int32_t streaming;  // 1: mark the output stores non-temporal (outputs much larger than the caches)
     int32_t raw_lambda;  // fraction from the unclamped source coordinate (see axis_tap)
+    int32_t interleave;  // 1: planes of Hs x Ws; C: channels-last images, a row is Ws pixels of C elements each
     float neg_zero;     // -0.0f, passed in so that fma(v, w, -0) is not folded back into a multiply
 };
 
@@ -54,8 +56,12 @@ __global__ __launch_bounds__(THREADS) void resize_band_lds_kernel(const T* __res
     const int lane = tid & 63;
 
     // ---- block geometry (uniform) ----
+    // Channels-last images are resized as planes whose rows are Ws * C elements: output element j of a row is channel
+    // j % C of pixel j / C, and its taps sit C elements apart.  Everything below counts row elements ("columns").
+    const int32_t ci = p.interleave;
+    const int32_t Wse = p.Ws * ci, Wde = p.Wd * ci;
     const int32_t c_begin = blockIdx.x * (THREADS * V);
-    const int32_t c_last = ((c_begin + THREADS * V < p.Wd) ? c_begin + THREADS * V : p.Wd) - 1;
+    const int32_t c_last = ((c_begin + THREADS * V < Wde) ? c_begin + THREADS * V : Wde) - 1;
     const int32_t h_begin = blockIdx.y * BAND;
     const int32_t h_end = (h_begin + BAND < p.Hd) ? h_begin + BAND : p.Hd;
     // gran 16 or 4: source rows on that grid, copied as they are.  gran 1: rows anywhere (an odd width of 16-bit
@@ -65,10 +71,10 @@ __global__ __launch_bounds__(THREADS) void resize_band_lds_kernel(const T* __res
     const bool shifted = p.gran == 1;
     const int32_t ge = shifted ? 1 : p.gran / (int)sizeof(T);  // elements per copy granule
     const uint32_t copy_unit = shifted ? 16u : (uint32_t)p.gran;
-    const int32_t xs_lo = axis_tap<HALF_PIXEL>(c_begin, p.scale_w, p.Ws).i0;
-    const int32_t xs_hi = axis_tap<HALF_PIXEL>(c_last, p.scale_w, p.Ws).i1;
+    const int32_t xs_lo = axis_tap<HALF_PIXEL>(c_begin / ci, p.scale_w, p.Ws).i0 * ci;
+    const int32_t xs_hi = axis_tap<HALF_PIXEL>(c_last / ci, p.scale_w, p.Ws).i1 * ci + ci - 1;
     const int32_t seg_col0 = xs_lo / ge * ge;
-    const int32_t seg_elems = (xs_hi + 1 - seg_col0 + ge - 1) / ge * ge;  // stays inside the row: Ws % ge == 0
+    const int32_t seg_elems = (xs_hi + 1 - seg_col0 + ge - 1) / ge * ge;  // stays inside the row: Wse % ge == 0
     const uint32_t seg_bytes = (uint32_t)seg_elems * (uint32_t)sizeof(T);
     const int32_t ys_lo = axis_tap<HALF_PIXEL>(h_begin, p.scale_h, p.Hs).i0;
     const int32_t ys_hi = axis_tap<HALF_PIXEL>(h_end - 1, p.scale_h, p.Hs).i1;
@@ -82,10 +88,12 @@ __global__ __launch_bounds__(THREADS) void resize_band_lds_kernel(const T* __res
 #pragma unroll
     for (int i = 0; i < V; i++) {
         int32_t c = col0 + i;
-        c = (c < p.Wd) ? c : p.Wd - 1;
-        const AxisTap t = axis_tap<HALF_PIXEL>(c, p.scale_w, p.Ws, p.raw_lambda);
-        to0[i] = (uint32_t)(t.i0 - seg_col0) * (uint32_t)sizeof(T);
-        to1[i] = (uint32_t)(t.i1 - seg_col0) * (uint32_t)sizeof(T);
+        c = (c < Wde) ? c : Wde - 1;
+        const int32_t px = (ci == 1) ? c : c / ci;
+        const int32_t ch = c - px * ci;
+        const AxisTap t = axis_tap<HALF_PIXEL>(px, p.scale_w, p.Ws, p.raw_lambda);
+        to0[i] = (uint32_t)(t.i0 * ci + ch - seg_col0) * (uint32_t)sizeof(T);
+        to1[i] = (uint32_t)(t.i1 * ci + ch - seg_col0) * (uint32_t)sizeof(T);
         dx[i] = t.lambda;
         omdx[i] = 1.0f - t.lambda;
     }
@@ -100,20 +108,20 @@ __global__ __launch_bounds__(THREADS) void resize_band_lds_kernel(const T* __res
         my_y1 = t.i1 - ys_lo;
         my_dy = t.lambda;
     }
-    const uint32_t out_row_bytes = (uint32_t)p.Wd * (uint32_t)sizeof(T);
-    const uint32_t out_off = (col0 < p.Wd) ? (uint32_t)col0 * (uint32_t)sizeof(T) : 0x80000000u;
-    const int32_t nvalid = (p.Wd - col0 < V) ? p.Wd - col0 : V;  // output columns of this lane inside the row
+    const uint32_t out_row_bytes = (uint32_t)Wde * (uint32_t)sizeof(T);
+    const uint32_t out_off = (col0 < Wde) ? (uint32_t)col0 * (uint32_t)sizeof(T) : 0x80000000u;
+    const int32_t nvalid = (Wde - col0 < V) ? Wde - col0 : V;  // output columns of this lane inside the row
     const uint32_t wave = __builtin_amdgcn_readfirstlane((uint32_t)tid >> 6);
     const float neg_zero = p.neg_zero;
 
     for (int64_t pl = blockIdx.z; pl < p.planes; pl += gridDim.z) {
         // ---- stage the source rows of this band ----
-        const char* src0 = reinterpret_cast<const char*>(x + (pl * p.Hs + ys_lo) * (int64_t)p.Ws + seg_col0);
+        const char* src0 = reinterpret_cast<const char*>(x + (pl * p.Hs + ys_lo) * (int64_t)Wse + seg_col0);
         const uint32_t chunk = 64u * copy_unit;
         const uint32_t chunks_per_row = (seg_bytes + (shifted ? 15u : 0u) + chunk - 1) / chunk;
         const uint32_t total_chunks = chunks_per_row * (uint32_t)rows;
         const uint32_t src0_low = (uint32_t)(reinterpret_cast<uintptr_t>(src0) & 15u);
-        const uint32_t row_low = (uint32_t)(((uint32_t)p.Ws * (uint32_t)sizeof(T)) & 15u);
+        const uint32_t row_low = (uint32_t)(((uint32_t)Wse * (uint32_t)sizeof(T)) & 15u);
         // bytes by which the copy of staged row r starts before the row's segment
         auto row_shift = [&](uint32_t r) -> uint32_t { return shifted ? ((src0_low + r * row_low) & 15u) : 0u; };
         for (uint32_t q = wave; q < total_chunks; q += NWAVES) {
@@ -124,7 +132,7 @@ __global__ __launch_bounds__(THREADS) void resize_band_lds_kernel(const T* __res
             const uint32_t limit = shifted ? ((seg_bytes + shift + 15u) & ~15u) : seg_bytes;
             if (lane_off < limit) {
                 const rs_global_cptr_t g =
-                    (rs_global_cptr_t)(src0 + (size_t)r * p.Ws * sizeof(T) - shift + lane_off);
+                    (rs_global_cptr_t)(src0 + (size_t)r * Wse * sizeof(T) - shift + lane_off);
                 const rs_lds_ptr_t l = (rs_lds_ptr_t)(lds + r * p.lds_pitch + cb);
                 if (copy_unit == 16u) {
                     __builtin_amdgcn_global_load_lds(g, l, 16, 0, 0);
@@ -136,7 +144,7 @@ __global__ __launch_bounds__(THREADS) void resize_band_lds_kernel(const T* __res
         __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
 
-        T* yp = y + (pl * p.Hd + h_begin) * (int64_t)p.Wd;
+        T* yp = y + (pl * p.Hd + h_begin) * (int64_t)Wde;
         float ha[V], hb[V];  // blended source rows ya and yb (row indices relative to ys_lo)
         int32_t ya = -1, yb = -1;
         auto blend_row = [&](float* hrow, int32_t ys) {
@@ -216,7 +224,7 @@ __global__ __launch_bounds__(THREADS) void resize_band_lds_kernel(const T* __res
                     }
                 }
             }
-            yp += p.Wd;
+            yp += Wde;
         }
         __syncthreads();  // everybody is done with the staged rows before the next plane overwrites them
     }

@@ -980,6 +980,14 @@ hipError_t run_resize(const ResizeArgs& a, hipStream_t stream)
         return hipGetLastError();
     }
     if (a.channels_last) {
+        if (!nhwc_vec_ok<T>(a)) {
+            // pixels that are not whole vectors: rows of Ws * C elements through the LDS-staged band kernel
+            bool handled = false;
+            const hipError_t e = run_resize_band_lds(a, stream, &handled);
+            if (handled || e != hipSuccess) {
+                return e;
+            }
+        }
         const int vb = nhwc_unit_bytes<T>(a);
         if (vb != 0) {
             // Units per lane.  Several units of 2 or 4 bytes per lane make the stores 16 bytes wide, which pays when
@@ -1099,6 +1107,9 @@ const char* resize_variant(const ResizeArgs& a)
         }
         if (vec) {
             return "nhwc_vec";
+        }
+        if (const char* lds_variant = resize_lds_variant(a)) {
+            return lds_variant;
         }
         int vb = 0;
         switch (a.elem) {

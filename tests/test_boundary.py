@@ -237,6 +237,8 @@ def test_upsample_template_selection(aclnn, desc):
     assert _up(aclnn, desc, inp=(2, 128, 128, 256), out=(2, 192, 192, 256), size=(192, 192), dt=f32,
                fmt=aclnn.ACL_FORMAT_NHWC, align=True)[2] == "nhwc_vec"
     assert _up(aclnn, desc, inp=(2, 12, 12, 5), out=(2, 18, 18, 5), size=(18, 18), dt=f32,
+               fmt=aclnn.ACL_FORMAT_NHWC, align=True)[2] == "nhwc_band_lds"
+    assert _up(aclnn, desc, inp=(2, 12, 12, 5), out=(2, 14, 14, 5), size=(14, 14), dt=f32,
                fmt=aclnn.ACL_FORMAT_NHWC, align=True)[2] == "nhwc_unit"
 
 
@@ -267,10 +269,14 @@ def test_upsample_template_selection_channels_last(aclnn, desc):
     # half-pixel centres and broadcast with align_corners
     assert variant((1, 8, 8, 32), (1, 3, 3, 32), f32, False) == "nhwc_four_weights"
     assert variant((1, 8, 8, 32), (1, 3, 3, 32), f16, False) == "nhwc_vec"
-    assert variant((1, 1, 1, 14), (1, 13, 7, 14), f32, False) == "nhwc_unit"      # 56-byte pixels: 8-byte units
-    assert variant((1, 1, 1, 7), (1, 13, 7, 7), f32, False) == "nhwc_unit"        # one element per unit
-    assert variant((1, 4, 4, 3), (1, 13, 7, 3), f32, False) == "nhwc_unit"        # three-channel images: 12 bytes
-    assert variant((1, 4, 4, 3), (1, 13, 7, 3), f16, False) == "nhwc_unit"        # ... and 6 bytes
+    # pixels that are not whole 16-byte vectors: images that at least double in area are staged in LDS as rows of
+    # W * C elements, the others move units of 12, 8, 6, 4 or 2 bytes
+    assert variant((1, 1, 1, 14), (1, 13, 7, 14), f32, False) == "nhwc_band_lds"
+    assert variant((1, 4, 4, 3), (1, 13, 7, 3), f16, False) == "nhwc_band_lds"
+    assert variant((1, 9, 9, 14), (1, 10, 8, 14), f32, False) == "nhwc_unit"      # 56-byte pixels: 8-byte units
+    assert variant((1, 9, 9, 7), (1, 10, 8, 7), f32, False) == "nhwc_unit"        # one element per unit
+    assert variant((1, 9, 9, 3), (1, 10, 8, 3), f32, False) == "nhwc_unit"        # three-channel images: 12 bytes
+    assert variant((1, 9, 9, 3), (1, 10, 8, 3), f16, False) == "nhwc_unit"        # ... and 6 bytes
     assert variant((1, 1, 1, 14), (1, 13, 7, 14), f32, True) == "broadcast"
     assert variant((1, 8, 8, 8), (1, 1, 1, 8), f32, True) == "first_pixel"
     assert variant((1, 8, 8, 32), (1, 1, 1, 32), f32, True) == "point_copy"

@@ -81,19 +81,37 @@ def test_upsample_nhwc(oracle, device, aclnn, dtype, align):
 
 
 @pytest.mark.parametrize("dtype", I.DTYPES)
-def test_upsample_nhwc_per_element_kernel(oracle, device, aclnn, dtype, monkeypatch):
-    """the per-element channels-last kernel (kept for band counts beyond the grid limit) is reachable through
-    OPSCV_RESIZE_VARIANT=generic and matches the oracle like the band kernels"""
+@pytest.mark.parametrize("forced", ["generic", "register"])
+def test_upsample_nhwc_kernels_behind_the_lds_variant(oracle, device, aclnn, dtype, forced, monkeypatch):
+    """OPSCV_RESIZE_VARIANT=generic reaches the per-element channels-last kernel (kept for band counts beyond the grid
+    limit), =register the unit kernel on shapes that the LDS-staged variant would take; both match the oracle"""
     torch = _torch()
-    monkeypatch.setenv("OPSCV_RESIZE_VARIANT", "generic")
+    monkeypatch.setenv("OPSCV_RESIZE_VARIANT", forced)
     rng = np.random.default_rng(29)
+    seen = set()
     for (N, C, H, W), size, align in [((2, 5, 7, 9), (14, 18), False), ((1, 3, 9, 6), (4, 11), True),
-                                      ((1, 7, 12, 10), (5, 23), False)]:
+                                      ((1, 7, 12, 10), (5, 23), False), ((2, 3, 9, 11), (20, 17), False),
+                                      ((1, 6, 5, 7), (11, 13), True), ((1, 10, 6, 4), (9, 9), False),
+                                      ((1, 9, 6, 4), (5, 10), False), ((1, 2, 6, 4), (9, 7), True),
+                                      ((1, 20, 5, 5), (12, 12), False)]:
         x = I.cast_np(rng.standard_normal((N, H, W, C)).astype(np.float32), dtype)
         ref = oracle.upsample_bilinear2d_nhwc(x, size, align, dtype=I.oracle_code(dtype))
-        y = aclnn.upsample_bilinear2d(I.to_torch(x, dtype, device), size, align, channels_last=True)
+        xt = I.to_torch(x, dtype, device)
+        y = torch.empty((N,) + tuple(size) + (C,), dtype=xt.dtype, device=device)
+        hs = [aclnn.tensor_handle(xt, aclnn.ACL_FORMAT_NHWC), aclnn.tensor_handle(y, aclnn.ACL_FORMAT_NHWC)]
+        arr = aclnn.create_int_array(list(size))
+        st, _, ex = aclnn.get_workspace_size_upsample_bilinear2d(hs[0], arr, align, 0.0, 0.0, hs[1])
+        assert st == 0
+        seen.add(aclnn.executor_variant(ex))
+        aclnn.destroy_executor(ex)
+        aclnn.destroy_int_array(arr)
+        for h in hs:
+            aclnn.destroy_tensor(h)
+        aclnn.upsample_bilinear2d(xt, size, align, out=y, channels_last=True)
         torch.cuda.synchronize()
         assert np.array_equal(_bits(I.from_torch(y, dtype), dtype), _bits(ref, dtype)), (dtype, N, C, H, W, align)
+    # 20 channels of fp32 are whole 16-byte vectors, which have a kernel of their own
+    assert seen - {"nhwc_vec"} == ({"nhwc_generic"} if forced == "generic" else {"nhwc_unit"})
 
 
 @pytest.mark.parametrize("dtype", I.DTYPES)
