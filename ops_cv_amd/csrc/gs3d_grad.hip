@@ -321,11 +321,24 @@ __global__ __launch_bounds__(kThreads) void gs3d_grad_input_kernel(const T* __re
             for (int k = 0; k < NT; k++) {
                 if ((pend & (1u << k)) && owner[tag_of(off[k], tag_mask)] == (key | ((uint32_t)(NT - 1 - k) << kLaneBits))) {
                     T* e = planes + off[k];
+                    if (nc == CB) {
+                        // all planes read before any is written: the channels' updates overlap
+                        float cur[CB];
 #pragma unroll
-                    for (int cb = 0; cb < CB; cb++) {
-                        if (cb < nc) {
-                            const float val = contribution3<T, INTERP>(go[cb], wt[k]);
-                            ElemIO<T>::store(e + cb * p.band_px, ElemIO<T>::load(e + cb * p.band_px) + val);
+                        for (int cb = 0; cb < CB; cb++) {
+                            cur[cb] = ElemIO<T>::load(e + cb * p.band_px);
+                        }
+#pragma unroll
+                        for (int cb = 0; cb < CB; cb++) {
+                            ElemIO<T>::store(e + cb * p.band_px, cur[cb] + contribution3<T, INTERP>(go[cb], wt[k]));
+                        }
+                    } else {
+#pragma unroll
+                        for (int cb = 0; cb < CB; cb++) {
+                            if (cb < nc) {
+                                const float val = contribution3<T, INTERP>(go[cb], wt[k]);
+                                ElemIO<T>::store(e + cb * p.band_px, ElemIO<T>::load(e + cb * p.band_px) + val);
+                            }
                         }
                     }
                     pend &= ~(1u << k);
