@@ -609,28 +609,32 @@ __global__ __launch_bounds__(kThreads) void resize_nearest_lds_kernel(const T* _
                                                                        int64_t outer, int32_t Hs, int32_t Ws,
                                                                        int32_t Hd, int32_t Wd, float scale_h,
                                                                        float scale_w, uint32_t slot_bytes,
-                                                                       int streaming)
+                                                                       int streaming, int32_t ci)
 {
+    // ci = 1: planes of Hs x Ws.  ci = C: channels-last images, resized as planes whose rows are Ws * C elements
+    // (element j of a row is channel j % C of pixel j / C); "columns" below are row elements.
     constexpr int V = 16 / (int)sizeof(T);
     extern __shared__ uint4 nearest_smem[];
     char* lds = reinterpret_cast<char*>(nearest_smem);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const uint32_t wave = __builtin_amdgcn_readfirstlane((uint32_t)tid >> 6);
+    const int32_t Wse = Ws * ci, Wde = Wd * ci;
     const int32_t col_first = blockIdx.x * kThreads * V;
-    const int32_t col_last = ((col_first + kThreads * V < Wd) ? col_first + kThreads * V : Wd) - 1;
-    const int32_t s_lo = nearest_src(col_first, scale_w, Ws) / V * V;
-    const int32_t s_hi = nearest_src(col_last, scale_w, Ws);
+    const int32_t col_last = ((col_first + kThreads * V < Wde) ? col_first + kThreads * V : Wde) - 1;
+    const int32_t s_lo = nearest_src(col_first / ci, scale_w, Ws) * ci / V * V;
+    const int32_t s_hi = nearest_src(col_last / ci, scale_w, Ws) * ci + ci - 1;
     const uint32_t seg_bytes = (uint32_t)((s_hi - s_lo) / V + 1) * 16u;
     const bool use_lds = seg_bytes <= slot_bytes;  // uniform; the launch sizes the slots so that this holds
     const int32_t e0 = col_first + tid * V;
-    const bool active = e0 < Wd;
-    const int nvalid = (Wd - e0 < V) ? Wd - e0 : V;
+    const bool active = e0 < Wde;
+    const int nvalid = (Wde - e0 < V) ? Wde - e0 : V;
     int32_t src_col[V];
 #pragma unroll
     for (int i = 0; i < V; i++) {
-        const int32_t c = (e0 + i < Wd) ? e0 + i : Wd - 1;
-        src_col[i] = nearest_src(c, scale_w, Ws);
+        const int32_t c = (e0 + i < Wde) ? e0 + i : Wde - 1;
+        const int32_t px = (ci == 1) ? c : c / ci;
+        src_col[i] = nearest_src(px, scale_w, Ws) * ci + (c - px * ci);
     }
     const int64_t rows = outer * Hd;
     for (int64_t r0 = (int64_t)blockIdx.y * kNearestBand; r0 < rows; r0 += (int64_t)gridDim.y * kNearestBand) {
@@ -647,7 +651,7 @@ __global__ __launch_bounds__(kThreads) void resize_nearest_lds_kernel(const T* _
                 src_row[j] = o * Hs + nearest_src(h, scale_h, Hs);
                 if (src_row[j] != prev) {
                     if (use_lds) {
-                        const char* src = reinterpret_cast<const char*>(x + src_row[j] * (int64_t)Ws + s_lo);
+                        const char* src = reinterpret_cast<const char*>(x + src_row[j] * (int64_t)Wse + s_lo);
                         for (uint32_t cb = wave * 1024u; cb < seg_bytes; cb += (kThreads / 64) * 1024u) {
                             const uint32_t lane_off = cb + (uint32_t)lane * 16u;
                             if (lane_off < seg_bytes) {
@@ -687,7 +691,7 @@ __global__ __launch_bounds__(kThreads) void resize_nearest_lds_kernel(const T* _
                             v[i] = seg[src_col[i] - s_lo];
                         }
                     } else {
-                        const T* src = x + src_row[j] * (int64_t)Ws;
+                        const T* src = x + src_row[j] * (int64_t)Wse;
 #pragma unroll
                         for (int i = 0; i < V; i++) {
                             v[i] = src[src_col[i]];
@@ -698,7 +702,7 @@ __global__ __launch_bounds__(kThreads) void resize_nearest_lds_kernel(const T* _
                 }
                 // rows of a width that is not a multiple of V start anywhere: the vector store is element-aligned,
                 // and the lane at the ragged end of a row stores its elements singly
-                T* dst = y + (r0 + j) * (int64_t)Wd + e0;
+                T* dst = y + (r0 + j) * (int64_t)Wde + e0;
                 if (nvalid == V) {
                     typedef uint32_t u32x4_any __attribute__((ext_vector_type(4), aligned(2)));
                     u32x4_any t;
@@ -844,6 +848,36 @@ int four_weights_unit(const ResizeArgs& a)
     return 1;
 }
 
+// LDS bytes per staged source-row segment of the nearest kernel that gathers out of LDS, 0 when that kernel does not
+// apply.  It serves NCHW planes and channels-last images whose pixels are not whole 16-byte vectors (rows of Ws * C
+// elements), with source rows on the 16-byte grid.  The slot is the longest source segment a chunk of kThreads
+// vectors can touch, with slack for the rounding of the per-column products; the kernel checks the real length and
+// gathers from global memory otherwise.
+template <typename T>
+uint64_t nearest_lds_slot(const ResizeArgs& a)
+{
+    constexpr int V = 16 / (int)sizeof(T);
+    const bool nhwc = a.channels_last != 0;
+    const int64_t ci = nhwc ? a.C : 1;
+    if (a.mode != ResizeMode::Nearest || reinterpret_cast<uintptr_t>(a.x) % 16 != 0 || (a.Ws * ci) % V != 0 ||
+        a.Ws * ci > INT32_MAX || a.Wd * ci > INT32_MAX) {
+        return 0;
+    }
+    if (nhwc && (a.C % V == 0 || reinterpret_cast<uintptr_t>(a.y) % sizeof(T) != 0)) {
+        return 0;  // whole vectors per pixel: one vector load per lane does it
+    }
+    if (nhwc && a.Hd * a.Wd < a.Hs * a.Ws) {
+        return 0;  // shrinking images: nothing is reused, the gather from memory is as fast (measured)
+    }
+    const char* v = getenv("OPSCV_NEAREST_VARIANT");
+    if (v != nullptr && v[0] == 'g') {
+        return 0;
+    }
+    const double span = (double)(kThreads * V) * (double)a.scale_w * 1.001 + 2.0 + 2.0 * V + 2.0 * (double)ci;
+    const uint64_t slot = ((uint64_t)(span * sizeof(T)) + 15u) / 16u * 16u;
+    return (slot * kNearestBand <= 64u * 1024u) ? slot : 0;
+}
+
 template <typename T>
 hipError_t run_resize(const ResizeArgs& a, hipStream_t stream)
 {
@@ -902,17 +936,13 @@ hipError_t run_resize(const ResizeArgs& a, hipStream_t stream)
                        (int32_t)a.C, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h, a.scale_w, \
                        streaming)
         const int streaming = (out_elems * (int64_t)sizeof(T) >= (128ll << 20)) ? 1 : 0;
-        if (!nhwc && reinterpret_cast<uintptr_t>(x) % 16 == 0 && a.Ws % V == 0 && !(getenv("OPSCV_NEAREST_VARIANT") && getenv("OPSCV_NEAREST_VARIANT")[0] == 'g')) {
-            // slot = the longest source segment a chunk of kThreads vectors can touch, with slack for the rounding of
-            // the per-column products; the kernel checks the real length and gathers from global memory otherwise
-            const double span = (double)(kThreads * V) * (double)a.scale_w * 1.001 + 2.0 + 2.0 * V;
-            const uint64_t slot = ((uint64_t)(span * sizeof(T)) + 15u) / 16u * 16u;
-            if (slot * kNearestBand <= 64u * 1024u) {
-                hipLaunchKernelGGL((resize_nearest_lds_kernel<T>), grid, dim3(kThreads), slot * kNearestBand, stream, x,
-                                   y, outer, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h,
-                                   a.scale_w, (uint32_t)slot, streaming);
-                return hipGetLastError();
-            }
+        if (const uint64_t slot = nearest_lds_slot<T>(a)) {
+            const int64_t vlanes = (row_elems + V - 1) / V;
+            dim3 lgrid((unsigned)((vlanes + kThreads - 1) / kThreads), (unsigned)(bands < 65535 ? bands : 65535));
+            hipLaunchKernelGGL((resize_nearest_lds_kernel<T>), lgrid, dim3(kThreads), slot * kNearestBand, stream, x, y,
+                               outer, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h, a.scale_w,
+                               (uint32_t)slot, streaming, (int32_t)(nhwc ? a.C : 1));
+            return hipGetLastError();
         }
         if (nhwc) {
             if (vec) {
@@ -1086,15 +1116,16 @@ const char* resize_variant(const ResizeArgs& a)
         case ResizeMode::PointCopy: return "point_copy";
         case ResizeMode::FourWeights: return "nhwc_four_weights";
         case ResizeMode::Nearest: {
-            if (a.channels_last) {
-                return "nearest_nhwc";
+            uint64_t slot = 0;
+            switch (a.elem) {
+                case Elem::F32: slot = nearest_lds_slot<float>(a); break;
+                case Elem::F16: slot = nearest_lds_slot<_Float16>(a); break;
+                case Elem::BF16: slot = nearest_lds_slot<__bf16>(a); break;
             }
-            // source rows of whole 16-byte vectors and slots that fit: the LDS-staged kernel (see run_resize)
-            const int64_t V = 16 / elem_size(a.elem);
-            const double span = 256.0 * (double)V * (double)a.scale_w * 1.001 + 2.0 + 2.0 * (double)V;
-            const uint64_t slot = ((uint64_t)(span * elem_size(a.elem)) + 15u) / 16u * 16u;
-            const bool lds = a.Ws % V == 0 && slot * kNearestBand <= 64u * 1024u;
-            return lds ? "nearest_nchw_lds" : "nearest_nchw";
+            if (a.channels_last) {
+                return slot != 0 ? "nearest_nhwc_lds" : "nearest_nhwc";
+            }
+            return slot != 0 ? "nearest_nchw_lds" : "nearest_nchw";
         }
         default: break;
     }

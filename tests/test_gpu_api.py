@@ -608,6 +608,40 @@ def test_resize_nearest_wide_rows(oracle, device, aclnn, dtype):
 
 
 @pytest.mark.parametrize("dtype", I.DTYPES)
+def test_resize_nearest_few_channels_last(oracle, device, aclnn, dtype):
+    """nearest on channels-last images whose pixels are not whole vectors: growing images with source rows on the
+    16-byte grid gather out of LDS (rows of W * C elements), the others from memory; several column chunks, ragged
+    row ends, non-integer factors"""
+    import torch
+    rng = np.random.default_rng(321)
+    cases = [((2, 8, 8, 3), (16, 24), True), ((1, 6, 16, 5), (7, 40), True), ((1, 5, 1000, 3), (9, 2100), True),
+             ((2, 4, 24, 1), (8, 50), True), ((1, 7, 8, 6), (9, 13), True), ((1, 7, 9, 3), (9, 13), False),
+             ((1, 12, 16, 3), (5, 7), False)]
+    for shape, (Ho, Wo), lds in cases:
+        N, H, W, C = shape
+        x = I.cast_np(rng.standard_normal(shape).astype(np.float32), dtype)
+        ref = oracle.resize_nearest(x, (Ho, Wo), channels_last=True, dtype=I.oracle_code(dtype))
+        xt = I.to_torch(x, dtype, device)
+        out = torch.empty((N, Ho, Wo, C), dtype=xt.dtype, device=device)
+        sc = aclnn.create_float_array([1.0, Ho / H, Wo / W, 1.0])
+        hs = [aclnn.tensor_handle(xt, aclnn.ACL_FORMAT_NHWC), aclnn.tensor_handle(out, aclnn.ACL_FORMAT_NHWC)]
+        st, _, ex = aclnn.get_workspace_size_resize(hs[0], sc, b"nearest", hs[1])
+        assert st == 0
+        variant = aclnn.executor_variant(ex)
+        aclnn.destroy_executor(ex)
+        aclnn.destroy_float_array(sc)
+        for h in hs:
+            aclnn.destroy_tensor(h)
+        # 16-bit rows of 9 * 3 elements are off the 16-byte grid; fp32 rows of 27 elements too
+        assert variant == ("nearest_nhwc_lds" if lds else "nearest_nhwc"), (shape, variant)
+        y = aclnn.resize(xt, (1.0, Ho / H, Wo / W, 1.0), "nearest", out=out, channels_last=True)
+        torch.cuda.synchronize()
+        got = I.from_torch(y, dtype)
+        view = np.uint32 if dtype == "fp32" else np.uint16
+        assert np.array_equal(got.view(view), ref.view(view)), (shape, Ho, Wo, dtype)
+
+
+@pytest.mark.parametrize("dtype", I.DTYPES)
 def test_resize_point_copy(oracle, device, aclnn, dtype):
     """channels-last shrinks by whole factors take the reference's point-copy template: bit-exact copies, also of
     infinities and NaNs, through aclnnUpsampleBilinear2d and aclnnResize; vector and scalar channel counts"""
