@@ -188,8 +188,9 @@ template <typename TI>
 __device__ __forceinline__ float visit_sum(const TI* base, int32_t pitch, int32_t y0, int32_t x0, int32_t in_y_start,
                                            int32_t in_x_start, float out_y_start, float out_x_start, float fh,
                                            float fw, float scale_h, float scale_w, float last_y, float last_x,
-                                           int32_t Hd, int32_t Wd)
+                                           int32_t Hd, int32_t Wd, int32_t ci = 1, int32_t ch = 0)
 {
+    // ci, ch: channels-last rows hold ci elements per pixel, this lane's channel is ch (x0 counts elements)
     float acc = 0.0f;
     float out_y = out_y_start;
     for (int32_t in_y = in_y_start; out_y < fh + 1.0f && in_y < Hd; in_y++) {
@@ -200,7 +201,7 @@ __device__ __forceinline__ float visit_sum(const TI* base, int32_t pitch, int32_
         for (int32_t in_x = in_x_start; out_x < fw + 1.0f && in_x < Wd; in_x++) {
             const float xc = __builtin_fmaxf(0.0f, __builtin_fminf(out_x, last_x));
             const float x_lerp = 1.0f - __builtin_fabsf(xc - fw);
-            acc += ElemIO<TI>::load(row + (in_x - x0)) * y_lerp * x_lerp;
+            acc += ElemIO<TI>::load(row + ((int64_t)in_x * ci + ch - x0)) * y_lerp * x_lerp;
             out_x += scale_w;
         }
         out_y += scale_h;
@@ -211,11 +212,13 @@ __device__ __forceinline__ float visit_sum(const TI* base, int32_t pitch, int32_
 // The same sum with the column part of the loop taken out: a lane keeps the weights of the (at most KX) columns it
 // visits -- computed once, by the same repeated additions -- and a row costs one LDS read, two products and an add
 // per column.  Column k of a lane with fewer than k + 1 visits leaves the sum alone.
-template <typename TI, int KX, int KMIN>
+template <typename TI, int KX, int KMIN, bool IL = false>
 __device__ __forceinline__ float visit_sum_fixed(const TI* tile_xy, int32_t pitch, int32_t y0, int32_t in_y_start,
                                                  int32_t nx, const float* xl, float out_y_start, float fh,
-                                                 float scale_h, float last_y, int32_t Hd, float neg_zero)
+                                                 float scale_h, float last_y, int32_t Hd, float neg_zero,
+                                                 int32_t ci = 1)
 {
+    const int32_t step = IL ? ci : 1;  // elements between the columns a lane visits
     float acc = 0.0f;
     float out_y = out_y_start;
     for (int32_t in_y = in_y_start; out_y < fh + 1.0f && in_y < Hd; in_y++) {
@@ -228,7 +231,7 @@ __device__ __forceinline__ float visit_sum_fixed(const TI* tile_xy, int32_t pitc
             // fma(g, w, -0) is g * w bit for bit and lets a 16-bit element be converted by the multiply itself; the
             // read of a column past the lane's last one may fetch anything (it stays inside LDS) and is dropped.
             // Every lane of the workgroup visits at least KMIN columns: those need no test.
-            const float t = __builtin_fmaf(ElemIO<TI>::load(row + k), y_lerp, neg_zero) * xl[k];
+            const float t = __builtin_fmaf(ElemIO<TI>::load(row + k * step), y_lerp, neg_zero) * xl[k];
             acc = (k < KMIN || k < nx) ? acc + t : acc;
         }
         out_y += scale_h;
@@ -243,10 +246,11 @@ __device__ __forceinline__ float visit_sum_fixed(const TI* tile_xy, int32_t pitc
 // column, two products and an add.
 constexpr int kRowWeights = 6;  // visited rows per outgoing row kept in registers (more: the loops above)
 
-template <int KX, int KMIN, int Q>
+template <int KX, int KMIN, int Q, bool IL = false>
 __device__ __forceinline__ float tile_sum_fixed(const float* lane_rows, int32_t pitch, int32_t n_rows, float lerp_pack,
-                                                int32_t nx, const float* xl, float neg_zero)
+                                                int32_t nx, const float* xl, float neg_zero, int32_t ci = 1)
 {
+    const int32_t step = IL ? ci : 1;  // elements between the columns a lane visits
     float acc = 0.0f;
 #pragma unroll
     for (int j = 0; j < kRowWeights; j++) {
@@ -257,7 +261,7 @@ __device__ __forceinline__ float tile_sum_fixed(const float* lane_rows, int32_t 
 #pragma unroll
             for (int k = 0; k < KX; k++) {
                 // fma(g, w, -0) is g * w bit for bit; the compiler may not fold it into the following product
-                const float t = __builtin_fmaf(lane_rows[k], y_lerp, neg_zero) * xl[k];
+                const float t = __builtin_fmaf(lane_rows[k * step], y_lerp, neg_zero) * xl[k];
                 acc = (k < KMIN || k < nx) ? acc + t : acc;
             }
             lane_rows += pitch;
@@ -270,7 +274,10 @@ constexpr int kTileCols = 128;
 constexpr int32_t kGradCapWords = 12288;  // at most 48 KB of LDS per workgroup (fp32 words, one per tile element)
 constexpr int kTileGroups = kGradThreads / kTileCols;  // row groups of a workgroup
 
-template <typename TI, typename TO, bool HALF_PIXEL>
+// IL: channels-last tensors, taken as planes whose rows are W * ci elements (element j of a row is channel j % ci of
+// pixel j / ci); "columns" then count row elements, a lane's visited columns sit ci elements apart, and the column
+// geometry (first visit, count, weights) is that of the lane's pixel.
+template <typename TI, typename TO, bool HALF_PIXEL, bool IL>
 __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI* __restrict__ g, TO* __restrict__ y,
                                                                         int64_t planes, int32_t Hs, int32_t Ws,
                                                                         int32_t Hd, int32_t Wd, float scale_h,
@@ -278,8 +285,10 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
                                                                         float inv_scale_w, int32_t tile_rows,
                                                                         int32_t cap_words, float neg_zero,
                                                                         uint32_t tiles_x, uint32_t tiles_y,
-                                                                        uint32_t plane_slots)
+                                                                        uint32_t plane_slots, int32_t ci_arg)
 {
+    const int32_t ci = IL ? ci_arg : 1;
+    const int32_t Wse = Ws * ci, Wde = Wd * ci;  // row elements
     // Workgroups are handed to the eight XCDs in turn, each with its own L2.  The launch is one-dimensional and padded
     // to a multiple of eight; workgroup L becomes tile (L % 8) * (count / 8) + L / 8, so that an XCD works through a
     // contiguous run of tiles and the rows and 128-byte lines that neighbouring tiles share are fetched from memory
@@ -312,9 +321,11 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
         return in;
     };
     const int32_t W = W0 + tx;
-    const bool col_ok = W < Ws;
-    const int32_t in_x_start = first_visit(col_ok ? W : W0, inv_scale_w, Wd);
-    const int32_t tile_x0 = first_visit(W0, inv_scale_w, Wd) / EPW * EPW;
+    const bool col_ok = W < Wse;
+    const int32_t px = IL ? (col_ok ? W : W0) / ci : (col_ok ? W : W0);  // pixel of this lane's column
+    const int32_t ch = IL ? (col_ok ? W : W0) - px * ci : 0;               // and its channel
+    const int32_t in_x_start = first_visit(px, inv_scale_w, Wd);
+    const int32_t tile_x0 = first_visit(IL ? W0 / ci : W0, inv_scale_w, Wd) * ci / EPW * EPW;
     const int32_t tile_y0 = first_visit(H0, inv_scale_h, Hd);
     if (threadIdx.x == 0) {
         s_x1 = 0;
@@ -329,7 +340,7 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
         // per wavefront (an atomic per lane is serialised lane by lane on the scalar unit)
         int32_t x_end = 0;
         if (col_ok) {
-            x_end = end_visit(W, in_x_start, scale_w, Wd);
+            x_end = end_visit(px, in_x_start, scale_w, Wd);
             nx = x_end - in_x_start;
         }
         int32_t m_end = x_end, m_nx = nx, m_min = col_ok ? nx : INT32_MAX;  // lanes past the last column do not count
@@ -352,7 +363,7 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
         }
     }
     __syncthreads();
-    const int32_t tile_x1 = (s_x1 + EPW - 1) / EPW * EPW;  // Wd is a multiple of EPW (host check): stays inside the row
+    const int32_t tile_x1 = (s_x1 * ci + EPW - 1) / EPW * EPW;  // rows are multiples of EPW (host check): stays inside
     const int32_t tile_y1 = s_y1;
     const int32_t pitch_w = (tile_x1 > tile_x0) ? (tile_x1 - tile_x0) / EPW : 0;
     const int32_t rows = (tile_y1 > tile_y0) ? tile_y1 - tile_y0 : 0;
@@ -362,7 +373,7 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
     const bool use_lds = (int64_t)rows * pitch <= cap_words;
     const float* tile = reinterpret_cast<const float*>(tile_words);
     const float out_x_start = ((float)in_x_start + offset) * scale_w - offset;
-    const float fw = (float)W;
+    const float fw = (float)px;
 
     // column weights of this lane, for the variants with a fixed column count
     constexpr int KMAX = 8;
@@ -381,7 +392,7 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
     const int32_t pw1 = (pitch_w > 0) ? pitch_w : 1;
     const int32_t ld_r0 = (int32_t)threadIdx.x / pw1, ld_c0 = (int32_t)threadIdx.x % pw1;
     const int32_t ld_dr = kGradThreads / pw1, ld_dc = kGradThreads % pw1;
-    const int32_t x_base = (nx > 0) ? in_x_start - tile_x0 : 0;
+    const int32_t x_base = (nx > 0) ? in_x_start * ci + ch - tile_x0 : 0;
 
     // rows visited by each of this wavefront's outgoing rows, and their weights (see tile_sum_fixed)
     constexpr int HQ = 8 / kTileGroups;  // outgoing rows per lane at the largest tile height
@@ -411,14 +422,14 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
 
     // Copy of the rectangle into LDS: word i of the tile is (row i / pitch_w, word i % pitch_w) of the rectangle.
     const int32_t total = rows * pitch_w;
-    const int32_t row_words = Wd / EPW;
+    const int32_t row_words = Wde / EPW;
 
     for (int64_t pl = block_z; pl < planes; pl += plane_slots) {
-        const TI* gp = g + pl * (int64_t)Hd * Wd;
+        const TI* gp = g + pl * (int64_t)Hd * Wde;
         if (use_lds) {
             // the pair (row, word) is advanced instead of divided
             int32_t r = ld_r0, cw = ld_c0;
-            const uint32_t* src = reinterpret_cast<const uint32_t*>(gp + (int64_t)tile_y0 * Wd + tile_x0);
+            const uint32_t* src = reinterpret_cast<const uint32_t*>(gp + (int64_t)tile_y0 * Wde + tile_x0);
 #pragma unroll 8
             for (int32_t i = threadIdx.x; i < total; i += kGradThreads) {
                 const uint32_t word = src[(int64_t)r * row_words + cw];
@@ -442,7 +453,7 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
             __syncthreads();
         }
         if (col_ok && use_lds && rows_fixed && nx_max <= 6) {
-            TO* yp = y + (pl * Hs + H0 + ty) * (int64_t)Ws + W;
+            TO* yp = y + (pl * Hs + H0 + ty) * (int64_t)Wse + W;
             // -0 in a vector register: with the row weight in a scalar one, a second scalar operand would be copied
             // into a vector register before every product
             const float neg_zero_v = as_fp32_value(neg_zero);
@@ -455,7 +466,7 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
                     const float* lane_rows = tile + (first_row - tile_y0) * pitch + x_base;
                     float acc;
 #define OPSCV_TILE_SUM(KX, KMIN) \
-    tile_sum_fixed<KX, KMIN, q>(lane_rows, pitch, n_rows, lerp_pack, nx, xl, neg_zero_v)
+    tile_sum_fixed<KX, KMIN, q, IL>(lane_rows, pitch, n_rows, lerp_pack, nx, xl, neg_zero_v, ci)
                     if (nx_max <= 4) {
                         acc = (nx_min >= 4) ? OPSCV_TILE_SUM(4, 4) : OPSCV_TILE_SUM(4, 0);
                     } else if (nx_max <= 5) {
@@ -464,7 +475,7 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
                         acc = (nx_min >= 4) ? OPSCV_TILE_SUM(6, 4) : OPSCV_TILE_SUM(6, 0);
                     }
 #undef OPSCV_TILE_SUM
-                    ElemIO<TO>::store(yp + (int64_t)q * kTileGroups * Ws, acc);
+                    ElemIO<TO>::store(yp + (int64_t)q * kTileGroups * Wse, acc);
                 }
             };
             static_assert(HQ == 4, "one call per outgoing row of a lane");
@@ -479,8 +490,8 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
                 float acc;
                 // separate call sites so that each is compiled for its own address space (LDS reads, global loads)
 #define OPSCV_VISIT(KX, KMIN)                                                                                       \
-    visit_sum_fixed<float, KX, KMIN>(tile + x_base, pitch, tile_y0, in_y_start, nx, xl, out_y_start, (float)H, scale_h,  \
-                                  last_y, Hd, neg_zero)
+    visit_sum_fixed<float, KX, KMIN, IL>(tile + x_base, pitch, tile_y0, in_y_start, nx, xl, out_y_start, (float)H,    \
+                                         scale_h, last_y, Hd, neg_zero, ci)
                 if (use_lds && nx_max <= 4) {
                     acc = (nx_min >= 4) ? OPSCV_VISIT(4, 4) : OPSCV_VISIT(4, 0);
                 } else if (use_lds && nx_max <= 5) {
@@ -491,13 +502,13 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
                     acc = OPSCV_VISIT(8, 0);
                 } else if (use_lds) {
                     acc = visit_sum<float>(tile, pitch, tile_y0, tile_x0, in_y_start, in_x_start, out_y_start,
-                                        out_x_start, (float)H, fw, scale_h, scale_w, last_y, last_x, Hd, Wd);
+                                        out_x_start, (float)H, fw, scale_h, scale_w, last_y, last_x, Hd, Wd, ci, ch);
                 } else {
-                    acc = visit_sum<TI>(gp, Wd, 0, 0, in_y_start, in_x_start, out_y_start, out_x_start, (float)H, fw,
-                                        scale_h, scale_w, last_y, last_x, Hd, Wd);
+                    acc = visit_sum<TI>(gp, Wde, 0, 0, in_y_start, in_x_start, out_y_start, out_x_start, (float)H, fw,
+                                        scale_h, scale_w, last_y, last_x, Hd, Wd, ci, ch);
                 }
 #undef OPSCV_VISIT
-                ElemIO<TO>::store(y + (pl * Hs + H) * (int64_t)Ws + W, acc);
+                ElemIO<TO>::store(y + (pl * Hs + H) * (int64_t)Wse + W, acc);
             }
         }
         if (use_lds) {
@@ -512,11 +523,14 @@ template <typename TI>
 int32_t lds_tile_rows(const ResizeGradArgs& a, int32_t cap_words, int32_t* need_words = nullptr)
 {
     constexpr int EPW = 4 / (int)sizeof(TI);
-    if (a.channels_last || a.user_scales || a.Wd % EPW != 0 || reinterpret_cast<uintptr_t>(a.x) % 4 != 0) {
+    const int64_t ci = a.channels_last ? a.C : 1;  // row elements per pixel
+    if (a.user_scales || (a.Wd * ci) % EPW != 0 || reinterpret_cast<uintptr_t>(a.x) % 4 != 0 ||
+        a.Ws * ci > INT32_MAX || a.Wd * ci > INT32_MAX) {
         return 0;
     }
     const double per_col = (double)a.Wd / (double)a.Ws, per_row = (double)a.Hd / (double)a.Hs;
-    const double cols = kTileCols * per_col + 2.0 * per_col + 2.0 + EPW;
+    // a tile of kTileCols outgoing elements visits that many times per_col incoming ones, plus two pixels either side
+    const double cols = kTileCols * per_col + (2.0 * per_col + 2.0) * (double)ci + EPW;
     for (int32_t rows = 8; rows >= kTileGroups; rows /= 2) {
         const double need = (rows * per_row + 2.0 * per_row + 2.0) * cols;  // fp32 words: one per element
         if (need <= (double)cap_words) {
@@ -540,27 +554,37 @@ hipError_t run(const ResizeGradArgs& a, hipStream_t stream)
     lds_words = (lds_words + 63) / 64 * 64;
     lds_words = lds_words < kCapWords ? lds_words : kCapWords;
     if (tile_rows > 0) {
-        const int64_t planes = a.N * a.C;
+        const int64_t ci = a.channels_last ? a.C : 1;
+        const int64_t planes = a.channels_last ? a.N : a.N * a.C;
+        const int64_t row_elems = a.Ws * ci;
         // A workgroup walks over several planes with the tile geometry and column weights it computed once; enough
         // workgroups are launched to keep every CU supplied (want_blocks), the rest of the planes are looped over.
-        const int64_t tiles = ((a.Ws + kTileCols - 1) / kTileCols) * ((a.Hs + tile_rows - 1) / tile_rows);
+        const int64_t tiles = ((row_elems + kTileCols - 1) / kTileCols) * ((a.Hs + tile_rows - 1) / tile_rows);
         const int64_t want_blocks = 8192;
         int64_t zdim = (want_blocks + tiles - 1) / tiles;
         zdim = zdim < planes ? zdim : planes;
         zdim = zdim < 65535 ? zdim : 65535;
-        const int64_t tiles_x = (a.Ws + kTileCols - 1) / kTileCols, tiles_y = (a.Hs + tile_rows - 1) / tile_rows;
+        const int64_t tiles_x = (row_elems + kTileCols - 1) / kTileCols, tiles_y = (a.Hs + tile_rows - 1) / tile_rows;
         const int64_t blocks = (tiles * zdim + 7) / 8 * 8;  // padded for the XCD mapping of the kernel
         if (tiles_y <= 65535 && blocks <= (int64_t)INT32_MAX) {
             const dim3 grid((unsigned)blocks);
-#define OPSCV_RGL(HP)                                                                                                \
-    hipLaunchKernelGGL((resize_grad_lds_kernel<TI, TO, HP>), grid, dim3(kGradThreads), lds_words * 4, stream,         \
+#define OPSCV_RGL(HP, IL)                                                                                            \
+    hipLaunchKernelGGL((resize_grad_lds_kernel<TI, TO, HP, IL>), grid, dim3(kGradThreads), lds_words * 4, stream,     \
                        (const TI*)a.x, (TO*)a.y, planes, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, \
                        a.scale_h, a.scale_w, a.inv_scale_h, a.inv_scale_w, tile_rows, lds_words, -0.0f,              \
-                       (uint32_t)tiles_x, (uint32_t)tiles_y, (uint32_t)zdim)
+                       (uint32_t)tiles_x, (uint32_t)tiles_y, (uint32_t)zdim, (int32_t)ci)
             if (a.half_pixel) {
-                OPSCV_RGL(true);
+                if (a.channels_last) {
+                    OPSCV_RGL(true, true);
+                } else {
+                    OPSCV_RGL(true, false);
+                }
             } else {
-                OPSCV_RGL(false);
+                if (a.channels_last) {
+                    OPSCV_RGL(false, true);
+                } else {
+                    OPSCV_RGL(false, false);
+                }
             }
 #undef OPSCV_RGL
             return hipGetLastError();

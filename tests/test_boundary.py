@@ -391,7 +391,10 @@ def test_upsample_backward_status_codes(aclnn, desc):
     # formats: equal, NCHW or NHWC; NHWC reads the four extents as N,H,W,C
     assert _ub(aclnn, desc, ofmt=aclnn.ACL_FORMAT_NHWC)[0] == INV
     assert _ub(aclnn, desc, grad=(1, 2, 2, 5), out=(1, 3, 3, 5), isize=(1, 3, 3, 5), fmt=aclnn.ACL_FORMAT_NHWC,
-               sh=0, sw=0) == (0, 0, "resize_grad_gather")
+               sh=0, sw=0) == (0, 0, "resize_grad_lds")
+    # 16-bit rows of an odd number of elements are not whole 4-byte words: the per-element gather
+    assert _ub(aclnn, desc, grad=(1, 2, 3, 5), out=(1, 3, 3, 5), osize=(2, 3), isize=(1, 3, 3, 5),
+               fmt=aclnn.ACL_FORMAT_NHWC, dt=aclnn.ACL_FLOAT16, sh=0, sw=0) == (0, 0, "resize_grad_gather")
     # equal sizes: a copy
     assert _ub(aclnn, desc, grad=(1, 1, 3, 3), osize=(3, 3), sh=1.0, sw=1.0)[2] == "copy"
 

@@ -311,7 +311,10 @@ def test_upsample_backward(oracle, device, aclnn, dtype, channels_last):
              # several column tiles and ragged row tiles of the LDS variant; an odd incoming width (16-bit types
              # then take the gather kernel); a x20 upscale whose tile exceeds the LDS capacity; a strong downscale
              ((1, 2, 37, 300), (75, 610), True, 0.0, 0.0), ((2, 1, 19, 131), (40, 263), False, 0.0, 0.0),
-             ((1, 1, 9, 130), (180, 2600), False, 0.0, 0.0), ((1, 2, 90, 260), (11, 40), True, 0.0, 0.0)]
+             ((1, 1, 9, 130), (180, 2600), False, 0.0, 0.0), ((1, 2, 90, 260), (11, 40), True, 0.0, 0.0),
+             # channel counts whose channels-last rows span several column tiles with taps 3, 16 and 40 elements apart
+             ((2, 3, 21, 131), (40, 262), False, 0.0, 0.0), ((1, 16, 9, 40), (20, 85), True, 0.0, 0.0),
+             ((1, 40, 6, 12), (13, 30), False, 0.0, 0.0)]
     for in_shape, (Ho, Wo), align, sh, sw in cases:
         N, C, H, W = in_shape
         g = I.cast_np(rng.standard_normal((N, C, Ho, Wo)).astype(np.float32), dtype)
