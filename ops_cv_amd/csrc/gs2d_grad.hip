@@ -390,15 +390,12 @@ hipError_t launch_interp(const GridSamplerGradArgs& a, hipStream_t stream)
             return hipErrorInvalidValue;
         }
         const dim3 grid((unsigned)bands, (unsigned)cgroups, (unsigned)a.N);
-        static bool attr_set = false;  // more than the default 64 KB of dynamic LDS may be asked for
-        if (!attr_set) {
-            const hipError_t ea = hipFuncSetAttribute(
-                reinterpret_cast<const void*>(gs2d_grad_input_kernel<T, INTERP, CBMAX>),
-                hipFuncAttributeMaxDynamicSharedMemorySize, kTagsMax * 4 + 4096 * CBMAX * (int)sizeof(T));
-            if (ea != hipSuccess) {
-                return ea;
-            }
-            attr_set = true;
+        static std::atomic<uint32_t> lds_allowed{0};  // more than the default 64 KB of dynamic LDS may be asked for
+        const hipError_t ea =
+            allow_dynamic_lds(reinterpret_cast<const void*>(gs2d_grad_input_kernel<T, INTERP, CBMAX>),
+                              kTagsMax * 4 + 4096 * CBMAX * (int)sizeof(T), lds_allowed);
+        if (ea != hipSuccess) {
+            return ea;
         }
         if (grouped) {
             hipLaunchKernelGGL((gs2d_grad_input_kernel<T, INTERP, CBMAX>), grid, dim3(kThreads),

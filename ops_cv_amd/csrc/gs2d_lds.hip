@@ -38,6 +38,12 @@ LdsPlan make_lds_plan(const GridSamplerArgs& a)
     if (a.interp == 2) {
         p.ppt = (out_plane >= 4 * kThreads) ? 2 : 1;  // sixteen tap offsets per pixel live in registers
     }
+    // Two neighbouring pixels per lane and store for 16-bit elements: needs every output plane to start on a 4-byte
+    // boundary and to hold whole pairs (fp16 N16 C256 64x64: 128-byte stores 17.1 us, 256-byte stores 16.2 us, and the
+    // lanes of a wavefront then read taps two columns apart, which halves the LDS bank conflicts of a smooth grid)
+    if (esz == 2 && p.ppt >= 4 && a.interp != 2 && out_plane % 2 == 0 && reinterpret_cast<uintptr_t>(a.y) % 4 == 0) {
+        p.adj = 2;
+    }
     const int64_t tile = (int64_t)kThreads * p.ppt;
     p.tiles_per_n = (uint32_t)((out_plane + tile - 1) / tile);
     // channels per workgroup: as many stages as possible (the pixel decisions are reused across them) while

@@ -33,28 +33,54 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
 constexpr uint32_t kBufferFlags = 0x00020000u;  // raw buffer, 32-bit data format
 
-template <typename T>
-__device__ __forceinline__ void load_grid_pair(const T* gp, bool pair_aligned, float* gx, float* gy)
+// The grid points (x, y interleaved, element type T) of COUNT pixels starting at `gp`, `stride` pixels apart, as raw
+// bits.  The loads carry no condition and no use between them, so they are in flight together: one memory latency
+// for all pixels of a lane (written per pixel with the alignment test inside, every load was followed by a wait).
+template <typename T, int COUNT>
+__device__ __forceinline__ void load_grid_points(const T* const* gp, bool pair_aligned, float* gx, float* gy)
 {
     if constexpr (sizeof(T) == 2) {
         if (pair_aligned) {
-            const uint32_t raw = *reinterpret_cast<const uint32_t*>(gp);
-            T lo = __builtin_bit_cast(T, (uint16_t)(raw & 0xFFFFu));
-            T hi = __builtin_bit_cast(T, (uint16_t)(raw >> 16));
-            *gx = ElemIO<T>::load(&lo);
-            *gy = ElemIO<T>::load(&hi);
+            uint32_t raw[COUNT];
+#pragma unroll
+            for (int j = 0; j < COUNT; j++) {
+                raw[j] = *reinterpret_cast<const uint32_t*>(gp[j]);
+            }
+#pragma unroll
+            for (int j = 0; j < COUNT; j++) {
+                T lo = __builtin_bit_cast(T, (uint16_t)(raw[j] & 0xFFFFu));
+                T hi = __builtin_bit_cast(T, (uint16_t)(raw[j] >> 16));
+                gx[j] = ElemIO<T>::load(&lo);
+                gy[j] = ElemIO<T>::load(&hi);
+            }
             return;
         }
     } else {
         if (pair_aligned) {
-            const float2 raw = *reinterpret_cast<const float2*>(gp);
-            *gx = raw.x;
-            *gy = raw.y;
+            float2 raw[COUNT];
+#pragma unroll
+            for (int j = 0; j < COUNT; j++) {
+                raw[j] = *reinterpret_cast<const float2*>(gp[j]);
+            }
+#pragma unroll
+            for (int j = 0; j < COUNT; j++) {
+                gx[j] = raw[j].x;
+                gy[j] = raw[j].y;
+            }
             return;
         }
     }
-    *gx = ElemIO<T>::load(gp);
-    *gy = ElemIO<T>::load(gp + 1);
+    T ex[COUNT], ey[COUNT];
+#pragma unroll
+    for (int j = 0; j < COUNT; j++) {
+        ex[j] = gp[j][0];
+        ey[j] = gp[j][1];
+    }
+#pragma unroll
+    for (int j = 0; j < COUNT; j++) {
+        gx[j] = ElemIO<T>::load(&ex[j]);
+        gy[j] = ElemIO<T>::load(&ey[j]);
+    }
 }
 
 // Raw tap values of one pixel from a staged plane (LDS reads only, no arithmetic, so that the reads of
@@ -62,13 +88,40 @@ __device__ __forceinline__ void load_grid_pair(const T* gp, bool pair_aligned, f
 // `taddr` holds absolute LDS addresses of the taps in the first plane of the ring (base of the LDS allocation
 // already added, once, in the prologue); `plane_off` is the compile-time distance of the plane being sampled, which
 // ends up in the instruction's immediate offset.
+// A tap value stays in a 32-bit register of its own (16-bit elements zero-extended, as the LDS read delivers them):
+// left as 16-bit objects the compiler packs two of them into one register, and the packing instruction waits for
+// the reads right behind their issue, which undoes the overlap of the reads with the previous plane's arithmetic.
 template <typename T, int NT>
-__device__ __forceinline__ void load_taps(uint32_t plane_off, const uint32_t* taddr, T* raw)
+__device__ __forceinline__ void load_taps(uint32_t plane_off, const uint32_t* taddr, uint32_t* raw)
 {
-    typedef const T __attribute__((address_space(3))) * lds_elem_ptr_t;
+    typedef typename std::conditional<sizeof(T) == 2, uint16_t, uint32_t>::type bits_t;
+    typedef const bits_t __attribute__((address_space(3))) * lds_bits_ptr_t;
 #pragma unroll
     for (int t = 0; t < NT; t++) {
-        raw[t] = *reinterpret_cast<lds_elem_ptr_t>((uintptr_t)(taddr[t] + plane_off));
+        raw[t] = (uint32_t)*reinterpret_cast<lds_bits_ptr_t>((uintptr_t)(taddr[t] + plane_off));
+    }
+}
+
+template <typename T>
+__device__ __forceinline__ float tap_value(uint32_t raw)
+{
+    if constexpr (std::is_same<T, float>::value) {
+        return __builtin_bit_cast(float, raw);
+    } else if constexpr (std::is_same<T, _Float16>::value) {
+        return (float)__builtin_bit_cast(_Float16, (uint16_t)raw);
+    } else {
+        return __builtin_bit_cast(float, raw << 16);
+    }
+}
+
+// ... and of a tap held as an element (the channels-last kernel loads vectors of elements)
+template <typename T, typename R>
+__device__ __forceinline__ float tap_value_of(const R& raw)
+{
+    if constexpr (std::is_same<R, uint32_t>::value && !std::is_same<T, uint32_t>::value) {
+        return tap_value<T>(raw);
+    } else {
+        return ElemIO<T>::load(&raw);
     }
 }
 
@@ -84,17 +137,17 @@ __device__ __forceinline__ void load_taps(uint32_t plane_off, const uint32_t* ta
 // multiply-adds, and so is the column of the four row results.  A tap outside the image reads the zero slot; a
 // row outside the image therefore evaluates to +0 like the reference's literal 0 (the products are zeros and at
 // least one of the two middle coefficients is positive, so the sum cannot be -0).
-template <typename T, int INTERP>
-__device__ __forceinline__ float blend(const T* raw, const float* tw, float neg_zero)
+template <typename T, int INTERP, typename R>
+__device__ __forceinline__ float blend(const R* raw, const float* tw, float neg_zero)
 {
     if (INTERP == 2) {
         float r[4];
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            float acc = __builtin_fmaf(ElemIO<T>::load(&raw[4 * j]), tw[0], neg_zero);
-            acc = __builtin_fmaf(tw[1], ElemIO<T>::load(&raw[4 * j + 1]), acc);
-            acc = __builtin_fmaf(tw[2], ElemIO<T>::load(&raw[4 * j + 2]), acc);
-            acc = __builtin_fmaf(tw[3], ElemIO<T>::load(&raw[4 * j + 3]), acc);
+            float acc = __builtin_fmaf(tap_value_of<T>(raw[4 * j]), tw[0], neg_zero);
+            acc = __builtin_fmaf(tw[1], tap_value_of<T>(raw[4 * j + 1]), acc);
+            acc = __builtin_fmaf(tw[2], tap_value_of<T>(raw[4 * j + 2]), acc);
+            acc = __builtin_fmaf(tw[3], tap_value_of<T>(raw[4 * j + 3]), acc);
             r[j] = acc;
         }
         float out = tw[4] * r[0];
@@ -104,13 +157,13 @@ __device__ __forceinline__ float blend(const T* raw, const float* tw, float neg_
         return as_fp32_value(out);
     }
     if (INTERP == 0) {
-        float out = __builtin_fmaf(ElemIO<T>::load(&raw[0]), tw[0], 0.0f);
-        out += __builtin_fmaf(ElemIO<T>::load(&raw[1]), tw[1], neg_zero);
-        out += __builtin_fmaf(ElemIO<T>::load(&raw[2]), tw[2], neg_zero);
-        out += __builtin_fmaf(ElemIO<T>::load(&raw[3]), tw[3], neg_zero);
+        float out = __builtin_fmaf(tap_value_of<T>(raw[0]), tw[0], 0.0f);
+        out += __builtin_fmaf(tap_value_of<T>(raw[1]), tw[1], neg_zero);
+        out += __builtin_fmaf(tap_value_of<T>(raw[2]), tw[2], neg_zero);
+        out += __builtin_fmaf(tap_value_of<T>(raw[3]), tw[3], neg_zero);
         return out;
     }
-    return ElemIO<T>::load(&raw[0]);
+    return tap_value_of<T>(raw[0]);
 }
 
 template <typename T>
@@ -122,6 +175,25 @@ __device__ __forceinline__ void buffer_store_elem(float v, __amdgpu_buffer_rsrc_
         T h;
         ElemIO<T>::store(&h, v);
         __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(uint16_t, h), rsrc, (int)byte_off, 0, 0);
+    }
+}
+
+// The results of ADJ neighbouring output pixels of one channel leave as one store: two 16-bit results as one dword
+// (each rounded to T on its own, exactly as the single store does), so a wavefront writes 256 contiguous bytes per
+// instruction instead of 128.  The caller guarantees a 4-byte aligned address (even pixel index, even plane size).
+template <typename T, int ADJ>
+__device__ __forceinline__ void buffer_store_group(const float* v, __amdgpu_buffer_rsrc_t rsrc, uint32_t byte_off)
+{
+    if constexpr (ADJ == 1) {
+        buffer_store_elem<T>(v[0], rsrc, byte_off);
+    } else {
+        static_assert(ADJ == 2 && sizeof(T) == 2, "pairs of 16-bit results only");
+        // one packed conversion instruction, each half rounded to nearest even like the single conversion
+        typedef float float_pair_t __attribute__((ext_vector_type(2)));
+        typedef T elem_pair_t __attribute__((ext_vector_type(2)));
+        const float_pair_t f = {v[0], v[1]};
+        const elem_pair_t e = __builtin_convertvector(f, elem_pair_t);
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, e), rsrc, (int)byte_off, 0, 0);
     }
 }
 
@@ -234,8 +306,8 @@ __device__ __forceinline__ void issue_stage_copy(const char* src, char* dst, uin
 //
 // SHIFTED_PLANES selects the layout for planes off the 16-byte grid (issue_stage_copy); it is a template parameter so
 // that the kernels for whole, aligned planes carry no trace of it.
-template <typename T, int INTERP, int PAD, bool ALIGN, int SWAVES, int LWAVES, int PPT, int CGS, int NBUF, int PITCH,
-          bool SHIFTED_PLANES = false>
+template <typename T, int INTERP, int PAD, bool ALIGN, int SWAVES, int LWAVES, int PPT, int ADJ, int CGS, int NBUF,
+          int PITCH, bool SHIFTED_PLANES = false>
 __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves_per_eu(1, 5))) void gs2d_lds_kernel(
     const T* __restrict__ x, const T* __restrict__ grid, T* __restrict__ y, int32_t C, int32_t H, int32_t W,
     int32_t out_plane, uint32_t tiles_per_n, uint32_t cblocks, int32_t chans_per_block, int32_t copy_gran,
@@ -317,35 +389,37 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
                 issue_stage_copy<4, LWAVES, CGS, PITCH>(src, dst, plane_bytes, planes_of(s), lwave, lane, lane * 4u);
             }
         };
-#pragma unroll
-        for (int s = 0; s < DEPTH; s++) {
-            if (s < nstages) {
-                start_stage(s, s);
-            }
+        // `issued` stages have been started; stage q goes to slot q % NBUF, which is free once the samplers are through
+        // the barrier of stage q - DEPTH (their reads of stage q - NBUF have returned by then)
+        int32_t issued = 0;
+        int fill = 0;  // slot of stage `issued`
+        auto issue_next = [&]() {
+            start_stage(issued, fill);
+            issued++;
+            fill = (fill + 1 == NBUF) ? 0 : fill + 1;
+        };
+        while (issued < DEPTH && issued < nstages) {
+            issue_next();
         }
-        int slot = 0;
         for (int32_t s = 0; s < nstages; s++) {
-            // outstanding after stage s has landed: the copies of stages s+1 .. min(s+DEPTH, nstages)-1
+            // outstanding once stage s has landed: the copies of stages s + 1 .. issued - 1
             if constexpr (shifted) {
                 uint32_t later_copies = 0;
-                for (int32_t q = s + 1; q < s + DEPTH && q < nstages; q++) {
+                for (int32_t q = s + 1; q < issued; q++) {
                     later_copies += shifted_copy_count(q);
                 }
                 wait_vmcnt(later_copies);
             } else {
                 int32_t later_planes = 0;
-                for (int32_t q = s + 1; q < s + DEPTH && q < nstages; q++) {
+                for (int32_t q = s + 1; q < issued; q++) {
                     later_planes += planes_of(q);
                 }
                 wait_vmcnt((uint32_t)later_planes * per_plane);
             }
             lds_barrier();
-            if (s + DEPTH < nstages) {
-                int refill = slot + DEPTH;
-                refill = (refill >= NBUF) ? refill - NBUF : refill;
-                start_stage(s + DEPTH, refill);
+            if (issued < nstages) {
+                issue_next();
             }
-            slot = (slot + 1 == NBUF) ? 0 : slot + 1;
         }
         return;
     }
@@ -357,20 +431,30 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
     }
 
     // per-pixel decisions, once for the whole channel range
+    // A lane owns PPT / ADJ groups of ADJ neighbouring pixels; the groups of a lane are STHREADS * ADJ pixels apart.
+    // With ADJ = 2 (16-bit elements) the two results of a channel leave as one 4-byte store, and the lanes of a
+    // wavefront read taps two source columns apart, i.e. from different LDS banks for an undistorted grid.
+    static_assert(PPT % ADJ == 0, "whole groups per lane");
+    constexpr int NGRP = PPT / ADJ;
     uint32_t toff[PPT][NT];
     float tw[PPT][NW];
-    uint32_t pixoff[PPT];  // byte offset of the pixel inside an output plane; out of range for lanes past the end
-    // all grid points of the lane are requested before the first is used: one memory latency, not PPT of them
+    uint32_t pixoff[NGRP];  // byte offset of the group inside an output plane; out of range for lanes past the end
     float gxs[PPT], gys[PPT];
     const T* gridn = grid + (int64_t)n * out_plane * 2;
+    const T* gptr[PPT];
 #pragma unroll
-    for (int j = 0; j < PPT; j++) {
-        const int32_t pix = (int32_t)tile * (STHREADS * PPT) + j * STHREADS + tid;
-        const bool valid = pix < out_plane;
-        const int32_t pc = valid ? pix : out_plane - 1;
-        pixoff[j] = valid ? (uint32_t)pc * (uint32_t)sizeof(T) : 0x80000000u;
-        load_grid_pair<T>(gridn + (int64_t)pc * 2, pair_aligned != 0, &gxs[j], &gys[j]);
+    for (int q = 0; q < NGRP; q++) {
+        const int32_t pix0 = (int32_t)tile * (STHREADS * PPT) + q * (STHREADS * ADJ) + tid * ADJ;
+        // the output plane holds a whole number of groups (the launch plan picks ADJ accordingly)
+        const bool valid = pix0 < out_plane;
+        const int32_t pc = valid ? pix0 : out_plane - ADJ;
+        pixoff[q] = valid ? (uint32_t)pc * (uint32_t)sizeof(T) : 0x80000000u;
+#pragma unroll
+        for (int a = 0; a < ADJ; a++) {
+            gptr[q * ADJ + a] = gridn + (int64_t)(pc + a) * 2;
+        }
     }
+    load_grid_points<T, PPT>(gptr, pair_aligned != 0, gxs, gys);
     // the bank-spreading layout exists for border padding only (see make_lds_plan)
     const uint32_t rs = (PAD == 1) ? (uint32_t)row_shift : 0u;
 #pragma unroll
@@ -465,75 +549,65 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
     T* yb = y + ((int64_t)n * C + c_begin) * out_plane;
     const uint32_t out_plane_bytes = (uint32_t)out_plane * (uint32_t)sizeof(T);
 
-    // `buf` is the byte offset of the stage's slot inside the ring
     // the bytes by which a plane's copy started early (SHIFTED_PLANES, see issue_stage_copy): the low four bits of the
-    // plane's first byte address, from those of the tensor's address and of the plane size
+    // plane's first byte address, from those of the tensor's address and of the plane size.  The shift makes the
+    // plane distance a run-time value where it is a literal otherwise (one more add per tap).
     const uint32_t addr_low = (uint32_t)(reinterpret_cast<uintptr_t>(x) & 15u);
     const uint32_t size_low = plane_bytes & 15u;
     const uint32_t first_plane = (uint32_t)n * (uint32_t)C + (uint32_t)c_begin;
-    // The shift makes the plane distance a run-time value where it is a literal otherwise (one more add per tap).
-    auto sample_stage = [&](int32_t s, uint32_t buf) {
-        constexpr bool SHIFTED = SHIFTED_PLANES;
-        auto plane_shift = [&](int32_t stage, int k) -> uint32_t {
-            if constexpr (SHIFTED) {
-                return (addr_low + (first_plane + (uint32_t)(stage * CGS + k)) * size_low) & 15u;
-            } else {
-                (void)stage;
-                (void)k;
-                return 0u;
-            }
-        };
-        const int32_t left = nchan - s * CGS;
-        T* ys = yb + (int64_t)s * CGS * out_plane;
-        if (left >= CGS) {
-            // software pipeline over the channels of the stage: the taps of channel k+1 are read from LDS
-            // while channel k is blended and stored
-            T raw[2][PPT][NT];
-#pragma unroll
-            for (int j = 0; j < PPT; j++) {
-                load_taps<T, NT>(buf + plane_shift(s, 0), toff[j], raw[0][j]);
-            }
-#pragma unroll
-            for (int k = 0; k < CGS; k++) {
-                if (k + 1 < CGS) {
-#pragma unroll
-                    for (int j = 0; j < PPT; j++) {
-                        load_taps<T, NT>(buf + (k + 1) * PITCH + plane_shift(s, k + 1), toff[j], raw[(k + 1) & 1][j]);
-                    }
-                }
-                const __amdgpu_buffer_rsrc_t rsrc =
-                    __builtin_amdgcn_make_buffer_rsrc(ys + (int64_t)k * out_plane, 0, out_plane_bytes, kBufferFlags);
-#pragma unroll
-                for (int j = 0; j < PPT; j++) {
-                    buffer_store_elem<T>(blend<T, INTERP>(raw[k & 1][j], tw[j], neg_zero), rsrc, pixoff[j]);
-                }
-            }
+    auto plane_shift = [&](int32_t p) -> uint32_t {
+        if constexpr (SHIFTED_PLANES) {
+            return (addr_low + (first_plane + (uint32_t)p) * size_low) & 15u;
         } else {
-            for (int k = 0; k < left; k++) {
-                const __amdgpu_buffer_rsrc_t rsrc =
-                    __builtin_amdgcn_make_buffer_rsrc(ys + (int64_t)k * out_plane, 0, out_plane_bytes, kBufferFlags);
-                T raw[PPT][NT];
-#pragma unroll
-                for (int j = 0; j < PPT; j++) {
-                    load_taps<T, NT>(buf + k * PITCH + plane_shift(s, k), toff[j], raw[j]);
-                }
-#pragma unroll
-                for (int j = 0; j < PPT; j++) {
-                    buffer_store_elem<T>(blend<T, INTERP>(raw[j], tw[j], neg_zero), rsrc, pixoff[j]);
-                }
-            }
+            (void)p;
+            return 0u;
         }
     };
-
-    // the ring, unrolled by NBUF so that the slot offset is an immediate; one barrier per stage, matched by the
-    // loaders' loop above
+    // One software pipeline over all planes of the block, across stage boundaries.  A lane keeps one set of tap
+    // registers per pixel; as soon as a pixel of plane p has been blended, its registers are reloaded with the taps
+    // of plane p + 1, so the LDS reads of a pixel are in flight while the lane's other pixels are blended and
+    // stored (the per-wavefront counter of outstanding LDS operations is exact in straight-line code, which is why
+    // nothing in the steady state is conditional: past the last plane the reload reads whatever the ring holds and
+    // the values are dropped).  The barrier that hands over a stage sits in front of the first read of the stage's
+    // first plane, inside the previous stage's last plane.  A wavefront's LDS reads have all returned when it
+    // enters the barrier (lgkmcnt(0)), so the loaders, which refill the previous stage's slot once they are through
+    // the same barrier, never overwrite a plane that is still being read.  The loop is unrolled over one turn of
+    // the ring (NBUF stages of CGS planes) so that a plane's offset in the ring is an immediate.
+    constexpr int UNR = NBUF * CGS;
+    uint32_t raw[PPT][NT];
     __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the zero-slot writes, before the first barrier publishes them
-    for (int32_t s = 0; s < nstages; s += NBUF) {
+    lds_barrier();                        // stage 0 has landed
 #pragma unroll
-        for (int u = 0; u < NBUF; u++) {
-            if (s + u < nstages) {
-                lds_barrier();
-                sample_stage(s + u, (uint32_t)(u * SLOT_BYTES));
+    for (int j = 0; j < PPT; j++) {
+        load_taps<T, NT>(plane_shift(0), toff[j], raw[j]);
+    }
+    for (int32_t b = 0; b < nchan; b += UNR) {
+#pragma unroll
+        for (int u = 0; u < UNR; u++) {
+            const int32_t p = b + u;
+            if (p >= nchan) {
+                break;
+            }
+            const int un = (u + 1) % UNR;  // a literal once the loop is unrolled
+            const uint32_t next_off = (uint32_t)((un / CGS) * SLOT_BYTES + (un % CGS) * PITCH) + plane_shift(p + 1);
+            const __amdgpu_buffer_rsrc_t rsrc =
+                __builtin_amdgcn_make_buffer_rsrc(yb + (int64_t)p * out_plane, 0, out_plane_bytes, kBufferFlags);
+#pragma unroll
+            for (int q = 0; q < NGRP; q++) {
+                float v[ADJ];
+#pragma unroll
+                for (int a = 0; a < ADJ; a++) {
+                    const int j = q * ADJ + a;
+                    v[a] = blend<T, INTERP>(raw[j], tw[j], neg_zero);
+                    if (j == 0 && un % CGS == 0 && p + 1 < nchan) {
+                        __builtin_amdgcn_s_waitcnt(0xC07F);
+                        lds_barrier();  // stage (p + 1) / CGS has landed
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    load_taps<T, NT>(next_off, toff[j], raw[j]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                buffer_store_group<T, ADJ>(v, rsrc, pixoff[q]);
             }
         }
     }

@@ -14,6 +14,7 @@ struct LdsPlan {
     bool ok = false;
     int cls = 0;  // index into kPitch / kCgs
     int ppt = 4;
+    int adj = 1;  // neighbouring output pixels per store (2: pairs of 16-bit results as one dword)
     int copy_gran = 16;
     int xcd_swizzle = 0;
     int row_shift = 0;  // 7 when the staged planes (128-byte rows) use the bank-spreading layout, else 0
@@ -36,18 +37,14 @@ constexpr int kNbuf[5] = {4, 4, 4, 4, 2};  // ring slots (stages resident in LDS
 
 LdsPlan make_lds_plan(const GridSamplerArgs& a);
 
-template <typename T, int I, int P, bool A, int PPT, int CGS, int NBUF, int PITCH, int LWAVES, bool SHIFTED>
+template <typename T, int I, int P, bool A, int PPT, int ADJ, int CGS, int NBUF, int PITCH, int LWAVES, bool SHIFTED>
 hipError_t launch_one(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t stream)
 {
-    auto kernel = gs2d_lds_kernel<T, I, P, A, kSamplerWaves, LWAVES, PPT, CGS, NBUF, PITCH, SHIFTED>;
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, kLdsLimit);
-        if (e != hipSuccess) {
-            return e;
-        }
-        attr_set = true;
+    auto kernel = gs2d_lds_kernel<T, I, P, A, kSamplerWaves, LWAVES, PPT, ADJ, CGS, NBUF, PITCH, SHIFTED>;
+    static std::atomic<uint32_t> lds_allowed{0};
+    const hipError_t ea = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kLdsLimit, lds_allowed);
+    if (ea != hipSuccess) {
+        return ea;
     }
     const int64_t esz = sizeof(T);
     const int pair_aligned = (reinterpret_cast<uintptr_t>(a.grid) % (2 * esz) == 0);
@@ -62,7 +59,14 @@ hipError_t launch_one(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t st
 template <typename T, int I, int P, bool A, int CLS, int PPT, bool SHIFTED>
 hipError_t launch_cls(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t stream)
 {
-    return launch_one<T, I, P, A, PPT, kCgs[CLS], kNbuf[CLS], kPitch[CLS], kLoaderWaves[CLS], SHIFTED>(a, p, stream);
+    // pairs of neighbouring pixels per store exist for 16-bit elements with four or eight pixels per lane
+    if constexpr (sizeof(T) == 2 && PPT >= 4) {
+        if (p.adj == 2) {
+            return launch_one<T, I, P, A, PPT, 2, kCgs[CLS], kNbuf[CLS], kPitch[CLS], kLoaderWaves[CLS], SHIFTED>(a, p,
+                                                                                                                 stream);
+        }
+    }
+    return launch_one<T, I, P, A, PPT, 1, kCgs[CLS], kNbuf[CLS], kPitch[CLS], kLoaderWaves[CLS], SHIFTED>(a, p, stream);
 }
 
 // Expands (interp, pad, align, size class, pixels per lane) for one element type and launches.  Eight pixels per

@@ -544,20 +544,15 @@ hipError_t launch_interp(const GridSampler3DGradArgs& a, hipStream_t stream)
             ranges = (const int32_t*)a.chunk_ranges;
         }
         // more than the default 64 KB of dynamic LDS
-        static bool attr_set = false;
-        if (!attr_set) {
-            hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void*>(gs3d_grad_input_kernel<T, INTERP, CBMAX>),
-                                                hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                kTagsMax * 4 + kBandMax * CBMAX * (int)sizeof(T));
-            if (ea == hipSuccess) {
-                ea = hipFuncSetAttribute(reinterpret_cast<const void*>(gs3d_grad_input_kernel<T, INTERP, 1>),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         kTagsMax * 4 + kBandMax * (int)sizeof(T));
-            }
-            if (ea != hipSuccess) {
-                return ea;
-            }
-            attr_set = true;
+        static std::atomic<uint32_t> lds_allowed{0}, lds_allowed_single{0};
+        hipError_t ea = allow_dynamic_lds(reinterpret_cast<const void*>(gs3d_grad_input_kernel<T, INTERP, CBMAX>),
+                                          kTagsMax * 4 + kBandMax * CBMAX * (int)sizeof(T), lds_allowed);
+        if (ea == hipSuccess) {
+            ea = allow_dynamic_lds(reinterpret_cast<const void*>(gs3d_grad_input_kernel<T, INTERP, 1>),
+                                   kTagsMax * 4 + kBandMax * (int)sizeof(T), lds_allowed_single);
+        }
+        if (ea != hipSuccess) {
+            return ea;
         }
         if (grouped) {
             hipLaunchKernelGGL((gs3d_grad_input_kernel<T, INTERP, CBMAX>), grid, dim3(kThreads),

@@ -3,9 +3,32 @@
 
 #include <hip/hip_runtime_api.h>
 
+#include <atomic>
+
 #include "acl_types.hpp"
 
 namespace opscv {
+
+// Raises a kernel's dynamic-LDS limit once per device.  `done` is a bit mask of the devices served (one static
+// object per kernel at the call site); setting the attribute twice is harmless, so concurrent first calls need no
+// lock, only the atomic mask.
+inline hipError_t allow_dynamic_lds(const void* kernel, int bytes, std::atomic<uint32_t>& done)
+{
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) {
+        return e;
+    }
+    const uint32_t bit = 1u << (dev & 31);
+    if (done.load(std::memory_order_acquire) & bit) {
+        return hipSuccess;
+    }
+    e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (e == hipSuccess) {
+        done.fetch_or(bit, std::memory_order_release);
+    }
+    return e;
+}
 
 // Record written per output pixel by the tap-dump kernel (28 bytes, no padding).
 struct TapRecord {

@@ -109,16 +109,14 @@ __device__ __forceinline__ float safe_downgrade(float x)
     return x;
 }
 
-// float -> int32 with saturation (the hardware conversion saturates; 2^31 is out of bounds either way)
+// float -> int32 with saturation: values from 2^31 up give INT32_MAX, values below -2^31 give INT32_MIN (either is out
+// of bounds for every caller) and NaN gives 0.  This is what the hardware conversion does by itself; spelled with
+// comparisons in C++ (where the out-of-range cast is undefined) it compiles to branches around the same instruction.
 __device__ __forceinline__ int32_t float_to_i32(float v)
 {
-    if (v >= 2147483648.0f) {
-        return INT32_MAX;
-    }
-    if (v < -2147483648.0f) {
-        return INT32_MIN;
-    }
-    return (int32_t)v;
+    int32_t r;
+    asm("v_cvt_i32_f32 %0, %1" : "=v"(r) : "v"(v));
+    return r;
 }
 
 // grid_sampler2_d_simt.h:219-234
