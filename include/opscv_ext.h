@@ -51,6 +51,28 @@ ACLNN_API aclnnStatus opscvGridSampler2DBicubicTaps(const void* grid, aclDataTyp
  */
 ACLNN_API const char* opscvExecutorVariant(const aclOpExecutor* executor);
 
+/*
+ * Size in bytes of the library-owned scratch array behind opscvGridSampler2DNoAlloc: the most that the non-contiguous
+ * views of one call may need for packing (each packed view takes its size rounded up to 256 bytes).
+ */
+#define OPSCV_NOALLOC_SCRATCH_BYTES (16u << 20)
+
+/*
+ * aclnnGridSampler2DGetWorkspaceSize + aclnnGridSampler2D as one call that allocates nothing, neither on the device
+ * nor on the host.  It has no counterpart in the reference; it is for callers that cannot allocate a workspace
+ * between the two phases: code under HIP graph capture, serving loops with a fixed memory plan, harnesses that
+ * forbid allocation.  Same arguments, validation, status codes and results as the two-phase pair.  Where that pair
+ * packs non-contiguous views into the caller's workspace (and scatters a non-contiguous output from it), this entry
+ * point uses a file-scope device array of OPSCV_NOALLOC_SCRATCH_BYTES bytes that every device holds from library load
+ * to process end.  A call whose views would need more returns ACLNN_ERR_PARAM_INVALID (161002) and launches nothing.
+ * Contiguous tensors and channels-last views use no scratch at all.  All calls on one device share the array: calls
+ * that overlap in time on one device (different streams, different threads) race on it and must be serialised by the
+ * caller; calls on one stream are ordered by the stream.  Asynchronous on `stream` like aclnnGridSampler2D.
+ */
+ACLNN_API aclnnStatus opscvGridSampler2DNoAlloc(const aclTensor* input, const aclTensor* grid,
+                                                int64_t interpolationMode, int64_t paddingMode, bool alignCorners,
+                                                aclTensor* out, aclrtStream stream);
+
 /* Library version string, e.g. "opscv-amd 0.1 (gfx950)". */
 ACLNN_API const char* opscvVersion(void);
 

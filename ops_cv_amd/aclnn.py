@@ -134,6 +134,8 @@ def load_library():
     L.opscvGridSampler2DBicubicTaps.argtypes = [vp, ctypes.c_int, i64, i64, i64, i64, i64, i64, ctypes.c_bool, vp, vp]
     L.opscvExecutorVariant.restype = ctypes.c_char_p
     L.opscvExecutorVariant.argtypes = [vp]
+    L.opscvGridSampler2DNoAlloc.restype = i32
+    L.opscvGridSampler2DNoAlloc.argtypes = [vp, vp, i64, i64, ctypes.c_bool, vp, vp]
     L.opscvVersion.restype = ctypes.c_char_p
     L.opscvVersion.argtypes = []
     _lib = L
@@ -339,6 +341,22 @@ def grid_sampler2d(inp, grid, interpolation_mode=0, padding_mode=0, align_corner
         for h in hs:
             destroy_tensor(h)
     return out
+
+
+NOALLOC_SCRATCH_BYTES = 16 << 20  # OPSCV_NOALLOC_SCRATCH_BYTES (include/opscv_ext.h)
+
+
+def grid_sampler2d_noalloc(inp, grid, out, interpolation_mode=0, padding_mode=0, align_corners=False, stream=None):
+    """opscvGridSampler2DNoAlloc on torch CUDA tensors: one call, no workspace; `out` is the caller's.  Returns the
+    status code (0 on success) so that a test can look at the refusals as well."""
+    L = load_library()
+    hs = [tensor_handle(inp), tensor_handle(grid), tensor_handle(out)]
+    try:
+        return L.opscvGridSampler2DNoAlloc(hs[0], hs[1], interpolation_mode, padding_mode, align_corners, hs[2],
+                                           _stream_handle(stream))
+    finally:
+        for h in hs:
+            destroy_tensor(h)
 
 
 def grid_sampler2d_backward(grad_out, inp, grid, interpolation_mode=0, padding_mode=0, align_corners=False,

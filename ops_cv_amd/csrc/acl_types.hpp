@@ -210,8 +210,22 @@ struct aclOpExecutor {
         uint64_t ws_offset = 0;
         int elem_bytes = 0;
     };
-    std::vector<Pack> pack_in;
-    std::vector<Pack> unpack_out;
+    // at most three inputs and two outputs per operator; fixed storage, so that planning never touches the heap
+    struct PackList {
+        static constexpr int kCapacity = 4;
+        Pack items[kCapacity];
+        int count = 0;
+        void push_back(const Pack& p)
+        {
+            if (count < kCapacity) {
+                items[count++] = p;
+            }
+        }
+        const Pack* begin() const { return items; }
+        const Pack* end() const { return items + count; }
+    };
+    PackList pack_in;
+    PackList unpack_out;
 };
 
 namespace opscv {

@@ -7,6 +7,7 @@
 
 #include "aclnn_grid_sampler2d.h"
 #include "executor.hpp"
+#include "opscv_ext.h"
 
 using namespace opscv;
 
@@ -100,24 +101,16 @@ bool check_shapes(const aclTensor* input, const aclTensor* grid, const aclTensor
 
 }  // namespace
 
-extern "C" {
+namespace {
 
-aclnnStatus aclnnGridSampler2DGetWorkspaceSize(const aclTensor* input, const aclTensor* grid,
-                                               int64_t interpolationMode, int64_t paddingMode, bool alignCorners,
-                                               aclTensor* out, uint64_t* workspaceSize, aclOpExecutor** executor)
+// Everything the first phase does except creating the executor: validation in the reference's order
+// (aclnn_grid_sampler2d.cpp:159-175) and the plan, written into `ex`.
+aclnnStatus plan_grid_sampler2d(const aclTensor* input, const aclTensor* grid, int64_t interpolationMode,
+                                int64_t paddingMode, bool alignCorners, aclTensor* out, aclOpExecutor* ex)
 {
-    std::unique_ptr<aclOpExecutor> ex(new (std::nothrow) aclOpExecutor());
-    if (!ex) {
-        set_error("aclnnGridSampler2D: cannot allocate the executor");
-        return ACLNN_ERR_INNER_CREATE_EXECUTOR;
-    }
     // 1. null pointers (aclnn_grid_sampler2d.cpp:55-61)
     if (input == nullptr || grid == nullptr || out == nullptr) {
         set_error("aclnnGridSampler2D: input, grid and out must not be NULL");
-        return ACLNN_ERR_PARAM_NULLPTR;
-    }
-    if (workspaceSize == nullptr || executor == nullptr) {
-        set_error("aclnnGridSampler2D: workspaceSize and executor must not be NULL");
         return ACLNN_ERR_PARAM_NULLPTR;
     }
     // 2. dtypes, 3. attributes, 4. shapes
@@ -127,8 +120,6 @@ aclnnStatus aclnnGridSampler2DGetWorkspaceSize(const aclTensor* input, const acl
     }
     // empty tensors are a successful no-op that still hands out an executor (aclnn_grid_sampler2d.cpp:280-285)
     if (input->empty() || grid->empty()) {
-        *workspaceSize = 0;
-        *executor = ex.release();
         return ACLNN_SUCCESS;
     }
     // The reference routes DOUBLE to a host-CPU kernel that is not part of its tree; it does not exist here.
@@ -168,11 +159,35 @@ aclnnStatus aclnnGridSampler2DGetWorkspaceSize(const aclTensor* input, const acl
         ex->in0.direct = (input->data == nullptr) ? nullptr : (char*)input->data + input->offset * (int64_t)esz;
         ex->out0.direct = (out->data == nullptr) ? nullptr : (char*)out->data + out->offset * (int64_t)esz;
     } else {
-        ex->in0 = plan_view(ex.get(), input, esz, false);
-        ex->out0 = plan_view(ex.get(), out, esz, true);
+        ex->in0 = plan_view(ex, input, esz, false);
+        ex->out0 = plan_view(ex, out, esz, true);
     }
-    ex->in1 = plan_view(ex.get(), grid, esz, false);
+    ex->in1 = plan_view(ex, grid, esz, false);
+    return ACLNN_SUCCESS;
+}
 
+}  // namespace
+
+extern "C" {
+
+aclnnStatus aclnnGridSampler2DGetWorkspaceSize(const aclTensor* input, const aclTensor* grid,
+                                               int64_t interpolationMode, int64_t paddingMode, bool alignCorners,
+                                               aclTensor* out, uint64_t* workspaceSize, aclOpExecutor** executor)
+{
+    std::unique_ptr<aclOpExecutor> ex(new (std::nothrow) aclOpExecutor());
+    if (!ex) {
+        set_error("aclnnGridSampler2D: cannot allocate the executor");
+        return ACLNN_ERR_INNER_CREATE_EXECUTOR;
+    }
+    if (input != nullptr && grid != nullptr && out != nullptr && (workspaceSize == nullptr || executor == nullptr)) {
+        set_error("aclnnGridSampler2D: workspaceSize and executor must not be NULL");
+        return ACLNN_ERR_PARAM_NULLPTR;
+    }
+    const aclnnStatus st =
+        plan_grid_sampler2d(input, grid, interpolationMode, paddingMode, alignCorners, out, ex.get());
+    if (st != ACLNN_SUCCESS) {
+        return st;
+    }
     *workspaceSize = ex->workspace_bytes;
     *executor = ex.release();
     return ACLNN_SUCCESS;
@@ -181,6 +196,35 @@ aclnnStatus aclnnGridSampler2DGetWorkspaceSize(const aclTensor* input, const acl
 aclnnStatus aclnnGridSampler2D(void* workspace, uint64_t workspaceSize, aclOpExecutor* executor, aclrtStream stream)
 {
     return run_executor(workspace, workspaceSize, executor, stream, OpKind::GridSampler2D, "aclnnGridSampler2D");
+}
+
+// Both phases in one call, with the library's static scratch array in the place of the caller's workspace.  The plan
+// lives on the stack (its packing lists have fixed storage), so the call allocates nothing on either side.
+aclnnStatus opscvGridSampler2DNoAlloc(const aclTensor* input, const aclTensor* grid, int64_t interpolationMode,
+                                      int64_t paddingMode, bool alignCorners, aclTensor* out, aclrtStream stream)
+{
+    aclOpExecutor ex;
+    const aclnnStatus st = plan_grid_sampler2d(input, grid, interpolationMode, paddingMode, alignCorners, out, &ex);
+    if (st != ACLNN_SUCCESS) {
+        return st;
+    }
+    void* scratch = nullptr;
+    if (ex.workspace_bytes > 0) {
+        uint64_t capacity = 0;
+        const hipError_t e = static_scratch(&scratch, &capacity);
+        if (e != hipSuccess) {
+            set_error("opscvGridSampler2DNoAlloc: the static scratch array is not available: %s",
+                      hipGetErrorString(e));
+            return ACLNN_ERR_RUNTIME_ERROR;
+        }
+        if (ex.workspace_bytes > capacity) {
+            set_error("opscvGridSampler2DNoAlloc: packing the non-contiguous views needs %llu bytes, the static "
+                      "scratch array holds %llu; use aclnnGridSampler2D with a workspace",
+                      (unsigned long long)ex.workspace_bytes, (unsigned long long)capacity);
+            return ACLNN_ERR_PARAM_INVALID;
+        }
+    }
+    return execute_plan(scratch, &ex, stream, "opscvGridSampler2DNoAlloc");
 }
 
 }  // extern "C"

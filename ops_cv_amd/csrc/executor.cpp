@@ -82,6 +82,11 @@ aclnnStatus run_executor(void* workspace, uint64_t workspace_size, aclOpExecutor
             return ACLNN_ERR_PARAM_INVALID;
         }
     }
+    return execute_plan(workspace, ex, stream, api);
+}
+
+aclnnStatus execute_plan(void* workspace, const aclOpExecutor* ex, aclrtStream stream, const char* api)
+{
     if (ex->kind == OpKind::Nop) {
         return ACLNN_SUCCESS;
     }

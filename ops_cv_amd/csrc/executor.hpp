@@ -1,6 +1,8 @@
 // Shared pieces of the two-phase API: planning of view packing and the second-phase runner.
 #pragma once
 
+#include <hip/hip_runtime_api.h>
+
 #include <memory>
 
 #include "acl_types.hpp"
@@ -24,5 +26,14 @@ inline void* resolve(const PlannedPtr& p, void* workspace)
 // launches the operator, scatters the packed output, frees the executor (always, also on failure).
 aclnnStatus run_executor(void* workspace, uint64_t workspace_size, aclOpExecutor* ex, aclrtStream stream,
                          OpKind expected, const char* api);
+
+// The work of the second phase for a planned executor that stays the caller's (nothing is freed): gathers packed
+// inputs into `workspace`, launches the operator, scatters the packed output.  `workspace` must hold
+// ex->workspace_bytes bytes.
+aclnnStatus execute_plan(void* workspace, const aclOpExecutor* ex, aclrtStream stream, const char* api);
+
+// File-scope device array that stands in for the caller's workspace in the entry points that must not allocate
+// (static_scratch.hip): address of this device's copy and its size in bytes.
+hipError_t static_scratch(void** ptr, uint64_t* bytes);
 
 }  // namespace opscv
