@@ -163,6 +163,11 @@ aclnnStatus plan_grid_sampler2d(const aclTensor* input, const aclTensor* grid, i
         ex->out0 = plan_view(ex, out, esz, true);
     }
     ex->in1 = plan_view(ex, grid, esz, false);
+    // what is known of the operands' addresses already now (a workspace slice is 256-byte aligned, like null): the
+    // kernel choice depends on their alignment, and opscvExecutorVariant reports it from this plan
+    a.x = ex->in0.in_workspace ? nullptr : ex->in0.direct;
+    a.grid = ex->in1.in_workspace ? nullptr : ex->in1.direct;
+    a.y = ex->out0.in_workspace ? nullptr : ex->out0.direct;
     return ACLNN_SUCCESS;
 }
 

@@ -74,6 +74,11 @@ inline bool gs_shapes_ok(const GridSamplerArgs& a)
 hipError_t run_gs2d_lds(const GridSamplerArgs& a, hipStream_t stream, bool* handled);
 const char* gs2d_lds_variant_name(const GridSamplerArgs& a);
 
+// Pair-layout LDS variant (gs2d_pair.hip): bilinear, 16-bit elements, several output pixels per input pixel; same
+// convention as run_gs2d_lds.
+hipError_t run_gs2d_pair(const GridSamplerArgs& a, hipStream_t stream, bool* handled);
+const char* gs2d_pair_variant_name(const GridSamplerArgs& a);
+
 // Channels-last variant (gs2d_nhwc.hip): a.x is (N,Hin,Win,C), a.y is (N,Hout,Wout,C).
 hipError_t run_gs2d_nhwc(const GridSamplerArgs& a, hipStream_t stream);
 

@@ -357,11 +357,17 @@ struct BicubicTapsLauncher {
 }  // namespace
 
 namespace {
-// OPSCV_GS_VARIANT=direct forces the direct kernel (benchmark knob)
+// OPSCV_GS_VARIANT=direct forces the direct kernel, OPSCV_GS_VARIANT=ring keeps the pair-layout variant out
+// (benchmark and test knobs)
 bool force_direct()
 {
     const char* v = getenv("OPSCV_GS_VARIANT");
     return v != nullptr && v[0] == 'd';
+}
+bool force_ring()
+{
+    const char* v = getenv("OPSCV_GS_VARIANT");
+    return v != nullptr && v[0] == 'r';
 }
 }  // namespace
 
@@ -371,7 +377,10 @@ const char* grid_sampler2d_variant(const GridSamplerArgs& a)
         return "nhwc";
     }
     if (!force_direct()) {
-        const char* n = gs2d_lds_variant_name(a);
+        const char* n = force_ring() ? nullptr : gs2d_pair_variant_name(a);
+        if (n == nullptr) {
+            n = gs2d_lds_variant_name(a);
+        }
         if (n != nullptr) {
             return n;
         }
@@ -395,7 +404,11 @@ hipError_t launch_grid_sampler2d(const GridSamplerArgs& a, hipStream_t stream)
     }
     if (!force_direct()) {
         bool handled = false;
-        hipError_t e = run_gs2d_lds(a, stream, &handled);
+        hipError_t e = force_ring() ? hipSuccess : run_gs2d_pair(a, stream, &handled);
+        if (handled || e != hipSuccess) {
+            return e;
+        }
+        e = run_gs2d_lds(a, stream, &handled);
         if (handled || e != hipSuccess) {
             return e;
         }

@@ -93,6 +93,46 @@ def test_grid_sampler_large_planes(oracle, device, dtype, interp):
         _assert_same_bits(y, y_ref, "gs-large %s %s" % (dtype, INTERP[interp]))
 
 
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("pad", [0, 1, 2])
+@pytest.mark.parametrize("align", [False, True])
+def test_grid_sampler_pair_layout_variant(oracle, device, dtype, pad, align, monkeypatch):
+    """the pair-layout kernel (bilinear, 16-bit elements, several output pixels per input pixel): every staged row
+    length class, row counts off the loader's blocks of sixteen, a ragged last pixel tile, coordinates outside the
+    image on every side and non-finite ones; bit for bit against the oracle and against the ring kernel"""
+    import torch
+    from ops_cv_amd import aclnn
+    rng = np.random.default_rng(1700 + pad * 10 + int(align))
+    for (N, C, H, W, Ho, Wo) in [(2, 9, 40, 32, 97, 98), (1, 16, 64, 64, 150, 152), (2, 8, 21, 96, 90, 91 * 2),
+                                 (1, 12, 128, 128, 250, 254), (1, 3, 5, 128, 64, 66)]:
+        x32 = rng.standard_normal((N, C, H, W)).astype(np.float32)
+        x32[0, 0, 0, :] = 3.0e4  # large values on the image border: a tap wrongly taken from outside would show
+        g32 = rng.uniform(-1.4, 1.4, (N, Ho, Wo, 2)).astype(np.float32)
+        sv = I.special_grid_values()
+        k = min(sv.size, Wo)
+        g32[0, 0, :k, 0] = sv[:k]
+        g32[0, 1, :k, 1] = sv[:k]
+        x, g = I.cast_np(x32, dtype), I.cast_np(g32, dtype)
+        xt, gt = I.to_torch(x, dtype, device), I.to_torch(g, dtype, device)
+        out = torch.empty((N, C, Ho, Wo), dtype=xt.dtype, device=device)
+        hs = [aclnn.tensor_handle(t) for t in (xt, gt, out)]
+        st, _, ex = aclnn.get_workspace_size_grid_sampler2d(hs[0], hs[1], 0, pad, align, hs[2])
+        assert st == 0
+        assert aclnn.executor_variant(ex).startswith("lds_pair_w"), aclnn.executor_variant(ex)
+        aclnn.destroy_executor(ex)
+        for h in hs:
+            aclnn.destroy_tensor(h)
+        y_ref = oracle.grid_sampler2d(x, g, 0, pad, align, dtype=I.oracle_code(dtype))
+        y = I.from_torch(aclnn.grid_sampler2d(xt, gt, 0, pad, align, out=out), dtype)
+        what = "gs-pair %s %s align=%s %s" % (dtype, PAD[pad], align, (N, C, H, W, Ho, Wo))
+        _check(y, y_ref, dtype, 0, what)
+        _assert_same_bits(y, y_ref, what)
+        monkeypatch.setenv("OPSCV_GS_VARIANT", "ring")
+        y_ring = I.from_torch(aclnn.grid_sampler2d(xt, gt, 0, pad, align), dtype)
+        monkeypatch.delenv("OPSCV_GS_VARIANT")
+        _assert_same_bits(y_ring, y_ref, what + " (ring kernel)")
+
+
 @pytest.mark.parametrize("dtype", I.DTYPES)
 @pytest.mark.parametrize("interp", [0, 1, 2])
 @pytest.mark.parametrize("pad", [0, 1, 2])
