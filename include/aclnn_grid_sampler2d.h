@@ -12,6 +12,17 @@
  *   shapes            : input (N,C,Hin,Win), grid (N,Hout,Wout,2), out (N,C,Hout,Wout); formats are ignored
  *   views             : arbitrary strides/offsets are honoured (packed through the workspace)
  * Validation order and status codes follow aclnn_grid_sampler2d.cpp:159-175.
+ *
+ * Which of the reference's kernels the arithmetic follows: image/grid_sampler2_d/op_kernel/arch35/
+ * grid_sampler2_d_simt.h (one fused multiply-add in the unnormalisation, non-finite source coordinates give NaN in
+ * every channel for bilinear and bicubic, zero for nearest).  On its newest part the reference's own
+ * aclnnGridSampler2D launches a different kernel for bilinear NCHW tensors (aclnn_grid_sampler2d.cpp:321-324 ->
+ * image/grid_sample/op_kernel/arch35/grid_sampler_2d_bilinear_smit.h), which agrees with the one followed here within
+ * the bilinear tolerance (1e-5 fp32, 1e-3 relative 16-bit) on finite grids but not beyond it in one case: a NaN or
+ * infinite grid value under zeros padding gives 0 there (grid_sampler_bilinear_smit_common.h:67-90 turns every
+ * non-finite coordinate into an out-of-range one) and NaN here.  It also unnormalises as ((g + 1) * size - 1) / 2,
+ * which can pick the neighbouring pair of corner pixels for coordinates within an ulp of a pixel centre (results stay
+ * within tolerance).
  */
 #ifndef OPSCV_ACLNN_GRID_SAMPLER2D_H_
 #define OPSCV_ACLNN_GRID_SAMPLER2D_H_

@@ -11,6 +11,13 @@
  *   outputSize  : {Hout, Wout}, must equal out's spatial sizes
  *   scalesH/W   : user multipliers (>= 0); 0 derives the ratio from the sizes.  Ignored when alignCorners.
  * Validation order and status codes follow aclnn_upsample_bilinear_2d.cpp:170-195 (NULL self/out -> 561103).
+ *
+ * The reference's kernel for its older parts (two matrix products with banded coefficient matrices,
+ * image/upsample_bilinear2d/op_kernel/upsample_bilinear2d_kernel.h:284-370, index rule
+ * upsample_bilinear2d_common.h:37-51) takes the same taps and weights, except that its second tap is the next pixel
+ * also at integer source coordinates, where the rule followed here blends the pixel with itself.  The two agree
+ * on finite data; next to an infinite or NaN pixel the matrix products turn 0 * inf into NaN where this
+ * implementation returns the pixel.
  */
 #ifndef OPSCV_ACLNN_UPSAMPLE_BILINEAR_2D_H_
 #define OPSCV_ACLNN_UPSAMPLE_BILINEAR_2D_H_

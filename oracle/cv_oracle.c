@@ -49,6 +49,12 @@
  *                                  with and without the chunk shift of several items per core.  Bit-level parity
  *                                  with the reference is "parity unpinned" for the reasons given for the 2-D
  *                                  backward; the accumulation order restated is that of its deterministic mode
+ *   oracle_grid_sampler2d_arch35, oracle_upsample_a2_axis_taps, oracle_upsample_bilinear2d_a2 : restatements of two
+ *                                  neighbouring implementations in the reference that no HIP kernel follows; kept
+ *                                  to show where they leave the mirrored kernels.  Pinned by closed forms (taps and
+ *                                  weights at hand-computed coordinates, zero output for non-finite grid values,
+ *                                  x2 upscale tap table) and by agreement with the mirrored oracle within tolerance
+ *                                  on finite data
  *   oracle_resize_scale          : float bit patterns held by the reference's tiling UT
  *                                  (image/resize_bilinear_v2/tests/ut/op_host/arch35/test_resize_bilinear_v2_tiling.cpp)
  */
@@ -1545,6 +1551,137 @@ int oracle_grid_sampler3d_backward(const void* gout, const void* x, const void* 
                         store_from_float(dgrid, dtype, o + a, (interp == 1 || C == 0) ? 0.0f : mult[a][t] * gi[a][t]);
                     }
                 }
+            }
+        }
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------------------------------
+ * Two neighbouring implementations of the same operators in the reference, restated only to show where their
+ * results leave those of the kernels this library mirrors (tests/test_oracle.py); no HIP kernel follows them.
+ * ---------------------------------------------------------------------------------------- */
+
+/* The 2-D bilinear kernel of the reference's GridSample operator, which is what its aclnnGridSampler2D launches on
+ * its newest part (aclnn_grid_sampler2d.cpp:321-324):
+ *   image/grid_sample/op_kernel/arch35/grid_sampler_2d_bilinear_smit.h:56-153 and
+ *   image/grid_sample/op_kernel/arch35/grid_sampler_bilinear_smit_common.h:36-90.
+ * It differs from grid_sampler2_d_simt.h (the source mirrored by oracle_grid_sampler2d) in four places: the
+ * unnormalisation is ((g + 1) * size - 1) / 2 instead of one fused multiply-add; reflection uses fmodf and the parity
+ * of the quotient; a non-finite coordinate becomes -100 also for bilinear, so that the sample lies outside and the
+ * output is 0 where the mirrored kernel writes NaN to every channel; and the weights are (1 - dh) * (1 - dw) with
+ * dh = y - floor(y), a tap outside contributing value 0 times its weight. */
+int oracle_grid_sampler2d_arch35(const void* x, const void* grid, void* y, int dtype, int64_t N, int64_t C,
+                                 int64_t Hin, int64_t Win, int64_t Hout, int64_t Wout, int padding_mode,
+                                 int align_corners)
+{
+    if (dtype < 0 || dtype > 2 || Hin <= 0 || Win <= 0 || padding_mode < 0 || padding_mode > 2) {
+        return -1;
+    }
+    for (int64_t n = 0; n < N; n++) {
+        for (int64_t h = 0; h < Hout; h++) {
+            for (int64_t w = 0; w < Wout; w++) {
+                const int64_t goff = ((n * Hout + h) * Wout + w) * 2;
+                float gw = load_as_float(grid, dtype, goff);
+                float gh = load_as_float(grid, dtype, goff + 1);
+                gh = oracle_gs3d_unnormalize(gh, (int32_t)Hin, align_corners);
+                gw = oracle_gs3d_unnormalize(gw, (int32_t)Win, align_corners);
+                gw = oracle_gs3d_clip(gw, (int32_t)Win, padding_mode, align_corners);
+                gh = oracle_gs3d_clip(gh, (int32_t)Hin, padding_mode, align_corners);
+                const float hf = floorf(gh), wf = floorf(gw);
+                const float dh = gh - hf, dw = gw - wf;
+                const int64_t h0 = gs3_index(hf), w0 = gs3_index(wf);
+                const int64_t h1 = gs3_index(hf + 1), w1 = gs3_index(wf + 1);
+                for (int64_t c = 0; c < C; c++) {
+                    const int64_t base = (n * C + c) * Hin * Win;
+                    float v = gs3_point_value(x, dtype, base, 0, h0, w0, 1, Hin, Win);
+                    float out = v * ((1.0f - dh) * (1.0f - dw));
+                    v = gs3_point_value(x, dtype, base, 0, h0, w1, 1, Hin, Win);
+                    out += v * ((1.0f - dh) * dw);
+                    v = gs3_point_value(x, dtype, base, 0, h1, w0, 1, Hin, Win);
+                    out += v * (dh * (1.0f - dw));
+                    v = gs3_point_value(x, dtype, base, 0, h1, w1, 1, Hin, Win);
+                    out += v * (dh * dw);
+                    store_from_float(y, dtype, ((n * C + c) * Hout + h) * Wout + w, out);
+                }
+            }
+        }
+    }
+    return 0;
+}
+
+/* Index and coefficient rule of the reference's matmul upsample kernel for its older parts, one axis:
+ *   image/upsample_bilinear2d/op_kernel/upsample_bilinear2d_common.h:37-51 (getCenterValue, getLambda),
+ *   image/upsample_bilinear2d/op_kernel/upsample_bilinear2d_kernel.h:299-318 (the coefficient matrices),
+ *   scale: image/upsample_bilinear2d/op_host/upsample_bilinear2d_tiling.cpp:142-157.
+ * src = scale * d (align_corners) or max(scale * (d + 0.5) - 0.5, 0); i0 = min(int(src), len - 1);
+ * i1 = min(i0 + 1, len - 1); i0 == i1 -> coefficient 1 on i0, else l1 = clamp(src - i0, 0, 1), l0 = 1 - l1. */
+int oracle_upsample_a2_axis_taps(int64_t len_src, int64_t len_dst, int align_corners, float user_scale, int32_t* i0,
+                                 int32_t* i1, float* l0, float* l1)
+{
+    float scale;
+    if (len_dst == len_src) {
+        scale = 1.0f;
+    } else if (align_corners) {
+        scale = (len_dst > 1) ? (float)(len_src - 1) / (float)(len_dst - 1) : 0.0f;
+    } else {
+        scale = (user_scale > 0.0f) ? user_scale : (float)len_src / (float)len_dst;
+    }
+    for (int64_t d = 0; d < len_dst; d++) {
+        float src;
+        if (align_corners) {
+            src = scale * (float)d;
+        } else {
+            src = scale * ((float)d + 0.5f) - 0.5f;
+            src = (src > 0.0f) ? src : 0.0f;
+        }
+        int64_t a = (int64_t)src;
+        a = (a < len_src - 1) ? a : len_src - 1;
+        int64_t b = (a + 1 < len_src - 1) ? a + 1 : len_src - 1;
+        i0[d] = (int32_t)a;
+        i1[d] = (int32_t)b;
+        if (a == b) {
+            l0[d] = 1.0f;
+            l1[d] = 0.0f;
+        } else {
+            float lam = src - (float)a;
+            lam = (lam > 0.0f) ? lam : 0.0f;
+            lam = (lam < 1.0f) ? lam : 1.0f;
+            l1[d] = lam;
+            l0[d] = 1.0f - lam;
+        }
+    }
+    return 0;
+}
+
+/* The result of that kernel with its two taps per axis (fp32; width first, then height, as its two matrix products
+ * go: upsample_bilinear2d_kernel.h:284-370).  The products with the zero entries of its banded coefficient
+ * matrices are not modelled: they add nothing for finite data and make more outputs NaN for non-finite data. */
+int oracle_upsample_bilinear2d_a2(const float* x, float* y, int64_t N, int64_t C, int64_t Hs, int64_t Ws, int64_t Hd,
+                                  int64_t Wd, int align_corners)
+{
+    if (Hs <= 0 || Ws <= 0 || Hd <= 0 || Wd <= 0 || Hd > 65536 || Wd > 65536) {
+        return -1;
+    }
+    static int32_t h0[65536], h1[65536], w0[65536], w1[65536];
+    static float hl0[65536], hl1[65536], wl0[65536], wl1[65536];
+    oracle_upsample_a2_axis_taps(Hs, Hd, align_corners, 0.0f, h0, h1, hl0, hl1);
+    oracle_upsample_a2_axis_taps(Ws, Wd, align_corners, 0.0f, w0, w1, wl0, wl1);
+    for (int64_t pl = 0; pl < N * C; pl++) {
+        const float* xp = x + pl * Hs * Ws;
+        for (int64_t i = 0; i < Hd; i++) {
+            for (int64_t j = 0; j < Wd; j++) {
+                float top = wl0[j] * xp[h0[i] * Ws + w0[j]];
+                float bot = wl0[j] * xp[h1[i] * Ws + w0[j]];
+                if (w1[j] != w0[j]) {
+                    top += wl1[j] * xp[h0[i] * Ws + w1[j]];
+                    bot += wl1[j] * xp[h1[i] * Ws + w1[j]];
+                }
+                float out = hl0[i] * top;
+                if (h1[i] != h0[i]) {
+                    out += hl1[i] * bot;
+                }
+                y[(pl * Hd + i) * Wd + j] = out;
             }
         }
     }

@@ -175,6 +175,15 @@ int oracle_grid_sampler3d_backward(const void* gout, const void* x, const void* 
                                    int dtype, int64_t N, int64_t C, int64_t D, int64_t H, int64_t W, int64_t Do,
                                    int64_t Ho, int64_t Wo, int interp, int pad, int align);
 
+/* Neighbouring implementations in the reference (not mirrored by any HIP kernel; see cv_oracle.c) */
+int oracle_grid_sampler2d_arch35(const void* x, const void* grid, void* y, int dtype, int64_t N, int64_t C,
+                                 int64_t Hin, int64_t Win, int64_t Hout, int64_t Wout, int padding_mode,
+                                 int align_corners);
+int oracle_upsample_a2_axis_taps(int64_t len_src, int64_t len_dst, int align_corners, float user_scale, int32_t* i0,
+                                 int32_t* i1, float* l0, float* l1);
+int oracle_upsample_bilinear2d_a2(const float* x, float* y, int64_t N, int64_t C, int64_t Hs, int64_t Ws, int64_t Hd,
+                                  int64_t Wd, int align_corners);
+
 int oracle_max_threads(void);
 
 #ifdef __cplusplus

@@ -112,6 +112,12 @@ def lib():
                                                                             ctypes.c_double]
     L.oracle_max_threads.restype = ctypes.c_int
     L.oracle_max_threads.argtypes = []
+    L.oracle_grid_sampler2d_arch35.restype = ctypes.c_int
+    L.oracle_grid_sampler2d_arch35.argtypes = [vp, vp, vp, ctypes.c_int] + [i64] * 6 + [ctypes.c_int, ctypes.c_int]
+    L.oracle_upsample_a2_axis_taps.restype = ctypes.c_int
+    L.oracle_upsample_a2_axis_taps.argtypes = [i64, i64, ctypes.c_int, ctypes.c_float, vp, vp, vp, vp]
+    L.oracle_upsample_bilinear2d_a2.restype = ctypes.c_int
+    L.oracle_upsample_bilinear2d_a2.argtypes = [vp, vp] + [i64] * 6 + [ctypes.c_int]
     _lib = L
     return L
 
@@ -277,6 +283,43 @@ def upsample_bilinear2d(x, out_hw, align=False, scales_h=0.0, scales_w=0.0, dtyp
                                           float(scales_h), float(scales_w), threads)
     if rc != 0:
         raise ValueError("oracle_upsample_bilinear2d rc=%d" % rc)
+    return y
+
+
+def grid_sampler2d_arch35(x, grid, pad=0, align=False, dtype=None):
+    """bilinear 2-D sampling by the rule of the reference's GridSample operator on its newest part (a neighbouring
+    implementation that no HIP kernel follows)"""
+    x = np.ascontiguousarray(x)
+    grid = np.ascontiguousarray(grid)
+    code = _code_of(x) if dtype is None else dtype
+    N, C, H, W = x.shape
+    _, Ho, Wo, _ = grid.shape
+    y = np.empty((N, C, Ho, Wo), dtype=x.dtype)
+    rc = lib().oracle_grid_sampler2d_arch35(_ptr(x), _ptr(grid), _ptr(y), code, N, C, H, W, Ho, Wo, pad,
+                                            int(bool(align)))
+    if rc != 0:
+        raise ValueError("oracle_grid_sampler2d_arch35 rc=%d" % rc)
+    return y
+
+
+def upsample_a2_axis_taps(len_src, len_dst, align=False, scale=0.0):
+    """(i0, i1, l0, l1) of the reference's matmul upsample kernel for one axis"""
+    i0 = np.zeros(len_dst, dtype=np.int32)
+    i1 = np.zeros(len_dst, dtype=np.int32)
+    l0 = np.zeros(len_dst, dtype=np.float32)
+    l1 = np.zeros(len_dst, dtype=np.float32)
+    lib().oracle_upsample_a2_axis_taps(len_src, len_dst, int(bool(align)), float(scale), _ptr(i0), _ptr(i1), _ptr(l0),
+                                       _ptr(l1))
+    return i0, i1, l0, l1
+
+
+def upsample_bilinear2d_a2(x, out_hw, align=False):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    N, C, Hs, Ws = x.shape
+    y = np.empty((N, C, out_hw[0], out_hw[1]), dtype=np.float32)
+    rc = lib().oracle_upsample_bilinear2d_a2(_ptr(x), _ptr(y), N, C, Hs, Ws, out_hw[0], out_hw[1], int(bool(align)))
+    if rc != 0:
+        raise ValueError("oracle_upsample_bilinear2d_a2 rc=%d" % rc)
     return y
 
 

@@ -942,3 +942,88 @@ def test_upsample_backward_equal_sizes_is_a_copy(oracle):
     yh = oracle.upsample_bilinear2d_backward(np.ascontiguousarray(g.transpose(0, 2, 3, 1)), (5, 7), False,
                                              channels_last=True, scales_h=2.0, scales_w=2.0)
     assert np.array_equal(yh.view(np.uint32), g.transpose(0, 2, 3, 1).view(np.uint32))
+
+
+# ---- neighbouring implementations in the reference that the kernels do not follow: where they leave the mirrored ones ----
+
+def test_arch35_grid_sample_rule_departs_at_non_finite_coordinates_and_near_ties(oracle):
+    """image/grid_sample/op_kernel/arch35/grid_sampler_bilinear_smit_common.h:67-90 maps a non-finite coordinate to
+    -100 for bilinear as well (output 0 under every padding that leaves it non-finite), where
+    grid_sampler2_d_simt.h:485-487, the kernel this library mirrors, writes NaN to every channel; and
+    grid_sampler_2d_bilinear_smit.h:135-141 unnormalises as ((g + 1) * size - 1) / 2, not with one fused multiply-add."""
+    rng = np.random.default_rng(31)
+    x = rng.standard_normal((1, 2, 6, 10)).astype(np.float32)
+    g = np.zeros((1, 1, 4, 2), dtype=np.float32)
+    g[0, 0, 0] = (np.nan, 0.0)
+    g[0, 0, 1] = (0.0, np.inf)
+    g[0, 0, 2] = (0.25, -0.5)      # an ordinary point
+    g[0, 0, 3] = (0.6999999, 0.0)  # W = 10: the fused form gives 7.9999995, the unfused one 8.0
+    mirrored = oracle.grid_sampler2d(x, g, 0, 0, False)
+    arch35 = oracle.grid_sampler2d_arch35(x, g, 0, False)
+    assert np.isnan(mirrored[0, :, 0, 0]).all() and np.isnan(mirrored[0, :, 0, 1]).all()
+    assert (arch35[0, :, 0, 0] == 0.0).all() and (arch35[0, :, 0, 1] == 0.0).all()
+    # closed form of the ordinary point: ix = ((1.25) * 10 - 1) / 2 = 5.75, iy = ((0.5) * 6 - 1) / 2 = 1.0
+    want = 0.25 * x[0, :, 1, 5] + 0.75 * x[0, :, 1, 6]
+    np.testing.assert_allclose(arch35[0, :, 0, 2], want, rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(mirrored[0, :, 0, 2], want, rtol=1e-6, atol=1e-6)
+    # the crafted point: different corner taps, results within the bilinear tolerance of each other all the same
+    f32 = np.float32
+    fused = f32(np.fma(f32(5.0), f32(0.6999999) + f32(1.0), f32(-0.5))) if hasattr(np, "fma") else None
+    unfused = f32((f32(0.6999999) + f32(1.0)) * f32(10.0) - f32(1.0)) / f32(2.0)
+    assert unfused == f32(8.0)
+    if fused is not None:
+        assert fused < f32(8.0)
+    iy = f32((f32(1.0) * f32(6.0) - f32(1.0)) / f32(2.0))  # 2.5 either way
+    assert iy == f32(2.5)
+    np.testing.assert_allclose(arch35[0, :, 0, 3], 0.5 * x[0, :, 2, 8] + 0.5 * x[0, :, 3, 8], rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(arch35[0, :, 0, 3], mirrored[0, :, 0, 3], atol=2e-5)
+    # border and reflection padding turn a NaN coordinate into 0 in both (clip maps NaN to 0): no departure there
+    for pad in (1, 2):
+        a = oracle.grid_sampler2d_arch35(x, g[:, :, :1], pad, False)
+        m = oracle.grid_sampler2d(x, g[:, :, :1], 0, pad, False)
+        assert np.isfinite(a).all() and np.isfinite(m).all()
+    # finite random grids, every padding and alignment: the two agree within the bilinear tolerance
+    gr = rng.uniform(-1.6, 1.6, (1, 9, 11, 2)).astype(np.float32)
+    for pad in (0, 1, 2):
+        for align in (False, True):
+            np.testing.assert_allclose(oracle.grid_sampler2d_arch35(x, gr, pad, align),
+                                       oracle.grid_sampler2d(x, gr, 0, pad, align), atol=1e-5)
+
+
+def test_a2_upsample_rule_departs_next_to_non_finite_pixels(oracle):
+    """image/upsample_bilinear2d/op_kernel/upsample_bilinear2d_common.h:37-51: the second tap is i0 + 1 (capped), also
+    when the source coordinate is an integer, where resize_bilinear_v2_simt_nchw.h:118-134 (mirrored) takes ceil = floor
+    and blends the pixel with itself.  Same taps and weights otherwise, so finite data agree; an infinite neighbour
+    makes the matmul kernel's 0 * inf a NaN where the mirrored kernel returns the pixel."""
+    # tap table of the reference's example: 4 -> 8 rows with align_corners (scale 3/7), 2 -> 4 columns
+    i0, i1, l0, l1 = oracle.upsample_a2_axis_taps(4, 8, True)
+    assert list(i0) == [0, 0, 0, 1, 1, 2, 2, 3] and list(i1) == [1, 1, 1, 2, 2, 3, 3, 3]
+    np.testing.assert_allclose(l1, [0, 3 / 7, 6 / 7, 2 / 7, 5 / 7, 1 / 7, 4 / 7, 0], atol=1e-6)
+    np.testing.assert_allclose(l0 + l1, 1.0, atol=1e-7)
+    assert l0[7] == 1.0  # the last row: both taps are the last pixel, coefficient one
+    j0, j1, m = oracle.upsample_axis_taps(4, 8, True)
+    assert list(j0) == list(i0)          # first taps agree everywhere ...
+    assert j1[0] == 0 and i1[0] == 1     # ... second taps differ at integer coordinates: the pixel itself / its neighbour
+    np.testing.assert_allclose(m, l1, atol=1e-6)
+    # half-pixel x2: coordinates -0.25 -> 0, 0.25, 0.75, 1.25 ...
+    i0, i1, l0, l1 = oracle.upsample_a2_axis_taps(3, 6, False)
+    assert list(i0) == [0, 0, 0, 1, 1, 2] and list(i1) == [1, 1, 1, 2, 2, 2]
+    np.testing.assert_allclose(l1, [0, 0.25, 0.75, 0.25, 0.75, 0], atol=1e-7)
+    # finite data: equal to the mirrored oracle within rounding; the reference's example values
+    x = np.arange(8, dtype=np.float32).reshape(1, 1, 4, 2)
+    a2 = oracle.upsample_bilinear2d_a2(x, (8, 4), True)
+    np.testing.assert_allclose(a2, oracle.upsample_bilinear2d(x, (8, 4), True), atol=1e-6)
+    np.testing.assert_allclose(a2[0, 0, 0], [0, 1 / 3, 2 / 3, 1], atol=1e-6)
+    rng = np.random.default_rng(33)
+    xr = rng.standard_normal((2, 3, 7, 9)).astype(np.float32)
+    for align in (False, True):
+        np.testing.assert_allclose(oracle.upsample_bilinear2d_a2(xr, (15, 20), align),
+                                   oracle.upsample_bilinear2d(xr, (15, 20), align), atol=1e-5)
+    # the departure: an infinite pixel right of an integer source coordinate
+    xi = np.ones((1, 1, 1, 3), dtype=np.float32)
+    xi[0, 0, 0, 1] = np.inf
+    a2 = oracle.upsample_bilinear2d_a2(xi, (1, 5), True)        # columns 0, 0.5, 1, 1.5, 2
+    mir = oracle.upsample_bilinear2d(xi, (1, 5), True)
+    assert mir[0, 0, 0, 0] == 1.0 and np.isnan(a2[0, 0, 0, 0])   # 1 * 1 + 0 * inf
+    assert mir[0, 0, 0, 4] == 1.0 and a2[0, 0, 0, 4] == 1.0       # last column: one tap in both
+    assert not np.isfinite(mir[0, 0, 0, 1]) and not np.isfinite(a2[0, 0, 0, 1])  # between the pixels neither is finite
