@@ -24,19 +24,27 @@ for _p in (ROOT, os.path.join(ROOT, "tests")):
 
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs summarised under profiles/ (scaled by a
-# plain copy of known size), keyed by (workload, kernel variant); anything else reports null
+# HBM bytes per launch measured with rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs (scaled by a plain copy of known
+# size), keyed by (workload, kernel variant the figure was measured on).  The figure is reported only when the run
+# picks that same variant, together with the summary file it comes from; anything else reports null.
 MEASURED_TRAFFIC = {
-    ("C3", "lds_ring_p8208_2x4"): 69.41e6,   # profiles/gs2d_lds_ring_C3_fp16_n16_c256.md
-    ("C4", "nchw_band_lds"): 1415.4e6,       # profiles/resize_band_lds_C4_fp16_4k_upscale.md
-    ("C2", "nchw_flat_lds"): 33.08e6,        # profiles/resize_flat_lds_C2_fp32_56_to_112.md
-    ("C5", "lds_ring_p32784_1x4"): 176.4e6,  # profiles/gs2d_lds_ring_C5_bf16_random_gather.md
-    ("V1", "gs3d_bilinear"): 38.67e6,        # profiles/gs3d_V1_fp16_22x4x16x64x64.md
-    ("G3", "gs2d_grad_ordered"): 255.3e6,    # profiles/gs2d_grad_G3_fp16_n16_c256.md (both kernels of a step)
-    ("W1", "gs3d_grad_ordered"): 140.0e6,    # profiles/gs3d_grad_W1_fp16_22x4x16x64x64.md (three kernels of a step)
-    ("B4", "resize_grad_lds"): 1340.0e6,     # profiles/resize_grad_lds_B4_fp16_4k.md
-    ("R4", "nearest_nchw_lds"): 1327.3e6,    # profiles/resize_nearest_lds_R4_fp16_4k.md
+    ("C3", "lds_ring_p8208_2x4"): (69.41e6, "profiles/gs2d_lds_ring_C3_fp16_n16_c256.md"),
+    ("C4", "nchw_band_lds"): (1415.4e6, "profiles/resize_band_lds_C4_fp16_4k_upscale.md"),
+    ("C2", "nchw_flat_lds"): (33.08e6, "profiles/resize_flat_lds_C2_fp32_56_to_112.md"),
+    ("C5", "lds_pair_w128"): (None, "profiles/gs2d_lds_pair_C5_bf16_random_gather.md"),
+    ("V1", "gs3d_bilinear"): (38.67e6, "profiles/gs3d_V1_fp16_22x4x16x64x64.md"),
+    ("G3", "gs2d_grad_ordered"): (255.3e6, "profiles/gs2d_grad_G3_fp16_n16_c256.md"),
+    ("W1", "gs3d_grad_ordered"): (140.0e6, "profiles/gs3d_grad_W1_fp16_22x4x16x64x64.md"),
+    ("B4", "resize_grad_lds"): (1340.0e6, "profiles/resize_grad_lds_B4_fp16_4k.md"),
+    ("R4", "nearest_nchw_lds"): (1327.3e6, "profiles/resize_nearest_lds_R4_fp16_4k.md"),
 }
+
+# the type the arithmetic runs in, per workload: every kernel of this path converts its 16-bit elements to fp32,
+# computes in fp32 (products and sums rounded separately, as the reference does) and rounds once on the way out
+ARITHMETIC = {"C1": "f32", "C2": "f32", "C3": "f32", "C4": "f32", "C5": "f32", "L1": "f32", "V1": "f32", "V1cl": "f32",
+              "G3": "f32", "W1": "f32", "B4": "f32", "R4": "f32"}
+
+MIN_TIMED_LAUNCHES = 50  # floor for the secondary workloads, whatever --steps says for the headline
 
 # name -> description of the workloads (shapes as in the baseline configuration list)
 GS_WORKLOADS = {
@@ -96,7 +104,13 @@ def make_up_input(name, seed_base):
     return I.cast_np(x32, w["dtype"])
 
 
+_BENCH_LIB = None
+
+
 def load_bench_lib():
+    global _BENCH_LIB
+    if _BENCH_LIB is not None:
+        return _BENCH_LIB
     path = os.path.join(ROOT, "ops_cv_amd", "libopscv_bench.so")
     if not os.path.exists(path):
         raise RuntimeError("libopscv_bench.so is not built: run `python -m ops_cv_amd.build`")
@@ -105,14 +119,14 @@ def load_bench_lib():
     pd = ctypes.POINTER(ctypes.c_double)
     L.opscv_bench_grid_sampler2d.restype = ctypes.c_int
     L.opscv_bench_grid_sampler2d.argtypes = [ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.c_int,
-                                            i64, i64, ctypes.c_bool, vp, u64, ctypes.c_int, vp, pd, pd]
+                                            i64, i64, ctypes.c_bool, vp, u64, ctypes.c_int, ctypes.c_int, vp, pd, pd]
     L.opscv_bench_upsample_bilinear2d.restype = ctypes.c_int
     L.opscv_bench_upsample_bilinear2d.argtypes = [ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.c_int, vp,
                                                  ctypes.c_bool, ctypes.c_double, ctypes.c_double, vp, u64,
-                                                 ctypes.c_int, vp, pd, pd]
+                                                 ctypes.c_int, ctypes.c_int, vp, pd, pd]
     L.opscv_bench_grid_sampler2d_backward.restype = ctypes.c_int
     L.opscv_bench_grid_sampler2d_backward.argtypes = [ctypes.POINTER(vp)] * 5 + [ctypes.c_int, i64, i64, ctypes.c_bool,
-                                                                                 vp, vp, u64, ctypes.c_int, vp, pd, pd]
+                                                                                 vp, vp, u64, ctypes.c_int, ctypes.c_int, vp, pd, pd]
     L.opscv_bench_grid_sampler3d_backward.restype = ctypes.c_int
     L.opscv_bench_grid_sampler3d_backward.argtypes = L.opscv_bench_grid_sampler2d_backward.argtypes
     L.opscv_bench_grid_sampler3d.restype = ctypes.c_int
@@ -120,13 +134,16 @@ def load_bench_lib():
     L.opscv_bench_upsample_bilinear2d_backward.restype = ctypes.c_int
     L.opscv_bench_upsample_bilinear2d_backward.argtypes = [ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.c_int, vp,
                                                           vp, ctypes.c_bool, ctypes.c_double, ctypes.c_double, vp,
-                                                          u64, ctypes.c_int, vp, pd, pd]
+                                                          u64, ctypes.c_int, ctypes.c_int, vp, pd, pd]
     L.opscv_bench_resize.restype = ctypes.c_int
     L.opscv_bench_resize.argtypes = [ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.c_int, vp, ctypes.c_char_p, vp,
-                                     u64, ctypes.c_int, vp, pd, pd]
+                                     u64, ctypes.c_int, ctypes.c_int, vp, pd, pd]
+    L.opscv_bench_host_us.restype = None
+    L.opscv_bench_host_us.argtypes = [pd, pd]
     L.opscv_bench_stream.restype = ctypes.c_int
     L.opscv_bench_stream.argtypes = [ctypes.POINTER(vp), ctypes.POINTER(vp), ctypes.c_int, u64, u64, ctypes.c_int, vp,
                                      pd]
+    _BENCH_LIB = L
     return L
 
 
@@ -172,6 +189,11 @@ class Timed:
         self.kernel_us = event_ms * 1e3 / steps
         self.step_ms = wall_ms / steps
         self.stream_us = None
+        # host time per call inside GetWorkspaceSize (validation + plan) and inside the second phase (launches only:
+        # the kernels run asynchronously), measured in the same loop
+        p1, p2 = ctypes.c_double(0), ctypes.c_double(0)
+        load_bench_lib().opscv_bench_host_us(ctypes.byref(p1), ctypes.byref(p2))
+        self.host_phase1_us, self.host_phase2_us = p1.value, p2.value
 
 
 def bench_gs(name, steps, warmup, interp=None, pad=None, align=None, sets=None, check=True, channels_last=False):
@@ -213,8 +235,8 @@ def bench_gs(name, steps, warmup, interp=None, pad=None, align=None, sets=None, 
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     ev, wall = ctypes.c_double(0), ctypes.c_double(0)
 
-    def run(k):
-        rc = L.opscv_bench_grid_sampler2d(ax, ag, ay, nsets, w["interp"], w["pad"], w["align"], None, 0, k, stream,
+    def run(k, warm=0):
+        rc = L.opscv_bench_grid_sampler2d(ax, ag, ay, nsets, w["interp"], w["pad"], w["align"], None, 0, warm, k, stream,
                                           ctypes.byref(ev), ctypes.byref(wall))
         if rc != 0:
             raise RuntimeError("bench loop failed rc=%d: %s" % (rc, aclnn.load_library().aclGetRecentErrMsg()))
@@ -225,7 +247,7 @@ def bench_gs(name, steps, warmup, interp=None, pad=None, align=None, sets=None, 
     aclnn.destroy_executor(ex)
     preheat(run, warmup)
     torch.cuda.synchronize()
-    t = run(steps)
+    t = run(steps, warmup)
     torch.cuda.synchronize()
     t.stream_us = stream_reference_us(L, xs, ys, steps, stream) if check else None
     torch.cuda.synchronize()
@@ -247,7 +269,7 @@ def bench_gs(name, steps, warmup, interp=None, pad=None, align=None, sets=None, 
     desc = "%s grid_sampler2d %s x%s grid%s %s %s align_corners=%s%s" % (
         name, w["dtype"], tuple(w["x"]), (N, Ho, Wo, 2), INTERP_NAMES[w["interp"]], PAD_NAMES[w["pad"]], w["align"],
         " channels_last views" if channels_last else "")
-    return dict(workload=desc, samples=samples, alg_bytes=alg_bytes, timed=t, variant=variant, parity=parity,
+    return dict(steps=steps, workload=desc, samples=samples, alg_bytes=alg_bytes, timed=t, variant=variant, parity=parity,
                 sets=nsets, cpu=(x0, g0, w), default_modes=(interp is None and pad is None and align is None and not channels_last))
 
 
@@ -279,9 +301,9 @@ def bench_up(name, steps, warmup, sets=None, check=True):
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     ev, wall = ctypes.c_double(0), ctypes.c_double(0)
 
-    def run(k):
+    def run(k, warm=0):
         rc = L.opscv_bench_upsample_bilinear2d(ax, ay, nsets, size, w["align"], w["scales"][0], w["scales"][1], None,
-                                               0, k, stream, ctypes.byref(ev), ctypes.byref(wall))
+                                               0, warm, k, stream, ctypes.byref(ev), ctypes.byref(wall))
         if rc != 0:
             raise RuntimeError("bench loop failed rc=%d: %s" % (rc, aclnn.load_library().aclGetRecentErrMsg()))
         return Timed(ev.value, wall.value, k)
@@ -292,7 +314,7 @@ def bench_up(name, steps, warmup, sets=None, check=True):
     aclnn.destroy_executor(ex)
     preheat(run, warmup)
     torch.cuda.synchronize()
-    t = run(steps)
+    t = run(steps, warmup)
     torch.cuda.synchronize()
     t.stream_us = stream_reference_us(L, xs, ys, steps, stream) if check else None
     torch.cuda.synchronize()
@@ -316,7 +338,7 @@ def bench_up(name, steps, warmup, sets=None, check=True):
     alg_bytes = (N * C * Hs * Ws + samples) * e
     desc = "%s upsample_bilinear2d %s %s->%s align_corners=%s" % (name, w["dtype"], tuple(w["x"]),
                                                                   (N, C, Hd, Wd), w["align"])
-    return dict(workload=desc, samples=samples, alg_bytes=alg_bytes, timed=t, variant=variant, parity=parity,
+    return dict(steps=steps, workload=desc, samples=samples, alg_bytes=alg_bytes, timed=t, variant=variant, parity=parity,
                 sets=nsets, cpu=(x0, w))
 
 
@@ -324,7 +346,7 @@ def _finish(L, run, xs, ys, steps, warmup, stream):
     import torch
     preheat(run, warmup)
     torch.cuda.synchronize()
-    t = run(steps)
+    t = run(steps, warmup)
     torch.cuda.synchronize()
     t.stream_us = stream_reference_us(L, xs, ys, steps, stream)
     torch.cuda.synchronize()
@@ -380,8 +402,8 @@ def bench_gs3d(steps, warmup, sets=4, channels_last=False):
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     ev, wall = ctypes.c_double(0), ctypes.c_double(0)
 
-    def run(k):
-        rc = L.opscv_bench_grid_sampler3d(ax_, ag, ay, sets, 0, 0, False, None, 0, k, stream, ctypes.byref(ev),
+    def run(k, warm=0):
+        rc = L.opscv_bench_grid_sampler3d(ax_, ag, ay, sets, 0, 0, False, None, 0, warm, k, stream, ctypes.byref(ev),
                                           ctypes.byref(wall))
         if rc != 0:
             raise RuntimeError("bench loop failed rc=%d: %s" % (rc, aclnn.load_library().aclGetRecentErrMsg()))
@@ -401,7 +423,7 @@ def bench_gs3d(steps, warmup, sets=4, channels_last=False):
             aclnn.destroy_tensor(h)
     samples = N * C * D * H * W
     alg = (N * C * D * H * W * 2 + N * D * H * W * 3) * esize(dtype)
-    return dict(workload="V1 grid_sampler3d fp16 x(22,4,16,64,64) grid(22,16,64,64,3) bilinear zeros "
+    return dict(steps=steps, workload="V1 grid_sampler3d fp16 x(22,4,16,64,64) grid(22,16,64,64,3) bilinear zeros "
                          "align_corners=False" + (" NDHWC tensors" if channels_last else ""), samples=samples, alg_bytes=alg, timed=t, variant=variant,
                 parity=parity, sets=sets, default_modes=True)
 
@@ -449,8 +471,8 @@ def bench_gs3d_backward(steps, warmup, sets=2, mask=(True, True)):
     work = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)  # the spans of the chunks of grid points
     wptr = ctypes.c_void_p(work.data_ptr())
 
-    def run(k):
-        rc = L.opscv_bench_grid_sampler3d_backward(*arrs, sets, 0, 0, False, m, wptr, ws_bytes, k, stream,
+    def run(k, warm=0):
+        rc = L.opscv_bench_grid_sampler3d_backward(*arrs, sets, 0, 0, False, m, wptr, ws_bytes, warm, k, stream,
                                                    ctypes.byref(ev), ctypes.byref(wall))
         if rc != 0:
             raise RuntimeError("bench loop failed rc=%d: %s" % (rc, aclnn.load_library().aclGetRecentErrMsg()))
@@ -468,7 +490,7 @@ def bench_gs3d_backward(steps, warmup, sets=2, mask=(True, True)):
     e = esize(dtype)
     # gradOutput read by both gradients' kernels, input read once, grid read twice, both gradients written
     alg = (2 * N * C * D * H * W + 2 * N * C * D * H * W + 3 * N * D * H * W * 3) * e
-    return dict(workload="W1 grid_sampler3d_backward fp16 x(22,4,16,64,64) grid(22,16,64,64,3) bilinear zeros "
+    return dict(steps=steps, workload="W1 grid_sampler3d_backward fp16 x(22,4,16,64,64) grid(22,16,64,64,3) bilinear zeros "
                          "align_corners=False both gradients", samples=N * C * D * H * W, alg_bytes=alg, timed=t,
                 variant=variant, parity=parity, sets=sets, default_modes=True)
 
@@ -504,8 +526,8 @@ def bench_gs_backward(steps, warmup, sets=4, mask=(True, True)):
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     ev, wall = ctypes.c_double(0), ctypes.c_double(0)
 
-    def run(k):
-        rc = L.opscv_bench_grid_sampler2d_backward(*arrs, sets, 0, 0, False, m, None, 0, k, stream, ctypes.byref(ev),
+    def run(k, warm=0):
+        rc = L.opscv_bench_grid_sampler2d_backward(*arrs, sets, 0, 0, False, m, None, 0, warm, k, stream, ctypes.byref(ev),
                                                    ctypes.byref(wall))
         if rc != 0:
             raise RuntimeError("bench loop failed rc=%d: %s" % (rc, aclnn.load_library().aclGetRecentErrMsg()))
@@ -528,7 +550,7 @@ def bench_gs_backward(steps, warmup, sets=4, mask=(True, True)):
     e = esize(dtype)
     # gradOutput read for both gradients' kernels, input read once, grid read, both gradients written
     alg = (N * C * Ho * Wo + 2 * N * C * H * W + 2 * N * Ho * Wo * 2) * e
-    return dict(workload="G3 grid_sampler2d_backward fp16 x(16,256,64,64) grid(16,64,64,2) bilinear zeros "
+    return dict(steps=steps, workload="G3 grid_sampler2d_backward fp16 x(16,256,64,64) grid(16,64,64,2) bilinear zeros "
                          "align_corners=False both gradients", samples=N * C * Ho * Wo, alg_bytes=alg, timed=t,
                 variant=variant, parity=parity, sets=sets, default_modes=True)
 
@@ -566,8 +588,8 @@ def bench_resize_like(kind, steps, warmup, sets=2):
     if kind == "backward":
         osz, isz = aclnn.create_int_array([Hd, Wd]), aclnn.create_int_array([N, C, Hs, Ws])
 
-        def run(k):
-            rc = L.opscv_bench_upsample_bilinear2d_backward(ax, ay, sets, osz, isz, True, 2.0, 2.0, None, 0, k, stream,
+        def run(k, warm=0):
+            rc = L.opscv_bench_upsample_bilinear2d_backward(ax, ay, sets, osz, isz, True, 2.0, 2.0, None, 0, warm, k, stream,
                                                             ctypes.byref(ev), ctypes.byref(wall))
             if rc != 0:
                 raise RuntimeError("bench loop failed rc=%d: %s" % (rc, aclnn.load_library().aclGetRecentErrMsg()))
@@ -580,8 +602,8 @@ def bench_resize_like(kind, steps, warmup, sets=2):
     else:
         sc = aclnn.create_float_array([1.0, 1.0, 2.0, 2.0])
 
-        def run(k):
-            rc = L.opscv_bench_resize(ax, ay, sets, sc, b"nearest", None, 0, k, stream, ctypes.byref(ev),
+        def run(k, warm=0):
+            rc = L.opscv_bench_resize(ax, ay, sets, sc, b"nearest", None, 0, warm, k, stream, ctypes.byref(ev),
                                       ctypes.byref(wall))
             if rc != 0:
                 raise RuntimeError("bench loop failed rc=%d: %s" % (rc, aclnn.load_library().aclGetRecentErrMsg()))
@@ -600,16 +622,18 @@ def bench_resize_like(kind, steps, warmup, sets=2):
         aclnn.destroy_tensor(h)
     samples = int(np.prod(out_shape))
     alg = (int(np.prod(in_shape)) + samples) * esize(dtype)
-    return dict(workload=desc, samples=samples, alg_bytes=alg, timed=t, variant=variant, parity=parity, sets=sets,
+    return dict(steps=steps, workload=desc, samples=samples, alg_bytes=alg, timed=t, variant=variant, parity=parity, sets=sets,
                 default_modes=True)
 
 
 def roofline_of(r):
     gbs = r["alg_bytes"] / (r["timed"].kernel_us * 1e-6) / 1e9
     name = r["workload"].split(" ")[0]
-    traffic = MEASURED_TRAFFIC.get((name, r["variant"])) if r.get("default_modes", True) else None
+    traffic, source = None, None
+    if r.get("default_modes", True):
+        traffic, source = MEASURED_TRAFFIC.get((name, r["variant"]), (None, None))
     out = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-           "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": traffic,
+           "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_source": source if traffic else None,
            "kernel_us": round(r["timed"].kernel_us, 3), "algorithmic_bytes": r["alg_bytes"],
            "kernel": r["variant"]}
     su = r["timed"].stream_us
@@ -620,11 +644,16 @@ def roofline_of(r):
     return out
 
 
+def host_of(r):
+    t = r["timed"]
+    return {"phase1_get_workspace_size": round(t.host_phase1_us, 3), "phase2_launch": round(t.host_phase2_us, 3)}
+
+
 def summary_of(r):
     t = r["timed"]
     return {"workload": r["workload"], "samples_per_s": r["samples"] / (t.step_ms * 1e-3),
-            "ms_per_step": round(t.step_ms, 6), "roofline": roofline_of(r), "parity_vs_oracle": r["parity"],
-            "tensor_sets": r["sets"]}
+            "ms_per_step": round(t.step_ms, 6), "roofline": roofline_of(r), "host_us_per_call": host_of(r),
+            "parity_vs_oracle": r["parity"], "tensor_sets": r["sets"], "timed_launches": r.get("steps")}
 
 
 def cpu_baseline_gs(x0, g0, w, budget_s=12.0):
@@ -730,11 +759,12 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        "dtype": ARITHMETIC[head],
         "data": "synthetic",
         "config": {"workload": r["workload"], "tensor_sets_rotated": r["sets"], "kernel": r["variant"],
                    "parity_vs_oracle": r["parity"]},
         "roofline": roofline_of(r),
+        "host_us_per_call": host_of(r),
     }
     try:
         props = torch.cuda.get_device_properties(0)
@@ -750,36 +780,36 @@ def main():
         line["cpu_baseline"] = None
     if not args.only:
         others = {}
+        # the secondary workloads are timed over at least MIN_TIMED_LAUNCHES launches each, so that their figures
+        # are reproducible whatever --steps asks for the headline
+        ko = max(MIN_TIMED_LAUNCHES, args.steps)
         if head == "C3":
             for interp in (0, 1):
                 for pad in (0, 1, 2):
                     if interp == 0 and pad == 0:
                         continue
-                    rr = bench_gs("C3", args.steps, args.warmup, interp=interp, pad=pad)
+                    rr = bench_gs("C3", ko, args.warmup, interp=interp, pad=pad)
                     others["C3_%s_%s" % (INTERP_NAMES[interp], PAD_NAMES[pad])] = summary_of(rr)
-            rr = bench_gs("C3", args.steps, args.warmup, sets=1)
+            rr = bench_gs("C3", ko, args.warmup, sets=1)
             others["C3_bilinear_zeros_same_buffers_every_step"] = summary_of(rr)
-            others["C3_bilinear_zeros_align_corners"] = summary_of(bench_gs("C3", args.steps, args.warmup, align=True))
-            others["C3_bilinear_zeros_channels_last"] = summary_of(bench_gs("C3", args.steps, args.warmup,
+            others["C3_bilinear_zeros_align_corners"] = summary_of(bench_gs("C3", ko, args.warmup, align=True))
+            others["C3_bilinear_zeros_channels_last"] = summary_of(bench_gs("C3", ko, args.warmup,
                                                                              channels_last=True))
             # the third interpolation mode on the same tensors (not part of the headline set)
-            others["C3_bicubic_zeros"] = summary_of(bench_gs("C3", max(10, args.steps // 2), args.warmup, interp=2))
+            others["C3_bicubic_zeros"] = summary_of(bench_gs("C3", ko, args.warmup, interp=2))
         for name in ("C1", "C5"):
             if name != head:
-                others[name] = summary_of(bench_gs(name, args.steps, args.warmup))
+                others[name] = summary_of(bench_gs(name, ko, args.warmup))
         for name in ("C2", "C4"):
             if name != head:
-                k = args.steps if name == "C2" else max(5, args.steps // 4)
-                others[name] = summary_of(bench_up(name, k, max(2, args.warmup // 4)))
+                others[name] = summary_of(bench_up(name, ko, args.warmup))
         # the entry points either side of the path, on shapes of the same scale
-        others["V1_grid_sampler3d"] = summary_of(bench_gs3d(max(10, args.steps // 2), args.warmup))
-        others["V1_grid_sampler3d_ndhwc"] = summary_of(bench_gs3d(max(10, args.steps // 2), args.warmup,
-                                                                  channels_last=True))
-        k4 = max(5, args.steps // 4)
-        others["G3_grid_sampler2d_backward"] = summary_of(bench_gs_backward(k4, max(2, args.warmup // 4)))
-        others["W1_grid_sampler3d_backward"] = summary_of(bench_gs3d_backward(k4, max(2, args.warmup // 4)))
-        others["B4_upsample_backward"] = summary_of(bench_resize_like("backward", k4, max(2, args.warmup // 4)))
-        others["R4_resize_nearest"] = summary_of(bench_resize_like("nearest", k4, max(2, args.warmup // 4)))
+        others["V1_grid_sampler3d"] = summary_of(bench_gs3d(ko, args.warmup))
+        others["V1_grid_sampler3d_ndhwc"] = summary_of(bench_gs3d(ko, args.warmup, channels_last=True))
+        others["G3_grid_sampler2d_backward"] = summary_of(bench_gs_backward(ko, args.warmup))
+        others["W1_grid_sampler3d_backward"] = summary_of(bench_gs3d_backward(ko, args.warmup))
+        others["B4_upsample_backward"] = summary_of(bench_resize_like("backward", ko, args.warmup))
+        others["R4_resize_nearest"] = summary_of(bench_resize_like("nearest", ko, args.warmup))
         line["other_workloads"] = others
     print(json.dumps(line))
 

@@ -56,7 +56,15 @@ extern "C" __attribute__((visibility("default"))) int opscv_bench_stream(
     if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) {
         return -1;
     }
+    // a few untimed launches right in front of the timed region, as the operator loops do
+    for (int k = 0; k < 10; k++) {
+        const int i = (steps + k) % sets;
+        hipLaunchKernelGGL(stream_kernel, dim3((unsigned)blocks), dim3(256), 0, s, (const uint4*)srcs[i],
+                           (uint4*)dsts[i], in_chunks, out_chunks);
+    }
     if (hipStreamSynchronize(s) != hipSuccess) {
+        (void)hipEventDestroy(e0);
+        (void)hipEventDestroy(e1);
         return -1;
     }
     (void)hipEventRecord(e0, s);
@@ -67,6 +75,8 @@ extern "C" __attribute__((visibility("default"))) int opscv_bench_stream(
     }
     (void)hipEventRecord(e1, s);
     if (hipEventSynchronize(e1) != hipSuccess || hipGetLastError() != hipSuccess) {
+        (void)hipEventDestroy(e0);
+        (void)hipEventDestroy(e1);
         return -1;
     }
     float ms = 0.0f;
