@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0
 # size), keyed by (workload, kernel variant the figure was measured on).  The figure is reported only when the run
 # picks that same variant, together with the summary file it comes from; anything else reports null.
 MEASURED_TRAFFIC = {
-    ("C3", "lds_ring_p8208_2x4"): (69.41e6, "profiles/gs2d_lds_ring_C3_fp16_n16_c256.md"),
+    ("C3", "lds_ring_p8208_1x6"): (None, "profiles/gs2d_lds_ring_C3_fp16_n16_c256.md"),
     ("C4", "nchw_band_lds"): (1415.4e6, "profiles/resize_band_lds_C4_fp16_4k_upscale.md"),
     ("C2", "nchw_flat_lds"): (33.08e6, "profiles/resize_flat_lds_C2_fp32_56_to_112.md"),
     ("C5", "lds_pair_w128"): (None, "profiles/gs2d_lds_pair_C5_bf16_random_gather.md"),

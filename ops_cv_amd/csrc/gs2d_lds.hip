@@ -41,7 +41,10 @@ LdsPlan make_lds_plan(const GridSamplerArgs& a)
     // Two neighbouring pixels per lane and store for 16-bit elements: needs every output plane to start on a 4-byte
     // boundary and to hold whole pairs (fp16 N16 C256 64x64: 128-byte stores 17.1 us, 256-byte stores 16.2 us, and the
     // lanes of a wavefront then read taps two columns apart, which halves the LDS bank conflicts of a smooth grid)
-    if (esz == 2 && p.ppt >= 4 && a.interp != 2 && out_plane % 2 == 0 && reinterpret_cast<uintptr_t>(a.y) % 4 == 0) {
+    // Not for border padding: coordinates clamped to the first or last column then put both pixels of a lane on one
+    // bank, next to their neighbours' (same case, border: 18.0 us with single pixels, 21.6 us with pairs).
+    if (esz == 2 && p.ppt >= 4 && a.interp != 2 && a.pad != 1 && out_plane % 2 == 0 &&
+        reinterpret_cast<uintptr_t>(a.y) % 4 == 0) {
         p.adj = 2;
     }
     const int64_t tile = (int64_t)kThreads * p.ppt;
@@ -89,7 +92,7 @@ const char* gs2d_lds_variant_name(const GridSamplerArgs& a)
     if (!p.ok) {
         return nullptr;
     }
-    static const char* names[5] = {"lds_ring_p2064_4x4", "lds_ring_p8208_2x4", "lds_ring_p16400_1x4",
+    static const char* names[5] = {"lds_ring_p2064_4x4", "lds_ring_p8208_1x6", "lds_ring_p16400_1x4",
                                    "lds_ring_p32784_1x4", "lds_ring_p81904_1x2"};
     return names[p.cls];
 }
