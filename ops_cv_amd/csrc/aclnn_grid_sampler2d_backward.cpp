@@ -186,6 +186,10 @@ aclnnStatus aclnnGridSampler2DBackwardGetWorkspaceSize(const aclTensor* gradOutp
     ex->in0 = plan_view(ex.get(), gradOutput, esz, false);
     ex->in1 = plan_view(ex.get(), input, esz, false);
     ex->in2 = plan_view(ex.get(), grid, esz, false);
+    // known now unless packed into the workspace (whose slices are 256-byte aligned): lets the variant query see the
+    // alignment the launch will see
+    a.x = ex->in1.in_workspace ? nullptr : ex->in1.direct;
+    a.gout = ex->in0.in_workspace ? nullptr : ex->in0.direct;
     ex->want_out0 = want_dx ? 1 : 0;
     ex->want_out1 = want_dgrid ? 1 : 0;
     if (want_dx) {

@@ -93,7 +93,10 @@ const char* opscvExecutorVariant(const aclOpExecutor* executor)
         case OpKind::GridSampler2D: return grid_sampler2d_variant(executor->gs);
         case OpKind::Resize: return resize_variant(executor->rs);
         case OpKind::ResizeGrad: return executor->rg.copy ? "copy" : resize_grad_variant(executor->rg);
-        case OpKind::GridSampler2DGrad: return "gs2d_grad_ordered";
+        case OpKind::GridSampler2DGrad:
+            // the grid gradient has a variant that stages the input planes through LDS
+            return (executor->want_out1 && gs2d_grad_grid_uses_lds(executor->gsg)) ? "gs2d_grad_ordered_lds"
+                                                                                   : "gs2d_grad_ordered";
         case OpKind::GridSampler3DGrad: return "gs3d_grad_ordered";
         case OpKind::GridSampler3D:
             if (executor->gs3.channels_last) {

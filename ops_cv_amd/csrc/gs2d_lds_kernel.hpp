@@ -207,17 +207,31 @@ __device__ __forceinline__ void wait_vmcnt_imm()
 }
 
 // Run-time `n` (wave-uniform, 0..63) -> the matching immediate form; larger values cannot be expressed and wait
-// for everything.
+// for everything.  The instruction only takes a literal, so the value is found by bisection: six scalar compares.
+// (Written as a switch over the 64 values it compiled into a chain of compare-and-branch blocks walked from 63
+// downwards, several hundred cycles per wait for the small counts a ring uses.)
+template <int LO, int HI>
+__device__ __forceinline__ void wait_vmcnt_between(uint32_t n)
+{
+    if constexpr (LO == HI) {
+        wait_vmcnt_imm<LO>();
+    } else {
+        constexpr int MID = (LO + HI) / 2;
+        if (n <= (uint32_t)MID) {
+            wait_vmcnt_between<LO, MID>(n);
+        } else {
+            wait_vmcnt_between<MID + 1, HI>(n);
+        }
+    }
+}
+
 __device__ __forceinline__ void wait_vmcnt(uint32_t n)
 {
-    switch (__builtin_amdgcn_readfirstlane(n)) {
-#define OPSCV_W(N) \
-    case N: wait_vmcnt_imm<N>(); break;
-#define OPSCV_W8(B) OPSCV_W(B) OPSCV_W(B + 1) OPSCV_W(B + 2) OPSCV_W(B + 3) OPSCV_W(B + 4) OPSCV_W(B + 5) OPSCV_W(B + 6) OPSCV_W(B + 7)
-        OPSCV_W8(0) OPSCV_W8(8) OPSCV_W8(16) OPSCV_W8(24) OPSCV_W8(32) OPSCV_W8(40) OPSCV_W8(48) OPSCV_W8(56)
-#undef OPSCV_W8
-#undef OPSCV_W
-        default: wait_vmcnt_imm<0>(); break;
+    n = __builtin_amdgcn_readfirstlane(n);
+    if (n > 63u) {
+        wait_vmcnt_imm<0>();
+    } else {
+        wait_vmcnt_between<0, 63>(n);
     }
 }
 

@@ -56,6 +56,10 @@ hipError_t launch_resize(const ResizeArgs& a, hipStream_t stream);
 hipError_t launch_resize_grad(const ResizeGradArgs& a, hipStream_t stream);
 const char* resize_grad_variant(const ResizeGradArgs& a);  // which kernel launch_resize_grad picks (x may be null)
 hipError_t launch_grid_sampler2d_grad(const GridSamplerGradArgs& a, hipStream_t stream);
+// grid gradient of the 2-D sampler with the input planes staged through LDS (gs2d_grad_lds.hip); *handled is false
+// when the shape does not qualify.  gs2d_grad_grid_uses_lds: whether it would run (pointers may still be null).
+hipError_t run_gs2d_grad_grid_lds(const GridSamplerGradArgs& a, hipStream_t stream, bool* handled);
+bool gs2d_grad_grid_uses_lds(const GridSamplerGradArgs& a);
 hipError_t launch_grid_sampler3d(const GridSampler3DArgs& a, hipStream_t stream);
 hipError_t launch_grid_sampler3d_grad(const GridSampler3DGradArgs& a, hipStream_t stream);
 // 32-bit words of GridSampler3DGradArgs::chunk_ranges that make the input gradient faster; 0 when it would not help

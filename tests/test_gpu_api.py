@@ -451,6 +451,57 @@ def test_grid_sampler2d_backward(oracle, device, aclnn, dtype, interp):
                         (what, N, C, H, W, Ho, Wo, pad, align)
 
 
+@pytest.mark.parametrize("dtype", I.DTYPES)
+def test_grid_sampler2d_backward_grid_gradient_lds_variant(oracle, device, aclnn, dtype):
+    """The grid gradient with the input planes staged through LDS (enough workgroups of 256 points, 16 channels or
+    more, planes of whole 4 KiB): bit for bit the oracle's channel-ordered sums, every padding and alignment, partial last tile, batch counts
+    that are and are not a multiple of 8, corners outside the image next to non-finite gradOutput values, special
+    grid values, every ring class"""
+    torch = _torch()
+    rng = np.random.default_rng(620)
+    # planes of 4, 8, 12 and 32 KiB for 16-bit elements, twice that for fp32 (the 32 KiB shape is halved): every ring
+    # class and several copy counts per loader
+    shapes = [(8, 16, 32, 64, 64, 64), (3, 17, 64, 64, 108, 104), (8, 19, 64, 96, 64, 64),
+              (2, 16, 64 if dtype == "fp32" else 128, 128, 128, 128)]
+    for (N, C, H, W, Ho, Wo) in shapes:
+        x = I.cast_np(rng.standard_normal((N, C, H, W)).astype(np.float32), dtype)
+        g32 = rng.uniform(-1.3, 1.3, (N, Ho, Wo, 2)).astype(np.float32)
+        flat = g32.reshape(-1, 2)
+        special = np.array([np.nan, np.inf, -np.inf, 1e30, -1e30, 1.0, -1.0, 0.0], np.float32)
+        for j in range(len(special)):
+            flat[j, j % 2] = special[j]
+        g = I.cast_np(g32, dtype)
+        go32 = rng.standard_normal((N, C, Ho, Wo)).astype(np.float32)
+        # non-finite incoming gradients, some at points whose corners fall outside the image
+        gof = go32.reshape(N, C, -1)
+        outside = np.argwhere(np.abs(g32.reshape(N, -1, 2)).max(axis=2) > 1.0)
+        for j, (n_, p_) in enumerate(outside[:12]):
+            gof[n_, j % C, p_] = (np.inf, -np.inf, np.nan)[j % 3]
+        gof[0, 1, 5] = np.inf
+        go = I.cast_np(go32, dtype)
+        for pad in range(3):
+            for align in (False, True):
+                tensors = [I.to_torch(v, dtype, device) for v in (go, x, g)]
+                hs = [aclnn.tensor_handle(t) for t in tensors + [tensors[1], tensors[2]]]
+                m = aclnn.create_bool_array([True, True])
+                st, ws, ex = aclnn.get_workspace_size_grid_sampler2d_backward(hs[0], hs[1], hs[2], 0, pad, align, m,
+                                                                              hs[3], hs[4])
+                assert st == 0 and aclnn.executor_variant(ex) == "gs2d_grad_ordered_lds"
+                assert aclnn.destroy_executor(ex) == 0
+                aclnn.destroy_bool_array(m)
+                for h in hs:
+                    aclnn.destroy_tensor(h)
+                rdx, rdg = oracle.grid_sampler2d_backward(go, x, g, 0, pad, align, dtype=I.oracle_code(dtype))
+                dx, dg = aclnn.grid_sampler2d_backward(I.to_torch(go, dtype, device), I.to_torch(x, dtype, device),
+                                                       I.to_torch(g, dtype, device), 0, pad, align)
+                torch.cuda.synchronize()
+                for got, ref, what in ((I.from_torch(dx, dtype), rdx, "dx"), (I.from_torch(dg, dtype), rdg, "dgrid")):
+                    rn = np.isnan(I.as_f32(ref, dtype))
+                    assert np.array_equal(np.isnan(I.as_f32(got, dtype)), rn), (what, N, C, H, W, pad, align)
+                    assert np.array_equal(np.where(rn, 0, _bits(got, dtype)), np.where(rn, 0, _bits(ref, dtype))), \
+                        (what, N, C, H, W, Ho, Wo, pad, align)
+
+
 def test_grid_sampler2d_backward_mask_views_and_torch(oracle, device, aclnn):
     torch = _torch()
     import torch.nn.functional as F
