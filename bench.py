@@ -30,7 +30,7 @@ HBM_PEAK_GBS = 8000.0
 MEASURED_TRAFFIC = {
     ("C3", "lds_ring_p8208_1x6"): (69.36e6, "profiles/gs2d_lds_ring_C3_fp16_n16_c256.md"),
     ("C4", "nchw_band_lds"): (1415.4e6, "profiles/resize_band_lds_C4_fp16_4k_upscale.md"),
-    ("C2", "nchw_flat_lds"): (33.08e6, "profiles/resize_flat_lds_C2_fp32_56_to_112.md"),
+    ("C2", "nchw_flat_lds"): (32.43e6, "profiles/resize_flat_lds_C2_fp32_56_to_112.md"),
     ("C5", "lds_pair_w128"): (176.3e6, "profiles/gs2d_lds_pair_C5_bf16_random_gather.md"),
     ("V1", "gs3d_bilinear"): (38.67e6, "profiles/gs3d_V1_fp16_22x4x16x64x64.md"),
     ("G3", "gs2d_grad_ordered_lds"): (137.3e6, "profiles/gs2d_grad_G3_fp16_n16_c256.md"),

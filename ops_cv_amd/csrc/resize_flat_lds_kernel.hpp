@@ -24,9 +24,9 @@ struct FlatLdsParams {
     int64_t planes;
     int32_t Hs, Ws, Hd, Wd;
     float scale_h, scale_w;
-    int32_t band_rows;  // output rows per workgroup (a multiple of rg)
+    int32_t band_rows;  // output rows per workgroup
     int32_t cl;         // column lanes = ceil(Wd / V)
-    int32_t rg;         // row groups = THREADS / cl
+    int32_t rg;         // row groups at work: at most THREADS / cl
     int32_t gran;       // bytes per lane of the asynchronous copy: 16 or 4; 1: 16 in the shifted layout (kernel)
     int32_t raw_lambda;  // fraction from the unclamped source coordinate (see axis_tap)
     float neg_zero;     // -0.0f, passed in so that fma(v, w, -0) is not folded back into a multiply
@@ -55,6 +55,34 @@ __global__ __launch_bounds__(THREADS) void resize_flat_lds_kernel(const T* __res
     const uint32_t src_row_bytes = (uint32_t)p.Ws * (uint32_t)sizeof(T);
     const uint32_t stage_bytes = (uint32_t)(ys_hi - ys_lo + 1) * src_row_bytes;
 
+    // The staging copy of a plane's band: gran 1 = source rows anywhere (an odd width of 16-bit elements, a view
+    // that starts anywhere).  The band's rows are one contiguous byte range; it is copied in 16-byte units from the
+    // boundary before its first byte to the boundary after its last (the bytes outside share an aligned unit with
+    // bytes inside, so they are readable) and lands `shift` bytes into LDS.
+    const uint32_t copy_unit = (p.gran == 1) ? 16u : (uint32_t)p.gran;
+    const uint32_t chunk = 64u * copy_unit;
+    auto stage = [&](int64_t pl) -> uint32_t {
+        const char* src0 = reinterpret_cast<const char*>(x + (pl * p.Hs + ys_lo) * (int64_t)p.Ws);
+        const uint32_t shift = (p.gran == 1) ? (uint32_t)(reinterpret_cast<uintptr_t>(src0) & 15u) : 0u;
+        const uint32_t copy_bytes = (p.gran == 1) ? ((stage_bytes + shift + 15u) & ~15u) : stage_bytes;
+        src0 -= shift;
+        for (uint32_t cb = wave * chunk; cb < copy_bytes; cb += NWAVES * chunk) {
+            const uint32_t lane_off = cb + (uint32_t)lane * copy_unit;
+            if (lane_off < copy_bytes) {
+                const rs_global_cptr_t g = (rs_global_cptr_t)(src0 + lane_off);
+                const rs_lds_ptr_t l = (rs_lds_ptr_t)(lds + cb);
+                if (copy_unit == 16u) {
+                    __builtin_amdgcn_global_load_lds(g, l, 16, 0, 0);
+                } else {
+                    __builtin_amdgcn_global_load_lds(g, l, 4, 0, 0);
+                }
+            }
+        }
+        return shift;
+    };
+    // the first plane's copy is on its way while the lanes work out their column taps
+    uint32_t shift = (blockIdx.y < p.planes) ? stage(blockIdx.y) : 0u;
+
     // ---- per-lane column taps ----
     const int32_t col0 = cvec * V;
     const int32_t nvalid = (p.Wd - col0 < V) ? p.Wd - col0 : V;  // output columns of this lane inside the row
@@ -74,29 +102,10 @@ __global__ __launch_bounds__(THREADS) void resize_flat_lds_kernel(const T* __res
     const uint32_t out_plane_bytes = (uint32_t)p.Hd * out_row_bytes;
     const uint32_t col_off = (uint32_t)col0 * (uint32_t)sizeof(T);
     const float neg_zero = p.neg_zero;
-    const uint32_t copy_unit = (p.gran == 1) ? 16u : (uint32_t)p.gran;
-    const uint32_t chunk = 64u * copy_unit;
 
     for (int64_t pl = blockIdx.y; pl < p.planes; pl += gridDim.y) {
-        // gran 1: source rows anywhere (an odd width of 16-bit elements, a view that starts anywhere).  The band's
-        // rows are one contiguous byte range; it is copied in 16-byte units from the boundary before its first byte to
-        // the boundary after its last (the bytes outside share an aligned unit with bytes inside, so they are
-        // readable) and lands `shift` bytes into LDS.
-        const char* src0 = reinterpret_cast<const char*>(x + (pl * p.Hs + ys_lo) * (int64_t)p.Ws);
-        const uint32_t shift = (p.gran == 1) ? (uint32_t)(reinterpret_cast<uintptr_t>(src0) & 15u) : 0u;
-        const uint32_t copy_bytes = (p.gran == 1) ? ((stage_bytes + shift + 15u) & ~15u) : stage_bytes;
-        src0 -= shift;
-        for (uint32_t cb = wave * chunk; cb < copy_bytes; cb += NWAVES * chunk) {
-            const uint32_t lane_off = cb + (uint32_t)lane * copy_unit;
-            if (lane_off < copy_bytes) {
-                const rs_global_cptr_t g = (rs_global_cptr_t)(src0 + lane_off);
-                const rs_lds_ptr_t l = (rs_lds_ptr_t)(lds + cb);
-                if (copy_unit == 16u) {
-                    __builtin_amdgcn_global_load_lds(g, l, 16, 0, 0);
-                } else {
-                    __builtin_amdgcn_global_load_lds(g, l, 4, 0, 0);
-                }
-            }
+        if (pl != (int64_t)blockIdx.y) {
+            shift = stage(pl);
         }
         __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
