@@ -526,18 +526,21 @@ def bench_gs_backward(steps, warmup, sets=4, mask=(True, True)):
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     ev, wall = ctypes.c_double(0), ctypes.c_double(0)
 
+    st, ws_bytes, ex = aclnn.get_workspace_size_grid_sampler2d_backward(hs[0][0], hs[1][0], hs[2][0], 0, 0, False, m,
+                                                                        hs[3][0], hs[4][0])
+    assert st == 0
+    variant = aclnn.executor_variant(ex)
+    aclnn.destroy_executor(ex)
+    work = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)  # the input gradient's contribution lists
+    wptr = ctypes.c_void_p(work.data_ptr()) if ws_bytes else None
+
     def run(k, warm=0):
-        rc = L.opscv_bench_grid_sampler2d_backward(*arrs, sets, 0, 0, False, m, None, 0, warm, k, stream, ctypes.byref(ev),
-                                                   ctypes.byref(wall))
+        rc = L.opscv_bench_grid_sampler2d_backward(*arrs, sets, 0, 0, False, m, wptr, ws_bytes, warm, k, stream,
+                                                   ctypes.byref(ev), ctypes.byref(wall))
         if rc != 0:
             raise RuntimeError("bench loop failed rc=%d: %s" % (rc, aclnn.load_library().aclGetRecentErrMsg()))
         return Timed(ev.value, wall.value, k)
 
-    st, _, ex = aclnn.get_workspace_size_grid_sampler2d_backward(hs[0][0], hs[1][0], hs[2][0], 0, 0, False, m,
-                                                                 hs[3][0], hs[4][0])
-    assert st == 0
-    variant = aclnn.executor_variant(ex)
-    aclnn.destroy_executor(ex)
     t = _finish(L, run, ts[0], ts[3], steps, warmup, stream)
     rdx, rdg = oracle_lib.grid_sampler2d_backward(*first, 0, 0, False, dtype=I.oracle_code(dtype))
     parity = _parity(I.from_torch(ts[3][0], dtype), rdx, dtype)

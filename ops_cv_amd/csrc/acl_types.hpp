@@ -128,6 +128,9 @@ struct GridSamplerGradArgs {
     const void* grid = nullptr;  // (N,Hout,Wout,2)
     void* dx = nullptr;          // (N,C,Hin,Win)
     void* dgrid = nullptr;       // (N,Hout,Wout,2)
+    // optional scratch of gs2d_grad_csr_words() 32-bit words: the per-element contribution lists of the input
+    // gradient (gs2d_grad_csr.hip); null: the input gradient is scattered with elections (gs2d_grad.hip)
+    void* scratch = nullptr;
 };
 
 // Backward of the 3-D sampler.  dx / dgrid may be null (output mask): that gradient is then not computed.

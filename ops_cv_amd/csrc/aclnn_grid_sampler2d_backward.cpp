@@ -7,6 +7,7 @@
 
 #include "aclnn_grid_sampler2d_backward.h"
 #include "executor.hpp"
+#include "kernels.hpp"
 
 using namespace opscv;
 
@@ -197,6 +198,15 @@ aclnnStatus aclnnGridSampler2DBackwardGetWorkspaceSize(const aclTensor* gradOutp
     }
     if (want_dgrid) {
         ex->out1 = plan_view(ex.get(), gridGrad, esz, true);
+    }
+    if (want_dx) {
+        // scratch of the input gradient's list variant (0 words when the shape does not qualify)
+        const int64_t words = gs2d_grad_csr_words(a);
+        if (words > 0) {
+            ex->scratch.in_workspace = true;
+            ex->scratch.ws_offset = (ex->workspace_bytes + 255) / 256 * 256;
+            ex->workspace_bytes = ex->scratch.ws_offset + (uint64_t)words * 4;
+        }
     }
     *workspaceSize = ex->workspace_bytes;
     *executor = ex.release();

@@ -120,6 +120,7 @@ aclnnStatus execute_plan(void* workspace, const aclOpExecutor* ex, aclrtStream s
         a.grid = resolve(ex->in2, workspace);
         a.dx = ex->want_out0 ? resolve(ex->out0, workspace) : nullptr;
         a.dgrid = ex->want_out1 ? resolve(ex->out1, workspace) : nullptr;
+        a.scratch = ex->scratch.in_workspace ? resolve(ex->scratch, workspace) : nullptr;
         if (a.gout == nullptr || a.x == nullptr || a.grid == nullptr || (ex->want_out0 && a.dx == nullptr) ||
             (ex->want_out1 && a.dgrid == nullptr)) {
             set_error("%s: tensor data pointer is NULL", api);

@@ -95,8 +95,13 @@ const char* opscvExecutorVariant(const aclOpExecutor* executor)
         case OpKind::ResizeGrad: return executor->rg.copy ? "copy" : resize_grad_variant(executor->rg);
         case OpKind::GridSampler2DGrad:
             // the grid gradient has a variant that stages the input planes through LDS
-            return (executor->want_out1 && gs2d_grad_grid_uses_lds(executor->gsg)) ? "gs2d_grad_ordered_lds"
-                                                                                   : "gs2d_grad_ordered";
+        {
+            // input gradient: elections or lists; grid gradient: one lane per point or the LDS-ring variant
+            const bool lists = executor->want_out0 && executor->scratch.in_workspace;
+            const bool rings = executor->want_out1 && gs2d_grad_grid_uses_lds(executor->gsg);
+            return lists ? (rings ? "gs2d_grad_lists_lds" : "gs2d_grad_lists")
+                         : (rings ? "gs2d_grad_ordered_lds" : "gs2d_grad_ordered");
+        }
         case OpKind::GridSampler3DGrad: return "gs3d_grad_ordered";
         case OpKind::GridSampler3D:
             if (executor->gs3.channels_last) {

@@ -388,7 +388,14 @@ hipError_t launch_interp(const GridSamplerGradArgs& a, hipStream_t stream)
     while (p.tags < p.band_px && p.tags < kTagsMax) {
         p.tags *= 2;
     }
-    if (a.dx != nullptr) {
+    bool dx_done = false;
+    if (a.dx != nullptr && INTERP == 0) {
+        const hipError_t e = run_gs2d_grad_input_csr(a, stream, &dx_done);
+        if (e != hipSuccess) {
+            return e;
+        }
+    }
+    if (a.dx != nullptr && !dx_done) {
         const int64_t bands = (plane_px + p.band_px - 1) / p.band_px;
         // 8 bytes of planes per band element: 4 channels of a 16-bit type, 2 of fp32 (48 KB of LDS with the tags, three
         // workgroups per compute unit); fewer channels than that run one per workgroup

@@ -1,0 +1,676 @@
+// Backward of grid_sampler2d for gfx950: gradient of the input (bilinear) as a gather over precomputed lists.
+//
+// The reference's deterministic mode (image/grid_sampler2_d_grad/op_kernel/arch35/grid_sampler2_d_grad_simt_det.h:
+// 75-101) fixes the order in which contributions reach an element of the gradient: the grid points of a batch item
+// in chunks of 256, per chunk corner after corner (nw, ne, sw, se), per corner point after point, every add rounded
+// to the element type.  Which points reach which element, through which corner and with what weight, depends on
+// the grid alone -- it is the same for every channel.  So instead of scattering per channel (gs2d_grad.hip elects, per
+// corner and round, who may add to an element: about 250 workgroup barriers per group of four planes), three kernels:
+//
+//   sort (one workgroup per batch item): the points are sorted by the cell (y0, x0) of their north-west corner -- a
+//     stable block radix sort of (cell, point) keys, so the points of a cell come out in ascending order -- and the
+//     start of every cell's run is noted.  The four corner weights of every point go to scratch memory beside them.
+//   lists (one lane per element, all CUs): element (y, x) is the nw corner of the points of cell (y, x), the ne corner
+//     of cell (y, x-1), the sw corner of cell (y-1, x) and the se corner of cell (y-1, x-1).  The up to eight points of
+//     each of the four runs are read at once, keyed (chunk, corner, point) and sorted in registers by a bitonic
+//     network: the element's contributions in exactly the reference's order.  A corner outside the image never comes
+//     up: no element asks for it.  The first eight (point, weight) pairs of an element go to a fixed slot, the rest to
+//     an overflow area.  A cell with more than eight points (points piled up on one spot) takes a walk with cursors
+//     instead of the network.
+//   apply (per batch item, tile of 512 elements, block of channels): a lane owns one element and holds its first
+//     eight contributions in registers (more: in LDS); the gradOutput planes of the channels stream through LDS
+//     (asynchronous global->LDS copies by a loader wavefront, two buffers), and per channel the lane folds
+//     gradOutput[point] * weight into its sum in list order with the reference's roundings.  No atomics, no
+//     elections; one barrier per group of planes.
+//
+// The result is the same sequence of rounded operations per element as the scatter in gs2d_grad.hip, bit for bit.
+#include <hip/hip_runtime.h>
+
+#include <rocprim/block/block_radix_sort.hpp>
+
+#include "gs2d_grad_math.hpp"
+#include "gs2d_lds_kernel.hpp"
+#include "kernels.hpp"
+
+namespace opscv {
+
+namespace {
+
+constexpr int kSortThreads = 1024;
+constexpr int kMaxIpt = 8;                        // points per sorting thread: up to 8192 grid points per batch item
+constexpr int kPointBits = 13;                    // 8192 points
+constexpr uint32_t kPointMask = (1u << kPointBits) - 1u;
+constexpr int kMaxCells = 16384;                  // (H + 1) * (W + 1)
+constexpr uint32_t kNoCell = 0xFFFFFFFFu;         // key of a point none of whose corners can be inside, and of padding
+constexpr int kChunkShift = 8;                    // 256 points per chunk of the accumulation order
+constexpr int kListThreads = 256;
+constexpr int kRun = 8;                           // points of a cell the sorting network takes
+constexpr int kApplyLanes = 512;                  // elements per workgroup of the apply kernel
+constexpr int kApplyLoaders = 2;                  // loader wavefronts
+constexpr int kApplyThreads = kApplyLanes + 64 * kApplyLoaders;
+constexpr int kHeld = 8;                          // contributions of an element kept in registers
+constexpr int kApplyBufBytes = 64 * 1024;         // the ring of gradOutput planes (twice that for planes over 16 KiB)
+constexpr int kApplyNbuf = 4;                     // its slots: three groups of planes on their way while one is read
+constexpr int kApplySpill = 1024;                 // contributions beyond the held ones that a workgroup keeps in LDS
+
+struct GradParams {
+    int32_t C, H, W, Ho, Wo;
+    int32_t pad, align;
+};
+
+// scratch of one batch item, offsets in 32-bit words
+struct CsrLayout {
+    uint32_t wts;         // 4 floats per point: the corner weights nw, ne, sw, se
+    uint32_t sorted;      // kSortThreads * ipt keys (cell << kPointBits | point), sorted
+    uint32_t cell_start;  // cells + 1 positions in `sorted`
+    uint32_t count;       // H * W list lengths
+    uint32_t held;        // H * W slots of kHeld (point, weight) pairs
+    uint32_t more_start;  // H * W positions in `more` (elements with more than kHeld contributions)
+    uint32_t more_used;   // 1 word: pairs handed out in `more`
+    uint32_t more;        // up to 4 * points (point, weight) pairs
+    uint32_t item_words;
+};
+
+CsrLayout make_layout(int64_t points, int64_t plane_px, int64_t cells, int ipt)
+{
+    auto align4 = [](uint32_t v) { return (v + 3u) & ~3u; };
+    CsrLayout l;
+    l.wts = 0;
+    l.sorted = (uint32_t)(4 * points);
+    l.cell_start = l.sorted + (uint32_t)(kSortThreads * ipt);
+    l.count = align4(l.cell_start + (uint32_t)cells + 1u);
+    l.held = align4(l.count + (uint32_t)plane_px);
+    l.more_start = l.held + (uint32_t)(2 * kHeld * plane_px);
+    l.more_used = align4(l.more_start + (uint32_t)plane_px);
+    l.more = l.more_used + 4u;
+    l.item_words = align4(l.more + (uint32_t)(8 * points));
+    return l;
+}
+
+template <typename T, int IPT>
+__global__ __launch_bounds__(kSortThreads) void gs2d_grad_csr_sort_kernel(const T* __restrict__ grid,
+                                                                           uint32_t* __restrict__ ws, GradParams p,
+                                                                           CsrLayout lay)
+{
+    using sort_t = rocprim::block_radix_sort<uint32_t, kSortThreads, IPT>;
+    __shared__ typename sort_t::storage_type sort_storage;
+    extern __shared__ uint32_t sorted_lds[];  // kSortThreads * IPT keys
+    const int32_t points = p.Ho * p.Wo;
+    const int32_t cells = (p.H + 1) * (p.W + 1);
+    const uint32_t cell_bits = 32u - (uint32_t)__builtin_clz((uint32_t)cells);  // `cells` itself fits: the sentinel
+    const int t = threadIdx.x;
+    const int64_t n = blockIdx.x;
+    uint32_t* wsn = ws + (size_t)n * lay.item_words;
+    float* wts = reinterpret_cast<float*>(wsn + lay.wts);
+    uint32_t* sorted = wsn + lay.sorted;
+    uint32_t* cell_start = wsn + lay.cell_start;
+    if (t == 0) {
+        wsn[lay.more_used] = 0u;
+    }
+
+    // keys (cell << kPointBits | point); the weights of every point go to scratch
+    uint32_t keys[IPT];
+#pragma unroll
+    for (int i = 0; i < IPT; i++) {
+        const int32_t pt = t * IPT + i;
+        keys[i] = kNoCell;
+        if (pt < points) {
+            GradTaps<T, 0> tp;
+            const int64_t idx = n * points + pt;
+            decide_grad_taps<T, 0>(tp, ElemIO<T>::load(grid + 2 * idx), ElemIO<T>::load(grid + 2 * idx + 1), p.H, p.W,
+                                   p.pad, p.align);
+            *reinterpret_cast<float4*>(wts + 4 * pt) = make_float4(tp.w[0], tp.w[1], tp.w[2], tp.w[3]);
+            if (tp.x0 >= -1 && tp.x0 < p.W && tp.y0 >= -1 && tp.y0 < p.H) {
+                const uint32_t cell = (uint32_t)(tp.y0 + 1) * (uint32_t)(p.W + 1) + (uint32_t)(tp.x0 + 1);
+                keys[i] = (cell << kPointBits) | (uint32_t)pt;
+            }
+        }
+    }
+    // The keys enter in ascending point order (a thread's points, and thread after thread) and the radix sort is
+    // stable, so sorting by the cell field alone leaves the points of a cell ascending; kNoCell (all ones in the sorted
+    // bits, more than any cell) comes last.
+    sort_t().sort(keys, sort_storage, kPointBits, kPointBits + cell_bits);
+#pragma unroll
+    for (int i = 0; i < IPT; i++) {
+        sorted_lds[t * IPT + i] = keys[i];
+        sorted[t * IPT + i] = keys[i];
+    }
+    __syncthreads();
+
+    // where every cell's run starts: the first position whose key is not below the cell's (a binary search per cell,
+    // cells shared out among the threads; a thread that walked from its key's predecessor to its key would cross
+    // thousands of empty cells alone where the grid leaves part of the image untouched)
+    constexpr uint32_t total = kSortThreads * IPT;
+    for (int32_t c = t; c <= cells; c += kSortThreads) {
+        const uint32_t want = (uint32_t)c << kPointBits;
+        uint32_t lo = 0, hi = total;
+        while (lo < hi) {
+            const uint32_t mid = (lo + hi) >> 1;
+            if (sorted_lds[mid] < want) {
+                lo = mid + 1;
+            } else {
+                hi = mid;
+            }
+        }
+        cell_start[c] = lo;
+    }
+}
+
+__device__ __forceinline__ uint2 pair_of(uint32_t pt, uint32_t corner, const float* wts)
+{
+    return make_uint2(pt, __builtin_bit_cast(uint32_t, wts[4u * pt + corner]));
+}
+
+__global__ __launch_bounds__(kListThreads) void gs2d_grad_csr_lists_kernel(uint32_t* __restrict__ ws, int32_t H,
+                                                                            int32_t W, uint32_t tiles, CsrLayout lay)
+{
+    const int64_t n = blockIdx.x / tiles;
+    const int32_t e = (int32_t)(blockIdx.x % tiles) * kListThreads + (int32_t)threadIdx.x;
+    if (e >= H * W) {
+        return;
+    }
+    uint32_t* wsn = ws + (size_t)n * lay.item_words;
+    const float* wts = reinterpret_cast<const float*>(wsn + lay.wts);
+    const uint32_t* sorted = wsn + lay.sorted;
+    const uint32_t* cell_start = wsn + lay.cell_start;
+    uint2* held = reinterpret_cast<uint2*>(wsn + lay.held) + (size_t)e * kHeld;
+    uint2* more = reinterpret_cast<uint2*>(wsn + lay.more);
+
+    const uint32_t y = (uint32_t)(e / W), x = (uint32_t)(e - (int32_t)y * W);
+    const uint32_t w1 = (uint32_t)(W + 1);
+    uint32_t cid[4], cur[4], end[4];
+    cid[0] = (y + 1u) * w1 + (x + 1u);  // nw corner of the points of cell (y, x)
+    cid[1] = (y + 1u) * w1 + x;         // ne corner of cell (y, x - 1)
+    cid[2] = y * w1 + (x + 1u);         // sw corner of cell (y - 1, x)
+    cid[3] = y * w1 + x;                // se corner of cell (y - 1, x - 1)
+    uint32_t cnt = 0;
+    bool crowded = false;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        cur[k] = cell_start[cid[k]];
+        end[k] = cell_start[cid[k] + 1];
+        cnt += end[k] - cur[k];
+        crowded = crowded || end[k] - cur[k] > (uint32_t)kRun;
+    }
+    wsn[lay.count + (uint32_t)e] = cnt;
+    uint32_t more_at = 0;
+    if (cnt > (uint32_t)kHeld) {
+        // the order in which elements get their place does not matter: nothing depends on where a list lies
+        more_at = atomicAdd(&wsn[lay.more_used], cnt - (uint32_t)kHeld);
+        wsn[lay.more_start + (uint32_t)e] = more_at;
+    }
+    auto put = [&](uint32_t i, uint32_t pt, uint32_t corner) {
+        const uint2 v = pair_of(pt, corner, wts);
+        if (i < (uint32_t)kHeld) {
+            held[i] = v;
+        } else {
+            more[more_at + i - (uint32_t)kHeld] = v;
+        }
+    };
+    if (!crowded) {
+        // all candidates at once (independent loads), keyed (chunk, corner, point), sorted by a bitonic network
+        uint32_t key[4 * kRun];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const uint32_t len = end[k] - cur[k];
+#pragma unroll
+            for (int i = 0; i < kRun; i++) {
+                const bool valid = (uint32_t)i < len;
+                const uint32_t pt = sorted[valid ? cur[k] + (uint32_t)i : 0u] & kPointMask;
+                key[k * kRun + i] =
+                    valid ? (((pt >> kChunkShift) << (kPointBits + 2)) | ((uint32_t)k << kPointBits) | pt) : 0xFFFFFFFFu;
+            }
+        }
+#pragma unroll
+        for (int size = 2; size <= 4 * kRun; size *= 2) {
+#pragma unroll
+            for (int stride = size / 2; stride > 0; stride /= 2) {
+#pragma unroll
+                for (int i = 0; i < 4 * kRun; i++) {
+                    const int l = i ^ stride;
+                    if (l > i) {
+                        const uint32_t lo = key[i] < key[l] ? key[i] : key[l];
+                        const uint32_t hi = key[i] < key[l] ? key[l] : key[i];
+                        const bool ascending = (i & size) == 0;
+                        key[i] = ascending ? lo : hi;
+                        key[l] = ascending ? hi : lo;
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4 * kRun; i++) {
+            if ((uint32_t)i < cnt) {
+                put((uint32_t)i, key[i] & kPointMask, (key[i] >> kPointBits) & 3u);
+            }
+        }
+        return;
+    }
+    // a run longer than the network takes: chunk by chunk, corner by corner, with a cursor into every run
+    uint32_t i = 0;
+    for (;;) {
+        uint32_t chunk = 0xFFFFFFFFu;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            if (cur[k] < end[k]) {
+                const uint32_t c = (sorted[cur[k]] & kPointMask) >> kChunkShift;
+                chunk = c < chunk ? c : chunk;
+            }
+        }
+        if (chunk == 0xFFFFFFFFu) {
+            break;
+        }
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            while (cur[k] < end[k]) {
+                const uint32_t pt = sorted[cur[k]] & kPointMask;
+                if ((pt >> kChunkShift) != chunk) {
+                    break;
+                }
+                put(i++, pt, (uint32_t)k);
+                cur[k]++;
+            }
+        }
+    }
+}
+
+// One more contribution: gradOutput times weight rounded to fp32 and then to the element type, added to the sum with
+// a rounding to the element type (grid_sampler2_d_grad_simt_det.h:75-101).
+//   fp16: weight and gradOutput are fp16 values, their exact product has 22 significant bits and so is exact in fp32;
+//     rounding it to fp16 is the fp16 product.  The fp32 sum of two fp16 values rounded to fp16 is the fp16 sum (24
+//     bits are 2 x 11 + 2: the double rounding cannot differ).  So the sum lives in an fp16 register and a
+//     contribution is one fp16 multiply and one fp16 add, with the same results bit for bit.
+//   bf16 has no such instructions, fp32 needs no rounding steps: the generic form, the fp32 product pinned so that the
+//     compiler cannot merge product and conversion into one instruction that rounds once.
+template <typename T>
+struct Fold {
+    typedef float acc_t;
+    static __device__ __forceinline__ acc_t zero() { return 0.0f; }
+    static __device__ __forceinline__ acc_t weight(float w) { return w; }
+    static __device__ __forceinline__ acc_t add(acc_t acc, uint32_t go_bits, acc_t w)
+    {
+        return rt<T>(acc + rt<T>(as_fp32_value(w * tap_value<T>(go_bits))));
+    }
+    static __device__ __forceinline__ void store(T* p, acc_t acc) { ElemIO<T>::store(p, acc); }
+};
+template <>
+struct Fold<_Float16> {
+    typedef _Float16 acc_t;
+    static __device__ __forceinline__ acc_t zero() { return (_Float16)0.0f; }
+    static __device__ __forceinline__ acc_t weight(float w) { return (_Float16)w; }  // exact: the weight is an fp16 value
+    static __device__ __forceinline__ acc_t add(acc_t acc, uint32_t go_bits, acc_t w)
+    {
+        const _Float16 val = w * __builtin_bit_cast(_Float16, (uint16_t)go_bits);
+        return acc + val;
+    }
+    static __device__ __forceinline__ void store(_Float16* p, acc_t acc) { *p = acc; }
+};
+
+template <typename T, int CB>
+__global__ __launch_bounds__(kApplyThreads) void gs2d_grad_csr_apply_kernel(
+    const T* __restrict__ gout, T* __restrict__ dx, const uint32_t* __restrict__ ws, GradParams p, CsrLayout lay,
+    uint32_t tiles, uint32_t cblocks, int32_t chans_per_block, int32_t xcd_swizzle)
+{
+    typedef Fold<T> F;
+    typedef typename F::acc_t acc_t;
+    extern __shared__ uint4 smem_raw[];
+    char* lds = reinterpret_cast<char*>(smem_raw);
+    __shared__ uint32_t spill_used;
+    const int tid = threadIdx.x;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane((uint32_t)tid >> 6);
+    const int32_t points = p.Ho * p.Wo;
+    const int32_t plane_px = p.H * p.W;
+    const uint32_t row_bytes = (uint32_t)points * (uint32_t)sizeof(T);  // one gradOutput plane
+    const uint32_t buf_bytes = (uint32_t)CB * row_bytes;
+    uint2* spill = reinterpret_cast<uint2*>(lds + (uint32_t)kApplyNbuf * buf_bytes);  // behind the ring
+
+    // all element tiles of one (batch item, channel block) on one XCD: they stream the same gradOutput planes
+    uint32_t group, tile;
+    if (xcd_swizzle) {
+        const uint32_t xcd = blockIdx.x & 7u, i = blockIdx.x >> 3;
+        group = (i / tiles) * 8u + xcd;
+        tile = i % tiles;
+    } else {
+        group = blockIdx.x / tiles;
+        tile = blockIdx.x % tiles;
+    }
+    const uint32_t cb = group % cblocks;
+    const int64_t n = group / cblocks;
+    const int32_t c_begin = (int32_t)cb * chans_per_block;
+    const int32_t c_end = (c_begin + chans_per_block < p.C) ? c_begin + chans_per_block : p.C;
+    const int32_t nchan = c_end - c_begin;
+    const int32_t steps = (nchan + CB - 1) / CB;
+    const T* go_n = gout + (n * p.C + c_begin) * (int64_t)points;
+    if (tid == 0) {
+        spill_used = 0u;
+    }
+
+    if (wave >= (uint32_t)(kApplyLanes / 64)) {
+        // ------------------------------------------------ loader wavefronts ------------------------------------
+        // A ring of kApplyNbuf slots: with two, a group of planes was asked for when the one before it had landed, and
+        // every step waited out a memory latency.  The copy loop is kept to a few instructions per KiB (a pointer that
+        // advances, no bounds test except for a last partial KiB): one wavefront issuing a general copy routine
+        // moved 16 KiB per microsecond, and the steps waited for that (43 us on fp16 N16 C256 64x64, where the
+        // arithmetic needs a quarter).
+        const uint32_t lwave = wave - (uint32_t)(kApplyLanes / 64);
+        const uint32_t lane = (uint32_t)tid & 63u;
+        auto bytes_of = [&](int32_t s) -> uint32_t {
+            const int32_t left = nchan - s * CB;
+            return (uint32_t)(left < CB ? left : CB) * row_bytes;  // the planes are neighbours in memory
+        };
+        // copy instructions this wavefront issues for a group of `bytes`: every kApplyLoaders-th KiB, the last one partial
+        auto copies_of = [&](uint32_t bytes) -> uint32_t {
+            const uint32_t kib = (bytes + 1023u) >> 10;
+            return (kib > lwave) ? (kib - lwave + kApplyLoaders - 1) / kApplyLoaders : 0u;
+        };
+        const uint32_t copies_full = copies_of(buf_bytes);
+        const char* src_lane = reinterpret_cast<const char*>(go_n) + lwave * 1024u + lane * 16u;
+        int32_t issued = 0;
+        auto issue_next = [&]() {
+            const uint32_t bytes = bytes_of(issued);
+            const char* src = src_lane + (size_t)issued * buf_bytes;
+            char* dst = lds + (uint32_t)(issued % kApplyNbuf) * buf_bytes + lwave * 1024u;
+            const uint32_t whole = bytes >> 10;
+            uint32_t j = lwave;
+            for (; j < whole; j += kApplyLoaders) {
+                __builtin_amdgcn_global_load_lds((global_cptr_t)src, (lds_ptr_t)dst, 16, 0, 0);
+                src += kApplyLoaders * 1024;
+                dst += kApplyLoaders * 1024;
+            }
+            if ((bytes & 1023u) != 0u && j == whole) {
+                if (lane * 16u < (bytes & 1023u)) {
+                    __builtin_amdgcn_global_load_lds((global_cptr_t)src, (lds_ptr_t)dst, 16, 0, 0);
+                }
+            }
+            issued++;
+        };
+        while (issued < kApplyNbuf - 1 && issued < steps) {
+            issue_next();
+        }
+        lds_barrier();  // the element lanes' set-up barrier
+        for (int32_t s = 0; s < steps; s++) {
+            // the planes of step s have landed when at most the copies of the groups after it are out
+            uint32_t later = 0;
+            for (int32_t q = s + 1; q < issued; q++) {
+                later += (q == steps - 1) ? copies_of(bytes_of(q)) : copies_full;
+            }
+            wait_vmcnt(later);
+            lds_barrier();  // ... and the slot of step s - 1 has been read for the last time
+            if (issued < steps) {
+                issue_next();
+            }
+        }
+        return;
+    }
+
+    // ---------------------------------------------------- element lanes ----------------------------------------
+    const uint32_t* wsn = ws + (size_t)n * lay.item_words;
+    const int32_t e = (int32_t)tile * kApplyLanes + tid;
+    const bool live = e < plane_px;
+    const uint32_t cnt = live ? wsn[lay.count + (uint32_t)e] : 0u;
+    uint32_t hoff[kHeld];  // byte offset of the point inside a gradOutput plane
+    acc_t hw[kHeld];
+    {
+        const uint4* slot = reinterpret_cast<const uint4*>(wsn + lay.held) + (size_t)(live ? e : 0) * (kHeld / 2);
+        uint4 raw[kHeld / 2];
+#pragma unroll
+        for (int k = 0; k < kHeld / 2; k++) {
+            raw[k] = slot[k];
+        }
+#pragma unroll
+        for (int k = 0; k < kHeld / 2; k++) {
+            const bool a = (uint32_t)(2 * k) < cnt, b = (uint32_t)(2 * k + 1) < cnt;
+            hoff[2 * k] = a ? raw[k].x * (uint32_t)sizeof(T) : 0u;
+            hw[2 * k] = F::weight(a ? __builtin_bit_cast(float, raw[k].y) : 0.0f);
+            hoff[2 * k + 1] = b ? raw[k].z * (uint32_t)sizeof(T) : 0u;
+            hw[2 * k + 1] = F::weight(b ? __builtin_bit_cast(float, raw[k].w) : 0.0f);
+        }
+    }
+    __syncthreads();  // spill_used is zero
+    // contributions beyond the held ones: a place in LDS while there is room, else they stay in scratch memory
+    const uint2* rest = nullptr;  // where the lane reads them in every step
+    bool rest_in_lds = false;
+    uint32_t rest_at = 0;
+    if (cnt > (uint32_t)kHeld) {
+        const uint32_t extra = cnt - (uint32_t)kHeld;
+        const uint2* src = reinterpret_cast<const uint2*>(wsn + lay.more) + wsn[lay.more_start + (uint32_t)e];
+        rest = src;
+        rest_at = atomicAdd(&spill_used, extra);
+        if (rest_at + extra <= (uint32_t)kApplySpill) {
+            rest_in_lds = true;
+            for (uint32_t i = 0; i < extra; i++) {
+                spill[rest_at + i] = src[i];
+            }
+        }
+    }
+    // the longest held list of the wavefront decides how many rounds its lanes run
+    uint32_t kmax = cnt < (uint32_t)kHeld ? cnt : (uint32_t)kHeld;
+    uint32_t cmax = cnt;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const uint32_t other = (uint32_t)__shfl_xor((int)kmax, o);
+        kmax = other > kmax ? other : kmax;
+        const uint32_t other2 = (uint32_t)__shfl_xor((int)cmax, o);
+        cmax = other2 > cmax ? other2 : cmax;
+    }
+    kmax = __builtin_amdgcn_readfirstlane(kmax);
+    const bool any_rest = __builtin_amdgcn_readfirstlane(cmax) > (uint32_t)kHeld;
+    T* dx_e = dx + (n * p.C + c_begin) * (int64_t)plane_px + (live ? e : 0);
+    // the lists are in registers or LDS from here on: nothing below waits for memory except an overfull spill area
+    __builtin_amdgcn_s_waitcnt(0);
+
+    typedef typename std::conditional<sizeof(T) == 2, uint16_t, uint32_t>::type bits_t;
+    typedef const bits_t __attribute__((address_space(3))) * lds_bits_ptr_t;
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
+    auto go_at = [&](uint32_t off) -> uint32_t {
+        return (uint32_t)*reinterpret_cast<lds_bits_ptr_t>((uintptr_t)(lds_base + off));
+    };
+    // R rounds of one step, straight-line: all gradOutput values first (raw bits, so that nothing waits between the
+    // reads), then the sums in list order; a lane whose list is shorter keeps its sum (a select, not arithmetic: a
+    // value read for a contribution that does not exist may be anything)
+    auto rounds = [&](auto r_tag, uint32_t buf_off, acc_t* acc) {
+        constexpr int R = decltype(r_tag)::value;
+        uint32_t raw[R][CB];
+#pragma unroll
+        for (int k = 0; k < R; k++) {
+#pragma unroll
+            for (int j = 0; j < CB; j++) {
+                raw[k][j] = go_at(buf_off + (uint32_t)j * row_bytes + hoff[k]);
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < R; k++) {
+            const bool mine = (uint32_t)k < cnt;
+#pragma unroll
+            for (int j = 0; j < CB; j++) {
+                const acc_t next = F::add(acc[j], raw[k][j], hw[k]);
+                acc[j] = mine ? next : acc[j];
+            }
+        }
+    };
+
+    for (int32_t s = 0; s < steps; s++) {
+        lds_barrier();  // the planes of step s have landed
+        const uint32_t buf_off = (uint32_t)(s % kApplyNbuf) * buf_bytes;
+        acc_t acc[CB];
+#pragma unroll
+        for (int j = 0; j < CB; j++) {
+            acc[j] = F::zero();
+        }
+        switch (kmax) {
+            case 0: break;
+            case 1: rounds(std::integral_constant<int, 1>{}, buf_off, acc); break;
+            case 2: rounds(std::integral_constant<int, 2>{}, buf_off, acc); break;
+            case 3: rounds(std::integral_constant<int, 3>{}, buf_off, acc); break;
+            case 4: rounds(std::integral_constant<int, 4>{}, buf_off, acc); break;
+            case 5: rounds(std::integral_constant<int, 5>{}, buf_off, acc); break;
+            case 6: rounds(std::integral_constant<int, 6>{}, buf_off, acc); break;
+            case 7: rounds(std::integral_constant<int, 7>{}, buf_off, acc); break;
+            default: rounds(std::integral_constant<int, 8>{}, buf_off, acc); break;
+        }
+        if (any_rest && cnt > (uint32_t)kHeld) {
+            for (uint32_t i = 0; i < cnt - (uint32_t)kHeld; i++) {
+                const uint2 v = rest_in_lds ? spill[rest_at + i] : rest[i];
+                const acc_t w = F::weight(__builtin_bit_cast(float, v.y));
+#pragma unroll
+                for (int j = 0; j < CB; j++) {
+                    acc[j] = F::add(acc[j], go_at(buf_off + (uint32_t)j * row_bytes + v.x * (uint32_t)sizeof(T)), w);
+                }
+            }
+        }
+        if (live) {
+#pragma unroll
+            for (int j = 0; j < CB; j++) {
+                if (s * CB + j < nchan) {
+                    F::store(dx_e + (int64_t)(s * CB + j) * plane_px, acc[j]);
+                }
+            }
+        }
+    }
+}
+
+struct CsrPlan {
+    bool ok = false;
+    int ipt = 1;
+    int cb = 1;
+    uint32_t tiles = 0, cblocks = 0;
+    int32_t chans_per_block = 0;
+    int xcd_swizzle = 0;
+    CsrLayout lay;
+};
+
+CsrPlan make_plan(const GridSamplerGradArgs& a)
+{
+    CsrPlan pl;
+    const int64_t esz = elem_size(a.elem);
+    const int64_t points = a.Hout * a.Wout, plane_px = a.Hin * a.Win;
+    const int64_t cells = (a.Hin + 1) * (a.Win + 1);
+    // what the kernels assume: the sort holds an item's points in one workgroup, a gradOutput plane is whole 16-byte
+    // units on 16-byte boundaries and fits a slot of the ring
+    if (a.interp != 0 || points > (int64_t)kSortThreads * kMaxIpt || cells > kMaxCells || (points * esz) % 16 != 0 ||
+        reinterpret_cast<uintptr_t>(a.gout) % 16 != 0 || points * esz > 2 * kApplyBufBytes / kApplyNbuf) {
+        return pl;
+    }
+    // worth three extra kernels only with channels to share the lists among
+    if (a.C < 8 || a.N * a.C > INT32_MAX) {
+        return pl;
+    }
+    pl.ipt = 1;
+    while ((int64_t)kSortThreads * pl.ipt < points) {
+        pl.ipt *= 2;
+    }
+    pl.cb = 4;
+    while (pl.cb > 1 && (int64_t)kApplyNbuf * pl.cb * points * esz > kApplyBufBytes) {
+        pl.cb /= 2;
+    }
+    pl.tiles = (uint32_t)((plane_px + kApplyLanes - 1) / kApplyLanes);
+    // channel blocks: about two workgroups per CU, whole groups of planes each
+    const int64_t base = a.N * pl.tiles;
+    int64_t cblocks = (512 + base - 1) / base;
+    const int64_t max_cblocks = (a.C + pl.cb - 1) / pl.cb;
+    cblocks = cblocks > max_cblocks ? max_cblocks : cblocks;
+    int64_t cpb = (a.C + cblocks - 1) / cblocks;
+    cpb = (cpb + pl.cb - 1) / pl.cb * pl.cb;
+    cblocks = (a.C + cpb - 1) / cpb;
+    const int64_t list_tiles = (plane_px + kListThreads - 1) / kListThreads;
+    if (base * cblocks > INT32_MAX || a.N * list_tiles > INT32_MAX) {
+        return pl;
+    }
+    pl.chans_per_block = (int32_t)cpb;
+    pl.cblocks = (uint32_t)cblocks;
+    pl.xcd_swizzle = ((a.N * cblocks) % 8 == 0) ? 1 : 0;
+    pl.lay = make_layout(points, plane_px, cells, pl.ipt);
+    pl.ok = true;
+    return pl;
+}
+
+template <typename T, int IPT>
+hipError_t launch_sort(const GridSamplerGradArgs& a, const CsrPlan& pl, const GradParams& p, hipStream_t stream)
+{
+    hipLaunchKernelGGL((gs2d_grad_csr_sort_kernel<T, IPT>), dim3((unsigned)a.N), dim3(kSortThreads),
+                       kSortThreads * IPT * 4, stream, (const T*)a.grid, (uint32_t*)a.scratch, p, pl.lay);
+    return hipGetLastError();
+}
+
+template <typename T, int CB>
+hipError_t launch_apply(const GridSamplerGradArgs& a, const CsrPlan& pl, const GradParams& p, hipStream_t stream)
+{
+    auto kernel = gs2d_grad_csr_apply_kernel<T, CB>;
+    constexpr int kLdsMax = 2 * kApplyBufBytes + kApplySpill * 8;
+    static std::atomic<uint32_t> lds_allowed{0};
+    const hipError_t ea = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kLdsMax, lds_allowed);
+    if (ea != hipSuccess) {
+        return ea;
+    }
+    const uint32_t blocks = (uint32_t)(a.N * pl.tiles * pl.cblocks);
+    const int lds_bytes = kApplyNbuf * CB * (int)(a.Hout * a.Wout) * (int)sizeof(T) + kApplySpill * 8;
+    hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kApplyThreads), lds_bytes, stream, (const T*)a.gout, (T*)a.dx,
+                       (const uint32_t*)a.scratch, p, pl.lay, pl.tiles, pl.cblocks, pl.chans_per_block, pl.xcd_swizzle);
+    return hipGetLastError();
+}
+
+template <typename T>
+hipError_t run_typed(const GridSamplerGradArgs& a, const CsrPlan& pl, hipStream_t stream)
+{
+    GradParams p{};
+    p.C = (int32_t)a.C;
+    p.H = (int32_t)a.Hin;
+    p.W = (int32_t)a.Win;
+    p.Ho = (int32_t)a.Hout;
+    p.Wo = (int32_t)a.Wout;
+    p.pad = a.pad;
+    p.align = a.align;
+    hipError_t e = hipErrorInvalidValue;
+    switch (pl.ipt) {
+        case 1: e = launch_sort<T, 1>(a, pl, p, stream); break;
+        case 2: e = launch_sort<T, 2>(a, pl, p, stream); break;
+        case 4: e = launch_sort<T, 4>(a, pl, p, stream); break;
+        case 8: e = launch_sort<T, 8>(a, pl, p, stream); break;
+        default: break;
+    }
+    if (e != hipSuccess) {
+        return e;
+    }
+    const uint32_t list_tiles = (uint32_t)((a.Hin * a.Win + kListThreads - 1) / kListThreads);
+    hipLaunchKernelGGL(gs2d_grad_csr_lists_kernel, dim3((unsigned)(a.N * list_tiles)), dim3(kListThreads), 0, stream,
+                       (uint32_t*)a.scratch, (int32_t)a.Hin, (int32_t)a.Win, list_tiles, pl.lay);
+    e = hipGetLastError();
+    if (e != hipSuccess) {
+        return e;
+    }
+    switch (pl.cb) {
+        case 4: return launch_apply<T, 4>(a, pl, p, stream);
+        case 2: return launch_apply<T, 2>(a, pl, p, stream);
+        case 1: return launch_apply<T, 1>(a, pl, p, stream);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace
+
+int64_t gs2d_grad_csr_words(const GridSamplerGradArgs& a)
+{
+    const CsrPlan pl = make_plan(a);
+    return pl.ok ? (int64_t)pl.lay.item_words * a.N : 0;
+}
+
+hipError_t run_gs2d_grad_input_csr(const GridSamplerGradArgs& a, hipStream_t stream, bool* handled)
+{
+    *handled = false;
+    if (a.dx == nullptr || a.scratch == nullptr) {
+        return hipSuccess;
+    }
+    const CsrPlan pl = make_plan(a);
+    if (!pl.ok) {
+        return hipSuccess;
+    }
+    *handled = true;
+    switch (a.elem) {
+        case Elem::F32: return run_typed<float>(a, pl, stream);
+        case Elem::F16: return run_typed<_Float16>(a, pl, stream);
+        case Elem::BF16: return run_typed<__bf16>(a, pl, stream);
+    }
+    return hipErrorInvalidValue;
+}
+
+}  // namespace opscv

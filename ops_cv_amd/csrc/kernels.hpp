@@ -60,6 +60,10 @@ hipError_t launch_grid_sampler2d_grad(const GridSamplerGradArgs& a, hipStream_t 
 // when the shape does not qualify.  gs2d_grad_grid_uses_lds: whether it would run (pointers may still be null).
 hipError_t run_gs2d_grad_grid_lds(const GridSamplerGradArgs& a, hipStream_t stream, bool* handled);
 bool gs2d_grad_grid_uses_lds(const GridSamplerGradArgs& a);
+// input gradient of the 2-D sampler as a gather over per-element contribution lists (gs2d_grad_csr.hip): 32-bit words
+// of GridSamplerGradArgs::scratch it needs, 0 when the shape does not qualify; *handled is false when it did not run
+int64_t gs2d_grad_csr_words(const GridSamplerGradArgs& a);
+hipError_t run_gs2d_grad_input_csr(const GridSamplerGradArgs& a, hipStream_t stream, bool* handled);
 hipError_t launch_grid_sampler3d(const GridSampler3DArgs& a, hipStream_t stream);
 hipError_t launch_grid_sampler3d_grad(const GridSampler3DGradArgs& a, hipStream_t stream);
 // 32-bit words of GridSampler3DGradArgs::chunk_ranges that make the input gradient faster; 0 when it would not help

@@ -486,7 +486,10 @@ def test_grid_sampler2d_backward_grid_gradient_lds_variant(oracle, device, aclnn
                 m = aclnn.create_bool_array([True, True])
                 st, ws, ex = aclnn.get_workspace_size_grid_sampler2d_backward(hs[0], hs[1], hs[2], 0, pad, align, m,
                                                                               hs[3], hs[4])
-                assert st == 0 and aclnn.executor_variant(ex) == "gs2d_grad_ordered_lds"
+                # the input gradient takes its list variant where an item's points fit one sorting workgroup
+                lists = Ho * Wo <= 8192
+                assert st == 0 and aclnn.executor_variant(ex) == ("gs2d_grad_lists_lds" if lists
+                                                                   else "gs2d_grad_ordered_lds")
                 assert aclnn.destroy_executor(ex) == 0
                 aclnn.destroy_bool_array(m)
                 for h in hs:
@@ -500,6 +503,61 @@ def test_grid_sampler2d_backward_grid_gradient_lds_variant(oracle, device, aclnn
                     assert np.array_equal(np.isnan(I.as_f32(got, dtype)), rn), (what, N, C, H, W, pad, align)
                     assert np.array_equal(np.where(rn, 0, _bits(got, dtype)), np.where(rn, 0, _bits(ref, dtype))), \
                         (what, N, C, H, W, Ho, Wo, pad, align)
+
+
+@pytest.mark.parametrize("dtype", I.DTYPES)
+def test_grid_sampler2d_backward_input_gradient_list_variant(oracle, device, aclnn, dtype):
+    """The input gradient as a gather over per-element contribution lists (8 channels or more, up to 8192 grid
+    points per item): bit for bit the oracle's chunk / corner / point order, with points piling up on few elements
+    (lists far longer than the eight entries a lane holds), elements nobody reaches, points outside the image,
+    non-finite gradOutput next to corners outside the image, every padding and alignment, channel counts that are not
+    a multiple of the planes staged together, plane sizes that leave a partial element tile"""
+    torch = _torch()
+    rng = np.random.default_rng(630)
+    for (N, C, H, W, Ho, Wo, kind) in [(2, 9, 7, 9, 24, 24, "pile"), (3, 8, 30, 40, 64, 64, "random"),
+                                        (1, 13, 64, 64, 90, 88, "smooth"), (2, 8, 20, 20, 32, 64, "outside")]:
+        x = I.cast_np(rng.standard_normal((N, C, H, W)).astype(np.float32), dtype)
+        if kind == "pile":
+            g32 = rng.choice(np.array([-0.93, -0.31, 0.02, 0.4, 0.77], np.float32), (N, Ho, Wo, 2))
+        elif kind == "smooth":
+            ys, xs = np.meshgrid(np.linspace(-1.05, 1.05, Ho), np.linspace(-1.05, 1.05, Wo), indexing="ij")
+            g32 = np.broadcast_to(np.stack([xs * 0.9 + ys * 0.1, ys * 0.95 - xs * 0.05], -1), (N, Ho, Wo, 2))
+            g32 = np.ascontiguousarray(g32, dtype=np.float32)
+        elif kind == "outside":
+            g32 = rng.uniform(-2.5, 2.5, (N, Ho, Wo, 2)).astype(np.float32)
+        else:
+            g32 = rng.uniform(-1.2, 1.2, (N, Ho, Wo, 2)).astype(np.float32)
+        flat = g32.reshape(-1, 2)
+        special = np.array([np.nan, np.inf, -np.inf, 1e30, -1e30, 1.0, -1.0, 0.0], np.float32)
+        for j in range(len(special)):
+            flat[j, j % 2] = special[j]
+        g = I.cast_np(g32, dtype)
+        go32 = rng.standard_normal((N, C, Ho, Wo)).astype(np.float32)
+        gof = go32.reshape(N, C, -1)
+        edge = np.argwhere(np.abs(g32.reshape(N, -1, 2)).max(axis=2) > 0.97)
+        for j, (n_, p_) in enumerate(edge[:10]):
+            gof[n_, j % C, p_] = (np.inf, -np.inf, np.nan)[j % 3]
+        go = I.cast_np(go32, dtype)
+        for pad in range(3):
+            for align in (False, True):
+                tensors = [I.to_torch(v, dtype, device) for v in (go, x, g)]
+                hs = [aclnn.tensor_handle(t) for t in tensors + [tensors[1], tensors[2]]]
+                m = aclnn.create_bool_array([True, True])
+                st, ws, ex = aclnn.get_workspace_size_grid_sampler2d_backward(hs[0], hs[1], hs[2], 0, pad, align, m,
+                                                                              hs[3], hs[4])
+                assert st == 0 and ws > 0 and aclnn.executor_variant(ex).startswith("gs2d_grad_lists")
+                assert aclnn.destroy_executor(ex) == 0
+                aclnn.destroy_bool_array(m)
+                for h in hs:
+                    aclnn.destroy_tensor(h)
+                rdx, rdg = oracle.grid_sampler2d_backward(go, x, g, 0, pad, align, dtype=I.oracle_code(dtype))
+                dx, dg = aclnn.grid_sampler2d_backward(*tensors, 0, pad, align)
+                torch.cuda.synchronize()
+                for got, ref, what in ((I.from_torch(dx, dtype), rdx, "dx"), (I.from_torch(dg, dtype), rdg, "dgrid")):
+                    rn = np.isnan(I.as_f32(ref, dtype))
+                    assert np.array_equal(np.isnan(I.as_f32(got, dtype)), rn), (what, kind, pad, align)
+                    assert np.array_equal(np.where(rn, 0, _bits(got, dtype)), np.where(rn, 0, _bits(ref, dtype))), \
+                        (what, kind, N, C, H, W, Ho, Wo, pad, align)
 
 
 def test_grid_sampler2d_backward_mask_views_and_torch(oracle, device, aclnn):
