@@ -304,6 +304,15 @@ struct Fold<_Float16> {
         return acc + val;
     }
     static __device__ __forceinline__ void store(_Float16* p, acc_t acc) { *p = acc; }
+    // two channels at once: the same two operations as packed fp16 instructions (each half rounds on its own)
+    typedef _Float16 pair_t __attribute__((ext_vector_type(2)));
+    static __device__ __forceinline__ pair_t add2(pair_t acc, uint32_t go_lo, uint32_t go_hi, acc_t w)
+    {
+        const pair_t go = {__builtin_bit_cast(_Float16, (uint16_t)go_lo), __builtin_bit_cast(_Float16, (uint16_t)go_hi)};
+        const pair_t ww = {w, w};
+        const pair_t val = ww * go;
+        return acc + val;
+    }
 };
 
 template <typename T, int CB>
@@ -478,13 +487,35 @@ __global__ __launch_bounds__(kApplyThreads) void gs2d_grad_csr_apply_kernel(
                 raw[k][j] = go_at(buf_off + (uint32_t)j * row_bytes + hoff[k]);
             }
         }
+        if constexpr (std::is_same<T, _Float16>::value && CB % 2 == 0) {
+            typename F::pair_t acc2[CB / 2];
 #pragma unroll
-        for (int k = 0; k < R; k++) {
-            const bool mine = (uint32_t)k < cnt;
+            for (int j = 0; j < CB / 2; j++) {
+                acc2[j] = typename F::pair_t{acc[2 * j], acc[2 * j + 1]};
+            }
 #pragma unroll
-            for (int j = 0; j < CB; j++) {
-                const acc_t next = F::add(acc[j], raw[k][j], hw[k]);
-                acc[j] = mine ? next : acc[j];
+            for (int k = 0; k < R; k++) {
+                const bool mine = (uint32_t)k < cnt;
+#pragma unroll
+                for (int j = 0; j < CB / 2; j++) {
+                    const typename F::pair_t next = F::add2(acc2[j], raw[k][2 * j], raw[k][2 * j + 1], hw[k]);
+                    acc2[j] = mine ? next : acc2[j];
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < CB / 2; j++) {
+                acc[2 * j] = acc2[j].x;
+                acc[2 * j + 1] = acc2[j].y;
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < R; k++) {
+                const bool mine = (uint32_t)k < cnt;
+#pragma unroll
+                for (int j = 0; j < CB; j++) {
+                    const acc_t next = F::add(acc[j], raw[k][j], hw[k]);
+                    acc[j] = mine ? next : acc[j];
+                }
             }
         }
     };
