@@ -37,10 +37,10 @@ namespace opscv {
 namespace {
 
 constexpr int kSortThreads = 1024;
-constexpr int kMaxIpt = 8;                        // points per sorting thread: up to 8192 grid points per batch item
-constexpr int kPointBits = 13;                    // 8192 points
+constexpr int kMaxIpt = 16;                       // points per sorting thread: up to 16384 grid points per batch item
+constexpr int kPointBits = 14;                    // 16384 points
 constexpr uint32_t kPointMask = (1u << kPointBits) - 1u;
-constexpr int kMaxCells = 16384;                  // (H + 1) * (W + 1)
+constexpr int kMaxCells = 32768;                  // (H + 1) * (W + 1): the keys keep 32 bits
 constexpr uint32_t kNoCell = 0xFFFFFFFFu;         // key of a point none of whose corners can be inside, and of padding
 constexpr int kChunkShift = 8;                    // 256 points per chunk of the accumulation order
 constexpr int kListThreads = 256;
@@ -618,6 +618,12 @@ CsrPlan make_plan(const GridSamplerGradArgs& a)
 template <typename T, int IPT>
 hipError_t launch_sort(const GridSamplerGradArgs& a, const CsrPlan& pl, const GradParams& p, hipStream_t stream)
 {
+    static std::atomic<uint32_t> lds_allowed{0};  // sixteen keys per thread take 64 KB beside the sort's own storage
+    const hipError_t ea = allow_dynamic_lds(reinterpret_cast<const void*>(gs2d_grad_csr_sort_kernel<T, IPT>),
+                                            kSortThreads * IPT * 4, lds_allowed);
+    if (ea != hipSuccess) {
+        return ea;
+    }
     hipLaunchKernelGGL((gs2d_grad_csr_sort_kernel<T, IPT>), dim3((unsigned)a.N), dim3(kSortThreads),
                        kSortThreads * IPT * 4, stream, (const T*)a.grid, (uint32_t*)a.scratch, p, pl.lay);
     return hipGetLastError();
@@ -657,6 +663,7 @@ hipError_t run_typed(const GridSamplerGradArgs& a, const CsrPlan& pl, hipStream_
         case 2: e = launch_sort<T, 2>(a, pl, p, stream); break;
         case 4: e = launch_sort<T, 4>(a, pl, p, stream); break;
         case 8: e = launch_sort<T, 8>(a, pl, p, stream); break;
+        case 16: e = launch_sort<T, 16>(a, pl, p, stream); break;
         default: break;
     }
     if (e != hipSuccess) {

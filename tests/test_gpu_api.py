@@ -486,8 +486,9 @@ def test_grid_sampler2d_backward_grid_gradient_lds_variant(oracle, device, aclnn
                 m = aclnn.create_bool_array([True, True])
                 st, ws, ex = aclnn.get_workspace_size_grid_sampler2d_backward(hs[0], hs[1], hs[2], 0, pad, align, m,
                                                                               hs[3], hs[4])
-                # the input gradient takes its list variant where an item's points fit one sorting workgroup
-                lists = Ho * Wo <= 8192
+                # the input gradient takes its list variant where an item's points fit one sorting workgroup and a
+                # gradOutput plane fits a slot of the ring
+                lists = Ho * Wo <= 16384 and Ho * Wo * (4 if dtype == "fp32" else 2) <= 32768
                 assert st == 0 and aclnn.executor_variant(ex) == ("gs2d_grad_lists_lds" if lists
                                                                    else "gs2d_grad_ordered_lds")
                 assert aclnn.destroy_executor(ex) == 0
@@ -507,15 +508,16 @@ def test_grid_sampler2d_backward_grid_gradient_lds_variant(oracle, device, aclnn
 
 @pytest.mark.parametrize("dtype", I.DTYPES)
 def test_grid_sampler2d_backward_input_gradient_list_variant(oracle, device, aclnn, dtype):
-    """The input gradient as a gather over per-element contribution lists (8 channels or more, up to 8192 grid
-    points per item): bit for bit the oracle's chunk / corner / point order, with points piling up on few elements
+    """The input gradient as a gather over per-element contribution lists (8 channels or more, up to 16384 grid
+    points per item and 32 KiB per gradOutput plane): bit for bit the oracle's chunk / corner / point order, with points piling up on few elements
     (lists far longer than the eight entries a lane holds), elements nobody reaches, points outside the image,
     non-finite gradOutput next to corners outside the image, every padding and alignment, channel counts that are not
     a multiple of the planes staged together, plane sizes that leave a partial element tile"""
     torch = _torch()
     rng = np.random.default_rng(630)
     for (N, C, H, W, Ho, Wo, kind) in [(2, 9, 7, 9, 24, 24, "pile"), (3, 8, 30, 40, 64, 64, "random"),
-                                        (1, 13, 64, 64, 90, 88, "smooth"), (2, 8, 20, 20, 32, 64, "outside")]:
+                                        (1, 13, 64, 64, 90, 88, "smooth"), (2, 8, 20, 20, 32, 64, "outside"),
+                                        (1, 8, 40, 44, 100, 64 if dtype == "fp32" else 128, "random")]:
         x = I.cast_np(rng.standard_normal((N, C, H, W)).astype(np.float32), dtype)
         if kind == "pile":
             g32 = rng.choice(np.array([-0.93, -0.31, 0.02, 0.4, 0.77], np.float32), (N, Ho, Wo, 2))
