@@ -139,3 +139,39 @@ def test_upsample_idx64_moves_the_template_threshold(oracle, device, aclnn):
             assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), "planes %s differ" % (sl,)
     finally:
         oracle.set_reference_cores(0)
+
+
+def test_grid_sampler_backward_beyond_2_31_elements(oracle, device, aclnn):
+    """aclnnGridSampler2DBackward with input, gradOutput and input gradient of more than 2^31 elements each, through the
+    list variant of the input gradient and the LDS-ring variant of the grid gradient.  The input gradient is checked on
+    the first and the last channels (a channel's gradient depends on that channel of gradOutput and on the grid only),
+    the grid gradient on the last batch item, whose sums run over planes that start beyond 2^31 elements."""
+    import torch
+    torch.manual_seed(17)
+    N, C, H, W, Ho, Wo = 9, 65535, 64, 64, 64, 64
+    assert N * C * H * W > TWO31 and N * C * Ho * Wo > TWO31
+    x = torch.randn((N, C, H, W), device=device, dtype=torch.float16)
+    go = torch.randn((N, C, Ho, Wo), device=device, dtype=torch.float16)
+    g = (torch.rand((N, Ho, Wo, 2), device=device) * 2.3 - 1.15).to(torch.float16)
+    dx = torch.empty_like(x)
+    dg = torch.empty_like(g)
+    hs = [aclnn.tensor_handle(t) for t in (go, x, g, dx, dg)]
+    m = aclnn.create_bool_array([True, True])
+    st, ws, ex = aclnn.get_workspace_size_grid_sampler2d_backward(hs[0], hs[1], hs[2], 0, 0, False, m, hs[3], hs[4])
+    assert st == 0 and aclnn.executor_variant(ex) == "gs2d_grad_lists_lds"
+    aclnn.destroy_executor(ex)
+    aclnn.destroy_bool_array(m)
+    for h in hs:
+        aclnn.destroy_tensor(h)
+    aclnn.grid_sampler2d_backward(go, x, g, 0, 0, False, (True, True), dx, dg)
+    torch.cuda.synchronize()
+    g_np = _f16(_bits(g))
+    code = I.oracle_code("fp16")
+    for sl in (slice(0, 3), slice(C - 3, C)):
+        rdx, _ = oracle.grid_sampler2d_backward(_f16(_bits(go[:, sl])), _f16(_bits(x[:, sl])), g_np, 0, 0, False,
+                                                dtype=code, want=(True, False))
+        assert np.array_equal(_bits(dx[:, sl]), rdx.view(np.uint16)), "input gradient, channels %s" % (sl,)
+    n = N - 1
+    _, rdg = oracle.grid_sampler2d_backward(_f16(_bits(go[n:])), _f16(_bits(x[n:])), g_np[n:], 0, 0, False, dtype=code,
+                                            want=(False, True))
+    assert np.array_equal(_bits(dg[n:]), rdg.view(np.uint16)), "grid gradient of the last batch item"
