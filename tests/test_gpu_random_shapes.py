@@ -195,6 +195,39 @@ def test_random_sampler_backward_and_3d(oracle, device, aclnn):
         torch.cuda.synchronize()
         _same(I.from_torch(dx, dtype), rdx, dtype, (case, "dx", dtype, N, C, H, W, Ho, Wo, interp, pad, align))
         _same(I.from_torch(dg, dtype), rdg, dtype, (case, "dgrid", dtype, N, C, H, W, Ho, Wo, interp, pad, align))
+    # shapes that the list variant of the input gradient takes (8 channels or more, gradOutput planes of whole
+    # 16-byte units) and, every other case, the LDS-ring variant of the grid gradient too (planes of whole 4 KiB, 128
+    # workgroups of 256 points or more)
+    for case in range(36):
+        dtype = I.DTYPES[case % 3]
+        esz = 4 if dtype == "fp32" else 2
+        C = int(rng.integers(8, 41))
+        if case % 2 == 0:
+            N = int(rng.integers(4, 10))
+            H, W = int(rng.choice([16, 32, 64])), int(rng.choice([32, 64])) * (2 if esz == 2 else 1)
+            Ho = Wo = 64
+            while N * ((Ho * Wo + 255) // 256) < 128:
+                N += 1
+        else:
+            N = int(rng.integers(1, 4))
+            H, W = _dims(rng, 2, 70, 2)
+            Ho, Wo = int(rng.integers(1, 80)), 8 * int(rng.integers(1, 12))
+        interp, pad, align = 0, int(rng.integers(0, 3)), bool(rng.integers(0, 2))
+        _say("gs2d backward lists", dtype, N, C, H, W, Ho, Wo, interp, pad, align)
+        x = I.cast_np(rng.standard_normal((N, C, H, W)).astype(np.float32), dtype)
+        g32 = rng.uniform(-1.3, 1.3, (N, Ho, Wo, 2)).astype(np.float32)
+        if case % 3 == 1:
+            g32 = _sprinkle(rng, g32, H, W, align)
+        if case % 4 == 3:
+            g32 = np.round(g32 * 4) / 4  # points pile up on few elements
+        g = I.cast_np(g32, dtype)
+        go = I.cast_np(rng.standard_normal((N, C, Ho, Wo)).astype(np.float32), dtype)
+        rdx, rdg = oracle.grid_sampler2d_backward(go, x, g, interp, pad, align, dtype=I.oracle_code(dtype))
+        dx, dg = aclnn.grid_sampler2d_backward(I.to_torch(go, dtype, device), I.to_torch(x, dtype, device),
+                                               I.to_torch(g, dtype, device), interp, pad, align)
+        torch.cuda.synchronize()
+        _same(I.from_torch(dx, dtype), rdx, dtype, (case, "dx lists", dtype, N, C, H, W, Ho, Wo, pad, align))
+        _same(I.from_torch(dg, dtype), rdg, dtype, (case, "dgrid lists", dtype, N, C, H, W, Ho, Wo, pad, align))
     for case in range(150):
         dtype = I.DTYPES[case % 3]
         N, C = _dims(rng, 1, 3, 1)[0], _dims(rng, 1, 20, 1)[0]
