@@ -315,7 +315,7 @@ struct Fold<_Float16> {
     }
 };
 
-template <typename T, int CB>
+template <typename T, int CB, int EPL>
 __global__ __launch_bounds__(kApplyThreads) void gs2d_grad_csr_apply_kernel(
     const T* __restrict__ gout, T* __restrict__ dx, const uint32_t* __restrict__ ws, GradParams p, CsrLayout lay,
     uint32_t tiles, uint32_t cblocks, int32_t chans_per_block, int32_t xcd_swizzle)
@@ -413,14 +413,24 @@ __global__ __launch_bounds__(kApplyThreads) void gs2d_grad_csr_apply_kernel(
     }
 
     // ---------------------------------------------------- element lanes ----------------------------------------
+    // A lane owns EPL elements, kApplyLanes apart (a workgroup's tile is EPL * kApplyLanes elements): with two, every
+    // gradOutput plane is staged by half as many workgroups, and the copies into LDS run at the rate the L2s deliver
+    // (268 MB in all for fp16 N16 C256 64x64 with one element per lane, 12 of the kernel's 34 us).
     const uint32_t* wsn = ws + (size_t)n * lay.item_words;
-    const int32_t e = (int32_t)tile * kApplyLanes + tid;
-    const bool live = e < plane_px;
-    const uint32_t cnt = live ? wsn[lay.count + (uint32_t)e] : 0u;
-    uint32_t hoff[kHeld];  // byte offset of the point inside a gradOutput plane
-    acc_t hw[kHeld];
-    {
-        const uint4* slot = reinterpret_cast<const uint4*>(wsn + lay.held) + (size_t)(live ? e : 0) * (kHeld / 2);
+    int32_t e[EPL];
+    bool live[EPL];
+    uint32_t cnt[EPL];
+    uint32_t hoff[EPL][kHeld];  // byte offset of the point inside a gradOutput plane
+    acc_t hw[EPL][kHeld];
+#pragma unroll
+    for (int i = 0; i < EPL; i++) {
+        e[i] = ((int32_t)tile * EPL + i) * kApplyLanes + tid;
+        live[i] = e[i] < plane_px;
+        cnt[i] = live[i] ? wsn[lay.count + (uint32_t)e[i]] : 0u;
+    }
+#pragma unroll
+    for (int i = 0; i < EPL; i++) {
+        const uint4* slot = reinterpret_cast<const uint4*>(wsn + lay.held) + (size_t)(live[i] ? e[i] : 0) * (kHeld / 2);
         uint4 raw[kHeld / 2];
 #pragma unroll
         for (int k = 0; k < kHeld / 2; k++) {
@@ -428,43 +438,51 @@ __global__ __launch_bounds__(kApplyThreads) void gs2d_grad_csr_apply_kernel(
         }
 #pragma unroll
         for (int k = 0; k < kHeld / 2; k++) {
-            const bool a = (uint32_t)(2 * k) < cnt, b = (uint32_t)(2 * k + 1) < cnt;
-            hoff[2 * k] = a ? raw[k].x * (uint32_t)sizeof(T) : 0u;
-            hw[2 * k] = F::weight(a ? __builtin_bit_cast(float, raw[k].y) : 0.0f);
-            hoff[2 * k + 1] = b ? raw[k].z * (uint32_t)sizeof(T) : 0u;
-            hw[2 * k + 1] = F::weight(b ? __builtin_bit_cast(float, raw[k].w) : 0.0f);
+            const bool a = (uint32_t)(2 * k) < cnt[i], b = (uint32_t)(2 * k + 1) < cnt[i];
+            hoff[i][2 * k] = a ? raw[k].x * (uint32_t)sizeof(T) : 0u;
+            hw[i][2 * k] = F::weight(a ? __builtin_bit_cast(float, raw[k].y) : 0.0f);
+            hoff[i][2 * k + 1] = b ? raw[k].z * (uint32_t)sizeof(T) : 0u;
+            hw[i][2 * k + 1] = F::weight(b ? __builtin_bit_cast(float, raw[k].w) : 0.0f);
         }
     }
     __syncthreads();  // spill_used is zero
     // contributions beyond the held ones: a place in LDS while there is room, else they stay in scratch memory
-    const uint2* rest = nullptr;  // where the lane reads them in every step
-    bool rest_in_lds = false;
-    uint32_t rest_at = 0;
-    if (cnt > (uint32_t)kHeld) {
-        const uint32_t extra = cnt - (uint32_t)kHeld;
-        const uint2* src = reinterpret_cast<const uint2*>(wsn + lay.more) + wsn[lay.more_start + (uint32_t)e];
-        rest = src;
-        rest_at = atomicAdd(&spill_used, extra);
-        if (rest_at + extra <= (uint32_t)kApplySpill) {
-            rest_in_lds = true;
-            for (uint32_t i = 0; i < extra; i++) {
-                spill[rest_at + i] = src[i];
+    const uint2* rest[EPL];  // where the lane reads them in every step
+    bool rest_in_lds[EPL];
+    uint32_t rest_at[EPL];
+    uint32_t kmax[EPL];
+    bool any_rest[EPL];
+#pragma unroll
+    for (int i = 0; i < EPL; i++) {
+        rest[i] = nullptr;
+        rest_in_lds[i] = false;
+        rest_at[i] = 0;
+        if (cnt[i] > (uint32_t)kHeld) {
+            const uint32_t extra = cnt[i] - (uint32_t)kHeld;
+            const uint2* src = reinterpret_cast<const uint2*>(wsn + lay.more) + wsn[lay.more_start + (uint32_t)e[i]];
+            rest[i] = src;
+            rest_at[i] = atomicAdd(&spill_used, extra);
+            if (rest_at[i] + extra <= (uint32_t)kApplySpill) {
+                rest_in_lds[i] = true;
+                for (uint32_t k = 0; k < extra; k++) {
+                    spill[rest_at[i] + k] = src[k];
+                }
             }
         }
-    }
-    // the longest held list of the wavefront decides how many rounds its lanes run
-    uint32_t kmax = cnt < (uint32_t)kHeld ? cnt : (uint32_t)kHeld;
-    uint32_t cmax = cnt;
+        // the longest held list of the wavefront decides how many rounds its lanes run
+        uint32_t km = cnt[i] < (uint32_t)kHeld ? cnt[i] : (uint32_t)kHeld;
+        uint32_t cm = cnt[i];
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        const uint32_t other = (uint32_t)__shfl_xor((int)kmax, o);
-        kmax = other > kmax ? other : kmax;
-        const uint32_t other2 = (uint32_t)__shfl_xor((int)cmax, o);
-        cmax = other2 > cmax ? other2 : cmax;
+        for (int o = 32; o > 0; o >>= 1) {
+            const uint32_t other = (uint32_t)__shfl_xor((int)km, o);
+            km = other > km ? other : km;
+            const uint32_t other2 = (uint32_t)__shfl_xor((int)cm, o);
+            cm = other2 > cm ? other2 : cm;
+        }
+        kmax[i] = __builtin_amdgcn_readfirstlane(km);
+        any_rest[i] = __builtin_amdgcn_readfirstlane(cm) > (uint32_t)kHeld;
     }
-    kmax = __builtin_amdgcn_readfirstlane(kmax);
-    const bool any_rest = __builtin_amdgcn_readfirstlane(cmax) > (uint32_t)kHeld;
-    T* dx_e = dx + (n * p.C + c_begin) * (int64_t)plane_px + (live ? e : 0);
+    T* dx_c = dx + (n * p.C + c_begin) * (int64_t)plane_px;
     // the lists are in registers or LDS from here on: nothing below waits for memory except an overfull spill area
     __builtin_amdgcn_s_waitcnt(0);
 
@@ -474,17 +492,17 @@ __global__ __launch_bounds__(kApplyThreads) void gs2d_grad_csr_apply_kernel(
     auto go_at = [&](uint32_t off) -> uint32_t {
         return (uint32_t)*reinterpret_cast<lds_bits_ptr_t>((uintptr_t)(lds_base + off));
     };
-    // R rounds of one step, straight-line: all gradOutput values first (raw bits, so that nothing waits between the
-    // reads), then the sums in list order; a lane whose list is shorter keeps its sum (a select, not arithmetic: a
-    // value read for a contribution that does not exist may be anything)
-    auto rounds = [&](auto r_tag, uint32_t buf_off, acc_t* acc) {
+    // R rounds of one step for one of the lane's elements, straight-line: all gradOutput values first (raw bits, so
+    // that nothing waits between the reads), then the sums in list order; a lane whose list is shorter keeps its sum
+    // (a select, not arithmetic: a value read for a contribution that does not exist may be anything)
+    auto rounds = [&](auto r_tag, uint32_t buf_off, const uint32_t* ho, const acc_t* w, uint32_t count, acc_t* acc) {
         constexpr int R = decltype(r_tag)::value;
         uint32_t raw[R][CB];
 #pragma unroll
         for (int k = 0; k < R; k++) {
 #pragma unroll
             for (int j = 0; j < CB; j++) {
-                raw[k][j] = go_at(buf_off + (uint32_t)j * row_bytes + hoff[k]);
+                raw[k][j] = go_at(buf_off + (uint32_t)j * row_bytes + ho[k]);
             }
         }
         if constexpr (std::is_same<T, _Float16>::value && CB % 2 == 0) {
@@ -495,10 +513,10 @@ __global__ __launch_bounds__(kApplyThreads) void gs2d_grad_csr_apply_kernel(
             }
 #pragma unroll
             for (int k = 0; k < R; k++) {
-                const bool mine = (uint32_t)k < cnt;
+                const bool mine = (uint32_t)k < count;
 #pragma unroll
                 for (int j = 0; j < CB / 2; j++) {
-                    const typename F::pair_t next = F::add2(acc2[j], raw[k][2 * j], raw[k][2 * j + 1], hw[k]);
+                    const typename F::pair_t next = F::add2(acc2[j], raw[k][2 * j], raw[k][2 * j + 1], w[k]);
                     acc2[j] = mine ? next : acc2[j];
                 }
             }
@@ -510,10 +528,10 @@ __global__ __launch_bounds__(kApplyThreads) void gs2d_grad_csr_apply_kernel(
         } else {
 #pragma unroll
             for (int k = 0; k < R; k++) {
-                const bool mine = (uint32_t)k < cnt;
+                const bool mine = (uint32_t)k < count;
 #pragma unroll
                 for (int j = 0; j < CB; j++) {
-                    const acc_t next = F::add(acc[j], raw[k][j], hw[k]);
+                    const acc_t next = F::add(acc[j], raw[k][j], w[k]);
                     acc[j] = mine ? next : acc[j];
                 }
             }
@@ -523,37 +541,40 @@ __global__ __launch_bounds__(kApplyThreads) void gs2d_grad_csr_apply_kernel(
     for (int32_t s = 0; s < steps; s++) {
         lds_barrier();  // the planes of step s have landed
         const uint32_t buf_off = (uint32_t)(s % kApplyNbuf) * buf_bytes;
-        acc_t acc[CB];
 #pragma unroll
-        for (int j = 0; j < CB; j++) {
-            acc[j] = F::zero();
-        }
-        switch (kmax) {
-            case 0: break;
-            case 1: rounds(std::integral_constant<int, 1>{}, buf_off, acc); break;
-            case 2: rounds(std::integral_constant<int, 2>{}, buf_off, acc); break;
-            case 3: rounds(std::integral_constant<int, 3>{}, buf_off, acc); break;
-            case 4: rounds(std::integral_constant<int, 4>{}, buf_off, acc); break;
-            case 5: rounds(std::integral_constant<int, 5>{}, buf_off, acc); break;
-            case 6: rounds(std::integral_constant<int, 6>{}, buf_off, acc); break;
-            case 7: rounds(std::integral_constant<int, 7>{}, buf_off, acc); break;
-            default: rounds(std::integral_constant<int, 8>{}, buf_off, acc); break;
-        }
-        if (any_rest && cnt > (uint32_t)kHeld) {
-            for (uint32_t i = 0; i < cnt - (uint32_t)kHeld; i++) {
-                const uint2 v = rest_in_lds ? spill[rest_at + i] : rest[i];
-                const acc_t w = F::weight(__builtin_bit_cast(float, v.y));
-#pragma unroll
-                for (int j = 0; j < CB; j++) {
-                    acc[j] = F::add(acc[j], go_at(buf_off + (uint32_t)j * row_bytes + v.x * (uint32_t)sizeof(T)), w);
-                }
-            }
-        }
-        if (live) {
+        for (int i = 0; i < EPL; i++) {
+            acc_t acc[CB];
 #pragma unroll
             for (int j = 0; j < CB; j++) {
-                if (s * CB + j < nchan) {
-                    F::store(dx_e + (int64_t)(s * CB + j) * plane_px, acc[j]);
+                acc[j] = F::zero();
+            }
+            switch (kmax[i]) {
+                case 0: break;
+                case 1: rounds(std::integral_constant<int, 1>{}, buf_off, hoff[i], hw[i], cnt[i], acc); break;
+                case 2: rounds(std::integral_constant<int, 2>{}, buf_off, hoff[i], hw[i], cnt[i], acc); break;
+                case 3: rounds(std::integral_constant<int, 3>{}, buf_off, hoff[i], hw[i], cnt[i], acc); break;
+                case 4: rounds(std::integral_constant<int, 4>{}, buf_off, hoff[i], hw[i], cnt[i], acc); break;
+                case 5: rounds(std::integral_constant<int, 5>{}, buf_off, hoff[i], hw[i], cnt[i], acc); break;
+                case 6: rounds(std::integral_constant<int, 6>{}, buf_off, hoff[i], hw[i], cnt[i], acc); break;
+                case 7: rounds(std::integral_constant<int, 7>{}, buf_off, hoff[i], hw[i], cnt[i], acc); break;
+                default: rounds(std::integral_constant<int, 8>{}, buf_off, hoff[i], hw[i], cnt[i], acc); break;
+            }
+            if (any_rest[i] && cnt[i] > (uint32_t)kHeld) {
+                for (uint32_t k = 0; k < cnt[i] - (uint32_t)kHeld; k++) {
+                    const uint2 v = rest_in_lds[i] ? spill[rest_at[i] + k] : rest[i][k];
+                    const acc_t w = F::weight(__builtin_bit_cast(float, v.y));
+#pragma unroll
+                    for (int j = 0; j < CB; j++) {
+                        acc[j] = F::add(acc[j], go_at(buf_off + (uint32_t)j * row_bytes + v.x * (uint32_t)sizeof(T)), w);
+                    }
+                }
+            }
+            if (live[i]) {
+#pragma unroll
+                for (int j = 0; j < CB; j++) {
+                    if (s * CB + j < nchan) {
+                        F::store(dx_c + (int64_t)(s * CB + j) * plane_px + e[i], acc[j]);
+                    }
                 }
             }
         }
@@ -564,6 +585,7 @@ struct CsrPlan {
     bool ok = false;
     int ipt = 1;
     int cb = 1;
+    int epl = 1;  // elements per lane of the apply kernel
     uint32_t tiles = 0, cblocks = 0;
     int32_t chans_per_block = 0;
     int xcd_swizzle = 0;
@@ -594,7 +616,12 @@ CsrPlan make_plan(const GridSamplerGradArgs& a)
     while (pl.cb > 1 && (int64_t)kApplyNbuf * pl.cb * points * esz > kApplyBufBytes) {
         pl.cb /= 2;
     }
-    pl.tiles = (uint32_t)((plane_px + kApplyLanes - 1) / kApplyLanes);
+    // two elements per lane where that still leaves workgroups for every CU
+    pl.epl = (plane_px >= 2 * kApplyLanes && a.N * ((plane_px + 2 * kApplyLanes - 1) / (2 * kApplyLanes)) *
+                                                      ((a.C + pl.cb - 1) / pl.cb) >= 512)
+                 ? 2
+                 : 1;
+    pl.tiles = (uint32_t)((plane_px + kApplyLanes * pl.epl - 1) / (kApplyLanes * pl.epl));
     // channel blocks: about two workgroups per CU, whole groups of planes each
     const int64_t base = a.N * pl.tiles;
     int64_t cblocks = (512 + base - 1) / base;
@@ -629,10 +656,10 @@ hipError_t launch_sort(const GridSamplerGradArgs& a, const CsrPlan& pl, const Gr
     return hipGetLastError();
 }
 
-template <typename T, int CB>
+template <typename T, int CB, int EPL>
 hipError_t launch_apply(const GridSamplerGradArgs& a, const CsrPlan& pl, const GradParams& p, hipStream_t stream)
 {
-    auto kernel = gs2d_grad_csr_apply_kernel<T, CB>;
+    auto kernel = gs2d_grad_csr_apply_kernel<T, CB, EPL>;
     constexpr int kLdsMax = 2 * kApplyBufBytes + kApplySpill * 8;
     static std::atomic<uint32_t> lds_allowed{0};
     const hipError_t ea = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kLdsMax, lds_allowed);
@@ -676,10 +703,13 @@ hipError_t run_typed(const GridSamplerGradArgs& a, const CsrPlan& pl, hipStream_
     if (e != hipSuccess) {
         return e;
     }
-    switch (pl.cb) {
-        case 4: return launch_apply<T, 4>(a, pl, p, stream);
-        case 2: return launch_apply<T, 2>(a, pl, p, stream);
-        case 1: return launch_apply<T, 1>(a, pl, p, stream);
+    switch (pl.cb * 4 + pl.epl) {
+        case 4 * 4 + 1: return launch_apply<T, 4, 1>(a, pl, p, stream);
+        case 4 * 4 + 2: return launch_apply<T, 4, 2>(a, pl, p, stream);
+        case 2 * 4 + 1: return launch_apply<T, 2, 1>(a, pl, p, stream);
+        case 2 * 4 + 2: return launch_apply<T, 2, 2>(a, pl, p, stream);
+        case 1 * 4 + 1: return launch_apply<T, 1, 1>(a, pl, p, stream);
+        case 1 * 4 + 2: return launch_apply<T, 1, 2>(a, pl, p, stream);
         default: return hipErrorInvalidValue;
     }
 }
