@@ -388,11 +388,23 @@ hipError_t launch_interp(const GridSamplerGradArgs& a, hipStream_t stream)
     while (p.tags < p.band_px && p.tags < kTagsMax) {
         p.tags *= 2;
     }
-    bool dx_done = false;
-    if (a.dx != nullptr && INTERP == 0) {
-        const hipError_t e = run_gs2d_grad_input_csr(a, stream, &dx_done);
+    // The grid gradient's LDS-ring kernel goes first where it runs: on its way it zeroes the words that the list
+    // variant of the input gradient wants zeroed, which saves that one a launch (4.7 us).  Whichever of the two reads
+    // gradOutput first reads it from HBM and leaves it in the last-level cache for the other; the grid gradient's
+    // kernel loses more by going first (3.7 us) than the list variant's last kernel gains (1 us), still a net gain.
+    bool dx_done = false, dgrid_done = false;
+    if (INTERP == 0) {
+        GradClear clear{};
+        const bool lists = gs2d_grad_csr_clear(a, &clear);
+        hipError_t e = run_gs2d_grad_grid_lds(a, stream, &dgrid_done, lists ? &clear : nullptr);
         if (e != hipSuccess) {
             return e;
+        }
+        if (lists) {
+            e = run_gs2d_grad_input_csr(a, stream, &dx_done, dgrid_done);
+            if (e != hipSuccess) {
+                return e;
+            }
         }
     }
     if (a.dx != nullptr && !dx_done) {
@@ -427,14 +439,7 @@ hipError_t launch_interp(const GridSamplerGradArgs& a, hipStream_t stream)
             return e;
         }
     }
-    if (a.dgrid != nullptr) {
-        if (INTERP == 0) {
-            bool handled = false;
-            const hipError_t e = run_gs2d_grad_grid_lds(a, stream, &handled);
-            if (e != hipSuccess || handled) {
-                return e;
-            }
-        }
+    if (a.dgrid != nullptr && !dgrid_done) {
         const int64_t total = a.N * a.Hout * a.Wout;
         const int64_t blocks = (total + kThreads - 1) / kThreads;
         if (blocks > INT32_MAX) {

@@ -5,15 +5,20 @@
 // in chunks of 256, per chunk corner after corner (nw, ne, sw, se), per corner point after point, every add rounded
 // to the element type.  Which points reach which element, through which corner and with what weight, depends on
 // the grid alone -- it is the same for every channel.  So instead of scattering per channel (gs2d_grad.hip elects, per
-// corner and round, who may add to an element: about 250 workgroup barriers per group of four planes), three kernels:
+// corner and round, who may add to an element: about 250 workgroup barriers per group of four planes), a few kernels:
 //
-//   sort (one workgroup per batch item): the points are sorted by the cell (y0, x0) of their north-west corner -- a
+//   slots (one lane per grid point, all CUs): the four corner weights of every point go to scratch memory, and the
+//     point takes one of the eight slots of the cell (y0, x0) of its north-west corner (an atomic count per cell: which
+//     slot a point gets depends on timing, which points a cell holds does not).  A cell with more than eight points
+//     flags its batch item.
+//   sort (one workgroup per flagged batch item, else it returns at once): the item's points are sorted by cell -- a
 //     stable block radix sort of (cell, point) keys, so the points of a cell come out in ascending order -- and the
-//     start of every cell's run is noted.  The four corner weights of every point go to scratch memory beside them.
+//     start of every cell's run is noted.
 //   lists (one lane per element, all CUs): element (y, x) is the nw corner of the points of cell (y, x), the ne corner
 //     of cell (y, x-1), the sw corner of cell (y-1, x) and the se corner of cell (y-1, x-1).  The up to eight points of
-//     each of the four runs are read at once, keyed (chunk, corner, point) and sorted in registers by a bitonic
-//     network: the element's contributions in exactly the reference's order.  A corner outside the image never comes
+//     each of the four cells are read at once (from the slots, or from the sorted runs of a flagged item), keyed
+//     (chunk, corner, point) and sorted in registers by a bitonic network: the element's contributions in exactly the
+//     reference's order, whatever order the slots were filled in.  A corner outside the image never comes
 //     up: no element asks for it.  The first eight (point, weight) pairs of an element go to a fixed slot, the rest to
 //     an overflow area.  A cell with more than eight points (points piled up on one spot) takes a walk with cursors
 //     instead of the network.
@@ -68,6 +73,9 @@ struct CsrLayout {
     uint32_t more_start;  // H * W positions in `more` (elements with more than kHeld contributions)
     uint32_t more_used;   // 1 word: pairs handed out in `more`
     uint32_t more;        // up to 4 * points (point, weight) pairs
+    uint32_t slot_count;  // cells counts of points per cell; behind them 2 words: the item's flag "a cell overflowed"
+                          // and the count of workgroups that have handed out their slots
+    uint32_t slots;       // cells * kRun points
     uint32_t item_words;
 };
 
@@ -83,32 +91,45 @@ CsrLayout make_layout(int64_t points, int64_t plane_px, int64_t cells, int ipt)
     l.more_start = l.held + (uint32_t)(2 * kHeld * plane_px);
     l.more_used = align4(l.more_start + (uint32_t)plane_px);
     l.more = l.more_used + 4u;
-    l.item_words = align4(l.more + (uint32_t)(8 * points));
+    l.slot_count = align4(l.more + (uint32_t)(8 * points));
+    l.slots = align4(l.slot_count + (uint32_t)cells + 2u);
+    l.item_words = align4(l.slots + (uint32_t)(kRun * cells));
     return l;
 }
 
+// zeroes the cell counts of every item, the two words behind them and the overflow counter (a kernel rather than a
+// memset: a caller may capture the launch sequence in a graph).  The backward's other kernel does the same on its way
+// when it runs first (GradClear).
+__global__ __launch_bounds__(256) void gs2d_grad_csr_clear_kernel(GradClear c)
+{
+    uint32_t* wsn = c.base + (size_t)blockIdx.y * c.item_words;
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i < c.count) {
+        wsn[c.first + i] = 0u;
+    }
+    if (i == 0) {
+        wsn[c.single] = 0u;
+    }
+}
+
+// The points of one item sorted by cell, and where every cell's run starts: all threads of a workgroup of
+// kSortThreads.
 template <typename T, int IPT>
-__global__ __launch_bounds__(kSortThreads) void gs2d_grad_csr_sort_kernel(const T* __restrict__ grid,
-                                                                           uint32_t* __restrict__ ws, GradParams p,
-                                                                           CsrLayout lay)
+__device__ __forceinline__ void sort_item(const T* __restrict__ grid, uint32_t* __restrict__ wsn, const GradParams& p,
+                                          const CsrLayout& lay, int64_t n,
+                                          typename rocprim::block_radix_sort<uint32_t, kSortThreads, IPT>::storage_type&
+                                              sort_storage,
+                                          uint32_t* sorted_lds)
 {
     using sort_t = rocprim::block_radix_sort<uint32_t, kSortThreads, IPT>;
-    __shared__ typename sort_t::storage_type sort_storage;
-    extern __shared__ uint32_t sorted_lds[];  // kSortThreads * IPT keys
     const int32_t points = p.Ho * p.Wo;
     const int32_t cells = (p.H + 1) * (p.W + 1);
     const uint32_t cell_bits = 32u - (uint32_t)__builtin_clz((uint32_t)cells);  // `cells` itself fits: the sentinel
     const int t = threadIdx.x;
-    const int64_t n = blockIdx.x;
-    uint32_t* wsn = ws + (size_t)n * lay.item_words;
-    float* wts = reinterpret_cast<float*>(wsn + lay.wts);
     uint32_t* sorted = wsn + lay.sorted;
     uint32_t* cell_start = wsn + lay.cell_start;
-    if (t == 0) {
-        wsn[lay.more_used] = 0u;
-    }
 
-    // keys (cell << kPointBits | point); the weights of every point go to scratch
+    // keys (cell << kPointBits | point)
     uint32_t keys[IPT];
 #pragma unroll
     for (int i = 0; i < IPT; i++) {
@@ -119,7 +140,6 @@ __global__ __launch_bounds__(kSortThreads) void gs2d_grad_csr_sort_kernel(const 
             const int64_t idx = n * points + pt;
             decide_grad_taps<T, 0>(tp, ElemIO<T>::load(grid + 2 * idx), ElemIO<T>::load(grid + 2 * idx + 1), p.H, p.W,
                                    p.pad, p.align);
-            *reinterpret_cast<float4*>(wts + 4 * pt) = make_float4(tp.w[0], tp.w[1], tp.w[2], tp.w[3]);
             if (tp.x0 >= -1 && tp.x0 < p.W && tp.y0 >= -1 && tp.y0 < p.H) {
                 const uint32_t cell = (uint32_t)(tp.y0 + 1) * (uint32_t)(p.W + 1) + (uint32_t)(tp.x0 + 1);
                 keys[i] = (cell << kPointBits) | (uint32_t)pt;
@@ -156,6 +176,63 @@ __global__ __launch_bounds__(kSortThreads) void gs2d_grad_csr_sort_kernel(const 
     }
 }
 
+// One lane per grid point (workgroups of kSortThreads points, `blocks_per_item` of them per batch item): weights to
+// scratch, a slot in the point's cell.  The workgroup of an item that finishes last sorts the item when one of its
+// cells overflowed -- it knows that it is the last from a count of finished workgroups, it waits for nobody, and it
+// reads nothing that the others wrote.
+template <typename T, int IPT>
+__global__ __launch_bounds__(kSortThreads) void gs2d_grad_csr_slots_kernel(const T* __restrict__ grid,
+                                                                            uint32_t* __restrict__ ws, GradParams p,
+                                                                            CsrLayout lay, uint32_t blocks_per_item)
+{
+    using sort_t = rocprim::block_radix_sort<uint32_t, kSortThreads, IPT>;
+    __shared__ typename sort_t::storage_type sort_storage;
+    __shared__ uint32_t sort_it;
+    extern __shared__ uint32_t sorted_lds[];  // kSortThreads * IPT keys
+    const int32_t points = p.Ho * p.Wo;
+    const uint32_t cells = (uint32_t)(p.H + 1) * (uint32_t)(p.W + 1);
+    const int t = threadIdx.x;
+    const int64_t n = blockIdx.x / blocks_per_item;
+    const int32_t pt = (int32_t)(blockIdx.x % blocks_per_item) * kSortThreads + t;
+    uint32_t* wsn = ws + (size_t)n * lay.item_words;
+    uint32_t* flag = wsn + lay.slot_count + cells;
+    uint32_t* finished = flag + 1;  // low half: workgroups of the item that are through; high half: those that flagged
+    bool crowded = false;
+    if (pt < points) {
+        float* wts = reinterpret_cast<float*>(wsn + lay.wts);
+        GradTaps<T, 0> tp;
+        const int64_t idx = n * points + pt;
+        decide_grad_taps<T, 0>(tp, ElemIO<T>::load(grid + 2 * idx), ElemIO<T>::load(grid + 2 * idx + 1), p.H, p.W,
+                               p.pad, p.align);
+        *reinterpret_cast<float4*>(wts + 4 * pt) = make_float4(tp.w[0], tp.w[1], tp.w[2], tp.w[3]);
+        if (tp.x0 >= -1 && tp.x0 < p.W && tp.y0 >= -1 && tp.y0 < p.H) {
+            const uint32_t cell = (uint32_t)(tp.y0 + 1) * (uint32_t)(p.W + 1) + (uint32_t)(tp.x0 + 1);
+            const uint32_t r = atomicAdd(&wsn[lay.slot_count + cell], 1u);
+            if (r < (uint32_t)kRun) {
+                wsn[lay.slots + cell * (uint32_t)kRun + r] = (uint32_t)pt;
+            } else {
+                crowded = true;  // the item is to be sorted
+            }
+        }
+    }
+    // The workgroup counts itself as finished, and in the same atomic says whether one of its points found its cell
+    // full: the workgroup that counts last has the flags of all the others in what the atomic returns.
+    const int any = __syncthreads_or(crowded ? 1 : 0);
+    if (t == 0) {
+        const uint32_t before = atomicAdd(finished, 1u + ((uint32_t)any << 16));
+        const bool last = (before & 0xFFFFu) == blocks_per_item - 1u;
+        const bool sort = last && ((before >> 16) != 0u || any != 0);
+        if (sort) {
+            *flag = 1u;  // for the kernel that makes the lists
+        }
+        sort_it = sort ? 1u : 0u;
+    }
+    __syncthreads();
+    if (sort_it != 0u) {
+        sort_item<T, IPT>(grid, wsn, p, lay, n, sort_storage, sorted_lds);
+    }
+}
+
 __device__ __forceinline__ uint2 pair_of(uint32_t pt, uint32_t corner, const float* wts)
 {
     return make_uint2(pt, __builtin_bit_cast(uint32_t, wts[4u * pt + corner]));
@@ -183,12 +260,21 @@ __global__ __launch_bounds__(kListThreads) void gs2d_grad_csr_lists_kernel(uint3
     cid[1] = (y + 1u) * w1 + x;         // ne corner of cell (y, x - 1)
     cid[2] = y * w1 + (x + 1u);         // sw corner of cell (y - 1, x)
     cid[3] = y * w1 + x;                // se corner of cell (y - 1, x - 1)
+    // the points of a cell: its slots, or, in an item where some cell overflowed its slots, its run in the sorted keys
+    const uint32_t cells = (uint32_t)(H + 1) * w1;
+    const bool from_runs = wsn[lay.slot_count + cells] != 0u;
+    const uint32_t* source = from_runs ? sorted : wsn + lay.slots;
     uint32_t cnt = 0;
     bool crowded = false;
 #pragma unroll
     for (int k = 0; k < 4; k++) {
-        cur[k] = cell_start[cid[k]];
-        end[k] = cell_start[cid[k] + 1];
+        if (from_runs) {
+            cur[k] = cell_start[cid[k]];
+            end[k] = cell_start[cid[k] + 1];
+        } else {
+            cur[k] = cid[k] * (uint32_t)kRun;
+            end[k] = cur[k] + wsn[lay.slot_count + cid[k]];
+        }
         cnt += end[k] - cur[k];
         crowded = crowded || end[k] - cur[k] > (uint32_t)kRun;
     }
@@ -216,7 +302,7 @@ __global__ __launch_bounds__(kListThreads) void gs2d_grad_csr_lists_kernel(uint3
 #pragma unroll
             for (int i = 0; i < kRun; i++) {
                 const bool valid = (uint32_t)i < len;
-                const uint32_t pt = sorted[valid ? cur[k] + (uint32_t)i : 0u] & kPointMask;
+                const uint32_t pt = source[valid ? cur[k] + (uint32_t)i : 0u] & kPointMask;
                 key[k * kRun + i] =
                     valid ? (((pt >> kChunkShift) << (kPointBits + 2)) | ((uint32_t)k << kPointBits) | pt) : 0xFFFFFFFFu;
             }
@@ -246,7 +332,8 @@ __global__ __launch_bounds__(kListThreads) void gs2d_grad_csr_lists_kernel(uint3
         }
         return;
     }
-    // a run longer than the network takes: chunk by chunk, corner by corner, with a cursor into every run
+    // a run longer than the network takes (only in an item that went through the sort): chunk by chunk, corner by
+    // corner, with a cursor into every run
     uint32_t i = 0;
     for (;;) {
         uint32_t chunk = 0xFFFFFFFFu;
@@ -605,7 +692,7 @@ CsrPlan make_plan(const GridSamplerGradArgs& a)
         return pl;
     }
     // worth three extra kernels only with channels to share the lists among
-    if (a.C < 8 || a.N * a.C > INT32_MAX) {
+    if (a.C < 8 || a.N * a.C > INT32_MAX || a.N > 65535) {  // the clear kernel indexes items by blockIdx.y
         return pl;
     }
     pl.ipt = 1;
@@ -631,7 +718,8 @@ CsrPlan make_plan(const GridSamplerGradArgs& a)
     cpb = (cpb + pl.cb - 1) / pl.cb * pl.cb;
     cblocks = (a.C + cpb - 1) / cpb;
     const int64_t list_tiles = (plane_px + kListThreads - 1) / kListThreads;
-    if (base * cblocks > INT32_MAX || a.N * list_tiles > INT32_MAX) {
+    if (base * cblocks > INT32_MAX || a.N * list_tiles > INT32_MAX ||
+        a.N * ((points + kSortThreads - 1) / kSortThreads) > INT32_MAX) {
         return pl;
     }
     pl.chans_per_block = (int32_t)cpb;
@@ -643,17 +731,30 @@ CsrPlan make_plan(const GridSamplerGradArgs& a)
 }
 
 template <typename T, int IPT>
-hipError_t launch_sort(const GridSamplerGradArgs& a, const CsrPlan& pl, const GradParams& p, hipStream_t stream)
+hipError_t launch_slots(const GridSamplerGradArgs& a, const CsrPlan& pl, const GradParams& p, hipStream_t stream)
 {
     static std::atomic<uint32_t> lds_allowed{0};  // sixteen keys per thread take 64 KB beside the sort's own storage
-    const hipError_t ea = allow_dynamic_lds(reinterpret_cast<const void*>(gs2d_grad_csr_sort_kernel<T, IPT>),
+    const hipError_t ea = allow_dynamic_lds(reinterpret_cast<const void*>(gs2d_grad_csr_slots_kernel<T, IPT>),
                                             kSortThreads * IPT * 4, lds_allowed);
     if (ea != hipSuccess) {
         return ea;
     }
-    hipLaunchKernelGGL((gs2d_grad_csr_sort_kernel<T, IPT>), dim3((unsigned)a.N), dim3(kSortThreads),
-                       kSortThreads * IPT * 4, stream, (const T*)a.grid, (uint32_t*)a.scratch, p, pl.lay);
+    const int64_t blocks_per_item = (a.Hout * a.Wout + kSortThreads - 1) / kSortThreads;
+    hipLaunchKernelGGL((gs2d_grad_csr_slots_kernel<T, IPT>), dim3((unsigned)(a.N * blocks_per_item)),
+                       dim3(kSortThreads), kSortThreads * IPT * 4, stream, (const T*)a.grid, (uint32_t*)a.scratch, p,
+                       pl.lay, (uint32_t)blocks_per_item);
     return hipGetLastError();
+}
+
+GradClear clear_of(const GridSamplerGradArgs& a, const CsrPlan& pl)
+{
+    GradClear c{};
+    c.base = (uint32_t*)a.scratch;
+    c.item_words = pl.lay.item_words;
+    c.first = pl.lay.slot_count;
+    c.count = (uint32_t)((a.Hin + 1) * (a.Win + 1)) + 2u;  // the counts, the flag, the count of finished workgroups
+    c.single = pl.lay.more_used;
+    return c;
 }
 
 template <typename T, int CB, int EPL>
@@ -674,7 +775,7 @@ hipError_t launch_apply(const GridSamplerGradArgs& a, const CsrPlan& pl, const G
 }
 
 template <typename T>
-hipError_t run_typed(const GridSamplerGradArgs& a, const CsrPlan& pl, hipStream_t stream)
+hipError_t run_typed(const GridSamplerGradArgs& a, const CsrPlan& pl, bool cleared, hipStream_t stream)
 {
     GradParams p{};
     p.C = (int32_t)a.C;
@@ -684,13 +785,23 @@ hipError_t run_typed(const GridSamplerGradArgs& a, const CsrPlan& pl, hipStream_
     p.Wo = (int32_t)a.Wout;
     p.pad = a.pad;
     p.align = a.align;
-    hipError_t e = hipErrorInvalidValue;
+    hipError_t e = hipSuccess;
+    if (!cleared) {
+        const GradClear c = clear_of(a, pl);
+        hipLaunchKernelGGL(gs2d_grad_csr_clear_kernel, dim3((c.count + 255u) / 256u, (unsigned)a.N), dim3(256), 0, stream,
+                           c);
+        e = hipGetLastError();
+        if (e != hipSuccess) {
+            return e;
+        }
+    }
+    e = hipErrorInvalidValue;
     switch (pl.ipt) {
-        case 1: e = launch_sort<T, 1>(a, pl, p, stream); break;
-        case 2: e = launch_sort<T, 2>(a, pl, p, stream); break;
-        case 4: e = launch_sort<T, 4>(a, pl, p, stream); break;
-        case 8: e = launch_sort<T, 8>(a, pl, p, stream); break;
-        case 16: e = launch_sort<T, 16>(a, pl, p, stream); break;
+        case 1: e = launch_slots<T, 1>(a, pl, p, stream); break;
+        case 2: e = launch_slots<T, 2>(a, pl, p, stream); break;
+        case 4: e = launch_slots<T, 4>(a, pl, p, stream); break;
+        case 8: e = launch_slots<T, 8>(a, pl, p, stream); break;
+        case 16: e = launch_slots<T, 16>(a, pl, p, stream); break;
         default: break;
     }
     if (e != hipSuccess) {
@@ -722,7 +833,19 @@ int64_t gs2d_grad_csr_words(const GridSamplerGradArgs& a)
     return pl.ok ? (int64_t)pl.lay.item_words * a.N : 0;
 }
 
-hipError_t run_gs2d_grad_input_csr(const GridSamplerGradArgs& a, hipStream_t stream, bool* handled)
+bool gs2d_grad_csr_clear(const GridSamplerGradArgs& a, GradClear* clear)
+{
+    if (a.dx == nullptr || a.scratch == nullptr) {
+        return false;
+    }
+    const CsrPlan pl = make_plan(a);
+    if (pl.ok) {
+        *clear = clear_of(a, pl);
+    }
+    return pl.ok;
+}
+
+hipError_t run_gs2d_grad_input_csr(const GridSamplerGradArgs& a, hipStream_t stream, bool* handled, bool cleared)
 {
     *handled = false;
     if (a.dx == nullptr || a.scratch == nullptr) {
@@ -734,9 +857,9 @@ hipError_t run_gs2d_grad_input_csr(const GridSamplerGradArgs& a, hipStream_t str
     }
     *handled = true;
     switch (a.elem) {
-        case Elem::F32: return run_typed<float>(a, pl, stream);
-        case Elem::F16: return run_typed<_Float16>(a, pl, stream);
-        case Elem::BF16: return run_typed<__bf16>(a, pl, stream);
+        case Elem::F32: return run_typed<float>(a, pl, cleared, stream);
+        case Elem::F16: return run_typed<_Float16>(a, pl, cleared, stream);
+        case Elem::BF16: return run_typed<__bf16>(a, pl, cleared, stream);
     }
     return hipErrorInvalidValue;
 }

@@ -69,7 +69,7 @@ template <typename T, int NBUF, int PITCH>
 __global__ __launch_bounds__(kThreadsLds) void gs2d_grad_grid_lds_kernel(
     const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ grid, T* __restrict__ dgrid, int32_t C,
     int32_t H, int32_t W, int32_t points, uint32_t tiles_per_n, int32_t pad, int32_t align, int32_t xcd_swizzle,
-    int32_t ahead_x, float neg_zero)
+    int32_t ahead_x, float neg_zero, GradClear clear)
 {
     static_assert(kUnroll % NBUF == 0, "a turn of the loop is whole turns of the ring");
     extern __shared__ uint4 smem_raw[];
@@ -244,6 +244,20 @@ __global__ __launch_bounds__(kThreadsLds) void gs2d_grad_grid_lds_kernel(
     // ---------------------------------------------------- point wavefronts -------------------------------------
     if (tid < NBUF * 4) {
         reinterpret_cast<uint32_t*>(lds + (tid >> 2) * PITCH + zero_off)[tid & 3] = 0u;
+    }
+    // words of scratch memory that a later kernel wants zeroed (none when clear.count is 0): the item's tiles share
+    // them out
+    if (clear.count != 0u) {
+        uint32_t* words = clear.base + (size_t)n * clear.item_words;
+        const uint32_t share = (clear.count + tiles_per_n - 1u) / tiles_per_n;
+        const uint32_t from = tile * share;
+        const uint32_t to = (from + share < clear.count) ? from + share : clear.count;
+        for (uint32_t i = from + (uint32_t)tid; i < to; i += (uint32_t)kPoints) {
+            words[clear.first + i] = 0u;
+        }
+        if (tile == 0u && tid == 0) {
+            words[clear.single] = 0u;
+        }
     }
     const int32_t pix = (int32_t)tile * kPoints + tid;
     const bool live = pix < points;
@@ -425,7 +439,7 @@ GridLdsPlan make_plan(const GridSamplerGradArgs& a)
 }
 
 template <typename T, int CLS>
-hipError_t launch_cls(const GridSamplerGradArgs& a, const GridLdsPlan& p, hipStream_t stream)
+hipError_t launch_cls(const GridSamplerGradArgs& a, const GridLdsPlan& p, const GradClear& clear, hipStream_t stream)
 {
     auto kernel = gs2d_grad_grid_lds_kernel<T, kGradNbuf[CLS], kGradPitch[CLS]>;
     constexpr int lds_bytes = kGradNbuf[CLS] * (kGradPitch[CLS] + kPoints * (int)sizeof(T)) + kDumpBytes;
@@ -446,17 +460,18 @@ hipError_t launch_cls(const GridSamplerGradArgs& a, const GridLdsPlan& p, hipStr
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kThreadsLds), lds_bytes, stream, (const T*)a.gout, (const T*)a.x,
                        (const T*)a.grid, (T*)a.dgrid, (int32_t)a.C, (int32_t)a.Hin, (int32_t)a.Win,
                        (int32_t)(a.Hout * a.Wout), p.tiles_per_n, (int32_t)a.pad, (int32_t)a.align, p.xcd_swizzle,
-                       (int32_t)ahead, -0.0f);
+                       (int32_t)ahead, -0.0f, clear);
     return hipGetLastError();
 }
 
 template <typename T>
-hipError_t launch_typed(const GridSamplerGradArgs& a, const GridLdsPlan& p, hipStream_t stream)
+hipError_t launch_typed(const GridSamplerGradArgs& a, const GridLdsPlan& p, const GradClear& clear,
+                        hipStream_t stream)
 {
     switch (p.cls) {
-        case 0: return launch_cls<T, 0>(a, p, stream);
-        case 1: return launch_cls<T, 1>(a, p, stream);
-        case 2: return launch_cls<T, 2>(a, p, stream);
+        case 0: return launch_cls<T, 0>(a, p, clear, stream);
+        case 1: return launch_cls<T, 1>(a, p, clear, stream);
+        case 2: return launch_cls<T, 2>(a, p, clear, stream);
         default: return hipErrorInvalidValue;
     }
 }
@@ -465,7 +480,8 @@ hipError_t launch_typed(const GridSamplerGradArgs& a, const GridLdsPlan& p, hipS
 
 bool gs2d_grad_grid_uses_lds(const GridSamplerGradArgs& a) { return make_plan(a).ok; }
 
-hipError_t run_gs2d_grad_grid_lds(const GridSamplerGradArgs& a, hipStream_t stream, bool* handled)
+hipError_t run_gs2d_grad_grid_lds(const GridSamplerGradArgs& a, hipStream_t stream, bool* handled,
+                                  const GradClear* clear_or_null)
 {
     *handled = false;
     if (a.dgrid == nullptr) {
@@ -476,10 +492,11 @@ hipError_t run_gs2d_grad_grid_lds(const GridSamplerGradArgs& a, hipStream_t stre
         return hipSuccess;
     }
     *handled = true;
+    const GradClear clear = (clear_or_null != nullptr) ? *clear_or_null : GradClear{};  // count 0, base null: nothing
     switch (a.elem) {
-        case Elem::F32: return launch_typed<float>(a, p, stream);
-        case Elem::F16: return launch_typed<_Float16>(a, p, stream);
-        case Elem::BF16: return launch_typed<__bf16>(a, p, stream);
+        case Elem::F32: return launch_typed<float>(a, p, clear, stream);
+        case Elem::F16: return launch_typed<_Float16>(a, p, clear, stream);
+        case Elem::BF16: return launch_typed<__bf16>(a, p, clear, stream);
     }
     return hipErrorInvalidValue;
 }

@@ -58,12 +58,26 @@ const char* resize_grad_variant(const ResizeGradArgs& a);  // which kernel launc
 hipError_t launch_grid_sampler2d_grad(const GridSamplerGradArgs& a, hipStream_t stream);
 // grid gradient of the 2-D sampler with the input planes staged through LDS (gs2d_grad_lds.hip); *handled is false
 // when the shape does not qualify.  gs2d_grad_grid_uses_lds: whether it would run (pointers may still be null).
-hipError_t run_gs2d_grad_grid_lds(const GridSamplerGradArgs& a, hipStream_t stream, bool* handled);
+// Words of scratch memory that one kernel zeroes on its way for a later one: per batch item (item_words apart) `count`
+// words from `first` on, and the word `single`.
+struct GradClear {
+    uint32_t* base;
+    uint32_t item_words;
+    uint32_t first;
+    uint32_t count;
+    uint32_t single;
+};
+// `clear`, when not null, is zeroed by the kernel if it runs (*handled).
+hipError_t run_gs2d_grad_grid_lds(const GridSamplerGradArgs& a, hipStream_t stream, bool* handled,
+                                  const GradClear* clear);
 bool gs2d_grad_grid_uses_lds(const GridSamplerGradArgs& a);
 // input gradient of the 2-D sampler as a gather over per-element contribution lists (gs2d_grad_csr.hip): 32-bit words
 // of GridSamplerGradArgs::scratch it needs, 0 when the shape does not qualify; *handled is false when it did not run
 int64_t gs2d_grad_csr_words(const GridSamplerGradArgs& a);
-hipError_t run_gs2d_grad_input_csr(const GridSamplerGradArgs& a, hipStream_t stream, bool* handled);
+// whether run_gs2d_grad_input_csr would run, and the words it wants zeroed first: `cleared` says that an earlier kernel
+// on the stream has done that, else it launches a kernel of its own for it
+bool gs2d_grad_csr_clear(const GridSamplerGradArgs& a, GradClear* clear);
+hipError_t run_gs2d_grad_input_csr(const GridSamplerGradArgs& a, hipStream_t stream, bool* handled, bool cleared);
 hipError_t launch_grid_sampler3d(const GridSampler3DArgs& a, hipStream_t stream);
 hipError_t launch_grid_sampler3d_grad(const GridSampler3DGradArgs& a, hipStream_t stream);
 // 32-bit words of GridSampler3DGradArgs::chunk_ranges that make the input gradient faster; 0 when it would not help

@@ -512,12 +512,14 @@ def test_grid_sampler2d_backward_input_gradient_list_variant(oracle, device, acl
     points per item and 32 KiB per gradOutput plane): bit for bit the oracle's chunk / corner / point order, with points piling up on few elements
     (lists far longer than the eight entries a lane holds), elements nobody reaches, points outside the image,
     non-finite gradOutput next to corners outside the image, every padding and alignment, channel counts that are not
-    a multiple of the planes staged together, plane sizes that leave a partial element tile"""
+    a multiple of the planes staged together, plane sizes that leave a partial element tile, batches where one item
+    takes the sorted path and the others the slots"""
     torch = _torch()
     rng = np.random.default_rng(630)
     for (N, C, H, W, Ho, Wo, kind) in [(2, 9, 7, 9, 24, 24, "pile"), (3, 8, 30, 40, 64, 64, "random"),
                                         (1, 13, 64, 64, 90, 88, "smooth"), (2, 8, 20, 20, 32, 64, "outside"),
-                                        (1, 8, 40, 44, 100, 64 if dtype == "fp32" else 128, "random")]:
+                                        (1, 8, 40, 44, 100, 64 if dtype == "fp32" else 128, "random"),
+                                        (3, 8, 48, 48, 40, 40, "mixed"), (8, 16, 64, 64, 64, 64, "mixed")]:
         x = I.cast_np(rng.standard_normal((N, C, H, W)).astype(np.float32), dtype)
         if kind == "pile":
             g32 = rng.choice(np.array([-0.93, -0.31, 0.02, 0.4, 0.77], np.float32), (N, Ho, Wo, 2))
@@ -527,6 +529,11 @@ def test_grid_sampler2d_backward_input_gradient_list_variant(oracle, device, acl
             g32 = np.ascontiguousarray(g32, dtype=np.float32)
         elif kind == "outside":
             g32 = rng.uniform(-2.5, 2.5, (N, Ho, Wo, 2)).astype(np.float32)
+        elif kind == "mixed":
+            # one item whose points pile up (its cells overflow their slots, the item is sorted) among items whose
+            # cells hold a few points each (lists straight from the slots); several workgroups of points per item
+            g32 = rng.uniform(-1.0, 1.0, (N, Ho, Wo, 2)).astype(np.float32)
+            g32[N // 2] = rng.choice(np.array([-0.93, -0.31, 0.02, 0.4, 0.77], np.float32), (Ho, Wo, 2))
         else:
             g32 = rng.uniform(-1.2, 1.2, (N, Ho, Wo, 2)).astype(np.float32)
         flat = g32.reshape(-1, 2)
