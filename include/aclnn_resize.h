@@ -12,7 +12,13 @@
  *     bilinear : align_corners = false, half-pixel centres, scale = in / out -- the same kernel as
  *                aclnnUpsampleBilinear2d with alignCorners = false and zero user scales
  *     nearest  : src = min(floor(dst * (in / out)), in - 1)
- *                (image/resize_nearest_neighbor_v2/op_kernel/arch35/resize_nearest_neighbor_v2_simt.h:103-124)
+ *                (image/resize_nearest_neighbor_v2/op_kernel/arch35/resize_nearest_neighbor_v2_simt.h:103-124);
+ *                NHWC upscales by whole factors with at least 128 bytes of channels per pixel and rows that fit the
+ *                reference device's unified buffer take the reference's replicating template instead,
+ *                src = dst / factor (.../op_host/arch35/resize_nearest_neighbor_v2_tiling_base.cpp:640-665,
+ *                .../op_kernel/arch35/resize_nearest_neighbor_v2_data_copy_nhwc.h:205-231): the same result up to
+ *                a factor of 40, different from the float rule from 41 on.  The buffer size mirrored is 253952
+ *                bytes unless the environment variable OPSCV_REFERENCE_UB_BYTES gives another.
  *   views     : arbitrary strides/offsets are honoured (packed through the workspace)
  */
 #ifndef OPSCV_ACLNN_RESIZE_H_

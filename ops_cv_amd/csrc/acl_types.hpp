@@ -168,6 +168,7 @@ struct ResizeArgs {
     int channels_last = 0;
     int raw_lambda = 0;  // NCHW bilinear: fraction taken from the unclamped source coordinate (see axis_tap)
     float scale_h = 1.0f, scale_w = 1.0f;
+    int32_t rep_h = 0, rep_w = 0;  // Nearest: whole upscale factors when source = destination / factor is the rule, else 0
     int64_t point_step_h = 1, point_step_w = 1;  // PointCopy: integer source stride per destination pixel
     int64_t N = 0, C = 0, Hs = 0, Ws = 0, Hd = 0, Wd = 0;
     const void* x = nullptr;

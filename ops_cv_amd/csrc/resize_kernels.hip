@@ -503,13 +503,25 @@ __global__ __launch_bounds__(kThreads) void resize_nhwc_four_weights_kernel(cons
 // Nearest-neighbour resize (align_corners = false, half_pixel_centers = false):
 //   src = min(floor(float(dst) * scale), len_src - 1)
 // image/resize_nearest_neighbor_v2/op_kernel/arch35/resize_nearest_neighbor_v2_simt.h:103-124.
-__device__ __forceinline__ int32_t nearest_src(int32_t d, float scale, int32_t len_src)
+// With rep > 0: src = dst / rep in integer arithmetic, the rule of the reference's channels-last template that
+// replicates every source pixel a whole number of times (resize_nearest_neighbor_v2_data_copy_nhwc.h:205-231; the
+// launch plan says when the reference takes it).  The two first differ at a factor of 41.
+__device__ __forceinline__ int32_t nearest_src(int32_t d, float scale, int32_t len_src, int32_t rep)
 {
+    if (rep > 0) {
+        return d / rep;
+    }
     const float f = __builtin_floorf((float)d * scale);
     // the reference converts to an unsigned index and clamps from above only; dst and scale are non-negative
     const int32_t i = (f >= 2147483648.0f) ? INT32_MAX : (int32_t)f;
     return (i < len_src - 1) ? i : len_src - 1;
 }
+
+// scales of the float rule, factors of the replicating rule (0: the float rule)
+struct NearestRule {
+    float scale_h, scale_w;
+    int32_t rep_h, rep_w;
+};
 
 constexpr int kNearestBand = 8;
 
@@ -519,8 +531,7 @@ constexpr int kNearestBand = 8;
 template <typename T, bool NHWC, bool VEC>
 __global__ __launch_bounds__(kThreads) void resize_nearest_kernel(const T* __restrict__ x, T* __restrict__ y,
                                                                    int64_t outer, int32_t C, int32_t Hs, int32_t Ws,
-                                                                   int32_t Hd, int32_t Wd, float scale_h, float scale_w,
-                                                                   int streaming)
+                                                                   int32_t Hd, int32_t Wd, NearestRule rule, int streaming)
 {
     constexpr int V = VEC ? 16 / (int)sizeof(T) : 1;
     const int64_t row_elems = NHWC ? (int64_t)Wd * C : (int64_t)Wd;
@@ -533,12 +544,12 @@ __global__ __launch_bounds__(kThreads) void resize_nearest_kernel(const T* __res
     if (NHWC) {
         const int32_t w = (int32_t)(e0 / C);
         const int32_t c = (int32_t)(e0 - (int64_t)w * C);
-        src_off[0] = (int64_t)nearest_src(w, scale_w, Ws) * C + c;
+        src_off[0] = (int64_t)nearest_src(w, rule.scale_w, Ws, rule.rep_w) * C + c;
     } else {
 #pragma unroll
         for (int i = 0; i < V; i++) {
             const int32_t col = ((int32_t)e0 + i < Wd) ? (int32_t)e0 + i : Wd - 1;  // past a ragged row end: unused
-            src_off[i] = nearest_src(col, scale_w, Ws);
+            src_off[i] = nearest_src(col, rule.scale_w, Ws, rule.rep_w);
         }
     }
     // NCHW rows of any width: the vector store is element-aligned, the lane at a ragged row end stores singly
@@ -551,7 +562,7 @@ __global__ __launch_bounds__(kThreads) void resize_nearest_kernel(const T* __res
       for (int64_t r = r0; r < r_end; r++) {
         const int64_t o = r / Hd;
         const int32_t h = (int32_t)(r - o * Hd);
-        const T* src = x + (o * Hs + nearest_src(h, scale_h, Hs)) * src_row_elems;
+        const T* src = x + (o * Hs + nearest_src(h, rule.scale_h, Hs, rule.rep_h)) * src_row_elems;
         T* dst = y + r * row_elems + e0;
         if (VEC) {
             uint4 packed;
@@ -607,9 +618,8 @@ __global__ __launch_bounds__(kThreads) void resize_nearest_kernel(const T* __res
 template <typename T>
 __global__ __launch_bounds__(kThreads) void resize_nearest_lds_kernel(const T* __restrict__ x, T* __restrict__ y,
                                                                        int64_t outer, int32_t Hs, int32_t Ws,
-                                                                       int32_t Hd, int32_t Wd, float scale_h,
-                                                                       float scale_w, uint32_t slot_bytes,
-                                                                       int streaming, int32_t ci)
+                                                                       int32_t Hd, int32_t Wd, NearestRule rule,
+                                                                       uint32_t slot_bytes, int streaming, int32_t ci)
 {
     // ci = 1: planes of Hs x Ws.  ci = C: channels-last images, resized as planes whose rows are Ws * C elements
     // (element j of a row is channel j % C of pixel j / C); "columns" below are row elements.
@@ -622,8 +632,8 @@ __global__ __launch_bounds__(kThreads) void resize_nearest_lds_kernel(const T* _
     const int32_t Wse = Ws * ci, Wde = Wd * ci;
     const int32_t col_first = blockIdx.x * kThreads * V;
     const int32_t col_last = ((col_first + kThreads * V < Wde) ? col_first + kThreads * V : Wde) - 1;
-    const int32_t s_lo = nearest_src(col_first / ci, scale_w, Ws) * ci / V * V;
-    const int32_t s_hi = nearest_src(col_last / ci, scale_w, Ws) * ci + ci - 1;
+    const int32_t s_lo = nearest_src(col_first / ci, rule.scale_w, Ws, rule.rep_w) * ci / V * V;
+    const int32_t s_hi = nearest_src(col_last / ci, rule.scale_w, Ws, rule.rep_w) * ci + ci - 1;
     const uint32_t seg_bytes = (uint32_t)((s_hi - s_lo) / V + 1) * 16u;
     const bool use_lds = seg_bytes <= slot_bytes;  // uniform; the launch sizes the slots so that this holds
     const int32_t e0 = col_first + tid * V;
@@ -634,7 +644,7 @@ __global__ __launch_bounds__(kThreads) void resize_nearest_lds_kernel(const T* _
     for (int i = 0; i < V; i++) {
         const int32_t c = (e0 + i < Wde) ? e0 + i : Wde - 1;
         const int32_t px = (ci == 1) ? c : c / ci;
-        src_col[i] = nearest_src(px, scale_w, Ws) * ci + (c - px * ci);
+        src_col[i] = nearest_src(px, rule.scale_w, Ws, rule.rep_w) * ci + (c - px * ci);
     }
     const int64_t rows = outer * Hd;
     for (int64_t r0 = (int64_t)blockIdx.y * kNearestBand; r0 < rows; r0 += (int64_t)gridDim.y * kNearestBand) {
@@ -648,7 +658,7 @@ __global__ __launch_bounds__(kThreads) void resize_nearest_lds_kernel(const T* _
             if (r < rows) {
                 const int64_t o = r / Hd;
                 const int32_t h = (int32_t)(r - o * Hd);
-                src_row[j] = o * Hs + nearest_src(h, scale_h, Hs);
+                src_row[j] = o * Hs + nearest_src(h, rule.scale_h, Hs, rule.rep_h);
                 if (src_row[j] != prev) {
                     if (use_lds) {
                         const char* src = reinterpret_cast<const char*>(x + src_row[j] * (int64_t)Wse + s_lo);
@@ -933,15 +943,15 @@ hipError_t run_resize(const ResizeArgs& a, hipStream_t stream)
         dim3 grid((unsigned)((lanes + kThreads - 1) / kThreads), (unsigned)(bands < 65535 ? bands : 65535));
 #define OPSCV_NEAREST(NHWC_, VEC_)                                                                                  \
     hipLaunchKernelGGL((resize_nearest_kernel<T, NHWC_, VEC_>), grid, dim3(kThreads), 0, stream, x, y, outer,      \
-                       (int32_t)a.C, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h, a.scale_w, \
-                       streaming)
+                       (int32_t)a.C, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, rule, streaming)
         const int streaming = (out_elems * (int64_t)sizeof(T) >= (128ll << 20)) ? 1 : 0;
+        const NearestRule rule{a.scale_h, a.scale_w, a.rep_h, a.rep_w};
         if (const uint64_t slot = nearest_lds_slot<T>(a)) {
             const int64_t vlanes = (row_elems + V - 1) / V;
             dim3 lgrid((unsigned)((vlanes + kThreads - 1) / kThreads), (unsigned)(bands < 65535 ? bands : 65535));
             hipLaunchKernelGGL((resize_nearest_lds_kernel<T>), lgrid, dim3(kThreads), slot * kNearestBand, stream, x, y,
-                               outer, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, a.scale_h, a.scale_w,
-                               (uint32_t)slot, streaming, (int32_t)(nhwc ? a.C : 1));
+                               outer, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, rule, (uint32_t)slot,
+                               streaming, (int32_t)(nhwc ? a.C : 1));
             return hipGetLastError();
         }
         if (nhwc) {

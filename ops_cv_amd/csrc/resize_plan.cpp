@@ -101,11 +101,60 @@ int64_t reference_vector_cores()
     return 64;  // the core count of the reference's tiling unit test (test_resize_bilinear_v2_tiling.cpp: {64, 245760})
 }
 
+// bytes of the reference device's unified buffer: OPSCV_REFERENCE_UB_BYTES, else that of the reference's tiling unit
+// test (test_resize_nearest_neighbor_v2_tiling.cpp: {64, 253952})
+static int64_t reference_ub_bytes()
+{
+    if (const char* v = getenv("OPSCV_REFERENCE_UB_BYTES")) {
+        const long long n = strtoll(v, nullptr, 10);
+        if (n > 0) {
+            return n;
+        }
+    }
+    return 253952;
+}
+
+// Whether the reference resizes this channels-last tensor with the template that replicates every source pixel a
+// whole number of times (IsMatchTiling_NHWC_UB2UB, resize_nearest_neighbor_v2_tiling_base.cpp:640-665, called with
+// align_corners = half_pixel_centers = false and no scales, aclnn_resize.cpp:278): an upscale by whole factors, 128
+// bytes of channels or more per pixel, a source row and an output row that fit the unified buffer twice, tensors under
+// 2^32 elements.  That template's index is destination / factor in integer arithmetic
+// (resize_nearest_neighbor_v2_data_copy_nhwc.h:205-231); floor(float(destination) * scale), the rule of every other
+// template, first differs from it at a factor of 41.
+static bool nearest_replicates(const ResizeArgs& a)
+{
+    if (!a.channels_last || a.Wd <= a.Ws || a.Hd < a.Hs || a.Wd % a.Ws != 0 || a.Hd % a.Hs != 0) {
+        return false;
+    }
+    const int64_t esz = elem_size(a.elem), block = 32;
+    const int64_t c_bytes = a.C * esz;
+    const bool whole_blocks = c_bytes % block == 0;
+    const int64_t c_padded = (c_bytes + block - 1) / block * block / esz;  // channels rounded up to whole blocks
+    if (whole_blocks ? c_padded * a.Ws * esz < 256 : c_bytes < 128) {
+        return false;
+    }
+    if ((a.Ws + a.Wd) * c_padded * esz * 2 > reference_ub_bytes()) {
+        return false;
+    }
+    if (a.N * a.C * a.Hs * a.Ws >= (int64_t)UINT32_MAX || a.N * a.C * a.Hd * a.Wd >= (int64_t)UINT32_MAX) {
+        return false;
+    }
+    if (whole_blocks && a.Wd * c_bytes < 4096) {
+        return false;
+    }
+    return a.Hd / a.Hs <= INT32_MAX && a.Wd / a.Ws <= INT32_MAX;
+}
+
 void plan_resize_nearest(ResizeArgs* a)
 {
     a->half_pixel = 0;
     a->scale_h = (float)a->Hs / (float)a->Hd;
     a->scale_w = (float)a->Ws / (float)a->Wd;
+    a->rep_h = a->rep_w = 0;
+    if (nearest_replicates(*a)) {
+        a->rep_h = (int32_t)(a->Hd / a->Hs);
+        a->rep_w = (int32_t)(a->Wd / a->Ws);
+    }
     a->mode = ResizeMode::Nearest;
     if (a->Hs == a->Hd && a->Ws == a->Wd) {
         a->mode = ResizeMode::Copy;  // every index maps to itself: floor(i * 1.0f) = i

@@ -22,6 +22,9 @@ int64_t reference_vector_cores();
 // Nearest-neighbour resize with align_corners = false and half_pixel_centers = false, the only combination
 // aclnnResize requests (image/resize_bilinear_v2/op_api/aclnn_resize.cpp:286-288): scale = in / out
 // (image/resize_nearest_neighbor_v2/op_host/arch35/resize_nearest_neighbor_v2_tiling_base.cpp:253-263).
+// Sets rep_h / rep_w where the reference would take its replicating channels-last template (:640-665), whose index is
+// destination / factor; that choice reads the size of the reference device's unified buffer, 253952 bytes unless
+// OPSCV_REFERENCE_UB_BYTES says otherwise.
 void plan_resize_nearest(ResizeArgs* a);
 
 }  // namespace opscv

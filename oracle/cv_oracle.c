@@ -27,6 +27,10 @@
  *                                  it by its zero weight too)
  *   oracle_resize_nearest        : integer-factor upscales equal element repetition, committed and live
  *                                  torch interpolate(mode="nearest") comparison (bit-exact: a pure copy)
+ *   oracle_nearest_nhwc_schedule : the strategies the reference's tiling UT names for its channels-last cases
+ *                                  (test_resize_nearest_neighbor_v2_tiling.cpp, tests 03-07, 11, 14, 15, platform
+ *                                  {64 cores, 253952 bytes}); the replicating rule it switches oracle_resize_nearest
+ *                                  to: numpy repeat, and the one place it leaves the float rule (factor 41)
  *   oracle_upsample_bilinear2d_backward : adjointness with the forward oracle (<forward(x), g> = <x, backward(g)>),
  *                                  gradient mass conservation, x2 closed form, live torch autograd comparison
  *   oracle_grid_sampler3d        : identity grid reproduces the volume, a grid constant in z reduces to the 2-D
@@ -721,6 +725,61 @@ static inline int64_t nearest_src(int64_t d, float scale, int64_t len_src)
     return (i < len_src - 1) ? i : len_src - 1;
 }
 
+static int64_t g_reference_ub_bytes = 253952;
+
+void oracle_set_reference_ub_bytes(int64_t bytes)
+{
+    g_reference_ub_bytes = bytes > 0 ? bytes : 253952;
+}
+
+static int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+/* resize_nearest_neighbor_v2_tiling_base.cpp:640-665 (IsMatchTiling_NHWC_UB2UB), 476-494 (IsMatchTiling_NHWC) and
+ * 667-713 (MatchTilingStrategyAndSetTilingKey) for a channels-last tensor with align_corners = half_pixel_centers =
+ * false and no scales given, which is how aclnnResize calls the operator (aclnn_resize.cpp:278). */
+int oracle_nearest_nhwc_schedule(int dtype, int64_t N, int64_t C, int64_t Hs, int64_t Ws, int64_t Hd, int64_t Wd)
+{
+    const int64_t esz = (dtype == ORACLE_F32) ? 4 : 2;
+    const int64_t block = 32; /* bytes of a unified-buffer block */
+    const int64_t ub = g_reference_ub_bytes, cores = g_reference_cores;
+    const int aligned = (C * esz) % block == 0;                     /* :233-236 */
+    const int64_t c_align = ceil_div64(C * esz, block) * block / esz; /* :237 */
+    int ub2ub = 1;
+    if (Wd <= Ws || Hd < Hs || Wd % Ws != 0 || Hd % Hs != 0) {
+        ub2ub = 0; /* an upscale by whole factors only */
+    } else if ((c_align * Ws * esz < 128 * 2 && c_align == C) || (C * esz < 128 && c_align != C)) {
+        ub2ub = 0; /* few channels */
+    } else if ((Ws + Wd) * c_align * esz * 2 > ub) {
+        ub2ub = 0; /* a source row and an output row, double-buffered, do not fit */
+    } else if (N * C * Hs * Ws >= (int64_t)UINT32_MAX || N * C * Hd * Wd >= (int64_t)UINT32_MAX) {
+        ub2ub = 0;
+    } else if (aligned && Wd * C * esz < 4096) {
+        ub2ub = 0; /* short rows */
+    }
+    if (ub2ub) {
+        const int64_t in_ub = Ws * c_align * esz * 2;
+        const int64_t out_ub = (Hd / Hs) * Wd * c_align * esz * 2;
+        int sch = (in_ub + out_ub <= ub) ? 6 : 7;
+        const int64_t n_factor = ceil_div64(N, cores), n_cores = ceil_div64(N, n_factor);
+        const int64_t h_factor = ceil_div64(Hs, cores), h_cores = ceil_div64(Hs, h_factor);
+        if (n_cores < cores && h_cores < cores) {
+            sch = 8;
+        }
+        return sch;
+    }
+    if (C * esz >= 128) {
+        const int64_t max_ub_num = ((ub / 2) / block) * block / esz;
+        if (aligned && (N * c_align < max_ub_num || C * esz < 256)) {
+            return 2;
+        }
+        return (c_align <= max_ub_num) ? 0 : 1;
+    }
+    if (Hs == Hd && Ws == Wd) {
+        return 4;
+    }
+    return (Hs == 1 && Ws == 1) ? 5 : 3;
+}
+
 int oracle_resize_nearest(const void* x, void* y, int dtype, int64_t N, int64_t C, int64_t Hs, int64_t Ws,
                           int64_t Hd, int64_t Wd, int channels_last)
 {
@@ -731,14 +790,25 @@ int oracle_resize_nearest(const void* x, void* y, int dtype, int64_t N, int64_t 
     /* resize_nearest_neighbor_v2_tiling_base.cpp:257,262 */
     const float scale_h = (float)Hs / (float)Hd;
     const float scale_w = (float)Ws / (float)Wd;
+    /* Schedules 6-8 replicate every source pixel Hd / Hs times down and Wd / Ws times across
+     * (resize_nearest_neighbor_v2_data_copy_nhwc.h:110-111,205-231): output (h, w) is source (h / kh, w / kw) in
+     * integer arithmetic, which floor(float(w) * scale) first misses at a factor of 41 (w = 41 gives 0). */
+    int64_t rep_h = 0, rep_w = 0;
+    if (channels_last) {
+        const int sch = oracle_nearest_nhwc_schedule(dtype, N, C, Hs, Ws, Hd, Wd);
+        if (sch >= 6 && sch <= 8) {
+            rep_h = Hd / Hs;
+            rep_w = Wd / Ws;
+        }
+    }
     const char* src = (const char*)x;
     char* dst = (char*)y;
     for (int64_t n = 0; n < N; n++) {
         for (int64_t c = 0; c < C; c++) {
             for (int64_t h = 0; h < Hd; h++) {
-                const int64_t sy = nearest_src(h, scale_h, Hs);
+                const int64_t sy = rep_h ? h / rep_h : nearest_src(h, scale_h, Hs);
                 for (int64_t w = 0; w < Wd; w++) {
-                    const int64_t sx = nearest_src(w, scale_w, Ws);
+                    const int64_t sx = rep_w ? w / rep_w : nearest_src(w, scale_w, Ws);
                     int64_t so, dof;
                     if (channels_last) {
                         so = ((n * Hs + sy) * Ws + sx) * C + c;

@@ -107,9 +107,19 @@ int oracle_upsample_bilinear2d(const void* x, void* y, int dtype, int64_t N, int
  * (image/resize_nearest_neighbor_v2/op_kernel/arch35/resize_nearest_neighbor_v2_simt.h:103-124, scale rule
  * image/resize_nearest_neighbor_v2/op_host/arch35/resize_nearest_neighbor_v2_tiling_base.cpp:253-263).
  * channels_last = 0: x is (N,C,Hs,Ws); 1: x is (N,Hs,Ws,C).
+ * One of the reference's channels-last templates does not use that rule: for an upscale by whole factors with
+ * enough channels and rows that fit its unified buffer it replicates every source pixel (src = dst / factor in
+ * integer arithmetic, resize_nearest_neighbor_v2_data_copy_nhwc.h:110-111,205-231); the float rule first differs from
+ * that at a factor of 41.  oracle_nearest_nhwc_schedule restates the choice
+ * (resize_nearest_neighbor_v2_tiling_base.cpp:476-494,640-713; returns the schedule id of
+ * resize_nearest_neighbor_v2_tiling_key.h, 6-8 are the replicating template) for the core count of
+ * oracle_set_reference_cores and the buffer size of oracle_set_reference_ub_bytes (default 253952, that of the
+ * reference's tiling UT); oracle_resize_nearest follows it for channels_last = 1.
  */
 int oracle_resize_nearest(const void* x, void* y, int dtype, int64_t N, int64_t C, int64_t Hs, int64_t Ws,
                           int64_t Hd, int64_t Wd, int channels_last);
+int oracle_nearest_nhwc_schedule(int dtype, int64_t N, int64_t C, int64_t Hs, int64_t Ws, int64_t Hd, int64_t Wd);
+void oracle_set_reference_ub_bytes(int64_t bytes);
 
 /*
  * Backward of the bilinear resize, deterministic gather formulation

@@ -102,6 +102,10 @@ def lib():
     L.oracle_grid_sampler3d_backward.argtypes = [vp] * 5 + [ctypes.c_int] + [i64] * 8 + [ctypes.c_int] * 3
     L.oracle_set_reference_cores.restype = None
     L.oracle_set_reference_cores.argtypes = [i64]
+    L.oracle_set_reference_ub_bytes.restype = None
+    L.oracle_set_reference_ub_bytes.argtypes = [i64]
+    L.oracle_nearest_nhwc_schedule.restype = ctypes.c_int
+    L.oracle_nearest_nhwc_schedule.argtypes = [ctypes.c_int, i64, i64, i64, i64, i64, i64]
     L.oracle_resize_uses_hw_split.restype = ctypes.c_int
     L.oracle_resize_uses_hw_split.argtypes = [i64] * 6
     L.oracle_upsample_bilinear2d_nhwc.restype = ctypes.c_int
@@ -326,6 +330,16 @@ def upsample_bilinear2d_a2(x, out_hw, align=False):
 def set_reference_cores(cores):
     """vector cores of the device the reference would run on (its NCHW template choice depends on it); 0 -> default"""
     lib().oracle_set_reference_cores(int(cores))
+
+
+def set_reference_ub_bytes(n):
+    """unified-buffer bytes of the device the reference would run on (gates its replicating nearest template); 0 -> default"""
+    lib().oracle_set_reference_ub_bytes(int(n))
+
+
+def nearest_nhwc_schedule(dtype_code, N, C, Hs, Ws, Hd, Wd):
+    """schedule id the reference's tiling picks for a channels-last nearest resize (6-8: the replicating template)"""
+    return int(lib().oracle_nearest_nhwc_schedule(dtype_code, N, C, Hs, Ws, Hd, Wd))
 
 
 def resize_uses_hw_split(N, C, Hs, Ws, Hd, Wd):

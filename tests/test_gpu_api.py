@@ -763,6 +763,68 @@ def test_resize_nearest_few_channels_last(oracle, device, aclnn, dtype):
 
 
 @pytest.mark.parametrize("dtype", I.DTYPES)
+def test_resize_nearest_replicating_template(oracle, device, aclnn, dtype, monkeypatch):
+    """nearest on channels-last images where the reference takes its replicating template (whole upscale factors,
+    128 bytes of channels or more, rows that fit its unified buffer): source = destination / factor, which the float
+    rule leaves at factors of 41 and up -- columns 41 and 82 of a 3 -> 123 upscale; next to it shapes that fail one
+    gate each and keep the float rule, and the unified-buffer size as an environment switch.  Pixels of whole vectors
+    (the gather from memory) and of 66 elements (the gather out of LDS)."""
+    import torch
+    rng = np.random.default_rng(322)
+    code = I.oracle_code(dtype)
+    esz = 4 if dtype == "fp32" else 2
+    wide = 128 // esz  # channels of 128 bytes
+    cases = [((2, 3, 3, wide), (6, 123)), ((1, 2, 3, 2 * wide), (2, 141)),     # x41, x47 along W
+             ((1, 1, 4, wide + 2), (41, 8)),                                    # x41 along H, pixels off the vector grid
+             ((1, 3, 3, wide // 2), (6, 123)),                                  # 64 bytes of channels: float rule
+             ((1, 3, 3, wide), (6, 124)),                                       # a factor that is not whole: float rule
+             ((1, 2, 3, 8 * wide), (2, 123))]                                   # rows beyond the buffer: float rule
+    replicating = [True, True, True, False, False, False]
+    for (shape, (Ho, Wo)), rep in zip(cases, replicating):
+        N, H, W, C = shape
+        assert (oracle.nearest_nhwc_schedule(code, N, C, H, W, Ho, Wo) in (6, 7, 8)) == rep, shape
+        x = I.cast_np(rng.standard_normal(shape).astype(np.float32), dtype)
+        ref = oracle.resize_nearest(x, (Ho, Wo), channels_last=True, dtype=code)
+        if rep:
+            assert np.array_equal(ref, np.repeat(np.repeat(x, Ho // H, axis=1), Wo // W, axis=2))
+        xt = I.to_torch(x, dtype, device)
+        out = torch.empty((N, Ho, Wo, C), dtype=xt.dtype, device=device)
+        y = aclnn.resize(xt, (1.0, Ho / H, Wo / W, 1.0), "nearest", out=out, channels_last=True)
+        torch.cuda.synchronize()
+        got = I.from_torch(y, dtype)
+        view = np.uint32 if dtype == "fp32" else np.uint16
+        assert np.array_equal(got.view(view), ref.view(view)), (shape, Ho, Wo, dtype)
+    # the same tensor as planes: the float rule, which differs at columns 41 and 82
+    x = I.cast_np(rng.standard_normal((1, 2, 3, wide)).astype(np.float32), dtype)
+    yl = aclnn.resize(I.to_torch(x, dtype, device), (1.0, 1.0, 41.0, 1.0), "nearest",
+                      out=torch.empty((1, 2, 123, wide), dtype=I.to_torch(x, dtype, device).dtype, device=device),
+                      channels_last=True)
+    xp = np.ascontiguousarray(x.transpose(0, 3, 1, 2))
+    yp = aclnn.resize(I.to_torch(xp, dtype, device), (1.0, 1.0, 1.0, 41.0), "nearest",
+                      out=torch.empty((1, wide, 2, 123), dtype=I.to_torch(x, dtype, device).dtype, device=device))
+    torch.cuda.synchronize()
+    gl, gp = I.from_torch(yl, dtype), I.from_torch(yp, dtype)
+    differ = [w for w in range(123) if not np.array_equal(gl[0, :, w, :], gp[0, :, :, w].T)]
+    assert differ == [41, 82]
+    # a larger unified buffer lets the last case above through
+    shape, (Ho, Wo) = cases[5]
+    N, H, W, C = shape
+    x = I.cast_np(rng.standard_normal(shape).astype(np.float32), dtype)
+    monkeypatch.setenv("OPSCV_REFERENCE_UB_BYTES", str(1 << 20))
+    oracle.set_reference_ub_bytes(1 << 20)
+    try:
+        ref = oracle.resize_nearest(x, (Ho, Wo), channels_last=True, dtype=code)
+        assert np.array_equal(ref, np.repeat(x, 41, axis=2))
+        xt = I.to_torch(x, dtype, device)
+        y = aclnn.resize(xt, (1.0, 1.0, 41.0, 1.0), "nearest",
+                         out=torch.empty((N, Ho, Wo, C), dtype=xt.dtype, device=device), channels_last=True)
+        torch.cuda.synchronize()
+        assert np.array_equal(I.from_torch(y, dtype), ref)
+    finally:
+        oracle.set_reference_ub_bytes(0)
+
+
+@pytest.mark.parametrize("dtype", I.DTYPES)
 def test_resize_point_copy(oracle, device, aclnn, dtype):
     """channels-last shrinks by whole factors take the reference's point-copy template: bit-exact copies, also of
     infinities and NaNs, through aclnnUpsampleBilinear2d and aclnnResize; vector and scalar channel counts"""

@@ -458,6 +458,66 @@ def test_resize_nearest_oracle(oracle):
                                         mode="nearest").numpy().astype(np.float16))
 
 
+def test_nearest_channels_last_replicating_template(oracle):
+    """resize_nearest_neighbor_v2_tiling_base.cpp:476-494,640-713: which template the reference picks for a
+    channels-last nearest resize, pinned on the strategies its tiling UT names for its own cases
+    (tests/ut/op_host/arch35/test_resize_nearest_neighbor_v2_tiling.cpp, platform {64 cores, 253952 bytes of unified
+    buffer}, fp32, shapes as (N, H, W, C)); and the rule of the replicating template
+    (resize_nearest_neighbor_v2_data_copy_nhwc.h:205-231): numpy's repeat, which the float rule leaves at a factor
+    of 41"""
+    ut = [  # (N, Hs, Ws, C) -> (Hd, Wd): does the UT name the replicating template ("UB2UB") for the case
+        ((64, 4, 32, 48), (4, 64), True),      # test 03: UB2UB W_OUT_ALL
+        ((2, 8, 32, 64), (16, 64), True),      # test 04: UB2UB CORE_NH
+        ((1, 8, 32, 64), (16, 75), False),     # test 05: a copy template (W factor not whole)
+        ((1, 4, 8, 128), (12, 20), False),     # test 06: a copy template
+        ((1, 2, 2, 128), (4, 5), False),       # test 07: a copy template
+        ((1, 8, 32, 63), (16, 75), False),     # test 11: a copy template, C not a whole block
+        ((1, 16, 64, 64), (8, 32), False),     # test 14: a downscale: "not-enlarged rejects UB2UB"
+        ((30, 100, 64, 128), (200, 128), True),  # test 15: UB2UB NOT_W_OUT_ALL
+    ]
+    # Which variant of the replicating template (6, 7, 8: how the work is cut) and which of the three copy templates
+    # (0, 1, 2) is taken changes no result, the UT asserts no key for these cases, and its comments on the variant do
+    # not always agree with the source (test 15 is named NOT_W_OUT_ALL, but 30 items and 50 row groups are both fewer
+    # than 64 cores, which tiling_base.cpp:679-685 sends to CORE_NH; test 11 says C = 63 was chosen to get past JHC,
+    # test 05 calls the same shape with C = 64 SmallC).  The restatement follows the source for the variant; what is
+    # asserted against the UT is the class, which decides the index rule.
+    for (N, Hs, Ws, C), (Hd, Wd), replicating in ut:
+        got = oracle.nearest_nhwc_schedule(0, N, C, Hs, Ws, Hd, Wd)
+        assert (got in (6, 7, 8)) == replicating and (replicating or got in (0, 1, 2)), (N, Hs, Ws, C, got)
+    assert oracle.nearest_nhwc_schedule(0, 64, 48, 4, 32, 4, 64) == 6   # test 03 also by variant: 64 items fill the cores
+    assert oracle.nearest_nhwc_schedule(0, 2, 64, 8, 32, 16, 64) == 8   # test 04 also by variant
+    # the gates of the replicating template, one at a time from a case that passes
+    base = dict(N=4, C=64, Hs=6, Ws=8, Hd=12, Wd=32)
+    sch = lambda **kw: oracle.nearest_nhwc_schedule(1, *[{**base, **kw}[k] for k in ("N", "C", "Hs", "Ws", "Hd", "Wd")])
+    assert sch() in (6, 7, 8)
+    assert sch(Wd=8) not in (6, 7, 8)            # W not enlarged
+    assert sch(Wd=36) not in (6, 7, 8)           # W factor not whole
+    assert sch(Hd=15) not in (6, 7, 8)           # H factor not whole
+    assert sch(Hd=3) not in (6, 7, 8)            # H reduced
+    assert sch(C=16) not in (6, 7, 8)            # 32 bytes of channels, a whole block, rows too short
+    assert sch(C=33) not in (6, 7, 8)            # 66 bytes of channels, not a whole block, under 128
+    assert sch(C=65) in (6, 7, 8)                # 130 bytes, not a whole block
+    assert sch(Ws=1, Wd=4, C=64) not in (6, 7, 8)   # source row under 256 bytes
+    assert sch(Ws=1, Wd=31) not in (6, 7, 8)     # aligned channels and an output row under 4096 bytes
+    assert sch(Ws=8, Wd=8 * 120, C=128) not in (6, 7, 8)  # (8 + 960) * 128 * 2 * 2 bytes do not fit the buffer
+    oracle.set_reference_ub_bytes(1 << 20)
+    assert sch(Ws=8, Wd=8 * 120, C=128) in (6, 7, 8)
+    oracle.set_reference_ub_bytes(0)
+    # the rule: repeat; and where the float rule differs
+    rng = np.random.default_rng(99)
+    x = rng.standard_normal((2, 3, 3, 64)).astype(np.float16)     # (N, H, W, C)
+    assert oracle.nearest_nhwc_schedule(1, 2, 64, 3, 3, 6, 123) in (6, 7, 8)
+    y = oracle.resize_nearest(x, (6, 123), channels_last=True)
+    assert np.array_equal(y, np.repeat(np.repeat(x, 2, axis=1), 41, axis=2))
+    yt = oracle.resize_nearest(np.ascontiguousarray(x.transpose(0, 3, 1, 2)), (6, 123))  # planes: the float rule
+    differ = [w for w in range(123) if not np.array_equal(yt[:, :, :, w], y[:, :, w, :].transpose(0, 2, 1))]
+    assert differ == [41, 82]  # floor(float(41) * float(3.0f / 123.0f)) = 0, not 1
+    x5 = rng.standard_normal((1, 4, 5, 64)).astype(np.float32)
+    y5 = oracle.resize_nearest(x5, (12, 35), channels_last=True)  # factors 3 and 7: both rules agree
+    assert oracle.nearest_nhwc_schedule(0, 1, 64, 4, 5, 12, 35) in (6, 7, 8)
+    assert np.array_equal(y5, np.repeat(np.repeat(x5, 3, axis=1), 7, axis=2))
+
+
 def test_upsample_backward_oracle(oracle):
     """resize_bilinear_v2_grad_simt_determine.h / _determine_scales.h: the gather form is the adjoint of the
     forward resize (<forward(x), g> = <x, backward(g)>), keeps the gradient mass when no source pixel is skipped,
