@@ -149,6 +149,9 @@ struct GridSampler3DGradArgs {
     // optional scratch of gs3d_grad_range_words() 32-bit words: the span of voxels every chunk of grid points
     // touches, which lets a band of the input gradient pass over the chunks that miss it; null: every chunk is looked at
     void* chunk_ranges = nullptr;
+    // optional scratch of gs3d_grad_list_words() 32-bit words, 16-byte aligned: cell slots and corner weights of the
+    // variant that gathers every voxel's contributions (gs3d_grad_lists.hip); null: the ordered kernel does all items
+    void* lists = nullptr;
 };
 
 enum class ResizeMode : int {

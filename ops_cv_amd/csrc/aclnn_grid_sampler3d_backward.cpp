@@ -210,12 +210,16 @@ aclnnStatus aclnnGridSampler3DBackwardGetWorkspaceSize(const aclTensor* gradOutp
         ex->out1 = plan_view(ex.get(), gridGrad, esz, true);
     }
     if (want_dx) {
-        // scratch of the input-gradient kernel: the voxel span of every chunk of grid points
-        const int64_t words = gs3d_grad_range_words(a);
-        if (words > 0) {
+        // scratch of the input-gradient kernels: the voxel span of every chunk of grid points, then (from the next
+        // 256-byte boundary) the cell slots and corner weights of the gather variant
+        const int64_t range_words = gs3d_grad_range_words(a);
+        const int64_t list_words = gs3d_grad_list_words(a);
+        if (range_words > 0 || list_words > 0) {
             ex->scratch.in_workspace = true;
             ex->scratch.ws_offset = (ex->workspace_bytes + 255) / 256 * 256;
-            ex->workspace_bytes = ex->scratch.ws_offset + (uint64_t)words * 4;
+            ex->workspace_bytes = ex->scratch.ws_offset + (list_words > 0 ? gs3d_grad_lists_offset(range_words) +
+                                                                                 (uint64_t)list_words * 4
+                                                                           : (uint64_t)range_words * 4);
         }
     }
     *workspaceSize = ex->workspace_bytes;

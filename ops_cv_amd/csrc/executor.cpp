@@ -134,7 +134,12 @@ aclnnStatus execute_plan(void* workspace, const aclOpExecutor* ex, aclrtStream s
         a.grid = resolve(ex->in2, workspace);
         a.dx = ex->want_out0 ? resolve(ex->out0, workspace) : nullptr;
         a.dgrid = ex->want_out1 ? resolve(ex->out1, workspace) : nullptr;
-        a.chunk_ranges = ex->scratch.in_workspace ? resolve(ex->scratch, workspace) : nullptr;
+        if (ex->scratch.in_workspace) {
+            char* scratch = static_cast<char*>(resolve(ex->scratch, workspace));
+            const int64_t range_words = gs3d_grad_range_words(a);
+            a.chunk_ranges = range_words > 0 ? scratch : nullptr;
+            a.lists = gs3d_grad_list_words(a) > 0 ? scratch + gs3d_grad_lists_offset(range_words) : nullptr;
+        }
         if (a.gout == nullptr || a.x == nullptr || a.grid == nullptr || (ex->want_out0 && a.dx == nullptr) ||
             (ex->want_out1 && a.dgrid == nullptr)) {
             set_error("%s: tensor data pointer is NULL", api);

@@ -102,7 +102,10 @@ const char* opscvExecutorVariant(const aclOpExecutor* executor)
             return lists ? (rings ? "gs2d_grad_lists_lds" : "gs2d_grad_lists")
                          : (rings ? "gs2d_grad_ordered_lds" : "gs2d_grad_ordered");
         }
-        case OpKind::GridSampler3DGrad: return "gs3d_grad_ordered";
+        case OpKind::GridSampler3DGrad:
+            // input gradient: a gather over every voxel's contributions, or elections in their order
+            return (executor->want_out0 && gs3d_grad_list_words(executor->gsg3) > 0) ? "gs3d_grad_lists"
+                                                                                      : "gs3d_grad_ordered";
         case OpKind::GridSampler3D:
             if (executor->gs3.channels_last) {
                 return executor->gs3.interp == 0 ? "gs3d_ndhwc_bilinear" : "gs3d_ndhwc_nearest";

@@ -22,119 +22,25 @@
 #include <type_traits>
 
 #include "gs2d_grad_math.hpp"
+#include "gs3d_grad_math.hpp"
 #include "kernels.hpp"
 
 namespace opscv {
 
 namespace {
 
-constexpr int kThreads = 256;  // also the chunk length of the accumulation order
+constexpr int kThreads = kChunkPoints3;  // a workgroup walks a chunk of the accumulation order, a lane per point
 constexpr uint32_t kLaneBits = 8;              // 256 points of a chunk
 constexpr uint32_t kKeyBits = kLaneBits + 3;   // ... times eight corners
 constexpr uint32_t kEpochMax = (1u << (32 - kKeyBits)) - 1;
 constexpr int kTagsMax = 4096;  // election tags of a band (bands of 8192 voxels share them in pairs: two workgroups per CU)
 constexpr int kBandMax = 8192;  // most voxels of the gradient a workgroup keeps in LDS
 
-struct Grad3Params {
-    int32_t C, D, H, W, points;
-    int32_t pad, align;
-    int32_t band_px;
-    int32_t items_per_core;
-    int32_t chunks;  // chunks a batch item is walked in, a possibly empty leading one included
-    int32_t tags;    // election tags, a power of two (tag_of)
-};
-
 // Tag of a band element.  Elements that share a tag are elected as if they were one; folding the high bits in keeps
 // neighbours along every axis (offsets 1, W, H * W, often powers of two) on different tags.
 __device__ __forceinline__ int32_t tag_of(int32_t off, int32_t tag_mask)
 {
     return (off ^ (off >> 10)) & tag_mask;
-}
-
-// Where the contributions of a grid point land in the (D, H, W) volume and with what weight.
-//   INTERP 0: eight corners, index = x-high + 2 * y-high + 4 * z-high; weight = rt<T>(wx * wy * wz)
-//   INTERP 1: one tap, weight 1
-// off[k] = -1 marks a corner outside the volume.
-template <typename T, int INTERP>
-struct GradTaps3 {
-    static constexpr int NT = (INTERP == 0) ? 8 : 1;
-    int32_t off[NT];
-    float w[NT];
-    float wx[2], wy[2], wz[2];  // per axis: weight of the low and of the high corner
-    int32_t x0, y0, z0;         // bilinear: the low corner
-    float mx, my, mz;           // chain-rule multipliers of the grid gradient
-};
-
-__device__ __forceinline__ int32_t next_index(int32_t i)
-{
-    return (i == INT32_MAX) ? i : i + 1;
-}
-
-template <typename T, int INTERP>
-__device__ __forceinline__ void decide_grad_taps3(GradTaps3<T, INTERP>& t, float gx, float gy, float gz, int32_t D,
-                                                  int32_t H, int32_t W, int pad, int align)
-{
-    // grid_sampler3_d_grad_simt_det.h:381-383
-    const float fx = source_index_set_grad<T>(gx, W, pad, align, &t.mx);
-    const float fy = source_index_set_grad<T>(gy, H, pad, align, &t.my);
-    const float fz = source_index_set_grad<T>(gz, D, pad, align, &t.mz);
-    if (INTERP == 1) {
-        // grid_sampler3_d_grad_simt_det.h:340-342
-        const int32_t xi = float_to_i32(__builtin_rintf(fx));
-        const int32_t yi = float_to_i32(__builtin_rintf(fy));
-        const int32_t zi = float_to_i32(__builtin_rintf(fz));
-        const bool in = (uint32_t)xi < (uint32_t)W && (uint32_t)yi < (uint32_t)H && (uint32_t)zi < (uint32_t)D;
-        t.off[0] = in ? (zi * H + yi) * W + xi : -1;
-        t.w[0] = 1.0f;
-        return;
-    }
-    // grid_sampler3_d_grad_simt_det.h:281-297
-    const int32_t x0 = float_to_i32(__builtin_floorf(fx));
-    const int32_t y0 = float_to_i32(__builtin_floorf(fy));
-    const int32_t z0 = float_to_i32(__builtin_floorf(fz));
-    const int32_t x1 = next_index(x0), y1 = next_index(y0), z1 = next_index(z0);
-    t.x0 = x0;
-    t.y0 = y0;
-    t.z0 = z0;
-    t.wx[0] = (float)x1 - fx;
-    t.wx[1] = fx - (float)x0;
-    t.wy[0] = (float)y1 - fy;
-    t.wy[1] = fy - (float)y0;
-    t.wz[0] = (float)z1 - fz;
-    t.wz[1] = fz - (float)z0;
-#pragma unroll
-    for (int k = 0; k < 8; k++) {
-        const int xs = k & 1, ys = (k >> 1) & 1, zs = k >> 2;
-        const int32_t cx = xs ? x1 : x0, cy = ys ? y1 : y0, cz = zs ? z1 : z0;
-        const bool in = (uint32_t)cx < (uint32_t)W && (uint32_t)cy < (uint32_t)H && (uint32_t)cz < (uint32_t)D;
-        t.off[k] = in ? (cz * H + cy) * W + cx : -1;
-        // the fp32 product is pinned before it is rounded to T (one rounding each, as in the reference)
-        t.w[k] = rt<T>(as_fp32_value(t.wx[xs] * t.wy[ys] * t.wz[zs]));
-    }
-}
-
-// What a corner adds: weight times incoming gradient in fp32, then rounded to the element type
-// (grid_sampler3_d_grad_simt_det.h:116-118,72-73).
-template <typename T, int INTERP>
-__device__ __forceinline__ float contribution3(float go, float w)
-{
-    if (INTERP == 1) {
-        return rt<T>(go);
-    }
-    return rt<T>(as_fp32_value(w * go));
-}
-
-// Thread of the chunk that holds the first grid point of batch item n.
-__device__ __forceinline__ int32_t chunk_phase(int64_t n, const Grad3Params& p)
-{
-    return (int32_t)(((n % p.items_per_core) * (int64_t)p.points) % kThreads);
-}
-
-// Chunks a batch item is walked in: with several items per core the first chunk of an item may start before its
-// first point.
-__host__ __device__ inline int32_t chunk_count(int64_t points, int64_t items_per_core)
-{
-    return (int32_t)(((items_per_core > 1 ? kThreads - 1 : 0) + points + kThreads - 1) / kThreads);
 }
 
 // Per (batch item, chunk): lowest and highest voxel any corner of the chunk's points lands on (lowest > highest for a
@@ -188,8 +94,14 @@ __global__ __launch_bounds__(kThreads) void gs3d_grad_range_kernel(const T* __re
 template <typename T, int INTERP, int CB>
 __global__ __launch_bounds__(kThreads) void gs3d_grad_input_kernel(const T* __restrict__ gout,
                                                                     const T* __restrict__ grid, T* __restrict__ dx,
-                                                                    const int32_t* __restrict__ ranges, Grad3Params p)
+                                                                    const int32_t* __restrict__ ranges, Grad3Params p,
+                                                                    const uint32_t* __restrict__ item_flags,
+                                                                    uint32_t flag_stride)
 {
+    // with item flags: only the items the gather variant left over (the same answer for the whole workgroup)
+    if (item_flags != nullptr && item_flags[(size_t)blockIdx.z * flag_stride] == 0u) {
+        return;
+    }
     using Taps = GradTaps3<T, INTERP>;
     constexpr int NT = Taps::NT;
     extern __shared__ uint32_t smem_u32[];
@@ -539,9 +451,22 @@ hipError_t launch_interp(const GridSampler3DGradArgs& a, hipStream_t stream)
             if (p.chunks > 0x7fffffff / 2) {
                 return hipErrorInvalidValue;
             }
+            ranges = (const int32_t*)a.chunk_ranges;
+        }
+        // The gather variant first, where it runs: it does every item but those with crowded cells or voxels, flags
+        // those, and notes the chunk spans on its way; the ordered kernel below then does the flagged items only.
+        const uint32_t* item_flags = nullptr;
+        uint32_t flag_stride = 0;
+        if (INTERP == 0) {
+            const hipError_t el = run_gs3d_grad_input_lists(a, p, const_cast<int32_t*>(ranges), stream, &item_flags,
+                                                            &flag_stride);
+            if (el != hipSuccess) {
+                return el;
+            }
+        }
+        if (ranges != nullptr && item_flags == nullptr) {
             hipLaunchKernelGGL((gs3d_grad_range_kernel<T, INTERP>), dim3((unsigned)p.chunks, (unsigned)a.N),
                                dim3(kThreads), 0, stream, (const T*)a.grid, (int32_t*)a.chunk_ranges, p);
-            ranges = (const int32_t*)a.chunk_ranges;
         }
         // more than the default 64 KB of dynamic LDS
         static std::atomic<uint32_t> lds_allowed{0}, lds_allowed_single{0};
@@ -557,11 +482,11 @@ hipError_t launch_interp(const GridSampler3DGradArgs& a, hipStream_t stream)
         if (grouped) {
             hipLaunchKernelGGL((gs3d_grad_input_kernel<T, INTERP, CBMAX>), grid, dim3(kThreads),
                                (size_t)p.tags * 4 + (size_t)p.band_px * CBMAX * sizeof(T), stream, (const T*)a.gout,
-                               (const T*)a.grid, (T*)a.dx, ranges, p);
+                               (const T*)a.grid, (T*)a.dx, ranges, p, item_flags, flag_stride);
         } else {
             hipLaunchKernelGGL((gs3d_grad_input_kernel<T, INTERP, 1>), grid, dim3(kThreads),
                                (size_t)p.tags * 4 + (size_t)p.band_px * sizeof(T), stream, (const T*)a.gout, (const T*)a.grid,
-                               (T*)a.dx, ranges, p);
+                               (T*)a.dx, ranges, p, item_flags, flag_stride);
         }
         const hipError_t e = hipGetLastError();
         if (e != hipSuccess) {

@@ -82,6 +82,11 @@ hipError_t launch_grid_sampler3d(const GridSampler3DArgs& a, hipStream_t stream)
 hipError_t launch_grid_sampler3d_grad(const GridSampler3DGradArgs& a, hipStream_t stream);
 // 32-bit words of GridSampler3DGradArgs::chunk_ranges that make the input gradient faster; 0 when it would not help
 int64_t gs3d_grad_range_words(const GridSampler3DGradArgs& a);
+// 32-bit words of GridSampler3DGradArgs::lists that the gather variant of the input gradient needs; 0 when the shape
+// does not qualify (gs3d_grad_lists.hip)
+int64_t gs3d_grad_list_words(const GridSampler3DGradArgs& a);
+// one scratch region holds both: the chunk spans at its start, the lists from this byte offset
+inline uint64_t gs3d_grad_lists_offset(int64_t range_words) { return ((uint64_t)range_words * 4 + 255) / 256 * 256; }
 
 // gather == true : strided view -> contiguous buffer;  false : contiguous buffer -> strided view
 hipError_t launch_strided_copy(const StridedView& v, void* contiguous, int elem_bytes, bool gather,

@@ -557,8 +557,11 @@ def test_grid_sampler3d_backward_status_codes(aclnn, desc):
     of aclnn_grid_sampler3d_backward.cpp:174-238"""
     INV, NULL = aclnn.ACLNN_ERR_PARAM_INVALID, aclnn.ACLNN_ERR_PARAM_NULLPTR
     # dtype_float16 / dtype_float32 / dtype_bf16: the unit test's shapes
-    for dt in (aclnn.ACL_FLOAT, aclnn.ACL_FLOAT16, aclnn.ACL_BF16):
-        assert _gsb3(aclnn, desc, dt=dt) == (0, 0, "gs3d_grad_ordered")
+    # bilinear asks for the scratch of the gather variant: per batch item four flag words, a count and eight 16-bit slots
+    # per cell of the (D+1) x (H+1) x (W+1) lattice of low corners (2 x 4 x 4 here), eight weights per grid point (4)
+    for dt, esz in ((aclnn.ACL_FLOAT, 4), (aclnn.ACL_FLOAT16, 2), (aclnn.ACL_BF16, 2)):
+        assert _gsb3(aclnn, desc, dt=dt) == (0, (4 + 32 + 4 * 32) * 4 + 4 * 8 * esz, "gs3d_grad_lists")
+        assert _gsb3(aclnn, desc, dt=dt, interp=1) == (0, 0, "gs3d_grad_ordered")
     # gradOutput_nullptr .. gridGrad_nullptr
     for missing in ("gout", "inp", "grid", "dx", "dgrid"):
         assert _gsb3(aclnn, desc, **{missing: None})[0] == NULL, missing
@@ -594,12 +597,15 @@ def test_grid_sampler3d_backward_status_codes(aclnn, desc):
     # channels-last: the format of input says where the channels are; such tensors are packed through the workspace
     nd = aclnn.ACL_FORMAT_NDHWC
     st, ws, v = _gsb3(aclnn, desc, gout=(1, 1, 2, 2, 5), inp=(1, 1, 3, 3, 5), fmt=nd)
-    assert st == 0 and v == "gs3d_grad_ordered" and ws >= (20 + 45 + 45) * 4
+    assert st == 0 and v == "gs3d_grad_lists" and ws >= (20 + 45 + 45) * 4
     assert _gsb3(aclnn, desc, gout=(1, 1, 2, 2, 4), inp=(1, 1, 3, 3, 5), fmt=nd)[0] == INV
     # volumes of more than one LDS band ask for scratch: two words per chunk of 256 grid points and batch item, only
-    # when the input gradient is wanted
+    # when the input gradient is wanted; the gather variant's scratch follows from the next 256-byte boundary
     big = dict(gout=(3, 1, 2, 30, 10), inp=(3, 1, 10, 30, 30), grid=(3, 2, 30, 10, 3))
-    assert _gsb3(aclnn, desc, **big)[:2] == (0, 3 * 3 * 2 * 4)
+    assert _gsb3(aclnn, desc, interp=1, **big)[:2] == (0, 3 * 3 * 2 * 4)
+    cells, points = 11 * 31 * 31, 600
+    per_item = ((4 + cells + 3) // 4 * 4 + 4 * cells) * 4 + points * 8 * 4
+    assert _gsb3(aclnn, desc, **big) == (0, 256 + 3 * per_item, "gs3d_grad_lists")
     assert _gsb3(aclnn, desc, mask=(False, True), **big)[:2] == (0, 0)
 
 

@@ -640,6 +640,76 @@ def test_grid_sampler3d_backward(oracle, device, aclnn, dtype, interp):
                         (what, N, C, D, H, W, Do, Ho, Wo, pad, align)
 
 
+@pytest.mark.parametrize("dtype", I.DTYPES)
+def test_grid_sampler3d_backward_gather_variant(oracle, device, aclnn, dtype, monkeypatch):
+    """The input gradient of the 3-D sampler as a gather over every voxel's contributions: bit for bit the oracle's
+    (chunk, corner, point) order on jittered lattices (about eight contributions per voxel), on denser grids (lists of
+    more than sixteen entries, some items handed to the ordered kernel because a voxel has more than 32), with one
+    piled-up item among lattice items, with channel counts around the group of four, and with more items than cores
+    (chunk boundaries that move from item to item).  Which items the gather did is read from the flag words it keeps
+    in the workspace, which is handed over full of ones."""
+    torch = _torch()
+    rng = np.random.default_rng(720)
+    code = I.oracle_code(dtype)
+    esz = 4 if dtype == "fp32" else 2
+
+    def lattice(N, Do, Ho, Wo, spread, jitter):
+        ax = [np.linspace(-1 + 1 / n, 1 - 1 / n, n) for n in (Do, Ho, Wo)]
+        gz, gy, gx = np.meshgrid(*ax, indexing="ij")
+        base = np.stack([gx, gy, gz], -1)[None].astype(np.float32)
+        g = base * rng.uniform(1 - spread, 1 + spread, (N, 1, 1, 1, 3)) + rng.uniform(-0.1, 0.1, (N, 1, 1, 1, 3))
+        return (g + rng.normal(0, jitter, g.shape)).astype(np.float32)
+
+    cases = [  # N, C, (D, H, W), (Do, Ho, Wo), kind, cores
+        (3, 5, (6, 12, 10), (6, 12, 10), "lattice", 2),
+        (2, 4, (5, 9, 33), (7, 12, 40), "dense", 64),
+        (3, 1, (4, 8, 8), (4, 8, 8), "mixed", 64),
+        (2, 6, (3, 20, 70), (3, 20, 70), "lattice", 64),
+        (5, 2, (4, 6, 6), (5, 8, 8), "dense", 2),
+        (5, 3, (5, 8, 8), (5, 8, 8), "lattice", 2),
+    ]
+    seen_gathered = seen_flagged = 0
+    try:
+        for (N, C, (D, H, W), (Do, Ho, Wo), kind, cores) in cases:
+            monkeypatch.setenv("OPSCV_REFERENCE_CORES", str(cores))
+            oracle.set_reference_cores(cores)
+            g32 = lattice(N, Do, Ho, Wo, 0.1, 0.03)
+            if kind == "mixed":
+                g32[1] = rng.choice(np.array([-0.5, 0.1, 0.6], np.float32), (Do, Ho, Wo, 3))
+            g = I.cast_np(g32, dtype)
+            x = I.cast_np(rng.standard_normal((N, C, D, H, W)).astype(np.float32), dtype)
+            go = I.cast_np(rng.standard_normal((N, C, Do, Ho, Wo)).astype(np.float32), dtype)
+            points, cells, vol = Do * Ho * Wo, (D + 1) * (H + 1) * (W + 1), D * H * W
+            for pad, align in ((0, False), (1, True), (2, False)):
+                ws = torch.full((64 << 20,), 0xFF, dtype=torch.uint8, device=device)
+                rdx, rdg = oracle.grid_sampler3d_backward(go, x, g, 0, pad, align, dtype=code)
+                dx, dg = aclnn.grid_sampler3d_backward(I.to_torch(go, dtype, device), I.to_torch(x, dtype, device),
+                                                       I.to_torch(g, dtype, device), 0, pad, align, workspace=ws)
+                torch.cuda.synchronize()
+                for got, ref, what in ((I.from_torch(dx, dtype), rdx, "dx"), (I.from_torch(dg, dtype), rdg, "dgrid")):
+                    assert np.array_equal(_bits(got, dtype), _bits(ref, dtype)), (what, kind, N, C, D, H, W, pad, align)
+                # the flag word of every item: first word of its scratch, behind the chunk spans (none for one band)
+                per_core = (N + cores - 1) // cores if N > cores else 1
+                chunks = ((255 if per_core > 1 else 0) + points + 255) // 256
+                range_bytes = N * 2 * chunks * 4 if vol > 2048 else 0  # bands of 2048 voxels or more
+                item_words = (((4 + cells + 3) // 4 * 4 + 4 * cells) * 4 + points * 8 * esz + 15) // 16 * 4
+                words = ws.view(torch.int32)
+                flags = [int(words[(range_bytes + 255) // 256 * 64 + n * item_words].item()) for n in range(N)]
+                assert all(f in (0, 1) for f in flags), flags
+                # (border and reflection padding fold the points beyond the volume onto its faces, edges and corners,
+                # which may crowd a cell there: only zeros padding keeps a lattice item's cells sparse for certain)
+                if kind == "mixed" and pad == 0:
+                    assert flags == [0, 1, 0], flags
+                if kind == "lattice" and pad == 0:
+                    assert flags == [0] * N, flags
+                seen_gathered += flags.count(0)
+                seen_flagged += flags.count(1)
+    finally:
+        oracle.set_reference_cores(64)
+        monkeypatch.delenv("OPSCV_REFERENCE_CORES")
+    assert seen_gathered > 0 and seen_flagged > 0
+
+
 def test_grid_sampler3d_backward_core_split_mask_layouts_and_torch(oracle, device, aclnn, monkeypatch):
     torch = _torch()
     import torch.nn.functional as F
