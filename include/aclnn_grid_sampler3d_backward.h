@@ -16,6 +16,8 @@
  *                       (N,D,H,W,C) extents, anything else (N,C,D,H,W)
  *   outputMask        : exactly two flags; a NULL mask or two false flags make the call a successful no-op
  *   views             : arbitrary strides/offsets are honoured (packed through the workspace)
+ *   workspace         : also asked for with dense tensors when inputGrad is wanted (scratch of the kernels: cell slots,
+ *                       corner weights and regrouped gradOutput of the bilinear gather, voxel spans of the chunks)
  * The result is deterministic: every element of inputGrad is the sum of its contributions in the order of the
  * reference's deterministic mode (grid points in chunks of 256; per chunk corner after corner, per corner point after
  * point; every add rounded to the tensor's element type).

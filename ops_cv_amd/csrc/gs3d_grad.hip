@@ -284,6 +284,8 @@ __global__ __launch_bounds__(kThreads) void gs3d_grad_grid_kernel(const T* __res
     if (idx >= total) {
         return;
     }
+    (void)gout;
+    (void)x;
     if (INTERP == 1) {
         // grid_sampler3_d_grad_simt_det.h:354-356
         ElemIO<T>::store(dgrid + 3 * idx, 0.0f);
@@ -291,113 +293,15 @@ __global__ __launch_bounds__(kThreads) void gs3d_grad_grid_kernel(const T* __res
         ElemIO<T>::store(dgrid + 3 * idx + 2, 0.0f);
         return;
     }
-    const int32_t points = p.points;
-    const int64_t n = idx / points;
-    const int32_t pt = (int32_t)(idx - n * points);
-    Taps tp;
-    decide_grad_taps3<T, INTERP>(tp, ElemIO<T>::load(grid + 3 * idx), ElemIO<T>::load(grid + 3 * idx + 1),
-                                 ElemIO<T>::load(grid + 3 * idx + 2), p.D, p.H, p.W, p.pad, p.align);
-    const int32_t vol = p.D * p.H * p.W;
-    const T* x_n = x + n * p.C * (int64_t)vol;
-    const T* go_n = gout + n * p.C * (int64_t)points + pt;
-    float gix = 0.0f, giy = 0.0f, giz = 0.0f;
-    bool ok[8];
-    int32_t o[8];
-#pragma unroll
-    for (int k = 0; k < 8; k++) {
-        ok[k] = tp.off[k] >= 0;
-        o[k] = ok[k] ? tp.off[k] : 0;
+    if constexpr (INTERP == 0) {
+        const int32_t points = p.points;
+        const int64_t n = idx / points;
+        const int32_t pt = (int32_t)(idx - n * points);
+        Taps tp;
+        decide_grad_taps3<T, INTERP>(tp, ElemIO<T>::load(grid + 3 * idx), ElemIO<T>::load(grid + 3 * idx + 1),
+                                     ElemIO<T>::load(grid + 3 * idx + 2), p.D, p.H, p.W, p.pad, p.align);
+        gs3d_point_grid_gradient<T>(tp, gout, x, dgrid, idx, n, pt, p);
     }
-    // grid_sampler3_d_grad_simt_det.h:119-124 and the seven corners after it: value times two distances times the
-    // incoming gradient, left to right, subtracted for a low corner of the axis and added for a high one
-    auto accumulate = [&](float go, const float* v) {
-#pragma unroll
-        for (int k = 0; k < 8; k++) {
-            const int xs = k & 1, ys = (k >> 1) & 1, zs = k >> 2;
-            if (ok[k]) {
-                const float tx = v[k] * tp.wy[ys] * tp.wz[zs] * go;
-                const float ty = v[k] * tp.wx[xs] * tp.wz[zs] * go;
-                const float tz = v[k] * tp.wx[xs] * tp.wy[ys] * go;
-                gix = xs ? gix + tx : gix - tx;
-                giy = ys ? giy + ty : giy - ty;
-                giz = zs ? giz + tz : giz - tz;
-            }
-        }
-    };
-    // The sums run over the channels in order; the loads do not depend on them and are issued a group ahead.
-    constexpr int U = 4;
-    int32_t c = 0;
-    if (p.W >= 2) {
-        // The low and high corner along x are neighbours in memory: one load of two elements (aligned to one element
-        // only) per row of corners instead of two halves the addresses the gather puts through the memory pipeline.
-        // The pair sits at column pb = clamp(x0, 0, W - 2), so it never leaves the row; which half is which corner
-        // follows from pb.  Corners outside the volume are skipped by accumulate() as before.
-        using PairBits = typename std::conditional<sizeof(T) == 2, uint32_t, uint64_t>::type;
-        const int32_t pb = (tp.x0 < 0) ? 0 : ((tp.x0 > p.W - 2) ? p.W - 2 : tp.x0);
-        const bool lo_w = (tp.x0 == pb), lo_e = (next_index(tp.x0) == pb);
-        int32_t rowoff[4];
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            const int32_t cy = (r & 1) ? next_index(tp.y0) : tp.y0, cz = (r >> 1) ? next_index(tp.z0) : tp.z0;
-            const bool in = (uint32_t)cy < (uint32_t)p.H && (uint32_t)cz < (uint32_t)p.D;
-            rowoff[r] = in ? (cz * p.H + cy) * p.W + pb : 0;
-        }
-        for (; c + U <= p.C; c += U) {
-            float go[U];
-            PairBits pr[U][4];
-#pragma unroll
-            for (int u = 0; u < U; u++) {
-                const T* xc = x_n + (int64_t)(c + u) * vol;
-                go[u] = ElemIO<T>::load(go_n + (int64_t)(c + u) * points);
-#pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    __builtin_memcpy(&pr[u][r], xc + rowoff[r], sizeof(PairBits));
-                }
-            }
-#pragma unroll
-            for (int u = 0; u < U; u++) {
-                float v[8];
-#pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    T two[2];
-                    __builtin_memcpy(two, &pr[u][r], sizeof(PairBits));
-                    const float lo = ElemIO<T>::load(&two[0]), hi = ElemIO<T>::load(&two[1]);
-                    v[2 * r] = lo_w ? lo : hi;
-                    v[2 * r + 1] = lo_e ? lo : hi;
-                }
-                accumulate(go[u], v);
-            }
-        }
-    }
-    for (; c + U <= p.C; c += U) {
-        float go[U], v[U][8];
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            const T* xc = x_n + (int64_t)(c + u) * vol;
-            go[u] = ElemIO<T>::load(go_n + (int64_t)(c + u) * points);
-#pragma unroll
-            for (int k = 0; k < 8; k++) {
-                v[u][k] = ElemIO<T>::load(xc + o[k]);
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            accumulate(go[u], v[u]);
-        }
-    }
-    for (; c < p.C; c++) {
-        const T* xc = x_n + (int64_t)c * vol;
-        float v[8];
-#pragma unroll
-        for (int k = 0; k < 8; k++) {
-            v[k] = ElemIO<T>::load(xc + o[k]);
-        }
-        accumulate(ElemIO<T>::load(go_n + (int64_t)c * points), v);
-    }
-    // grid_sampler3_d_grad_simt_det.h:324-326: product in fp32, then the conversion
-    ElemIO<T>::store(dgrid + 3 * idx, as_fp32_value(tp.mx * gix));
-    ElemIO<T>::store(dgrid + 3 * idx + 1, as_fp32_value(tp.my * giy));
-    ElemIO<T>::store(dgrid + 3 * idx + 2, as_fp32_value(tp.mz * giz));
 }
 
 // Voxels per band.  Every workgroup is a chain of dependent LDS round trips, so the chip is filled by workgroups
@@ -435,6 +339,7 @@ hipError_t launch_interp(const GridSampler3DGradArgs& a, hipStream_t stream)
     while (p.tags < p.band_px && p.tags < kTagsMax) {
         p.tags *= 2;
     }
+    bool dgrid_done = false;  // the gather variant's first kernel computes the grid gradient on its way
     if (a.dx != nullptr) {
         const int64_t bands = (vol + p.band_px - 1) / p.band_px;
         // 8 bytes of gradient per band voxel: 4 channels of a 16-bit type, 2 of fp32 (96 KB of LDS with the election
@@ -459,7 +364,7 @@ hipError_t launch_interp(const GridSampler3DGradArgs& a, hipStream_t stream)
         uint32_t flag_stride = 0;
         if (INTERP == 0) {
             const hipError_t el = run_gs3d_grad_input_lists(a, p, const_cast<int32_t*>(ranges), stream, &item_flags,
-                                                            &flag_stride);
+                                                            &flag_stride, &dgrid_done);
             if (el != hipSuccess) {
                 return el;
             }
@@ -493,7 +398,7 @@ hipError_t launch_interp(const GridSampler3DGradArgs& a, hipStream_t stream)
             return e;
         }
     }
-    if (a.dgrid != nullptr) {
+    if (a.dgrid != nullptr && !dgrid_done) {
         const int64_t total = a.N * (int64_t)p.points;
         const int64_t blocks = (total + kThreads - 1) / kThreads;
         if (blocks > INT32_MAX) {

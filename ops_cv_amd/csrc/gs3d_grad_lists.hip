@@ -25,6 +25,8 @@
 // fp16 22x4x16x64x64 with a registration-style warp: 297 us (ordered kernel) -> see the profile of that workload.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "gs3d_grad_math.hpp"
 #include "kernels.hpp"
 
@@ -46,19 +48,22 @@ struct Lists3Layout {
                       // cell's 16-byte slot record made the slots kernel 17 us slower on fp16 22x4x16x64x64)
     uint32_t slots;   // kCellSlots 16-bit point numbers per cell and two unused ones: one 16-byte load per cell
     uint32_t wts;     // eight weights of the element type per point
+    uint32_t go4;     // gradOutput with the channels of a group of four side by side: [group][point][4]
     uint32_t item_words;
 };
 
 inline uint32_t align4(uint64_t v) { return (uint32_t)((v + 3u) & ~(uint64_t)3u); }
 
-Lists3Layout make_layout(int64_t cells, int64_t points, int64_t esz)
+Lists3Layout make_layout(int64_t cells, int64_t points, int64_t esz, int64_t channels)
 {
     Lists3Layout l;
     l.flag = 0;
     l.counts = 4;
     l.slots = align4((uint64_t)l.counts + (uint64_t)cells);
     l.wts = align4((uint64_t)l.slots + (uint64_t)cells * 4);
-    l.item_words = align4((uint64_t)l.wts + (uint64_t)points * 8 * (uint64_t)esz / 4);
+    l.go4 = align4((uint64_t)l.wts + (uint64_t)points * 8 * (uint64_t)esz / 4);
+    const uint64_t groups = ((uint64_t)channels + kChanBlock - 1) / kChanBlock;
+    l.item_words = align4((uint64_t)l.go4 + groups * (uint64_t)points * kChanBlock * (uint64_t)esz / 4);
     return l;
 }
 
@@ -84,11 +89,15 @@ __global__ __launch_bounds__(256) void gs3d_lists_clear_kernel(uint32_t* __restr
     }
 }
 
-template <typename T>
+// GRID: the lane goes on to the gradient of its grid point -- the corner decisions are the same, and the atomics
+// and stores above are on their way while the corners of the input are read.
+template <typename T, bool GRID>
 __global__ __launch_bounds__(kLThreads) void gs3d_lists_slots_kernel(const T* __restrict__ grid,
+                                                                      const T* __restrict__ gout,
                                                                       uint32_t* __restrict__ ws,
                                                                       int32_t* __restrict__ ranges, Grad3Params p,
-                                                                      Lists3Layout lay, int32_t N)
+                                                                      Lists3Layout lay, int32_t N,
+                                                                      const T* __restrict__ x, T* __restrict__ dgrid)
 {
     using Taps = GradTaps3<T, 0>;
     __shared__ int32_t s_lo[kLThreads / 64], s_hi[kLThreads / 64];
@@ -122,6 +131,26 @@ __global__ __launch_bounds__(kLThreads) void gs3d_lists_slots_kernel(const T* __
             reinterpret_cast<uint4*>(wts)[0] = reinterpret_cast<const uint4*>(w8)[0];
             reinterpret_cast<uint4*>(wts)[1] = reinterpret_cast<const uint4*>(w8)[1];
         }
+        // gradOutput of the point, four channels side by side: the gather then takes them with one load (past the
+        // last channel the last one again, never used)
+        {
+            const T* go_n = gout + n * p.C * (int64_t)p.points + pt;
+            T* go4 = reinterpret_cast<T*>(wsn + lay.go4);
+            for (int32_t c0 = 0; c0 < p.C; c0 += kChanBlock) {
+                T four[kChanBlock];
+#pragma unroll
+                for (int j = 0; j < kChanBlock; j++) {
+                    const int32_t c = (c0 + j < p.C) ? c0 + j : p.C - 1;
+                    four[j] = go_n[(int64_t)c * p.points];
+                }
+                T* dst = go4 + ((size_t)(c0 / kChanBlock) * p.points + pt) * kChanBlock;
+                if constexpr (sizeof(T) == 2) {
+                    *reinterpret_cast<uint2*>(dst) = *reinterpret_cast<const uint2*>(four);
+                } else {
+                    *reinterpret_cast<uint4*>(dst) = *reinterpret_cast<const uint4*>(four);
+                }
+            }
+        }
         // the cell of the low corner; a point none of whose corners is inside the volume has no cell
         if (tp.x0 >= -1 && tp.x0 < p.W && tp.y0 >= -1 && tp.y0 < p.H && tp.z0 >= -1 && tp.z0 < p.D) {
             const uint32_t cell = ((uint32_t)(tp.z0 + 1) * (uint32_t)(p.H + 1) + (uint32_t)(tp.y0 + 1)) *
@@ -133,6 +162,9 @@ __global__ __launch_bounds__(kLThreads) void gs3d_lists_slots_kernel(const T* __
             } else {
                 wsn[lay.flag] = 1u;
             }
+        }
+        if constexpr (GRID) {
+            gs3d_point_grid_gradient<T>(tp, gout, x, dgrid, n * (int64_t)p.points + pt, n, pt, p);
         }
     }
     if (ranges == nullptr) {
@@ -222,7 +254,7 @@ __device__ __forceinline__ void sort_list(uint32_t* mine, uint32_t len)
 }
 
 template <typename T>
-__global__ __launch_bounds__(kLThreads) void gs3d_lists_gather_kernel(const T* __restrict__ gout, T* __restrict__ dx,
+__global__ __launch_bounds__(kLThreads) void gs3d_lists_gather_kernel(T* __restrict__ dx,
                                                                        uint32_t* __restrict__ ws, Grad3Params p,
                                                                        Lists3Layout lay, uint32_t tiles,
                                                                        uint32_t cblocks, int32_t chans_per_block,
@@ -311,13 +343,9 @@ __global__ __launch_bounds__(kLThreads) void gs3d_lists_gather_kernel(const T* _
     const uint32_t last = len > 0 ? len - 1u : 0u;
     for (int32_t c0 = c_begin; c0 < c_end; c0 += kChanBlock) {
         const int32_t nc = (c_end - c0 < kChanBlock) ? c_end - c0 : kChanBlock;
-        // byte offsets from the item's gradOutput in 32 bits (launch plan): one address register pair for all loads
-        const char* go_n = reinterpret_cast<const char*>(gout + n * p.C * (int64_t)p.points);
-        uint32_t chan_off[kChanBlock];
-#pragma unroll
-        for (int j = 0; j < kChanBlock; j++) {
-            chan_off[j] = (uint32_t)(c0 + (j < nc ? j : nc - 1)) * (uint32_t)p.points * (uint32_t)sizeof(T);
-        }
+        // the group's gradOutput, four channels per point (byte offsets in 32 bits: launch plan)
+        const char* go4 = reinterpret_cast<const char*>(wsn + lay.go4) +
+                          (size_t)(c0 / kChanBlock) * p.points * (kChanBlock * sizeof(T));
         acc_t acc[kChanBlock];
 #pragma unroll
         for (int j = 0; j < kChanBlock; j++) {
@@ -328,10 +356,9 @@ __global__ __launch_bounds__(kLThreads) void gs3d_lists_gather_kernel(const T* _
             const uint32_t key = mine[(i < last ? i : last) * kLThreads];
             const uint32_t pt = key & 0xFFFFu, k = (key >> kPtBits) & 7u;
             w = *reinterpret_cast<const T*>(wts + (pt * 8u + k) * (uint32_t)sizeof(T));
-#pragma unroll
-            for (int j = 0; j < kChanBlock; j++) {
-                g[j] = *reinterpret_cast<const T*>(go_n + (chan_off[j] + pt * (uint32_t)sizeof(T)));
-            }
+            typedef typename std::conditional<sizeof(T) == 2, uint2, uint4>::type four_t;
+            const four_t four = *reinterpret_cast<const four_t*>(go4 + pt * (uint32_t)(kChanBlock * sizeof(T)));
+            __builtin_memcpy(g, &four, sizeof(four));
         };
         if (len > 0) {
             fetch(0, wa, ga);
@@ -378,8 +405,12 @@ Lists3Plan make_plan(const GridSampler3DGradArgs& a)
         a.C * points * esz > (int64_t)UINT32_MAX) {
         return pl;
     }
+    const int64_t groups = (a.C + kChanBlock - 1) / kChanBlock;
+    if (4 + cells * 5 + points * 8 * esz / 4 + groups * points * kChanBlock * esz / 4 + 16 > (int64_t)1 << 31) {
+        return pl;  // an item's scratch is indexed in 32 bits
+    }
     pl.cells = cells;
-    pl.lay = make_layout(cells, points, esz);
+    pl.lay = make_layout(cells, points, esz, a.C);
     pl.tiles = (uint32_t)((vol + kLThreads - 1) / kLThreads);
     // channel blocks: lanes enough for the chip (a lane walks its list once per four channels)
     const int64_t base = a.N * pl.tiles;
@@ -412,14 +443,21 @@ hipError_t run_typed(const GridSampler3DGradArgs& a, const Lists3Plan& pl, const
         return e;
     }
     const uint32_t item_slots = 8u * (uint32_t)((a.N + 7) / 8);  // items, rounded up to whole turns of the XCDs
-    hipLaunchKernelGGL((gs3d_lists_slots_kernel<T>), dim3(item_slots * (uint32_t)p.chunks), dim3(kLThreads), 0, stream,
-                       (const T*)a.grid, ws, ranges, p, pl.lay, (int32_t)a.N);
+    if (a.dgrid != nullptr) {
+        hipLaunchKernelGGL((gs3d_lists_slots_kernel<T, true>), dim3(item_slots * (uint32_t)p.chunks), dim3(kLThreads), 0,
+                           stream, (const T*)a.grid, (const T*)a.gout, ws, ranges, p, pl.lay, (int32_t)a.N,
+                           (const T*)a.x, (T*)a.dgrid);
+    } else {
+        hipLaunchKernelGGL((gs3d_lists_slots_kernel<T, false>), dim3(item_slots * (uint32_t)p.chunks), dim3(kLThreads),
+                           0, stream, (const T*)a.grid, (const T*)a.gout, ws, ranges, p, pl.lay, (int32_t)a.N,
+                           (const T*)nullptr, (T*)nullptr);
+    }
     e = hipGetLastError();
     if (e != hipSuccess) {
         return e;
     }
     hipLaunchKernelGGL((gs3d_lists_gather_kernel<T>), dim3(item_slots * pl.tiles * pl.cblocks), dim3(kLThreads), 0,
-                       stream, (const T*)a.gout, (T*)a.dx, ws, p, pl.lay, pl.tiles, pl.cblocks, pl.chans_per_block,
+                       stream, (T*)a.dx, ws, p, pl.lay, pl.tiles, pl.cblocks, pl.chans_per_block,
                        (int32_t)a.N);
     return hipGetLastError();
 }
@@ -433,10 +471,12 @@ int64_t gs3d_grad_list_words(const GridSampler3DGradArgs& a)
 }
 
 hipError_t run_gs3d_grad_input_lists(const GridSampler3DGradArgs& a, const Grad3Params& p, int32_t* ranges,
-                                     hipStream_t stream, const uint32_t** item_flags, uint32_t* flag_stride)
+                                     hipStream_t stream, const uint32_t** item_flags, uint32_t* flag_stride,
+                                     bool* dgrid_done)
 {
     *item_flags = nullptr;
     *flag_stride = 0;
+    *dgrid_done = false;
     if (a.dx == nullptr || a.lists == nullptr) {
         return hipSuccess;
     }
@@ -446,6 +486,7 @@ hipError_t run_gs3d_grad_input_lists(const GridSampler3DGradArgs& a, const Grad3
     }
     *item_flags = (const uint32_t*)a.lists + pl.lay.flag;
     *flag_stride = pl.lay.item_words;
+    *dgrid_done = a.dgrid != nullptr;
     switch (a.elem) {
         case Elem::F32: return run_typed<float>(a, pl, p, ranges, stream);
         case Elem::F16: return run_typed<_Float16>(a, pl, p, ranges, stream);

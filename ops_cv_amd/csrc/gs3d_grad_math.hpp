@@ -6,6 +6,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "acl_types.hpp"
 #include "gs2d_grad_math.hpp"
 
@@ -108,11 +110,125 @@ __host__ __device__ inline int32_t chunk_count(int64_t points, int64_t items_per
     return (int32_t)(((items_per_core > 1 ? kChunkPoints3 - 1 : 0) + points + kChunkPoints3 - 1) / kChunkPoints3);
 }
 
+// The gradient of one grid point (bilinear): the sums over the channels of value times two distances times the
+// incoming gradient for the eight corners, then the chain-rule multipliers (grid_sampler3_d_grad_simt_det.h:98-330).
+// `idx` is the point's number among all points of the batch, n its batch item, pt its number within the item.
+template <typename T>
+__device__ __forceinline__ void gs3d_point_grid_gradient(const GradTaps3<T, 0>& tp, const T* __restrict__ gout,
+                                                         const T* __restrict__ x, T* __restrict__ dgrid, int64_t idx,
+                                                         int64_t n, int32_t pt, const Grad3Params& p)
+{
+    const int32_t points = p.points;
+    const int32_t vol = p.D * p.H * p.W;
+    const T* x_n = x + n * p.C * (int64_t)vol;
+    const T* go_n = gout + n * p.C * (int64_t)points + pt;
+    float gix = 0.0f, giy = 0.0f, giz = 0.0f;
+    bool ok[8];
+    int32_t o[8];
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        ok[k] = tp.off[k] >= 0;
+        o[k] = ok[k] ? tp.off[k] : 0;
+    }
+    // grid_sampler3_d_grad_simt_det.h:119-124 and the seven corners after it: value times two distances times the
+    // incoming gradient, left to right, subtracted for a low corner of the axis and added for a high one
+    auto accumulate = [&](float go, const float* v) {
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const int xs = k & 1, ys = (k >> 1) & 1, zs = k >> 2;
+            if (ok[k]) {
+                const float tx = v[k] * tp.wy[ys] * tp.wz[zs] * go;
+                const float ty = v[k] * tp.wx[xs] * tp.wz[zs] * go;
+                const float tz = v[k] * tp.wx[xs] * tp.wy[ys] * go;
+                gix = xs ? gix + tx : gix - tx;
+                giy = ys ? giy + ty : giy - ty;
+                giz = zs ? giz + tz : giz - tz;
+            }
+        }
+    };
+    // The sums run over the channels in order; the loads do not depend on them and are issued a group ahead.
+    constexpr int U = 4;
+    int32_t c = 0;
+    if (p.W >= 2) {
+        // The low and high corner along x are neighbours in memory: one load of two elements (aligned to one element
+        // only) per row of corners instead of two halves the addresses the gather puts through the memory pipeline.
+        // The pair sits at column pb = clamp(x0, 0, W - 2), so it never leaves the row; which half is which corner
+        // follows from pb.  Corners outside the volume are skipped by accumulate() as before.
+        using PairBits = typename std::conditional<sizeof(T) == 2, uint32_t, uint64_t>::type;
+        const int32_t pb = (tp.x0 < 0) ? 0 : ((tp.x0 > p.W - 2) ? p.W - 2 : tp.x0);
+        const bool lo_w = (tp.x0 == pb), lo_e = (next_index(tp.x0) == pb);
+        int32_t rowoff[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int32_t cy = (r & 1) ? next_index(tp.y0) : tp.y0, cz = (r >> 1) ? next_index(tp.z0) : tp.z0;
+            const bool in = (uint32_t)cy < (uint32_t)p.H && (uint32_t)cz < (uint32_t)p.D;
+            rowoff[r] = in ? (cz * p.H + cy) * p.W + pb : 0;
+        }
+        for (; c + U <= p.C; c += U) {
+            float go[U];
+            PairBits pr[U][4];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const T* xc = x_n + (int64_t)(c + u) * vol;
+                go[u] = ElemIO<T>::load(go_n + (int64_t)(c + u) * points);
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    __builtin_memcpy(&pr[u][r], xc + rowoff[r], sizeof(PairBits));
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                float v[8];
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    T two[2];
+                    __builtin_memcpy(two, &pr[u][r], sizeof(PairBits));
+                    const float lo = ElemIO<T>::load(&two[0]), hi = ElemIO<T>::load(&two[1]);
+                    v[2 * r] = lo_w ? lo : hi;
+                    v[2 * r + 1] = lo_e ? lo : hi;
+                }
+                accumulate(go[u], v);
+            }
+        }
+    }
+    for (; c + U <= p.C; c += U) {
+        float go[U], v[U][8];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const T* xc = x_n + (int64_t)(c + u) * vol;
+            go[u] = ElemIO<T>::load(go_n + (int64_t)(c + u) * points);
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                v[u][k] = ElemIO<T>::load(xc + o[k]);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            accumulate(go[u], v[u]);
+        }
+    }
+    for (; c < p.C; c++) {
+        const T* xc = x_n + (int64_t)c * vol;
+        float v[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            v[k] = ElemIO<T>::load(xc + o[k]);
+        }
+        accumulate(ElemIO<T>::load(go_n + (int64_t)c * points), v);
+    }
+    // grid_sampler3_d_grad_simt_det.h:324-326: product in fp32, then the conversion
+    ElemIO<T>::store(dgrid + 3 * idx, as_fp32_value(tp.mx * gix));
+    ElemIO<T>::store(dgrid + 3 * idx + 1, as_fp32_value(tp.my * giy));
+    ElemIO<T>::store(dgrid + 3 * idx + 2, as_fp32_value(tp.mz * giz));
+}
+
 // The gather variant of the input gradient (gs3d_grad_lists.hip).  Runs when a.lists is set and the shape qualifies:
 // *item_flags then points at a word per batch item, `*flag_stride` words apart, that is non-zero for the items it
 // leaves to the ordered kernel, which has to run after it for those; otherwise *item_flags is null and nothing was
-// launched.  `ranges` (may be null) receives the voxel span of every chunk, as from gs3d_grad_range_kernel.
+// launched.  `ranges` (may be null) receives the voxel span of every chunk, as from gs3d_grad_range_kernel.  When
+// a.dgrid is set, its first kernel computes the gradient of the grid as well (*dgrid_done).
 hipError_t run_gs3d_grad_input_lists(const GridSampler3DGradArgs& a, const Grad3Params& p, int32_t* ranges,
-                                     hipStream_t stream, const uint32_t** item_flags, uint32_t* flag_stride);
+                                     hipStream_t stream, const uint32_t** item_flags, uint32_t* flag_stride,
+                                     bool* dgrid_done);
 
 }  // namespace opscv

@@ -692,7 +692,8 @@ def test_grid_sampler3d_backward_gather_variant(oracle, device, aclnn, dtype, mo
                 per_core = (N + cores - 1) // cores if N > cores else 1
                 chunks = ((255 if per_core > 1 else 0) + points + 255) // 256
                 range_bytes = N * 2 * chunks * 4 if vol > 2048 else 0  # bands of 2048 voxels or more
-                item_words = (((4 + cells + 3) // 4 * 4 + 4 * cells) * 4 + points * 8 * esz + 15) // 16 * 4
+                item_words = (((4 + cells + 3) // 4 * 4 + 4 * cells) * 4 + points * 8 * esz +
+                              (C + 3) // 4 * points * 4 * esz + 15) // 16 * 4
                 words = ws.view(torch.int32)
                 flags = [int(words[(range_bytes + 255) // 256 * 64 + n * item_words].item()) for n in range(N)]
                 assert all(f in (0, 1) for f in flags), flags
