@@ -9,9 +9,10 @@
 // scatter becomes a gather, as for the 2-D sampler (gs2d_grad_csr.hip):
 //
 //   slots (one lane per grid point, workgroups along the reference's chunks): the eight corner weights of the point go
-//     to scratch memory, and the point takes one of the six slots of the cell (z0, y0, x0) of its low corner (an
-//     atomic count per cell: which slot a point gets depends on timing, which points a cell holds does not).  A cell
-//     with more than six points flags its batch item.  The workgroup also notes the span of voxels its chunk
+//     to scratch memory, and the point takes one of the eight slots of the cell (z0, y0, x0) of its low corner (an
+//     atomic count per cell: which slot a point gets depends on timing, which points a cell holds does not).  A point
+//     that finds its cell full goes to a short overflow list of the item, where the voxels of a crowded cell look for
+//     it; an item with more than 1024 such points is flagged.  The workgroup also notes the span of voxels its chunk
 //     touches, which the ordered kernel wants should the item be flagged.
 //   gather (one lane per voxel): voxel (z, y, x) is corner (xs, ys, zs) of the points of cell (z - zs, y - ys, x - xs).
 //     The lane collects the points of its eight cells, keyed (chunk, corner, point), into a list of its own in LDS,
@@ -35,18 +36,20 @@ namespace opscv {
 namespace {
 
 constexpr int kLThreads = kChunkPoints3;
-constexpr int kCellSlots = 6;   // points a cell can hold
+constexpr int kCellSlots = 8;   // points a cell can hold in its slot record
+constexpr int kOverflowMax = 1024;  // points of an item that found their cell's record full and wait in a list
 constexpr int kListMax = 32;    // contributions a voxel's list can hold
 constexpr int kChanBlock = 4;   // channels per walk of a list
 constexpr uint32_t kPtBits = 16;
 
 // 32-bit words of scratch per batch item
 struct Lists3Layout {
-    uint32_t flag;    // 4 words; [0] != 0: the item is left to the ordered kernel
+    uint32_t flag;    // 4 words; [0] != 0: the item is left to the ordered kernel; [1]: points in the overflow list
     uint32_t counts;  // one per cell of the (D + 1) x (H + 1) x (W + 1) lattice of low corners.  Dense, apart from the
                       // slots: the atomics of neighbouring points then meet in few cache lines (a count inside the
                       // cell's 16-byte slot record made the slots kernel 17 us slower on fp16 22x4x16x64x64)
-    uint32_t slots;   // kCellSlots 16-bit point numbers per cell and two unused ones: one 16-byte load per cell
+    uint32_t slots;   // kCellSlots 16-bit point numbers per cell: one 16-byte load per cell
+    uint32_t overflow;  // kOverflowMax (cell, point) pairs: the points beyond the eighth of a cell
     uint32_t wts;     // eight weights of the element type per point
     uint32_t go4;     // gradOutput with the channels of a group of four side by side: [group][point][4]
     uint32_t item_words;
@@ -60,7 +63,8 @@ Lists3Layout make_layout(int64_t cells, int64_t points, int64_t esz, int64_t cha
     l.flag = 0;
     l.counts = 4;
     l.slots = align4((uint64_t)l.counts + (uint64_t)cells);
-    l.wts = align4((uint64_t)l.slots + (uint64_t)cells * 4);
+    l.overflow = align4((uint64_t)l.slots + (uint64_t)cells * 4);
+    l.wts = align4((uint64_t)l.overflow + 2u * kOverflowMax);
     l.go4 = align4((uint64_t)l.wts + (uint64_t)points * 8 * (uint64_t)esz / 4);
     const uint64_t groups = ((uint64_t)channels + kChanBlock - 1) / kChanBlock;
     l.item_words = align4((uint64_t)l.go4 + groups * (uint64_t)points * kChanBlock * (uint64_t)esz / 4);
@@ -160,7 +164,14 @@ __global__ __launch_bounds__(kLThreads) void gs3d_lists_slots_kernel(const T* __
             if (r < (uint32_t)kCellSlots) {
                 reinterpret_cast<uint16_t*>(wsn + lay.slots + (size_t)cell * 4)[r] = (uint16_t)pt;
             } else {
-                wsn[lay.flag] = 1u;
+                // the record is full: the point waits in the item's overflow list, where the voxels of a crowded cell
+                // look for it; an item with more of those than the list holds is left to the ordered kernel
+                const uint32_t o = atomicAdd(&wsn[lay.flag + 1], 1u);
+                if (o < (uint32_t)kOverflowMax) {
+                    reinterpret_cast<uint2*>(wsn + lay.overflow)[o] = make_uint2(cell, (uint32_t)pt);
+                } else {
+                    wsn[lay.flag] = 1u;
+                }
             }
         }
         if constexpr (GRID) {
@@ -299,10 +310,11 @@ __global__ __launch_bounds__(kLThreads) void gs3d_lists_gather_kernel(T* __restr
         rec[k] = slots[cell];
     }
     uint32_t len = 0;
+    bool crowded = false;
 #pragma unroll
     for (int k = 0; k < 8; k++) {
-        cnt[k] = cnt[k] < (uint32_t)kCellSlots ? cnt[k] : (uint32_t)kCellSlots;  // more: the item is flagged
         len += cnt[k];
+        crowded = crowded || cnt[k] > (uint32_t)kCellSlots;
     }
     if (len > (uint32_t)kListMax) {
         wsn[lay.flag] = 1u;  // the ordered kernel redoes the item
@@ -315,7 +327,7 @@ __global__ __launch_bounds__(kLThreads) void gs3d_lists_gather_kernel(T* __restr
 #pragma unroll
     for (int k = 0; k < 8; k++) {
         // a cell holds a point or two as a rule: those without a loop
-        const uint32_t have = cnt[k];
+        const uint32_t have = cnt[k] < (uint32_t)kCellSlots ? cnt[k] : (uint32_t)kCellSlots;
         if (have > 0u) {
             mine[at * kLThreads] = key_of(rec[k].x & 0xFFFFu, (uint32_t)k);
         }
@@ -323,10 +335,27 @@ __global__ __launch_bounds__(kLThreads) void gs3d_lists_gather_kernel(T* __restr
             mine[(at + 1u) * kLThreads] = key_of(rec[k].x >> 16, (uint32_t)k);
         }
         for (uint32_t i = 2; i < have; i++) {
-            const uint32_t pt = (((i < 4u) ? rec[k].y : rec[k].z) >> ((i & 1u) * 16u)) & 0xFFFFu;
-            mine[(at + i) * kLThreads] = key_of(pt, (uint32_t)k);
+            const uint32_t word = (i < 4u) ? rec[k].y : ((i < 6u) ? rec[k].z : rec[k].w);
+            mine[(at + i) * kLThreads] = key_of((word >> ((i & 1u) * 16u)) & 0xFFFFu, (uint32_t)k);
         }
         at += have;
+    }
+    if (crowded) {
+        // the points of a crowded cell beyond its record: the item's overflow list holds them, with their cell
+        const uint32_t listed = wsn[lay.flag + 1] < (uint32_t)kOverflowMax ? wsn[lay.flag + 1] : (uint32_t)kOverflowMax;
+        const uint2* waiting = reinterpret_cast<const uint2*>(wsn + lay.overflow);
+        const uint32_t xb = (uint32_t)x + 1u, yb = (uint32_t)y + 1u, zb = (uint32_t)z + 1u;
+        for (uint32_t i = 0; i < listed; i++) {
+            const uint2 e = waiting[i];
+            // which corner of this voxel the waiting point's cell is, if any
+            const uint32_t cx = e.x % w1, cyz = e.x / w1;
+            const uint32_t cy = cyz % h1, cz = cyz / h1;
+            const uint32_t xs = xb - cx, ys = yb - cy, zs = zb - cz;
+            if (xs <= 1u && ys <= 1u && zs <= 1u) {
+                mine[at * kLThreads] = key_of(e.y, xs + 2u * ys + 4u * zs);
+                at++;
+            }
+        }
     }
     // Sort, ascending keys = the reference's order: the list goes through registers and a bitonic network of 16 keys,
     // or of 32 where a lane of the wavefront has more (past its end a list is padded with the largest key).  An
@@ -406,7 +435,8 @@ Lists3Plan make_plan(const GridSampler3DGradArgs& a)
         return pl;
     }
     const int64_t groups = (a.C + kChanBlock - 1) / kChanBlock;
-    if (4 + cells * 5 + points * 8 * esz / 4 + groups * points * kChanBlock * esz / 4 + 16 > (int64_t)1 << 31) {
+    if (4 + cells * 5 + 2 * kOverflowMax + points * 8 * esz / 4 + groups * points * kChanBlock * esz / 4 + 16 >
+        (int64_t)1 << 31) {
         return pl;  // an item's scratch is indexed in 32 bits
     }
     pl.cells = cells;

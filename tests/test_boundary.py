@@ -558,10 +558,11 @@ def test_grid_sampler3d_backward_status_codes(aclnn, desc):
     INV, NULL = aclnn.ACLNN_ERR_PARAM_INVALID, aclnn.ACLNN_ERR_PARAM_NULLPTR
     # dtype_float16 / dtype_float32 / dtype_bf16: the unit test's shapes
     # bilinear asks for the scratch of the gather variant: per batch item four flag words, a count and eight 16-bit slots
-    # per cell of the (D+1) x (H+1) x (W+1) lattice of low corners (2 x 4 x 4 here), eight weights per grid point (4)
-    # and gradOutput once more, in groups of four channels
+    # per cell of the (D+1) x (H+1) x (W+1) lattice of low corners (2 x 4 x 4 here), an overflow list of 1024 (cell,
+    # point) pairs, eight weights per grid point (4) and gradOutput once more, in groups of four channels
     for dt, esz in ((aclnn.ACL_FLOAT, 4), (aclnn.ACL_FLOAT16, 2), (aclnn.ACL_BF16, 2)):
-        assert _gsb3(aclnn, desc, dt=dt) == (0, (4 + 32 + 4 * 32) * 4 + 4 * 8 * esz + 4 * 4 * esz, "gs3d_grad_lists")
+        assert _gsb3(aclnn, desc, dt=dt) == (0, (4 + 32 + 4 * 32 + 2048) * 4 + 4 * 8 * esz + 4 * 4 * esz,
+                                             "gs3d_grad_lists")
         assert _gsb3(aclnn, desc, dt=dt, interp=1) == (0, 0, "gs3d_grad_ordered")
     # gradOutput_nullptr .. gridGrad_nullptr
     for missing in ("gout", "inp", "grid", "dx", "dgrid"):
@@ -605,7 +606,7 @@ def test_grid_sampler3d_backward_status_codes(aclnn, desc):
     big = dict(gout=(3, 1, 2, 30, 10), inp=(3, 1, 10, 30, 30), grid=(3, 2, 30, 10, 3))
     assert _gsb3(aclnn, desc, interp=1, **big)[:2] == (0, 3 * 3 * 2 * 4)
     cells, points = 11 * 31 * 31, 600
-    per_item = ((4 + cells + 3) // 4 * 4 + 4 * cells) * 4 + points * 8 * 4 + points * 4 * 4
+    per_item = ((4 + cells + 3) // 4 * 4 + 4 * cells + 2048) * 4 + points * 8 * 4 + points * 4 * 4
     assert _gsb3(aclnn, desc, **big) == (0, 256 + 3 * per_item, "gs3d_grad_lists")
     assert _gsb3(aclnn, desc, mask=(False, True), **big)[:2] == (0, 0)
 

@@ -645,7 +645,8 @@ def test_grid_sampler3d_backward_gather_variant(oracle, device, aclnn, dtype, mo
     """The input gradient of the 3-D sampler as a gather over every voxel's contributions: bit for bit the oracle's
     (chunk, corner, point) order on jittered lattices (about eight contributions per voxel), on denser grids (lists of
     more than sixteen entries, some items handed to the ordered kernel because a voxel has more than 32), with one
-    piled-up item among lattice items, with channel counts around the group of four, and with more items than cores
+    piled-up item among lattice items, with a cell that overflows its slots into the item's overflow list, with
+    channel counts around the group of four, and with more items than cores
     (chunk boundaries that move from item to item).  Which items the gather did is read from the flag words it keeps
     in the workspace, which is handed over full of ones."""
     torch = _torch()
@@ -664,6 +665,7 @@ def test_grid_sampler3d_backward_gather_variant(oracle, device, aclnn, dtype, mo
         (3, 5, (6, 12, 10), (6, 12, 10), "lattice", 2),
         (2, 4, (5, 9, 33), (7, 12, 40), "dense", 64),
         (3, 1, (4, 8, 8), (4, 8, 8), "mixed", 64),
+        (2, 3, (4, 8, 8), (4, 8, 8), "crowded", 64),
         (2, 6, (3, 20, 70), (3, 20, 70), "lattice", 64),
         (5, 2, (4, 6, 6), (5, 8, 8), "dense", 2),
         (5, 3, (5, 8, 8), (5, 8, 8), "lattice", 2),
@@ -675,7 +677,11 @@ def test_grid_sampler3d_backward_gather_variant(oracle, device, aclnn, dtype, mo
             oracle.set_reference_cores(cores)
             g32 = lattice(N, Do, Ho, Wo, 0.1, 0.03)
             if kind == "mixed":
-                g32[1] = rng.choice(np.array([-0.5, 0.1, 0.6], np.float32), (Do, Ho, Wo, 3))
+                g32[1] = np.float32(0.1)  # every point of the item on one spot: lists far beyond what a voxel holds
+            if kind == "crowded":
+                # a lattice with a dozen points moved onto one spot: that cell overflows its eight slots and its voxels
+                # find the rest in the item's overflow list; the item is still the gather's
+                g32[:, 0, :2, :6] = np.float32(0.3)
             g = I.cast_np(g32, dtype)
             x = I.cast_np(rng.standard_normal((N, C, D, H, W)).astype(np.float32), dtype)
             go = I.cast_np(rng.standard_normal((N, C, Do, Ho, Wo)).astype(np.float32), dtype)
@@ -692,7 +698,7 @@ def test_grid_sampler3d_backward_gather_variant(oracle, device, aclnn, dtype, mo
                 per_core = (N + cores - 1) // cores if N > cores else 1
                 chunks = ((255 if per_core > 1 else 0) + points + 255) // 256
                 range_bytes = N * 2 * chunks * 4 if vol > 2048 else 0  # bands of 2048 voxels or more
-                item_words = (((4 + cells + 3) // 4 * 4 + 4 * cells) * 4 + points * 8 * esz +
+                item_words = (((4 + cells + 3) // 4 * 4 + 4 * cells + 2048) * 4 + points * 8 * esz +
                               (C + 3) // 4 * points * 4 * esz + 15) // 16 * 4
                 words = ws.view(torch.int32)
                 flags = [int(words[(range_bytes + 255) // 256 * 64 + n * item_words].item()) for n in range(N)]
@@ -703,6 +709,10 @@ def test_grid_sampler3d_backward_gather_variant(oracle, device, aclnn, dtype, mo
                     assert flags == [0, 1, 0], flags
                 if kind == "lattice" and pad == 0:
                     assert flags == [0] * N, flags
+                if kind == "crowded" and pad == 0:
+                    assert flags == [0] * N, flags
+                    overflowed = [int(words[(range_bytes + 255) // 256 * 64 + n * item_words + 1].item()) for n in range(N)]
+                    assert all(o >= 4 for o in overflowed), overflowed
                 seen_gathered += flags.count(0)
                 seen_flagged += flags.count(1)
     finally:
