@@ -274,7 +274,7 @@ __global__ __launch_bounds__(kThreads) void gs3d_grad_input_kernel(const T* __re
     }
 }
 
-template <typename T, int INTERP>
+template <typename T, int INTERP, int U>
 __global__ __launch_bounds__(kThreads) void gs3d_grad_grid_kernel(const T* __restrict__ gout, const T* __restrict__ x,
                                                                    const T* __restrict__ grid, T* __restrict__ dgrid,
                                                                    int64_t total, Grad3Params p)
@@ -300,7 +300,7 @@ __global__ __launch_bounds__(kThreads) void gs3d_grad_grid_kernel(const T* __res
         Taps tp;
         decide_grad_taps3<T, INTERP>(tp, ElemIO<T>::load(grid + 3 * idx), ElemIO<T>::load(grid + 3 * idx + 1),
                                      ElemIO<T>::load(grid + 3 * idx + 2), p.D, p.H, p.W, p.pad, p.align);
-        gs3d_point_grid_gradient<T>(tp, gout, x, dgrid, idx, n, pt, p);
+        gs3d_point_grid_gradient<T, U>(tp, gout, x, dgrid, idx, n, pt, p);
     }
 }
 
@@ -404,8 +404,13 @@ hipError_t launch_interp(const GridSampler3DGradArgs& a, hipStream_t stream)
         if (blocks > INT32_MAX) {
             return hipErrorInvalidValue;
         }
-        hipLaunchKernelGGL((gs3d_grad_grid_kernel<T, INTERP>), dim3((unsigned)blocks), dim3(kThreads), 0, stream,
-                           (const T*)a.gout, (const T*)a.x, (const T*)a.grid, (T*)a.dgrid, total, p);
+        if (total < kGridGradFewPoints) {
+            hipLaunchKernelGGL((gs3d_grad_grid_kernel<T, INTERP, 4>), dim3((unsigned)blocks), dim3(kThreads), 0, stream,
+                               (const T*)a.gout, (const T*)a.x, (const T*)a.grid, (T*)a.dgrid, total, p);
+        } else {
+            hipLaunchKernelGGL((gs3d_grad_grid_kernel<T, INTERP, 1>), dim3((unsigned)blocks), dim3(kThreads), 0, stream,
+                               (const T*)a.gout, (const T*)a.x, (const T*)a.grid, (T*)a.dgrid, total, p);
+        }
         return hipGetLastError();
     }
     return hipSuccess;

@@ -95,7 +95,7 @@ __global__ __launch_bounds__(256) void gs3d_lists_clear_kernel(uint32_t* __restr
 
 // GRID: the lane goes on to the gradient of its grid point -- the corner decisions are the same, and the atomics
 // and stores above are on their way while the corners of the input are read.
-template <typename T, bool GRID>
+template <typename T, int GRID>
 __global__ __launch_bounds__(kLThreads) void gs3d_lists_slots_kernel(const T* __restrict__ grid,
                                                                       const T* __restrict__ gout,
                                                                       uint32_t* __restrict__ ws,
@@ -174,8 +174,8 @@ __global__ __launch_bounds__(kLThreads) void gs3d_lists_slots_kernel(const T* __
                 }
             }
         }
-        if constexpr (GRID) {
-            gs3d_point_grid_gradient<T>(tp, gout, x, dgrid, n * (int64_t)p.points + pt, n, pt, p);
+        if constexpr (GRID > 0) {  // GRID: channels in flight together (gs3d_point_grid_gradient)
+            gs3d_point_grid_gradient<T, GRID>(tp, gout, x, dgrid, n * (int64_t)p.points + pt, n, pt, p);
         }
     }
     if (ranges == nullptr) {
@@ -473,14 +473,16 @@ hipError_t run_typed(const GridSampler3DGradArgs& a, const Lists3Plan& pl, const
         return e;
     }
     const uint32_t item_slots = 8u * (uint32_t)((a.N + 7) / 8);  // items, rounded up to whole turns of the XCDs
-    if (a.dgrid != nullptr) {
-        hipLaunchKernelGGL((gs3d_lists_slots_kernel<T, true>), dim3(item_slots * (uint32_t)p.chunks), dim3(kLThreads), 0,
-                           stream, (const T*)a.grid, (const T*)a.gout, ws, ranges, p, pl.lay, (int32_t)a.N,
-                           (const T*)a.x, (T*)a.dgrid);
+    const dim3 slots_grid(item_slots * (uint32_t)p.chunks);
+    if (a.dgrid != nullptr && a.N * (int64_t)p.points < kGridGradFewPoints) {
+        hipLaunchKernelGGL((gs3d_lists_slots_kernel<T, 4>), slots_grid, dim3(kLThreads), 0, stream, (const T*)a.grid,
+                           (const T*)a.gout, ws, ranges, p, pl.lay, (int32_t)a.N, (const T*)a.x, (T*)a.dgrid);
+    } else if (a.dgrid != nullptr) {
+        hipLaunchKernelGGL((gs3d_lists_slots_kernel<T, 1>), slots_grid, dim3(kLThreads), 0, stream, (const T*)a.grid,
+                           (const T*)a.gout, ws, ranges, p, pl.lay, (int32_t)a.N, (const T*)a.x, (T*)a.dgrid);
     } else {
-        hipLaunchKernelGGL((gs3d_lists_slots_kernel<T, false>), dim3(item_slots * (uint32_t)p.chunks), dim3(kLThreads),
-                           0, stream, (const T*)a.grid, (const T*)a.gout, ws, ranges, p, pl.lay, (int32_t)a.N,
-                           (const T*)nullptr, (T*)nullptr);
+        hipLaunchKernelGGL((gs3d_lists_slots_kernel<T, 0>), slots_grid, dim3(kLThreads), 0, stream, (const T*)a.grid,
+                           (const T*)a.gout, ws, ranges, p, pl.lay, (int32_t)a.N, (const T*)nullptr, (T*)nullptr);
     }
     e = hipGetLastError();
     if (e != hipSuccess) {

@@ -113,7 +113,11 @@ __host__ __device__ inline int32_t chunk_count(int64_t points, int64_t items_per
 // The gradient of one grid point (bilinear): the sums over the channels of value times two distances times the
 // incoming gradient for the eight corners, then the chain-rule multipliers (grid_sampler3_d_grad_simt_det.h:98-330).
 // `idx` is the point's number among all points of the batch, n its batch item, pt its number within the item.
-template <typename T>
+// U: channels whose loads are in flight together.  Four need about 150 vector registers (three wavefronts per SIMD),
+// one about 76 (six): with grid points for four wavefronts per SIMD and more, the wavefronts hide the latency better
+// than the unrolling does (fp16 22x4x16x64x64: 34.0 us with four, 29.1 us with one; 2x64x16x64x64: 32.0 and 41.5 us).
+constexpr int64_t kGridGradFewPoints = 256 * 4 * 4 * 64;  // below: U = 4
+template <typename T, int U>
 __device__ __forceinline__ void gs3d_point_grid_gradient(const GradTaps3<T, 0>& tp, const T* __restrict__ gout,
                                                          const T* __restrict__ x, T* __restrict__ dgrid, int64_t idx,
                                                          int64_t n, int32_t pt, const Grad3Params& p)
@@ -147,7 +151,6 @@ __device__ __forceinline__ void gs3d_point_grid_gradient(const GradTaps3<T, 0>& 
         }
     };
     // The sums run over the channels in order; the loads do not depend on them and are issued a group ahead.
-    constexpr int U = 4;
     int32_t c = 0;
     if (p.W >= 2) {
         // The low and high corner along x are neighbours in memory: one load of two elements (aligned to one element
