@@ -231,6 +231,118 @@ __global__ __launch_bounds__(kThreads) void gs3d_kernel(const T* __restrict__ x,
     }
 }
 
+// The bilinear kernel for two-byte elements, rows of two columns and more and volumes below 2^31 elements: the same
+// results as gs3d_kernel from fewer instructions, which is what bounds either (their wavefronts keep the SIMDs'
+// instruction issue busy for most of the kernel's time; memory is far from its limits).  Per channel a lane makes four
+// loads of a pair of neighbouring columns, as gs3d_kernel does, but
+//  * one byte-permute instruction per pair puts the value of column w0 into the low half and that of w1 into the high
+//    half and zeroes the half whose corner lies outside the volume (selector bytes 0x0c give zero bytes), in place of
+//    two conversions and four selects: the selector of a row is made once per point;
+//  * the loads are unconditional (a row without a valid corner reads the volume's first pair and its selector zeroes
+//    both halves), so no branches around them;
+//  * offsets inside a volume are 32-bit.
+// Products and sums per element exactly as in gs3d_kernel.
+typedef uint32_t UnalignedWord __attribute__((aligned(2)));  // a pair of two-byte elements, aligned to one of them
+constexpr uint32_t kSelLow = 0x0100u, kSelHigh = 0x0302u, kSelZero = 0x0c0cu;
+
+template <typename T>
+__device__ __forceinline__ float half_value(uint32_t word, bool high)
+{
+    if constexpr (std::is_same<T, __bf16>::value) {
+        return __builtin_bit_cast(float, high ? (word & 0xffff0000u) : (word << 16));
+    } else {
+        return (float)__builtin_bit_cast(_Float16, (uint16_t)(high ? (word >> 16) : (word & 0xffffu)));
+    }
+}
+
+template <typename T, int PAD, bool ALIGN>
+__global__ __launch_bounds__(kThreads) void gs3d_pair16_kernel(const T* __restrict__ x, const T* __restrict__ grid,
+                                                                T* __restrict__ y, Gs3dParams p)
+{
+    static_assert(sizeof(T) == 2, "pairs of two-byte elements");
+    const int64_t pt = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (pt >= p.points) {
+        return;
+    }
+    const int64_t n = pt / p.out_vol;
+    const int64_t sp = pt - n * p.out_vol;
+    const T* g = grid + pt * 3;
+    const float gw = ElemIO<T>::load(g);
+    const float gh = ElemIO<T>::load(g + 1);
+    const float gd = ElemIO<T>::load(g + 2);
+    const float pd = clip3<PAD, ALIGN>(unnormalize3<ALIGN>(gd, p.Din), p.Din);
+    const float pw = clip3<PAD, ALIGN>(unnormalize3<ALIGN>(gw, p.Win), p.Win);
+    const float ph = clip3<PAD, ALIGN>(unnormalize3<ALIGN>(gh, p.Hin), p.Hin);
+
+    const uint32_t in_plane = (uint32_t)p.Hin * (uint32_t)p.Win;
+    const uint32_t in_vol = (uint32_t)p.Din * in_plane;
+    const int32_t c_begin = blockIdx.y * p.chan_chunk;
+    const int32_t c_end = (c_begin + p.chan_chunk < p.C) ? c_begin + p.chan_chunk : p.C;
+    const T* xc = x + (n * p.C + c_begin) * (int64_t)in_vol;
+    T* yc = y + (n * p.C + c_begin) * p.out_vol + sp;
+
+    const float fd = __builtin_floorf(pd), fh = __builtin_floorf(ph), fw = __builtin_floorf(pw);
+    const float dd = pd - fd, dh = ph - fh, dw = pw - fw;
+    const int32_t d0 = float_to_i32(fd), d1 = float_to_i32(fd + 1.0f);
+    const int32_t h0 = float_to_i32(fh), h1 = float_to_i32(fh + 1.0f);
+    const int32_t w0 = float_to_i32(fw), w1 = float_to_i32(fw + 1.0f);
+    const bool vd0 = d0 >= 0 && d0 < p.Din, vd1 = d1 >= 0 && d1 < p.Din;
+    const bool vh0 = h0 >= 0 && h0 < p.Hin, vh1 = h1 >= 0 && h1 < p.Hin;
+    const bool vw0 = w0 >= 0 && w0 < p.Win, vw1 = w1 >= 0 && w1 < p.Win;
+    float wt[8];
+    wt[0] = (1.0f - dw) * (1.0f - dh) * (1.0f - dd);
+    wt[1] = dw * (1.0f - dh) * (1.0f - dd);
+    wt[2] = (1.0f - dw) * dh * (1.0f - dd);
+    wt[3] = dw * dh * (1.0f - dd);
+    wt[4] = (1.0f - dw) * (1.0f - dh) * dd;
+    wt[5] = dw * (1.0f - dh) * dd;
+    wt[6] = (1.0f - dw) * dh * dd;
+    wt[7] = dw * dh * dd;
+    // the pair of a row starts at column pb = clamp(w0, 0, Win - 2); a valid corner sits in its low half if its column
+    // is pb and in its high half otherwise
+    const int32_t pb = (w0 < 0) ? 0 : ((w0 > p.Win - 2) ? p.Win - 2 : w0);
+    const uint32_t at_w0 = (w0 == pb) ? kSelLow : kSelHigh, at_w1 = (w1 == pb) ? kSelLow : kSelHigh;
+    typedef const __attribute__((address_space(1))) T* GlobalRow;  // keeps the loads below global ones, not flat
+    GlobalRow row[4];
+    uint32_t sel[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const bool vdh = ((r & 2) ? vd1 : vd0) && ((r & 1) ? vh1 : vh0);
+        const bool k0 = vdh && vw0, k1 = vdh && vw1;
+        const uint32_t d = (uint32_t)((r & 2) ? d1 : d0), h = (uint32_t)((r & 1) ? h1 : h0);
+        sel[r] = (k0 ? at_w0 : kSelZero) | ((k1 ? at_w1 : kSelZero) << 16);
+        row[r] = (GlobalRow)(xc + ((k0 || k1) ? d * in_plane + h * (uint32_t)p.Win + (uint32_t)pb : 0u));
+    }
+    auto fetch = [&](uint32_t (&pairs)[4]) {
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            pairs[r] = *(const __attribute__((address_space(1), aligned(2))) UnalignedWord*)row[r];
+            row[r] += in_vol;
+        }
+    };
+    auto blend_and_store = [&](const uint32_t (&pairs)[4]) {
+        float v[8];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const uint32_t m = __builtin_amdgcn_perm(pairs[r], pairs[r], sel[r]);
+            v[2 * r] = half_value<T>(m, false);
+            v[2 * r + 1] = half_value<T>(m, true);
+        }
+        float acc = v[0] * wt[0];
+#pragma unroll
+        for (int k = 1; k < 8; k++) {
+            acc += v[k] * wt[k];
+        }
+        ElemIO<T>::store(yc, acc);
+        yc += p.out_vol;
+    };
+    for (int32_t c = c_begin; c < c_end; c++) {
+        uint32_t pairs[4];
+        fetch(pairs);
+        blend_and_store(pairs);
+    }
+}
+
 // Channels-last (NDHWC) variant: the C values of a voxel are contiguous, so a corner is one load of up to 16 bytes
 // instead of C scattered two- or four-byte loads.  A lane owns one unit of UE consecutive channels of one output
 // point (consecutive lanes own consecutive units, so loads and stores of neighbouring lanes are contiguous); the
@@ -383,6 +495,13 @@ hipError_t launch_one(const GridSampler3DArgs& a, hipStream_t stream)
     const int64_t ychunks = (a.C + p.chan_chunk - 1) / p.chan_chunk;
     if (pblocks > INT32_MAX || ychunks > 65535) {
         return hipErrorInvalidValue;
+    }
+    if constexpr (sizeof(T) == 2 && INTERP == 0) {
+        if (a.Win >= 2 && a.Din * a.Hin * a.Win <= INT32_MAX) {
+            hipLaunchKernelGGL((gs3d_pair16_kernel<T, PAD, ALIGN>), dim3((unsigned)pblocks, (unsigned)ychunks),
+                               dim3(kThreads), 0, stream, (const T*)a.x, (const T*)a.grid, (T*)a.y, p);
+            return hipGetLastError();
+        }
     }
     hipLaunchKernelGGL((gs3d_kernel<T, INTERP, PAD, ALIGN>), dim3((unsigned)pblocks, (unsigned)ychunks),
                        dim3(kThreads), 0, stream, (const T*)a.x, (const T*)a.grid, (T*)a.y, p);
