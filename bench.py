@@ -32,6 +32,7 @@ MEASURED_TRAFFIC = {
     ("C4", "nchw_band_lds"): (1415.4e6, "profiles/resize_band_lds_C4_fp16_4k_upscale.md"),
     ("C2", "nchw_flat_lds"): (32.43e6, "profiles/resize_flat_lds_C2_fp32_56_to_112.md"),
     ("C5", "lds_pair_w128"): (176.3e6, "profiles/gs2d_lds_pair_C5_bf16_random_gather.md"),
+    ("L1", "box_lds"): (742.5e6, "profiles/gs2d_box_L1_fp16_1080p.md"),
     ("V1", "gs3d_bilinear"): (38.72e6, "profiles/gs3d_V1_fp16_22x4x16x64x64.md"),
     ("G3", "gs2d_grad_lists_lds"): (182.8e6, "profiles/gs2d_grad_G3_fp16_n16_c256.md"),
     ("W1", "gs3d_grad_lists"): (200.1e6, "profiles/gs3d_grad_W1_fp16_22x4x16x64x64.md"),

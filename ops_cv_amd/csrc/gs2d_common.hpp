@@ -79,6 +79,11 @@ const char* gs2d_lds_variant_name(const GridSamplerArgs& a);
 hipError_t run_gs2d_pair(const GridSamplerArgs& a, hipStream_t stream, bool* handled);
 const char* gs2d_pair_variant_name(const GridSamplerArgs& a);
 
+// Box variant (gs2d_box.hip): bilinear, 16-bit elements, planes beyond the LDS variants; the box of input pixels that a
+// tile of output pixels reads goes through LDS.  Same convention as run_gs2d_lds.
+hipError_t run_gs2d_box(const GridSamplerArgs& a, hipStream_t stream, bool* handled);
+const char* gs2d_box_variant_name(const GridSamplerArgs& a);
+
 // Channels-last variant (gs2d_nhwc.hip): a.x is (N,Hin,Win,C), a.y is (N,Hout,Wout,C).
 hipError_t run_gs2d_nhwc(const GridSamplerArgs& a, hipStream_t stream);
 

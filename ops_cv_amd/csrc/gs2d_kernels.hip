@@ -381,6 +381,9 @@ const char* grid_sampler2d_variant(const GridSamplerArgs& a)
         if (n == nullptr) {
             n = gs2d_lds_variant_name(a);
         }
+        if (n == nullptr) {
+            n = gs2d_box_variant_name(a);
+        }
         if (n != nullptr) {
             return n;
         }
@@ -409,6 +412,10 @@ hipError_t launch_grid_sampler2d(const GridSamplerArgs& a, hipStream_t stream)
             return e;
         }
         e = run_gs2d_lds(a, stream, &handled);
+        if (handled || e != hipSuccess) {
+            return e;
+        }
+        e = run_gs2d_box(a, stream, &handled);
         if (handled || e != hipSuccess) {
             return e;
         }

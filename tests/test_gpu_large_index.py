@@ -48,7 +48,7 @@ def _variant(aclnn, x, g, y, interp, pad, align):
     return v
 
 
-@pytest.mark.parametrize("case", ["lds_ring", "lds_pair", "direct", "nhwc"])
+@pytest.mark.parametrize("case", ["lds_ring", "lds_pair", "direct", "box_lds", "box_lds_scattered", "nhwc"])
 def test_grid_sampler_beyond_2_31_elements(oracle, device, aclnn, case):
     import torch
     torch.manual_seed(11)
@@ -56,19 +56,25 @@ def test_grid_sampler_beyond_2_31_elements(oracle, device, aclnn, case):
         N, C, H, W, Ho, Wo, interp, pad, align = 2, 140000, 128, 64, 128, 64, 0, 0, False
     elif case == "lds_pair":    # output beyond 2^31 elements through the pair-layout kernel
         N, C, H, W, Ho, Wo, interp, pad, align = 1, 40000, 64, 32, 240, 240, 0, 1, True
-    elif case == "direct":      # planes far beyond LDS: the direct kernel
+    elif case == "direct":      # planes far beyond LDS: the direct kernel (nearest samples; bicubic and fp32 too)
+        N, C, H, W, Ho, Wo, interp, pad, align = 1, 2100, 1024, 1024, 1024, 1024, 1, 2, False
+    elif case.startswith("box_lds"):  # planes far beyond LDS, bilinear: a tile's box of the input through LDS
         N, C, H, W, Ho, Wo, interp, pad, align = 1, 2100, 1024, 1024, 1024, 1024, 0, 2, False
     else:                       # channels-last views of NHWC memory
         N, C, H, W, Ho, Wo, interp, pad, align = 1, 2100, 1024, 1024, 1024, 1024, 1, 0, False
     assert N * C * Ho * Wo >= TWO31
     x = torch.randn((N, C, H, W), device=device, dtype=torch.float16)
     g = (torch.rand((N, Ho, Wo, 2), device=device) * 2.3 - 1.15).to(torch.float16)
+    if case == "box_lds":
+        # a smooth warp, so that the tiles' boxes fit (scattered points, the case after this one, take the kernel's
+        # pair loads instead)
+        g = torch.from_numpy(I.affine_grid(np.random.default_rng(11), N, Ho, Wo)).to(device).to(torch.float16)
     y = torch.empty((N, C, Ho, Wo), device=device, dtype=torch.float16)
     if case == "nhwc":
         x = x.contiguous(memory_format=torch.channels_last)
         y = y.contiguous(memory_format=torch.channels_last)
     v = _variant(aclnn, x, g, y, interp, pad, align)
-    assert v.startswith(case), v
+    assert v.startswith("box_lds" if case.startswith("box_lds") else case), v
     aclnn.grid_sampler2d(x, g, interp, pad, align, out=y)
     torch.cuda.synchronize()
     _check_sampler_channels(oracle, x, g, y, interp, pad, align, [slice(0, 2), slice(C // 2, C // 2 + 2),
