@@ -55,7 +55,7 @@ GS_WORKLOADS = {
                sets=8),
     "C5": dict(dtype="bf16", x=(8, 128, 128, 128), grid=(8, 256, 256), kind="random", interp=0, pad=1, align=True,
                sets=3),
-    # not a BASELINE configuration: input planes of 4 MB, far beyond LDS, which only the direct kernel serves
+    # not a BASELINE configuration: input planes of 4 MB, far beyond the LDS variants (image warps)
     "L1": dict(dtype="fp16", x=(2, 32, 1080, 1920), grid=(2, 1080, 1920), kind="affine", interp=0, pad=0, align=False,
                sets=2),
 }
@@ -807,6 +807,9 @@ def main():
         for name in ("C2", "C4"):
             if name != head:
                 others[name] = summary_of(bench_up(name, ko, args.warmup))
+        if head != "L1":
+            # not a BASELINE configuration: planes beyond LDS (1080p), the shape image warps come in
+            others["L1_sampler_1080p_planes"] = summary_of(bench_gs("L1", min(ko, 50), min(args.warmup, 5)))
         # the entry points either side of the path, on shapes of the same scale
         others["V1_grid_sampler3d"] = summary_of(bench_gs3d(ko, args.warmup))
         others["V1_grid_sampler3d_ndhwc"] = summary_of(bench_gs3d(ko, args.warmup, channels_last=True))
