@@ -109,6 +109,42 @@ def test_random_grid_sampler2d_large_planes(oracle, device, aclnn):
         _same(I.from_torch(y, dtype), ref, dtype, (case, dtype, N, C, H, W, Ho, Wo, interp, pad, align))
 
 
+def test_random_grid_sampler2d_box_variant(oracle, device, aclnn):
+    """planes beyond the LDS variants under smooth warps of random angle and scale, 16-bit elements: tiles whose box of
+    input pixels goes through LDS, next to tiles that fall back to loads from global memory (strong minification,
+    sprinkled special values), tiles cut by the edges of the output, channel counts of every remainder"""
+    import torch
+    rng = np.random.default_rng(9005 + SEED_SHIFT)
+    for case in range(30):
+        dtype = ("fp16", "bf16")[case % 2]
+        N, C = int(rng.integers(1, 3)), int(rng.integers(1, 10))
+        H = int(rng.integers(120, 400))
+        W = 8 * int(rng.integers((41000 // H) // 8 + 1, 60))  # rows of whole 16-byte units, planes above 80 KB
+        Ho = int(rng.integers(32, 200))
+        Wo = 2 * int(rng.integers(32, 120))
+        pad, align = int(rng.integers(0, 3)), bool(rng.integers(0, 2))
+        deg = float(rng.choice([5.0, 30.0, 90.0]))
+        lo = float(rng.choice([0.3, 0.8, 1.0]))
+        _say("gs2d box", dtype, N, C, H, W, Ho, Wo, pad, align, deg, lo)
+        x = I.cast_np(rng.standard_normal((N, C, H, W)).astype(np.float32), dtype)
+        g32 = I.affine_grid(rng, N, Ho, Wo, max_deg=deg, scale=(lo, lo * 1.5), shift=0.3)
+        if case % 3 == 1:
+            g32 = _sprinkle(rng, g32, H, W, align)
+        g = I.cast_np(g32, dtype)
+        tx, tg = I.to_torch(x, dtype, device), I.to_torch(g, dtype, device)
+        ty = torch.empty((N, C, Ho, Wo), dtype=tx.dtype, device=device)
+        hs = [aclnn.tensor_handle(t) for t in (tx, tg, ty)]
+        st, _, ex = aclnn.get_workspace_size_grid_sampler2d(hs[0], hs[1], 0, pad, align, hs[2])
+        assert st == 0 and aclnn.executor_variant(ex) == "box_lds", (H, W, Ho, Wo)
+        aclnn.destroy_executor(ex)
+        for h in hs:
+            aclnn.destroy_tensor(h)
+        ref = oracle.grid_sampler2d(x, g, 0, pad, align, dtype=I.oracle_code(dtype))
+        y = aclnn.grid_sampler2d(tx, tg, 0, pad, align)
+        torch.cuda.synchronize()
+        _same(I.from_torch(y, dtype), ref, dtype, (case, dtype, N, C, H, W, Ho, Wo, pad, align, deg, lo))
+
+
 def test_random_resize_family(oracle, device, aclnn, monkeypatch):
     import torch
     rng = np.random.default_rng(9002 + SEED_SHIFT)
