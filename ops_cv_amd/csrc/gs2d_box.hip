@@ -218,11 +218,12 @@ __global__ __launch_bounds__(kBoxThreads) void gs2d_box_kernel(const T* __restri
     uint32_t toff[kBoxPpl][4];
 #pragma unroll
     for (int j = 0; j < kBoxPpl; j++) {
+        // a lane off the image decided a pixel of some other tile: its taps are not in this box, it reads the zeros
         const uint32_t o_nw = (y0[j] - (uint32_t)y_lo) * pitch + (x0[j] * 2u - byte_lo);
-        toff[j][0] = (in_y0[j] && in_x0[j]) ? o_nw : kBoxZero;
-        toff[j][1] = (in_y0[j] && in_x1[j]) ? o_nw + 2u : kBoxZero;
-        toff[j][2] = (in_y1[j] && in_x0[j]) ? o_nw + pitch : kBoxZero;
-        toff[j][3] = (in_y1[j] && in_x1[j]) ? o_nw + pitch + 2u : kBoxZero;
+        toff[j][0] = (live[j] && in_y0[j] && in_x0[j]) ? o_nw : kBoxZero;
+        toff[j][1] = (live[j] && in_y0[j] && in_x1[j]) ? o_nw + 2u : kBoxZero;
+        toff[j][2] = (live[j] && in_y1[j] && in_x0[j]) ? o_nw + pitch : kBoxZero;
+        toff[j][3] = (live[j] && in_y1[j] && in_x1[j]) ? o_nw + pitch + 2u : kBoxZero;
     }
     // copying: eight lanes a box row, lane k of them its k-th unit; the same unit of every channel of a group
     const uint32_t my_unit = tid % kBoxRowUnits, my_row = tid / kBoxRowUnits;
