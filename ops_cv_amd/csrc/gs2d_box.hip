@@ -1,4 +1,4 @@
-// Grid sampler 2-D forward, bilinear, 16-bit elements, input planes too large for the LDS variants: box variant.
+// Grid sampler 2-D forward, 16-bit elements, input planes too large for the LDS variants: box variant.
 //
 // Same arithmetic as the other variants (sampler_math.hpp, blend() in gs2d_lds_kernel.hpp; reference kernel
 // image/grid_sampler2_d/op_kernel/arch35/grid_sampler2_d_simt.h:303-339,461-514).  The direct kernel reads every tap
@@ -10,8 +10,8 @@
 // eight lanes a row -- into LDS and takes the taps from there with two-byte LDS reads.  The box of a tile under a
 // smooth warp is little larger than the tile turned and scaled.  Two channel groups are on their way in registers
 // while one is sampled (two LDS buffers, a barrier per group).  A tile whose box does not fit (scattered points,
-// strong minification) falls back, the whole workgroup together, to pair loads from global memory as the direct
-// kernel makes them.
+// strong minification) falls back, the whole workgroup together, to loads from global memory as the direct
+// kernel makes them (bilinear: the west and east tap of a row as one load).
 // fp16 2x32x1080x1920, warps of up to 30 degrees: 318 us direct, 202 us here.
 #include <hip/hip_runtime.h>
 
@@ -63,11 +63,15 @@ struct BoxParams {
     float neg_zero;
 };
 
-template <typename T, int PAD, bool ALIGN>
+template <typename T, int INTERP, int PAD, bool ALIGN>
 __global__ __launch_bounds__(kBoxThreads) void gs2d_box_kernel(const T* __restrict__ x, const T* __restrict__ grid,
                                                                 T* __restrict__ y, BoxParams p)
 {
     static_assert(sizeof(T) == 2, "two-byte elements");
+    // taps per axis: bilinear 2 x 2, nearest 1, bicubic 4 x 4; tap (r, k) is row by[r], column bx[k]
+    constexpr int NA = (INTERP == 0) ? 2 : (INTERP == 1 ? 1 : 4);
+    constexpr int NT = NA * NA;
+    constexpr int NW = (INTERP == 2) ? 8 : 4;
     __shared__ __attribute__((aligned(16))) char lds[2 * kBoxBuf];
     __shared__ int32_t s_box[4];  // lowest column and row, highest column and row a tap of the tile lies in
     const uint32_t tid = threadIdx.x;
@@ -87,15 +91,15 @@ __global__ __launch_bounds__(kBoxThreads) void gs2d_box_kernel(const T* __restri
     const T* xc = x + (n * p.C + c_begin) * in_plane;
     T* ybase = y + (n * p.C + c_begin) * out_plane;
 
-    // the decisions of decide_pixel() (sampler_math.hpp; grid_sampler2_d_simt.h:479-498, 307-316) without branches,
-    // as in the LDS kernels, for the lane's kBoxPpl pixels
+    // the decisions of decide_pixel() / decide_bicubic() (sampler_math.hpp; grid_sampler2_d_simt.h:479-503, 307-316,
+    // 341-349, 379-412), bilinear and nearest without branches as in the LDS kernels, for the lane's kBoxPpl pixels
     const int32_t ox0 = (int32_t)(tx * kTileW + kBoxPpl * (tid % kRowLanes));
     const int32_t oy = (int32_t)(ty * kTileH + tid / kRowLanes);
     bool live[kBoxPpl];
     uint32_t out_off[kBoxPpl];  // byte offset in an output plane; out of the plane's range for lanes off the image
-    uint32_t x0[kBoxPpl], y0[kBoxPpl];
-    bool in_x0[kBoxPpl], in_x1[kBoxPpl], in_y0[kBoxPpl], in_y1[kBoxPpl];
-    float tw[kBoxPpl][4];
+    uint32_t bx[kBoxPpl][NA], by[kBoxPpl][NA];  // tap columns and rows
+    bool okx[kBoxPpl][NA], oky[kBoxPpl][NA];    // ... inside the image (none for a non-finite source coordinate)
+    float tw[kBoxPpl][NW];
     const uint32_t uw = (uint32_t)p.W, uh = (uint32_t)p.H;
     float gxs[kBoxPpl], gys[kBoxPpl];
 #pragma unroll
@@ -110,28 +114,60 @@ __global__ __launch_bounds__(kBoxThreads) void gs2d_box_kernel(const T* __restri
     }
 #pragma unroll
     for (int j = 0; j < kBoxPpl; j++) {
-        float ix = compute_source_index<PAD, ALIGN>(gxs[j], p.W);
-        float iy = compute_source_index<PAD, ALIGN>(gys[j], p.H);
-        const bool finite = __builtin_fabsf(ix) < __builtin_inff() && __builtin_fabsf(iy) < __builtin_inff();
-        const bool x_far = ix > 2147483646.0f || ix < -2147483648.0f;  // safe_downgrade: -> -100, always outside
-        const bool y_far = iy > 2147483646.0f || iy < -2147483648.0f;
-        ix = x_far ? -100.0f : ix;
-        iy = y_far ? -100.0f : iy;
-        const float ixf = __builtin_floorf(ix), iyf = __builtin_floorf(iy);
-        x0[j] = (uint32_t)float_to_i32(ixf);
-        y0[j] = (uint32_t)float_to_i32(iyf);
-        in_x0[j] = x0[j] < uw && finite;
-        in_x1[j] = x0[j] + 1u < uw && finite;
-        in_y0[j] = y0[j] < uh;
-        in_y1[j] = y0[j] + 1u < uh;
-        const float wx1 = ix - ixf, wx0 = ixf + 1.0f - ix;
-        const float wy1 = iy - iyf, wy0 = iyf + 1.0f - iy;
-        // non-finite source coordinate: every tap reads zeros and 0 * NaN makes every channel NaN, as the reference
-        // writes (grid_sampler2_d_simt.h:485-487)
-        tw[j][0] = finite ? wx0 * wy0 : __builtin_nanf("");
-        tw[j][1] = wx1 * wy0;
-        tw[j][2] = wx0 * wy1;
-        tw[j][3] = wx1 * wy1;
+        if constexpr (INTERP == 2) {
+            const BicubicTap b = decide_bicubic<PAD, ALIGN>(gxs[j], gys[j], p.H, p.W);
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                bx[j][k] = (uint32_t)b.bx[k];
+                by[j][k] = (uint32_t)b.by[k];
+                okx[j][k] = b.bx[k] >= 0 && b.bx[k] < p.W && !b.flag;
+                oky[j][k] = b.by[k] >= 0 && b.by[k] < p.H;
+                tw[j][k] = b.cx[k];
+                tw[j][4 + k] = b.cy[k];
+            }
+            if (b.flag) {
+                tw[j][0] = __builtin_nanf("");  // 0 * NaN: every channel becomes NaN, as the reference writes
+            }
+        } else {
+            float ix = compute_source_index<PAD, ALIGN>(gxs[j], p.W);
+            float iy = compute_source_index<PAD, ALIGN>(gys[j], p.H);
+            const bool finite = __builtin_fabsf(ix) < __builtin_inff() && __builtin_fabsf(iy) < __builtin_inff();
+            const bool x_far = ix > 2147483646.0f || ix < -2147483648.0f;  // safe_downgrade: -> -100, always outside
+            const bool y_far = iy > 2147483646.0f || iy < -2147483648.0f;
+            if constexpr (INTERP == 0) {
+                ix = x_far ? -100.0f : ix;
+                iy = y_far ? -100.0f : iy;
+                const float ixf = __builtin_floorf(ix), iyf = __builtin_floorf(iy);
+                bx[j][0] = (uint32_t)float_to_i32(ixf);
+                by[j][0] = (uint32_t)float_to_i32(iyf);
+                bx[j][1] = bx[j][0] + 1u;  // wraps at INT32_MAX: out of bounds either way
+                by[j][1] = by[j][0] + 1u;
+                okx[j][0] = bx[j][0] < uw && finite;
+                okx[j][1] = bx[j][1] < uw && finite;
+                oky[j][0] = by[j][0] < uh;
+                oky[j][1] = by[j][1] < uh;
+                const float wx1 = ix - ixf, wx0 = ixf + 1.0f - ix;
+                const float wy1 = iy - iyf, wy0 = iyf + 1.0f - iy;
+                // non-finite source coordinate: every tap reads zeros and 0 * NaN makes every channel NaN, as the
+                // reference writes (grid_sampler2_d_simt.h:485-487)
+                tw[j][0] = finite ? wx0 * wy0 : __builtin_nanf("");
+                tw[j][1] = wx1 * wy0;
+                tw[j][2] = wx0 * wy1;
+                tw[j][3] = wx1 * wy1;
+            } else {
+                ix = (x_far || !finite) ? -100.0f : ix;
+                iy = (y_far || !finite) ? -100.0f : iy;
+                // round half to even from floor, fraction and parity (grid_sampler2_d_simt.h:219-234)
+                const float xf = __builtin_floorf(ix), yf = __builtin_floorf(iy);
+                const float fx = ix - xf, fy = iy - yf;
+                const uint32_t xi = (uint32_t)float_to_i32(xf), yi = (uint32_t)float_to_i32(yf);
+                bx[j][0] = xi + ((fx > 0.5f || (fx == 0.5f && (xi & 1u))) ? 1u : 0u);
+                by[j][0] = yi + ((fy > 0.5f || (fy == 0.5f && (yi & 1u))) ? 1u : 0u);
+                okx[j][0] = bx[j][0] < uw;
+                oky[j][0] = by[j][0] < uh;
+                tw[j][0] = tw[j][1] = tw[j][2] = tw[j][3] = 0.0f;
+            }
+        }
     }
 
     if (tid < 4) {
@@ -142,14 +178,19 @@ __global__ __launch_bounds__(kBoxThreads) void gs2d_box_kernel(const T* __restri
     }
     __syncthreads();
     {
-        // the columns and rows inside the image among a pixel's two each; a pixel with none on an axis reads nothing
+        // the columns and rows inside the image among a pixel's taps; a pixel with none on an axis reads nothing
         int32_t lo_x = INT32_MAX, lo_y = INT32_MAX, hi_x = -1, hi_y = -1;
 #pragma unroll
         for (int j = 0; j < kBoxPpl; j++) {
-            const int32_t lx = in_x0[j] ? (int32_t)x0[j] : (in_x1[j] ? (int32_t)x0[j] + 1 : INT32_MAX);
-            const int32_t hx = in_x1[j] ? (int32_t)x0[j] + 1 : (in_x0[j] ? (int32_t)x0[j] : -1);
-            const int32_t ly = in_y0[j] ? (int32_t)y0[j] : (in_y1[j] ? (int32_t)y0[j] + 1 : INT32_MAX);
-            const int32_t hy = in_y1[j] ? (int32_t)y0[j] + 1 : (in_y0[j] ? (int32_t)y0[j] : -1);
+            int32_t lx = INT32_MAX, ly = INT32_MAX, hx = -1, hy = -1;
+#pragma unroll
+            for (int k = 0; k < NA; k++) {
+                const int32_t cx = (int32_t)bx[j][k], cy = (int32_t)by[j][k];
+                lx = (okx[j][k] && cx < lx) ? cx : lx;
+                hx = (okx[j][k] && cx > hx) ? cx : hx;
+                ly = (oky[j][k] && cy < ly) ? cy : ly;
+                hy = (oky[j][k] && cy > hy) ? cy : hy;
+            }
             if (live[j] && hx >= 0 && hy >= 0) {
                 lo_x = lx < lo_x ? lx : lo_x;
                 hi_x = hx > hi_x ? hx : hi_x;
@@ -179,51 +220,86 @@ __global__ __launch_bounds__(kBoxThreads) void gs2d_box_kernel(const T* __restri
     const uint32_t pitch = upr * 16u;
 
     if (rows * pitch > kBoxZero || upr > kBoxRowUnits || rows > kBoxRows) {
-        // ------------------------------------------------ the box does not fit: pair loads from global memory ---
-        // The west and east tap of a row as one load of two elements from column pb = clamp(x0, 0, W - 2); one
-        // byte-permute puts the west value in the low half, the east value in the high half and zeroes the half whose
-        // tap is outside the image; a row without a valid tap reads the plane's first pair, zeroed the same way.
+        // ------------------------------------------------ the box does not fit: loads from global memory ---------
 #pragma unroll
         for (int j = 0; j < kBoxPpl; j++) {
             if (!live[j]) {
                 continue;
             }
-            const int32_t sx0 = (int32_t)x0[j];
-            const int32_t pb = (sx0 < 0) ? 0 : ((sx0 > p.W - 2) ? p.W - 2 : sx0);
-            const uint32_t at_w = (sx0 == pb) ? kSelLow : kSelHigh, at_e = ((int32_t)(x0[j] + 1u) == pb) ? kSelLow : kSelHigh;
-            const uint32_t sel_n = ((in_y0[j] && in_x0[j]) ? at_w : kSelZero) | (((in_y0[j] && in_x1[j]) ? at_e : kSelZero) << 16);
-            const uint32_t sel_s = ((in_y1[j] && in_x0[j]) ? at_w : kSelZero) | (((in_y1[j] && in_x1[j]) ? at_e : kSelZero) << 16);
-            typedef const __attribute__((address_space(1))) T* GlobalRow;
-            const bool any_x = in_x0[j] || in_x1[j];
-            GlobalRow pn = (GlobalRow)(xc + ((in_y0[j] && any_x) ? (int64_t)y0[j] * p.W + pb : 0));
-            GlobalRow ps = (GlobalRow)(xc + ((in_y1[j] && any_x) ? (int64_t)(y0[j] + 1u) * p.W + pb : 0));
             T* yc = reinterpret_cast<T*>(reinterpret_cast<char*>(ybase) + out_off[j]);
+            if constexpr (INTERP == 0) {
+                // The west and east tap of a row as one load of two elements from column pb = clamp(x0, 0, W - 2); one
+                // byte-permute puts the west value in the low half, the east value in the high half and zeroes the
+                // half whose tap is outside the image; a row without a valid tap reads the plane's first pair, zeroed
+                // the same way.
+                const int32_t sx0 = (int32_t)bx[j][0];
+                const int32_t pb = (sx0 < 0) ? 0 : ((sx0 > p.W - 2) ? p.W - 2 : sx0);
+                const uint32_t at_w = (sx0 == pb) ? kSelLow : kSelHigh, at_e = ((int32_t)bx[j][1] == pb) ? kSelLow : kSelHigh;
+                const uint32_t sel_n = ((oky[j][0] && okx[j][0]) ? at_w : kSelZero) | (((oky[j][0] && okx[j][1]) ? at_e : kSelZero) << 16);
+                const uint32_t sel_s = ((oky[j][1] && okx[j][0]) ? at_w : kSelZero) | (((oky[j][1] && okx[j][1]) ? at_e : kSelZero) << 16);
+                typedef const __attribute__((address_space(1))) T* GlobalRow;
+                const bool any_x = okx[j][0] || okx[j][1];
+                GlobalRow pn = (GlobalRow)(xc + ((oky[j][0] && any_x) ? (int64_t)by[j][0] * p.W + pb : 0));
+                GlobalRow ps = (GlobalRow)(xc + ((oky[j][1] && any_x) ? (int64_t)by[j][1] * p.W + pb : 0));
 #pragma unroll 4
-            for (int32_t c = c_begin; c < c_end; c++) {
-                const uint32_t north = *(const __attribute__((address_space(1), aligned(2))) UnalignedWord*)pn;
-                const uint32_t south = *(const __attribute__((address_space(1), aligned(2))) UnalignedWord*)ps;
-                const uint32_t mn = __builtin_amdgcn_perm(north, north, sel_n);
-                const uint32_t ms = __builtin_amdgcn_perm(south, south, sel_s);
-                const uint32_t raw[4] = {mn & 0xffffu, mn >> 16, ms & 0xffffu, ms >> 16};
-                ElemIO<T>::store(yc, blend<T, 0>(raw, tw[j], p.neg_zero));
-                pn += in_plane;
-                ps += in_plane;
-                yc += out_plane;
+                for (int32_t c = c_begin; c < c_end; c++) {
+                    const uint32_t north = *(const __attribute__((address_space(1), aligned(2))) UnalignedWord*)pn;
+                    const uint32_t south = *(const __attribute__((address_space(1), aligned(2))) UnalignedWord*)ps;
+                    const uint32_t mn = __builtin_amdgcn_perm(north, north, sel_n);
+                    const uint32_t ms = __builtin_amdgcn_perm(south, south, sel_s);
+                    const uint32_t raw[4] = {mn & 0xffffu, mn >> 16, ms & 0xffffu, ms >> 16};
+                    ElemIO<T>::store(yc, blend<T, 0>(raw, tw[j], p.neg_zero));
+                    pn += in_plane;
+                    ps += in_plane;
+                    yc += out_plane;
+                }
+            } else {
+                // one load per tap, none with a branch around it: a tap outside the image reads the plane's first
+                // element and is replaced by zero
+                uint32_t at[NT];  // element offsets in a plane (planes hold fewer than 2^31 elements)
+                bool ok[NT];
+#pragma unroll
+                for (int r = 0; r < NA; r++) {
+#pragma unroll
+                    for (int k = 0; k < NA; k++) {
+                        ok[r * NA + k] = oky[j][r] && okx[j][k];
+                        at[r * NA + k] = ok[r * NA + k] ? by[j][r] * uw + bx[j][k] : 0u;
+                    }
+                }
+                const __attribute__((address_space(1))) uint16_t* xp =
+                    (const __attribute__((address_space(1))) uint16_t*)xc;
+                for (int32_t c = c_begin; c < c_end; c++) {
+                    uint32_t raw[NT];
+#pragma unroll
+                    for (int i = 0; i < NT; i++) {
+                        raw[i] = xp[at[i]];
+                    }
+#pragma unroll
+                    for (int i = 0; i < NT; i++) {
+                        raw[i] = ok[i] ? raw[i] : 0u;
+                    }
+                    ElemIO<T>::store(yc, blend<T, INTERP>(raw, tw[j], p.neg_zero));
+                    xp += in_plane;
+                    yc += out_plane;
+                }
             }
         }
         return;
     }
 
-    // LDS byte offsets of the four taps in a channel's box
-    uint32_t toff[kBoxPpl][4];
+    // LDS byte offsets of the taps in a channel's box
+    uint32_t toff[kBoxPpl][NT];
 #pragma unroll
     for (int j = 0; j < kBoxPpl; j++) {
         // a lane off the image decided a pixel of some other tile: its taps are not in this box, it reads the zeros
-        const uint32_t o_nw = (y0[j] - (uint32_t)y_lo) * pitch + (x0[j] * 2u - byte_lo);
-        toff[j][0] = (live[j] && in_y0[j] && in_x0[j]) ? o_nw : kBoxZero;
-        toff[j][1] = (live[j] && in_y0[j] && in_x1[j]) ? o_nw + 2u : kBoxZero;
-        toff[j][2] = (live[j] && in_y1[j] && in_x0[j]) ? o_nw + pitch : kBoxZero;
-        toff[j][3] = (live[j] && in_y1[j] && in_x1[j]) ? o_nw + pitch + 2u : kBoxZero;
+#pragma unroll
+        for (int r = 0; r < NA; r++) {
+            const uint32_t row = (by[j][r] - (uint32_t)y_lo) * pitch - byte_lo;
+#pragma unroll
+            for (int k = 0; k < NA; k++) {
+                toff[j][r * NA + k] = (live[j] && oky[j][r] && okx[j][k]) ? row + bx[j][k] * 2u : kBoxZero;
+            }
+        }
     }
     // copying: eight lanes a box row, lane k of them its k-th unit; the same unit of every channel of a group
     const uint32_t my_unit = tid % kBoxRowUnits, my_row = tid / kBoxRowUnits;
@@ -270,12 +346,12 @@ __global__ __launch_bounds__(kBoxThreads) void gs2d_box_kernel(const T* __restri
             float v[kBoxPpl];
 #pragma unroll
             for (int j = 0; j < kBoxPpl; j++) {
-                uint32_t raw[4];
+                uint32_t raw[NT];
 #pragma unroll
-                for (int k = 0; k < 4; k++) {
+                for (int k = 0; k < NT; k++) {
                     raw[k] = *reinterpret_cast<const uint16_t*>(lds + buf * kBoxBuf + cc * kBoxChanBytes + toff[j][k]);
                 }
-                v[j] = blend<T, 0>(raw, tw[j], p.neg_zero);
+                v[j] = blend<T, INTERP>(raw, tw[j], p.neg_zero);
             }
             buffer_store_group<T, kBoxPpl>(v, rsrc, out_off[0]);
         }
@@ -302,7 +378,7 @@ __global__ __launch_bounds__(kBoxThreads) void gs2d_box_kernel(const T* __restri
 #undef OPSCV_BOX_STASH
 }
 
-template <typename T, int PAD, bool ALIGN>
+template <typename T, int INTERP, int PAD, bool ALIGN>
 hipError_t launch_box(const GridSamplerArgs& a, hipStream_t stream)
 {
     BoxParams p;
@@ -326,30 +402,41 @@ hipError_t launch_box(const GridSamplerArgs& a, hipStream_t stream)
     p.chan_chunk = (int32_t)per;
     const int64_t by = (a.C + per - 1) / per;
     p.neg_zero = -0.0f;
-    hipLaunchKernelGGL((gs2d_box_kernel<T, PAD, ALIGN>), dim3((unsigned)tiles, (unsigned)by), dim3(kBoxThreads), 0,
+    hipLaunchKernelGGL((gs2d_box_kernel<T, INTERP, PAD, ALIGN>), dim3((unsigned)tiles, (unsigned)by), dim3(kBoxThreads), 0,
                        stream, (const T*)a.x, (const T*)a.grid, (T*)a.y, p);
     return hipGetLastError();
+}
+
+template <typename T, int INTERP>
+hipError_t launch_box_interp(const GridSamplerArgs& a, hipStream_t stream)
+{
+    switch (a.pad * 2 + a.align) {
+        case 0: return launch_box<T, INTERP, 0, false>(a, stream);
+        case 1: return launch_box<T, INTERP, 0, true>(a, stream);
+        case 2: return launch_box<T, INTERP, 1, false>(a, stream);
+        case 3: return launch_box<T, INTERP, 1, true>(a, stream);
+        case 4: return launch_box<T, INTERP, 2, false>(a, stream);
+        case 5: return launch_box<T, INTERP, 2, true>(a, stream);
+        default: return hipErrorInvalidValue;
+    }
 }
 
 template <typename T>
 hipError_t launch_box_typed(const GridSamplerArgs& a, hipStream_t stream)
 {
-    switch (a.pad * 2 + a.align) {
-        case 0: return launch_box<T, 0, false>(a, stream);
-        case 1: return launch_box<T, 0, true>(a, stream);
-        case 2: return launch_box<T, 1, false>(a, stream);
-        case 3: return launch_box<T, 1, true>(a, stream);
-        case 4: return launch_box<T, 2, false>(a, stream);
-        case 5: return launch_box<T, 2, true>(a, stream);
+    switch (a.interp) {
+        case 0: return launch_box_interp<T, 0>(a, stream);
+        case 1: return launch_box_interp<T, 1>(a, stream);
+        case 2: return launch_box_interp<T, 2>(a, stream);
         default: return hipErrorInvalidValue;
     }
 }
 
-// What the kernel assumes: bilinear samples of two-byte elements; input rows of whole 16-byte units on 16-byte
+// What the kernel assumes: two-byte elements; input rows of whole 16-byte units on 16-byte
 // boundaries, two columns or more; output planes that fill the tiles; counts that fit the launch.
 bool box_applies(const GridSamplerArgs& a)
 {
-    if (a.elem == Elem::F32 || a.interp != 0 || a.channels_last) {
+    if (a.elem == Elem::F32 || a.interp < 0 || a.interp > 2 || a.channels_last) {
         return false;
     }
     if (a.Win < 2 || (a.Win * 2) % 16 != 0 || reinterpret_cast<uintptr_t>(a.x) % 16 != 0) {

@@ -383,15 +383,16 @@ def test_grid_sampler3d(oracle, device, aclnn, dtype, interp):
                     (N, C, D, H, W, Do, Ho, Wo, pad, align)
 
 
+@pytest.mark.parametrize("interp", [0, 1, 2])
 @pytest.mark.parametrize("dtype", ["fp16", "bf16"])
-def test_grid_sampler2d_box_variant(oracle, device, aclnn, dtype):
-    """Bilinear samples of 16-bit elements on planes beyond the LDS variants (80 KB): a tile of 32 x 16 output pixels copies
+def test_grid_sampler2d_box_variant(oracle, device, aclnn, dtype, interp):
+    """Samples of 16-bit elements on planes beyond the LDS variants (80 KB), every interpolation mode: a tile of 32 x 16 output pixels copies
     the box of input pixels it reads into LDS.  Smooth warps (boxes that fit), scattered points and strong
     minification (boxes that do not: pair loads from global memory), a batch item whose points all lie outside the
     image, special grid values, tiles cut by the right and lower edge, channel counts that are not whole groups of
     four, few tiles (runs of channels to different workgroups); every padding and alignment; bit for bit the oracle"""
     torch = _torch()
-    rng = np.random.default_rng(640)
+    rng = np.random.default_rng(640 + interp)
     cases = [
         # N, C, H, W, Ho, Wo, kind
         (2, 5, 208, 200, 70, 100, "affine"),
@@ -421,26 +422,26 @@ def test_grid_sampler2d_box_variant(oracle, device, aclnn, dtype):
                 tx, tg = I.to_torch(x, dtype, device), I.to_torch(g, dtype, device)
                 ty = torch.empty((N, C, Ho, Wo), dtype=tx.dtype, device=device)
                 hs = [aclnn.tensor_handle(t) for t in (tx, tg, ty)]
-                st, _, ex = aclnn.get_workspace_size_grid_sampler2d(hs[0], hs[1], 0, pad, align, hs[2])
+                st, _, ex = aclnn.get_workspace_size_grid_sampler2d(hs[0], hs[1], interp, pad, align, hs[2])
                 assert st == 0 and aclnn.executor_variant(ex) == "box_lds", (N, C, H, W, Ho, Wo)
                 aclnn.destroy_executor(ex)
                 for h in hs:
                     aclnn.destroy_tensor(h)
-                ref = oracle.grid_sampler2d(x, g, 0, pad, align, dtype=I.oracle_code(dtype))
-                y = aclnn.grid_sampler2d(tx, tg, 0, pad, align)
+                ref = oracle.grid_sampler2d(x, g, interp, pad, align, dtype=I.oracle_code(dtype))
+                y = aclnn.grid_sampler2d(tx, tg, interp, pad, align)
                 torch.cuda.synchronize()
                 got = I.from_torch(y, dtype)
                 rn = np.isnan(I.as_f32(ref, dtype))
-                assert np.array_equal(np.isnan(I.as_f32(got, dtype)), rn), (kind, N, C, H, W, pad, align)
+                assert np.array_equal(np.isnan(I.as_f32(got, dtype)), rn), (kind, interp, N, C, H, W, pad, align)
                 assert np.array_equal(np.where(rn, 0, _bits(got, dtype)), np.where(rn, 0, _bits(ref, dtype))), \
-                    (kind, N, C, H, W, Ho, Wo, pad, align)
+                    (kind, interp, N, C, H, W, Ho, Wo, pad, align)
     # shapes the variant leaves to the direct kernel: rows of odd length, rows that are not whole 16-byte units
     for (H, W, Ho, Wo) in [(208, 200, 64, 65), (208, 204, 64, 64)]:
         tx = I.to_torch(I.cast_np(rng.standard_normal((1, 2, H, W)).astype(np.float32), dtype), dtype, device)
         tg = I.to_torch(I.cast_np(I.affine_grid(rng, 1, Ho, Wo), dtype), dtype, device)
         ty = torch.empty((1, 2, Ho, Wo), dtype=tx.dtype, device=device)
         hs = [aclnn.tensor_handle(t) for t in (tx, tg, ty)]
-        st, _, ex = aclnn.get_workspace_size_grid_sampler2d(hs[0], hs[1], 0, 0, False, hs[2])
+        st, _, ex = aclnn.get_workspace_size_grid_sampler2d(hs[0], hs[1], interp, 0, False, hs[2])
         assert st == 0 and aclnn.executor_variant(ex) == "direct", (H, W, Ho, Wo)
         aclnn.destroy_executor(ex)
         for h in hs:

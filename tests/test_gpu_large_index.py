@@ -56,8 +56,8 @@ def test_grid_sampler_beyond_2_31_elements(oracle, device, aclnn, case):
         N, C, H, W, Ho, Wo, interp, pad, align = 2, 140000, 128, 64, 128, 64, 0, 0, False
     elif case == "lds_pair":    # output beyond 2^31 elements through the pair-layout kernel
         N, C, H, W, Ho, Wo, interp, pad, align = 1, 40000, 64, 32, 240, 240, 0, 1, True
-    elif case == "direct":      # planes far beyond LDS: the direct kernel (nearest samples; bicubic and fp32 too)
-        N, C, H, W, Ho, Wo, interp, pad, align = 1, 2100, 1024, 1024, 1024, 1024, 1, 2, False
+    elif case == "direct":      # planes far beyond LDS: the direct kernel (output rows of odd length; fp32 too)
+        N, C, H, W, Ho, Wo, interp, pad, align = 1, 2100, 1024, 1024, 1023, 1025, 1, 2, False  # rows of odd length
     elif case.startswith("box_lds"):  # planes far beyond LDS, bilinear: a tile's box of the input through LDS
         N, C, H, W, Ho, Wo, interp, pad, align = 1, 2100, 1024, 1024, 1024, 1024, 0, 2, False
     else:                       # channels-last views of NHWC memory

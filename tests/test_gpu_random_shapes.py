@@ -122,10 +122,10 @@ def test_random_grid_sampler2d_box_variant(oracle, device, aclnn):
         W = 8 * int(rng.integers((41000 // H) // 8 + 1, 60))  # rows of whole 16-byte units, planes above 80 KB
         Ho = int(rng.integers(32, 200))
         Wo = 2 * int(rng.integers(32, 120))
-        pad, align = int(rng.integers(0, 3)), bool(rng.integers(0, 2))
+        interp, pad, align = int(rng.integers(0, 3)), int(rng.integers(0, 3)), bool(rng.integers(0, 2))
         deg = float(rng.choice([5.0, 30.0, 90.0]))
         lo = float(rng.choice([0.3, 0.8, 1.0]))
-        _say("gs2d box", dtype, N, C, H, W, Ho, Wo, pad, align, deg, lo)
+        _say("gs2d box", dtype, N, C, H, W, Ho, Wo, interp, pad, align, deg, lo)
         x = I.cast_np(rng.standard_normal((N, C, H, W)).astype(np.float32), dtype)
         g32 = I.affine_grid(rng, N, Ho, Wo, max_deg=deg, scale=(lo, lo * 1.5), shift=0.3)
         if case % 3 == 1:
@@ -134,15 +134,15 @@ def test_random_grid_sampler2d_box_variant(oracle, device, aclnn):
         tx, tg = I.to_torch(x, dtype, device), I.to_torch(g, dtype, device)
         ty = torch.empty((N, C, Ho, Wo), dtype=tx.dtype, device=device)
         hs = [aclnn.tensor_handle(t) for t in (tx, tg, ty)]
-        st, _, ex = aclnn.get_workspace_size_grid_sampler2d(hs[0], hs[1], 0, pad, align, hs[2])
+        st, _, ex = aclnn.get_workspace_size_grid_sampler2d(hs[0], hs[1], interp, pad, align, hs[2])
         assert st == 0 and aclnn.executor_variant(ex) == "box_lds", (H, W, Ho, Wo)
         aclnn.destroy_executor(ex)
         for h in hs:
             aclnn.destroy_tensor(h)
-        ref = oracle.grid_sampler2d(x, g, 0, pad, align, dtype=I.oracle_code(dtype))
-        y = aclnn.grid_sampler2d(tx, tg, 0, pad, align)
+        ref = oracle.grid_sampler2d(x, g, interp, pad, align, dtype=I.oracle_code(dtype))
+        y = aclnn.grid_sampler2d(tx, tg, interp, pad, align)
         torch.cuda.synchronize()
-        _same(I.from_torch(y, dtype), ref, dtype, (case, dtype, N, C, H, W, Ho, Wo, pad, align, deg, lo))
+        _same(I.from_torch(y, dtype), ref, dtype, (case, dtype, N, C, H, W, Ho, Wo, interp, pad, align, deg, lo))
 
 
 def test_random_resize_family(oracle, device, aclnn, monkeypatch):
