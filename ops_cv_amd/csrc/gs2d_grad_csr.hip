@@ -31,6 +31,8 @@
 // The result is the same sequence of rounded operations per element as the scatter in gs2d_grad.hip, bit for bit.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include <rocprim/block/block_radix_sort.hpp>
 
 #include "gs2d_grad_math.hpp"
@@ -294,41 +296,60 @@ __global__ __launch_bounds__(kListThreads) void gs2d_grad_csr_lists_kernel(uint3
         }
     };
     if (!crowded) {
-        // all candidates at once (independent loads), keyed (chunk, corner, point), sorted by a bitonic network
-        uint32_t key[4 * kRun];
+        // all candidates at once (independent loads), keyed (chunk, corner, point), sorted by a bitonic network.  The
+        // network takes R candidates from each of the four cells; R is the smallest of 2, 4 and 8 that covers the
+        // fullest cell of any lane of the wavefront (a cell of a smooth grid holds a point or two: 8 loads and a
+        // network of 8 keys instead of 32 and 32).
+        auto sort_and_put = [&](auto r_tag) {
+            constexpr int R = decltype(r_tag)::value;
+            uint32_t key[4 * R];
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const uint32_t len = end[k] - cur[k];
+            for (int k = 0; k < 4; k++) {
+                const uint32_t len = end[k] - cur[k];
 #pragma unroll
-            for (int i = 0; i < kRun; i++) {
-                const bool valid = (uint32_t)i < len;
-                const uint32_t pt = source[valid ? cur[k] + (uint32_t)i : 0u] & kPointMask;
-                key[k * kRun + i] =
-                    valid ? (((pt >> kChunkShift) << (kPointBits + 2)) | ((uint32_t)k << kPointBits) | pt) : 0xFFFFFFFFu;
+                for (int i = 0; i < R; i++) {
+                    const bool valid = (uint32_t)i < len;
+                    const uint32_t pt = source[valid ? cur[k] + (uint32_t)i : 0u] & kPointMask;
+                    key[k * R + i] = valid ? (((pt >> kChunkShift) << (kPointBits + 2)) | ((uint32_t)k << kPointBits) | pt)
+                                           : 0xFFFFFFFFu;
+                }
             }
-        }
 #pragma unroll
-        for (int size = 2; size <= 4 * kRun; size *= 2) {
+            for (int size = 2; size <= 4 * R; size *= 2) {
 #pragma unroll
-            for (int stride = size / 2; stride > 0; stride /= 2) {
+                for (int stride = size / 2; stride > 0; stride /= 2) {
 #pragma unroll
-                for (int i = 0; i < 4 * kRun; i++) {
-                    const int l = i ^ stride;
-                    if (l > i) {
-                        const uint32_t lo = key[i] < key[l] ? key[i] : key[l];
-                        const uint32_t hi = key[i] < key[l] ? key[l] : key[i];
-                        const bool ascending = (i & size) == 0;
-                        key[i] = ascending ? lo : hi;
-                        key[l] = ascending ? hi : lo;
+                    for (int i = 0; i < 4 * R; i++) {
+                        const int l = i ^ stride;
+                        if (l > i) {
+                            const uint32_t lo = key[i] < key[l] ? key[i] : key[l];
+                            const uint32_t hi = key[i] < key[l] ? key[l] : key[i];
+                            const bool ascending = (i & size) == 0;
+                            key[i] = ascending ? lo : hi;
+                            key[l] = ascending ? hi : lo;
+                        }
                     }
                 }
             }
-        }
 #pragma unroll
-        for (int i = 0; i < 4 * kRun; i++) {
-            if ((uint32_t)i < cnt) {
-                put((uint32_t)i, key[i] & kPointMask, (key[i] >> kPointBits) & 3u);
+            for (int i = 0; i < 4 * R; i++) {
+                if ((uint32_t)i < cnt) {
+                    put((uint32_t)i, key[i] & kPointMask, (key[i] >> kPointBits) & 3u);
+                }
             }
+        };
+        uint32_t fullest = 0;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            fullest = (end[k] - cur[k] > fullest) ? end[k] - cur[k] : fullest;
+        }
+        static_assert(kRun == 8, "the three sizes below end at a cell's eight slots");
+        if (__builtin_amdgcn_ballot_w64(fullest > 4u) != 0) {
+            sort_and_put(std::integral_constant<int, 8>{});
+        } else if (__builtin_amdgcn_ballot_w64(fullest > 2u) != 0) {
+            sort_and_put(std::integral_constant<int, 4>{});
+        } else {
+            sort_and_put(std::integral_constant<int, 2>{});
         }
         return;
     }
