@@ -1,9 +1,29 @@
 // Grid sampler 2-D forward, LDS-staged variant: plan selection (device code in gs2d_lds_kernel.hpp).
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include "gs2d_lds_launch.hpp"
 
 namespace opscv {
+
+// CUs of the current device (256 on MI355X; also the answer where no device can be asked, as in host-only planning).
+static int compute_unit_count()
+{
+    static std::atomic<int> cached{0};
+    int v = cached.load(std::memory_order_relaxed);
+    if (v == 0) {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
+            (void)hipGetLastError();
+            cus = 256;
+        }
+        v = cus;
+        cached.store(v, std::memory_order_relaxed);
+    }
+    return v;
+}
 
 LdsPlan make_lds_plan(const GridSamplerArgs& a)
 {
@@ -70,6 +90,23 @@ LdsPlan make_lds_plan(const GridSamplerArgs& a)
     p.cblocks = (uint32_t)cblocks;
     if (a.N * p.tiles_per_n * cblocks > INT32_MAX) {
         return p;
+    }
+    // Exactly two workgroups per CU: the one that reaches a CU first keeps ahead of the one that joins it for the
+    // whole kernel (its wavefronts are the older ones wherever the CU arbitrates) and ends about five stages earlier,
+    // after which the CU runs half empty.  The launch hands out workgroups in index order and channel blocks are
+    // numbered with the index (gs2d_lds_kernel.hpp), so the lower half of the channel blocks are those first
+    // workgroups: they take 5 channels for every 3 of the upper half (fp16 N16 C256 64x64: 13.9 us with 16 + 16,
+    // 13.3 with 19 + 13, 12.9 with 20 + 12; the measured stage rates while both run are 2.2 and 1.45 per microsecond).
+    // A wrong guess about who comes first costs balance, never correctness.
+    if (cgs == 1 && cblocks % 2 == 0 && cpb >= 8 && a.C == cblocks * cpb &&
+        a.N * p.tiles_per_n * cblocks == 2 * (int64_t)compute_unit_count() && (a.N * cblocks / 2) % 8 == 0) {
+        const int64_t wide = (cpb * 5 + 2) / 4;
+        const int64_t narrow = 2 * cpb - wide;
+        if (narrow >= 1) {
+            p.wide_blocks = (uint32_t)(cblocks / 2);
+            p.chans_wide = (int32_t)wide;
+            p.chans_per_block = (int32_t)narrow;
+        }
     }
     p.copy_gran = plain ? 16 : 2;  // 2: 16-byte units in the shifted layout
     // Bank-spreading layout (gs2d_lds_kernel.hpp): rows of exactly 128 bytes, 16-byte copy granule.  Only for

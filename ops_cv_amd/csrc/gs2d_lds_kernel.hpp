@@ -13,7 +13,8 @@
 //   * a tap outside the image points at a 16-byte slot of zeros behind each staged plane, which reproduces the
 //     reference's "skip the tap" exactly (0 * w adds nothing) without per-channel selects;
 //   * every output channel plane is written once, 64 consecutive pixels per wavefront store, through a buffer
-//     descriptor whose range check drops the lanes of a partial last tile.
+//     descriptor whose range check drops the lanes of a partial last tile.  The stores (and the loads of the grid
+//     points) carry the non-temporal hint; the plane copies do not.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -36,7 +37,22 @@ constexpr uint32_t kBufferFlags = 0x00020000u;  // raw buffer, 32-bit data forma
 // The grid points (x, y interleaved, element type T) of COUNT pixels starting at `gp`, `stride` pixels apart, as raw
 // bits.  The loads carry no condition and no use between them, so they are in flight together: one memory latency
 // for all pixels of a lane (written per pixel with the alignment test inside, every load was followed by a wait).
-template <typename T, int COUNT>
+//
+// STREAM: the loads carry the non-temporal hint.  A kernel whose results leave through non-temporal stores must load
+// its grid points the same way: on this part ordinary loads issued by the same kernel take the advantage of the
+// streaming stores away again (fp16 N16 C256 64x64: 16.0 us with ordinary loads and stores, 17.3 us with ordinary
+// loads and streaming stores, 14.3 us with both streaming).
+template <typename V, bool STREAM>
+__device__ __forceinline__ V load_maybe_streaming(const V* p)
+{
+    if constexpr (STREAM) {
+        return __builtin_nontemporal_load(p);
+    } else {
+        return *p;
+    }
+}
+
+template <typename T, int COUNT, bool STREAM = false>
 __device__ __forceinline__ void load_grid_points(const T* const* gp, bool pair_aligned, float* gx, float* gy)
 {
     if constexpr (sizeof(T) == 2) {
@@ -44,7 +60,7 @@ __device__ __forceinline__ void load_grid_points(const T* const* gp, bool pair_a
             uint32_t raw[COUNT];
 #pragma unroll
             for (int j = 0; j < COUNT; j++) {
-                raw[j] = *reinterpret_cast<const uint32_t*>(gp[j]);
+                raw[j] = load_maybe_streaming<uint32_t, STREAM>(reinterpret_cast<const uint32_t*>(gp[j]));
             }
 #pragma unroll
             for (int j = 0; j < COUNT; j++) {
@@ -57,10 +73,11 @@ __device__ __forceinline__ void load_grid_points(const T* const* gp, bool pair_a
         }
     } else {
         if (pair_aligned) {
-            float2 raw[COUNT];
+            typedef float float_pair_t __attribute__((ext_vector_type(2)));
+            float_pair_t raw[COUNT];
 #pragma unroll
             for (int j = 0; j < COUNT; j++) {
-                raw[j] = *reinterpret_cast<const float2*>(gp[j]);
+                raw[j] = load_maybe_streaming<float_pair_t, STREAM>(reinterpret_cast<const float_pair_t*>(gp[j]));
             }
 #pragma unroll
             for (int j = 0; j < COUNT; j++) {
@@ -70,16 +87,18 @@ __device__ __forceinline__ void load_grid_points(const T* const* gp, bool pair_a
             return;
         }
     }
-    T ex[COUNT], ey[COUNT];
+    typedef typename std::conditional<sizeof(T) == 2, uint16_t, uint32_t>::type bits_t;
+    bits_t ex[COUNT], ey[COUNT];
 #pragma unroll
     for (int j = 0; j < COUNT; j++) {
-        ex[j] = gp[j][0];
-        ey[j] = gp[j][1];
+        ex[j] = load_maybe_streaming<bits_t, STREAM>(reinterpret_cast<const bits_t*>(gp[j]));
+        ey[j] = load_maybe_streaming<bits_t, STREAM>(reinterpret_cast<const bits_t*>(gp[j]) + 1);
     }
 #pragma unroll
     for (int j = 0; j < COUNT; j++) {
-        gx[j] = ElemIO<T>::load(&ex[j]);
-        gy[j] = ElemIO<T>::load(&ey[j]);
+        const T tx = __builtin_bit_cast(T, ex[j]), ty = __builtin_bit_cast(T, ey[j]);
+        gx[j] = ElemIO<T>::load(&tx);
+        gy[j] = ElemIO<T>::load(&ty);
     }
 }
 
@@ -166,26 +185,32 @@ __device__ __forceinline__ float blend(const R* raw, const float* tw, float neg_
     return tap_value_of<T>(raw[0]);
 }
 
-template <typename T>
+// cache-policy operand of the buffer stores: 0 = ordinary, 2 = non-temporal (streaming: the line is written through
+// and not kept, so the end of the kernel has no dirty lines to write back)
+constexpr int kStoreOrdinary = 0;
+constexpr int kStoreStreaming = 2;
+
+template <typename T, bool STREAM = false>
 __device__ __forceinline__ void buffer_store_elem(float v, __amdgpu_buffer_rsrc_t rsrc, uint32_t byte_off)
 {
+    constexpr int AUX = STREAM ? kStoreStreaming : kStoreOrdinary;
     if constexpr (sizeof(T) == 4) {
-        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), rsrc, (int)byte_off, 0, 0);
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), rsrc, (int)byte_off, 0, AUX);
     } else {
         T h;
         ElemIO<T>::store(&h, v);
-        __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(uint16_t, h), rsrc, (int)byte_off, 0, 0);
+        __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(uint16_t, h), rsrc, (int)byte_off, 0, AUX);
     }
 }
 
 // The results of ADJ neighbouring output pixels of one channel leave as one store: two 16-bit results as one dword
 // (each rounded to T on its own, exactly as the single store does), so a wavefront writes 256 contiguous bytes per
 // instruction instead of 128.  The caller guarantees a 4-byte aligned address (even pixel index, even plane size).
-template <typename T, int ADJ>
+template <typename T, int ADJ, bool STREAM = false>
 __device__ __forceinline__ void buffer_store_group(const float* v, __amdgpu_buffer_rsrc_t rsrc, uint32_t byte_off)
 {
     if constexpr (ADJ == 1) {
-        buffer_store_elem<T>(v[0], rsrc, byte_off);
+        buffer_store_elem<T, STREAM>(v[0], rsrc, byte_off);
     } else {
         static_assert(ADJ == 2 && sizeof(T) == 2, "pairs of 16-bit results only");
         // one packed conversion instruction, each half rounded to nearest even like the single conversion
@@ -193,7 +218,8 @@ __device__ __forceinline__ void buffer_store_group(const float* v, __amdgpu_buff
         typedef T elem_pair_t __attribute__((ext_vector_type(2)));
         const float_pair_t f = {v[0], v[1]};
         const elem_pair_t e = __builtin_convertvector(f, elem_pair_t);
-        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, e), rsrc, (int)byte_off, 0, 0);
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, e), rsrc, (int)byte_off, 0,
+                                              STREAM ? kStoreStreaming : kStoreOrdinary);
     }
 }
 
@@ -254,6 +280,33 @@ __device__ __forceinline__ void lds_barrier()
 // plane onto itself.  The copy applies it to the source address (the LDS side of the asynchronous copy is fixed per
 // lane); a copy instruction covers eight whole rows starting at a multiple of 1 KiB, so the permuted source offset
 // of a lane inside that block is a per-lane constant.  The samplers apply it once per tap when they compute offsets.
+// Division of a block index by a launch constant without the hardware's reciprocal sequence (a dependent chain of
+// conversions and a reciprocal that every wavefront of the kernel would walk before it knows its work): the host hands
+// over m = ceil(2^s / d), s = 31 + ceil(log2 d), and floor(x / d) = (x * m) >> s for every x < 2^31.
+struct FastDiv {
+    uint32_t mul = 0x80000000u;
+    uint32_t shift = 31;
+    uint32_t div = 1;
+};
+
+inline FastDiv make_fast_div(uint32_t d)
+{
+    FastDiv f;
+    uint32_t l = 0;
+    while ((1ull << l) < d) {
+        l++;
+    }
+    f.shift = 31 + l;
+    f.mul = (uint32_t)(((1ull << f.shift) + d - 1) / d);
+    f.div = d;
+    return f;
+}
+
+__device__ __forceinline__ uint32_t fast_div(uint32_t x, const FastDiv& f)
+{
+    return (uint32_t)(((uint64_t)x * f.mul) >> f.shift);
+}
+
 __device__ __forceinline__ uint32_t lds_swizzle(uint32_t byte_off, uint32_t row_shift)
 {
     return row_shift ? (byte_off ^ (((byte_off >> row_shift) & 7u) << 4)) : byte_off;
@@ -289,17 +342,28 @@ __device__ __forceinline__ void issue_stage_copy(const char* src, char* dst, uin
                 sp -= shift;
                 copy_bytes = (shift + plane_bytes + 15u) & ~15u;
             }
-            for (uint32_t base = lwave * CHUNK; base < copy_bytes; base += LWAVES * CHUNK) {
-                if (base + lane_off < copy_bytes) {
-                    // lane_src_off: the chunk of this 1 KiB block that belongs at the lane's LDS position
-                    const global_cptr_t gsrc = (global_cptr_t)(sp + base + lane_src_off);
-                    const lds_ptr_t ldst = (lds_ptr_t)(dp + base);
-                    // the size operand must be a literal
-                    if constexpr (G == 16) {
-                        __builtin_amdgcn_global_load_lds(gsrc, ldst, 16, 0, 0);
-                    } else {
-                        __builtin_amdgcn_global_load_lds(gsrc, ldst, 4, 0, 0);
-                    }
+            // whole chunks first, without a per-lane test (no exec-mask bookkeeping between the copy instructions:
+            // 13.2 -> 12.9 us on fp16 N16 C256 64x64), then the one partial chunk if this wavefront is its owner
+            const uint32_t whole_bytes = copy_bytes - copy_bytes % CHUNK;
+            uint32_t base = lwave * CHUNK;
+            for (; base < whole_bytes; base += LWAVES * CHUNK) {
+                // lane_src_off: the chunk of this 1 KiB block that belongs at the lane's LDS position
+                const global_cptr_t gsrc = (global_cptr_t)(sp + base + lane_src_off);
+                const lds_ptr_t ldst = (lds_ptr_t)(dp + base);
+                // the size operand must be a literal
+                if constexpr (G == 16) {
+                    __builtin_amdgcn_global_load_lds(gsrc, ldst, 16, 0, 0);
+                } else {
+                    __builtin_amdgcn_global_load_lds(gsrc, ldst, 4, 0, 0);
+                }
+            }
+            if (base < copy_bytes && base + lane_off < copy_bytes) {
+                const global_cptr_t gsrc = (global_cptr_t)(sp + base + lane_src_off);
+                const lds_ptr_t ldst = (lds_ptr_t)(dp + base);
+                if constexpr (G == 16) {
+                    __builtin_amdgcn_global_load_lds(gsrc, ldst, 16, 0, 0);
+                } else {
+                    __builtin_amdgcn_global_load_lds(gsrc, ldst, 4, 0, 0);
                 }
             }
         }
@@ -323,9 +387,9 @@ __device__ __forceinline__ void issue_stage_copy(const char* src, char* dst, uin
 template <typename T, int INTERP, int PAD, bool ALIGN, int SWAVES, int LWAVES, int PPT, int ADJ, int CGS, int NBUF,
           int PITCH, bool SHIFTED_PLANES = false>
 __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves_per_eu(1, 5))) void gs2d_lds_kernel(
-    const T* __restrict__ x, const T* __restrict__ grid, T* __restrict__ y, int32_t C, int32_t H, int32_t W,
-    int32_t out_plane, uint32_t tiles_per_n, uint32_t cblocks, int32_t chans_per_block, int32_t copy_gran,
-    int32_t pair_aligned, int32_t xcd_swizzle, int32_t row_shift, float neg_zero)
+    const T* __restrict__ x, const T* __restrict__ grid, T* __restrict__ y, FastDiv N, int32_t C, int32_t H, int32_t W,
+    int32_t out_plane, FastDiv tiles_per_n, int32_t chans_per_block, uint32_t wide_blocks,
+    int32_t chans_wide, int32_t copy_gran, int32_t pair_aligned, int32_t xcd_swizzle, int32_t row_shift, float neg_zero)
 {
     extern __shared__ uint4 smem_raw[];
     char* lds = reinterpret_cast<char*>(smem_raw);
@@ -337,28 +401,37 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
     const int tid = threadIdx.x;
     const uint32_t wave = __builtin_amdgcn_readfirstlane((uint32_t)tid >> 6);
 
-    // Block -> (group = (n, channel block), tile).  Workgroups are handed to the 8 XCDs round-robin by index;
+    // Block -> (group = (channel block, n), tile).  Workgroups are handed to the 8 XCDs round-robin by index;
     // with the swizzle all tiles of one group (they read the same input planes) land on the same XCD next to
-    // each other in time, so the planes are fetched into one L2 once.
+    // each other in time, so the planes are fetched into one L2 once.  Groups are numbered with the batch item
+    // fastest: the workgroups that run at the same time then cover every batch item (with the channel block
+    // fastest, the first half of the launch worked on the first half of both tensors, the second half on the rest:
+    // 14.5 against 13.0 us on fp16 N16 C256 64x64), and an XCD sees the grids of N / 8 batch items only.
     uint32_t group, tile;
     if (xcd_swizzle) {
         const uint32_t xcd = blockIdx.x & 7u;
         const uint32_t i = blockIdx.x >> 3;
-        group = (i / tiles_per_n) * 8u + xcd;
-        tile = i % tiles_per_n;
+        const uint32_t k = fast_div(i, tiles_per_n);
+        group = k * 8u + xcd;
+        tile = i - k * tiles_per_n.div;
     } else {
-        group = blockIdx.x / tiles_per_n;
-        tile = blockIdx.x % tiles_per_n;
+        group = fast_div(blockIdx.x, tiles_per_n);
+        tile = blockIdx.x - group * tiles_per_n.div;
     }
-    const uint32_t cb = group % cblocks;
-    const uint32_t n = group / cblocks;
+    const uint32_t cb = fast_div(group, N);
+    const uint32_t n = group - cb * N.div;
 
     const int32_t plane_elems = H * W;
     const uint32_t plane_bytes = (uint32_t)plane_elems * (uint32_t)sizeof(T);
     // behind the plane, which in the shifted layout (copy_gran == 2) may sit up to 14 bytes into its slot
     const uint32_t zero_off = round_up16(plane_bytes + (SHIFTED_PLANES ? 14u : 0u));
-    const int32_t c_begin = (int32_t)cb * chans_per_block;
-    const int32_t c_end = (c_begin + chans_per_block < C) ? c_begin + chans_per_block : C;
+    // The first `wide_blocks` channel blocks take `chans_wide` channels each, the others `chans_per_block` (see
+    // make_lds_plan: the workgroup that reaches a CU first runs ahead of the one that shares the CU with it).
+    const bool wide = cb < wide_blocks;
+    const int32_t my_chans = wide ? chans_wide : chans_per_block;
+    const int32_t c_begin = wide ? (int32_t)cb * chans_wide
+                                 : (int32_t)wide_blocks * chans_wide + (int32_t)(cb - wide_blocks) * chans_per_block;
+    const int32_t c_end = (c_begin + my_chans < C) ? c_begin + my_chans : C;
     const int32_t nchan = c_end - c_begin;
     const int32_t nstages = (nchan + CGS - 1) / CGS;
 
@@ -435,6 +508,10 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
                 issue_next();
             }
         }
+        // the samplers' barrier behind the last plane of a full last stage (see their loop)
+        if (nchan % CGS == 0) {
+            lds_barrier();
+        }
         return;
     }
 
@@ -468,7 +545,7 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
             gptr[q * ADJ + a] = gridn + (int64_t)(pc + a) * 2;
         }
     }
-    load_grid_points<T, PPT>(gptr, pair_aligned != 0, gxs, gys);
+    load_grid_points<T, PPT, true>(gptr, pair_aligned != 0, gxs, gys);
     // the bank-spreading layout exists for border padding only (see make_lds_plan)
     const uint32_t rs = (PAD == 1) ? (uint32_t)row_shift : 0u;
 #pragma unroll
@@ -595,6 +672,11 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
     for (int j = 0; j < PPT; j++) {
         load_taps<T, NT>(plane_shift(0), toff[j], raw[j]);
     }
+    // Every plane runs the same straight-line body, barrier included (behind the block's last plane the loaders add
+    // one more barrier to meet it).  With the barrier under a condition of its own ("is there a next plane") two
+    // paths met in front of the next blend, and the compiler, merging their counts of outstanding LDS reads, made
+    // every plane wait for all sixteen of its reads before the first product (14.0 against 12.9 us on fp16 N16 C256
+    // 64x64).
     for (int32_t b = 0; b < nchan; b += UNR) {
 #pragma unroll
         for (int u = 0; u < UNR; u++) {
@@ -613,15 +695,15 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
                 for (int a = 0; a < ADJ; a++) {
                     const int j = q * ADJ + a;
                     v[a] = blend<T, INTERP>(raw[j], tw[j], neg_zero);
-                    if (j == 0 && un % CGS == 0 && p + 1 < nchan) {
+                    if (j == 0 && un % CGS == 0) {
                         __builtin_amdgcn_s_waitcnt(0xC07F);
-                        lds_barrier();  // stage (p + 1) / CGS has landed
+                        lds_barrier();  // stage (p + 1) / CGS has landed (or, behind the last plane, nothing)
                     }
                     __builtin_amdgcn_sched_barrier(0);
                     load_taps<T, NT>(next_off, toff[j], raw[j]);
                     __builtin_amdgcn_sched_barrier(0);
                 }
-                buffer_store_group<T, ADJ>(v, rsrc, pixoff[q]);
+                buffer_store_group<T, ADJ, true>(v, rsrc, pixoff[q]);
             }
         }
     }

@@ -21,6 +21,9 @@ struct LdsPlan {
     uint32_t lds_bytes = 0;
     uint32_t tiles_per_n = 0, cblocks = 0;
     int32_t chans_per_block = 0;
+    // the first `wide_blocks` channel blocks take `chans_wide` channels each (0: all blocks alike)
+    uint32_t wide_blocks = 0;
+    int32_t chans_wide = 0;
 };
 
 constexpr int kSamplerWaves = 8;  // 512 lanes own output pixels
@@ -52,9 +55,9 @@ hipError_t launch_one(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t st
     const int pair_aligned = (reinterpret_cast<uintptr_t>(a.grid) % (2 * esz) == 0);
     const uint32_t blocks = (uint32_t)(a.N * p.tiles_per_n * p.cblocks);
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3((kSamplerWaves + LWAVES) * 64), p.lds_bytes, stream, (const T*)a.x, (const T*)a.grid,
-                       (T*)a.y, (int32_t)a.C, (int32_t)a.Hin, (int32_t)a.Win, (int32_t)(a.Hout * a.Wout),
-                       p.tiles_per_n, p.cblocks, p.chans_per_block, p.copy_gran, pair_aligned, p.xcd_swizzle, p.row_shift,
-                       -0.0f);
+                       (T*)a.y, make_fast_div((uint32_t)a.N), (int32_t)a.C, (int32_t)a.Hin, (int32_t)a.Win, (int32_t)(a.Hout * a.Wout),
+                       make_fast_div(p.tiles_per_n), p.chans_per_block, p.wide_blocks, p.chans_wide, p.copy_gran,
+                       pair_aligned, p.xcd_swizzle, p.row_shift, -0.0f);
     return hipGetLastError();
 }
 
