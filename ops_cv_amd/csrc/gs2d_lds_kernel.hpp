@@ -370,6 +370,123 @@ __device__ __forceinline__ void issue_stage_copy(const char* src, char* dst, uin
     }
 }
 
+// The per-pixel decisions of one lane: tap offsets (LDS byte offsets inside a staged plane, `zero_off` for a tap outside
+// the image) and weights for its PPT pixels.  Padding mode and align_corners are run-time, wave-uniform values
+// (kernel arguments; scalar branches around the clip and reflect steps): the decisions run once per workgroup,
+// outside the channel loop, so one kernel serves all six combinations at no cost to the loop.
+// SWIZZLED: the staged planes use the bank-spreading layout (`rs` = its row shift); without it `rs` is not looked at,
+// so the plain layout pays nothing per tap.
+// Source coordinates of COUNT grid points for one (padding mode, align_corners) pair, and the one wave-uniform switch
+// that picks the pair.  All coordinates of a lane are computed inside one branch, so the chains of the lane's pixels
+// interleave as they do with the modes fixed at compile time (a branch per coordinate cost 0.3 us on fp16 N16 C256
+// 64x64: each chain then waited out its own latencies).
+template <int PAD, bool ALIGN, int COUNT>
+__device__ __forceinline__ void source_indices(const float* gxs, const float* gys, int32_t H, int32_t W, float* ixs,
+                                               float* iys)
+{
+#pragma unroll
+    for (int j = 0; j < COUNT; j++) {
+        ixs[j] = compute_source_index<PAD, ALIGN>(gxs[j], W);
+        iys[j] = compute_source_index<PAD, ALIGN>(gys[j], H);
+    }
+}
+
+template <int COUNT>
+__device__ __forceinline__ void source_indices_rt(const float* gxs, const float* gys, int32_t H, int32_t W, int32_t pad,
+                                                  bool align, float* ixs, float* iys)
+{
+    switch (pad * 2 + (align ? 1 : 0)) {
+        case 0: source_indices<0, false, COUNT>(gxs, gys, H, W, ixs, iys); break;
+        case 1: source_indices<0, true, COUNT>(gxs, gys, H, W, ixs, iys); break;
+        case 2: source_indices<1, false, COUNT>(gxs, gys, H, W, ixs, iys); break;
+        case 3: source_indices<1, true, COUNT>(gxs, gys, H, W, ixs, iys); break;
+        case 4: source_indices<2, false, COUNT>(gxs, gys, H, W, ixs, iys); break;
+        default: source_indices<2, true, COUNT>(gxs, gys, H, W, ixs, iys); break;
+    }
+}
+
+template <typename T, int INTERP, int PPT, int NT, int NW, bool SWIZZLED>
+__device__ __forceinline__ void decide_lane_pixels(const float* gxs, const float* gys, int32_t H, int32_t W,
+                                                   uint32_t row_shift, uint32_t zero_off, int32_t pad, bool align,
+                                                   uint32_t (*toff)[NT], float (*tw)[NW])
+{
+    const uint32_t rs = SWIZZLED ? row_shift : 0u;
+    float ixs[PPT], iys[PPT];
+    if constexpr (INTERP != 2) {
+        source_indices_rt<PPT>(gxs, gys, H, W, pad, align, ixs, iys);
+    }
+#pragma unroll
+    for (int j = 0; j < PPT; j++) {
+        if constexpr (INTERP == 2) {
+            const BicubicTap b = decide_bicubic_rt(gxs[j], gys[j], H, W, pad, align);
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const bool row_in = b.by[r] >= 0 && b.by[r] < H && !b.flag;
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    const bool in = row_in && b.bx[k] >= 0 && b.bx[k] < W;
+                    toff[j][4 * r + k] =
+                        in ? lds_swizzle(((uint32_t)b.by[r] * (uint32_t)W + (uint32_t)b.bx[k]) * (uint32_t)sizeof(T), rs)
+                           : zero_off;
+                }
+                tw[j][r] = b.cx[r];
+                tw[j][4 + r] = b.cy[r];
+            }
+            if (b.flag) {
+                tw[j][0] = __builtin_nanf("");  // 0 * NaN: every channel becomes NaN, as the reference writes
+            }
+            continue;
+        }
+        // Bilinear and nearest: the decisions of decide_pixel() (sampler_math.hpp; grid_sampler2_d_simt.h:479-498,
+        // 307-316, 341-349) written without branches -- this prologue runs once per workgroup for every one of its
+        // pixels and is on the critical path to the first sampled stage, so its instruction count matters.
+        // Bounds tests are single unsigned compares (a negative index is a huge unsigned one), tap offsets follow
+        // from the north-west one by modular arithmetic, and the "+1" of an index saturated at INT32_MAX wraps to
+        // 0x80000000, which is out of bounds like the saturated value itself.
+        float ix = ixs[j];
+        float iy = iys[j];
+        const bool finite = __builtin_fabsf(ix) < __builtin_inff() && __builtin_fabsf(iy) < __builtin_inff();
+        const bool x_far = ix > 2147483646.0f || ix < -2147483648.0f;  // safe_downgrade: -> -100, always outside
+        const bool y_far = iy > 2147483646.0f || iy < -2147483648.0f;
+        const uint32_t uw = (uint32_t)W, uh = (uint32_t)H, es = (uint32_t)sizeof(T);
+        if (INTERP == 0) {
+            ix = x_far ? -100.0f : ix;
+            iy = y_far ? -100.0f : iy;
+            const float ixf = __builtin_floorf(ix), iyf = __builtin_floorf(iy);
+            const uint32_t x0 = (uint32_t)float_to_i32(ixf), y0 = (uint32_t)float_to_i32(iyf);
+            const uint32_t x1 = x0 + 1u, y1 = y0 + 1u;
+            const bool in_x0 = x0 < uw && finite, in_x1 = x1 < uw && finite;
+            const bool in_y0 = y0 < uh, in_y1 = y1 < uh;
+            const uint32_t o_nw = (y0 * uw + x0) * es;
+            const uint32_t o_sw = o_nw + uw * es;
+            toff[j][0] = (in_y0 && in_x0) ? lds_swizzle(o_nw, rs) : zero_off;
+            toff[j][1] = (in_y0 && in_x1) ? lds_swizzle(o_nw + es, rs) : zero_off;
+            toff[j][2] = (in_y1 && in_x0) ? lds_swizzle(o_sw, rs) : zero_off;
+            toff[j][3] = (in_y1 && in_x1) ? lds_swizzle(o_sw + es, rs) : zero_off;
+            const float wx1 = ix - ixf, wx0 = ixf + 1.0f - ix;
+            const float wy1 = iy - iyf, wy0 = iyf + 1.0f - iy;
+            // non-finite source coordinate: every tap reads the zero slot and 0 * NaN makes every channel NaN,
+            // as the reference writes (grid_sampler2_d_simt.h:485-487)
+            tw[j][0] = finite ? wx0 * wy0 : __builtin_nanf("");
+            tw[j][1] = wx1 * wy0;
+            tw[j][2] = wx0 * wy1;
+            tw[j][3] = wx1 * wy1;
+        } else {
+            ix = (x_far || !finite) ? -100.0f : ix;
+            iy = (y_far || !finite) ? -100.0f : iy;
+            // round half to even from floor, fraction and parity (grid_sampler2_d_simt.h:219-234)
+            const float xf = __builtin_floorf(ix), yf = __builtin_floorf(iy);
+            const float fx = ix - xf, fy = iy - yf;
+            const uint32_t xi = (uint32_t)float_to_i32(xf), yi = (uint32_t)float_to_i32(yf);
+            const uint32_t xr = xi + ((fx > 0.5f || (fx == 0.5f && (xi & 1u))) ? 1u : 0u);
+            const uint32_t yr = yi + ((fy > 0.5f || (fy == 0.5f && (yi & 1u))) ? 1u : 0u);
+            const bool in = xr < uw && yr < uh;
+            toff[j][0] = in ? lds_swizzle((yr * uw + xr) * es, rs) : zero_off;
+            tw[j][0] = tw[j][1] = tw[j][2] = tw[j][3] = 0.0f;
+        }
+    }
+}
+
 // LDS layout: a ring of NBUF stage slots, each CGS planes at PITCH bytes (PITCH >= padded plane size + 16,
 // compile-time so that a tap address is "register + immediate").  Stage s lives in slot s % NBUF and up to
 // NBUF-1 later stages are in flight while it is sampled.
@@ -384,12 +501,13 @@ __device__ __forceinline__ void issue_stage_copy(const char* src, char* dst, uin
 //
 // SHIFTED_PLANES selects the layout for planes off the 16-byte grid (issue_stage_copy); it is a template parameter so
 // that the kernels for whole, aligned planes carry no trace of it.
-template <typename T, int INTERP, int PAD, bool ALIGN, int SWAVES, int LWAVES, int PPT, int ADJ, int CGS, int NBUF,
-          int PITCH, bool SHIFTED_PLANES = false>
+template <typename T, int INTERP, int SWAVES, int LWAVES, int PPT, int ADJ, int CGS, int NBUF, int PITCH,
+          bool SHIFTED_PLANES = false>
 __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves_per_eu(1, 5))) void gs2d_lds_kernel(
     const T* __restrict__ x, const T* __restrict__ grid, T* __restrict__ y, FastDiv N, int32_t C, int32_t H, int32_t W,
     int32_t out_plane, FastDiv tiles_per_n, int32_t chans_per_block, uint32_t wide_blocks,
-    int32_t chans_wide, int32_t copy_gran, int32_t pair_aligned, int32_t xcd_swizzle, int32_t row_shift, float neg_zero)
+    int32_t chans_wide, int32_t copy_gran, int32_t pair_aligned, int32_t xcd_swizzle, int32_t row_shift, int32_t pad,
+    int32_t align, float neg_zero)
 {
     extern __shared__ uint4 smem_raw[];
     char* lds = reinterpret_cast<char*>(smem_raw);
@@ -463,7 +581,7 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
             }
             return total;
         };
-        const uint32_t lane_src16 = lds_swizzle(lane * 16u, (PAD == 1) ? (uint32_t)row_shift : 0u);
+        const uint32_t lane_src16 = lds_swizzle(lane * 16u, (uint32_t)row_shift);
         auto start_stage = [&](int32_t s, int slot) {
             const char* src = xb + (size_t)s * stage_bytes;
             char* dst = lds + slot * SLOT_BYTES;
@@ -546,78 +664,12 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
         }
     }
     load_grid_points<T, PPT, true>(gptr, pair_aligned != 0, gxs, gys);
-    // the bank-spreading layout exists for border padding only (see make_lds_plan)
-    const uint32_t rs = (PAD == 1) ? (uint32_t)row_shift : 0u;
-#pragma unroll
-    for (int j = 0; j < PPT; j++) {
-        const float gx = gxs[j], gy = gys[j];
-        if constexpr (INTERP == 2) {
-            const BicubicTap b = decide_bicubic<PAD, ALIGN>(gx, gy, H, W);
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const bool row_in = b.by[r] >= 0 && b.by[r] < H && !b.flag;
-#pragma unroll
-                for (int k = 0; k < 4; k++) {
-                    const bool in = row_in && b.bx[k] >= 0 && b.bx[k] < W;
-                    toff[j][4 * r + k] =
-                        in ? lds_swizzle(((uint32_t)b.by[r] * (uint32_t)W + (uint32_t)b.bx[k]) * (uint32_t)sizeof(T), rs)
-                           : zero_off;
-                }
-                tw[j][r] = b.cx[r];
-                tw[j][4 + r] = b.cy[r];
-            }
-            if (b.flag) {
-                tw[j][0] = __builtin_nanf("");  // 0 * NaN: every channel becomes NaN, as the reference writes
-            }
-            continue;
-        }
-        // Bilinear and nearest: the decisions of decide_pixel() (sampler_math.hpp; grid_sampler2_d_simt.h:479-498,
-        // 307-316, 341-349) written without branches -- this prologue runs once per workgroup for every one of its
-        // pixels and is on the critical path to the first sampled stage, so its instruction count matters.
-        // Bounds tests are single unsigned compares (a negative index is a huge unsigned one), tap offsets follow
-        // from the north-west one by modular arithmetic, and the "+1" of an index saturated at INT32_MAX wraps to
-        // 0x80000000, which is out of bounds like the saturated value itself.
-        float ix = compute_source_index<PAD, ALIGN>(gx, W);
-        float iy = compute_source_index<PAD, ALIGN>(gy, H);
-        const bool finite = __builtin_fabsf(ix) < __builtin_inff() && __builtin_fabsf(iy) < __builtin_inff();
-        const bool x_far = ix > 2147483646.0f || ix < -2147483648.0f;  // safe_downgrade: -> -100, always outside
-        const bool y_far = iy > 2147483646.0f || iy < -2147483648.0f;
-        const uint32_t uw = (uint32_t)W, uh = (uint32_t)H, es = (uint32_t)sizeof(T);
-        if (INTERP == 0) {
-            ix = x_far ? -100.0f : ix;
-            iy = y_far ? -100.0f : iy;
-            const float ixf = __builtin_floorf(ix), iyf = __builtin_floorf(iy);
-            const uint32_t x0 = (uint32_t)float_to_i32(ixf), y0 = (uint32_t)float_to_i32(iyf);
-            const uint32_t x1 = x0 + 1u, y1 = y0 + 1u;
-            const bool in_x0 = x0 < uw && finite, in_x1 = x1 < uw && finite;
-            const bool in_y0 = y0 < uh, in_y1 = y1 < uh;
-            const uint32_t o_nw = (y0 * uw + x0) * es;
-            const uint32_t o_sw = o_nw + uw * es;
-            toff[j][0] = (in_y0 && in_x0) ? lds_swizzle(o_nw, rs) : zero_off;
-            toff[j][1] = (in_y0 && in_x1) ? lds_swizzle(o_nw + es, rs) : zero_off;
-            toff[j][2] = (in_y1 && in_x0) ? lds_swizzle(o_sw, rs) : zero_off;
-            toff[j][3] = (in_y1 && in_x1) ? lds_swizzle(o_sw + es, rs) : zero_off;
-            const float wx1 = ix - ixf, wx0 = ixf + 1.0f - ix;
-            const float wy1 = iy - iyf, wy0 = iyf + 1.0f - iy;
-            // non-finite source coordinate: every tap reads the zero slot and 0 * NaN makes every channel NaN,
-            // as the reference writes (grid_sampler2_d_simt.h:485-487)
-            tw[j][0] = finite ? wx0 * wy0 : __builtin_nanf("");
-            tw[j][1] = wx1 * wy0;
-            tw[j][2] = wx0 * wy1;
-            tw[j][3] = wx1 * wy1;
-        } else {
-            ix = (x_far || !finite) ? -100.0f : ix;
-            iy = (y_far || !finite) ? -100.0f : iy;
-            // round half to even from floor, fraction and parity (grid_sampler2_d_simt.h:219-234)
-            const float xf = __builtin_floorf(ix), yf = __builtin_floorf(iy);
-            const float fx = ix - xf, fy = iy - yf;
-            const uint32_t xi = (uint32_t)float_to_i32(xf), yi = (uint32_t)float_to_i32(yf);
-            const uint32_t xr = xi + ((fx > 0.5f || (fx == 0.5f && (xi & 1u))) ? 1u : 0u);
-            const uint32_t yr = yi + ((fy > 0.5f || (fy == 0.5f && (yi & 1u))) ? 1u : 0u);
-            const bool in = xr < uw && yr < uh;
-            toff[j][0] = in ? lds_swizzle((yr * uw + xr) * es, rs) : zero_off;
-            tw[j][0] = tw[j][1] = tw[j][2] = tw[j][3] = 0.0f;
-        }
+    // the bank-spreading layout exists for border padding only (see make_lds_plan: row_shift is 0 otherwise)
+    const uint32_t rs = (uint32_t)row_shift;
+    if (rs != 0u) {
+        decide_lane_pixels<T, INTERP, PPT, NT, NW, true>(gxs, gys, H, W, rs, zero_off, pad, align != 0, toff, tw);
+    } else {
+        decide_lane_pixels<T, INTERP, PPT, NT, NW, false>(gxs, gys, H, W, rs, zero_off, pad, align != 0, toff, tw);
     }
 
     // tap offsets become absolute LDS addresses (left as offsets, the compiler re-adds the allocation's base to

@@ -42,10 +42,10 @@ constexpr int kNbuf[5] = {4, 6, 4, 4, 2};  // ring slots (stages resident in LDS
 
 LdsPlan make_lds_plan(const GridSamplerArgs& a);
 
-template <typename T, int I, int P, bool A, int PPT, int ADJ, int CGS, int NBUF, int PITCH, int LWAVES, bool SHIFTED>
+template <typename T, int I, int PPT, int ADJ, int CGS, int NBUF, int PITCH, int LWAVES, bool SHIFTED>
 hipError_t launch_one(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t stream)
 {
-    auto kernel = gs2d_lds_kernel<T, I, P, A, kSamplerWaves, LWAVES, PPT, ADJ, CGS, NBUF, PITCH, SHIFTED>;
+    auto kernel = gs2d_lds_kernel<T, I, kSamplerWaves, LWAVES, PPT, ADJ, CGS, NBUF, PITCH, SHIFTED>;
     static std::atomic<uint32_t> lds_allowed{0};
     const hipError_t ea = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kLdsLimit, lds_allowed);
     if (ea != hipSuccess) {
@@ -57,63 +57,63 @@ hipError_t launch_one(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t st
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3((kSamplerWaves + LWAVES) * 64), p.lds_bytes, stream, (const T*)a.x, (const T*)a.grid,
                        (T*)a.y, make_fast_div((uint32_t)a.N), (int32_t)a.C, (int32_t)a.Hin, (int32_t)a.Win, (int32_t)(a.Hout * a.Wout),
                        make_fast_div(p.tiles_per_n), p.chans_per_block, p.wide_blocks, p.chans_wide, p.copy_gran,
-                       pair_aligned, p.xcd_swizzle, p.row_shift, -0.0f);
+                       pair_aligned, p.xcd_swizzle, p.row_shift, (int32_t)a.pad, (int32_t)(a.align != 0), -0.0f);
     return hipGetLastError();
 }
 
-template <typename T, int I, int P, bool A, int CLS, int PPT, bool SHIFTED>
+template <typename T, int I, int CLS, int PPT, bool SHIFTED>
 hipError_t launch_cls(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t stream)
 {
     // pairs of neighbouring pixels per store exist for 16-bit elements with four or eight pixels per lane
     if constexpr (sizeof(T) == 2 && PPT >= 4) {
         if (p.adj == 2) {
-            return launch_one<T, I, P, A, PPT, 2, kCgs[CLS], kNbuf[CLS], kPitch[CLS], kLoaderWaves[CLS], SHIFTED>(a, p,
+            return launch_one<T, I, PPT, 2, kCgs[CLS], kNbuf[CLS], kPitch[CLS], kLoaderWaves[CLS], SHIFTED>(a, p,
                                                                                                                  stream);
         }
     }
-    return launch_one<T, I, P, A, PPT, 1, kCgs[CLS], kNbuf[CLS], kPitch[CLS], kLoaderWaves[CLS], SHIFTED>(a, p, stream);
+    return launch_one<T, I, PPT, 1, kCgs[CLS], kNbuf[CLS], kPitch[CLS], kLoaderWaves[CLS], SHIFTED>(a, p, stream);
 }
 
-// Expands (interp, pad, align, size class, pixels per lane) for one element type and launches.  Eight pixels per
-// lane exist for the two large-plane classes only.
+// Expands (interp, size class, pixels per lane) for one element type and launches; padding mode and align_corners are
+// run-time arguments of the kernel.  Eight pixels per lane exist for the two large-plane classes only.
 template <typename T, bool SHIFTED>
 struct LdsTypedLauncher {
     const GridSamplerArgs& a;
     const LdsPlan& p;
     hipStream_t stream;
-    template <typename U, int I, int P, bool A>
-    hipError_t operator()() const
+    template <int I>
+    hipError_t run() const
     {
         if constexpr (I == 2) {
             // bicubic keeps sixteen tap offsets per pixel: one or two pixels per lane
             switch (p.cls * 16 + p.ppt) {
-                case 0 * 16 + 1: return launch_cls<T, I, P, A, 0, 1, SHIFTED>(a, p, stream);
-                case 0 * 16 + 2: return launch_cls<T, I, P, A, 0, 2, SHIFTED>(a, p, stream);
-                case 1 * 16 + 1: return launch_cls<T, I, P, A, 1, 1, SHIFTED>(a, p, stream);
-                case 1 * 16 + 2: return launch_cls<T, I, P, A, 1, 2, SHIFTED>(a, p, stream);
-                case 2 * 16 + 1: return launch_cls<T, I, P, A, 2, 1, SHIFTED>(a, p, stream);
-                case 2 * 16 + 2: return launch_cls<T, I, P, A, 2, 2, SHIFTED>(a, p, stream);
-                case 3 * 16 + 1: return launch_cls<T, I, P, A, 3, 1, SHIFTED>(a, p, stream);
-                case 3 * 16 + 2: return launch_cls<T, I, P, A, 3, 2, SHIFTED>(a, p, stream);
-                case 4 * 16 + 1: return launch_cls<T, I, P, A, 4, 1, SHIFTED>(a, p, stream);
-                case 4 * 16 + 2: return launch_cls<T, I, P, A, 4, 2, SHIFTED>(a, p, stream);
+                case 0 * 16 + 1: return launch_cls<T, I, 0, 1, SHIFTED>(a, p, stream);
+                case 0 * 16 + 2: return launch_cls<T, I, 0, 2, SHIFTED>(a, p, stream);
+                case 1 * 16 + 1: return launch_cls<T, I, 1, 1, SHIFTED>(a, p, stream);
+                case 1 * 16 + 2: return launch_cls<T, I, 1, 2, SHIFTED>(a, p, stream);
+                case 2 * 16 + 1: return launch_cls<T, I, 2, 1, SHIFTED>(a, p, stream);
+                case 2 * 16 + 2: return launch_cls<T, I, 2, 2, SHIFTED>(a, p, stream);
+                case 3 * 16 + 1: return launch_cls<T, I, 3, 1, SHIFTED>(a, p, stream);
+                case 3 * 16 + 2: return launch_cls<T, I, 3, 2, SHIFTED>(a, p, stream);
+                case 4 * 16 + 1: return launch_cls<T, I, 4, 1, SHIFTED>(a, p, stream);
+                case 4 * 16 + 2: return launch_cls<T, I, 4, 2, SHIFTED>(a, p, stream);
                 default: return hipErrorInvalidValue;
             }
         }
         switch (p.cls * 16 + p.ppt) {
-            case 0 * 16 + 1: return launch_cls<T, I, P, A, 0, 1, SHIFTED>(a, p, stream);
-            case 0 * 16 + 4: return launch_cls<T, I, P, A, 0, 4, SHIFTED>(a, p, stream);
-            case 1 * 16 + 1: return launch_cls<T, I, P, A, 1, 1, SHIFTED>(a, p, stream);
-            case 1 * 16 + 4: return launch_cls<T, I, P, A, 1, 4, SHIFTED>(a, p, stream);
-            case 2 * 16 + 1: return launch_cls<T, I, P, A, 2, 1, SHIFTED>(a, p, stream);
-            case 2 * 16 + 4: return launch_cls<T, I, P, A, 2, 4, SHIFTED>(a, p, stream);
-            case 2 * 16 + 8: return launch_cls<T, I, P, A, 2, 8, SHIFTED>(a, p, stream);
-            case 3 * 16 + 1: return launch_cls<T, I, P, A, 3, 1, SHIFTED>(a, p, stream);
-            case 3 * 16 + 4: return launch_cls<T, I, P, A, 3, 4, SHIFTED>(a, p, stream);
-            case 3 * 16 + 8: return launch_cls<T, I, P, A, 3, 8, SHIFTED>(a, p, stream);
-            case 4 * 16 + 1: return launch_cls<T, I, P, A, 4, 1, SHIFTED>(a, p, stream);
-            case 4 * 16 + 4: return launch_cls<T, I, P, A, 4, 4, SHIFTED>(a, p, stream);
-            case 4 * 16 + 8: return launch_cls<T, I, P, A, 4, 8, SHIFTED>(a, p, stream);
+            case 0 * 16 + 1: return launch_cls<T, I, 0, 1, SHIFTED>(a, p, stream);
+            case 0 * 16 + 4: return launch_cls<T, I, 0, 4, SHIFTED>(a, p, stream);
+            case 1 * 16 + 1: return launch_cls<T, I, 1, 1, SHIFTED>(a, p, stream);
+            case 1 * 16 + 4: return launch_cls<T, I, 1, 4, SHIFTED>(a, p, stream);
+            case 2 * 16 + 1: return launch_cls<T, I, 2, 1, SHIFTED>(a, p, stream);
+            case 2 * 16 + 4: return launch_cls<T, I, 2, 4, SHIFTED>(a, p, stream);
+            case 2 * 16 + 8: return launch_cls<T, I, 2, 8, SHIFTED>(a, p, stream);
+            case 3 * 16 + 1: return launch_cls<T, I, 3, 1, SHIFTED>(a, p, stream);
+            case 3 * 16 + 4: return launch_cls<T, I, 3, 4, SHIFTED>(a, p, stream);
+            case 3 * 16 + 8: return launch_cls<T, I, 3, 8, SHIFTED>(a, p, stream);
+            case 4 * 16 + 1: return launch_cls<T, I, 4, 1, SHIFTED>(a, p, stream);
+            case 4 * 16 + 4: return launch_cls<T, I, 4, 4, SHIFTED>(a, p, stream);
+            case 4 * 16 + 8: return launch_cls<T, I, 4, 8, SHIFTED>(a, p, stream);
             default: return hipErrorInvalidValue;
         }
     }
@@ -123,7 +123,13 @@ struct LdsTypedLauncher {
 template <typename T, bool SHIFTED>
 hipError_t lds_launch_typed(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t stream)
 {
-    return dispatch_modes<T>(a, LdsTypedLauncher<T, SHIFTED>{a, p, stream});
+    const LdsTypedLauncher<T, SHIFTED> launcher{a, p, stream};
+    switch (a.interp) {
+        case 0: return launcher.template run<0>();
+        case 1: return launcher.template run<1>();
+        case 2: return launcher.template run<2>();
+        default: return hipErrorInvalidValue;
+    }
 }
 
 extern template hipError_t lds_launch_typed<float, false>(const GridSamplerArgs&, const LdsPlan&, hipStream_t);

@@ -98,6 +98,30 @@ __device__ __forceinline__ float compute_source_index(float coord, int32_t size)
     return compute_coordinates<PAD, ALIGN>(unnormalize<ALIGN>(coord, size), size);
 }
 
+// The same with padding mode and align_corners as run-time, wave-uniform values (kernel arguments): each branch is the
+// instantiation above, so the arithmetic is identical; the branches are scalar.
+__device__ __forceinline__ float unnormalize_rt(float coord, int32_t size, bool align)
+{
+    return align ? unnormalize<true>(coord, size) : unnormalize<false>(coord, size);
+}
+
+__device__ __forceinline__ float compute_coordinates_rt(float coord, int32_t size, int32_t pad, bool align)
+{
+    if (pad == 1) {
+        coord = clip_coordinates(coord, size);
+    } else if (pad == 2) {
+        coord = align ? reflect_coordinates(coord, 0.0f, 2.0f * (float)(size - 1))
+                      : reflect_coordinates(coord, -0.5f, 2.0f * (float)size);
+        coord = clip_coordinates(coord, size);
+    }
+    return coord;
+}
+
+__device__ __forceinline__ float compute_source_index_rt(float coord, int32_t size, int32_t pad, bool align)
+{
+    return compute_coordinates_rt(unnormalize_rt(coord, size, align), size, pad, align);
+}
+
 __device__ __forceinline__ bool nan_or_inf(float x) { return __builtin_isnan(x) || __builtin_isinf(x); }
 
 // grid_sampler2_d_simt.h:209-215
@@ -259,6 +283,43 @@ __device__ __forceinline__ BicubicTap decide_bicubic(float gx, float gy, int32_t
     for (int k = 0; k < 4; k++) {
         t.bx[k] = safe_float_to_i32(compute_coordinates<PAD, ALIGN>(ixf + (float)(k - 1), W));
         t.by[k] = safe_float_to_i32(compute_coordinates<PAD, ALIGN>(iyf + (float)(k - 1), H));
+    }
+    t.cx[0] = cubic_convolution2(tx + 1.0f, A);
+    t.cx[1] = cubic_convolution1(tx, A);
+    t.cx[2] = cubic_convolution1(1.0f - tx, A);
+    t.cx[3] = cubic_convolution2(2.0f - tx, A);
+    t.cy[0] = cubic_convolution2(ty + 1.0f, A);
+    t.cy[1] = cubic_convolution1(ty, A);
+    t.cy[2] = cubic_convolution1(1.0f - ty, A);
+    t.cy[3] = cubic_convolution2(2.0f - ty, A);
+    return t;
+}
+
+// decide_bicubic with run-time padding mode and align_corners (see compute_coordinates_rt)
+__device__ __forceinline__ BicubicTap decide_bicubic_rt(float gx, float gy, int32_t H, int32_t W, int32_t pad, bool align)
+{
+    constexpr float A = -0.75f;
+    BicubicTap t;
+    const float ix = unnormalize_rt(gx, W, align);
+    const float iy = unnormalize_rt(gy, H, align);
+    t.flag = 0;
+    if (nan_or_inf(ix) || nan_or_inf(iy)) {
+        t.flag = 1;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            t.bx[k] = t.by[k] = 0;
+            t.cx[k] = t.cy[k] = 0.0f;
+        }
+        return t;
+    }
+    const float ixf = __builtin_floorf(ix);
+    const float iyf = __builtin_floorf(iy);
+    const float tx = ix - ixf;
+    const float ty = iy - iyf;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        t.bx[k] = safe_float_to_i32(compute_coordinates_rt(ixf + (float)(k - 1), W, pad, align));
+        t.by[k] = safe_float_to_i32(compute_coordinates_rt(iyf + (float)(k - 1), H, pad, align));
     }
     t.cx[0] = cubic_convolution2(tx + 1.0f, A);
     t.cx[1] = cubic_convolution1(tx, A);
