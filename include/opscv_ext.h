@@ -73,6 +73,14 @@ ACLNN_API aclnnStatus opscvGridSampler2DNoAlloc(const aclTensor* input, const ac
                                                 int64_t interpolationMode, int64_t paddingMode, bool alignCorners,
                                                 aclTensor* out, aclrtStream stream);
 
+/*
+ * Revision of the data movement of a kernel variant (the names opscvExecutorVariant returns): a small integer that
+ * goes up whenever a change to the variant's kernels changes which bytes they move or how (loads, stores, staging,
+ * work split).  A counter measurement of memory traffic is valid for the revision it was taken on; the benchmark
+ * reports such a figure only while the revision matches.  Unknown names return 0.
+ */
+ACLNN_API int32_t opscvVariantRevision(const char* variant);
+
 /* Library version string, e.g. "opscv-amd 0.1 (gfx950)". */
 ACLNN_API const char* opscvVersion(void);
 

@@ -138,6 +138,8 @@ def load_library():
     L.opscvGridSampler2DNoAlloc.argtypes = [vp, vp, i64, i64, ctypes.c_bool, vp, vp]
     L.opscvVersion.restype = ctypes.c_char_p
     L.opscvVersion.argtypes = []
+    L.opscvVariantRevision.restype = ctypes.c_int32
+    L.opscvVariantRevision.argtypes = [ctypes.c_char_p]
     _lib = L
     return L
 
@@ -281,6 +283,11 @@ def destroy_executor(handle):
 
 def executor_variant(handle):
     return load_library().opscvExecutorVariant(handle).decode()
+
+
+def variant_revision(name):
+    """Revision of the data movement of a kernel variant (opscvVariantRevision)."""
+    return int(load_library().opscvVariantRevision(name.encode()))
 
 
 # ----------------------------------------------------------------------------------------------------

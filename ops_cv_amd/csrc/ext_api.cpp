@@ -3,6 +3,8 @@
 
 #include <hip/hip_runtime_api.h>
 
+#include <cstring>
+
 #include "acl_types.hpp"
 #include "kernels.hpp"
 
@@ -114,6 +116,36 @@ const char* opscvExecutorVariant(const aclOpExecutor* executor)
         default: break;
     }
     return "";
+}
+
+int32_t opscvVariantRevision(const char* variant)
+{
+    // longest matching prefix wins; bump an entry with the change that alters the variant's memory traffic
+    static const struct {
+        const char* prefix;
+        int32_t revision;
+    } table[] = {
+        // 2 (ring and pair variants): streaming stores and grid loads, batch-fastest block order; ring: 5:3 channel split
+        {"lds_ring", 2},
+        {"lds_pair", 2},       {"box_lds", 1},          {"direct", 1},          {"nhwc", 1},
+        {"nchw_band_lds", 1},  {"nchw_flat_lds", 1},    {"nchw_band", 1},       {"nchw_generic", 1},
+        {"nhwc_", 1},          {"nearest_", 1},         {"copy", 1},            {"point_copy", 1},
+        {"broadcast", 1},      {"first_pixel", 1},      {"resize_grad", 1},     {"gs2d_grad", 1},
+        {"gs3d_grad", 1},      {"gs3d_", 1},
+    };
+    if (variant == nullptr) {
+        return 0;
+    }
+    int32_t best = 0;
+    size_t best_len = 0;
+    for (const auto& e : table) {
+        const size_t n = strlen(e.prefix);
+        if (strncmp(variant, e.prefix, n) == 0 && n >= best_len) {
+            best = e.revision;
+            best_len = n;
+        }
+    }
+    return best;
 }
 
 const char* opscvVersion(void) { return "opscv-amd 0.1 (gfx950)"; }

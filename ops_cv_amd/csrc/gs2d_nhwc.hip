@@ -13,6 +13,8 @@
 // one element per lane and step.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "gs2d_common.hpp"
 #include "gs2d_lds_kernel.hpp"
 #include "kernels.hpp"
@@ -106,8 +108,14 @@ __global__ __launch_bounds__(kNhwcThreads) void gs2d_nhwc_kernel(const T* __rest
         const int64_t p = first + (int64_t)j * groups;
         live[j] = p < total_pixels;
         pix[j] = live[j] ? p : total_pixels - 1;
-        gx[j] = ElemIO<T>::load(grid + 2 * pix[j]);
-        gy[j] = ElemIO<T>::load(grid + 2 * pix[j] + 1);
+        // grid points and results stream (non-temporal hint), the tap loads do not: see load_grid_points in
+        // gs2d_lds_kernel.hpp
+        typedef typename std::conditional<sizeof(T) == 2, uint16_t, uint32_t>::type bits_t;
+        const bits_t* gp = reinterpret_cast<const bits_t*>(grid + 2 * pix[j]);
+        const T ex = __builtin_bit_cast(T, __builtin_nontemporal_load(gp));
+        const T ey = __builtin_bit_cast(T, __builtin_nontemporal_load(gp + 1));
+        gx[j] = ElemIO<T>::load(&ex);
+        gy[j] = ElemIO<T>::load(&ey);
     }
     NhwcPixel<NT, NW> px[PIX];
     const T* xn[PIX];
@@ -156,11 +164,13 @@ __global__ __launch_bounds__(kNhwcThreads) void gs2d_nhwc_kernel(const T* __rest
             if (live[j]) {
                 T* yp = y + pix[j] * C + c;
                 if constexpr (VEC) {
-                    uint4 packed;
+                    typedef uint32_t dwordx4_t __attribute__((ext_vector_type(4)));
+                    dwordx4_t packed;
                     __builtin_memcpy(&packed, outv, 16);
-                    *reinterpret_cast<uint4*>(yp) = packed;
+                    __builtin_nontemporal_store(packed, reinterpret_cast<dwordx4_t*>(yp));
                 } else {
-                    yp[0] = outv[0];
+                    typedef typename std::conditional<sizeof(T) == 2, uint16_t, uint32_t>::type bits_t;
+                    __builtin_nontemporal_store(__builtin_bit_cast(bits_t, outv[0]), reinterpret_cast<bits_t*>(yp));
                 }
             }
         }

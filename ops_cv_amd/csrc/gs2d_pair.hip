@@ -89,9 +89,9 @@ hipError_t pair_launch_one(const GridSamplerArgs& a, const PairPlan& p, hipStrea
     const int pair_aligned = (reinterpret_cast<uintptr_t>(a.grid) % 4 == 0);
     const uint32_t blocks = (uint32_t)(a.N * p.tiles_per_n * p.cblocks);
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3((kPairSamplerWaves + kPairLoaderWaves) * 64), p.lds_bytes, stream,
-                       (const T*)a.x, (const T*)a.grid, (T*)a.y, (int32_t)a.C, (int32_t)a.Hin, (int32_t)a.Win,
-                       (int32_t)(a.Hout * a.Wout), p.tiles_per_n, p.cblocks, p.chans_per_block, pair_aligned,
-                       p.xcd_swizzle, -0.0f);
+                       (const T*)a.x, (const T*)a.grid, (T*)a.y, make_fast_div((uint32_t)a.N), (int32_t)a.C,
+                       (int32_t)a.Hin, (int32_t)a.Win, (int32_t)(a.Hout * a.Wout), make_fast_div(p.tiles_per_n),
+                       p.chans_per_block, pair_aligned, p.xcd_swizzle, -0.0f);
     return hipGetLastError();
 }
 

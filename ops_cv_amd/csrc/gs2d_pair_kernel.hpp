@@ -72,9 +72,9 @@ __device__ __forceinline__ float blend_pairs(uint32_t north, uint32_t south, con
 // spreads the sixteen rows a wavefront covers over all banks (a 16-way conflict otherwise).
 template <typename T, int PAD, bool ALIGN, int SWAVES, int LWAVES, int PPT, int PITCH, int RMAX>
 __global__ __launch_bounds__((SWAVES + LWAVES) * 64) void gs2d_pair_kernel(
-    const T* __restrict__ x, const T* __restrict__ grid, T* __restrict__ y, int32_t C, int32_t H, int32_t W,
-    int32_t out_plane, uint32_t tiles_per_n, uint32_t cblocks, int32_t chans_per_block, int32_t pair_aligned,
-    int32_t xcd_swizzle, float neg_zero)
+    const T* __restrict__ x, const T* __restrict__ grid, T* __restrict__ y, FastDiv N, int32_t C, int32_t H, int32_t W,
+    int32_t out_plane, FastDiv tiles_per_n, int32_t chans_per_block, int32_t pair_aligned, int32_t xcd_swizzle,
+    float neg_zero)
 {
     static_assert(sizeof(T) == 2, "pairs of 16-bit elements");
     static_assert(PPT % 2 == 0, "two neighbouring pixels per store");
@@ -91,18 +91,21 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) void gs2d_pair_kernel(
     const int tid = threadIdx.x;
     const uint32_t wave = __builtin_amdgcn_readfirstlane((uint32_t)tid >> 6);
 
+    // groups (channel block, n) are numbered with the batch item fastest, as in the ring kernel (gs2d_lds_kernel.hpp):
+    // the workgroups in flight together cover every batch item (bf16 N8 C128 128x128 -> 256x256: 51.5 -> 49.0 us)
     uint32_t group, tile;
     if (xcd_swizzle) {
         const uint32_t xcd = blockIdx.x & 7u;
         const uint32_t i = blockIdx.x >> 3;
-        group = (i / tiles_per_n) * 8u + xcd;
-        tile = i % tiles_per_n;
+        const uint32_t k = fast_div(i, tiles_per_n);
+        group = k * 8u + xcd;
+        tile = i - k * tiles_per_n.div;
     } else {
-        group = blockIdx.x / tiles_per_n;
-        tile = blockIdx.x % tiles_per_n;
+        group = fast_div(blockIdx.x, tiles_per_n);
+        tile = blockIdx.x - group * tiles_per_n.div;
     }
-    const uint32_t cb = group % cblocks;
-    const uint32_t n = group / cblocks;
+    const uint32_t cb = fast_div(group, N);
+    const uint32_t n = group - cb * N.div;
     const int32_t plane_elems = H * W;
     const int32_t c_begin = (int32_t)cb * chans_per_block;
     const int32_t c_end = (c_begin + chans_per_block < C) ? c_begin + chans_per_block : C;
@@ -224,7 +227,10 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) void gs2d_pair_kernel(
         gptr[2 * q] = gridn + (int64_t)pc * 2;
         gptr[2 * q + 1] = gridn + (int64_t)(pc + 1) * 2;
     }
-    load_grid_points<T, PPT>(gptr, pair_aligned != 0, gxs, gys);
+    // grid points and results stream (non-temporal hint), the plane loads of the loaders do not: see
+    // load_grid_points in gs2d_lds_kernel.hpp (bf16 N8 C128 128x128 -> 256x256: 69.3 -> 51.0 us; with streaming plane
+    // loads as well 102 us)
+    load_grid_points<T, PPT, true>(gptr, pair_aligned != 0, gxs, gys);
     uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
     asm volatile("" : "+s"(lds_base));  // kept as a value: seen as the allocation's symbol it is re-added per use
     const uint32_t outside = ((uint32_t)H + 1u) * ROW_STEP;  // rows H + 1 and H + 2: zeros for both pairs
@@ -296,7 +302,7 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) void gs2d_pair_kernel(
                     read_pixel(j, next_off);
                     __builtin_amdgcn_sched_barrier(0);
                 }
-                buffer_store_group<T, 2>(v, rsrc, pixoff[q]);
+                buffer_store_group<T, 2, true>(v, rsrc, pixoff[q]);
             }
         }
     }
