@@ -208,7 +208,7 @@ __global__ __launch_bounds__(kThreads) void gs3d_kernel(const T* __restrict__ x,
             for (int k = 1; k < 8; k++) {
                 acc += v[k] * wt[k];
             }
-            ElemIO<T>::store(yc, acc);
+            store_streaming<T>(yc, acc);
             xc += in_vol;
             yc += p.out_vol;
         }
@@ -225,7 +225,7 @@ __global__ __launch_bounds__(kThreads) void gs3d_kernel(const T* __restrict__ x,
         for (int k = 1; k < 8; k++) {
             acc += v[k] * wt[k];
         }
-        ElemIO<T>::store(yc, acc);
+        store_streaming<T>(yc, acc);
         xc += in_vol;
         yc += p.out_vol;
     }
@@ -333,7 +333,7 @@ __global__ __launch_bounds__(kThreads) void gs3d_pair16_kernel(const T* __restri
         for (int k = 1; k < 8; k++) {
             acc += v[k] * wt[k];
         }
-        ElemIO<T>::store(yc, acc);
+        store_streaming<T>(yc, acc);
         yc += p.out_vol;
     };
     for (int32_t c = c_begin; c < c_end; c++) {

@@ -14,7 +14,9 @@ namespace {
 
 constexpr int kBand = 12;               // output rows per workgroup (measured best on the 4K x2 upscale)
 constexpr int kLdsBudget = 64 * 1024;   // per workgroup, so that at least two are resident per CU
-constexpr int64_t kStreamingBytes = 128ll << 20;  // outputs beyond this are written with non-temporal stores
+// outputs from this size on are written with non-temporal stores (written through instead of left dirty in L2 for the
+// end of the kernel to write back)
+constexpr int64_t kStreamingBytes = 1ll << 20;
 
 struct BandPlan {
     bool ok = false;

@@ -11,7 +11,9 @@
 //   * A lane computes its column taps once; it then walks the band rows  hb + group, hb + group + rg, ...  and
 //     evaluates the reference formula per output element from eight (fp32: four-byte, else two-byte) LDS reads
 //     per column pair -- same operations in the same order as the per-pixel reference.
-//   * One 16-byte store per lane and row through a buffer descriptor over the output plane.
+//   * One 16-byte store per lane and row through a buffer descriptor over the output plane, non-temporal (the lines
+//     are written through instead of staying dirty in L2 for the end of the kernel to write back: fp32 8x64x56x56 ->
+//     112x112 8.7 -> 6.7 us).
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -142,7 +144,7 @@ __global__ __launch_bounds__(THREADS) void resize_flat_lds_kernel(const T* __res
             const uint32_t out_off = (uint32_t)h * out_row_bytes + col_off;
             if (nvalid == V) {
                 // rows of a width that is not a multiple of V start anywhere: the store is element-aligned
-                __builtin_amdgcn_raw_buffer_store_b128(packed, rsrc, (int)out_off, 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b128(packed, rsrc, (int)out_off, 0, 2);
             } else {
                 // the lane that holds the ragged end of the row stores its elements singly
 #pragma unroll
@@ -150,10 +152,10 @@ __global__ __launch_bounds__(THREADS) void resize_flat_lds_kernel(const T* __res
                     if (i < nvalid) {
                         if constexpr (sizeof(T) == 4) {
                             __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, outv[i]), rsrc,
-                                                                  (int)(out_off + i * 4), 0, 0);
+                                                                  (int)(out_off + i * 4), 0, 2);
                         } else {
                             __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(uint16_t, outv[i]), rsrc,
-                                                                  (int)(out_off + i * 2), 0, 0);
+                                                                  (int)(out_off + i * 2), 0, 2);
                         }
                     }
                 }

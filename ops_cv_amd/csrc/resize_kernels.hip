@@ -27,6 +27,10 @@ constexpr int kThreads = 256;
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 // 16-byte store that bypasses the caches (for outputs much larger than them)
+// Outputs from this size on are written with non-temporal stores: the lines are written through instead of staying
+// dirty in L2 until the end of the kernel writes them back (fp32 8x64x56x56 -> 112x112, 25.7 MB of output: 8.7 -> 6.7 us).
+constexpr int64_t kResizeStreamingBytes = 1ll << 20;
+
 __device__ __forceinline__ void store_streaming(uint4* dst, uint4 v)
 {
     u32x4_t t;
@@ -944,7 +948,7 @@ hipError_t run_resize(const ResizeArgs& a, hipStream_t stream)
 #define OPSCV_NEAREST(NHWC_, VEC_)                                                                                  \
     hipLaunchKernelGGL((resize_nearest_kernel<T, NHWC_, VEC_>), grid, dim3(kThreads), 0, stream, x, y, outer,      \
                        (int32_t)a.C, (int32_t)a.Hs, (int32_t)a.Ws, (int32_t)a.Hd, (int32_t)a.Wd, rule, streaming)
-        const int streaming = (out_elems * (int64_t)sizeof(T) >= (128ll << 20)) ? 1 : 0;
+        const int streaming = (out_elems * (int64_t)sizeof(T) >= kResizeStreamingBytes) ? 1 : 0;
         const NearestRule rule{a.scale_h, a.scale_w, a.rep_h, a.rep_w};
         if (const uint64_t slot = nearest_lds_slot<T>(a)) {
             const int64_t vlanes = (row_elems + V - 1) / V;
@@ -975,7 +979,7 @@ hipError_t run_resize(const ResizeArgs& a, hipStream_t stream)
         const int ue = four_weights_unit<T>(a);
         const int64_t row_units = a.Wd * (a.C / ue);
         const int64_t rows = a.N * a.Hd;
-        const int streaming = (out_elems * (int64_t)sizeof(T) >= (128ll << 20)) ? 1 : 0;
+        const int streaming = (out_elems * (int64_t)sizeof(T) >= kResizeStreamingBytes) ? 1 : 0;
         dim3 grid((unsigned)((row_units + kThreads - 1) / kThreads), (unsigned)(rows < 65535 ? rows : 65535));
 #define OPSCV_FOUR(HP, UE)                                                                                           \
     hipLaunchKernelGGL((resize_nhwc_four_weights_kernel<T, HP, UE>), grid, dim3(kThreads), 0, stream, x, y, a.N,      \
@@ -1005,7 +1009,7 @@ hipError_t run_resize(const ResizeArgs& a, hipStream_t stream)
         constexpr int V = 16 / (int)sizeof(T);
         const int64_t row_vecs = a.Wd * (a.C / V);
         const int64_t bands = (a.Hd + kNhwcBand - 1) / kNhwcBand;
-        const int streaming = (out_elems * (int64_t)sizeof(T) >= (128ll << 20)) ? 1 : 0;
+        const int streaming = (out_elems * (int64_t)sizeof(T) >= kResizeStreamingBytes) ? 1 : 0;
         dim3 grid((unsigned)((row_vecs + kThreads - 1) / kThreads), (unsigned)bands,
                   (unsigned)(a.N < 65535 ? a.N : 65535));
         if (a.half_pixel) {

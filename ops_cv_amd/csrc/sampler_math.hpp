@@ -39,6 +39,20 @@ struct ElemIO<__bf16> {
     static __device__ __forceinline__ void store(__bf16* p, float v) { *p = (__bf16)v; }
 };
 
+// Store of one element with the non-temporal hint (same rounding as ElemIO<T>::store): for results that are written
+// once and not read again by the kernel, so that they are written through instead of staying dirty in L2.
+template <typename T>
+__device__ __forceinline__ void store_streaming(T* p, float v)
+{
+    T e;
+    ElemIO<T>::store(&e, v);
+    if constexpr (sizeof(T) == 4) {
+        __builtin_nontemporal_store(__builtin_bit_cast(uint32_t, e), reinterpret_cast<uint32_t*>(p));
+    } else {
+        __builtin_nontemporal_store(__builtin_bit_cast(uint16_t, e), reinterpret_cast<uint16_t*>(p));
+    }
+}
+
 // grid_sampler2_d_simt.h:125-132
 template <bool ALIGN>
 __device__ __forceinline__ float unnormalize(float coord, int32_t size)
