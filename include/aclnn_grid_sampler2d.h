@@ -23,6 +23,15 @@
  * non-finite coordinate into an out-of-range one) and NaN here.  It also unnormalises as ((g + 1) * size - 1) / 2,
  * which can pick the neighbouring pair of corner pixels for coordinates within an ulp of a pixel centre (results stay
  * within tolerance).
+ *
+ * A caller that replaces the reference library on that part and wants its results, non-finite grid values included,
+ * selects that second kernel's arithmetic for the bilinear mode with the process-wide option "grid_sampler2d_rule" = 1
+ * (opscvSetOption in opscv_ext.h, or OPSCV_GRID_SAMPLER2D_RULE=arch35 in the environment when the library is loaded):
+ * unnormalisation ((g + 1) * size - 1) / 2, reflection with fmodf, every non-finite coordinate turned into -100 (a zero
+ * sample), weights (1 - dh)(1 - dw) ..., grid_sampler_2d_bilinear_smit.h:67-153 and
+ * grid_sampler_bilinear_smit_common.h:36-90.  The option is read by the first phase and kept in the executor; nearest
+ * and bicubic are not affected (the reference serves them with other kernels on that part).  The default stays the
+ * rule described above.
  */
 #ifndef OPSCV_ACLNN_GRID_SAMPLER2D_H_
 #define OPSCV_ACLNN_GRID_SAMPLER2D_H_

@@ -74,6 +74,31 @@ ACLNN_API aclnnStatus opscvGridSampler2DNoAlloc(const aclTensor* input, const ac
                                                 aclTensor* out, aclrtStream stream);
 
 /*
+ * Process-wide options.  They start from the environment, read once when the library first needs one of them, and
+ * change only through opscvSetOption afterwards; every GetWorkspaceSize call copies the values it needs into its
+ * executor, so a second phase runs with the options of its first phase and never looks at the environment.
+ *
+ *   name                    environment (initial value)      values
+ *   "grid_sampler2d_rule"   OPSCV_GRID_SAMPLER2D_RULE=arch35  0 (default): bilinear coordinates as in the reference's
+ *                                                            GridSampler2D kernel (grid_sampler2_d_simt.h);
+ *                                                            1: as in the kernel its aclnnGridSampler2D launches on
+ *                                                            its newest part (see aclnn_grid_sampler2d.h)
+ *   "reference_cores"       OPSCV_REFERENCE_CORES            vector cores of the reference's device (default 64): its
+ *                                                            choice between two resize templates and the chunk phase
+ *                                                            of the 3-D sampler gradient read it
+ *   "reference_ub_bytes"    OPSCV_REFERENCE_UB_BYTES         unified buffer of the reference's device (default
+ *                                                            253952): gates its replicating nearest-resize template
+ *   "gs_variant"            OPSCV_GS_VARIANT=direct|ring     0 automatic, 1 direct kernel, 2 no pair-layout variant
+ *   "resize_variant"        OPSCV_RESIZE_VARIANT=generic|register|band   0 automatic, 1 per-element kernels,
+ *                                                            2 register-band kernel, 3 no flat LDS kernel
+ *   "nearest_variant"       OPSCV_NEAREST_VARIANT=gather     0 automatic, 1 gather from memory
+ * The last three pick among kernels with identical results (tests and benchmarks use them); the first three can
+ * change result bits.  Returns ACLNN_ERR_PARAM_INVALID for an unknown name or a value out of range.
+ */
+ACLNN_API aclnnStatus opscvSetOption(const char* name, int64_t value);
+ACLNN_API aclnnStatus opscvGetOption(const char* name, int64_t* value);
+
+/*
  * Revision of the data movement of a kernel variant (the names opscvExecutorVariant returns): a small integer that
  * goes up whenever a change to the variant's kernels changes which bytes they move or how (loads, stores, staging,
  * work split).  A counter measurement of memory traffic is valid for the revision it was taken on; the benchmark

@@ -138,6 +138,10 @@ def load_library():
     L.opscvGridSampler2DNoAlloc.argtypes = [vp, vp, i64, i64, ctypes.c_bool, vp, vp]
     L.opscvVersion.restype = ctypes.c_char_p
     L.opscvVersion.argtypes = []
+    L.opscvSetOption.restype = ctypes.c_int
+    L.opscvSetOption.argtypes = [ctypes.c_char_p, ctypes.c_int64]
+    L.opscvGetOption.restype = ctypes.c_int
+    L.opscvGetOption.argtypes = [ctypes.c_char_p, ctypes.POINTER(ctypes.c_int64)]
     L.opscvVariantRevision.restype = ctypes.c_int32
     L.opscvVariantRevision.argtypes = [ctypes.c_char_p]
     _lib = L
@@ -283,6 +287,37 @@ def destroy_executor(handle):
 
 def executor_variant(handle):
     return load_library().opscvExecutorVariant(handle).decode()
+
+
+def set_option(name, value):
+    """opscvSetOption; raises on an unknown name or a value out of range."""
+    st = load_library().opscvSetOption(name.encode(), int(value))
+    if st != ACLNN_SUCCESS:
+        raise AclnnError("opscvSetOption(%r, %r)" % (name, value), st)
+
+
+def get_option(name):
+    v = ctypes.c_int64(0)
+    st = load_library().opscvGetOption(name.encode(), ctypes.byref(v))
+    if st != ACLNN_SUCCESS:
+        raise AclnnError("opscvGetOption(%r)" % name, st)
+    return v.value
+
+
+class option:
+    """Context manager: an option set for the block and restored afterwards."""
+
+    def __init__(self, name, value):
+        self.name, self.value = name, value
+
+    def __enter__(self):
+        self.saved = get_option(self.name)
+        set_option(self.name, self.value)
+        return self
+
+    def __exit__(self, *exc):
+        set_option(self.name, self.saved)
+        return False
 
 
 def variant_revision(name):

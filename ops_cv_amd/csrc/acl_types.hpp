@@ -97,6 +97,9 @@ struct GridSamplerArgs {
     int pad = 0;
     int align = 0;
     int channels_last = 0;  // 1: x is (N,Hin,Win,C) and y is (N,Hout,Wout,C) in memory
+    // values of the process-wide options (options.hpp) at the time of the first phase:
+    int rule = 0;           // bilinear coordinate rule: 0 grid_sampler2_d_simt.h, 1 the arch35 GridSample kernel
+    int force_variant = 0;  // GsVariant: 0 automatic choice, 1 direct kernel, 2 no pair-layout variant
     int64_t N = 0, C = 0, Hin = 0, Win = 0, Hout = 0, Wout = 0;
     const void* x = nullptr;
     const void* grid = nullptr;
@@ -170,6 +173,9 @@ struct ResizeArgs {
     int half_pixel = 1;
     int channels_last = 0;
     int raw_lambda = 0;  // NCHW bilinear: fraction taken from the unclamped source coordinate (see axis_tap)
+    // values of the process-wide options (options.hpp) at the time of the first phase:
+    int force_variant = 0;  // ResizeVariant: 0 automatic, 1 per-element kernels, 2 register band, 3 no flat LDS kernel
+    int force_nearest = 0;  // NearestVariant: 0 automatic, 1 gather from memory (no LDS staging)
     float scale_h = 1.0f, scale_w = 1.0f;
     int32_t rep_h = 0, rep_w = 0;  // Nearest: whole upscale factors when source = destination / factor is the rule, else 0
     int64_t point_step_h = 1, point_step_w = 1;  // PointCopy: integer source stride per destination pixel

@@ -7,6 +7,7 @@
 
 #include "aclnn_grid_sampler2d.h"
 #include "executor.hpp"
+#include "options.hpp"
 #include "opscv_ext.h"
 
 using namespace opscv;
@@ -141,6 +142,12 @@ aclnnStatus plan_grid_sampler2d(const aclTensor* input, const aclTensor* grid, i
 
     ex->kind = OpKind::GridSampler2D;
     GridSamplerArgs& a = ex->gs;
+    // the process-wide options as they are now; the second phase runs with these whatever is set in between
+    const Options opt = current_options();
+    a.force_variant = opt.gs_variant;
+    // the second coordinate rule exists for the bilinear mode only (the reference's arch35 GridSample kernel is
+    // bilinear; its nearest and bicubic modes take other kernels, which are not mirrored)
+    a.rule = (interpolationMode == 0) ? opt.grid_sampler2d_rule : kRuleGridSampler2D;
     a.elem = elem;
     a.interp = (int)interpolationMode;
     a.pad = (int)paddingMode;
@@ -154,7 +161,9 @@ aclnnStatus plan_grid_sampler2d(const aclTensor* input, const aclTensor* grid, i
     const int esz = elem_size(elem);
     // Views that are dense in channels-last order (what a framework hands over for its channels_last memory
     // format) are sampled in place by the channels-last kernel instead of being repacked to NCHW and back.
-    if (!input->contiguous() && !out->contiguous() && channels_last_dense(input) && channels_last_dense(out)) {
+    // (the channels-last kernel implements the first coordinate rule only: under the second, such views are packed)
+    if (a.rule == kRuleGridSampler2D && !input->contiguous() && !out->contiguous() && channels_last_dense(input) &&
+        channels_last_dense(out)) {
         a.channels_last = 1;
         ex->in0.direct = (input->data == nullptr) ? nullptr : (char*)input->data + input->offset * (int64_t)esz;
         ex->out0.direct = (out->data == nullptr) ? nullptr : (char*)out->data + out->offset * (int64_t)esz;

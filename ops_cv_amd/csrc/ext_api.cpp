@@ -7,6 +7,7 @@
 
 #include "acl_types.hpp"
 #include "kernels.hpp"
+#include "options.hpp"
 
 using namespace opscv;
 
@@ -118,6 +119,32 @@ const char* opscvExecutorVariant(const aclOpExecutor* executor)
     return "";
 }
 
+aclnnStatus opscvSetOption(const char* name, int64_t value)
+{
+    if (name == nullptr) {
+        set_error("opscvSetOption: name must not be NULL");
+        return ACLNN_ERR_PARAM_NULLPTR;
+    }
+    if (!set_option(name, value)) {
+        set_error("opscvSetOption: unknown option '%s' or value %lld out of its range", name, (long long)value);
+        return ACLNN_ERR_PARAM_INVALID;
+    }
+    return ACLNN_SUCCESS;
+}
+
+aclnnStatus opscvGetOption(const char* name, int64_t* value)
+{
+    if (name == nullptr || value == nullptr) {
+        set_error("opscvGetOption: name and value must not be NULL");
+        return ACLNN_ERR_PARAM_NULLPTR;
+    }
+    if (!get_option(name, value)) {
+        set_error("opscvGetOption: unknown option '%s'", name);
+        return ACLNN_ERR_PARAM_INVALID;
+    }
+    return ACLNN_SUCCESS;
+}
+
 int32_t opscvVariantRevision(const char* variant)
 {
     // longest matching prefix wins; bump an entry with the change that alters the variant's memory traffic
@@ -127,7 +154,7 @@ int32_t opscvVariantRevision(const char* variant)
     } table[] = {
         // 2 (ring and pair variants): streaming stores and grid loads, batch-fastest block order; ring: 5:3 channel split
         {"lds_ring", 2},
-        {"lds_pair", 2},       {"box_lds", 1},          {"direct", 1},          {"nhwc", 1},
+        {"lds_pair", 2},       {"box_lds", 1},          {"direct", 1},          {"direct_arch35", 1},          {"nhwc", 1},
         {"nchw_band_lds", 1},  {"nchw_flat_lds", 1},    {"nchw_band", 1},       {"nchw_generic", 1},
         {"nhwc_", 1},          {"nearest_", 1},         {"copy", 1},            {"point_copy", 1},
         {"broadcast", 1},      {"first_pixel", 1},      {"resize_grad", 1},     {"gs2d_grad", 1},

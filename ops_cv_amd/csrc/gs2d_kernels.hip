@@ -16,6 +16,7 @@
 
 #include "gs2d_common.hpp"
 #include "kernels.hpp"
+#include "options.hpp"
 #include "sampler_math.hpp"
 
 namespace opscv {
@@ -216,6 +217,63 @@ __global__ __launch_bounds__(kDirectThreads) void gs2d_direct_kernel(const T* __
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// Bilinear sampling by the second coordinate rule (option "grid_sampler2d_rule" = 1), for every shape the LDS ring
+// does not take: the arithmetic of the kernel that the reference's aclnnGridSampler2D launches for NCHW tensors on its
+// arch35 part, image/grid_sample/op_kernel/arch35/grid_sampler_2d_bilinear_smit.h:67-153 with
+// grid_sampler_bilinear_smit_common.h:36-90 -- unnormalise as ((g + 1) * size - 1) / 2, reflect with fmodf, a
+// non-finite coordinate becomes -100 (a zero sample), weights (1 - dh)(1 - dw) ..., the sum starts with the bare first
+// product, a corner outside the image counts as the value 0.  One lane per output pixel, decisions hoisted out of the
+// channel loop (the reference repeats them per channel; they do not depend on it).
+// ---------------------------------------------------------------------------------------------------------
+template <typename T, int PAD, bool ALIGN>
+__global__ __launch_bounds__(kDirectThreads) void gs2d_arch35_kernel(const T* __restrict__ x,
+                                                                      const T* __restrict__ grid,
+                                                                      T* __restrict__ y, int64_t total_pixels,
+                                                                      int32_t C_all, int32_t H, int32_t W,
+                                                                      int64_t out_plane, int32_t chan_chunk)
+{
+    const int32_t c_first = (int32_t)blockIdx.y * chan_chunk;
+    const int32_t C = (c_first + chan_chunk < C_all) ? chan_chunk : C_all - c_first;
+    const int64_t in_plane = (int64_t)H * W;
+    const int64_t stride = (int64_t)gridDim.x * kDirectThreads;
+    for (int64_t p = (int64_t)blockIdx.x * kDirectThreads + threadIdx.x; p < total_pixels; p += stride) {
+        const int64_t n = p / out_plane;
+        const int64_t rem = p - n * out_plane;
+        const float gw = ElemIO<T>::load(grid + 2 * p);
+        const float gh = ElemIO<T>::load(grid + 2 * p + 1);
+        const float pw = clip3<PAD, ALIGN>(unnormalize3<ALIGN>(gw, W), W);
+        const float ph = clip3<PAD, ALIGN>(unnormalize3<ALIGN>(gh, H), H);
+        const float hf = __builtin_floorf(ph), wf = __builtin_floorf(pw);
+        const float dh = ph - hf, dw = pw - wf;
+        // corner indices from the floats floor and floor + 1 (saturating conversion: anything beyond int32 lies
+        // outside every image, like the reference's out-of-range conversion)
+        const int32_t h0 = float_to_i32(hf), w0 = float_to_i32(wf);
+        const int32_t h1 = float_to_i32(hf + 1.0f), w1 = float_to_i32(wf + 1.0f);
+        const bool in[4] = {within(h0, w0, H, W), within(h0, w1, H, W), within(h1, w0, H, W), within(h1, w1, H, W)};
+        const int64_t off[4] = {in[0] ? (int64_t)h0 * W + w0 : 0, in[1] ? (int64_t)h0 * W + w1 : 0,
+                                in[2] ? (int64_t)h1 * W + w0 : 0, in[3] ? (int64_t)h1 * W + w1 : 0};
+        const float wt[4] = {(1.0f - dh) * (1.0f - dw), (1.0f - dh) * dw, dh * (1.0f - dw), dh * dw};
+        const T* xp = x + (n * C_all + c_first) * in_plane;
+        T* yp = y + (n * C_all + c_first) * out_plane + rem;
+#pragma unroll 4
+        for (int32_t c = 0; c < C; c++) {
+            float v[4];
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                v[k] = in[k] ? ElemIO<T>::load(xp + off[k]) : 0.0f;
+            }
+            float out = v[0] * wt[0];
+            out += v[1] * wt[1];
+            out += v[2] * wt[2];
+            out += v[3] * wt[3];
+            ElemIO<T>::store(yp, out);
+            xp += in_plane;
+            yp += out_plane;
+        }
+    }
+}
+
 template <typename T, int INTERP, int PAD, bool ALIGN>
 __global__ __launch_bounds__(kDirectThreads) void gs2d_taps_kernel(const T* __restrict__ grid,
                                                                     TapRecord* __restrict__ taps,
@@ -295,6 +353,25 @@ hipError_t run_direct(const GridSamplerArgs& a, hipStream_t stream)
     return hipGetLastError();
 }
 
+template <typename T, int PAD, bool ALIGN>
+hipError_t run_arch35(const GridSamplerArgs& a, hipStream_t stream)
+{
+    const int64_t total = a.N * a.Hout * a.Wout;
+    const int blocks = blocks_for(total, kDirectThreads);
+    int64_t chunks = (8192 + blocks - 1) / blocks;  // as run_direct
+    chunks = chunks < a.C ? chunks : a.C;
+    chunks = chunks < 1 ? 1 : chunks;
+    const int64_t chan_chunk = (a.C + chunks - 1) / chunks;
+    const int64_t grid_y = (a.C + chan_chunk - 1) / chan_chunk;
+    if (grid_y > 65535) {
+        return hipErrorInvalidValue;
+    }
+    hipLaunchKernelGGL((gs2d_arch35_kernel<T, PAD, ALIGN>), dim3((unsigned)blocks, (unsigned)grid_y),
+                       dim3(kDirectThreads), 0, stream, (const T*)a.x, (const T*)a.grid, (T*)a.y, total,
+                       (int32_t)a.C, (int32_t)a.Hin, (int32_t)a.Win, a.Hout * a.Wout, (int32_t)chan_chunk);
+    return hipGetLastError();
+}
+
 template <typename T, int INTERP, int PAD, bool ALIGN>
 hipError_t run_taps(const GridSamplerArgs& a, TapRecord* taps, hipStream_t stream)
 {
@@ -332,6 +409,20 @@ struct DirectLauncher {
     }
 };
 
+struct Arch35Launcher {
+    const GridSamplerArgs& a;
+    hipStream_t stream;
+    template <typename T, int I, int P, bool A>
+    hipError_t operator()() const
+    {
+        if constexpr (I == 0) {
+            return run_arch35<T, P, A>(a, stream);
+        } else {
+            return hipErrorInvalidValue;
+        }
+    }
+};
+
 struct TapsLauncher {
     const GridSamplerArgs& a;
     TapRecord* taps;
@@ -357,27 +448,26 @@ struct BicubicTapsLauncher {
 }  // namespace
 
 namespace {
-// OPSCV_GS_VARIANT=direct forces the direct kernel, OPSCV_GS_VARIANT=ring keeps the pair-layout variant out
+// option "gs_variant" as captured by the first phase: the direct kernel forced, or the pair-layout variant kept out
 // (benchmark and test knobs)
-bool force_direct()
-{
-    const char* v = getenv("OPSCV_GS_VARIANT");
-    return v != nullptr && v[0] == 'd';
-}
-bool force_ring()
-{
-    const char* v = getenv("OPSCV_GS_VARIANT");
-    return v != nullptr && v[0] == 'r';
-}
+bool force_direct(const GridSamplerArgs& a) { return a.force_variant == kGsDirect; }
+bool force_ring(const GridSamplerArgs& a) { return a.force_variant == kGsRing; }
 }  // namespace
+
+// The second coordinate rule (bilinear only) is implemented by the LDS ring and by a direct kernel of its own.
+static bool second_rule(const GridSamplerArgs& a) { return a.rule != kRuleGridSampler2D && a.interp == 0; }
 
 const char* grid_sampler2d_variant(const GridSamplerArgs& a)
 {
+    if (second_rule(a)) {
+        const char* n = force_direct(a) ? nullptr : gs2d_lds_variant_name(a);
+        return n != nullptr ? n : "direct_arch35";
+    }
     if (a.channels_last) {
         return "nhwc";
     }
-    if (!force_direct()) {
-        const char* n = force_ring() ? nullptr : gs2d_pair_variant_name(a);
+    if (!force_direct(a)) {
+        const char* n = force_ring(a) ? nullptr : gs2d_pair_variant_name(a);
         if (n == nullptr) {
             n = gs2d_lds_variant_name(a);
         }
@@ -402,12 +492,25 @@ hipError_t launch_grid_sampler2d(const GridSamplerArgs& a, hipStream_t stream)
     if (a.x == nullptr || a.grid == nullptr || a.y == nullptr) {
         return hipErrorInvalidValue;
     }
+    if (second_rule(a)) {
+        if (a.channels_last) {
+            return hipErrorInvalidValue;  // the first phase packs such views under this rule
+        }
+        if (!force_direct(a)) {
+            bool handled = false;
+            const hipError_t e = run_gs2d_lds(a, stream, &handled);
+            if (handled || e != hipSuccess) {
+                return e;
+            }
+        }
+        return dispatch_elem(a, Arch35Launcher{a, stream});
+    }
     if (a.channels_last) {
         return run_gs2d_nhwc(a, stream);
     }
-    if (!force_direct()) {
+    if (!force_direct(a)) {
         bool handled = false;
-        hipError_t e = force_ring() ? hipSuccess : run_gs2d_pair(a, stream, &handled);
+        hipError_t e = force_ring(a) ? hipSuccess : run_gs2d_pair(a, stream, &handled);
         if (handled || e != hipSuccess) {
             return e;
         }

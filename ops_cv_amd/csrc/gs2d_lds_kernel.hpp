@@ -156,8 +156,12 @@ __device__ __forceinline__ float tap_value_of(const R& raw)
 // multiply-adds, and so is the column of the four row results.  A tap outside the image reads the zero slot; a
 // row outside the image therefore evaluates to +0 like the reference's literal 0 (the products are zeros and at
 // least one of the two middle coefficients is positive, so the sum cannot be -0).
+//
+// `first` is the addend of the first bilinear product: +0 for "0 + nw" as above; -0 gives the bare product "nw" with
+// which the reference's second bilinear kernel starts its sum (grid_sampler_2d_bilinear_smit.h:78-82), which differs
+// in the sign of a zero result only.
 template <typename T, int INTERP, typename R>
-__device__ __forceinline__ float blend(const R* raw, const float* tw, float neg_zero)
+__device__ __forceinline__ float blend(const R* raw, const float* tw, float neg_zero, float first = 0.0f)
 {
     if (INTERP == 2) {
         float r[4];
@@ -176,7 +180,7 @@ __device__ __forceinline__ float blend(const R* raw, const float* tw, float neg_
         return as_fp32_value(out);
     }
     if (INTERP == 0) {
-        float out = __builtin_fmaf(tap_value_of<T>(raw[0]), tw[0], 0.0f);
+        float out = __builtin_fmaf(tap_value_of<T>(raw[0]), tw[0], first);
         out += __builtin_fmaf(tap_value_of<T>(raw[1]), tw[1], neg_zero);
         out += __builtin_fmaf(tap_value_of<T>(raw[2]), tw[2], neg_zero);
         out += __builtin_fmaf(tap_value_of<T>(raw[3]), tw[3], neg_zero);
@@ -391,10 +395,33 @@ __device__ __forceinline__ void source_indices(const float* gxs, const float* gy
     }
 }
 
+// ... by the second coordinate rule (sampler_math.hpp: unnormalize3, clip3): always finite, -100 for what was not
+template <int PAD, bool ALIGN, int COUNT>
+__device__ __forceinline__ void source_indices_arch35(const float* gxs, const float* gys, int32_t H, int32_t W,
+                                                      float* ixs, float* iys)
+{
+#pragma unroll
+    for (int j = 0; j < COUNT; j++) {
+        ixs[j] = clip3<PAD, ALIGN>(unnormalize3<ALIGN>(gxs[j], W), W);
+        iys[j] = clip3<PAD, ALIGN>(unnormalize3<ALIGN>(gys[j], H), H);
+    }
+}
+
 template <int COUNT>
 __device__ __forceinline__ void source_indices_rt(const float* gxs, const float* gys, int32_t H, int32_t W, int32_t pad,
-                                                  bool align, float* ixs, float* iys)
+                                                  bool align, bool arch35, float* ixs, float* iys)
 {
+    if (arch35) {
+        switch (pad * 2 + (align ? 1 : 0)) {
+            case 0: source_indices_arch35<0, false, COUNT>(gxs, gys, H, W, ixs, iys); break;
+            case 1: source_indices_arch35<0, true, COUNT>(gxs, gys, H, W, ixs, iys); break;
+            case 2: source_indices_arch35<1, false, COUNT>(gxs, gys, H, W, ixs, iys); break;
+            case 3: source_indices_arch35<1, true, COUNT>(gxs, gys, H, W, ixs, iys); break;
+            case 4: source_indices_arch35<2, false, COUNT>(gxs, gys, H, W, ixs, iys); break;
+            default: source_indices_arch35<2, true, COUNT>(gxs, gys, H, W, ixs, iys); break;
+        }
+        return;
+    }
     switch (pad * 2 + (align ? 1 : 0)) {
         case 0: source_indices<0, false, COUNT>(gxs, gys, H, W, ixs, iys); break;
         case 1: source_indices<0, true, COUNT>(gxs, gys, H, W, ixs, iys); break;
@@ -408,12 +435,12 @@ __device__ __forceinline__ void source_indices_rt(const float* gxs, const float*
 template <typename T, int INTERP, int PPT, int NT, int NW, bool SWIZZLED>
 __device__ __forceinline__ void decide_lane_pixels(const float* gxs, const float* gys, int32_t H, int32_t W,
                                                    uint32_t row_shift, uint32_t zero_off, int32_t pad, bool align,
-                                                   uint32_t (*toff)[NT], float (*tw)[NW])
+                                                   bool arch35, uint32_t (*toff)[NT], float (*tw)[NW])
 {
     const uint32_t rs = SWIZZLED ? row_shift : 0u;
     float ixs[PPT], iys[PPT];
     if constexpr (INTERP != 2) {
-        source_indices_rt<PPT>(gxs, gys, H, W, pad, align, ixs, iys);
+        source_indices_rt<PPT>(gxs, gys, H, W, pad, align, arch35 && INTERP == 0, ixs, iys);
     }
 #pragma unroll
     for (int j = 0; j < PPT; j++) {
@@ -454,6 +481,8 @@ __device__ __forceinline__ void decide_lane_pixels(const float* gxs, const float
             iy = y_far ? -100.0f : iy;
             const float ixf = __builtin_floorf(ix), iyf = __builtin_floorf(iy);
             const uint32_t x0 = (uint32_t)float_to_i32(ixf), y0 = (uint32_t)float_to_i32(iyf);
+            // the second rule takes the east / south index from the float "floor + 1"
+            // (grid_sampler_2d_bilinear_smit.h:84-99), which is the integer "+ 1" for every index a staged plane has
             const uint32_t x1 = x0 + 1u, y1 = y0 + 1u;
             const bool in_x0 = x0 < uw && finite, in_x1 = x1 < uw && finite;
             const bool in_y0 = y0 < uh, in_y1 = y1 < uh;
@@ -463,10 +492,13 @@ __device__ __forceinline__ void decide_lane_pixels(const float* gxs, const float
             toff[j][1] = (in_y0 && in_x1) ? lds_swizzle(o_nw + es, rs) : zero_off;
             toff[j][2] = (in_y1 && in_x0) ? lds_swizzle(o_sw, rs) : zero_off;
             toff[j][3] = (in_y1 && in_x1) ? lds_swizzle(o_sw + es, rs) : zero_off;
-            const float wx1 = ix - ixf, wx0 = ixf + 1.0f - ix;
-            const float wy1 = iy - iyf, wy0 = iyf + 1.0f - iy;
+            // weights: (x0 + 1 - ix), (ix - x0) by the first rule; (1 - d), d with d = ix - floor(ix) by the second
+            // (grid_sampler_2d_bilinear_smit.h:72-76)
+            const float wx1 = ix - ixf, wx0 = arch35 ? 1.0f - wx1 : ixf + 1.0f - ix;
+            const float wy1 = iy - iyf, wy0 = arch35 ? 1.0f - wy1 : iyf + 1.0f - iy;
             // non-finite source coordinate: every tap reads the zero slot and 0 * NaN makes every channel NaN,
-            // as the reference writes (grid_sampler2_d_simt.h:485-487)
+            // as the reference writes (grid_sampler2_d_simt.h:485-487); under the second rule the coordinate has
+            // become -100 by now and the sample is zero
             tw[j][0] = finite ? wx0 * wy0 : __builtin_nanf("");
             tw[j][1] = wx1 * wy0;
             tw[j][2] = wx0 * wy1;
@@ -507,7 +539,7 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
     const T* __restrict__ x, const T* __restrict__ grid, T* __restrict__ y, FastDiv N, int32_t C, int32_t H, int32_t W,
     int32_t out_plane, FastDiv tiles_per_n, int32_t chans_per_block, uint32_t wide_blocks,
     int32_t chans_wide, int32_t copy_gran, int32_t pair_aligned, int32_t xcd_swizzle, int32_t row_shift, int32_t pad,
-    int32_t align, float neg_zero)
+    int32_t align, int32_t rule, float neg_zero)
 {
     extern __shared__ uint4 smem_raw[];
     char* lds = reinterpret_cast<char*>(smem_raw);
@@ -666,11 +698,16 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
     load_grid_points<T, PPT, true>(gptr, pair_aligned != 0, gxs, gys);
     // the bank-spreading layout exists for border padding only (see make_lds_plan: row_shift is 0 otherwise)
     const uint32_t rs = (uint32_t)row_shift;
+    // `rule` != 0: the coordinate rule of the reference's second bilinear kernel (bilinear only)
+    const bool arch35 = rule != 0;
     if (rs != 0u) {
-        decide_lane_pixels<T, INTERP, PPT, NT, NW, true>(gxs, gys, H, W, rs, zero_off, pad, align != 0, toff, tw);
+        decide_lane_pixels<T, INTERP, PPT, NT, NW, true>(gxs, gys, H, W, rs, zero_off, pad, align != 0, arch35, toff,
+                                                         tw);
     } else {
-        decide_lane_pixels<T, INTERP, PPT, NT, NW, false>(gxs, gys, H, W, rs, zero_off, pad, align != 0, toff, tw);
+        decide_lane_pixels<T, INTERP, PPT, NT, NW, false>(gxs, gys, H, W, rs, zero_off, pad, align != 0, arch35, toff,
+                                                          tw);
     }
+    const float first_zero = arch35 ? neg_zero : 0.0f;
 
     // tap offsets become absolute LDS addresses (left as offsets, the compiler re-adds the allocation's base to
     // every tap in every stage)
@@ -746,7 +783,7 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
 #pragma unroll
                 for (int a = 0; a < ADJ; a++) {
                     const int j = q * ADJ + a;
-                    v[a] = blend<T, INTERP>(raw[j], tw[j], neg_zero);
+                    v[a] = blend<T, INTERP>(raw[j], tw[j], neg_zero, first_zero);
                     if (j == 0 && un % CGS == 0) {
                         __builtin_amdgcn_s_waitcnt(0xC07F);
                         lds_barrier();  // stage (p + 1) / CGS has landed (or, behind the last plane, nothing)

@@ -57,7 +57,8 @@ hipError_t launch_one(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t st
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3((kSamplerWaves + LWAVES) * 64), p.lds_bytes, stream, (const T*)a.x, (const T*)a.grid,
                        (T*)a.y, make_fast_div((uint32_t)a.N), (int32_t)a.C, (int32_t)a.Hin, (int32_t)a.Win, (int32_t)(a.Hout * a.Wout),
                        make_fast_div(p.tiles_per_n), p.chans_per_block, p.wide_blocks, p.chans_wide, p.copy_gran,
-                       pair_aligned, p.xcd_swizzle, p.row_shift, (int32_t)a.pad, (int32_t)(a.align != 0), -0.0f);
+                       pair_aligned, p.xcd_swizzle, p.row_shift, (int32_t)a.pad, (int32_t)(a.align != 0), (int32_t)a.rule,
+                       -0.0f);
     return hipGetLastError();
 }
 

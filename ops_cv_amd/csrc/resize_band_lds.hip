@@ -5,6 +5,7 @@
 #include <cstdlib>
 
 #include "kernels.hpp"
+#include "options.hpp"
 #include "resize_band_lds_kernel.hpp"
 #include "resize_flat_lds_kernel.hpp"
 
@@ -123,8 +124,8 @@ BandPlan make_plan(const ResizeArgs& a)
     bp.p.streaming = (a.N * a.C * a.Hd * a.Wd * (int64_t)sizeof(T) >= kStreamingBytes) ? 1 : 0;
     bp.lds_bytes = (uint32_t)bytes;
     bp.grid = dim3((unsigned)cblocks, (unsigned)bands, (unsigned)(planes < 65535 ? planes : 65535));
-    const char* v = getenv("OPSCV_RESIZE_VARIANT");
-    bp.ok = !(v != nullptr && (v[0] == 'g' || v[0] == 'r'));  // generic / register-band forced (benchmark knob)
+    // generic / register-band forced (benchmark knob, option "resize_variant")
+    bp.ok = !(a.force_variant == kResizeGeneric || a.force_variant == kResizeRegisterBand);
     return bp;
 }
 
@@ -225,9 +226,8 @@ FlatPlan make_flat_plan(const ResizeArgs& a)
     fp.p.raw_lambda = a.raw_lambda;
     fp.lds_bytes = (uint32_t)(((int64_t)rows * a.Ws * (int64_t)sizeof(T) + (gran == 1 ? 15 : 0) + 15) / 16 * 16);
     fp.grid = dim3((unsigned)bands, (unsigned)(planes < 65535 ? planes : 65535));
-    const char* v = getenv("OPSCV_RESIZE_VARIANT");
-    // generic / register-band / LDS band forced (benchmark knob)
-    fp.ok = !(v != nullptr && (v[0] == 'g' || v[0] == 'r' || v[0] == 'b'));
+    // generic / register-band / LDS band forced (benchmark knob, option "resize_variant")
+    fp.ok = a.force_variant == kResizeAuto;
     return fp;
 }
 

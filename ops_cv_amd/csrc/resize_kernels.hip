@@ -14,6 +14,7 @@
 #include <type_traits>
 
 #include "kernels.hpp"
+#include "options.hpp"
 #include "resize_band_lds_kernel.hpp"
 #include "resize_math.hpp"
 #include "sampler_math.hpp"
@@ -808,8 +809,7 @@ bool band_variant_ok(const ResizeArgs& a)
     if ((a.Hd + kBand - 1) / kBand > 65535) {
         return false;
     }
-    const char* v = getenv("OPSCV_RESIZE_VARIANT");
-    return !(v != nullptr && v[0] == 'g');  // OPSCV_RESIZE_VARIANT=generic forces the generic kernel
+    return a.force_variant != kResizeGeneric;  // option "resize_variant" = generic forces the generic kernel
 }
 
 // The vector NHWC variant moves whole 16-byte runs of channels.
@@ -832,8 +832,7 @@ int nhwc_unit_bytes(const ResizeArgs& a)
         reinterpret_cast<uintptr_t>(a.x) % esz != 0 || reinterpret_cast<uintptr_t>(a.y) % esz != 0) {
         return 0;
     }
-    const char* v = getenv("OPSCV_RESIZE_VARIANT");
-    if (v != nullptr && v[0] == 'g') {
+    if (a.force_variant == kResizeGeneric) {
         return 0;
     }
     const int64_t pixel_bytes = a.C * esz;
@@ -883,8 +882,7 @@ uint64_t nearest_lds_slot(const ResizeArgs& a)
     if (nhwc && a.Hd * a.Wd < a.Hs * a.Ws) {
         return 0;  // shrinking images: nothing is reused, the gather from memory is as fast (measured)
     }
-    const char* v = getenv("OPSCV_NEAREST_VARIANT");
-    if (v != nullptr && v[0] == 'g') {
+    if (a.force_nearest == kNearestGather) {
         return 0;
     }
     const double span = (double)(kThreads * V) * (double)a.scale_w * 1.001 + 2.0 + 2.0 * V + 2.0 * (double)ci;

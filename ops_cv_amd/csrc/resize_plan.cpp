@@ -1,5 +1,7 @@
 #include "resize_plan.hpp"
 
+#include "options.hpp"
+
 #include <cfloat>
 #include <cmath>
 #include <cstdint>
@@ -50,6 +52,9 @@ static bool point_copy_steps(const ResizeArgs& a, bool align_corners, int64_t* s
 
 void plan_resize(ResizeArgs* a, bool align_corners, float user_scale_h, float user_scale_w)
 {
+    const Options opt = current_options();
+    a->force_variant = opt.resize_variant;
+    a->force_nearest = opt.nearest_variant;
     a->half_pixel = align_corners ? 0 : 1;
     a->scale_h = resize_axis_scale(a->Hs, a->Hd, align_corners, user_scale_h);
     a->scale_w = resize_axis_scale(a->Ws, a->Wd, align_corners, user_scale_w);
@@ -90,29 +95,12 @@ void plan_resize(ResizeArgs* a, bool align_corners, float user_scale_h, float us
     }
 }
 
-int64_t reference_vector_cores()
-{
-    if (const char* v = getenv("OPSCV_REFERENCE_CORES")) {
-        const long n = strtol(v, nullptr, 10);
-        if (n > 0) {
-            return n;
-        }
-    }
-    return 64;  // the core count of the reference's tiling unit test (test_resize_bilinear_v2_tiling.cpp: {64, 245760})
-}
+// option "reference_cores" (options.hpp): 64 unless set, the core count of the reference's tiling unit test
+int64_t reference_vector_cores() { return current_options().reference_cores; }
 
-// bytes of the reference device's unified buffer: OPSCV_REFERENCE_UB_BYTES, else that of the reference's tiling unit
-// test (test_resize_nearest_neighbor_v2_tiling.cpp: {64, 253952})
-static int64_t reference_ub_bytes()
-{
-    if (const char* v = getenv("OPSCV_REFERENCE_UB_BYTES")) {
-        const long long n = strtoll(v, nullptr, 10);
-        if (n > 0) {
-            return n;
-        }
-    }
-    return 253952;
-}
+// bytes of the reference device's unified buffer, option "reference_ub_bytes": 253952 unless set, that of the
+// reference's tiling unit test
+static int64_t reference_ub_bytes() { return current_options().reference_ub_bytes; }
 
 // Whether the reference resizes this channels-last tensor with the template that replicates every source pixel a
 // whole number of times (IsMatchTiling_NHWC_UB2UB, resize_nearest_neighbor_v2_tiling_base.cpp:640-665, called with
@@ -147,6 +135,9 @@ static bool nearest_replicates(const ResizeArgs& a)
 
 void plan_resize_nearest(ResizeArgs* a)
 {
+    const Options opt = current_options();
+    a->force_variant = opt.resize_variant;
+    a->force_nearest = opt.nearest_variant;
     a->half_pixel = 0;
     a->scale_h = (float)a->Hs / (float)a->Hd;
     a->scale_w = (float)a->Ws / (float)a->Wd;

@@ -346,6 +346,72 @@ __device__ __forceinline__ BicubicTap decide_bicubic_rt(float gx, float gy, int3
     return t;
 }
 
+// ---- the coordinate rule of the reference's GridSample operator on its arch35 part ----
+// (the 3-D sampler follows it; the 2-D sampler offers it as its second rule: the kernel that the reference's
+// aclnnGridSampler2D launches there, image/grid_sample/op_kernel/arch35/grid_sampler_2d_bilinear_smit.h:109-153)
+
+// grid_sampler_bilinear_smit_common.h:37-46 (size is an unsigned index type there: size - 1 is converted to
+// float for the comparison, the replacement value is float(size) - 1)
+__device__ __forceinline__ float clip3_coordinates(float coord, int32_t size)
+{
+    coord = (coord < 0.0f) ? 0.0f : coord;
+    coord = (coord > (float)(size - 1)) ? (float)size - 1.0f : coord;
+    if (__builtin_isnan(coord) || __builtin_isinf(coord)) {
+        return 0.0f;
+    }
+    return coord;
+}
+
+// grid_sampler_bilinear_smit_common.h:48-66.  `low2` is twiceLow (0 or -1), `span2` is twiceHigh - twiceLow.
+// The parity of floor(coord / span) is taken from the float itself: every float of 2^24 or more is an even
+// integer, below that the conversion to an integer is exact.
+__device__ __forceinline__ float reflect3_coordinates(float coord, int32_t low2, int64_t span2)
+{
+    if (span2 == 0) {
+        return 0.0f;
+    }
+    const float mn = (float)low2 / 2.0f;
+    const float span = (float)span2 / 2.0f;
+    coord = __builtin_fabsf(coord - mn);
+    const float extra = __builtin_fmodf(coord, span);
+    const float fl = __builtin_floorf(coord / span);
+    const bool odd = (fl < 16777216.0f) && (((int32_t)fl & 1) != 0);
+    if (!odd) {
+        return extra + mn;
+    }
+    return span - extra + mn;
+}
+
+// grid_sampler_bilinear_smit_common.h:76-92
+template <int PAD, bool ALIGN>
+__device__ __forceinline__ float clip3(float coord, int32_t size)
+{
+    if (PAD == 1) {
+        coord = clip3_coordinates(coord, size);
+    } else if (PAD == 2) {
+        if (ALIGN) {
+            coord = reflect3_coordinates(coord, 0, 2 * ((int64_t)size - 1));
+        } else {
+            coord = reflect3_coordinates(coord, -1, 2 * (int64_t)size);
+        }
+        coord = clip3_coordinates(coord, size);
+    }
+    if (nan_or_inf(coord)) {
+        return -100.0f;
+    }
+    return coord;
+}
+
+// grid_sampler_3d_bilinear_smit.h:171-179
+template <bool ALIGN>
+__device__ __forceinline__ float unnormalize3(float g, int32_t size)
+{
+    if (ALIGN) {
+        return (g + 1.0f) / 2.0f * (float)(size - 1);
+    }
+    return ((g + 1.0f) * (float)size - 1.0f) / 2.0f;
+}
+
 __device__ __forceinline__ bool within(int32_t h, int32_t w, int32_t H, int32_t W)
 {
     return h >= 0 && h < H && w >= 0 && w < W;

@@ -33,3 +33,22 @@ def device():
     if not torch.cuda.is_available():
         pytest.fail("GPU tests need a GPU: the HIP path has no CPU fallback")
     return torch.device("cuda:0")
+
+
+OPTION_NAMES = ("gs_variant", "resize_variant", "nearest_variant", "reference_cores", "reference_ub_bytes",
+                "grid_sampler2d_rule")
+
+
+@pytest.fixture(autouse=True)
+def _library_options_restored():
+    """The library's process-wide options (opscvSetOption) are put back after every test that changed them."""
+    try:
+        from ops_cv_amd import aclnn as a
+        a.load_library()
+    except Exception:  # the library is not built: the tests that need it fail on their own
+        yield
+        return
+    saved = {n: a.get_option(n) for n in OPTION_NAMES}
+    yield
+    for n, v in saved.items():
+        a.set_option(n, v)

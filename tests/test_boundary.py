@@ -623,3 +623,39 @@ def test_resize_template_selection_point_copy(aclnn, desc):
     # NCHW never takes the template
     assert _rs(aclnn, desc, inp=(1, 32, 9, 15), out=(1, 32, 3, 5), scales=(1, 1, 1 / 3, 1 / 3), mode=b"bilinear")[2] != \
         "point_copy"
+
+
+def test_options_api_and_rule_captured_at_phase_one(aclnn):
+    """opscvSetOption / opscvGetOption: names, ranges, defaults; the bilinear coordinate rule goes into the executor at
+    phase 1 (the variant name of a shape beyond LDS shows it) and applies to the bilinear mode only"""
+    defaults = {"gs_variant": 0, "resize_variant": 0, "nearest_variant": 0, "reference_cores": 64,
+                "reference_ub_bytes": 253952, "grid_sampler2d_rule": 0}
+    for name, value in defaults.items():
+        assert aclnn.get_option(name) == value, name
+    L = aclnn.load_library()
+    assert L.opscvSetOption(b"no_such_option", 1) == 161002
+    assert L.opscvSetOption(b"grid_sampler2d_rule", 2) == 161002
+    assert L.opscvSetOption(b"reference_cores", 0) == 161002
+    assert L.opscvSetOption(None, 0) == 161001
+    assert aclnn.get_option("grid_sampler2d_rule") == 0
+    f16 = aclnn.ACL_FLOAT16
+
+    def variant(interp):
+        hs = [aclnn.create_tensor((1, 2, 300, 310), f16), aclnn.create_tensor((1, 20, 24, 2), f16),
+              aclnn.create_tensor((1, 2, 20, 24), f16)]
+        st, ws, ex = aclnn.get_workspace_size_grid_sampler2d(hs[0], hs[1], interp, 0, False, hs[2])
+        assert st == 0 and ws == 0
+        v = aclnn.executor_variant(ex)
+        aclnn.destroy_executor(ex)
+        for h in hs:
+            aclnn.destroy_tensor(h)
+        return v
+
+    assert variant(0) == "direct"
+    with aclnn.option("grid_sampler2d_rule", 1):
+        assert variant(0) == "direct_arch35"
+        assert variant(1) == "direct"  # nearest: the rule does not apply
+    assert variant(0) == "direct"
+    with aclnn.option("gs_variant", 1):
+        assert aclnn.get_option("gs_variant") == 1
+    assert aclnn.get_option("gs_variant") == 0

@@ -83,10 +83,10 @@ def test_upsample_nhwc(oracle, device, aclnn, dtype, align):
 @pytest.mark.parametrize("dtype", I.DTYPES)
 @pytest.mark.parametrize("forced", ["generic", "register"])
 def test_upsample_nhwc_kernels_behind_the_lds_variant(oracle, device, aclnn, dtype, forced, monkeypatch):
-    """OPSCV_RESIZE_VARIANT=generic reaches the per-element channels-last kernel (kept for band counts beyond the grid
-    limit), =register the unit kernel on shapes that the LDS-staged variant would take; both match the oracle"""
+    """Option resize_variant = generic reaches the per-element channels-last kernel (kept for band counts beyond the grid
+    limit), = register the unit kernel on shapes that the LDS-staged variant would take; both match the oracle"""
     torch = _torch()
-    monkeypatch.setenv("OPSCV_RESIZE_VARIANT", forced)
+    aclnn.set_option("resize_variant", {"generic": 1, "register": 2}[forced])
     rng = np.random.default_rng(29)
     seen = set()
     for (N, C, H, W), size, align in [((2, 5, 7, 9), (14, 18), False), ((1, 3, 9, 6), (4, 11), True),
@@ -738,7 +738,7 @@ def test_grid_sampler3d_backward_gather_variant(oracle, device, aclnn, dtype, mo
     seen_gathered = seen_flagged = 0
     try:
         for (N, C, (D, H, W), (Do, Ho, Wo), kind, cores) in cases:
-            monkeypatch.setenv("OPSCV_REFERENCE_CORES", str(cores))
+            aclnn.set_option("reference_cores", cores)
             oracle.set_reference_cores(cores)
             g32 = lattice(N, Do, Ho, Wo, 0.1, 0.03)
             if kind == "mixed":
@@ -782,7 +782,7 @@ def test_grid_sampler3d_backward_gather_variant(oracle, device, aclnn, dtype, mo
                 seen_flagged += flags.count(1)
     finally:
         oracle.set_reference_cores(64)
-        monkeypatch.delenv("OPSCV_REFERENCE_CORES")
+        aclnn.set_option("reference_cores", 64)
     assert seen_gathered > 0 and seen_flagged > 0
 
 
@@ -802,7 +802,7 @@ def test_grid_sampler3d_backward_core_split_mask_layouts_and_torch(oracle, devic
         results = []
         try:
             for cores in (2, 64):
-                monkeypatch.setenv("OPSCV_REFERENCE_CORES", str(cores))
+                aclnn.set_option("reference_cores", cores)
                 oracle.set_reference_cores(cores)
                 rdx, rdg = oracle.grid_sampler3d_backward(go, x, g, 0, 1, False)
                 dx, dg = aclnn.grid_sampler3d_backward(*(torch.from_numpy(a).to(device) for a in (go, x, g)), 0, 1,
@@ -813,7 +813,7 @@ def test_grid_sampler3d_backward_core_split_mask_layouts_and_torch(oracle, devic
                 results.append(rdx)
         finally:
             oracle.set_reference_cores(64)
-            monkeypatch.delenv("OPSCV_REFERENCE_CORES")
+            aclnn.set_option("reference_cores", 64)
         # the order is visible in fp16
         assert not np.array_equal(results[0].view(np.uint16), results[1].view(np.uint16))
     # masks, strided views, channels-last, torch autograd (fp32)
@@ -956,7 +956,7 @@ def test_resize_nearest_replicating_template(oracle, device, aclnn, dtype, monke
     shape, (Ho, Wo) = cases[5]
     N, H, W, C = shape
     x = I.cast_np(rng.standard_normal(shape).astype(np.float32), dtype)
-    monkeypatch.setenv("OPSCV_REFERENCE_UB_BYTES", str(1 << 20))
+    aclnn.set_option("reference_ub_bytes", 1 << 20)
     oracle.set_reference_ub_bytes(1 << 20)
     try:
         ref = oracle.resize_nearest(x, (Ho, Wo), channels_last=True, dtype=code)

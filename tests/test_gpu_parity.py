@@ -127,9 +127,8 @@ def test_grid_sampler_pair_layout_variant(oracle, device, dtype, pad, align, mon
         what = "gs-pair %s %s align=%s %s" % (dtype, PAD[pad], align, (N, C, H, W, Ho, Wo))
         _check(y, y_ref, dtype, 0, what)
         _assert_same_bits(y, y_ref, what)
-        monkeypatch.setenv("OPSCV_GS_VARIANT", "ring")
-        y_ring = I.from_torch(aclnn.grid_sampler2d(xt, gt, 0, pad, align), dtype)
-        monkeypatch.delenv("OPSCV_GS_VARIANT")
+        with aclnn.option("gs_variant", 2):  # the pair-layout variant kept out
+            y_ring = I.from_torch(aclnn.grid_sampler2d(xt, gt, 0, pad, align), dtype)
         _assert_same_bits(y_ring, y_ref, what + " (ring kernel)")
 
 
@@ -146,6 +145,94 @@ def test_grid_sampler_special_coordinates(oracle, device, dtype, interp, pad, al
         y, y_ref = _run_gs(oracle, device, x32, g32, dtype, interp, pad, align)
         _check(y, y_ref, dtype, interp, "gs-special %s %s %s align=%s %s" % (dtype, INTERP[interp], PAD[pad], align,
                                                                               (H, W)))
+
+
+@pytest.mark.parametrize("dtype", I.DTYPES)
+@pytest.mark.parametrize("pad", [0, 1, 2])
+@pytest.mark.parametrize("align", [False, True])
+def test_grid_sampler_second_coordinate_rule(oracle, device, dtype, pad, align):
+    """option grid_sampler2d_rule = 1: bilinear sampling as the reference's aclnnGridSampler2D computes it on its arch35
+    part (grid_sampler_2d_bilinear_smit.h:109-153, grid_sampler_bilinear_smit_common.h:36-90), against the oracle's
+    restatement of that kernel: the special coordinates (ties, borders, 1e10, inf, NaN -- zeros here, where the
+    default rule writes NaN), random and affine grids, shapes served by the LDS ring, by the direct kernel (planes
+    beyond LDS, the ring switched off), channels-last and strided views; bit for bit.  The first phase fixes the rule:
+    an executor planned under one rule runs under it whatever the option says at the second phase."""
+    import torch
+    from ops_cv_amd import aclnn
+    rng = np.random.default_rng(3500 + pad * 10 + int(align))
+    code = I.oracle_code(dtype)
+    variants = set()
+
+    def run(x32, g32, forced=0, channels_last=False):
+        x, g = I.cast_np(x32, dtype), I.cast_np(g32, dtype)
+        ref = oracle.grid_sampler2d_arch35(x, g, pad, align, dtype=code)
+        xt, gt = I.to_torch(x, dtype, device), I.to_torch(g, dtype, device)
+        out = None
+        if channels_last:
+            xt = xt.contiguous(memory_format=torch.channels_last)
+            out = torch.empty((x.shape[0], x.shape[1], g.shape[1], g.shape[2]), dtype=xt.dtype,
+                              device=device).contiguous(memory_format=torch.channels_last)
+        if out is None:
+            out = torch.empty((x.shape[0], x.shape[1], g.shape[1], g.shape[2]), dtype=xt.dtype, device=device)
+        with aclnn.option("grid_sampler2d_rule", 1), aclnn.option("gs_variant", forced):
+            hs = [aclnn.tensor_handle(t) for t in (xt, gt, out)]
+            st, _, ex = aclnn.get_workspace_size_grid_sampler2d(hs[0], hs[1], 0, pad, align, hs[2])
+            assert st == 0
+            variants.add(aclnn.executor_variant(ex))
+            aclnn.destroy_executor(ex)
+            for h in hs:
+                aclnn.destroy_tensor(h)
+            y = aclnn.grid_sampler2d(xt, gt, 0, pad, align, out=out)
+        torch.cuda.synchronize()
+        what = "gs second rule %s %s align=%s %s forced=%d cl=%s" % (dtype, PAD[pad], align, x.shape, forced,
+                                                                     channels_last)
+        got = I.from_torch(y, dtype)
+        assert not np.isnan(I.as_f32(got, dtype)).any() or np.isnan(I.as_f32(x, dtype)).any(), what
+        _check(got, ref, dtype, 0, what)
+        _assert_same_bits(got, ref, what)
+        return got
+
+    special = I.special_grid()
+    for (H, W) in [(5, 8), (10, 10), (1, 7), (64, 64)]:
+        x32 = rng.standard_normal((1, 3, H, W)).astype(np.float32)
+        run(x32, special)
+        run(x32, special, forced=1)
+    for (N, C, H, W, Ho, Wo) in [(2, 5, 13, 17, 19, 23), (1, 16, 64, 64, 32, 32), (2, 8, 1, 1, 7, 5),
+                                 (1, 3, 40, 70, 64, 96)]:
+        x32 = rng.standard_normal((N, C, H, W)).astype(np.float32)
+        g32 = rng.uniform(-1.4, 1.4, (N, Ho, Wo, 2)).astype(np.float32)
+        run(x32, g32)
+        run(x32, g32, forced=1)
+        run(x32, g32, channels_last=True)
+    x32 = rng.standard_normal((2, 32, 64, 64)).astype(np.float32)
+    run(x32, I.affine_grid(rng, 2, 64, 64))
+    # planes beyond LDS: the rule's own direct kernel
+    x32 = rng.standard_normal((1, 2, 300, 310)).astype(np.float32)
+    run(x32, I.affine_grid(rng, 1, 120, 130))
+    assert any(v.startswith("lds_ring") for v in variants) and "direct_arch35" in variants, variants
+    # the default rule on a non-finite coordinate differs (NaN in every channel), so the switch is not vacuous ...
+    x32 = rng.standard_normal((1, 2, 6, 6)).astype(np.float32)
+    g32 = np.zeros((1, 1, 2, 2), np.float32)
+    g32[0, 0, 1, 0] = np.nan
+    y_default, _ = _run_gs(oracle, device, x32, g32, dtype, 0, pad, align)
+    y_second = run(x32, g32)
+    if pad == 0:
+        assert np.isnan(I.as_f32(y_default, dtype)[0, :, 0, 1]).all()
+    assert (I.as_f32(y_second, dtype)[0, :, 0, 1] == (0.0 if pad == 0 else I.as_f32(y_second, dtype)[0, :, 0, 1])).all()
+    # ... and an executor keeps the rule of its first phase
+    x, g = I.cast_np(x32, dtype), I.cast_np(g32, dtype)
+    xt, gt = I.to_torch(x, dtype, device), I.to_torch(g, dtype, device)
+    out = torch.empty((1, 2, 1, 2), dtype=xt.dtype, device=device)
+    hs = [aclnn.tensor_handle(t) for t in (xt, gt, out)]
+    with aclnn.option("grid_sampler2d_rule", 1):
+        st, ws, ex = aclnn.get_workspace_size_grid_sampler2d(hs[0], hs[1], 0, pad, align, hs[2])
+        assert st == 0 and ws == 0
+    assert aclnn.get_option("grid_sampler2d_rule") == 0
+    assert aclnn.load_library().aclnnGridSampler2D(None, 0, ex, aclnn._stream_handle(None)) == 0
+    torch.cuda.synchronize()
+    for h in hs:
+        aclnn.destroy_tensor(h)
+    assert np.array_equal(I.from_torch(out, dtype).view(np.uint8), y_second.view(np.uint8))
 
 
 @pytest.mark.parametrize("dtype", I.DTYPES)
@@ -238,11 +325,11 @@ def test_upsample_hw_split_template(oracle, device, dtype, monkeypatch):
     cases = [((1, 2, 56, 56), (112, 112), 0, 0), ((1, 1, 33, 65), (67, 200), 0, 0), ((1, 3, 64, 32), (200, 64), 0, 0),
              ((1, 1, 700, 8), (1400, 16), 0, 0), ((2, 2, 20, 300), (47, 1031), 0, 0), ((1, 2, 16, 600), (40, 1536), 0, 0),
              ((2, 3, 30, 36), (75, 54), 2.5, 1.5), ((1, 2, 40, 40), (24, 48), 0, 0)]
-    monkeypatch.setenv("OPSCV_REFERENCE_CORES", "1")
+    aclnn.set_option("reference_cores", 1)
     differs = 0
     try:
         for forced in ("", "b", "r", "g"):
-            monkeypatch.setenv("OPSCV_RESIZE_VARIANT", forced)
+            aclnn.set_option("resize_variant", {"": 0, "g": 1, "r": 2, "b": 3}[forced])
             for shape, out_hw, sh, sw in cases:
                 x32 = rng.standard_normal(shape).astype(np.float32)
                 oracle.set_reference_cores(1)

@@ -149,7 +149,7 @@ def test_random_resize_family(oracle, device, aclnn, monkeypatch):
     import torch
     rng = np.random.default_rng(9002 + SEED_SHIFT)
     # the reference picks its NCHW template by output pixels against cores * 1024: four cores put both templates in reach
-    monkeypatch.setenv("OPSCV_REFERENCE_CORES", "4")
+    aclnn.set_option("reference_cores", 4)
     oracle.set_reference_cores(4)
     try:
         _random_resize_family(oracle, device, aclnn, torch, rng)
