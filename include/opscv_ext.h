@@ -68,6 +68,12 @@ ACLNN_API const char* opscvExecutorVariant(const aclOpExecutor* executor);
  * Contiguous tensors and channels-last views use no scratch at all.  All calls on one device share the array: calls
  * that overlap in time on one device (different streams, different threads) race on it and must be serialised by the
  * caller; calls on one stream are ordered by the stream.  Asynchronous on `stream` like aclnnGridSampler2D.
+ *
+ * Under stream capture: the first call on a device asks the runtime for the address of that device's copy of the
+ * array, and the first launch of a kernel variant on a device sets that kernel's shared-memory attribute; neither may
+ * be recorded.  Make one ordinary (uncaptured) call with the same dtype, modes and shapes on the device before the
+ * capture begins; every later call, captured or not, only launches kernels.  The packing and clearing steps are
+ * kernels (no memset node is recorded).
  */
 ACLNN_API aclnnStatus opscvGridSampler2DNoAlloc(const aclTensor* input, const aclTensor* grid,
                                                 int64_t interpolationMode, int64_t paddingMode, bool alignCorners,
@@ -92,7 +98,9 @@ ACLNN_API aclnnStatus opscvGridSampler2DNoAlloc(const aclTensor* input, const ac
  *   "resize_variant"        OPSCV_RESIZE_VARIANT=generic|register|band   0 automatic, 1 per-element kernels,
  *                                                            2 register-band kernel, 3 no flat LDS kernel
  *   "nearest_variant"       OPSCV_NEAREST_VARIANT=gather     0 automatic, 1 gather from memory
- * The last three pick among kernels with identical results (tests and benchmarks use them); the first three can
+ *   "gs3d_grad_variant"     OPSCV_GS3D_GRAD_VARIANT=ordered|gather   0 automatic, 1 ordered kernel, 2 gather variant
+ *                                                            wherever it can run (input gradient of the 3-D sampler)
+ * The last four pick among kernels with identical results (tests and benchmarks use them); the first three can
  * change result bits.  Returns ACLNN_ERR_PARAM_INVALID for an unknown name or a value out of range.
  */
 ACLNN_API aclnnStatus opscvSetOption(const char* name, int64_t value);

@@ -144,6 +144,7 @@ struct GridSampler3DGradArgs {
     int align = 0;
     int64_t N = 0, C = 0, Din = 0, Hin = 0, Win = 0, Dout = 0, Hout = 0, Wout = 0;
     int64_t items_per_core = 1;  // batch items the reference walks as one run of grid points (chunk boundaries)
+    int force_variant = 0;       // option "gs3d_grad_variant" at the first phase: 0 automatic, 1 ordered kernel, 2 gather
     const void* gout = nullptr;  // (N,C,Dout,Hout,Wout)
     const void* x = nullptr;     // (N,C,Din,Hin,Win)
     const void* grid = nullptr;  // (N,Dout,Hout,Wout,3)
@@ -228,17 +229,24 @@ struct aclOpExecutor {
         static constexpr int kCapacity = 4;
         Pack items[kCapacity];
         int count = 0;
-        void push_back(const Pack& p)
+        // false when the list is full (the entry is dropped: the caller must fail the plan)
+        bool push_back(const Pack& p)
         {
-            if (count < kCapacity) {
-                items[count++] = p;
+            if (count >= kCapacity) {
+                return false;
             }
+            items[count++] = p;
+            return true;
         }
         const Pack* begin() const { return items; }
         const Pack* end() const { return items + count; }
     };
     PackList pack_in;
     PackList unpack_out;
+    // a view that needed packing found its list full: the plan is unusable and the first phase reports
+    // ACLNN_ERR_INNER (no operator has that many views today; a future one would fail loudly instead of
+    // reading an unpacked workspace slice)
+    bool pack_overflow = false;
 };
 
 namespace opscv {

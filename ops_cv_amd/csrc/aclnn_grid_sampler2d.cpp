@@ -177,7 +177,7 @@ aclnnStatus plan_grid_sampler2d(const aclTensor* input, const aclTensor* grid, i
     a.x = ex->in0.in_workspace ? nullptr : ex->in0.direct;
     a.grid = ex->in1.in_workspace ? nullptr : ex->in1.direct;
     a.y = ex->out0.in_workspace ? nullptr : ex->out0.direct;
-    return ACLNN_SUCCESS;
+    return plan_status(ex, "aclnnGridSampler2D");
 }
 
 }  // namespace

@@ -208,6 +208,9 @@ aclnnStatus aclnnGridSampler2DBackwardGetWorkspaceSize(const aclTensor* gradOutp
             ex->workspace_bytes = ex->scratch.ws_offset + (uint64_t)words * 4;
         }
     }
+    if (const aclnnStatus ps = plan_status(ex.get(), "aclnnGridSampler2DBackward"); ps != ACLNN_SUCCESS) {
+        return ps;
+    }
     *workspaceSize = ex->workspace_bytes;
     *executor = ex.release();
     return ACLNN_SUCCESS;

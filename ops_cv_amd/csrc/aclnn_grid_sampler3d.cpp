@@ -189,6 +189,9 @@ aclnnStatus aclnnGridSampler3DGetWorkspaceSize(const aclTensor* input, const acl
     }
     ex->in1 = plan_view(ex.get(), grid, esz, false);
 
+    if (const aclnnStatus ps = plan_status(ex.get(), "aclnnGridSampler3D"); ps != ACLNN_SUCCESS) {
+        return ps;
+    }
     *workspaceSize = ex->workspace_bytes;
     *executor = ex.release();
     return ACLNN_SUCCESS;

@@ -7,6 +7,7 @@
 
 #include "aclnn_grid_sampler3d_backward.h"
 #include "executor.hpp"
+#include "options.hpp"
 #include "kernels.hpp"
 #include "resize_plan.hpp"
 
@@ -193,6 +194,7 @@ aclnnStatus aclnnGridSampler3DBackwardGetWorkspaceSize(const aclTensor* gradOutp
     // (image/grid_sampler3_d_grad/op_host/grid_sampler3_d_grad_tiling.cpp:183-191)
     const int64_t cores = reference_vector_cores();
     a.items_per_core = (a.N > cores) ? (a.N + cores - 1) / cores : 1;
+    a.force_variant = current_options().gs3d_grad_variant;
     const int esz = elem_size(elem);
     // The kernels work on (N,C,D,H,W) operands.  Channels-last tensors are those operands seen through a permuted
     // view, packed (and the gradient scattered) like any other non-contiguous view.
@@ -221,6 +223,9 @@ aclnnStatus aclnnGridSampler3DBackwardGetWorkspaceSize(const aclTensor* gradOutp
                                                                                  (uint64_t)list_words * 4
                                                                            : (uint64_t)range_words * 4);
         }
+    }
+    if (const aclnnStatus ps = plan_status(ex.get(), "aclnnGridSampler3DBackward"); ps != ACLNN_SUCCESS) {
+        return ps;
     }
     *workspaceSize = ex->workspace_bytes;
     *executor = ex.release();

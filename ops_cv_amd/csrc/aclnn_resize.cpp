@@ -136,6 +136,9 @@ aclnnStatus aclnnResizeGetWorkspaceSize(const aclTensor* self, const aclFloatArr
     const int esz = elem_size(elem);
     ex->in0 = plan_view(ex.get(), self, esz, false);
     ex->out0 = plan_view(ex.get(), out, esz, true);
+    if (const aclnnStatus ps = plan_status(ex.get(), "aclnnResize"); ps != ACLNN_SUCCESS) {
+        return ps;
+    }
     *workspaceSize = ex->workspace_bytes;
     *executor = ex.release();
     return ACLNN_SUCCESS;

@@ -161,6 +161,9 @@ aclnnStatus aclnnUpsampleBilinear2dGetWorkspaceSize(const aclTensor* self, const
     ex->in0 = plan_view(ex.get(), self, esz, false);
     ex->out0 = plan_view(ex.get(), out, esz, true);
 
+    if (const aclnnStatus ps = plan_status(ex.get(), "aclnnUpsampleBilinear2d"); ps != ACLNN_SUCCESS) {
+        return ps;
+    }
     *workspaceSize = ex->workspace_bytes;
     *executor = ex.release();
     return ACLNN_SUCCESS;

@@ -172,6 +172,9 @@ aclnnStatus aclnnUpsampleBilinear2dBackwardGetWorkspaceSize(const aclTensor* gra
                         : 0;
     ex->in0 = plan_view(ex.get(), gradOut, elem_size(ein), false);
     ex->out0 = plan_view(ex.get(), out, elem_size(eout), true);
+    if (const aclnnStatus ps = plan_status(ex.get(), "aclnnUpsampleBilinear2dBackward"); ps != ACLNN_SUCCESS) {
+        return ps;
+    }
     *workspaceSize = ex->workspace_bytes;
     *executor = ex.release();
     return ACLNN_SUCCESS;

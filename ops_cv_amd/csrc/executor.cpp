@@ -45,12 +45,19 @@ PlannedPtr plan_view(aclOpExecutor* ex, const aclTensor* t, int elem_bytes, bool
     ex->workspace_bytes = pk.ws_offset + (uint64_t)t->numel() * (uint64_t)elem_bytes;
     p.in_workspace = true;
     p.ws_offset = pk.ws_offset;
-    if (is_output) {
-        ex->unpack_out.push_back(pk);
-    } else {
-        ex->pack_in.push_back(pk);
+    if (!(is_output ? ex->unpack_out.push_back(pk) : ex->pack_in.push_back(pk))) {
+        ex->pack_overflow = true;
     }
     return p;
+}
+
+aclnnStatus plan_status(const aclOpExecutor* ex, const char* api)
+{
+    if (ex->pack_overflow) {
+        set_error("%s: more strided views than the plan can pack", api);
+        return ACLNN_ERR_INNER;
+    }
+    return ACLNN_SUCCESS;
 }
 
 aclnnStatus run_executor(void* workspace, uint64_t workspace_size, aclOpExecutor* ex, aclrtStream stream,
@@ -81,6 +88,12 @@ aclnnStatus run_executor(void* workspace, uint64_t workspace_size, aclOpExecutor
                       (unsigned long long)workspace_size, (unsigned long long)ex->workspace_bytes);
             return ACLNN_ERR_PARAM_INVALID;
         }
+        // the slices handed to the kernels are cut at multiples of 256 bytes from the workspace's start and are read
+        // and written with 16-byte vector accesses and 32-bit atomics
+        if (reinterpret_cast<uintptr_t>(workspace) % kWorkspaceAlignment != 0) {
+            set_error("%s: the workspace must start on a %d-byte boundary", api, (int)kWorkspaceAlignment);
+            return ACLNN_ERR_PARAM_INVALID;
+        }
     }
     return execute_plan(workspace, ex, stream, api);
 }
@@ -89,6 +102,10 @@ aclnnStatus execute_plan(void* workspace, const aclOpExecutor* ex, aclrtStream s
 {
     if (ex->kind == OpKind::Nop) {
         return ACLNN_SUCCESS;
+    }
+    if (ex->pack_overflow) {
+        set_error("%s: more strided views than the plan can pack", api);
+        return ACLNN_ERR_INNER;
     }
     hipStream_t s = (hipStream_t)stream;
     for (const auto& pk : ex->pack_in) {

@@ -17,6 +17,14 @@ namespace opscv {
 PlannedPtr plan_view(aclOpExecutor* ex, const aclTensor* t, int elem_bytes, bool is_output,
                      const int* perm = nullptr);
 
+// alignment the second phase asks of the caller's workspace pointer (hipMalloc returns 256-byte aligned memory; a
+// byte-offset slice of a larger buffer may not be)
+constexpr uintptr_t kWorkspaceAlignment = 16;
+
+// What every first phase returns when planning went wrong inside the library (today: more strided views than the
+// packing lists hold).
+aclnnStatus plan_status(const aclOpExecutor* ex, const char* api);
+
 inline void* resolve(const PlannedPtr& p, void* workspace)
 {
     return p.in_workspace ? (void*)((char*)workspace + p.ws_offset) : p.direct;

@@ -30,6 +30,7 @@
 
 #include "gs3d_grad_math.hpp"
 #include "kernels.hpp"
+#include "options.hpp"
 
 namespace opscv {
 
@@ -415,6 +416,13 @@ __global__ __launch_bounds__(kLThreads) void gs3d_lists_gather_kernel(T* __restr
     }
 }
 
+// profitability limits of the gather variant (see make_plan).  Measured on fp16 volumes, four channels, input gradient
+// and grid gradient together, ordered kernel / gather: 1 voxel per grid point 313 / 97 us (22 x 16x64x64), 4 voxels 83 /
+// 41 us, 16 voxels 35 / 38 us, 32 voxels 35 / 50 us, 128 voxels 56 / 262 us (2 x 128^3), 4096 voxels 80 / 2049 us
+// (256^3 with 4096 points).
+constexpr int64_t kSparseVoxelsPerPoint = 8;
+constexpr int64_t kMaxScratchBytes = (int64_t)1 << 30;
+
 struct Lists3Plan {
     bool ok = false;
     Lists3Layout lay;
@@ -435,9 +443,22 @@ Lists3Plan make_plan(const GridSampler3DGradArgs& a)
         return pl;
     }
     const int64_t groups = (a.C + kChanBlock - 1) / kChanBlock;
-    if (4 + cells * 5 + 2 * kOverflowMax + points * 8 * esz / 4 + groups * points * kChanBlock * esz / 4 + 16 >
-        (int64_t)1 << 31) {
+    const int64_t item_words_estimate =
+        4 + cells * 5 + 2 * kOverflowMax + points * 8 * esz / 4 + groups * points * kChanBlock * esz / 4 + 16;
+    if (item_words_estimate > (int64_t)1 << 31) {
         return pl;  // an item's scratch is indexed in 32 bits
+    }
+    if (a.force_variant == kGs3dGradOrdered) {
+        return pl;
+    }
+    if (a.force_variant != kGs3dGradGather) {
+        // The gather spends a lane, eight cell look-ups and five words of scratch on every voxel whether grid points
+        // fall near it or not, the ordered kernel works per grid point: a volume sampled at few points (below one
+        // point per kSparseVoxelsPerPoint voxels) stays with the ordered kernel, and so does a call whose scratch
+        // would pass kMaxScratchBytes.
+        if (points * kSparseVoxelsPerPoint < vol || item_words_estimate * 4 * a.N > kMaxScratchBytes) {
+            return pl;
+        }
     }
     pl.cells = cells;
     pl.lay = make_layout(cells, points, esz, a.C);

@@ -19,6 +19,7 @@ struct Store {
     // the unified buffer of the reference's tiling unit test (test_resize_nearest_neighbor_v2_tiling.cpp: {64, 253952})
     std::atomic<int64_t> reference_ub_bytes{253952};
     std::atomic<int64_t> grid_sampler2d_rule{kRuleGridSampler2D};
+    std::atomic<int64_t> gs3d_grad_variant{kGs3dGradAuto};
 };
 
 long long positive_env(const char* name)
@@ -54,6 +55,9 @@ Store& store()
         if (const long long n = positive_env("OPSCV_REFERENCE_UB_BYTES")) {
             s.reference_ub_bytes = n;
         }
+        if (const char* v = getenv("OPSCV_GS3D_GRAD_VARIANT")) {
+            s.gs3d_grad_variant = (v[0] == 'o') ? kGs3dGradOrdered : (v[0] == 'g' ? kGs3dGradGather : kGs3dGradAuto);
+        }
         if (const char* v = getenv("OPSCV_GRID_SAMPLER2D_RULE")) {
             s.grid_sampler2d_rule = (strcmp(v, "arch35") == 0 || strcmp(v, "1") == 0) ? kRuleGridSampleArch35
                                                                                        : kRuleGridSampler2D;
@@ -75,6 +79,7 @@ const Entry kEntries[] = {
     {"reference_cores", &Store::reference_cores, 1, INT64_MAX},
     {"reference_ub_bytes", &Store::reference_ub_bytes, 1, INT64_MAX},
     {"grid_sampler2d_rule", &Store::grid_sampler2d_rule, kRuleGridSampler2D, kRuleGridSampleArch35},
+    {"gs3d_grad_variant", &Store::gs3d_grad_variant, kGs3dGradAuto, kGs3dGradGather},
 };
 
 const Entry* find(const char* name)
@@ -102,6 +107,7 @@ Options current_options()
     o.reference_cores = s.reference_cores.load(std::memory_order_relaxed);
     o.reference_ub_bytes = s.reference_ub_bytes.load(std::memory_order_relaxed);
     o.grid_sampler2d_rule = (int32_t)s.grid_sampler2d_rule.load(std::memory_order_relaxed);
+    o.gs3d_grad_variant = (int32_t)s.gs3d_grad_variant.load(std::memory_order_relaxed);
     return o;
 }
 

@@ -36,7 +36,7 @@ def device():
 
 
 OPTION_NAMES = ("gs_variant", "resize_variant", "nearest_variant", "reference_cores", "reference_ub_bytes",
-                "grid_sampler2d_rule")
+                "grid_sampler2d_rule", "gs3d_grad_variant")
 
 
 @pytest.fixture(autouse=True)

@@ -607,7 +607,10 @@ def test_grid_sampler3d_backward_status_codes(aclnn, desc):
     assert _gsb3(aclnn, desc, interp=1, **big)[:2] == (0, 3 * 3 * 2 * 4)
     cells, points = 11 * 31 * 31, 600
     per_item = ((4 + cells + 3) // 4 * 4 + 4 * cells + 2048) * 4 + points * 8 * 4 + points * 4 * 4
-    assert _gsb3(aclnn, desc, **big) == (0, 256 + 3 * per_item, "gs3d_grad_lists")
+    # (fifteen voxels per grid point: the ordered kernel by itself, the gather when asked for)
+    assert _gsb3(aclnn, desc, **big) == (0, 3 * 3 * 2 * 4, "gs3d_grad_ordered")
+    with aclnn.option("gs3d_grad_variant", 2):
+        assert _gsb3(aclnn, desc, **big) == (0, 256 + 3 * per_item, "gs3d_grad_lists")
     assert _gsb3(aclnn, desc, mask=(False, True), **big)[:2] == (0, 0)
 
 
@@ -629,7 +632,7 @@ def test_options_api_and_rule_captured_at_phase_one(aclnn):
     """opscvSetOption / opscvGetOption: names, ranges, defaults; the bilinear coordinate rule goes into the executor at
     phase 1 (the variant name of a shape beyond LDS shows it) and applies to the bilinear mode only"""
     defaults = {"gs_variant": 0, "resize_variant": 0, "nearest_variant": 0, "reference_cores": 64,
-                "reference_ub_bytes": 253952, "grid_sampler2d_rule": 0}
+                "reference_ub_bytes": 253952, "grid_sampler2d_rule": 0, "gs3d_grad_variant": 0}
     for name, value in defaults.items():
         assert aclnn.get_option(name) == value, name
     L = aclnn.load_library()
@@ -659,3 +662,63 @@ def test_options_api_and_rule_captured_at_phase_one(aclnn):
     with aclnn.option("gs_variant", 1):
         assert aclnn.get_option("gs_variant") == 1
     assert aclnn.get_option("gs_variant") == 0
+
+
+def test_grid_sampler3d_backward_gather_variant_is_gated_on_point_density(aclnn):
+    """the gather variant of the 3-D sampler's input gradient pays per voxel, the ordered kernel per grid point: phase 1
+    takes the gather (and its scratch) only up to eight voxels per grid point, and option gs3d_grad_variant overrides"""
+    f16 = aclnn.ACL_FLOAT16
+
+    def plan(vol, pts, N=2, C=4):
+        D, H, W = vol
+        Do, Ho, Wo = pts
+        hs = [aclnn.create_tensor((N, C, Do, Ho, Wo), f16, aclnn.ACL_FORMAT_NCDHW),
+              aclnn.create_tensor((N, C, D, H, W), f16, aclnn.ACL_FORMAT_NCDHW),
+              aclnn.create_tensor((N, Do, Ho, Wo, 3), f16),
+              aclnn.create_tensor((N, C, D, H, W), f16, aclnn.ACL_FORMAT_NCDHW),
+              aclnn.create_tensor((N, Do, Ho, Wo, 3), f16)]
+        mask = aclnn.create_bool_array([True, True])
+        st, ws, ex = aclnn.get_workspace_size_grid_sampler3d_backward(hs[0], hs[1], hs[2], 0, 0, False, mask, hs[3],
+                                                                      hs[4])
+        assert st == 0
+        v = aclnn.executor_variant(ex)
+        aclnn.destroy_executor(ex)
+        for h in hs:
+            aclnn.destroy_tensor(h)
+        aclnn.destroy_bool_array(mask)
+        return v, ws
+
+    dense = plan((16, 32, 32), (16, 32, 32))        # one voxel per point
+    edge_in = plan((16, 32, 32), (4, 16, 32))       # eight voxels per point: still the gather
+    edge_out = plan((16, 32, 32), (4, 16, 31))      # a little over eight
+    sparse = plan((64, 64, 64), (4, 16, 16))        # 256 voxels per point
+    assert dense[0] == "gs3d_grad_lists" and edge_in[0] == "gs3d_grad_lists"
+    assert edge_out[0] == "gs3d_grad_ordered" and sparse[0] == "gs3d_grad_ordered"
+    # the ordered kernel asks for the chunk spans only: kilobytes, where the gather of the sparse case would want
+    # five words per lattice cell (several megabytes per batch item)
+    assert sparse[1] < 64 * 1024 < (1 << 20) < plan((16, 64, 64), (16, 64, 64))[1]
+    with aclnn.option("gs3d_grad_variant", 1):
+        assert plan((16, 32, 32), (16, 32, 32))[0] == "gs3d_grad_ordered"
+    with aclnn.option("gs3d_grad_variant", 2):
+        forced = plan((64, 64, 64), (4, 16, 16))
+        assert forced[0] == "gs3d_grad_lists" and forced[1] > 5 * 4 * 65 ** 3
+
+
+def test_second_phase_refuses_a_misaligned_workspace(aclnn):
+    """the kernels read and write their workspace slices with 16-byte accesses and 32-bit atomics: a workspace that
+    does not start on a 16-byte boundary is refused before anything is launched (and the executor is consumed)"""
+    import ctypes
+    f32 = aclnn.ACL_FLOAT
+    L = aclnn.load_library()
+    # a transposed input view needs packing, hence a workspace
+    hs = [aclnn.create_tensor((1, 2, 4, 6), f32, strides=(48, 24, 1, 4)), aclnn.create_tensor((1, 3, 3, 2), f32),
+          aclnn.create_tensor((1, 2, 3, 3), f32)]
+    st, ws, ex = aclnn.get_workspace_size_grid_sampler2d(hs[0], hs[1], 0, 0, False, hs[2])
+    assert st == 0 and ws >= 48 * 4
+    assert L.aclnnGridSampler2D(ctypes.c_void_p(0x7f0000001008), ws, ex, None) == 161002
+    assert b"16-byte boundary" in L.aclGetRecentErrMsg()
+    # the executor is gone: a second use is refused as not live
+    st, ws, ex = aclnn.get_workspace_size_grid_sampler2d(hs[0], hs[1], 0, 0, False, hs[2])
+    assert L.aclnnGridSampler2D(None, ws, ex, None) == 161001
+    for h in hs:
+        aclnn.destroy_tensor(h)

@@ -786,6 +786,34 @@ def test_grid_sampler3d_backward_gather_variant(oracle, device, aclnn, dtype, mo
     assert seen_gathered > 0 and seen_flagged > 0
 
 
+def test_grid_sampler3d_backward_sparse_volume_takes_the_ordered_kernel(oracle, device, aclnn):
+    """a volume sampled at few points (more than eight voxels per grid point) stays with the ordered kernel; forced
+    either way the two variants give the oracle's bits"""
+    torch = _torch()
+    rng = np.random.default_rng(733)
+    N, C, (D, H, W), (Do, Ho, Wo) = 2, 5, (12, 20, 24), (3, 9, 10)
+    x = rng.standard_normal((N, C, D, H, W)).astype(np.float16)
+    g = rng.uniform(-1.05, 1.05, (N, Do, Ho, Wo, 3)).astype(np.float16)
+    go = rng.standard_normal((N, C, Do, Ho, Wo)).astype(np.float16)
+    rdx, rdg = oracle.grid_sampler3d_backward(go, x, g, 0, 0, False)
+    xt, gt, got = (torch.from_numpy(a).to(device) for a in (x, g, go))
+    hs = [aclnn.tensor_handle(t, aclnn.ACL_FORMAT_NCDHW) for t in (got, xt)] + [aclnn.tensor_handle(gt)]
+    hs += [aclnn.tensor_handle(torch.empty_like(xt), aclnn.ACL_FORMAT_NCDHW), aclnn.tensor_handle(torch.empty_like(gt))]
+    mask = aclnn.create_bool_array([True, True])
+    st, _, ex = aclnn.get_workspace_size_grid_sampler3d_backward(hs[0], hs[1], hs[2], 0, 0, False, mask, hs[3], hs[4])
+    assert st == 0 and aclnn.executor_variant(ex) == "gs3d_grad_ordered"
+    aclnn.destroy_executor(ex)
+    for h in hs:
+        aclnn.destroy_tensor(h)
+    aclnn.destroy_bool_array(mask)
+    for forced in (0, 1, 2):
+        with aclnn.option("gs3d_grad_variant", forced):
+            dx, dg = aclnn.grid_sampler3d_backward(got, xt, gt, 0, 0, False)
+        torch.cuda.synchronize()
+        assert np.array_equal(dx.cpu().numpy().view(np.uint16), rdx.view(np.uint16)), forced
+        assert np.array_equal(dg.cpu().numpy().view(np.uint16), rdg.view(np.uint16)), forced
+
+
 def test_grid_sampler3d_backward_core_split_mask_layouts_and_torch(oracle, device, aclnn, monkeypatch):
     torch = _torch()
     import torch.nn.functional as F

@@ -92,3 +92,41 @@ def test_no_alloc_rejects_what_does_not_fit_and_bad_arguments(device, aclnn):
     h = aclnn.tensor_handle(x)
     assert L.opscvGridSampler2DNoAlloc(h, None, 0, 0, False, h, None) == aclnn.ACLNN_ERR_PARAM_NULLPTR
     aclnn.destroy_tensor(h)
+
+
+def test_no_alloc_in_a_graph_on_strided_views(device, aclnn):
+    """The entry point under stream capture, after one warm call on the device (which looks up the static array and
+    sets kernel attributes): the recorded graph packs the strided views into the static array, samples and scatters
+    the result into a window; every replay on new data equals the two-phase call on the same views."""
+    import torch
+    rng = np.random.default_rng(79)
+    shape = (2, 19, 23, 30, 17, 21)
+    N, C, H, W, Ho, Wo = shape
+    for dtype in ("fp16", "fp32"):
+        xt, gv = _views(torch, device, dtype, rng, *shape)
+        x_store, g_store = xt.transpose(2, 3), gv  # x_store is the dense buffer behind the transposed view
+        big = torch.full((N, C, Ho, Wo + 4), 3.0, dtype=xt.dtype, device=device)
+        win = big[:, :, :, 2:2 + Wo]
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            assert aclnn.grid_sampler2d_noalloc(xt, gv, win, 0, 0, False) == 0  # the warm call
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            st = aclnn.grid_sampler2d_noalloc(xt, gv, win, 0, 0, False)
+        assert st == 0, aclnn.load_library().aclGetRecentErrMsg()
+        for r in range(3):
+            x_new, g_new = _views(torch, device, dtype, rng, *shape)
+            x_store.copy_(x_new.transpose(2, 3))
+            g_store.copy_(g_new)
+            big.fill_(3.0)
+            graph.replay()
+            torch.cuda.synchronize()
+            want = aclnn.grid_sampler2d(x_new, g_new, 0, 0, False)
+            torch.cuda.synchronize()
+            got = I.from_torch(win.contiguous(), dtype).view(np.uint8)
+            assert np.array_equal(got, I.from_torch(want, dtype).view(np.uint8)), (dtype, r)
+            edge = I.as_f32(I.from_torch(big, dtype), dtype)
+            assert (edge[..., :2] == 3.0).all() and (edge[..., 2 + Wo:] == 3.0).all()
