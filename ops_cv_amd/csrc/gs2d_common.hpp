@@ -78,6 +78,9 @@ const char* gs2d_lds_variant_name(const GridSamplerArgs& a);
 // convention as run_gs2d_lds.
 hipError_t run_gs2d_pair(const GridSamplerArgs& a, hipStream_t stream, bool* handled);
 const char* gs2d_pair_variant_name(const GridSamplerArgs& a);
+// ... and its bicubic counterpart (gs2d_bicubic_pair.hip); both are reached through the two functions above
+hipError_t run_gs2d_bicubic_pair(const GridSamplerArgs& a, hipStream_t stream, bool* handled);
+const char* gs2d_bicubic_pair_variant_name(const GridSamplerArgs& a);
 
 // Box variant (gs2d_box.hip): bilinear, 16-bit elements, planes beyond the LDS variants; the box of input pixels that a
 // tile of output pixels reads goes through LDS.  Same convention as run_gs2d_lds.

@@ -121,6 +121,9 @@ struct PairLauncher {
 
 const char* gs2d_pair_variant_name(const GridSamplerArgs& a)
 {
+    if (a.interp == 2) {
+        return gs2d_bicubic_pair_variant_name(a);
+    }
     const PairPlan p = make_pair_plan(a);
     if (!p.ok) {
         return nullptr;
@@ -131,6 +134,9 @@ const char* gs2d_pair_variant_name(const GridSamplerArgs& a)
 
 hipError_t run_gs2d_pair(const GridSamplerArgs& a, hipStream_t stream, bool* handled)
 {
+    if (a.interp == 2) {
+        return run_gs2d_bicubic_pair(a, stream, handled);
+    }
     *handled = false;
     const PairPlan p = make_pair_plan(a);
     if (!p.ok) {

@@ -132,6 +132,51 @@ def test_grid_sampler_pair_layout_variant(oracle, device, dtype, pad, align, mon
         _assert_same_bits(y_ring, y_ref, what + " (ring kernel)")
 
 
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("pad", [0, 1])
+@pytest.mark.parametrize("align", [False, True])
+def test_grid_sampler_bicubic_pair_layout_variant(oracle, device, dtype, pad, align):
+    """the bicubic pair-layout kernel (16-bit elements, zeros and border padding): every staged row length class and
+    every loader class (one, two, five runs per lane), row counts off the loader's blocks of sixteen, a ragged last
+    pixel tile, one and many channels per workgroup, coordinates outside the image on every side (where the padding
+    entries at the row ends and the row of zeros are read), huge and non-finite ones; bit for bit against the oracle
+    and against the ring kernel"""
+    import torch
+    from ops_cv_amd import aclnn
+    rng = np.random.default_rng(1900 + pad * 10 + int(align))
+    for (N, C, H, W, Ho, Wo) in [(2, 9, 40, 32, 47, 48), (16, 3, 64, 64, 64, 64), (2, 8, 21, 96, 60, 62),
+                                 (1, 5, 100, 64, 90, 92), (1, 12, 128, 128, 130, 134), (1, 1, 5, 128, 32, 34)]:
+        x32 = rng.standard_normal((N, C, H, W)).astype(np.float32)
+        x32[0, 0, 0, :] = 3.0e4  # large values on the image border: a tap wrongly taken from outside would show
+        x32[0, 0, :, 0] = -2.0e4
+        x32[0, 0, :, W - 1] = 1.0e4
+        g32 = rng.uniform(-1.5, 1.5, (N, Ho, Wo, 2)).astype(np.float32)
+        sv = I.special_grid_values()
+        k = min(sv.size, Wo)
+        g32[0, 0, :k, 0] = sv[:k]
+        g32[0, 1, :k, 1] = sv[:k]
+        g32[0, 2, :k, 0] = sv[:k]
+        g32[0, 2, :k, 1] = sv[:k][::-1]
+        x, g = I.cast_np(x32, dtype), I.cast_np(g32, dtype)
+        xt, gt = I.to_torch(x, dtype, device), I.to_torch(g, dtype, device)
+        out = torch.empty((N, C, Ho, Wo), dtype=xt.dtype, device=device)
+        hs = [aclnn.tensor_handle(t) for t in (xt, gt, out)]
+        st, _, ex = aclnn.get_workspace_size_grid_sampler2d(hs[0], hs[1], 2, pad, align, hs[2])
+        assert st == 0
+        assert aclnn.executor_variant(ex).startswith("lds_pair_bicubic_w"), aclnn.executor_variant(ex)
+        aclnn.destroy_executor(ex)
+        for h in hs:
+            aclnn.destroy_tensor(h)
+        y_ref = oracle.grid_sampler2d(x, g, 2, pad, align, dtype=I.oracle_code(dtype))
+        y = I.from_torch(aclnn.grid_sampler2d(xt, gt, 2, pad, align, out=out), dtype)
+        what = "gs-bicubic-pair %s %s align=%s %s" % (dtype, PAD[pad], align, (N, C, H, W, Ho, Wo))
+        _check(y, y_ref, dtype, 2, what)
+        _assert_same_bits(y, y_ref, what)
+        with aclnn.option("gs_variant", 2):  # the pair-layout variants kept out
+            y_ring = I.from_torch(aclnn.grid_sampler2d(xt, gt, 2, pad, align), dtype)
+        _assert_same_bits(y, y_ring, what + " (against the ring kernel)")
+
+
 @pytest.mark.parametrize("dtype", I.DTYPES)
 @pytest.mark.parametrize("interp", [0, 1, 2])
 @pytest.mark.parametrize("pad", [0, 1, 2])
