@@ -111,11 +111,10 @@ LdsPlan make_lds_plan(const GridSamplerArgs& a)
     p.copy_gran = plain ? 16 : 2;  // 2: 16-byte units in the shifted layout
     // Bank-spreading layout (gs2d_lds_kernel.hpp): rows of exactly 128 bytes, 16-byte copy granule.  Only for
     // border padding, where clamped coordinates pile up on the first and last column (one bank in the plain
-    // layout: 21.2 -> 18.7 us on the fp16 N16 C256 64x64 case).  Elsewhere the plain layout is the better one: the
-    // bank then depends on x alone and the lanes of a wavefront have different x (zeros padding on the same case:
-    // 17.7 us plain, 18.5 us permuted).
+    // layout).  Elsewhere the plain layout is the better one: the bank then depends on x alone and the lanes of a
+    // wavefront have different x.
     if (a.pad == 1 && p.copy_gran == 16 && a.Win * esz == 128) {
-        p.row_shift = 7;
+        p.row_shift = 7 | (2 << 8);  // rows of 128 bytes, rotated by two chunks per row
     }
     // all tiles of one (n, channel block) group on one XCD: needs the group count to be a multiple of 8
     p.xcd_swizzle = ((a.N * cblocks) % 8 == 0) ? 1 : 0;

@@ -276,14 +276,18 @@ __device__ __forceinline__ void lds_barrier()
     asm volatile("" ::: "memory");
 }
 
-// Bank-spreading layout of a staged plane whose rows are exactly 128 bytes (row_shift = 7; 0 = plain layout).
-// LDS has 32 four-byte banks, i.e. 128 bytes per "line"; with that row pitch column x of every row falls into the
-// same bank, and coordinates clamped to the first or last column (border padding) make a wavefront read one bank
-// 64 times.  The 16-byte chunks of each line are therefore permuted by the low three bits of the row number:
-// byte offset o of the plane lives at o ^ ((row & 7) << 4).  The permutation stays inside the line, so it maps the
-// plane onto itself.  The copy applies it to the source address (the LDS side of the asynchronous copy is fixed per
-// lane); a copy instruction covers eight whole rows starting at a multiple of 1 KiB, so the permuted source offset
-// of a lane inside that block is a per-lane constant.  The samplers apply it once per tap when they compute offsets.
+// Bank-spreading layout of a staged plane whose rows are exactly 128 bytes (row_shift = 7 | turn << 8; 0 = plain
+// layout).  LDS has 32 four-byte banks, i.e. 128 bytes per "line"; with that row pitch column x of every row falls into
+// the same bank, and coordinates clamped to the first or last column (border padding) make a wavefront read one bank
+// 64 times.  The eight 16-byte chunks of each line are therefore rotated by `turn` chunks per row: byte offset o of the
+// plane lives in chunk (chunk(o) + turn * row) mod 8 of its line, which shifts consecutive rows by 4 * turn banks
+// (fp16 N16 C256 64x64, border: plain layout 21.2 us; chunks permuted by row & 7 instead 16.1 us; turn 2: 14.9, 4: 15.1,
+// 6: 15.0, 7: 19.2).  The rotation stays inside the line, so it maps the plane onto itself.  The copy applies its
+// inverse to the source address (the LDS side of the asynchronous copy is fixed per lane); a copy instruction covers
+// eight whole rows starting at a multiple of 1 KiB, so the source offset of a lane inside that block is a per-lane
+// constant.  The samplers apply it once per tap when they compute offsets.  Where the lanes of a wavefront already
+// read different columns (zeros and reflection padding with two neighbouring pixels per lane) any shift between rows
+// makes them meet more often: 13.1 us plain, 20 to 24 us rotated.
 // Division of a block index by a launch constant without the hardware's reciprocal sequence (a dependent chain of
 // conversions and a reciprocal that every wavefront of the kernel would walk before it knows its work): the host hands
 // over m = ceil(2^s / d), s = 31 + ceil(log2 d), and floor(x / d) = (x * m) >> s for every x < 2^31.
@@ -313,7 +317,22 @@ __device__ __forceinline__ uint32_t fast_div(uint32_t x, const FastDiv& f)
 
 __device__ __forceinline__ uint32_t lds_swizzle(uint32_t byte_off, uint32_t row_shift)
 {
-    return row_shift ? (byte_off ^ (((byte_off >> row_shift) & 7u) << 4)) : byte_off;
+    if (row_shift == 0u) {
+        return byte_off;
+    }
+    const uint32_t turn = row_shift >> 8, row = byte_off >> 7;
+    return (byte_off & ~0x70u) | ((((byte_off >> 4) + turn * row) & 7u) << 4);
+}
+
+// The chunk of a 1 KiB block (eight rows starting at a multiple of eight) that belongs at LDS position `byte_off` of
+// the block: the inverse of lds_swizzle.
+__device__ __forceinline__ uint32_t lds_unswizzle(uint32_t byte_off, uint32_t row_shift)
+{
+    if (row_shift == 0u) {
+        return byte_off;
+    }
+    const uint32_t turn = row_shift >> 8, row = byte_off >> 7;
+    return (byte_off & ~0x70u) | ((((byte_off >> 4) - turn * row) & 7u) << 4);
 }
 
 // Starts the asynchronous copy of `nch` consecutive input planes (plane_bytes each, contiguous in global memory
@@ -613,7 +632,7 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
             }
             return total;
         };
-        const uint32_t lane_src16 = lds_swizzle(lane * 16u, (uint32_t)row_shift);
+        const uint32_t lane_src16 = lds_unswizzle(lane * 16u, (uint32_t)row_shift);
         auto start_stage = [&](int32_t s, int slot) {
             const char* src = xb + (size_t)s * stage_bytes;
             char* dst = lds + slot * SLOT_BYTES;

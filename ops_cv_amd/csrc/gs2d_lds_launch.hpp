@@ -17,7 +17,7 @@ struct LdsPlan {
     int adj = 1;  // neighbouring output pixels per store (2: pairs of 16-bit results as one dword)
     int copy_gran = 16;
     int xcd_swizzle = 0;
-    int row_shift = 0;  // 7 when the staged planes (128-byte rows) use the bank-spreading layout, else 0
+    int row_shift = 0;  // 7 | turn << 8 when the staged planes (128-byte rows) use the bank-spreading layout, else 0
     uint32_t lds_bytes = 0;
     uint32_t tiles_per_n = 0, cblocks = 0;
     int32_t chans_per_block = 0;
