@@ -399,7 +399,12 @@ struct Fold {
     {
         return rt<T>(acc + rt<T>(as_fp32_value(w * tap_value<T>(go_bits))));
     }
-    static __device__ __forceinline__ void store(T* p, acc_t acc) { ElemIO<T>::store(p, acc); }
+    static __device__ __forceinline__ void store(T* p, acc_t acc)
+    {
+        T v;
+        ElemIO<T>::store(&v, acc);
+        __builtin_nontemporal_store(v, p);  // the gradient streams out: written once, not read again by this kernel
+    }
 };
 template <>
 struct Fold<_Float16> {
@@ -411,7 +416,7 @@ struct Fold<_Float16> {
         const _Float16 val = w * __builtin_bit_cast(_Float16, (uint16_t)go_bits);
         return acc + val;
     }
-    static __device__ __forceinline__ void store(_Float16* p, acc_t acc) { *p = acc; }
+    static __device__ __forceinline__ void store(_Float16* p, acc_t acc) { __builtin_nontemporal_store(acc, p); }
     // two channels at once: the same two operations as packed fp16 instructions (each half rounds on its own)
     typedef _Float16 pair_t __attribute__((ext_vector_type(2)));
     static __device__ __forceinline__ pair_t add2(pair_t acc, uint32_t go_lo, uint32_t go_hi, acc_t w)

@@ -218,7 +218,7 @@ struct Fold3 {
     {
         return rt<T>(acc + contribution3<T, 0>(ElemIO<T>::load(&go), ElemIO<T>::load(&w)));
     }
-    static __device__ __forceinline__ void store(T* p, acc_t acc) { ElemIO<T>::store(p, acc); }
+    static __device__ __forceinline__ void store(T* p, acc_t acc) { store_streaming<T>(p, acc); }
 };
 template <>
 struct Fold3<_Float16> {
@@ -229,7 +229,7 @@ struct Fold3<_Float16> {
         const _Float16 val = w * go;
         return acc + val;
     }
-    static __device__ __forceinline__ void store(_Float16* p, acc_t acc) { *p = acc; }
+    static __device__ __forceinline__ void store(_Float16* p, acc_t acc) { __builtin_nontemporal_store(acc, p); }
 };
 
 // The first NK entries of a lane's list (every kLThreads-th word from `mine`), sorted ascending through registers.

@@ -475,7 +475,7 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
                         acc = (nx_min >= 4) ? OPSCV_TILE_SUM(6, 4) : OPSCV_TILE_SUM(6, 0);
                     }
 #undef OPSCV_TILE_SUM
-                    ElemIO<TO>::store(yp + (int64_t)q * kTileGroups * Wse, acc);
+                    store_streaming<TO>(yp + (int64_t)q * kTileGroups * Wse, acc);
                 }
             };
             static_assert(HQ == 4, "one call per outgoing row of a lane");
@@ -508,7 +508,7 @@ __global__ __launch_bounds__(kGradThreads) void resize_grad_lds_kernel(const TI*
                                         scale_h, scale_w, last_y, last_x, Hd, Wd, ci, ch);
                 }
 #undef OPSCV_VISIT
-                ElemIO<TO>::store(y + (pl * Hs + H) * (int64_t)Wse + W, acc);
+                store_streaming<TO>(y + (pl * Hs + H) * (int64_t)Wse + W, acc);
             }
         }
         if (use_lds) {
