@@ -46,7 +46,11 @@ MEASURED_TRAFFIC = {
 # the type the arithmetic runs in, per workload: every kernel of this path converts its 16-bit elements to fp32,
 # computes in fp32 (products and sums rounded separately, as the reference does) and rounds once on the way out
 ARITHMETIC = {"C1": "f32", "C2": "f32", "C3": "f32", "C4": "f32", "C5": "f32", "L1": "f32", "V1": "f32", "V1cl": "f32",
-              "G3": "f32", "W1": "f32", "B4": "f32", "R4": "f32"}
+              "G3": "f32", "W1": "f32", "W1s": "f32", "B4": "f32", "R4": "f32"}
+
+# few grid points in a large volume (128 voxels a point): the input gradient of the 3-D sampler keeps its ordered kernel
+# here (the gather variant walks every voxel's cells and is 4 to 25 times slower on such shapes)
+W1_SPARSE = dict(shape=(4, 4, 64, 128, 128), points=(8, 32, 32), label="W1s")
 
 MIN_TIMED_LAUNCHES = 50  # floor for the secondary workloads, whatever --steps says for the headline
 
@@ -438,9 +442,10 @@ def bench_gs3d(steps, warmup, sets=4, channels_last=False):
                 parity=parity, sets=sets, default_modes=True)
 
 
-def bench_gs3d_backward(steps, warmup, sets=2, mask=(True, True)):
+def bench_gs3d_backward(steps, warmup, sets=2, mask=(True, True), shape=(22, 4, 16, 64, 64), points=None, label="W1"):
     """Backward of the volumetric workload (fp16 22 x 4 x 16 x 64 x 64, the same registration-style warp): both
-    gradients."""
+    gradients.  `points` (Do, Ho, Wo): a grid coarser than the volume (W1s: few points in a large volume, where the
+    library keeps its ordered kernel for the input gradient)."""
     import numpy as np
     import torch
     import inputs as I
@@ -448,19 +453,20 @@ def bench_gs3d_backward(steps, warmup, sets=2, mask=(True, True)):
     from ops_cv_amd import aclnn
     dev = torch.device("cuda:0")
     L = load_bench_lib()
-    N, C, D, H, W = 22, 4, 16, 64, 64
+    N, C, D, H, W = shape
+    Do, Ho, Wo = points if points is not None else (D, H, W)
     dtype = "fp16"
     ts, hs = [[] for _ in range(5)], [[] for _ in range(5)]
     first = None
     for s in range(sets):
         rng = np.random.default_rng(3100 + s)
         x = I.cast_np(rng.standard_normal((N, C, D, H, W)).astype(np.float32), dtype)
-        ax = [np.linspace(-1, 1, n, dtype=np.float32) for n in (D, H, W)]
+        ax = [np.linspace(-1, 1, n, dtype=np.float32) for n in (Do, Ho, Wo)]
         gz, gy, gx = np.meshgrid(*ax, indexing="ij")
         base = np.stack([gx, gy, gz], -1)[None]
         g = base * rng.uniform(0.9, 1.1, (N, 1, 1, 1, 3)) + rng.uniform(-0.1, 0.1, (N, 1, 1, 1, 3))
         g = I.cast_np((g + rng.normal(0, 0.01, g.shape)).astype(np.float32), dtype)
-        go = I.cast_np(rng.standard_normal((N, C, D, H, W)).astype(np.float32), dtype)
+        go = I.cast_np(rng.standard_normal((N, C, Do, Ho, Wo)).astype(np.float32), dtype)
         if s == 0:
             first = (go, x, g)
         tens = [I.to_torch(go, dtype, dev), I.to_torch(x, dtype, dev), I.to_torch(g, dtype, dev)]
@@ -499,10 +505,11 @@ def bench_gs3d_backward(steps, warmup, sets=2, mask=(True, True)):
     aclnn.destroy_bool_array(m)
     e = esize(dtype)
     # gradOutput read by both gradients' kernels, input read once, grid read twice, both gradients written
-    alg = (2 * N * C * D * H * W + 2 * N * C * D * H * W + 3 * N * D * H * W * 3) * e
-    return dict(steps=steps, workload="W1 grid_sampler3d_backward fp16 x(22,4,16,64,64) grid(22,16,64,64,3) bilinear zeros "
-                         "align_corners=False both gradients", samples=N * C * D * H * W, alg_bytes=alg, timed=t,
-                variant=variant, parity=parity, sets=sets, default_modes=True)
+    alg = (2 * N * C * Do * Ho * Wo + 2 * N * C * D * H * W + 3 * N * Do * Ho * Wo * 3) * e
+    return dict(steps=steps, workload="%s grid_sampler3d_backward fp16 x(%d,%d,%d,%d,%d) grid(%d,%d,%d,%d,3) bilinear zeros "
+                         "align_corners=False both gradients" % (label, N, C, D, H, W, N, Do, Ho, Wo),
+                samples=N * C * Do * Ho * Wo, alg_bytes=alg, timed=t, variant=variant, parity=parity, sets=sets,
+                default_modes=True)
 
 
 def bench_gs_backward(steps, warmup, sets=4, mask=(True, True)):
@@ -713,7 +720,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="C3", help="headline workload: C1..C5, L1 (sampler on 1080p planes), or one of the neighbouring entry points V1 (3-D sampler), G3 "
-                         "(sampler backward), W1 (3-D sampler backward), B4 (resize backward), R4 (nearest resize)")
+                         "(sampler backward), W1 (3-D sampler backward; W1s: few points in a large volume), B4 (resize backward), R4 (nearest resize)")
     ap.add_argument("--only", action="store_true", help="skip the other workloads and the CPU baseline")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -760,6 +767,8 @@ def main():
         r = bench_gs_backward(args.steps, args.warmup)
     elif head == "W1":
         r = bench_gs3d_backward(args.steps, args.warmup)
+    elif head == "W1s":
+        r = bench_gs3d_backward(args.steps, args.warmup, **W1_SPARSE)
     elif head == "B4":
         r = bench_resize_like("backward", args.steps, args.warmup)
     elif head == "R4":
@@ -835,6 +844,8 @@ def main():
         others["V1_grid_sampler3d_ndhwc"] = summary_of(bench_gs3d(ko, args.warmup, channels_last=True))
         others["G3_grid_sampler2d_backward"] = summary_of(bench_gs_backward(ko, args.warmup))
         others["W1_grid_sampler3d_backward"] = summary_of(bench_gs3d_backward(ko, args.warmup))
+        others["W1s_grid_sampler3d_backward_sparse_volume"] = summary_of(bench_gs3d_backward(min(ko, 50), min(args.warmup, 5),
+                                                                                           **W1_SPARSE))
         others["B4_upsample_backward"] = summary_of(bench_resize_like("backward", ko, args.warmup))
         others["R4_resize_nearest"] = summary_of(bench_resize_like("nearest", ko, args.warmup))
         line["other_workloads"] = others
