@@ -77,10 +77,10 @@ PairPlan make_pair_plan(const GridSamplerArgs& a)
     return p;
 }
 
-template <typename T, int P, bool A, int PITCH>
+template <typename T, int PITCH>
 hipError_t pair_launch_one(const GridSamplerArgs& a, const PairPlan& p, hipStream_t stream)
 {
-    auto kernel = gs2d_pair_kernel<T, P, A, kPairSamplerWaves, kPairLoaderWaves, kPairPpt, PITCH, kPairRmax>;
+    auto kernel = gs2d_pair_kernel<T, kPairSamplerWaves, kPairLoaderWaves, kPairPpt, PITCH, kPairRmax>;
     static std::atomic<uint32_t> lds_allowed{0};
     const hipError_t ea = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kLdsLimit, lds_allowed);
     if (ea != hipSuccess) {
@@ -91,31 +91,21 @@ hipError_t pair_launch_one(const GridSamplerArgs& a, const PairPlan& p, hipStrea
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3((kPairSamplerWaves + kPairLoaderWaves) * 64), p.lds_bytes, stream,
                        (const T*)a.x, (const T*)a.grid, (T*)a.y, make_fast_div((uint32_t)a.N), (int32_t)a.C,
                        (int32_t)a.Hin, (int32_t)a.Win, (int32_t)(a.Hout * a.Wout), make_fast_div(p.tiles_per_n),
-                       p.chans_per_block, pair_aligned, p.xcd_swizzle, -0.0f);
+                       p.chans_per_block, pair_aligned, p.xcd_swizzle, (int32_t)a.pad, (int32_t)(a.align != 0), -0.0f);
     return hipGetLastError();
 }
 
 template <typename T>
-struct PairLauncher {
-    const GridSamplerArgs& a;
-    const PairPlan& p;
-    hipStream_t stream;
-    template <typename U, int I, int P, bool A>
-    hipError_t operator()() const
-    {
-        if constexpr (I != 0) {
-            return hipErrorInvalidValue;
-        } else {
-            switch (p.cls) {
-                case 0: return pair_launch_one<T, P, A, kPairPitches[0]>(a, p, stream);
-                case 1: return pair_launch_one<T, P, A, kPairPitches[1]>(a, p, stream);
-                case 2: return pair_launch_one<T, P, A, kPairPitches[2]>(a, p, stream);
-                case 3: return pair_launch_one<T, P, A, kPairPitches[3]>(a, p, stream);
-                default: return hipErrorInvalidValue;
-            }
-        }
+hipError_t pair_launch_typed(const GridSamplerArgs& a, const PairPlan& p, hipStream_t stream)
+{
+    switch (p.cls) {
+        case 0: return pair_launch_one<T, kPairPitches[0]>(a, p, stream);
+        case 1: return pair_launch_one<T, kPairPitches[1]>(a, p, stream);
+        case 2: return pair_launch_one<T, kPairPitches[2]>(a, p, stream);
+        case 3: return pair_launch_one<T, kPairPitches[3]>(a, p, stream);
+        default: return hipErrorInvalidValue;
     }
-};
+}
 
 }  // namespace
 
@@ -143,10 +133,13 @@ hipError_t run_gs2d_pair(const GridSamplerArgs& a, hipStream_t stream, bool* han
         return hipSuccess;
     }
     *handled = true;
-    if (a.elem == Elem::F16) {
-        return dispatch_modes<_Float16>(a, PairLauncher<_Float16>{a, p, stream});
+    if (a.pad < 0 || a.pad > 2) {
+        return hipErrorInvalidValue;
     }
-    return dispatch_modes<__bf16>(a, PairLauncher<__bf16>{a, p, stream});
+    if (a.elem == Elem::F16) {
+        return pair_launch_typed<_Float16>(a, p, stream);
+    }
+    return pair_launch_typed<__bf16>(a, p, stream);
 }
 
 }  // namespace opscv

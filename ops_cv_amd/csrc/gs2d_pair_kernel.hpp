@@ -70,11 +70,11 @@ __device__ __forceinline__ float blend_pairs(uint32_t north, uint32_t south, con
 // the tensor 16-byte aligned and PITCH >= W + 4.  The lanes of a write instruction are 128 bytes apart along a row,
 // i.e. on the same banks; the distance between staged rows is therefore an odd multiple of 16 bytes modulo 128, which
 // spreads the sixteen rows a wavefront covers over all banks (a 16-way conflict otherwise).
-template <typename T, int PAD, bool ALIGN, int SWAVES, int LWAVES, int PPT, int PITCH, int RMAX>
+template <typename T, int SWAVES, int LWAVES, int PPT, int PITCH, int RMAX>
 __global__ __launch_bounds__((SWAVES + LWAVES) * 64) void gs2d_pair_kernel(
     const T* __restrict__ x, const T* __restrict__ grid, T* __restrict__ y, FastDiv N, int32_t C, int32_t H, int32_t W,
     int32_t out_plane, FastDiv tiles_per_n, int32_t chans_per_block, int32_t pair_aligned, int32_t xcd_swizzle,
-    float neg_zero)
+    int32_t pad, int32_t align, float neg_zero)
 {
     static_assert(sizeof(T) == 2, "pairs of 16-bit elements");
     static_assert(PPT % 2 == 0, "two neighbouring pixels per store");
@@ -234,11 +234,15 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) void gs2d_pair_kernel(
     uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
     asm volatile("" : "+s"(lds_base));  // kept as a value: seen as the allocation's symbol it is re-added per use
     const uint32_t outside = ((uint32_t)H + 1u) * ROW_STEP;  // rows H + 1 and H + 2: zeros for both pairs
+    // padding mode and align_corners are kernel arguments: one wave-uniform switch around the source coordinates of all
+    // the lane's pixels (they act once per pixel, outside the channel loop)
+    float ixs[PPT], iys[PPT];
+    source_indices_rt<PPT>(gxs, gys, H, W, pad, align != 0, false, ixs, iys);
 #pragma unroll
     for (int j = 0; j < PPT; j++) {
         // the decisions of decide_pixel() (sampler_math.hpp; grid_sampler2_d_simt.h:479-498, 307-316) without branches
-        float ix = compute_source_index<PAD, ALIGN>(gxs[j], W);
-        float iy = compute_source_index<PAD, ALIGN>(gys[j], H);
+        float ix = ixs[j];
+        float iy = iys[j];
         const bool finite = __builtin_fabsf(ix) < __builtin_inff() && __builtin_fabsf(iy) < __builtin_inff();
         const bool x_far = ix > 2147483646.0f || ix < -2147483648.0f;  // safe_downgrade: -> -100, always outside
         const bool y_far = iy > 2147483646.0f || iy < -2147483648.0f;
