@@ -18,11 +18,11 @@
 //   row r, dword 4 + k    (v[r][k-1], v[r][k]) for k = -4 .. W + 3, padded as above
 //   row H                 zeros
 // The two ring slots are interleaved row by row (row q of slot s at byte q * row_step + s * PITCH * 4), so that the slot
-// is an immediate offset of the read.  `row_step` is a kernel argument: by how many banks consecutive rows are shifted
-// against each other decides how often the lanes of a wavefront, which follow a slanted line through the plane, meet
-// on a bank, and the kernel's time with it (fp16 N16 C256 64x64, rotations up to 30 degrees: 35.5 us with a shift of 12
-// banks, 38.4 with 20, 44 with 16, 67 with none); it must be an odd number of 16-byte units, which spreads the sixteen
-// rows that the lanes of a loader's 16-byte write cover over all banks.
+// is an immediate offset of the read.  `row_step` is a kernel argument: it must be an odd number of 16-byte units, which
+// spreads the sixteen rows that the lanes of a loader's 16-byte write cover over all banks, and by how many banks it
+// shifts consecutive rows against each other decides how often the lanes of a sampler wavefront, which follow a
+// slanted line through the plane, meet on a bank (fp16 N16 C256 64x64, rotations up to 30 degrees: 35.5 us with a
+// shift of 12 banks, 38.4 with 20, 55.8 with 28, 60.7 with 4; even numbers of 16-byte units: 44 with 16, 67 with none).
 //
 // Workgroup roles, loader scheme and the samplers' rotating-register pipeline are those of gs2d_pair_kernel.hpp.  One
 // output pixel per lane and store: the lanes of a wavefront then read neighbouring entries (with two neighbouring
