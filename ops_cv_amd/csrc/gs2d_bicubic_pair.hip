@@ -54,7 +54,9 @@ BicubicPairPlan make_plan(const GridSamplerArgs& a)
     const uint32_t step = row_step((uint32_t)kPitches[p.cls]);
     p.row_step = step;
     const int64_t lds = (a.Hin + 1) * (int64_t)step;
-    const int64_t runs = a.Hin * (a.Win / 32);
+    // the loaders number their runs in blocks of sixteen rows (gs2d_bicubic_pair_kernel.hpp): a last, partial block
+    // takes the run numbers of a whole one
+    const int64_t runs = (a.Hin + 15) / 16 * 16 * (a.Win / 32);
     constexpr int64_t group_lanes = (kLoaderWaves / 2) * 64;
     if (lds > kLdsLimit || runs > (int64_t)kRunsPerLane[2] * group_lanes) {
         return p;

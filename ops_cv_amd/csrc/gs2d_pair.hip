@@ -48,7 +48,8 @@ PairPlan make_pair_plan(const GridSamplerArgs& a)
     p.cls = (int)(a.Win / 32) - 1;
     const uint32_t step = pair_row_step((uint32_t)kPairPitches[p.cls]);
     const int64_t lds = (a.Hin + 3) * (int64_t)step;
-    const int64_t runs = a.Hin * (a.Win / 32);
+    // the loaders number their runs in blocks of sixteen rows: a last, partial block takes the numbers of a whole one
+    const int64_t runs = (a.Hin + 15) / 16 * 16 * (a.Win / 32);
     if (lds > kLdsLimit || runs > (int64_t)kPairRmax * (kPairLoaderWaves / 2) * 64) {
         return p;
     }

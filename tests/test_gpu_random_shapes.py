@@ -87,6 +87,53 @@ def test_random_grid_sampler2d(oracle, device, aclnn):
         _same(I.from_torch(y, dtype), ref, dtype, (case, dtype, N, C, H, W, Ho, Wo, interp, pad, align, cl))
 
 
+def test_random_grid_sampler2d_pair_layouts(oracle, device, aclnn):
+    """rows of 32, 64, 96 or 128 16-bit elements, where the pair-layout kernels take bilinear samples of large output
+    planes and bicubic samples under zeros and border padding: random row counts, channel counts of every remainder,
+    odd output widths (which send the case to another variant: checked all the same), smooth and scattered grids with
+    special values sprinkled in; the variant that ran is counted so that the sweep cannot miss both kernels"""
+    import torch
+    rng = np.random.default_rng(9006 + SEED_SHIFT)
+    seen = {}
+    for case in range(60):
+        dtype = ("fp16", "bf16")[case % 2]
+        N, C = int(rng.integers(1, 4)), int(rng.integers(1, 20))
+        H, W = int(rng.integers(1, 130)), 32 * int(rng.integers(1, 5))
+        interp = (0, 2)[case % 3 != 0]
+        pad, align = int(rng.integers(0, 3)), bool(rng.integers(0, 2))
+        if interp == 0:
+            Ho, Wo = int(rng.integers(2 * H, 3 * H + 8)), int(rng.integers(2 * W, 2 * W + 40))  # several pixels per input pixel
+        else:
+            Ho, Wo = int(rng.integers(1, 140)), int(rng.integers(1, 140))
+            if case % 5 != 0:  # mostly what the bicubic pair kernel takes: zeros or border padding, whole pixel pairs
+                pad = int(rng.integers(0, 2))
+                Wo += Wo % 2
+        _say("gs2d pair", dtype, N, C, H, W, Ho, Wo, interp, pad, align)
+        x = I.cast_np(rng.standard_normal((N, C, H, W)).astype(np.float32), dtype)
+        if case % 4 == 0:
+            g32 = I.affine_grid(rng, N, Ho, Wo, max_deg=40.0, scale=(0.6, 1.4), shift=0.4)
+        else:
+            g32 = rng.uniform(-1.5, 1.5, (N, Ho, Wo, 2)).astype(np.float32)
+        if case % 2 == 1:
+            g32 = _sprinkle(rng, g32, H, W, align)
+        g = I.cast_np(g32, dtype)
+        tx, tg = I.to_torch(x, dtype, device), I.to_torch(g, dtype, device)
+        ty = torch.empty((N, C, Ho, Wo), dtype=tx.dtype, device=device)
+        hs = [aclnn.tensor_handle(t) for t in (tx, tg, ty)]
+        st, _, ex = aclnn.get_workspace_size_grid_sampler2d(hs[0], hs[1], interp, pad, align, hs[2])
+        assert st == 0
+        variant = aclnn.executor_variant(ex)
+        seen[variant.split("_w")[0]] = seen.get(variant.split("_w")[0], 0) + 1
+        aclnn.destroy_executor(ex)
+        for h in hs:
+            aclnn.destroy_tensor(h)
+        ref = oracle.grid_sampler2d(x, g, interp, pad, align, dtype=I.oracle_code(dtype))
+        y = aclnn.grid_sampler2d(tx, tg, interp, pad, align, out=ty)
+        torch.cuda.synchronize()
+        _same(I.from_torch(y, dtype), ref, dtype, (case, dtype, N, C, H, W, Ho, Wo, interp, pad, align, variant))
+    assert seen.get("lds_pair", 0) >= 3 and seen.get("lds_pair_bicubic", 0) >= 5, seen
+
+
 def test_random_grid_sampler2d_large_planes(oracle, device, aclnn):
     """input planes from a few KB to beyond the largest LDS class (the direct kernel), few channels"""
     import torch
