@@ -291,8 +291,8 @@ def upsample_bilinear2d(x, out_hw, align=False, scales_h=0.0, scales_w=0.0, dtyp
 
 
 def grid_sampler2d_arch35(x, grid, pad=0, align=False, dtype=None):
-    """bilinear 2-D sampling by the rule of the reference's GridSample operator on its newest part (a neighbouring
-    implementation that no HIP kernel follows)"""
+    """bilinear 2-D sampling by the rule of the reference's GridSample operator on its newest part (what the library
+    computes under option grid_sampler2d_rule = 1)"""
     x = np.ascontiguousarray(x)
     grid = np.ascontiguousarray(grid)
     code = _code_of(x) if dtype is None else dtype

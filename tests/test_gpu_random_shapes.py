@@ -87,6 +87,38 @@ def test_random_grid_sampler2d(oracle, device, aclnn):
         _same(I.from_torch(y, dtype), ref, dtype, (case, dtype, N, C, H, W, Ho, Wo, interp, pad, align, cl))
 
 
+def test_random_grid_sampler2d_second_rule(oracle, device, aclnn):
+    """option grid_sampler2d_rule = 1 over random shapes, padding modes and views, against the oracle's restatement of
+    the reference's second bilinear kernel"""
+    import torch
+    rng = np.random.default_rng(9007 + SEED_SHIFT)
+    for case in range(90):
+        dtype = I.DTYPES[case % 3]
+        N, C = _dims(rng, 1, 5, 1)[0], _dims(rng, 1, 40, 1)[0]
+        H, W = _dims(rng, 1, 150, 2)
+        Ho, Wo = _dims(rng, 1, 120, 2)
+        pad, align = int(rng.integers(0, 3)), bool(rng.integers(0, 2))
+        cl = case % 5 == 4
+        _say("gs2d rule 1", dtype, N, C, H, W, Ho, Wo, pad, align, cl)
+        x = I.cast_np(rng.standard_normal((N, C, H, W)).astype(np.float32), dtype)
+        g32 = rng.uniform(-1.4, 1.4, (N, Ho, Wo, 2)).astype(np.float32)
+        if case % 2 == 1:
+            g32 = _sprinkle(rng, g32, H, W, align)
+        g = I.cast_np(g32, dtype)
+        ref = oracle.grid_sampler2d_arch35(x, g, pad, align, dtype=I.oracle_code(dtype))
+        xt, gt = I.to_torch(x, dtype, device), I.to_torch(g, dtype, device)
+        with aclnn.option("grid_sampler2d_rule", 1):
+            if cl:
+                xt = xt.contiguous(memory_format=torch.channels_last)
+                out = torch.empty((N, C, Ho, Wo), dtype=xt.dtype,
+                                  device=device).contiguous(memory_format=torch.channels_last)
+                y = aclnn.grid_sampler2d(xt, gt, 0, pad, align, out=out).contiguous()
+            else:
+                y = aclnn.grid_sampler2d(xt, gt, 0, pad, align)
+        torch.cuda.synchronize()
+        _same(I.from_torch(y, dtype), ref, dtype, (case, dtype, N, C, H, W, Ho, Wo, pad, align, cl))
+
+
 def test_random_grid_sampler2d_pair_layouts(oracle, device, aclnn):
     """rows of 32, 64, 96 or 128 16-bit elements, where the pair-layout kernels take bilinear samples of large output
     planes and bicubic samples under zeros and border padding: random row counts, channel counts of every remainder,
