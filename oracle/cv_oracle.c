@@ -54,8 +54,9 @@
  *                                  with the reference is "parity unpinned" for the reasons given for the 2-D
  *                                  backward; the accumulation order restated is that of its deterministic mode
  *   oracle_grid_sampler2d_arch35, oracle_upsample_a2_axis_taps, oracle_upsample_bilinear2d_a2 : restatements of two
- *                                  neighbouring implementations in the reference that no HIP kernel follows; kept
- *                                  to show where they leave the mirrored kernels.  Pinned by closed forms (taps and
+ *                                  neighbouring implementations in the reference; the first is the checker of the
+ *                                  library's second bilinear rule (option grid_sampler2d_rule = 1), the other two no
+ *                                  HIP kernel follows (kept to show where they leave the mirrored kernels).  Pinned by closed forms (taps and
  *                                  weights at hand-computed coordinates, zero output for non-finite grid values,
  *                                  x2 upscale tap table) and by agreement with the mirrored oracle within tolerance
  *                                  on finite data
@@ -1628,8 +1629,9 @@ int oracle_grid_sampler3d_backward(const void* gout, const void* x, const void* 
 }
 
 /* ------------------------------------------------------------------------------------------
- * Two neighbouring implementations of the same operators in the reference, restated only to show where their
- * results leave those of the kernels this library mirrors (tests/test_oracle.py); no HIP kernel follows them.
+ * Two neighbouring implementations of the same operators in the reference, restated to show where their results
+ * leave those of the kernels this library mirrors by default (tests/test_oracle.py).  The first is also the checker
+ * of the library's second bilinear rule; no HIP kernel follows the second.
  * ---------------------------------------------------------------------------------------- */
 
 /* The 2-D bilinear kernel of the reference's GridSample operator, which is what its aclnnGridSampler2D launches on
