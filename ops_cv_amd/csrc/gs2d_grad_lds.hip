@@ -53,18 +53,6 @@ __device__ __forceinline__ void touch_line(const char* p, char* dump)
 }
 constexpr int kDumpBytes = 256;
 
-// The last planes of a ring: plane by plane, wait until at most the K, K - 1, ... 0 planes after it (PP copies each)
-// are outstanding, and hand it over.
-template <int K, int PP>
-__device__ __forceinline__ void ring_rundown()
-{
-    wait_vmcnt_imm<K * PP>();
-    lds_barrier();
-    if constexpr (K > 0) {
-        ring_rundown<K - 1, PP>();
-    }
-}
-
 template <typename T, int NBUF, int PITCH>
 __global__ __launch_bounds__(kThreadsLds) void gs2d_grad_grid_lds_kernel(
     const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ grid, T* __restrict__ dgrid, int32_t C,

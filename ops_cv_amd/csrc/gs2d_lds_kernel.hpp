@@ -276,6 +276,18 @@ __device__ __forceinline__ void lds_barrier()
     asm volatile("" ::: "memory");
 }
 
+// The last stages of a ring whose stages are PP copy instructions each: stage by stage, wait until at most the K,
+// K - 1, ... 0 stages after it are outstanding, and hand it over.
+template <int K, int PP>
+__device__ __forceinline__ void ring_rundown()
+{
+    wait_vmcnt_imm<K * PP>();
+    lds_barrier();
+    if constexpr (K > 0) {
+        ring_rundown<K - 1, PP>();
+    }
+}
+
 // Bank-spreading layout of a staged plane whose rows are exactly 128 bytes (row_shift = 7 | turn << 8; 0 = plain
 // layout).  LDS has 32 four-byte banks, i.e. 128 bytes per "line"; with that row pitch column x of every row falls into
 // the same bank, and coordinates clamped to the first or last column (border padding) make a wavefront read one bank
@@ -645,6 +657,68 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
                 issue_stage_copy<4, LWAVES, CGS, PITCH>(src, dst, plane_bytes, planes_of(s), lwave, lane, lane * 4u);
             }
         };
+        // The usual case has a loop of its own: single-plane stages of whole, aligned planes whose 1 KiB chunks divide
+        // evenly among the loaders (PP copies each, a compile-time number) and at least as many stages as the ring
+        // runs ahead.  A loader's step per stage -- wait, barrier, issue -- is in the chain of barriers that every
+        // stage goes through, and at the start of the kernel the loaders' first DEPTH stages are what the samplers
+        // wait for.  The general loop below finds the wait count of every stage at run time (a sum over the stages in
+        // flight, then six compares and branches to reach the matching literal) and tests bounds around every copy:
+        // about a hundred scalar instructions and two dozen taken branches per stage, 0.3 us of a wavefront's time.
+        // Here the counts are literals and the copies unconditional: steady state while the ring is full, then an
+        // unrolled run-down.
+        if constexpr (!shifted && CGS == 1) {
+            const uint32_t share = (uint32_t)LWAVES * 1024u;
+            if (copy_gran == 16 && plane_bytes % share == 0u && nstages >= DEPTH) {
+                auto ring_loop = [&](auto pp_tag) {
+                    constexpr int PP = decltype(pp_tag)::value;
+                    if constexpr ((DEPTH - 1) * PP <= 63 && PP * LWAVES * 1024 + 16 <= PITCH) {
+                        const char* src = xb + lwave * 1024u + lane_src16;  // this lane's 16 bytes of the first chunk
+                        uint32_t slot_off = lwave * 1024u;                  // the chunk's place in the slot being filled
+                        int fill = 0;
+                        auto issue = [&]() {
+#pragma unroll
+                            for (int j = 0; j < PP; j++) {
+                                __builtin_amdgcn_global_load_lds((global_cptr_t)(src + j * (LWAVES * 1024)),
+                                                                 (lds_ptr_t)(lds + slot_off + j * (LWAVES * 1024)), 16,
+                                                                 0, 0);
+                            }
+                            src += plane_bytes;
+                            fill = (fill + 1 == NBUF) ? 0 : fill + 1;
+                            slot_off = (uint32_t)fill * SLOT_BYTES + lwave * 1024u;
+                        };
+#pragma unroll
+                        for (int i = 0; i < DEPTH; i++) {
+                            issue();
+                        }
+                        for (int32_t s = 0; s < nstages - DEPTH; s++) {
+                            wait_vmcnt_imm<(DEPTH - 1) * PP>();  // stage s has landed: the DEPTH - 1 after it may be out
+                            lds_barrier();                       // ... and the slot of stage s - 1 is free
+                            issue();
+                        }
+                        ring_rundown<DEPTH - 1, PP>();
+                        lds_barrier();  // the samplers' barrier behind the last plane (see their loop)
+                        return true;
+                    } else {
+                        return false;
+                    }
+                };
+                bool done = false;
+                switch (plane_bytes / share) {
+                    case 1: done = ring_loop(std::integral_constant<int, 1>{}); break;
+                    case 2: done = ring_loop(std::integral_constant<int, 2>{}); break;
+                    case 3: done = ring_loop(std::integral_constant<int, 3>{}); break;
+                    case 4: done = ring_loop(std::integral_constant<int, 4>{}); break;
+                    case 5: done = ring_loop(std::integral_constant<int, 5>{}); break;
+                    case 6: done = ring_loop(std::integral_constant<int, 6>{}); break;
+                    case 7: done = ring_loop(std::integral_constant<int, 7>{}); break;
+                    case 8: done = ring_loop(std::integral_constant<int, 8>{}); break;
+                    default: break;
+                }
+                if (done) {
+                    return;
+                }
+            }
+        }
         // `issued` stages have been started; stage q goes to slot q % NBUF, which is free once the samplers are through
         // the barrier of stage q - DEPTH (their reads of stage q - NBUF have returned by then)
         int32_t issued = 0;
