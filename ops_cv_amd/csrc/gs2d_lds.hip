@@ -92,21 +92,30 @@ LdsPlan make_lds_plan(const GridSamplerArgs& a)
         return p;
     }
     // Exactly two workgroups per CU: the one that reaches a CU first keeps ahead of the one that joins it for the
-    // whole kernel (its wavefronts are the older ones wherever the CU arbitrates) and ends about five stages earlier,
-    // after which the CU runs half empty.  The launch hands out workgroups in index order and channel blocks are
-    // numbered with the index (gs2d_lds_kernel.hpp), so the lower half of the channel blocks are those first
-    // workgroups: they take 5 channels for every 3 of the upper half (fp16 N16 C256 64x64: 13.9 us with 16 + 16,
-    // 13.3 with 19 + 13, 12.9 with 20 + 12; the measured stage rates while both run are 2.2 and 1.45 per microsecond).
+    // whole kernel (its wavefronts are the older ones wherever the CU arbitrates), after which the CU runs half empty.
+    // The launch hands out workgroups in index order and channel blocks are numbered with the index
+    // (gs2d_lds_kernel.hpp), so the lower half of the channel blocks are those first workgroups and take more
+    // channels than the upper half.  fp16 N16 C256 64x64, channels in contiguous ranges: 13.9 us with 16 + 16, 13.3
+    // with 19 + 13, 12.9 with 20 + 12 (the stage rates measured while both ran were 2.2 and 1.45 per microsecond).
+    // With the channels dealt out in turn (below) and the loaders' literal-count loop: 13.2 us with 16 + 16, 12.9
+    // with 20 + 12, 12.5 with 22 + 10, 12.6 with 24 + 8, 13.1 with 26 + 6.
     // A wrong guess about who comes first costs balance, never correctness.
     if (cgs == 1 && cblocks % 2 == 0 && cpb >= 8 && a.C == cblocks * cpb &&
         a.N * p.tiles_per_n * cblocks == 2 * (int64_t)compute_unit_count() && (a.N * cblocks / 2) % 8 == 0) {
-        const int64_t wide = (cpb * 5 + 2) / 4;
+        const int64_t wide = plain ? (cpb * 11 + 4) / 8 : (cpb * 5 + 2) / 4;
         const int64_t narrow = 2 * cpb - wide;
         if (narrow >= 1) {
             p.wide_blocks = (uint32_t)(cblocks / 2);
             p.chans_wide = (int32_t)wide;
             p.chans_per_block = (int32_t)narrow;
         }
+    }
+    // Channels dealt out to the channel blocks in turn rather than in contiguous ranges (single-plane stages, whole
+    // aligned planes, every block's count exact): at any moment the workgroups of a batch item then read neighbouring
+    // planes and write neighbouring planes, instead of sixteen streams 160 KB apart (fp16 N16 C256 64x64: 13.4 ->
+    // 13.0 us before the split above was set again, 12.5 with it).
+    if (cgs == 1 && plain && cblocks > 1 && a.C == cblocks * cpb) {
+        p.chan_stride = (int32_t)cblocks;
     }
     p.copy_gran = plain ? 16 : 2;  // 2: 16-byte units in the shifted layout
     // Bank-spreading layout (gs2d_lds_kernel.hpp): rows of exactly 128 bytes, 16-byte copy granule.  Only for

@@ -569,7 +569,7 @@ template <typename T, int INTERP, int SWAVES, int LWAVES, int PPT, int ADJ, int 
 __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves_per_eu(1, 5))) void gs2d_lds_kernel(
     const T* __restrict__ x, const T* __restrict__ grid, T* __restrict__ y, FastDiv N, int32_t C, int32_t H, int32_t W,
     int32_t out_plane, FastDiv tiles_per_n, int32_t chans_per_block, uint32_t wide_blocks,
-    int32_t chans_wide, int32_t copy_gran, int32_t pair_aligned, int32_t xcd_swizzle, int32_t row_shift, int32_t pad,
+    int32_t chans_wide, int32_t chan_stride, int32_t copy_gran, int32_t pair_aligned, int32_t xcd_swizzle, int32_t row_shift, int32_t pad,
     int32_t align, int32_t rule, float neg_zero)
 {
     extern __shared__ uint4 smem_raw[];
@@ -610,18 +610,38 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
     // make_lds_plan: the workgroup that reaches a CU first runs ahead of the one that shares the CU with it).
     const bool wide = cb < wide_blocks;
     const int32_t my_chans = wide ? chans_wide : chans_per_block;
-    const int32_t c_begin = wide ? (int32_t)cb * chans_wide
-                                 : (int32_t)wide_blocks * chans_wide + (int32_t)(cb - wide_blocks) * chans_per_block;
-    const int32_t c_end = (c_begin + my_chans < C) ? c_begin + my_chans : C;
-    const int32_t nchan = c_end - c_begin;
+    // Which channels: a contiguous range [c_begin, c_end), or -- `chan_stride` != 0, single-plane stages, every block's
+    // count exact -- channels dealt out in turn: block cb takes cb, cb + chan_stride, ... while all blocks draw
+    // (`chans_per_block` turns), and the wide blocks then share out the rest among themselves, wide_blocks apart.
+    // Both are  first + j * step1  for the block's j-th channel up to j = switch_at, and step2 apart from there on.
+    int32_t first, step1, step2, nchan;
+    if (chan_stride != 0) {
+        first = (int32_t)cb;
+        step1 = chan_stride;
+        step2 = (int32_t)wide_blocks;
+        nchan = my_chans;
+    } else {
+        const int32_t c_begin = wide ? (int32_t)cb * chans_wide
+                                     : (int32_t)wide_blocks * chans_wide + (int32_t)(cb - wide_blocks) * chans_per_block;
+        const int32_t c_end = (c_begin + my_chans < C) ? c_begin + my_chans : C;
+        first = c_begin;
+        step1 = 1;
+        step2 = 1;
+        nchan = c_end - c_begin;
+    }
+    const int32_t switch_at = chans_per_block;
+    // the block's j-th channel
+    auto chan_of = [&](int32_t j) -> int32_t {
+        return first + (j < switch_at ? j * step1 : switch_at * step1 + (j - switch_at) * step2);
+    };
     const int32_t nstages = (nchan + CGS - 1) / CGS;
 
     if (wave >= (uint32_t)SWAVES) {
         // ------------------------------------------------ loader wavefronts ------------------------------------
         const uint32_t lwave = wave - SWAVES;
         const uint32_t lane = (uint32_t)tid & 63u;
-        const char* xb = reinterpret_cast<const char*>(x + ((int64_t)n * C + c_begin) * plane_elems);
-        const size_t stage_bytes = (size_t)CGS * plane_bytes;
+        const char* xn = reinterpret_cast<const char*>(x + (int64_t)n * C * plane_elems);  // the batch item's planes
+        const char* xb = xn + (size_t)first * plane_bytes;                                  // the block's first plane
         // copy instructions this wavefront issues per plane
         constexpr bool shifted = SHIFTED_PLANES;  // 16-byte granule, planes off the 16-byte grid (see issue_stage_copy)
         const uint32_t chunk = 64u * (uint32_t)(shifted ? 16 : copy_gran);
@@ -646,7 +666,7 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
         };
         const uint32_t lane_src16 = lds_unswizzle(lane * 16u, (uint32_t)row_shift);
         auto start_stage = [&](int32_t s, int slot) {
-            const char* src = xb + (size_t)s * stage_bytes;
+            const char* src = xn + (size_t)chan_of(s * CGS) * plane_bytes;
             char* dst = lds + slot * SLOT_BYTES;
             if constexpr (shifted) {
                 issue_stage_copy<16, LWAVES, CGS, PITCH, true>(src, dst, plane_bytes, planes_of(s), lwave, lane,
@@ -675,6 +695,7 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
                         const char* src = xb + lwave * 1024u + lane_src16;  // this lane's 16 bytes of the first chunk
                         uint32_t slot_off = lwave * 1024u;                  // the chunk's place in the slot being filled
                         int fill = 0;
+                        int32_t turn = 0;  // the block's channel being asked for
                         auto issue = [&]() {
 #pragma unroll
                             for (int j = 0; j < PP; j++) {
@@ -682,7 +703,8 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
                                                                  (lds_ptr_t)(lds + slot_off + j * (LWAVES * 1024)), 16,
                                                                  0, 0);
                             }
-                            src += plane_bytes;
+                            src += (size_t)(turn < switch_at ? step1 : step2) * plane_bytes;
+                            turn++;
                             fill = (fill + 1 == NBUF) ? 0 : fill + 1;
                             slot_off = (uint32_t)fill * SLOT_BYTES + lwave * 1024u;
                         };
@@ -819,7 +841,7 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
         }
     }
 
-    T* yb = y + ((int64_t)n * C + c_begin) * out_plane;
+    T* yplane = y + ((int64_t)n * C + first) * out_plane;  // the output plane of the channel being blended
     const uint32_t out_plane_bytes = (uint32_t)out_plane * (uint32_t)sizeof(T);
 
     // the bytes by which a plane's copy started early (SHIFTED_PLANES, see issue_stage_copy): the low four bits of the
@@ -827,7 +849,7 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
     // plane distance a run-time value where it is a literal otherwise (one more add per tap).
     const uint32_t addr_low = (uint32_t)(reinterpret_cast<uintptr_t>(x) & 15u);
     const uint32_t size_low = plane_bytes & 15u;
-    const uint32_t first_plane = (uint32_t)n * (uint32_t)C + (uint32_t)c_begin;
+    const uint32_t first_plane = (uint32_t)n * (uint32_t)C + (uint32_t)first;
     auto plane_shift = [&](int32_t p) -> uint32_t {
         if constexpr (SHIFTED_PLANES) {
             return (addr_low + (first_plane + (uint32_t)p) * size_low) & 15u;
@@ -869,7 +891,8 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
             const int un = (u + 1) % UNR;  // a literal once the loop is unrolled
             const uint32_t next_off = (uint32_t)((un / CGS) * SLOT_BYTES + (un % CGS) * PITCH) + plane_shift(p + 1);
             const __amdgpu_buffer_rsrc_t rsrc =
-                __builtin_amdgcn_make_buffer_rsrc(yb + (int64_t)p * out_plane, 0, out_plane_bytes, kBufferFlags);
+                __builtin_amdgcn_make_buffer_rsrc(yplane, 0, out_plane_bytes, kBufferFlags);
+            yplane += (int64_t)(p < switch_at ? step1 : step2) * out_plane;
 #pragma unroll
             for (int q = 0; q < NGRP; q++) {
                 float v[ADJ];
