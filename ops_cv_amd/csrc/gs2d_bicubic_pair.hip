@@ -30,6 +30,11 @@ struct BicubicPairPlan {
     uint32_t lds_bytes = 0;
     uint32_t tiles_per_n = 0, cblocks = 0;
     int32_t chans_per_block = 0;
+    // as in the ring kernel's plan (gs2d_lds_launch.hpp): the first `wide_blocks` channel blocks take `chans_wide`
+    // channels each, and channels are dealt out in turn, `chan_stride` apart, when that is not 0
+    uint32_t wide_blocks = 0;
+    int32_t chans_wide = 0;
+    int32_t chan_stride = 0;
     int xcd_swizzle = 0;
     uint32_t row_step = 0;
 };
@@ -86,6 +91,24 @@ BicubicPairPlan make_plan(const GridSamplerArgs& a)
     if (a.N * p.tiles_per_n * cblocks > INT32_MAX) {
         return p;
     }
+    // Exactly two workgroups per CU: the first to reach a CU runs ahead of the second (gs2d_lds.hip), so the lower half
+    // of the channel blocks takes 5 channels for every 3 of the upper half; and channels are dealt out in turn where
+    // every block's count is exact (fp16 N16 C256 64x64: 35.6 us with 32 + 32 in contiguous ranges, 35.5 dealt out,
+    // 35.2 with 36 + 28, 34.8 with 40 + 24, 34.9 with 44 + 20, 35.8 with 48 + 16: the LDS, not the schedule, bounds
+    // this kernel).
+    if (a.C == cblocks * cpb && cblocks > 1) {
+        if (cblocks % 2 == 0 && cpb >= 8 && a.N * p.tiles_per_n * cblocks == 2 * (int64_t)compute_unit_count() &&
+            (a.N * cblocks / 2) % 8 == 0) {
+            const int64_t wide = (cpb * 5 + 2) / 4;
+            const int64_t narrow = 2 * cpb - wide;
+            if (narrow >= 1) {
+                p.wide_blocks = (uint32_t)(cblocks / 2);
+                p.chans_wide = (int32_t)wide;
+                p.chans_per_block = (int32_t)narrow;
+            }
+        }
+        p.chan_stride = (int32_t)cblocks;
+    }
     p.xcd_swizzle = ((a.N * cblocks) % 8 == 0) ? 1 : 0;
     p.ok = true;
     return p;
@@ -105,7 +128,7 @@ hipError_t launch_one(const GridSamplerArgs& a, const BicubicPairPlan& p, hipStr
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3((kSamplerWaves + kLoaderWaves) * 64), p.lds_bytes, stream,
                        (const T*)a.x, (const T*)a.grid, (T*)a.y, make_fast_div((uint32_t)a.N), (int32_t)a.C,
                        (int32_t)a.Hin, (int32_t)a.Win, (int32_t)(a.Hout * a.Wout), make_fast_div(p.tiles_per_n),
-                       p.chans_per_block, pair_aligned, p.xcd_swizzle, p.row_step, (int32_t)a.pad, (int32_t)(a.align != 0),
+                       p.chans_per_block, p.wide_blocks, p.chans_wide, p.chan_stride, pair_aligned, p.xcd_swizzle, p.row_step, (int32_t)a.pad, (int32_t)(a.align != 0),
                        -0.0f);
     return hipGetLastError();
 }

@@ -66,7 +66,8 @@ __device__ __forceinline__ float blend_bicubic_pairs(const uint32_t* raw, const 
 template <typename T, int SWAVES, int LWAVES, int PPT, int PITCH, int RMAX, int ADJ>
 __global__ __launch_bounds__((SWAVES + LWAVES) * 64) void gs2d_bicubic_pair_kernel(
     const T* __restrict__ x, const T* __restrict__ grid, T* __restrict__ y, FastDiv N, int32_t C, int32_t H, int32_t W,
-    int32_t out_plane, FastDiv tiles_per_n, int32_t chans_per_block, int32_t pair_aligned, int32_t xcd_swizzle,
+    int32_t out_plane, FastDiv tiles_per_n, int32_t chans_per_block, uint32_t wide_blocks, int32_t chans_wide,
+    int32_t chan_stride, int32_t pair_aligned, int32_t xcd_swizzle,
     uint32_t row_step, int32_t pad, int32_t align, float neg_zero)
 {
     static_assert(sizeof(T) == 2, "pairs of 16-bit elements");
@@ -101,9 +102,29 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) void gs2d_bicubic_pair_kern
     const uint32_t cb = fast_div(group, N);
     const uint32_t n = group - cb * N.div;
     const int32_t plane_elems = H * W;
-    const int32_t c_begin = (int32_t)cb * chans_per_block;
-    const int32_t c_end = (c_begin + chans_per_block < C) ? c_begin + chans_per_block : C;
-    const int32_t nchan = c_end - c_begin;
+    // Which channels, as in the ring kernel (gs2d_lds_kernel.hpp): a contiguous range, or -- `chan_stride` != 0,
+    // every block's count exact -- channels dealt out in turn, the first `wide_blocks` blocks taking `chans_wide`
+    // each and the others `chans_per_block`.  The block's j-th channel is  first + j * step1  up to j = switch_at and
+    // step2 apart from there on.
+    const bool wide = cb < wide_blocks;
+    int32_t first, step1, step2, nchan;
+    if (chan_stride != 0) {
+        first = (int32_t)cb;
+        step1 = chan_stride;
+        step2 = (int32_t)wide_blocks;
+        nchan = wide ? chans_wide : chans_per_block;
+    } else {
+        const int32_t c_begin = (int32_t)cb * chans_per_block;
+        const int32_t c_end = (c_begin + chans_per_block < C) ? c_begin + chans_per_block : C;
+        first = c_begin;
+        step1 = 1;
+        step2 = 1;
+        nchan = c_end - c_begin;
+    }
+    const int32_t switch_at = chans_per_block;
+    auto chan_of = [&](int32_t j) -> int32_t {
+        return first + (j < switch_at ? j * step1 : switch_at * step1 + (j - switch_at) * step2);
+    };
 
     if (wave >= (uint32_t)SWAVES) {
         // ------------------------------------------------ loader wavefronts ------------------------------------
@@ -114,7 +135,7 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) void gs2d_bicubic_pair_kern
         const uint32_t lwave = wave - SWAVES;
         const uint32_t g = lwave / (LWAVES / 2);
         const uint32_t lg = (lwave % (LWAVES / 2)) * 64u + ((uint32_t)tid & 63u);
-        const char* xb = reinterpret_cast<const char*>(x + ((int64_t)n * C + c_begin) * plane_elems);
+        const char* xn = reinterpret_cast<const char*>(x + (int64_t)n * C * plane_elems);  // the batch item's planes
         const size_t plane_bytes = (size_t)plane_elems * 2u;
         const uint32_t rpr = (uint32_t)W / 32u;  // runs per row
         typedef uint32_t dwordx4_t __attribute__((ext_vector_type(4)));
@@ -139,7 +160,7 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) void gs2d_bicubic_pair_kern
         const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
         int32_t done = 0;  // barriers this wavefront has been through
         for (int32_t p = (int32_t)g; p < nchan; p += 2) {
-            const char* sp = xb + (size_t)p * plane_bytes;
+            const char* sp = xn + (size_t)chan_of(p) * plane_bytes;
 #pragma unroll
             for (int i = 0; i < RMAX; i++) {
                 if (dst[i] != 0xFFFFFFFFu) {
@@ -252,7 +273,7 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) void gs2d_bicubic_pair_kern
         }
     }
 
-    T* yb = y + ((int64_t)n * C + c_begin) * out_plane;
+    T* yn = y + (int64_t)n * C * out_plane;  // the batch item's output planes
     const uint32_t out_plane_bytes = (uint32_t)out_plane * 2u;
     typedef const uint32_t __attribute__((address_space(3))) * lds_dw_ptr_t;
     uint32_t raw[PPT][8];
@@ -283,7 +304,7 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) void gs2d_bicubic_pair_kern
             }
             const uint32_t next_off = (u == 0) ? ROW_BYTES : 0u;  // slot of plane p + 1
             const __amdgpu_buffer_rsrc_t rsrc =
-                __builtin_amdgcn_make_buffer_rsrc(yb + (int64_t)p * out_plane, 0, out_plane_bytes, kBufferFlags);
+                __builtin_amdgcn_make_buffer_rsrc(yn + (int64_t)chan_of(p) * out_plane, 0, out_plane_bytes, kBufferFlags);
 #pragma unroll
             for (int q = 0; q < NGRP; q++) {
                 float v[ADJ];

@@ -90,4 +90,7 @@ const char* gs2d_box_variant_name(const GridSamplerArgs& a);
 // Channels-last variant (gs2d_nhwc.hip): a.x is (N,Hin,Win,C), a.y is (N,Hout,Wout,C).
 hipError_t run_gs2d_nhwc(const GridSamplerArgs& a, hipStream_t stream);
 
+// CUs of the current device (256 on MI355X; also the answer where no device can be asked); gs2d_lds.hip
+int compute_unit_count();
+
 }  // namespace opscv

@@ -8,7 +8,7 @@
 namespace opscv {
 
 // CUs of the current device (256 on MI355X; also the answer where no device can be asked, as in host-only planning).
-static int compute_unit_count()
+int compute_unit_count()
 {
     static std::atomic<int> cached{0};
     int v = cached.load(std::memory_order_relaxed);
