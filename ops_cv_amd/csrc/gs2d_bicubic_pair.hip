@@ -125,11 +125,22 @@ hipError_t launch_one(const GridSamplerArgs& a, const BicubicPairPlan& p, hipStr
     }
     const int pair_aligned = (reinterpret_cast<uintptr_t>(a.grid) % 4 == 0);
     const uint32_t blocks = (uint32_t)(a.N * p.tiles_per_n * p.cblocks);
+    // A wavefront's 64 pixels are a block of 16 columns by 4 rows of the output where its size allows, not 64
+    // consecutive pixels: under a smooth grid the lanes' taps then lie in a compact patch of the plane, many lanes
+    // read the same pair (one bank access serves them all) and the patch's rows fall on different banks, where the
+    // taps of 64 pixels in a row are strung along a slanted line through half the plane (fp16 N16 C256 64x64,
+    // rotations of up to 30 degrees: 34.8 us in rows, 35.9 with 32 x 2, 31.9 with 16 x 4, 37.5 with 8 x 8 whose stores
+    // are 16-byte pieces, 56.1 with 4 x 16; the row step of 12 banks stays the best one: 31.8 us, as 20; 4 and 28: 40).
+    int32_t bw_shift = 0, blocks_per_row = 0;
+    if (a.Wout % 16 == 0 && a.Hout % 4 == 0) {
+        bw_shift = 4;
+        blocks_per_row = (int32_t)(a.Wout / 16);
+    }
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3((kSamplerWaves + kLoaderWaves) * 64), p.lds_bytes, stream,
                        (const T*)a.x, (const T*)a.grid, (T*)a.y, make_fast_div((uint32_t)a.N), (int32_t)a.C,
                        (int32_t)a.Hin, (int32_t)a.Win, (int32_t)(a.Hout * a.Wout), make_fast_div(p.tiles_per_n),
-                       p.chans_per_block, p.wide_blocks, p.chans_wide, p.chan_stride, pair_aligned, p.xcd_swizzle, p.row_step, (int32_t)a.pad, (int32_t)(a.align != 0),
-                       -0.0f);
+                       p.chans_per_block, p.wide_blocks, p.chans_wide, p.chan_stride, pair_aligned, p.xcd_swizzle,
+                       p.row_step, (int32_t)a.pad, (int32_t)(a.align != 0), bw_shift, blocks_per_row, -0.0f);
     return hipGetLastError();
 }
 

@@ -68,7 +68,7 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) void gs2d_bicubic_pair_kern
     const T* __restrict__ x, const T* __restrict__ grid, T* __restrict__ y, FastDiv N, int32_t C, int32_t H, int32_t W,
     int32_t out_plane, FastDiv tiles_per_n, int32_t chans_per_block, uint32_t wide_blocks, int32_t chans_wide,
     int32_t chan_stride, int32_t pair_aligned, int32_t xcd_swizzle,
-    uint32_t row_step, int32_t pad, int32_t align, float neg_zero)
+    uint32_t row_step, int32_t pad, int32_t align, int32_t bw_shift, int32_t blocks_per_row, float neg_zero)
 {
     static_assert(sizeof(T) == 2, "pairs of 16-bit elements");
     static_assert(PPT % ADJ == 0, "whole groups of neighbouring pixels per store");
@@ -241,8 +241,17 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) void gs2d_bicubic_pair_kern
     const T* gptr[PPT];
 #pragma unroll
     for (int q = 0; q < NGRP; q++) {
-        const int32_t pix0 = (int32_t)tile * (STHREADS * PPT) + q * (STHREADS * ADJ) + tid * ADJ;
-        const bool valid = pix0 < out_plane;  // the output plane holds whole groups (launch plan)
+        int32_t pix0 = (int32_t)tile * (STHREADS * PPT) + q * (STHREADS * ADJ) + tid * ADJ;
+        bool valid = pix0 < out_plane;  // the output plane holds whole groups (launch plan)
+        if (ADJ == 1 && bw_shift != 0) {
+            // a wavefront's 64 pixels as a block of 2^bw_shift columns by 64 >> bw_shift rows
+            const int32_t unit = pix0 >> 6;
+            const int32_t lane = tid & 63;
+            const int32_t bx = lane & ((1 << bw_shift) - 1), by = lane >> bw_shift;
+            const int32_t brow = unit / blocks_per_row, bcol = unit - brow * blocks_per_row;
+            pix0 = (brow * (64 >> bw_shift) + by) * (blocks_per_row << bw_shift) + (bcol << bw_shift) + bx;
+            valid = unit < (out_plane >> 6);
+        }
         const int32_t pc = valid ? pix0 : out_plane - ADJ;
         pixoff[q] = valid ? (uint32_t)pc * 2u : 0x80000000u;
 #pragma unroll
