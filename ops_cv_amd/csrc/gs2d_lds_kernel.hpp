@@ -734,6 +734,7 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
                     case 6: done = ring_loop(std::integral_constant<int, 6>{}); break;
                     case 7: done = ring_loop(std::integral_constant<int, 7>{}); break;
                     case 8: done = ring_loop(std::integral_constant<int, 8>{}); break;
+                    case 16: done = ring_loop(std::integral_constant<int, 16>{}); break;
                     default: break;
                 }
                 if (done) {
