@@ -431,7 +431,8 @@ struct Fold<_Float16> {
 template <typename T, int CB, int EPL>
 __global__ __launch_bounds__(kApplyThreads) void gs2d_grad_csr_apply_kernel(
     const T* __restrict__ gout, T* __restrict__ dx, const uint32_t* __restrict__ ws, GradParams p, CsrLayout lay,
-    uint32_t tiles, uint32_t cblocks, int32_t chans_per_block, int32_t xcd_swizzle)
+    uint32_t tiles, uint32_t cblocks, int32_t chans_per_block, int32_t xcd_swizzle, uint32_t items_fastest,
+    uint32_t wide_blocks, int32_t chans_wide, int32_t unit_stride)
 {
     typedef Fold<T> F;
     typedef typename F::acc_t acc_t;
@@ -456,13 +457,35 @@ __global__ __launch_bounds__(kApplyThreads) void gs2d_grad_csr_apply_kernel(
         group = blockIdx.x / tiles;
         tile = blockIdx.x % tiles;
     }
-    const uint32_t cb = group % cblocks;
-    const int64_t n = group / cblocks;
-    const int32_t c_begin = (int32_t)cb * chans_per_block;
-    const int32_t c_end = (c_begin + chans_per_block < p.C) ? c_begin + chans_per_block : p.C;
-    const int32_t nchan = c_end - c_begin;
+    // groups numbered with the batch item fastest (`items_fastest` = N, else 0): an XCD then sees the lists of N / 8
+    // items only, and the channel blocks with the low numbers are the workgroups handed out first
+    const uint32_t cb = items_fastest ? group / items_fastest : group % cblocks;
+    const int64_t n = items_fastest ? group % items_fastest : group / cblocks;
+    // A step works on a unit of CB neighbouring channels.  Which units: a contiguous range, or -- `unit_stride` != 0,
+    // every block's count exact -- units dealt out in turn, the first `wide_blocks` blocks taking `chans_wide`
+    // channels each and the others `chans_per_block` (see gs2d_lds.hip for the why of both).  The block's s-th unit
+    // is  first + s * step1  up to s = switch_at and step2 apart from there on.
+    const bool wide = cb < wide_blocks;
+    int32_t first, step1, step2, nchan;
+    if (unit_stride != 0) {
+        first = (int32_t)cb;
+        step1 = unit_stride;
+        step2 = (int32_t)wide_blocks;
+        nchan = wide ? chans_wide : chans_per_block;
+    } else {
+        const int32_t c_begin = (int32_t)cb * chans_per_block;
+        const int32_t c_end = (c_begin + chans_per_block < p.C) ? c_begin + chans_per_block : p.C;
+        first = c_begin / CB;
+        step1 = 1;
+        step2 = 1;
+        nchan = c_end - c_begin;
+    }
+    const int32_t switch_at = chans_per_block / CB;
+    auto unit_of = [&](int32_t s) -> int32_t {
+        return first + (s < switch_at ? s * step1 : switch_at * step1 + (s - switch_at) * step2);
+    };
     const int32_t steps = (nchan + CB - 1) / CB;
-    const T* go_n = gout + (n * p.C + c_begin) * (int64_t)points;
+    const T* go_n = gout + n * p.C * (int64_t)points;  // the batch item's gradOutput planes
     if (tid == 0) {
         spill_used = 0u;
     }
@@ -490,7 +513,7 @@ __global__ __launch_bounds__(kApplyThreads) void gs2d_grad_csr_apply_kernel(
         int32_t issued = 0;
         auto issue_next = [&]() {
             const uint32_t bytes = bytes_of(issued);
-            const char* src = src_lane + (size_t)issued * buf_bytes;
+            const char* src = src_lane + (size_t)unit_of(issued) * buf_bytes;
             char* dst = lds + (uint32_t)(issued % kApplyNbuf) * buf_bytes + lwave * 1024u;
             const uint32_t whole = bytes >> 10;
             uint32_t j = lwave;
@@ -595,7 +618,7 @@ __global__ __launch_bounds__(kApplyThreads) void gs2d_grad_csr_apply_kernel(
         kmax[i] = __builtin_amdgcn_readfirstlane(km);
         any_rest[i] = __builtin_amdgcn_readfirstlane(cm) > (uint32_t)kHeld;
     }
-    T* dx_c = dx + (n * p.C + c_begin) * (int64_t)plane_px;
+    T* dx_n = dx + n * p.C * (int64_t)plane_px;  // the batch item's gradient planes
     // the lists are in registers or LDS from here on: nothing below waits for memory except an overfull spill area
     __builtin_amdgcn_s_waitcnt(0);
 
@@ -686,7 +709,7 @@ __global__ __launch_bounds__(kApplyThreads) void gs2d_grad_csr_apply_kernel(
 #pragma unroll
                 for (int j = 0; j < CB; j++) {
                     if (s * CB + j < nchan) {
-                        F::store(dx_c + (int64_t)(s * CB + j) * plane_px + e[i], acc[j]);
+                        F::store(dx_n + (int64_t)(unit_of(s) * CB + j) * plane_px + e[i], acc[j]);
                     }
                 }
             }
@@ -702,6 +725,10 @@ struct CsrPlan {
     uint32_t tiles = 0, cblocks = 0;
     int32_t chans_per_block = 0;
     int xcd_swizzle = 0;
+    uint32_t items_fastest = 0;  // N when the apply kernel numbers its groups with the batch item fastest
+    uint32_t wide_blocks = 0;    // the first channel blocks take chans_wide channels each ...
+    int32_t chans_wide = 0;
+    int32_t unit_stride = 0;     // ... and units of cb channels are dealt out in turn, this many apart
     CsrLayout lay;
 };
 
@@ -751,6 +778,26 @@ CsrPlan make_plan(const GridSamplerGradArgs& a)
     pl.chans_per_block = (int32_t)cpb;
     pl.cblocks = (uint32_t)cblocks;
     pl.xcd_swizzle = ((a.N * cblocks) % 8 == 0) ? 1 : 0;
+    // The apply kernel numbers its groups with the batch item fastest where the items fill the XCDs evenly: an XCD then
+    // reads the lists of N / 8 items only (with the channel block fastest every XCD read every item's lists), and the
+    // channel blocks with the low numbers are the workgroups that are handed out first.
+    if (a.N % 8 == 0) {
+        pl.items_fastest = (uint32_t)a.N;
+    }
+    // Units of cb channels dealt out to the channel blocks in turn where every block's count is exact, and, with
+    // exactly two workgroups per CU, 5 channels for the first of a CU for every 3 of the second (gs2d_lds.hip has the
+    // why; backward of fp16 N16 C256 64x64, both gradients: 77.0 us with 32 + 32, 75.6 with 36 + 28, 74.9 with 38 + 26
+    // and 40 + 24, 75.7 with 42 + 22, 76.7 with 44 + 20).
+    if (a.C == cblocks * cpb && cblocks > 1) {
+        const int64_t wide = (cpb * 5 / 4) / pl.cb * pl.cb;
+        if (pl.items_fastest != 0 && cblocks % 2 == 0 && base * cblocks == 2 * (int64_t)compute_unit_count() &&
+            (a.N * cblocks / 2) % 8 == 0 && wide > cpb && wide < 2 * cpb) {
+            pl.wide_blocks = (uint32_t)(cblocks / 2);
+            pl.chans_wide = (int32_t)wide;
+            pl.chans_per_block = (int32_t)(2 * cpb - wide);
+        }
+        pl.unit_stride = (int32_t)cblocks;
+    }
     pl.lay = make_layout(points, plane_px, cells, pl.ipt);
     pl.ok = true;
     return pl;
@@ -796,7 +843,8 @@ hipError_t launch_apply(const GridSamplerGradArgs& a, const CsrPlan& pl, const G
     const uint32_t blocks = (uint32_t)(a.N * pl.tiles * pl.cblocks);
     const int lds_bytes = kApplyNbuf * CB * (int)(a.Hout * a.Wout) * (int)sizeof(T) + kApplySpill * 8;
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kApplyThreads), lds_bytes, stream, (const T*)a.gout, (T*)a.dx,
-                       (const uint32_t*)a.scratch, p, pl.lay, pl.tiles, pl.cblocks, pl.chans_per_block, pl.xcd_swizzle);
+                       (const uint32_t*)a.scratch, p, pl.lay, pl.tiles, pl.cblocks, pl.chans_per_block, pl.xcd_swizzle,
+                       pl.items_fastest, pl.wide_blocks, pl.chans_wide, pl.unit_stride);
     return hipGetLastError();
 }
 

@@ -101,4 +101,7 @@ const char* resize_lds_variant(const ResizeArgs& a);
 const char* grid_sampler2d_variant(const GridSamplerArgs& a);
 const char* resize_variant(const ResizeArgs& a);
 
+// CUs of the current device (256 on MI355X; also the answer where no device can be asked); gs2d_lds.hip
+int compute_unit_count();
+
 }  // namespace opscv

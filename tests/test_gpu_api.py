@@ -605,6 +605,28 @@ def test_grid_sampler2d_backward_grid_gradient_lds_variant(oracle, device, aclnn
                         (what, N, C, H, W, Ho, Wo, pad, align)
 
 
+@pytest.mark.parametrize("dtype", ("fp16", "fp32"))
+def test_grid_sampler2d_backward_launch_of_two_workgroups_per_cu(oracle, device, aclnn, dtype):
+    """a shape whose last kernel (the gather over the contribution lists) is launched as exactly two workgroups per CU
+    of a 256-CU part: the channel blocks handed out first take 10 channels, the others 6, in units dealt out in turn;
+    every channel's gradient must still be written once"""
+    torch = _torch()
+    rng = np.random.default_rng(640)
+    N, C, H, W, Ho, Wo = 16, 64, 64, 64, 64, 64
+    x = I.cast_np(rng.standard_normal((N, C, H, W)).astype(np.float32), dtype)
+    g = I.cast_np(I.affine_grid(rng, N, Ho, Wo), dtype)
+    go32 = rng.standard_normal((N, C, Ho, Wo)).astype(np.float32)
+    # every channel different from its neighbours by a constant, so that a channel taken twice or skipped shows
+    go32 += np.arange(C, dtype=np.float32).reshape(1, C, 1, 1) / 4
+    go = I.cast_np(go32, dtype)
+    tensors = [I.to_torch(v, dtype, device) for v in (go, x, g)]
+    rdx, rdg = oracle.grid_sampler2d_backward(go, x, g, 0, 0, False, dtype=I.oracle_code(dtype))
+    dx, dg = aclnn.grid_sampler2d_backward(*tensors, 0, 0, False)
+    torch.cuda.synchronize()
+    for got, ref, what in ((I.from_torch(dx, dtype), rdx, "dx"), (I.from_torch(dg, dtype), rdg, "dgrid")):
+        assert np.array_equal(_bits(got, dtype), _bits(ref, dtype)), what
+
+
 @pytest.mark.parametrize("dtype", I.DTYPES)
 def test_grid_sampler2d_backward_input_gradient_list_variant(oracle, device, aclnn, dtype):
     """The input gradient as a gather over per-element contribution lists (8 channels or more, up to 16384 grid
