@@ -385,6 +385,440 @@ __global__ __launch_bounds__(kThreadsLds) void gs2d_grad_grid_lds_kernel(
     }
 }
 
+
+// ---------------------------------------------------------------------------------------------------------------------
+// Two lanes per grid point.  The kernel above has one point wavefront per SIMD, and whatever that wavefront waits for
+// (a barrier, an LDS read) the SIMD waits for.  Here the lanes 2i and 2i + 1 of a wavefront own one grid point and the
+// channels of one parity each: a step is two planes, each lane reads the corners and the gradOutput value of its own
+// plane and forms its eight terms, and then both lanes add all sixteen terms of the step to the two running sums in
+// the reference's order -- the even channel's eight first, fetched from the even lane by a quad permutation that
+// rides on the add instruction, then the odd channel's.  Both lanes of a pair hold the same sums throughout; the even
+// one stores them.  Per step a lane issues 20 + 16 arithmetic instructions instead of 2 x 29, and a workgroup of 256
+// points has eight point wavefronts, two per SIMD, with half as many barriers each.  Needs an even channel count.
+constexpr int kPointWaves2 = 8;
+constexpr int kThreadsLds2 = (kPointWaves2 + kCopyWaves + 1) * 64;
+constexpr int kUnrollSteps = 8;  // steps per turn of the unrolled loop
+
+template <int CTRL>
+__device__ __forceinline__ float quad_from(float v)
+{
+    return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+
+template <typename T, int NBUF, int PITCH>
+__global__ __launch_bounds__(kThreadsLds2) void gs2d_grad_grid_lds2_kernel(
+    const T* __restrict__ gout, const T* __restrict__ x, const T* __restrict__ grid, T* __restrict__ dgrid, int32_t C,
+    int32_t H, int32_t W, int32_t points, uint32_t tiles_per_n, int32_t pad, int32_t align, int32_t xcd_swizzle,
+    int32_t ahead_x, float neg_zero, GradClear clear, int32_t Wo)
+{
+    constexpr int SBUF = NBUF / 2;  // steps the ring holds
+    static_assert(NBUF % 2 == 0 && kUnrollSteps % SBUF == 0, "a turn of the loop is whole turns of the ring");
+    static_assert(SBUF >= 4, "two steps held by the point wavefronts, two or more on their way");
+    extern __shared__ uint4 smem_raw[];
+    char* lds = reinterpret_cast<char*>(smem_raw);
+    constexpr int DEPTH = SBUF - 2;  // steps in flight ahead of the one whose values are being used
+    constexpr uint32_t GOUT_PITCH = kPoints * sizeof(T);
+    constexpr uint32_t GOUT_RING = NBUF * PITCH;
+    constexpr uint32_t DUMP = GOUT_RING + NBUF * GOUT_PITCH;
+    constexpr uint32_t BOX = DUMP + kDumpBytes;  // 4 words per point wavefront: the corners' row and column ranges
+    const int tid = threadIdx.x;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane((uint32_t)tid >> 6);
+
+    uint32_t n, tile;
+    if (xcd_swizzle) {
+        const uint32_t xcd = blockIdx.x & 7u, i = blockIdx.x >> 3;
+        n = (i / tiles_per_n) * 8u + xcd;
+        tile = i % tiles_per_n;
+    } else {
+        n = blockIdx.x / tiles_per_n;
+        tile = blockIdx.x % tiles_per_n;
+    }
+    const int32_t plane_elems = H * W;
+    const uint32_t plane_bytes = (uint32_t)plane_elems * (uint32_t)sizeof(T);
+    const uint32_t zero_off = round_up16(plane_bytes);
+    // the workgroup's 256 points are a block of 16 x 16 of the output (launch plan: both extents multiples of 16)
+    const uint32_t tiles_per_row = (uint32_t)Wo / 16u;
+    const uint32_t trow = tile / tiles_per_row, tcol = tile - trow * tiles_per_row;
+    // The box of the plane that the block's corners lie in, after the point wavefronts have published it (barrier):
+    // rows [ylo, yhi], columns [xa, xa + wb) on 16-byte boundaries.  Only the box is staged, as consecutive 16-byte
+    // units: unit u holds columns 8 / sizeof(T) * 2 ... of row ylo + u / row_units.
+    struct Box {
+        int32_t ylo, rows, xa, wb;
+    };
+    auto read_box = [&]() -> Box {
+        const int32_t* bw = reinterpret_cast<const int32_t*>(lds + BOX);
+        int32_t ylo = INT32_MAX, yhi = -1, xlo = INT32_MAX, xhi = -1;
+        for (int w8 = 0; w8 < kPointWaves2; w8++) {
+            const int32_t a = bw[w8 * 4 + 0], b2 = bw[w8 * 4 + 1], c2 = bw[w8 * 4 + 2], d2 = bw[w8 * 4 + 3];
+            ylo = a < ylo ? a : ylo;
+            yhi = b2 > yhi ? b2 : yhi;
+            xlo = c2 < xlo ? c2 : xlo;
+            xhi = d2 > xhi ? d2 : xhi;
+        }
+        constexpr int32_t EPU = 16 / (int32_t)sizeof(T);  // elements per 16-byte unit
+        Box bx;
+        if (yhi < 0) {  // no corner inside the image: a box of one unit that nobody reads
+            bx.ylo = 0;
+            bx.rows = 1;
+            bx.xa = 0;
+            bx.wb = EPU;
+        } else {
+            bx.ylo = ylo;
+            bx.rows = yhi - ylo + 1;
+            bx.xa = xlo / EPU * EPU;
+            const int32_t xe = (xhi + EPU) / EPU * EPU;  // one past the last column, rounded up
+            bx.wb = (xe < W ? xe : W) - bx.xa;
+        }
+        bx.ylo = __builtin_amdgcn_readfirstlane(bx.ylo);
+        bx.rows = __builtin_amdgcn_readfirstlane(bx.rows);
+        bx.xa = __builtin_amdgcn_readfirstlane(bx.xa);
+        bx.wb = __builtin_amdgcn_readfirstlane(bx.wb);
+        return bx;
+    };
+    const int32_t steps_real = C / 2;                                                  // C is even (launch plan)
+    const int32_t steps = (steps_real + kUnrollSteps - 1) / kUnrollSteps * kUnrollSteps;  // steps the workgroup walks
+
+    if (wave == (uint32_t)(kPointWaves2 + kCopyWaves)) {
+        // ------------------------------------------------ prefetch wavefront -----------------------------------
+        const uint32_t lane = (uint32_t)tid & 63u;
+        char* dump = lds + DUMP;
+        const char* xb = reinterpret_cast<const char*>(x + (int64_t)n * C * plane_elems);
+        const bool whole_lines = (reinterpret_cast<uintptr_t>(xb) % 128u == 0) && (plane_bytes % 128u == 0);
+        const uint32_t touches = plane_bytes / 128u + (whole_lines ? 0u : 1u);
+        int32_t mine = (int32_t)tile;
+        auto touch_plane = [&](int32_t c) {
+            if (c == mine) {
+                mine += (int32_t)tiles_per_n;
+                if (c < C) {
+                    const char* pl = xb + (size_t)c * plane_bytes;
+                    for (uint32_t j = lane; j < touches; j += 64u) {
+                        const uint32_t off = j * 128u;
+                        touch_line(pl + (off < plane_bytes ? off : plane_bytes - 1u), dump);
+                    }
+                }
+            }
+        };
+        // the block's sixteen gradOutput segments of a channel (32 or 64 bytes each): sixteen lanes per channel
+        const size_t gstep = (size_t)4 * points * sizeof(T);
+        const char* gp = reinterpret_cast<const char*>(gout + ((int64_t)n * C + (lane >> 4)) * points +
+                                                       (int64_t)(trow * 16u + (lane & 15u)) * Wo + tcol * 16u);
+        int32_t gc = (int32_t)(lane >> 4);
+        auto touch_gout = [&]() {
+            if (gc < C) {
+                touch_line(gp, dump);
+            }
+            gp += gstep;
+            gc += 4;
+        };
+        for (int32_t c = 0; c < ahead_x; c++) {
+            touch_plane(c);
+        }
+        for (int32_t c0 = 0; c0 < kAheadGout; c0 += 4) {
+            touch_gout();
+        }
+        lds_barrier();  // the box is published (nothing to do with it here)
+        for (int32_t s = 0; s <= steps + 1; s++) {
+            touch_plane(2 * s + ahead_x);
+            touch_plane(2 * s + 1 + ahead_x);
+            if ((s & 1) == 0) {
+                touch_gout();
+            }
+            lds_barrier();  // keeps pace with the ring: one barrier per step, and two more
+        }
+        wait_vmcnt_imm<0>();
+        return;
+    }
+    if (wave >= (uint32_t)kPointWaves2) {
+        // ------------------------------------------------ loader wavefronts ------------------------------------
+        const uint32_t lwave = wave - kPointWaves2;
+        const uint32_t lane = (uint32_t)tid & 63u;
+        const char* xb = reinterpret_cast<const char*>(x + (int64_t)n * C * plane_elems);
+        lds_barrier();  // the box is published
+        const Box box = read_box();
+        constexpr int32_t EPU = 16 / (int32_t)sizeof(T);
+        const uint32_t row_units = (uint32_t)(box.wb / EPU);
+        const uint32_t units = (uint32_t)box.rows * row_units;    // 16-byte units of the box
+        const uint32_t instrs = (units + 63u) / 64u;              // copy instructions per plane, all loaders together
+        const uint32_t my_instrs = (instrs > lwave) ? (instrs - lwave + kCopyWaves - 1) / kCopyWaves : 0u;
+        auto ring_loop = [&](auto pp_tag, auto go_tag) {
+            constexpr int PP = decltype(pp_tag)::value;  // copies per plane of this loader
+            constexpr int GO = decltype(go_tag)::value;
+            constexpr int PER_STEP = 2 * (PP + GO);
+            // The lane's 16 bytes of its wavefront's j-th instruction: unit (j * loaders + lwave) * 64 + lane of the
+            // box; a lane past the box's last unit copies the last unit again (its LDS place, behind the box, is
+            // nobody's).
+            uint32_t goffs[PP > 0 ? PP : 1];
+#pragma unroll
+            for (int j = 0; j < PP; j++) {
+                uint32_t u = ((uint32_t)j * kCopyWaves + lwave) * 64u + lane;
+                u = u < units ? u : units - 1u;
+                const uint32_t row = u / row_units, col = u - row * row_units;
+                goffs[j] = (((uint32_t)box.ylo + row) * (uint32_t)W + (uint32_t)box.xa + col * (uint32_t)EPU) *
+                           (uint32_t)sizeof(T);
+            }
+            const char* src = xb;
+            uint32_t slot_off = lwave * 1024u;
+            // gradOutput of the block: per channel 256 values in point order, sixteen segments of sixteen points
+            constexpr uint32_t GLANES = kPoints * sizeof(T) / 16u;
+            const uint32_t p0 = lane * (uint32_t)EPU;  // the lane's first point
+            const char* gsrc = reinterpret_cast<const char*>(
+                gout + (int64_t)n * C * points + (int64_t)(trow * 16u + (p0 >> 4)) * Wo + tcol * 16u + (p0 & 15u));
+            const bool glane = lane < GLANES;
+            const size_t gstep = (size_t)points * sizeof(T);
+            uint32_t gslot_off = GOUT_RING;
+            int fill = 0;  // step slot being filled
+            auto issue = [&]() {
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+#pragma unroll
+                    for (int j = 0; j < PP; j++) {
+                        __builtin_amdgcn_global_load_lds(
+                            (global_cptr_t)(src + (size_t)h * plane_bytes + goffs[j]),
+                            (lds_ptr_t)(lds + slot_off + h * PITCH + j * (kCopyWaves * 1024)), 16, 0, 0);
+                    }
+                }
+                if constexpr (GO) {
+                    if (glane) {
+                        __builtin_amdgcn_global_load_lds((global_cptr_t)gsrc, (lds_ptr_t)(lds + gslot_off), 16, 0, 0);
+                        __builtin_amdgcn_global_load_lds((global_cptr_t)(gsrc + gstep),
+                                                         (lds_ptr_t)(lds + gslot_off + GOUT_PITCH), 16, 0, 0);
+                    }
+                    gsrc += 2 * gstep;
+                }
+                src += (size_t)2 * plane_bytes;
+                fill = (fill + 1 == SBUF) ? 0 : fill + 1;
+                slot_off = (uint32_t)fill * (2 * PITCH) + lwave * 1024u;
+                gslot_off = GOUT_RING + (uint32_t)fill * (2 * GOUT_PITCH);
+            };
+            for (int i = 0; i < DEPTH; i++) {
+                issue();
+            }
+            for (int32_t s = 0; s < steps_real - DEPTH; s++) {
+                wait_vmcnt_imm<(DEPTH - 1) * PER_STEP>();  // step s has landed: the DEPTH - 1 after it may be out
+                lds_barrier();                             // ... and the slots of step s - 2 are free
+                issue();
+            }
+            ring_rundown<DEPTH - 1, PER_STEP>();
+            for (int32_t s = steps_real; s <= steps + 1; s++) {
+                lds_barrier();
+            }
+        };
+        auto with_pp = [&](auto pp_tag) {
+            constexpr int PP = decltype(pp_tag)::value;
+            if constexpr ((SBUF - 3) * 2 * (PP + 1) <= 63 && PP * kCopyWaves * 1024 + 16 <= PITCH + kCopyWaves * 1024) {
+                if (lwave == 0) {
+                    ring_loop(pp_tag, std::integral_constant<int, 1>{});
+                } else {
+                    ring_loop(pp_tag, std::integral_constant<int, 0>{});
+                }
+            } else {
+                for (int32_t s = 0; s <= steps + 1; s++) {
+                    lds_barrier();
+                }
+            }
+        };
+        switch (my_instrs) {  // at most plane_bytes / 4 KiB, which the launch plan limits to 4
+            case 0: with_pp(std::integral_constant<int, 0>{}); break;
+            case 1: with_pp(std::integral_constant<int, 1>{}); break;
+            case 2: with_pp(std::integral_constant<int, 2>{}); break;
+            case 3: with_pp(std::integral_constant<int, 3>{}); break;
+            default: with_pp(std::integral_constant<int, 4>{}); break;
+        }
+        return;
+    }
+
+    // ---------------------------------------------------- point wavefronts -------------------------------------
+    if (tid < NBUF * 4) {
+        reinterpret_cast<uint32_t*>(lds + (tid >> 2) * PITCH + zero_off)[tid & 3] = 0u;
+    }
+    if (clear.count != 0u) {
+        uint32_t* words = clear.base + (size_t)n * clear.item_words;
+        const uint32_t share = (clear.count + tiles_per_n - 1u) / tiles_per_n;
+        const uint32_t from = tile * share;
+        const uint32_t to = (from + share < clear.count) ? from + share : clear.count;
+        for (uint32_t i = from + (uint32_t)tid; i < to; i += (uint32_t)(kPointWaves2 * 64)) {
+            words[clear.first + i] = 0u;
+        }
+        if (tile == 0u && tid == 0) {
+            words[clear.single] = 0u;
+        }
+    }
+    const uint32_t parity = (uint32_t)tid & 1u;  // the lane's channels: parity, parity + 2, ...
+    const int32_t pt = tid >> 1;                 // its point inside the block: row pt / 16, column pt % 16
+    const int32_t pix = (int32_t)((trow * 16u + (uint32_t)(pt >> 4)) * (uint32_t)Wo + tcol * 16u + (uint32_t)(pt & 15));
+    const bool live = true;  // whole blocks only (launch plan)
+    const int64_t idx = (int64_t)n * points + pix;
+    GradTaps<T, 0> tp;
+    decide_grad_taps<T, 0>(tp, ElemIO<T>::load(grid + 2 * idx), ElemIO<T>::load(grid + 2 * idx + 1), H, W, pad, align);
+    // the rows and columns of the lane's corners inside the image, then of the wavefront's, for the box
+    {
+        const int32_t x1 = (tp.x0 == INT32_MAX) ? tp.x0 : tp.x0 + 1, y1 = (tp.y0 == INT32_MAX) ? tp.y0 : tp.y0 + 1;
+        const bool in0 = tp.off[0] >= 0, in1 = tp.off[1] >= 0, in2 = tp.off[2] >= 0, in3 = tp.off[3] >= 0;
+        int32_t ylo = INT32_MAX, yhi = -1, xlo = INT32_MAX, xhi = -1;
+        if (in0 || in1) {
+            ylo = tp.y0;
+            yhi = tp.y0;
+        }
+        if (in2 || in3) {
+            ylo = ylo < y1 ? ylo : y1;
+            yhi = y1;
+        }
+        if (in0 || in2) {
+            xlo = tp.x0;
+            xhi = tp.x0;
+        }
+        if (in1 || in3) {
+            xlo = xlo < x1 ? xlo : x1;
+            xhi = x1;
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const int32_t a = __shfl_xor(ylo, o), b2 = __shfl_xor(yhi, o), c2 = __shfl_xor(xlo, o), d2 = __shfl_xor(xhi, o);
+            ylo = a < ylo ? a : ylo;
+            yhi = b2 > yhi ? b2 : yhi;
+            xlo = c2 < xlo ? c2 : xlo;
+            xhi = d2 > xhi ? d2 : xhi;
+        }
+        if ((tid & 63) == 0) {
+            int32_t* bw = reinterpret_cast<int32_t*>(lds + BOX) + wave * 4u;
+            bw[0] = ylo;
+            bw[1] = yhi;
+            bw[2] = xlo;
+            bw[3] = xhi;
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    lds_barrier();  // every wavefront's ranges are in LDS
+    const Box box = read_box();
+    const float dxe = (float)(tp.x0 == INT32_MAX ? tp.x0 : tp.x0 + 1) - tp.fx, dxw = tp.fx - (float)tp.x0;
+    const float dys = (float)(tp.y0 == INT32_MAX ? tp.y0 : tp.y0 + 1) - tp.fy, dyn = tp.fy - (float)tp.y0;
+    uint32_t taddr[4], taddr_hi[4];  // in the first step slot, and in step slot SBUF / 2
+    uint32_t keep[4];
+    {
+        uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
+        asm volatile("" : "+s"(lds_base));
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const bool in = tp.off[k] >= 0;
+            // the corner's place in the staged box
+            const int32_t cy = (k < 2) ? tp.y0 : tp.y0 + 1, cx = (k & 1) ? tp.x0 + 1 : tp.x0;
+            const uint32_t boff = (uint32_t)((cy - box.ylo) * box.wb + (cx - box.xa)) * (uint32_t)sizeof(T);
+            taddr[k] = lds_base + parity * PITCH + (in ? boff : zero_off);
+            asm volatile("" : "+v"(taddr[k]));
+            taddr_hi[k] = taddr[k] + (SBUF / 2) * (2 * PITCH);
+            asm volatile("" : "+v"(taddr_hi[k]));
+            keep[k] = in ? 0xFFFFFFFFu : 0u;
+        }
+    }
+    uint32_t gaddr;
+    {
+        uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
+        asm volatile("" : "+s"(lds_base));
+        gaddr = lds_base + GOUT_RING + parity * GOUT_PITCH + (uint32_t)pt * (uint32_t)sizeof(T);
+        asm volatile("" : "+v"(gaddr));
+    }
+    float gix = 0.0f, giy = 0.0f;
+    auto term = [&](uint32_t vraw, float d, uint32_t gobits) -> float {
+        const float t = __builtin_fmaf(tap_value<T>(vraw), d, neg_zero);
+        return __builtin_fmaf(tap_value<T>(gobits), t, neg_zero);
+    };
+    uint32_t r0[5], r1[5];  // four corners and the gradOutput value of the lane's plane of step s and of step s + 1
+    auto read_one = [&](int slot, int k, uint32_t* r) {  // slot: step slot
+        if (k == 4) {
+            load_taps<T, 1>((uint32_t)(slot * 2 * GOUT_PITCH), &gaddr, r + 4);
+        } else if (slot < SBUF / 2) {
+            load_taps<T, 1>((uint32_t)(slot * 2 * PITCH), taddr + k, r + k);
+        } else {
+            load_taps<T, 1>((uint32_t)((slot - SBUF / 2) * 2 * PITCH), taddr_hi + k, r + k);
+        }
+    };
+    auto read_step = [&](int slot, uint32_t* r) {
+#pragma unroll
+        for (int k = 0; k < 5; k++) {
+            read_one(slot, k, r);
+        }
+    };
+    constexpr int kFromEven = 0xA0;  // quad permutation [0, 0, 2, 2]: the even lane of each pair
+    constexpr int kFromOdd = 0xF5;   // [1, 1, 3, 3]: the odd lane
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // the zero-slot writes, before the first barrier publishes them
+    lds_barrier();                        // step 0 has landed
+    read_step(0, r0);
+    lds_barrier();                        // step 1 has landed
+    read_step(1 % SBUF, r1);
+    auto turn = [&](auto masked, int32_t b) {
+#pragma unroll
+        for (int u = 0; u < kUnrollSteps; u++) {
+            const int32_t st = b + u;
+            uint32_t v0 = r0[0], v1 = r0[1], v2 = r0[2], v3 = r0[3], g = r0[4];
+            uint32_t r2[5];
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_waitcnt(0xC57F);  // lgkmcnt(5): the reads of step st are back
+            lds_barrier();                       // step st + 2 has landed (or there is none)
+            __builtin_amdgcn_sched_barrier(0);
+            if constexpr (decltype(masked)::value) {
+                const uint32_t m = (st < steps_real) ? 0xFFFFFFFFu : 0u;
+                v0 &= m;
+                v1 &= m;
+                v2 &= m;
+                v3 &= m;
+                g &= m;
+            }
+            const uint32_t g0 = g & keep[0], g1 = g & keep[1], g2 = g & keep[2], g3 = g & keep[3];
+            const int slot = (u + 2) % SBUF;
+            // the lane's own eight terms (grid_sampler2_d_grad_simt_det.h:150-185), the reads of step st + 2 between them
+            read_one(slot, 0, r2);
+            __builtin_amdgcn_sched_barrier(0);
+            const float t0x = term(v0, dys, g0), t0y = term(v0, dxe, g0);
+            __builtin_amdgcn_sched_barrier(0);
+            read_one(slot, 1, r2);
+            __builtin_amdgcn_sched_barrier(0);
+            const float t1x = term(v1, dys, g1), t1y = term(v1, dxw, g1);
+            __builtin_amdgcn_sched_barrier(0);
+            read_one(slot, 2, r2);
+            __builtin_amdgcn_sched_barrier(0);
+            const float t2x = term(v2, dyn, g2), t2y = term(v2, dxe, g2);
+            __builtin_amdgcn_sched_barrier(0);
+            read_one(slot, 3, r2);
+            read_one(slot, 4, r2);
+            __builtin_amdgcn_sched_barrier(0);
+            const float t3x = term(v3, dyn, g3), t3y = term(v3, dxw, g3);
+            // both channels' terms onto the running sums, the even channel first
+            gix -= quad_from<kFromEven>(t0x);
+            giy -= quad_from<kFromEven>(t0y);
+            gix += quad_from<kFromEven>(t1x);
+            giy -= quad_from<kFromEven>(t1y);
+            gix -= quad_from<kFromEven>(t2x);
+            giy += quad_from<kFromEven>(t2y);
+            gix += quad_from<kFromEven>(t3x);
+            giy += quad_from<kFromEven>(t3y);
+            gix -= quad_from<kFromOdd>(t0x);
+            giy -= quad_from<kFromOdd>(t0y);
+            gix += quad_from<kFromOdd>(t1x);
+            giy -= quad_from<kFromOdd>(t1y);
+            gix -= quad_from<kFromOdd>(t2x);
+            giy += quad_from<kFromOdd>(t2y);
+            gix += quad_from<kFromOdd>(t3x);
+            giy += quad_from<kFromOdd>(t3y);
+#pragma unroll
+            for (int k = 0; k < 5; k++) {
+                r0[k] = r1[k];
+                r1[k] = r2[k];
+            }
+        }
+    };
+    int32_t b = 0;
+    for (; b + kUnrollSteps <= steps_real; b += kUnrollSteps) {
+        turn(std::false_type{}, b);
+    }
+    if (b < steps_real) {
+        turn(std::true_type{}, b);
+    }
+    if (live && parity == 0u) {
+        ElemIO<T>::store(dgrid + 2 * idx, as_fp32_value(tp.mx * gix));
+        ElemIO<T>::store(dgrid + 2 * idx + 1, as_fp32_value(tp.my * giy));
+    }
+}
+
 struct GridLdsPlan {
     bool ok = false;
     int cls = 0;
@@ -427,8 +861,42 @@ GridLdsPlan make_plan(const GridSamplerGradArgs& a)
 }
 
 template <typename T, int CLS>
+hipError_t launch_cls2(const GridSamplerGradArgs& a, const GridLdsPlan& p, const GradClear& clear, hipStream_t stream)
+{
+    auto kernel = gs2d_grad_grid_lds2_kernel<T, kGradNbuf[CLS], kGradPitch[CLS]>;
+    // the rings, the prefetch wavefront's dump area, and four words per point wavefront for the box
+    constexpr int lds_bytes = kGradNbuf[CLS] * (kGradPitch[CLS] + kPoints * (int)sizeof(T)) + kDumpBytes + kPointWaves2 * 16;
+    static_assert(lds_bytes <= kLdsLimit, "the rings fit a CU's LDS");
+    static std::atomic<uint32_t> lds_allowed{0};
+    const hipError_t ea = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), lds_bytes, lds_allowed);
+    if (ea != hipSuccess) {
+        return ea;
+    }
+    const uint32_t blocks = (uint32_t)(a.N * p.tiles_per_n);
+    const int64_t plane_bytes = a.Hin * a.Win * (int64_t)sizeof(T);
+    int64_t ahead = 262144 / plane_bytes;
+    ahead = ahead > 64 ? 64 : ahead;
+    if (ahead < kGradNbuf[CLS]) {
+        ahead = kGradNbuf[CLS];
+    }
+    hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kThreadsLds2), lds_bytes, stream, (const T*)a.gout, (const T*)a.x,
+                       (const T*)a.grid, (T*)a.dgrid, (int32_t)a.C, (int32_t)a.Hin, (int32_t)a.Win,
+                       (int32_t)(a.Hout * a.Wout), p.tiles_per_n, (int32_t)a.pad, (int32_t)a.align, p.xcd_swizzle,
+                       (int32_t)ahead, -0.0f, clear, (int32_t)a.Wout);
+    return hipGetLastError();
+}
+
+template <typename T, int CLS>
 hipError_t launch_cls(const GridSamplerGradArgs& a, const GridLdsPlan& p, const GradClear& clear, hipStream_t stream)
 {
+    if constexpr (CLS <= 1) {
+        // two lanes per grid point and the planes' boxes only: an even channel count with steps enough to fill the
+        // ring, an output of whole 16 x 16 blocks, input rows of whole 16-byte units
+        if (a.C % 2 == 0 && a.C / 2 >= kGradNbuf[CLS] / 2 && a.Wout % 16 == 0 && a.Hout % 16 == 0 &&
+            a.Win % (16 / (int)sizeof(T)) == 0 && a.Hin * a.Win * (int64_t)sizeof(T) <= 4 * kCopyWaves * 1024) {
+            return launch_cls2<T, CLS>(a, p, clear, stream);
+        }
+    }
     auto kernel = gs2d_grad_grid_lds_kernel<T, kGradNbuf[CLS], kGradPitch[CLS]>;
     constexpr int lds_bytes = kGradNbuf[CLS] * (kGradPitch[CLS] + kPoints * (int)sizeof(T)) + kDumpBytes;
     static_assert(lds_bytes <= kLdsLimit, "the rings fit a CU's LDS");

@@ -605,6 +605,45 @@ def test_grid_sampler2d_backward_grid_gradient_lds_variant(oracle, device, aclnn
                         (what, N, C, H, W, Ho, Wo, pad, align)
 
 
+@pytest.mark.parametrize("dtype", I.DTYPES)
+def test_grid_sampler2d_backward_grid_gradient_box_variant(oracle, device, aclnn, dtype):
+    """The grid gradient with two lanes per grid point and only the box of each plane staged that a 16 x 16 block of
+    grid points reaches (even channel counts, outputs of whole 16 x 16 blocks): smooth grids whose boxes are a small
+    part of the plane, a batch item whose points all lie outside the image (empty boxes), blocks that straddle the
+    image's edge, random grids (the box is the whole plane), special grid values, both plane size classes, channel
+    counts that leave a partial turn of the unrolled loop, every padding and alignment"""
+    torch = _torch()
+    rng = np.random.default_rng(650)
+    shapes = [(8, 16, 64, 64, 64, 64), (8, 22, 32, 64, 48, 96), (4, 36, 64, 128 if dtype != "fp32" else 64, 64, 128)]
+    for (N, C, H, W, Ho, Wo) in shapes:
+        x = I.cast_np(rng.standard_normal((N, C, H, W)).astype(np.float32), dtype)
+        g32 = I.affine_grid(rng, N, Ho, Wo)
+        g32[1] = g32[1] * 0.2 + 3.0                                   # every point outside the image
+        g32[2] = rng.uniform(-1.2, 1.2, (Ho, Wo, 2)).astype(np.float32)  # the box is the whole plane
+        g32[3] = g32[3] * 0.3 + 0.85                                  # a small patch across the image's corner
+        flat = g32[0].reshape(-1, 2)
+        special = np.array([np.nan, np.inf, -np.inf, 1e30, -1e30, 1.0, -1.0, 0.0], np.float32)
+        for j in range(len(special)):
+            flat[17 * j + 3, j % 2] = special[j]
+        g = I.cast_np(g32, dtype)
+        go32 = rng.standard_normal((N, C, Ho, Wo)).astype(np.float32)
+        go32 += np.arange(C, dtype=np.float32).reshape(1, C, 1, 1) / 8
+        go32[0, 1, 0, 5] = np.inf
+        go32[3, C - 1, Ho - 1, Wo - 1] = np.nan
+        go = I.cast_np(go32, dtype)
+        for pad in range(3):
+            for align in (False, True):
+                rdx, rdg = oracle.grid_sampler2d_backward(go, x, g, 0, pad, align, dtype=I.oracle_code(dtype))
+                dx, dg = aclnn.grid_sampler2d_backward(I.to_torch(go, dtype, device), I.to_torch(x, dtype, device),
+                                                       I.to_torch(g, dtype, device), 0, pad, align)
+                torch.cuda.synchronize()
+                for got, ref, what in ((I.from_torch(dx, dtype), rdx, "dx"), (I.from_torch(dg, dtype), rdg, "dgrid")):
+                    rn = np.isnan(I.as_f32(ref, dtype))
+                    assert np.array_equal(np.isnan(I.as_f32(got, dtype)), rn), (what, N, C, H, W, pad, align)
+                    assert np.array_equal(np.where(rn, 0, _bits(got, dtype)), np.where(rn, 0, _bits(ref, dtype))), \
+                        (what, N, C, H, W, Ho, Wo, pad, align)
+
+
 @pytest.mark.parametrize("dtype", ("fp16", "fp32"))
 def test_grid_sampler2d_backward_launch_of_two_workgroups_per_cu(oracle, device, aclnn, dtype):
     """a shape whose last kernel (the gather over the contribution lists) is launched as exactly two workgroups per CU
