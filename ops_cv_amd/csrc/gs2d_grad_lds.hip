@@ -388,22 +388,21 @@ __global__ __launch_bounds__(kThreadsLds) void gs2d_grad_grid_lds_kernel(
 
 // ---------------------------------------------------------------------------------------------------------------------
 // Two lanes per grid point.  The kernel above has one point wavefront per SIMD, and whatever that wavefront waits for
-// (a barrier, an LDS read) the SIMD waits for.  Here the lanes 2i and 2i + 1 of a wavefront own one grid point and the
-// channels of one parity each: a step is two planes, each lane reads the corners and the gradOutput value of its own
-// plane and forms its eight terms, and then both lanes add all sixteen terms of the step to the two running sums in
-// the reference's order -- the even channel's eight first, fetched from the even lane by a quad permutation that
-// rides on the add instruction, then the odd channel's.  Both lanes of a pair hold the same sums throughout; the even
-// one stores them.  Per step a lane issues 20 + 16 arithmetic instructions instead of 2 x 29, and a workgroup of 256
-// points has eight point wavefronts, two per SIMD, with half as many barriers each.  Needs an even channel count.
+// (a barrier, an LDS read) the SIMD waits for.  Here the lanes 2i and 2i + 1 of a wavefront own one grid point and one
+// component of its gradient each: both read the four corners and the gradOutput value of every plane, the even lane
+// multiplies by the row distances and keeps the x sum, the odd lane by the column distances and keeps the y sum.  The
+// two sums are independent chains in the reference too, so nothing is exchanged and each sum sees its terms in the
+// reference's order.  A step is two planes (half as many barriers); per step a lane issues 32 arithmetic instructions
+// where a lane of the kernel above issues 58, and a workgroup of 256 points has eight point wavefronts, two per SIMD.
+// Needs an even channel count.
+//
+// Only the box of each plane is staged that the workgroup's points reach: the 256 points are a block of 16 x 16 of the
+// output, whose corners under a smooth grid lie in a small part of the plane.  The point wavefronts find the box first
+// (rows and columns of the corners inside the image, reduced over the wavefronts through LDS), the loaders copy it
+// as consecutive 16-byte units, the corners' LDS offsets are taken inside the box.
 constexpr int kPointWaves2 = 8;
 constexpr int kThreadsLds2 = (kPointWaves2 + kCopyWaves + 1) * 64;
 constexpr int kUnrollSteps = 8;  // steps per turn of the unrolled loop
-
-template <int CTRL>
-__device__ __forceinline__ float quad_from(float v)
-{
-    return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
-}
 
 template <typename T, int NBUF, int PITCH>
 __global__ __launch_bounds__(kThreadsLds2) void gs2d_grad_grid_lds2_kernel(
@@ -643,10 +642,10 @@ __global__ __launch_bounds__(kThreadsLds2) void gs2d_grad_grid_lds2_kernel(
             words[clear.single] = 0u;
         }
     }
-    const uint32_t parity = (uint32_t)tid & 1u;  // the lane's channels: parity, parity + 2, ...
+    const uint32_t parity = (uint32_t)tid & 1u;  // the lane's sum: 0 the x component of the point's gradient, 1 the y
     const int32_t pt = tid >> 1;                 // its point inside the block: row pt / 16, column pt % 16
     const int32_t pix = (int32_t)((trow * 16u + (uint32_t)(pt >> 4)) * (uint32_t)Wo + tcol * 16u + (uint32_t)(pt & 15));
-    const bool live = true;  // whole blocks only (launch plan)
+    // (whole blocks only -- launch plan -- so every lane's point exists)
     const int64_t idx = (int64_t)n * points + pix;
     GradTaps<T, 0> tp;
     decide_grad_taps<T, 0>(tp, ElemIO<T>::load(grid + 2 * idx), ElemIO<T>::load(grid + 2 * idx + 1), H, W, pad, align);
@@ -703,7 +702,7 @@ __global__ __launch_bounds__(kThreadsLds2) void gs2d_grad_grid_lds2_kernel(
             // the corner's place in the staged box
             const int32_t cy = (k < 2) ? tp.y0 : tp.y0 + 1, cx = (k & 1) ? tp.x0 + 1 : tp.x0;
             const uint32_t boff = (uint32_t)((cy - box.ylo) * box.wb + (cx - box.xa)) * (uint32_t)sizeof(T);
-            taddr[k] = lds_base + parity * PITCH + (in ? boff : zero_off);
+            taddr[k] = lds_base + (in ? boff : zero_off);
             asm volatile("" : "+v"(taddr[k]));
             taddr_hi[k] = taddr[k] + (SBUF / 2) * (2 * PITCH);
             asm volatile("" : "+v"(taddr_hi[k]));
@@ -714,32 +713,42 @@ __global__ __launch_bounds__(kThreadsLds2) void gs2d_grad_grid_lds2_kernel(
     {
         uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
         asm volatile("" : "+s"(lds_base));
-        gaddr = lds_base + GOUT_RING + parity * GOUT_PITCH + (uint32_t)pt * (uint32_t)sizeof(T);
+        gaddr = lds_base + GOUT_RING + (uint32_t)pt * (uint32_t)sizeof(T);
         asm volatile("" : "+v"(gaddr));
     }
-    float gix = 0.0f, giy = 0.0f;
+    // The lane's four signed distances: its sum takes  -t0 +t1 -t2 +t3  of the products with the row distances (x
+    // component) or  -t0 -t1 +t2 +t3  of those with the column distances (y component), grid_sampler2_d_grad_simt_det.h:
+    // 150-185; the sign goes into the distance (a - b is a + (-b) bit for bit, and negating a factor negates the
+    // rounded product), so that both lanes run the same instructions.
+    float dk[4];
+    dk[0] = parity ? -dxe : -dys;
+    dk[1] = parity ? -dxw : dys;
+    dk[2] = parity ? dxe : -dyn;
+    dk[3] = parity ? dxw : dyn;
+    float acc = 0.0f;
+    // (v * d) * go as two fused multiply-adds onto -0: bit for bit the two rounded products
     auto term = [&](uint32_t vraw, float d, uint32_t gobits) -> float {
         const float t = __builtin_fmaf(tap_value<T>(vraw), d, neg_zero);
         return __builtin_fmaf(tap_value<T>(gobits), t, neg_zero);
     };
-    uint32_t r0[5], r1[5];  // four corners and the gradOutput value of the lane's plane of step s and of step s + 1
+    // reads 0..4: the corners and the gradOutput value of the step's first plane, 5..9: of its second
+    uint32_t r0[10], r1[10];
     auto read_one = [&](int slot, int k, uint32_t* r) {  // slot: step slot
-        if (k == 4) {
-            load_taps<T, 1>((uint32_t)(slot * 2 * GOUT_PITCH), &gaddr, r + 4);
+        const int h = k / 5, c = k % 5;
+        if (c == 4) {
+            load_taps<T, 1>((uint32_t)((slot * 2 + h) * GOUT_PITCH), &gaddr, r + k);
         } else if (slot < SBUF / 2) {
-            load_taps<T, 1>((uint32_t)(slot * 2 * PITCH), taddr + k, r + k);
+            load_taps<T, 1>((uint32_t)((slot * 2 + h) * PITCH), taddr + c, r + k);
         } else {
-            load_taps<T, 1>((uint32_t)((slot - SBUF / 2) * 2 * PITCH), taddr_hi + k, r + k);
+            load_taps<T, 1>((uint32_t)(((slot - SBUF / 2) * 2 + h) * PITCH), taddr_hi + c, r + k);
         }
     };
     auto read_step = [&](int slot, uint32_t* r) {
 #pragma unroll
-        for (int k = 0; k < 5; k++) {
+        for (int k = 0; k < 10; k++) {
             read_one(slot, k, r);
         }
     };
-    constexpr int kFromEven = 0xA0;  // quad permutation [0, 0, 2, 2]: the even lane of each pair
-    constexpr int kFromOdd = 0xF5;   // [1, 1, 3, 3]: the odd lane
     __builtin_amdgcn_s_waitcnt(0xC07F);  // the zero-slot writes, before the first barrier publishes them
     lds_barrier();                        // step 0 has landed
     read_step(0, r0);
@@ -749,58 +758,41 @@ __global__ __launch_bounds__(kThreadsLds2) void gs2d_grad_grid_lds2_kernel(
 #pragma unroll
         for (int u = 0; u < kUnrollSteps; u++) {
             const int32_t st = b + u;
-            uint32_t v0 = r0[0], v1 = r0[1], v2 = r0[2], v3 = r0[3], g = r0[4];
-            uint32_t r2[5];
+            uint32_t cur[10];
+#pragma unroll
+            for (int k = 0; k < 10; k++) {
+                cur[k] = r0[k];
+            }
+            uint32_t r2[10];
             __builtin_amdgcn_sched_barrier(0);
-            __builtin_amdgcn_s_waitcnt(0xC57F);  // lgkmcnt(5): the reads of step st are back
+            __builtin_amdgcn_s_waitcnt(0xCA7F);  // lgkmcnt(10): the reads of step st are back
             lds_barrier();                       // step st + 2 has landed (or there is none)
             __builtin_amdgcn_sched_barrier(0);
             if constexpr (decltype(masked)::value) {
                 const uint32_t m = (st < steps_real) ? 0xFFFFFFFFu : 0u;
-                v0 &= m;
-                v1 &= m;
-                v2 &= m;
-                v3 &= m;
-                g &= m;
-            }
-            const uint32_t g0 = g & keep[0], g1 = g & keep[1], g2 = g & keep[2], g3 = g & keep[3];
-            const int slot = (u + 2) % SBUF;
-            // the lane's own eight terms (grid_sampler2_d_grad_simt_det.h:150-185), the reads of step st + 2 between them
-            read_one(slot, 0, r2);
-            __builtin_amdgcn_sched_barrier(0);
-            const float t0x = term(v0, dys, g0), t0y = term(v0, dxe, g0);
-            __builtin_amdgcn_sched_barrier(0);
-            read_one(slot, 1, r2);
-            __builtin_amdgcn_sched_barrier(0);
-            const float t1x = term(v1, dys, g1), t1y = term(v1, dxw, g1);
-            __builtin_amdgcn_sched_barrier(0);
-            read_one(slot, 2, r2);
-            __builtin_amdgcn_sched_barrier(0);
-            const float t2x = term(v2, dyn, g2), t2y = term(v2, dxe, g2);
-            __builtin_amdgcn_sched_barrier(0);
-            read_one(slot, 3, r2);
-            read_one(slot, 4, r2);
-            __builtin_amdgcn_sched_barrier(0);
-            const float t3x = term(v3, dyn, g3), t3y = term(v3, dxw, g3);
-            // both channels' terms onto the running sums, the even channel first
-            gix -= quad_from<kFromEven>(t0x);
-            giy -= quad_from<kFromEven>(t0y);
-            gix += quad_from<kFromEven>(t1x);
-            giy -= quad_from<kFromEven>(t1y);
-            gix -= quad_from<kFromEven>(t2x);
-            giy += quad_from<kFromEven>(t2y);
-            gix += quad_from<kFromEven>(t3x);
-            giy += quad_from<kFromEven>(t3y);
-            gix -= quad_from<kFromOdd>(t0x);
-            giy -= quad_from<kFromOdd>(t0y);
-            gix += quad_from<kFromOdd>(t1x);
-            giy -= quad_from<kFromOdd>(t1y);
-            gix -= quad_from<kFromOdd>(t2x);
-            giy += quad_from<kFromOdd>(t2y);
-            gix += quad_from<kFromOdd>(t3x);
-            giy += quad_from<kFromOdd>(t3y);
 #pragma unroll
-            for (int k = 0; k < 5; k++) {
+                for (int k = 0; k < 10; k++) {
+                    cur[k] &= m;
+                }
+            }
+            const int slot = (u + 2) % SBUF;
+            // the reads of step st + 2 go out one or two at a time between the terms of step st
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const uint32_t g = cur[5 * h + 4];
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    read_one(slot, 5 * h + k, r2);
+                    if (k == 3) {
+                        read_one(slot, 5 * h + 4, r2);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    acc += term(cur[5 * h + k], dk[k], g & keep[k]);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < 10; k++) {
                 r0[k] = r1[k];
                 r1[k] = r2[k];
             }
@@ -813,10 +805,8 @@ __global__ __launch_bounds__(kThreadsLds2) void gs2d_grad_grid_lds2_kernel(
     if (b < steps_real) {
         turn(std::true_type{}, b);
     }
-    if (live && parity == 0u) {
-        ElemIO<T>::store(dgrid + 2 * idx, as_fp32_value(tp.mx * gix));
-        ElemIO<T>::store(dgrid + 2 * idx + 1, as_fp32_value(tp.my * giy));
-    }
+    // products in fp32 first, then the conversion
+    ElemIO<T>::store(dgrid + 2 * idx + parity, as_fp32_value((parity ? tp.my : tp.mx) * acc));
 }
 
 struct GridLdsPlan {
