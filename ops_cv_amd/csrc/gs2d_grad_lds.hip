@@ -1,4 +1,6 @@
 // Backward of grid_sampler2d for gfx950: gradient of the grid (bilinear), input planes staged through LDS.
+// Two kernels: one lane per grid point with whole planes staged (described first), and, further down, two lanes per
+// point with only the box of each plane staged that a block of points reaches, for the shapes that allow it.
 //
 // Same arithmetic, in the same order, as the one-lane-per-point kernel in gs2d_grad.hip (reference:
 // image/grid_sampler2_d_grad/op_kernel/arch35/grid_sampler2_d_grad_simt_det.h:103-196): a lane owns one grid point
