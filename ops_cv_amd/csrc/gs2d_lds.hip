@@ -25,7 +25,17 @@ int compute_unit_count()
     return v;
 }
 
+static LdsPlan make_lds_plan_rows(const GridSamplerArgs& a, bool pad_rows);
+
 LdsPlan make_lds_plan(const GridSamplerArgs& a)
+{
+    // rows padded to a multiple of 128 bytes where that applies and the plan can keep the promise that goes with it
+    // (the loaders' literal-count loop is the one that pads)
+    const LdsPlan padded = make_lds_plan_rows(a, true);
+    return padded.ok ? padded : make_lds_plan_rows(a, false);
+}
+
+static LdsPlan make_lds_plan_rows(const GridSamplerArgs& a, bool pad_rows)
 {
     LdsPlan p;
     const int64_t esz = elem_size(a.elem);
@@ -37,7 +47,19 @@ LdsPlan make_lds_plan(const GridSamplerArgs& a)
     if (!plain && xa % esz != 0) {
         return p;  // a misaligned tensor: leave it to the direct variant
     }
-    const int64_t need = ((plane_bytes + (plain ? 0 : 14) + 15) & ~(int64_t)15) + 16;
+    // staged rows: the plane's rows, or each padded to a multiple of 128 bytes (rows of whole 16-byte units that are
+    // not one already; see the loaders' loop in gs2d_lds_kernel.hpp for why)
+    const int64_t row_bytes = a.Win * esz;
+    const bool padded = pad_rows && plain && row_bytes % 16 == 0 && row_bytes % 128 != 0;
+    if (pad_rows && !padded) {
+        return p;  // nothing to pad: the caller plans without
+    }
+    const int64_t lds_row_bytes = padded ? (row_bytes + 127) / 128 * 128 : row_bytes;
+    const int64_t staged_bytes = a.Hin * lds_row_bytes;
+    p.lds_w = (int32_t)(lds_row_bytes / esz);
+    // a padded plane is copied in whole 1 KiB chunks that must stay in front of the slot of zeros
+    const int64_t need = padded ? (staged_bytes + 1023) / 1024 * 1024 + 16
+                                : ((plane_bytes + (plain ? 0 : 14) + 15) & ~(int64_t)15) + 16;
     const int64_t out_plane = a.Hout * a.Wout;
     // output-plane byte offsets are kept in 32 bits (and below the out-of-range marker 0x80000000)
     if (out_plane * esz >= ((int64_t)1 << 31) || need > kPitch[4]) {
@@ -122,11 +144,22 @@ LdsPlan make_lds_plan(const GridSamplerArgs& a)
     // border padding, where clamped coordinates pile up on the first and last column (one bank in the plain
     // layout).  Elsewhere the plain layout is the better one: the bank then depends on x alone and the lanes of a
     // wavefront have different x.
-    if (a.pad == 1 && p.copy_gran == 16 && a.Win * esz == 128) {
+    if (a.pad == 1 && p.copy_gran == 16 && lds_row_bytes == 128) {
         p.row_shift = 7 | (2 << 8);  // rows of 128 bytes, rotated by two chunks per row
     }
     // all tiles of one (n, channel block) group on one XCD: needs the group count to be a multiple of 8
     p.xcd_swizzle = ((a.N * cblocks) % 8 == 0) ? 1 : 0;
+    if (padded) {
+        // Only the loaders' literal-count loop pads rows; what it asks for (gs2d_lds_kernel.hpp): single-plane
+        // stages, every block with at least as many channels as the ring runs ahead, and a copy count per loader
+        // that the loop is instantiated for.
+        const int64_t last_block = a.C - (cblocks - 1) * cpb;  // channels of the last block (contiguous ranges)
+        int64_t fewest = p.wide_blocks != 0 ? p.chans_per_block : (last_block < cpb ? last_block : cpb);
+        const int64_t copies = ((staged_bytes + 1023) / 1024 + kLoaderWaves[p.cls] - 1) / kLoaderWaves[p.cls];
+        if (cgs != 1 || fewest < kNbuf[p.cls] - 1 || copies > 16 || (kNbuf[p.cls] - 2) * copies > 63) {
+            return p;
+        }
+    }
     p.ok = true;
     return p;
 }

@@ -465,9 +465,10 @@ __device__ __forceinline__ void source_indices_rt(const float* gxs, const float*
 
 template <typename T, int INTERP, int PPT, int NT, int NW, bool SWIZZLED>
 __device__ __forceinline__ void decide_lane_pixels(const float* gxs, const float* gys, int32_t H, int32_t W,
-                                                   uint32_t row_shift, uint32_t zero_off, int32_t pad, bool align,
-                                                   bool arch35, uint32_t (*toff)[NT], float (*tw)[NW])
+                                                   uint32_t ldsw, uint32_t row_shift, uint32_t zero_off, int32_t pad,
+                                                   bool align, bool arch35, uint32_t (*toff)[NT], float (*tw)[NW])
 {
+    // ldsw: elements per staged row (W, or more where the loaders pad the rows -- see the kernel)
     const uint32_t rs = SWIZZLED ? row_shift : 0u;
     float ixs[PPT], iys[PPT];
     if constexpr (INTERP != 2) {
@@ -484,7 +485,7 @@ __device__ __forceinline__ void decide_lane_pixels(const float* gxs, const float
                 for (int k = 0; k < 4; k++) {
                     const bool in = row_in && b.bx[k] >= 0 && b.bx[k] < W;
                     toff[j][4 * r + k] =
-                        in ? lds_swizzle(((uint32_t)b.by[r] * (uint32_t)W + (uint32_t)b.bx[k]) * (uint32_t)sizeof(T), rs)
+                        in ? lds_swizzle(((uint32_t)b.by[r] * ldsw + (uint32_t)b.bx[k]) * (uint32_t)sizeof(T), rs)
                            : zero_off;
                 }
                 tw[j][r] = b.cx[r];
@@ -517,8 +518,8 @@ __device__ __forceinline__ void decide_lane_pixels(const float* gxs, const float
             const uint32_t x1 = x0 + 1u, y1 = y0 + 1u;
             const bool in_x0 = x0 < uw && finite, in_x1 = x1 < uw && finite;
             const bool in_y0 = y0 < uh, in_y1 = y1 < uh;
-            const uint32_t o_nw = (y0 * uw + x0) * es;
-            const uint32_t o_sw = o_nw + uw * es;
+            const uint32_t o_nw = (y0 * ldsw + x0) * es;
+            const uint32_t o_sw = o_nw + ldsw * es;
             toff[j][0] = (in_y0 && in_x0) ? lds_swizzle(o_nw, rs) : zero_off;
             toff[j][1] = (in_y0 && in_x1) ? lds_swizzle(o_nw + es, rs) : zero_off;
             toff[j][2] = (in_y1 && in_x0) ? lds_swizzle(o_sw, rs) : zero_off;
@@ -544,7 +545,7 @@ __device__ __forceinline__ void decide_lane_pixels(const float* gxs, const float
             const uint32_t xr = xi + ((fx > 0.5f || (fx == 0.5f && (xi & 1u))) ? 1u : 0u);
             const uint32_t yr = yi + ((fy > 0.5f || (fy == 0.5f && (yi & 1u))) ? 1u : 0u);
             const bool in = xr < uw && yr < uh;
-            toff[j][0] = in ? lds_swizzle((yr * uw + xr) * es, rs) : zero_off;
+            toff[j][0] = in ? lds_swizzle((yr * ldsw + xr) * es, rs) : zero_off;
             tw[j][0] = tw[j][1] = tw[j][2] = tw[j][3] = 0.0f;
         }
     }
@@ -570,7 +571,7 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
     const T* __restrict__ x, const T* __restrict__ grid, T* __restrict__ y, FastDiv N, int32_t C, int32_t H, int32_t W,
     int32_t out_plane, FastDiv tiles_per_n, int32_t chans_per_block, uint32_t wide_blocks,
     int32_t chans_wide, int32_t chan_stride, int32_t copy_gran, int32_t pair_aligned, int32_t xcd_swizzle, int32_t row_shift, int32_t pad,
-    int32_t align, int32_t rule, float neg_zero)
+    int32_t align, int32_t rule, int32_t ldsw, float neg_zero)
 {
     extern __shared__ uint4 smem_raw[];
     char* lds = reinterpret_cast<char*>(smem_raw);
@@ -605,7 +606,9 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
     const int32_t plane_elems = H * W;
     const uint32_t plane_bytes = (uint32_t)plane_elems * (uint32_t)sizeof(T);
     // behind the plane, which in the shifted layout (copy_gran == 2) may sit up to 14 bytes into its slot
-    const uint32_t zero_off = round_up16(plane_bytes + (SHIFTED_PLANES ? 14u : 0u));
+    // the slot of zeros sits in the last 16 bytes of a plane's pitch: behind any plane, wherever it ends, and behind
+    // whatever a plane's last, partial copy writes past the plane's end (see the loaders' loop)
+    constexpr uint32_t zero_off = (uint32_t)PITCH - 16u;
     // The first `wide_blocks` channel blocks take `chans_wide` channels each, the others `chans_per_block` (see
     // make_lds_plan: the workgroup that reaches a CU first runs ahead of the one that shares the CU with it).
     const bool wide = cb < wide_blocks;
@@ -677,9 +680,9 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
                 issue_stage_copy<4, LWAVES, CGS, PITCH>(src, dst, plane_bytes, planes_of(s), lwave, lane, lane * 4u);
             }
         };
-        // The usual case has a loop of its own: single-plane stages of whole, aligned planes whose 1 KiB chunks divide
-        // evenly among the loaders (PP copies each, a compile-time number) and at least as many stages as the ring
-        // runs ahead.  A loader's step per stage -- wait, barrier, issue -- is in the chain of barriers that every
+        // The usual case has a loop of its own: single-plane stages of planes of whole 16-byte units on the 16-byte
+        // grid (each loader has a fixed number of copies per plane, PP, a compile-time number in the loop) and at
+        // least as many stages as the ring runs ahead.  A loader's step per stage -- wait, barrier, issue -- is in the chain of barriers that every
         // stage goes through, and at the start of the kernel the loaders' first DEPTH stages are what the samplers
         // wait for.  The general loop below finds the wait count of every stage at run time (a sum over the stages in
         // flight, then six compares and branches to reach the matching literal) and tests bounds around every copy:
@@ -687,19 +690,42 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
         // Here the counts are literals and the copies unconditional: steady state while the ring is full, then an
         // unrolled run-down.
         if constexpr (!shifted && CGS == 1) {
-            const uint32_t share = (uint32_t)LWAVES * 1024u;
-            if (copy_gran == 16 && plane_bytes % share == 0u && nstages >= DEPTH) {
+            // 1 KiB chunks of a plane, shared out round-robin: this wavefront's copies per plane.  The last chunk may be
+            // partial: its lanes past the plane's end copy the plane's last 16 bytes again (no masked copy, no read
+            // past the tensor), which land behind the plane and in front of the slot of zeros.
+            // A staged row is the plane's row, or -- `ldsw` > W, set by the launch plan for rows that are not a multiple
+            // of 128 bytes -- the row padded to one: the copy then goes row by row through per-lane source offsets.
+            // With rows of 112 bytes, say, consecutive rows are 28 banks apart, and along a line of slope 1 : 8 (a
+            // rotation by 7 degrees) the lanes of a wavefront all read the same bank; rows of 128 bytes put a
+            // column on the same bank in every row, so that lanes with different columns never collide (fp16 N16 C256
+            // 56x56 under rotations of up to 30 degrees: 21.8 us with rows as they are).
+            const uint32_t row_b = (uint32_t)W * (uint32_t)sizeof(T), lrow_b = (uint32_t)ldsw * (uint32_t)sizeof(T);
+            const uint32_t staged_bytes = (uint32_t)H * lrow_b;
+            const uint32_t chunks1k = (staged_bytes + 1023u) / 1024u;
+            const uint32_t my_copies = (chunks1k > lwave) ? (chunks1k - lwave + LWAVES - 1) / LWAVES : 0u;
+            if (copy_gran == 16 && chunks1k * 1024u <= (uint32_t)PITCH - 16u && nstages >= DEPTH) {
                 auto ring_loop = [&](auto pp_tag) {
                     constexpr int PP = decltype(pp_tag)::value;
-                    if constexpr ((DEPTH - 1) * PP <= 63 && PP * LWAVES * 1024 + 16 <= PITCH) {
-                        const char* src = xb + lwave * 1024u + lane_src16;  // this lane's 16 bytes of the first chunk
-                        uint32_t slot_off = lwave * 1024u;                  // the chunk's place in the slot being filled
+                    if constexpr ((DEPTH - 1) * PP <= 63 && PP * LWAVES * 1024 <= PITCH - 16 + (LWAVES - 1) * 1024) {
+                        // this lane's 16 bytes of the wavefront's j-th chunk, as an offset into the plane
+                        uint32_t lane_off[PP > 0 ? PP : 1];
+#pragma unroll
+                        for (int j = 0; j < PP; j++) {
+                            uint32_t o = ((uint32_t)j * LWAVES + lwave) * 1024u + lane_src16;  // in the staged plane
+                            if (lrow_b != row_b) {
+                                const uint32_t row = o / lrow_b, col = o - row * lrow_b;
+                                o = (col < row_b) ? row * row_b + col : plane_bytes;  // padding: any bytes will do
+                            }
+                            lane_off[j] = o < plane_bytes ? o : plane_bytes - 16u;
+                        }
+                        const char* src = xn + (size_t)first * plane_bytes;  // the plane being asked for
+                        uint32_t slot_off = lwave * 1024u;                  // the first chunk's place in the slot being filled
                         int fill = 0;
                         int32_t turn = 0;  // the block's channel being asked for
                         auto issue = [&]() {
 #pragma unroll
                             for (int j = 0; j < PP; j++) {
-                                __builtin_amdgcn_global_load_lds((global_cptr_t)(src + j * (LWAVES * 1024)),
+                                __builtin_amdgcn_global_load_lds((global_cptr_t)(src + lane_off[j]),
                                                                  (lds_ptr_t)(lds + slot_off + j * (LWAVES * 1024)), 16,
                                                                  0, 0);
                             }
@@ -725,7 +751,8 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
                     }
                 };
                 bool done = false;
-                switch (plane_bytes / share) {
+                switch (my_copies) {
+                    case 0: done = ring_loop(std::integral_constant<int, 0>{}); break;
                     case 1: done = ring_loop(std::integral_constant<int, 1>{}); break;
                     case 2: done = ring_loop(std::integral_constant<int, 2>{}); break;
                     case 3: done = ring_loop(std::integral_constant<int, 3>{}); break;
@@ -734,6 +761,13 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
                     case 6: done = ring_loop(std::integral_constant<int, 6>{}); break;
                     case 7: done = ring_loop(std::integral_constant<int, 7>{}); break;
                     case 8: done = ring_loop(std::integral_constant<int, 8>{}); break;
+                    case 9: done = ring_loop(std::integral_constant<int, 9>{}); break;
+                    case 10: done = ring_loop(std::integral_constant<int, 10>{}); break;
+                    case 11: done = ring_loop(std::integral_constant<int, 11>{}); break;
+                    case 12: done = ring_loop(std::integral_constant<int, 12>{}); break;
+                    case 13: done = ring_loop(std::integral_constant<int, 13>{}); break;
+                    case 14: done = ring_loop(std::integral_constant<int, 14>{}); break;
+                    case 15: done = ring_loop(std::integral_constant<int, 15>{}); break;
                     case 16: done = ring_loop(std::integral_constant<int, 16>{}); break;
                     default: break;
                 }
@@ -817,10 +851,10 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
     // `rule` != 0: the coordinate rule of the reference's second bilinear kernel (bilinear only)
     const bool arch35 = rule != 0;
     if (rs != 0u) {
-        decide_lane_pixels<T, INTERP, PPT, NT, NW, true>(gxs, gys, H, W, rs, zero_off, pad, align != 0, arch35, toff,
+        decide_lane_pixels<T, INTERP, PPT, NT, NW, true>(gxs, gys, H, W, (uint32_t)ldsw, rs, zero_off, pad, align != 0, arch35, toff,
                                                          tw);
     } else {
-        decide_lane_pixels<T, INTERP, PPT, NT, NW, false>(gxs, gys, H, W, rs, zero_off, pad, align != 0, arch35, toff,
+        decide_lane_pixels<T, INTERP, PPT, NT, NW, false>(gxs, gys, H, W, (uint32_t)ldsw, rs, zero_off, pad, align != 0, arch35, toff,
                                                           tw);
     }
     const float first_zero = arch35 ? neg_zero : 0.0f;

@@ -27,6 +27,8 @@ struct LdsPlan {
     // != 0: channels are dealt out to the channel blocks in turn, this many apart (the number of blocks), instead of
     // a contiguous range per block
     int32_t chan_stride = 0;
+    // elements per staged row: Win, or Win's row padded to a multiple of 128 bytes (gs2d_lds_kernel.hpp, loaders)
+    int32_t lds_w = 0;
 };
 
 constexpr int kSamplerWaves = 8;  // 512 lanes own output pixels
@@ -60,7 +62,7 @@ hipError_t launch_one(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t st
     hipLaunchKernelGGL(kernel, dim3(blocks), dim3((kSamplerWaves + LWAVES) * 64), p.lds_bytes, stream, (const T*)a.x, (const T*)a.grid,
                        (T*)a.y, make_fast_div((uint32_t)a.N), (int32_t)a.C, (int32_t)a.Hin, (int32_t)a.Win, (int32_t)(a.Hout * a.Wout),
                        make_fast_div(p.tiles_per_n), p.chans_per_block, p.wide_blocks, p.chans_wide, p.chan_stride, p.copy_gran,
-                       pair_aligned, p.xcd_swizzle, p.row_shift, (int32_t)a.pad, (int32_t)(a.align != 0), (int32_t)a.rule,
+                       pair_aligned, p.xcd_swizzle, p.row_shift, (int32_t)a.pad, (int32_t)(a.align != 0), (int32_t)a.rule, p.lds_w,
                        -0.0f);
     return hipGetLastError();
 }

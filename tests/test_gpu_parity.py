@@ -180,6 +180,44 @@ def test_grid_sampler_bicubic_pair_layout_variant(oracle, device, dtype, pad, al
 @pytest.mark.parametrize("dtype", I.DTYPES)
 @pytest.mark.parametrize("interp", [0, 1, 2])
 @pytest.mark.parametrize("pad", [0, 1, 2])
+def test_grid_sampler_rows_padded_in_lds(oracle, device, dtype, interp, pad):
+    """input rows of whole 16-byte units that are not a multiple of 128 bytes (40, 48, 56, 24, 72 ... elements), which
+    the ring kernel stages with every row padded to one: enough channels for the loaders' literal-count loop, a
+    channel count that leaves a short last block, too few channels for that loop (rows as they are), planes whose
+    padded size moves them to the next size class, border padding (the rotated layout on padded rows of 128 bytes),
+    smooth and scattered grids with special values; bit for bit against the oracle"""
+    import torch
+    from ops_cv_amd import aclnn
+    rng = np.random.default_rng(2100 + interp * 10 + pad)
+    d = 2 if dtype == "fp32" else 1  # the same row bytes for every element type
+    # the launch plan pads rows only when every workgroup gets at least as many channels as the ring runs ahead, so
+    # the shapes have channels to spare: 10 per block with the uneven split of two workgroups per CU, 12 per block,
+    # 11 with a short last block of 5, 2 per block (rows stay as they are), and planes that move up a size class
+    shapes = [(16, 160, 56, 56 // d, 56, 56), (32, 180, 40, 40 // d, 40, 40), (16, 170, 48, 48 // d, 64, 64),
+              (16, 32, 56, 56 // d, 40, 40), (16, 160, 66, 56 // d, 64, 64)]
+    for (N, C, H, W, Ho, Wo) in shapes:
+        x32 = rng.standard_normal((N, C, H, W)).astype(np.float32)
+        x32[:, :, :, W - 1] += 100.0  # the last column of every row: a tap taken from the padding would show
+        x32[:, :, H - 1, :] -= 50.0
+        g32 = I.affine_grid(rng, N, Ho, Wo)
+        g32[N // 2] = rng.uniform(-1.3, 1.3, (Ho, Wo, 2)).astype(np.float32)
+        sv = I.special_grid_values()
+        k = min(sv.size, Wo)
+        g32[0, 0, :k, 0] = sv[:k]
+        g32[0, 1, :k, 1] = sv[:k]
+        x, g = I.cast_np(x32, dtype), I.cast_np(g32, dtype)
+        xt, gt = I.to_torch(x, dtype, device), I.to_torch(g, dtype, device)
+        y_ref = oracle.grid_sampler2d(x, g, interp, pad, False, dtype=I.oracle_code(dtype))
+        with aclnn.option("gs_variant", 2):  # the ring kernel also where a pair-layout variant would take the shape
+            y = I.from_torch(aclnn.grid_sampler2d(xt, gt, interp, pad, False), dtype)
+        what = "gs-padded-rows %s %s %s %s" % (dtype, interp, PAD[pad], (N, C, H, W, Ho, Wo))
+        _check(y, y_ref, dtype, interp, what)
+        _assert_same_bits(y, y_ref, what)
+
+
+@pytest.mark.parametrize("dtype", I.DTYPES)
+@pytest.mark.parametrize("interp", [0, 1, 2])
+@pytest.mark.parametrize("pad", [0, 1, 2])
 @pytest.mark.parametrize("align", [False, True])
 def test_grid_sampler_special_coordinates(oracle, device, dtype, interp, pad, align):
     """ties, borders, 1e10, inf and NaN grid values (what the reference handles at grid_sampler2_d_simt.h:136-247)"""
