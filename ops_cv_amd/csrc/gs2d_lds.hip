@@ -2,6 +2,7 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <cstdint>
 
 #include "gs2d_lds_launch.hpp"
 
@@ -74,7 +75,9 @@ static LdsPlan make_lds_plan_rows(const GridSamplerArgs& a, bool pad_rows)
     // pixels per lane: every tile of an output plane streams all staged input planes through LDS again, so large
     // output planes over large input planes take eight (half the tiles, half the LDS fill traffic)
     p.ppt = (out_plane >= 2 * kThreads) ? 4 : 1;
-    if (p.cls >= 2 && out_plane >= 32 * kThreads) {
+    // (from 8192 output pixels on: fp16 N16 C128 96x96 -> 96x96 27.0 us with four, 22.1 with eight; 112x112 43.4 and
+    // 28.4; fp32 N8 C128 96x96 34.7 and 25.1)
+    if (p.cls >= 2 && out_plane >= 16 * kThreads) {
         p.ppt = 8;
     }
     if (a.interp == 2) {
@@ -97,17 +100,30 @@ static LdsPlan make_lds_plan_rows(const GridSamplerArgs& a, bool pad_rows)
     // 95 us with 32 channels per workgroup, 87 us with 64)
     const int64_t want_blocks = (p.lds_bytes > kLdsLimit / 2) ? 256 : 512;
     const int64_t base = a.N * p.tiles_per_n;
-    int64_t cblocks = (want_blocks + base - 1) / base;
     const int64_t max_cblocks = (a.C + cgs - 1) / cgs;
-    if (cblocks > max_cblocks) {
-        cblocks = max_cblocks;
+    // Enough channel blocks to reach that count, or one block fewer where the count would spill into a second round
+    // of workgroups: the cost of a choice is rounds times channels per block (fp16 N16 C128 96x96, 80 (item, tile)
+    // pairs, one workgroup per CU: four channel blocks are 320 workgroups, a round and a quarter, 36.5 us; three are
+    // 240).
+    int64_t cblocks = 1, cpb = a.C;
+    {
+        int64_t best_cost = INT64_MAX;
+        const int64_t up = (want_blocks + base - 1) / base;
+        for (int64_t cand = up; cand >= up - 1; cand--) {
+            int64_t cb = cand > max_cblocks ? max_cblocks : cand;
+            cb = cb < 1 ? 1 : cb;
+            int64_t per = (a.C + cb - 1) / cb;
+            per = (per + cgs - 1) / cgs * cgs;
+            cb = (a.C + per - 1) / per;
+            const int64_t rounds = (base * cb + want_blocks - 1) / want_blocks;
+            const int64_t cost = rounds * per;
+            if (cost < best_cost) {
+                best_cost = cost;
+                cblocks = cb;
+                cpb = per;
+            }
+        }
     }
-    if (cblocks < 1) {
-        cblocks = 1;
-    }
-    int64_t cpb = (a.C + cblocks - 1) / cblocks;
-    cpb = (cpb + cgs - 1) / cgs * cgs;
-    cblocks = (a.C + cpb - 1) / cpb;
     p.chans_per_block = (int32_t)cpb;
     p.cblocks = (uint32_t)cblocks;
     if (a.N * p.tiles_per_n * cblocks > INT32_MAX) {
