@@ -216,6 +216,37 @@ def test_grid_sampler_rows_padded_in_lds(oracle, device, dtype, interp, pad):
 
 
 @pytest.mark.parametrize("dtype", I.DTYPES)
+@pytest.mark.parametrize("interp", [0, 1])
+@pytest.mark.parametrize("pad", [0, 1, 2])
+def test_grid_sampler_large_output_planes(oracle, device, dtype, interp, pad):
+    """output planes of 8192 pixels and more over planes of the large size classes (eight pixels per lane in the ring
+    kernel), with batch sizes and channel counts for which the launch plan takes one channel block fewer than would
+    fill the CUs: an uneven last block, a single block, blocks of one channel; bit for bit against the oracle"""
+    import torch
+    from ops_cv_amd import aclnn
+    rng = np.random.default_rng(2200 + interp * 10 + pad)
+    d = 2 if dtype == "fp32" else 1
+    shapes = [(16, 24, 96, 96 // d, 96, 96), (8, 7, 96, 96 // d, 112, 112), (3, 40, 80, 96 // d, 96, 100),
+              (16, 3, 96, 96 // d, 128, 65)]
+    for (N, C, H, W, Ho, Wo) in shapes:
+        x32 = rng.standard_normal((N, C, H, W)).astype(np.float32)
+        g32 = I.affine_grid(rng, N, Ho, Wo)
+        g32[N // 2] = rng.uniform(-1.3, 1.3, (Ho, Wo, 2)).astype(np.float32)
+        sv = I.special_grid_values()
+        k = min(sv.size, Wo)
+        g32[0, 0, :k, 0] = sv[:k]
+        g32[0, 1, :k, 1] = sv[:k]
+        x, g = I.cast_np(x32, dtype), I.cast_np(g32, dtype)
+        xt, gt = I.to_torch(x, dtype, device), I.to_torch(g, dtype, device)
+        y_ref = oracle.grid_sampler2d(x, g, interp, pad, False, dtype=I.oracle_code(dtype))
+        with aclnn.option("gs_variant", 2):  # the ring kernel also where a pair-layout variant would take the shape
+            y = I.from_torch(aclnn.grid_sampler2d(xt, gt, interp, pad, False), dtype)
+        what = "gs-large-planes %s %s %s %s" % (dtype, interp, PAD[pad], (N, C, H, W, Ho, Wo))
+        _check(y, y_ref, dtype, interp, what)
+        _assert_same_bits(y, y_ref, what)
+
+
+@pytest.mark.parametrize("dtype", I.DTYPES)
 @pytest.mark.parametrize("interp", [0, 1, 2])
 @pytest.mark.parametrize("pad", [0, 1, 2])
 @pytest.mark.parametrize("align", [False, True])
