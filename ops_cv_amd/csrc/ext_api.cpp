@@ -157,7 +157,7 @@ int32_t opscvVariantRevision(const char* variant)
         {"lds_pair", 2},       {"lds_pair_bicubic", 2}, {"box_lds", 1},          {"direct", 1},          {"direct_arch35", 1},          {"nhwc", 1},
         {"nchw_band_lds", 1},  {"nchw_flat_lds", 1},    {"nchw_band", 1},       {"nchw_generic", 1},
         {"nhwc_", 1},          {"nearest_", 1},         {"copy", 1},            {"point_copy", 1},
-        {"broadcast", 1},      {"first_pixel", 1},      {"resize_grad", 1},     {"gs2d_grad", 3},
+        {"broadcast", 1},      {"first_pixel", 1},      {"resize_grad", 1},     {"gs2d_grad", 4},
         {"gs3d_grad", 1},      {"gs3d_", 1},
     };
     if (variant == nullptr) {

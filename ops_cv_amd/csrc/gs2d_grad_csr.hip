@@ -55,6 +55,14 @@ constexpr int kRun = 8;                           // points of a cell the sortin
 constexpr int kApplyLanes = 512;                  // elements per workgroup of the apply kernel
 constexpr int kApplyLoaders = 2;                  // loader wavefronts
 constexpr int kApplyThreads = kApplyLanes + 64 * kApplyLoaders;
+// The interleaved layout of 16-bit planes (apply kernel): loader wavefronts that interleave through registers, the
+// 16-byte loads each of their lanes has per step (units of a plane times planes), the steps whose loads they keep on
+// their way, the slots of LDS
+constexpr int kPairLoaders = 4;
+constexpr int kPairThreads = kApplyLanes + 64 * kPairLoaders;
+constexpr int kPairLoads = 8;
+constexpr int kPairDepth = 2;
+constexpr int kPairNbuf = 2;
 constexpr int kHeld = 8;                          // contributions of an element kept in registers
 constexpr int kApplyBufBytes = 64 * 1024;         // the ring of gradOutput planes (twice that for planes over 16 KiB)
 constexpr int kApplyNbuf = 4;                     // its slots: three groups of planes on their way while one is read
@@ -428,8 +436,8 @@ struct Fold<_Float16> {
     }
 };
 
-template <typename T, int CB, int EPL>
-__global__ __launch_bounds__(kApplyThreads) void gs2d_grad_csr_apply_kernel(
+template <typename T, int CB, int EPL, bool PAIRS>
+__global__ __launch_bounds__(PAIRS ? kPairThreads : kApplyThreads, PAIRS ? 6 : 1) void gs2d_grad_csr_apply_kernel(
     const T* __restrict__ gout, T* __restrict__ dx, const uint32_t* __restrict__ ws, GradParams p, CsrLayout lay,
     uint32_t tiles, uint32_t cblocks, int32_t chans_per_block, int32_t xcd_swizzle, uint32_t items_fastest,
     uint32_t wide_blocks, int32_t chans_wide, int32_t unit_stride)
@@ -445,7 +453,17 @@ __global__ __launch_bounds__(kApplyThreads) void gs2d_grad_csr_apply_kernel(
     const int32_t plane_px = p.H * p.W;
     const uint32_t row_bytes = (uint32_t)points * (uint32_t)sizeof(T);  // one gradOutput plane
     const uint32_t buf_bytes = (uint32_t)CB * row_bytes;
-    uint2* spill = reinterpret_cast<uint2*>(lds + (uint32_t)kApplyNbuf * buf_bytes);  // behind the ring
+    // Interleaved layout (PAIRS: 16-bit elements, two or four channels per step): a slot of LDS holds the planes of a
+    // step interleaved -- point p is CB neighbouring 16-bit values, one per channel -- and 16 bytes of zeros behind
+    // them.  One 4- or 8-byte LDS read then serves all channels of a contribution, and a contribution that a lane
+    // does not have reads the zeros with weight 0: adding +0 changes no sum (a sum that starts at +0 is never -0), so
+    // the rounds need no selects.  The copy engine cannot interleave, so the loaders go through registers.
+    // fp16 N16 C256 64x64, this kernel: 29.7 us with the planes side by side (two per step), 25.4 with two interleaved.
+    static_assert(!PAIRS || ((CB == 2 || CB == 4) && sizeof(T) == 2), "the interleaved layout is 16-bit planes");
+    const uint32_t pair_pitch = buf_bytes + 16u;
+    const uint32_t pair_zero = buf_bytes;  // offset of the zeros inside a slot
+    uint2* spill = reinterpret_cast<uint2*>(lds + (PAIRS ? (uint32_t)kPairNbuf * pair_pitch
+                                                         : (uint32_t)kApplyNbuf * buf_bytes));  // behind the ring
 
     // all element tiles of one (batch item, channel block) on one XCD: they stream the same gradOutput planes
     uint32_t group, tile;
@@ -499,6 +517,92 @@ __global__ __launch_bounds__(kApplyThreads) void gs2d_grad_csr_apply_kernel(
         // arithmetic needs a quarter).
         const uint32_t lwave = wave - (uint32_t)(kApplyLanes / 64);
         const uint32_t lane = (uint32_t)tid & 63u;
+        if constexpr (PAIRS) {
+            // Every lane takes UPL 16-byte units (eight points) of every plane of a step: CB loads per unit, the
+            // halves interleaved, CB 16-byte LDS writes.  The loads of kPairDepth steps are on their way at any time;
+            // they are issued on every path alike, those past the last step from one address all lanes share (one
+            // cache line), so that the compiler's count of outstanding loads at every use is the same on all paths
+            // and exact.  Slot s % 2 is written between the barriers of steps s - 1 and s, while the element lanes
+            // read the other one.
+            constexpr int UPL = kPairLoads / CB;
+            typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+            typedef u32x4 __attribute__((address_space(3))) * lds_u32x4_ptr_t;
+            const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
+            const uint32_t lid = lwave * 64u + lane;
+            const uint32_t units = row_bytes >> 4;
+            if (lid < (uint32_t)kPairNbuf) {
+                *reinterpret_cast<lds_u32x4_ptr_t>((uintptr_t)(lds_base + lid * pair_pitch + pair_zero)) =
+                    u32x4{0u, 0u, 0u, 0u};
+            }
+            uint32_t unit[UPL];
+            bool mine[UPL];
+#pragma unroll
+            for (int u = 0; u < UPL; u++) {
+                unit[u] = lid + (uint32_t)u * (64u * kPairLoaders);
+                mine[u] = unit[u] < units;
+                unit[u] = mine[u] ? unit[u] : units - 1u;  // a lane without a unit reads the last one again
+            }
+            const char* go_bytes = reinterpret_cast<const char*>(go_n);
+            u32x4 regs[kPairDepth][UPL][CB];
+            auto issue = [&](u32x4 (*r)[CB], int32_t s) {
+                const bool real = s < steps;
+                const char* base = go_bytes + (real ? (size_t)unit_of(s) * buf_bytes : (size_t)0);
+                const int32_t left = real ? nchan - s * CB : 0;  // planes of a last, partial step: the first again
+#pragma unroll
+                for (int u = 0; u < UPL; u++) {
+                    const uint32_t off = real ? unit[u] * 16u : 0u;
+#pragma unroll
+                    for (int j = 0; j < CB; j++) {
+                        const uint32_t plane = (j < left) ? (uint32_t)j * row_bytes : 0u;
+                        r[u][j] = *reinterpret_cast<const u32x4*>(base + plane + off);
+                    }
+                }
+            };
+            // the low halves of two dwords in one, and the high halves
+            auto lows = [](uint32_t a, uint32_t b) -> uint32_t { return (a & 0xFFFFu) | (b << 16); };
+            auto highs = [](uint32_t a, uint32_t b) -> uint32_t { return (a >> 16) | (b & 0xFFFF0000u); };
+#pragma unroll
+            for (int k = 0; k < kPairDepth; k++) {
+                issue(regs[k], k);
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the zeros are written
+            lds_barrier();                                       // the element lanes' set-up barrier
+            for (int32_t s0 = 0; s0 < steps; s0 += kPairDepth) {
+#pragma unroll
+                for (int k = 0; k < kPairDepth; k++) {
+                    const int32_t s = s0 + k;
+                    if (s < steps) {
+                        const uint32_t slot = lds_base + ((uint32_t)s & 1u) * pair_pitch;
+#pragma unroll
+                        for (int u = 0; u < UPL; u++) {
+                            if (mine[u]) {
+                                const uint32_t at = slot + unit[u] * (16u * CB);
+                                if constexpr (CB == 2) {
+                                    const u32x4 a = regs[k][u][0], b = regs[k][u][1];
+                                    const u32x4 lo = {lows(a.x, b.x), highs(a.x, b.x), lows(a.y, b.y), highs(a.y, b.y)};
+                                    const u32x4 hi = {lows(a.z, b.z), highs(a.z, b.z), lows(a.w, b.w), highs(a.w, b.w)};
+                                    *reinterpret_cast<lds_u32x4_ptr_t>((uintptr_t)at) = lo;
+                                    *reinterpret_cast<lds_u32x4_ptr_t>((uintptr_t)(at + 16u)) = hi;
+                                } else {
+                                    const u32x4 a = regs[k][u][0], b = regs[k][u][1], c = regs[k][u][2],
+                                                d = regs[k][u][3];
+#pragma unroll
+                                    for (int q = 0; q < 4; q++) {  // dword q of a plane: points 2q and 2q + 1
+                                        const u32x4 two = {lows(a[q], b[q]), lows(c[q], d[q]), highs(a[q], b[q]),
+                                                           highs(c[q], d[q])};
+                                        *reinterpret_cast<lds_u32x4_ptr_t>((uintptr_t)(at + 16u * (uint32_t)q)) = two;
+                                    }
+                                }
+                            }
+                        }
+                        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                        lds_barrier();  // step s is in its slot, and the other slot has been read for the last time
+                    }
+                    issue(regs[k], s + kPairDepth);
+                }
+            }
+            return;
+        }
         auto bytes_of = [&](int32_t s) -> uint32_t {
             const int32_t left = nchan - s * CB;
             return (uint32_t)(left < CB ? left : CB) * row_bytes;  // the planes are neighbours in memory
@@ -575,9 +679,11 @@ __global__ __launch_bounds__(kApplyThreads) void gs2d_grad_csr_apply_kernel(
 #pragma unroll
         for (int k = 0; k < kHeld / 2; k++) {
             const bool a = (uint32_t)(2 * k) < cnt[i], b = (uint32_t)(2 * k + 1) < cnt[i];
-            hoff[i][2 * k] = a ? raw[k].x * (uint32_t)sizeof(T) : 0u;
+            constexpr uint32_t point_bytes = PAIRS ? (uint32_t)(2 * CB) : (uint32_t)sizeof(T);
+            const uint32_t none = PAIRS ? pair_zero : 0u;
+            hoff[i][2 * k] = a ? raw[k].x * point_bytes : none;
             hw[i][2 * k] = F::weight(a ? __builtin_bit_cast(float, raw[k].y) : 0.0f);
-            hoff[i][2 * k + 1] = b ? raw[k].z * (uint32_t)sizeof(T) : 0u;
+            hoff[i][2 * k + 1] = b ? raw[k].z * point_bytes : none;
             hw[i][2 * k + 1] = F::weight(b ? __builtin_bit_cast(float, raw[k].w) : 0.0f);
         }
     }
@@ -628,11 +734,59 @@ __global__ __launch_bounds__(kApplyThreads) void gs2d_grad_csr_apply_kernel(
     auto go_at = [&](uint32_t off) -> uint32_t {
         return (uint32_t)*reinterpret_cast<lds_bits_ptr_t>((uintptr_t)(lds_base + off));
     };
+    // all channels of a point in the interleaved layout: CB / 2 dwords
+    typedef uint32_t group_t __attribute__((ext_vector_type(CB >= 2 ? CB / 2 : 1)));
+    typedef const group_t __attribute__((address_space(3))) * lds_group_ptr_t;
+    auto group_at = [&](uint32_t off) -> group_t {
+        return *reinterpret_cast<lds_group_ptr_t>((uintptr_t)(lds_base + off));
+    };
+    auto dword_of = [](const group_t& g, int j) -> uint32_t { return g[CB >= 4 ? j : 0]; };
     // R rounds of one step for one of the lane's elements, straight-line: all gradOutput values first (raw bits, so
     // that nothing waits between the reads), then the sums in list order; a lane whose list is shorter keeps its sum
     // (a select, not arithmetic: a value read for a contribution that does not exist may be anything)
     auto rounds = [&](auto r_tag, uint32_t buf_off, const uint32_t* ho, const acc_t* w, uint32_t count, acc_t* acc) {
         constexpr int R = decltype(r_tag)::value;
+        if constexpr (PAIRS) {
+            // one read per contribution; a contribution the lane does not have is zeros times weight 0
+            (void)count;
+            group_t got[R];
+#pragma unroll
+            for (int k = 0; k < R; k++) {
+                got[k] = group_at(buf_off + ho[k]);
+            }
+            if constexpr (std::is_same<T, _Float16>::value) {
+                typename F::pair_t acc2[CB / 2];
+#pragma unroll
+                for (int j = 0; j < CB / 2; j++) {
+                    acc2[j] = typename F::pair_t{acc[2 * j], acc[2 * j + 1]};
+                }
+#pragma unroll
+                for (int k = 0; k < R; k++) {
+                    const typename F::pair_t ww = {w[k], w[k]};
+#pragma unroll
+                    for (int j = 0; j < CB / 2; j++) {
+                        const typename F::pair_t val = ww * __builtin_bit_cast(typename F::pair_t, dword_of(got[k], j));
+                        acc2[j] = acc2[j] + val;
+                    }
+                }
+#pragma unroll
+                for (int j = 0; j < CB / 2; j++) {
+                    acc[2 * j] = acc2[j].x;
+                    acc[2 * j + 1] = acc2[j].y;
+                }
+            } else {
+#pragma unroll
+                for (int k = 0; k < R; k++) {
+#pragma unroll
+                    for (int j = 0; j < CB / 2; j++) {
+                        const uint32_t two = dword_of(got[k], j);
+                        acc[2 * j] = F::add(acc[2 * j], two & 0xFFFFu, w[k]);
+                        acc[2 * j + 1] = F::add(acc[2 * j + 1], two >> 16, w[k]);
+                    }
+                }
+            }
+            return;
+        }
         uint32_t raw[R][CB];
 #pragma unroll
         for (int k = 0; k < R; k++) {
@@ -676,7 +830,7 @@ __global__ __launch_bounds__(kApplyThreads) void gs2d_grad_csr_apply_kernel(
 
     for (int32_t s = 0; s < steps; s++) {
         lds_barrier();  // the planes of step s have landed
-        const uint32_t buf_off = (uint32_t)(s % kApplyNbuf) * buf_bytes;
+        const uint32_t buf_off = PAIRS ? ((uint32_t)s & 1u) * pair_pitch : (uint32_t)(s % kApplyNbuf) * buf_bytes;
 #pragma unroll
         for (int i = 0; i < EPL; i++) {
             acc_t acc[CB];
@@ -699,9 +853,20 @@ __global__ __launch_bounds__(kApplyThreads) void gs2d_grad_csr_apply_kernel(
                 for (uint32_t k = 0; k < cnt[i] - (uint32_t)kHeld; k++) {
                     const uint2 v = rest_in_lds[i] ? spill[rest_at[i] + k] : rest[i][k];
                     const acc_t w = F::weight(__builtin_bit_cast(float, v.y));
+                    if constexpr (PAIRS) {
+                        const group_t got = group_at(buf_off + v.x * (uint32_t)(2 * CB));
 #pragma unroll
-                    for (int j = 0; j < CB; j++) {
-                        acc[j] = F::add(acc[j], go_at(buf_off + (uint32_t)j * row_bytes + v.x * (uint32_t)sizeof(T)), w);
+                        for (int j = 0; j < CB / 2; j++) {
+                            const uint32_t two = dword_of(got, j);
+                            acc[2 * j] = F::add(acc[2 * j], two & 0xFFFFu, w);
+                            acc[2 * j + 1] = F::add(acc[2 * j + 1], two >> 16, w);
+                        }
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < CB; j++) {
+                            acc[j] = F::add(acc[j],
+                                            go_at(buf_off + (uint32_t)j * row_bytes + v.x * (uint32_t)sizeof(T)), w);
+                        }
                     }
                 }
             }
@@ -722,6 +887,7 @@ struct CsrPlan {
     int ipt = 1;
     int cb = 1;
     int epl = 1;  // elements per lane of the apply kernel
+    bool pairs = false;  // the apply kernel's paired layout
     uint32_t tiles = 0, cblocks = 0;
     int32_t chans_per_block = 0;
     int xcd_swizzle = 0;
@@ -755,6 +921,12 @@ CsrPlan make_plan(const GridSamplerGradArgs& a)
     pl.cb = 4;
     while (pl.cb > 1 && (int64_t)kApplyNbuf * pl.cb * points * esz > kApplyBufBytes) {
         pl.cb /= 2;
+    }
+    // the interleaved layout: 16-bit elements, four channels per step for planes of up to 8 KiB and two for planes of
+    // up to 16 KiB (what the loaders' lanes cover with kPairLoads loads each; two slots of LDS either way)
+    if (esz == 2 && points * esz <= 16 * 64 * kPairLoaders * (kPairLoads / 2)) {
+        pl.pairs = true;
+        pl.cb = (points * esz <= 16 * 64 * kPairLoaders * (kPairLoads / 4)) ? 4 : 2;
     }
     // two elements per lane where that still leaves workgroups for every CU
     pl.epl = (plane_px >= 2 * kApplyLanes && a.N * ((plane_px + 2 * kApplyLanes - 1) / (2 * kApplyLanes)) *
@@ -830,10 +1002,10 @@ GradClear clear_of(const GridSamplerGradArgs& a, const CsrPlan& pl)
     return c;
 }
 
-template <typename T, int CB, int EPL>
+template <typename T, int CB, int EPL, bool PAIRS = false>
 hipError_t launch_apply(const GridSamplerGradArgs& a, const CsrPlan& pl, const GradParams& p, hipStream_t stream)
 {
-    auto kernel = gs2d_grad_csr_apply_kernel<T, CB, EPL>;
+    auto kernel = gs2d_grad_csr_apply_kernel<T, CB, EPL, PAIRS>;
     constexpr int kLdsMax = 2 * kApplyBufBytes + kApplySpill * 8;
     static std::atomic<uint32_t> lds_allowed{0};
     const hipError_t ea = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kLdsMax, lds_allowed);
@@ -841,8 +1013,9 @@ hipError_t launch_apply(const GridSamplerGradArgs& a, const CsrPlan& pl, const G
         return ea;
     }
     const uint32_t blocks = (uint32_t)(a.N * pl.tiles * pl.cblocks);
-    const int lds_bytes = kApplyNbuf * CB * (int)(a.Hout * a.Wout) * (int)sizeof(T) + kApplySpill * 8;
-    hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kApplyThreads), lds_bytes, stream, (const T*)a.gout, (T*)a.dx,
+    const int plane_bytes = (int)(a.Hout * a.Wout) * (int)sizeof(T);
+    const int lds_bytes = (PAIRS ? kPairNbuf * (CB * plane_bytes + 16) : kApplyNbuf * CB * plane_bytes) + kApplySpill * 8;
+    hipLaunchKernelGGL(kernel, dim3(blocks), dim3(PAIRS ? kPairThreads : kApplyThreads), lds_bytes, stream, (const T*)a.gout, (T*)a.dx,
                        (const uint32_t*)a.scratch, p, pl.lay, pl.tiles, pl.cblocks, pl.chans_per_block, pl.xcd_swizzle,
                        pl.items_fastest, pl.wide_blocks, pl.chans_wide, pl.unit_stride);
     return hipGetLastError();
@@ -887,6 +1060,17 @@ hipError_t run_typed(const GridSamplerGradArgs& a, const CsrPlan& pl, bool clear
     e = hipGetLastError();
     if (e != hipSuccess) {
         return e;
+    }
+    if constexpr (sizeof(T) == 2) {
+        if (pl.pairs) {
+            switch (pl.cb * 4 + pl.epl) {
+                case 4 * 4 + 1: return launch_apply<T, 4, 1, true>(a, pl, p, stream);
+                case 4 * 4 + 2: return launch_apply<T, 4, 2, true>(a, pl, p, stream);
+                case 2 * 4 + 1: return launch_apply<T, 2, 1, true>(a, pl, p, stream);
+                case 2 * 4 + 2: return launch_apply<T, 2, 2, true>(a, pl, p, stream);
+                default: return hipErrorInvalidValue;
+            }
+        }
     }
     switch (pl.cb * 4 + pl.epl) {
         case 4 * 4 + 1: return launch_apply<T, 4, 1>(a, pl, p, stream);

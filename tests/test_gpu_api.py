@@ -729,6 +729,43 @@ def test_grid_sampler2d_backward_input_gradient_list_variant(oracle, device, acl
                         (what, kind, N, C, H, W, Ho, Wo, pad, align)
 
 
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+def test_grid_sampler2d_backward_interleaved_planes(oracle, device, aclnn, dtype):
+    """16-bit gradOutput planes staged interleaved by the gather over the contribution lists: four channels per step
+    (planes of up to 8 KiB) and two (up to 16 KiB), channel counts that leave one, two or three planes for the last
+    step, planes that are not whole loads for every loader lane, a plane whose first point holds a non-finite value
+    (a contribution that a lane does not have must not read it), lists longer than a lane holds; bit for bit"""
+    torch = _torch()
+    rng = np.random.default_rng(650)
+    for (N, C, H, W, Ho, Wo, kind) in [(2, 9, 20, 24, 24, 40, "random"), (2, 10, 20, 24, 24, 40, "smooth"),
+                                        (3, 11, 33, 31, 40, 40, "smooth"), (1, 9, 64, 64, 72, 96, "smooth"),
+                                        (2, 12, 48, 40, 64, 128, "random"), (2, 16, 12, 12, 40, 48, "pile"),
+                                        (16, 24, 64, 64, 64, 64, "smooth")]:
+        x = I.cast_np(rng.standard_normal((N, C, H, W)).astype(np.float32), dtype)
+        if kind == "smooth":
+            g32 = I.affine_grid(rng, N, Ho, Wo)
+        elif kind == "pile":
+            g32 = rng.choice(np.array([-0.9, -0.3, 0.05, 0.45, 0.8], np.float32), (N, Ho, Wo, 2))
+        else:
+            g32 = rng.uniform(-1.1, 1.1, (N, Ho, Wo, 2)).astype(np.float32)
+        g = I.cast_np(g32, dtype)
+        go32 = rng.standard_normal((N, C, Ho, Wo)).astype(np.float32)
+        go32 += np.arange(C, dtype=np.float32).reshape(1, C, 1, 1) / 4
+        # the first point of some planes is infinite; its own grid point is moved far outside the image, so that no
+        # element takes it and the reference's result stays finite
+        go32[:, ::3, 0, 0] = np.inf
+        g32[:, 0, 0, :] = 5.0
+        g = I.cast_np(g32, dtype)
+        go = I.cast_np(go32, dtype)
+        tensors = [I.to_torch(v, dtype, device) for v in (go, x, g)]
+        rdx, rdg = oracle.grid_sampler2d_backward(go, x, g, 0, 0, False, dtype=I.oracle_code(dtype))
+        assert np.isfinite(I.as_f32(rdx, dtype)).all()
+        dx, dg = aclnn.grid_sampler2d_backward(*tensors, 0, 0, False)
+        torch.cuda.synchronize()
+        for got, ref, what in ((I.from_torch(dx, dtype), rdx, "dx"), (I.from_torch(dg, dtype), rdg, "dgrid")):
+            assert np.array_equal(_bits(got, dtype), _bits(ref, dtype)), (what, kind, N, C, H, W, Ho, Wo)
+
+
 def test_grid_sampler2d_backward_mask_views_and_torch(oracle, device, aclnn):
     torch = _torch()
     import torch.nn.functional as F
