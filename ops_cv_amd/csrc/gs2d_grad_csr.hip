@@ -24,9 +24,10 @@
 //     instead of the network.
 //   apply (per batch item, tile of 512 elements, block of channels): a lane owns one element and holds its first
 //     eight contributions in registers (more: in LDS); the gradOutput planes of the channels stream through LDS
-//     (asynchronous global->LDS copies by a loader wavefront, two buffers), and per channel the lane folds
-//     gradOutput[point] * weight into its sum in list order with the reference's roundings.  No atomics, no
-//     elections; one barrier per group of planes.
+//     (asynchronous global->LDS copies by loader wavefronts into a ring of slots; 16-bit planes of up to 16 KiB
+//     instead go through the loaders' registers and lie in LDS interleaved, all channels of a point side by side, so
+//     that one read serves them all), and per channel the lane folds gradOutput[point] * weight into its sum in list
+//     order with the reference's roundings.  No atomics, no elections; one barrier per group of planes.
 //
 // The result is the same sequence of rounded operations per element as the scatter in gs2d_grad.hip, bit for bit.
 #include <hip/hip_runtime.h>
