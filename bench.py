@@ -37,7 +37,7 @@ MEASURED_TRAFFIC = {
     ("C5", "lds_pair_w128"): (170.05e6, 2, "profiles/gs2d_lds_pair_C5_bf16_random_gather.md"),
     ("L1", "box_lds"): (742.5e6, 1, "profiles/gs2d_box_L1_fp16_1080p.md"),
     ("V1", "gs3d_bilinear"): (38.72e6, 1, "profiles/gs3d_V1_fp16_22x4x16x64x64.md"),
-    ("G3", "gs2d_grad_lists_lds"): (151.4e6, 4, "profiles/gs2d_grad_G3_fp16_n16_c256.md"),
+    ("G3", "gs2d_grad_lists_lds"): (151.8e6, 4, "profiles/gs2d_grad_G3_fp16_n16_c256.md"),
     ("W1", "gs3d_grad_lists"): (200.1e6, 1, "profiles/gs3d_grad_W1_fp16_22x4x16x64x64.md"),
     ("B4", "resize_grad_lds"): (1340.0e6, 1, "profiles/resize_grad_lds_B4_fp16_4k.md"),
     ("R4", "nearest_nchw_lds"): (1327.3e6, 1, "profiles/resize_nearest_lds_R4_fp16_4k.md"),

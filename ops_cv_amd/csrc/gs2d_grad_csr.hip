@@ -273,7 +273,18 @@ __global__ __launch_bounds__(kListThreads) void gs2d_grad_csr_lists_kernel(uint3
     cid[3] = y * w1 + x;                // se corner of cell (y - 1, x - 1)
     // the points of a cell: its slots, or, in an item where some cell overflowed its slots, its run in the sorted keys
     const uint32_t cells = (uint32_t)(H + 1) * w1;
-    const bool from_runs = wsn[lay.slot_count + cells] != 0u;
+    // One round of loads for the usual case: the item's flag, the four cells' counts and, unasked, the first two slots
+    // of every cell (a cell of a smooth grid holds a point or two) -- not flag, then counts, then slots, each waiting
+    // for the one before.
+    const uint32_t flag = wsn[lay.slot_count + cells];
+    uint32_t slot_cnt[4];
+    uint2 first_two[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        slot_cnt[k] = wsn[lay.slot_count + cid[k]];
+        first_two[k] = *reinterpret_cast<const uint2*>(wsn + lay.slots + cid[k] * (uint32_t)kRun);
+    }
+    const bool from_runs = flag != 0u;
     const uint32_t* source = from_runs ? sorted : wsn + lay.slots;
     uint32_t cnt = 0;
     bool crowded = false;
@@ -284,7 +295,7 @@ __global__ __launch_bounds__(kListThreads) void gs2d_grad_csr_lists_kernel(uint3
             end[k] = cell_start[cid[k] + 1];
         } else {
             cur[k] = cid[k] * (uint32_t)kRun;
-            end[k] = cur[k] + wsn[lay.slot_count + cid[k]];
+            end[k] = cur[k] + slot_cnt[k];
         }
         cnt += end[k] - cur[k];
         crowded = crowded || end[k] - cur[k] > (uint32_t)kRun;
@@ -318,7 +329,12 @@ __global__ __launch_bounds__(kListThreads) void gs2d_grad_csr_lists_kernel(uint3
 #pragma unroll
                 for (int i = 0; i < R; i++) {
                     const bool valid = (uint32_t)i < len;
-                    const uint32_t pt = source[valid ? cur[k] + (uint32_t)i : 0u] & kPointMask;
+                    uint32_t pt;
+                    if (R == 2 && !from_runs) {
+                        pt = (i == 0 ? first_two[k].x : first_two[k].y) & kPointMask;  // already here
+                    } else {
+                        pt = source[valid ? cur[k] + (uint32_t)i : 0u] & kPointMask;
+                    }
                     key[k * R + i] = valid ? (((pt >> kChunkShift) << (kPointBits + 2)) | ((uint32_t)k << kPointBits) | pt)
                                            : 0xFFFFFFFFu;
                 }
