@@ -154,6 +154,7 @@ int32_t opscvVariantRevision(const char* variant)
     } table[] = {
         // 2 (ring and pair variants): streaming stores and grid loads, batch-fastest block order; ring: 5:3 channel split
         {"lds_ring", 4},
+        {"lds_ring_pairs", 1},
         {"lds_pair", 2},       {"lds_pair_bicubic", 2}, {"box_lds", 1},          {"direct", 1},          {"direct_arch35", 1},          {"nhwc", 1},
         {"nchw_band_lds", 1},  {"nchw_flat_lds", 1},    {"nchw_band", 1},       {"nchw_generic", 1},
         {"nhwc_", 1},          {"nearest_", 1},         {"copy", 1},            {"point_copy", 1},

@@ -451,7 +451,7 @@ namespace {
 // option "gs_variant" as captured by the first phase: the direct kernel forced, or the pair-layout variant kept out
 // (benchmark and test knobs)
 bool force_direct(const GridSamplerArgs& a) { return a.force_variant == kGsDirect; }
-bool force_ring(const GridSamplerArgs& a) { return a.force_variant == kGsRing; }
+bool force_ring(const GridSamplerArgs& a) { return a.force_variant == kGsRing || a.force_variant == kGsRingSingle; }
 }  // namespace
 
 // The second coordinate rule (bilinear only) is implemented by the LDS ring and by a direct kernel of its own.

@@ -5,6 +5,7 @@
 #include <cstdint>
 
 #include "gs2d_lds_launch.hpp"
+#include "options.hpp"
 
 namespace opscv {
 
@@ -176,6 +177,18 @@ static LdsPlan make_lds_plan_rows(const GridSamplerArgs& a, bool pad_rows)
             return p;
         }
     }
+    // Two channels per stage, interleaved in LDS (gs2d_lds_kernel.hpp, CHANNEL_PAIRS): bilinear samples of 16-bit
+    // elements in the 8 KiB class with four pixels per lane, plain unpadded layout, every block's channels in pairs.
+    {
+        const int64_t last_block = a.C - (int64_t)(cblocks - 1) * cpb;
+        const bool even_counts = p.wide_blocks != 0 ? (p.chans_wide % 2 == 0 && p.chans_per_block % 2 == 0)
+                                                    : (cpb % 2 == 0 && last_block % 2 == 0);
+        if (a.interp == 0 && esz == 2 && p.cls == 1 && p.ppt == 4 && plain && !padded && p.row_shift == 0 &&
+            p.copy_gran == 16 && a.C % 2 == 0 && even_counts && a.force_variant != kGsRingSingle) {
+            p.chan_pairs = true;
+            p.lds_bytes = (uint32_t)(kPairsNbuf * kPairsPitch);
+        }
+    }
     p.ok = true;
     return p;
 }
@@ -188,7 +201,7 @@ const char* gs2d_lds_variant_name(const GridSamplerArgs& a)
     }
     static const char* names[5] = {"lds_ring_p2064_4x4", "lds_ring_p8208_1x6", "lds_ring_p16400_1x4",
                                    "lds_ring_p32784_1x4", "lds_ring_p81904_1x2"};
-    return names[p.cls];
+    return p.chan_pairs ? "lds_ring_pairs_p16400_2x2" : names[p.cls];
 }
 
 hipError_t run_gs2d_lds(const GridSamplerArgs& a, hipStream_t stream, bool* handled)
@@ -199,6 +212,9 @@ hipError_t run_gs2d_lds(const GridSamplerArgs& a, hipStream_t stream, bool* hand
         return hipSuccess;
     }
     *handled = true;
+    if (p.chan_pairs) {
+        return lds_launch_channel_pairs(a, p, stream);
+    }
     const bool shifted = p.copy_gran == 2;
     switch (a.elem) {
         case Elem::F32:

@@ -29,7 +29,15 @@ struct LdsPlan {
     int32_t chan_stride = 0;
     // elements per staged row: Win, or Win's row padded to a multiple of 128 bytes (gs2d_lds_kernel.hpp, loaders)
     int32_t lds_w = 0;
+    // two neighbouring channels per stage, interleaved in LDS (gs2d_lds_kernel.hpp, CHANNEL_PAIRS); the channel counts
+    // above stay in channels, the launch halves them
+    bool chan_pairs = false;
 };
+
+// the channel-pair kernels' LDS: two slots of two 8 KiB planes and the zeros
+constexpr int kPairsPitch = 16400;
+constexpr int kPairsNbuf = 2;
+constexpr int kPairsLoaderWaves = 4;
 
 constexpr int kSamplerWaves = 8;  // 512 lanes own output pixels
 // loader wavefronts per size class (the 16 KiB class as the 8 KiB one): enough that (NBUF-2) stages of one loader's copy instructions fit the
@@ -137,6 +145,9 @@ hipError_t lds_launch_typed(const GridSamplerArgs& a, const LdsPlan& p, hipStrea
         default: return hipErrorInvalidValue;
     }
 }
+
+// the CHANNEL_PAIRS kernels (16-bit elements, bilinear, the 8 KiB class with four pixels per lane): gs2d_lds_pairs.hip
+hipError_t lds_launch_channel_pairs(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t stream);
 
 extern template hipError_t lds_launch_typed<float, false>(const GridSamplerArgs&, const LdsPlan&, hipStream_t);
 extern template hipError_t lds_launch_typed<_Float16, false>(const GridSamplerArgs&, const LdsPlan&, hipStream_t);

@@ -73,7 +73,7 @@ struct Entry {
 };
 
 const Entry kEntries[] = {
-    {"gs_variant", &Store::gs_variant, kGsAuto, kGsRing},
+    {"gs_variant", &Store::gs_variant, kGsAuto, kGsRingSingle},
     {"resize_variant", &Store::resize_variant, kResizeAuto, kResizeLdsBand},
     {"nearest_variant", &Store::nearest_variant, kNearestAuto, kNearestGather},
     {"reference_cores", &Store::reference_cores, 1, INT64_MAX},

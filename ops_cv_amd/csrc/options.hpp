@@ -11,7 +11,8 @@
 
 namespace opscv {
 
-enum GsVariant : int32_t { kGsAuto = 0, kGsDirect = 1, kGsRing = 2 };
+// (kGsRingSingle: the ring kernel with one channel per stage, where two interleaved channels would be the choice)
+enum GsVariant : int32_t { kGsAuto = 0, kGsDirect = 1, kGsRing = 2, kGsRingSingle = 3 };
 enum ResizeVariant : int32_t { kResizeAuto = 0, kResizeGeneric = 1, kResizeRegisterBand = 2, kResizeLdsBand = 3 };
 enum NearestVariant : int32_t { kNearestAuto = 0, kNearestGather = 1 };
 enum GsRule : int32_t { kRuleGridSampler2D = 0, kRuleGridSampleArch35 = 1 };
