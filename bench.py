@@ -32,6 +32,7 @@ HBM_PEAK_GBS = 8000.0
 # and thereby retires the figure until the counters are read again.
 MEASURED_TRAFFIC = {
     ("C3", "lds_ring_p8208_1x6"): (67.58e6, 4, "profiles/gs2d_lds_ring_C3_fp16_n16_c256.md"),
+    ("C3", "lds_ring_pairs_p16400_2x2"): (67.59e6, 1, "profiles/gs2d_lds_ring_pairs_C3_fp16_n16_c256.md"),
     ("C4", "nchw_band_lds"): (1415.4e6, 1, "profiles/resize_band_lds_C4_fp16_4k_upscale.md"),
     ("C2", "nchw_flat_lds"): (32.43e6, 1, "profiles/resize_flat_lds_C2_fp32_56_to_112.md"),
     ("C5", "lds_pair_w128"): (170.05e6, 2, "profiles/gs2d_lds_pair_C5_bf16_random_gather.md"),

@@ -215,6 +215,58 @@ def test_grid_sampler_rows_padded_in_lds(oracle, device, dtype, interp, pad):
         _assert_same_bits(y, y_ref, what)
 
 
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("pad", [0, 2])
+@pytest.mark.parametrize("align", [False, True])
+def test_grid_sampler_channel_pairs_in_lds(oracle, device, dtype, pad, align):
+    """bilinear samples of 16-bit planes of up to 8 KiB with an even channel count, which the ring kernel stages two
+    channels at a time, interleaved: planes that are not whole loads for every loader lane, a last channel block
+    shorter than the others, the uneven split of two workgroups per CU, fewer stages than the loaders keep on their
+    way, both coordinate rules; bit for bit against the oracle and against the same kernel with
+    single-channel stages"""
+    import torch
+    from ops_cv_amd import aclnn
+    rng = np.random.default_rng(2300 + pad * 10 + int(align))
+    # (the launch plan takes channel pairs where every channel block gets an even number of channels: 4 per block,
+    # 2 with a last block of 2, 6 on planes of 200 16-byte units, 4 with 25 blocks, 2 = a single stage per block,
+    # and the headline's 22 + 10)
+    shapes = [(16, 64, 64, 64, 64, 64), (16, 26, 64, 64, 64, 64), (32, 48, 25, 64, 64, 64), (8, 100, 62, 64, 33, 70),
+              (64, 12, 48, 64, 40, 40), (16, 256, 64, 64, 64, 64)]
+    for (N, C, H, W, Ho, Wo) in shapes:
+        x32 = rng.standard_normal((N, C, H, W)).astype(np.float32)
+        x32 += np.arange(C, dtype=np.float32).reshape(1, C, 1, 1)  # a channel taken for its neighbour shows
+        g32 = I.affine_grid(rng, N, Ho, Wo)
+        g32[N // 2] = rng.uniform(-1.3, 1.3, (Ho, Wo, 2)).astype(np.float32)
+        sv = I.special_grid_values()
+        k = min(sv.size, Wo)
+        g32[0, 0, :k, 0] = sv[:k]
+        g32[0, 1, :k, 1] = sv[:k]
+        x, g = I.cast_np(x32, dtype), I.cast_np(g32, dtype)
+        xt, gt = I.to_torch(x, dtype, device), I.to_torch(g, dtype, device)
+        what = "gs-channel-pairs %s %s align=%s %s" % (dtype, PAD[pad], align, (N, C, H, W, Ho, Wo))
+        with aclnn.option("gs_variant", 2):  # the ring kernel also where a pair-layout variant would take the shape
+            out = torch.empty((N, C, Ho, Wo), dtype=xt.dtype, device=device)
+            hs = [aclnn.tensor_handle(t) for t in (xt, gt, out)]
+            st, _, ex = aclnn.get_workspace_size_grid_sampler2d(hs[0], hs[1], 0, pad, align, hs[2])
+            assert st == 0
+            assert aclnn.executor_variant(ex).startswith("lds_ring_pairs"), (what, aclnn.executor_variant(ex))
+            aclnn.destroy_executor(ex)
+            for h in hs:
+                aclnn.destroy_tensor(h)
+            y = I.from_torch(aclnn.grid_sampler2d(xt, gt, 0, pad, align), dtype)
+        y_ref = oracle.grid_sampler2d(x, g, 0, pad, align, dtype=I.oracle_code(dtype))
+        _check(y, y_ref, dtype, 0, what)
+        _assert_same_bits(y, y_ref, what)
+        with aclnn.option("gs_variant", 3):  # single-channel stages
+            y_single = I.from_torch(aclnn.grid_sampler2d(xt, gt, 0, pad, align), dtype)
+        _assert_same_bits(y, y_single, what + " (against single-channel stages)")
+        if not align:
+            with aclnn.option("gs_variant", 2), aclnn.option("grid_sampler2d_rule", 1):
+                y2 = I.from_torch(aclnn.grid_sampler2d(xt, gt, 0, pad, align), dtype)
+            y2_ref = oracle.grid_sampler2d_arch35(x, g, pad, align, dtype=I.oracle_code(dtype))
+            _assert_same_bits(y2, y2_ref, what + " (second rule)")
+
+
 @pytest.mark.parametrize("dtype", I.DTYPES)
 @pytest.mark.parametrize("interp", [0, 1])
 @pytest.mark.parametrize("pad", [0, 1, 2])
