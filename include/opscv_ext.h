@@ -94,7 +94,7 @@ ACLNN_API aclnnStatus opscvGridSampler2DNoAlloc(const aclTensor* input, const ac
  *                                                            of the 3-D sampler gradient read it
  *   "reference_ub_bytes"    OPSCV_REFERENCE_UB_BYTES         unified buffer of the reference's device (default
  *                                                            253952): gates its replicating nearest-resize template
- *   "gs_variant"            OPSCV_GS_VARIANT=direct|ring     0 automatic, 1 direct kernel, 2 no pair-layout variant,
+ *   "gs_variant"            OPSCV_GS_VARIANT=direct|ring|single   0 automatic, 1 direct kernel, 2 no pair-layout variant,
  *                                                            3 as 2 and single-channel stages in the ring kernel
  *   "resize_variant"        OPSCV_RESIZE_VARIANT=generic|register|band   0 automatic, 1 per-element kernels,
  *                                                            2 register-band kernel, 3 no flat LDS kernel

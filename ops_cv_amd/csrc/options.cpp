@@ -38,7 +38,7 @@ Store& store()
     static std::once_flag once;
     std::call_once(once, [] {
         if (const char* v = getenv("OPSCV_GS_VARIANT")) {
-            s.gs_variant = (v[0] == 'd') ? kGsDirect : (v[0] == 'r' ? kGsRing : kGsAuto);
+            s.gs_variant = (v[0] == 'd') ? kGsDirect : (v[0] == 'r' ? kGsRing : (v[0] == 's' ? kGsRingSingle : kGsAuto));
         }
         if (const char* v = getenv("OPSCV_RESIZE_VARIANT")) {
             s.resize_variant = (v[0] == 'g') ? kResizeGeneric

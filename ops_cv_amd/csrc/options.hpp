@@ -19,7 +19,7 @@ enum GsRule : int32_t { kRuleGridSampler2D = 0, kRuleGridSampleArch35 = 1 };
 enum Gs3dGradVariant : int32_t { kGs3dGradAuto = 0, kGs3dGradOrdered = 1, kGs3dGradGather = 2 };
 
 struct Options {
-    int32_t gs_variant = kGsAuto;            // OPSCV_GS_VARIANT = direct | ring
+    int32_t gs_variant = kGsAuto;            // OPSCV_GS_VARIANT = direct | ring | single
     int32_t resize_variant = kResizeAuto;    // OPSCV_RESIZE_VARIANT = generic | register | band
     int32_t nearest_variant = kNearestAuto;  // OPSCV_NEAREST_VARIANT = gather
     int64_t reference_cores = 64;            // OPSCV_REFERENCE_CORES
