@@ -183,10 +183,15 @@ static LdsPlan make_lds_plan_rows(const GridSamplerArgs& a, bool pad_rows)
         const int64_t last_block = a.C - (int64_t)(cblocks - 1) * cpb;
         const bool even_counts = p.wide_blocks != 0 ? (p.chans_wide % 2 == 0 && p.chans_per_block % 2 == 0)
                                                     : (cpb % 2 == 0 && last_block % 2 == 0);
-        if (a.interp == 0 && esz == 2 && p.cls == 1 && p.ppt == 4 && plain && !padded && p.row_shift == 0 &&
-            p.copy_gran == 16 && a.C % 2 == 0 && even_counts && a.force_variant != kGsRingSingle) {
+        if (a.interp == 0 && esz == 2 && p.cls == 1 && p.ppt == 4 && plain && !padded && p.copy_gran == 16 &&
+            a.C % 2 == 0 && even_counts && a.force_variant != kGsRingSingle) {
             p.chan_pairs = true;
             p.lds_bytes = (uint32_t)(kPairsNbuf * kPairsPitch);
+            if (p.row_shift != 0) {
+                // an element is four bytes wide here: one chunk per row shifts a column by eight banks, as two do in
+                // the single-channel layout
+                p.row_shift = 7 | (1 << 8);
+            }
         }
     }
     p.ok = true;

@@ -707,7 +707,9 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
                                 const u32x4 a = regs[k][u][0], b = regs[k][u][1];
                                 const u32x4 lo = {lows(a.x, b.x), highs(a.x, b.x), lows(a.y, b.y), highs(a.y, b.y)};
                                 const u32x4 hi = {lows(a.z, b.z), highs(a.z, b.z), lows(a.w, b.w), highs(a.w, b.w)};
-                                const uint32_t at = slot + unit[u] * 32u;
+                                // (the bank-spreading layout moves whole 16-byte chunks of the plane, which are the
+                                // 32-byte pieces here)
+                                const uint32_t at = slot + 2u * lds_swizzle(unit[u] * 16u, (uint32_t)row_shift);
                                 *reinterpret_cast<lds_u32x4_ptr_t>((uintptr_t)at) = lo;
                                 *reinterpret_cast<lds_u32x4_ptr_t>((uintptr_t)(at + 16u)) = hi;
                             }

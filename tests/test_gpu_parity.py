@@ -216,13 +216,13 @@ def test_grid_sampler_rows_padded_in_lds(oracle, device, dtype, interp, pad):
 
 
 @pytest.mark.parametrize("dtype", ["fp16", "bf16"])
-@pytest.mark.parametrize("pad", [0, 2])
+@pytest.mark.parametrize("pad", [0, 1, 2])
 @pytest.mark.parametrize("align", [False, True])
 def test_grid_sampler_channel_pairs_in_lds(oracle, device, dtype, pad, align):
     """bilinear samples of 16-bit planes of up to 8 KiB with an even channel count, which the ring kernel stages two
     channels at a time, interleaved: planes that are not whole loads for every loader lane, a last channel block
     shorter than the others, the uneven split of two workgroups per CU, fewer stages than the loaders keep on their
-    way, both coordinate rules; bit for bit against the oracle and against the same kernel with
+    way, border padding on rows of 128 bytes (the rotated layout) and on other rows, both coordinate rules; bit for bit against the oracle and against the same kernel with
     single-channel stages"""
     import torch
     from ops_cv_amd import aclnn
