@@ -739,7 +739,7 @@ __global__ __launch_bounds__(PAIRS ? kPairThreads : kApplyThreads, PAIRS ? 6 : 1
             cm = other2 > cm ? other2 : cm;
         }
         kmax[i] = __builtin_amdgcn_readfirstlane(km);
-        any_rest[i] = __builtin_amdgcn_readfirstlane(cm) > (uint32_t)kHeld;
+        any_rest[i] = (uint32_t)__builtin_amdgcn_readfirstlane(cm) > (uint32_t)kHeld;
     }
     T* dx_n = dx + n * p.C * (int64_t)plane_px;  // the batch item's gradient planes
     // the lists are in registers or LDS from here on: nothing below waits for memory except an overfull spill area
