@@ -166,6 +166,53 @@ def test_random_grid_sampler2d_pair_layouts(oracle, device, aclnn):
     assert seen.get("lds_pair", 0) >= 3 and seen.get("lds_pair_bicubic", 0) >= 5, seen
 
 
+def test_random_grid_sampler2d_channel_pairs(oracle, device, aclnn):
+    """bilinear samples of 16-bit planes between 2 and 8 KiB with enough batch items and channels that the ring kernel
+    gives every channel block several channels: where that count is even it stages two channels at a time
+    (interleaved in LDS), where it is odd or the rows get padded it does not -- checked all the same, and the
+    variant that ran is counted so that the sweep cannot miss the interleaved stages.  Random row counts and widths,
+    every padding, both alignments, smooth and scattered grids with special values sprinkled in."""
+    import torch
+    rng = np.random.default_rng(9008 + SEED_SHIFT)
+    seen = {}
+    for case in range(36):
+        dtype = ("fp16", "bf16")[case % 2]
+        N = int(rng.choice([8, 16, 24, 32]))
+        C = int(rng.integers(8, 40)) * (2 if case % 4 != 3 else 1)
+        W = 64 if case % 3 != 2 else 8 * int(rng.integers(3, 13))
+        H = int(rng.integers(max(2, 1100 // W), 4096 // W + 1))  # planes above the 2 KiB class, up to 8 KiB
+        Ho, Wo = int(rng.integers(24, 80)), int(rng.integers(24, 80))
+        pad, align = int(rng.integers(0, 3)), bool(rng.integers(0, 2))
+        _say("gs2d channel pairs", dtype, N, C, H, W, Ho, Wo, pad, align)
+        x32 = rng.standard_normal((N, C, H, W)).astype(np.float32)
+        x32 += np.arange(C, dtype=np.float32).reshape(1, C, 1, 1)
+        x = I.cast_np(x32, dtype)
+        if case % 3 == 0:
+            g32 = rng.uniform(-1.4, 1.4, (N, Ho, Wo, 2)).astype(np.float32)
+        else:
+            g32 = I.affine_grid(rng, N, Ho, Wo, max_deg=40.0, scale=(0.6, 1.4), shift=0.4)
+        if case % 2 == 1:
+            g32 = _sprinkle(rng, g32, H, W, align)
+        g = I.cast_np(g32, dtype)
+        tx, tg = I.to_torch(x, dtype, device), I.to_torch(g, dtype, device)
+        ty = torch.empty((N, C, Ho, Wo), dtype=tx.dtype, device=device)
+        with aclnn.option("gs_variant", 2):  # the ring kernel also where a pair-layout variant would take the shape
+            hs = [aclnn.tensor_handle(t) for t in (tx, tg, ty)]
+            st, _, ex = aclnn.get_workspace_size_grid_sampler2d(hs[0], hs[1], 0, pad, align, hs[2])
+            assert st == 0
+            variant = aclnn.executor_variant(ex)
+            key = "pairs" if variant.startswith("lds_ring_pairs") else "other"
+            seen[key] = seen.get(key, 0) + 1
+            aclnn.destroy_executor(ex)
+            for h in hs:
+                aclnn.destroy_tensor(h)
+            y = aclnn.grid_sampler2d(tx, tg, 0, pad, align, out=ty)
+            torch.cuda.synchronize()
+        ref = oracle.grid_sampler2d(x, g, 0, pad, align, dtype=I.oracle_code(dtype))
+        _same(I.from_torch(y, dtype), ref, dtype, (case, dtype, N, C, H, W, Ho, Wo, pad, align, variant))
+    assert seen.get("pairs", 0) >= 8, seen
+
+
 def test_random_grid_sampler2d_large_planes(oracle, device, aclnn):
     """input planes from a few KB to beyond the largest LDS class (the direct kernel), few channels"""
     import torch
