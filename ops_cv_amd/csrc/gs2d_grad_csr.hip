@@ -561,17 +561,22 @@ __global__ __launch_bounds__(PAIRS ? kPairThreads : kApplyThreads, PAIRS ? 6 : 1
             }
             const char* go_bytes = reinterpret_cast<const char*>(go_n);
             u32x4 regs[kPairDepth][UPL][CB];
+            // A load that has nothing to fetch -- past the last step, or a plane that a last, partial step does not
+            // have -- reads an address of its own near the start of the planes: were two of a lane's loads to ask for
+            // the same address, the compiler would make the second a register copy of the first, and a copy waits
+            // for its load (`s_waitcnt vmcnt(0)` behind the loads of every step, which is the end of the prefetch).
             auto issue = [&](u32x4 (*r)[CB], int32_t s) {
                 const bool real = s < steps;
                 const char* base = go_bytes + (real ? (size_t)unit_of(s) * buf_bytes : (size_t)0);
-                const int32_t left = real ? nchan - s * CB : 0;  // planes of a last, partial step: the first again
+                const int32_t left = real ? nchan - s * CB : 0;
 #pragma unroll
                 for (int u = 0; u < UPL; u++) {
-                    const uint32_t off = real ? unit[u] * 16u : 0u;
 #pragma unroll
                     for (int j = 0; j < CB; j++) {
-                        const uint32_t plane = (j < left) ? (uint32_t)j * row_bytes : 0u;
-                        r[u][j] = *reinterpret_cast<const u32x4*>(base + plane + off);
+                        const uint32_t spare = (uint32_t)(u * CB + j) * 16u;
+                        const uint32_t idle = spare < row_bytes ? spare : row_bytes - 16u;
+                        const uint32_t off = (j < left) ? (uint32_t)j * row_bytes + unit[u] * 16u : idle;
+                        r[u][j] = *reinterpret_cast<const u32x4*>(base + off);
                     }
                 }
             };
