@@ -73,6 +73,8 @@ inline bool gs_shapes_ok(const GridSamplerArgs& a)
 // its assumptions (input plane too large for LDS); the caller then falls back to the direct variant.
 hipError_t run_gs2d_lds(const GridSamplerArgs& a, hipStream_t stream, bool* handled);
 const char* gs2d_lds_variant_name(const GridSamplerArgs& a);
+// whether that variant would stage two channels at a time, interleaved (gs2d_lds_kernel.hpp, CHANNEL_PAIRS)
+bool gs2d_lds_channel_pairs(const GridSamplerArgs& a);
 
 // Pair-layout LDS variant (gs2d_pair.hip): bilinear, 16-bit elements, several output pixels per input pixel; same
 // convention as run_gs2d_lds.

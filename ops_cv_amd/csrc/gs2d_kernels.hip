@@ -452,6 +452,14 @@ namespace {
 // (benchmark and test knobs)
 bool force_direct(const GridSamplerArgs& a) { return a.force_variant == kGsDirect; }
 bool force_ring(const GridSamplerArgs& a) { return a.force_variant == kGsRing || a.force_variant == kGsRingSingle; }
+// Bilinear samples that the ring kernel takes two channels at a time go there rather than to the pair-layout kernel,
+// up to eight output pixels per input pixel (fp16 N16 C128 64x64 -> 128x128: 18.5 us against the pair layout's 21.9,
+// -> 160x160 29.5 against 41.5, bf16 N8 C128 32x128 -> 80x320 16.4 against 25.2; beyond, the pair layout's twelve pixels
+// per lane stage every plane less often: fp16 N16 C64 64x64 -> 192x192 26.2 against 20.6).
+bool ring_before_pair(const GridSamplerArgs& a)
+{
+    return a.interp == 0 && a.Hout * a.Wout <= 8 * a.Hin * a.Win && gs2d_lds_channel_pairs(a);
+}
 }  // namespace
 
 // The second coordinate rule (bilinear only) is implemented by the LDS ring and by a direct kernel of its own.
@@ -467,7 +475,7 @@ const char* grid_sampler2d_variant(const GridSamplerArgs& a)
         return "nhwc";
     }
     if (!force_direct(a)) {
-        const char* n = force_ring(a) ? nullptr : gs2d_pair_variant_name(a);
+        const char* n = (force_ring(a) || ring_before_pair(a)) ? nullptr : gs2d_pair_variant_name(a);
         if (n == nullptr) {
             n = gs2d_lds_variant_name(a);
         }
@@ -510,7 +518,7 @@ hipError_t launch_grid_sampler2d(const GridSamplerArgs& a, hipStream_t stream)
     }
     if (!force_direct(a)) {
         bool handled = false;
-        hipError_t e = force_ring(a) ? hipSuccess : run_gs2d_pair(a, stream, &handled);
+        hipError_t e = (force_ring(a) || ring_before_pair(a)) ? hipSuccess : run_gs2d_pair(a, stream, &handled);
         if (handled || e != hipSuccess) {
             return e;
         }

@@ -166,7 +166,25 @@ static LdsPlan make_lds_plan_rows(const GridSamplerArgs& a, bool pad_rows)
     }
     // all tiles of one (n, channel block) group on one XCD: needs the group count to be a multiple of 8
     p.xcd_swizzle = ((a.N * cblocks) % 8 == 0) ? 1 : 0;
-    if (padded) {
+    // Two channels per stage, interleaved in LDS (gs2d_lds_kernel.hpp, CHANNEL_PAIRS): bilinear samples of 16-bit
+    // elements in the 8 KiB class with four pixels per lane, plain layout (rows padded or not), every block's channels
+    // in pairs.
+    {
+        const int64_t last_block = a.C - (int64_t)(cblocks - 1) * cpb;
+        const bool even_counts = p.wide_blocks != 0 ? (p.chans_wide % 2 == 0 && p.chans_per_block % 2 == 0)
+                                                    : (cpb % 2 == 0 && last_block % 2 == 0);
+        if (a.interp == 0 && esz == 2 && p.cls == 1 && p.ppt == 4 && plain && p.copy_gran == 16 &&
+            2 * staged_bytes + 16 <= kPairsPitch && a.C % 2 == 0 && even_counts && a.force_variant != kGsRingSingle) {
+            p.chan_pairs = true;
+            p.lds_bytes = (uint32_t)(kPairsNbuf * kPairsPitch);
+            if (p.row_shift != 0) {
+                // an element is four bytes wide here: one chunk per row shifts a column by eight banks, as two do in
+                // the single-channel layout
+                p.row_shift = 7 | (1 << 8);
+            }
+        }
+    }
+    if (padded && !p.chan_pairs) {
         // Only the loaders' literal-count loop pads rows; what it asks for (gs2d_lds_kernel.hpp): single-plane
         // stages, every block with at least as many channels as the ring runs ahead, and a copy count per loader
         // that the loop is instantiated for.
@@ -175,23 +193,6 @@ static LdsPlan make_lds_plan_rows(const GridSamplerArgs& a, bool pad_rows)
         const int64_t copies = ((staged_bytes + 1023) / 1024 + kLoaderWaves[p.cls] - 1) / kLoaderWaves[p.cls];
         if (cgs != 1 || fewest < kNbuf[p.cls] - 1 || copies > 16 || (kNbuf[p.cls] - 2) * copies > 63) {
             return p;
-        }
-    }
-    // Two channels per stage, interleaved in LDS (gs2d_lds_kernel.hpp, CHANNEL_PAIRS): bilinear samples of 16-bit
-    // elements in the 8 KiB class with four pixels per lane, plain unpadded layout, every block's channels in pairs.
-    {
-        const int64_t last_block = a.C - (int64_t)(cblocks - 1) * cpb;
-        const bool even_counts = p.wide_blocks != 0 ? (p.chans_wide % 2 == 0 && p.chans_per_block % 2 == 0)
-                                                    : (cpb % 2 == 0 && last_block % 2 == 0);
-        if (a.interp == 0 && esz == 2 && p.cls == 1 && p.ppt == 4 && plain && !padded && p.copy_gran == 16 &&
-            a.C % 2 == 0 && even_counts && a.force_variant != kGsRingSingle) {
-            p.chan_pairs = true;
-            p.lds_bytes = (uint32_t)(kPairsNbuf * kPairsPitch);
-            if (p.row_shift != 0) {
-                // an element is four bytes wide here: one chunk per row shifts a column by eight banks, as two do in
-                // the single-channel layout
-                p.row_shift = 7 | (1 << 8);
-            }
         }
     }
     p.ok = true;
@@ -207,6 +208,12 @@ const char* gs2d_lds_variant_name(const GridSamplerArgs& a)
     static const char* names[5] = {"lds_ring_p2064_4x4", "lds_ring_p8208_1x6", "lds_ring_p16400_1x4",
                                    "lds_ring_p32784_1x4", "lds_ring_p81904_1x2"};
     return p.chan_pairs ? "lds_ring_pairs_p16400_2x2" : names[p.cls];
+}
+
+bool gs2d_lds_channel_pairs(const GridSamplerArgs& a)
+{
+    const LdsPlan p = make_lds_plan(a);
+    return p.ok && p.chan_pairs;
 }
 
 hipError_t run_gs2d_lds(const GridSamplerArgs& a, hipStream_t stream, bool* handled)

@@ -668,13 +668,22 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
             const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds;
             const uint32_t lid = lwave * 64u + lane;
             const uint32_t units = plane_bytes >> 4;
-            uint32_t unit[UPL];
+            uint32_t unit[UPL], place[UPL];
             bool mine[UPL];
 #pragma unroll
             for (int u = 0; u < UPL; u++) {
                 unit[u] = lid + (uint32_t)u * (64u * LWAVES);
                 mine[u] = unit[u] < units;
                 unit[u] = mine[u] ? unit[u] : units - 1u;  // a lane without a unit reads the last one again
+                // Where the unit's 32 bytes go in a slot: twice its offset in the single-channel layout, which is
+                // the unit's offset in the plane, or -- `ldsw` > W, rows padded to a multiple of 128 bytes (a row is
+                // whole units) -- row by row; the bank-spreading layout moves whole 16-byte chunks of that layout.
+                uint32_t staged = unit[u] * 16u;
+                if (ldsw != W) {
+                    const uint32_t elem = unit[u] * 8u, row = elem / (uint32_t)W;
+                    staged = (row * (uint32_t)ldsw + (elem - row * (uint32_t)W)) * 2u;
+                }
+                place[u] = 2u * lds_swizzle(staged, (uint32_t)row_shift);
             }
             u32x4 regs[RDEPTH][UPL][2];
             auto issue = [&](u32x4 (*r)[2], int32_t st) {
@@ -707,9 +716,7 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
                                 const u32x4 a = regs[k][u][0], b = regs[k][u][1];
                                 const u32x4 lo = {lows(a.x, b.x), highs(a.x, b.x), lows(a.y, b.y), highs(a.y, b.y)};
                                 const u32x4 hi = {lows(a.z, b.z), highs(a.z, b.z), lows(a.w, b.w), highs(a.w, b.w)};
-                                // (the bank-spreading layout moves whole 16-byte chunks of the plane, which are the
-                                // 32-byte pieces here)
-                                const uint32_t at = slot + 2u * lds_swizzle(unit[u] * 16u, (uint32_t)row_shift);
+                                const uint32_t at = slot + place[u];
                                 *reinterpret_cast<lds_u32x4_ptr_t>((uintptr_t)at) = lo;
                                 *reinterpret_cast<lds_u32x4_ptr_t>((uintptr_t)(at + 16u)) = hi;
                             }
