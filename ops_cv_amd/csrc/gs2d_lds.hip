@@ -189,10 +189,18 @@ static LdsPlan make_lds_plan_rows(const GridSamplerArgs& a, bool pad_rows)
         const int64_t last_block = a.C - (int64_t)(cblocks - 1) * cpb;
         const bool even_counts = p.wide_blocks != 0 ? (p.chans_wide % 2 == 0 && p.chans_per_block % 2 == 0)
                                                     : (cpb % 2 == 0 && last_block % 2 == 0);
-        if (a.interp == 0 && esz == 2 && p.cls == 1 && p.ppt == 4 && plain && p.copy_gran == 16 &&
-            2 * staged_bytes + 16 <= kPairsPitch && a.C % 2 == 0 && even_counts && a.force_variant != kGsRingSingle) {
+        const bool small = p.cls == 1 && p.ppt == 4 && 2 * staged_bytes + 16 <= kPairsPitch;
+        // The 16 KiB class where there are at least two output pixels per input pixel (eight pixels per lane then):
+        // fp16 N16 C128 96x64 -> 192x128 45.0 us with single channels, 29.3 in pairs (the pair layout of
+        // gs2d_pair.hip: 55.8), bf16 N8 C128 64x128 -> 128x256 26.1 and 22.3 (24.4).  One output pixel per input
+        // pixel is the loaders' game, and theirs is the better one with the copy engine: 96x64 -> 96x64 24.0 and 27.1.
+        const bool large = p.cls == 2 && p.ppt == 8 && 2 * staged_bytes + 16 <= kPairsPitchLarge &&
+                           out_plane >= 2 * a.Hin * a.Win;
+        if (a.interp == 0 && esz == 2 && (small || large) && plain && p.copy_gran == 16 && a.C % 2 == 0 &&
+            even_counts && a.force_variant != kGsRingSingle) {
             p.chan_pairs = true;
-            p.lds_bytes = (uint32_t)(kPairsNbuf * kPairsPitch);
+            p.pairs_pitch = small ? kPairsPitch : kPairsPitchLarge;
+            p.lds_bytes = (uint32_t)(kPairsNbuf * p.pairs_pitch);
             if (p.row_shift != 0) {
                 // an element is four bytes wide here: one chunk per row shifts a column by eight banks, as two do in
                 // the single-channel layout
@@ -223,7 +231,8 @@ const char* gs2d_lds_variant_name(const GridSamplerArgs& a)
     }
     static const char* names[5] = {"lds_ring_p2064_4x4", "lds_ring_p8208_1x6", "lds_ring_p16400_1x4",
                                    "lds_ring_p32784_1x4", "lds_ring_p81904_1x2"};
-    return p.chan_pairs ? "lds_ring_pairs_p16400_2x2" : names[p.cls];
+    return p.chan_pairs ? (p.pairs_pitch == kPairsPitch ? "lds_ring_pairs_p16400_2x2" : "lds_ring_pairs_p32784_2x2")
+                        : names[p.cls];
 }
 
 bool gs2d_lds_channel_pairs(const GridSamplerArgs& a)

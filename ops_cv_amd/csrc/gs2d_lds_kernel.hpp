@@ -662,7 +662,7 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
             // same on all paths and exact.  Slot s % 2 is written between the barriers of stages s - 1 and s, while
             // the samplers read the other one.
             constexpr int UPL = ((PITCH - 16) / 2 / 16 + LWAVES * 64 - 1) / (LWAVES * 64);
-            constexpr int RDEPTH = 3;
+            constexpr int RDEPTH = UPL <= 2 ? 3 : 2;  // 48 or 64 registers of loads
             typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
             typedef u32x4 __attribute__((address_space(3))) * lds_u32x4_ptr_t;
             const uint32_t lds_base = (uint32_t)(uintptr_t)(lds_ptr_t)lds;

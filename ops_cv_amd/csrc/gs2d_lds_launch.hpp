@@ -32,10 +32,12 @@ struct LdsPlan {
     // two neighbouring channels per stage, interleaved in LDS (gs2d_lds_kernel.hpp, CHANNEL_PAIRS); the channel counts
     // above stay in channels, the launch halves them
     bool chan_pairs = false;
+    int32_t pairs_pitch = 0;  // kPairsPitch or kPairsPitchLarge
 };
 
-// the channel-pair kernels' LDS: two slots of two 8 KiB planes and the zeros
+// the channel-pair kernels' LDS: two slots of two planes of the 8 KiB or of the 16 KiB class and the zeros
 constexpr int kPairsPitch = 16400;
+constexpr int kPairsPitchLarge = 32784;
 constexpr int kPairsNbuf = 2;
 constexpr int kPairsLoaderWaves = 4;
 

@@ -5,10 +5,10 @@ namespace opscv {
 
 namespace {
 
-template <typename T, int ADJ>
+template <typename T, int PPT, int ADJ, int PITCH>
 hipError_t launch_pairs(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t stream)
 {
-    auto kernel = gs2d_lds_kernel<T, 0, kSamplerWaves, kPairsLoaderWaves, 4, ADJ, 1, kPairsNbuf, kPairsPitch, false, true>;
+    auto kernel = gs2d_lds_kernel<T, 0, kSamplerWaves, kPairsLoaderWaves, PPT, ADJ, 1, kPairsNbuf, PITCH, false, true>;
     static std::atomic<uint32_t> lds_allowed{0};
     const hipError_t ea = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kLdsLimit, lds_allowed);
     if (ea != hipSuccess) {
@@ -26,17 +26,29 @@ hipError_t launch_pairs(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t 
     return hipGetLastError();
 }
 
+template <typename T, int PPT, int PITCH>
+hipError_t launch_pairs_adj(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t stream)
+{
+    return p.adj == 2 ? launch_pairs<T, PPT, 2, PITCH>(a, p, stream) : launch_pairs<T, PPT, 1, PITCH>(a, p, stream);
+}
+
 template <typename T>
 hipError_t launch_pairs_typed(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t stream)
 {
-    return p.adj == 2 ? launch_pairs<T, 2>(a, p, stream) : launch_pairs<T, 1>(a, p, stream);
+    if (p.pairs_pitch == kPairsPitch && p.ppt == 4) {
+        return launch_pairs_adj<T, 4, kPairsPitch>(a, p, stream);
+    }
+    if (p.pairs_pitch == kPairsPitchLarge && p.ppt == 8) {
+        return launch_pairs_adj<T, 8, kPairsPitchLarge>(a, p, stream);
+    }
+    return hipErrorInvalidValue;
 }
 
 }  // namespace
 
 hipError_t lds_launch_channel_pairs(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t stream)
 {
-    if (!p.chan_pairs || p.ppt != 4) {
+    if (!p.chan_pairs) {
         return hipErrorInvalidValue;
     }
     switch (a.elem) {

@@ -230,10 +230,11 @@ def test_grid_sampler_channel_pairs_in_lds(oracle, device, dtype, pad, align):
     # (the launch plan takes channel pairs where every channel block gets an even number of channels: 4 per block,
     # 2 with a last block of 2, 6 on planes of 200 16-byte units, 4 with 25 blocks, 2 = a single stage per block,
     # and the headline's 22 + 10)
-    # and, last, rows of 112, 80 and 96 bytes, which are staged padded to 128: 56 x 56, 40 x 40 and 48 x 44 planes)
+    # then rows of 112, 80 and 96 bytes, which are staged padded to 128: 56 x 56, 40 x 40 and 48 x 44 planes; last,
+    # planes of the 16 KiB class with two output pixels or more per input pixel)
     shapes = [(16, 64, 64, 64, 64, 64), (16, 26, 64, 64, 64, 64), (32, 48, 25, 64, 64, 64), (8, 100, 62, 64, 33, 70),
               (64, 12, 48, 64, 40, 40), (16, 256, 64, 64, 64, 64), (16, 64, 56, 56, 56, 56), (32, 48, 40, 40, 64, 64),
-              (16, 96, 44, 48, 50, 60)]
+              (16, 96, 44, 48, 50, 60), (16, 64, 96, 64, 192, 128), (8, 96, 64, 128, 100, 180)]
     for (N, C, H, W, Ho, Wo) in shapes:
         x32 = rng.standard_normal((N, C, H, W)).astype(np.float32)
         x32 += np.arange(C, dtype=np.float32).reshape(1, C, 1, 1)  # a channel taken for its neighbour shows
