@@ -75,6 +75,8 @@ hipError_t run_gs2d_lds(const GridSamplerArgs& a, hipStream_t stream, bool* hand
 const char* gs2d_lds_variant_name(const GridSamplerArgs& a);
 // whether that variant would stage two channels at a time, interleaved (gs2d_lds_kernel.hpp, CHANNEL_PAIRS)
 bool gs2d_lds_channel_pairs(const GridSamplerArgs& a);
+// ... and the average number of channels that a channel block then takes (0 where it stages single channels)
+int64_t gs2d_lds_channel_pairs_per_block(const GridSamplerArgs& a);
 
 // Pair-layout LDS variant (gs2d_pair.hip): bilinear, 16-bit elements, several output pixels per input pixel; same
 // convention as run_gs2d_lds.

@@ -456,8 +456,17 @@ bool force_ring(const GridSamplerArgs& a) { return a.force_variant == kGsRing ||
 // up to eight output pixels per input pixel (fp16 N16 C128 64x64 -> 128x128: 18.5 us against the pair layout's 21.9,
 // -> 160x160 29.5 against 41.5, bf16 N8 C128 32x128 -> 80x320 16.4 against 25.2; beyond, the pair layout's twelve pixels
 // per lane stage every plane less often: fp16 N16 C64 64x64 -> 192x192 26.2 against 20.6).
+// Bicubic samples under zeros padding likewise where a plane is above 4 KiB and a channel block takes 32 channels or
+// more, over which the sixteen tap offsets of a pixel are decided once (fp16 N16 C256 64x64 -> 64x64: 29.1 us
+// against the bicubic pair layout's 31.5, 40x96 28.4 against 35.0, 128x32 31.4 against 38.9; planes of 32x64 19.0
+// against 14.0, N8 C64 64x64 with eight channels per block 11.9 against 7.6).  Under border padding the pair layout's
+// staged margins win (64x64: 43.9 against 31.0); reflection has no pair layout and comes here anyway.
+constexpr int64_t kBicubicRingChannels = 32;  // 16 per block: 19.6 us against 17.5, 24: 24.1 against 24.3
 bool ring_before_pair(const GridSamplerArgs& a)
 {
+    if (a.interp == 2) {
+        return a.pad == 0 && a.Hin * a.Win * 2 > 4096 && gs2d_lds_channel_pairs_per_block(a) >= kBicubicRingChannels;
+    }
     return a.interp == 0 && a.Hout * a.Wout <= 8 * a.Hin * a.Win && gs2d_lds_channel_pairs(a);
 }
 }  // namespace

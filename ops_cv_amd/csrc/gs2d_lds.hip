@@ -126,9 +126,9 @@ static LdsPlan make_lds_plan_rows(const GridSamplerArgs& a, bool pad_rows)
             cb = cb < 1 ? 1 : cb;
             int64_t per = (a.C + cb - 1) / cb;
             per = (per + cgs - 1) / cgs * cgs;
-            // (16-bit bilinear: an even count lets the kernel take two channels per stage; worth one more channel
+            // (16-bit bilinear and bicubic: an even count lets the kernel take two channels per stage; worth one more channel
             // where a block has eight or more)
-            if (esz == 2 && a.interp == 0 && per >= 8 && per % 2 != 0 && a.C % 2 == 0) {
+            if (esz == 2 && a.interp != 1 && per >= 8 && per % 2 != 0 && a.C % 2 == 0) {
                 per++;
             }
             cb = (a.C + per - 1) / per;
@@ -157,7 +157,13 @@ static LdsPlan make_lds_plan_rows(const GridSamplerArgs& a, bool pad_rows)
     // A wrong guess about who comes first costs balance, never correctness.
     if (cgs == 1 && cblocks % 2 == 0 && cpb >= 8 && a.C == cblocks * cpb &&
         a.N * p.tiles_per_n * cblocks == 2 * (int64_t)compute_unit_count() && (a.N * cblocks / 2) % 8 == 0) {
-        const int64_t wide = plain ? (cpb * 11 + 4) / 8 : (cpb * 5 + 2) / 4;
+        int64_t wide = plain ? (cpb * 11 + 4) / 8 : (cpb * 5 + 2) / 4;
+        // 16-bit bilinear and bicubic samples: even counts on both sides, so that the kernel can take two channels per
+        // stage (below).  fp16 N16 C128 64x64 -> 64x64, eight channels per block on average: 11 + 5 in single stages
+        // 7.9 us, 10 + 6 in pairs 7.4, 12 + 4 in pairs 7.1; bicubic 29.7, 19.6 and 19.5.
+        if (esz == 2 && a.interp != 1 && plain && cpb % 2 == 0 && wide % 2 != 0 && a.force_variant != kGsRingSingle) {
+            wide++;
+        }
         const int64_t narrow = 2 * cpb - wide;
         if (narrow >= 1) {
             p.wide_blocks = (uint32_t)(cblocks / 2);
@@ -189,14 +195,15 @@ static LdsPlan make_lds_plan_rows(const GridSamplerArgs& a, bool pad_rows)
         const int64_t last_block = a.C - (int64_t)(cblocks - 1) * cpb;
         const bool even_counts = p.wide_blocks != 0 ? (p.chans_wide % 2 == 0 && p.chans_per_block % 2 == 0)
                                                     : (cpb % 2 == 0 && last_block % 2 == 0);
-        const bool small = p.cls == 1 && p.ppt == 4 && 2 * staged_bytes + 16 <= kPairsPitch;
+        // (bicubic: one or two pixels per lane, sixteen 4-byte reads per pixel for both channels)
+        const bool small = p.cls == 1 && (a.interp == 2 ? p.ppt <= 2 : p.ppt == 4) && 2 * staged_bytes + 16 <= kPairsPitch;
         // The 16 KiB class where there are at least two output pixels per input pixel (eight pixels per lane then):
         // fp16 N16 C128 96x64 -> 192x128 45.0 us with single channels, 29.3 in pairs (the pair layout of
         // gs2d_pair.hip: 55.8), bf16 N8 C128 64x128 -> 128x256 26.1 and 22.3 (24.4).  One output pixel per input
         // pixel is the loaders' game, and theirs is the better one with the copy engine: 96x64 -> 96x64 24.0 and 27.1.
         const bool large = p.cls == 2 && p.ppt == 8 && 2 * staged_bytes + 16 <= kPairsPitchLarge &&
                            out_plane >= 2 * a.Hin * a.Win;
-        if (a.interp == 0 && esz == 2 && (small || large) && plain && p.copy_gran == 16 && a.C % 2 == 0 &&
+        if (a.interp != 1 && esz == 2 && (small || (large && a.interp == 0)) && plain && p.copy_gran == 16 && a.C % 2 == 0 &&
             even_counts && a.force_variant != kGsRingSingle) {
             p.chan_pairs = true;
             p.pairs_pitch = small ? kPairsPitch : kPairsPitchLarge;
@@ -239,6 +246,12 @@ bool gs2d_lds_channel_pairs(const GridSamplerArgs& a)
 {
     const LdsPlan p = make_lds_plan(a);
     return p.ok && p.chan_pairs;
+}
+
+int64_t gs2d_lds_channel_pairs_per_block(const GridSamplerArgs& a)
+{
+    const LdsPlan p = make_lds_plan(a);
+    return (p.ok && p.chan_pairs) ? a.C / (int64_t)p.cblocks : 0;
 }
 
 hipError_t run_gs2d_lds(const GridSamplerArgs& a, hipStream_t stream, bool* handled)

@@ -610,8 +610,8 @@ __global__ __launch_bounds__((SWAVES + LWAVES) * 64) __attribute__((amdgpu_waves
     const uint32_t cb = fast_div(group, N);
     const uint32_t n = group - cb * N.div;
 
-    static_assert(!CHANNEL_PAIRS || (sizeof(T) == 2 && INTERP == 0 && CGS == 1 && NBUF == 2 && !SHIFTED_PLANES),
-                  "channel pairs: 16-bit bilinear, one pair per stage, two slots");
+    static_assert(!CHANNEL_PAIRS || (sizeof(T) == 2 && INTERP != 1 && CGS == 1 && NBUF == 2 && !SHIFTED_PLANES),
+                  "channel pairs: 16-bit bilinear or bicubic, one pair per stage, two slots");
     constexpr int PLANES = CHANNEL_PAIRS ? 2 : 1;  // planes that a "channel" of the block's channel loop stands for
     const int32_t plane_elems = H * W;
     const uint32_t plane_bytes = (uint32_t)plane_elems * (uint32_t)sizeof(T);

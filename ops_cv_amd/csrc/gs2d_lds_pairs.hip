@@ -5,10 +5,10 @@ namespace opscv {
 
 namespace {
 
-template <typename T, int PPT, int ADJ, int PITCH>
+template <typename T, int PPT, int ADJ, int PITCH, int INTERP = 0>
 hipError_t launch_pairs(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t stream)
 {
-    auto kernel = gs2d_lds_kernel<T, 0, kSamplerWaves, kPairsLoaderWaves, PPT, ADJ, 1, kPairsNbuf, PITCH, false, true>;
+    auto kernel = gs2d_lds_kernel<T, INTERP, kSamplerWaves, kPairsLoaderWaves, PPT, ADJ, 1, kPairsNbuf, PITCH, false, true>;
     static std::atomic<uint32_t> lds_allowed{0};
     const hipError_t ea = allow_dynamic_lds(reinterpret_cast<const void*>(kernel), kLdsLimit, lds_allowed);
     if (ea != hipSuccess) {
@@ -35,6 +35,15 @@ hipError_t launch_pairs_adj(const GridSamplerArgs& a, const LdsPlan& p, hipStrea
 template <typename T>
 hipError_t launch_pairs_typed(const GridSamplerArgs& a, const LdsPlan& p, hipStream_t stream)
 {
+    if (a.interp == 2) {  // bicubic: one or two pixels per lane, single stores
+        if (p.pairs_pitch == kPairsPitch && p.ppt == 2) {
+            return launch_pairs<T, 2, 1, kPairsPitch, 2>(a, p, stream);
+        }
+        if (p.pairs_pitch == kPairsPitch && p.ppt == 1) {
+            return launch_pairs<T, 1, 1, kPairsPitch, 2>(a, p, stream);
+        }
+        return hipErrorInvalidValue;
+    }
     if (p.pairs_pitch == kPairsPitch && p.ppt == 4) {
         return launch_pairs_adj<T, 4, kPairsPitch>(a, p, stream);
     }

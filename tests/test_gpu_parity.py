@@ -270,6 +270,54 @@ def test_grid_sampler_channel_pairs_in_lds(oracle, device, dtype, pad, align):
             _assert_same_bits(y2, y2_ref, what + " (second rule)")
 
 
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("pad", [0, 1, 2])
+@pytest.mark.parametrize("align", [False, True])
+def test_grid_sampler_bicubic_channel_pairs_in_lds(oracle, device, dtype, pad, align):
+    """bicubic samples (grid_sampler2_d_simt.h:362-458) of 16-bit planes of up to 8 KiB with an even channel count
+    through the ring kernel's interleaved stages (sixteen 4-byte reads per pixel serve two channels): one and two
+    pixels per lane, rows of 128 bytes and padded rows, a short last channel block, the uneven split of two workgroups
+    per CU; bit for bit against the oracle and against the same kernel with single-channel stages.  Reflection is the
+    padding that no pair-layout kernel takes, so there the automatic choice is checked as well."""
+    import torch
+    from ops_cv_amd import aclnn
+    rng = np.random.default_rng(2400 + pad * 10 + int(align))
+    shapes = [(16, 64, 64, 64, 64, 64), (16, 26, 64, 64, 20, 24), (32, 48, 25, 64, 64, 64), (8, 100, 62, 64, 33, 70),
+              (16, 256, 64, 64, 64, 64), (16, 64, 56, 56, 56, 56), (16, 96, 44, 48, 50, 60), (16, 128, 32, 128, 32, 128)]
+    pairs_seen = 0
+    for (N, C, H, W, Ho, Wo) in shapes:
+        x32 = rng.standard_normal((N, C, H, W)).astype(np.float32)
+        x32 += np.arange(C, dtype=np.float32).reshape(1, C, 1, 1)  # a channel taken for its neighbour shows
+        g32 = I.affine_grid(rng, N, Ho, Wo)
+        g32[N // 2] = rng.uniform(-1.3, 1.3, (Ho, Wo, 2)).astype(np.float32)
+        sv = I.special_grid_values()
+        k = min(sv.size, Wo)
+        g32[0, 0, :k, 0] = sv[:k]
+        g32[0, 1, :k, 1] = sv[:k]
+        x, g = I.cast_np(x32, dtype), I.cast_np(g32, dtype)
+        xt, gt = I.to_torch(x, dtype, device), I.to_torch(g, dtype, device)
+        what = "gs-bicubic-channel-pairs %s %s align=%s %s" % (dtype, PAD[pad], align, (N, C, H, W, Ho, Wo))
+        y_ref = oracle.grid_sampler2d(x, g, 2, pad, align, dtype=I.oracle_code(dtype))
+        for variant_option in ((2, 0) if pad == 2 else (2,)):
+            with aclnn.option("gs_variant", variant_option):
+                out = torch.empty((N, C, Ho, Wo), dtype=xt.dtype, device=device)
+                hs = [aclnn.tensor_handle(t) for t in (xt, gt, out)]
+                st, _, ex = aclnn.get_workspace_size_grid_sampler2d(hs[0], hs[1], 2, pad, align, hs[2])
+                assert st == 0
+                variant = aclnn.executor_variant(ex)
+                aclnn.destroy_executor(ex)
+                for h in hs:
+                    aclnn.destroy_tensor(h)
+                pairs_seen += int(variant.startswith("lds_ring_pairs"))
+                y = I.from_torch(aclnn.grid_sampler2d(xt, gt, 2, pad, align), dtype)
+            _check(y, y_ref, dtype, 2, what + " " + variant)
+            _assert_same_bits(y, y_ref, what + " " + variant)
+        with aclnn.option("gs_variant", 3):  # single-channel stages
+            y_single = I.from_torch(aclnn.grid_sampler2d(xt, gt, 2, pad, align), dtype)
+        _assert_same_bits(y, y_single, what + " (against single-channel stages)")
+    assert pairs_seen >= 6, pairs_seen
+
+
 @pytest.mark.parametrize("dtype", I.DTYPES)
 @pytest.mark.parametrize("interp", [0, 1])
 @pytest.mark.parametrize("pad", [0, 1, 2])

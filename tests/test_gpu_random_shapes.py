@@ -167,7 +167,7 @@ def test_random_grid_sampler2d_pair_layouts(oracle, device, aclnn):
 
 
 def test_random_grid_sampler2d_channel_pairs(oracle, device, aclnn):
-    """bilinear samples of 16-bit planes between 2 and 8 KiB with enough batch items and channels that the ring kernel
+    """bilinear and (every third case) bicubic samples of 16-bit planes between 2 and 8 KiB with enough batch items and channels that the ring kernel
     gives every channel block several channels: where that count is even it stages two channels at a time
     (interleaved in LDS), where it is odd or the rows get padded it does not -- checked all the same, and the
     variant that ran is counted so that the sweep cannot miss the interleaved stages.  Random row counts and widths,
@@ -183,7 +183,8 @@ def test_random_grid_sampler2d_channel_pairs(oracle, device, aclnn):
         H = int(rng.integers(max(2, 1100 // W), 4096 // W + 1))  # planes above the 2 KiB class, up to 8 KiB
         Ho, Wo = int(rng.integers(24, 80)), int(rng.integers(24, 80))
         pad, align = int(rng.integers(0, 3)), bool(rng.integers(0, 2))
-        _say("gs2d channel pairs", dtype, N, C, H, W, Ho, Wo, pad, align)
+        interp = 2 if case % 3 == 1 else 0
+        _say("gs2d channel pairs", dtype, N, C, H, W, Ho, Wo, interp, pad, align)
         x32 = rng.standard_normal((N, C, H, W)).astype(np.float32)
         x32 += np.arange(C, dtype=np.float32).reshape(1, C, 1, 1)
         x = I.cast_np(x32, dtype)
@@ -198,19 +199,19 @@ def test_random_grid_sampler2d_channel_pairs(oracle, device, aclnn):
         ty = torch.empty((N, C, Ho, Wo), dtype=tx.dtype, device=device)
         with aclnn.option("gs_variant", 2):  # the ring kernel also where a pair-layout variant would take the shape
             hs = [aclnn.tensor_handle(t) for t in (tx, tg, ty)]
-            st, _, ex = aclnn.get_workspace_size_grid_sampler2d(hs[0], hs[1], 0, pad, align, hs[2])
+            st, _, ex = aclnn.get_workspace_size_grid_sampler2d(hs[0], hs[1], interp, pad, align, hs[2])
             assert st == 0
             variant = aclnn.executor_variant(ex)
-            key = "pairs" if variant.startswith("lds_ring_pairs") else "other"
+            key = ("pairs" if variant.startswith("lds_ring_pairs") else "other") + ("_bicubic" if interp == 2 else "")
             seen[key] = seen.get(key, 0) + 1
             aclnn.destroy_executor(ex)
             for h in hs:
                 aclnn.destroy_tensor(h)
-            y = aclnn.grid_sampler2d(tx, tg, 0, pad, align, out=ty)
+            y = aclnn.grid_sampler2d(tx, tg, interp, pad, align, out=ty)
             torch.cuda.synchronize()
-        ref = oracle.grid_sampler2d(x, g, 0, pad, align, dtype=I.oracle_code(dtype))
-        _same(I.from_torch(y, dtype), ref, dtype, (case, dtype, N, C, H, W, Ho, Wo, pad, align, variant))
-    assert seen.get("pairs", 0) >= 8, seen
+        ref = oracle.grid_sampler2d(x, g, interp, pad, align, dtype=I.oracle_code(dtype))
+        _same(I.from_torch(y, dtype), ref, dtype, (case, dtype, N, C, H, W, Ho, Wo, interp, pad, align, variant))
+    assert seen.get("pairs", 0) >= 6 and seen.get("pairs_bicubic", 0) >= 3, seen
 
 
 def test_random_grid_sampler2d_large_planes(oracle, device, aclnn):
