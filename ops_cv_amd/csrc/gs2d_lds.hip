@@ -42,7 +42,9 @@ LdsPlan make_lds_plan(const GridSamplerArgs& a)
     // padded, 10.8 in pairs; rows of 80 elements 12.6 and 12.0; rows of 72, which shift by eight banks a row in the
     // interleaved layout, 13.1 and 14.3).
     const LdsPlan as_is = make_lds_plan_rows(a, false);
-    if (as_is.ok && as_is.chan_pairs && a.Win % 32 == 0) {
+    // (bicubic: sixteen reads per pixel and channel make the single-channel stages the slower choice whatever the rows:
+    // fp16 N16 C256 48x80 51.0 us padded, 35.4 in pairs; 50x72 51.8 and 42.2; border padding 64.9 and 37.3)
+    if (as_is.ok && as_is.chan_pairs && (a.Win % 32 == 0 || a.interp == 2)) {
         return as_is;
     }
     return padded.ok ? padded : as_is;
