@@ -465,7 +465,11 @@ constexpr int64_t kBicubicRingChannels = 32;  // 16 per block: 19.6 us against 1
 bool ring_before_pair(const GridSamplerArgs& a)
 {
     if (a.interp == 2) {
-        return a.pad == 0 && a.Hin * a.Win * 2 > 4096 && gs2d_lds_channel_pairs_per_block(a) >= kBicubicRingChannels;
+        // (planes above 8 KiB, whose pair layout leaves room for fewer workgroups: from 16 channels per block on -- fp16
+        // N16 C128 96x64 -> 96x64, 21 per block, 27.2 us against 41.9)
+        const int64_t plane_bytes = a.Hin * a.Win * 2;
+        const int64_t enough = plane_bytes > 8192 ? kBicubicRingChannels / 2 : kBicubicRingChannels;
+        return a.pad == 0 && plane_bytes > 4096 && gs2d_lds_channel_pairs_per_block(a) >= enough;
     }
     return a.interp == 0 && a.Hout * a.Wout <= 8 * a.Hin * a.Win && gs2d_lds_channel_pairs(a);
 }

@@ -205,7 +205,12 @@ static LdsPlan make_lds_plan_rows(const GridSamplerArgs& a, bool pad_rows)
         // pixel is the loaders' game, and theirs is the better one with the copy engine: 96x64 -> 96x64 24.0 and 27.1.
         const bool large = p.cls == 2 && p.ppt == 8 && 2 * staged_bytes + 16 <= kPairsPitchLarge &&
                            out_plane >= 2 * a.Hin * a.Win;
-        if (a.interp != 1 && esz == 2 && (small || (large && a.interp == 0)) && plain && p.copy_gran == 16 && a.C % 2 == 0 &&
+        // (bicubic in that class: one or two pixels per lane again, whatever the output's size -- the LDS reads set the
+        // pace there, not the loaders: fp16 N16 C256 96x80 -> 96x80 100.0 -> 63.7 us, border 181.9 -> 80.2; N16 C128
+        // 128x64 57.5 -> 33.7; rows of 80 elements padded to 128 in this class rather than interleaved as they are in
+        // the smaller one: 48x80 35.4 -> 32.6, 40x88 42.4 -> 31.4, border 37.3 -> 41.5 and 42.3 -> 37.5)
+        const bool large_bicubic = a.interp == 2 && p.cls == 2 && p.ppt <= 2 && 2 * staged_bytes + 16 <= kPairsPitchLarge;
+        if (a.interp != 1 && esz == 2 && (small || (large && a.interp == 0) || large_bicubic) && plain && p.copy_gran == 16 && a.C % 2 == 0 &&
             even_counts && a.force_variant != kGsRingSingle) {
             p.chan_pairs = true;
             p.pairs_pitch = small ? kPairsPitch : kPairsPitchLarge;

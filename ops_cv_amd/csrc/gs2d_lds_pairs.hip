@@ -1,4 +1,4 @@
-// LDS-staged grid sampler kernels with two channels per stage interleaved in LDS (16-bit elements, bilinear).
+// LDS-staged grid sampler kernels with two channels per stage interleaved in LDS (16-bit elements, bilinear and bicubic).
 #include "gs2d_lds_launch.hpp"
 
 namespace opscv {
@@ -41,6 +41,12 @@ hipError_t launch_pairs_typed(const GridSamplerArgs& a, const LdsPlan& p, hipStr
         }
         if (p.pairs_pitch == kPairsPitch && p.ppt == 1) {
             return launch_pairs<T, 1, 1, kPairsPitch, 2>(a, p, stream);
+        }
+        if (p.pairs_pitch == kPairsPitchLarge && p.ppt == 2) {
+            return launch_pairs<T, 2, 1, kPairsPitchLarge, 2>(a, p, stream);
+        }
+        if (p.pairs_pitch == kPairsPitchLarge && p.ppt == 1) {
+            return launch_pairs<T, 1, 1, kPairsPitchLarge, 2>(a, p, stream);
         }
         return hipErrorInvalidValue;
     }

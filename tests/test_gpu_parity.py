@@ -274,7 +274,7 @@ def test_grid_sampler_channel_pairs_in_lds(oracle, device, dtype, pad, align):
 @pytest.mark.parametrize("pad", [0, 1, 2])
 @pytest.mark.parametrize("align", [False, True])
 def test_grid_sampler_bicubic_channel_pairs_in_lds(oracle, device, dtype, pad, align):
-    """bicubic samples (grid_sampler2_d_simt.h:362-458) of 16-bit planes of up to 8 KiB with an even channel count
+    """bicubic samples (grid_sampler2_d_simt.h:362-458) of 16-bit planes of up to 16 KiB with an even channel count
     through the ring kernel's interleaved stages (sixteen 4-byte reads per pixel serve two channels): one and two
     pixels per lane, rows of 128 bytes and padded rows, a short last channel block, the uneven split of two workgroups
     per CU; bit for bit against the oracle and against the same kernel with single-channel stages.  Reflection is the
@@ -284,7 +284,8 @@ def test_grid_sampler_bicubic_channel_pairs_in_lds(oracle, device, dtype, pad, a
     rng = np.random.default_rng(2400 + pad * 10 + int(align))
     shapes = [(16, 64, 64, 64, 64, 64), (16, 26, 64, 64, 20, 24), (32, 48, 25, 64, 64, 64), (8, 100, 62, 64, 33, 70),
               (16, 256, 64, 64, 64, 64), (16, 64, 56, 56, 56, 56), (16, 96, 44, 48, 50, 60), (16, 128, 32, 128, 32, 128),
-              (16, 64, 48, 80, 40, 40), (16, 128, 50, 72, 60, 64)]  # rows of 160 and 144 bytes: interleaved as they are
+              (16, 64, 48, 80, 40, 40), (16, 128, 50, 72, 60, 64),  # rows of 160 and 144 bytes: interleaved as they are
+              (16, 64, 96, 64, 48, 64), (8, 32, 64, 128, 40, 50), (8, 64, 80, 96, 50, 70)]  # planes of the 16 KiB class
     pairs_seen = 0
     for (N, C, H, W, Ho, Wo) in shapes:
         x32 = rng.standard_normal((N, C, H, W)).astype(np.float32)
@@ -316,7 +317,7 @@ def test_grid_sampler_bicubic_channel_pairs_in_lds(oracle, device, dtype, pad, a
         with aclnn.option("gs_variant", 3):  # single-channel stages
             y_single = I.from_torch(aclnn.grid_sampler2d(xt, gt, 2, pad, align), dtype)
         _assert_same_bits(y, y_single, what + " (against single-channel stages)")
-    assert pairs_seen >= 8, pairs_seen
+    assert pairs_seen >= 9, pairs_seen
 
 
 @pytest.mark.parametrize("dtype", I.DTYPES)
