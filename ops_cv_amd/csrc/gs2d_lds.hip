@@ -143,6 +143,19 @@ static LdsPlan make_lds_plan_rows(const GridSamplerArgs& a, bool pad_rows)
             }
         }
     }
+    // Bicubic samples with two pixels per lane: sixteen tap offsets and sixteen tap values per pixel leave the CU room
+    // for one workgroup of this kernel (87 registers a lane), so 512 workgroups run as two rounds of 256, and every
+    // round pays the decisions of its pixels.  Where one workgroup per CU divides the channels evenly, that is the
+    // launch: fp16 N16 C256 64x64 -> 64x64 in channel pairs 29.1 -> 25.3 us (reflection 36.7 -> 31.9), N16 C128
+    // 64x128 33.3 -> 29.3, 128x64 33.7 -> 30.4.  (Other counts keep the finer blocks, which balance better than a
+    // round and a fraction: N16 C256 72x72, 176 (item, tile) pairs, 63.3 us with three blocks against 77.1 with two.)
+    if (a.interp == 2 && p.ppt == 2 && cgs == 1) {
+        const int64_t cus = compute_unit_count();
+        if (base <= cus && cus % base == 0 && a.C % (cus / base) == 0) {
+            cblocks = cus / base;
+            cpb = a.C / cblocks;
+        }
+    }
     p.chans_per_block = (int32_t)cpb;
     p.cblocks = (uint32_t)cblocks;
     if (a.N * p.tiles_per_n * cblocks > INT32_MAX) {
