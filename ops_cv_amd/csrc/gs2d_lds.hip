@@ -149,7 +149,11 @@ static LdsPlan make_lds_plan_rows(const GridSamplerArgs& a, bool pad_rows)
     // launch: fp16 N16 C256 64x64 -> 64x64 in channel pairs 29.1 -> 25.3 us (reflection 36.7 -> 31.9), N16 C128
     // 64x128 33.3 -> 29.3, 128x64 33.7 -> 30.4.  (Other counts keep the finer blocks, which balance better than a
     // round and a fraction: N16 C256 72x72, 176 (item, tile) pairs, 63.3 us with three blocks against 77.1 with two.)
-    if (a.interp == 2 && p.ppt == 2 && cgs == 1) {
+    // Likewise the bilinear channel pairs of the 16 KiB class (eight pixels per lane, 106 registers; the condition is
+    // the one under which the plan below takes them): bf16 N8 C128 64x128 -> 128x256 22.3 -> 18.7 us, fp16 N16 C128
+    // 38.7 -> 34.7, fp16 N16 C64 96x64 -> 256x128 20.9 -> 17.8.
+    const bool large_pairs = esz == 2 && a.interp == 0 && p.cls == 2 && p.ppt == 8 && out_plane >= 2 * a.Hin * a.Win;
+    if ((a.interp == 2 && p.ppt == 2 && cgs == 1) || large_pairs) {
         const int64_t cus = compute_unit_count();
         if (base <= cus && cus % base == 0 && a.C % (cus / base) == 0) {
             cblocks = cus / base;

@@ -234,7 +234,8 @@ def test_grid_sampler_channel_pairs_in_lds(oracle, device, dtype, pad, align):
     # planes of the 16 KiB class with two output pixels or more per input pixel)
     shapes = [(16, 64, 64, 64, 64, 64), (16, 26, 64, 64, 64, 64), (32, 48, 25, 64, 64, 64), (8, 100, 62, 64, 33, 70),
               (64, 12, 48, 64, 40, 40), (16, 256, 64, 64, 64, 64), (16, 64, 56, 56, 56, 56), (32, 48, 40, 40, 64, 64),
-              (16, 96, 44, 48, 50, 60), (16, 64, 96, 64, 192, 128), (8, 96, 64, 128, 100, 180)]
+              (16, 96, 44, 48, 50, 60), (16, 64, 96, 64, 192, 128), (8, 96, 64, 128, 100, 180),
+              (8, 32, 64, 128, 128, 256)]  # the last: 64 (item, tile) pairs, one workgroup per CU with 8 channels each
     for (N, C, H, W, Ho, Wo) in shapes:
         x32 = rng.standard_normal((N, C, H, W)).astype(np.float32)
         x32 += np.arange(C, dtype=np.float32).reshape(1, C, 1, 1)  # a channel taken for its neighbour shows
